@@ -1,0 +1,261 @@
+"""ctypes front end of the CPU oracle (``oracle/tract_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` as the checker; never by the product package.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libtract_oracle.so")
+
+FMT_Q8_0, FMT_Q4_0, FMT_Q8_1 = 2, 3, 4
+BLOCK_BYTES = {FMT_Q8_0: 34, FMT_Q4_0: 18, FMT_Q8_1: 36}
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (a few hundred ms)."""
+    src = os.path.join(_HERE, "tract_oracle.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-s", "-C", _HERE, "-B" if force else "-s"])
+    return _SO
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        L = C.CDLL(_SO)
+        sz, vp, i, f = C.c_size_t, C.c_void_p, C.c_int, C.c_float
+        L.orc_f32_to_f16.restype = C.c_uint16
+        L.orc_f32_to_f16.argtypes = [f]
+        L.orc_f16_to_f32.restype = f
+        L.orc_f16_to_f32.argtypes = [C.c_uint16]
+        L.orc_f32_to_f16_n.argtypes = [vp, vp, sz]
+        L.orc_f16_to_f32_n.argtypes = [vp, vp, sz]
+        L.orc_block_bytes.restype = sz
+        L.orc_block_bytes.argtypes = [i]
+        L.orc_quant.argtypes = [i, i, vp, sz, vp]
+        L.orc_dequant.argtypes = [i, i, vp, sz, vp]
+        L.orc_kv_new.restype = vp
+        L.orc_kv_new.argtypes = [sz, sz]
+        L.orc_kv_free.argtypes = [vp]
+        for n in ("len", "capacity", "reallocs"):
+            fn = getattr(L, "orc_kv_" + n)
+            fn.restype = sz
+            fn.argtypes = [vp]
+        L.orc_kv_buffer.restype = vp
+        L.orc_kv_buffer.argtypes = [vp]
+        L.orc_kv_push.argtypes = [vp, vp, sz]
+        L.orc_kv_valid_contiguous.argtypes = [vp, vp]
+        L.orc_concat_append.restype = vp
+        L.orc_concat_append.argtypes = [vp, sz, vp, sz, sz, sz]
+        L.orc_free.argtypes = [vp]
+        L.orc_flash_sdpa_f32.argtypes = [vp, vp, vp, vp] + [sz] * 6 + [sz] * 3 + [sz, sz, i, i, f, vp, i]
+        L.orc_flash_sdpa_eval_f16.argtypes = [vp, vp, vp, vp] + [sz] * 6 + [sz, sz, i, i, f, vp, i]
+        L.orc_naive_sdpa_f64.argtypes = [vp, vp, vp, vp] + [sz] * 6 + [sz, sz, i, i, f, vp]
+        L.orc_max_threads.restype = i
+        L.orc_decode_step_f16.argtypes = [vp] * 5 + [sz] * 5 + [i, vp, C.POINTER(vp), C.POINTER(vp)]
+        _lib = L
+    return _lib
+
+
+def _p(a: np.ndarray | None):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+# ----------------------------------------------------------------------------- f16
+def f32_to_f16_bits(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    lib().orc_f32_to_f16_n(_p(x), _p(out), x.size)
+    return out
+
+
+def f16_bits_to_f32(h: np.ndarray) -> np.ndarray:
+    h = np.ascontiguousarray(h, dtype=np.uint16)
+    out = np.empty(h.shape, dtype=np.float32)
+    lib().orc_f16_to_f32_n(_p(h), _p(out), h.size)
+    return out
+
+
+# ----------------------------------------------------------------------------- block quant
+def quant(fmt: int, x: np.ndarray) -> np.ndarray:
+    """BlockQuant::quant_f32 / quant_f16: blocks of 32 along the last axis.
+
+    Returns uint8 array of shape x.shape[:-1] + (D/32 * block_bytes,)."""
+    assert x.dtype in (np.float32, np.float16) and x.shape[-1] % 32 == 0
+    x = np.ascontiguousarray(x)
+    bb = BLOCK_BYTES[fmt]
+    out = np.empty(x.shape[:-1] + (x.shape[-1] // 32 * bb,), dtype=np.uint8)
+    rc = lib().orc_quant(fmt, int(x.dtype == np.float16), _p(x), x.size, _p(out))
+    assert rc == 0
+    return out
+
+
+def dequant(fmt: int, q: np.ndarray, dtype=np.float32) -> np.ndarray:
+    """BlockQuant::dequant_f32 / dequant_f16 of a canonical block byte array."""
+    q = np.ascontiguousarray(q, dtype=np.uint8)
+    bb = BLOCK_BYTES[fmt]
+    assert q.shape[-1] % bb == 0
+    d = q.shape[-1] // bb * 32
+    out = np.empty(q.shape[:-1] + (d,), dtype=dtype)
+    rc = lib().orc_dequant(fmt, int(dtype == np.float16), _p(q), out.size, _p(out))
+    assert rc == 0
+    return out
+
+
+# ----------------------------------------------------------------------------- kv cache
+class InPlaceKvCache:
+    """InPlaceKvCache (inplace_kv_cache.rs:28-114) over numpy arrays; `axis` is the
+    sequence axis of the pushed tensors."""
+
+    def __init__(self, axis: int):
+        self.axis = axis
+        self._h = None
+        self._shape = None
+        self._dtype = None
+
+    def push(self, x: np.ndarray) -> None:
+        x = np.ascontiguousarray(x)
+        if self._h is None:
+            outer = int(np.prod(x.shape[: self.axis], dtype=np.int64))
+            inner = int(np.prod(x.shape[self.axis + 1:], dtype=np.int64)) * x.dtype.itemsize
+            self._h = lib().orc_kv_new(outer, inner)
+            self._shape, self._dtype = list(x.shape), x.dtype
+        assert x.dtype == self._dtype
+        assert lib().orc_kv_push(self._h, _p(x), x.shape[self.axis]) == 0
+
+    def len(self) -> int:
+        return 0 if self._h is None else lib().orc_kv_len(self._h)
+
+    def capacity(self) -> int:
+        return 0 if self._h is None else lib().orc_kv_capacity(self._h)
+
+    def reallocs(self) -> int:
+        return 0 if self._h is None else lib().orc_kv_reallocs(self._h)
+
+    def valid_contiguous(self) -> np.ndarray:
+        shape = list(self._shape)
+        shape[self.axis] = self.len()
+        out = np.empty(shape, dtype=self._dtype)
+        lib().orc_kv_valid_contiguous(self._h, _p(out))
+        return out
+
+    def __del__(self):
+        if self._h is not None and _lib is not None:
+            _lib.orc_kv_free(self._h)
+            self._h = None
+
+
+def concat_append(past: np.ndarray | None, new: np.ndarray, axis: int) -> np.ndarray:
+    """DynKeyValueCacheState::eval (dyn_kv_cache.rs:158-174): fresh concat."""
+    new = np.ascontiguousarray(new)
+    if past is None:
+        return new.copy()
+    past = np.ascontiguousarray(past)
+    outer = int(np.prod(new.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(new.shape[axis + 1:], dtype=np.int64)) * new.dtype.itemsize
+    ptr = lib().orc_concat_append(_p(past), past.shape[axis], _p(new), new.shape[axis], outer, inner)
+    shape = list(new.shape)
+    shape[axis] = past.shape[axis] + new.shape[axis]
+    n = int(np.prod(shape, dtype=np.int64)) * new.dtype.itemsize
+    out = np.frombuffer(C.string_at(ptr, n), dtype=new.dtype).reshape(shape).copy()
+    lib().orc_free(ptr)
+    return out
+
+
+# ----------------------------------------------------------------------------- attention
+def _as4(q, k, v, mask):
+    r3 = q.ndim == 3
+    if r3:
+        q, k, v = q[:, None], k[:, None], v[:, None]
+        if mask is not None:
+            mask = mask[:, None]
+    return q, k, v, mask, r3
+
+
+def flash_sdpa(q, k, v, mask=None, causal=False, scale=None, threads=1):
+    """FlashSdpaOp::eval (flash_sdpa.rs:103-163).  f32 or f16 inputs (rank 3 or 4);
+    output has Q's shape and dtype."""
+    q, k, v, mask, r3 = _as4(q, k, v, mask)
+    B, Hq, Sq, D = q.shape
+    _, Hkv, Sk, _ = k.shape
+    mb, mh = (mask.shape[0], mask.shape[1]) if mask is not None else (1, 1)
+    if mask is not None:
+        mask = np.ascontiguousarray(np.broadcast_to(mask, (mb, mh, Sq, Sk)))
+    hs, sc = (0, 0.0) if scale is None else (1, float(scale))
+    if q.dtype == np.float16:
+        qq, kk, vv = (np.ascontiguousarray(a, dtype=np.float16) for a in (q, k, v))
+        mm = None if mask is None else np.ascontiguousarray(mask, dtype=np.float16)
+        out = np.empty(q.shape, dtype=np.float16)
+        lib().orc_flash_sdpa_eval_f16(_p(qq), _p(kk), _p(vv), _p(mm), B, Hq, Hkv, Sq, Sk, D, mb, mh,
+                                      int(causal), hs, sc, _p(out), threads)
+    else:
+        qq, kk, vv = (np.ascontiguousarray(a, dtype=np.float32) for a in (q, k, v))
+        mm = None if mask is None else np.ascontiguousarray(mask, dtype=np.float32)
+        out = np.empty(q.shape, dtype=np.float32)
+        lib().orc_flash_sdpa_f32(_p(qq), _p(kk), _p(vv), _p(mm), B, Hq, Hkv, Sq, Sk, D,
+                                 Hkv * Sk * D, Sk * D, D, mb, mh, int(causal), hs, sc, _p(out), threads)
+    return out[:, 0] if r3 else out
+
+
+def flash_sdpa_view(q, kbuf, vbuf, length, causal=False, scale=None, threads=1):
+    """flash_attention_gqa over zero-copy [0..length] views of capacity buffers
+    [B,Hkv,cap,D] f32 — what InPlaceKvSdpaState::eval does (inplace_kv_cache.rs:191-216)."""
+    B, Hq, Sq, D = q.shape
+    _, Hkv, cap, _ = kbuf.shape
+    assert kbuf.dtype == np.float32 and kbuf.flags.c_contiguous and vbuf.flags.c_contiguous
+    qq = np.ascontiguousarray(q, dtype=np.float32)
+    out = np.empty(q.shape, dtype=np.float32)
+    hs, sc = (0, 0.0) if scale is None else (1, float(scale))
+    lib().orc_flash_sdpa_f32(_p(qq), _p(kbuf), _p(vbuf), None, B, Hq, Hkv, Sq, length, D,
+                             Hkv * cap * D, cap * D, D, 1, 1, int(causal), hs, sc, _p(out), threads)
+    return out
+
+
+def naive_sdpa_f64(q, k, v, mask=None, causal=False, scale=None):
+    """Textbook softmax(QK^T*scale+mask)V in f64 over the f32 images of the inputs."""
+    q, k, v, mask, r3 = _as4(q, k, v, mask)
+    B, Hq, Sq, D = q.shape
+    _, Hkv, Sk, _ = k.shape
+    mb, mh = (mask.shape[0], mask.shape[1]) if mask is not None else (1, 1)
+    qq, kk, vv = (np.ascontiguousarray(a, dtype=np.float32) for a in (q, k, v))
+    mm = None
+    if mask is not None:
+        mm = np.ascontiguousarray(np.broadcast_to(mask, (mb, mh, Sq, Sk)), dtype=np.float32)
+    out = np.empty(q.shape, dtype=np.float64)
+    hs, sc = (0, 0.0) if scale is None else (1, float(scale))
+    lib().orc_naive_sdpa_f64(_p(qq), _p(kk), _p(vv), _p(mm), B, Hq, Hkv, Sq, Sk, D, mb, mh,
+                             int(causal), hs, sc, _p(out))
+    return out[:, 0] if r3 else out
+
+
+def decode_step_f16(q, k_past, v_past, k_new, v_new, threads=1):
+    """One decode step of the reference's default CPU path with its costs (concat
+    reallocation of K and V, whole-tensor f32 casts).  Returns (out, K, V)."""
+    B, Hq, _, D = q.shape
+    _, Hkv, T, _ = k_past.shape
+    out = np.empty(q.shape, dtype=np.float16)
+    kp, vp = C.c_void_p(), C.c_void_p()
+    lib().orc_decode_step_f16(_p(q), _p(k_past), _p(v_past), _p(k_new), _p(v_new), B, Hq, Hkv, T, D,
+                              threads, _p(out), C.byref(kp), C.byref(vp))
+    n = B * Hkv * (T + 1) * D
+    k = np.ctypeslib.as_array(C.cast(kp, C.POINTER(C.c_uint16)), shape=(n,)).view(np.float16).reshape(B, Hkv, T + 1, D).copy()
+    v = np.ctypeslib.as_array(C.cast(vp, C.POINTER(C.c_uint16)), shape=(n,)).view(np.float16).reshape(B, Hkv, T + 1, D).copy()
+    lib().orc_free(kp)
+    lib().orc_free(vp)
+    return out, k, v
+
+
+def max_threads() -> int:
+    return lib().orc_max_threads()
