@@ -1,0 +1,190 @@
+/*
+ * tract_rocm.h — C ABI of the MI355X (gfx950) KV-cache + attention path.
+ *
+ * This is the surface a `tract-rocm` runtime crate binds through FFI: plain
+ * pointers, sizes and integer handles, no C++ or framework types.  Each entry point
+ * names the interface of the tract tree it stands in for (paths relative to the
+ * tract source tree, version 0.23.6-pre).
+ *
+ * Conventions
+ *  - Every call returns 0 on success and 1 on failure; the message of the last
+ *    failure on the calling thread is returned by trocm_last_error() and stays
+ *    valid until the next failing call on that thread (same contract as tract's own
+ *    C API, api/ffi/src/lib.rs:18-62).  Null pointers are reported, never
+ *    dereferenced (api/ffi/src/lib.rs:83-92).
+ *  - `stream` is a hipStream_t passed as void*.  Work is asynchronous and ordered by
+ *    stream, one stream per host thread like cuda/src/context.rs:37-43.  NULL selects
+ *    the library's own per-thread stream, never the legacy default stream.
+ *  - Tensors are device pointers.  Shapes follow tract's attention layout
+ *    [batch, heads, tokens, head_dim] with head_dim contiguous; rank-3 tensors are
+ *    the heads == 1 case.  Strides are in elements unless the name says bytes.
+ *  - All entry points may be called from several threads at once on distinct
+ *    streams, caches and workspaces.
+ */
+#ifndef TRACT_ROCM_H
+#define TRACT_ROCM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
+
+/* Element / storage formats.  Q8_0 and Q4_0 are 32-element blocks along head_dim
+ * with one f16 scale per block (canonical block bytes: linalg/src/frame/block_quant/
+ * q4_0.rs:19-45, and q8_1.rs:20-48 without its `sum` field). */
+typedef enum {
+    TROCM_F32 = 0,
+    TROCM_F16 = 1,
+    TROCM_Q8_0 = 2,
+    TROCM_Q4_0 = 3
+} trocm_dtype;
+
+/* ---- runtime ------------------------------------------------------------------ */
+
+/* Select `device` and create the library context; idempotent.  Stands in for
+ * cuda_context() (cuda/src/context.rs:28-35) / Runtime::check (core/src/runtime.rs:23-34). */
+int trocm_init(int device);
+
+/* Message of the last failing call on this thread (api/ffi/src/lib.rs:44-62). */
+const char *trocm_last_error(void);
+
+/* Device properties useful to a caller's scheduler: compute units, bytes of HBM. */
+int trocm_device_info(int *compute_units, size_t *hbm_bytes, char *name, size_t name_len);
+
+/* ---- device memory and streams: DeviceContext (gpu/src/device.rs:13-35) ---------- */
+
+/* uninitialized_device_tensor (gpu/src/device.rs:15-19): 256-byte aligned device memory. */
+int trocm_malloc(void **ptr, size_t bytes);
+int trocm_free(void *ptr);
+/* tensor_to_device (gpu/src/device.rs:14) / DeviceTensor::to_host (gpu/src/tensor/mod.rs:180-187).
+ * Asynchronous on `stream`; the host buffer must stay alive until the stream is synchronised. */
+int trocm_h2d(void *dst_device, const void *src_host, size_t bytes, void *stream);
+int trocm_d2h(void *dst_host, const void *src_device, size_t bytes, void *stream);
+int trocm_memset(void *dst_device, int byte_value, size_t bytes, void *stream);
+int trocm_stream_create(void **stream);
+int trocm_stream_destroy(void *stream);
+/* DeviceContext::synchronize (gpu/src/device.rs:25) for one stream / for the device. */
+int trocm_stream_sync(void *stream);
+int trocm_device_sync(void);
+
+/* DeviceContext::copy_nd (gpu/src/device.rs:26-35; CUDA: cuda/src/kernels/array/dispatch.rs:11-46):
+ * strided N-d copy, rank 1..6, elem_size 1/2/4/8/16 bytes, strides in elements (may be
+ * 0 for broadcast sources, never negative), byte offsets added to the base pointers. */
+int trocm_copy_nd(void *dst, size_t dst_offset_bytes, const int64_t *dst_strides, const void *src,
+                  size_t src_offset_bytes, const int64_t *src_strides, const int64_t *shape, int rank,
+                  int elem_size, void *stream);
+
+/* ---- in-place KV cache: InPlaceKvCache (transformers/src/ops/inplace_kv_cache.rs:28-114),
+ *      replacing GpuDynKVCacheState::eval's reallocate-and-concat (gpu/src/ops/dyn_kv_cache.rs:58-113)
+ *
+ * One cache holds one tensor (K or V) of logical shape [batch, kv_heads, len, head_dim]
+ * in a device buffer of `capacity` tokens.  Storage formats:
+ *   F32/F16  [batch, kv_heads, capacity, head_dim]
+ *   Q8_0     codes [batch, kv_heads, capacity, head_dim] int8  + scales [.., capacity, head_dim/32] f16
+ *   Q4_0     codes [batch, kv_heads, capacity, head_dim/2] (16 canonical nibble bytes per block)
+ *            + scales [.., capacity, head_dim/32] f16
+ * The device layout of the quantised formats is private; trocm_kv_export() emits the
+ * canonical block bytes (scale then codes, blocks row-major along head_dim). */
+typedef struct trocm_kv_cache trocm_kv_cache;
+
+/* InPlaceKvCache::new (:37-39).  Allocates nothing until the first append or reserve. */
+int trocm_kv_cache_create(trocm_kv_cache **out, int storage_format, int64_t batch, int64_t kv_heads,
+                          int64_t head_dim);
+int trocm_kv_cache_destroy(trocm_kv_cache *cache);
+/* len() / capacity() / reallocs() (:41-53). */
+int trocm_kv_cache_len(const trocm_kv_cache *cache, int64_t *len);
+int trocm_kv_cache_capacity(const trocm_kv_cache *cache, int64_t *capacity);
+int trocm_kv_cache_reallocs(const trocm_kv_cache *cache, int64_t *reallocs);
+/* Pre-allocate room for `capacity` tokens (no counterpart in the CPU op, whose Vec-like
+ * growth starts from the first chunk; a device caller that knows its context budget
+ * avoids every later reallocation).  Never shrinks; keeps the valid region. */
+int trocm_kv_cache_reserve(trocm_kv_cache *cache, int64_t capacity, void *stream);
+/* push (:55-85): append `n_new` tokens read from `src` ([batch, kv_heads, n_new, head_dim]
+ * of src_dtype F32 or F16, element strides src_strides[4]; fused Move views are legal inputs
+ * of the device cache op, cuda/src/rewrite_rules/fuse_axis_op.rs:13-27).  Growth rule (:61-80):
+ * first chunk seeds capacity = n_new; else if len+n_new > capacity the buffer is replaced by
+ * one of max(2*capacity, len+n_new) tokens holding the valid region.  A quantised cache
+ * quantises on the way in; an F32/F16 cache requires src_dtype == storage_format. */
+int trocm_kv_append(trocm_kv_cache *cache, const void *src, int src_dtype, const int64_t *src_strides,
+                    int64_t n_new, void *stream);
+/* DynKeyValueCacheState::truncate (transformers/src/ops/dyn_kv_cache.rs:112-119): keep the first
+ * `len` tokens (speculative-decoding rollback).  Fails on an empty cache like the reference. */
+int trocm_kv_cache_truncate(trocm_kv_cache *cache, int64_t len);
+/* valid_contiguous (:100-103) / OpState::save_to (:222-228): write the valid region, dense,
+ * to `dst_device`: [batch, kv_heads, len, row_bytes] with row_bytes = trocm_kv_row_bytes(). */
+int trocm_kv_export(const trocm_kv_cache *cache, void *dst_device, void *stream);
+/* Bytes of one token of one head in the canonical export: head_dim*4, head_dim*2,
+ * head_dim/32*34 or head_dim/32*18. */
+int trocm_kv_row_bytes(const trocm_kv_cache *cache, size_t *bytes);
+/* OpStateFreeze::freeze (:262-272): an independent deep copy (same len, capacity = len). */
+int trocm_kv_cache_clone(const trocm_kv_cache *cache, trocm_kv_cache **out, void *stream);
+/* Raw view for kernels written against the cache: base pointers and capacity.
+ * `scales` is NULL for F32/F16. */
+int trocm_kv_cache_raw(const trocm_kv_cache *cache, void **data, void **scales, int64_t *capacity);
+
+/* ---- block quantisation as a tensor op: BlockQuant::{quant_f32,quant_f16,dequant_f32,dequant_f16}
+ *      (linalg/src/frame/block_quant/mod.rs:48-108) ------------------------------------------- */
+
+/* `n_elems` (multiple of 32) contiguous elements -> canonical blocks. */
+int trocm_block_quant(int format, const void *src, int src_dtype, size_t n_elems, void *dst_blocks,
+                      void *stream);
+int trocm_block_dequant(int format, const void *src_blocks, size_t n_elems, void *dst, int dst_dtype,
+                        void *stream);
+
+/* ---- attention -------------------------------------------------------------------------- */
+
+/* Scratch for split-K partial results and arrival counters.  The arena planner of the
+ * device layer does not model scratch (gpu/src/memory/schema.rs:56-128), so the op state
+ * owns one workspace and passes it to every call.  trocm_sdpa_workspace_init() must run
+ * once on a new workspace (it zeroes the counters); kernels leave it ready for the next
+ * call.  Two calls that overlap in time must not share a workspace. */
+int trocm_sdpa_workspace_bytes(int64_t batch, int64_t q_heads, int64_t q_len, int64_t head_dim,
+                               size_t *bytes);
+int trocm_sdpa_workspace_init(void *workspace, size_t bytes, void *stream);
+
+/* Sdpa (transformers/src/ops/sdpa.rs:83-89, semantics :131-227; CUDA dispatch
+ * cuda/src/kernels/flash_attn.rs:82-189): out = softmax(q k^T * scale + mask) v.
+ *   q, out : [batch, q_heads, q_len, head_dim] dense, dtype `dtype` (F32 or F16)
+ *   k, v   : [batch, kv_heads, kv_len, head_dim] of the same dtype, element strides
+ *            kv_strides[3] for batch, head, token (head_dim contiguous); q_heads must
+ *            be a multiple of kv_heads, kv head = q head / group (sdpa.rs:156-164)
+ *   mask   : optional additive [mask_batch, mask_heads, q_len, kv_len] dense, of `dtype`,
+ *            mask_batch in {1, batch}, mask_heads in {1, q_heads}; must be NULL when causal
+ *            (sdpa.rs:297-299)
+ *   scale  : NaN selects the default 1/sqrt(head_dim) (sdpa.rs:177-181)
+ *   causal : key j visible to query i iff j <= i + (kv_len - q_len) (flash_sdpa.rs:279-288) */
+int trocm_sdpa(const void *q, const void *k, const void *v, const void *mask, void *out, int dtype,
+               int64_t batch, int64_t q_heads, int64_t kv_heads, int64_t q_len, int64_t kv_len,
+               int64_t head_dim, const int64_t *kv_strides, int64_t mask_batch, int64_t mask_heads,
+               float scale, int causal, void *workspace, size_t workspace_bytes, void *stream);
+
+/* The consumer half of InPlaceKvSdpaState::eval (inplace_kv_cache.rs:191-216): attention of
+ * q over the valid [0..len] region of a K cache and a V cache, read in place (the device
+ * twin of valid_view, :90-95), with fused dequantisation for Q8_0/Q4_0 caches.
+ * q, out: [batch, q_heads, q_len, head_dim] dense of q_dtype (F32 or F16). */
+int trocm_sdpa_cached(const void *q, int q_dtype, int64_t q_heads, int64_t q_len,
+                      const trocm_kv_cache *k_cache, const trocm_kv_cache *v_cache, void *out,
+                      float scale, int causal, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Ragged multi-sequence decode: `n_seq` independent sequences, each with its own K and V
+ * cache (batch == 1 each, same heads/head_dim/format) and its own length; one query token
+ * per sequence.  q, out: [n_seq, q_heads, 1, head_dim].  The reference has no ragged batch:
+ * its statement of the same result is a dense batch padded to the longest sequence with an
+ * additive mask whose padded columns are <= -65504 (flash_sdpa.rs:261-268). */
+int trocm_sdpa_decode_ragged(const void *q, int q_dtype, int64_t q_heads, int64_t n_seq,
+                             trocm_kv_cache *const *k_caches, trocm_kv_cache *const *v_caches,
+                             void *out, float scale, void *workspace, size_t workspace_bytes,
+                             void *stream);
+
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRACT_ROCM_H */

@@ -1,0 +1,52 @@
+"""CPU-side checks of the boundary: the shared library loads without a GPU and exports
+every symbol that include/tract_rocm.h declares; the host mirror refuses to run without
+the device instead of falling back."""
+import os
+import re
+import subprocess
+
+import pytest
+
+from tests.conftest import ROOT
+
+
+def _header_symbols():
+    text = open(os.path.join(ROOT, "include", "tract_rocm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(trocm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from tract_amd import _lib
+    lib = _lib.load()
+    names = _header_symbols()
+    assert len(names) >= 30
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in tract_rocm.h but not exported"
+    assert set(_lib.SIGNATURES) == set(names)
+    out = subprocess.check_output(["nm", "-D", "--defined-only", _lib.LIB_PATH], text=True)
+    exported = set(re.findall(r" T (trocm_[a-z0-9_]+)", out))
+    assert exported == set(names)
+
+
+def test_header_is_plain_c():
+    src = '#include "tract_rocm.h"\nint main(void){return (int)sizeof(trocm_dtype) == 0;}\n'
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"), "-x", "c", "-",
+                    "-fsyntax-only"], input=src, text=True, check=True)
+
+
+def test_error_convention_without_device():
+    import tract_amd
+    from tract_amd import _lib
+    lib = _lib.load()
+    if lib.trocm_init(0) == 0:
+        pytest.skip("GPU present")
+    # KO + message, and no fallback path: the runtime cannot be created
+    assert b"HIP device" in lib.trocm_last_error()
+    with pytest.raises(tract_amd.TractRocmError):
+        tract_amd.runtime_for_name("rocm")
+    with pytest.raises(tract_amd.TractRocmError):
+        tract_amd.runtime_for_name("cuda")
+    # null pointers are reported, never dereferenced
+    assert lib.trocm_kv_cache_len(None, None) == 1
+    assert b"null pointer" in lib.trocm_last_error()

@@ -1,0 +1,176 @@
+"""Attention on the GPU vs the oracle (FlashSdpaOp restatement) and the f64 textbook
+form.  Tolerances are the path's contract: max-abs 1e-3 for f32, 2e-2 for f16."""
+import os
+
+import numpy as np
+import pytest
+
+import tract_amd
+from oracle import oracle as orc
+from tests import cases
+from tests.gpu_util import max_abs, rt  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.dtype(np.float32): 1e-3, np.dtype(np.float16): 2e-2}
+
+
+@pytest.mark.parametrize("name", sorted(cases.sdpa_literal_cases()))
+def test_literal_suite_cases(rt, name):
+    q, k, v, mask, scale, causal = cases.sdpa_literal_cases()[name]
+    got = tract_amd.Sdpa(scale=scale, datum_type=q.dtype, is_causal=causal).eval(q, k, v, mask).to_numpy()
+    want = orc.flash_sdpa(q, k, v, mask=mask, causal=causal, scale=scale)
+    assert got.dtype == q.dtype and got.shape == want.shape
+    assert max_abs(got, want) <= TOL[q.dtype]
+    assert max_abs(got, cases.textbook_sdpa(q, k, v, mask, scale, causal)) <= TOL[q.dtype]
+
+
+@pytest.mark.parametrize("name,causal,scale", [("simple-causal-f32", True, None), ("simple-non-causal-f32", False, None),
+                                               ("simple-scale-f32", False, 1.3)])
+def test_reference_golden_f32(rt, golden_dir, name, causal, scale):
+    z = np.load(os.path.join(golden_dir, "ref_sdpa", name, "io.npz"))
+    x = z["input_0"]
+    got = tract_amd.Sdpa(scale=scale, is_causal=causal).eval(x, x, x).to_numpy()
+    assert max_abs(got, z["output_0"]) <= 1e-5
+
+
+def test_reference_golden_mask_and_f16(rt, golden_dir):
+    d = os.path.join(golden_dir, "ref_sdpa")
+    z = np.load(os.path.join(d, "simple-mask-f32", "io.npz"))
+    raw = np.fromfile(os.path.join(d, "simple-mask-f32", "v0.dat"), dtype=np.uint8)
+    mask = np.ascontiguousarray(np.broadcast_to(raw[128:].view(np.float32).reshape(1, 2, 1), (1, 2, 2)))
+    got = tract_amd.Sdpa().eval(z["input_0"], z["input_1"], z["input_2"], mask).to_numpy()
+    assert max_abs(got, z["output_0"]) <= 1e-5
+    z = np.load(os.path.join(d, "simple-f16", "io.npz"))
+    x = z["input_0"].astype(np.float16)
+    got = tract_amd.Sdpa(datum_type=np.float16).eval(x, x, x).to_numpy()
+    assert max_abs(got, z["output_0"]) <= 2e-3
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal", [
+    (1, 2, 2, 16, 24, 8, False), (1, 4, 2, 1, 33, 8, True), (2, 8, 2, 70, 70, 16, True),
+    (1, 4, 1, 5, 133, 64, True), (2, 6, 3, 40, 97, 32, False), (1, 3, 1, 2, 300, 80, True),
+])
+def test_generic_shapes(rt, dt, B, Hq, Hkv, Sq, Sk, D, causal):
+    rng = np.random.default_rng(7)
+    q = rng.standard_normal((B, Hq, Sq, D), dtype=np.float32).astype(dt)
+    k = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(dt)
+    v = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(dt)
+    got = tract_amd.Sdpa(datum_type=dt, is_causal=causal).eval(q, k, v).to_numpy()
+    assert max_abs(got, orc.flash_sdpa(q, k, v, causal=causal)) <= TOL[np.dtype(dt)]
+    assert max_abs(got, cases.textbook_sdpa(q, k, v, causal=causal)) <= TOL[np.dtype(dt)]
+
+
+def test_padding_mask_equals_shorter_sequence(rt):
+    rng = np.random.default_rng(8)
+    B, Hq, Hkv, Sq, Sk, D = 2, 4, 2, 3, 80, 16
+    q = rng.standard_normal((B, Hq, Sq, D), dtype=np.float32)
+    k = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32)
+    v = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32)
+    lens = [50, 80]
+    mask = np.zeros((B, 1, Sq, Sk), dtype=np.float32)
+    for b, n in enumerate(lens):
+        mask[b, :, :, n:] = np.finfo(np.float32).min
+    got = tract_amd.Sdpa().eval(q, k, v, mask).to_numpy()
+    assert max_abs(got, orc.flash_sdpa(q, k, v, mask=mask)) <= 1e-3
+    for b, n in enumerate(lens):
+        assert max_abs(got[b:b + 1], cases.textbook_sdpa(q[b:b + 1], k[b:b + 1, :, :n], v[b:b + 1, :, :n])) <= 1e-5
+
+
+@pytest.mark.parametrize("dt,B,Hq,Hkv,D,T", [
+    (np.float16, 1, 32, 8, 128, 1), (np.float16, 1, 32, 8, 128, 31), (np.float16, 1, 32, 8, 128, 32),
+    (np.float16, 2, 32, 8, 128, 33), (np.float16, 1, 32, 8, 128, 1000), (np.float16, 2, 32, 8, 128, 4097),
+    (np.float32, 1, 32, 32, 64, 1), (np.float32, 1, 32, 32, 64, 255), (np.float32, 2, 8, 4, 64, 513),
+    (np.float16, 1, 8, 8, 64, 300), (np.float16, 1, 16, 2, 64, 777), (np.float32, 1, 4, 2, 128, 200),
+    (np.float16, 3, 8, 4, 128, 129), (np.float16, 1, 6, 2, 128, 100), (np.float16, 1, 8, 8, 96, 64),
+])
+def test_decode_split_k(rt, dt, B, Hq, Hkv, D, T):
+    """Sq == 1 through the split-K kernel (and the generic one where no fast kernel fits),
+    on caches with spare capacity (the tail holds NaN and must never be read)."""
+    rng = np.random.default_rng(100 + T)
+    q = (rng.standard_normal((B, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(dt)
+    k = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(dt)
+    v = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(dt)
+    st = tract_amd.InPlaceKvSdpa(axis=2, causal=True).state()
+    cap = T + 37
+    for c in (st.k, st.v):
+        c.reserve(cap, like=(k.shape, k.dtype))
+        import ctypes as C
+        from tract_amd._lib import call
+        data = C.c_void_p()
+        call("trocm_kv_cache_raw", c.handle, C.byref(data), None, None)
+        call("trocm_memset", data, 0xFF, B * Hkv * cap * D * np.dtype(dt).itemsize, None)  # NaN fill
+    out = st.eval([q, k, v]).to_numpy()
+    want = orc.flash_sdpa(q, k, v, causal=True)
+    assert not np.isnan(out).any()
+    assert max_abs(out, want) <= TOL[np.dtype(dt)]
+    assert max_abs(out, cases.textbook_sdpa(q, k, v, causal=True)) <= (2e-3 if dt == np.float16 else 2e-5)
+
+
+@pytest.mark.parametrize("splits", [1, 2, 3, 7, 64])
+def test_decode_any_split_count_agrees(rt, splits, monkeypatch):
+    # The split merge is exact in real arithmetic (log-sum-exp identity).
+    import subprocess, sys, json
+    code = f"""
+import os, json, numpy as np
+os.environ['TROCM_DECODE_SPLITS']='{splits}'
+import tract_amd
+tract_amd.runtime_for_name('rocm')
+rng=np.random.default_rng(5)
+q=(rng.standard_normal((2,32,1,128),dtype=np.float32)/11.3).astype(np.float16)
+k=rng.standard_normal((2,8,3000,128),dtype=np.float32).astype(np.float16)
+v=rng.standard_normal((2,8,3000,128),dtype=np.float32).astype(np.float16)
+st=tract_amd.InPlaceKvSdpa(2,True).state()
+o=st.eval([q,k,v]).to_numpy()
+print(json.dumps(o.astype(np.float32).reshape(-1).tolist()))
+"""
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, check=True,
+                         cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__)))).stdout
+    got = np.array(json.loads(out.strip().splitlines()[-1]), dtype=np.float32).reshape(2, 32, 1, 128)
+    rng = np.random.default_rng(5)
+    q = (rng.standard_normal((2, 32, 1, 128), dtype=np.float32) / 11.3).astype(np.float16)
+    k = rng.standard_normal((2, 8, 3000, 128), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((2, 8, 3000, 128), dtype=np.float32).astype(np.float16)
+    assert max_abs(got, cases.textbook_sdpa(q, k, v)) <= 2e-3
+
+
+def test_inplace_kv_sdpa_decode_loop_cfg1(rt):
+    """cfg1: B=1, 32 q heads = 32 kv heads, D=64, f32, cache grows 0 -> 256 one token per
+    step with causal attention at each step; fused op vs {concat cache, FlashSdpaOp}."""
+    B, H, D, T = 1, 32, 64, 256
+    q = cases.seeded_normal(cases.cfg_seed(1, "q"), (T, B, H, 1, D))
+    k = cases.seeded_normal(cases.cfg_seed(1, "k"), (T, B, H, 1, D))
+    v = cases.seeded_normal(cases.cfg_seed(1, "v"), (T, B, H, 1, D))
+    st = tract_amd.InPlaceKvSdpa(axis=2, causal=True, scale=None).state()
+    kc = vc = None
+    worst = 0.0
+    for t in range(T):
+        out = st.eval([q[t], k[t], v[t]]).to_numpy()
+        kc, vc = orc.concat_append(kc, k[t], 2), orc.concat_append(vc, v[t], 2)
+        if t % 8 == 0 or t > 250:
+            worst = max(worst, max_abs(out, orc.flash_sdpa(q[t], kc, vc, causal=True)))
+    assert st.k.len() == T and st.k.capacity() == 256 and st.k.reallocs() == 8
+    assert worst <= 1e-3
+    saved = []
+    st.save_to(saved)
+    assert saved[0].tobytes() == kc.tobytes() and saved[1].tobytes() == vc.tobytes()
+
+
+def test_ragged_decode_small(rt):
+    rng = np.random.default_rng(21)
+    Hq, Hkv, D = 32, 8, 128
+    lens = [1, 31, 64, 200, 1025]
+    ks, vs, qs = [], [], []
+    kcs, vcs = [], []
+    for n in lens:
+        k = rng.standard_normal((1, Hkv, n, D), dtype=np.float32).astype(np.float16)
+        v = rng.standard_normal((1, Hkv, n, D), dtype=np.float32).astype(np.float16)
+        kc, vc = tract_amd.InPlaceKvCache(2), tract_amd.InPlaceKvCache(2)
+        kc.push(k), vc.push(v)
+        ks.append(k), vs.append(v), kcs.append(kc), vcs.append(vc)
+    q = (rng.standard_normal((len(lens), Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    out = tract_amd.sdpa_decode_ragged(tract_amd.DeviceTensor.from_numpy(q), kcs, vcs).to_numpy()
+    for i in range(len(lens)):
+        want = orc.flash_sdpa(q[i:i + 1], ks[i], vs[i], causal=True)
+        assert max_abs(out[i:i + 1], want) <= 2e-2

@@ -1,0 +1,13 @@
+"""tract_amd — MI355X (gfx950) implementation of tract's KV-cache hot path.
+
+The product is ``libtract_rocm.so`` (hand-written HIP behind the C ABI of
+``include/tract_rocm.h``).  This package is the host-side mirror of the tract
+operators on that path (``InPlaceKvCache``, ``InPlaceKvSdpa``, ``DynKeyValueCache``,
+``Sdpa``, the Q4_0/Q8_0 ``BlockQuant`` formats) over that ABI, used by the tests and
+the benchmark the way a ``tract-rocm`` crate would use it through FFI.
+"""
+from ._lib import F16, F32, Q4_0, Q8_0, TractRocmError  # noqa: F401
+from .runtime import (DeviceTensor, RocmRuntime, Stream, Workspace, runtime_for_name,  # noqa: F401
+                      synchronize)
+from .ops import (BlockQuant, DynKeyValueCache, DynKeyValueCacheState, InPlaceKvCache,  # noqa: F401
+                  InPlaceKvSdpa, InPlaceKvSdpaState, Sdpa, Q4_0_FORMAT, Q8_0_FORMAT, sdpa_decode_ragged)

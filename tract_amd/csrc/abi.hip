@@ -1,0 +1,598 @@
+// Host side of libtract_rocm.so: the C ABI declared in include/tract_rocm.h.
+// Runtime context, error convention, device memory, the in-place capacity-doubling KV
+// cache and the dispatch of attention calls to the kernels.
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <math.h>
+#include <mutex>
+#include <new>
+#include <vector>
+#include "common.h"
+
+namespace trocm {
+
+// ---- error convention (api/ffi/src/lib.rs:18-62) -----------------------------------------
+static thread_local char g_last_error[1024] = "";
+
+int fail(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    return 1;
+}
+
+// ---- context ---------------------------------------------------------------------------------
+static std::mutex g_init_mutex;
+static int g_device = -1;
+static int g_compute_units = 0;
+static size_t g_hbm_bytes = 0;
+static char g_name[256] = "";
+
+struct ThreadStream {
+    hipStream_t s = nullptr;
+    ~ThreadStream() {
+        // Streams of exiting threads are left to the runtime: destroying them here can run
+        // after the HIP runtime itself has been torn down.
+    }
+};
+static thread_local ThreadStream g_thread_stream;
+
+int ensure_init() {
+    if (g_device >= 0) return 0;
+    return fail("trocm_init() has not been called");
+}
+
+int num_compute_units() { return g_compute_units > 0 ? g_compute_units : 256; }
+
+int resolve_stream(void *stream, hipStream_t *out) {
+    if (ensure_init()) return 1;
+    if (stream) {
+        *out = (hipStream_t)stream;
+        return 0;
+    }
+    if (!g_thread_stream.s) {
+        TROCM_HIP(hipSetDevice(g_device));
+        TROCM_HIP(hipStreamCreateWithFlags(&g_thread_stream.s, hipStreamNonBlocking));
+    }
+    *out = g_thread_stream.s;
+    return 0;
+}
+
+}  // namespace trocm
+
+using namespace trocm;
+
+// ---- KV cache object -------------------------------------------------------------------------
+struct trocm_kv_cache {
+    int fmt;
+    int64_t B, H, D;
+    int64_t len, cap, reallocs;
+    void *data;    // F32/F16 rows, or the code plane
+    void *scales;  // f16 scale plane of the quantised formats
+};
+
+static size_t plane_bytes(const trocm_kv_cache *c, int64_t cap) {
+    return (size_t)c->B * c->H * cap * device_row_bytes(c->fmt, c->D);
+}
+static size_t scale_plane_bytes(const trocm_kv_cache *c, int64_t cap) {
+    return is_quant(c->fmt) ? (size_t)c->B * c->H * cap * (c->D / 32) * 2 : 0;
+}
+
+// Copy the first `len` tokens of planes with capacity `src_cap` into planes of `dst_cap`.
+static int copy_valid(const trocm_kv_cache *c, void *dst, void *dst_scales, int64_t dst_cap, const void *src,
+                      const void *src_scales, int64_t src_cap, int64_t len, hipStream_t s) {
+    if (len == 0) return 0;
+    CopyNd d;
+    d.rank = 2;
+    int64_t rb = (int64_t)device_row_bytes(c->fmt, c->D);
+    d.shape[0] = c->B * c->H;
+    d.shape[1] = len * rb;
+    d.dst_stride[0] = dst_cap * rb;
+    d.src_stride[0] = src_cap * rb;
+    d.dst_stride[1] = d.src_stride[1] = 1;
+    if (launch_copy_nd(dst, src, d, 1, s)) return 1;
+    if (is_quant(c->fmt)) {
+        int64_t sb = c->D / 32 * 2;
+        d.shape[1] = len * sb;
+        d.dst_stride[0] = dst_cap * sb;
+        d.src_stride[0] = src_cap * sb;
+        if (launch_copy_nd(dst_scales, src_scales, d, 1, s)) return 1;
+    }
+    return 0;
+}
+
+// Replace the buffers by ones of `new_cap` tokens holding the valid region
+// (grow(), transformers/src/ops/inplace_kv_cache.rs:106-113; the tail stays uninitialised).
+static int regrow(trocm_kv_cache *c, int64_t new_cap, hipStream_t s) {
+    void *nd = nullptr, *ns = nullptr;
+    size_t pb = plane_bytes(c, new_cap), sb = scale_plane_bytes(c, new_cap);
+    hipError_t e = hipMalloc(&nd, pb ? pb : 16);
+    if (e != hipSuccess)
+        return fail("allocating a KV cache of %lld tokens (%zu bytes) failed: %s", (long long)new_cap, pb,
+                    hipGetErrorString(e));
+    if (sb) {
+        e = hipMalloc(&ns, sb);
+        if (e != hipSuccess) {
+            (void)hipFree(nd);
+            return fail("allocating KV cache scales (%zu bytes) failed: %s", sb, hipGetErrorString(e));
+        }
+    }
+    if (c->data && c->len) {
+        if (copy_valid(c, nd, ns, new_cap, c->data, c->scales, c->cap, c->len, s)) {
+            (void)hipFree(nd);
+            if (ns) (void)hipFree(ns);
+            return 1;
+        }
+    }
+    if (c->data) {
+        // The old buffers may still be read by work queued on the stream.
+        TROCM_HIP(hipStreamSynchronize(s));
+        TROCM_HIP(hipFree(c->data));
+        if (c->scales) TROCM_HIP(hipFree(c->scales));
+    }
+    c->data = nd;
+    c->scales = ns;
+    c->cap = new_cap;
+    return 0;
+}
+
+extern "C" {
+
+// ---- runtime -------------------------------------------------------------------------------
+int trocm_init(int device) {
+    std::lock_guard<std::mutex> lock(g_init_mutex);
+    if (g_device >= 0) {
+        TROCM_REQUIRE(g_device == device, "Context is already set on device %d", g_device);  // gpu/src/device.rs:129-137
+        return 0;
+    }
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n == 0)
+        return fail("no HIP device available (%s)", e != hipSuccess ? hipGetErrorString(e) : "device count is 0");
+    TROCM_REQUIRE(device >= 0 && device < n, "device %d out of range (found %d)", device, n);
+    TROCM_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    TROCM_HIP(hipGetDeviceProperties(&prop, device));
+    TROCM_REQUIRE(strncmp(prop.gcnArchName, "gfx950", 6) == 0,
+                  "this library is built for gfx950 (MI355X); device %d is %s", device, prop.gcnArchName);
+    g_compute_units = prop.multiProcessorCount;
+    g_hbm_bytes = prop.totalGlobalMem;
+    snprintf(g_name, sizeof(g_name), "%s (%s)", prop.name, prop.gcnArchName);
+    g_device = device;
+    return 0;
+}
+
+const char *trocm_last_error(void) { return g_last_error; }
+
+int trocm_device_info(int *compute_units, size_t *hbm_bytes, char *name, size_t name_len) {
+    if (ensure_init()) return 1;
+    if (compute_units) *compute_units = g_compute_units;
+    if (hbm_bytes) *hbm_bytes = g_hbm_bytes;
+    if (name && name_len) snprintf(name, name_len, "%s", g_name);
+    return 0;
+}
+
+// ---- memory and streams ----------------------------------------------------------------------
+int trocm_malloc(void **ptr, size_t bytes) {
+    TROCM_NOT_NULL(ptr);
+    if (ensure_init()) return 1;
+    *ptr = nullptr;
+    hipError_t e = hipMalloc(ptr, bytes ? bytes : 16);
+    if (e != hipSuccess) return fail("device allocation of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+    return 0;
+}
+
+int trocm_free(void *ptr) {
+    if (!ptr) return 0;
+    TROCM_HIP(hipFree(ptr));
+    return 0;
+}
+
+int trocm_h2d(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes == 0) return 0;
+    TROCM_NOT_NULL(dst);
+    TROCM_NOT_NULL(src);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    TROCM_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s));
+    return 0;
+}
+
+int trocm_d2h(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes == 0) return 0;
+    TROCM_NOT_NULL(dst);
+    TROCM_NOT_NULL(src);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    TROCM_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s));
+    return 0;
+}
+
+int trocm_memset(void *dst, int value, size_t bytes, void *stream) {
+    if (bytes == 0) return 0;
+    TROCM_NOT_NULL(dst);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    TROCM_HIP(hipMemsetAsync(dst, value, bytes, s));
+    return 0;
+}
+
+int trocm_stream_create(void **stream) {
+    TROCM_NOT_NULL(stream);
+    if (ensure_init()) return 1;
+    hipStream_t s;
+    TROCM_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = (void *)s;
+    return 0;
+}
+
+int trocm_stream_destroy(void *stream) {
+    if (!stream) return 0;
+    TROCM_HIP(hipStreamDestroy((hipStream_t)stream));
+    return 0;
+}
+
+int trocm_stream_sync(void *stream) {
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    TROCM_HIP(hipStreamSynchronize(s));
+    return 0;
+}
+
+int trocm_device_sync(void) {
+    if (ensure_init()) return 1;
+    TROCM_HIP(hipDeviceSynchronize());
+    return 0;
+}
+
+int trocm_copy_nd(void *dst, size_t dst_offset_bytes, const int64_t *dst_strides, const void *src,
+                  size_t src_offset_bytes, const int64_t *src_strides, const int64_t *shape, int rank, int elem_size,
+                  void *stream) {
+    TROCM_NOT_NULL(dst);
+    TROCM_NOT_NULL(src);
+    TROCM_NOT_NULL(dst_strides);
+    TROCM_NOT_NULL(src_strides);
+    TROCM_NOT_NULL(shape);
+    TROCM_REQUIRE(rank >= 1 && rank <= 6, "copy_nd: rank %d not in 1..6", rank);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    CopyNd d;
+    d.rank = rank;
+    for (int i = 0; i < rank; i++) {
+        d.shape[i] = shape[i];
+        d.dst_stride[i] = dst_strides[i] * elem_size;
+        d.src_stride[i] = src_strides[i] * elem_size;
+    }
+    return launch_copy_nd((char *)dst + dst_offset_bytes, (const char *)src + src_offset_bytes, d, elem_size, s);
+}
+
+// ---- KV cache ----------------------------------------------------------------------------------
+int trocm_kv_cache_create(trocm_kv_cache **out, int fmt, int64_t batch, int64_t kv_heads, int64_t head_dim) {
+    TROCM_NOT_NULL(out);
+    if (ensure_init()) return 1;
+    TROCM_REQUIRE(fmt >= TROCM_F32 && fmt <= TROCM_Q4_0, "unknown storage format %d", fmt);
+    TROCM_REQUIRE(batch >= 1 && kv_heads >= 1 && head_dim >= 1, "kv cache: batch, kv_heads and head_dim must be >= 1");
+    TROCM_REQUIRE(!is_quant(fmt) || head_dim % 32 == 0,
+                  "quantised KV cache needs head_dim %% 32 == 0, got %lld", (long long)head_dim);
+    trocm_kv_cache *c = new (std::nothrow) trocm_kv_cache();
+    TROCM_REQUIRE(c != nullptr, "out of host memory");
+    c->fmt = fmt;
+    c->B = batch, c->H = kv_heads, c->D = head_dim;
+    c->len = c->cap = c->reallocs = 0;
+    c->data = c->scales = nullptr;
+    *out = c;
+    return 0;
+}
+
+int trocm_kv_cache_destroy(trocm_kv_cache *c) {
+    if (!c) return 0;
+    int rc = 0;
+    if (c->data && hipFree(c->data) != hipSuccess) rc = fail("hipFree of a KV cache failed");
+    if (c->scales && hipFree(c->scales) != hipSuccess) rc = fail("hipFree of KV cache scales failed");
+    delete c;
+    return rc;
+}
+
+int trocm_kv_cache_len(const trocm_kv_cache *c, int64_t *len) {
+    TROCM_NOT_NULL(c);
+    TROCM_NOT_NULL(len);
+    *len = c->len;
+    return 0;
+}
+int trocm_kv_cache_capacity(const trocm_kv_cache *c, int64_t *capacity) {
+    TROCM_NOT_NULL(c);
+    TROCM_NOT_NULL(capacity);
+    *capacity = c->cap;
+    return 0;
+}
+int trocm_kv_cache_reallocs(const trocm_kv_cache *c, int64_t *reallocs) {
+    TROCM_NOT_NULL(c);
+    TROCM_NOT_NULL(reallocs);
+    *reallocs = c->reallocs;
+    return 0;
+}
+
+int trocm_kv_cache_reserve(trocm_kv_cache *c, int64_t capacity, void *stream) {
+    TROCM_NOT_NULL(c);
+    TROCM_REQUIRE(capacity >= 0, "reserve: negative capacity");
+    if (capacity <= c->cap) return 0;
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    return regrow(c, capacity, s);
+}
+
+int trocm_kv_append(trocm_kv_cache *c, const void *src, int src_dtype, const int64_t *src_strides, int64_t n_new,
+                    void *stream) {
+    TROCM_NOT_NULL(c);
+    TROCM_REQUIRE(n_new >= 0, "append: negative token count");
+    if (n_new == 0) return 0;  // inplace_kv_cache.rs:57-59
+    TROCM_NOT_NULL(src);
+    TROCM_NOT_NULL(src_strides);
+    TROCM_REQUIRE(src_dtype == TROCM_F32 || src_dtype == TROCM_F16, "append: source dtype must be F32 or F16");
+    TROCM_REQUIRE(is_quant(c->fmt) || src_dtype == c->fmt,
+                  "append: source dtype %d does not match the cache's storage format %d", src_dtype, c->fmt);
+    for (int i = 0; i < 4; i++) TROCM_REQUIRE(src_strides[i] >= 0, "append: negative source strides are not supported");
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    // growth rule, inplace_kv_cache.rs:61-80
+    if (c->cap == 0) {
+        if (regrow(c, n_new, s)) return 1;
+    } else if (c->len + n_new > c->cap) {
+        int64_t new_cap = c->cap * 2 > c->len + n_new ? c->cap * 2 : c->len + n_new;
+        if (regrow(c, new_cap, s)) return 1;
+        c->reallocs += 1;
+    }
+    if (is_quant(c->fmt)) {
+        QuantAppend a;
+        a.fmt = c->fmt, a.src_dtype = src_dtype;
+        a.B = c->B, a.H = c->H, a.S = n_new, a.D = c->D;
+        for (int i = 0; i < 4; i++) a.ss[i] = src_strides[i];
+        a.cap = c->cap, a.t0 = c->len;
+        a.src = src, a.codes = c->data, a.scales = c->scales;
+        if (launch_quant_append(a, s)) return 1;
+    } else {
+        int64_t es = (int64_t)elem_bytes(c->fmt);
+        CopyNd d;
+        d.rank = 4;
+        d.shape[0] = c->B, d.shape[1] = c->H, d.shape[2] = n_new, d.shape[3] = c->D;
+        for (int i = 0; i < 4; i++) d.src_stride[i] = src_strides[i] * es;
+        d.dst_stride[0] = c->H * c->cap * c->D * es;
+        d.dst_stride[1] = c->cap * c->D * es;
+        d.dst_stride[2] = c->D * es;
+        d.dst_stride[3] = es;
+        if (launch_copy_nd((char *)c->data + c->len * c->D * es, src, d, (int)es, s)) return 1;
+    }
+    c->len += n_new;
+    return 0;
+}
+
+int trocm_kv_cache_truncate(trocm_kv_cache *c, int64_t len) {
+    TROCM_NOT_NULL(c);
+    TROCM_REQUIRE(c->data != nullptr, "Can not truncate a zero-len kv-cache value");  // dyn_kv_cache.rs:112-119
+    TROCM_REQUIRE(len >= 0 && len <= c->len, "truncate: length %lld out of range 0..=%lld", (long long)len,
+                  (long long)c->len);
+    c->len = len;
+    return 0;
+}
+
+int trocm_kv_row_bytes(const trocm_kv_cache *c, size_t *bytes) {
+    TROCM_NOT_NULL(c);
+    TROCM_NOT_NULL(bytes);
+    *bytes = canonical_row_bytes(c->fmt, c->D);
+    return 0;
+}
+
+int trocm_kv_export(const trocm_kv_cache *c, void *dst, void *stream) {
+    TROCM_NOT_NULL(c);
+    if (c->len == 0) return 0;
+    TROCM_NOT_NULL(dst);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    if (is_quant(c->fmt))
+        return launch_quant_export(c->fmt, c->B, c->H, c->len, c->cap, c->D, c->data, c->scales, dst, s);
+    CopyNd d;
+    d.rank = 2;
+    int64_t rb = (int64_t)device_row_bytes(c->fmt, c->D);
+    d.shape[0] = c->B * c->H;
+    d.shape[1] = c->len * rb;
+    d.dst_stride[0] = c->len * rb;
+    d.src_stride[0] = c->cap * rb;
+    d.dst_stride[1] = d.src_stride[1] = 1;
+    return launch_copy_nd(dst, c->data, d, 1, s);
+}
+
+int trocm_kv_cache_clone(const trocm_kv_cache *c, trocm_kv_cache **out, void *stream) {
+    TROCM_NOT_NULL(c);
+    TROCM_NOT_NULL(out);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    trocm_kv_cache *n = nullptr;
+    if (trocm_kv_cache_create(&n, c->fmt, c->B, c->H, c->D)) return 1;
+    if (c->cap) {
+        if (regrow(n, c->cap, s)) {
+            trocm_kv_cache_destroy(n);
+            return 1;
+        }
+        if (copy_valid(c, n->data, n->scales, n->cap, c->data, c->scales, c->cap, c->len, s)) {
+            trocm_kv_cache_destroy(n);
+            return 1;
+        }
+    }
+    n->len = c->len;
+    n->reallocs = c->reallocs;
+    *out = n;
+    return 0;
+}
+
+int trocm_kv_cache_raw(const trocm_kv_cache *c, void **data, void **scales, int64_t *capacity) {
+    TROCM_NOT_NULL(c);
+    if (data) *data = c->data;
+    if (scales) *scales = c->scales;
+    if (capacity) *capacity = c->cap;
+    return 0;
+}
+
+// ---- block quantisation as a tensor op ---------------------------------------------------------
+int trocm_block_quant(int format, const void *src, int src_dtype, size_t n_elems, void *dst_blocks, void *stream) {
+    TROCM_REQUIRE(format == TROCM_Q8_0 || format == TROCM_Q4_0, "block_quant: format must be Q8_0 or Q4_0");
+    TROCM_REQUIRE(src_dtype == TROCM_F32 || src_dtype == TROCM_F16, "block_quant: source dtype must be F32 or F16");
+    TROCM_REQUIRE(n_elems % 32 == 0, "block_quant: %zu elements is not a multiple of the block length 32", n_elems);
+    if (n_elems == 0) return 0;
+    TROCM_NOT_NULL(src);
+    TROCM_NOT_NULL(dst_blocks);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    return launch_block_quant(format, src, src_dtype, n_elems, dst_blocks, s);
+}
+
+int trocm_block_dequant(int format, const void *src_blocks, size_t n_elems, void *dst, int dst_dtype, void *stream) {
+    TROCM_REQUIRE(format == TROCM_Q8_0 || format == TROCM_Q4_0, "block_dequant: format must be Q8_0 or Q4_0");
+    TROCM_REQUIRE(dst_dtype == TROCM_F32 || dst_dtype == TROCM_F16, "block_dequant: output dtype must be F32 or F16");
+    TROCM_REQUIRE(n_elems % 32 == 0, "block_dequant: %zu elements is not a multiple of the block length 32", n_elems);
+    if (n_elems == 0) return 0;
+    TROCM_NOT_NULL(src_blocks);
+    TROCM_NOT_NULL(dst);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    return launch_block_dequant(format, src_blocks, n_elems, dst, dst_dtype, s);
+}
+
+// ---- attention -----------------------------------------------------------------------------------
+int trocm_sdpa_workspace_bytes(int64_t batch, int64_t q_heads, int64_t q_len, int64_t head_dim, size_t *bytes) {
+    TROCM_NOT_NULL(bytes);
+    TROCM_REQUIRE(batch >= 0 && q_heads >= 0 && q_len >= 0 && head_dim >= 0, "workspace_bytes: negative dimension");
+    (void)q_len;
+    *bytes = decode_workspace_bytes(batch, q_heads, head_dim);
+    return 0;
+}
+
+int trocm_sdpa_workspace_init(void *workspace, size_t bytes, void *stream) {
+    TROCM_NOT_NULL(workspace);
+    TROCM_REQUIRE(bytes >= kWsCounterBytes, "workspace of %zu bytes is smaller than the counter area", bytes);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    TROCM_HIP(hipMemsetAsync(workspace, 0, kWsCounterBytes, s));
+    return 0;
+}
+
+static int dispatch_sdpa(const SdpaArgs &a, hipStream_t s) {
+    if (a.B == 0 || a.Hq == 0 || a.Sq == 0 || a.D == 0) return 0;
+    int rc = 2;
+    if (a.Sq == 1) rc = launch_sdpa_decode(a, s);
+    if (rc == 2) rc = launch_sdpa_prefill(a, s);
+    if (rc == 2) rc = launch_sdpa_generic(a, s);
+    return rc;
+}
+
+int trocm_sdpa(const void *q, const void *k, const void *v, const void *mask, void *out, int dtype, int64_t batch,
+               int64_t q_heads, int64_t kv_heads, int64_t q_len, int64_t kv_len, int64_t head_dim,
+               const int64_t *kv_strides, int64_t mask_batch, int64_t mask_heads, float scale, int causal,
+               void *workspace, size_t workspace_bytes, void *stream) {
+    TROCM_NOT_NULL(q);
+    TROCM_NOT_NULL(k);
+    TROCM_NOT_NULL(v);
+    TROCM_NOT_NULL(out);
+    TROCM_REQUIRE(dtype == TROCM_F32 || dtype == TROCM_F16, "sdpa: dtype must be F32 or F16");
+    TROCM_REQUIRE(batch >= 0 && q_heads >= 0 && kv_heads >= 1 && q_len >= 0 && kv_len >= 0 && head_dim >= 0,
+                  "sdpa: negative dimension");
+    TROCM_REQUIRE(q_heads % kv_heads == 0, "Q heads (%lld) must be a multiple of K/V heads (%lld)", (long long)q_heads,
+                  (long long)kv_heads);  // sdpa.rs:325-330
+    TROCM_REQUIRE(!(causal && mask), "Mask cannot be provided if is_causal=true");  // sdpa.rs:297-299
+    if (mask) {
+        TROCM_REQUIRE(mask_batch == 1 || mask_batch == batch, "sdpa: mask batch must be 1 or %lld", (long long)batch);
+        TROCM_REQUIRE(mask_heads == 1 || mask_heads == q_heads, "sdpa: mask heads must be 1 or %lld", (long long)q_heads);
+    }
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    SdpaArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = q, a.out = out, a.q_dtype = dtype, a.kv_fmt = dtype;
+    a.k = k, a.v = v;
+    a.B = batch, a.Hq = q_heads, a.Hkv = kv_heads, a.Sq = q_len, a.Sk = kv_len, a.D = head_dim;
+    if (kv_strides) {
+        a.kv_stride_b = kv_strides[0], a.kv_stride_h = kv_strides[1], a.kv_stride_t = kv_strides[2];
+        TROCM_REQUIRE(a.kv_stride_b >= 0 && a.kv_stride_h >= 0 && a.kv_stride_t >= 0, "sdpa: negative K/V strides");
+    } else {
+        a.kv_stride_t = head_dim, a.kv_stride_h = kv_len * head_dim, a.kv_stride_b = kv_heads * kv_len * head_dim;
+    }
+    a.mask = mask, a.mask_b = mask ? mask_batch : 1, a.mask_h = mask ? mask_heads : 1;
+    a.scale = isnan(scale) ? 1.0f / sqrtf((float)head_dim) : scale;  // sdpa.rs:177-181
+    a.causal = causal;
+    a.workspace = workspace, a.workspace_bytes = workspace_bytes;
+    if (kv_len == 0) {  // nothing to attend to: zeros, like the CPU op's zero-initialised output (flash_sdpa.rs:253)
+        TROCM_HIP(hipMemsetAsync(out, 0, (size_t)batch * q_heads * q_len * head_dim * elem_bytes(dtype), s));
+        return 0;
+    }
+    return dispatch_sdpa(a, s);
+}
+
+int trocm_sdpa_cached(const void *q, int q_dtype, int64_t q_heads, int64_t q_len, const trocm_kv_cache *kc,
+                      const trocm_kv_cache *vc, void *out, float scale, int causal, void *workspace,
+                      size_t workspace_bytes, void *stream) {
+    TROCM_NOT_NULL(q);
+    TROCM_NOT_NULL(kc);
+    TROCM_NOT_NULL(vc);
+    TROCM_NOT_NULL(out);
+    TROCM_REQUIRE(q_dtype == TROCM_F32 || q_dtype == TROCM_F16, "sdpa: q dtype must be F32 or F16");
+    TROCM_REQUIRE(kc->fmt == vc->fmt && kc->B == vc->B && kc->H == vc->H && kc->D == vc->D,
+                  "K and V caches differ in format or shape");
+    TROCM_REQUIRE(kc->len == vc->len, "K/V lengths must match (%lld vs %lld)", (long long)kc->len, (long long)vc->len);
+    TROCM_REQUIRE(kc->cap == vc->cap, "K/V capacities must match (%lld vs %lld)", (long long)kc->cap, (long long)vc->cap);
+    TROCM_REQUIRE(kc->len > 0, "empty kv-cache");  // inplace_kv_cache.rs:91
+    TROCM_REQUIRE(q_heads % kc->H == 0, "Q heads (%lld) must be a multiple of K/V heads (%lld)", (long long)q_heads,
+                  (long long)kc->H);
+    TROCM_REQUIRE(is_quant(kc->fmt) || kc->fmt == q_dtype, "q dtype %d does not match the cache format %d", q_dtype,
+                  kc->fmt);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    SdpaArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = q, a.out = out, a.q_dtype = q_dtype, a.kv_fmt = kc->fmt;
+    a.k = kc->data, a.v = vc->data, a.k_scales = kc->scales, a.v_scales = vc->scales;
+    a.B = kc->B, a.Hq = q_heads, a.Hkv = kc->H, a.Sq = q_len, a.Sk = kc->len, a.D = kc->D;
+    a.kv_stride_t = kc->D, a.kv_stride_h = kc->cap * kc->D, a.kv_stride_b = kc->H * kc->cap * kc->D;
+    a.mask_b = a.mask_h = 1;
+    a.scale = isnan(scale) ? 1.0f / sqrtf((float)kc->D) : scale;
+    a.causal = causal;
+    a.workspace = workspace, a.workspace_bytes = workspace_bytes;
+    return dispatch_sdpa(a, s);
+}
+
+int trocm_sdpa_decode_ragged(const void *q, int q_dtype, int64_t q_heads, int64_t n_seq,
+                             trocm_kv_cache *const *k_caches, trocm_kv_cache *const *v_caches, void *out, float scale,
+                             void *workspace, size_t workspace_bytes, void *stream) {
+    TROCM_NOT_NULL(q);
+    TROCM_NOT_NULL(k_caches);
+    TROCM_NOT_NULL(v_caches);
+    TROCM_NOT_NULL(out);
+    TROCM_REQUIRE(n_seq >= 1, "ragged decode: n_seq must be >= 1");
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    std::vector<RaggedSeq> seqs((size_t)n_seq);
+    const trocm_kv_cache *k0 = k_caches[0];
+    TROCM_NOT_NULL(k0);
+    for (int64_t i = 0; i < n_seq; i++) {
+        const trocm_kv_cache *kc = k_caches[i], *vc = v_caches[i];
+        TROCM_NOT_NULL(kc);
+        TROCM_NOT_NULL(vc);
+        TROCM_REQUIRE(kc->B == 1 && vc->B == 1, "ragged decode: every per-sequence cache must have batch == 1");
+        TROCM_REQUIRE(kc->fmt == k0->fmt && vc->fmt == k0->fmt && kc->H == k0->H && vc->H == k0->H && kc->D == k0->D &&
+                          vc->D == k0->D,
+                      "ragged decode: caches differ in format or shape (sequence %lld)", (long long)i);
+        TROCM_REQUIRE(kc->len == vc->len && kc->cap == vc->cap, "K/V lengths must match (sequence %lld)", (long long)i);
+        TROCM_REQUIRE(kc->len > 0, "empty kv-cache (sequence %lld)", (long long)i);
+        seqs[(size_t)i] = RaggedSeq{kc->data, vc->data, kc->scales, vc->scales, kc->len, kc->cap};
+    }
+    TROCM_REQUIRE(q_heads % k0->H == 0, "Q heads (%lld) must be a multiple of K/V heads (%lld)", (long long)q_heads,
+                  (long long)k0->H);
+    TROCM_REQUIRE(is_quant(k0->fmt) || k0->fmt == q_dtype, "q dtype %d does not match the cache format %d", q_dtype,
+                  k0->fmt);
+    float sc = isnan(scale) ? 1.0f / sqrtf((float)k0->D) : scale;
+    return launch_sdpa_decode_ragged(q, out, q_dtype, k0->fmt, n_seq, q_heads, k0->H, k0->D, seqs.data(), sc, workspace,
+                                     workspace_bytes, s);
+}
+
+}  // extern "C"

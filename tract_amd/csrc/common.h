@@ -1,0 +1,120 @@
+// Internal declarations shared by the translation units of libtract_rocm.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include "../../include/tract_rocm.h"
+
+namespace trocm {
+
+// ---- error convention: 0 = OK, 1 = KO + thread-local message --------------------------
+int fail(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+
+#define TROCM_REQUIRE(cond, ...)                 \
+    do {                                         \
+        if (!(cond)) return ::trocm::fail(__VA_ARGS__); \
+    } while (0)
+
+#define TROCM_NOT_NULL(p) TROCM_REQUIRE((p) != nullptr, "unexpected null pointer argument: %s", #p)
+
+#define TROCM_HIP(expr)                                                                   \
+    do {                                                                                  \
+        hipError_t e__ = (expr);                                                          \
+        if (e__ != hipSuccess)                                                            \
+            return ::trocm::fail("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e__), __FILE__, __LINE__); \
+    } while (0)
+
+// Resolves the `void *stream` argument of the C ABI: NULL -> this thread's own stream.
+int resolve_stream(void *stream, hipStream_t *out);
+int ensure_init();
+int num_compute_units();
+
+static inline size_t elem_bytes(int dtype) { return dtype == TROCM_F32 ? 4 : dtype == TROCM_F16 ? 2 : 0; }
+static inline bool is_quant(int fmt) { return fmt == TROCM_Q8_0 || fmt == TROCM_Q4_0; }
+// Canonical bytes of one token row of one head.
+static inline size_t canonical_row_bytes(int fmt, int64_t d) {
+    switch (fmt) {
+        case TROCM_F32: return (size_t)d * 4;
+        case TROCM_F16: return (size_t)d * 2;
+        case TROCM_Q8_0: return (size_t)d / 32 * 34;
+        case TROCM_Q4_0: return (size_t)d / 32 * 18;
+    }
+    return 0;
+}
+// Bytes of one token row in the device code plane (F32/F16: the row itself).
+static inline size_t device_row_bytes(int fmt, int64_t d) {
+    switch (fmt) {
+        case TROCM_F32: return (size_t)d * 4;
+        case TROCM_F16: return (size_t)d * 2;
+        case TROCM_Q8_0: return (size_t)d;
+        case TROCM_Q4_0: return (size_t)d / 2;
+    }
+    return 0;
+}
+
+// ---- kernels' launchers (each in its own .hip file) ------------------------------------
+
+// Strided N-d copy, strides in BYTES, rank <= 6.
+struct CopyNd {
+    int rank;
+    int64_t shape[6];
+    int64_t dst_stride[6];
+    int64_t src_stride[6];
+};
+int launch_copy_nd(void *dst, const void *src, const CopyNd &desc, int elem_size, hipStream_t s);
+
+// Quantise [rows, d] (row r of the source at src + b*ss[0] + h*ss[1] + t*ss[2] elements, element
+// stride ss[3]) into the code/scale planes of a cache at token offset t0.
+struct QuantAppend {
+    int fmt, src_dtype;
+    int64_t B, H, S, D;
+    int64_t ss[4];          // source element strides
+    int64_t cap, t0;        // destination capacity (tokens) and first token
+    const void *src;
+    void *codes, *scales;
+};
+int launch_quant_append(const QuantAppend &a, hipStream_t s);
+// Canonical export of the quantised planes: dst [B,H,len, D/32 * block_bytes].
+int launch_quant_export(int fmt, int64_t B, int64_t H, int64_t len, int64_t cap, int64_t D,
+                        const void *codes, const void *scales, void *dst, hipStream_t s);
+// Dequantise canonical blocks to a dense f32/f16 tensor.
+int launch_block_quant(int fmt, const void *src, int src_dtype, size_t n_elems, void *dst, hipStream_t s);
+int launch_block_dequant(int fmt, const void *blocks, size_t n_elems, void *dst, int dst_dtype, hipStream_t s);
+
+// Attention.  One description for every kernel.
+struct SdpaArgs {
+    const void *q;
+    void *out;
+    int q_dtype;            // F32 / F16 (q and out)
+    int kv_fmt;             // F32 / F16 / Q8_0 / Q4_0
+    const void *k, *v;      // code planes (or plain tensors)
+    const void *k_scales, *v_scales;
+    int64_t B, Hq, Hkv, Sq, Sk, D;
+    int64_t kv_stride_b, kv_stride_h, kv_stride_t;       // in ELEMENTS of the logical [.., D] tensor rows
+    const void *mask;       // of q_dtype, [mask_b, mask_h, Sq, Sk]
+    int64_t mask_b, mask_h;
+    float scale;
+    int causal;
+    void *workspace;
+    size_t workspace_bytes;
+};
+int launch_sdpa_generic(const SdpaArgs &a, hipStream_t s);
+// Split-K decode (Sq == 1).  Returns 2 when the shape is not covered by a fast kernel.
+int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s);
+// MFMA prefill.  Returns 2 when the shape is not covered.
+int launch_sdpa_prefill(const SdpaArgs &a, hipStream_t s);
+
+// Ragged decode: per-sequence descriptors live in pinned host memory owned by the library.
+struct RaggedSeq {
+    const void *k, *v, *k_scales, *v_scales;
+    int64_t len, cap;
+};
+int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt, int64_t n_seq, int64_t Hq,
+                              int64_t Hkv, int64_t D, const RaggedSeq *seqs, float scale, void *workspace,
+                              size_t workspace_bytes, hipStream_t s);
+
+// Workspace layout: [counters: kWsCounters ints][partials ...]
+constexpr size_t kWsCounterBytes = 64 * 1024;   // 16384 arrival counters
+size_t decode_workspace_bytes(int64_t B, int64_t Hq, int64_t D);
+
+}  // namespace trocm

@@ -1,0 +1,136 @@
+// Strided N-d copy for gfx950: the device side of DeviceContext::copy_nd
+// (gpu/src/device.rs:26-35).  The host collapses the description to the fewest
+// dimensions and the widest vector (up to 16 bytes) that strides and alignment allow, so
+// that a KV-cache append or growth moves whole 128-bit words with consecutive lanes on
+// consecutive addresses; HBM bandwidth is the only bound.
+#include "common.h"
+
+namespace trocm {
+namespace {
+
+struct CopyDev {
+    int rank;
+    uint32_t shape[6];
+    int64_t dst_stride[6];  // bytes
+    int64_t src_stride[6];  // bytes
+};
+
+template <typename V, typename Index>
+__global__ __launch_bounds__(256) void copy_nd_kernel(char *__restrict__ dst, const char *__restrict__ src,
+                                                      CopyDev p, Index total) {
+    Index step = (Index)gridDim.x * blockDim.x;
+    for (Index idx = (Index)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += step) {
+        Index rem = idx;
+        int64_t doff = 0, soff = 0;
+#pragma unroll
+        for (int d = 5; d >= 0; --d) {
+            if (d < p.rank) {
+                Index q = rem / p.shape[d];
+                uint32_t i = (uint32_t)(rem - q * p.shape[d]);
+                rem = q;
+                doff += (int64_t)i * p.dst_stride[d];
+                soff += (int64_t)i * p.src_stride[d];
+            }
+        }
+        *reinterpret_cast<V *>(dst + doff) = *reinterpret_cast<const V *>(src + soff);
+    }
+}
+
+template <typename V>
+int launch_typed(char *dst, const char *src, const CopyDev &p, uint64_t total, hipStream_t s) {
+    const int block = 256;
+    uint64_t blocks = (total + block - 1) / block;
+    uint64_t max_blocks = (uint64_t)num_compute_units() * 32;
+    if (blocks > max_blocks) blocks = max_blocks;
+    if (total < (1ull << 31))
+        hipLaunchKernelGGL((copy_nd_kernel<V, uint32_t>), dim3((unsigned)blocks), dim3(block), 0, s, dst, src, p,
+                           (uint32_t)total);
+    else
+        hipLaunchKernelGGL((copy_nd_kernel<V, uint64_t>), dim3((unsigned)blocks), dim3(block), 0, s, dst, src, p,
+                           (uint64_t)total);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("copy_nd launch failed: %s", hipGetErrorString(e));
+    return 0;
+}
+
+}  // namespace
+
+int launch_copy_nd(void *dst_v, const void *src_v, const CopyNd &in, int elem_size, hipStream_t s) {
+    TROCM_REQUIRE(in.rank >= 1 && in.rank <= 6, "copy_nd: rank %d not in 1..6", in.rank);
+    TROCM_REQUIRE(elem_size == 1 || elem_size == 2 || elem_size == 4 || elem_size == 8 || elem_size == 16,
+                  "copy_nd: unsupported element size %d", elem_size);
+    // 1. drop unit dims, detect empty zones
+    int64_t shape[6], ds[6], ss[6];
+    int rank = 0;
+    for (int d = 0; d < in.rank; d++) {
+        TROCM_REQUIRE(in.shape[d] >= 0, "copy_nd: negative dimension");
+        TROCM_REQUIRE(in.dst_stride[d] >= 0 && in.src_stride[d] >= 0, "copy_nd: negative strides are not supported");
+        if (in.shape[d] == 0) return 0;
+        TROCM_REQUIRE(in.shape[d] < (1ll << 32), "copy_nd: dimension %lld too large", (long long)in.shape[d]);
+        if (in.shape[d] == 1) continue;
+        shape[rank] = in.shape[d];
+        ds[rank] = in.dst_stride[d];
+        ss[rank] = in.src_stride[d];
+        rank++;
+    }
+    if (rank == 0) {
+        shape[0] = 1;
+        ds[0] = ss[0] = elem_size;
+        rank = 1;
+    }
+    // 2. merge dims that are contiguous in both tensors (outer stride == inner stride * inner extent)
+    for (int d = rank - 2; d >= 0; d--) {
+        if (ds[d] == ds[d + 1] * shape[d + 1] && ss[d] == ss[d + 1] * shape[d + 1] &&
+            shape[d] * shape[d + 1] < (1ll << 32)) {
+            shape[d] *= shape[d + 1];
+            ds[d] = ds[d + 1];
+            ss[d] = ss[d + 1];
+            for (int e = d + 1; e < rank - 1; e++) {
+                shape[e] = shape[e + 1];
+                ds[e] = ds[e + 1];
+                ss[e] = ss[e + 1];
+            }
+            rank--;
+        }
+    }
+    // 3. widen the element when the innermost dim is dense in both tensors
+    int vec = elem_size;
+    if (ds[rank - 1] == elem_size && ss[rank - 1] == elem_size) {
+        for (int cand = 16; cand > elem_size; cand >>= 1) {
+            bool ok = ((uintptr_t)dst_v % cand == 0) && ((uintptr_t)src_v % cand == 0) &&
+                      ((shape[rank - 1] * elem_size) % cand == 0);
+            for (int d = 0; d < rank - 1 && ok; d++) ok = (ds[d] % cand == 0) && (ss[d] % cand == 0);
+            if (ok) {
+                vec = cand;
+                break;
+            }
+        }
+        if (vec != elem_size) {
+            shape[rank - 1] = shape[rank - 1] * elem_size / vec;
+            ds[rank - 1] = ss[rank - 1] = vec;
+        }
+    } else {
+        TROCM_REQUIRE((uintptr_t)dst_v % elem_size == 0 && (uintptr_t)src_v % elem_size == 0,
+                      "copy_nd: pointers not aligned to the element size");
+    }
+    CopyDev p;
+    p.rank = rank;
+    uint64_t total = 1;
+    for (int d = 0; d < 6; d++) {
+        p.shape[d] = d < rank ? (uint32_t)shape[d] : 1;
+        p.dst_stride[d] = d < rank ? ds[d] : 0;
+        p.src_stride[d] = d < rank ? ss[d] : 0;
+        if (d < rank) total *= (uint64_t)shape[d];
+    }
+    char *dst = (char *)dst_v;
+    const char *src = (const char *)src_v;
+    switch (vec) {
+        case 1: return launch_typed<uint8_t>(dst, src, p, total, s);
+        case 2: return launch_typed<uint16_t>(dst, src, p, total, s);
+        case 4: return launch_typed<uint32_t>(dst, src, p, total, s);
+        case 8: return launch_typed<uint2>(dst, src, p, total, s);
+        default: return launch_typed<uint4>(dst, src, p, total, s);
+    }
+}
+
+}  // namespace trocm

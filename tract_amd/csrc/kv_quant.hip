@@ -1,0 +1,307 @@
+// Q8_0 / Q4_0 block quantisation on KV append, canonical export and dequantisation.
+//
+// Stored bytes must equal what tract's CPU block quantisers produce
+// (linalg/src/frame/block_quant/q4_0.rs:19-45, q8_1.rs:20-48 without the `sum`
+// field), so every floating-point step is spelled out: no contraction of a*b+c (this
+// file is compiled with -ffp-contract=off and uses the _rn intrinsics), IEEE division,
+// round-half-away for Q8 codes, truncation for Q4 codes, RNE for the f16 scale.
+//
+// Device layout (private): a code plane with one row per token ([D] int8 for Q8_0,
+// [D/2] bytes = 16 canonical nibble bytes per block for Q4_0) and a scale plane with
+// D/32 f16 per token, so that decode can read both with aligned 128-bit loads.
+//
+// Each block is scanned by one thread in element order: the quantiser's "first element
+// with strictly largest |v|" rule is order dependent, and a 32-element block is 64-128
+// bytes, so one lane reads whole 128-bit words.  The work is HBM-bound (reads 2-4 bytes
+// and writes ~1 byte per element).
+#include <hip/hip_fp16.h>
+#include "common.h"
+
+namespace trocm {
+namespace {
+
+__device__ __forceinline__ float load_elem(const float *p) { return *p; }
+__device__ __forceinline__ float load_elem(const __half *p) { return __half2float(*p); }
+
+// Rust `f32 as i8`: truncate toward zero, saturate, NaN -> 0.
+__device__ __forceinline__ int sat_i8(float x) {
+    if (x != x) return 0;
+    if (x <= -128.0f) return -128;
+    if (x >= 127.0f) return 127;
+    return (int)x;
+}
+
+// f32::round(): half away from zero.  x - trunc(x) is exact, so the comparison is too.
+__device__ __forceinline__ float round_half_away(float x) {
+    float t = truncf(x);
+    float d = __fsub_rn(x, t);
+    if (fabsf(d) >= 0.5f) t = __fadd_rn(t, copysignf(1.0f, x));
+    return t;
+}
+
+// Signed value of the first element with strictly largest magnitude (q4_0.rs:27-34).
+__device__ __forceinline__ float signed_first_absmax(const float (&v)[32]) {
+    float amax = 0.0f, mx = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+        float a = fabsf(v[i]);
+        if (amax < a) {
+            amax = a;
+            mx = v[i];
+        }
+    }
+    return mx;
+}
+
+// Q8: returns the f16 scale bits, codes packed 4 per word in element order.
+__device__ __forceinline__ uint16_t quant_q8(const float (&v)[32], uint32_t (&codes)[8]) {
+    float mx = signed_first_absmax(v);
+    float scale = __fdiv_rn(mx, 127.0f);                               // q8_1.rs:39
+    float r = (scale == 0.0f) ? 0.0f : __fdiv_rn(1.0f, scale);         // q8_1.rs:40
+#pragma unroll
+    for (int w = 0; w < 8; w++) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            int c = sat_i8(round_half_away(__fmul_rn(v[w * 4 + b], r)));  // q8_1.rs:45
+            word |= (uint32_t)(c & 0xff) << (8 * b);
+        }
+        codes[w] = word;
+    }
+    return __half_as_ushort(__float2half_rn(scale));
+}
+
+// Q4: byte j = code(elem j) | code(elem j+16) << 4 (q4_0.rs:39-44, helpers.rs:62-68).
+__device__ __forceinline__ uint16_t quant_q4(const float (&v)[32], uint32_t (&codes)[4]) {
+    float mx = signed_first_absmax(v);
+    float scale = __fdiv_rn(mx, -8.0f);                                // q4_0.rs:35
+    float r = (scale == 0.0f) ? 0.0f : __fdiv_rn(1.0f, scale);         // q4_0.rs:36
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            int j = w * 4 + b;
+            int lo = sat_i8(__fadd_rn(__fmul_rn(v[j], r), 8.5f));
+            int hi = sat_i8(__fadd_rn(__fmul_rn(v[j + 16], r), 8.5f));
+            lo = lo < 15 ? lo : 15;
+            hi = hi < 15 ? hi : 15;
+            uint32_t byte = ((uint32_t)lo & 0xffu) | (((uint32_t)hi << 4) & 0xffu);
+            word |= (byte & 0xffu) << (8 * b);
+        }
+        codes[w] = word;
+    }
+    return __half_as_ushort(__float2half_rn(scale));
+}
+
+template <typename SrcT>
+__device__ __forceinline__ void load_block(const SrcT *p, int64_t stride, bool vec, float (&v)[32]) {
+    if (vec) {  // dense and 16-byte aligned: whole 128-bit words
+        constexpr int kPerWord = 16 / sizeof(SrcT);
+        const uint4 *w = reinterpret_cast<const uint4 *>(p);
+#pragma unroll
+        for (int i = 0; i < 32 / kPerWord; i++) {
+            uint4 x = w[i];
+            const SrcT *e = reinterpret_cast<const SrcT *>(&x);
+#pragma unroll
+            for (int j = 0; j < kPerWord; j++) v[i * kPerWord + j] = load_elem(e + j);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 32; i++) v[i] = load_elem(p + i * stride);
+    }
+}
+
+struct QuantAppendDev {
+    int fmt;
+    int vec;
+    int64_t B, H, S, D;
+    int64_t ss[4];
+    int64_t cap, t0;
+    const void *src;
+    uint8_t *codes;
+    uint16_t *scales;
+    int64_t n_blocks;
+};
+
+template <typename SrcT>
+__global__ __launch_bounds__(256) void quant_append_kernel(QuantAppendDev a) {
+    int64_t nb = a.D / 32;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < a.n_blocks;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        int64_t blk = idx % nb;
+        int64_t rem = idx / nb;
+        int64_t t = rem % a.S;
+        rem /= a.S;
+        int64_t h = rem % a.H;
+        int64_t b = rem / a.H;
+        const SrcT *p = (const SrcT *)a.src + b * a.ss[0] + h * a.ss[1] + t * a.ss[2] + blk * 32 * a.ss[3];
+        float v[32];
+        load_block(p, a.ss[3], a.vec != 0, v);
+        int64_t row = (b * a.H + h) * a.cap + a.t0 + t;
+        if (a.fmt == TROCM_Q8_0) {
+            uint32_t c[8];
+            uint16_t d = quant_q8(v, c);
+            uint4 *dst = reinterpret_cast<uint4 *>(a.codes + row * a.D + blk * 32);
+            dst[0] = make_uint4(c[0], c[1], c[2], c[3]);
+            dst[1] = make_uint4(c[4], c[5], c[6], c[7]);
+            a.scales[row * nb + blk] = d;
+        } else {
+            uint32_t c[4];
+            uint16_t d = quant_q4(v, c);
+            *reinterpret_cast<uint4 *>(a.codes + row * (a.D / 2) + blk * 16) = make_uint4(c[0], c[1], c[2], c[3]);
+            a.scales[row * nb + blk] = d;
+        }
+    }
+}
+
+// Canonical export: [B,H,len, nb * (2 + code bytes)], 2-byte aligned stores.
+__global__ __launch_bounds__(256) void quant_export_kernel(int fmt, int64_t BH, int64_t len, int64_t cap, int64_t D,
+                                                           const uint8_t *__restrict__ codes,
+                                                           const uint16_t *__restrict__ scales,
+                                                           uint16_t *__restrict__ dst) {
+    int64_t nb = D / 32;
+    int64_t total = BH * len * nb;
+    int cw = fmt == TROCM_Q8_0 ? 16 : 8;  // code bytes / 2
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        int64_t blk = idx % nb;
+        int64_t rem = idx / nb;
+        int64_t t = rem % len;
+        int64_t bh = rem / len;
+        int64_t row = bh * cap + t;
+        const uint16_t *c = reinterpret_cast<const uint16_t *>(codes + (row * nb + blk) * (cw * 2));
+        uint16_t *o = dst + ((bh * len + t) * nb + blk) * (1 + cw);
+        o[0] = scales[row * nb + blk];
+        for (int i = 0; i < cw; i++) o[1 + i] = c[i];
+    }
+}
+
+// Canonical blocks from a dense tensor (BlockQuant::quant_f32/quant_f16 as a tensor op).
+template <typename SrcT>
+__global__ __launch_bounds__(256) void block_quant_kernel(int fmt, const SrcT *__restrict__ src, int64_t n_blocks,
+                                                          bool vec, uint16_t *__restrict__ dst) {
+    int cw = fmt == TROCM_Q8_0 ? 16 : 8;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n_blocks;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        float v[32];
+        load_block(src + idx * 32, 1, vec, v);
+        uint16_t *o = dst + idx * (1 + cw);
+        if (fmt == TROCM_Q8_0) {
+            uint32_t c[8];
+            o[0] = quant_q8(v, c);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                o[1 + 2 * i] = (uint16_t)(c[i] & 0xffff);
+                o[2 + 2 * i] = (uint16_t)(c[i] >> 16);
+            }
+        } else {
+            uint32_t c[4];
+            o[0] = quant_q4(v, c);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                o[1 + 2 * i] = (uint16_t)(c[i] & 0xffff);
+                o[2 + 2 * i] = (uint16_t)(c[i] >> 16);
+            }
+        }
+    }
+}
+
+// BlockQuant::dequant_f32 / dequant_f16 (block_quant/mod.rs:78-108; q4_0.rs:82-95, q8_1.rs:50-63):
+// the product is formed in the output type: for f16 the f32 product is rounded to f16.
+template <typename DstT>
+__global__ __launch_bounds__(256) void block_dequant_kernel(int fmt, const uint8_t *__restrict__ blocks,
+                                                            int64_t n_blocks, DstT *__restrict__ dst) {
+    int bb = fmt == TROCM_Q8_0 ? 34 : 18;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n_blocks;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const uint8_t *q = blocks + idx * bb;
+        float d = __half2float(__ushort_as_half((uint16_t)(q[0] | (q[1] << 8))));
+        DstT *o = dst + idx * 32;
+        if (fmt == TROCM_Q8_0) {
+            for (int i = 0; i < 32; i++) o[i] = (DstT)__fmul_rn((float)(int8_t)q[2 + i], d);
+        } else {
+            for (int j = 0; j < 16; j++) {
+                int lo = q[2 + j] & 0xf, hi = q[2 + j] >> 4;
+                o[j] = (DstT)__fmul_rn((float)(lo - 8), d);
+                o[j + 16] = (DstT)__fmul_rn((float)(hi - 8), d);
+            }
+        }
+    }
+}
+
+int grid_for(int64_t n) {
+    int64_t blocks = (n + 255) / 256;
+    int64_t cap = (int64_t)num_compute_units() * 16;
+    return (int)(blocks < 1 ? 1 : (blocks > cap ? cap : blocks));
+}
+
+int check_launch(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("%s launch failed: %s", what, hipGetErrorString(e));
+    return 0;
+}
+
+}  // namespace
+
+int launch_quant_append(const QuantAppend &a, hipStream_t s) {
+    TROCM_REQUIRE(a.D % 32 == 0, "quantised KV cache needs head_dim %% 32 == 0, got %lld", (long long)a.D);
+    QuantAppendDev d;
+    d.fmt = a.fmt;
+    d.B = a.B, d.H = a.H, d.S = a.S, d.D = a.D;
+    for (int i = 0; i < 4; i++) d.ss[i] = a.ss[i];
+    d.cap = a.cap, d.t0 = a.t0;
+    d.src = a.src;
+    d.codes = (uint8_t *)a.codes;
+    d.scales = (uint16_t *)a.scales;
+    d.n_blocks = a.B * a.H * a.S * (a.D / 32);
+    if (d.n_blocks == 0) return 0;
+    size_t es = elem_bytes(a.src_dtype);
+    // 128-bit loads need a dense innermost axis and every block start on a 16-byte boundary
+    // (blocks are 32 elements = 64 or 128 bytes, so only the base and outer strides matter).
+    bool vec = a.ss[3] == 1 && ((uintptr_t)a.src % 16 == 0);
+    for (int i = 0; i < 3 && vec; i++) vec = (a.ss[i] * (int64_t)es) % 16 == 0;
+    d.vec = vec;
+    int grid = grid_for(d.n_blocks);
+    if (a.src_dtype == TROCM_F16)
+        hipLaunchKernelGGL(quant_append_kernel<__half>, dim3(grid), dim3(256), 0, s, d);
+    else
+        hipLaunchKernelGGL(quant_append_kernel<float>, dim3(grid), dim3(256), 0, s, d);
+    return check_launch("quant_append");
+}
+
+int launch_quant_export(int fmt, int64_t B, int64_t H, int64_t len, int64_t cap, int64_t D, const void *codes,
+                        const void *scales, void *dst, hipStream_t s) {
+    int64_t total = B * H * len * (D / 32);
+    if (total == 0) return 0;
+    hipLaunchKernelGGL(quant_export_kernel, dim3(grid_for(total)), dim3(256), 0, s, fmt, B * H, len, cap, D,
+                       (const uint8_t *)codes, (const uint16_t *)scales, (uint16_t *)dst);
+    return check_launch("quant_export");
+}
+
+int launch_block_quant(int fmt, const void *src, int src_dtype, size_t n_elems, void *dst, hipStream_t s) {
+    int64_t nb = (int64_t)(n_elems / 32);
+    if (nb == 0) return 0;
+    bool vec = (uintptr_t)src % 16 == 0;
+    if (src_dtype == TROCM_F16)
+        hipLaunchKernelGGL(block_quant_kernel<__half>, dim3(grid_for(nb)), dim3(256), 0, s, fmt, (const __half *)src,
+                           nb, vec, (uint16_t *)dst);
+    else
+        hipLaunchKernelGGL(block_quant_kernel<float>, dim3(grid_for(nb)), dim3(256), 0, s, fmt, (const float *)src, nb,
+                           vec, (uint16_t *)dst);
+    return check_launch("block_quant");
+}
+
+int launch_block_dequant(int fmt, const void *blocks, size_t n_elems, void *dst, int dst_dtype, hipStream_t s) {
+    int64_t nb = (int64_t)(n_elems / 32);
+    if (nb == 0) return 0;
+    if (dst_dtype == TROCM_F16)
+        hipLaunchKernelGGL(block_dequant_kernel<__half>, dim3(grid_for(nb)), dim3(256), 0, s, fmt,
+                           (const uint8_t *)blocks, nb, (__half *)dst);
+    else
+        hipLaunchKernelGGL(block_dequant_kernel<float>, dim3(grid_for(nb)), dim3(256), 0, s, fmt,
+                           (const uint8_t *)blocks, nb, (float *)dst);
+    return check_launch("block_dequant");
+}
+
+}  // namespace trocm

@@ -1,0 +1,482 @@
+// Split-K flash-decode attention for gfx950 (q_len == 1), GQA head sharing.
+//
+// Work decomposition
+//   grid = (splits, kv_heads, batch); one 256-thread workgroup (4 wavefronts of 64)
+//   owns a contiguous range of 32-token tiles of one (batch, kv head) and serves all G
+//   query heads of that KV head from a single read of K and V.  Wave w takes tiles
+//   w, w+4, ... of the range; every wave keeps its own online-softmax state.
+//
+// Per 32-token tile, per wave
+//   K  : the 32 rows are fetched with coalesced 128-bit loads (consecutive lanes,
+//        consecutive bytes), parked in registers while the previous tile is computed,
+//        then stored to a wave-private LDS tile with a per-row rotation of the 16-byte
+//        chunks so that the transposed read below is bank-conflict free.
+//   QK : lanes 2t and 2t+1 read the two halves of row t from LDS and form the G dot
+//        products of token t against the query vectors (broadcast reads from LDS); one
+//        DPP exchange joins the halves, no other cross-lane traffic.
+//   softmax: tile maximum per head by a DPP wave reduction; p = exp2(s - m) per lane.
+//   PV : p goes through LDS; the wave regroups as 4 row groups x 16 lanes, lane j owning
+//        head_dim/16 output columns; V rows come straight from HBM, coalesced, prefetched
+//        one tile ahead.
+//
+// Combination
+//   waves are merged through LDS; if the launch has several splits, each workgroup
+//   stores its unnormalised (O, m, l) to the workspace, takes a ticket from an arrival
+//   counter and the last one to arrive merges all splits and writes the output, so one
+//   launch does the whole job.  Logits are kept in log2 units (scale * log2 e folded in).
+//
+// Roofline: HBM-bound.  Algorithmic bytes per launch = 2*B*Hkv*T*D*e (K and V once per KV
+// head) + Q read + O write.
+#include <hip/hip_fp16.h>
+#include <string.h>
+#include <stdlib.h>
+#include "common.h"
+
+namespace trocm {
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+constexpr int kTile = 32;
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+struct DecodeDev {
+    const char *q;
+    char *out;
+    const char *k, *v;
+    int64_t kv_stride_b, kv_stride_h, kv_stride_t;  // bytes
+    int T;                                          // valid tokens
+    int tiles_per_split, nsplit;
+    int Hq, Hkv;
+    float scale_log2;
+    float *part_o;   // [B*Hkv*nsplit][G*D]
+    float *part_ml;  // [B*Hkv*nsplit][2*G]
+    int *counters;   // [B*Hkv]
+};
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float readlane_f(float x, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
+}
+// DPP controls: row_ror:n rotates within a row of 16 lanes; quad_perm[1,0,3,2] swaps neighbours.
+constexpr int kRowRor1 = 0x121, kRowRor2 = 0x122, kRowRor4 = 0x124, kRowRor8 = 0x128, kSwapPairs = 0xB1;
+
+__device__ __forceinline__ float wave_max(float x) {
+    x = fmaxf(x, dpp_f<kRowRor8>(x));
+    x = fmaxf(x, dpp_f<kRowRor4>(x));
+    x = fmaxf(x, dpp_f<kRowRor2>(x));
+    x = fmaxf(x, dpp_f<kRowRor1>(x));
+    return fmaxf(fmaxf(readlane_f(x, 0), readlane_f(x, 16)), fmaxf(readlane_f(x, 32), readlane_f(x, 48)));
+}
+__device__ __forceinline__ float wave_sum(float x) {
+    x += dpp_f<kRowRor8>(x);
+    x += dpp_f<kRowRor4>(x);
+    x += dpp_f<kRowRor2>(x);
+    x += dpp_f<kRowRor1>(x);
+    return (readlane_f(x, 0) + readlane_f(x, 16)) + (readlane_f(x, 32) + readlane_f(x, 48));
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// 16 bytes of K against 16 bytes of Q: 8 f16 products or 4 f32 products, f32 accumulate.
+template <typename T>
+__device__ __forceinline__ float dot16(const u32x4 &k, const u32x4 &q, float acc);
+template <>
+__device__ __forceinline__ float dot16<__half>(const u32x4 &k, const u32x4 &q, float acc) {
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, k[i]), __builtin_bit_cast(half2_t, q[i]), acc, false);
+    return acc;
+}
+template <>
+__device__ __forceinline__ float dot16<float>(const u32x4 &k, const u32x4 &q, float acc) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc = fmaf(__builtin_bit_cast(float, k[i]), __builtin_bit_cast(float, q[i]), acc);
+    return acc;
+}
+
+// The slice of a V row owned by one lane in the PV phase: EPL = D/16 elements.
+template <typename T, int EPL>
+struct VSlice;
+template <>
+struct VSlice<__half, 8> { typedef half8_t type; };
+template <>
+struct VSlice<__half, 4> { typedef half4_t type; };
+template <>
+struct VSlice<float, 8> { typedef float8_t type; };
+template <>
+struct VSlice<float, 4> { typedef float4_t type; };
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float x);
+template <>
+__device__ __forceinline__ __half from_f32<__half>(float x) { return __float2half_rn(x); }
+template <>
+__device__ __forceinline__ float from_f32<float>(float x) { return x; }
+
+// Rotation of the 16-byte chunks of LDS row t.  A 128-bit LDS read pass covers 16 lanes =
+// 8 rows x 2 half rows; with this rotation they fall into 16 different 16-byte bank groups.
+template <int CPR>
+__device__ __forceinline__ int rot(int row) {
+    return CPR == 8 ? (row >> 1) : row;
+}
+
+template <typename T, int D, int G>
+__global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1) void sdpa_decode_kernel(DecodeDev p) {
+    constexpr int RB = D * sizeof(T);   // bytes of one K/V row: 128, 256 or 512
+    constexpr int CPR = RB / 16;        // 16-byte chunks per row: 8, 16, 32
+    constexpr int HC = CPR / 2;         // chunks per half row (one QK lane)
+    constexpr int KL = kTile * CPR / 64;  // K loads per lane per tile
+    constexpr int EPL = D / 16;         // output columns per lane in the PV phase
+    constexpr int VI = kTile / 4;       // V rows per lane per tile
+    typedef typename VSlice<T, EPL>::type vslice_t;
+    static_assert(RB == 128 || RB == 256 || RB == 512, "unsupported row size");
+
+    __shared__ u32x4 lds_k[kWaves][kTile * CPR];
+    __shared__ u32x4 lds_q[G * CPR];
+    __shared__ float lds_p[kWaves][kTile * G];
+    __shared__ int lds_ticket;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int w = tid >> 6;
+    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+
+    // ---- stage the G query vectors of this KV head ------------------------------------
+    {
+        const u32x4 *qg = reinterpret_cast<const u32x4 *>(p.q + ((int64_t)b * p.Hq + (int64_t)kvh * G) * RB);
+        for (int i = tid; i < G * CPR; i += kThreads) lds_q[i] = qg[i];
+    }
+    __syncthreads();
+
+    const char *kbase = p.k + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+    const char *vbase = p.v + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+    const int n_tiles = (p.T + kTile - 1) / kTile;
+    const int tile_begin = split * p.tiles_per_split;
+    const int tile_end = min(n_tiles, tile_begin + p.tiles_per_split);
+    const int last_tok = p.T - 1;
+
+    float m[G], l[G], o[G][EPL];
+#pragma unroll
+    for (int h = 0; h < G; h++) {
+        m[h] = -INFINITY;
+        l[h] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; e++) o[h][e] = 0.0f;
+    }
+
+    // K load j of a tile fetches 16-byte chunk (j*64 + lane) of the tile, i.e. row
+    // (j*64+lane)/CPR, chunk (j*64+lane)%CPR: consecutive lanes, consecutive bytes.
+    // LDS slot of (row, chunk c): row*CPR + ((c + rot(row)) mod CPR).
+    const int rg = lane >> 4, j16 = lane & 15;
+    const int qk_row = lane >> 1, qk_half = lane & 1;
+    u32x4 kreg[KL];
+    vslice_t vreg[VI];
+    auto issue_k = [&](int tile) {
+        const int t0 = tile * kTile;
+#pragma unroll
+        for (int j = 0; j < KL; j++) {
+            int L = j * 64 + lane;
+            int row = L / CPR, c = L % CPR;
+            int tok = min(t0 + row, last_tok);
+            kreg[j] = *reinterpret_cast<const u32x4 *>(kbase + (int64_t)tok * p.kv_stride_t + c * 16);
+        }
+    };
+    auto issue_v = [&](int tile) {
+        const int t0 = tile * kTile;
+#pragma unroll
+        for (int i = 0; i < VI; i++) {
+            int tok = min(t0 + 4 * i + rg, last_tok);
+            vreg[i] = *reinterpret_cast<const vslice_t *>(vbase + (int64_t)tok * p.kv_stride_t +
+                                                          j16 * (int)sizeof(vslice_t));
+        }
+    };
+
+    int tile = tile_begin + w;
+    if (tile < tile_end) {
+        issue_k(tile);
+        issue_v(tile);
+    }
+
+    for (; tile < tile_end; tile += kWaves) {
+        const int t0 = tile * kTile;
+        // 1. park the K tile in LDS (rotated chunks); its registers are then refilled
+#pragma unroll
+        for (int j = 0; j < KL; j++) {
+            int L = j * 64 + lane;
+            int row = L / CPR, c = L % CPR;
+            lds_k[w][row * CPR + ((c + rot<CPR>(row)) & (CPR - 1))] = kreg[j];
+        }
+        const bool more = tile + kWaves < tile_end;
+        if (more) issue_k(tile + kWaves);
+
+        // 2. scores of token (t0 + qk_row): this lane covers chunks [qk_half*HC, +HC)
+        float s[G];
+#pragma unroll
+        for (int h = 0; h < G; h++) s[h] = 0.0f;
+#pragma unroll
+        for (int cc = 0; cc < HC; cc++) {
+            int c = qk_half * HC + cc;
+            u32x4 kc = lds_k[w][qk_row * CPR + ((c + rot<CPR>(qk_row)) & (CPR - 1))];
+#pragma unroll
+            for (int h = 0; h < G; h++) s[h] = dot16<T>(kc, lds_q[h * CPR + c], s[h]);
+        }
+        const bool valid = (t0 + qk_row) < p.T;
+        // 3. online softmax (wave-uniform running maximum per head)
+        float pr[G];
+#pragma unroll
+        for (int h = 0; h < G; h++) {
+            float full = s[h] + dpp_f<kSwapPairs>(s[h]);  // join the two half rows
+            float sv = valid ? full * p.scale_log2 : -INFINITY;
+            float m_new = fmaxf(m[h], wave_max(sv));
+            float alpha = fast_exp2(m[h] - m_new);
+            pr[h] = fast_exp2(sv - m_new);
+            l[h] = l[h] * alpha + pr[h];  // both lanes of a pair add p: halved at the end
+            m[h] = m_new;
+#pragma unroll
+            for (int e = 0; e < EPL; e++) o[h][e] *= alpha;
+        }
+        if (qk_half == 0) {
+            if constexpr (G == 4) {
+                float4_t t4 = {pr[0], pr[1], pr[2], pr[3]};
+                *reinterpret_cast<float4_t *>(&lds_p[w][qk_row * G]) = t4;
+            } else {
+#pragma unroll
+                for (int h = 0; h < G; h++) lds_p[w][qk_row * G + h] = pr[h];
+            }
+        }
+        // 4. O += P V (row group rg takes tokens 4*i + rg)
+#pragma unroll
+        for (int i = 0; i < VI; i++) {
+            float pp[G];
+            if constexpr (G == 4) {
+                float4_t t4 = *reinterpret_cast<const float4_t *>(&lds_p[w][(4 * i + rg) * G]);
+                pp[0] = t4[0], pp[1] = t4[1], pp[2] = t4[2], pp[3] = t4[3];
+            } else {
+#pragma unroll
+                for (int h = 0; h < G; h++) pp[h] = lds_p[w][(4 * i + rg) * G + h];
+            }
+            vslice_t vv = vreg[i];
+#pragma unroll
+            for (int e = 0; e < EPL; e++) {
+                float vf = (float)vv[e];
+#pragma unroll
+                for (int h = 0; h < G; h++) o[h][e] = fmaf(pp[h], vf, o[h][e]);
+            }
+        }
+        // 5. V of the wave's next tile (in flight while the next tile's QK runs)
+        if (more) issue_v(tile + kWaves);
+    }
+
+    // ---- merge the 4 row groups of the wave, then the 4 waves through LDS ----------------
+#pragma unroll
+    for (int h = 0; h < G; h++) {
+        l[h] = 0.5f * wave_sum(l[h]);
+#pragma unroll
+        for (int e = 0; e < EPL; e++) {
+            float x = o[h][e];
+            x += __shfl_xor(x, 16, 64);
+            x += __shfl_xor(x, 32, 64);
+            o[h][e] = x;
+        }
+    }
+    __syncthreads();  // every wave is done with its K tile: the space is reused below
+    float *comb = reinterpret_cast<float *>(&lds_k[0][0]);  // [kWaves][G*D + 2*G]
+    constexpr int kCombStride = G * D + 2 * G;
+    static_assert(sizeof(float) * kWaves * kCombStride <= sizeof(u32x4) * kWaves * kTile * CPR, "combine buffer");
+    if (rg == 0) {
+#pragma unroll
+        for (int h = 0; h < G; h++)
+#pragma unroll
+            for (int e = 0; e < EPL; e++) comb[w * kCombStride + h * D + j16 * EPL + e] = o[h][e];
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int h = 0; h < G; h++) {
+            comb[w * kCombStride + G * D + h] = m[h];
+            comb[w * kCombStride + G * D + G + h] = l[h];
+        }
+    }
+    __syncthreads();
+
+    const int64_t bh = (int64_t)b * p.Hkv + kvh;
+    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)b * p.Hq + (int64_t)kvh * G) * D;
+    for (int idx = tid; idx < G * D; idx += kThreads) {
+        int h = idx / D;
+        float mm = -INFINITY;
+#pragma unroll
+        for (int ww = 0; ww < kWaves; ww++) mm = fmaxf(mm, comb[ww * kCombStride + G * D + h]);
+        float acc = 0.0f, ll = 0.0f;
+#pragma unroll
+        for (int ww = 0; ww < kWaves; ww++) {
+            float f = fast_exp2(comb[ww * kCombStride + G * D + h] - mm);
+            acc += comb[ww * kCombStride + idx] * f;
+            ll += comb[ww * kCombStride + G * D + G + h] * f;
+        }
+        if (p.nsplit == 1) {
+            out[idx] = from_f32<T>(acc / ll);
+        } else {
+            int64_t slot = bh * p.nsplit + split;
+            p.part_o[slot * (G * D) + idx] = acc;
+            if ((idx % D) == 0) {
+                p.part_ml[slot * (2 * G) + h] = mm;
+                p.part_ml[slot * (2 * G) + G + h] = ll;
+            }
+        }
+    }
+    if (p.nsplit == 1) return;
+
+    // ---- last workgroup to arrive merges the splits ---------------------------------------
+    __threadfence();  // release: partials visible device-wide before the ticket is taken
+    __syncthreads();
+    if (tid == 0) lds_ticket = __hip_atomic_fetch_add(&p.counters[bh], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (lds_ticket != p.nsplit - 1) return;
+    __threadfence();  // acquire: see every other workgroup's partials
+    for (int idx = tid; idx < G * D; idx += kThreads) {
+        int h = idx / D;
+        float mm = -INFINITY;
+        for (int sp = 0; sp < p.nsplit; sp++)
+            mm = fmaxf(mm, __hip_atomic_load(&p.part_ml[(bh * p.nsplit + sp) * (2 * G) + h], __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT));
+        float acc = 0.0f, ll = 0.0f;
+        for (int sp = 0; sp < p.nsplit; sp++) {
+            int64_t slot = bh * p.nsplit + sp;
+            float f = fast_exp2(
+                __hip_atomic_load(&p.part_ml[slot * (2 * G) + h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - mm);
+            acc += __hip_atomic_load(&p.part_o[slot * (G * D) + idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+            ll += __hip_atomic_load(&p.part_ml[slot * (2 * G) + G + h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+        }
+        out[idx] = from_f32<T>(acc / ll);
+    }
+    if (tid == 0) __hip_atomic_store(&p.counters[bh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+}
+
+template <typename T, int D>
+int launch_g(const DecodeDev &p, int G, dim3 grid, hipStream_t s) {
+    switch (G) {
+        case 1: hipLaunchKernelGGL((sdpa_decode_kernel<T, D, 1>), grid, dim3(kThreads), 0, s, p); break;
+        case 2: hipLaunchKernelGGL((sdpa_decode_kernel<T, D, 2>), grid, dim3(kThreads), 0, s, p); break;
+        case 4: hipLaunchKernelGGL((sdpa_decode_kernel<T, D, 4>), grid, dim3(kThreads), 0, s, p); break;
+        case 8: hipLaunchKernelGGL((sdpa_decode_kernel<T, D, 8>), grid, dim3(kThreads), 0, s, p); break;
+        default: return 2;
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("sdpa_decode launch failed: %s", hipGetErrorString(e));
+    return 0;
+}
+
+}  // namespace
+
+// Partials: at most kMaxSplitRows rows of (D + 2) floats per query head.
+constexpr int64_t kMaxSplitRows = 8192;
+
+size_t decode_workspace_bytes(int64_t B, int64_t Hq, int64_t D) {
+    int64_t rows = B * Hq > kMaxSplitRows ? B * Hq : kMaxSplitRows;
+    return kWsCounterBytes + (size_t)rows * (size_t)(D + 2) * sizeof(float) + 256;
+}
+
+// Number of splits: enough workgroups to fill every CU twice over, never less than four
+// tiles per workgroup when the context allows it, bounded by the workspace.
+static int choose_splits(int64_t BH, int64_t G, int n_tiles) {
+    static int forced = -1;
+    if (forced < 0) {
+        const char *e = getenv("TROCM_DECODE_SPLITS");  // experiment knob, like tract's declare_knob!
+        forced = e ? atoi(e) : 0;
+    }
+    int64_t target = (int64_t)num_compute_units() * 2;
+    int64_t ns = forced > 0 ? forced : (target + BH - 1) / BH;
+    int64_t max_by_tiles = (n_tiles + kWaves - 1) / kWaves;
+    if (ns > max_by_tiles) ns = max_by_tiles;
+    int64_t max_by_ws = kMaxSplitRows / (BH * G);
+    if (ns > max_by_ws) ns = max_by_ws;
+    if (ns < 1) ns = 1;
+    return (int)ns;
+}
+
+int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
+    if (a.Sq != 1 || a.mask != nullptr) return 2;
+    if (a.kv_fmt != TROCM_F16 && a.kv_fmt != TROCM_F32) return 2;
+    if (a.q_dtype != a.kv_fmt) return 2;
+    if (a.D != 64 && a.D != 128) return 2;
+    if (a.Hq % a.Hkv) return 2;
+    int64_t G = a.Hq / a.Hkv;
+    if (G != 1 && G != 2 && G != 4 && G != 8) return 2;
+    size_t es = elem_bytes(a.kv_fmt);
+    // 128-bit loads: rows and bases must be 16-byte aligned
+    if ((a.kv_stride_b * es) % 16 || (a.kv_stride_h * es) % 16 || (a.kv_stride_t * es) % 16) return 2;
+    if ((uintptr_t)a.k % 16 || (uintptr_t)a.v % 16 || (uintptr_t)a.q % 16) return 2;
+    if (a.Sk <= 0 || a.Sk > (1ll << 30)) return 2;
+    int64_t BH = a.B * a.Hkv;
+    if (BH > (int64_t)(kWsCounterBytes / sizeof(int)) || a.B > 65535 || a.Hkv > 65535) return 2;
+
+    int n_tiles = (int)((a.Sk + kTile - 1) / kTile);
+    int nsplit = choose_splits(BH, G, n_tiles);
+    int tps = (n_tiles + nsplit - 1) / nsplit;
+    nsplit = (n_tiles + tps - 1) / tps;  // no empty split
+    if (nsplit > 1) {
+        TROCM_NOT_NULL(a.workspace);
+        size_t need = kWsCounterBytes + (size_t)BH * nsplit * G * (a.D + 2) * sizeof(float);
+        TROCM_REQUIRE(a.workspace_bytes >= need, "sdpa workspace too small: %zu bytes given, %zu needed",
+                      a.workspace_bytes, need);
+    }
+    DecodeDev p;
+    p.q = (const char *)a.q;
+    p.out = (char *)a.out;
+    p.k = (const char *)a.k;
+    p.v = (const char *)a.v;
+    p.kv_stride_b = a.kv_stride_b * es;
+    p.kv_stride_h = a.kv_stride_h * es;
+    p.kv_stride_t = a.kv_stride_t * es;
+    p.T = (int)a.Sk;
+    p.tiles_per_split = tps;
+    p.nsplit = nsplit;
+    p.Hq = (int)a.Hq;
+    p.Hkv = (int)a.Hkv;
+    p.scale_log2 = a.scale * 1.4426950408889634f;
+    p.counters = (int *)a.workspace;
+    p.part_ml = (float *)((char *)a.workspace + kWsCounterBytes);
+    p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * G;
+    dim3 grid(nsplit, (unsigned)a.Hkv, (unsigned)a.B);
+    if (a.kv_fmt == TROCM_F16)
+        return a.D == 128 ? launch_g<__half, 128>(p, (int)G, grid, s) : launch_g<__half, 64>(p, (int)G, grid, s);
+    return a.D == 128 ? launch_g<float, 128>(p, (int)G, grid, s) : launch_g<float, 64>(p, (int)G, grid, s);
+}
+
+}  // namespace trocm
+
+namespace trocm {
+// Ragged decode, first form: one split-K launch per sequence on the caller's stream
+// (launches on one stream are ordered, so the sequences can share the workspace).
+int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt, int64_t n_seq, int64_t Hq, int64_t Hkv,
+                              int64_t D, const RaggedSeq *seqs, float scale, void *workspace, size_t workspace_bytes,
+                              hipStream_t s) {
+    size_t es = elem_bytes(q_dtype);
+    for (int64_t i = 0; i < n_seq; i++) {
+        SdpaArgs a;
+        memset(&a, 0, sizeof(a));
+        a.q = (const char *)q + (size_t)i * Hq * D * es;
+        a.out = (char *)out + (size_t)i * Hq * D * es;
+        a.q_dtype = q_dtype, a.kv_fmt = kv_fmt;
+        a.k = seqs[i].k, a.v = seqs[i].v, a.k_scales = seqs[i].k_scales, a.v_scales = seqs[i].v_scales;
+        a.B = 1, a.Hq = Hq, a.Hkv = Hkv, a.Sq = 1, a.Sk = seqs[i].len, a.D = D;
+        a.kv_stride_t = D, a.kv_stride_h = seqs[i].cap * D, a.kv_stride_b = Hkv * seqs[i].cap * D;
+        a.mask_b = a.mask_h = 1;
+        a.scale = scale;
+        a.workspace = workspace, a.workspace_bytes = workspace_bytes;
+        int rc = launch_sdpa_decode(a, s);
+        if (rc == 2) rc = launch_sdpa_generic(a, s);
+        if (rc) return rc;
+    }
+    return 0;
+}
+}  // namespace trocm

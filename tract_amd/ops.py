@@ -1,0 +1,395 @@
+"""Host-side mirror of tract's KV-cache operators over the rocm C ABI.
+
+Names, arguments and error behaviour follow the reference operators so that the
+parity tests read like tract's own unit tests:
+
+* ``InPlaceKvCache``      transformers/src/ops/inplace_kv_cache.rs:28-114
+* ``InPlaceKvSdpa``/State transformers/src/ops/inplace_kv_cache.rs:131-290
+* ``DynKeyValueCache``/State transformers/src/ops/dyn_kv_cache.rs:90-183 (device twin:
+  gpu/src/ops/dyn_kv_cache.rs:8-125), here backed by the in-place cache
+* ``Sdpa``                transformers/src/ops/sdpa.rs:83-89, 296-356
+* ``BlockQuant``          linalg/src/frame/block_quant/mod.rs:36-108 (Q4_0; Q8_0 = Q8_1 without sum)
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import numpy as np
+
+from . import _lib
+from ._lib import F16, F32, Q4_0, Q8_0, TractRocmError, call
+from .runtime import DeviceTensor, Workspace, _sh, dtype_code
+
+_I64x4 = C.c_int64 * 4
+_I64x3 = C.c_int64 * 3
+
+
+def _as_device(x, stream=None) -> DeviceTensor:
+    return x if isinstance(x, DeviceTensor) else DeviceTensor.from_numpy(np.asarray(x), stream)
+
+
+def _canon4(shape):
+    """[B,H,S,D] view of a rank-3 ([B,S,D]) or rank-4 shape."""
+    if len(shape) == 4:
+        return tuple(shape)
+    if len(shape) == 3:
+        return (shape[0], 1, shape[1], shape[2])
+    raise TractRocmError(f"Inputs must be of rank 3 or 4, found {len(shape)}")
+
+
+class InPlaceKvCache:
+    """Geometric-growth in-place cache along `axis` (the token axis, rank-2)."""
+
+    def __init__(self, axis: int, storage_format: int | None = None):
+        self.axis = axis
+        self.storage_format = storage_format  # None: same as the first pushed tensor
+        self._h = None
+        self._shape = None
+        self._dtype = None
+
+    # -- lifetime
+    def _create(self, shape, dtype):
+        if self.axis != len(shape) - 2:
+            raise TractRocmError(f"kv-cache axis {self.axis} unsupported: the token axis must be rank-2")
+        B, H, _, D = _canon4(shape)
+        fmt = dtype_code(dtype) if self.storage_format is None else self.storage_format
+        h = C.c_void_p()
+        call("trocm_kv_cache_create", C.byref(h), fmt, B, H, D)
+        self._h, self._shape, self._dtype, self.storage_format = h, tuple(shape), np.dtype(dtype), fmt
+
+    def __del__(self):
+        try:
+            if self._h:
+                _lib.load().trocm_kv_cache_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+    # -- InPlaceKvCache API
+    def _get(self, what) -> int:
+        if self._h is None:
+            return 0
+        v = C.c_int64()
+        call("trocm_kv_cache_" + what, self._h, C.byref(v))
+        return v.value
+
+    def len(self) -> int:
+        return self._get("len")
+
+    def is_empty(self) -> bool:
+        return self.len() == 0
+
+    def capacity(self) -> int:
+        return self._get("capacity")
+
+    def reallocs(self) -> int:
+        return self._get("reallocs")
+
+    def reserve(self, capacity: int, like=None, stream=None) -> None:
+        if self._h is None:
+            if like is None:
+                raise TractRocmError("reserve on a cache that has seen no tensor needs `like=(shape, dtype)`")
+            self._create(*like)
+        call("trocm_kv_cache_reserve", self._h, capacity, _sh(stream))
+
+    def push(self, x, strides=None, stream=None) -> None:
+        """Append `x` ([.., S, D] device tensor or numpy array) along the token axis.
+        `strides`: element strides of a non-dense source view (shape stays x.shape)."""
+        t = _as_device(x, stream)
+        if self._h is None:
+            if t.shape[self.axis if self.axis >= 0 else 0] == 0:
+                return
+            self._create(t.shape, t.dtype)
+        if len(t.shape) != len(self._shape):
+            raise TractRocmError("rank mismatch in kv-cache push")
+        want = list(self._shape)
+        got = list(t.shape)
+        want[self.axis] = got[self.axis] = 0
+        if want != got:
+            raise TractRocmError(f"kv-cache push: shape {t.shape} does not match the cache's {self._shape} off-axis")
+        B, H, S, D = _canon4(t.shape)
+        st = strides if strides is not None else t.strides()
+        if len(st) == 3:
+            st = (st[0], 0, st[1], st[2])
+        call("trocm_kv_append", self._h, t.ptr, dtype_code(t.dtype), _I64x4(*st), S, _sh(stream))
+
+    def truncate(self, length: int) -> None:
+        if self._h is None:
+            raise TractRocmError("Can not truncate a zero-len kv-cache value")
+        call("trocm_kv_cache_truncate", self._h, length)
+
+    def row_bytes(self) -> int:
+        n = C.c_size_t()
+        call("trocm_kv_row_bytes", self._h, C.byref(n))
+        return n.value
+
+    def valid_contiguous(self, stream=None) -> np.ndarray:
+        """Dense host copy of the valid [0..len] region: the tensor for F32/F16 storage, the
+        canonical block bytes `[.., len, D/32*block_bytes]` (uint8) for Q8_0/Q4_0."""
+        if self._h is None:
+            raise TractRocmError("empty kv-cache")
+        n = self.len()
+        shape = list(self._shape)
+        shape[self.axis] = n
+        if self.storage_format in (F32, F16):
+            out = DeviceTensor(shape, np.float32 if self.storage_format == F32 else np.float16)
+        else:
+            shape[-1] = self.row_bytes()
+            out = DeviceTensor(shape, np.uint8)
+        call("trocm_kv_export", self._h, out.ptr, _sh(stream))
+        return out.to_numpy(stream)
+
+    def clone(self, stream=None) -> "InPlaceKvCache":
+        c = InPlaceKvCache(self.axis, self.storage_format)
+        if self._h is not None:
+            h = C.c_void_p()
+            call("trocm_kv_cache_clone", self._h, C.byref(h), _sh(stream))
+            c._h, c._shape, c._dtype = h, self._shape, self._dtype
+        return c
+
+    @property
+    def handle(self):
+        return self._h
+
+
+def _scale_arg(scale) -> float:
+    return float("nan") if scale is None else float(scale)
+
+
+class Sdpa:
+    """Scaled dot-product attention on plain device tensors (sdpa.rs:83-89)."""
+
+    def __init__(self, scale=None, datum_type=np.float32, acc_datum_type=np.float32, is_causal=False):
+        self.scale, self.datum_type, self.acc_datum_type, self.is_causal = scale, datum_type, acc_datum_type, is_causal
+        self._ws = None
+
+    def output_facts(self, q_shape, k_shape, v_shape, mask_shape=None):
+        """sdpa.rs:296-356."""
+        if self.is_causal and mask_shape is not None:
+            raise TractRocmError("Mask cannot be provided if is_causal=true")
+        rank = len(q_shape)
+        if rank not in (3, 4):
+            raise TractRocmError("Input tensors must be 3D or 4D")
+        if len(k_shape) != rank or len(v_shape) != rank:
+            raise TractRocmError(f"Q, K and V should have the same rank {rank}")
+        if rank == 4 and q_shape[1] % k_shape[1] != 0:
+            raise TractRocmError(f"Q heads ({q_shape[1]}) must be a multiple of K/V heads ({k_shape[1]})")
+        return tuple(q_shape[:-1]) + (v_shape[-1],)
+
+    def eval(self, q, k, v, mask=None, stream=None) -> DeviceTensor:
+        q, k, v = (_as_device(t, stream) for t in (q, k, v))
+        m = None if mask is None else _as_device(mask, stream)
+        self.output_facts(q.shape, k.shape, v.shape, None if m is None else m.shape)
+        if not (q.dtype == k.dtype == v.dtype) or (m is not None and m.dtype != q.dtype):
+            raise TractRocmError("Q, K, V and mask must share a datum type")
+        B, Hq, Sq, D = _canon4(q.shape)
+        _, Hkv, Sk, Dk = _canon4(k.shape)
+        if _canon4(v.shape) != (B, Hkv, Sk, D) or Dk != D:
+            raise TractRocmError("K/V shape mismatch")
+        mb = mh = 1
+        if m is not None:
+            ms = _canon4(m.shape)
+            if ms[2:] != (Sq, Sk):
+                raise TractRocmError(f"mask shape {m.shape} does not end in [q_len, kv_len]")
+            mb, mh = ms[0], ms[1]
+        out = DeviceTensor(q.shape, q.dtype)
+        if self._ws is None or self._ws_key != (B, Hq, D):
+            self._ws, self._ws_key = Workspace(B, Hq, Sq, D, stream), (B, Hq, D)
+        call("trocm_sdpa", q.ptr, k.ptr, v.ptr, None if m is None else m.ptr, out.ptr, dtype_code(q.dtype),
+             B, Hq, Hkv, Sq, Sk, D, None, mb, mh, _scale_arg(self.scale), int(self.is_causal),
+             self._ws.ptr, self._ws.nbytes, _sh(stream))
+        return out
+
+
+class InPlaceKvSdpa:
+    """Fused in-place KV-cache + attention op: inputs [Q, K_new, V_new], output Q-shaped."""
+
+    def __init__(self, axis: int = 2, causal: bool = True, scale=None, storage_format: int | None = None):
+        self.axis, self.causal, self.scale, self.storage_format = axis, causal, scale, storage_format
+
+    def name(self) -> str:
+        return "InPlaceKvSdpa"
+
+    def is_stateless(self) -> bool:
+        return False
+
+    def state(self) -> "InPlaceKvSdpaState":
+        return InPlaceKvSdpaState(self.axis, self.causal, self.scale, self.storage_format)
+
+    def output_facts(self, *shapes):
+        if len(shapes) != 3:
+            raise TractRocmError("InPlaceKvSdpa expects [Q, K_new, V_new]")
+        return tuple(shapes[0])
+
+
+class InPlaceKvSdpaState:
+    def __init__(self, axis, causal, scale, storage_format=None):
+        self.axis, self.causal, self.scale, self.storage_format = axis, causal, scale, storage_format
+        self.k = InPlaceKvCache(axis, storage_format)
+        self.v = InPlaceKvCache(axis, storage_format)
+        self._ws = None
+        self._ws_key = None
+
+    def eval(self, inputs, stream=None) -> DeviceTensor:
+        if len(inputs) != 3:
+            raise TractRocmError("InPlaceKvSdpa expects [Q, K_new, V_new]")
+        q, k_new, v_new = (_as_device(t, stream) for t in inputs)
+        self.k.push(k_new, stream=stream)
+        self.v.push(v_new, stream=stream)
+        return self.attend(q, stream)
+
+    def attend(self, q: DeviceTensor, stream=None, out: DeviceTensor | None = None) -> DeviceTensor:
+        B, Hq, Sq, D = _canon4(q.shape)
+        if out is None:
+            out = DeviceTensor(q.shape, q.dtype)
+        if self._ws is None or self._ws_key != (B, Hq, D):
+            self._ws, self._ws_key = Workspace(B, Hq, Sq, D, stream), (B, Hq, D)
+        if self.k.handle is None:
+            raise TractRocmError("empty kv-cache")
+        call("trocm_sdpa_cached", q.ptr, dtype_code(q.dtype), Hq, Sq, self.k.handle, self.v.handle, out.ptr,
+             _scale_arg(self.scale), int(self.causal), self._ws.ptr, self._ws.nbytes, _sh(stream))
+        return out
+
+    def save_to(self, states: list) -> None:
+        if not self.k.is_empty():
+            states.append(self.k.valid_contiguous())
+            states.append(self.v.valid_contiguous())
+
+    def load_from(self, states) -> None:
+        it = iter(states)
+        k = next(it, None)
+        if k is not None:
+            v = next(it, None)
+            if v is None:
+                raise TractRocmError("InPlaceKvSdpa load_from: expected V state after K")
+            self.k = InPlaceKvCache(self.axis, self.storage_format)
+            self.v = InPlaceKvCache(self.axis, self.storage_format)
+            self.k.push(k)
+            self.v.push(v)
+
+    def freeze(self) -> "InPlaceKvSdpaState":
+        f = InPlaceKvSdpaState(self.axis, self.causal, self.scale, self.storage_format)
+        f.k, f.v = self.k.clone(), self.v.clone()
+        return f
+
+    def unfreeze(self) -> "InPlaceKvSdpaState":
+        return self.freeze()
+
+
+class DynKeyValueCache:
+    """The dynamic KV-cache op (dyn_kv_cache.rs:177-183): one input, output = whole cache."""
+
+    def __init__(self, name: str, axis: int, storage_format: int | None = None):
+        self.name, self.axis, self.storage_format = name, axis, storage_format
+
+    def is_stateless(self) -> bool:
+        return False
+
+    def state(self) -> "DynKeyValueCacheState":
+        return DynKeyValueCacheState(self.name, self.axis, self.storage_format)
+
+
+class DynKeyValueCacheState:
+    def __init__(self, name, axis, storage_format=None):
+        self.name, self.axis = name, axis
+        self.kv_cache = InPlaceKvCache(axis, storage_format)
+
+    def eval(self, x, stream=None) -> InPlaceKvCache:
+        """Appends in place and returns the cache itself: consumers read (buffer, capacity, len)
+        instead of a freshly concatenated tensor."""
+        self.kv_cache.push(x, stream=stream)
+        return self.kv_cache
+
+    def resolve_symbols(self) -> int:
+        """The value bound to the past-length symbol P (dyn_kv_cache.rs:153-156)."""
+        return self.kv_cache.len()
+
+    def truncate(self, length: int) -> None:
+        if self.kv_cache.handle is None:
+            raise TractRocmError("Can not truncate a zero-len kv-cache value")
+        self.kv_cache.truncate(length)
+
+    def save_to(self, states: list) -> None:
+        if self.kv_cache.handle is None:
+            raise TractRocmError(f"KV cache {self.name} was never initialized")
+        states.append(self.kv_cache.valid_contiguous())
+
+    def load_from(self, states) -> None:
+        it = iter(states)
+        t = next(it, None)
+        if t is None:
+            raise TractRocmError("Not enough state initializers")
+        self.kv_cache = InPlaceKvCache(self.axis, self.kv_cache.storage_format)
+        self.kv_cache.push(t)
+
+    def freeze(self) -> "DynKeyValueCacheState":
+        f = DynKeyValueCacheState(self.name, self.axis, self.kv_cache.storage_format)
+        f.kv_cache = self.kv_cache.clone()
+        return f
+
+    unfreeze = freeze
+
+
+class BlockQuant:
+    """A block-quantisation format as a tensor op (block_quant/mod.rs:36-108)."""
+
+    def __init__(self, fmt: int, name: str, block_bytes: int):
+        self.fmt, self.name, self._bb = fmt, name, block_bytes
+
+    def block_len(self) -> int:
+        return 32
+
+    def block_bytes(self) -> int:
+        return self._bb
+
+    def _quant(self, x: np.ndarray, stream=None) -> np.ndarray:
+        if x.size % 32:
+            raise TractRocmError(f"{x.size} elements is not a multiple of the block length 32")
+        src = DeviceTensor.from_numpy(x, stream)
+        dst = DeviceTensor((x.size // 32 * self._bb,), np.uint8)
+        call("trocm_block_quant", self.fmt, src.ptr, dtype_code(x.dtype), x.size, dst.ptr, _sh(stream))
+        return dst.to_numpy(stream)
+
+    def quant_f32(self, x, stream=None) -> np.ndarray:
+        return self._quant(np.ascontiguousarray(x, dtype=np.float32), stream)
+
+    def quant_f16(self, x, stream=None) -> np.ndarray:
+        return self._quant(np.ascontiguousarray(x, dtype=np.float16), stream)
+
+    def _dequant(self, blob, dtype, stream=None) -> np.ndarray:
+        blob = np.ascontiguousarray(blob, dtype=np.uint8).reshape(-1)
+        if blob.size % self._bb:
+            raise TractRocmError(f"{blob.size} bytes is not a multiple of the block size {self._bb}")
+        n = blob.size // self._bb * 32
+        src = DeviceTensor.from_numpy(blob, stream)
+        dst = DeviceTensor((n,), dtype)
+        call("trocm_block_dequant", self.fmt, src.ptr, n, dst.ptr, dtype_code(dtype), _sh(stream))
+        return dst.to_numpy(stream)
+
+    def dequant_f32(self, blob, stream=None) -> np.ndarray:
+        return self._dequant(blob, np.float32, stream)
+
+    def dequant_f16(self, blob, stream=None) -> np.ndarray:
+        return self._dequant(blob, np.float16, stream)
+
+
+Q4_0_FORMAT = BlockQuant(Q4_0, "Q4_0", 18)
+Q8_0_FORMAT = BlockQuant(Q8_0, "Q8_0", 34)
+
+
+def sdpa_decode_ragged(q: DeviceTensor, k_caches, v_caches, scale=None, workspace: Workspace | None = None,
+                       stream=None, out: DeviceTensor | None = None) -> DeviceTensor:
+    """One decode step for `n_seq` independent sequences with their own caches and lengths.
+    q: [n_seq, Hq, 1, D]."""
+    n, Hq, _, D = q.shape
+    if len(k_caches) != n or len(v_caches) != n:
+        raise TractRocmError("ragged decode: one K and one V cache per sequence expected")
+    if out is None:
+        out = DeviceTensor(q.shape, q.dtype)
+    ws = workspace or Workspace(n, Hq, 1, D, stream)
+    ks = (C.c_void_p * n)(*[c.handle for c in k_caches])
+    vs = (C.c_void_p * n)(*[c.handle for c in v_caches])
+    call("trocm_sdpa_decode_ragged", q.ptr, dtype_code(q.dtype), Hq, n, ks, vs, out.ptr, _scale_arg(scale),
+         ws.ptr, ws.nbytes, _sh(stream))
+    return out
