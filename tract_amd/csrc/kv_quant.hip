@@ -23,6 +23,16 @@ namespace {
 __device__ __forceinline__ float load_elem(const float *p) { return *p; }
 __device__ __forceinline__ float load_elem(const __half *p) { return __half2float(*p); }
 
+// f32 -> f16, round to nearest even, as its own instruction.  The empty asm keeps the
+// compiler from folding a preceding multiply into a mixed-precision fma whose +0 addend
+// would turn a -0 product into +0 (the reference keeps the sign of zero).
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float x) {
+    asm volatile("" : "+v"(x));
+    return __half_as_ushort(__float2half_rn(x));
+}
+__device__ __forceinline__ void store_out(float *p, float x) { *p = x; }
+__device__ __forceinline__ void store_out(__half *p, float x) { *p = __ushort_as_half(f32_to_f16_bits(x)); }
+
 // Rust `f32 as i8`: truncate toward zero, saturate, NaN -> 0.
 __device__ __forceinline__ int sat_i8(float x) {
     if (x != x) return 0;
@@ -68,7 +78,7 @@ __device__ __forceinline__ uint16_t quant_q8(const float (&v)[32], uint32_t (&co
         }
         codes[w] = word;
     }
-    return __half_as_ushort(__float2half_rn(scale));
+    return f32_to_f16_bits(scale);
 }
 
 // Q4: byte j = code(elem j) | code(elem j+16) << 4 (q4_0.rs:39-44, helpers.rs:62-68).
@@ -91,7 +101,7 @@ __device__ __forceinline__ uint16_t quant_q4(const float (&v)[32], uint32_t (&co
         }
         codes[w] = word;
     }
-    return __half_as_ushort(__float2half_rn(scale));
+    return f32_to_f16_bits(scale);
 }
 
 template <typename SrcT>
@@ -219,12 +229,12 @@ __global__ __launch_bounds__(256) void block_dequant_kernel(int fmt, const uint8
         float d = __half2float(__ushort_as_half((uint16_t)(q[0] | (q[1] << 8))));
         DstT *o = dst + idx * 32;
         if (fmt == TROCM_Q8_0) {
-            for (int i = 0; i < 32; i++) o[i] = (DstT)__fmul_rn((float)(int8_t)q[2 + i], d);
+            for (int i = 0; i < 32; i++) store_out(o + i, __fmul_rn((float)(int8_t)q[2 + i], d));
         } else {
             for (int j = 0; j < 16; j++) {
                 int lo = q[2 + j] & 0xf, hi = q[2 + j] >> 4;
-                o[j] = (DstT)__fmul_rn((float)(lo - 8), d);
-                o[j + 16] = (DstT)__fmul_rn((float)(hi - 8), d);
+                store_out(o + j, __fmul_rn((float)(lo - 8), d));
+                store_out(o + j + 16, __fmul_rn((float)(hi - 8), d));
             }
         }
     }

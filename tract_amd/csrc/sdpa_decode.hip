@@ -88,19 +88,30 @@ __device__ __forceinline__ float wave_sum(float x) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // 16 bytes of K against 16 bytes of Q: 8 f16 products or 4 f32 products, f32 accumulate.
+// Vector elements are copied into scalars before any bit cast.
+__device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+
 template <typename T>
-__device__ __forceinline__ float dot16(const u32x4 &k, const u32x4 &q, float acc);
+__device__ __forceinline__ float dot16(u32x4 k, u32x4 q, float acc);
 template <>
-__device__ __forceinline__ float dot16<__half>(const u32x4 &k, const u32x4 &q, float acc) {
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, k[i]), __builtin_bit_cast(half2_t, q[i]), acc, false);
+__device__ __forceinline__ float dot16<__half>(u32x4 k, u32x4 q, float acc) {
+    uint32_t k0 = k.x, k1 = k.y, k2 = k.z, k3 = k.w;
+    uint32_t q0 = q.x, q1 = q.y, q2 = q.z, q3 = q.w;
+    acc = __builtin_amdgcn_fdot2(as_half2(k0), as_half2(q0), acc, false);
+    acc = __builtin_amdgcn_fdot2(as_half2(k1), as_half2(q1), acc, false);
+    acc = __builtin_amdgcn_fdot2(as_half2(k2), as_half2(q2), acc, false);
+    acc = __builtin_amdgcn_fdot2(as_half2(k3), as_half2(q3), acc, false);
     return acc;
 }
 template <>
-__device__ __forceinline__ float dot16<float>(const u32x4 &k, const u32x4 &q, float acc) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) acc = fmaf(__builtin_bit_cast(float, k[i]), __builtin_bit_cast(float, q[i]), acc);
+__device__ __forceinline__ float dot16<float>(u32x4 k, u32x4 q, float acc) {
+    uint32_t k0 = k.x, k1 = k.y, k2 = k.z, k3 = k.w;
+    uint32_t q0 = q.x, q1 = q.y, q2 = q.z, q3 = q.w;
+    acc = fmaf(as_f32(k0), as_f32(q0), acc);
+    acc = fmaf(as_f32(k1), as_f32(q1), acc);
+    acc = fmaf(as_f32(k2), as_f32(q2), acc);
+    acc = fmaf(as_f32(k3), as_f32(q3), acc);
     return acc;
 }
 
