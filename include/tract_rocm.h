@@ -72,6 +72,14 @@ int trocm_stream_destroy(void *stream);
 int trocm_stream_sync(void *stream);
 int trocm_device_sync(void);
 
+/* Per-launch timing with event pairs, the device profiler's mechanism
+ * (cuda/src/context.rs:363-453, cuda/src/kernels/launch_args.rs:77-90). */
+int trocm_event_create(void **event);
+int trocm_event_destroy(void *event);
+int trocm_event_record(void *event, void *stream);
+/* Waits for `stop`, then returns the time between the two events in milliseconds. */
+int trocm_event_elapsed_ms(void *start, void *stop, float *ms);
+
 /* DeviceContext::copy_nd (gpu/src/device.rs:26-35; CUDA: cuda/src/kernels/array/dispatch.rs:11-46):
  * strided N-d copy, rank 1..6, elem_size 1/2/4/8/16 bytes, strides in elements (may be
  * 0 for broadcast sources, never negative), byte offsets added to the base pointers. */
@@ -112,6 +120,11 @@ int trocm_kv_cache_reserve(trocm_kv_cache *cache, int64_t capacity, void *stream
  * quantises on the way in; an F32/F16 cache requires src_dtype == storage_format. */
 int trocm_kv_append(trocm_kv_cache *cache, const void *src, int src_dtype, const int64_t *src_strides,
                     int64_t n_new, void *stream);
+/* The two pushes of InPlaceKvSdpaState::eval (inplace_kv_cache.rs:199-204) in one call and, for
+ * F32/F16 caches with dense rows, one kernel launch: k_src and v_src share dtype and strides. */
+int trocm_kv_append_pair(trocm_kv_cache *k_cache, trocm_kv_cache *v_cache, const void *k_src,
+                         const void *v_src, int src_dtype, const int64_t *src_strides, int64_t n_new,
+                         void *stream);
 /* DynKeyValueCacheState::truncate (transformers/src/ops/dyn_kv_cache.rs:112-119): keep the first
  * `len` tokens (speculative-decoding rollback).  Fails on an empty cache like the reference. */
 int trocm_kv_cache_truncate(trocm_kv_cache *cache, int64_t len);
@@ -121,7 +134,7 @@ int trocm_kv_export(const trocm_kv_cache *cache, void *dst_device, void *stream)
 /* Bytes of one token of one head in the canonical export: head_dim*4, head_dim*2,
  * head_dim/32*34 or head_dim/32*18. */
 int trocm_kv_row_bytes(const trocm_kv_cache *cache, size_t *bytes);
-/* OpStateFreeze::freeze (:262-272): an independent deep copy (same len, capacity = len). */
+/* OpStateFreeze::freeze (:262-272): an independent deep copy (same len, capacity, reallocs). */
 int trocm_kv_cache_clone(const trocm_kv_cache *cache, trocm_kv_cache **out, void *stream);
 /* Raw view for kernels written against the cache: base pointers and capacity.
  * `scales` is NULL for F32/F16. */
@@ -141,8 +154,9 @@ int trocm_block_dequant(int format, const void *src_blocks, size_t n_elems, void
 /* Scratch for split-K partial results and arrival counters.  The arena planner of the
  * device layer does not model scratch (gpu/src/memory/schema.rs:56-128), so the op state
  * owns one workspace and passes it to every call.  trocm_sdpa_workspace_init() must run
- * once on a new workspace (it zeroes the counters); kernels leave it ready for the next
- * call.  Two calls that overlap in time must not share a workspace. */
+ * once on a new workspace (it zeroes the header area reserved for kernel-side counters);
+ * kernels leave it ready for the next call.  Two calls that overlap in time must not share
+ * a workspace. */
 int trocm_sdpa_workspace_bytes(int64_t batch, int64_t q_heads, int64_t q_len, int64_t head_dim,
                                size_t *bytes);
 int trocm_sdpa_workspace_init(void *workspace, size_t bytes, void *stream);
@@ -170,6 +184,14 @@ int trocm_sdpa(const void *q, const void *k, const void *v, const void *mask, vo
 int trocm_sdpa_cached(const void *q, int q_dtype, int64_t q_heads, int64_t q_len,
                       const trocm_kv_cache *k_cache, const trocm_kv_cache *v_cache, void *out,
                       float scale, int causal, void *workspace, size_t workspace_bytes, void *stream);
+
+/* InPlaceKvSdpaState::eval (inplace_kv_cache.rs:191-216) as one call: push k_new and v_new
+ * ([batch, kv_heads, n_new, head_dim] of `dtype`, element strides kv_new_strides[4] or NULL for
+ * dense) into the caches, then attend q ([batch, q_heads, n_new, head_dim] dense) over them. */
+int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_new, int dtype,
+                               int64_t q_heads, int64_t n_new, const int64_t *kv_new_strides,
+                               trocm_kv_cache *k_cache, trocm_kv_cache *v_cache, void *out, float scale,
+                               int causal, void *workspace, size_t workspace_bytes, void *stream);
 
 /* Ragged multi-sequence decode: `n_seq` independent sequences, each with its own K and V
  * cache (batch == 1 each, same heads/head_dim/format) and its own length; one query token

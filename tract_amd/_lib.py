@@ -37,6 +37,10 @@ SIGNATURES = {
     "trocm_stream_destroy": [_vp],
     "trocm_stream_sync": [_vp],
     "trocm_device_sync": [],
+    "trocm_event_create": [C.POINTER(_vp)],
+    "trocm_event_destroy": [_vp],
+    "trocm_event_record": [_vp, _vp],
+    "trocm_event_elapsed_ms": [_vp, _vp, C.POINTER(_f)],
     "trocm_copy_nd": [_vp, _sz, _pi64, _vp, _sz, _pi64, _pi64, _i, _i, _vp],
     "trocm_kv_cache_create": [C.POINTER(_vp), _i, _i64, _i64, _i64],
     "trocm_kv_cache_destroy": [_vp],
@@ -45,6 +49,7 @@ SIGNATURES = {
     "trocm_kv_cache_reallocs": [_vp, _pi64],
     "trocm_kv_cache_reserve": [_vp, _i64, _vp],
     "trocm_kv_append": [_vp, _vp, _i, _pi64, _i64, _vp],
+    "trocm_kv_append_pair": [_vp, _vp, _vp, _vp, _i, _pi64, _i64, _vp],
     "trocm_kv_cache_truncate": [_vp, _i64],
     "trocm_kv_export": [_vp, _vp, _vp],
     "trocm_kv_row_bytes": [_vp, C.POINTER(_sz)],
@@ -57,6 +62,7 @@ SIGNATURES = {
     "trocm_sdpa": [_vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i64, _i64, _i64, _i64, _pi64, _i64, _i64, _f, _i,
                    _vp, _sz, _vp],
     "trocm_sdpa_cached": [_vp, _i, _i64, _i64, _vp, _vp, _vp, _f, _i, _vp, _sz, _vp],
+    "trocm_inplace_kv_sdpa_eval": [_vp, _vp, _vp, _i, _i64, _i64, _pi64, _vp, _vp, _vp, _f, _i, _vp, _sz, _vp],
     "trocm_sdpa_decode_ragged": [_vp, _i, _i64, _i64, C.POINTER(_vp), C.POINTER(_vp), _vp, _f, _vp, _sz, _vp],
 }
 _RESTYPES = {"trocm_last_error": C.c_char_p}

@@ -248,6 +248,38 @@ int trocm_device_sync(void) {
     return 0;
 }
 
+int trocm_event_create(void **event) {
+    TROCM_NOT_NULL(event);
+    if (ensure_init()) return 1;
+    hipEvent_t e;
+    TROCM_HIP(hipEventCreate(&e));
+    *event = (void *)e;
+    return 0;
+}
+
+int trocm_event_destroy(void *event) {
+    if (!event) return 0;
+    TROCM_HIP(hipEventDestroy((hipEvent_t)event));
+    return 0;
+}
+
+int trocm_event_record(void *event, void *stream) {
+    TROCM_NOT_NULL(event);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    TROCM_HIP(hipEventRecord((hipEvent_t)event, s));
+    return 0;
+}
+
+int trocm_event_elapsed_ms(void *start, void *stop, float *ms) {
+    TROCM_NOT_NULL(start);
+    TROCM_NOT_NULL(stop);
+    TROCM_NOT_NULL(ms);
+    TROCM_HIP(hipEventSynchronize((hipEvent_t)stop));
+    TROCM_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return 0;
+}
+
 int trocm_copy_nd(void *dst, size_t dst_offset_bytes, const int64_t *dst_strides, const void *src,
                   size_t src_offset_bytes, const int64_t *src_strides, const int64_t *shape, int rank, int elem_size,
                   void *stream) {
@@ -324,20 +356,15 @@ int trocm_kv_cache_reserve(trocm_kv_cache *c, int64_t capacity, void *stream) {
     return regrow(c, capacity, s);
 }
 
-int trocm_kv_append(trocm_kv_cache *c, const void *src, int src_dtype, const int64_t *src_strides, int64_t n_new,
-                    void *stream) {
-    TROCM_NOT_NULL(c);
-    TROCM_REQUIRE(n_new >= 0, "append: negative token count");
-    if (n_new == 0) return 0;  // inplace_kv_cache.rs:57-59
+// Argument checks and the growth rule of push (inplace_kv_cache.rs:55-80).
+static int append_prepare(trocm_kv_cache *c, const void *src, int src_dtype, const int64_t *src_strides, int64_t n_new,
+                          hipStream_t s) {
     TROCM_NOT_NULL(src);
     TROCM_NOT_NULL(src_strides);
     TROCM_REQUIRE(src_dtype == TROCM_F32 || src_dtype == TROCM_F16, "append: source dtype must be F32 or F16");
     TROCM_REQUIRE(is_quant(c->fmt) || src_dtype == c->fmt,
                   "append: source dtype %d does not match the cache's storage format %d", src_dtype, c->fmt);
     for (int i = 0; i < 4; i++) TROCM_REQUIRE(src_strides[i] >= 0, "append: negative source strides are not supported");
-    hipStream_t s;
-    if (resolve_stream(stream, &s)) return 1;
-    // growth rule, inplace_kv_cache.rs:61-80
     if (c->cap == 0) {
         if (regrow(c, n_new, s)) return 1;
     } else if (c->len + n_new > c->cap) {
@@ -345,6 +372,12 @@ int trocm_kv_append(trocm_kv_cache *c, const void *src, int src_dtype, const int
         if (regrow(c, new_cap, s)) return 1;
         c->reallocs += 1;
     }
+    return 0;
+}
+
+// Write the new tokens at [len, len + n_new) (capacity is already sufficient).
+static int append_write(trocm_kv_cache *c, const void *src, int src_dtype, const int64_t *src_strides, int64_t n_new,
+                        hipStream_t s) {
     if (is_quant(c->fmt)) {
         QuantAppend a;
         a.fmt = c->fmt, a.src_dtype = src_dtype;
@@ -352,20 +385,64 @@ int trocm_kv_append(trocm_kv_cache *c, const void *src, int src_dtype, const int
         for (int i = 0; i < 4; i++) a.ss[i] = src_strides[i];
         a.cap = c->cap, a.t0 = c->len;
         a.src = src, a.codes = c->data, a.scales = c->scales;
-        if (launch_quant_append(a, s)) return 1;
-    } else {
-        int64_t es = (int64_t)elem_bytes(c->fmt);
-        CopyNd d;
-        d.rank = 4;
-        d.shape[0] = c->B, d.shape[1] = c->H, d.shape[2] = n_new, d.shape[3] = c->D;
-        for (int i = 0; i < 4; i++) d.src_stride[i] = src_strides[i] * es;
-        d.dst_stride[0] = c->H * c->cap * c->D * es;
-        d.dst_stride[1] = c->cap * c->D * es;
-        d.dst_stride[2] = c->D * es;
-        d.dst_stride[3] = es;
-        if (launch_copy_nd((char *)c->data + c->len * c->D * es, src, d, (int)es, s)) return 1;
+        return launch_quant_append(a, s);
     }
+    int64_t es = (int64_t)elem_bytes(c->fmt);
+    CopyNd d;
+    d.rank = 4;
+    d.shape[0] = c->B, d.shape[1] = c->H, d.shape[2] = n_new, d.shape[3] = c->D;
+    for (int i = 0; i < 4; i++) d.src_stride[i] = src_strides[i] * es;
+    d.dst_stride[0] = c->H * c->cap * c->D * es;
+    d.dst_stride[1] = c->cap * c->D * es;
+    d.dst_stride[2] = c->D * es;
+    d.dst_stride[3] = es;
+    return launch_copy_nd((char *)c->data + c->len * c->D * es, src, d, (int)es, s);
+}
+
+int trocm_kv_append(trocm_kv_cache *c, const void *src, int src_dtype, const int64_t *src_strides, int64_t n_new,
+                    void *stream) {
+    TROCM_NOT_NULL(c);
+    TROCM_REQUIRE(n_new >= 0, "append: negative token count");
+    if (n_new == 0) return 0;  // inplace_kv_cache.rs:57-59
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    if (append_prepare(c, src, src_dtype, src_strides, n_new, s)) return 1;
+    if (append_write(c, src, src_dtype, src_strides, n_new, s)) return 1;
     c->len += n_new;
+    return 0;
+}
+
+int trocm_kv_append_pair(trocm_kv_cache *kc, trocm_kv_cache *vc, const void *k_src, const void *v_src, int src_dtype,
+                         const int64_t *src_strides, int64_t n_new, void *stream) {
+    TROCM_NOT_NULL(kc);
+    TROCM_NOT_NULL(vc);
+    TROCM_REQUIRE(n_new >= 0, "append: negative token count");
+    TROCM_REQUIRE(kc->fmt == vc->fmt && kc->B == vc->B && kc->H == vc->H && kc->D == vc->D,
+                  "K and V caches differ in format or shape");
+    if (n_new == 0) return 0;
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    if (append_prepare(kc, k_src, src_dtype, src_strides, n_new, s)) return 1;
+    if (append_prepare(vc, v_src, src_dtype, src_strides, n_new, s)) return 1;
+    int rc = 2;
+    if (!is_quant(kc->fmt) && src_strides[3] == 1 && kc->cap == vc->cap && kc->len == vc->len) {
+        int64_t es = (int64_t)elem_bytes(kc->fmt);
+        AppendPair a;
+        a.src[0] = k_src, a.src[1] = v_src;
+        a.dst[0] = (char *)kc->data + kc->len * kc->D * es;
+        a.dst[1] = (char *)vc->data + vc->len * vc->D * es;
+        a.B = kc->B, a.H = kc->H, a.S = n_new, a.row_bytes = kc->D * es;
+        for (int i = 0; i < 3; i++) a.src_stride[i] = src_strides[i] * es;
+        a.dst_stride[0] = kc->H * kc->cap * kc->D * es, a.dst_stride[1] = kc->cap * kc->D * es, a.dst_stride[2] = kc->D * es;
+        rc = launch_append_pair(a, s);
+    }
+    if (rc == 2) {
+        rc = append_write(kc, k_src, src_dtype, src_strides, n_new, s);
+        if (!rc) rc = append_write(vc, v_src, src_dtype, src_strides, n_new, s);
+    }
+    if (rc) return rc;
+    kc->len += n_new;
+    vc->len += n_new;
     return 0;
 }
 
@@ -559,6 +636,20 @@ int trocm_sdpa_cached(const void *q, int q_dtype, int64_t q_heads, int64_t q_len
     a.causal = causal;
     a.workspace = workspace, a.workspace_bytes = workspace_bytes;
     return dispatch_sdpa(a, s);
+}
+
+int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_new, int dtype, int64_t q_heads,
+                               int64_t n_new, const int64_t *kv_new_strides, trocm_kv_cache *kc, trocm_kv_cache *vc,
+                               void *out, float scale, int causal, void *workspace, size_t workspace_bytes,
+                               void *stream) {
+    TROCM_NOT_NULL(kc);
+    int64_t dense[4];
+    if (!kv_new_strides) {
+        dense[3] = 1, dense[2] = kc->D, dense[1] = n_new * kc->D, dense[0] = kc->H * n_new * kc->D;
+        kv_new_strides = dense;
+    }
+    if (trocm_kv_append_pair(kc, vc, k_new, v_new, dtype, kv_new_strides, n_new, stream)) return 1;
+    return trocm_sdpa_cached(q, dtype, q_heads, n_new, kc, vc, out, scale, causal, workspace, workspace_bytes, stream);
 }
 
 int trocm_sdpa_decode_ragged(const void *q, int q_dtype, int64_t q_heads, int64_t n_seq,

@@ -63,6 +63,18 @@ struct CopyNd {
 };
 int launch_copy_nd(void *dst, const void *src, const CopyNd &desc, int elem_size, hipStream_t s);
 
+// Two same-shaped appends (K and V) in one launch; rows dense, everything 16-byte aligned.
+// Returns 2 when the shapes do not qualify (the caller then issues two copy_nd).
+struct AppendPair {
+    const void *src[2];
+    void *dst[2];           // already offset to the first appended token
+    int64_t B, H, S;
+    int64_t row_bytes;
+    int64_t src_stride[3];  // bytes: batch, head, token (same for both tensors)
+    int64_t dst_stride[3];
+};
+int launch_append_pair(const AppendPair &a, hipStream_t s);
+
 // Quantise [rows, d] (row r of the source at src + b*ss[0] + h*ss[1] + t*ss[2] elements, element
 // stride ss[3]) into the code/scale planes of a cache at token offset t0.
 struct QuantAppend {

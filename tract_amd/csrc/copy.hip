@@ -53,7 +53,62 @@ int launch_typed(char *dst, const char *src, const CopyDev &p, uint64_t total, h
     return 0;
 }
 
+// K and V appended in one launch: blockIdx.y selects the tensor.  Rows of `row_bytes`
+// (a multiple of 16) are dense in source and destination; 16 bytes per thread.
+struct AppendPairDev {
+    const char *src[2];
+    char *dst[2];
+    int64_t src_stride[3];  // bytes: batch, head, token
+    int64_t dst_stride[3];
+    uint32_t H, S, chunks_per_row;
+    uint32_t total;  // B*H*S*chunks_per_row
+};
+
+__global__ __launch_bounds__(256) void append_pair_kernel(AppendPairDev p) {
+    const char *src = p.src[blockIdx.y];
+    char *dst = p.dst[blockIdx.y];
+    for (uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x; idx < p.total; idx += gridDim.x * blockDim.x) {
+        uint32_t c = idx % p.chunks_per_row;
+        uint32_t r = idx / p.chunks_per_row;
+        uint32_t t = r % p.S;
+        r /= p.S;
+        uint32_t h = r % p.H;
+        uint32_t b = r / p.H;
+        const uint4 *sp = reinterpret_cast<const uint4 *>(src + b * p.src_stride[0] + h * p.src_stride[1] +
+                                                          t * p.src_stride[2] + (int64_t)c * 16);
+        uint4 *dp = reinterpret_cast<uint4 *>(dst + b * p.dst_stride[0] + h * p.dst_stride[1] + t * p.dst_stride[2] +
+                                              (int64_t)c * 16);
+        *dp = *sp;
+    }
+}
+
 }  // namespace
+
+int launch_append_pair(const AppendPair &a, hipStream_t s) {
+    AppendPairDev p;
+    uint64_t total = (uint64_t)a.B * a.H * a.S * (a.row_bytes / 16);
+    if (total == 0) return 0;
+    if (a.row_bytes % 16 || total >= (1ull << 31)) return 2;
+    for (int t = 0; t < 2; t++) {
+        if ((uintptr_t)a.src[t] % 16 || (uintptr_t)a.dst[t] % 16) return 2;
+        p.src[t] = (const char *)a.src[t];
+        p.dst[t] = (char *)a.dst[t];
+    }
+    for (int i = 0; i < 3; i++) {
+        if (a.src_stride[i] % 16 || a.dst_stride[i] % 16) return 2;
+        p.src_stride[i] = a.src_stride[i];
+        p.dst_stride[i] = a.dst_stride[i];
+    }
+    p.H = (uint32_t)a.H, p.S = (uint32_t)a.S, p.chunks_per_row = (uint32_t)(a.row_bytes / 16);
+    p.total = (uint32_t)total;
+    uint64_t blocks = (total + 255) / 256;
+    uint64_t cap = (uint64_t)num_compute_units() * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(append_pair_kernel, dim3((unsigned)blocks, 2), dim3(256), 0, s, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("append_pair launch failed: %s", hipGetErrorString(e));
+    return 0;
+}
 
 int launch_copy_nd(void *dst_v, const void *src_v, const CopyNd &in, int elem_size, hipStream_t s) {
     TROCM_REQUIRE(in.rank >= 1 && in.rank <= 6, "copy_nd: rank %d not in 1..6", in.rank);

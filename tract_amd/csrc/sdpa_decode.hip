@@ -21,9 +21,11 @@
 //
 // Combination
 //   waves are merged through LDS; if the launch has several splits, each workgroup
-//   stores its unnormalised (O, m, l) to the workspace, takes a ticket from an arrival
-//   counter and the last one to arrive merges all splits and writes the output, so one
-//   launch does the whole job.  Logits are kept in log2 units (scale * log2 e folded in).
+//   stores its unnormalised (O, m, l) to the workspace and a second, tiny launch on the
+//   same stream merges the splits of every (batch, kv head) and writes the output.  (A
+//   single-launch "last workgroup merges" scheme needs device-scope release/acquire fences,
+//   i.e. an L2 write-back and invalidate per workgroup on this multi-XCD part; measured, that
+//   tripled the kernel time.)  Logits are kept in log2 units (scale * log2 e folded in).
 //
 // Roofline: HBM-bound.  Algorithmic bytes per launch = 2*B*Hkv*T*D*e (K and V once per KV
 // head) + Q read + O write.
@@ -57,7 +59,6 @@ struct DecodeDev {
     float scale_log2;
     float *part_o;   // [B*Hkv*nsplit][G*D]
     float *part_ml;  // [B*Hkv*nsplit][2*G]
-    int *counters;   // [B*Hkv]
 };
 
 template <int CTRL>
@@ -134,6 +135,28 @@ __device__ __forceinline__ __half from_f32<__half>(float x) { return __float2hal
 template <>
 __device__ __forceinline__ float from_f32<float>(float x) { return x; }
 
+// Merge the per-split partials (O, m, l) of one (batch, kv head) and write the output rows.
+template <typename T, int D, int G>
+__device__ __forceinline__ void merge_splits(const DecodeDev &p, int64_t bh, T *out, int tid) {
+    for (int idx = tid; idx < G * D; idx += kThreads) {
+        const int h = idx / D;
+        const float *ml = p.part_ml + bh * p.nsplit * (2 * G);
+        const float *po = p.part_o + bh * p.nsplit * (G * D) + idx;
+        auto ld = [&](const float *a) { return *a; };
+        float mm = -INFINITY;
+#pragma unroll 4
+        for (int sp = 0; sp < p.nsplit; sp++) mm = fmaxf(mm, ld(ml + sp * (2 * G) + h));
+        float acc = 0.0f, ll = 0.0f;
+#pragma unroll 4
+        for (int sp = 0; sp < p.nsplit; sp++) {
+            float f = fast_exp2(ld(ml + sp * (2 * G) + h) - mm);
+            acc += ld(po + (int64_t)sp * (G * D)) * f;
+            ll += ld(ml + sp * (2 * G) + G + h) * f;
+        }
+        out[idx] = from_f32<T>(acc / ll);
+    }
+}
+
 // Rotation of the 16-byte chunks of LDS row t.  A 128-bit LDS read pass covers 16 lanes =
 // 8 rows x 2 half rows; with this rotation they fall into 16 different 16-byte bank groups.
 template <int CPR>
@@ -155,7 +178,6 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     __shared__ u32x4 lds_k[kWaves][kTile * CPR];
     __shared__ u32x4 lds_q[G * CPR];
     __shared__ float lds_p[kWaves][kTile * G];
-    __shared__ int lds_ticket;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -188,27 +210,52 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     // K load j of a tile fetches 16-byte chunk (j*64 + lane) of the tile, i.e. row
     // (j*64+lane)/CPR, chunk (j*64+lane)%CPR: consecutive lanes, consecutive bytes.
     // LDS slot of (row, chunk c): row*CPR + ((c + rot(row)) mod CPR).
+    // Addresses are a wave-uniform tile base plus per-lane 32-bit offsets that never change;
+    // only the one partial tile at the end of the sequence clamps its rows to the last token.
     const int rg = lane >> 4, j16 = lane & 15;
     const int qk_row = lane >> 1, qk_half = lane & 1;
+    const uint32_t stride_t = (uint32_t)p.kv_stride_t;
+    uint32_t k_off[KL], k_slot[KL], v_off[VI];
+#pragma unroll
+    for (int j = 0; j < KL; j++) {
+        int L = j * 64 + lane;
+        int row = L / CPR, c = L % CPR;
+        k_off[j] = (uint32_t)row * stride_t + (uint32_t)c * 16u;
+        k_slot[j] = row * CPR + ((c + rot<CPR>(row)) & (CPR - 1));
+    }
+#pragma unroll
+    for (int i = 0; i < VI; i++) v_off[i] = (uint32_t)(4 * i + rg) * stride_t + (uint32_t)j16 * (uint32_t)sizeof(vslice_t);
+
     u32x4 kreg[KL];
     vslice_t vreg[VI];
     auto issue_k = [&](int tile) {
         const int t0 = tile * kTile;
+        const char *base = kbase + (int64_t)t0 * p.kv_stride_t;
+        if (t0 + kTile <= p.T) {
 #pragma unroll
-        for (int j = 0; j < KL; j++) {
-            int L = j * 64 + lane;
-            int row = L / CPR, c = L % CPR;
-            int tok = min(t0 + row, last_tok);
-            kreg[j] = *reinterpret_cast<const u32x4 *>(kbase + (int64_t)tok * p.kv_stride_t + c * 16);
+            for (int j = 0; j < KL; j++) kreg[j] = *reinterpret_cast<const u32x4 *>(base + k_off[j]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < KL; j++) {
+                int L = j * 64 + lane;
+                int row = min(L / CPR, last_tok - t0), c = L % CPR;
+                kreg[j] = *reinterpret_cast<const u32x4 *>(base + (uint32_t)row * stride_t + (uint32_t)c * 16u);
+            }
         }
     };
     auto issue_v = [&](int tile) {
         const int t0 = tile * kTile;
+        const char *base = vbase + (int64_t)t0 * p.kv_stride_t;
+        if (t0 + kTile <= p.T) {
 #pragma unroll
-        for (int i = 0; i < VI; i++) {
-            int tok = min(t0 + 4 * i + rg, last_tok);
-            vreg[i] = *reinterpret_cast<const vslice_t *>(vbase + (int64_t)tok * p.kv_stride_t +
-                                                          j16 * (int)sizeof(vslice_t));
+            for (int i = 0; i < VI; i++) vreg[i] = *reinterpret_cast<const vslice_t *>(base + v_off[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < VI; i++) {
+                int row = min(4 * i + rg, last_tok - t0);
+                vreg[i] = *reinterpret_cast<const vslice_t *>(base + (uint32_t)row * stride_t +
+                                                              (uint32_t)j16 * (uint32_t)sizeof(vslice_t));
+            }
         }
     };
 
@@ -217,16 +264,14 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
         issue_k(tile);
         issue_v(tile);
     }
+    const u32x4 *lds_krow = &lds_k[w][qk_row * CPR];
+    const int qk_rot = rot<CPR>(qk_row) + qk_half * HC;
 
     for (; tile < tile_end; tile += kWaves) {
         const int t0 = tile * kTile;
         // 1. park the K tile in LDS (rotated chunks); its registers are then refilled
 #pragma unroll
-        for (int j = 0; j < KL; j++) {
-            int L = j * 64 + lane;
-            int row = L / CPR, c = L % CPR;
-            lds_k[w][row * CPR + ((c + rot<CPR>(row)) & (CPR - 1))] = kreg[j];
-        }
+        for (int j = 0; j < KL; j++) lds_k[w][k_slot[j]] = kreg[j];
         const bool more = tile + kWaves < tile_end;
         if (more) issue_k(tile + kWaves);
 
@@ -234,12 +279,11 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
         float s[G];
 #pragma unroll
         for (int h = 0; h < G; h++) s[h] = 0.0f;
-#pragma unroll
+#pragma unroll 2
         for (int cc = 0; cc < HC; cc++) {
-            int c = qk_half * HC + cc;
-            u32x4 kc = lds_k[w][qk_row * CPR + ((c + rot<CPR>(qk_row)) & (CPR - 1))];
+            u32x4 kc = lds_krow[(cc + qk_rot) & (CPR - 1)];
 #pragma unroll
-            for (int h = 0; h < G; h++) s[h] = dot16<T>(kc, lds_q[h * CPR + c], s[h]);
+            for (int h = 0; h < G; h++) s[h] = dot16<T>(kc, lds_q[h * CPR + qk_half * HC + cc], s[h]);
         }
         const bool valid = (t0 + qk_row) < p.T;
         // 3. online softmax (wave-uniform running maximum per head)
@@ -344,41 +388,31 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
             }
         }
     }
-    if (p.nsplit == 1) return;
+}
 
-    // ---- last workgroup to arrive merges the splits ---------------------------------------
-    __threadfence();  // release: partials visible device-wide before the ticket is taken
-    __syncthreads();
-    if (tid == 0) lds_ticket = __hip_atomic_fetch_add(&p.counters[bh], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (lds_ticket != p.nsplit - 1) return;
-    __threadfence();  // acquire: see every other workgroup's partials
-    for (int idx = tid; idx < G * D; idx += kThreads) {
-        int h = idx / D;
-        float mm = -INFINITY;
-        for (int sp = 0; sp < p.nsplit; sp++)
-            mm = fmaxf(mm, __hip_atomic_load(&p.part_ml[(bh * p.nsplit + sp) * (2 * G) + h], __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_AGENT));
-        float acc = 0.0f, ll = 0.0f;
-        for (int sp = 0; sp < p.nsplit; sp++) {
-            int64_t slot = bh * p.nsplit + sp;
-            float f = fast_exp2(
-                __hip_atomic_load(&p.part_ml[slot * (2 * G) + h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - mm);
-            acc += __hip_atomic_load(&p.part_o[slot * (G * D) + idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
-            ll += __hip_atomic_load(&p.part_ml[slot * (2 * G) + G + h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
-        }
-        out[idx] = from_f32<T>(acc / ll);
-    }
-    if (tid == 0) __hip_atomic_store(&p.counters[bh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+// Merge launch: grid (kv_heads, batch), runs after the split kernel on the same stream.
+template <typename T, int D, int G>
+__global__ __launch_bounds__(kThreads) void sdpa_decode_merge_kernel(DecodeDev p) {
+    const int kvh = blockIdx.x, b = blockIdx.y;
+    const int64_t bh = (int64_t)b * p.Hkv + kvh;
+    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)b * p.Hq + (int64_t)kvh * G) * D;
+    merge_splits<T, D, G>(p, bh, out, threadIdx.x);
+}
+
+template <typename T, int D, int G>
+void launch_both(const DecodeDev &p, dim3 grid, hipStream_t s) {
+    hipLaunchKernelGGL((sdpa_decode_kernel<T, D, G>), grid, dim3(kThreads), 0, s, p);
+    if (p.nsplit > 1)
+        hipLaunchKernelGGL((sdpa_decode_merge_kernel<T, D, G>), dim3(grid.y, grid.z), dim3(kThreads), 0, s, p);
 }
 
 template <typename T, int D>
 int launch_g(const DecodeDev &p, int G, dim3 grid, hipStream_t s) {
     switch (G) {
-        case 1: hipLaunchKernelGGL((sdpa_decode_kernel<T, D, 1>), grid, dim3(kThreads), 0, s, p); break;
-        case 2: hipLaunchKernelGGL((sdpa_decode_kernel<T, D, 2>), grid, dim3(kThreads), 0, s, p); break;
-        case 4: hipLaunchKernelGGL((sdpa_decode_kernel<T, D, 4>), grid, dim3(kThreads), 0, s, p); break;
-        case 8: hipLaunchKernelGGL((sdpa_decode_kernel<T, D, 8>), grid, dim3(kThreads), 0, s, p); break;
+        case 1: launch_both<T, D, 1>(p, grid, s); break;
+        case 2: launch_both<T, D, 2>(p, grid, s); break;
+        case 4: launch_both<T, D, 4>(p, grid, s); break;
+        case 8: launch_both<T, D, 8>(p, grid, s); break;
         default: return 2;
     }
     hipError_t e = hipGetLastError();
@@ -396,16 +430,19 @@ size_t decode_workspace_bytes(int64_t B, int64_t Hq, int64_t D) {
     return kWsCounterBytes + (size_t)rows * (size_t)(D + 2) * sizeof(float) + 256;
 }
 
-// Number of splits: enough workgroups to fill every CU twice over, never less than four
-// tiles per workgroup when the context allows it, bounded by the workspace.
+// Number of splits.  Measured on MI355X (8k context, f16, G=4): one workgroup per compute
+// unit is the sweet spot -- each wave already keeps a 16 KiB tile in flight, so more
+// workgroups add merge work and scheduling rounds without adding bandwidth (B=8: 4 splits
+// = 256 workgroups 45.9 us; 8 splits 48.9 us; 32 splits 55.5 us).  Never fewer than one
+// tile per wave, bounded by the workspace.
 static int choose_splits(int64_t BH, int64_t G, int n_tiles) {
     static int forced = -1;
     if (forced < 0) {
         const char *e = getenv("TROCM_DECODE_SPLITS");  // experiment knob, like tract's declare_knob!
         forced = e ? atoi(e) : 0;
     }
-    int64_t target = (int64_t)num_compute_units() * 2;
-    int64_t ns = forced > 0 ? forced : (target + BH - 1) / BH;
+    int64_t target = (int64_t)num_compute_units();
+    int64_t ns = forced > 0 ? forced : (target + BH / 2) / BH;
     int64_t max_by_tiles = (n_tiles + kWaves - 1) / kWaves;
     if (ns > max_by_tiles) ns = max_by_tiles;
     int64_t max_by_ws = kMaxSplitRows / (BH * G);
@@ -454,7 +491,7 @@ int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
     p.Hq = (int)a.Hq;
     p.Hkv = (int)a.Hkv;
     p.scale_log2 = a.scale * 1.4426950408889634f;
-    p.counters = (int *)a.workspace;
+
     p.part_ml = (float *)((char *)a.workspace + kWsCounterBytes);
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * G;
     dim3 grid(nsplit, (unsigned)a.Hkv, (unsigned)a.B);

@@ -101,18 +101,20 @@ class InPlaceKvCache:
             if t.shape[self.axis if self.axis >= 0 else 0] == 0:
                 return
             self._create(t.shape, t.dtype)
-        if len(t.shape) != len(self._shape):
-            raise TractRocmError("rank mismatch in kv-cache push")
-        want = list(self._shape)
-        got = list(t.shape)
-        want[self.axis] = got[self.axis] = 0
-        if want != got:
-            raise TractRocmError(f"kv-cache push: shape {t.shape} does not match the cache's {self._shape} off-axis")
+        self._check_push_shape(t.shape)
         B, H, S, D = _canon4(t.shape)
         st = strides if strides is not None else t.strides()
         if len(st) == 3:
             st = (st[0], 0, st[1], st[2])
         call("trocm_kv_append", self._h, t.ptr, dtype_code(t.dtype), _I64x4(*st), S, _sh(stream))
+
+    def _check_push_shape(self, shape) -> None:
+        if len(shape) != len(self._shape):
+            raise TractRocmError("rank mismatch in kv-cache push")
+        want, got = list(self._shape), list(shape)
+        want[self.axis] = got[self.axis] = 0
+        if want != got:
+            raise TractRocmError(f"kv-cache push: shape {tuple(shape)} does not match the cache's {self._shape} off-axis")
 
     def truncate(self, length: int) -> None:
         if self._h is None:
@@ -235,9 +237,29 @@ class InPlaceKvSdpaState:
         if len(inputs) != 3:
             raise TractRocmError("InPlaceKvSdpa expects [Q, K_new, V_new]")
         q, k_new, v_new = (_as_device(t, stream) for t in inputs)
-        self.k.push(k_new, stream=stream)
-        self.v.push(v_new, stream=stream)
-        return self.attend(q, stream)
+        return self.eval_into(q, k_new, v_new, None, stream)
+
+    def eval_into(self, q: DeviceTensor, k_new: DeviceTensor, v_new: DeviceTensor, out: DeviceTensor | None = None,
+                  stream=None) -> DeviceTensor:
+        """`eval` on device tensors with a caller-provided output: one C call per step (the two
+        pushes share a launch) once the caches exist."""
+        fused = (self.k.handle is not None and self.v.handle is not None and k_new.shape == v_new.shape
+                 and k_new.dtype == v_new.dtype == q.dtype and len(q.shape) == len(k_new.shape)
+                 and q.shape[self.axis] == k_new.shape[self.axis])
+        if not fused:
+            self.k.push(k_new, stream=stream)
+            self.v.push(v_new, stream=stream)
+            return self.attend(q, stream, out)
+        self.k._check_push_shape(k_new.shape)
+        B, Hq, Sq, D = _canon4(q.shape)
+        if out is None:
+            out = DeviceTensor(q.shape, q.dtype)
+        if self._ws is None or self._ws_key != (B, Hq, D):
+            self._ws, self._ws_key = Workspace(B, Hq, Sq, D, stream), (B, Hq, D)
+        call("trocm_inplace_kv_sdpa_eval", q.ptr, k_new.ptr, v_new.ptr, dtype_code(q.dtype), Hq, Sq, None,
+             self.k.handle, self.v.handle, out.ptr, _scale_arg(self.scale), int(self.causal),
+             self._ws.ptr, self._ws.nbytes, _sh(stream))
+        return out
 
     def attend(self, q: DeviceTensor, stream=None, out: DeviceTensor | None = None) -> DeviceTensor:
         B, Hq, Sq, D = _canon4(q.shape)

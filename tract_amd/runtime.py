@@ -77,6 +77,32 @@ class Stream:
             pass
 
 
+class Event:
+    """A HIP event; `Event.elapsed_ms(a, b)` waits for b."""
+
+    def __init__(self):
+        h = C.c_void_p()
+        call("trocm_event_create", C.byref(h))
+        self.handle = h
+
+    def record(self, stream=None):
+        call("trocm_event_record", self.handle, _sh(stream))
+
+    @staticmethod
+    def elapsed_ms(start: "Event", stop: "Event") -> float:
+        ms = C.c_float()
+        call("trocm_event_elapsed_ms", start.handle, stop.handle, C.byref(ms))
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self.handle:
+                _lib.load().trocm_event_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
 def _sh(stream):
     return stream.handle if isinstance(stream, Stream) else stream
 
