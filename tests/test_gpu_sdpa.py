@@ -174,3 +174,55 @@ def test_ragged_decode_small(rt):
     for i in range(len(lens)):
         want = orc.flash_sdpa(q[i:i + 1], ks[i], vs[i], causal=True)
         assert max_abs(out[i:i + 1], want) <= 2e-2
+
+
+@pytest.mark.parametrize("fmt_name", ["Q8_0", "Q4_0"])
+@pytest.mark.parametrize("B,Hq,Hkv,T", [(1, 32, 8, 1), (2, 32, 8, 100), (2, 32, 8, 1025), (1, 8, 8, 333), (1, 16, 2, 64),
+                                         (1, 24, 8, 77)])
+def test_decode_quantised_cache(rt, fmt_name, B, Hq, Hkv, T):
+    """cfg4 (reduced): K/V quantised on append, 1% outlier channels x20, decode with fused
+    dequantisation.  Oracle: FlashSdpaOp over the dequantised blocks (f16 dequant like
+    BlockQuant::dequant_f16, then the f16 eval path)."""
+    D = 128
+    dev_fmt = getattr(tract_amd, fmt_name)
+    orc_fmt = getattr(orc, "FMT_" + fmt_name)
+    rng = np.random.default_rng(cases.cfg_seed(4, "chan") + T)
+    chan = rng.choice(Hkv * D, size=max(1, Hkv * D // 100), replace=False)
+
+    def outliers(x):
+        xf = x.transpose(0, 2, 1, 3).reshape(B, -1, Hkv * D).astype(np.float32)
+        xf[:, :, chan] *= 20
+        return xf.reshape(B, -1, Hkv, D).transpose(0, 2, 1, 3).astype(np.float16)
+
+    k = outliers(cases.seeded_normal(cases.cfg_seed(4, "k") + T, (B, Hkv, T, D)))
+    v = outliers(cases.seeded_normal(cases.cfg_seed(4, "v") + T, (B, Hkv, T, D)))
+    q = (cases.seeded_normal(cases.cfg_seed(4, "q") + T, (B, Hq, 1, D)) / np.sqrt(D)).astype(np.float16)
+    st = tract_amd.InPlaceKvSdpa(axis=2, causal=True, storage_format=dev_fmt).state()
+    st.k.reserve(T + 19, like=(k.shape, k.dtype))
+    st.v.reserve(T + 19, like=(v.shape, v.dtype))
+    out = st.eval([q, k, v]).to_numpy()
+    kq, vq = orc.quant(orc_fmt, k), orc.quant(orc_fmt, v)
+    assert st.k.valid_contiguous().tobytes() == kq.tobytes() and st.v.valid_contiguous().tobytes() == vq.tobytes()
+    kd, vd = orc.dequant(orc_fmt, kq, np.float16), orc.dequant(orc_fmt, vq, np.float16)
+    want = orc.flash_sdpa(q, kd, vd, causal=True)
+    assert not np.isnan(out).any()
+    assert max_abs(out, want) <= 2e-2
+    # attributable: against f32 dequantisation in f64 the fused kernel is much closer
+    exact = cases.textbook_sdpa(q, orc.dequant(orc_fmt, kq, np.float32), orc.dequant(orc_fmt, vq, np.float32))
+    # (the output is f16: allow its rounding, half an ulp relative, on the outlier-channel magnitudes)
+    assert np.allclose(out.astype(np.float64), exact, rtol=1.5e-3, atol=2e-3)
+
+
+def test_quantised_cache_with_f32_queries_uses_generic_kernel(rt):
+    rng = np.random.default_rng(31)
+    B, Hq, Hkv, T, D = 1, 4, 2, 50, 64
+    k = rng.standard_normal((B, Hkv, T, D), dtype=np.float32)
+    v = rng.standard_normal((B, Hkv, T, D), dtype=np.float32)
+    q = rng.standard_normal((B, Hq, 3, D), dtype=np.float32) / 8
+    for dev_fmt, orc_fmt in ((tract_amd.Q8_0, orc.FMT_Q8_0), (tract_amd.Q4_0, orc.FMT_Q4_0)):
+        st = tract_amd.InPlaceKvSdpa(axis=2, causal=False, storage_format=dev_fmt).state()
+        st.k.push(k), st.v.push(v)
+        out = st.attend(tract_amd.DeviceTensor.from_numpy(q)).to_numpy()
+        kd = orc.dequant(orc_fmt, orc.quant(orc_fmt, k))
+        vd = orc.dequant(orc_fmt, orc.quant(orc_fmt, v))
+        assert max_abs(out, orc.flash_sdpa(q, kd, vd)) <= 1e-3

@@ -25,7 +25,8 @@ COMMON = [
 ]
 # per-file extra flags: the quantiser must not contract a*b+c into an fma
 EXTRA = {"kv_quant.hip": ["-ffp-contract=off"]}
-SOURCES = ["abi.hip", "copy.hip", "kv_quant.hip", "sdpa_generic.hip", "sdpa_decode.hip", "sdpa_prefill.hip"]
+SOURCES = ["abi.hip", "copy.hip", "kv_quant.hip", "sdpa_generic.hip", "sdpa_decode.hip", "sdpa_decode_quant.hip",
+           "sdpa_prefill.hip"]
 
 
 def _newer(target: str, deps: list[str]) -> bool:
@@ -46,7 +47,7 @@ def _run(cmd: list[str]) -> None:
 
 def build(force: bool = False, verbose: bool = True) -> str:
     os.makedirs(OBJ, exist_ok=True)
-    headers = [os.path.join(CSRC, "common.h"), os.path.join(HERE, "..", "include", "tract_rocm.h"), __file__]
+    headers = [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "decode_common.h"), os.path.join(HERE, "..", "include", "tract_rocm.h"), __file__]
     jobs = []
     objs = []
     for src in SOURCES:

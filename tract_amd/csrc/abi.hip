@@ -558,7 +558,7 @@ int trocm_sdpa_workspace_init(void *workspace, size_t bytes, void *stream) {
 static int dispatch_sdpa(const SdpaArgs &a, hipStream_t s) {
     if (a.B == 0 || a.Hq == 0 || a.Sq == 0 || a.D == 0) return 0;
     int rc = 2;
-    if (a.Sq == 1) rc = launch_sdpa_decode(a, s);
+    if (a.Sq == 1) rc = is_quant(a.kv_fmt) ? launch_sdpa_decode_quant(a, s) : launch_sdpa_decode(a, s);
     if (rc == 2) rc = launch_sdpa_prefill(a, s);
     if (rc == 2) rc = launch_sdpa_generic(a, s);
     return rc;

@@ -1,0 +1,150 @@
+// Pieces shared by the split-K decode kernels (plain and quantised KV): launch geometry,
+// kernel parameters, DPP wave reductions and the split-merge kernel.
+#pragma once
+#include <hip/hip_fp16.h>
+#include <string.h>
+#include <stdlib.h>
+#include "common.h"
+
+namespace trocm {
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+constexpr int kTile = 32;
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+struct DecodeDev {
+    const char *q;
+    char *out;
+    const char *k, *v;
+    int64_t kv_stride_b, kv_stride_h, kv_stride_t;  // bytes
+    int T;                                          // valid tokens
+    int tiles_per_split, nsplit;
+    int Hq, Hkv;
+    float scale_log2;
+    float *part_o;   // [B*Hkv*nsplit][G*D]
+    float *part_ml;  // [B*Hkv*nsplit][2*G]
+    // quantised KV only: f16 scale planes, [B, Hkv, cap, D/32]
+    const char *k_scales, *v_scales;
+    int64_t sc_stride_b, sc_stride_h;  // bytes
+};
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float readlane_f(float x, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
+}
+// DPP controls: row_ror:n rotates within a row of 16 lanes; quad_perm[1,0,3,2] swaps neighbours.
+constexpr int kRowRor1 = 0x121, kRowRor2 = 0x122, kRowRor4 = 0x124, kRowRor8 = 0x128, kSwapPairs = 0xB1;
+
+__device__ __forceinline__ float wave_max(float x) {
+    x = fmaxf(x, dpp_f<kRowRor8>(x));
+    x = fmaxf(x, dpp_f<kRowRor4>(x));
+    x = fmaxf(x, dpp_f<kRowRor2>(x));
+    x = fmaxf(x, dpp_f<kRowRor1>(x));
+    return fmaxf(fmaxf(readlane_f(x, 0), readlane_f(x, 16)), fmaxf(readlane_f(x, 32), readlane_f(x, 48)));
+}
+__device__ __forceinline__ float wave_sum(float x) {
+    x += dpp_f<kRowRor8>(x);
+    x += dpp_f<kRowRor4>(x);
+    x += dpp_f<kRowRor2>(x);
+    x += dpp_f<kRowRor1>(x);
+    return (readlane_f(x, 0) + readlane_f(x, 16)) + (readlane_f(x, 32) + readlane_f(x, 48));
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// 16 bytes of K against 16 bytes of Q: 8 f16 products or 4 f32 products, f32 accumulate.
+// Vector elements are copied into scalars before any bit cast.
+__device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+
+template <typename T>
+__device__ __forceinline__ float dot16(u32x4 k, u32x4 q, float acc);
+template <>
+__device__ __forceinline__ float dot16<__half>(u32x4 k, u32x4 q, float acc) {
+    uint32_t k0 = k.x, k1 = k.y, k2 = k.z, k3 = k.w;
+    uint32_t q0 = q.x, q1 = q.y, q2 = q.z, q3 = q.w;
+    acc = __builtin_amdgcn_fdot2(as_half2(k0), as_half2(q0), acc, false);
+    acc = __builtin_amdgcn_fdot2(as_half2(k1), as_half2(q1), acc, false);
+    acc = __builtin_amdgcn_fdot2(as_half2(k2), as_half2(q2), acc, false);
+    acc = __builtin_amdgcn_fdot2(as_half2(k3), as_half2(q3), acc, false);
+    return acc;
+}
+template <>
+__device__ __forceinline__ float dot16<float>(u32x4 k, u32x4 q, float acc) {
+    uint32_t k0 = k.x, k1 = k.y, k2 = k.z, k3 = k.w;
+    uint32_t q0 = q.x, q1 = q.y, q2 = q.z, q3 = q.w;
+    acc = fmaf(as_f32(k0), as_f32(q0), acc);
+    acc = fmaf(as_f32(k1), as_f32(q1), acc);
+    acc = fmaf(as_f32(k2), as_f32(q2), acc);
+    acc = fmaf(as_f32(k3), as_f32(q3), acc);
+    return acc;
+}
+
+// The slice of a V row owned by one lane in the PV phase: EPL = D/16 elements.
+template <typename T, int EPL>
+struct VSlice;
+template <>
+struct VSlice<__half, 8> { typedef half8_t type; };
+template <>
+struct VSlice<__half, 4> { typedef half4_t type; };
+template <>
+struct VSlice<float, 8> { typedef float8_t type; };
+template <>
+struct VSlice<float, 4> { typedef float4_t type; };
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float x);
+template <>
+__device__ __forceinline__ __half from_f32<__half>(float x) { return __float2half_rn(x); }
+template <>
+__device__ __forceinline__ float from_f32<float>(float x) { return x; }
+
+// Merge the per-split partials (O, m, l) of one (batch, kv head) and write the output rows.
+template <typename T, int D, int G>
+__device__ __forceinline__ void merge_splits(const DecodeDev &p, int64_t bh, T *out, int tid) {
+    for (int idx = tid; idx < G * D; idx += kThreads) {
+        const int h = idx / D;
+        const float *ml = p.part_ml + bh * p.nsplit * (2 * G);
+        const float *po = p.part_o + bh * p.nsplit * (G * D) + idx;
+        auto ld = [&](const float *a) { return *a; };
+        float mm = -INFINITY;
+#pragma unroll 4
+        for (int sp = 0; sp < p.nsplit; sp++) mm = fmaxf(mm, ld(ml + sp * (2 * G) + h));
+        float acc = 0.0f, ll = 0.0f;
+#pragma unroll 4
+        for (int sp = 0; sp < p.nsplit; sp++) {
+            float f = fast_exp2(ld(ml + sp * (2 * G) + h) - mm);
+            acc += ld(po + (int64_t)sp * (G * D)) * f;
+            ll += ld(ml + sp * (2 * G) + G + h) * f;
+        }
+        out[idx] = from_f32<T>(acc / ll);
+    }
+}
+
+// Merge launch: grid (kv_heads, batch), runs after the split kernel on the same stream.
+template <typename T, int D, int G>
+__global__ __launch_bounds__(kThreads) void sdpa_decode_merge_kernel(DecodeDev p) {
+    const int kvh = blockIdx.x, b = blockIdx.y;
+    const int64_t bh = (int64_t)b * p.Hkv + kvh;
+    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)b * p.Hq + (int64_t)kvh * G) * D;
+    merge_splits<T, D, G>(p, bh, out, threadIdx.x);
+}
+
+}  // namespace
+
+// Partials: at most kMaxSplitRows rows of (D + 2) floats per query head.
+constexpr int64_t kMaxSplitRows = 8192;
+int choose_decode_splits(int64_t BH, int64_t G, int n_tiles);
+
+}  // namespace trocm

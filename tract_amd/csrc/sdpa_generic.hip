@@ -16,6 +16,8 @@ namespace {
 
 struct GenericDev {
     const void *q, *k, *v, *mask;
+    const void *k_scales, *v_scales;  // quantised K/V: f16 scale planes
+    int kv_fmt;
     void *out;
     int64_t B, Hq, Hkv, Sq, Sk, D;
     int64_t kv_stride_b, kv_stride_h, kv_stride_t;  // elements
@@ -28,6 +30,49 @@ __device__ __forceinline__ float ld(const float *p) { return *p; }
 __device__ __forceinline__ float ld(const __half *p) { return __half2float(*p); }
 __device__ __forceinline__ void st(float *p, float x) { *p = x; }
 __device__ __forceinline__ void st(__half *p, float x) { *p = __float2half_rn(x); }
+
+// Element (token j, column d) of a K or V plane of one (batch, kv head).  Plain formats: a row
+// of T; quantised formats: code and block scale, dequantised as code * d in f32
+// (linalg/src/frame/block_quant/q4_0.rs:82-95, q8_1.rs:50-63).
+template <typename T>
+struct KvReader {
+    const T *rows;
+    const uint8_t *codes;
+    const uint16_t *scales;
+    int64_t stride_t;  // elements between token rows (plain) -- quantised rows are dense
+    int fmt, D;
+    __device__ __forceinline__ float at(int64_t j, int d) const {
+        if (fmt == TROCM_Q8_0) {
+            float sc = __half2float(__ushort_as_half(scales[j * (D / 32) + d / 32]));
+            return (float)(int8_t)codes[j * D + d] * sc;
+        }
+        if (fmt == TROCM_Q4_0) {
+            float sc = __half2float(__ushort_as_half(scales[j * (D / 32) + d / 32]));
+            int e = d & 31;
+            uint8_t byte = codes[j * (D / 2) + (d / 32) * 16 + (e & 15)];
+            int nib = e < 16 ? (byte & 15) : (byte >> 4);
+            return (float)(nib - 8) * sc;
+        }
+        return ld(rows + j * stride_t + d);
+    }
+};
+
+template <typename T>
+__device__ __forceinline__ KvReader<T> make_reader(const GenericDev &p, const void *plane, const void *scales, int64_t b,
+                                                   int64_t kvh) {
+    KvReader<T> r;
+    r.fmt = p.kv_fmt, r.D = (int)p.D, r.stride_t = p.kv_stride_t;
+    r.rows = nullptr, r.codes = nullptr, r.scales = nullptr;
+    if (p.kv_fmt == TROCM_Q8_0 || p.kv_fmt == TROCM_Q4_0) {
+        int64_t row0 = (b * p.kv_stride_b + kvh * p.kv_stride_h) / p.D;  // first token row of this (batch, head)
+        int64_t rb = p.kv_fmt == TROCM_Q8_0 ? p.D : p.D / 2;
+        r.codes = (const uint8_t *)plane + row0 * rb;
+        r.scales = (const uint16_t *)scales + row0 * (p.D / 32);
+    } else {
+        r.rows = (const T *)plane + b * p.kv_stride_b + kvh * p.kv_stride_h;
+    }
+    return r;
+}
 
 template <typename T>
 __global__ __launch_bounds__(64) void sdpa_generic_kernel(GenericDev p) {
@@ -44,8 +89,8 @@ __global__ __launch_bounds__(64) void sdpa_generic_kernel(GenericDev p) {
     const int D = (int)p.D;
 
     const T *q = (const T *)p.q + ((b * p.Hq + qh) * p.Sq + i) * p.D;
-    const T *k = (const T *)p.k + b * p.kv_stride_b + kvh * p.kv_stride_h;
-    const T *v = (const T *)p.v + b * p.kv_stride_b + kvh * p.kv_stride_h;
+    const KvReader<T> k = make_reader<T>(p, p.k, p.k_scales, b, kvh);
+    const KvReader<T> v = make_reader<T>(p, p.v, p.v_scales, b, kvh);
     T *out = (T *)p.out + ((b * p.Hq + qh) * p.Sq + i) * p.D;
     const T *mask = nullptr;
     if (p.mask) {
@@ -63,9 +108,8 @@ __global__ __launch_bounds__(64) void sdpa_generic_kernel(GenericDev p) {
         n_vis = lim < 0 ? 0 : (lim < p.Sk ? lim : p.Sk);
     }
     auto score = [&](int64_t j) {
-        const T *kr = k + j * p.kv_stride_t;
         float acc = 0.0f;
-        for (int d = 0; d < D; d++) acc = fmaf(lds_q[d], ld(kr + d), acc);
+        for (int d = 0; d < D; d++) acc = fmaf(lds_q[d], k.at(j, d), acc);
         acc *= p.scale;
         if (mask) acc += ld(mask + j);
         return acc;
@@ -90,11 +134,10 @@ __global__ __launch_bounds__(64) void sdpa_generic_kernel(GenericDev p) {
             int64_t n = n_vis - j0 < 64 ? n_vis - j0 : 64;
             for (int64_t jj = 0; jj < n; jj++) {
                 float pp = lds_p[jj];
-                const T *vr = v + (j0 + jj) * p.kv_stride_t;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     int d = lane + 64 * e;
-                    if (d < D) o[e] = fmaf(pp, ld(vr + d), o[e]);
+                    if (d < D) o[e] = fmaf(pp, v.at(j0 + jj, d), o[e]);
                 }
             }
         }
@@ -111,14 +154,16 @@ __global__ __launch_bounds__(64) void sdpa_generic_kernel(GenericDev p) {
 }  // namespace
 
 int launch_sdpa_generic(const SdpaArgs &a, hipStream_t s) {
-    TROCM_REQUIRE(a.kv_fmt == TROCM_F32 || a.kv_fmt == TROCM_F16, "generic sdpa: quantised K/V not supported");
-    TROCM_REQUIRE(a.q_dtype == a.kv_fmt, "generic sdpa: Q and K/V must share a dtype");
+    const bool quant = a.kv_fmt == TROCM_Q8_0 || a.kv_fmt == TROCM_Q4_0;
+    TROCM_REQUIRE(quant || a.q_dtype == a.kv_fmt, "generic sdpa: Q and K/V must share a dtype");
+    TROCM_REQUIRE(!quant || (a.D % 32 == 0 && a.kv_stride_t == a.D), "generic sdpa: quantised K/V needs dense rows and head_dim %% 32 == 0");
     TROCM_REQUIRE(a.D >= 1 && a.D <= 512, "generic sdpa: head_dim %lld not in 1..512", (long long)a.D);
     int64_t rows = a.B * a.Hq * a.Sq;
     if (rows == 0) return 0;
     TROCM_REQUIRE(rows < (1ll << 31), "generic sdpa: too many query rows");
     GenericDev p;
     p.q = a.q, p.k = a.k, p.v = a.v, p.mask = a.mask, p.out = a.out;
+    p.k_scales = a.k_scales, p.v_scales = a.v_scales, p.kv_fmt = a.kv_fmt;
     p.B = a.B, p.Hq = a.Hq, p.Hkv = a.Hkv, p.Sq = a.Sq, p.Sk = a.Sk, p.D = a.D;
     p.kv_stride_b = a.kv_stride_b, p.kv_stride_h = a.kv_stride_h, p.kv_stride_t = a.kv_stride_t;
     p.mask_b = a.mask_b, p.mask_h = a.mask_h;
