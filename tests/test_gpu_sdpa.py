@@ -226,3 +226,62 @@ def test_quantised_cache_with_f32_queries_uses_generic_kernel(rt):
         kd = orc.dequant(orc_fmt, orc.quant(orc_fmt, k))
         vd = orc.dequant(orc_fmt, orc.quant(orc_fmt, v))
         assert max_abs(out, orc.flash_sdpa(q, kd, vd)) <= 1e-3
+
+
+@pytest.mark.parametrize("dt,Hq,Hkv,D,n_seq,lo,hi", [
+    (np.float16, 32, 8, 128, 24, 1, 3000), (np.float32, 8, 8, 64, 7, 30, 900), (np.float16, 16, 2, 64, 40, 1, 400),
+    (np.float16, 6, 2, 128, 5, 10, 300),   # group size 3: per-sequence fall-back
+])
+def test_ragged_decode_many_sequences(rt, dt, Hq, Hkv, D, n_seq, lo, hi):
+    """cfg5 (reduced): independent sequences with their own capacity-doubling caches and
+    lengths; every sequence must equal the batch-1 oracle.  Two decode steps with an append
+    in between, so lengths (and the work plan) change from call to call."""
+    rng = np.random.default_rng(cases.cfg_seed(5, "len"))
+    lens = rng.integers(lo, hi, size=n_seq, endpoint=True)
+    kcs, vcs, ks, vs = [], [], [], []
+    for n in lens:
+        k = rng.standard_normal((1, Hkv, int(n), D), dtype=np.float32).astype(dt)
+        v = rng.standard_normal((1, Hkv, int(n), D), dtype=np.float32).astype(dt)
+        kc, vc = tract_amd.InPlaceKvCache(2), tract_amd.InPlaceKvCache(2)
+        kc.push(k), vc.push(v)
+        kcs.append(kc), vcs.append(vc), ks.append(k), vs.append(v)
+    ws = tract_amd.Workspace(n_seq, Hq, 1, D)
+    for step in range(2):
+        q = (rng.standard_normal((n_seq, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(dt)
+        out = tract_amd.sdpa_decode_ragged(tract_amd.DeviceTensor.from_numpy(q), kcs, vcs, workspace=ws).to_numpy()
+        assert not np.isnan(out).any()
+        for i in range(n_seq):
+            want = orc.flash_sdpa(q[i:i + 1], ks[i], vs[i], causal=True)
+            assert max_abs(out[i:i + 1], want) <= TOL[np.dtype(dt)], f"sequence {i} len {ks[i].shape[2]}"
+        for i in range(n_seq):  # append one token to every sequence
+            kn = rng.standard_normal((1, Hkv, 1, D), dtype=np.float32).astype(dt)
+            vn = rng.standard_normal((1, Hkv, 1, D), dtype=np.float32).astype(dt)
+            kcs[i].push(kn), vcs[i].push(vn)
+            ks[i], vs[i] = np.concatenate([ks[i], kn], axis=2), np.concatenate([vs[i], vn], axis=2)
+
+
+def test_ragged_equals_padded_batch_with_mask(rt):
+    """The reference's statement of a ragged batch: a dense batch padded to the longest
+    sequence with an additive mask whose padded columns are <= -65504 (flash_sdpa.rs:261-268)."""
+    rng = np.random.default_rng(77)
+    Hq, Hkv, D = 8, 2, 64
+    lens = [5, 64, 33, 100]
+    Tmax = max(lens)
+    kp = np.zeros((len(lens), Hkv, Tmax, D), np.float32)
+    vp = np.zeros((len(lens), Hkv, Tmax, D), np.float32)
+    mask = np.zeros((len(lens), 1, 1, Tmax), np.float32)
+    kcs, vcs = [], []
+    for i, n in enumerate(lens):
+        k = rng.standard_normal((1, Hkv, n, D), dtype=np.float32)
+        v = rng.standard_normal((1, Hkv, n, D), dtype=np.float32)
+        kp[i, :, :n], vp[i, :, :n] = k[0], v[0]
+        mask[i, :, :, n:] = -65504.0
+        kc, vc = tract_amd.InPlaceKvCache(2), tract_amd.InPlaceKvCache(2)
+        kc.push(k), vc.push(v)
+        kcs.append(kc), vcs.append(vc)
+    q = rng.standard_normal((len(lens), Hq, 1, D), dtype=np.float32) / 8
+    got = tract_amd.sdpa_decode_ragged(tract_amd.DeviceTensor.from_numpy(q), kcs, vcs).to_numpy()
+    want = orc.flash_sdpa(q, kp, vp, mask=mask)
+    assert max_abs(got, want) <= 1e-3
+    dense = tract_amd.Sdpa().eval(q, kp, vp, mask).to_numpy()
+    assert max_abs(got, dense) <= 1e-5

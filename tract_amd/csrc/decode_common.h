@@ -36,6 +36,17 @@ struct DecodeDev {
     int64_t sc_stride_b, sc_stride_h;  // bytes
 };
 
+// Ragged batches: one work item = a tile range of one sequence (device copies of the host plan).
+struct RaggedItem {
+    const char *k, *v;   // planes of the sequence (kv head 0)
+    int64_t stride_h;    // bytes between kv heads
+    int T, tile_begin, tile_end;
+    int seq, split, nsplit, slot0;
+};
+struct RaggedSeqSlots {
+    int slot0, nsplit;
+};
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_f(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
@@ -111,22 +122,25 @@ template <>
 __device__ __forceinline__ float from_f32<float>(float x) { return x; }
 
 // Merge the per-split partials (O, m, l) of one (batch, kv head) and write the output rows.
+// Partial records `first`, `first + stride`, ... (`nsplit` of them).
 template <typename T, int D, int G>
-__device__ __forceinline__ void merge_splits(const DecodeDev &p, int64_t bh, T *out, int tid) {
+__device__ __forceinline__ void merge_splits(const DecodeDev &p, int64_t first, int64_t stride, int nsplit, T *out,
+                                             int tid) {
     for (int idx = tid; idx < G * D; idx += kThreads) {
         const int h = idx / D;
-        const float *ml = p.part_ml + bh * p.nsplit * (2 * G);
-        const float *po = p.part_o + bh * p.nsplit * (G * D) + idx;
+        const float *ml = p.part_ml + first * (2 * G);
+        const float *po = p.part_o + first * (G * D) + idx;
+        const int64_t ml_step = stride * (2 * G), po_step = stride * (G * D);
         auto ld = [&](const float *a) { return *a; };
         float mm = -INFINITY;
 #pragma unroll 4
-        for (int sp = 0; sp < p.nsplit; sp++) mm = fmaxf(mm, ld(ml + sp * (2 * G) + h));
+        for (int sp = 0; sp < nsplit; sp++) mm = fmaxf(mm, ld(ml + sp * ml_step + h));
         float acc = 0.0f, ll = 0.0f;
 #pragma unroll 4
-        for (int sp = 0; sp < p.nsplit; sp++) {
-            float f = fast_exp2(ld(ml + sp * (2 * G) + h) - mm);
-            acc += ld(po + (int64_t)sp * (G * D)) * f;
-            ll += ld(ml + sp * (2 * G) + G + h) * f;
+        for (int sp = 0; sp < nsplit; sp++) {
+            float f = fast_exp2(ld(ml + sp * ml_step + h) - mm);
+            acc += ld(po + sp * po_step) * f;
+            ll += ld(ml + sp * ml_step + G + h) * f;
         }
         out[idx] = from_f32<T>(acc / ll);
     }
@@ -138,7 +152,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_decode_merge_kernel(DecodeDev p
     const int kvh = blockIdx.x, b = blockIdx.y;
     const int64_t bh = (int64_t)b * p.Hkv + kvh;
     T *out = reinterpret_cast<T *>(p.out) + ((int64_t)b * p.Hq + (int64_t)kvh * G) * D;
-    merge_splits<T, D, G>(p, bh, out, threadIdx.x);
+    merge_splits<T, D, G>(p, bh * p.nsplit, 1, p.nsplit, out, threadIdx.x);
 }
 
 }  // namespace

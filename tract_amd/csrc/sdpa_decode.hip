@@ -41,8 +41,19 @@ __device__ __forceinline__ int rot(int row) {
     return CPR == 8 ? (row >> 1) : row;
 }
 
+// What one workgroup has to do: a tile range of one (sequence, kv head), and where its result goes.
+struct DecodeWork {
+    const char *q;      // the G query rows of this kv head
+    char *out;          // the G output rows
+    const char *kbase, *vbase;
+    int T;              // valid tokens of the sequence
+    int tile_begin, tile_end;
+    bool direct;        // single split: write the output rows; else store partials at `part`
+    int64_t part;       // index of the partial record
+};
+
 template <typename T, int D, int G>
-__global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1) void sdpa_decode_kernel(DecodeDev p) {
+__device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork &wk) {
     constexpr int RB = D * sizeof(T);   // bytes of one K/V row: 128, 256 or 512
     constexpr int CPR = RB / 16;        // 16-byte chunks per row: 8, 16, 32
     constexpr int HC = CPR / 2;         // chunks per half row (one QK lane)
@@ -59,21 +70,18 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int w = tid >> 6;
-    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
 
     // ---- stage the G query vectors of this KV head ------------------------------------
     {
-        const u32x4 *qg = reinterpret_cast<const u32x4 *>(p.q + ((int64_t)b * p.Hq + (int64_t)kvh * G) * RB);
+        const u32x4 *qg = reinterpret_cast<const u32x4 *>(wk.q);
         for (int i = tid; i < G * CPR; i += kThreads) lds_q[i] = qg[i];
     }
     __syncthreads();
 
-    const char *kbase = p.k + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
-    const char *vbase = p.v + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
-    const int n_tiles = (p.T + kTile - 1) / kTile;
-    const int tile_begin = split * p.tiles_per_split;
-    const int tile_end = min(n_tiles, tile_begin + p.tiles_per_split);
-    const int last_tok = p.T - 1;
+    const char *kbase = wk.kbase, *vbase = wk.vbase;
+    const int seq_T = wk.T;
+    const int tile_begin = wk.tile_begin, tile_end = wk.tile_end;
+    const int last_tok = seq_T - 1;
 
     float m[G], l[G], o[G][EPL];
 #pragma unroll
@@ -108,7 +116,7 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     auto issue_k = [&](int tile) {
         const int t0 = tile * kTile;
         const char *base = kbase + (int64_t)t0 * p.kv_stride_t;
-        if (t0 + kTile <= p.T) {
+        if (t0 + kTile <= seq_T) {
 #pragma unroll
             for (int j = 0; j < KL; j++) kreg[j] = *reinterpret_cast<const u32x4 *>(base + k_off[j]);
         } else {
@@ -123,7 +131,7 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     auto issue_v = [&](int tile) {
         const int t0 = tile * kTile;
         const char *base = vbase + (int64_t)t0 * p.kv_stride_t;
-        if (t0 + kTile <= p.T) {
+        if (t0 + kTile <= seq_T) {
 #pragma unroll
             for (int i = 0; i < VI; i++) vreg[i] = *reinterpret_cast<const vslice_t *>(base + v_off[i]);
         } else {
@@ -162,7 +170,7 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
 #pragma unroll
             for (int h = 0; h < G; h++) s[h] = dot16<T>(kc, lds_q[h * CPR + qk_half * HC + cc], s[h]);
         }
-        const bool valid = (t0 + qk_row) < p.T;
+        const bool valid = (t0 + qk_row) < seq_T;
         // 3. online softmax (wave-uniform running maximum per head)
         float pr[G];
 #pragma unroll
@@ -240,8 +248,7 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     }
     __syncthreads();
 
-    const int64_t bh = (int64_t)b * p.Hkv + kvh;
-    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)b * p.Hq + (int64_t)kvh * G) * D;
+    T *out = reinterpret_cast<T *>(wk.out);
     for (int idx = tid; idx < G * D; idx += kThreads) {
         int h = idx / D;
         float mm = -INFINITY;
@@ -254,10 +261,10 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
             acc += comb[ww * kCombStride + idx] * f;
             ll += comb[ww * kCombStride + G * D + G + h] * f;
         }
-        if (p.nsplit == 1) {
+        if (wk.direct) {
             out[idx] = from_f32<T>(acc / ll);
         } else {
-            int64_t slot = bh * p.nsplit + split;
+            int64_t slot = wk.part;
             p.part_o[slot * (G * D) + idx] = acc;
             if ((idx % D) == 0) {
                 p.part_ml[slot * (2 * G) + h] = mm;
@@ -265,6 +272,58 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
             }
         }
     }
+}
+
+// Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.
+template <typename T, int D, int G>
+__global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1) void sdpa_decode_kernel(DecodeDev p) {
+    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    DecodeWork wk;
+    const int64_t row = ((int64_t)b * p.Hq + (int64_t)kvh * G) * D * (int64_t)sizeof(T);
+    wk.q = p.q + row;
+    wk.out = p.out + row;
+    wk.kbase = p.k + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+    wk.vbase = p.v + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+    wk.T = p.T;
+    const int n_tiles = (p.T + kTile - 1) / kTile;
+    wk.tile_begin = split * p.tiles_per_split;
+    wk.tile_end = min(n_tiles, wk.tile_begin + p.tiles_per_split);
+    wk.direct = p.nsplit == 1;
+    wk.part = ((int64_t)b * p.Hkv + kvh) * p.nsplit + split;
+    decode_body<T, D, G>(p, wk);
+}
+
+// Ragged batch: grid (work items, kv_heads).  An item is a tile range of one sequence; the
+// host cuts every sequence into ranges of about the same number of tiles, so that 64
+// sequences whose lengths differ 64-fold still load all compute units evenly.
+template <typename T, int D, int G>
+__global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1) void sdpa_decode_ragged_kernel(
+    DecodeDev p, const RaggedItem *__restrict__ items) {
+    const RaggedItem it = items[blockIdx.x];
+    const int kvh = blockIdx.y;
+    DecodeWork wk;
+    const int64_t row = ((int64_t)it.seq * p.Hq + (int64_t)kvh * G) * D * (int64_t)sizeof(T);
+    wk.q = p.q + row;
+    wk.out = p.out + row;
+    wk.kbase = it.k + (int64_t)kvh * it.stride_h;
+    wk.vbase = it.v + (int64_t)kvh * it.stride_h;
+    wk.T = it.T;
+    wk.tile_begin = it.tile_begin;
+    wk.tile_end = it.tile_end;
+    wk.direct = it.nsplit == 1;
+    wk.part = ((int64_t)it.slot0 + it.split) * p.Hkv + kvh;
+    decode_body<T, D, G>(p, wk);
+}
+
+// Merge launch of the ragged batch: grid (kv_heads, sequences).
+template <typename T, int D, int G>
+__global__ __launch_bounds__(kThreads) void sdpa_decode_ragged_merge_kernel(DecodeDev p,
+                                                                             const RaggedSeqSlots *__restrict__ seqs) {
+    const int kvh = blockIdx.x, seq = blockIdx.y;
+    const RaggedSeqSlots ss = seqs[seq];
+    if (ss.nsplit <= 1) return;
+    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)seq * p.Hq + (int64_t)kvh * G) * D;
+    merge_splits<T, D, G>(p, (int64_t)ss.slot0 * p.Hkv + kvh, p.Hkv, ss.nsplit, out, threadIdx.x);
 }
 
 template <typename T, int D, int G>
@@ -368,11 +427,62 @@ int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
 }  // namespace trocm
 
 namespace trocm {
-// Ragged decode, first form: one split-K launch per sequence on the caller's stream
-// (launches on one stream are ordered, so the sequences can share the workspace).
-int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt, int64_t n_seq, int64_t Hq, int64_t Hkv,
-                              int64_t D, const RaggedSeq *seqs, float scale, void *workspace, size_t workspace_bytes,
-                              hipStream_t s) {
+namespace {
+
+// Pinned staging for the per-call plan of a ragged launch (a few KiB): a small ring per host
+// thread, each slot guarded by an event so that a slot is not rewritten while its copy is
+// still in flight.
+constexpr int kStageSlots = 4;
+struct StageSlot {
+    void *host = nullptr;
+    hipEvent_t done = nullptr;
+    bool in_flight = false;
+};
+thread_local StageSlot g_stage[kStageSlots];
+thread_local int g_stage_next = 0;
+
+int acquire_stage(StageSlot **out) {
+    StageSlot &sl = g_stage[g_stage_next];
+    g_stage_next = (g_stage_next + 1) % kStageSlots;
+    if (!sl.host) {
+        TROCM_HIP(hipHostMalloc(&sl.host, kWsCounterBytes, hipHostMallocDefault));
+        TROCM_HIP(hipEventCreateWithFlags(&sl.done, hipEventDisableTiming));
+    } else if (sl.in_flight) {
+        TROCM_HIP(hipEventSynchronize(sl.done));
+    }
+    sl.in_flight = false;
+    *out = &sl;
+    return 0;
+}
+
+template <typename T, int D, int G>
+void launch_ragged(const DecodeDev &p, const RaggedItem *items, int n_items, const RaggedSeqSlots *seqs, int n_seq,
+                   bool any_split, hipStream_t s) {
+    hipLaunchKernelGGL((sdpa_decode_ragged_kernel<T, D, G>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+    if (any_split)
+        hipLaunchKernelGGL((sdpa_decode_ragged_merge_kernel<T, D, G>), dim3(p.Hkv, n_seq), dim3(kThreads), 0, s, p, seqs);
+}
+
+template <typename T, int D>
+int launch_ragged_g(const DecodeDev &p, int G, const RaggedItem *items, int n_items, const RaggedSeqSlots *seqs,
+                    int n_seq, bool any_split, hipStream_t s) {
+    switch (G) {
+        case 1: launch_ragged<T, D, 1>(p, items, n_items, seqs, n_seq, any_split, s); break;
+        case 2: launch_ragged<T, D, 2>(p, items, n_items, seqs, n_seq, any_split, s); break;
+        case 4: launch_ragged<T, D, 4>(p, items, n_items, seqs, n_seq, any_split, s); break;
+        case 8: launch_ragged<T, D, 8>(p, items, n_items, seqs, n_seq, any_split, s); break;
+        default: return 2;
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("ragged sdpa_decode launch failed: %s", hipGetErrorString(e));
+    return 0;
+}
+
+// One launch per sequence on the caller's stream: the fall-back for shapes and formats the
+// ragged kernel does not cover (launches on one stream are ordered, so they share the workspace).
+int ragged_per_sequence(const void *q, void *out, int q_dtype, int kv_fmt, int64_t n_seq, int64_t Hq, int64_t Hkv,
+                        int64_t D, const RaggedSeq *seqs, float scale, void *workspace, size_t workspace_bytes,
+                        hipStream_t s) {
     size_t es = elem_bytes(q_dtype);
     for (int64_t i = 0; i < n_seq; i++) {
         SdpaArgs a;
@@ -386,10 +496,104 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
         a.mask_b = a.mask_h = 1;
         a.scale = scale;
         a.workspace = workspace, a.workspace_bytes = workspace_bytes;
-        int rc = launch_sdpa_decode(a, s);
+        int rc = is_quant(kv_fmt) ? launch_sdpa_decode_quant(a, s) : launch_sdpa_decode(a, s);
         if (rc == 2) rc = launch_sdpa_generic(a, s);
         if (rc) return rc;
     }
     return 0;
+}
+
+}  // namespace
+
+// Ragged decode: one launch for all sequences.  The host cuts the sequences into work items
+// of about equal tile counts, uploads the plan (items + per-sequence slot ranges) into the
+// head of the workspace, and the kernels index it by blockIdx.
+int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt, int64_t n_seq, int64_t Hq, int64_t Hkv,
+                              int64_t D, const RaggedSeq *seqs, float scale, void *workspace, size_t workspace_bytes,
+                              hipStream_t s) {
+    const int64_t G = Hq / Hkv;
+    const size_t es = elem_bytes(kv_fmt);
+    bool fast = (kv_fmt == TROCM_F16 || kv_fmt == TROCM_F32) && q_dtype == kv_fmt && (D == 64 || D == 128) &&
+                (G == 1 || G == 2 || G == 4 || G == 8) && workspace != nullptr && (uintptr_t)q % 16 == 0 &&
+                n_seq <= 2048 && Hkv <= 65535;
+    for (int64_t i = 0; i < n_seq && fast; i++)
+        fast = (uintptr_t)seqs[i].k % 16 == 0 && (uintptr_t)seqs[i].v % 16 == 0 && seqs[i].len < (1ll << 30) &&
+               (seqs[i].cap * D * es) % 16 == 0;
+    if (!fast)
+        return ragged_per_sequence(q, out, q_dtype, kv_fmt, n_seq, Hq, Hkv, D, seqs, scale, workspace, workspace_bytes, s);
+
+    // ---- plan ----------------------------------------------------------------------------------
+    int64_t total_tiles = 0;
+    for (int64_t i = 0; i < n_seq; i++) total_tiles += (seqs[i].len + kTile - 1) / kTile;
+    const int64_t rows_cap = (int64_t)((workspace_bytes - kWsCounterBytes) / ((D + 2) * sizeof(float)));
+    const int64_t max_items_ws = rows_cap / Hq;  // every item may need a partial record per q head
+    const int64_t max_items_tbl =
+        ((int64_t)kWsCounterBytes - n_seq * (int64_t)sizeof(RaggedSeqSlots)) / (int64_t)sizeof(RaggedItem);
+    const int64_t max_items = max_items_ws < max_items_tbl ? max_items_ws : max_items_tbl;
+    TROCM_REQUIRE(workspace_bytes > kWsCounterBytes && max_items >= n_seq,
+                  "sdpa workspace too small for %lld sequences (%zu bytes)", (long long)n_seq, workspace_bytes);
+    int64_t tiles_per_item = (total_tiles + num_compute_units() - 1) / num_compute_units();
+    if (tiles_per_item < kWaves) tiles_per_item = kWaves;
+    int64_t n_items = 0;
+    for (;;) {
+        n_items = 0;
+        for (int64_t i = 0; i < n_seq; i++) {
+            int64_t tiles = (seqs[i].len + kTile - 1) / kTile;
+            n_items += (tiles + tiles_per_item - 1) / tiles_per_item;
+        }
+        if (n_items <= max_items) break;
+        tiles_per_item += (tiles_per_item + 3) / 4;
+    }
+    StageSlot *stage;
+    if (acquire_stage(&stage)) return 1;
+    RaggedItem *items = (RaggedItem *)stage->host;
+    RaggedSeqSlots *slots = (RaggedSeqSlots *)(items + n_items);
+    int64_t it = 0;
+    bool any_split = false;
+    for (int64_t i = 0; i < n_seq; i++) {
+        int64_t tiles = (seqs[i].len + kTile - 1) / kTile;
+        int64_t ns = (tiles + tiles_per_item - 1) / tiles_per_item;
+        int64_t tps = (tiles + ns - 1) / ns;
+        ns = (tiles + tps - 1) / tps;
+        slots[i].slot0 = (int)it;
+        slots[i].nsplit = (int)ns;
+        any_split |= ns > 1;
+        for (int64_t sp = 0; sp < ns; sp++, it++) {
+            RaggedItem &r = items[it];
+            r.k = (const char *)seqs[i].k;
+            r.v = (const char *)seqs[i].v;
+            r.stride_h = seqs[i].cap * D * (int64_t)es;
+            r.T = (int)seqs[i].len;
+            r.tile_begin = (int)(sp * tps);
+            r.tile_end = (int)((sp + 1) * tps < tiles ? (sp + 1) * tps : tiles);
+            r.seq = (int)i, r.split = (int)sp, r.nsplit = (int)ns, r.slot0 = slots[i].slot0;
+        }
+    }
+    n_items = it;
+    // the seq table sits right after the items actually emitted
+    RaggedSeqSlots *slots_packed = (RaggedSeqSlots *)(items + n_items);
+    if (slots_packed != slots) memmove(slots_packed, slots, (size_t)n_seq * sizeof(RaggedSeqSlots));
+    size_t plan_bytes = (size_t)n_items * sizeof(RaggedItem) + (size_t)n_seq * sizeof(RaggedSeqSlots);
+    TROCM_HIP(hipMemcpyAsync(workspace, stage->host, plan_bytes, hipMemcpyHostToDevice, s));
+    TROCM_HIP(hipEventRecord(stage->done, s));
+    stage->in_flight = true;
+
+    DecodeDev p;
+    memset(&p, 0, sizeof(p));
+    p.q = (const char *)q;
+    p.out = (char *)out;
+    p.kv_stride_t = D * (int64_t)es;
+    p.Hq = (int)Hq;
+    p.Hkv = (int)Hkv;
+    p.scale_log2 = scale * 1.4426950408889634f;
+    p.part_ml = (float *)((char *)workspace + kWsCounterBytes);
+    p.part_o = p.part_ml + (size_t)n_items * Hkv * 2 * G;
+    const RaggedItem *d_items = (const RaggedItem *)workspace;
+    const RaggedSeqSlots *d_slots = (const RaggedSeqSlots *)(d_items + n_items);
+    if (kv_fmt == TROCM_F16)
+        return D == 128 ? launch_ragged_g<__half, 128>(p, (int)G, d_items, (int)n_items, d_slots, (int)n_seq, any_split, s)
+                        : launch_ragged_g<__half, 64>(p, (int)G, d_items, (int)n_items, d_slots, (int)n_seq, any_split, s);
+    return D == 128 ? launch_ragged_g<float, 128>(p, (int)G, d_items, (int)n_items, d_slots, (int)n_seq, any_split, s)
+                    : launch_ragged_g<float, 64>(p, (int)G, d_items, (int)n_items, d_slots, (int)n_seq, any_split, s);
 }
 }  // namespace trocm
