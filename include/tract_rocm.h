@@ -100,9 +100,22 @@ int trocm_copy_nd(void *dst, size_t dst_offset_bytes, const int64_t *dst_strides
  * canonical block bytes (scale then codes, blocks row-major along head_dim). */
 typedef struct trocm_kv_cache trocm_kv_cache;
 
+/* A pool is ONE device allocation from which many caches take (and, on growth, exchange)
+ * their planes: the arrangement for many independent sequences, each with its own
+ * capacity-doubling cache.  It stands where DeviceMemoryPool (gpu/src/memory/pool.rs) stands
+ * for per-run tensors, but for state that lives across runs.  Caches created in a pool
+ * fail with a message when the pool is exhausted; destroy them before the pool. */
+typedef struct trocm_kv_pool trocm_kv_pool;
+int trocm_kv_pool_create(trocm_kv_pool **out, size_t bytes);
+int trocm_kv_pool_destroy(trocm_kv_pool *pool);
+int trocm_kv_pool_stats(trocm_kv_pool *pool, size_t *bytes_total, size_t *bytes_in_use, size_t *largest_free,
+                        void **base);
+
 /* InPlaceKvCache::new (:37-39).  Allocates nothing until the first append or reserve. */
 int trocm_kv_cache_create(trocm_kv_cache **out, int storage_format, int64_t batch, int64_t kv_heads,
                           int64_t head_dim);
+int trocm_kv_cache_create_in_pool(trocm_kv_cache **out, trocm_kv_pool *pool, int storage_format,
+                                  int64_t batch, int64_t kv_heads, int64_t head_dim);
 int trocm_kv_cache_destroy(trocm_kv_cache *cache);
 /* len() / capacity() / reallocs() (:41-53). */
 int trocm_kv_cache_len(const trocm_kv_cache *cache, int64_t *len);

@@ -142,3 +142,44 @@ def test_copy_nd_general(rt):
     I2 = C.c_int64 * 2
     call("trocm_copy_nd", d_dst.ptr, 0, I2(7, 1), d_src.ptr, 0, I2(0, 1), I2(4, 7), 2, 4, None)
     assert np.array_equal(d_dst.to_numpy(), np.broadcast_to(src, (4, 7)))
+
+
+def test_pool_backed_caches_share_one_allocation(rt):
+    """cfg5's memory arrangement: per-sequence capacity-doubling caches carved from one device
+    allocation; growth exchanges planes inside the pool; exhaustion is an error, not a fault."""
+    rng = np.random.default_rng(6)
+    H, D = 2, 64
+    pool = tract_amd.KvPool(4 << 20)
+    base, total = pool.stats()["base"], pool.stats()["bytes_total"]
+    caches, refs = [], []
+    for i in range(6):
+        c, r = tract_amd.InPlaceKvCache(2, pool=pool), orc.InPlaceKvCache(2)
+        x = rng.standard_normal((1, H, 3 + 5 * i, D)).astype(np.float16)
+        c.push(x), r.push(x)
+        caches.append(c), refs.append(r)
+    for step in range(70):  # single-token growth: every cache doubles several times inside the pool
+        for c, r in zip(caches, refs):
+            x = rng.standard_normal((1, H, 1, D)).astype(np.float16)
+            c.push(x), r.push(x)
+    for c, r in zip(caches, refs):
+        assert (c.len(), c.capacity(), c.reallocs()) == (r.len(), r.capacity(), r.reallocs())
+        assert c.valid_contiguous().tobytes() == r.valid_contiguous().tobytes()
+        ptr, _, cap = c.raw()
+        assert base <= ptr and ptr + H * cap * D * 2 <= base + total
+    used = pool.stats()["bytes_in_use"]
+    assert used >= sum(H * c.capacity() * D * 2 for c in caches)
+    # a quantised cache in the same pool
+    qc = tract_amd.InPlaceKvCache(2, storage_format=tract_amd.Q4_0, pool=pool)
+    x = rng.standard_normal((1, H, 40, D)).astype(np.float16)
+    qc.push(x)
+    assert qc.valid_contiguous().tobytes() == orc.quant(orc.FMT_Q4_0, x).tobytes()
+    # exhaustion
+    big = tract_amd.InPlaceKvCache(2, pool=pool)
+    with pytest.raises(tract_amd.TractRocmError, match="pool exhausted"):
+        big.push(np.zeros((1, H, 40000, D), np.float16))
+    with pytest.raises(tract_amd.TractRocmError, match="live caches"):
+        pool.close()
+    for c in caches + [qc, big]:
+        c.close()
+    assert pool.stats()["bytes_in_use"] == 0 and pool.stats()["largest_free"] == total
+    pool.close()

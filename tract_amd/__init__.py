@@ -9,5 +9,5 @@ the benchmark the way a ``tract-rocm`` crate would use it through FFI.
 from ._lib import F16, F32, Q4_0, Q8_0, TractRocmError  # noqa: F401
 from .runtime import (DeviceTensor, Event, RocmRuntime, Stream, Workspace, runtime_for_name,  # noqa: F401
                       synchronize)
-from .ops import (BlockQuant, DynKeyValueCache, DynKeyValueCacheState, InPlaceKvCache,  # noqa: F401
+from .ops import (BlockQuant, DynKeyValueCache, DynKeyValueCacheState, InPlaceKvCache, KvPool,  # noqa: F401
                   InPlaceKvSdpa, InPlaceKvSdpaState, Sdpa, Q4_0_FORMAT, Q8_0_FORMAT, sdpa_decode_ragged)

@@ -43,6 +43,10 @@ SIGNATURES = {
     "trocm_event_elapsed_ms": [_vp, _vp, C.POINTER(_f)],
     "trocm_copy_nd": [_vp, _sz, _pi64, _vp, _sz, _pi64, _pi64, _i, _i, _vp],
     "trocm_kv_cache_create": [C.POINTER(_vp), _i, _i64, _i64, _i64],
+    "trocm_kv_cache_create_in_pool": [C.POINTER(_vp), _vp, _i, _i64, _i64, _i64],
+    "trocm_kv_pool_create": [C.POINTER(_vp), _sz],
+    "trocm_kv_pool_destroy": [_vp],
+    "trocm_kv_pool_stats": [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_vp)],
     "trocm_kv_cache_destroy": [_vp],
     "trocm_kv_cache_len": [_vp, _pi64],
     "trocm_kv_cache_capacity": [_vp, _pi64],

@@ -6,6 +6,8 @@
 #include <stdlib.h>
 #include <string.h>
 #include <math.h>
+#include <iterator>
+#include <map>
 #include <mutex>
 #include <new>
 #include <vector>
@@ -65,6 +67,58 @@ int resolve_stream(void *stream, hipStream_t *out) {
 
 using namespace trocm;
 
+// ---- KV pool: one device allocation carved into per-cache planes ------------------------------
+// (the role of DeviceMemoryPool, gpu/src/memory/pool.rs, for state that outlives a run).
+// Address-ordered first fit with coalescing; 256-byte granularity; guarded by a mutex.
+struct trocm_kv_pool {
+    char *base = nullptr;
+    size_t bytes = 0, in_use = 0;
+    int64_t live_caches = 0;
+    std::map<size_t, size_t> free_list;  // offset -> size
+    std::map<size_t, size_t> used;       // offset -> size
+    std::mutex mu;
+};
+
+static void *pool_alloc(trocm_kv_pool *pool, size_t bytes) {
+    bytes = (bytes + 255) & ~(size_t)255;
+    if (bytes == 0) bytes = 256;
+    std::lock_guard<std::mutex> lock(pool->mu);
+    for (auto it = pool->free_list.begin(); it != pool->free_list.end(); ++it) {
+        if (it->second >= bytes) {
+            size_t off = it->first, rest = it->second - bytes;
+            pool->free_list.erase(it);
+            if (rest) pool->free_list[off + bytes] = rest;
+            pool->used[off] = bytes;
+            pool->in_use += bytes;
+            return pool->base + off;
+        }
+    }
+    return nullptr;
+}
+
+static void pool_free(trocm_kv_pool *pool, void *ptr) {
+    std::lock_guard<std::mutex> lock(pool->mu);
+    size_t off = (size_t)((char *)ptr - pool->base);
+    auto u = pool->used.find(off);
+    if (u == pool->used.end()) return;
+    size_t size = u->second;
+    pool->used.erase(u);
+    pool->in_use -= size;
+    auto next = pool->free_list.lower_bound(off);
+    if (next != pool->free_list.end() && off + size == next->first) {  // merge with the block after
+        size += next->second;
+        next = pool->free_list.erase(next);
+    }
+    if (next != pool->free_list.begin()) {  // merge with the block before
+        auto prev = std::prev(next);
+        if (prev->first + prev->second == off) {
+            prev->second += size;
+            return;
+        }
+    }
+    pool->free_list[off] = size;
+}
+
 // ---- KV cache object -------------------------------------------------------------------------
 struct trocm_kv_cache {
     int fmt;
@@ -72,7 +126,33 @@ struct trocm_kv_cache {
     int64_t len, cap, reallocs;
     void *data;    // F32/F16 rows, or the code plane
     void *scales;  // f16 scale plane of the quantised formats
+    trocm_kv_pool *pool;  // where the planes live; NULL = their own hipMalloc
 };
+
+static int plane_alloc(trocm_kv_cache *c, void **ptr, size_t bytes, const char *what) {
+    if (c->pool) {
+        *ptr = pool_alloc(c->pool, bytes);
+        if (!*ptr) {
+            std::lock_guard<std::mutex> lock(c->pool->mu);
+            return fail("KV pool exhausted: %s of %zu bytes does not fit (%zu of %zu bytes in use)", what, bytes,
+                        c->pool->in_use, c->pool->bytes);
+        }
+        return 0;
+    }
+    hipError_t e = hipMalloc(ptr, bytes ? bytes : 16);
+    if (e != hipSuccess) return fail("allocating %s (%zu bytes) failed: %s", what, bytes, hipGetErrorString(e));
+    return 0;
+}
+
+static int plane_free(trocm_kv_cache *c, void *ptr) {
+    if (!ptr) return 0;
+    if (c->pool) {
+        pool_free(c->pool, ptr);
+        return 0;
+    }
+    TROCM_HIP(hipFree(ptr));
+    return 0;
+}
 
 static size_t plane_bytes(const trocm_kv_cache *c, int64_t cap) {
     return (size_t)c->B * c->H * cap * device_row_bytes(c->fmt, c->D);
@@ -109,29 +189,23 @@ static int copy_valid(const trocm_kv_cache *c, void *dst, void *dst_scales, int6
 static int regrow(trocm_kv_cache *c, int64_t new_cap, hipStream_t s) {
     void *nd = nullptr, *ns = nullptr;
     size_t pb = plane_bytes(c, new_cap), sb = scale_plane_bytes(c, new_cap);
-    hipError_t e = hipMalloc(&nd, pb ? pb : 16);
-    if (e != hipSuccess)
-        return fail("allocating a KV cache of %lld tokens (%zu bytes) failed: %s", (long long)new_cap, pb,
-                    hipGetErrorString(e));
-    if (sb) {
-        e = hipMalloc(&ns, sb);
-        if (e != hipSuccess) {
-            (void)hipFree(nd);
-            return fail("allocating KV cache scales (%zu bytes) failed: %s", sb, hipGetErrorString(e));
-        }
+    if (plane_alloc(c, &nd, pb, "a KV cache plane")) return 1;
+    if (sb && plane_alloc(c, &ns, sb, "a KV cache scale plane")) {
+        (void)plane_free(c, nd);
+        return 1;
     }
     if (c->data && c->len) {
         if (copy_valid(c, nd, ns, new_cap, c->data, c->scales, c->cap, c->len, s)) {
-            (void)hipFree(nd);
-            if (ns) (void)hipFree(ns);
+            (void)plane_free(c, nd);
+            (void)plane_free(c, ns);
             return 1;
         }
     }
     if (c->data) {
         // The old buffers may still be read by work queued on the stream.
         TROCM_HIP(hipStreamSynchronize(s));
-        TROCM_HIP(hipFree(c->data));
-        if (c->scales) TROCM_HIP(hipFree(c->scales));
+        if (plane_free(c, c->data)) return 1;
+        if (plane_free(c, c->scales)) return 1;
     }
     c->data = nd;
     c->scales = ns;
@@ -315,17 +389,72 @@ int trocm_kv_cache_create(trocm_kv_cache **out, int fmt, int64_t batch, int64_t 
     c->B = batch, c->H = kv_heads, c->D = head_dim;
     c->len = c->cap = c->reallocs = 0;
     c->data = c->scales = nullptr;
+    c->pool = nullptr;
     *out = c;
+    return 0;
+}
+
+int trocm_kv_cache_create_in_pool(trocm_kv_cache **out, trocm_kv_pool *pool, int fmt, int64_t batch, int64_t kv_heads,
+                                  int64_t head_dim) {
+    TROCM_NOT_NULL(pool);
+    if (trocm_kv_cache_create(out, fmt, batch, kv_heads, head_dim)) return 1;
+    (*out)->pool = pool;
+    std::lock_guard<std::mutex> lock(pool->mu);
+    pool->live_caches += 1;
     return 0;
 }
 
 int trocm_kv_cache_destroy(trocm_kv_cache *c) {
     if (!c) return 0;
-    int rc = 0;
-    if (c->data && hipFree(c->data) != hipSuccess) rc = fail("hipFree of a KV cache failed");
-    if (c->scales && hipFree(c->scales) != hipSuccess) rc = fail("hipFree of KV cache scales failed");
+    int rc = plane_free(c, c->data);
+    rc |= plane_free(c, c->scales);
+    if (c->pool) {
+        std::lock_guard<std::mutex> lock(c->pool->mu);
+        c->pool->live_caches -= 1;
+    }
     delete c;
     return rc;
+}
+
+int trocm_kv_pool_create(trocm_kv_pool **out, size_t bytes) {
+    TROCM_NOT_NULL(out);
+    if (ensure_init()) return 1;
+    TROCM_REQUIRE(bytes >= 256, "kv pool: size must be at least 256 bytes");
+    bytes &= ~(size_t)255;
+    trocm_kv_pool *p = new (std::nothrow) trocm_kv_pool();
+    TROCM_REQUIRE(p != nullptr, "out of host memory");
+    hipError_t e = hipMalloc((void **)&p->base, bytes);
+    if (e != hipSuccess) {
+        delete p;
+        return fail("allocating a KV pool of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+    }
+    p->bytes = bytes;
+    p->free_list[0] = bytes;
+    *out = p;
+    return 0;
+}
+
+int trocm_kv_pool_destroy(trocm_kv_pool *p) {
+    if (!p) return 0;
+    TROCM_REQUIRE(p->live_caches == 0, "kv pool still has %lld live caches", (long long)p->live_caches);
+    TROCM_HIP(hipFree(p->base));
+    delete p;
+    return 0;
+}
+
+int trocm_kv_pool_stats(trocm_kv_pool *p, size_t *bytes_total, size_t *bytes_in_use, size_t *largest_free,
+                        void **base) {
+    TROCM_NOT_NULL(p);
+    std::lock_guard<std::mutex> lock(p->mu);
+    if (bytes_total) *bytes_total = p->bytes;
+    if (bytes_in_use) *bytes_in_use = p->in_use;
+    if (largest_free) {
+        size_t m = 0;
+        for (auto &kv : p->free_list) m = kv.second > m ? kv.second : m;
+        *largest_free = m;
+    }
+    if (base) *base = p->base;
+    return 0;
 }
 
 int trocm_kv_cache_len(const trocm_kv_cache *c, int64_t *len) {
@@ -487,7 +616,9 @@ int trocm_kv_cache_clone(const trocm_kv_cache *c, trocm_kv_cache **out, void *st
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
     trocm_kv_cache *n = nullptr;
-    if (trocm_kv_cache_create(&n, c->fmt, c->B, c->H, c->D)) return 1;
+    if (c->pool ? trocm_kv_cache_create_in_pool(&n, c->pool, c->fmt, c->B, c->H, c->D)
+                : trocm_kv_cache_create(&n, c->fmt, c->B, c->H, c->D))
+        return 1;
     if (c->cap) {
         if (regrow(n, c->cap, s)) {
             trocm_kv_cache_destroy(n);

@@ -38,11 +38,33 @@ def _canon4(shape):
     raise TractRocmError(f"Inputs must be of rank 3 or 4, found {len(shape)}")
 
 
+class KvPool:
+    """One device allocation shared by many caches (per-sequence capacity-doubling caches of a
+    ragged batch)."""
+
+    def __init__(self, nbytes: int):
+        h = C.c_void_p()
+        call("trocm_kv_pool_create", C.byref(h), nbytes)
+        self.handle = h
+
+    def stats(self) -> dict:
+        total, used, largest, base = C.c_size_t(), C.c_size_t(), C.c_size_t(), C.c_void_p()
+        call("trocm_kv_pool_stats", self.handle, C.byref(total), C.byref(used), C.byref(largest), C.byref(base))
+        return {"bytes_total": total.value, "bytes_in_use": used.value, "largest_free": largest.value,
+                "base": base.value}
+
+    def close(self) -> None:
+        if self.handle:
+            call("trocm_kv_pool_destroy", self.handle)
+            self.handle = None
+
+
 class InPlaceKvCache:
     """Geometric-growth in-place cache along `axis` (the token axis, rank-2)."""
 
-    def __init__(self, axis: int, storage_format: int | None = None):
+    def __init__(self, axis: int, storage_format: int | None = None, pool: KvPool | None = None):
         self.axis = axis
+        self.pool = pool
         self.storage_format = storage_format  # None: same as the first pushed tensor
         self._h = None
         self._shape = None
@@ -55,7 +77,10 @@ class InPlaceKvCache:
         B, H, _, D = _canon4(shape)
         fmt = dtype_code(dtype) if self.storage_format is None else self.storage_format
         h = C.c_void_p()
-        call("trocm_kv_cache_create", C.byref(h), fmt, B, H, D)
+        if self.pool is not None:
+            call("trocm_kv_cache_create_in_pool", C.byref(h), self.pool.handle, fmt, B, H, D)
+        else:
+            call("trocm_kv_cache_create", C.byref(h), fmt, B, H, D)
         self._h, self._shape, self._dtype, self.storage_format = h, tuple(shape), np.dtype(dtype), fmt
 
     def __del__(self):
@@ -143,12 +168,24 @@ class InPlaceKvCache:
         return out.to_numpy(stream)
 
     def clone(self, stream=None) -> "InPlaceKvCache":
-        c = InPlaceKvCache(self.axis, self.storage_format)
+        c = InPlaceKvCache(self.axis, self.storage_format, self.pool)
         if self._h is not None:
             h = C.c_void_p()
             call("trocm_kv_cache_clone", self._h, C.byref(h), _sh(stream))
             c._h, c._shape, c._dtype = h, self._shape, self._dtype
         return c
+
+    def close(self) -> None:
+        """Release the device planes now (otherwise at garbage collection)."""
+        if self._h:
+            call("trocm_kv_cache_destroy", self._h)
+            self._h = None
+
+    def raw(self):
+        """(data pointer, scales pointer or None, capacity) of the device planes."""
+        d, sc, cap = C.c_void_p(), C.c_void_p(), C.c_int64()
+        call("trocm_kv_cache_raw", self._h, C.byref(d), C.byref(sc), C.byref(cap))
+        return d.value, sc.value, cap.value
 
     @property
     def handle(self):
