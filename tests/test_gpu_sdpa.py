@@ -285,3 +285,48 @@ def test_ragged_equals_padded_batch_with_mask(rt):
     assert max_abs(got, want) <= 1e-3
     dense = tract_amd.Sdpa().eval(q, kp, vp, mask).to_numpy()
     assert max_abs(got, dense) <= 1e-5
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal", [
+    (1, 4, 1, 32, 32, 128, True), (1, 4, 2, 64, 64, 128, True), (1, 8, 2, 100, 100, 128, True),
+    (1, 4, 4, 33, 200, 128, True), (2, 8, 2, 77, 301, 128, False), (1, 32, 8, 128, 384, 128, True),
+    (2, 32, 8, 512, 512, 128, True),      # >= 256 workgroups: 128-query tiles (4x1 waves)
+    (1, 32, 8, 200, 712, 128, True),      # 64-query tiles (2x2 waves), ragged edges
+    (1, 8, 8, 90, 90, 64, True), (2, 64, 8, 256, 300, 64, False), (1, 4, 2, 2, 9, 128, True),
+])
+def test_prefill_mfma(rt, B, Hq, Hkv, Sq, Sk, D, causal):
+    rng = np.random.default_rng(1000 + Sq + Sk)
+    q = (rng.standard_normal((B, Hq, Sq, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    k = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(np.float16)
+    got = tract_amd.Sdpa(datum_type=np.float16, is_causal=causal).eval(q, k, v).to_numpy()
+    want = orc.flash_sdpa(q, k, v, causal=causal, threads=8)
+    assert not np.isnan(got).any()
+    assert max_abs(got, want) <= 2e-2
+    assert max_abs(got, cases.textbook_sdpa(q, k, v, causal=causal)) <= 4e-3
+
+
+def test_chunked_prefill_into_cache_cfg3_reduced(rt):
+    """cfg3 (reduced to 8 chunks of 96 tokens): each chunk is appended to the in-place cache,
+    then attends causally to the whole cache so far (q_len 96, kv_len 96*c), reading K/V from
+    the capacity buffer.  The concatenated outputs equal one causal pass over all tokens."""
+    rng = np.random.default_rng(cases.cfg_seed(3, "q"))
+    B, Hq, Hkv, D, S, C = 1, 32, 8, 128, 96, 8
+    q = (cases.seeded_normal(cases.cfg_seed(3, "q"), (B, Hq, S * C, D)) / np.sqrt(D)).astype(np.float16)
+    k = cases.seeded_normal(cases.cfg_seed(3, "k"), (B, Hkv, S * C, D), np.float16)
+    v = cases.seeded_normal(cases.cfg_seed(3, "v"), (B, Hkv, S * C, D), np.float16)
+    st = tract_amd.InPlaceKvSdpa(axis=2, causal=True).state()
+    outs = []
+    for c in range(C):
+        sl = slice(c * S, (c + 1) * S)
+        outs.append(st.eval([q[:, :, sl], k[:, :, sl], v[:, :, sl]]).to_numpy())
+        assert st.k.len() == (c + 1) * S
+    got = np.concatenate(outs, axis=2)
+    assert st.k.capacity() == 768 and st.k.reallocs() == 3
+    assert st.k.valid_contiguous().tobytes() == k.tobytes()
+    want = orc.flash_sdpa(q, k, v, causal=True, threads=8)
+    assert max_abs(got, want) <= 2e-2
+    # chunk c on its own against the oracle with the bottom-right aligned causal rule
+    c = 5
+    one = orc.flash_sdpa(q[:, :, c * S:(c + 1) * S], k[:, :, :(c + 1) * S], v[:, :, :(c + 1) * S], causal=True, threads=8)
+    assert max_abs(outs[c], one) <= 2e-2

@@ -1,5 +1,300 @@
-// MFMA prefill attention for gfx950 (placeholder dispatch until the kernel lands).
+// MFMA prefill attention for gfx950: q_len > 1, f16 in/out, f32 accumulate, causal
+// (bottom-right aligned) or unmasked, GQA, K/V read in place from the capacity buffer.
+//
+// Formulation (transposed, so that every per-query softmax scalar lives in one lane):
+//   S^T = K . Q^T      v_mfma_f32_32x32x16_f16, A = K rows (key-major, contraction over d),
+//                      B = Q rows held in registers for the whole kernel
+//   O^T = V^T . P^T    A = V^T fragments, B = P^T taken straight from the S^T accumulators
+//                      (rounded to f16), contraction over keys
+// In the 32x32 accumulator layout a lane holds ONE query column (lane % 32) and 16 of the 32
+// rows (keys, or output features): row maxima and sums over keys are in-lane reductions plus
+// one exchange between the two half-waves, and the rescaling factors of the online softmax
+// apply to the lane's own O^T registers.
+//
+// A wave owns 32 queries and, per workgroup tile, 64 keys.  The 4 waves of a workgroup are
+// arranged WM x WN: WM query groups (BLOCK_M = 32*WM) times WN key slices (BLOCK_N = 64*WN);
+// waves that share queries keep separate online-softmax states and are merged through LDS at
+// the end.  4x1 suits long query chunks, 2x2 keeps all four SIMDs busy when there are few
+// query tiles.
+//
+// K tile: global -> registers (prefetched one tile ahead) -> LDS, row-major, rows padded by 16
+// bytes (conflict-free 128-bit fragment reads).  V tile: the MFMA wants 8 consecutive KEYS per
+// lane for a fixed feature, but V rows are feature-major, so V is stored transposed in LDS
+// ([feature][key]) with the keys of each group of 16 permuted into the order in which the
+// S^T accumulator registers hold them; a V^T fragment is then one 128-bit LDS read.
+//
+// Roofline: MFMA-bound.  FLOPs = 4 * B * Hq * D * (visible query-key pairs).
+#include <hip/hip_fp16.h>
+#include <string.h>
+#include <stdlib.h>
 #include "common.h"
+
 namespace trocm {
-int launch_sdpa_prefill(const SdpaArgs &, hipStream_t) { return 2; }
+namespace {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+
+struct PrefillDev {
+    const _Float16 *q;
+    _Float16 *out;
+    const _Float16 *k, *v;
+    int64_t kv_stride_b, kv_stride_h, kv_stride_t;  // elements
+    int B, Hq, Hkv, Sq, Sk;
+    int causal;
+    int n_qtiles;
+    float scale_log2;
+};
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Position of key `k16` (0..15) inside its group of 16 in the transposed V tile: lane half hb
+// of the MFMA contraction holds, in order, accumulator rows 4hb..4hb+3 and 8+4hb..8+4hb+3.
+__device__ __forceinline__ int vt_pos(int k16) { return 8 * ((k16 >> 2) & 1) + 4 * (k16 >> 3) + (k16 & 3); }
+
+template <int D, int WM, int WN>
+__global__ __launch_bounds__(kThreads, 1) void sdpa_prefill_kernel(PrefillDev p) {
+    constexpr int BLOCK_M = 32 * WM, BLOCK_N = 64 * WN;
+    constexpr int KS = D / 16;            // contraction steps of Q K^T
+    constexpr int DB = D / 32;            // 32-feature blocks of the output
+    constexpr int KROW = D + 8;           // halfs per K row in LDS
+    constexpr int VROW = BLOCK_N + 8;     // halfs per V^T row in LDS
+    constexpr int NL = BLOCK_N * D / 8 / kThreads;  // 128-bit loads per thread per tile and tensor
+    static_assert(WM * WN == 4, "four waves per workgroup");
+
+    __shared__ __attribute__((aligned(16))) _Float16 lds_k[BLOCK_N * KROW];
+    __shared__ __attribute__((aligned(16))) _Float16 lds_vt[D * VROW];
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int hb = lane >> 5, l32 = lane & 31;
+    const int wm = w % WM, wn = w / WM;
+
+    // workgroup -> (kv head fastest, so that consecutive workgroup ids, which the hardware deals
+    // round-robin to the 8 XCDs, keep one kv head's K/V in one XCD's L2), longest query tiles first
+    int id = blockIdx.x;
+    const int kvh = id % p.Hkv;
+    id /= p.Hkv;
+    const int G = p.Hq / p.Hkv;
+    const int g = id % G;
+    id /= G;
+    const int qt = p.n_qtiles - 1 - (id % p.n_qtiles);
+    const int b = id / p.n_qtiles;
+    const int qh = kvh * G + g;
+
+    const int off = p.Sk - p.Sq;          // query i sees keys j <= i + off when causal
+    const int q0 = qt * BLOCK_M + 32 * wm;  // first query of this wave
+    const int my_q = q0 + l32;
+    const _Float16 *qrow = p.q + (((int64_t)b * p.Hq + qh) * p.Sq + min(my_q, p.Sq - 1)) * D;
+    const _Float16 *kbase = p.k + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+    const _Float16 *vbase = p.v + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+
+    // Q^T fragments: query = lane % 32, features 16*ks + 8*hb .. +8
+    half8_t qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = *reinterpret_cast<const half8_t *>(qrow + 16 * ks + 8 * hb);
+
+    // key tiles this workgroup needs
+    const int wg_q_last = min(qt * BLOCK_M + BLOCK_M, p.Sq) - 1;
+    const int last_key = p.causal ? min(p.Sk - 1, wg_q_last + off) : p.Sk - 1;
+    const int n_kt = last_key / BLOCK_N + 1;
+    const int wave_q_last = min(q0 + 31, p.Sq - 1);
+
+    float m_run = -INFINITY, l_run = 0.0f;
+    float16_t o[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
+
+    u32x4 kpre[NL], vpre[NL];
+    auto prefetch = [&](int kt) {
+#pragma unroll
+        for (int j = 0; j < NL; j++) {
+            int c = j * kThreads + tid;
+            int key = c / (D / 8), dc = c % (D / 8);
+            int64_t row = min(kt * BLOCK_N + key, p.Sk - 1);
+            kpre[j] = *reinterpret_cast<const u32x4 *>(kbase + row * p.kv_stride_t + dc * 8);
+            vpre[j] = *reinterpret_cast<const u32x4 *>(vbase + row * p.kv_stride_t + dc * 8);
+        }
+    };
+    prefetch(0);
+
+    for (int kt = 0; kt < n_kt; kt++) {
+        __syncthreads();  // everyone is done reading the previous tile
+#pragma unroll
+        for (int j = 0; j < NL; j++) {
+            int c = j * kThreads + tid;
+            int key = c / (D / 8), dc = c % (D / 8);
+            *reinterpret_cast<u32x4 *>(&lds_k[key * KROW + dc * 8]) = kpre[j];
+            int pos = (key & ~15) + vt_pos(key & 15);
+            uint32_t vw[4] = {vpre[j].x, vpre[j].y, vpre[j].z, vpre[j].w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint16_t lo = (uint16_t)(vw[i] & 0xffffu), hi = (uint16_t)(vw[i] >> 16);
+                *reinterpret_cast<uint16_t *>(&lds_vt[(dc * 8 + 2 * i) * VROW + pos]) = lo;
+                *reinterpret_cast<uint16_t *>(&lds_vt[(dc * 8 + 2 * i + 1) * VROW + pos]) = hi;
+            }
+        }
+        __syncthreads();
+        if (kt + 1 < n_kt) prefetch(kt + 1);
+
+        const int k_lo = kt * BLOCK_N + 64 * wn;  // first key of this wave's slice
+        const bool active = k_lo < p.Sk && (!p.causal || k_lo <= wave_q_last + off);
+        if (!active) continue;
+
+        // ---- S^T = K Q^T : 2 key blocks of 32 x 32 queries -------------------------------------
+        float16_t s[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[kb][r] = 0.0f;
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                half8_t kf = *reinterpret_cast<const half8_t *>(&lds_k[(64 * wn + 32 * kb + l32) * KROW + 16 * ks + 8 * hb]);
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s[kb], 0, 0, 0);
+            }
+        }
+        // ---- online softmax for query lane%32 over this lane's 32 keys ---------------------------
+        const bool need_mask = (k_lo + 64 > p.Sk) || (p.causal && (k_lo + 63 > q0 + off));
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                float x = s[kb][r] * p.scale_log2;
+                if (need_mask) {
+                    int key = k_lo + 32 * kb + 8 * (r >> 2) + 4 * hb + (r & 3);
+                    bool vis = key < p.Sk && (!p.causal || key <= my_q + off);
+                    x = vis ? x : -INFINITY;
+                }
+                s[kb][r] = x;
+                tmax = fmaxf(tmax, x);
+            }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m_run, tmax);
+        const float m_ref = (m_new == -INFINITY) ? 0.0f : m_new;  // nothing visible yet: keep everything at zero
+        const float alpha = fast_exp2(m_run - m_ref);
+        float psum = 0.0f;
+        half8_t pf[4];  // P^T fragments: contraction step st takes accumulator rows 8*(st%2)..+8 of block st/2
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float pv = fast_exp2(s[st >> 1][8 * (st & 1) + i] - m_ref);
+                psum += pv;
+                pf[st][i] = (_Float16)pv;
+            }
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[db][r] *= alpha;
+        // ---- O^T += V^T P^T ------------------------------------------------------------------------
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+                half8_t vf = *reinterpret_cast<const half8_t *>(&lds_vt[(32 * db + l32) * VROW + 64 * wn + 16 * st + 8 * hb]);
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[st], o[db], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- merge the two lane halves' sums, then the WN key slices through LDS ---------------------
+    l_run += __shfl_xor(l_run, 32, 64);
+    if constexpr (WN > 1) {
+        __syncthreads();  // the tiles are dead: reuse their space
+        float *xo = reinterpret_cast<float *>(lds_k);  // [WM][64 lanes][DB*16] + m, l
+        constexpr int kPer = DB * 16 + 2;
+        static_assert(sizeof(float) * WM * 64 * kPer <= sizeof(_Float16) * (BLOCK_N * KROW), "merge buffer");
+        float *mine = xo + ((size_t)wm * 64 + lane) * kPer;
+        if (wn == 1) {
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) mine[db * 16 + r] = o[db][r];
+            mine[DB * 16] = m_run;
+            mine[DB * 16 + 1] = l_run;
+        }
+        __syncthreads();
+        if (wn == 1) return;
+        const float m_o = mine[DB * 16], l_o = mine[DB * 16 + 1];
+        const float mm = fmaxf(m_run, m_o);
+        const float m_ref = (mm == -INFINITY) ? 0.0f : mm;
+        const float fa = fast_exp2(m_run - m_ref), fb = fast_exp2(m_o - m_ref);
+        l_run = l_run * fa + l_o * fb;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[db][r] = o[db][r] * fa + mine[db * 16 + r] * fb;
+    }
+    if (my_q >= p.Sq) return;
+    const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+    _Float16 *orow = p.out + (((int64_t)b * p.Hq + qh) * p.Sq + my_q) * D;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int rq = 0; rq < 4; rq++) {
+            half4_t h4;
+#pragma unroll
+            for (int i = 0; i < 4; i++) h4[i] = (_Float16)(o[db][4 * rq + i] * inv);
+            *reinterpret_cast<half4_t *>(orow + 32 * db + 8 * rq + 4 * hb) = h4;
+        }
+}
+
+template <int D, int WM, int WN>
+int launch_cfg(const PrefillDev &p0, hipStream_t s) {
+    PrefillDev p = p0;
+    constexpr int BLOCK_M = 32 * WM;
+    p.n_qtiles = (p.Sq + BLOCK_M - 1) / BLOCK_M;
+    int64_t wgs = (int64_t)p.B * p.Hq * p.n_qtiles;
+    if (wgs >= (1ll << 31)) return 2;
+    hipLaunchKernelGGL((sdpa_prefill_kernel<D, WM, WN>), dim3((unsigned)wgs), dim3(kThreads), 0, s, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("sdpa_prefill launch failed: %s", hipGetErrorString(e));
+    return 0;
+}
+
+}  // namespace
+
+int launch_sdpa_prefill(const SdpaArgs &a, hipStream_t s) {
+    if (a.q_dtype != TROCM_F16 || a.kv_fmt != TROCM_F16 || a.mask != nullptr) return 2;
+    if (a.D != 128 && a.D != 64) return 2;
+    if (a.Sq < 2 || a.Sk < 1 || a.Hq % a.Hkv) return 2;
+    if (a.causal && a.Sk < a.Sq) return 2;  // some queries would see nothing: the generic kernel owns that case
+    if (a.Sk >= (1ll << 30) || a.Sq >= (1ll << 30) || a.B >= (1ll << 20)) return 2;
+    if ((a.kv_stride_b % 8) || (a.kv_stride_h % 8) || (a.kv_stride_t % 8)) return 2;  // 128-bit row loads
+    if ((uintptr_t)a.q % 16 || (uintptr_t)a.k % 16 || (uintptr_t)a.v % 16 || (uintptr_t)a.out % 8) return 2;
+    PrefillDev p;
+    memset(&p, 0, sizeof(p));
+    p.q = (const _Float16 *)a.q;
+    p.out = (_Float16 *)a.out;
+    p.k = (const _Float16 *)a.k;
+    p.v = (const _Float16 *)a.v;
+    p.kv_stride_b = a.kv_stride_b, p.kv_stride_h = a.kv_stride_h, p.kv_stride_t = a.kv_stride_t;
+    p.B = (int)a.B, p.Hq = (int)a.Hq, p.Hkv = (int)a.Hkv, p.Sq = (int)a.Sq, p.Sk = (int)a.Sk;
+    p.causal = a.causal;
+    p.scale_log2 = a.scale * 1.4426950408889634f;
+    // 4x1 (128 queries per workgroup) when that still gives every compute unit a workgroup,
+    // else 2x2 (64 queries, keys split over two wave pairs)
+    static int forced = -1;
+    if (forced < 0) {
+        const char *e = getenv("TROCM_PREFILL_SHAPE");  // experiment knob: 41 or 22
+        forced = e ? atoi(e) : 0;
+    }
+    int64_t wgs_41 = a.B * a.Hq * ((a.Sq + 127) / 128);
+    bool use41 = forced ? forced == 41 : wgs_41 >= num_compute_units();
+    if (a.D == 128) return use41 ? launch_cfg<128, 4, 1>(p, s) : launch_cfg<128, 2, 2>(p, s);
+    return use41 ? launch_cfg<64, 4, 1>(p, s) : launch_cfg<64, 2, 2>(p, s);
+}
+
 }  // namespace trocm
