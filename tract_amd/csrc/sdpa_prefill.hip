@@ -17,11 +17,15 @@
 // the end.  4x1 suits long query chunks, 2x2 keeps all four SIMDs busy when there are few
 // query tiles.
 //
-// K tile: global -> registers (prefetched one tile ahead) -> LDS, row-major, rows padded by 16
-// bytes (conflict-free 128-bit fragment reads).  V tile: the MFMA wants 8 consecutive KEYS per
-// lane for a fixed feature, but V rows are feature-major, so V is stored transposed in LDS
-// ([feature][key]) with the keys of each group of 16 permuted into the order in which the
-// S^T accumulator registers hold them; a V^T fragment is then one 128-bit LDS read.
+// K and V tiles: global -> registers (prefetched one tile ahead) -> LDS, both row-major with
+// padded rows, written with 128-bit stores.  K fragments are plain 128-bit LDS reads.  For V
+// the MFMA wants 8 KEYS per lane at a fixed feature while V rows are feature-major: the
+// fragments are read with gfx950's transposing LDS load (ds_read_b64_tr_b16).  Measured
+// semantics of that load: in each block of 16 lanes, lane i receives element i%4 of the four
+// 8-byte rows addressed by lanes i/4, i/4+4, i/4+8, i/4+12.  So source lane s of a block points
+// at V[key(s/4)][16 features of the block + 4*(s%4)] and lane i comes back with 4 keys of its
+// own feature; two such loads give the 8 keys of one contraction step, in the order in which
+// the S^T accumulator registers hold them (rows 4hb..4hb+3, then 8+4hb..8+4hb+3).
 //
 // Roofline: MFMA-bound.  FLOPs = 4 * B * Hq * D * (visible query-key pairs).
 #include <hip/hip_fp16.h>
@@ -36,6 +40,7 @@ typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef short short4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
 
@@ -52,22 +57,25 @@ struct PrefillDev {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// Position of key `k16` (0..15) inside its group of 16 in the transposed V tile: lane half hb
-// of the MFMA contraction holds, in order, accumulator rows 4hb..4hb+3 and 8+4hb..8+4hb+3.
-__device__ __forceinline__ int vt_pos(int k16) { return 8 * ((k16 >> 2) & 1) + 4 * (k16 >> 3) + (k16 & 3); }
+// Transposing 64-bit LDS load of 16-bit elements (see the header comment for its lane mapping).
+__device__ __forceinline__ half4_t lds_read_tr16(const _Float16 *lds_ptr) {
+    typedef __attribute__((address_space(3))) short4_t *lds_v4_ptr;
+    short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_ptr)(uintptr_t)(uint32_t)(uintptr_t)lds_ptr);
+    return __builtin_bit_cast(half4_t, r);
+}
 
 template <int D, int WM, int WN>
 __global__ __launch_bounds__(kThreads, 1) void sdpa_prefill_kernel(PrefillDev p) {
     constexpr int BLOCK_M = 32 * WM, BLOCK_N = 64 * WN;
     constexpr int KS = D / 16;            // contraction steps of Q K^T
     constexpr int DB = D / 32;            // 32-feature blocks of the output
-    constexpr int KROW = D + 8;           // halfs per K row in LDS
-    constexpr int VROW = BLOCK_N + 8;     // halfs per V^T row in LDS
+    constexpr int KROW = D + 8;           // halfs per K row in LDS: 128-bit reads of 16 rows hit 64 distinct banks
+    constexpr int VROW = D + 16;          // halfs per V row in LDS: the 4 rows of a transposing read sit 8 banks apart
     constexpr int NL = BLOCK_N * D / 8 / kThreads;  // 128-bit loads per thread per tile and tensor
     static_assert(WM * WN == 4, "four waves per workgroup");
 
     __shared__ __attribute__((aligned(16))) _Float16 lds_k[BLOCK_N * KROW];
-    __shared__ __attribute__((aligned(16))) _Float16 lds_vt[D * VROW];
+    __shared__ __attribute__((aligned(16))) _Float16 lds_v[BLOCK_N * VROW];
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int hb = lane >> 5, l32 = lane & 31;
@@ -130,14 +138,7 @@ __global__ __launch_bounds__(kThreads, 1) void sdpa_prefill_kernel(PrefillDev p)
             int c = j * kThreads + tid;
             int key = c / (D / 8), dc = c % (D / 8);
             *reinterpret_cast<u32x4 *>(&lds_k[key * KROW + dc * 8]) = kpre[j];
-            int pos = (key & ~15) + vt_pos(key & 15);
-            uint32_t vw[4] = {vpre[j].x, vpre[j].y, vpre[j].z, vpre[j].w};
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                uint16_t lo = (uint16_t)(vw[i] & 0xffffu), hi = (uint16_t)(vw[i] >> 16);
-                *reinterpret_cast<uint16_t *>(&lds_vt[(dc * 8 + 2 * i) * VROW + pos]) = lo;
-                *reinterpret_cast<uint16_t *>(&lds_vt[(dc * 8 + 2 * i + 1) * VROW + pos]) = hi;
-            }
+            *reinterpret_cast<u32x4 *>(&lds_v[key * VROW + dc * 8]) = vpre[j];
         }
         __syncthreads();
         if (kt + 1 < n_kt) prefetch(kt + 1);
@@ -199,11 +200,16 @@ __global__ __launch_bounds__(kThreads, 1) void sdpa_prefill_kernel(PrefillDev p)
 #pragma unroll
             for (int r = 0; r < 16; r++) o[db][r] *= alpha;
         // ---- O^T += V^T P^T ------------------------------------------------------------------------
+        // This lane as a SOURCE of the transposing loads: key row (lane%16)/4 of a group of four,
+        // features 16*(lane/16 % 2) + 4*(lane%4) of the 32-feature block.
+        const _Float16 *vsrc = &lds_v[(64 * wn + 4 * hb + ((lane & 15) >> 2)) * VROW + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)];
 #pragma unroll
         for (int st = 0; st < 4; st++) {
 #pragma unroll
             for (int db = 0; db < DB; db++) {
-                half8_t vf = *reinterpret_cast<const half8_t *>(&lds_vt[(32 * db + l32) * VROW + 64 * wn + 16 * st + 8 * hb]);
+                half4_t lo = lds_read_tr16(vsrc + (16 * st) * VROW + 32 * db);      // keys 16st + 4hb + 0..3
+                half4_t hi = lds_read_tr16(vsrc + (16 * st + 8) * VROW + 32 * db);  // keys 16st + 8 + 4hb + 0..3
+                half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
                 o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[st], o[db], 0, 0, 0);
             }
         }
