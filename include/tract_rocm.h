@@ -216,6 +216,15 @@ int trocm_sdpa_decode_ragged(const void *q, int q_dtype, int64_t q_heads, int64_
                              void *out, float scale, void *workspace, size_t workspace_bytes,
                              void *stream);
 
+/* One decode step of a ragged batch as one call: append k_new[i], v_new[i] (dense
+ * [n_seq, kv_heads, 1, head_dim] of `dtype`) to sequence i's caches, then attend q[i] over them.
+ * Per sequence this is InPlaceKvSdpaState::eval (inplace_kv_cache.rs:191-216).  On F32/F16 caches
+ * the attention kernel stores the new tokens itself: one launch (plus the split merge) per step. */
+int trocm_inplace_kv_sdpa_eval_ragged(const void *q, const void *k_new, const void *v_new, int dtype,
+                                      int64_t q_heads, int64_t n_seq, trocm_kv_cache *const *k_caches,
+                                      trocm_kv_cache *const *v_caches, void *out, float scale,
+                                      void *workspace, size_t workspace_bytes, void *stream);
+
 #if defined(__GNUC__)
 #pragma GCC visibility pop
 #endif

@@ -330,3 +330,69 @@ def test_chunked_prefill_into_cache_cfg3_reduced(rt):
     c = 5
     one = orc.flash_sdpa(q[:, :, c * S:(c + 1) * S], k[:, :, :(c + 1) * S], v[:, :, :(c + 1) * S], causal=True, threads=8)
     assert max_abs(outs[c], one) <= 2e-2
+
+
+@pytest.mark.parametrize("dt,Hq,Hkv,D", [(np.float16, 32, 8, 128), (np.float32, 8, 8, 64), (np.float16, 6, 2, 128)])
+def test_fused_step_appends_in_the_attention_launch(rt, dt, Hq, Hkv, D):
+    """InPlaceKvSdpaState::eval as ONE call per step: the new token is read from the inputs and
+    stored into the cache by the decode kernel.  Cache bytes must stay identical to concat and
+    the output must match the oracle, across tile boundaries and across a capacity doubling."""
+    rng = np.random.default_rng(2024)
+    B, T0 = 2, 29
+    k = rng.standard_normal((B, Hkv, T0, D), dtype=np.float32).astype(dt)
+    v = rng.standard_normal((B, Hkv, T0, D), dtype=np.float32).astype(dt)
+    st = tract_amd.InPlaceKvSdpa(axis=2, causal=True).state()
+    st.k.push(k), st.v.push(v)
+    kc, vc = k, v
+    for step in range(40):  # 29 -> 69 tokens: crosses tiles of 32 and the 29 -> 58 -> 116 doublings
+        q = (rng.standard_normal((B, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(dt)
+        kn = rng.standard_normal((B, Hkv, 1, D), dtype=np.float32).astype(dt)
+        vn = rng.standard_normal((B, Hkv, 1, D), dtype=np.float32).astype(dt)
+        out = st.eval([q, kn, vn]).to_numpy()
+        kc, vc = orc.concat_append(kc, kn, 2), orc.concat_append(vc, vn, 2)
+        assert st.k.len() == kc.shape[2] == st.v.len()
+        assert max_abs(out, orc.flash_sdpa(q, kc, vc, causal=True)) <= TOL[np.dtype(dt)], f"step {step}"
+        if step % 7 == 0 or step == 39:
+            assert st.k.valid_contiguous().tobytes() == kc.tobytes()
+            assert st.v.valid_contiguous().tobytes() == vc.tobytes()
+    assert st.k.capacity() == 116 and st.k.reallocs() == 2
+
+
+def test_fused_ragged_step(rt):
+    rng = np.random.default_rng(4242)
+    Hq, Hkv, D, n_seq = 32, 8, 128, 9
+    lens = [1, 31, 32, 33, 63, 64, 500, 1000, 2047]
+    pool = tract_amd.KvPool(64 << 20)
+    kcs, vcs, ks, vs = [], [], [], []
+    for n in lens:
+        k = rng.standard_normal((1, Hkv, n, D), dtype=np.float32).astype(np.float16)
+        v = rng.standard_normal((1, Hkv, n, D), dtype=np.float32).astype(np.float16)
+        kc, vc = tract_amd.InPlaceKvCache(2, pool=pool), tract_amd.InPlaceKvCache(2, pool=pool)
+        kc.push(k), vc.push(v)
+        kcs.append(kc), vcs.append(vc), ks.append(k), vs.append(v)
+    ws = tract_amd.Workspace(n_seq, Hq, 1, D)
+    for step in range(3):
+        q = (rng.standard_normal((n_seq, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+        kn = rng.standard_normal((n_seq, Hkv, 1, D), dtype=np.float32).astype(np.float16)
+        vn = rng.standard_normal((n_seq, Hkv, 1, D), dtype=np.float32).astype(np.float16)
+        out = tract_amd.inplace_kv_sdpa_eval_ragged(
+            tract_amd.DeviceTensor.from_numpy(q), tract_amd.DeviceTensor.from_numpy(kn),
+            tract_amd.DeviceTensor.from_numpy(vn), kcs, vcs, workspace=ws).to_numpy()
+        for i in range(n_seq):
+            ks[i] = np.concatenate([ks[i], kn[i:i + 1]], axis=2)
+            vs[i] = np.concatenate([vs[i], vn[i:i + 1]], axis=2)
+            assert kcs[i].len() == ks[i].shape[2]
+            assert max_abs(out[i:i + 1], orc.flash_sdpa(q[i:i + 1], ks[i], vs[i], causal=True)) <= 2e-2
+    for i in range(n_seq):
+        assert kcs[i].valid_contiguous().tobytes() == ks[i].tobytes()
+        assert vcs[i].valid_contiguous().tobytes() == vs[i].tobytes()
+    # quantised caches take the explicit-append route behind the same call
+    qk, qv = tract_amd.InPlaceKvCache(2, storage_format=tract_amd.Q8_0), tract_amd.InPlaceKvCache(2, storage_format=tract_amd.Q8_0)
+    qk.push(ks[6]), qv.push(vs[6])
+    q1 = (rng.standard_normal((1, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    kn = rng.standard_normal((1, Hkv, 1, D), dtype=np.float32).astype(np.float16)
+    out = tract_amd.inplace_kv_sdpa_eval_ragged(tract_amd.DeviceTensor.from_numpy(q1), tract_amd.DeviceTensor.from_numpy(kn),
+                                                tract_amd.DeviceTensor.from_numpy(kn), [qk], [qv]).to_numpy()
+    kd = orc.dequant(orc.FMT_Q8_0, orc.quant(orc.FMT_Q8_0, np.concatenate([ks[6], kn], axis=2)), np.float16)
+    vd = orc.dequant(orc.FMT_Q8_0, orc.quant(orc.FMT_Q8_0, np.concatenate([vs[6], kn], axis=2)), np.float16)
+    assert qk.len() == ks[6].shape[2] + 1 and max_abs(out, orc.flash_sdpa(q1, kd, vd, causal=True)) <= 2e-2

@@ -67,6 +67,8 @@ SIGNATURES = {
                    _vp, _sz, _vp],
     "trocm_sdpa_cached": [_vp, _i, _i64, _i64, _vp, _vp, _vp, _f, _i, _vp, _sz, _vp],
     "trocm_inplace_kv_sdpa_eval": [_vp, _vp, _vp, _i, _i64, _i64, _pi64, _vp, _vp, _vp, _f, _i, _vp, _sz, _vp],
+    "trocm_inplace_kv_sdpa_eval_ragged": [_vp, _vp, _vp, _i, _i64, _i64, C.POINTER(_vp), C.POINTER(_vp), _vp, _f, _vp,
+                                          _sz, _vp],
     "trocm_sdpa_decode_ragged": [_vp, _i, _i64, _i64, C.POINTER(_vp), C.POINTER(_vp), _vp, _f, _vp, _sz, _vp],
 }
 _RESTYPES = {"trocm_last_error": C.c_char_p}

@@ -769,23 +769,65 @@ int trocm_sdpa_cached(const void *q, int q_dtype, int64_t q_heads, int64_t q_len
     return dispatch_sdpa(a, s);
 }
 
+// Shared argument block of an attention call over two caches.
+static void cached_args(SdpaArgs &a, const void *q, int q_dtype, int64_t q_heads, int64_t q_len,
+                        const trocm_kv_cache *kc, const trocm_kv_cache *vc, int64_t kv_len, void *out, float scale,
+                        int causal, void *workspace, size_t workspace_bytes) {
+    memset(&a, 0, sizeof(a));
+    a.q = q, a.out = out, a.q_dtype = q_dtype, a.kv_fmt = kc->fmt;
+    a.k = kc->data, a.v = vc->data, a.k_scales = kc->scales, a.v_scales = vc->scales;
+    a.B = kc->B, a.Hq = q_heads, a.Hkv = kc->H, a.Sq = q_len, a.Sk = kv_len, a.D = kc->D;
+    a.kv_stride_t = kc->D, a.kv_stride_h = kc->cap * kc->D, a.kv_stride_b = kc->H * kc->cap * kc->D;
+    a.mask_b = a.mask_h = 1;
+    a.scale = isnan(scale) ? 1.0f / sqrtf((float)kc->D) : scale;
+    a.causal = causal;
+    a.workspace = workspace, a.workspace_bytes = workspace_bytes;
+}
+
 int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_new, int dtype, int64_t q_heads,
                                int64_t n_new, const int64_t *kv_new_strides, trocm_kv_cache *kc, trocm_kv_cache *vc,
                                void *out, float scale, int causal, void *workspace, size_t workspace_bytes,
                                void *stream) {
     TROCM_NOT_NULL(kc);
+    TROCM_NOT_NULL(vc);
     int64_t dense[4];
-    if (!kv_new_strides) {
-        dense[3] = 1, dense[2] = kc->D, dense[1] = n_new * kc->D, dense[0] = kc->H * n_new * kc->D;
+    dense[3] = 1, dense[2] = kc->D, dense[1] = n_new * kc->D, dense[0] = kc->H * n_new * kc->D;
+    bool is_dense = kv_new_strides == nullptr;
+    if (!is_dense) {
+        is_dense = true;
+        for (int i = 0; i < 4; i++) is_dense = is_dense && kv_new_strides[i] == dense[i];
+    } else {
         kv_new_strides = dense;
+    }
+    // Decode step on a plain-format cache: the attention kernel reads the new token from the
+    // inputs and stores it into the cache itself -- one launch instead of append + attention.
+    if (n_new == 1 && is_dense && !is_quant(kc->fmt) && dtype == kc->fmt && q && k_new && v_new && out &&
+        kc->fmt == vc->fmt && kc->B == vc->B && kc->H == vc->H && kc->D == vc->D && kc->len == vc->len &&
+        q_heads % kc->H == 0) {
+        hipStream_t s;
+        if (resolve_stream(stream, &s)) return 1;
+        if (append_prepare(kc, k_new, dtype, kv_new_strides, 1, s)) return 1;
+        if (append_prepare(vc, v_new, dtype, kv_new_strides, 1, s)) return 1;
+        if (kc->cap == vc->cap) {
+            SdpaArgs a;
+            cached_args(a, q, dtype, q_heads, 1, kc, vc, kc->len + 1, out, scale, causal, workspace, workspace_bytes);
+            a.k_new = k_new, a.v_new = v_new;
+            int rc = launch_sdpa_decode(a, s);
+            if (rc == 0) {
+                kc->len += 1;
+                vc->len += 1;
+                return 0;
+            }
+            if (rc != 2) return rc;
+        }
     }
     if (trocm_kv_append_pair(kc, vc, k_new, v_new, dtype, kv_new_strides, n_new, stream)) return 1;
     return trocm_sdpa_cached(q, dtype, q_heads, n_new, kc, vc, out, scale, causal, workspace, workspace_bytes, stream);
 }
 
-int trocm_sdpa_decode_ragged(const void *q, int q_dtype, int64_t q_heads, int64_t n_seq,
-                             trocm_kv_cache *const *k_caches, trocm_kv_cache *const *v_caches, void *out, float scale,
-                             void *workspace, size_t workspace_bytes, void *stream) {
+static int ragged_common(const void *q, const void *k_new, const void *v_new, int q_dtype, int64_t q_heads,
+                         int64_t n_seq, trocm_kv_cache *const *k_caches, trocm_kv_cache *const *v_caches, void *out,
+                         float scale, void *workspace, size_t workspace_bytes, void *stream) {
     TROCM_NOT_NULL(q);
     TROCM_NOT_NULL(k_caches);
     TROCM_NOT_NULL(v_caches);
@@ -793,28 +835,82 @@ int trocm_sdpa_decode_ragged(const void *q, int q_dtype, int64_t q_heads, int64_
     TROCM_REQUIRE(n_seq >= 1, "ragged decode: n_seq must be >= 1");
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
+    const bool fused = k_new != nullptr;
+    if (fused) TROCM_NOT_NULL(v_new);
     std::vector<RaggedSeq> seqs((size_t)n_seq);
-    const trocm_kv_cache *k0 = k_caches[0];
+    trocm_kv_cache *k0 = k_caches[0];
     TROCM_NOT_NULL(k0);
     for (int64_t i = 0; i < n_seq; i++) {
-        const trocm_kv_cache *kc = k_caches[i], *vc = v_caches[i];
+        trocm_kv_cache *kc = k_caches[i], *vc = v_caches[i];
         TROCM_NOT_NULL(kc);
         TROCM_NOT_NULL(vc);
         TROCM_REQUIRE(kc->B == 1 && vc->B == 1, "ragged decode: every per-sequence cache must have batch == 1");
         TROCM_REQUIRE(kc->fmt == k0->fmt && vc->fmt == k0->fmt && kc->H == k0->H && vc->H == k0->H && kc->D == k0->D &&
                           vc->D == k0->D,
                       "ragged decode: caches differ in format or shape (sequence %lld)", (long long)i);
-        TROCM_REQUIRE(kc->len == vc->len && kc->cap == vc->cap, "K/V lengths must match (sequence %lld)", (long long)i);
-        TROCM_REQUIRE(kc->len > 0, "empty kv-cache (sequence %lld)", (long long)i);
-        seqs[(size_t)i] = RaggedSeq{kc->data, vc->data, kc->scales, vc->scales, kc->len, kc->cap};
+        TROCM_REQUIRE(kc->len == vc->len, "K/V lengths must match (sequence %lld)", (long long)i);
     }
     TROCM_REQUIRE(q_heads % k0->H == 0, "Q heads (%lld) must be a multiple of K/V heads (%lld)", (long long)q_heads,
                   (long long)k0->H);
     TROCM_REQUIRE(is_quant(k0->fmt) || k0->fmt == q_dtype, "q dtype %d does not match the cache format %d", q_dtype,
                   k0->fmt);
+    const int64_t row_elems = k0->H * k0->D;  // one sequence's new token, all kv heads
+    const size_t es = elem_bytes(q_dtype);
+    int64_t dense[4] = {row_elems, k0->D, k0->D, 1};
+    bool in_kernel = fused && !is_quant(k0->fmt);
+    if (fused) {  // growth first (may reallocate), for every sequence
+        for (int64_t i = 0; i < n_seq; i++) {
+            const char *kn = (const char *)k_new + (size_t)i * row_elems * es, *vn = (const char *)v_new + (size_t)i * row_elems * es;
+            if (append_prepare(k_caches[i], kn, q_dtype, dense, 1, s)) return 1;
+            if (append_prepare(v_caches[i], vn, q_dtype, dense, 1, s)) return 1;
+        }
+    }
     float sc = isnan(scale) ? 1.0f / sqrtf((float)k0->D) : scale;
-    return launch_sdpa_decode_ragged(q, out, q_dtype, k0->fmt, n_seq, q_heads, k0->H, k0->D, seqs.data(), sc, workspace,
-                                     workspace_bytes, s);
+    auto append_explicitly = [&]() -> int {
+        for (int64_t i = 0; i < n_seq; i++) {
+            const char *kn = (const char *)k_new + (size_t)i * row_elems * es, *vn = (const char *)v_new + (size_t)i * row_elems * es;
+            if (append_write(k_caches[i], kn, q_dtype, dense, 1, s)) return 1;
+            if (append_write(v_caches[i], vn, q_dtype, dense, 1, s)) return 1;
+            k_caches[i]->len += 1, v_caches[i]->len += 1;
+        }
+        return 0;
+    };
+    if (fused && !in_kernel && append_explicitly()) return 1;
+    for (;;) {
+        for (int64_t i = 0; i < n_seq; i++) {
+            const trocm_kv_cache *kc = k_caches[i], *vc = v_caches[i];
+            TROCM_REQUIRE(kc->cap == vc->cap, "K/V capacities must match (sequence %lld)", (long long)i);
+            int64_t len = kc->len + (in_kernel ? 1 : 0);
+            TROCM_REQUIRE(len > 0, "empty kv-cache (sequence %lld)", (long long)i);
+            seqs[(size_t)i] = RaggedSeq{kc->data, vc->data, kc->scales, vc->scales, len, kc->cap};
+        }
+        int rc = launch_sdpa_decode_ragged(q, out, q_dtype, k0->fmt, n_seq, q_heads, k0->H, k0->D, seqs.data(), sc,
+                                           workspace, workspace_bytes, in_kernel ? k_new : nullptr,
+                                           in_kernel ? v_new : nullptr, s);
+        if (rc == 0 && in_kernel)
+            for (int64_t i = 0; i < n_seq; i++) k_caches[i]->len += 1, v_caches[i]->len += 1;
+        if (rc != 2) return rc;
+        if (!in_kernel) return fail("ragged decode: no kernel covers this shape");
+        // the kernel cannot append in place for this shape: append explicitly, then attend
+        in_kernel = false;
+        if (append_explicitly()) return 1;
+    }
+}
+
+int trocm_sdpa_decode_ragged(const void *q, int q_dtype, int64_t q_heads, int64_t n_seq,
+                             trocm_kv_cache *const *k_caches, trocm_kv_cache *const *v_caches, void *out, float scale,
+                             void *workspace, size_t workspace_bytes, void *stream) {
+    return ragged_common(q, nullptr, nullptr, q_dtype, q_heads, n_seq, k_caches, v_caches, out, scale, workspace,
+                         workspace_bytes, stream);
+}
+
+int trocm_inplace_kv_sdpa_eval_ragged(const void *q, const void *k_new, const void *v_new, int dtype, int64_t q_heads,
+                                      int64_t n_seq, trocm_kv_cache *const *k_caches, trocm_kv_cache *const *v_caches,
+                                      void *out, float scale, void *workspace, size_t workspace_bytes, void *stream) {
+    TROCM_NOT_NULL(k_new);
+    TROCM_NOT_NULL(v_new);
+    return ragged_common(q, k_new, v_new, dtype, q_heads, n_seq, k_caches, v_caches, out, scale, workspace,
+                         workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -101,6 +101,9 @@ struct SdpaArgs {
     int kv_fmt;             // F32 / F16 / Q8_0 / Q4_0
     const void *k, *v;      // code planes (or plain tensors)
     const void *k_scales, *v_scales;
+    // fused append (split-K decode of plain formats only): the new token's K and V rows, dense
+    // [B, Hkv, 1, D]; they are token Sk-1, read from here and stored into the cache by the kernel
+    const void *k_new, *v_new;
     int64_t B, Hq, Hkv, Sq, Sk, D;
     int64_t kv_stride_b, kv_stride_h, kv_stride_t;       // in ELEMENTS of the logical [.., D] tensor rows
     const void *mask;       // of q_dtype, [mask_b, mask_h, Sq, Sk]
@@ -123,9 +126,11 @@ struct RaggedSeq {
     const void *k, *v, *k_scales, *v_scales;
     int64_t len, cap;
 };
+// k_new/v_new: optional fused append, dense [n_seq, Hkv, 1, D] (then seqs[i].len already counts
+// the new token).  Returns 2 when a fused append was asked for but the fast kernel does not apply.
 int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt, int64_t n_seq, int64_t Hq,
                               int64_t Hkv, int64_t D, const RaggedSeq *seqs, float scale, void *workspace,
-                              size_t workspace_bytes, hipStream_t s);
+                              size_t workspace_bytes, const void *k_new, const void *v_new, hipStream_t s);
 
 // Workspace layout: [counters: kWsCounters ints][partials ...]
 constexpr size_t kWsCounterBytes = 64 * 1024;   // 16384 arrival counters

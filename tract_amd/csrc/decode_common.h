@@ -34,6 +34,8 @@ struct DecodeDev {
     // quantised KV only: f16 scale planes, [B, Hkv, cap, D/32]
     const char *k_scales, *v_scales;
     int64_t sc_stride_b, sc_stride_h;  // bytes
+    // fused append (plain formats): the step's new K/V rows, dense [B or n_seq, Hkv, 1, D]; NULL = none
+    const char *k_new, *v_new;
 };
 
 // Ragged batches: one work item = a tile range of one sequence (device copies of the host plan).

@@ -46,7 +46,8 @@ struct DecodeWork {
     const char *q;      // the G query rows of this kv head
     char *out;          // the G output rows
     const char *kbase, *vbase;
-    int T;              // valid tokens of the sequence
+    const char *k_new, *v_new;  // fused append: the row of token T-1 is read from here and stored to the cache
+    int T;              // valid tokens of the sequence (including a fused new token)
     int tile_begin, tile_end;
     bool direct;        // single split: write the output rows; else store partials at `part`
     int64_t part;       // index of the partial record
@@ -80,6 +81,7 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
 
     const char *kbase = wk.kbase, *vbase = wk.vbase;
     const int seq_T = wk.T;
+    const int cache_T = wk.k_new ? seq_T - 1 : seq_T;  // tokens already stored in the cache
     const int tile_begin = wk.tile_begin, tile_end = wk.tile_end;
     const int last_tok = seq_T - 1;
 
@@ -116,30 +118,38 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
     auto issue_k = [&](int tile) {
         const int t0 = tile * kTile;
         const char *base = kbase + (int64_t)t0 * p.kv_stride_t;
-        if (t0 + kTile <= seq_T) {
+        if (t0 + kTile <= cache_T) {
 #pragma unroll
             for (int j = 0; j < KL; j++) kreg[j] = *reinterpret_cast<const u32x4 *>(base + k_off[j]);
         } else {
+            // the sequence's last tile: rows past the end repeat the last token; a fused new token
+            // comes from the step's input and is written to its place in the cache on the way
 #pragma unroll
             for (int j = 0; j < KL; j++) {
                 int L = j * 64 + lane;
                 int row = min(L / CPR, last_tok - t0), c = L % CPR;
-                kreg[j] = *reinterpret_cast<const u32x4 *>(base + (uint32_t)row * stride_t + (uint32_t)c * 16u);
+                const char *cache_ptr = base + (uint32_t)row * stride_t + (uint32_t)c * 16u;
+                const bool is_new = wk.k_new != nullptr && t0 + row == last_tok;
+                kreg[j] = *reinterpret_cast<const u32x4 *>(is_new ? wk.k_new + c * 16 : cache_ptr);
+                if (is_new && L / CPR == last_tok - t0) *reinterpret_cast<u32x4 *>(const_cast<char *>(cache_ptr)) = kreg[j];
             }
         }
     };
     auto issue_v = [&](int tile) {
         const int t0 = tile * kTile;
         const char *base = vbase + (int64_t)t0 * p.kv_stride_t;
-        if (t0 + kTile <= seq_T) {
+        if (t0 + kTile <= cache_T) {
 #pragma unroll
             for (int i = 0; i < VI; i++) vreg[i] = *reinterpret_cast<const vslice_t *>(base + v_off[i]);
         } else {
 #pragma unroll
             for (int i = 0; i < VI; i++) {
                 int row = min(4 * i + rg, last_tok - t0);
-                vreg[i] = *reinterpret_cast<const vslice_t *>(base + (uint32_t)row * stride_t +
-                                                              (uint32_t)j16 * (uint32_t)sizeof(vslice_t));
+                const char *cache_ptr = base + (uint32_t)row * stride_t + (uint32_t)j16 * (uint32_t)sizeof(vslice_t);
+                const bool is_new = wk.v_new != nullptr && t0 + row == last_tok;
+                vreg[i] = *reinterpret_cast<const vslice_t *>(is_new ? wk.v_new + j16 * (int)sizeof(vslice_t) : cache_ptr);
+                if (is_new && 4 * i + rg == last_tok - t0)
+                    *reinterpret_cast<vslice_t *>(const_cast<char *>(cache_ptr)) = vreg[i];
             }
         }
     };
@@ -284,6 +294,9 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     wk.out = p.out + row;
     wk.kbase = p.k + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
     wk.vbase = p.v + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+    const int64_t new_row = ((int64_t)b * p.Hkv + kvh) * D * (int64_t)sizeof(T);
+    wk.k_new = p.k_new ? p.k_new + new_row : nullptr;
+    wk.v_new = p.v_new ? p.v_new + new_row : nullptr;
     wk.T = p.T;
     const int n_tiles = (p.T + kTile - 1) / kTile;
     wk.tile_begin = split * p.tiles_per_split;
@@ -307,6 +320,9 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     wk.out = p.out + row;
     wk.kbase = it.k + (int64_t)kvh * it.stride_h;
     wk.vbase = it.v + (int64_t)kvh * it.stride_h;
+    const int64_t new_row = ((int64_t)it.seq * p.Hkv + kvh) * D * (int64_t)sizeof(T);
+    wk.k_new = p.k_new ? p.k_new + new_row : nullptr;
+    wk.v_new = p.v_new ? p.v_new + new_row : nullptr;
     wk.T = it.T;
     wk.tile_begin = it.tile_begin;
     wk.tile_end = it.tile_end;
@@ -402,6 +418,7 @@ int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
                       a.workspace_bytes, need);
     }
     DecodeDev p;
+    memset(&p, 0, sizeof(p));
     p.q = (const char *)a.q;
     p.out = (char *)a.out;
     p.k = (const char *)a.k;
@@ -415,7 +432,9 @@ int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
     p.Hq = (int)a.Hq;
     p.Hkv = (int)a.Hkv;
     p.scale_log2 = a.scale * 1.4426950408889634f;
-
+    p.k_new = (const char *)a.k_new;
+    p.v_new = (const char *)a.v_new;
+    if (p.k_new && (p.v_new == nullptr || (uintptr_t)p.k_new % 16 || (uintptr_t)p.v_new % 16)) return 2;
     p.part_ml = (float *)((char *)a.workspace + kWsCounterBytes);
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * G;
     dim3 grid(nsplit, (unsigned)a.Hkv, (unsigned)a.B);
@@ -510,7 +529,7 @@ int ragged_per_sequence(const void *q, void *out, int q_dtype, int kv_fmt, int64
 // head of the workspace, and the kernels index it by blockIdx.
 int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt, int64_t n_seq, int64_t Hq, int64_t Hkv,
                               int64_t D, const RaggedSeq *seqs, float scale, void *workspace, size_t workspace_bytes,
-                              hipStream_t s) {
+                              const void *k_new, const void *v_new, hipStream_t s) {
     const int64_t G = Hq / Hkv;
     const size_t es = elem_bytes(kv_fmt);
     bool fast = (kv_fmt == TROCM_F16 || kv_fmt == TROCM_F32) && q_dtype == kv_fmt && (D == 64 || D == 128) &&
@@ -519,8 +538,11 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     for (int64_t i = 0; i < n_seq && fast; i++)
         fast = (uintptr_t)seqs[i].k % 16 == 0 && (uintptr_t)seqs[i].v % 16 == 0 && seqs[i].len < (1ll << 30) &&
                (seqs[i].cap * D * es) % 16 == 0;
-    if (!fast)
+    if (k_new && ((uintptr_t)k_new % 16 || (uintptr_t)v_new % 16)) fast = false;
+    if (!fast) {
+        if (k_new) return 2;  // the caller appends explicitly, then calls again without a fused append
         return ragged_per_sequence(q, out, q_dtype, kv_fmt, n_seq, Hq, Hkv, D, seqs, scale, workspace, workspace_bytes, s);
+    }
 
     // ---- plan ----------------------------------------------------------------------------------
     int64_t total_tiles = 0;
@@ -586,6 +608,8 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     p.Hq = (int)Hq;
     p.Hkv = (int)Hkv;
     p.scale_log2 = scale * 1.4426950408889634f;
+    p.k_new = (const char *)k_new;
+    p.v_new = (const char *)v_new;
     p.part_ml = (float *)((char *)workspace + kWsCounterBytes);
     p.part_o = p.part_ml + (size_t)n_items * Hkv * 2 * G;
     const RaggedItem *d_items = (const RaggedItem *)workspace;

@@ -452,3 +452,23 @@ def sdpa_decode_ragged(q: DeviceTensor, k_caches, v_caches, scale=None, workspac
     call("trocm_sdpa_decode_ragged", q.ptr, dtype_code(q.dtype), Hq, n, ks, vs, out.ptr, _scale_arg(scale),
          ws.ptr, ws.nbytes, _sh(stream))
     return out
+
+
+def inplace_kv_sdpa_eval_ragged(q: DeviceTensor, k_new: DeviceTensor, v_new: DeviceTensor, k_caches, v_caches,
+                                scale=None, workspace: Workspace | None = None, stream=None,
+                                out: DeviceTensor | None = None) -> DeviceTensor:
+    """One decode step for `n_seq` independent sequences: append k_new[i], v_new[i]
+    ([n_seq, Hkv, 1, D]) to sequence i's caches and attend q[i] ([n_seq, Hq, 1, D]) over them."""
+    n, Hq, _, D = q.shape
+    if len(k_caches) != n or len(v_caches) != n:
+        raise TractRocmError("ragged decode: one K and one V cache per sequence expected")
+    if k_new.shape != v_new.shape or k_new.shape[0] != n or k_new.shape[2] != 1:
+        raise TractRocmError("ragged decode: k_new / v_new must be [n_seq, kv_heads, 1, head_dim]")
+    if out is None:
+        out = DeviceTensor(q.shape, q.dtype)
+    ws = workspace or Workspace(n, Hq, 1, D, stream)
+    ks = (C.c_void_p * n)(*[c.handle for c in k_caches])
+    vs = (C.c_void_p * n)(*[c.handle for c in v_caches])
+    call("trocm_inplace_kv_sdpa_eval_ragged", q.ptr, k_new.ptr, v_new.ptr, dtype_code(q.dtype), Hq, n, ks, vs,
+         out.ptr, _scale_arg(scale), ws.ptr, ws.nbytes, _sh(stream))
+    return out
