@@ -144,6 +144,130 @@ def cpu_baseline(B, budget_s=20.0):
     }
 
 
+def time_calls(ta, fn, iters):
+    """Average microseconds of fn() over `iters` back-to-back calls (HIP events on the stream)."""
+    for _ in range(3):
+        fn()
+    ta.synchronize()
+    e0, e1 = ta.Event(), ta.Event()
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    return ta.Event.elapsed_ms(e0, e1) / iters * 1e3
+
+
+def base_line(args, workload, value, unit, ms_per_step, dtype, roofline, extra):
+    line = {
+        "metric": "decode-attn over KV cache: achieved HBM GB/s (% of peak) + us/token at 8k ctx",
+        "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype, "data": "synthetic", "config": {"workload": workload}, "roofline": roofline,
+    }
+    line.update(extra)
+    return line
+
+
+def run_cfg3(ta, args):
+    """Chunked prefill: 8 chunks of 512 tokens appended to an empty cache, each followed by causal
+    attention of the chunk over the cache so far.  MFMA-bound; value = causal-effective TFLOP/s."""
+    S, C = 512, 8
+    st = ta.InPlaceKvSdpa(axis=2, causal=True).state()
+    per_chunk, tot_us, tot_fl = [], 0.0, 0.0
+    for c in range(1, C + 1):
+        k = seeded_f16(cfg_seed(3, "k") + c, (1, HKV, S, D))
+        v = seeded_f16(cfg_seed(3, "v") + c, (1, HKV, S, D))
+        st.k.push(k), st.v.push(v)
+        q = ta.DeviceTensor.from_numpy((seeded_f16(cfg_seed(3, "q") + c, (1, HQ, S, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16))
+        out = ta.DeviceTensor((1, HQ, S, D), np.float16)
+        us = time_calls(ta, lambda: st.attend(q, out=out), 20)
+        pairs = S * (S * c) - S * (S - 1) // 2
+        fl = 4.0 * HQ * D * pairs
+        per_chunk.append({"kv_len": S * c, "us": round(us, 2), "tflops": round(fl / us / 1e6, 1)})
+        tot_us += us
+        tot_fl += fl
+    tf = tot_fl / tot_us / 1e6
+    roof = {"bound": "mfma", "kernel": "sdpa_prefill_kernel<128,2,2>", "achieved": round(tf, 1), "peak": 2500.0,
+            "unit": "TFLOP/s", "frac": round(tf / 2500.0, 4), "traffic": None}
+    return base_line(args, "cfg3: chunked prefill, 8 x 512 tokens into an empty cache, causal SDPA of each chunk over "
+                     "the cache so far (32q/8kv d=128 f16, batch 1); attention launches only", round(tf, 1), "TFLOP/s",
+                     round(tot_us / C / 1e3, 5), "f16", roof, {"chunks": per_chunk, "total_us": round(tot_us, 1)})
+
+
+def run_cfg4(ta, args):
+    """Block-quantised KV cache, batch 8, contexts 4096 and 16384, decode with fused dequant."""
+    res = {}
+    for name, fmt, ek in (("q8_0", ta.Q8_0, 34 / 32), ("q4_0", ta.Q4_0, 18 / 32), ("f16", None, 2.0)):
+        for T in (4096, 16384):
+            B = 8
+            st = ta.InPlaceKvSdpa(axis=2, causal=True, storage_format=fmt).state()
+            rng = np.random.default_rng(cfg_seed(4, "k"))
+            chan = rng.choice(HKV * D, size=10, replace=False)
+            for b0 in range(0, B, 2):  # build two sequences at a time to bound host memory
+                pass
+            k = seeded_f16(cfg_seed(4, "k") + T, (B, HKV, T, D)).astype(np.float32)
+            kf = k.transpose(0, 2, 1, 3).reshape(B, T, HKV * D)
+            kf[:, :, chan] *= 20.0
+            k = kf.reshape(B, T, HKV, D).transpose(0, 2, 1, 3).astype(np.float16)
+            for c in (st.k, st.v):
+                c.reserve(T + 128, like=(k.shape, k.dtype))
+                c.push(k)
+            q = ta.DeviceTensor.from_numpy((seeded_f16(cfg_seed(4, "q"), (B, HQ, 1, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16))
+            out = ta.DeviceTensor((B, HQ, 1, D), np.float16)
+            us = time_calls(ta, lambda: st.attend(q, out=out), 100)
+            by = 2 * B * HKV * T * D * ek + 2 * B * HQ * D * 2
+            res[f"{name}_ctx{T}"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by)}
+    head = res["q8_0_ctx16384"]
+    roof = {"bound": "hbm", "kernel": "sdpa_decode_q_kernel<Q8_0,4>", "achieved": head["gbs"], "peak": HBM_PEAK_GBS,
+            "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4), "traffic": None}
+    return base_line(args, "cfg4: decode over a Q8_0 / Q4_0 quantised KV cache (fused dequant), batch 8, contexts 4096 "
+                     "and 16384, 1% outlier channels x20; attention launches only; headline = Q8_0 at 16384",
+                     head["gbs"], "GB/s", round(head["us"] / 1e3, 5), "q8_0/f16", roof, {"cases": res})
+
+
+def run_cfg5(ta, args):
+    """Ragged multi-sequence decode: 64 sequences with their own capacity-doubling caches carved
+    from one pool, lengths uniform in [512, 32768]; a step appends one token to every sequence
+    and attends within each sequence's own length (one fused call)."""
+    n_seq = 64
+    rng = np.random.default_rng(cfg_seed(5, "q") + 3)
+    lens = rng.integers(512, 32768, size=n_seq, endpoint=True)
+    pool = ta.KvPool(int(lens.sum()) * HKV * D * 2 * 2 * 3 + (64 << 20))
+    kcs, vcs = [], []
+    for i, n in enumerate(lens):
+        k = seeded_f16(cfg_seed(5, "k") + i, (1, HKV, int(n), D))
+        kc, vc = ta.InPlaceKvCache(2, pool=pool), ta.InPlaceKvCache(2, pool=pool)
+        kc.push(k), vc.push(k)
+        kcs.append(kc), vcs.append(vc)
+    ws = ta.Workspace(n_seq, HQ, 1, D)
+    n = args.steps + args.warmup
+    steps = min(args.steps, 64)
+    n = steps + args.warmup
+    qs = [ta.DeviceTensor.from_numpy((seeded_f16(cfg_seed(5, "q") + i, (n_seq, HQ, 1, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16)) for i in range(n)]
+    kn = [ta.DeviceTensor.from_numpy(seeded_f16(cfg_seed(5, "k") + 1000 + i, (n_seq, HKV, 1, D))) for i in range(n)]
+    out = ta.DeviceTensor((n_seq, HQ, 1, D), np.float16)
+    for i in range(args.warmup):
+        ta.inplace_kv_sdpa_eval_ragged(qs[i], kn[i], kn[i], kcs, vcs, workspace=ws, out=out)
+    ta.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.warmup, n):
+        ta.inplace_kv_sdpa_eval_ragged(qs[i], kn[i], kn[i], kcs, vcs, workspace=ws, out=out)
+    ta.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    tot = int(sum(c.len() for c in kcs))
+    by = 2 * HKV * D * 2 * tot + 2 * n_seq * HQ * D * 2 + 2 * n_seq * HKV * D * 2
+    us_k = time_calls(ta, lambda: ta.sdpa_decode_ragged(qs[0], kcs, vcs, workspace=ws, out=out), 20)
+    roof = {"bound": "hbm", "kernel": "sdpa_decode_ragged_kernel<f16,128,4>", "achieved": round(by / us_k / 1e3, 1),
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(by / us_k / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
+            "kernel_us": round(us_k, 2), "algorithmic_bytes_per_launch": int(by)}
+    st = pool.stats()
+    return base_line(args, f"cfg5: ragged decode, 64 sequences (lengths 512..32768, sum {tot}), per-sequence "
+                     "capacity-doubling caches in one pool, one fused append+attention call per step",
+                     round(by / dt / 1e9, 1), "GB/s", round(dt * 1e3, 5), "f16", roof,
+                     {"steps": steps, "us_per_step": round(dt * 1e6, 1), "pool_bytes": st["bytes_total"],
+                      "pool_in_use": st["bytes_in_use"], "pct_of_hbm_peak": round(100 * by / dt / 1e9 / HBM_PEAK_GBS, 2)})
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -153,6 +277,9 @@ def main():
     ap.add_argument("--other-batches", type=str, default="1,32")
     ap.add_argument("--kernel-iters", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5"],
+                    help="cfg2 (default) is the configuration the metric is quoted on; the others print one line "
+                         "of the same shape for the remaining configurations")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this path is measured on one GPU; --gpus {args.gpus} is not supported "
@@ -161,6 +288,11 @@ def main():
 
     import tract_amd as ta
     rt = ta.runtime_for_name("rocm")
+    if args.workload != "cfg2":
+        line = {"cfg3": run_cfg3, "cfg4": run_cfg4, "cfg5": run_cfg5}[args.workload](ta, args)
+        line["device"] = rt.device_name
+        print(json.dumps(line))
+        return
     main_res = run_batch(ta, args.batch, args.steps, args.warmup, args.kernel_iters)
 
     # parity spot check of the last output against the oracle (checker only)

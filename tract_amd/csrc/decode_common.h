@@ -161,6 +161,6 @@ __global__ __launch_bounds__(kThreads) void sdpa_decode_merge_kernel(DecodeDev p
 
 // Partials: at most kMaxSplitRows rows of (D + 2) floats per query head.
 constexpr int64_t kMaxSplitRows = 8192;
-int choose_decode_splits(int64_t BH, int64_t G, int n_tiles);
+int choose_decode_splits(int64_t BH, int64_t G, int n_tiles, int wg_per_cu);
 
 }  // namespace trocm

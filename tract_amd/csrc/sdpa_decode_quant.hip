@@ -372,7 +372,7 @@ int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s) {
     if ((cap_h * rb) % 16 || (cap_b * rb) % 16) return 2;
 
     int n_tiles = (int)((a.Sk + kTile - 1) / kTile);
-    int nsplit = choose_decode_splits(BH, G, n_tiles);
+    int nsplit = choose_decode_splits(BH, G, n_tiles, 2);
     int tps = (n_tiles + nsplit - 1) / nsplit;
     nsplit = (n_tiles + tps - 1) / tps;
     if (nsplit > 1) {
