@@ -1,0 +1,262 @@
+// tract_rocm.hpp — C++17 host-side mirror of tract's KV-cache operators over the C ABI of
+// tract_rocm.h.  Header-only; names, argument meaning and error behaviour follow the reference
+// operators (the same mirror exists in Python, tract_amd/ops.py):
+//   InPlaceKvCache            transformers/src/ops/inplace_kv_cache.rs:28-114
+//   InPlaceKvSdpa / State     transformers/src/ops/inplace_kv_cache.rs:131-290
+//   Sdpa                      transformers/src/ops/sdpa.rs:83-89, 296-356
+//   runtime_for_name          core/src/runtime.rs:223-250
+// Every failing ABI call becomes a trocm::Error carrying the library's message, the way a
+// TractResult Err carries its context.
+#pragma once
+#include <cmath>
+#include <cstdint>
+#include <memory>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+#include "tract_rocm.h"
+
+namespace trocm {
+
+struct Error : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+inline void check(int rc) {
+    if (rc != 0) throw Error(trocm_last_error());
+}
+
+enum class DatumType { F32 = TROCM_F32, F16 = TROCM_F16 };
+inline size_t size_of(DatumType dt) { return dt == DatumType::F32 ? 4 : 2; }
+
+class Runtime {
+   public:
+    std::string name() const { return "rocm"; }
+    void check() const { trocm::check(trocm_device_sync()); }
+};
+inline Runtime runtime_for_name(const std::string &name, int device = 0) {
+    if (name != "rocm") throw Error("Runtime \"" + name + "\" not found: only \"rocm\" is registered here");
+    check(trocm_init(device));
+    return Runtime();
+}
+
+// A dense device tensor (shape + datum type); move-only owner of its allocation.
+class DeviceTensor {
+   public:
+    DeviceTensor() = default;
+    DeviceTensor(std::vector<int64_t> shape, DatumType dt) : shape_(std::move(shape)), dt_(dt) {
+        check(trocm_malloc(&ptr_, bytes()));
+    }
+    DeviceTensor(const DeviceTensor &) = delete;
+    DeviceTensor &operator=(const DeviceTensor &) = delete;
+    DeviceTensor(DeviceTensor &&o) noexcept { *this = std::move(o); }
+    DeviceTensor &operator=(DeviceTensor &&o) noexcept {
+        std::swap(ptr_, o.ptr_), std::swap(shape_, o.shape_), std::swap(dt_, o.dt_);
+        return *this;
+    }
+    ~DeviceTensor() {
+        if (ptr_) trocm_free(ptr_);
+    }
+    static DeviceTensor from_host(const void *host, std::vector<int64_t> shape, DatumType dt) {
+        DeviceTensor t(std::move(shape), dt);
+        check(trocm_h2d(t.ptr_, host, t.bytes(), nullptr));
+        check(trocm_stream_sync(nullptr));
+        return t;
+    }
+    void to_host(void *host) const {
+        check(trocm_d2h(host, ptr_, bytes(), nullptr));
+        check(trocm_stream_sync(nullptr));
+    }
+    size_t len() const {
+        size_t n = 1;
+        for (auto d : shape_) n *= (size_t)d;
+        return n;
+    }
+    size_t bytes() const { return len() * size_of(dt_); }
+    const std::vector<int64_t> &shape() const { return shape_; }
+    DatumType datum_type() const { return dt_; }
+    void *ptr() const { return ptr_; }
+
+   private:
+    void *ptr_ = nullptr;
+    std::vector<int64_t> shape_;
+    DatumType dt_ = DatumType::F32;
+};
+
+// Geometric-growth in-place cache along the token axis of [B, H, S, D] tensors (axis 2).
+class InPlaceKvCache {
+   public:
+    explicit InPlaceKvCache(size_t axis, std::optional<int> storage_format = std::nullopt)
+        : axis_(axis), fmt_(storage_format) {}
+    InPlaceKvCache(const InPlaceKvCache &) = delete;
+    InPlaceKvCache &operator=(const InPlaceKvCache &) = delete;
+    InPlaceKvCache(InPlaceKvCache &&o) noexcept { *this = std::move(o); }
+    InPlaceKvCache &operator=(InPlaceKvCache &&o) noexcept {
+        std::swap(h_, o.h_), std::swap(axis_, o.axis_), std::swap(fmt_, o.fmt_), std::swap(shape_, o.shape_);
+        return *this;
+    }
+    ~InPlaceKvCache() {
+        if (h_) trocm_kv_cache_destroy(h_);
+    }
+
+    int64_t len() const { return get(trocm_kv_cache_len); }
+    bool is_empty() const { return len() == 0; }
+    int64_t capacity() const { return get(trocm_kv_cache_capacity); }
+    int64_t reallocs() const { return get(trocm_kv_cache_reallocs); }
+
+    // Append `input` along the axis, in place; O(input) amortised.
+    void push(const DeviceTensor &input) {
+        const auto &sh = input.shape();
+        if (sh.size() != 4 || axis_ != 2) throw Error("kv-cache push: [B,H,S,D] tensors with axis 2 are supported");
+        if (sh[2] == 0) return;
+        if (!h_) {
+            int fmt = fmt_.value_or((int)input.datum_type());
+            check(trocm_kv_cache_create(&h_, fmt, sh[0], sh[1], sh[3]));
+            shape_ = sh;
+        } else if (sh[0] != shape_[0] || sh[1] != shape_[1] || sh[3] != shape_[3]) {
+            throw Error("rank mismatch in kv-cache push");
+        }
+        int64_t strides[4] = {sh[1] * sh[2] * sh[3], sh[2] * sh[3], sh[3], 1};
+        check(trocm_kv_append(h_, input.ptr(), (int)input.datum_type(), strides, sh[2], nullptr));
+    }
+    void truncate(int64_t len) {
+        if (!h_) throw Error("Can not truncate a zero-len kv-cache value");
+        check(trocm_kv_cache_truncate(h_, len));
+    }
+    // Dense copy of the valid [0..len] region as raw bytes (canonical block bytes when quantised).
+    std::vector<uint8_t> valid_contiguous() const {
+        if (!h_) throw Error("empty kv-cache");
+        size_t row = 0;
+        check(trocm_kv_row_bytes(h_, &row));
+        size_t n = (size_t)shape_[0] * shape_[1] * (size_t)len() * row;
+        void *dev = nullptr;
+        check(trocm_malloc(&dev, n));
+        std::vector<uint8_t> host(n);
+        int rc = trocm_kv_export(h_, dev, nullptr);
+        if (!rc) rc = trocm_d2h(host.data(), dev, n, nullptr);
+        if (!rc) rc = trocm_stream_sync(nullptr);
+        trocm_free(dev);
+        check(rc);
+        return host;
+    }
+    InPlaceKvCache clone() const {
+        InPlaceKvCache c(axis_, fmt_);
+        if (h_) {
+            check(trocm_kv_cache_clone(h_, &c.h_, nullptr));
+            c.shape_ = shape_;
+        }
+        return c;
+    }
+    trocm_kv_cache *handle() const { return h_; }
+
+   private:
+    int64_t get(int (*fn)(const trocm_kv_cache *, int64_t *)) const {
+        if (!h_) return 0;
+        int64_t v = 0;
+        check(fn(h_, &v));
+        return v;
+    }
+    trocm_kv_cache *h_ = nullptr;
+    size_t axis_ = 2;
+    std::optional<int> fmt_;
+    std::vector<int64_t> shape_;
+};
+
+// Split-K scratch owned by an op state.
+class Workspace {
+   public:
+    Workspace(int64_t batch, int64_t q_heads, int64_t q_len, int64_t head_dim) {
+        check(trocm_sdpa_workspace_bytes(batch, q_heads, q_len, head_dim, &bytes_));
+        check(trocm_malloc(&ptr_, bytes_));
+        check(trocm_sdpa_workspace_init(ptr_, bytes_, nullptr));
+    }
+    Workspace(const Workspace &) = delete;
+    Workspace &operator=(const Workspace &) = delete;
+    ~Workspace() {
+        if (ptr_) trocm_free(ptr_);
+    }
+    void *ptr() const { return ptr_; }
+    size_t bytes() const { return bytes_; }
+
+   private:
+    void *ptr_ = nullptr;
+    size_t bytes_ = 0;
+};
+
+// Scaled dot-product attention on plain device tensors.
+struct Sdpa {
+    std::optional<float> scale;
+    bool is_causal = false;
+    DeviceTensor eval(const DeviceTensor &q, const DeviceTensor &k, const DeviceTensor &v,
+                      const DeviceTensor *mask = nullptr) const {
+        if (is_causal && mask) throw Error("Mask cannot be provided if is_causal=true");
+        const auto &qs = q.shape(), &ks = k.shape();
+        if (qs.size() != 4 || ks.size() != 4 || v.shape() != ks) throw Error("Input tensors must be 4D here");
+        DeviceTensor out(qs, q.datum_type());
+        Workspace ws(qs[0], qs[1], qs[2], qs[3]);
+        check(trocm_sdpa(q.ptr(), k.ptr(), v.ptr(), mask ? mask->ptr() : nullptr, out.ptr(), (int)q.datum_type(), qs[0],
+                         qs[1], ks[1], qs[2], ks[2], qs[3], nullptr, mask ? mask->shape()[0] : 1,
+                         mask ? mask->shape()[1] : 1, scale.value_or(NAN), is_causal, ws.ptr(), ws.bytes(), nullptr));
+        check(trocm_stream_sync(nullptr));
+        return out;
+    }
+};
+
+// Fused in-place KV-cache + attention op: inputs [Q, K_new, V_new], output Q-shaped.
+class InPlaceKvSdpaState {
+   public:
+    InPlaceKvSdpaState(size_t axis, bool causal, std::optional<float> scale, std::optional<int> fmt = std::nullopt)
+        : axis_(axis), causal_(causal), scale_(scale), fmt_(fmt), k(axis, fmt), v(axis, fmt) {}
+
+    DeviceTensor eval(const DeviceTensor &q, const DeviceTensor &k_new, const DeviceTensor &v_new) {
+        k.push(k_new);
+        v.push(v_new);
+        const auto &qs = q.shape();
+        if (!ws_) ws_ = std::make_unique<Workspace>(qs[0], qs[1], qs[2], qs[3]);
+        DeviceTensor out(qs, q.datum_type());
+        check(trocm_sdpa_cached(q.ptr(), (int)q.datum_type(), qs[1], qs[2], k.handle(), v.handle(), out.ptr(),
+                                scale_.value_or(NAN), causal_, ws_->ptr(), ws_->bytes(), nullptr));
+        return out;
+    }
+    // [K_valid, V_valid] as raw bytes; empty when nothing was pushed.
+    void save_to(std::vector<std::vector<uint8_t>> &states) const {
+        if (!k.is_empty()) {
+            states.push_back(k.valid_contiguous());
+            states.push_back(v.valid_contiguous());
+        }
+    }
+    void load_from(const DeviceTensor &k_state, const DeviceTensor &v_state) {
+        k = InPlaceKvCache(axis_, fmt_);
+        v = InPlaceKvCache(axis_, fmt_);
+        k.push(k_state);
+        v.push(v_state);
+    }
+    InPlaceKvSdpaState freeze() const {
+        InPlaceKvSdpaState f(axis_, causal_, scale_, fmt_);
+        f.k = k.clone();
+        f.v = v.clone();
+        return f;
+    }
+
+   private:
+    size_t axis_;
+    bool causal_;
+    std::optional<float> scale_;
+    std::optional<int> fmt_;
+    std::unique_ptr<Workspace> ws_;
+
+   public:
+    InPlaceKvCache k, v;
+};
+
+struct InPlaceKvSdpa {
+    size_t axis = 2;
+    bool causal = true;
+    std::optional<float> scale;
+    std::string name() const { return "InPlaceKvSdpa"; }
+    bool is_stateless() const { return false; }
+    InPlaceKvSdpaState state() const { return InPlaceKvSdpaState(axis, causal, scale); }
+};
+
+}  // namespace trocm

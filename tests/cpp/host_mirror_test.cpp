@@ -1,0 +1,178 @@
+// C++ twin of tract's unit tests for the in-place KV cache and the fused op
+// (transformers/src/ops/inplace_kv_cache.rs:366-418, 456-491, 595-658, 898-942), run against
+// the rocm library through the C++ host mirror.  References are written in the test, as the
+// reference's own tests do: plain concatenation and naive f32 attention.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+#include "tract_rocm.hpp"
+
+using namespace trocm;
+
+#define EXPECT(cond)                                                          \
+    do {                                                                      \
+        if (!(cond)) {                                                        \
+            std::fprintf(stderr, "FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); \
+            return 1;                                                         \
+        }                                                                     \
+    } while (0)
+
+// deterministic filler (seq_tensor of the reference tests)
+static std::vector<float> seq_tensor(size_t n, float start) {
+    std::vector<float> v(n);
+    for (size_t i = 0; i < n; i++) v[i] = start + 0.001f * (float)(i % 977) - 0.3f * (float)(i % 7);
+    return v;
+}
+
+// naive GQA attention over [B,H,S,D] f32, causal bottom-right aligned
+static std::vector<float> naive(const std::vector<float> &q, const std::vector<float> &k, const std::vector<float> &v,
+                                int B, int Hq, int Hkv, int Sq, int Sk, int D, bool causal) {
+    std::vector<float> out((size_t)B * Hq * Sq * D);
+    const float scale = 1.0f / std::sqrt((float)D);
+    std::vector<float> s(Sk);
+    for (int b = 0; b < B; b++)
+        for (int h = 0; h < Hq; h++) {
+            int kh = h / (Hq / Hkv);
+            for (int i = 0; i < Sq; i++) {
+                float mx = -INFINITY;
+                int vis = causal ? std::min(Sk, i + (Sk - Sq) + 1) : Sk;
+                for (int j = 0; j < vis; j++) {
+                    float a = 0;
+                    for (int d = 0; d < D; d++) a += q[(((size_t)b * Hq + h) * Sq + i) * D + d] * k[(((size_t)b * Hkv + kh) * Sk + j) * D + d];
+                    s[j] = a * scale;
+                    mx = std::fmax(mx, s[j]);
+                }
+                float sum = 0;
+                for (int j = 0; j < vis; j++) sum += (s[j] = std::exp(s[j] - mx));
+                for (int d = 0; d < D; d++) {
+                    float a = 0;
+                    for (int j = 0; j < vis; j++) a += s[j] * v[(((size_t)b * Hkv + kh) * Sk + j) * D + d];
+                    out[(((size_t)b * Hq + h) * Sq + i) * D + d] = a / sum;
+                }
+            }
+        }
+    return out;
+}
+
+// concat along axis 2 of [B,H,*,D]
+static void concat(std::vector<float> &acc, int &len, const std::vector<float> &x, int B, int H, int n, int D) {
+    std::vector<float> out((size_t)B * H * (len + n) * D);
+    for (int bh = 0; bh < B * H; bh++) {
+        std::memcpy(&out[(size_t)bh * (len + n) * D], acc.data() + (size_t)bh * len * D, sizeof(float) * len * D);
+        std::memcpy(&out[((size_t)bh * (len + n) + len) * D], x.data() + (size_t)bh * n * D, sizeof(float) * n * D);
+    }
+    acc.swap(out);
+    len += n;
+}
+
+int main() {
+    try {
+        Runtime rt = runtime_for_name("rocm");
+        rt.check();
+        bool threw = false;
+        try {
+            runtime_for_name("cuda");
+        } catch (const Error &) {
+            threw = true;
+        }
+        EXPECT(threw);
+
+        // inplace_matches_concat + realloc count (inplace_kv_cache.rs:366-418)
+        {
+            const int B = 1, H = 4, D = 16;
+            InPlaceKvCache c(2);
+            std::vector<float> ref;
+            int len = 0;
+            for (int step = 0; step < 1024; step++) {
+                auto x = seq_tensor((size_t)B * H * D, (float)step);
+                c.push(DeviceTensor::from_host(x.data(), {B, H, 1, D}, DatumType::F32));
+                if (step < 70 || step == 1023) concat(ref, len, x, B, H, 1, D);
+            }
+            EXPECT(c.len() == 1024 && c.capacity() == 1024 && c.reallocs() <= 12);
+            InPlaceKvCache c2(2);
+            std::vector<float> ref2;
+            int len2 = 0;
+            int chunks[] = {3, 1, 7, 1, 30, 2};
+            for (int n : chunks) {
+                auto x = seq_tensor((size_t)B * H * n * D, (float)n);
+                c2.push(DeviceTensor::from_host(x.data(), {B, H, n, D}, DatumType::F32));
+                concat(ref2, len2, x, B, H, n, D);
+                auto got = c2.valid_contiguous();
+                EXPECT(got.size() == ref2.size() * 4 && std::memcmp(got.data(), ref2.data(), got.size()) == 0);
+            }
+            EXPECT(c2.len() == 44 && c2.capacity() == 84);  // 3 -> 6 -> 12 -> 42 -> 84
+            // truncate + clone (dyn_kv_cache.rs:112-119, :262-272)
+            InPlaceKvCache frozen = c2.clone();
+            c2.truncate(10);
+            EXPECT(c2.len() == 10 && frozen.len() == 44);
+            bool bad = false;
+            try {
+                c2.truncate(11);
+            } catch (const Error &) {
+                bad = true;
+            }
+            EXPECT(bad);
+        }
+
+        // fused op vs {concat, naive attention}, GQA + causal, decode loop (inplace_kv_cache.rs:595-658)
+        {
+            const int B = 2, Hq = 8, Hkv = 2, D = 64;
+            InPlaceKvSdpaState st = InPlaceKvSdpa{2, true, std::nullopt}.state();
+            std::vector<float> kc, vc;
+            int klen = 0, vlen = 0;
+            double worst = 0;
+            int lens[] = {40, 1, 1, 1, 5, 1};
+            for (int n : lens) {
+                auto q = seq_tensor((size_t)B * Hq * n * D, 0.1f * n), k = seq_tensor((size_t)B * Hkv * n * D, 0.2f * n),
+                     v = seq_tensor((size_t)B * Hkv * n * D, 0.3f * n);
+                for (auto &x : q) x *= 0.05f;
+                for (auto &x : k) x *= 0.1f;
+                DeviceTensor out = st.eval(DeviceTensor::from_host(q.data(), {B, Hq, n, D}, DatumType::F32),
+                                           DeviceTensor::from_host(k.data(), {B, Hkv, n, D}, DatumType::F32),
+                                           DeviceTensor::from_host(v.data(), {B, Hkv, n, D}, DatumType::F32));
+                concat(kc, klen, k, B, Hkv, n, D);
+                concat(vc, vlen, v, B, Hkv, n, D);
+                std::vector<float> got(out.len());
+                out.to_host(got.data());
+                auto want = naive(q, kc, vc, B, Hq, Hkv, n, klen, D, true);
+                for (size_t i = 0; i < got.size(); i++) worst = std::fmax(worst, std::fabs((double)got[i] - want[i]));
+            }
+            EXPECT(worst < 1e-3);
+            // save / load resume is exact (inplace_kv_cache.rs:898-942)
+            std::vector<std::vector<uint8_t>> saved;
+            st.save_to(saved);
+            EXPECT(saved.size() == 2 && saved[0].size() == kc.size() * 4);
+            EXPECT(std::memcmp(saved[0].data(), kc.data(), saved[0].size()) == 0);
+            EXPECT(std::memcmp(saved[1].data(), vc.data(), saved[1].size()) == 0);
+            InPlaceKvSdpaState st2 = InPlaceKvSdpa{2, true, std::nullopt}.state();
+            st2.load_from(DeviceTensor::from_host(saved[0].data(), {B, Hkv, klen, D}, DatumType::F32),
+                          DeviceTensor::from_host(saved[1].data(), {B, Hkv, klen, D}, DatumType::F32));
+            EXPECT(st2.k.len() == klen && st2.k.valid_contiguous() == saved[0]);
+        }
+
+        // Sdpa: mask rejected when causal (sdpa.rs:297-299)
+        {
+            auto x = seq_tensor(2 * 4 * 8, 0.f);
+            DeviceTensor t = DeviceTensor::from_host(x.data(), {1, 2, 4, 8}, DatumType::F32);
+            Sdpa op{std::nullopt, true};
+            bool bad = false;
+            try {
+                op.eval(t, t, t, &t);
+            } catch (const Error &e) {
+                bad = std::string(e.what()).find("Mask cannot be provided") != std::string::npos;
+            }
+            EXPECT(bad);
+            Sdpa nc{1.3f, false};
+            DeviceTensor o = nc.eval(t, t, t);
+            std::vector<float> got(o.len());
+            o.to_host(got.data());
+            EXPECT(std::isfinite(got[0]));
+        }
+        std::printf("host_mirror_test: all checks passed\n");
+        return 0;
+    } catch (const std::exception &e) {
+        std::fprintf(stderr, "host_mirror_test: exception: %s\n", e.what());
+        return 2;
+    }
+}
