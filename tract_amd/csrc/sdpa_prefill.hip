@@ -11,11 +11,16 @@
 // one exchange between the two half-waves, and the rescaling factors of the online softmax
 // apply to the lane's own O^T registers.
 //
-// A wave owns 32 queries and, per workgroup tile, 64 keys.  The 4 waves of a workgroup are
+// A wave owns 32 queries and, per workgroup tile, 64 keys.  The waves of a workgroup are
 // arranged WM x WN: WM query groups (BLOCK_M = 32*WM) times WN key slices (BLOCK_N = 64*WN);
 // waves that share queries keep separate online-softmax states and are merged through LDS at
-// the end.  4x1 suits long query chunks, 2x2 keeps all four SIMDs busy when there are few
-// query tiles.
+// the end.  Eight waves per workgroup put two waves on every SIMD; because the two barriers per
+// tile keep them in the same phase this gains only about 5 % over four waves (307 -> 321 TFLOP/s
+// on 8 x 512-token chunks).  2x4 (64 queries per workgroup) keeps every compute unit busy when
+// there are few query tiles, 4x2 (128 queries) halves the K/V staging per query when there are
+// many.  HG query heads of one KV head can
+// share a workgroup (the WM waves are split HG ways): the K/V tile staged into LDS then feeds
+// HG times more MFMA work, which is what GQA allows and what bounds small-batch prefill.
 //
 // K and V tiles: global -> registers (prefetched one tile ahead) -> LDS, both row-major with
 // padded rows, written with 128-bit stores.  K fragments are plain 128-bit LDS reads.  For V
@@ -42,7 +47,6 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef short short4_t __attribute__((ext_vector_type(4)));
 
-constexpr int kThreads = 256;
 
 struct PrefillDev {
     const _Float16 *q;
@@ -64,18 +68,23 @@ __device__ __forceinline__ half4_t lds_read_tr16(const _Float16 *lds_ptr) {
     return __builtin_bit_cast(half4_t, r);
 }
 
-template <int D, int WM, int WN>
-__global__ __launch_bounds__(kThreads, 1) void sdpa_prefill_kernel(PrefillDev p) {
-    constexpr int BLOCK_M = 32 * WM, BLOCK_N = 64 * WN;
+template <int D, int WM, int WN, int HG>
+__global__ __launch_bounds__(64 * WM * WN) void sdpa_prefill_kernel(PrefillDev p) {
+    constexpr int kThreads = 64 * WM * WN;
+    constexpr int QB = WM / HG;           // 32-query blocks per workgroup
+    constexpr int BLOCK_M = 32 * QB, BLOCK_N = 64 * WN;
+    static_assert(WM % HG == 0, "waves split evenly over the heads of a workgroup");
     constexpr int KS = D / 16;            // contraction steps of Q K^T
     constexpr int DB = D / 32;            // 32-feature blocks of the output
     constexpr int KROW = D + 8;           // halfs per K row in LDS: 128-bit reads of 16 rows hit 64 distinct banks
     constexpr int VROW = D + 16;          // halfs per V row in LDS: the 4 rows of a transposing read sit 8 banks apart
     constexpr int NL = BLOCK_N * D / 8 / kThreads;  // 128-bit loads per thread per tile and tensor
-    static_assert(WM * WN == 4, "four waves per workgroup");
+    static_assert(WM * WN == 4 || WM * WN == 8, "four or eight waves per workgroup");
+    static_assert(NL >= 1 && NL * 8 * kThreads == BLOCK_N * D, "tile loads must divide evenly");
 
-    __shared__ __attribute__((aligned(16))) _Float16 lds_k[BLOCK_N * KROW];
-    __shared__ __attribute__((aligned(16))) _Float16 lds_v[BLOCK_N * VROW];
+    __shared__ __attribute__((aligned(16))) _Float16 lds_all[BLOCK_N * (KROW + VROW)];
+    _Float16 *lds_k = lds_all;
+    _Float16 *lds_v = lds_all + BLOCK_N * KROW;
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int hb = lane >> 5, l32 = lane & 31;
@@ -87,14 +96,14 @@ __global__ __launch_bounds__(kThreads, 1) void sdpa_prefill_kernel(PrefillDev p)
     const int kvh = id % p.Hkv;
     id /= p.Hkv;
     const int G = p.Hq / p.Hkv;
-    const int g = id % G;
-    id /= G;
+    const int gg = id % (G / HG);         // group of HG query heads of this kv head
+    id /= (G / HG);
     const int qt = p.n_qtiles - 1 - (id % p.n_qtiles);
     const int b = id / p.n_qtiles;
-    const int qh = kvh * G + g;
+    const int qh = kvh * G + gg * HG + (wm % HG);
 
     const int off = p.Sk - p.Sq;          // query i sees keys j <= i + off when causal
-    const int q0 = qt * BLOCK_M + 32 * wm;  // first query of this wave
+    const int q0 = qt * BLOCK_M + 32 * (wm / HG);  // first query of this wave
     const int my_q = q0 + l32;
     const _Float16 *qrow = p.q + (((int64_t)b * p.Hq + qh) * p.Sq + min(my_q, p.Sq - 1)) * D;
     const _Float16 *kbase = p.k + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
@@ -219,11 +228,11 @@ __global__ __launch_bounds__(kThreads, 1) void sdpa_prefill_kernel(PrefillDev p)
     l_run += __shfl_xor(l_run, 32, 64);
     if constexpr (WN > 1) {
         __syncthreads();  // the tiles are dead: reuse their space
-        float *xo = reinterpret_cast<float *>(lds_k);  // [WM][64 lanes][DB*16] + m, l
+        float *xo = reinterpret_cast<float *>(lds_all);  // [WN-1][WM][64 lanes][DB*16 + 2]
         constexpr int kPer = DB * 16 + 2;
-        static_assert(sizeof(float) * WM * 64 * kPer <= sizeof(_Float16) * (BLOCK_N * KROW), "merge buffer");
-        float *mine = xo + ((size_t)wm * 64 + lane) * kPer;
-        if (wn == 1) {
+        static_assert(sizeof(float) * (WN - 1) * WM * 64 * kPer <= sizeof(_Float16) * BLOCK_N * (KROW + VROW), "merge buffer");
+        if (wn > 0) {
+            float *mine = xo + (((size_t)(wn - 1) * WM + wm) * 64 + lane) * kPer;
 #pragma unroll
             for (int db = 0; db < DB; db++)
 #pragma unroll
@@ -232,16 +241,21 @@ __global__ __launch_bounds__(kThreads, 1) void sdpa_prefill_kernel(PrefillDev p)
             mine[DB * 16 + 1] = l_run;
         }
         __syncthreads();
-        if (wn == 1) return;
-        const float m_o = mine[DB * 16], l_o = mine[DB * 16 + 1];
-        const float mm = fmaxf(m_run, m_o);
-        const float m_ref = (mm == -INFINITY) ? 0.0f : mm;
-        const float fa = fast_exp2(m_run - m_ref), fb = fast_exp2(m_o - m_ref);
-        l_run = l_run * fa + l_o * fb;
+        if (wn > 0) return;
 #pragma unroll
-        for (int db = 0; db < DB; db++)
+        for (int other = 1; other < WN; other++) {
+            const float *theirs = xo + (((size_t)(other - 1) * WM + wm) * 64 + lane) * kPer;
+            const float m_o = theirs[DB * 16], l_o = theirs[DB * 16 + 1];
+            const float mm = fmaxf(m_run, m_o);
+            const float m_ref = (mm == -INFINITY) ? 0.0f : mm;
+            const float fa = fast_exp2(m_run - m_ref), fb = fast_exp2(m_o - m_ref);
+            l_run = l_run * fa + l_o * fb;
+            m_run = mm;
 #pragma unroll
-            for (int r = 0; r < 16; r++) o[db][r] = o[db][r] * fa + mine[db * 16 + r] * fb;
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[db][r] = o[db][r] * fa + theirs[db * 16 + r] * fb;
+        }
     }
     if (my_q >= p.Sq) return;
     const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
@@ -257,14 +271,15 @@ __global__ __launch_bounds__(kThreads, 1) void sdpa_prefill_kernel(PrefillDev p)
         }
 }
 
-template <int D, int WM, int WN>
+template <int D, int WM, int WN, int HG>
 int launch_cfg(const PrefillDev &p0, hipStream_t s) {
     PrefillDev p = p0;
-    constexpr int BLOCK_M = 32 * WM;
+    constexpr int BLOCK_M = 32 * WM / HG;
+    if ((p.Hq / p.Hkv) % HG) return 2;
     p.n_qtiles = (p.Sq + BLOCK_M - 1) / BLOCK_M;
-    int64_t wgs = (int64_t)p.B * p.Hq * p.n_qtiles;
+    int64_t wgs = (int64_t)p.B * (p.Hq / HG) * p.n_qtiles;
     if (wgs >= (1ll << 31)) return 2;
-    hipLaunchKernelGGL((sdpa_prefill_kernel<D, WM, WN>), dim3((unsigned)wgs), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((sdpa_prefill_kernel<D, WM, WN, HG>), dim3((unsigned)wgs), dim3(64 * WM * WN), 0, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("sdpa_prefill launch failed: %s", hipGetErrorString(e));
     return 0;
@@ -290,17 +305,36 @@ int launch_sdpa_prefill(const SdpaArgs &a, hipStream_t s) {
     p.B = (int)a.B, p.Hq = (int)a.Hq, p.Hkv = (int)a.Hkv, p.Sq = (int)a.Sq, p.Sk = (int)a.Sk;
     p.causal = a.causal;
     p.scale_log2 = a.scale * 1.4426950408889634f;
-    // 4x1 (128 queries per workgroup) when that still gives every compute unit a workgroup,
-    // else 2x2 (64 queries, keys split over two wave pairs)
+    // Shapes, named WM WN HG: 4 2 1 = 128 queries of one head; 2 4 1 = 64 queries, keys split four
+    // ways; 4 2 4 = 32 queries of each of 4 heads of a kv head; 8 1 4 = 64 queries x 4 heads.
+    // TROCM_PREFILL_SHAPE=<WM><WN><HG> forces one (experiments).
     static int forced = -1;
     if (forced < 0) {
-        const char *e = getenv("TROCM_PREFILL_SHAPE");  // experiment knob: 41 or 22
+        const char *e = getenv("TROCM_PREFILL_SHAPE");
         forced = e ? atoi(e) : 0;
     }
-    int64_t wgs_41 = a.B * a.Hq * ((a.Sq + 127) / 128);
-    bool use41 = forced ? forced == 41 : wgs_41 >= num_compute_units();
-    if (a.D == 128) return use41 ? launch_cfg<128, 4, 1>(p, s) : launch_cfg<128, 2, 2>(p, s);
-    return use41 ? launch_cfg<64, 4, 1>(p, s) : launch_cfg<64, 2, 2>(p, s);
+    const int64_t G = a.Hq / a.Hkv;
+    int shape = forced;
+    if (!shape) {
+        (void)G;
+        int64_t wgs_421 = a.B * a.Hq * ((a.Sq + 127) / 128);
+        shape = wgs_421 >= num_compute_units() ? 421 : 241;
+    }
+#define TROCM_PREFILL_CASES(DD)                                        \
+    switch (shape) {                                                   \
+        case 411: return launch_cfg<DD, 4, 1, 1>(p, s);                \
+        case 221: return launch_cfg<DD, 2, 2, 1>(p, s);                \
+        case 421: return launch_cfg<DD, 4, 2, 1>(p, s);                \
+        case 241: return launch_cfg<DD, 2, 4, 1>(p, s);                \
+        case 424: return launch_cfg<DD, 4, 2, 4>(p, s);                \
+        case 814: return launch_cfg<DD, 8, 1, 4>(p, s);                \
+        default: return fail("unknown prefill shape %d", shape);       \
+    }
+    if (a.D == 128) {
+        TROCM_PREFILL_CASES(128)
+    }
+    TROCM_PREFILL_CASES(64)
+#undef TROCM_PREFILL_CASES
 }
 
 }  // namespace trocm
