@@ -192,7 +192,7 @@ def run_cfg3(ta, args):
         tot_us += us
         tot_fl += fl
     tf = tot_fl / tot_us / 1e6
-    roof = {"bound": "mfma", "kernel": "sdpa_prefill_kernel<128,2,2>", "achieved": round(tf, 1), "peak": 2500.0,
+    roof = {"bound": "mfma", "kernel": "sdpa_prefill_pp_kernel<128,4> (+ sdpa_prefill_merge_kernel<128>)", "achieved": round(tf, 1), "peak": 2500.0,
             "unit": "TFLOP/s", "frac": round(tf / 2500.0, 4), "traffic": None}
     return base_line(args, "cfg3: chunked prefill, 8 x 512 tokens into an empty cache, causal SDPA of each chunk over "
                      "the cache so far (32q/8kv d=128 f16, batch 1); attention launches only", round(tf, 1), "TFLOP/s",

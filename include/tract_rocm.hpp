@@ -213,7 +213,9 @@ class InPlaceKvSdpaState {
         k.push(k_new);
         v.push(v_new);
         const auto &qs = q.shape();
-        if (!ws_) ws_ = std::make_unique<Workspace>(qs[0], qs[1], qs[2], qs[3]);
+        size_t need = 0;
+        check(trocm_sdpa_workspace_bytes(qs[0], qs[1], qs[2], qs[3], &need));
+        if (!ws_ || ws_->bytes() < need) ws_ = std::make_unique<Workspace>(qs[0], qs[1], qs[2], qs[3]);
         DeviceTensor out(qs, q.datum_type());
         check(trocm_sdpa_cached(q.ptr(), (int)q.datum_type(), qs[1], qs[2], k.handle(), v.handle(), out.ptr(),
                                 scale_.value_or(NAN), causal_, ws_->ptr(), ws_->bytes(), nullptr));

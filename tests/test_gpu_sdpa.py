@@ -306,6 +306,81 @@ def test_prefill_mfma(rt, B, Hq, Hkv, Sq, Sk, D, causal):
     assert max_abs(got, cases.textbook_sdpa(q, k, v, causal=causal)) <= 4e-3
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal", [
+    (1, 2, 2, 256, 256, 128, True),       # one head per workgroup (8 query blocks), key splits
+    (1, 3, 3, 300, 1000, 128, True),      # ... ragged, last query tile mostly empty
+    (1, 4, 2, 128, 640, 128, True),       # two heads per workgroup
+    (2, 12, 2, 130, 515, 128, False),     # group of 6: two heads per workgroup, three workgroups per kv head
+    (1, 32, 8, 512, 2048, 128, True),     # four heads per workgroup, four key splits (the chunked-prefill shape)
+    (1, 8, 2, 64, 4096, 128, True),       # few queries, long cache: 16 key splits
+    (1, 8, 2, 33, 65, 128, True),         # second tile of 1 key
+    (3, 8, 8, 256, 256, 64, True), (1, 16, 4, 96, 1500, 64, False),
+    (16, 32, 8, 64, 64, 128, True),       # enough workgroups without splitting
+])
+def test_prefill_grouped_heads_and_key_splits(rt, B, Hq, Hkv, Sq, Sk, D, causal):
+    rng = np.random.default_rng(2000 + Sq + Sk + Hq)
+    q = (rng.standard_normal((B, Hq, Sq, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    k = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(np.float16)
+    k[:, :, Sk // 3] *= 6.0   # an outlier key: the running maximum moves late and the splits' maxima differ
+    got = tract_amd.Sdpa(datum_type=np.float16, is_causal=causal).eval(q, k, v).to_numpy()
+    want = orc.flash_sdpa(q, k, v, causal=causal, threads=8)
+    assert not np.isnan(got).any()
+    assert max_abs(got, want) <= 2e-2
+    assert max_abs(got, cases.textbook_sdpa(q, k, v, causal=causal)) <= 4e-3
+
+
+_PREFILL_ENV_CODE = """
+import os, sys, numpy as np
+import tract_amd
+tract_amd.runtime_for_name('rocm')
+rng=np.random.default_rng(77)
+q=(rng.standard_normal((1,32,192,128),dtype=np.float32)/11.3).astype(np.float16)
+k=rng.standard_normal((1,8,1100,128),dtype=np.float32).astype(np.float16)
+v=rng.standard_normal((1,8,1100,128),dtype=np.float32).astype(np.float16)
+o=tract_amd.Sdpa(datum_type=np.float16,is_causal=True).eval(q,k,v).to_numpy()
+sys.stdout.buffer.write(o.tobytes())
+"""
+
+
+@pytest.mark.parametrize("env", [{"TROCM_PREFILL_SPLITS": "1"}, {"TROCM_PREFILL_SPLITS": "2"},
+                                 {"TROCM_PREFILL_SPLITS": "5"}, {"TROCM_PREFILL_SPLITS": "16"},
+                                 {"TROCM_PREFILL_HG": "1"}, {"TROCM_PREFILL_HG": "2"}, {"TROCM_PREFILL_PP": "0"}])
+def test_prefill_any_split_count_and_head_grouping_agree(rt, env):
+    """The key-split merge is exact in real arithmetic and the head grouping only changes which
+    workgroup computes a head: every setting must agree with the textbook form."""
+    import subprocess, sys
+    e = dict(os.environ)
+    e.update(env)
+    out = subprocess.run([sys.executable, "-c", _PREFILL_ENV_CODE], capture_output=True, check=True, env=e,
+                         cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__)))).stdout
+    got = np.frombuffer(out[-1 * 32 * 192 * 128 * 2:], dtype=np.float16).reshape(1, 32, 192, 128)
+    rng = np.random.default_rng(77)
+    q = (rng.standard_normal((1, 32, 192, 128), dtype=np.float32) / 11.3).astype(np.float16)
+    k = rng.standard_normal((1, 8, 1100, 128), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((1, 8, 1100, 128), dtype=np.float32).astype(np.float16)
+    assert max_abs(got, cases.textbook_sdpa(q, k, v, causal=True)) <= 4e-3
+
+
+def test_prefill_with_a_workspace_too_small_for_key_splits(rt):
+    """A caller may hand over a workspace sized for decode only: prefill then runs unsplit."""
+    from tract_amd._lib import call
+    from tract_amd.runtime import DeviceTensor, Workspace
+    B, Hq, Hkv, Sq, Sk, D = 1, 32, 8, 512, 1024, 128
+    rng = np.random.default_rng(4)
+    q = (rng.standard_normal((B, Hq, Sq, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    k = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(np.float16)
+    ws = Workspace(B, Hq, 1, D)
+    assert ws.nbytes < Workspace.bytes_for(B, Hq, Sq, D)
+    dq, dk, dv = (DeviceTensor.from_numpy(t) for t in (q, k, v))
+    out = DeviceTensor(q.shape, q.dtype)
+    for wsp, wsn in ((ws.ptr, ws.nbytes), (None, 0)):
+        call("trocm_sdpa", dq.ptr, dk.ptr, dv.ptr, None, out.ptr, 1, B, Hq, Hkv, Sq, Sk, D, None, 1, 1,
+             float("nan"), 1, wsp, wsn, None)
+        assert max_abs(out.to_numpy(), cases.textbook_sdpa(q, k, v, causal=True)) <= 4e-3
+
+
 def test_chunked_prefill_into_cache_cfg3_reduced(rt):
     """cfg3 (reduced to 8 chunks of 96 tokens): each chunk is appended to the in-place cache,
     then attends causally to the whole cache so far (q_len 96, kv_len 96*c), reading K/V from

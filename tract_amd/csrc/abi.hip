@@ -672,8 +672,9 @@ int trocm_block_dequant(int format, const void *src_blocks, size_t n_elems, void
 int trocm_sdpa_workspace_bytes(int64_t batch, int64_t q_heads, int64_t q_len, int64_t head_dim, size_t *bytes) {
     TROCM_NOT_NULL(bytes);
     TROCM_REQUIRE(batch >= 0 && q_heads >= 0 && q_len >= 0 && head_dim >= 0, "workspace_bytes: negative dimension");
-    (void)q_len;
-    *bytes = decode_workspace_bytes(batch, q_heads, head_dim);
+    size_t need = decode_workspace_bytes(batch, q_heads, head_dim);
+    size_t prefill = kWsCounterBytes + prefill_workspace_bytes(batch, q_heads, q_len, head_dim);
+    *bytes = need > prefill ? need : prefill;
     return 0;
 }
 
@@ -690,6 +691,7 @@ static int dispatch_sdpa(const SdpaArgs &a, hipStream_t s) {
     if (a.B == 0 || a.Hq == 0 || a.Sq == 0 || a.D == 0) return 0;
     int rc = 2;
     if (a.Sq == 1) rc = is_quant(a.kv_fmt) ? launch_sdpa_decode_quant(a, s) : launch_sdpa_decode(a, s);
+    if (rc == 2 && a.Sq > 1) rc = launch_sdpa_prefill_pp(a, s);
     if (rc == 2) rc = launch_sdpa_prefill(a, s);
     if (rc == 2) rc = launch_sdpa_generic(a, s);
     return rc;

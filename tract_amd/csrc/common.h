@@ -120,6 +120,10 @@ int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s);
 int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s);
 // MFMA prefill.  Returns 2 when the shape is not covered.
 int launch_sdpa_prefill(const SdpaArgs &a, hipStream_t s);
+// MFMA prefill for q_len >= 32: staggered waves, GQA heads sharing K/V tiles, key splits across
+// workgroups (partials in the workspace after the counter area).  Returns 2 when not covered.
+int launch_sdpa_prefill_pp(const SdpaArgs &a, hipStream_t s);
+size_t prefill_workspace_bytes(int64_t B, int64_t Hq, int64_t Sq, int64_t D);
 
 // Ragged decode: per-sequence descriptors live in pinned host memory owned by the library.
 struct RaggedSeq {

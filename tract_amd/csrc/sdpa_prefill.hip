@@ -113,6 +113,11 @@ __global__ __launch_bounds__(64 * WM * WN) void sdpa_prefill_kernel(PrefillDev p
     half8_t qf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) qf[ks] = *reinterpret_cast<const half8_t *>(qrow + 16 * ks + 8 * hb);
+    // Settle the Q loads here.  Otherwise the compiler must assume they may still be in flight at
+    // the top of the tile loop and waits for vmcnt(0) at their first use there, which also waits
+    // for the K/V prefetch issued a few instructions earlier and exposes its whole latency.
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) asm volatile("" : "+v"(qf[ks]));
 
     // key tiles this workgroup needs
     const int wg_q_last = min(qt * BLOCK_M + BLOCK_M, p.Sq) - 1;

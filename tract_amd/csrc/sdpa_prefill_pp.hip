@@ -1,0 +1,445 @@
+// MFMA prefill attention for gfx950, throughput version for q_len >= 32 (GQA heads share K/V tiles).
+// f16 in/out, f32 accumulate, causal (bottom-right aligned) or unmasked, GQA, K/V read in place.
+//
+// Same transposed formulation as sdpa_prefill.hip (S^T = K.Q^T, O^T = V^T.P^T with 32x32x16 MFMAs,
+// every softmax scalar of a query in one lane).  What differs is how a compute unit is kept busy:
+//
+//  * One workgroup = 8 waves = 8 different (query head, 32-query block) pairs that all read the
+//    SAME 64-key K/V tile: HG query heads of one kv head (GQA) x 8/HG query blocks.  A tile
+//    staged into LDS once feeds 8 waves, so staging traffic per MFMA is a quarter of what a
+//    one-head 64-query workgroup needs.
+//  * K and V tiles are double buffered in LDS and fetched two tiles ahead through registers, so a
+//    tile costs one barrier and the global-memory latency stays hidden.  (Running the two waves
+//    of a SIMD half an iteration apart, so that one's softmax would overlap the other's MFMAs,
+//    was tried and measured no faster: the hardware already interleaves them.)
+//  * Few workgroups (small batch) are spread over the chip by splitting the key range over
+//    several workgroups.  Each writes its normalised partial output in f16 plus (m, l) to the
+//    workspace, laid out exactly as the accumulator registers are (so every store instruction
+//    covers 512 contiguous bytes), and a small kernel merges them.
+//  * The output accumulators are rescaled only when some query's running maximum moved.
+//
+// Roofline: MFMA-bound.  FLOPs = 4 * B * Hq * D * (visible query-key pairs).
+#include <hip/hip_fp16.h>
+#include <string.h>
+#include <stdlib.h>
+#include "common.h"
+
+namespace trocm {
+namespace {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef short short4_t __attribute__((ext_vector_type(4)));
+
+struct PrefillPP {
+    const _Float16 *q;
+    _Float16 *out;
+    const _Float16 *k, *v;
+    int64_t kv_stride_b, kv_stride_h, kv_stride_t;  // elements
+    int B, Hq, Hkv, Sq, Sk;
+    int causal;
+    int n_qtiles, nsplit;
+    float scale_log2;
+    // Partials of key split s and 32-query block wb (= (b * Hq + qh) * n_qb32 + q / 32):
+    _Float16 *part_o;   // [nsplit][n_wb][D / 4][32 queries][4 features], normalised by l
+    float *part_ml;     // [nsplit][n_wb][2][32 queries]: m (log2 domain), then l
+    int n_qb32;
+    int64_t n_wb;
+};
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Transposing 64-bit LDS load of 16-bit elements: in each block of 16 lanes, lane i receives
+// element i%4 of the four 8-byte rows addressed by lanes i/4, i/4+4, i/4+8, i/4+12.
+__device__ __forceinline__ half4_t lds_read_tr16(const _Float16 *lds_ptr) {
+    typedef __attribute__((address_space(3))) short4_t *lds_v4_ptr;
+    short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_ptr)(uintptr_t)(uint32_t)(uintptr_t)lds_ptr);
+    return __builtin_bit_cast(half4_t, r);
+}
+
+constexpr int kWavesPP = 8, kThreadsPP = 64 * kWavesPP, kTileN = 64;
+
+template <int D, int HG>
+__global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p) {
+    constexpr int QB = kWavesPP / HG;     // 32-query blocks per workgroup
+    constexpr int BLOCK_M = 32 * QB;
+    constexpr int KS = D / 16;            // contraction steps of Q K^T
+    constexpr int DB = D / 32;            // 32-feature blocks of the output
+    constexpr int KROW = D + 8;           // halfs per K row in LDS: 128-bit reads of 16 rows hit 64 distinct banks
+    constexpr int VROW = D + 16;          // halfs per V row in LDS: the 4 rows of a transposing read sit 8 banks apart
+    constexpr int NL = kTileN * D / 8 / kThreadsPP;  // 128-bit loads per thread per tile and tensor
+    static_assert(NL >= 1 && NL * 8 * kThreadsPP == kTileN * D, "tile loads must divide evenly");
+
+    __shared__ __attribute__((aligned(16))) _Float16 lds_k[2][kTileN * KROW];
+    __shared__ __attribute__((aligned(16))) _Float16 lds_v[2][kTileN * VROW];
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int hb = lane >> 5, l32 = lane & 31;
+
+    // workgroup -> (kv head fastest: consecutive workgroup ids go round-robin to the 8 XCDs, so
+    // one kv head's K/V stays in one XCD's L2), head group, key split, query tile (longest first)
+    int id = blockIdx.x;
+    const int kvh = id % p.Hkv;
+    id /= p.Hkv;
+    const int G = p.Hq / p.Hkv;
+    const int gg = id % (G / HG);
+    id /= (G / HG);
+    const int split = id % p.nsplit;
+    id /= p.nsplit;
+    const int qt = p.n_qtiles - 1 - (id % p.n_qtiles);
+    const int b = id / p.n_qtiles;
+    const int qh = kvh * G + gg * HG + (w % HG);
+
+    const int off = p.Sk - p.Sq;          // query i sees keys j <= i + off when causal
+    const int q0 = qt * BLOCK_M + 32 * (w / HG);  // first query of this wave
+    const int my_q = q0 + l32;
+    const bool wave_has_queries = q0 < p.Sq;
+    const _Float16 *qrow = p.q + (((int64_t)b * p.Hq + qh) * p.Sq + min(my_q, p.Sq - 1)) * D;
+    const _Float16 *kbase = p.k + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+    const _Float16 *vbase = p.v + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+
+    // key tiles of this workgroup: its share of the tiles its last query sees
+    const int wg_q_last = min(qt * BLOCK_M + BLOCK_M, p.Sq) - 1;
+    const int last_key = p.causal ? min(p.Sk - 1, wg_q_last + off) : p.Sk - 1;
+    const int n_kt = last_key / kTileN + 1;
+    const int per = (n_kt + p.nsplit - 1) / p.nsplit;
+    const int t_begin = split * per;
+    const int n_it = max(0, min(n_kt, t_begin + per) - t_begin);
+    const int wave_q_last = min(q0 + 31, p.Sq - 1);
+
+    float m_run = -INFINITY, l_run = 0.0f;   // m_run in the log2 domain, already scaled
+    float16_t o[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
+
+    half8_t qf[KS];
+    u32x4 kpre[NL], vpre[NL];
+    auto prefetch = [&](int kt) {
+#pragma unroll
+        for (int j = 0; j < NL; j++) {
+            int c = j * kThreadsPP + tid;
+            int key = c / (D / 8), dc = c % (D / 8);
+            int64_t row = min(kt * kTileN + key, p.Sk - 1);
+            kpre[j] = *reinterpret_cast<const u32x4 *>(kbase + row * p.kv_stride_t + dc * 8);
+            vpre[j] = *reinterpret_cast<const u32x4 *>(vbase + row * p.kv_stride_t + dc * 8);
+        }
+    };
+    auto stage = [&](int kbuf, int vbuf) {
+#pragma unroll
+        for (int j = 0; j < NL; j++) {
+            int c = j * kThreadsPP + tid;
+            int key = c / (D / 8), dc = c % (D / 8);
+            *reinterpret_cast<u32x4 *>(&lds_k[kbuf][key * KROW + dc * 8]) = kpre[j];
+            *reinterpret_cast<u32x4 *>(&lds_v[vbuf][key * VROW + dc * 8]) = vpre[j];
+        }
+    };
+
+    // does this wave have anything to do on tile kt?
+    auto tile_active = [&](int kt) { return wave_has_queries && (!p.causal || kt * kTileN <= wave_q_last + off); };
+
+    // ---- S^T = K Q^T : 2 key blocks of 32 x 32 queries ---------------------------------------------
+    auto qk = [&](int kbuf, float16_t (&s)[2]) {
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[kb][r] = 0.0f;
+        const _Float16 *kt_base = &lds_k[kbuf][l32 * KROW + 8 * hb];
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                half8_t kf = *reinterpret_cast<const half8_t *>(kt_base + (32 * kb) * KROW + 16 * ks);
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s[kb], 0, 0, 0);
+            }
+        }
+    };
+
+    // ---- online softmax for query lane%32 over this lane's 32 keys; leaves P^T fragments in pf ----
+    auto softmax = [&](int kt, float16_t (&s)[2], half8_t (&pf)[4]) {
+        const int k_lo = kt * kTileN;
+        const bool need_mask = (k_lo + kTileN > p.Sk) || (p.causal && (k_lo + kTileN - 1 > q0 + off));
+        if (need_mask) {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    int key = k_lo + 32 * kb + 8 * (r >> 2) + 4 * hb + (r & 3);
+                    bool vis = key < p.Sk && (!p.causal || key <= my_q + off);
+                    s[kb][r] = vis ? s[kb][r] : -INFINITY;
+                }
+        }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) tmax = fmaxf(tmax, s[kb][r]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m_run, tmax * p.scale_log2);  // scale > 0: the maximum commutes with the scaling
+        const float m_ref = (m_new == -INFINITY) ? 0.0f : m_new;  // nothing visible yet: keep everything at zero
+        float psum = 0.0f;
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float pv = fast_exp2(__builtin_fmaf(s[st >> 1][8 * (st & 1) + i], p.scale_log2, -m_ref));
+                psum += pv;
+                pf[st][i] = (_Float16)pv;
+            }
+        }
+        const bool moved = m_new != m_run;
+        const float alpha = fast_exp2(m_run - m_ref);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[db][r] *= alpha;
+        }
+    };
+
+    // ---- O^T += V^T P^T ---------------------------------------------------------------------------------
+    // This lane as a SOURCE of the transposing loads: key row (lane%16)/4 of a group of four,
+    // features 16*(lane/16 % 2) + 4*(lane%4) of the 32-feature block.
+    const int vsrc_off = (4 * hb + ((lane & 15) >> 2)) * VROW + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    auto pv = [&](int vbuf, half8_t (&pf)[4]) {
+        const _Float16 *vsrc = &lds_v[vbuf][vsrc_off];
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+                half4_t lo = lds_read_tr16(vsrc + (16 * st) * VROW + 32 * db);      // keys 16st + 4hb + 0..3
+                half4_t hi = lds_read_tr16(vsrc + (16 * st + 8) * VROW + 32 * db);  // keys 16st + 8 + 4hb + 0..3
+                half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[st], o[db], 0, 0, 0);
+            }
+        }
+    };
+
+    if (n_it > 0) prefetch(t_begin);   // issued before the Q loads: both latencies overlap
+    // Q^T fragments: query = lane % 32, features 16*ks + 8*hb .. +8
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = *reinterpret_cast<const half8_t *>(qrow + 16 * ks + 8 * hb);
+    // Settle the Q loads here.  Otherwise the compiler must assume they may still be in flight at
+    // the top of the tile loop and waits for vmcnt(0) at their first use there, which also waits
+    // for the K/V prefetch issued a few instructions earlier and exposes its whole latency.
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) asm volatile("" : "+v"(qf[ks]));
+
+    if (n_it > 0) {
+        stage(0, 0);
+        if (n_it > 1) prefetch(t_begin + 1);
+    }
+    for (int it = 0; it < n_it; it++) {
+        __syncthreads();   // tile `it` is in LDS; every wave is done with the buffers about to be overwritten
+        const int cur = it & 1;
+        if (it + 1 < n_it) {
+            stage(cur ^ 1, cur ^ 1);
+            if (it + 2 < n_it) prefetch(t_begin + it + 2);
+        }
+        const int kt = t_begin + it;
+        if (tile_active(kt)) {
+            float16_t s[2];
+            half8_t pf[4];
+            qk(cur, s);
+            softmax(kt, s, pf);
+            pv(cur, pf);
+        }
+    }
+
+    l_run += __shfl_xor(l_run, 32, 64);
+    if (!wave_has_queries) return;
+    if (p.nsplit == 1) {
+        if (my_q >= p.Sq) return;
+        const int64_t row = ((int64_t)b * p.Hq + qh) * p.Sq + my_q;
+        const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+        _Float16 *orow = p.out + row * D;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int rq = 0; rq < 4; rq++) {
+                half4_t h4;
+#pragma unroll
+                for (int i = 0; i < 4; i++) h4[i] = (_Float16)(o[db][4 * rq + i] * inv);
+                *reinterpret_cast<half4_t *>(orow + 32 * db + 8 * rq + 4 * hb) = h4;
+            }
+    } else {
+        const int64_t wb = ((int64_t)b * p.Hq + qh) * p.n_qb32 + (q0 >> 5);
+        const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+        _Float16 *po = p.part_o + ((int64_t)split * p.n_wb + wb) * (32 * D) + l32 * 4;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int rq = 0; rq < 4; rq++) {
+                half4_t h4;
+#pragma unroll
+                for (int i = 0; i < 4; i++) h4[i] = (_Float16)(o[db][4 * rq + i] * inv);
+                *reinterpret_cast<half4_t *>(po + (8 * db + 2 * rq + hb) * 128) = h4;
+            }
+        p.part_ml[((int64_t)split * p.n_wb + wb) * 64 + lane] = hb ? l_run : m_run;
+    }
+}
+
+// Merge of the key splits, one workgroup per 32-query block:
+//   out = sum_s w_s O_s / sum_s w_s,   w_s = l_s 2^(m_s - max m),   O_s normalised partial outputs.
+template <int D>
+__global__ __launch_bounds__(256) void sdpa_prefill_merge_kernel(PrefillPP p) {
+    constexpr int kMaxSplits = 16;
+    constexpr int OROW = D + 8;
+    __shared__ float wts[kMaxSplits][32];
+    __shared__ __attribute__((aligned(16))) _Float16 tile[32 * OROW];
+    const int64_t wb = blockIdx.x;
+    const int tid = threadIdx.x;
+    if (tid < 32) {
+        float mm = -INFINITY;
+        for (int sp = 0; sp < p.nsplit; sp++) mm = fmaxf(mm, p.part_ml[((int64_t)sp * p.n_wb + wb) * 64 + tid]);
+        const float m_ref = (mm == -INFINITY) ? 0.0f : mm;
+        float total = 0.0f;
+        for (int sp = 0; sp < p.nsplit; sp++) {
+            const float *ml = p.part_ml + ((int64_t)sp * p.n_wb + wb) * 64;
+            const float wgt = ml[32 + tid] * fast_exp2(ml[tid] - m_ref);
+            wts[sp][tid] = wgt;
+            total += wgt;
+        }
+        const float inv = total > 0.0f ? 1.0f / total : 0.0f;
+        for (int sp = 0; sp < p.nsplit; sp++) wts[sp][tid] *= inv;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < D / 32; j++) {
+        const int idx = j * 256 + tid;       // (feature group, query) in the partials' order
+        const int fg = idx >> 5, q = idx & 31;
+        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int sp = 0; sp < p.nsplit; sp++) {
+            const half4_t h = *reinterpret_cast<const half4_t *>(p.part_o + ((int64_t)sp * p.n_wb + wb) * (32 * D) + idx * 4);
+            const float wgt = wts[sp][q];
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[i] += wgt * (float)h[i];
+        }
+        half4_t h4;
+#pragma unroll
+        for (int i = 0; i < 4; i++) h4[i] = (_Float16)acc[i];
+        *reinterpret_cast<half4_t *>(&tile[q * OROW + fg * 4]) = h4;
+    }
+    __syncthreads();
+    const int64_t bh = wb / p.n_qb32;
+    const int q_first = (int)(wb % p.n_qb32) * 32;
+#pragma unroll
+    for (int j = 0; j < D / 64; j++) {
+        const int idx = j * 256 + tid;       // (query, 16-byte segment of its row)
+        const int q = idx / (D / 8), seg = idx % (D / 8);
+        if (q_first + q < p.Sq)
+            *reinterpret_cast<u32x4 *>(p.out + (bh * p.Sq + q_first + q) * D + seg * 8) =
+                *reinterpret_cast<const u32x4 *>(&tile[q * OROW + seg * 8]);
+    }
+}
+
+template <int D, int HG>
+int launch_cfg(const PrefillPP &p, int64_t wgs, hipStream_t s) {
+    hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("sdpa_prefill_pp launch failed: %s", hipGetErrorString(e));
+    if (p.nsplit > 1) {
+        hipLaunchKernelGGL((sdpa_prefill_merge_kernel<D>), dim3((unsigned)p.n_wb), dim3(256), 0, s, p);
+        e = hipGetLastError();
+        if (e != hipSuccess) return fail("sdpa_prefill_merge launch failed: %s", hipGetErrorString(e));
+    }
+    return 0;
+}
+
+template <int D>
+int launch_hg(const PrefillPP &p, int hg, int64_t wgs, hipStream_t s) {
+    switch (hg) {
+        case 4: return launch_cfg<D, 4>(p, wgs, s);
+        case 2: return launch_cfg<D, 2>(p, wgs, s);
+        default: return launch_cfg<D, 1>(p, wgs, s);
+    }
+}
+
+int env_int(const char *name, int dflt) {
+    const char *e = getenv(name);
+    return e ? atoi(e) : dflt;
+}
+
+}  // namespace
+
+static size_t split_bytes(int64_t n_wb, int64_t D) { return (size_t)n_wb * (32 * (size_t)D * sizeof(_Float16) + 64 * sizeof(float)); }
+
+// Upper bound of the partial-result area the staggered prefill kernel may use for this shape.
+size_t prefill_workspace_bytes(int64_t B, int64_t Hq, int64_t Sq, int64_t D) {
+    if (Sq < 2 || (D != 64 && D != 128)) return 0;
+    const int64_t wgs1 = B * ((Hq + 3) / 4) * ((Sq + 63) / 64);  // about the fewest workgroups any head grouping gives
+    const int64_t cus = 256;
+    if (wgs1 >= cus) return 0;
+    int64_t ns = (cus + wgs1 - 1) / wgs1;
+    if (ns > 16) ns = 16;
+    return (size_t)ns * split_bytes(B * Hq * ((Sq + 31) / 32), D) + 256;
+}
+
+int launch_sdpa_prefill_pp(const SdpaArgs &a, hipStream_t s) {
+    if (a.q_dtype != TROCM_F16 || a.kv_fmt != TROCM_F16 || a.mask != nullptr) return 2;
+    if (a.D != 128 && a.D != 64) return 2;
+    if (a.Sq < 2 || a.Sk < 1 || a.Hq % a.Hkv) return 2;
+    if (!(a.scale > 0.0f)) return 2;       // the running maximum is taken before scaling
+    if (a.causal && a.Sk < a.Sq) return 2;  // some queries would see nothing: the generic kernel owns that case
+    if (a.Sk >= (1ll << 30) || a.Sq >= (1ll << 30) || a.B >= (1ll << 20)) return 2;
+    if ((a.kv_stride_b % 8) || (a.kv_stride_h % 8) || (a.kv_stride_t % 8)) return 2;  // 128-bit row loads
+    if ((uintptr_t)a.q % 16 || (uintptr_t)a.k % 16 || (uintptr_t)a.v % 16 || (uintptr_t)a.out % 8) return 2;
+    static const int enabled = env_int("TROCM_PREFILL_PP", 1);
+    if (!enabled) return 2;
+    static const int forced_hg = env_int("TROCM_PREFILL_HG", 0);
+    static const int forced_split = env_int("TROCM_PREFILL_SPLITS", 0);
+    const int64_t G = a.Hq / a.Hkv;
+    int hg = G % 4 == 0 ? 4 : G % 2 == 0 ? 2 : 1;
+    if (forced_hg && G % forced_hg == 0 && (forced_hg == 1 || forced_hg == 2 || forced_hg == 4)) hg = forced_hg;
+    const int block_m = 32 * kWavesPP / hg;
+    const int64_t n_qtiles = (a.Sq + block_m - 1) / block_m;
+    // Waves whose 32-query block lies past q_len idle: leave short prompts to the smaller kernel.
+    if (a.Sq * 2 < n_qtiles * block_m) return 2;
+
+    PrefillPP p;
+    memset(&p, 0, sizeof(p));
+    p.q = (const _Float16 *)a.q;
+    p.out = (_Float16 *)a.out;
+    p.k = (const _Float16 *)a.k;
+    p.v = (const _Float16 *)a.v;
+    p.kv_stride_b = a.kv_stride_b, p.kv_stride_h = a.kv_stride_h, p.kv_stride_t = a.kv_stride_t;
+    p.B = (int)a.B, p.Hq = (int)a.Hq, p.Hkv = (int)a.Hkv, p.Sq = (int)a.Sq, p.Sk = (int)a.Sk;
+    p.causal = a.causal;
+    p.scale_log2 = a.scale * 1.4426950408889634f;
+    p.n_qtiles = (int)n_qtiles;
+    p.n_qb32 = (int)((a.Sq + 31) / 32);
+    p.n_wb = a.B * a.Hq * p.n_qb32;
+
+    const int64_t wgs1 = a.B * (a.Hq / hg) * n_qtiles;
+    const int64_t cus = num_compute_units();
+    int64_t ns = 1;
+    if (wgs1 < cus) {
+        ns = (cus + wgs1 - 1) / wgs1;
+        const int64_t tiles = (a.Sk + kTileN - 1) / kTileN;
+        if (ns > tiles / 2) ns = tiles / 2;   // at least two tiles per split
+        if (ns > 16) ns = 16;
+    }
+    if (forced_split > 0) ns = forced_split;
+    const size_t per_split = split_bytes(p.n_wb, a.D);
+    const size_t avail = a.workspace && a.workspace_bytes > kWsCounterBytes + 256 ? a.workspace_bytes - kWsCounterBytes - 256 : 0;
+    if (ns > 1 && (size_t)ns * per_split > avail) ns = (int64_t)(avail / per_split);
+    if (ns < 1) ns = 1;
+    p.nsplit = (int)ns;
+    if (ns > 1) {
+        char *base = (char *)a.workspace + kWsCounterBytes;
+        base += (256 - ((uintptr_t)base & 255)) & 255;
+        p.part_o = (_Float16 *)base;
+        p.part_ml = (float *)(base + (size_t)ns * p.n_wb * 32 * a.D * sizeof(_Float16));
+    }
+    const int64_t wgs = wgs1 * ns;
+    if (wgs >= (1ll << 31)) return 2;
+    return a.D == 128 ? launch_hg<128>(p, hg, wgs, s) : launch_hg<64>(p, hg, wgs, s);
+}
+
+}  // namespace trocm

@@ -233,7 +233,7 @@ class Sdpa:
                 raise TractRocmError(f"mask shape {m.shape} does not end in [q_len, kv_len]")
             mb, mh = ms[0], ms[1]
         out = DeviceTensor(q.shape, q.dtype)
-        if self._ws is None or self._ws_key != (B, Hq, D):
+        if self._ws is None or self._ws_key != (B, Hq, D) or self._ws.nbytes < Workspace.bytes_for(B, Hq, Sq, D):
             self._ws, self._ws_key = Workspace(B, Hq, Sq, D, stream), (B, Hq, D)
         call("trocm_sdpa", q.ptr, k.ptr, v.ptr, None if m is None else m.ptr, out.ptr, dtype_code(q.dtype),
              B, Hq, Hkv, Sq, Sk, D, None, mb, mh, _scale_arg(self.scale), int(self.is_causal),
@@ -291,7 +291,7 @@ class InPlaceKvSdpaState:
         B, Hq, Sq, D = _canon4(q.shape)
         if out is None:
             out = DeviceTensor(q.shape, q.dtype)
-        if self._ws is None or self._ws_key != (B, Hq, D):
+        if self._ws is None or self._ws_key != (B, Hq, D) or self._ws.nbytes < Workspace.bytes_for(B, Hq, Sq, D):
             self._ws, self._ws_key = Workspace(B, Hq, Sq, D, stream), (B, Hq, D)
         call("trocm_inplace_kv_sdpa_eval", q.ptr, k_new.ptr, v_new.ptr, dtype_code(q.dtype), Hq, Sq, None,
              self.k.handle, self.v.handle, out.ptr, _scale_arg(self.scale), int(self.causal),
@@ -302,7 +302,7 @@ class InPlaceKvSdpaState:
         B, Hq, Sq, D = _canon4(q.shape)
         if out is None:
             out = DeviceTensor(q.shape, q.dtype)
-        if self._ws is None or self._ws_key != (B, Hq, D):
+        if self._ws is None or self._ws_key != (B, Hq, D) or self._ws.nbytes < Workspace.bytes_for(B, Hq, Sq, D):
             self._ws, self._ws_key = Workspace(B, Hq, Sq, D, stream), (B, Hq, D)
         if self.k.handle is None:
             raise TractRocmError("empty kv-cache")

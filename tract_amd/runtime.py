@@ -159,10 +159,14 @@ class Workspace:
     """Persistent split-K scratch owned by an op state (the arena planner does not model
     scratch, gpu/src/memory/schema.rs:56-128)."""
 
-    def __init__(self, batch: int, q_heads: int, q_len: int, head_dim: int, stream=None):
+    @staticmethod
+    def bytes_for(batch: int, q_heads: int, q_len: int, head_dim: int) -> int:
         n = C.c_size_t()
         call("trocm_sdpa_workspace_bytes", batch, q_heads, q_len, head_dim, C.byref(n))
-        self.nbytes = n.value
+        return n.value
+
+    def __init__(self, batch: int, q_heads: int, q_len: int, head_dim: int, stream=None):
+        self.nbytes = Workspace.bytes_for(batch, q_heads, q_len, head_dim)
         self.buf = DeviceTensor((self.nbytes,), np.uint8)
         call("trocm_sdpa_workspace_init", self.buf.ptr, self.nbytes, _sh(stream))
         call("trocm_stream_sync", _sh(stream))
