@@ -169,7 +169,9 @@ int trocm_block_dequant(int format, const void *src_blocks, size_t n_elems, void
  * owns one workspace and passes it to every call.  trocm_sdpa_workspace_init() must run
  * once on a new workspace (it zeroes the header area reserved for kernel-side counters);
  * kernels leave it ready for the next call.  Two calls that overlap in time must not share
- * a workspace. */
+ * a workspace.  The size covers decode for (batch, q_heads, head_dim) and, for q_len > 1,
+ * the partial results of a prefill whose key range is split over workgroups; a call made
+ * with a smaller (or NULL) workspace still succeeds, with fewer splits. */
 int trocm_sdpa_workspace_bytes(int64_t batch, int64_t q_heads, int64_t q_len, int64_t head_dim,
                                size_t *bytes);
 int trocm_sdpa_workspace_init(void *workspace, size_t bytes, void *stream);
