@@ -36,6 +36,9 @@ struct DecodeDev {
     int64_t sc_stride_b, sc_stride_h;  // bytes
     // fused append (plain formats): the step's new K/V rows, dense [B or n_seq, Hkv, 1, D]; NULL = none
     const char *k_new, *v_new;
+    // dense f16/f32 kernel: 1 = the splits of a sequence take groups of kWaves tiles round-robin
+    // (concurrent workgroups then read neighbouring addresses), 0 = contiguous tile ranges
+    int interleave;
 };
 
 // Ragged batches: one work item = a tile range of one sequence (device copies of the host plan).

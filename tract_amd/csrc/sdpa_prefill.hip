@@ -14,13 +14,10 @@
 // A wave owns 32 queries and, per workgroup tile, 64 keys.  The waves of a workgroup are
 // arranged WM x WN: WM query groups (BLOCK_M = 32*WM) times WN key slices (BLOCK_N = 64*WN);
 // waves that share queries keep separate online-softmax states and are merged through LDS at
-// the end.  Eight waves per workgroup put two waves on every SIMD; because the two barriers per
-// tile keep them in the same phase this gains only about 5 % over four waves (307 -> 321 TFLOP/s
-// on 8 x 512-token chunks).  2x4 (64 queries per workgroup) keeps every compute unit busy when
-// there are few query tiles, 4x2 (128 queries) halves the K/V staging per query when there are
-// many.  HG query heads of one KV head can
-// share a workgroup (the WM waves are split HG ways): the K/V tile staged into LDS then feeds
-// HG times more MFMA work, which is what GQA allows and what bounds small-batch prefill.
+// the end.  2x2 (64 queries per workgroup) keeps more compute units busy when there are few
+// query tiles, 4x2 (eight waves, 128 queries) halves the K/V staging per query when there are
+// many.  This kernel serves prompts too short for sdpa_prefill_pp.hip, whose grouped-head
+// workgroups are the fast path.
 //
 // K and V tiles: global -> registers (prefetched one tile ahead) -> LDS, both row-major with
 // padded rows, written with 128-bit stores.  K fragments are plain 128-bit LDS reads.  For V
@@ -310,8 +307,8 @@ int launch_sdpa_prefill(const SdpaArgs &a, hipStream_t s) {
     p.B = (int)a.B, p.Hq = (int)a.Hq, p.Hkv = (int)a.Hkv, p.Sq = (int)a.Sq, p.Sk = (int)a.Sk;
     p.causal = a.causal;
     p.scale_log2 = a.scale * 1.4426950408889634f;
-    // Shapes, named WM WN HG: 4 2 1 = 128 queries of one head; 2 4 1 = 64 queries, keys split four
-    // ways; 4 2 4 = 32 queries of each of 4 heads of a kv head; 8 1 4 = 64 queries x 4 heads.
+    // Shapes, named WM WN HG: 4 1 1 = four waves, 128 queries of one head; 2 2 1 = four waves, 64
+    // queries, keys split two ways; 4 2 1 = eight waves, 128 queries, keys split two ways.
     // TROCM_PREFILL_SHAPE=<WM><WN><HG> forces one (experiments).
     static int forced = -1;
     if (forced < 0) {
@@ -323,16 +320,13 @@ int launch_sdpa_prefill(const SdpaArgs &a, hipStream_t s) {
     if (!shape) {
         (void)G;
         int64_t wgs_421 = a.B * a.Hq * ((a.Sq + 127) / 128);
-        shape = wgs_421 >= num_compute_units() ? 421 : 241;
+        shape = wgs_421 >= num_compute_units() ? 421 : 221;
     }
 #define TROCM_PREFILL_CASES(DD)                                        \
     switch (shape) {                                                   \
         case 411: return launch_cfg<DD, 4, 1, 1>(p, s);                \
         case 221: return launch_cfg<DD, 2, 2, 1>(p, s);                \
         case 421: return launch_cfg<DD, 4, 2, 1>(p, s);                \
-        case 241: return launch_cfg<DD, 2, 4, 1>(p, s);                \
-        case 424: return launch_cfg<DD, 4, 2, 4>(p, s);                \
-        case 814: return launch_cfg<DD, 8, 1, 4>(p, s);                \
         default: return fail("unknown prefill shape %d", shape);       \
     }
     if (a.D == 128) {
