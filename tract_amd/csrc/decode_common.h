@@ -126,38 +126,53 @@ __device__ __forceinline__ __half from_f32<__half>(float x) { return __float2hal
 template <>
 __device__ __forceinline__ float from_f32<float>(float x) { return x; }
 
-// Merge the per-split partials (O, m, l) of one (batch, kv head) and write the output rows.
-// Partial records `first`, `first + stride`, ... (`nsplit` of them).
+// Merge the per-split partials (O, m, l) of ONE query head h of a (batch, kv head) and write its
+// output row; called by a workgroup of D threads, one output element per thread.  Partial records
+// `first`, `first + stride`, ... (`nsplit` of them).  The (m, l) pairs go through LDS once and the
+// O loads of different splits are independent, so the chain is two memory latencies long however
+// many splits there are (with one thread looping over splits and heads a B=1 merge took as long
+// as the attention itself).
+constexpr int kMergeChunk = 256;
 template <typename T, int D, int G>
-__device__ __forceinline__ void merge_splits(const DecodeDev &p, int64_t first, int64_t stride, int nsplit, T *out,
-                                             int tid) {
-    for (int idx = tid; idx < G * D; idx += kThreads) {
-        const int h = idx / D;
-        const float *ml = p.part_ml + first * (2 * G);
-        const float *po = p.part_o + first * (G * D) + idx;
-        const int64_t ml_step = stride * (2 * G), po_step = stride * (G * D);
-        auto ld = [&](const float *a) { return *a; };
-        float mm = -INFINITY;
-#pragma unroll 4
-        for (int sp = 0; sp < nsplit; sp++) mm = fmaxf(mm, ld(ml + sp * ml_step + h));
-        float acc = 0.0f, ll = 0.0f;
-#pragma unroll 4
-        for (int sp = 0; sp < nsplit; sp++) {
-            float f = fast_exp2(ld(ml + sp * ml_step + h) - mm);
-            acc += ld(po + sp * po_step) * f;
-            ll += ld(ml + sp * ml_step + G + h) * f;
+__device__ __forceinline__ void merge_head(const DecodeDev &p, int64_t first, int64_t stride, int nsplit, int h,
+                                           T *out_row, int tid) {
+    __shared__ float lds_m[kMergeChunk], lds_l[kMergeChunk];
+    float m_run = -INFINITY, acc = 0.0f, ll = 0.0f;
+    for (int base = 0; base < nsplit; base += kMergeChunk) {
+        const int n = min(kMergeChunk, nsplit - base);
+        if (base) __syncthreads();
+        for (int sp = tid; sp < n; sp += D) {
+            const float *ml = p.part_ml + (first + (int64_t)(base + sp) * stride) * (2 * G);
+            lds_m[sp] = ml[h];
+            lds_l[sp] = ml[G + h];
         }
-        out[idx] = from_f32<T>(acc / ll);
+        __syncthreads();
+        float cm = -INFINITY;
+        for (int sp = 0; sp < n; sp++) cm = fmaxf(cm, lds_m[sp]);
+        const float m_new = fmaxf(m_run, cm);
+        const float keep = fast_exp2(m_run - m_new);   // 0 on the first chunk
+        acc *= keep;
+        ll *= keep;
+        m_run = m_new;
+        const float *po = p.part_o + (first + (int64_t)base * stride) * (G * D) + h * D + tid;
+        const int64_t po_step = stride * (G * D);
+#pragma unroll 8
+        for (int sp = 0; sp < n; sp++) {
+            const float f = fast_exp2(lds_m[sp] - m_new);
+            acc += po[sp * po_step] * f;
+            ll += lds_l[sp] * f;
+        }
     }
+    out_row[tid] = from_f32<T>(acc / ll);
 }
 
-// Merge launch: grid (kv_heads, batch), runs after the split kernel on the same stream.
+// Merge launch: grid (kv_heads, batch, G), D threads; runs after the split kernel on the same stream.
 template <typename T, int D, int G>
-__global__ __launch_bounds__(kThreads) void sdpa_decode_merge_kernel(DecodeDev p) {
-    const int kvh = blockIdx.x, b = blockIdx.y;
+__global__ __launch_bounds__(D) void sdpa_decode_merge_kernel(DecodeDev p) {
+    const int kvh = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
     const int64_t bh = (int64_t)b * p.Hkv + kvh;
-    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)b * p.Hq + (int64_t)kvh * G) * D;
-    merge_splits<T, D, G>(p, bh * p.nsplit, 1, p.nsplit, out, threadIdx.x);
+    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)b * p.Hq + (int64_t)kvh * G + h) * D;
+    merge_head<T, D, G>(p, bh * p.nsplit, 1, p.nsplit, h, out, threadIdx.x);
 }
 
 }  // namespace

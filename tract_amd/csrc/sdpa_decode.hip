@@ -340,22 +340,21 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     decode_body<T, D, G>(p, wk);
 }
 
-// Merge launch of the ragged batch: grid (kv_heads, sequences).
+// Merge launch of the ragged batch: grid (kv_heads, sequences, G), D threads.
 template <typename T, int D, int G>
-__global__ __launch_bounds__(kThreads) void sdpa_decode_ragged_merge_kernel(DecodeDev p,
-                                                                             const RaggedSeqSlots *__restrict__ seqs) {
-    const int kvh = blockIdx.x, seq = blockIdx.y;
+__global__ __launch_bounds__(D) void sdpa_decode_ragged_merge_kernel(DecodeDev p, const RaggedSeqSlots *__restrict__ seqs) {
+    const int kvh = blockIdx.x, seq = blockIdx.y, h = blockIdx.z;
     const RaggedSeqSlots ss = seqs[seq];
     if (ss.nsplit <= 1) return;
-    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)seq * p.Hq + (int64_t)kvh * G) * D;
-    merge_splits<T, D, G>(p, (int64_t)ss.slot0 * p.Hkv + kvh, p.Hkv, ss.nsplit, out, threadIdx.x);
+    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)seq * p.Hq + (int64_t)kvh * G + h) * D;
+    merge_head<T, D, G>(p, (int64_t)ss.slot0 * p.Hkv + kvh, p.Hkv, ss.nsplit, h, out, threadIdx.x);
 }
 
 template <typename T, int D, int G>
 void launch_both(const DecodeDev &p, dim3 grid, hipStream_t s) {
     hipLaunchKernelGGL((sdpa_decode_kernel<T, D, G>), grid, dim3(kThreads), 0, s, p);
     if (p.nsplit > 1)
-        hipLaunchKernelGGL((sdpa_decode_merge_kernel<T, D, G>), dim3(grid.y, grid.z), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((sdpa_decode_merge_kernel<T, D, G>), dim3(grid.y, grid.z, G), dim3(D), 0, s, p);
 }
 
 template <typename T, int D>
@@ -494,7 +493,7 @@ void launch_ragged(const DecodeDev &p, const RaggedItem *items, int n_items, con
                    bool any_split, hipStream_t s) {
     hipLaunchKernelGGL((sdpa_decode_ragged_kernel<T, D, G>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
     if (any_split)
-        hipLaunchKernelGGL((sdpa_decode_ragged_merge_kernel<T, D, G>), dim3(p.Hkv, n_seq), dim3(kThreads), 0, s, p, seqs);
+        hipLaunchKernelGGL((sdpa_decode_ragged_merge_kernel<T, D, G>), dim3(p.Hkv, n_seq, G), dim3(D), 0, s, p, seqs);
 }
 
 template <typename T, int D>

@@ -334,7 +334,7 @@ template <int FMT, int G>
 int launch_one(const DecodeDev &p, dim3 grid, hipStream_t s) {
     hipLaunchKernelGGL((sdpa_decode_q_kernel<FMT, G>), grid, dim3(kThreads), 0, s, p);
     if (p.nsplit > 1)
-        hipLaunchKernelGGL((sdpa_decode_merge_kernel<__half, kD, G>), dim3(grid.y, grid.z), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((sdpa_decode_merge_kernel<__half, kD, G>), dim3(grid.y, grid.z, G), dim3(kD), 0, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("sdpa_decode (quantised KV) launch failed: %s", hipGetErrorString(e));
     return 0;
