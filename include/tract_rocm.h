@@ -162,6 +162,27 @@ int trocm_block_quant(int format, const void *src, int src_dtype, size_t n_elems
 int trocm_block_dequant(int format, const void *src_blocks, size_t n_elems, void *dst, int dst_dtype,
                         void *stream);
 
+/* ---- element-wise neighbours of the cache ------------------------------------------------- */
+
+/* Cast between F32 and F16 (core `Cast` as the GPU backends run it,
+ * cuda/src/kernels/array/cast.rs:21-47, :92): F32 -> F16 rounds to nearest even, F16 -> F32
+ * is exact, same type copies.  n_elems dense elements. */
+int trocm_cast(const void *src, int src_dtype, void *dst, int dst_dtype, size_t n_elems, void *stream);
+
+/* ApplyRope (transformers/src/ops/apply_rope.rs:169-176): out = x * cos + RotateHalf(x) * sin,
+ * every product and the sum rounded to `dtype` like the CPU op.  Rank 2..4, inner dimension
+ * even; strides in elements, NULL = dense.  cos and sin share `cos_sin_strides`, given for
+ * the input's rank with 0 on broadcast axes (what compute_broadcast_strides produces in
+ * cuda/src/kernels/nn/apply_rope.rs:75-81). */
+int trocm_apply_rope(const void *input, const void *cos, const void *sin, void *out, int dtype, int rank,
+                     const int64_t *shape, const int64_t *in_strides, const int64_t *cos_sin_strides,
+                     const int64_t *out_strides, void *stream);
+
+/* RotateHalf (transformers/src/ops/apply_rope.rs:58-76): out = concat(-x[.., h..], x[.., ..h])
+ * along the innermost axis, h = half of it.  Rank 1..4. */
+int trocm_rotate_half(const void *input, void *out, int dtype, int rank, const int64_t *shape,
+                      const int64_t *in_strides, const int64_t *out_strides, void *stream);
+
 /* ---- attention -------------------------------------------------------------------------- */
 
 /* Scratch for split-K partial results and arrival counters.  The arena planner of the

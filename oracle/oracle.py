@@ -42,6 +42,8 @@ def lib() -> C.CDLL:
         L.orc_f16_to_f32.argtypes = [C.c_uint16]
         L.orc_f32_to_f16_n.argtypes = [vp, vp, sz]
         L.orc_f16_to_f32_n.argtypes = [vp, vp, sz]
+        L.orc_rotate_half.argtypes = [i, vp, vp, sz, sz]
+        L.orc_apply_rope.argtypes = [i, vp, vp, vp, vp, i, vp, vp]
         L.orc_block_bytes.restype = sz
         L.orc_block_bytes.argtypes = [i]
         L.orc_quant.argtypes = [i, i, vp, sz, vp]
@@ -259,3 +261,32 @@ def decode_step_f16(q, k_past, v_past, k_new, v_new, threads=1):
 
 def max_threads() -> int:
     return lib().orc_max_threads()
+
+
+def rotate_half(x: np.ndarray) -> np.ndarray:
+    """RotateHalf (apply_rope.rs:58-76) on a dense f32/f16 array."""
+    x = np.ascontiguousarray(x)
+    out = np.empty_like(x)
+    inner = x.shape[-1]
+    lib().orc_rotate_half(int(x.dtype == np.float16), _p(x), _p(out), x.size // max(inner, 1), inner)
+    return out
+
+
+def apply_rope(x: np.ndarray, cos: np.ndarray, sin: np.ndarray) -> np.ndarray:
+    """ApplyRope (apply_rope.rs:169-176): x*cos + rotate_half(x)*sin in x's datum type; cos and
+    sin (same shape) broadcast against x numpy-style."""
+    x = np.ascontiguousarray(x)
+    assert cos.shape == sin.shape and cos.dtype == sin.dtype == x.dtype and 2 <= x.ndim <= 4
+    cos, sin = np.ascontiguousarray(cos), np.ascontiguousarray(sin)
+    pad = (1,) * (x.ndim - cos.ndim) + cos.shape
+    strides, acc = [], 1
+    for d in range(x.ndim - 1, -1, -1):
+        assert pad[d] in (1, x.shape[d])
+        strides.append(0 if pad[d] == 1 and x.shape[d] != 1 else acc)
+        acc *= pad[d]
+    strides = strides[::-1]
+    out = np.empty_like(x)
+    shp = (C.c_size_t * x.ndim)(*x.shape)
+    cs = (C.c_size_t * x.ndim)(*strides)
+    lib().orc_apply_rope(int(x.dtype == np.float16), _p(x), _p(cos), _p(sin), _p(out), x.ndim, shp, cs)
+    return out

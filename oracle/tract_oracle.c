@@ -25,6 +25,12 @@
  *                          crate matrixmultiply 0.3.10 whose summation order is not
  *                          part of the reference tree.
  *
+ *   RotateHalf / ApplyRope  pinned: RotateHalf twice == negation (the reference's own unit
+ *                          test, apply_rope.rs:257-277), an independent numpy
+ *                          concatenate form, the rotation closed forms (norm of each
+ *                          pair kept, angles add); f16 arithmetic is the `half` crate's
+ *                          (operate in f32, round to f16 after every operation)
+ *
  * Build: gcc -O2 -fno-fast-math -ffp-contract=off (Rust never contracts a*b+c).
  */
 #include <math.h>
@@ -637,4 +643,70 @@ ORC_API void orc_decode_step_f16(const uint16_t *q, const uint16_t *k_past, cons
     orc_flash_sdpa_eval_f16(q, kc, vc, NULL, B, Hq, Hkv, 1, T + 1, D, 1, 1, 1, 0, 0.0f, out, threads);
     *k_out = kc;
     *v_out = vc;
+}
+
+/* ------------------------------------------------------------------------- */
+/* RotateHalf and ApplyRope (transformers/src/ops/apply_rope.rs).              */
+/* Dense row-major input of shape[0..rank), rank <= 4; cos/sin given with      */
+/* element strides for the input's rank, 0 on broadcast axes.                  */
+/* ------------------------------------------------------------------------- */
+
+/* f16 * f16 and f16 + f16 as crate `half` computes them without native fp16
+ * arithmetic: widen, operate in f32, round to f16. */
+static inline uint16_t h_mul(uint16_t a, uint16_t b) { return orc_f32_to_f16(orc_f16_to_f32(a) * orc_f16_to_f32(b)); }
+static inline uint16_t h_add(uint16_t a, uint16_t b) { return orc_f32_to_f16(orc_f16_to_f32(a) + orc_f16_to_f32(b)); }
+
+/* apply_rope.rs:58-76: tensor[.., 0..h] = -input[.., h..]; tensor[.., h..] = input[.., 0..h] */
+ORC_API void orc_rotate_half(int is_f16, const void *in, void *out, size_t rows, size_t inner) {
+    size_t h = inner / 2;
+    for (size_t r = 0; r < rows; r++) {
+        if (is_f16) {
+            const uint16_t *x = (const uint16_t *)in + r * inner;
+            uint16_t *y = (uint16_t *)out + r * inner;
+            for (size_t i = 0; i < h; i++) {
+                y[i] = (uint16_t)(x[i + h] ^ 0x8000u); /* Neg flips the sign bit */
+                y[i + h] = x[i];
+            }
+        } else {
+            const float *x = (const float *)in + r * inner;
+            float *y = (float *)out + r * inner;
+            for (size_t i = 0; i < h; i++) {
+                y[i] = -x[i + h];
+                y[i + h] = x[i];
+            }
+        }
+    }
+}
+
+/* apply_rope.rs:169-176: Add(Mul(input, cos), Mul(RotateHalf(input), sin)), each op in the
+ * input's datum type with numpy-style broadcasting of cos and sin. */
+ORC_API void orc_apply_rope(int is_f16, const void *in, const void *cosv, const void *sinv, void *out, int rank,
+                            const size_t *shape, const size_t *cs_strides) {
+    size_t sh[4] = {1, 1, 1, 1}, cs[4] = {0, 0, 0, 0};
+    for (int d = 0; d < rank; d++) {
+        sh[4 - rank + d] = shape[d];
+        cs[4 - rank + d] = cs_strides[d];
+    }
+    size_t inner = sh[3], h = inner / 2;
+    size_t rows = sh[0] * sh[1] * sh[2];
+    void *rot = malloc(rows * inner * (is_f16 ? 2 : 4));
+    orc_rotate_half(is_f16, in, rot, rows, inner);
+    (void)h;
+    for (size_t i0 = 0; i0 < sh[0]; i0++)
+        for (size_t i1 = 0; i1 < sh[1]; i1++)
+            for (size_t i2 = 0; i2 < sh[2]; i2++)
+                for (size_t i3 = 0; i3 < sh[3]; i3++) {
+                    size_t e = ((i0 * sh[1] + i1) * sh[2] + i2) * sh[3] + i3;
+                    size_t c = i0 * cs[0] + i1 * cs[1] + i2 * cs[2] + i3 * cs[3];
+                    if (is_f16) {
+                        const uint16_t *x = in, *r = rot, *co = cosv, *si = sinv;
+                        ((uint16_t *)out)[e] = h_add(h_mul(x[e], co[c]), h_mul(r[e], si[c]));
+                    } else {
+                        const float *x = in, *r = rot, *co = cosv, *si = sinv;
+                        float a = x[e] * co[c];
+                        float b = r[e] * si[c];
+                        ((float *)out)[e] = a + b;
+                    }
+                }
+    free(rot);
 }

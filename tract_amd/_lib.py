@@ -61,6 +61,9 @@ SIGNATURES = {
     "trocm_kv_cache_raw": [_vp, C.POINTER(_vp), C.POINTER(_vp), _pi64],
     "trocm_block_quant": [_i, _vp, _i, _sz, _vp, _vp],
     "trocm_block_dequant": [_i, _vp, _sz, _vp, _i, _vp],
+    "trocm_cast": [_vp, _i, _vp, _i, _sz, _vp],
+    "trocm_apply_rope": [_vp, _vp, _vp, _vp, _i, _i, _pi64, _pi64, _pi64, _pi64, _vp],
+    "trocm_rotate_half": [_vp, _vp, _i, _i, _pi64, _pi64, _pi64, _vp],
     "trocm_sdpa_workspace_bytes": [_i64, _i64, _i64, _i64, C.POINTER(_sz)],
     "trocm_sdpa_workspace_init": [_vp, _sz, _vp],
     "trocm_sdpa": [_vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i64, _i64, _i64, _i64, _pi64, _i64, _i64, _f, _i,

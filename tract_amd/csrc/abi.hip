@@ -668,6 +668,57 @@ int trocm_block_dequant(int format, const void *src_blocks, size_t n_elems, void
     return launch_block_dequant(format, src_blocks, n_elems, dst, dst_dtype, s);
 }
 
+// ---- element-wise neighbours: cast, RotateHalf, ApplyRope ---------------------------------------
+int trocm_cast(const void *src, int src_dtype, void *dst, int dst_dtype, size_t n_elems, void *stream) {
+    TROCM_REQUIRE((src_dtype == TROCM_F32 || src_dtype == TROCM_F16) && (dst_dtype == TROCM_F32 || dst_dtype == TROCM_F16),
+                  "cast: only F32 and F16 are handled here (got %d -> %d)", src_dtype, dst_dtype);
+    if (n_elems == 0) return 0;
+    TROCM_NOT_NULL(src);
+    TROCM_NOT_NULL(dst);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    return launch_cast(src, src_dtype, dst, dst_dtype, n_elems, s);
+}
+
+static int rope_common(const void *input, const void *cos, const void *sin, void *out, int dtype, int rank,
+                       const int64_t *shape, const int64_t *in_strides, const int64_t *cs_strides,
+                       const int64_t *out_strides, int rotate_only, void *stream) {
+    const char *what = rotate_only ? "rotate_half" : "apply_rope";
+    TROCM_REQUIRE(dtype == TROCM_F32 || dtype == TROCM_F16, "Unsupported dt %d for %s", dtype, what);
+    TROCM_NOT_NULL(shape);
+    // apply_rope.rs (cuda kernels) :72-73: rank 2..4; RotateHalf takes any rank >= 1 (here up to 4)
+    TROCM_REQUIRE(rank >= (rotate_only ? 1 : 2) && rank <= 4, "%s: unsupported rank %d", what, rank);
+    int64_t n = 1;
+    for (int d = 0; d < rank; d++) {
+        TROCM_REQUIRE(shape[d] >= 0, "%s: negative dimension", what);
+        n *= shape[d];
+    }
+    TROCM_REQUIRE(shape[rank - 1] % 2 == 0,
+                  "RotateHalf possible only if the most inner dimension of the shape is divisible by 2 (got %lld)",
+                  (long long)shape[rank - 1]);  // apply_rope.rs:64-68
+    if (n == 0) return 0;
+    TROCM_NOT_NULL(input);
+    TROCM_NOT_NULL(out);
+    if (!rotate_only) {
+        TROCM_NOT_NULL(cos);
+        TROCM_NOT_NULL(sin);
+    }
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    return launch_apply_rope(input, cos, sin, out, dtype, rank, shape, in_strides, cs_strides, out_strides, rotate_only, s);
+}
+
+int trocm_apply_rope(const void *input, const void *cos, const void *sin, void *out, int dtype, int rank,
+                     const int64_t *shape, const int64_t *in_strides, const int64_t *cos_sin_strides,
+                     const int64_t *out_strides, void *stream) {
+    return rope_common(input, cos, sin, out, dtype, rank, shape, in_strides, cos_sin_strides, out_strides, 0, stream);
+}
+
+int trocm_rotate_half(const void *input, void *out, int dtype, int rank, const int64_t *shape,
+                      const int64_t *in_strides, const int64_t *out_strides, void *stream) {
+    return rope_common(input, nullptr, nullptr, out, dtype, rank, shape, in_strides, nullptr, out_strides, 1, stream);
+}
+
 // ---- attention -----------------------------------------------------------------------------------
 int trocm_sdpa_workspace_bytes(int64_t batch, int64_t q_heads, int64_t q_len, int64_t head_dim, size_t *bytes) {
     TROCM_NOT_NULL(bytes);

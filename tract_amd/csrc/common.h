@@ -93,6 +93,13 @@ int launch_quant_export(int fmt, int64_t B, int64_t H, int64_t len, int64_t cap,
 int launch_block_quant(int fmt, const void *src, int src_dtype, size_t n_elems, void *dst, hipStream_t s);
 int launch_block_dequant(int fmt, const void *blocks, size_t n_elems, void *dst, int dst_dtype, hipStream_t s);
 
+// Element-wise neighbours of the cache: cast f32 <-> f16, RotateHalf, ApplyRope (rank <= 4, element
+// strides, NULL = dense; cos/sin strides are 0 on broadcast axes).
+int launch_cast(const void *src, int src_dtype, void *dst, int dst_dtype, size_t n, hipStream_t s);
+int launch_apply_rope(const void *x, const void *cos, const void *sin, void *y, int dtype, int rank,
+                      const int64_t *shape, const int64_t *in_strides, const int64_t *cs_strides,
+                      const int64_t *out_strides, int rotate_only, hipStream_t s);
+
 // Attention.  One description for every kernel.
 struct SdpaArgs {
     const void *q;

@@ -9,6 +9,9 @@ parity tests read like tract's own unit tests:
   gpu/src/ops/dyn_kv_cache.rs:8-125), here backed by the in-place cache
 * ``Sdpa``                transformers/src/ops/sdpa.rs:83-89, 296-356
 * ``BlockQuant``          linalg/src/frame/block_quant/mod.rs:36-108 (Q4_0; Q8_0 = Q8_1 without sum)
+* ``ApplyRope``/``RotateHalf`` transformers/src/ops/apply_rope.rs:44-86, 150-188 (device twin:
+  cuda/src/kernels/nn/apply_rope.rs:41-129)
+* ``Cast``                cuda/src/kernels/array/cast.rs:17-90 (f32 <-> f16 only)
 """
 from __future__ import annotations
 
@@ -472,3 +475,87 @@ def inplace_kv_sdpa_eval_ragged(q: DeviceTensor, k_new: DeviceTensor, v_new: Dev
     call("trocm_inplace_kv_sdpa_eval_ragged", q.ptr, k_new.ptr, v_new.ptr, dtype_code(q.dtype), Hq, n, ks, vs,
          out.ptr, _scale_arg(scale), ws.ptr, ws.nbytes, _sh(stream))
     return out
+
+
+def _broadcast_strides(x_shape, c_shape):
+    """Element strides of a dense tensor of shape ``c_shape`` broadcast against ``x_shape``
+    (0 on broadcast axes), for x's rank: cuda/src/kernels/utils.rs compute_broadcast_strides."""
+    if len(c_shape) > len(x_shape):
+        raise TractRocmError("cos/sin rank exceeds the input rank")
+    pad = (1,) * (len(x_shape) - len(c_shape)) + tuple(c_shape)
+    out, acc = [], 1
+    for d in range(len(x_shape) - 1, -1, -1):
+        if pad[d] not in (1, x_shape[d]):
+            raise TractRocmError(f"cos/sin shape {tuple(c_shape)} does not broadcast against {tuple(x_shape)}")
+        out.append(0 if pad[d] == 1 and x_shape[d] != 1 else acc)
+        acc *= pad[d]
+    return out[::-1]
+
+
+class RotateHalf:
+    """Y = Concat(Neg(Slice(X, h.., -1)), Slice(X, ..h, -1)), h = half the innermost axis."""
+
+    def name(self) -> str:
+        return "RotateHalf"
+
+    def is_stateless(self) -> bool:
+        return True
+
+    def output_facts(self, shape):
+        return tuple(shape)
+
+    def eval(self, x, stream=None) -> DeviceTensor:
+        x = _as_device(x, stream)
+        out = DeviceTensor(x.shape, x.dtype)
+        shp = (C.c_int64 * len(x.shape))(*x.shape)
+        call("trocm_rotate_half", x.ptr, out.ptr, dtype_code(x.dtype), len(x.shape), shp, None, None, _sh(stream))
+        return out
+
+
+class ApplyRope:
+    """Y = X * Cos + RotateHalf(X) * Sin, inputs [X, Cos, Sin]; Cos and Sin share a shape that
+    broadcasts against X."""
+
+    @staticmethod
+    def is_supported_dt(dt) -> bool:
+        return np.dtype(dt) in (np.dtype(np.float32), np.dtype(np.float16))
+
+    def name(self) -> str:
+        return "ApplyRope"
+
+    def is_stateless(self) -> bool:
+        return True
+
+    def output_facts(self, x_shape, cos_shape=None, sin_shape=None):
+        return tuple(x_shape)
+
+    def eval(self, x, cos, sin, stream=None, out: DeviceTensor | None = None) -> DeviceTensor:
+        x, cos, sin = (_as_device(t, stream) for t in (x, cos, sin))
+        if not (x.dtype == cos.dtype == sin.dtype):
+            raise TractRocmError("input, cos and sin must share a datum type")
+        if tuple(cos.shape) != tuple(sin.shape):
+            raise TractRocmError("cos and sin must have the same shape")
+        cs = _broadcast_strides(x.shape, cos.shape)
+        if out is None:
+            out = DeviceTensor(x.shape, x.dtype)
+        n = len(x.shape)
+        call("trocm_apply_rope", x.ptr, cos.ptr, sin.ptr, out.ptr, dtype_code(x.dtype), n, (C.c_int64 * n)(*x.shape),
+             None, (C.c_int64 * n)(*cs), None, _sh(stream))
+        return out
+
+
+class Cast:
+    """Cast between f32 and f16 (round to nearest even on the way down)."""
+
+    def __init__(self, to):
+        self.to = np.dtype(to)
+
+    def name(self) -> str:
+        return "Cast"
+
+    def eval(self, x, stream=None) -> DeviceTensor:
+        x = _as_device(x, stream)
+        out = DeviceTensor(x.shape, self.to)
+        call("trocm_cast", x.ptr, dtype_code(x.dtype), out.ptr, dtype_code(self.to), int(np.prod(x.shape, dtype=np.int64)),
+             _sh(stream))
+        return out
