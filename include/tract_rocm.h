@@ -116,6 +116,15 @@ int trocm_kv_cache_create(trocm_kv_cache **out, int storage_format, int64_t batc
                           int64_t head_dim);
 int trocm_kv_cache_create_in_pool(trocm_kv_cache **out, trocm_kv_pool *pool, int storage_format,
                                   int64_t batch, int64_t kv_heads, int64_t head_dim);
+/* WindowKvCache::new (transformers/src/ops/window_kv_cache.rs:80-93): a fixed-capacity ring
+ * buffer of `window` token slots for models trained with sliding-window attention.  Appends
+ * overwrite the oldest slots once full (push, :111-143); len() <= window; the valid slots
+ * are [0, len) in physical (rotated) order, which is all decode attention needs.  The
+ * buffer is allocated at the first append; reserve and truncate are refused. */
+int trocm_kv_cache_create_window(trocm_kv_cache **out, int storage_format, int64_t batch, int64_t kv_heads,
+                                 int64_t head_dim, int64_t window);
+/* window (0 for an ordinary cache) and the next write position. */
+int trocm_kv_cache_window(const trocm_kv_cache *cache, int64_t *window, int64_t *cursor);
 int trocm_kv_cache_destroy(trocm_kv_cache *cache);
 /* len() / capacity() / reallocs() (:41-53). */
 int trocm_kv_cache_len(const trocm_kv_cache *cache, int64_t *len);
@@ -228,6 +237,14 @@ int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_n
                                int64_t q_heads, int64_t n_new, const int64_t *kv_new_strides,
                                trocm_kv_cache *k_cache, trocm_kv_cache *v_cache, void *out, float scale,
                                int causal, void *workspace, size_t workspace_bytes, void *stream);
+
+/* WindowKvSdpaState::eval (transformers/src/ops/window_kv_cache.rs:216-239): append K_new and
+ * V_new to the two sliding-window caches, then attend Q to every valid slot without a causal
+ * mask (the ring buffer is the window).  Arguments as trocm_inplace_kv_sdpa_eval. */
+int trocm_window_kv_sdpa_eval(const void *q, const void *k_new, const void *v_new, int dtype, int64_t q_heads,
+                              int64_t n_new, const int64_t *kv_new_strides, trocm_kv_cache *k_cache,
+                              trocm_kv_cache *v_cache, void *out, float scale, void *workspace,
+                              size_t workspace_bytes, void *stream);
 
 /* Ragged multi-sequence decode: `n_seq` independent sequences, each with its own K and V
  * cache (batch == 1 each, same heads/head_dim/format) and its own length; one query token

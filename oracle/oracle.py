@@ -42,6 +42,15 @@ def lib() -> C.CDLL:
         L.orc_f16_to_f32.argtypes = [C.c_uint16]
         L.orc_f32_to_f16_n.argtypes = [vp, vp, sz]
         L.orc_f16_to_f32_n.argtypes = [vp, vp, sz]
+        L.orc_win_new.restype = vp
+        L.orc_win_new.argtypes = [sz, sz, sz]
+        L.orc_win_free.argtypes = [vp]
+        for n in ("len", "cursor", "capacity"):
+            fn = getattr(L, "orc_win_" + n)
+            fn.restype = sz
+            fn.argtypes = [vp]
+        L.orc_win_push.argtypes = [vp, vp, sz]
+        L.orc_win_valid.argtypes = [vp, vp]
         L.orc_rotate_half.argtypes = [i, vp, vp, sz, sz]
         L.orc_apply_rope.argtypes = [i, vp, vp, vp, vp, i, vp, vp]
         L.orc_block_bytes.restype = sz
@@ -290,3 +299,40 @@ def apply_rope(x: np.ndarray, cos: np.ndarray, sin: np.ndarray) -> np.ndarray:
     cs = (C.c_size_t * x.ndim)(*strides)
     lib().orc_apply_rope(int(x.dtype == np.float16), _p(x), _p(cos), _p(sin), _p(out), x.ndim, shp, cs)
     return out
+
+
+class WindowKvCache:
+    """WindowKvCache (window_kv_cache.rs:80-154) over [B, H, S, D] arrays, token axis 2."""
+
+    def __init__(self, window: int):
+        assert window > 0
+        self.window, self._h, self._like = window, None, None
+
+    def push(self, x: np.ndarray) -> None:
+        x = np.ascontiguousarray(x)
+        if x.shape[2] == 0:
+            return
+        if self._h is None:
+            self._like = (x.shape, x.dtype)
+            self._h = lib().orc_win_new(x.shape[0] * x.shape[1], self.window, x.shape[3] * x.dtype.itemsize)
+        lib().orc_win_push(self._h, _p(x), x.shape[2])
+
+    def len(self) -> int:
+        return 0 if self._h is None else lib().orc_win_len(self._h)
+
+    def cursor(self) -> int:
+        return 0 if self._h is None else lib().orc_win_cursor(self._h)
+
+    def capacity(self) -> int:
+        return 0 if self._h is None else lib().orc_win_capacity(self._h)
+
+    def valid_view(self) -> np.ndarray:
+        shape, dt = self._like
+        out = np.empty((shape[0], shape[1], self.len(), shape[3]), dt)
+        lib().orc_win_valid(self._h, _p(out))
+        return out
+
+    def __del__(self):
+        if self._h is not None and _lib is not None:
+            _lib.orc_win_free(self._h)
+            self._h = None

@@ -25,6 +25,10 @@
  *                          crate matrixmultiply 0.3.10 whose summation order is not
  *                          part of the reference tree.
  *
+ *   window (ring) cache     pinned: the reference's unit tests (window_kv_cache.rs:342-374:
+ *                          last-w-as-a-set, chunk larger than the window), hand-derived
+ *                          slot layouts for the wrap-around case, windowed attention ==
+ *                          attention over the last w tokens (:407-466)
  *   RotateHalf / ApplyRope  pinned: RotateHalf twice == negation (the reference's own unit
  *                          test, apply_rope.rs:257-277), an independent numpy
  *                          concatenate form, the rotation closed forms (norm of each
@@ -709,4 +713,64 @@ ORC_API void orc_apply_rope(int is_f16, const void *in, const void *cosv, const 
                     }
                 }
     free(rot);
+}
+
+/* ------------------------------------------------------------------------- */
+/* WindowKvCache (transformers/src/ops/window_kv_cache.rs:80-154): ring buffer  */
+/* of `window` rows per (batch, head); rows are opaque byte strings.            */
+/* ------------------------------------------------------------------------- */
+typedef struct {
+    size_t outer, window, row_bytes, len, cursor;
+    unsigned char *buf; /* [outer][window][row_bytes], allocated on first push */
+} orc_win;
+
+ORC_API orc_win *orc_win_new(size_t outer, size_t window, size_t row_bytes) {
+    orc_win *c = (orc_win *)calloc(1, sizeof(orc_win));
+    c->outer = outer, c->window = window, c->row_bytes = row_bytes;
+    return c;
+}
+ORC_API void orc_win_free(orc_win *c) {
+    if (c) free(c->buf);
+    free(c);
+}
+ORC_API size_t orc_win_len(const orc_win *c) { return c->len; }
+ORC_API size_t orc_win_cursor(const orc_win *c) { return c->cursor; }
+ORC_API size_t orc_win_capacity(const orc_win *c) { return c->buf ? c->window : 0; } /* :98-100 */
+
+/* buf[.., dst0 .. dst0+n) = src[.., src0 .. src0+n) along the token axis (assign_slice) */
+static void win_assign(orc_win *c, size_t dst0, const unsigned char *src, size_t n_new, size_t src0, size_t n) {
+    for (size_t o = 0; o < c->outer; o++)
+        memcpy(c->buf + (o * c->window + dst0) * c->row_bytes, src + (o * n_new + src0) * c->row_bytes, n * c->row_bytes);
+}
+
+/* push, :111-143.  src is [outer][n_new][row_bytes]. */
+ORC_API void orc_win_push(orc_win *c, const void *srcv, size_t n_new) {
+    const unsigned char *src = (const unsigned char *)srcv;
+    if (n_new == 0) return;                                                       /* :113-115 */
+    if (!c->buf) c->buf = (unsigned char *)malloc(c->outer * c->window * c->row_bytes); /* :101-108 */
+    size_t w = c->window;
+    if (n_new >= w) {                                                             /* :119-126 */
+        win_assign(c, 0, src, n_new, n_new - w, w);
+        c->cursor = 0;
+        c->len = w;
+        return;
+    }
+    size_t end = c->cursor + n_new;                                               /* :129 */
+    if (end <= w) {
+        win_assign(c, c->cursor, src, n_new, 0, n_new);
+        c->cursor = end == w ? 0 : end;
+    } else {
+        size_t first = w - c->cursor;
+        win_assign(c, c->cursor, src, n_new, 0, first);
+        win_assign(c, 0, src, n_new, first, n_new - first);
+        c->cursor = n_new - first;
+    }
+    c->len = c->len + n_new < w ? c->len + n_new : w;                             /* :141 */
+}
+
+/* valid_view, :145-152: slots [0, len) in physical order, copied out dense [outer][len][row_bytes] */
+ORC_API void orc_win_valid(const orc_win *c, void *dstv) {
+    unsigned char *dst = (unsigned char *)dstv;
+    for (size_t o = 0; o < c->outer; o++)
+        memcpy(dst + o * c->len * c->row_bytes, c->buf + o * c->window * c->row_bytes, c->len * c->row_bytes);
 }

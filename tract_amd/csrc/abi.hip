@@ -127,6 +127,9 @@ struct trocm_kv_cache {
     void *data;    // F32/F16 rows, or the code plane
     void *scales;  // f16 scale plane of the quantised formats
     trocm_kv_pool *pool;  // where the planes live; NULL = their own hipMalloc
+    // sliding-window (ring buffer) mode, window_kv_cache.rs:80-87: capacity fixed at `window`,
+    // `cursor` = next write position; 0 = ordinary growing cache
+    int64_t window, cursor;
 };
 
 static int plane_alloc(trocm_kv_cache *c, void **ptr, size_t bytes, const char *what) {
@@ -390,7 +393,23 @@ int trocm_kv_cache_create(trocm_kv_cache **out, int fmt, int64_t batch, int64_t 
     c->len = c->cap = c->reallocs = 0;
     c->data = c->scales = nullptr;
     c->pool = nullptr;
+    c->window = c->cursor = 0;
     *out = c;
+    return 0;
+}
+
+int trocm_kv_cache_create_window(trocm_kv_cache **out, int fmt, int64_t batch, int64_t kv_heads, int64_t head_dim,
+                                 int64_t window) {
+    TROCM_REQUIRE(window > 0, "window must be > 0");  // window_kv_cache.rs:91
+    if (trocm_kv_cache_create(out, fmt, batch, kv_heads, head_dim)) return 1;
+    (*out)->window = window;
+    return 0;
+}
+
+int trocm_kv_cache_window(const trocm_kv_cache *c, int64_t *window, int64_t *cursor) {
+    TROCM_NOT_NULL(c);
+    if (window) *window = c->window;
+    if (cursor) *cursor = c->cursor;
     return 0;
 }
 
@@ -479,6 +498,7 @@ int trocm_kv_cache_reallocs(const trocm_kv_cache *c, int64_t *reallocs) {
 int trocm_kv_cache_reserve(trocm_kv_cache *c, int64_t capacity, void *stream) {
     TROCM_NOT_NULL(c);
     TROCM_REQUIRE(capacity >= 0, "reserve: negative capacity");
+    TROCM_REQUIRE(c->window == 0, "reserve: a sliding-window cache has a fixed capacity of %lld", (long long)c->window);
     if (capacity <= c->cap) return 0;
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
@@ -494,6 +514,10 @@ static int append_prepare(trocm_kv_cache *c, const void *src, int src_dtype, con
     TROCM_REQUIRE(is_quant(c->fmt) || src_dtype == c->fmt,
                   "append: source dtype %d does not match the cache's storage format %d", src_dtype, c->fmt);
     for (int i = 0; i < 4; i++) TROCM_REQUIRE(src_strides[i] >= 0, "append: negative source strides are not supported");
+    if (c->window) {  // window_kv_cache.rs:101-108: the ring buffer is allocated once, at the window
+        if (c->cap == 0 && regrow(c, c->window, s)) return 1;
+        return 0;
+    }
     if (c->cap == 0) {
         if (regrow(c, n_new, s)) return 1;
     } else if (c->len + n_new > c->cap) {
@@ -504,15 +528,16 @@ static int append_prepare(trocm_kv_cache *c, const void *src, int src_dtype, con
     return 0;
 }
 
-// Write the new tokens at [len, len + n_new) (capacity is already sufficient).
-static int append_write(trocm_kv_cache *c, const void *src, int src_dtype, const int64_t *src_strides, int64_t n_new,
-                        hipStream_t s) {
+// Write source tokens [s0, s0 + n_new) at cache positions [t0, t0 + n_new) (inside the capacity).
+static int append_write_at(trocm_kv_cache *c, const void *src0, int src_dtype, const int64_t *src_strides, int64_t s0,
+                           int64_t n_new, int64_t t0, hipStream_t s) {
+    const void *src = (const char *)src0 + s0 * src_strides[2] * (int64_t)elem_bytes(src_dtype);
     if (is_quant(c->fmt)) {
         QuantAppend a;
         a.fmt = c->fmt, a.src_dtype = src_dtype;
         a.B = c->B, a.H = c->H, a.S = n_new, a.D = c->D;
         for (int i = 0; i < 4; i++) a.ss[i] = src_strides[i];
-        a.cap = c->cap, a.t0 = c->len;
+        a.cap = c->cap, a.t0 = t0;
         a.src = src, a.codes = c->data, a.scales = c->scales;
         return launch_quant_append(a, s);
     }
@@ -525,7 +550,37 @@ static int append_write(trocm_kv_cache *c, const void *src, int src_dtype, const
     d.dst_stride[1] = c->cap * c->D * es;
     d.dst_stride[2] = c->D * es;
     d.dst_stride[3] = es;
-    return launch_copy_nd((char *)c->data + c->len * c->D * es, src, d, (int)es, s);
+    return launch_copy_nd((char *)c->data + t0 * c->D * es, src, d, (int)es, s);
+}
+
+// Ring-buffer push of a sliding-window cache (window_kv_cache.rs:111-143).
+static int window_write(trocm_kv_cache *c, const void *src, int src_dtype, const int64_t *src_strides, int64_t n_new,
+                        hipStream_t s) {
+    const int64_t w = c->window;
+    if (n_new >= w) {  // only the last w tokens survive, laid out [0, w); the cursor resets
+        if (append_write_at(c, src, src_dtype, src_strides, n_new - w, w, 0, s)) return 1;
+        c->cursor = 0;
+        c->len = w;
+        return 0;
+    }
+    const int64_t end = c->cursor + n_new;
+    if (end <= w) {
+        if (append_write_at(c, src, src_dtype, src_strides, 0, n_new, c->cursor, s)) return 1;
+        c->cursor = end == w ? 0 : end;
+    } else {
+        const int64_t first = w - c->cursor;
+        if (append_write_at(c, src, src_dtype, src_strides, 0, first, c->cursor, s)) return 1;
+        if (append_write_at(c, src, src_dtype, src_strides, first, n_new - first, 0, s)) return 1;
+        c->cursor = n_new - first;
+    }
+    c->len = c->len + n_new < w ? c->len + n_new : w;
+    return 0;
+}
+
+// Write the new tokens at [len, len + n_new) (capacity is already sufficient).
+static int append_write(trocm_kv_cache *c, const void *src, int src_dtype, const int64_t *src_strides, int64_t n_new,
+                        hipStream_t s) {
+    return append_write_at(c, src, src_dtype, src_strides, 0, n_new, c->len, s);
 }
 
 int trocm_kv_append(trocm_kv_cache *c, const void *src, int src_dtype, const int64_t *src_strides, int64_t n_new,
@@ -536,6 +591,7 @@ int trocm_kv_append(trocm_kv_cache *c, const void *src, int src_dtype, const int
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
     if (append_prepare(c, src, src_dtype, src_strides, n_new, s)) return 1;
+    if (c->window) return window_write(c, src, src_dtype, src_strides, n_new, s);
     if (append_write(c, src, src_dtype, src_strides, n_new, s)) return 1;
     c->len += n_new;
     return 0;
@@ -551,8 +607,13 @@ int trocm_kv_append_pair(trocm_kv_cache *kc, trocm_kv_cache *vc, const void *k_s
     if (n_new == 0) return 0;
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
+    TROCM_REQUIRE(kc->window == vc->window, "K and V caches differ in window");
     if (append_prepare(kc, k_src, src_dtype, src_strides, n_new, s)) return 1;
     if (append_prepare(vc, v_src, src_dtype, src_strides, n_new, s)) return 1;
+    if (kc->window) {
+        if (window_write(kc, k_src, src_dtype, src_strides, n_new, s)) return 1;
+        return window_write(vc, v_src, src_dtype, src_strides, n_new, s);
+    }
     int rc = 2;
     if (!is_quant(kc->fmt) && src_strides[3] == 1 && kc->cap == vc->cap && kc->len == vc->len) {
         int64_t es = (int64_t)elem_bytes(kc->fmt);
@@ -578,6 +639,7 @@ int trocm_kv_append_pair(trocm_kv_cache *kc, trocm_kv_cache *vc, const void *k_s
 int trocm_kv_cache_truncate(trocm_kv_cache *c, int64_t len) {
     TROCM_NOT_NULL(c);
     TROCM_REQUIRE(c->data != nullptr, "Can not truncate a zero-len kv-cache value");  // dyn_kv_cache.rs:112-119
+    TROCM_REQUIRE(c->window == 0, "truncate: a sliding-window cache does not keep its tokens in order");
     TROCM_REQUIRE(len >= 0 && len <= c->len, "truncate: length %lld out of range 0..=%lld", (long long)len,
                   (long long)c->len);
     c->len = len;
@@ -631,6 +693,7 @@ int trocm_kv_cache_clone(const trocm_kv_cache *c, trocm_kv_cache **out, void *st
     }
     n->len = c->len;
     n->reallocs = c->reallocs;
+    n->window = c->window, n->cursor = c->cursor;
     *out = n;
     return 0;
 }
@@ -855,7 +918,7 @@ int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_n
     // Decode step on a plain-format cache: the attention kernel reads the new token from the
     // inputs and stores it into the cache itself -- one launch instead of append + attention.
     if (n_new == 1 && is_dense && !is_quant(kc->fmt) && dtype == kc->fmt && q && k_new && v_new && out &&
-        kc->fmt == vc->fmt && kc->B == vc->B && kc->H == vc->H && kc->D == vc->D && kc->len == vc->len &&
+        kc->window == 0 && vc->window == 0 && kc->fmt == vc->fmt && kc->B == vc->B && kc->H == vc->H && kc->D == vc->D && kc->len == vc->len &&
         q_heads % kc->H == 0) {
         hipStream_t s;
         if (resolve_stream(stream, &s)) return 1;
@@ -876,6 +939,22 @@ int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_n
     }
     if (trocm_kv_append_pair(kc, vc, k_new, v_new, dtype, kv_new_strides, n_new, stream)) return 1;
     return trocm_sdpa_cached(q, dtype, q_heads, n_new, kc, vc, out, scale, causal, workspace, workspace_bytes, stream);
+}
+
+// WindowKvSdpaState::eval (window_kv_cache.rs:216-239): push K_new / V_new into the ring buffers,
+// then attend to every valid slot in physical order without a causal mask -- the ring buffer
+// already bounds which keys are visible, and attention does not depend on the order of the keys.
+int trocm_window_kv_sdpa_eval(const void *q, const void *k_new, const void *v_new, int dtype, int64_t q_heads,
+                              int64_t n_new, const int64_t *kv_new_strides, trocm_kv_cache *kc, trocm_kv_cache *vc,
+                              void *out, float scale, void *workspace, size_t workspace_bytes, void *stream) {
+    TROCM_NOT_NULL(kc);
+    TROCM_NOT_NULL(vc);
+    TROCM_REQUIRE(kc->window > 0 && vc->window == kc->window, "window_kv_sdpa: K and V must be sliding-window caches of one window");
+    int64_t dense[4];
+    dense[3] = 1, dense[2] = kc->D, dense[1] = n_new * kc->D, dense[0] = kc->H * n_new * kc->D;
+    if (!kv_new_strides) kv_new_strides = dense;
+    if (trocm_kv_append_pair(kc, vc, k_new, v_new, dtype, kv_new_strides, n_new, stream)) return 1;
+    return trocm_sdpa_cached(q, dtype, q_heads, n_new, kc, vc, out, scale, 0, workspace, workspace_bytes, stream);
 }
 
 static int ragged_common(const void *q, const void *k_new, const void *v_new, int q_dtype, int64_t q_heads,
@@ -902,6 +981,8 @@ static int ragged_common(const void *q, const void *k_new, const void *v_new, in
                           vc->D == k0->D,
                       "ragged decode: caches differ in format or shape (sequence %lld)", (long long)i);
         TROCM_REQUIRE(kc->len == vc->len, "K/V lengths must match (sequence %lld)", (long long)i);
+        TROCM_REQUIRE(!fused || (kc->window == 0 && vc->window == 0),
+                      "ragged fused step: sliding-window caches are not supported (sequence %lld)", (long long)i);
     }
     TROCM_REQUIRE(q_heads % k0->H == 0, "Q heads (%lld) must be a multiple of K/V heads (%lld)", (long long)q_heads,
                   (long long)k0->H);

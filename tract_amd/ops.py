@@ -9,6 +9,7 @@ parity tests read like tract's own unit tests:
   gpu/src/ops/dyn_kv_cache.rs:8-125), here backed by the in-place cache
 * ``Sdpa``                transformers/src/ops/sdpa.rs:83-89, 296-356
 * ``BlockQuant``          linalg/src/frame/block_quant/mod.rs:36-108 (Q4_0; Q8_0 = Q8_1 without sum)
+* ``WindowKvCache``, ``WindowKvSdpa``/State transformers/src/ops/window_kv_cache.rs:80-154, 156-239
 * ``ApplyRope``/``RotateHalf`` transformers/src/ops/apply_rope.rs:44-86, 150-188 (device twin:
   cuda/src/kernels/nn/apply_rope.rs:41-129)
 * ``Cast``                cuda/src/kernels/array/cast.rs:17-90 (f32 <-> f16 only)
@@ -195,6 +196,44 @@ class InPlaceKvCache:
         return self._h
 
 
+class WindowKvCache(InPlaceKvCache):
+    """Fixed-capacity sliding-window KV cache (ring buffer) along `axis`: once `window` slots are
+    full an append overwrites the oldest; the valid slots are [0, len) in physical order."""
+
+    def __init__(self, axis: int, window: int, storage_format: int | None = None):
+        if window <= 0:
+            raise TractRocmError("window must be > 0")
+        super().__init__(axis, storage_format)
+        self.window = window
+
+    def _create(self, shape, dtype):
+        if self.axis != len(shape) - 2:
+            raise TractRocmError(f"kv-cache axis {self.axis} unsupported: the token axis must be rank-2")
+        B, H, _, D = _canon4(shape)
+        fmt = dtype_code(dtype) if self.storage_format is None else self.storage_format
+        h = C.c_void_p()
+        call("trocm_kv_cache_create_window", C.byref(h), fmt, B, H, D, self.window)
+        self._h, self._shape, self._dtype, self.storage_format = h, tuple(shape), np.dtype(dtype), fmt
+
+    def cursor(self) -> int:
+        if self._h is None:
+            return 0
+        w, c = C.c_int64(), C.c_int64()
+        call("trocm_kv_cache_window", self._h, C.byref(w), C.byref(c))
+        return c.value
+
+    def valid_view(self, stream=None) -> np.ndarray:
+        return self.valid_contiguous(stream)
+
+    def clone(self, stream=None) -> "WindowKvCache":
+        c = WindowKvCache(self.axis, self.window, self.storage_format)
+        if self._h is not None:
+            h = C.c_void_p()
+            call("trocm_kv_cache_clone", self._h, C.byref(h), _sh(stream))
+            c._h, c._shape, c._dtype = h, self._shape, self._dtype
+        return c
+
+
 def _scale_arg(scale) -> float:
     return float("nan") if scale is None else float(scale)
 
@@ -336,6 +375,64 @@ class InPlaceKvSdpaState:
         return f
 
     def unfreeze(self) -> "InPlaceKvSdpaState":
+        return self.freeze()
+
+
+class WindowKvSdpa:
+    """Fused sliding-window KV-cache + attention (decode): inputs [Q, K_new, V_new], each
+    [B, H, S, D]; output has Q's shape.  The bounded cache is the sliding window."""
+
+    def __init__(self, axis: int = 2, window: int = 4096, scale=None, storage_format: int | None = None):
+        self.axis, self.window, self.scale, self.storage_format = axis, window, scale, storage_format
+
+    def name(self) -> str:
+        return "WindowKvSdpa"
+
+    def is_stateless(self) -> bool:
+        return False
+
+    def state(self) -> "WindowKvSdpaState":
+        return WindowKvSdpaState(self.axis, self.window, self.scale, self.storage_format)
+
+    def output_facts(self, *shapes):
+        if len(shapes) != 3:
+            raise TractRocmError("WindowKvSdpa expects [Q, K_new, V_new]")
+        return tuple(shapes[0])
+
+
+class WindowKvSdpaState:
+    def __init__(self, axis, window, scale, storage_format=None):
+        self.axis, self.window, self.scale, self.storage_format = axis, window, scale, storage_format
+        self.k = WindowKvCache(axis, window, storage_format)
+        self.v = WindowKvCache(axis, window, storage_format)
+        self._ws = None
+
+    def eval(self, inputs, stream=None, out: DeviceTensor | None = None) -> DeviceTensor:
+        if len(inputs) != 3:
+            raise TractRocmError("WindowKvSdpa expects [Q, K_new, V_new]")
+        q, k_new, v_new = (_as_device(t, stream) for t in inputs)
+        if k_new.shape != v_new.shape or not (q.dtype == k_new.dtype == v_new.dtype):
+            raise TractRocmError("K_new and V_new must share shape and datum type with Q's type")
+        for c, t in ((self.k, k_new), (self.v, v_new)):
+            if c.handle is None:
+                c._create(t.shape, t.dtype)
+            c._check_push_shape(t.shape)
+        B, Hq, Sq, D = _canon4(q.shape)
+        S = _canon4(k_new.shape)[2]
+        if out is None:
+            out = DeviceTensor(q.shape, q.dtype)
+        if self._ws is None or self._ws.nbytes < Workspace.bytes_for(B, Hq, Sq, D):
+            self._ws = Workspace(B, Hq, Sq, D, stream)
+        call("trocm_window_kv_sdpa_eval", q.ptr, k_new.ptr, v_new.ptr, dtype_code(q.dtype), Hq, S, None,
+             self.k.handle, self.v.handle, out.ptr, _scale_arg(self.scale), self._ws.ptr, self._ws.nbytes, _sh(stream))
+        return out
+
+    def freeze(self) -> "WindowKvSdpaState":
+        f = WindowKvSdpaState(self.axis, self.window, self.scale, self.storage_format)
+        f.k, f.v = self.k.clone(), self.v.clone()
+        return f
+
+    def unfreeze(self) -> "WindowKvSdpaState":
         return self.freeze()
 
 
