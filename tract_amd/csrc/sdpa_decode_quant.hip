@@ -9,10 +9,11 @@
 //   QK : dot2 accumulates sum q_i (1024 + u_i) per 32-element block; the constant part
 //        (1152 or 1032 times the block sum of q, computed once per workgroup) is subtracted
 //        and the block scale d applied:  s += d * (dot - bias * qsum).
-//   PV : (1024 + u) - bias is exact in f16; p * d is formed once per token and head and the
-//        update is a mixed-precision fma per element.
+//   PV : (1024 + u) - bias is exact in f16 and (code * d) rounded to f16 is the reference's
+//        dequantised value; two tokens share a dot2 against the f16 pair (p_a, p_b).
 // The reference dequantises to f16 ((code * d) rounded to f16, q4_0.rs:82-95) before its f32
-// attention; here the product stays in f32, a difference below half an f16 ulp per element.
+// attention; V is formed exactly so, for K the product with d stays in f32 (a difference below
+// half an f16 ulp per element).
 //
 // Roofline: HBM-bound on paper (34/32 or 18/32 bytes per element) but the vector ALU work
 // per byte is 2-4x that of f16, so these kernels are ALU-limited before they are
@@ -224,48 +225,66 @@ __global__ __launch_bounds__(kThreads, G <= 4 ? 2 : 1) void sdpa_decode_q_kernel
             for (int h = 0; h < G; h++) s[h] = fmaf(d, acc[h] - lds_qsum[h * kNB + blk], s[h]);
         }
         const bool valid = (t0 + qk_row) < p.T;
-        float pr[G];
+        float pr[G], alpha[G];
+        bool moved = false;
 #pragma unroll
         for (int h = 0; h < G; h++) {
             float full = s[h] + dpp_f<kSwapPairs>(s[h]);
             float sv = valid ? full * p.scale_log2 : -INFINITY;
             float m_new = fmaxf(m[h], wave_max(sv));
-            float alpha = fast_exp2(m[h] - m_new);
+            alpha[h] = fast_exp2(m[h] - m_new);
             pr[h] = fast_exp2(sv - m_new);
-            l[h] = l[h] * alpha + pr[h];
+            l[h] = l[h] * alpha[h] + pr[h];
+            moved = moved || (m_new != m[h]);
             m[h] = m_new;
+        }
+        if (moved) {  // wave-uniform: the running maxima rarely move after the first tiles
 #pragma unroll
-            for (int e = 0; e < EPL; e++) o[h][e] *= alpha;
+            for (int h = 0; h < G; h++)
+#pragma unroll
+                for (int e = 0; e < EPL; e++) o[h][e] *= alpha[h];
         }
         if (qk_half == 0) {
 #pragma unroll
             for (int h = 0; h < G; h++) lds_p[w][qk_row * G + h] = pr[h];
         }
-        // ---- O += P V with fused dequantisation
+        // ---- O += P V with fused dequantisation, two tokens per dot2 ---------------------------
+        // Tokens 4*(2j)+rg and 4*(2j+1)+rg of this lane are paired: their code bytes are interleaved
+        // (one v_perm per two elements) and turned into halves 1024+u; a packed subtract (exact) and
+        // a packed multiply form (code_a * d_a, code_b * d_b) rounded once to f16 -- the reference's
+        // dequantised values (q4_0.rs:82-95).  dot2 with the f16 pair (p_a, p_b) accumulates in f32.
 #pragma unroll
-        for (int i = 0; i < VI; i++) {
-            const float d = __half2float(__ushort_as_half(vsreg[i]));
-            float pd[G];
-#pragma unroll
-            for (int h = 0; h < G; h++) pd[h] = lds_p[w][(4 * i + rg) * G + h] * d;
-            half2_t c2[4];
+        for (int j = 0; j < VI / 2; j++) {
+            const int ia = 2 * j, ib = 2 * j + 1;
+            const half2_t dpair = as_half2((uint32_t)vsreg[ia] | ((uint32_t)vsreg[ib] << 16));
             const half2_t bias = {(_Float16)Q::kBias, (_Float16)Q::kBias};
+            half2_t pp[G];
+#pragma unroll
+            for (int h = 0; h < G; h++) {
+                pp[h][0] = (_Float16)lds_p[w][(4 * ia + rg) * G + h];
+                pp[h][1] = (_Float16)lds_p[w][(4 * ib + rg) * G + h];
+            }
+            uint32_t wa[2], wb[2];
             if constexpr (FMT == TROCM_Q8_0) {
-                uint32_t x0 = vreg[i].x ^ 0x80808080u, x1 = vreg[i].y ^ 0x80808080u;
-                c2[0] = magic_lo(x0) - bias, c2[1] = magic_hi(x0) - bias;
-                c2[2] = magic_lo(x1) - bias, c2[3] = magic_hi(x1) - bias;
+                wa[0] = vreg[ia].x ^ 0x80808080u, wa[1] = vreg[ia].y ^ 0x80808080u;
+                wb[0] = vreg[ib].x ^ 0x80808080u, wb[1] = vreg[ib].y ^ 0x80808080u;
             } else {
-                uint32_t x = vreg[i];
-                uint32_t lo = x & 0x0F0F0F0Fu, hi = (x >> 4) & 0x0F0F0F0Fu;
-                c2[0] = magic_lo(lo) - bias, c2[1] = magic_hi(lo) - bias;
-                c2[2] = magic_lo(hi) - bias, c2[3] = magic_hi(hi) - bias;
+                wa[0] = vreg[ia] & 0x0F0F0F0Fu, wa[1] = (vreg[ia] >> 4) & 0x0F0F0F0Fu;
+                wb[0] = vreg[ib] & 0x0F0F0F0Fu, wb[1] = (vreg[ib] >> 4) & 0x0F0F0F0Fu;
             }
 #pragma unroll
-            for (int e = 0; e < EPL; e++) {
-                float vf = (float)(c2[e >> 1][e & 1]);
+            for (int wd = 0; wd < 2; wd++) {
+                // bytes (a0, b0, a1, b1) and (a2, b2, a3, b3) of this word's four elements
+                const uint32_t t01 = perm(wa[wd], wb[wd], 0x01050004u), t23 = perm(wa[wd], wb[wd], 0x03070206u);
+                half2_t v2[4] = {magic_lo(t01), magic_hi(t01), magic_lo(t23), magic_hi(t23)};
 #pragma unroll
-                for (int h = 0; h < G; h++) o[h][e] = fmaf(pd[h], vf, o[h][e]);
+                for (int i = 0; i < 4; i++) {
+                    const half2_t vd = (v2[i] - bias) * dpair;
+#pragma unroll
+                    for (int h = 0; h < G; h++) o[h][4 * wd + i] = __builtin_amdgcn_fdot2(vd, pp[h], o[h][4 * wd + i], false);
+                }
             }
+            __builtin_amdgcn_sched_barrier(0);  // one token pair at a time: keeps the register count down
         }
         if (more) issue_v(tile + kWaves);
     }
