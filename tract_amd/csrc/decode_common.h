@@ -39,6 +39,9 @@ struct DecodeDev {
     // dense f16/f32 kernel: 1 = the splits of a sequence take groups of kWaves tiles round-robin
     // (concurrent workgroups then read neighbouring addresses), 0 = contiguous tile ranges
     int interleave;
+    // != NULL: arrival counters (one int per (batch, kv head), zero between launches); the last
+    // workgroup of a sequence-head to arrive merges the splits itself and no merge launch follows
+    int *counters;
 };
 
 // Ragged batches: one work item = a tile range of one sequence (device copies of the host plan).
@@ -133,6 +136,7 @@ __device__ __forceinline__ float from_f32<float>(float x) { return x; }
 // many splits there are (with one thread looping over splits and heads a B=1 merge took as long
 // as the attention itself).
 constexpr int kMergeChunk = 256;
+constexpr int kTailMergeMax = 8;   // most splits the in-kernel (last workgroup) merge handles
 template <typename T, int D, int G>
 __device__ __forceinline__ void merge_head(const DecodeDev &p, int64_t first, int64_t stride, int nsplit, int h,
                                            T *out_row, int tid) {
