@@ -158,9 +158,11 @@ int trocm_kv_export(const trocm_kv_cache *cache, void *dst_device, void *stream)
 int trocm_kv_row_bytes(const trocm_kv_cache *cache, size_t *bytes);
 /* OpStateFreeze::freeze (:262-272): an independent deep copy (same len, capacity, reallocs). */
 int trocm_kv_cache_clone(const trocm_kv_cache *cache, trocm_kv_cache **out, void *stream);
-/* Raw view for kernels written against the cache: base pointers and capacity.
+/* Raw view for kernels written against the cache: base pointers and the row pitch in tokens
+ * (the planes are [batch, kv_heads, pitch, ...]; pitch >= capacity, large caches pad their rows
+ * by 1/32 so that half-full power-of-two rows do not leave an address bit unused).
  * `scales` is NULL for F32/F16. */
-int trocm_kv_cache_raw(const trocm_kv_cache *cache, void **data, void **scales, int64_t *capacity);
+int trocm_kv_cache_raw(const trocm_kv_cache *cache, void **data, void **scales, int64_t *pitch);
 
 /* ---- block quantisation as a tensor op: BlockQuant::{quant_f32,quant_f16,dequant_f32,dequant_f16}
  *      (linalg/src/frame/block_quant/mod.rs:48-108) ------------------------------------------- */

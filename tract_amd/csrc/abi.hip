@@ -124,6 +124,7 @@ struct trocm_kv_cache {
     int fmt;
     int64_t B, H, D;
     int64_t len, cap, reallocs;
+    int64_t pitch;  // tokens between the rows of consecutive heads in the planes (>= cap, see pitch_for)
     void *data;    // F32/F16 rows, or the code plane
     void *scales;  // f16 scale plane of the quantised formats
     trocm_kv_pool *pool;  // where the planes live; NULL = their own hipMalloc
@@ -155,6 +156,22 @@ static int plane_free(trocm_kv_cache *c, void *ptr) {
     }
     TROCM_HIP(hipFree(ptr));
     return 0;
+}
+
+// Row pitch (tokens between the rows of consecutive (batch, head) pairs) for a capacity.
+// Capacities double, so `cap * row_bytes` is a large power of two for the usual head sizes, and a
+// cache that is half full (the state right after a doubling) then leaves one address bit constant
+// over the whole working set: measured on MI355X, decode over such a layout is 7 % slower than
+// over densely packed rows (57.5 us against 53.5 us, batch 8, 8226 tokens in 16384-token rows).
+// 1/32 of padding per row removes the effect (52.9 us).  TROCM_KV_PITCH_PAD=<tokens> overrides.
+static int64_t pitch_for(int64_t cap) {
+    static int64_t forced = -2;
+    if (forced == -2) {
+        const char *e = getenv("TROCM_KV_PITCH_PAD");
+        forced = e ? atoll(e) : -1;
+    }
+    if (forced >= 0) return cap + forced;
+    return cap >= 2048 ? cap + ((cap / 32 + 7) & ~(int64_t)7) : cap;
 }
 
 static size_t plane_bytes(const trocm_kv_cache *c, int64_t cap) {
@@ -191,14 +208,15 @@ static int copy_valid(const trocm_kv_cache *c, void *dst, void *dst_scales, int6
 // (grow(), transformers/src/ops/inplace_kv_cache.rs:106-113; the tail stays uninitialised).
 static int regrow(trocm_kv_cache *c, int64_t new_cap, hipStream_t s) {
     void *nd = nullptr, *ns = nullptr;
-    size_t pb = plane_bytes(c, new_cap), sb = scale_plane_bytes(c, new_cap);
+    const int64_t new_pitch = pitch_for(new_cap);
+    size_t pb = plane_bytes(c, new_pitch), sb = scale_plane_bytes(c, new_pitch);
     if (plane_alloc(c, &nd, pb, "a KV cache plane")) return 1;
     if (sb && plane_alloc(c, &ns, sb, "a KV cache scale plane")) {
         (void)plane_free(c, nd);
         return 1;
     }
     if (c->data && c->len) {
-        if (copy_valid(c, nd, ns, new_cap, c->data, c->scales, c->cap, c->len, s)) {
+        if (copy_valid(c, nd, ns, new_pitch, c->data, c->scales, c->pitch, c->len, s)) {
             (void)plane_free(c, nd);
             (void)plane_free(c, ns);
             return 1;
@@ -213,6 +231,7 @@ static int regrow(trocm_kv_cache *c, int64_t new_cap, hipStream_t s) {
     c->data = nd;
     c->scales = ns;
     c->cap = new_cap;
+    c->pitch = new_pitch;
     return 0;
 }
 
@@ -390,7 +409,7 @@ int trocm_kv_cache_create(trocm_kv_cache **out, int fmt, int64_t batch, int64_t 
     TROCM_REQUIRE(c != nullptr, "out of host memory");
     c->fmt = fmt;
     c->B = batch, c->H = kv_heads, c->D = head_dim;
-    c->len = c->cap = c->reallocs = 0;
+    c->len = c->cap = c->reallocs = c->pitch = 0;
     c->data = c->scales = nullptr;
     c->pool = nullptr;
     c->window = c->cursor = 0;
@@ -537,7 +556,7 @@ static int append_write_at(trocm_kv_cache *c, const void *src0, int src_dtype, c
         a.fmt = c->fmt, a.src_dtype = src_dtype;
         a.B = c->B, a.H = c->H, a.S = n_new, a.D = c->D;
         for (int i = 0; i < 4; i++) a.ss[i] = src_strides[i];
-        a.cap = c->cap, a.t0 = t0;
+        a.cap = c->pitch, a.t0 = t0;
         a.src = src, a.codes = c->data, a.scales = c->scales;
         return launch_quant_append(a, s);
     }
@@ -546,8 +565,8 @@ static int append_write_at(trocm_kv_cache *c, const void *src0, int src_dtype, c
     d.rank = 4;
     d.shape[0] = c->B, d.shape[1] = c->H, d.shape[2] = n_new, d.shape[3] = c->D;
     for (int i = 0; i < 4; i++) d.src_stride[i] = src_strides[i] * es;
-    d.dst_stride[0] = c->H * c->cap * c->D * es;
-    d.dst_stride[1] = c->cap * c->D * es;
+    d.dst_stride[0] = c->H * c->pitch * c->D * es;
+    d.dst_stride[1] = c->pitch * c->D * es;
     d.dst_stride[2] = c->D * es;
     d.dst_stride[3] = es;
     return launch_copy_nd((char *)c->data + t0 * c->D * es, src, d, (int)es, s);
@@ -623,7 +642,7 @@ int trocm_kv_append_pair(trocm_kv_cache *kc, trocm_kv_cache *vc, const void *k_s
         a.dst[1] = (char *)vc->data + vc->len * vc->D * es;
         a.B = kc->B, a.H = kc->H, a.S = n_new, a.row_bytes = kc->D * es;
         for (int i = 0; i < 3; i++) a.src_stride[i] = src_strides[i] * es;
-        a.dst_stride[0] = kc->H * kc->cap * kc->D * es, a.dst_stride[1] = kc->cap * kc->D * es, a.dst_stride[2] = kc->D * es;
+        a.dst_stride[0] = kc->H * kc->pitch * kc->D * es, a.dst_stride[1] = kc->pitch * kc->D * es, a.dst_stride[2] = kc->D * es;
         rc = launch_append_pair(a, s);
     }
     if (rc == 2) {
@@ -660,14 +679,14 @@ int trocm_kv_export(const trocm_kv_cache *c, void *dst, void *stream) {
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
     if (is_quant(c->fmt))
-        return launch_quant_export(c->fmt, c->B, c->H, c->len, c->cap, c->D, c->data, c->scales, dst, s);
+        return launch_quant_export(c->fmt, c->B, c->H, c->len, c->pitch, c->D, c->data, c->scales, dst, s);
     CopyNd d;
     d.rank = 2;
     int64_t rb = (int64_t)device_row_bytes(c->fmt, c->D);
     d.shape[0] = c->B * c->H;
     d.shape[1] = c->len * rb;
     d.dst_stride[0] = c->len * rb;
-    d.src_stride[0] = c->cap * rb;
+    d.src_stride[0] = c->pitch * rb;
     d.dst_stride[1] = d.src_stride[1] = 1;
     return launch_copy_nd(dst, c->data, d, 1, s);
 }
@@ -686,7 +705,7 @@ int trocm_kv_cache_clone(const trocm_kv_cache *c, trocm_kv_cache **out, void *st
             trocm_kv_cache_destroy(n);
             return 1;
         }
-        if (copy_valid(c, n->data, n->scales, n->cap, c->data, c->scales, c->cap, c->len, s)) {
+        if (copy_valid(c, n->data, n->scales, n->pitch, c->data, c->scales, c->pitch, c->len, s)) {
             trocm_kv_cache_destroy(n);
             return 1;
         }
@@ -702,7 +721,7 @@ int trocm_kv_cache_raw(const trocm_kv_cache *c, void **data, void **scales, int6
     TROCM_NOT_NULL(c);
     if (data) *data = c->data;
     if (scales) *scales = c->scales;
-    if (capacity) *capacity = c->cap;
+    if (capacity) *capacity = c->pitch;
     return 0;
 }
 
@@ -877,7 +896,7 @@ int trocm_sdpa_cached(const void *q, int q_dtype, int64_t q_heads, int64_t q_len
     a.q = q, a.out = out, a.q_dtype = q_dtype, a.kv_fmt = kc->fmt;
     a.k = kc->data, a.v = vc->data, a.k_scales = kc->scales, a.v_scales = vc->scales;
     a.B = kc->B, a.Hq = q_heads, a.Hkv = kc->H, a.Sq = q_len, a.Sk = kc->len, a.D = kc->D;
-    a.kv_stride_t = kc->D, a.kv_stride_h = kc->cap * kc->D, a.kv_stride_b = kc->H * kc->cap * kc->D;
+    a.kv_stride_t = kc->D, a.kv_stride_h = kc->pitch * kc->D, a.kv_stride_b = kc->H * kc->pitch * kc->D;
     a.mask_b = a.mask_h = 1;
     a.scale = isnan(scale) ? 1.0f / sqrtf((float)kc->D) : scale;
     a.causal = causal;
@@ -893,7 +912,7 @@ static void cached_args(SdpaArgs &a, const void *q, int q_dtype, int64_t q_heads
     a.q = q, a.out = out, a.q_dtype = q_dtype, a.kv_fmt = kc->fmt;
     a.k = kc->data, a.v = vc->data, a.k_scales = kc->scales, a.v_scales = vc->scales;
     a.B = kc->B, a.Hq = q_heads, a.Hkv = kc->H, a.Sq = q_len, a.Sk = kv_len, a.D = kc->D;
-    a.kv_stride_t = kc->D, a.kv_stride_h = kc->cap * kc->D, a.kv_stride_b = kc->H * kc->cap * kc->D;
+    a.kv_stride_t = kc->D, a.kv_stride_h = kc->pitch * kc->D, a.kv_stride_b = kc->H * kc->pitch * kc->D;
     a.mask_b = a.mask_h = 1;
     a.scale = isnan(scale) ? 1.0f / sqrtf((float)kc->D) : scale;
     a.causal = causal;
@@ -1016,7 +1035,7 @@ static int ragged_common(const void *q, const void *k_new, const void *v_new, in
             TROCM_REQUIRE(kc->cap == vc->cap, "K/V capacities must match (sequence %lld)", (long long)i);
             int64_t len = kc->len + (in_kernel ? 1 : 0);
             TROCM_REQUIRE(len > 0, "empty kv-cache (sequence %lld)", (long long)i);
-            seqs[(size_t)i] = RaggedSeq{kc->data, vc->data, kc->scales, vc->scales, len, kc->cap};
+            seqs[(size_t)i] = RaggedSeq{kc->data, vc->data, kc->scales, vc->scales, len, kc->pitch};
         }
         int rc = launch_sdpa_decode_ragged(q, out, q_dtype, k0->fmt, n_seq, q_heads, k0->H, k0->D, seqs.data(), sc,
                                            workspace, workspace_bytes, in_kernel ? k_new : nullptr,
