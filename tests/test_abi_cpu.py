@@ -50,3 +50,18 @@ def test_error_convention_without_device():
     # null pointers are reported, never dereferenced
     assert lib.trocm_kv_cache_len(None, None) == 1
     assert b"null pointer" in lib.trocm_last_error()
+
+
+def test_no_kernel_spills_registers():
+    """A kernel that spills to scratch still computes the right thing and runs several times
+    slower (it happened twice while these kernels were written); the build records hipcc's
+    per-kernel resource usage and this test reads it."""
+    from tract_amd.build import resource_usage
+    usage = resource_usage()
+    assert len(usage) > 50
+    spilling = {k: v for k, v in usage.items() if v.get("VGPRs Spill", 0) or v.get("SGPRs Spill", 0) or v.get("ScratchSize [bytes/lane]", 0)}
+    assert not spilling, spilling
+    # the kernels that must keep two waves per SIMD resident do
+    for name, v in usage.items():
+        if "sdpa_prefill_pp_kernel" in name:
+            assert v["Occupancy [waves/SIMD]"] >= 2, (name, v)

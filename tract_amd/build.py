@@ -6,6 +6,7 @@ to this file (``tract_amd/libtract_rocm.so``); objects go to ``tract_amd/csrc/bu
 from __future__ import annotations
 
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -22,6 +23,7 @@ COMMON = [
     "-fhip-fp32-correctly-rounded-divide-sqrt", "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
+    "-Rpass-analysis=kernel-resource-usage",   # per-kernel registers / spills / LDS, kept beside the objects
 ]
 # per-file extra flags: the quantiser must not contract a*b+c into an fma
 EXTRA = {"kv_quant.hip": ["-ffp-contract=off"], "elementwise.hip": ["-ffp-contract=off"]}
@@ -38,11 +40,44 @@ def _newer(target: str, deps: list[str]) -> bool:
 
 def _run(cmd: list[str]) -> None:
     p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in p.stdout.splitlines() if "packed-fp32-ops" not in l)
+    lines = [l for l in p.stdout.splitlines() if "packed-fp32-ops" not in l]
+    remarks = [l.split("remark: ", 1)[1].split(" [-Rpass", 1)[0].strip() for l in lines if "[-Rpass-analysis=kernel-resource-usage]" in l]
+    kept, pending, in_remark = [], [], False
+    for l in lines:   # drop the remarks together with their source-context and include-stack lines
+        if "-Rpass-analysis=kernel-resource-usage" in l:
+            pending, in_remark = [], True
+        elif l.startswith("In file included from"):
+            pending.append(l)
+        elif in_remark and re.match(r"^\s*(\d+\s*)?\|", l):
+            pass
+        else:
+            kept += pending + [l]
+            pending, in_remark = [], False
+    out = "\n".join(kept)
     if p.returncode != 0:
         raise RuntimeError("command failed: " + " ".join(cmd) + "\n" + out)
+    if "-c" in cmd:
+        with open(cmd[cmd.index("-o") + 1] + ".usage.txt", "w") as f:
+            f.write("\n".join(remarks) + "\n")
     if out.strip():
         print(out)
+
+
+def resource_usage() -> dict:
+    """{kernel symbol: {"VGPRs": n, "VGPRs Spill": n, "ScratchSize [bytes/lane]": n, ...}} of the last
+    build (hipcc's kernel-resource-usage remarks), building first if an object is stale."""
+    build(verbose=False)
+    res = {}
+    for src in SOURCES:
+        path = os.path.join(OBJ, src.replace(".hip", ".o")) + ".usage.txt"
+        cur = None
+        for line in open(path):
+            key, _, val = line.strip().partition(": ")
+            if key == "Function Name":
+                cur = res.setdefault(val, {"source": src})
+            elif cur is not None and val.strip().lstrip("-").isdigit():
+                cur[key] = int(val)
+    return res
 
 
 def build(force: bool = False, verbose: bool = True) -> str:
@@ -54,7 +89,7 @@ def build(force: bool = False, verbose: bool = True) -> str:
         s = os.path.join(CSRC, src)
         o = os.path.join(OBJ, src.replace(".hip", ".o"))
         objs.append(o)
-        if force or not _newer(o, [s] + headers):
+        if force or not _newer(o, [s] + headers) or not os.path.exists(o + ".usage.txt"):
             jobs.append([HIPCC] + COMMON + EXTRA.get(src, []) + ["-c", s, "-o", o])
     if jobs:
         if verbose:
