@@ -94,7 +94,21 @@ class InPlaceKvCache {
     InPlaceKvCache(InPlaceKvCache &&o) noexcept { *this = std::move(o); }
     InPlaceKvCache &operator=(InPlaceKvCache &&o) noexcept {
         std::swap(h_, o.h_), std::swap(axis_, o.axis_), std::swap(fmt_, o.fmt_), std::swap(shape_, o.shape_);
+        std::swap(window_, o.window_);
         return *this;
+    }
+    // WindowKvCache::new (window_kv_cache.rs:89-93): the same object in ring-buffer mode.
+    static InPlaceKvCache window(size_t axis, int64_t window, std::optional<int> storage_format = std::nullopt) {
+        if (window <= 0) throw Error("window must be > 0");
+        InPlaceKvCache c(axis, storage_format);
+        c.window_ = window;
+        return c;
+    }
+    int64_t cursor() const {
+        if (!h_) return 0;
+        int64_t w = 0, c = 0;
+        check(trocm_kv_cache_window(h_, &w, &c));
+        return c;
     }
     ~InPlaceKvCache() {
         if (h_) trocm_kv_cache_destroy(h_);
@@ -112,7 +126,10 @@ class InPlaceKvCache {
         if (sh[2] == 0) return;
         if (!h_) {
             int fmt = fmt_.value_or((int)input.datum_type());
-            check(trocm_kv_cache_create(&h_, fmt, sh[0], sh[1], sh[3]));
+            if (window_ > 0)
+                check(trocm_kv_cache_create_window(&h_, fmt, sh[0], sh[1], sh[3], window_));
+            else
+                check(trocm_kv_cache_create(&h_, fmt, sh[0], sh[1], sh[3]));
             shape_ = sh;
         } else if (sh[0] != shape_[0] || sh[1] != shape_[1] || sh[3] != shape_[3]) {
             throw Error("rank mismatch in kv-cache push");
@@ -142,6 +159,7 @@ class InPlaceKvCache {
     }
     InPlaceKvCache clone() const {
         InPlaceKvCache c(axis_, fmt_);
+        c.window_ = window_;
         if (h_) {
             check(trocm_kv_cache_clone(h_, &c.h_, nullptr));
             c.shape_ = shape_;
@@ -158,6 +176,7 @@ class InPlaceKvCache {
         return v;
     }
     trocm_kv_cache *h_ = nullptr;
+    int64_t window_ = 0;
     size_t axis_ = 2;
     std::optional<int> fmt_;
     std::vector<int64_t> shape_;
@@ -259,6 +278,83 @@ struct InPlaceKvSdpa {
     std::string name() const { return "InPlaceKvSdpa"; }
     bool is_stateless() const { return false; }
     InPlaceKvSdpaState state() const { return InPlaceKvSdpaState(axis, causal, scale); }
+};
+
+// Fused sliding-window KV-cache + attention (window_kv_cache.rs:156-239): inputs [Q, K_new, V_new].
+class WindowKvSdpaState {
+   public:
+    WindowKvSdpaState(size_t axis, int64_t window, std::optional<float> scale, std::optional<int> fmt = std::nullopt)
+        : scale_(scale), k(InPlaceKvCache::window(axis, window, fmt)), v(InPlaceKvCache::window(axis, window, fmt)) {}
+    DeviceTensor eval(const DeviceTensor &q, const DeviceTensor &k_new, const DeviceTensor &v_new) {
+        k.push(k_new);   // WindowKvSdpaState::eval, :224-225
+        v.push(v_new);
+        const auto &qs = q.shape();
+        size_t need = 0;
+        check(trocm_sdpa_workspace_bytes(qs[0], qs[1], qs[2], qs[3], &need));
+        if (!ws_ || ws_->bytes() < need) ws_ = std::make_unique<Workspace>(qs[0], qs[1], qs[2], qs[3]);
+        DeviceTensor out(qs, q.datum_type());
+        // the ring buffer bounds which keys are visible: attend to all of them, no causal mask (:232-236)
+        check(trocm_sdpa_cached(q.ptr(), (int)q.datum_type(), qs[1], qs[2], k.handle(), v.handle(), out.ptr(),
+                                scale_.value_or(NAN), 0, ws_->ptr(), ws_->bytes(), nullptr));
+        return out;
+    }
+
+   private:
+    std::optional<float> scale_;
+    std::unique_ptr<Workspace> ws_;
+
+   public:
+    InPlaceKvCache k, v;
+};
+
+struct WindowKvSdpa {
+    size_t axis = 2;
+    int64_t window = 4096;
+    std::optional<float> scale;
+    std::string name() const { return "WindowKvSdpa"; }
+    bool is_stateless() const { return false; }
+    WindowKvSdpaState state() const { return WindowKvSdpaState(axis, window, scale); }
+};
+
+// RotateHalf / ApplyRope (transformers/src/ops/apply_rope.rs:58-76, 169-176) and Cast on dense tensors;
+// cos and sin share a shape that broadcasts against x (trailing-aligned).
+struct RotateHalf {
+    DeviceTensor eval(const DeviceTensor &x) const {
+        DeviceTensor out(x.shape(), x.datum_type());
+        check(trocm_rotate_half(x.ptr(), out.ptr(), (int)x.datum_type(), (int)x.shape().size(), x.shape().data(), nullptr,
+                                nullptr, nullptr));
+        return out;
+    }
+};
+
+struct ApplyRope {
+    DeviceTensor eval(const DeviceTensor &x, const DeviceTensor &cos, const DeviceTensor &sin) const {
+        if (cos.shape() != sin.shape()) throw Error("cos and sin must have the same shape");
+        const auto &xs = x.shape(), &cs = cos.shape();
+        if (cs.size() > xs.size()) throw Error("cos/sin rank exceeds the input rank");
+        std::vector<int64_t> strides(xs.size(), 0);
+        int64_t acc = 1;
+        for (size_t i = 0; i < xs.size(); i++) {
+            size_t d = xs.size() - 1 - i;
+            int64_t cd = i < cs.size() ? cs[cs.size() - 1 - i] : 1;
+            if (cd != 1 && cd != xs[d]) throw Error("cos/sin shape does not broadcast against the input");
+            strides[d] = (cd == 1 && xs[d] != 1) ? 0 : acc;
+            acc *= cd;
+        }
+        DeviceTensor out(xs, x.datum_type());
+        check(trocm_apply_rope(x.ptr(), cos.ptr(), sin.ptr(), out.ptr(), (int)x.datum_type(), (int)xs.size(), xs.data(),
+                               nullptr, strides.data(), nullptr, nullptr));
+        return out;
+    }
+};
+
+struct Cast {
+    DatumType to;
+    DeviceTensor eval(const DeviceTensor &x) const {
+        DeviceTensor out(x.shape(), to);
+        check(trocm_cast(x.ptr(), (int)x.datum_type(), out.ptr(), (int)to, x.len(), nullptr));
+        return out;
+    }
 };
 
 }  // namespace trocm

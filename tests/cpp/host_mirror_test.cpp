@@ -2,6 +2,7 @@
 // (transformers/src/ops/inplace_kv_cache.rs:366-418, 456-491, 595-658, 898-942), run against
 // the rocm library through the C++ host mirror.  References are written in the test, as the
 // reference's own tests do: plain concatenation and naive f32 attention.
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -168,6 +169,90 @@ int main() {
             std::vector<float> got(o.len());
             o.to_host(got.data());
             EXPECT(std::isfinite(got[0]));
+        }
+        // window_holds_last_w_as_a_set + prefill_chunk_larger_than_window_keeps_last_w (window_kv_cache.rs:342-374)
+        {
+            const int w = 4;
+            InPlaceKvCache c = InPlaceKvCache::window(2, w);
+            for (int t = 0; t < 10; t++) {
+                float x = (float)t;
+                c.push(DeviceTensor::from_host(&x, {1, 1, 1, 1}, DatumType::F32));
+                EXPECT(c.len() <= w);
+                auto bytes = c.valid_contiguous();
+                std::vector<float> got(bytes.size() / 4);
+                std::memcpy(got.data(), bytes.data(), bytes.size());
+                std::sort(got.begin(), got.end());
+                for (size_t i = 0; i < got.size(); i++) EXPECT(got[i] == (float)(t + 1 - (int)got.size() + (int)i));
+            }
+            EXPECT(c.capacity() == w && c.cursor() == 10 % w);
+            InPlaceKvCache big = InPlaceKvCache::window(2, 3);
+            float chunk[7] = {0, 1, 2, 3, 4, 5, 6};
+            big.push(DeviceTensor::from_host(chunk, {1, 1, 7, 1}, DatumType::F32));
+            auto bytes = big.valid_contiguous();
+            float got[3];
+            std::memcpy(got, bytes.data(), 12);
+            EXPECT(got[0] == 4.f && got[1] == 5.f && got[2] == 6.f && big.cursor() == 0);
+        }
+
+        // window_sdpa_decode_matches_last_w_in_model (window_kv_cache.rs:468-527)
+        {
+            const int B = 1, H = 2, D = 16, W = 5;
+            WindowKvSdpaState st = WindowKvSdpa{2, W, std::nullopt}.state();
+            auto mk = [&](float base) {
+                std::vector<float> v((size_t)B * H * D);
+                for (size_t i = 0; i < v.size(); i++) v[i] = base + std::sin((float)i * 0.013f);
+                return v;
+            };
+            std::vector<float> kf, vf;
+            int len = 0, vlen = 0;
+            for (int t = 0; t < 15; t++) {
+                auto q = mk(9.0f + t * 0.1f), k = mk(1.0f + t * 0.07f), v = mk(5.0f - t * 0.05f);
+                DeviceTensor o = st.eval(DeviceTensor::from_host(q.data(), {B, H, 1, D}, DatumType::F32),
+                                         DeviceTensor::from_host(k.data(), {B, H, 1, D}, DatumType::F32),
+                                         DeviceTensor::from_host(v.data(), {B, H, 1, D}, DatumType::F32));
+                std::vector<float> got(o.len());
+                o.to_host(got.data());
+                concat(kf, len, k, B, H, 1, D);
+                concat(vf, vlen, v, B, H, 1, D);
+                const int n = std::min(len, W);
+                std::vector<float> kl((size_t)B * H * n * D), vl(kl.size());
+                for (int bh = 0; bh < B * H; bh++)
+                    for (int j = 0; j < n; j++) {
+                        std::memcpy(&kl[((size_t)bh * n + j) * D], &kf[((size_t)bh * len + len - n + j) * D], sizeof(float) * D);
+                        std::memcpy(&vl[((size_t)bh * n + j) * D], &vf[((size_t)bh * len + len - n + j) * D], sizeof(float) * D);
+                    }
+                auto want = naive(q, kl, vl, B, H, H, 1, n, D, false);
+                for (size_t i = 0; i < want.size(); i++) EXPECT(std::fabs(want[i] - got[i]) <= 1e-3f);
+            }
+        }
+
+        // test_rotate_half (apply_rope.rs:257-277) and ApplyRope against its definition
+        {
+            const int R = 10, C = 64;
+            std::vector<float> x((size_t)R * C), cs(x.size()), sn(x.size());
+            for (size_t i = 0; i < x.size(); i++) x[i] = (float)i, cs[i] = std::cos((float)i), sn[i] = std::sin((float)i);
+            DeviceTensor dx = DeviceTensor::from_host(x.data(), {R, C}, DatumType::F32);
+            DeviceTensor twice = RotateHalf{}.eval(RotateHalf{}.eval(dx));
+            std::vector<float> back(x.size());
+            twice.to_host(back.data());
+            for (size_t i = 0; i < x.size(); i++) EXPECT(-back[i] == x[i]);
+            DeviceTensor y = ApplyRope{}.eval(dx, DeviceTensor::from_host(cs.data(), {R, C}, DatumType::F32),
+                                              DeviceTensor::from_host(sn.data(), {R, C}, DatumType::F32));
+            std::vector<float> got(x.size());
+            y.to_host(got.data());
+            for (int r = 0; r < R; r++)
+                for (int c = 0; c < C; c++) {
+                    size_t i = (size_t)r * C + c;
+                    float rot = c < C / 2 ? -x[i + C / 2] : x[i - C / 2];
+                    volatile float a = x[i] * cs[i];   // each operation rounded on its own, like the CPU op
+                    volatile float b = rot * sn[i];
+                    EXPECT(got[i] == a + b);
+                }
+            DeviceTensor h = Cast{DatumType::F16}.eval(dx);
+            DeviceTensor f = Cast{DatumType::F32}.eval(h);
+            std::vector<float> rt2(x.size());
+            f.to_host(rt2.data());
+            for (size_t i = 0; i < x.size(); i++) EXPECT(rt2[i] == x[i]);   // integers up to 2048 are exact in f16
         }
         std::printf("host_mirror_test: all checks passed\n");
         return 0;
