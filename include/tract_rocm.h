@@ -164,6 +164,29 @@ int trocm_kv_cache_clone(const trocm_kv_cache *cache, trocm_kv_cache **out, void
  * `scales` is NULL for F32/F16. */
 int trocm_kv_cache_raw(const trocm_kv_cache *cache, void **data, void **scales, int64_t *pitch);
 
+/* Append tokens given as canonical blocks in device memory, [batch, kv_heads, n_tokens,
+ * head_dim/32 * block_bytes] (the layout trocm_kv_export writes): OpState::load_from
+ * (dyn_kv_cache.rs:121-140) for a quantised cache without dequantising.  Quantised, ordinary
+ * (not sliding-window) caches only; grows like an append. */
+int trocm_kv_import_blocks(trocm_kv_cache *cache, const void *blocks_device, int64_t n_tokens, void *stream);
+
+/* ---- NNEF tensor files (.dat), host memory only (nnef/src/tensors.rs) --------------------------
+ * The 128-byte header (tensors.rs:10-25) for the tensors of this path.  `item` is a storage
+ * format: TROCM_F32 / TROCM_F16 (vendor 0, item type 0; write_tensor :196-233), TROCM_Q4_0
+ * (vendor 'TR', item type 0x3040, shape flattened to rank 2; write_block_quant_value :300-322)
+ * or TROCM_Q8_0, written as tract's Q8_1 blocks of 36 bytes under item type 0x3081.
+ * trocm_dat_header_read (read_tensor :62-95, read_block_quant_value :275-298) also accepts
+ * item types 0x2040 (flag LEGACY_Q4_PACKING: convert the payload with
+ * trocm_dat_q4_0_legacy_to_gguf, tensors.rs:250-273) and 0x3080; Q8 payloads are Q8_1 blocks
+ * (flag Q8_1_BLOCKS: strip the sums with trocm_q8_1_to_q8_0 before trocm_kv_import_blocks). */
+#define TROCM_DAT_LEGACY_Q4_PACKING 1
+#define TROCM_DAT_Q8_1_BLOCKS 2
+int trocm_dat_header_write(void *dst128, int item, int rank, const int64_t *dims, size_t data_bytes);
+int trocm_dat_header_read(const void *src128, int *item, int *rank, int64_t *dims8, size_t *data_bytes, int *flags);
+int trocm_dat_q4_0_legacy_to_gguf(void *blocks, size_t bytes);
+int trocm_q8_1_to_q8_0(const void *src_36, void *dst_34, size_t n_blocks);
+int trocm_q8_0_to_q8_1(const void *src_34, void *dst_36, size_t n_blocks);
+
 /* ---- block quantisation as a tensor op: BlockQuant::{quant_f32,quant_f16,dequant_f32,dequant_f16}
  *      (linalg/src/frame/block_quant/mod.rs:48-108) ------------------------------------------- */
 

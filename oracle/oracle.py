@@ -336,3 +336,49 @@ class WindowKvCache:
         if self._h is not None and _lib is not None:
             _lib.orc_win_free(self._h)
             self._h = None
+
+
+# ---- NNEF tensor files (nnef/src/tensors.rs), restated with `struct` -------------------------------
+_DAT_VENDOR_TRACT = (ord("T") << 8) | ord("R")   # tensors.rs:8
+
+
+def dat_header_fields(data: bytes) -> dict:
+    """The 128-byte header (tensors.rs:10-25), little endian, field by field."""
+    import struct
+    magic0, magic1, vmaj, vmin, size, rank = struct.unpack_from("<BBBBII", data, 0)
+    dims = struct.unpack_from("<8I", data, 12)
+    bits, item, vendor = struct.unpack_from("<IHH", data, 44)
+    return {"magic": (magic0, magic1), "version": (vmaj, vmin), "data_size_bytes": size, "rank": rank,
+            "dims": dims[:rank], "bits_per_item": bits, "item_type": item, "item_type_vendor": vendor,
+            "rest_is_zero": not any(data[52:128])}
+
+
+def dat_write_plain(a: np.ndarray) -> bytes:
+    """write_tensor for f32 / f16 (tensors.rs:186-248): vendor 0, item type 0."""
+    import struct
+    a = np.require(a, requirements="C")
+    dims = list(a.shape) + [0] * (8 - a.ndim)
+    head = struct.pack("<BBBBII8IIHH", 0x4E, 0xEF, 1, 0, a.nbytes, a.ndim, *dims, a.dtype.itemsize * 8, 0, 0)
+    return head + b"\0" * (128 - len(head)) + a.tobytes()
+
+
+def dat_write_block_quant(item_type: int, blocks: bytes, shape) -> bytes:
+    """write_block_quant_value (tensors.rs:300-322): shape flattened to [prod(leading), last]."""
+    import struct
+    m = int(np.prod(shape[:-1], dtype=np.int64))
+    dims = [m, shape[-1]] + [0] * 6
+    head = struct.pack("<BBBBII8IIHH", 0x4E, 0xEF, 1, 0, len(blocks), 2, *dims, 0xFFFFFFFF, item_type, _DAT_VENDOR_TRACT)
+    return head + b"\0" * (128 - len(head)) + bytes(blocks)
+
+
+def q4_0_legacy_to_gguf(blocks: np.ndarray) -> np.ndarray:
+    """tract_to_gguf_q4_0_packing (tensors.rs:250-273), statement by statement."""
+    out = np.array(blocks, dtype=np.uint8).reshape(-1, 18).copy()
+    for b in range(out.shape[0]):
+        nibbles = out[b, 2:18]            # a view: written in place, from the top down, like the reference
+        second = nibbles[8:].copy()
+        for i in range(15, -1, -1):
+            lsb = (nibbles[i // 2] & 0x0F) if i % 2 == 0 else ((nibbles[i // 2] & 0xF0) >> 4)
+            msb = ((second[i // 2] & 0x0F) << 4) if i % 2 == 0 else (second[i // 2] & 0xF0)
+            nibbles[i] = msb | lsb
+    return out.reshape(blocks.shape)

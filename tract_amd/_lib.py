@@ -59,6 +59,12 @@ SIGNATURES = {
     "trocm_kv_row_bytes": [_vp, C.POINTER(_sz)],
     "trocm_kv_cache_clone": [_vp, C.POINTER(_vp), _vp],
     "trocm_kv_cache_raw": [_vp, C.POINTER(_vp), C.POINTER(_vp), _pi64],
+    "trocm_kv_import_blocks": [_vp, _vp, _i64, _vp],
+    "trocm_dat_header_write": [_vp, _i, _i, _pi64, _sz],
+    "trocm_dat_header_read": [_vp, C.POINTER(_i), C.POINTER(_i), _pi64, C.POINTER(_sz), C.POINTER(_i)],
+    "trocm_dat_q4_0_legacy_to_gguf": [_vp, _sz],
+    "trocm_q8_1_to_q8_0": [_vp, _vp, _sz],
+    "trocm_q8_0_to_q8_1": [_vp, _vp, _sz],
     "trocm_block_quant": [_i, _vp, _i, _sz, _vp, _vp],
     "trocm_block_dequant": [_i, _vp, _sz, _vp, _i, _vp],
     "trocm_cast": [_vp, _i, _vp, _i, _sz, _vp],

@@ -717,6 +717,31 @@ int trocm_kv_cache_clone(const trocm_kv_cache *c, trocm_kv_cache **out, void *st
     return 0;
 }
 
+// Append `n_tokens` tokens given as canonical blocks on the device ([batch, kv_heads, n_tokens,
+// head_dim/32 * block_bytes], what trocm_kv_export writes): load_from of a quantised state without
+// a round trip through floats.
+int trocm_kv_import_blocks(trocm_kv_cache *c, const void *blocks, int64_t n_tokens, void *stream) {
+    TROCM_NOT_NULL(c);
+    TROCM_REQUIRE(is_quant(c->fmt), "import_blocks: the cache stores plain %s tensors, append them instead",
+                  c->fmt == TROCM_F32 ? "f32" : "f16");
+    TROCM_REQUIRE(c->window == 0, "import_blocks: not supported for a sliding-window cache");
+    TROCM_REQUIRE(n_tokens >= 0, "import_blocks: negative token count");
+    if (n_tokens == 0) return 0;
+    TROCM_NOT_NULL(blocks);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    if (c->cap == 0) {
+        if (regrow(c, n_tokens, s)) return 1;
+    } else if (c->len + n_tokens > c->cap) {
+        int64_t new_cap = c->cap * 2 > c->len + n_tokens ? c->cap * 2 : c->len + n_tokens;
+        if (regrow(c, new_cap, s)) return 1;
+        c->reallocs += 1;
+    }
+    if (launch_quant_import(c->fmt, c->B, c->H, n_tokens, c->pitch, c->len, c->D, blocks, c->data, c->scales, s)) return 1;
+    c->len += n_tokens;
+    return 0;
+}
+
 int trocm_kv_cache_raw(const trocm_kv_cache *c, void **data, void **scales, int64_t *capacity) {
     TROCM_NOT_NULL(c);
     if (data) *data = c->data;

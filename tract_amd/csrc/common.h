@@ -89,6 +89,9 @@ int launch_quant_append(const QuantAppend &a, hipStream_t s);
 // Canonical export of the quantised planes: dst [B,H,len, D/32 * block_bytes].
 int launch_quant_export(int fmt, int64_t B, int64_t H, int64_t len, int64_t cap, int64_t D,
                         const void *codes, const void *scales, void *dst, hipStream_t s);
+// Canonical import: blocks [B,H,n, D/32 * block_bytes] into the planes at tokens [t0, t0 + n).
+int launch_quant_import(int fmt, int64_t B, int64_t H, int64_t n, int64_t pitch, int64_t t0, int64_t D, const void *blocks,
+                        void *codes, void *scales, hipStream_t s);
 // Dequantise canonical blocks to a dense f32/f16 tensor.
 int launch_block_quant(int fmt, const void *src, int src_dtype, size_t n_elems, void *dst, hipStream_t s);
 int launch_block_dequant(int fmt, const void *blocks, size_t n_elems, void *dst, int dst_dtype, hipStream_t s);

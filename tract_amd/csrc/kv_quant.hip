@@ -187,6 +187,28 @@ __global__ __launch_bounds__(256) void quant_export_kernel(int fmt, int64_t BH, 
     }
 }
 
+// Canonical import, the inverse of the export: blocks [B,H,n, nb * (2 + code bytes)] are split into
+// the code and scale planes at tokens [t0, t0 + n) of every (batch, head) row.
+__global__ __launch_bounds__(256) void quant_import_kernel(int fmt, int64_t BH, int64_t n, int64_t pitch, int64_t t0,
+                                                           int64_t D, const uint16_t *__restrict__ src,
+                                                           uint8_t *__restrict__ codes, uint16_t *__restrict__ scales) {
+    int64_t nb = D / 32;
+    int64_t total = BH * n * nb;
+    int cw = fmt == TROCM_Q8_0 ? 16 : 8;  // code bytes / 2
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        int64_t blk = idx % nb;
+        int64_t rem = idx / nb;
+        int64_t t = rem % n;
+        int64_t bh = rem / n;
+        int64_t row = bh * pitch + t0 + t;
+        const uint16_t *i16 = src + ((bh * n + t) * nb + blk) * (1 + cw);
+        uint16_t *c = reinterpret_cast<uint16_t *>(codes + (row * nb + blk) * (cw * 2));
+        scales[row * nb + blk] = i16[0];
+        for (int i = 0; i < cw; i++) c[i] = i16[1 + i];
+    }
+}
+
 // Canonical blocks from a dense tensor (BlockQuant::quant_f32/quant_f16 as a tensor op).
 template <typename SrcT>
 __global__ __launch_bounds__(256) void block_quant_kernel(int fmt, const SrcT *__restrict__ src, int64_t n_blocks,
@@ -287,6 +309,15 @@ int launch_quant_export(int fmt, int64_t B, int64_t H, int64_t len, int64_t cap,
     hipLaunchKernelGGL(quant_export_kernel, dim3(grid_for(total)), dim3(256), 0, s, fmt, B * H, len, cap, D,
                        (const uint8_t *)codes, (const uint16_t *)scales, (uint16_t *)dst);
     return check_launch("quant_export");
+}
+
+int launch_quant_import(int fmt, int64_t B, int64_t H, int64_t n, int64_t pitch, int64_t t0, int64_t D, const void *blocks,
+                        void *codes, void *scales, hipStream_t s) {
+    int64_t total = B * H * n * (D / 32);
+    if (total == 0) return 0;
+    hipLaunchKernelGGL(quant_import_kernel, dim3(grid_for(total)), dim3(256), 0, s, fmt, B * H, n, pitch, t0, D,
+                       (const uint16_t *)blocks, (uint8_t *)codes, (uint16_t *)scales);
+    return check_launch("quant_import");
 }
 
 int launch_block_quant(int fmt, const void *src, int src_dtype, size_t n_elems, void *dst, hipStream_t s) {

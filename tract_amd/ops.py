@@ -171,6 +171,40 @@ class InPlaceKvCache:
         call("trocm_kv_export", self._h, out.ptr, _sh(stream))
         return out.to_numpy(stream)
 
+    def save_dat(self, stream=None) -> bytes:
+        """The valid region as an NNEF tensor file: a rank-4 f32/f16 tensor, or the canonical blocks
+        of a quantised cache (no dequantisation) under the flattened shape [B*H*len, D]."""
+        from . import dat
+        v = self.valid_contiguous(stream)
+        if self.storage_format in (F32, F16):
+            return dat.write_tensor(v)
+        B, H, _, D = _canon4(self._shape)
+        return dat.write_block_quant(self.storage_format, v, (B * H * self.len(), D))
+
+    def load_dat(self, data: bytes, like=None, stream=None) -> None:
+        """Append the tokens of an NNEF tensor file written by `save_dat`.  A quantised file records
+        only [rows, D]: `like=(shape, dtype)` gives batch and heads when the cache is still empty."""
+        from . import dat
+        item, shape, payload = dat.read_tensor(data)
+        if item in (F32, F16):
+            self.push(payload, stream=stream)
+            return
+        if self._h is None:
+            if like is None:
+                raise TractRocmError("load_dat of block-quantised data into an empty cache needs `like=(shape, dtype)`")
+            if self.storage_format is None:
+                self.storage_format = item
+            self._create(*like)
+        if self.storage_format != item:
+            raise TractRocmError("the file's block format differs from the cache's storage format")
+        B, H, _, D = _canon4(self._shape)
+        if shape[-1] != D or shape[0] % (B * H):
+            raise TractRocmError(f"file shape {shape} does not match a cache of {B} x {H} heads of {D}")
+        n = shape[0] // (B * H)
+        dev = DeviceTensor.from_numpy(payload, stream)
+        call("trocm_kv_import_blocks", self._h, dev.ptr, n, _sh(stream))
+        call("trocm_stream_sync", _sh(stream))
+
     def clone(self, stream=None) -> "InPlaceKvCache":
         c = InPlaceKvCache(self.axis, self.storage_format, self.pool)
         if self._h is not None:
