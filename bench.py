@@ -32,11 +32,11 @@ sys.path.insert(0, ROOT)
 HQ, HKV, D, CTX = 32, 8, 128, 8192
 LAYERS = 4
 HBM_PEAK_GBS = 8000.0
-# HBM traffic of one decode-attention launch at the default arguments (batch 8, context 8328 in
-# the kernel loop), from two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE),
-# each counter scaled by what it reads for the 128 MiB prefill copy of known size: FETCH_SIZE
-# 133477.5 x 1.9991 KiB + WRITE_SIZE 520 x 1.000 KiB.
-PMC_TRAFFIC_BYTES_B8_CTX8328 = int((133477.5 * 1.9991 + 520.0) * 1024)
+# HBM traffic of one decode-attention launch at the default arguments (batch 8, context 8226 in the
+# kernel loop), from two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE), each
+# counter scaled by what it reads for the 128 MiB prefill copy of known size: FETCH_SIZE
+# 132120.1 x 1.9991 KiB + WRITE_SIZE 650 x 1.000 KiB.
+PMC_TRAFFIC_BYTES_B8_CTX8226 = int((132120.1 * 1.9991 + 650.0) * 1024)
 
 
 def cfg_seed(cfg, what):
@@ -367,7 +367,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(main_res["kernel_gbs"] / HBM_PEAK_GBS, 4),
-            "traffic": PMC_TRAFFIC_BYTES_B8_CTX8328 if (args.batch, args.steps, args.warmup) == (8, 128, 8) else None,
+            "traffic": PMC_TRAFFIC_BYTES_B8_CTX8226 if (args.batch, args.steps, args.warmup) == (8, 128, 8) else None,
             "kernel_us": round(main_res["kernel_us"], 3),
             "algorithmic_bytes_per_launch": main_res["kernel_bytes"],
             "cache_resident_achieved": round(main_res["cache_resident_kernel_gbs"], 2),
