@@ -296,6 +296,77 @@ def run_cfg5(ta, args):
                       "pool_in_use": st["bytes_in_use"], "pct_of_hbm_peak": round(100 * by / dt / 1e9 / HBM_PEAK_GBS, 2)})
 
 
+def run_ops(ta, args):
+    """The ops either side of the cache (RoPE, cast) and the sliding-window decode step, each against
+    its HBM roofline, with the oracle timed on the host for the same ops (smaller sample)."""
+    from oracle import oracle as orc
+    res = {}
+    rng = np.random.default_rng(7)
+    # RoPE on a prefill chunk: Q [1, 32, 4096, 128] f16 against [4096, 128] tables, rotating over 8 inputs (> 256 MB)
+    S = 4096
+    xs = [ta.DeviceTensor.from_numpy(rng.standard_normal((1, HQ, S, D)).astype(np.float16)) for _ in range(8)]
+    ang = rng.uniform(-3, 3, (S, D)).astype(np.float32)
+    cos, sin = ta.DeviceTensor.from_numpy(np.cos(ang).astype(np.float16)), ta.DeviceTensor.from_numpy(np.sin(ang).astype(np.float16))
+    out = ta.DeviceTensor((1, HQ, S, D), np.float16)
+    rope, turn = ta.ApplyRope(), [0]
+
+    def one_rope():
+        rope.eval(xs[turn[0] % 8], cos, sin, out=out)
+        turn[0] += 1
+
+    us = time_calls(ta, one_rope, 80)
+    by = 2 * HQ * S * D * 2 + 2 * S * D * 2   # x read, y written, tables once
+    res["apply_rope_f16_1x32x4096x128"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": by}
+    # cast f32 -> f16, 64 Mi elements, rotating over 4 inputs
+    n = 64 << 20
+    cs = [ta.DeviceTensor.from_numpy(rng.standard_normal(n, dtype=np.float32)) for _ in range(4)]
+    cast = ta.Cast(np.float16)
+    us = time_calls(ta, lambda: cast.eval(cs[0]), 3)   # warm the allocator path once
+    dst = ta.DeviceTensor((n,), np.float16)
+    from tract_amd._lib import call
+
+    def one_cast():
+        call("trocm_cast", cs[turn[0] % 4].ptr, 0, dst.ptr, 1, n, None)
+        turn[0] += 1
+
+    us = time_calls(ta, one_cast, 40)
+    res["cast_f32_f16_64Mi"] = {"us": round(us, 2), "gbs": round(n * 6 / us / 1e3, 1), "bytes": n * 6}
+    # sliding-window decode step: batch 8, window 4096, full ring (append wraps), 4 layers
+    W, B = 4096, 8
+    sts = [ta.WindowKvSdpa(axis=2, window=W).state() for _ in range(4)]
+    k0 = rng.standard_normal((B, HKV, W + 100, D)).astype(np.float16)
+    q0 = ta.DeviceTensor.from_numpy((rng.standard_normal((B, HQ, W + 100, D)) / np.sqrt(D)).astype(np.float16))
+    for st in sts:
+        st.eval([q0, k0, k0])
+    del q0
+    q1 = ta.DeviceTensor.from_numpy((rng.standard_normal((B, HQ, 1, D)) / np.sqrt(D)).astype(np.float16))
+    k1 = ta.DeviceTensor.from_numpy(rng.standard_normal((B, HKV, 1, D)).astype(np.float16))
+    o1 = ta.DeviceTensor((B, HQ, 1, D), np.float16)
+
+    def one_win():
+        sts[turn[0] % 4].eval([q1, k1, k1], out=o1)
+        turn[0] += 1
+
+    us = time_calls(ta, one_win, 100)
+    by = algorithmic_bytes(B, W)
+    res["window_kv_sdpa_step_b8_w4096"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by)}
+    # the oracle on the host for the same ops, on a bounded sample
+    xh = rng.standard_normal((1, 4, S, D)).astype(np.float16)
+    t0 = time.perf_counter()
+    orc.apply_rope(xh, np.cos(ang).astype(np.float16), np.sin(ang).astype(np.float16))
+    t_rope = (time.perf_counter() - t0) * (HQ / 4)
+    cpu = {"value": round(res["apply_rope_f16_1x32x4096x128"]["bytes"] / t_rope / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+           "sample": "ApplyRope of 4 of the 32 heads with the scalar C restatement, scaled to 32"}
+    head = res["apply_rope_f16_1x32x4096x128"]
+    roof = {"bound": "hbm", "kernel": "apply_rope_vec_kernel<f16>", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(head["gbs"] / HBM_PEAK_GBS, 4), "traffic": None}
+    line = base_line(args, "ops: ApplyRope on a 4096-token prefill chunk (32 heads, d=128, f16), cast f32->f16 of 64 Mi "
+                     "elements, sliding-window decode step (batch 8, window 4096); inputs rotate so that launches read HBM",
+                     head["gbs"], "GB/s", round(head["us"] / 1e3, 5), "f16", roof, {"cases": res})
+    line["cpu_baseline"] = cpu
+    return line
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -305,7 +376,7 @@ def main():
     ap.add_argument("--other-batches", type=str, default="1,32")
     ap.add_argument("--kernel-iters", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5"],
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "ops"],
                     help="cfg2 (default) is the configuration the metric is quoted on; the others print one line "
                          "of the same shape for the remaining configurations")
     args = ap.parse_args()
@@ -317,7 +388,7 @@ def main():
     import tract_amd as ta
     rt = ta.runtime_for_name("rocm")
     if args.workload != "cfg2":
-        line = {"cfg3": run_cfg3, "cfg4": run_cfg4, "cfg5": run_cfg5}[args.workload](ta, args)
+        line = {"cfg3": run_cfg3, "cfg4": run_cfg4, "cfg5": run_cfg5, "ops": run_ops}[args.workload](ta, args)
         line["device"] = rt.device_name
         print(json.dumps(line))
         return
