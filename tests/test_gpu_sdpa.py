@@ -108,6 +108,39 @@ def test_decode_split_k(rt, dt, B, Hq, Hkv, D, T):
     assert max_abs(out, cases.textbook_sdpa(q, k, v, causal=True)) <= (2e-3 if dt == np.float16 else 2e-5)
 
 
+@pytest.mark.parametrize("kind", ["random", "padding_min", "padding_inf", "leading_inf"])
+@pytest.mark.parametrize("dt,B,Hq,Hkv,D,T,mb,mh", [
+    (np.float16, 2, 32, 8, 128, 3000, 2, 1), (np.float16, 2, 32, 8, 128, 1025, 1, 32), (np.float16, 3, 8, 8, 64, 333, 3, 8),
+    (np.float32, 2, 8, 4, 64, 513, 2, 1), (np.float32, 1, 4, 2, 128, 200, 1, 4), (np.float16, 1, 16, 2, 128, 97, 1, 1),
+])
+def test_decode_with_additive_mask(rt, kind, dt, B, Hq, Hkv, D, T, mb, mh):
+    """Sq == 1 with a mask input [mask_b, mask_h, 1, T] (broadcast over batch and/or heads), the form in
+    which exported decoders state padding and windows (cuda/src/kernels/flash_attn.rs:138-143): served
+    by the split-K kernel.  Padded columns at the reference's finite minimum, at -inf, and -inf over
+    whole leading tiles (a tile, a wave or a split that sees nothing must contribute nothing)."""
+    rng = np.random.default_rng(200 + T)
+    q = (rng.standard_normal((B, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(dt)
+    k = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(dt)
+    v = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(dt)
+    mask = np.zeros((mb, mh, 1, T), dtype=np.float32)
+    if kind == "random":
+        mask = rng.standard_normal((mb, mh, 1, T), dtype=np.float32) * 3
+    else:
+        lo = -np.inf if kind.endswith("inf") else float(np.finfo(dt).min)
+        for b in range(mb):
+            for h in range(mh):
+                n = int(rng.integers(1, T))
+                if kind == "leading_inf":
+                    mask[b, h, 0, :T - n] = lo
+                else:
+                    mask[b, h, 0, n:] = lo
+    mask = mask.astype(dt)
+    got = tract_amd.Sdpa(datum_type=dt).eval(q, k, v, mask).to_numpy()
+    assert not np.isnan(got).any()
+    assert max_abs(got, orc.flash_sdpa(q, k, v, mask=mask)) <= TOL[np.dtype(dt)]
+    assert max_abs(got, cases.textbook_sdpa(q, k, v, mask)) <= (2e-3 if dt == np.float16 else 2e-5)
+
+
 @pytest.mark.parametrize("splits", [1, 2, 3, 7, 64])
 def test_decode_any_split_count_agrees(rt, splits, monkeypatch):
     # The split merge is exact in real arithmetic (log-sum-exp identity).
@@ -328,6 +361,46 @@ def test_prefill_grouped_heads_and_key_splits(rt, B, Hq, Hkv, Sq, Sk, D, causal)
     assert not np.isnan(got).any()
     assert max_abs(got, want) <= 2e-2
     assert max_abs(got, cases.textbook_sdpa(q, k, v, causal=causal)) <= 4e-3
+
+
+@pytest.mark.parametrize("kind", ["random", "causal_min", "causal_inf", "window_inf"])
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,mb,mh", [
+    (1, 32, 8, 512, 2048, 128, 1, 1),     # the chunked-prefill shape, one mask for all heads, key splits
+    (2, 8, 2, 130, 516, 128, 2, 8),       # a mask per batch and head
+    (1, 4, 2, 128, 641, 128, 1, 4),       # odd row length: element-wise mask loads
+    (2, 12, 2, 77, 302, 128, 2, 1), (3, 8, 8, 256, 256, 64, 1, 1), (1, 16, 4, 96, 1500, 64, 1, 16),
+    (1, 2, 2, 256, 256, 128, 1, 2),
+])
+def test_prefill_with_additive_mask(rt, kind, B, Hq, Hkv, Sq, Sk, D, mb, mh):
+    """q_len > 1 with a mask input [mask_b, mask_h, q_len, kv_len] (cuda/src/kernels/flash_attn.rs:138-143),
+    served by the MFMA kernel.  A causal mask stated as an input, with the reference's finite minimum
+    (sdpa.rs:550-553) or -inf above the diagonal, must reproduce is_causal; a banded (sliding-window)
+    mask leaves whole tiles and whole key splits with nothing visible."""
+    rng = np.random.default_rng(3000 + Sq + Sk + Hq)
+    q = (rng.standard_normal((B, Hq, Sq, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    k = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(np.float16)
+    i = np.arange(Sq)[:, None] + (Sk - Sq)
+    j = np.arange(Sk)[None, :]
+    if kind == "random":
+        mask = rng.standard_normal((mb, mh, Sq, Sk), dtype=np.float32) * 3
+    else:
+        lo = -np.inf if kind.endswith("inf") else float(np.finfo(np.float16).min)
+        hidden = j > i
+        if kind == "window_inf":
+            hidden = hidden | (j < i - 100)
+        mask = np.broadcast_to(np.where(hidden, lo, 0.0).astype(np.float32), (mb, mh, Sq, Sk)).copy()
+    mask = mask.astype(np.float16)
+    got = tract_amd.Sdpa(datum_type=np.float16).eval(q, k, v, mask).to_numpy()
+    assert not np.isnan(got).any()
+    if kind != "window_inf":
+        # (the CPU kernel starts from m = -inf and yields NaN for a row whose first key tile is all -inf
+        # while other rows of the tile are not, flash_sdpa.rs:309-316; the band is held to the f64 form)
+        assert max_abs(got, orc.flash_sdpa(q, k, v, mask=mask, threads=8)) <= 2e-2
+    assert max_abs(got, cases.textbook_sdpa(q, k, v, mask)) <= 4e-3
+    if kind.startswith("causal"):
+        same = tract_amd.Sdpa(datum_type=np.float16, is_causal=True).eval(q, k, v).to_numpy()
+        assert max_abs(got, same) <= 2e-3
 
 
 _PREFILL_ENV_CODE = """

@@ -42,6 +42,9 @@ struct DecodeDev {
     // != NULL: arrival counters (one int per (batch, kv head), zero between launches); the last
     // workgroup of a sequence-head to arrive merges the splits itself and no merge launch follows
     int *counters;
+    // additive mask of the q/out dtype, [mask_b, mask_h, 1, T] (NULL = none); byte strides, 0 on a broadcast axis
+    const char *mask;
+    int64_t mask_stride_b, mask_stride_h;
 };
 
 // Ragged batches: one work item = a tile range of one sequence (device copies of the host plan).

@@ -57,6 +57,8 @@ struct DecodeWork {
     int *counter;
     int nsplit;
     int64_t part_first, part_stride;
+    const char *mask;   // additive mask row of this kv head's first query head (NULL = none), token 0
+    int64_t mask_stride_h;
 };
 
 template <typename T, int D, int G>
@@ -121,9 +123,28 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
 
     u32x4 kreg[KL];
     vslice_t vreg[VI];
+    // Additive mask values of this lane's token, one per query head, fetched together with the tile's K
+    // (one tile ahead).  Rows past the end read the last token's value; they are discarded below.
+    const bool has_mask = wk.mask != nullptr;
+    T mreg[G];
+#pragma unroll
+    for (int h = 0; h < G; h++) mreg[h] = from_f32<T>(0.0f);
+    auto issue_mask = [&](int tile) {
+        const T *mrow = reinterpret_cast<const T *>(wk.mask) + min(tile * kTile + qk_row, last_tok);
+        if (wk.mask_stride_h == 0) {
+            const T v = *mrow;
+#pragma unroll
+            for (int h = 0; h < G; h++) mreg[h] = v;
+        } else {
+#pragma unroll
+            for (int h = 0; h < G; h++)
+                mreg[h] = *reinterpret_cast<const T *>(reinterpret_cast<const char *>(mrow) + h * wk.mask_stride_h);
+        }
+    };
     auto issue_k = [&](int tile) {
         const int t0 = tile * kTile;
         const char *base = kbase + (int64_t)t0 * p.kv_stride_t;
+        if (has_mask) issue_mask(tile);
         if (t0 + kTile <= cache_T) {
 #pragma unroll
             for (int j = 0; j < KL; j++) kreg[j] = *reinterpret_cast<const u32x4 *>(base + k_off[j]);
@@ -173,6 +194,9 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
         // 1. park the K tile in LDS (rotated chunks); its registers are then refilled
 #pragma unroll
         for (int j = 0; j < KL; j++) lds_k[w][k_slot[j]] = kreg[j];
+        float madd[G];
+#pragma unroll
+        for (int h = 0; h < G; h++) madd[h] = (float)mreg[h] * 1.4426950408889634f;
         const bool more = tile + tile_step < tile_end;
         if (more) issue_k(tile + tile_step);
 
@@ -193,9 +217,12 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
         for (int h = 0; h < G; h++) {
             float full = s[h] + dpp_f<kSwapPairs>(s[h]);  // join the two half rows
             float sv = valid ? full * p.scale_log2 : -INFINITY;
+            if (has_mask) sv += madd[h];
             float m_new = fmaxf(m[h], wave_max(sv));
-            float alpha = fast_exp2(m[h] - m_new);
-            pr[h] = fast_exp2(sv - m_new);
+            // a tile whose every token is masked with -inf must leave the state untouched, not NaN
+            const float m_ref = (has_mask && m_new == -INFINITY) ? 0.0f : m_new;
+            float alpha = fast_exp2(m[h] - m_ref);
+            pr[h] = fast_exp2(sv - m_ref);
             l[h] = l[h] * alpha + pr[h];  // both lanes of a pair add p: halved at the end
             m[h] = m_new;
 #pragma unroll
@@ -270,10 +297,12 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
         float mm = -INFINITY;
 #pragma unroll
         for (int ww = 0; ww < kWaves; ww++) mm = fmaxf(mm, comb[ww * kCombStride + G * D + h]);
+        // a range masked out entirely with -inf yields the neutral record (0, -inf, 0), not NaN
+        const float mm_ref = mm == -INFINITY ? 0.0f : mm;
         float acc = 0.0f, ll = 0.0f;
 #pragma unroll
         for (int ww = 0; ww < kWaves; ww++) {
-            float f = fast_exp2(comb[ww * kCombStride + G * D + h] - mm);
+            float f = fast_exp2(comb[ww * kCombStride + G * D + h] - mm_ref);
             acc += comb[ww * kCombStride + idx] * f;
             ll += comb[ww * kCombStride + G * D + G + h] * f;
         }
@@ -377,6 +406,8 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     wk.nsplit = p.nsplit;
     wk.part_first = bh * p.nsplit;
     wk.part_stride = 1;
+    wk.mask = p.mask ? p.mask + (int64_t)b * p.mask_stride_b + (int64_t)kvh * G * p.mask_stride_h : nullptr;
+    wk.mask_stride_h = p.mask_stride_h;
     decode_body<T, D, G>(p, wk);
 }
 
@@ -407,6 +438,8 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     wk.nsplit = it.nsplit;
     wk.part_first = (int64_t)it.slot0 * p.Hkv + kvh;
     wk.part_stride = p.Hkv;
+    wk.mask = nullptr;
+    wk.mask_stride_h = 0;
     decode_body<T, D, G>(p, wk);
 }
 
@@ -471,7 +504,7 @@ int choose_decode_splits(int64_t BH, int64_t G, int n_tiles, int wg_per_cu) {
 }
 
 int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
-    if (a.Sq != 1 || a.mask != nullptr) return 2;
+    if (a.Sq != 1) return 2;
     if (a.kv_fmt != TROCM_F16 && a.kv_fmt != TROCM_F32) return 2;
     if (a.q_dtype != a.kv_fmt) return 2;
     if (a.D != 64 && a.D != 128) return 2;
@@ -519,6 +552,11 @@ int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
     p.k_new = (const char *)a.k_new;
     p.v_new = (const char *)a.v_new;
     if (p.k_new && (p.v_new == nullptr || (uintptr_t)p.k_new % 16 || (uintptr_t)p.v_new % 16)) return 2;
+    if (a.mask) {   // [mask_b, mask_h, 1, Sk] dense
+        p.mask = (const char *)a.mask;
+        p.mask_stride_h = a.mask_h > 1 ? a.Sk * (int64_t)es : 0;
+        p.mask_stride_b = a.mask_b > 1 ? a.mask_h * a.Sk * (int64_t)es : 0;
+    }
     p.part_ml = (float *)((char *)a.workspace + kWsCounterBytes);
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * G;
     // With few splits the last workgroup of a (batch, kv head) to arrive merges them itself; with many

@@ -48,6 +48,10 @@ struct PrefillPP {
     float *part_ml;     // [nsplit][n_wb][2][32 queries]: m (log2 domain), then l
     int n_qb32;
     int64_t n_wb;
+    // additive mask [mask_b, mask_h, Sq, Sk] of f16 (masked kernels only); element strides, 0 on a broadcast axis
+    const _Float16 *mask;
+    int64_t mask_stride_b, mask_stride_h;
+    int mask_vec;       // rows allow 8-byte loads (Sk % 4 == 0 and an 8-byte aligned base)
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -62,7 +66,7 @@ __device__ __forceinline__ half4_t lds_read_tr16(const _Float16 *lds_ptr) {
 
 constexpr int kWavesPP = 8, kThreadsPP = 64 * kWavesPP, kTileN = 64;
 
-template <int D, int HG>
+template <int D, int HG, bool MASK>
 __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p) {
     constexpr int QB = kWavesPP / HG;     // 32-query blocks per workgroup
     constexpr int BLOCK_M = 32 * QB;
@@ -139,6 +143,27 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
         }
     };
 
+    // Mask values of this lane's query for the 32 keys it owns in a tile: 8 groups of 4 consecutive
+    // keys, fetched one tile ahead (issued right after the previous tile's softmax has consumed them).
+    half4_t mpre[MASK ? 8 : 1];
+    const _Float16 *mrow = nullptr;
+    if constexpr (MASK)
+        mrow = p.mask + (int64_t)b * p.mask_stride_b + (int64_t)qh * p.mask_stride_h + (int64_t)min(my_q, p.Sq - 1) * p.Sk;
+    auto prefetch_mask = [&](int kt) {
+        if constexpr (MASK) {
+#pragma unroll
+            for (int g = 0; g < 8; g++) {
+                const int key0 = kt * kTileN + 32 * (g >> 2) + 8 * (g & 3) + 4 * hb;
+                if (p.mask_vec) {
+                    mpre[g] = *reinterpret_cast<const half4_t *>(mrow + min(key0, p.Sk - 4));
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) mpre[g][i] = mrow[min(key0 + i, p.Sk - 1)];
+                }
+            }
+        }
+    };
+
     // does this wave have anything to do on tile kt?
     auto tile_active = [&](int kt) { return wave_has_queries && (!p.causal || kt * kTileN <= wave_q_last + off); };
 
@@ -162,6 +187,14 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
     // ---- online softmax for query lane%32 over this lane's 32 keys; leaves P^T fragments in pf ----
     auto softmax = [&](int kt, float16_t (&s)[2], half8_t (&pf)[4]) {
         const int k_lo = kt * kTileN;
+        if constexpr (MASK) {
+            // logits in the log2 domain, mask added: the maximum below is then taken after the scaling
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    s[kb][r] = __builtin_fmaf((float)mpre[4 * kb + (r >> 2)][r & 3], 1.4426950408889634f, s[kb][r] * p.scale_log2);
+        }
         const bool need_mask = (k_lo + kTileN > p.Sk) || (p.causal && (k_lo + kTileN - 1 > q0 + off));
         if (need_mask) {
 #pragma unroll
@@ -179,14 +212,15 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
 #pragma unroll
             for (int r = 0; r < 16; r++) tmax = fmaxf(tmax, s[kb][r]);
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float m_new = fmaxf(m_run, tmax * p.scale_log2);  // scale > 0: the maximum commutes with the scaling
+        const float m_new = fmaxf(m_run, MASK ? tmax : tmax * p.scale_log2);  // scale > 0: the maximum commutes with the scaling
         const float m_ref = (m_new == -INFINITY) ? 0.0f : m_new;  // nothing visible yet: keep everything at zero
         float psum = 0.0f;
 #pragma unroll
         for (int st = 0; st < 4; st++) {
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                float pv = fast_exp2(__builtin_fmaf(s[st >> 1][8 * (st & 1) + i], p.scale_log2, -m_ref));
+                const float sx = s[st >> 1][8 * (st & 1) + i];
+                float pv = fast_exp2(MASK ? sx - m_ref : __builtin_fmaf(sx, p.scale_log2, -m_ref));
                 psum += pv;
                 pf[st][i] = (_Float16)pv;
             }
@@ -234,6 +268,7 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
     if (n_it > 0) {
         stage(0, 0);
         if (n_it > 1) prefetch(t_begin + 1);
+        prefetch_mask(t_begin);
     }
     for (int it = 0; it < n_it; it++) {
         __syncthreads();   // tile `it` is in LDS; every wave is done with the buffers about to be overwritten
@@ -248,6 +283,7 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
             half8_t pf[4];
             qk(cur, s);
             softmax(kt, s, pf);
+            if (it + 1 < n_it) prefetch_mask(kt + 1);
             pv(cur, pf);
         }
     }
@@ -341,7 +377,10 @@ __global__ __launch_bounds__(256) void sdpa_prefill_merge_kernel(PrefillPP p) {
 
 template <int D, int HG>
 int launch_cfg(const PrefillPP &p, int64_t wgs, hipStream_t s) {
-    hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
+    if (p.mask)
+        hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG, true>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
+    else
+        hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG, false>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("sdpa_prefill_pp launch failed: %s", hipGetErrorString(e));
     if (p.nsplit > 1) {
@@ -382,7 +421,8 @@ size_t prefill_workspace_bytes(int64_t B, int64_t Hq, int64_t Sq, int64_t D) {
 }
 
 int launch_sdpa_prefill_pp(const SdpaArgs &a, hipStream_t s) {
-    if (a.q_dtype != TROCM_F16 || a.kv_fmt != TROCM_F16 || a.mask != nullptr) return 2;
+    if (a.q_dtype != TROCM_F16 || a.kv_fmt != TROCM_F16) return 2;
+    if (a.mask && a.causal) return 2;
     if (a.D != 128 && a.D != 64) return 2;
     if (a.Sq < 2 || a.Sk < 1 || a.Hq % a.Hkv) return 2;
     if (!(a.scale > 0.0f)) return 2;       // the running maximum is taken before scaling
@@ -415,6 +455,12 @@ int launch_sdpa_prefill_pp(const SdpaArgs &a, hipStream_t s) {
     p.n_qtiles = (int)n_qtiles;
     p.n_qb32 = (int)((a.Sq + 31) / 32);
     p.n_wb = a.B * a.Hq * p.n_qb32;
+    if (a.mask) {   // [mask_b, mask_h, Sq, Sk] dense
+        p.mask = (const _Float16 *)a.mask;
+        p.mask_stride_h = a.mask_h > 1 ? a.Sq * a.Sk : 0;
+        p.mask_stride_b = a.mask_b > 1 ? a.mask_h * a.Sq * a.Sk : 0;
+        p.mask_vec = a.Sk % 4 == 0 && (uintptr_t)a.mask % 8 == 0;
+    }
 
     const int64_t wgs1 = a.B * (a.Hq / hg) * n_qtiles;
     const int64_t cus = num_compute_units();
