@@ -350,6 +350,41 @@ def run_ops(ta, args):
     us = time_calls(ta, one_win, 100)
     by = algorithmic_bytes(B, W)
     res["window_kv_sdpa_step_b8_w4096"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by)}
+    del sts, xs, cs
+    # mask inputs on the fast attention kernels: decode (batch 8, 8192 tokens, padding mask [8,1,1,T]) over
+    # 4 layers' K/V, and a 512-query chunk over 4096 keys with the causal mask stated as an input [1,1,512,4096]
+    T = 8192
+    kvs = [(ta.DeviceTensor.from_numpy(rng.standard_normal((B, HKV, T, D)).astype(np.float16)),
+            ta.DeviceTensor.from_numpy(rng.standard_normal((B, HKV, T, D)).astype(np.float16))) for _ in range(4)]
+    pad = np.zeros((B, 1, 1, T), np.float16)
+    for b in range(B):
+        pad[b, :, :, T - 37 * b:] = np.finfo(np.float16).min
+    pad = ta.DeviceTensor.from_numpy(pad)
+    sd = ta.Sdpa(datum_type=np.float16)
+
+    def one_masked(masked):
+        kk, vv = kvs[turn[0] % 4]
+        sd.eval(q1, kk, vv, pad if masked else None, out=o1)
+        turn[0] += 1
+
+    by = algorithmic_bytes(B, T)
+    for name, masked in (("decode_b8_ctx8192_padding_mask", True), ("decode_b8_ctx8192_no_mask", False)):
+        us = time_calls(ta, lambda: one_masked(masked), 100)
+        res[name] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by)}
+    Sq, Sk = 512, 4096
+    qp = ta.DeviceTensor.from_numpy((rng.standard_normal((1, HQ, Sq, D)) / np.sqrt(D)).astype(np.float16))
+    op = ta.DeviceTensor((1, HQ, Sq, D), np.float16)
+    cm = np.where(np.arange(Sk)[None, :] > np.arange(Sq)[:, None] + (Sk - Sq), np.finfo(np.float16).min, 0).astype(np.float16)
+    cm = ta.DeviceTensor.from_numpy(cm.reshape(1, 1, Sq, Sk))
+    kk, vv = kvs[0]
+    kp = ta.DeviceTensor.from_numpy(kk.to_numpy()[:1, :, :Sk].copy())
+    vp = ta.DeviceTensor.from_numpy(vv.to_numpy()[:1, :, :Sk].copy())
+    sc = ta.Sdpa(datum_type=np.float16, is_causal=True)
+    fl = 4.0 * HQ * D * (Sq * Sk - Sq * (Sq - 1) / 2)
+    us = time_calls(ta, lambda: sd.eval(qp, kp, vp, cm, out=op), 50)
+    res["prefill_512x4096_causal_as_mask_input"] = {"us": round(us, 2), "tflops": round(fl / us / 1e6, 1)}
+    us = time_calls(ta, lambda: sc.eval(qp, kp, vp, out=op), 50)
+    res["prefill_512x4096_is_causal"] = {"us": round(us, 2), "tflops": round(fl / us / 1e6, 1)}
     # the oracle on the host for the same ops, on a bounded sample
     xh = rng.standard_normal((1, 4, S, D)).astype(np.float16)
     t0 = time.perf_counter()

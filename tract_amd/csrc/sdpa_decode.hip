@@ -61,7 +61,7 @@ struct DecodeWork {
     int64_t mask_stride_h;
 };
 
-template <typename T, int D, int G>
+template <typename T, int D, int G, bool MASK>
 __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork &wk) {
     constexpr int RB = D * sizeof(T);   // bytes of one K/V row: 128, 256 or 512
     constexpr int CPR = RB / 16;        // 16-byte chunks per row: 8, 16, 32
@@ -78,7 +78,7 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int w = tid >> 6;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, and the compiler is told so: tile bases stay in scalar registers
 
     // ---- stage the G query vectors of this KV head ------------------------------------
     {
@@ -123,28 +123,25 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
 
     u32x4 kreg[KL];
     vslice_t vreg[VI];
-    // Additive mask values of this lane's token, one per query head, fetched together with the tile's K
-    // (one tile ahead).  Rows past the end read the last token's value; they are discarded below.
-    const bool has_mask = wk.mask != nullptr;
+    // Additive mask values of this lane's token, one per query head, fetched one tile ahead, right after
+    // the softmax that consumed the previous ones (so no second copy stays live across the QK phase: the
+    // G=4 kernel has no register to spare, and a spill reload in the loop waits for vmcnt(0), i.e. for
+    // every prefetch in flight).  Rows past the end read the last token's value; they are discarded
+    // below.  The masked kernel is a separate instantiation and always issues G loads (a head stride
+    // of 0 when the mask is shared), so that the compiler can count outstanding loads exactly.
+    constexpr bool has_mask = MASK;
     T mreg[G];
 #pragma unroll
     for (int h = 0; h < G; h++) mreg[h] = from_f32<T>(0.0f);
     auto issue_mask = [&](int tile) {
-        const T *mrow = reinterpret_cast<const T *>(wk.mask) + min(tile * kTile + qk_row, last_tok);
-        if (wk.mask_stride_h == 0) {
-            const T v = *mrow;
+        // wave-uniform row bases plus one 32-bit lane offset
+        const uint32_t moff = (uint32_t)min(tile * kTile + qk_row, last_tok) * (uint32_t)sizeof(T);
 #pragma unroll
-            for (int h = 0; h < G; h++) mreg[h] = v;
-        } else {
-#pragma unroll
-            for (int h = 0; h < G; h++)
-                mreg[h] = *reinterpret_cast<const T *>(reinterpret_cast<const char *>(mrow) + h * wk.mask_stride_h);
-        }
+        for (int h = 0; h < G; h++) mreg[h] = *reinterpret_cast<const T *>(wk.mask + h * wk.mask_stride_h + moff);
     };
     auto issue_k = [&](int tile) {
         const int t0 = tile * kTile;
         const char *base = kbase + (int64_t)t0 * p.kv_stride_t;
-        if (has_mask) issue_mask(tile);
         if (t0 + kTile <= cache_T) {
 #pragma unroll
             for (int j = 0; j < KL; j++) kreg[j] = *reinterpret_cast<const u32x4 *>(base + k_off[j]);
@@ -183,6 +180,7 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
 
     int tile = tile_begin + w;
     if (tile < tile_end) {
+        if constexpr (has_mask) issue_mask(tile);
         issue_k(tile);
         issue_v(tile);
     }
@@ -194,9 +192,6 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
         // 1. park the K tile in LDS (rotated chunks); its registers are then refilled
 #pragma unroll
         for (int j = 0; j < KL; j++) lds_k[w][k_slot[j]] = kreg[j];
-        float madd[G];
-#pragma unroll
-        for (int h = 0; h < G; h++) madd[h] = (float)mreg[h] * 1.4426950408889634f;
         const bool more = tile + tile_step < tile_end;
         if (more) issue_k(tile + tile_step);
 
@@ -217,7 +212,7 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
         for (int h = 0; h < G; h++) {
             float full = s[h] + dpp_f<kSwapPairs>(s[h]);  // join the two half rows
             float sv = valid ? full * p.scale_log2 : -INFINITY;
-            if (has_mask) sv += madd[h];
+            if constexpr (has_mask) sv = __builtin_fmaf((float)mreg[h], 1.4426950408889634f, sv);
             float m_new = fmaxf(m[h], wave_max(sv));
             // a tile whose every token is masked with -inf must leave the state untouched, not NaN
             const float m_ref = (has_mask && m_new == -INFINITY) ? 0.0f : m_new;
@@ -227,6 +222,9 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
             m[h] = m_new;
 #pragma unroll
             for (int e = 0; e < EPL; e++) o[h][e] *= alpha;
+        }
+        if constexpr (has_mask) {
+            if (more) issue_mask(tile + tile_step);
         }
         if (qk_half == 0) {
             if constexpr (G == 4) {
@@ -376,7 +374,7 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
 }
 
 // Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.
-template <typename T, int D, int G>
+template <typename T, int D, int G, bool MASK>
 __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1) void sdpa_decode_kernel(DecodeDev p) {
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     DecodeWork wk;
@@ -406,9 +404,9 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     wk.nsplit = p.nsplit;
     wk.part_first = bh * p.nsplit;
     wk.part_stride = 1;
-    wk.mask = p.mask ? p.mask + (int64_t)b * p.mask_stride_b + (int64_t)kvh * G * p.mask_stride_h : nullptr;
+    wk.mask = MASK ? p.mask + (int64_t)b * p.mask_stride_b + (int64_t)kvh * G * p.mask_stride_h : nullptr;
     wk.mask_stride_h = p.mask_stride_h;
-    decode_body<T, D, G>(p, wk);
+    decode_body<T, D, G, MASK>(p, wk);
 }
 
 // Ragged batch: grid (work items, kv_heads).  An item is a tile range of one sequence; the
@@ -440,7 +438,7 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     wk.part_stride = p.Hkv;
     wk.mask = nullptr;
     wk.mask_stride_h = 0;
-    decode_body<T, D, G>(p, wk);
+    decode_body<T, D, G, false>(p, wk);
 }
 
 // Merge launch of the ragged batch: grid (kv_heads, sequences, G), D threads.
@@ -455,7 +453,10 @@ __global__ __launch_bounds__(D) void sdpa_decode_ragged_merge_kernel(DecodeDev p
 
 template <typename T, int D, int G>
 void launch_both(const DecodeDev &p, dim3 grid, hipStream_t s) {
-    hipLaunchKernelGGL((sdpa_decode_kernel<T, D, G>), grid, dim3(kThreads), 0, s, p);
+    if (p.mask)
+        hipLaunchKernelGGL((sdpa_decode_kernel<T, D, G, true>), grid, dim3(kThreads), 0, s, p);
+    else
+        hipLaunchKernelGGL((sdpa_decode_kernel<T, D, G, false>), grid, dim3(kThreads), 0, s, p);
     if (p.nsplit > 1 && p.counters == nullptr)
         hipLaunchKernelGGL((sdpa_decode_merge_kernel<T, D, G>), dim3(grid.y, grid.z, G), dim3(D), 0, s, p);
 }

@@ -292,7 +292,7 @@ class Sdpa:
             raise TractRocmError(f"Q heads ({q_shape[1]}) must be a multiple of K/V heads ({k_shape[1]})")
         return tuple(q_shape[:-1]) + (v_shape[-1],)
 
-    def eval(self, q, k, v, mask=None, stream=None) -> DeviceTensor:
+    def eval(self, q, k, v, mask=None, stream=None, out=None) -> DeviceTensor:
         q, k, v = (_as_device(t, stream) for t in (q, k, v))
         m = None if mask is None else _as_device(mask, stream)
         self.output_facts(q.shape, k.shape, v.shape, None if m is None else m.shape)
@@ -308,7 +308,10 @@ class Sdpa:
             if ms[2:] != (Sq, Sk):
                 raise TractRocmError(f"mask shape {m.shape} does not end in [q_len, kv_len]")
             mb, mh = ms[0], ms[1]
-        out = DeviceTensor(q.shape, q.dtype)
+        if out is None:
+            out = DeviceTensor(q.shape, q.dtype)
+        elif tuple(out.shape) != tuple(q.shape) or out.dtype != q.dtype:
+            raise TractRocmError("out must have Q's shape and datum type")
         if self._ws is None or self._ws_key != (B, Hq, D) or self._ws.nbytes < Workspace.bytes_for(B, Hq, Sq, D):
             self._ws, self._ws_key = Workspace(B, Hq, Sq, D, stream), (B, Hq, D)
         call("trocm_sdpa", q.ptr, k.ptr, v.ptr, None if m is None else m.ptr, out.ptr, dtype_code(q.dtype),
