@@ -74,7 +74,7 @@ __global__ __launch_bounds__(kThreads, G <= 4 ? 2 : 1) void sdpa_decode_q_kernel
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int w = tid >> 6;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, and the compiler is told so
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
 
     {

@@ -83,7 +83,7 @@ __global__ __launch_bounds__(64 * WM * WN) void sdpa_prefill_kernel(PrefillDev p
     _Float16 *lds_k = lds_all;
     _Float16 *lds_v = lds_all + BLOCK_N * KROW;
 
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hb = lane >> 5, l32 = lane & 31;
     const int wm = w % WM, wn = w / WM;
 

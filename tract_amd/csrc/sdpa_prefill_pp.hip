@@ -52,6 +52,9 @@ struct PrefillPP {
     const _Float16 *mask;
     int64_t mask_stride_b, mask_stride_h;
     int mask_vec;       // rows allow 8-byte loads (Sk % 4 == 0 and an 8-byte aligned base)
+    // != NULL: arrival counters, one per (batch, query tile, head group, kv head), zero between launches;
+    // the last key split of a tile to arrive merges the partials itself and no merge launch follows
+    int *counters;
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -80,7 +83,7 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
     __shared__ __attribute__((aligned(16))) _Float16 lds_k[2][kTileN * KROW];
     __shared__ __attribute__((aligned(16))) _Float16 lds_v[2][kTileN * VROW];
 
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hb = lane >> 5, l32 = lane & 31;
 
     // workgroup -> (kv head fastest: consecutive workgroup ids go round-robin to the 8 XCDs, so
@@ -289,9 +292,8 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
     }
 
     l_run += __shfl_xor(l_run, 32, 64);
-    if (!wave_has_queries) return;
     if (p.nsplit == 1) {
-        if (my_q >= p.Sq) return;
+        if (!wave_has_queries || my_q >= p.Sq) return;
         const int64_t row = ((int64_t)b * p.Hq + qh) * p.Sq + my_q;
         const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
         _Float16 *orow = p.out + row * D;
@@ -304,10 +306,18 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
                 for (int i = 0; i < 4; i++) h4[i] = (_Float16)(o[db][4 * rq + i] * inv);
                 *reinterpret_cast<half4_t *>(orow + 32 * db + 8 * rq + 4 * hb) = h4;
             }
-    } else {
-        const int64_t wb = ((int64_t)b * p.Hq + qh) * p.n_qb32 + (q0 >> 5);
+        return;
+    }
+    // ---- key splits: store this split's normalised partial -----------------------------------------
+    // With arrival counters the stores are agent-scope write-through stores: they are visible to every
+    // compute unit of the device once they complete, so no cache write-back is needed before the
+    // workgroup signals its arrival.
+    const bool tail_merge = p.counters != nullptr;
+    const int64_t wb = ((int64_t)b * p.Hq + qh) * p.n_qb32 + (q0 >> 5);
+    if (wave_has_queries) {
         const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
         _Float16 *po = p.part_o + ((int64_t)split * p.n_wb + wb) * (32 * D) + l32 * 4;
+        float *pml = p.part_ml + ((int64_t)split * p.n_wb + wb) * 64 + lane;
 #pragma unroll
         for (int db = 0; db < DB; db++)
 #pragma unroll
@@ -315,10 +325,103 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
                 half4_t h4;
 #pragma unroll
                 for (int i = 0; i < 4; i++) h4[i] = (_Float16)(o[db][4 * rq + i] * inv);
-                *reinterpret_cast<half4_t *>(po + (8 * db + 2 * rq + hb) * 128) = h4;
+                _Float16 *dst = po + (8 * db + 2 * rq + hb) * 128;
+                if (tail_merge)
+                    __hip_atomic_store(reinterpret_cast<uint64_t *>(dst), __builtin_bit_cast(uint64_t, h4), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                else
+                    *reinterpret_cast<half4_t *>(dst) = h4;
             }
-        p.part_ml[((int64_t)split * p.n_wb + wb) * 64 + lane] = hb ? l_run : m_run;
+        if (tail_merge)
+            __hip_atomic_store(pml, hb ? l_run : m_run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else
+            *pml = hb ? l_run : m_run;
     }
+    if (!tail_merge) return;
+
+    // ---- the last split of this tile to arrive merges all of them ------------------------------------
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's partial stores have completed
+    __syncthreads();                                     // ... and so have the whole workgroup's
+    __shared__ int s_last;
+    if (tid == 0) {
+        int *counter = p.counters + (((int64_t)b * p.n_qtiles + qt) * (G / HG) + gg) * p.Hkv + kvh;
+        const int arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = arrived == p.nsplit - 1;
+        if (s_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+    }
+    __syncthreads();
+    if (!s_last || !wave_has_queries) return;
+    // Every wave merges its own 32-query block: out = sum_s w_s O_s, w_s = l_s 2^(m_s - max m) / sum.
+    // The weights go through a wave-private corner of the (now idle) K tile buffer; the partial
+    // outputs are laid out as the accumulators are, so each lane reads back exactly its own elements,
+    // two splits in flight at a time.
+    constexpr int kMaxSplits = 16, kMergeBatch = 2;
+    auto aload_f = [](const float *a) { return __hip_atomic_load(a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    float *wts = reinterpret_cast<float *>(&lds_k[0][0]) + w * (kMaxSplits * 32);
+    {
+        float mv[kMaxSplits], lv[kMaxSplits];
+#pragma unroll
+        for (int sp = 0; sp < kMaxSplits; sp++) {
+            const float *ml = p.part_ml + ((int64_t)min(sp, p.nsplit - 1) * p.n_wb + wb) * 64;
+            mv[sp] = aload_f(ml + l32);
+            lv[sp] = aload_f(ml + 32 + l32);
+        }
+        float mm = -INFINITY;
+#pragma unroll
+        for (int sp = 0; sp < kMaxSplits; sp++) mm = fmaxf(mm, mv[sp]);
+        const float m_ref = (mm == -INFINITY) ? 0.0f : mm;
+        float total = 0.0f;
+#pragma unroll
+        for (int sp = 0; sp < kMaxSplits; sp++) {
+            lv[sp] = sp < p.nsplit ? lv[sp] * fast_exp2(mv[sp] - m_ref) : 0.0f;
+            total += lv[sp];
+        }
+        const float inv = total > 0.0f ? 1.0f / total : 0.0f;
+        if (hb == 0) {
+#pragma unroll
+            for (int sp = 0; sp < kMaxSplits; sp++) wts[sp * 32 + l32] = lv[sp] * inv;
+        }
+    }
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
+    for (int s0 = 0; s0 < p.nsplit; s0 += kMergeBatch) {
+        uint64_t raw[kMergeBatch][DB * 4];
+#pragma unroll
+        for (int j = 0; j < kMergeBatch; j++) {
+            const _Float16 *po = p.part_o + ((int64_t)min(s0 + j, p.nsplit - 1) * p.n_wb + wb) * (32 * D) + l32 * 4;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++)
+                    raw[j][db * 4 + rq] = __hip_atomic_load(reinterpret_cast<const uint64_t *>(po + (8 * db + 2 * rq + hb) * 128),
+                                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int j = 0; j < kMergeBatch; j++) {
+            const float wgt = s0 + j < p.nsplit ? wts[(s0 + j) * 32 + l32] : 0.0f;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    const half4_t h4 = __builtin_bit_cast(half4_t, raw[j][db * 4 + rq]);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) o[db][4 * rq + i] += wgt * (float)h4[i];
+                }
+        }
+    }
+    if (my_q >= p.Sq) return;
+    _Float16 *orow = p.out + (((int64_t)b * p.Hq + qh) * p.Sq + my_q) * D;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int rq = 0; rq < 4; rq++) {
+            half4_t h4;
+#pragma unroll
+            for (int i = 0; i < 4; i++) h4[i] = (_Float16)o[db][4 * rq + i];
+            *reinterpret_cast<half4_t *>(orow + 32 * db + 8 * rq + 4 * hb) = h4;
+        }
 }
 
 // Merge of the key splits, one workgroup per 32-query block:
@@ -383,7 +486,7 @@ int launch_cfg(const PrefillPP &p, int64_t wgs, hipStream_t s) {
         hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG, false>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("sdpa_prefill_pp launch failed: %s", hipGetErrorString(e));
-    if (p.nsplit > 1) {
+    if (p.nsplit > 1 && p.counters == nullptr) {
         hipLaunchKernelGGL((sdpa_prefill_merge_kernel<D>), dim3((unsigned)p.n_wb), dim3(256), 0, s, p);
         e = hipGetLastError();
         if (e != hipSuccess) return fail("sdpa_prefill_merge launch failed: %s", hipGetErrorString(e));
@@ -471,7 +574,7 @@ int launch_sdpa_prefill_pp(const SdpaArgs &a, hipStream_t s) {
         if (ns > tiles / 2) ns = tiles / 2;   // at least two tiles per split
         if (ns > 16) ns = 16;
     }
-    if (forced_split > 0) ns = forced_split;
+    if (forced_split > 0) ns = forced_split < 16 ? forced_split : 16;   // the merges handle at most 16 splits
     const size_t per_split = split_bytes(p.n_wb, a.D);
     const size_t avail = a.workspace && a.workspace_bytes > kWsCounterBytes + 256 ? a.workspace_bytes - kWsCounterBytes - 256 : 0;
     if (ns > 1 && (size_t)ns * per_split > avail) ns = (int64_t)(avail / per_split);
@@ -482,6 +585,10 @@ int launch_sdpa_prefill_pp(const SdpaArgs &a, hipStream_t s) {
         base += (256 - ((uintptr_t)base & 255)) & 255;
         p.part_o = (_Float16 *)base;
         p.part_ml = (float *)(base + (size_t)ns * p.n_wb * 32 * a.D * sizeof(_Float16));
+        // With few enough tiles for the counter area the last split to arrive merges (no second launch);
+        // TROCM_PREFILL_TAIL_MERGE=0 keeps the merge launch.
+        static const int tail_merge = env_int("TROCM_PREFILL_TAIL_MERGE", 1);
+        if (tail_merge && ns <= 16 && wgs1 <= (int64_t)(kWsCounterBytes / sizeof(int))) p.counters = (int *)a.workspace;
     }
     const int64_t wgs = wgs1 * ns;
     if (wgs >= (1ll << 31)) return 2;
