@@ -971,7 +971,7 @@ int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_n
         if (kc->cap == vc->cap) {
             SdpaArgs a;
             cached_args(a, q, dtype, q_heads, 1, kc, vc, kc->len + 1, out, scale, causal, workspace, workspace_bytes);
-            a.k_new = k_new, a.v_new = v_new;
+            a.k_new = k_new, a.v_new = v_new, a.new_pos = -1;
             int rc = launch_sdpa_decode(a, s);
             if (rc == 0) {
                 kc->len += 1;
@@ -996,7 +996,36 @@ int trocm_window_kv_sdpa_eval(const void *q, const void *k_new, const void *v_ne
     TROCM_REQUIRE(kc->window > 0 && vc->window == kc->window, "window_kv_sdpa: K and V must be sliding-window caches of one window");
     int64_t dense[4];
     dense[3] = 1, dense[2] = kc->D, dense[1] = n_new * kc->D, dense[0] = kc->H * n_new * kc->D;
-    if (!kv_new_strides) kv_new_strides = dense;
+    bool is_dense = kv_new_strides == nullptr;
+    if (!is_dense) {
+        is_dense = true;
+        for (int i = 0; i < 4; i++) is_dense = is_dense && kv_new_strides[i] == dense[i];
+    } else {
+        kv_new_strides = dense;
+    }
+    // Decode step on a plain-format ring: the attention kernel reads the new token from the inputs and
+    // stores it at the cursor itself -- one launch instead of append + attention.
+    if (n_new == 1 && is_dense && !is_quant(kc->fmt) && dtype == kc->fmt && q && k_new && v_new && out && kc->fmt == vc->fmt &&
+        kc->B == vc->B && kc->H == vc->H && kc->D == vc->D && kc->len == vc->len && kc->cursor == vc->cursor &&
+        q_heads % kc->H == 0) {
+        hipStream_t s;
+        if (resolve_stream(stream, &s)) return 1;
+        if (append_prepare(kc, k_new, dtype, kv_new_strides, 1, s)) return 1;
+        if (append_prepare(vc, v_new, dtype, kv_new_strides, 1, s)) return 1;
+        if (kc->cap == vc->cap && kc->cap == kc->window) {
+            const int64_t w = kc->window, new_len = kc->len + 1 < w ? kc->len + 1 : w;
+            SdpaArgs a;
+            cached_args(a, q, dtype, q_heads, 1, kc, vc, new_len, out, scale, 0, workspace, workspace_bytes);
+            a.k_new = k_new, a.v_new = v_new, a.new_pos = kc->cursor;
+            int rc = launch_sdpa_decode(a, s);
+            if (rc == 0) {
+                kc->cursor = vc->cursor = kc->cursor + 1 == w ? 0 : kc->cursor + 1;
+                kc->len = vc->len = new_len;
+                return 0;
+            }
+            if (rc != 2) return rc;
+        }
+    }
     if (trocm_kv_append_pair(kc, vc, k_new, v_new, dtype, kv_new_strides, n_new, stream)) return 1;
     return trocm_sdpa_cached(q, dtype, q_heads, n_new, kc, vc, out, scale, 0, workspace, workspace_bytes, stream);
 }

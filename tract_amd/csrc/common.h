@@ -114,6 +114,7 @@ struct SdpaArgs {
     // fused append (split-K decode of plain formats only): the new token's K and V rows, dense
     // [B, Hkv, 1, D]; they are token Sk-1, read from here and stored into the cache by the kernel
     const void *k_new, *v_new;
+    int64_t new_pos;        // token index the fused new token is stored at; < 0 means Sk - 1 (ring buffers pass the cursor)
     int64_t B, Hq, Hkv, Sq, Sk, D;
     int64_t kv_stride_b, kv_stride_h, kv_stride_t;       // in ELEMENTS of the logical [.., D] tensor rows
     const void *mask;       // of q_dtype, [mask_b, mask_h, Sq, Sk]

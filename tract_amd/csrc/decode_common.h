@@ -36,6 +36,7 @@ struct DecodeDev {
     int64_t sc_stride_b, sc_stride_h;  // bytes
     // fused append (plain formats): the step's new K/V rows, dense [B or n_seq, Hkv, 1, D]; NULL = none
     const char *k_new, *v_new;
+    int new_pos;   // token index of the fused new token (T - 1 for a growing cache, the cursor of a ring buffer)
     // dense f16/f32 kernel: 1 = the splits of a sequence take groups of kWaves tiles round-robin
     // (concurrent workgroups then read neighbouring addresses), 0 = contiguous tile ranges
     int interleave;

@@ -46,7 +46,8 @@ struct DecodeWork {
     const char *q;      // the G query rows of this kv head
     char *out;          // the G output rows
     const char *kbase, *vbase;
-    const char *k_new, *v_new;  // fused append: the row of token T-1 is read from here and stored to the cache
+    const char *k_new, *v_new;  // fused append: the row of token new_pos is read from here and stored to the cache
+    int new_pos;
     int T;              // valid tokens of the sequence (including a fused new token)
     int tile_begin, tile_end;
     int tile_step;      // distance between a wave's successive tiles (kWaves for a contiguous range)
@@ -89,7 +90,9 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
 
     const char *kbase = wk.kbase, *vbase = wk.vbase;
     const int seq_T = wk.T;
-    const int cache_T = wk.k_new ? seq_T - 1 : seq_T;  // tokens already stored in the cache
+    const int new_pos = wk.k_new ? wk.new_pos : -1;   // the token that comes from the step's input, if any
+    // a tile takes the plain path when it is full and does not hold the new token
+    auto plain_tile = [&](int t0) { return t0 + kTile <= seq_T && !(new_pos >= t0 && new_pos < t0 + kTile); };
     const int tile_begin = wk.tile_begin, tile_end = wk.tile_end, tile_step = wk.tile_step;
     const int last_tok = seq_T - 1;
 
@@ -142,27 +145,28 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
     auto issue_k = [&](int tile) {
         const int t0 = tile * kTile;
         const char *base = kbase + (int64_t)t0 * p.kv_stride_t;
-        if (t0 + kTile <= cache_T) {
+        if (plain_tile(t0)) {
 #pragma unroll
             for (int j = 0; j < KL; j++) kreg[j] = *reinterpret_cast<const u32x4 *>(base + k_off[j]);
         } else {
-            // the sequence's last tile: rows past the end repeat the last token; a fused new token
-            // comes from the step's input and is written to its place in the cache on the way
+            // the sequence's last tile and the tile of a fused new token: rows past the end repeat the
+            // last token; the new token comes from the step's input and is written to its place in
+            // the cache on the way
 #pragma unroll
             for (int j = 0; j < KL; j++) {
                 int L = j * 64 + lane;
                 int row = min(L / CPR, last_tok - t0), c = L % CPR;
                 const char *cache_ptr = base + (uint32_t)row * stride_t + (uint32_t)c * 16u;
-                const bool is_new = wk.k_new != nullptr && t0 + row == last_tok;
+                const bool is_new = t0 + row == new_pos;
                 kreg[j] = *reinterpret_cast<const u32x4 *>(is_new ? wk.k_new + c * 16 : cache_ptr);
-                if (is_new && L / CPR == last_tok - t0) *reinterpret_cast<u32x4 *>(const_cast<char *>(cache_ptr)) = kreg[j];
+                if (is_new && L / CPR == new_pos - t0) *reinterpret_cast<u32x4 *>(const_cast<char *>(cache_ptr)) = kreg[j];
             }
         }
     };
     auto issue_v = [&](int tile) {
         const int t0 = tile * kTile;
         const char *base = vbase + (int64_t)t0 * p.kv_stride_t;
-        if (t0 + kTile <= cache_T) {
+        if (plain_tile(t0)) {
 #pragma unroll
             for (int i = 0; i < VI; i++) vreg[i] = *reinterpret_cast<const vslice_t *>(base + v_off[i]);
         } else {
@@ -170,9 +174,9 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
             for (int i = 0; i < VI; i++) {
                 int row = min(4 * i + rg, last_tok - t0);
                 const char *cache_ptr = base + (uint32_t)row * stride_t + (uint32_t)j16 * (uint32_t)sizeof(vslice_t);
-                const bool is_new = wk.v_new != nullptr && t0 + row == last_tok;
+                const bool is_new = t0 + row == new_pos;
                 vreg[i] = *reinterpret_cast<const vslice_t *>(is_new ? wk.v_new + j16 * (int)sizeof(vslice_t) : cache_ptr);
-                if (is_new && 4 * i + rg == last_tok - t0)
+                if (is_new && 4 * i + rg == new_pos - t0)
                     *reinterpret_cast<vslice_t *>(const_cast<char *>(cache_ptr)) = vreg[i];
             }
         }
@@ -387,6 +391,7 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     wk.k_new = p.k_new ? p.k_new + new_row : nullptr;
     wk.v_new = p.v_new ? p.v_new + new_row : nullptr;
     wk.T = p.T;
+    wk.new_pos = p.new_pos;
     const int n_tiles = (p.T + kTile - 1) / kTile;
     if (p.interleave) {
         wk.tile_begin = split * kWaves;
@@ -427,6 +432,7 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     wk.k_new = p.k_new ? p.k_new + new_row : nullptr;
     wk.v_new = p.v_new ? p.v_new + new_row : nullptr;
     wk.T = it.T;
+    wk.new_pos = it.T - 1;
     wk.tile_begin = it.tile_begin;
     wk.tile_end = it.tile_end;
     wk.tile_step = kWaves;
@@ -552,6 +558,7 @@ int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
     p.scale_log2 = a.scale * 1.4426950408889634f;
     p.k_new = (const char *)a.k_new;
     p.v_new = (const char *)a.v_new;
+    p.new_pos = a.new_pos >= 0 ? (int)a.new_pos : (int)a.Sk - 1;
     if (p.k_new && (p.v_new == nullptr || (uintptr_t)p.k_new % 16 || (uintptr_t)p.v_new % 16)) return 2;
     if (a.mask) {   // [mask_b, mask_h, 1, Sk] dense
         p.mask = (const char *)a.mask;
