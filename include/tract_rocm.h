@@ -238,8 +238,11 @@ int trocm_sdpa_workspace_init(void *workspace, size_t bytes, void *stream);
  *            kv_strides[3] for batch, head, token (head_dim contiguous); q_heads must
  *            be a multiple of kv_heads, kv head = q head / group (sdpa.rs:156-164)
  *   mask   : optional additive [mask_batch, mask_heads, q_len, kv_len] dense, of `dtype`,
- *            mask_batch in {1, batch}, mask_heads in {1, q_heads}; must be NULL when causal
- *            (sdpa.rs:297-299)
+ *            mask_batch in {1, batch}, mask_heads in {1, q_heads} (the broadcast the CUDA
+ *            dispatch expresses with zero strides, cuda/src/kernels/flash_attn.rs:138-143);
+ *            must be NULL when causal (sdpa.rs:297-299).  Values may be finite minima
+ *            (sdpa.rs:550-553) or -inf; a row masked entirely with -inf yields NaN, as on the
+ *            CPU.  The split-K decode and MFMA prefill kernels take the mask themselves.
  *   scale  : NaN selects the default 1/sqrt(head_dim) (sdpa.rs:177-181)
  *   causal : key j visible to query i iff j <= i + (kv_len - q_len) (flash_sdpa.rs:279-288) */
 int trocm_sdpa(const void *q, const void *k, const void *v, const void *mask, void *out, int dtype,
@@ -265,7 +268,9 @@ int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_n
 
 /* WindowKvSdpaState::eval (transformers/src/ops/window_kv_cache.rs:216-239): append K_new and
  * V_new to the two sliding-window caches, then attend Q to every valid slot without a causal
- * mask (the ring buffer is the window).  Arguments as trocm_inplace_kv_sdpa_eval. */
+ * mask (the ring buffer is the window).  Arguments as trocm_inplace_kv_sdpa_eval.  A
+ * single-token step on F32/F16 rings is one launch: the attention kernel stores the token at
+ * the cursor. */
 int trocm_window_kv_sdpa_eval(const void *q, const void *k_new, const void *v_new, int dtype, int64_t q_heads,
                               int64_t n_new, const int64_t *kv_new_strides, trocm_kv_cache *k_cache,
                               trocm_kv_cache *v_cache, void *out, float scale, void *workspace,
