@@ -385,6 +385,25 @@ def run_ops(ta, args):
     res["prefill_512x4096_causal_as_mask_input"] = {"us": round(us, 2), "tflops": round(fl / us / 1e6, 1)}
     us = time_calls(ta, lambda: sc.eval(qp, kp, vp, out=op), 50)
     res["prefill_512x4096_is_causal"] = {"us": round(us, 2), "tflops": round(fl / us / 1e6, 1)}
+    del kvs, kp, vp
+    # Q4_0 weights x one activation row (the decode-time projections of an 8B-class decoder), f16; each
+    # shape rotates over 8 weight matrices so that launches read HBM
+    gemm = ta.GgmlGemm()
+    for n_, k_ in ((14336, 4096), (4096, 14336), (4096, 4096)):
+        blob = rng.integers(0, 256, (n_, k_ // 32 * 18), dtype=np.uint8)
+        blob[:, 1::18] = (blob[:, 1::18] & 0x03) | 0x28      # scales: small finite f16 values
+        ws = [ta.Q40Weights(blob, 1, n_, k_) for _ in range(8)]
+        xa = ta.DeviceTensor.from_numpy(rng.standard_normal((1, 1, k_)).astype(np.float16))
+        oa = ta.DeviceTensor((1, 1, n_), np.float16)
+
+        def one_mv():
+            gemm.eval(xa, ws[turn[0] % 8], out=oa)
+            turn[0] += 1
+
+        us = time_calls(ta, one_mv, 200)
+        by = n_ * (k_ // 32) * 18 + 2 * k_ + 2 * n_
+        res[f"q4_0_matvec_f16_n{n_}_k{k_}"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": by}
+        del ws
     # the oracle on the host for the same ops, on a bounded sample
     xh = rng.standard_normal((1, 4, S, D)).astype(np.float16)
     t0 = time.perf_counter()

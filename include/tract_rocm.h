@@ -196,6 +196,30 @@ int trocm_block_quant(int format, const void *src, int src_dtype, size_t n_elems
 int trocm_block_dequant(int format, const void *src_blocks, size_t n_elems, void *dst, int dst_dtype,
                         void *stream);
 
+/* ---- Q4_0 weights x a few activation rows: the decode-time projections ------------------------
+ *
+ * The matrix-vector arm of GgmlGemm (cuda/src/kernels/matmul/mod.rs:575-627; taken for m <= 8,
+ * :605-606; `dispatch_ggml_matvec_q40` :481-529): weights [batch, n, k] in Q4_0 blocks along k
+ * (BlockQuantStorage rows, linalg/src/frame/block_quant/storage.rs:14-59), activations
+ * [act_batch, m, k], output [act_batch, m, n] in the activations' type; act_batch must be a
+ * multiple of the weights' batch (:488).  Result: the product with the dequantised weights, the
+ * definition the reference's own test holds its kernel to (mod.rs:864-890). */
+typedef struct trocm_q4_weights trocm_q4_weights;
+
+/* Device copy of `batch * n` rows of k/32 canonical 18-byte blocks (device pointer, row-major, no
+ * padding; the reference pads rows to 512 elements for its kernel, cuda/src/utils.rs:252-280, which
+ * this layout does not need).  k must be a multiple of 32 (utils.rs:253). */
+int trocm_q4_0_weights_create(trocm_q4_weights **out, const void *blocks_device, int64_t batch, int64_t n,
+                              int64_t k, void *stream);
+int trocm_q4_0_weights_destroy(trocm_q4_weights *weights);
+int trocm_q4_0_weights_shape(const trocm_q4_weights *weights, int64_t *batch, int64_t *n, int64_t *k);
+/* The canonical blocks back (byte-identical to what was loaded). */
+int trocm_q4_0_weights_export(const trocm_q4_weights *weights, void *dst_blocks_device, void *stream);
+/* out[b, i, j] = sum_k act[b, i, k] * w[b / (act_batch / batch), j, k]; act and out dense, F32 or F16,
+ * act 16-byte aligned, m <= 8. */
+int trocm_q4_0_matvec(const trocm_q4_weights *weights, const void *act, int act_dtype, int64_t act_batch,
+                      int64_t m, void *out, void *stream);
+
 /* ---- element-wise neighbours of the cache ------------------------------------------------- */
 
 /* Cast between F32 and F16 (core `Cast` as the GPU backends run it,

@@ -357,4 +357,46 @@ struct Cast {
     }
 };
 
+// Q4_0 weights [batch, n, k] on the device and their product with a few activation rows: the
+// matrix-vector arm of GgmlGemm (cuda/src/kernels/matmul/mod.rs:575-627, m <= 8).
+class Q40Weights {
+   public:
+    // `blocks`: batch * n rows of k/32 canonical 18-byte blocks in host memory
+    Q40Weights(const void *blocks, int64_t batch, int64_t n, int64_t k) : batch_(batch), n_(n), k_(k) {
+        if (k % 32) throw Error("k is not a whole number of 32-element blocks");
+        const size_t bytes = (size_t)batch * n * (k / 32) * 18;
+        void *dev = nullptr;
+        check(trocm_malloc(&dev, bytes));
+        int rc = trocm_h2d(dev, blocks, bytes, nullptr);
+        if (rc == 0) rc = trocm_q4_0_weights_create(&w_, dev, batch, n, k, nullptr);
+        if (rc == 0) rc = trocm_stream_sync(nullptr);
+        trocm_free(dev);
+        check(rc);
+    }
+    Q40Weights(const Q40Weights &) = delete;
+    Q40Weights &operator=(const Q40Weights &) = delete;
+    ~Q40Weights() {
+        if (w_) trocm_q4_0_weights_destroy(w_);
+    }
+    int64_t batch() const { return batch_; }
+    int64_t n() const { return n_; }
+    int64_t k() const { return k_; }
+    trocm_q4_weights *handle() const { return w_; }
+
+   private:
+    trocm_q4_weights *w_ = nullptr;
+    int64_t batch_, n_, k_;
+};
+
+struct GgmlGemm {
+    // activations [b, m, k] (f32 or f16) x weights [b_w, n, k] -> [b, m, n]
+    DeviceTensor eval(const DeviceTensor &act, const Q40Weights &w) const {
+        const auto &as = act.shape();
+        if (as.size() != 3 || as[2] != w.k()) throw Error("activations must be [batch, m, k]");
+        DeviceTensor out({as[0], as[1], w.n()}, act.datum_type());
+        check(trocm_q4_0_matvec(w.handle(), act.ptr(), (int)act.datum_type(), as[0], as[1], out.ptr(), nullptr));
+        return out;
+    }
+};
+
 }  // namespace trocm

@@ -57,6 +57,7 @@ def lib() -> C.CDLL:
         L.orc_block_bytes.argtypes = [i]
         L.orc_quant.argtypes = [i, i, vp, sz, vp]
         L.orc_dequant.argtypes = [i, i, vp, sz, vp]
+        L.orc_q4_0_matvec.argtypes = [vp, sz, sz, sz, vp, i, sz, sz, vp]
         L.orc_kv_new.restype = vp
         L.orc_kv_new.argtypes = [sz, sz]
         L.orc_kv_free.argtypes = [vp]
@@ -121,6 +122,20 @@ def dequant(fmt: int, q: np.ndarray, dtype=np.float32) -> np.ndarray:
     d = q.shape[-1] // bb * 32
     out = np.empty(q.shape[:-1] + (d,), dtype=dtype)
     rc = lib().orc_dequant(fmt, int(dtype == np.float16), _p(q), out.size, _p(out))
+    assert rc == 0
+    return out
+
+
+def q4_0_matvec(blocks: np.ndarray, act: np.ndarray) -> np.ndarray:
+    """GgmlGemm's Q4_0 matrix-vector arm as its test defines it (cuda/src/kernels/matmul/mod.rs:864-890):
+    blocks uint8 [w_batch, n, k/32*18], act [act_batch, m, k] f32 or f16 -> [act_batch, m, n]."""
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    act = np.ascontiguousarray(act)
+    wb, n, rb = blocks.shape
+    ab, m, k = act.shape
+    assert rb == k // 32 * 18 and act.dtype in (np.float32, np.float16)
+    out = np.empty((ab, m, n), dtype=act.dtype)
+    rc = lib().orc_q4_0_matvec(_p(blocks), wb, n, k, _p(act), int(act.dtype == np.float16), ab, m, _p(out))
     assert rc == 0
     return out
 

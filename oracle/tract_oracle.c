@@ -34,6 +34,10 @@
  *                          concatenate form, the rotation closed forms (norm of each
  *                          pair kept, angles add); f16 arithmetic is the `half` crate's
  *                          (operate in f32, round to f16 after every operation)
+ *   Q4_0 matrix-vector      pinned (tolerance): == numpy's product with the (pinned) dequantised
+ *                          weights in f64, a hand-built block whose dot product is known in
+ *                          closed form, linearity in the activations; exact f32 bits unpinned
+ *                          (summation order of the CPU matrix product)
  *
  * Build: gcc -O2 -fno-fast-math -ffp-contract=off (Rust never contracts a*b+c).
  */
@@ -318,6 +322,51 @@ ORC_API int orc_dequant(int fmt, int dst_f16, const uint8_t *src, size_t n_elems
             if (fmt == 3) orc_q4_0_dequant_block_f32(q, o);
             else if (fmt == 2) orc_q8_0_dequant_block_f32(q, o);
             else orc_q8_1_dequant_block_f32(q, o);
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Q4_0 weights x activations: out[b, i, j] = sum_k act[b, i, k] * w[b / ratio, j, k], the product the */
+/* reference holds its GPU kernel to (cuda/src/kernels/matmul/mod.rs:864-890): the weights pass         */
+/* through Q4_0.simulate_precision_loss (quantise + dequantise in the activations' type,               */
+/* block_quant/mod.rs:110-155) and then a plain matrix product in that type.  Here the blocks are       */
+/* given; each is dequantised in the activations' type (f16: rounded to f16, q4_0.rs:82-95) and the     */
+/* dot product accumulates in f32 in k order (the exact f32 bits of the CPU product depend on the      */
+/* matrix-multiply kernel's summation order and are not pinned; callers compare within a tolerance).   */
+/* ------------------------------------------------------------------------- */
+ORC_API int orc_q4_0_matvec(const uint8_t *blocks, size_t w_batch, size_t n, size_t k, const void *act, int f16,
+                            size_t act_batch, size_t m, void *out) {
+    if (k % QK || w_batch == 0 || act_batch % w_batch) return 1;
+    const size_t ratio = act_batch / w_batch, nb = k / QK, rb = nb * 18;
+    long long total = (long long)act_batch * (long long)n;
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static)
+#endif
+    for (long long bj = 0; bj < total; bj++) {
+        const size_t b = (size_t)bj / n, j = (size_t)bj % n;
+        const uint8_t *row = blocks + ((b / ratio) * n + j) * rb;
+        for (size_t i = 0; i < m; i++) {
+            float acc = 0.0f;
+            for (size_t blk = 0; blk < nb; blk++) {
+                float w[QK];
+                if (f16) {
+                    uint16_t h[QK];
+                    orc_q4_0_dequant_block_f16(row + blk * 18, h);
+                    for (int e = 0; e < QK; e++) w[e] = orc_f16_to_f32(h[e]);
+                } else {
+                    orc_q4_0_dequant_block_f32(row + blk * 18, w);
+                }
+                for (int e = 0; e < QK; e++) {
+                    const size_t kk = blk * QK + e;
+                    const float x = f16 ? orc_f16_to_f32(((const uint16_t *)act)[(b * m + i) * k + kk])
+                                        : ((const float *)act)[(b * m + i) * k + kk];
+                    acc += w[e] * x;
+                }
+            }
+            if (f16) ((uint16_t *)out)[(b * m + i) * n + j] = orc_f32_to_f16(acc);
+            else ((float *)out)[(b * m + i) * n + j] = acc;
         }
     }
     return 0;

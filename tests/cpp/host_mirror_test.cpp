@@ -254,6 +254,30 @@ int main() {
             f.to_host(rt2.data());
             for (size_t i = 0; i < x.size(); i++) EXPECT(rt2[i] == x[i]);   // integers up to 2048 are exact in f16
         }
+        // Q4_0 weights x activations: every block holds the nibbles i % 16 (the table of q4_0.rs:722-739),
+        // so sums over whole blocks and single elements are known in closed form
+        {
+            const int N = 4, K = 96;
+            const float scales[N] = {0.5f, 0.25f, 1.0f, 2.0f};
+            const uint16_t scale_bits[N] = {0x3800, 0x3400, 0x3C00, 0x4000};
+            std::vector<uint8_t> blocks((size_t)N * (K / 32) * 18);
+            for (int j = 0; j < N; j++)
+                for (int b = 0; b < K / 32; b++) {
+                    uint8_t *blk = &blocks[((size_t)j * (K / 32) + b) * 18];
+                    blk[0] = (uint8_t)(scale_bits[j] & 0xff), blk[1] = (uint8_t)(scale_bits[j] >> 8);
+                    for (int i = 0; i < 16; i++) blk[2 + i] = (uint8_t)((i % 16) | (((16 + i) % 16) << 4));
+                }
+            Q40Weights w(blocks.data(), 1, N, K);
+            std::vector<float> ones(K, 1.0f), e(K, 0.0f), got(N);
+            GgmlGemm{}.eval(DeviceTensor::from_host(ones.data(), {1, 1, K}, DatumType::F32), w).to_host(got.data());
+            for (int j = 0; j < N; j++) EXPECT(got[j] == scales[j] * -48.0f);   // 3 blocks x sum(i % 16 - 8) = 3 x -16
+            e[37] = 1.0f;   // block 1, element 5: (5 - 8) * d
+            GgmlGemm{}.eval(DeviceTensor::from_host(e.data(), {1, 1, K}, DatumType::F32), w).to_host(got.data());
+            for (int j = 0; j < N; j++) EXPECT(got[j] == scales[j] * -3.0f);
+            e[37] = 0.0f, e[16] = 1.0f;   // a high nibble: element 16 has code 0
+            GgmlGemm{}.eval(DeviceTensor::from_host(e.data(), {1, 1, K}, DatumType::F32), w).to_host(got.data());
+            for (int j = 0; j < N; j++) EXPECT(got[j] == scales[j] * -8.0f);
+        }
         std::printf("host_mirror_test: all checks passed\n");
         return 0;
     } catch (const std::exception &e) {

@@ -1,0 +1,95 @@
+"""Q4_0 weights x a few activation rows on the GPU (the matrix-vector arm of GgmlGemm,
+cuda/src/kernels/matmul/mod.rs:575-627) vs the oracle and the f64 product with the dequantised
+weights.  Tolerance: relative to 1 + |reference|, 1e-4 for f32 and 4e-3 for f16 activations (the
+reference's own test allows Approximation::VeryApproximate, mod.rs:776-786)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import tract_amd
+from oracle import oracle as orc
+from tests.gpu_util import rt  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+Q4 = 3
+
+
+def rel_err(got, want):
+    return float(np.max(np.abs(got.astype(np.float64) - want) / (1 + np.abs(want))))
+
+
+def f64_product(blocks, act, dt):
+    wd = orc.dequant(Q4, blocks, dt).astype(np.float64)
+    return np.einsum("bmk,bnk->bmn", act.astype(np.float64), np.repeat(wd, act.shape[0] // wd.shape[0], axis=0))
+
+
+# (b, m, k, n) of the reference's matrix-vector cases (mod.rs:709-724, with k rounded up to whole
+# blocks) plus decoder shapes: ragged n, k that is not a multiple of 64 blocks, k beyond one LDS chunk
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+@pytest.mark.parametrize("wb,ab,m,n,k", [
+    (1, 1, 1, 1, 32), (2, 2, 1, 2, 64), (2, 2, 2, 7, 128), (1, 4, 1, 1, 64), (1, 1, 5, 1, 32), (1, 2, 8, 2, 64),
+    (1, 1, 1, 4096, 4096), (1, 1, 1, 1000, 2080), (1, 1, 3, 515, 4096), (1, 2, 4, 130, 1024), (1, 1, 6, 77, 2048),
+    (1, 1, 7, 33, 992), (1, 1, 8, 200, 8192), (1, 1, 1, 64, 20480), (2, 4, 2, 50, 14336),
+])
+def test_matvec_matches_the_oracle(rt, dt, wb, ab, m, n, k):
+    rng = np.random.default_rng(n + k + m)
+    w = (rng.standard_normal((wb, n, k)) * 0.05).astype(np.float32)
+    w[:, :, ::97] *= 8.0    # outliers: blocks with very different scales
+    act = rng.standard_normal((ab, m, k)).astype(dt)
+    blocks = orc.quant(Q4, w)
+    wq = tract_amd.Q40Weights(blocks, wb, n, k)
+    got = tract_amd.GgmlGemm().eval(act, wq).to_numpy()
+    assert got.dtype == dt and got.shape == (ab, m, n)
+    tol = 1e-4 if dt == np.float32 else 4e-3
+    assert rel_err(got, f64_product(blocks, act, dt)) <= tol
+    if n * k * ab * m <= 1 << 24:
+        assert rel_err(got, orc.q4_0_matvec(blocks, act).astype(np.float64)) <= tol
+
+
+def test_closed_form_blocks(rt):
+    """Nibbles i % 16 in every block (the table of q4_0.rs:722-739): sums of whole blocks and single
+    elements are known exactly, low and high nibbles alike."""
+    n, k = 4, 96
+    scales = np.array([0.5, 0.25, 1.0, 2.0], np.float32)
+    codes = np.arange(32) % 16
+    packed = (codes[:16] | (codes[16:] << 4)).astype(np.uint8)
+    blocks = np.zeros((1, n, 3 * 18), np.uint8)
+    for j in range(n):
+        for b in range(3):
+            blocks[0, j, b * 18:b * 18 + 2] = np.array([scales[j]], np.float16).view(np.uint8)
+            blocks[0, j, b * 18 + 2:b * 18 + 18] = packed
+    wq = tract_amd.Q40Weights(blocks, 1, n, k)
+    gemm = tract_amd.GgmlGemm()
+    for dt in (np.float32, np.float16):
+        assert np.array_equal(gemm.eval(np.ones((1, 1, k), dt), wq).to_numpy()[0, 0], (scales * -48.0).astype(dt))
+        for pos, code in ((37, 5), (16, 0), (95, 15), (0, 0)):
+            e = np.zeros((1, 1, k), dt)
+            e[0, 0, pos] = 1
+            assert np.array_equal(gemm.eval(e, wq).to_numpy()[0, 0], (scales * (code - 8)).astype(dt))
+
+
+def test_weights_round_trip_and_quantize(rt):
+    rng = np.random.default_rng(9)
+    w = rng.standard_normal((2, 37, 160)).astype(np.float32)
+    blocks = orc.quant(Q4, w)
+    wq = tract_amd.Q40Weights(blocks, 2, 37, 160)
+    assert np.array_equal(wq.blocks(), blocks)              # the canonical bytes come back unchanged
+    wq2 = tract_amd.Q40Weights.quantize(w)                  # quantised on the device: same bytes as the oracle
+    assert np.array_equal(wq2.blocks(), blocks)
+
+
+def test_error_paths(rt):
+    blocks = np.zeros((1, 4, 2 * 18), np.uint8)
+    wq = tract_amd.Q40Weights(blocks, 1, 4, 64)
+    with pytest.raises(tract_amd.TractRocmError, match="whole number of 32-element blocks"):
+        tract_amd.Q40Weights(np.zeros(18, np.uint8), 1, 1, 40)
+    with pytest.raises(tract_amd.TractRocmError, match="at most 8"):
+        tract_amd.GgmlGemm().eval(np.zeros((1, 9, 64), np.float32), wq)
+    with pytest.raises(tract_amd.TractRocmError, match="do not match"):
+        tract_amd.GgmlGemm().eval(np.zeros((1, 1, 32), np.float32), wq)
+    w2 = tract_amd.Q40Weights(np.zeros((2, 4, 2 * 18), np.uint8), 2, 4, 64)
+    with pytest.raises(tract_amd.TractRocmError, match="not a multiple of the weights' batch"):
+        tract_amd.GgmlGemm().eval(np.zeros((3, 1, 64), np.float32), w2)
+    out = tract_amd.GgmlGemm().eval(np.zeros((0, 1, 64), np.float32).reshape(0, 1, 64), wq)
+    assert out.shape == (0, 1, 4)

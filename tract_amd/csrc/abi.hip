@@ -750,6 +750,93 @@ int trocm_kv_cache_raw(const trocm_kv_cache *c, void **data, void **scales, int6
     return 0;
 }
 
+// ---- Q4_0 weights and the decode-time projection --------------------------------------------------
+}  // extern "C" (the struct below is opaque to C callers)
+
+struct trocm_q4_weights {
+    int64_t batch, n, k;
+    void *codes, *scales;   // [batch * n, k/2] bytes and [batch * n, k/32] f16
+};
+
+extern "C" {
+
+int trocm_q4_0_weights_create(trocm_q4_weights **out, const void *blocks, int64_t batch, int64_t n, int64_t k,
+                              void *stream) {
+    TROCM_NOT_NULL(out);
+    *out = nullptr;
+    TROCM_REQUIRE(batch >= 1 && n >= 1 && k >= 32, "q4_0 weights: empty shape [%lld, %lld, %lld]", (long long)batch,
+                  (long long)n, (long long)k);
+    TROCM_REQUIRE(k % 32 == 0, "q4_0 weights: k = %lld is not a whole number of 32-element blocks", (long long)k);  // utils.rs:253
+    TROCM_REQUIRE(batch * n < (1ll << 31) && k < (1ll << 31), "q4_0 weights: shape too large");
+    TROCM_NOT_NULL(blocks);
+    if (ensure_init()) return 1;
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    trocm_q4_weights *w = new (std::nothrow) trocm_q4_weights();
+    TROCM_REQUIRE(w != nullptr, "out of host memory");
+    w->batch = batch, w->n = n, w->k = k;
+    const int64_t rows = batch * n;
+    hipError_t e = hipMalloc(&w->codes, (size_t)rows * (size_t)(k / 2));
+    if (e == hipSuccess) e = hipMalloc(&w->scales, (size_t)rows * (size_t)(k / 32) * 2);
+    if (e != hipSuccess) {
+        if (w->codes) (void)hipFree(w->codes);
+        delete w;
+        return fail("q4_0 weights: hipMalloc failed: %s", hipGetErrorString(e));
+    }
+    if (launch_quant_import(TROCM_Q4_0, 1, 1, rows, rows, 0, k, blocks, w->codes, w->scales, s)) {
+        (void)hipFree(w->codes);
+        (void)hipFree(w->scales);
+        delete w;
+        return 1;
+    }
+    *out = w;
+    return 0;
+}
+
+int trocm_q4_0_weights_destroy(trocm_q4_weights *w) {
+    if (!w) return 0;
+    TROCM_HIP(hipDeviceSynchronize());
+    TROCM_HIP(hipFree(w->codes));
+    TROCM_HIP(hipFree(w->scales));
+    delete w;
+    return 0;
+}
+
+int trocm_q4_0_weights_shape(const trocm_q4_weights *w, int64_t *batch, int64_t *n, int64_t *k) {
+    TROCM_NOT_NULL(w);
+    if (batch) *batch = w->batch;
+    if (n) *n = w->n;
+    if (k) *k = w->k;
+    return 0;
+}
+
+int trocm_q4_0_weights_export(const trocm_q4_weights *w, void *dst_blocks, void *stream) {
+    TROCM_NOT_NULL(w);
+    TROCM_NOT_NULL(dst_blocks);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    const int64_t rows = w->batch * w->n;
+    return launch_quant_export(TROCM_Q4_0, 1, 1, rows, rows, w->k, w->codes, w->scales, dst_blocks, s);
+}
+
+int trocm_q4_0_matvec(const trocm_q4_weights *w, const void *act, int act_dtype, int64_t act_batch, int64_t m, void *out,
+                      void *stream) {
+    TROCM_NOT_NULL(w);
+    TROCM_REQUIRE(act_dtype == TROCM_F32 || act_dtype == TROCM_F16, "q4_0_matvec: activations must be F32 or F16");
+    TROCM_REQUIRE(act_batch >= 0 && m >= 0, "q4_0_matvec: negative dimension");
+    TROCM_REQUIRE(m <= 8, "q4_0_matvec: m = %lld activation rows; the matrix-vector kernel takes at most 8", (long long)m);  // mod.rs:605
+    if (act_batch == 0 || m == 0) return 0;                                      // mod.rs:586-588
+    TROCM_REQUIRE(act_batch % w->batch == 0, "q4_0_matvec: activation batch %lld is not a multiple of the weights' batch %lld",
+                  (long long)act_batch, (long long)w->batch);                     // mod.rs:488
+    TROCM_REQUIRE(act_batch <= 65535, "q4_0_matvec: batch too large");
+    TROCM_NOT_NULL(act);
+    TROCM_NOT_NULL(out);
+    TROCM_REQUIRE((uintptr_t)act % 16 == 0, "q4_0_matvec: activations must be 16-byte aligned");
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    return launch_q4_0_matvec(w->codes, w->scales, w->batch, w->n, w->k, act, act_dtype, act_batch, m, out, s);
+}
+
 // ---- block quantisation as a tensor op ---------------------------------------------------------
 int trocm_block_quant(int format, const void *src, int src_dtype, size_t n_elems, void *dst_blocks, void *stream) {
     TROCM_REQUIRE(format == TROCM_Q8_0 || format == TROCM_Q4_0, "block_quant: format must be Q8_0 or Q4_0");

@@ -103,6 +103,11 @@ int launch_apply_rope(const void *x, const void *cos, const void *sin, void *y, 
                       const int64_t *shape, const int64_t *in_strides, const int64_t *cs_strides,
                       const int64_t *out_strides, int rotate_only, hipStream_t s);
 
+// Q4_0 weights (code plane [w_batch, n, k/2], scale plane [w_batch, n, k/32]) times m <= 8 activation
+// rows: out[b, i, j] = sum_k act[b, i, k] * w[b * w_batch / act_batch, j, k]; act and out of act_dtype.
+int launch_q4_0_matvec(const void *codes, const void *scales, int64_t w_batch, int64_t n, int64_t k, const void *act,
+                       int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s);
+
 // Attention.  One description for every kernel.
 struct SdpaArgs {
     const void *q;

@@ -23,7 +23,7 @@ import numpy as np
 
 from . import _lib
 from ._lib import F16, F32, Q4_0, Q8_0, TractRocmError, call
-from .runtime import DeviceTensor, Workspace, _sh, dtype_code
+from .runtime import DeviceTensor, Workspace, _sh, dtype_code, synchronize
 
 _I64x4 = C.c_int64 * 4
 _I64x3 = C.c_int64 * 3
@@ -572,6 +572,78 @@ class BlockQuant:
 
 Q4_0_FORMAT = BlockQuant(Q4_0, "Q4_0", 18)
 Q8_0_FORMAT = BlockQuant(Q8_0, "Q8_0", 34)
+
+
+class Q40Weights:
+    """Q4_0 weights [batch, n, k] resident on the device (BlockQuantStorage rows of k/32 blocks,
+    block_quant/storage.rs:14-59), as the matrix-vector arm of GgmlGemm takes them."""
+
+    def __init__(self, blocks, batch: int, n: int, k: int, stream=None):
+        if k % 32:
+            raise TractRocmError(f"k = {k} is not a whole number of 32-element blocks")
+        if isinstance(blocks, DeviceTensor):
+            src = blocks
+        else:
+            src = DeviceTensor.from_numpy(np.ascontiguousarray(blocks, dtype=np.uint8).reshape(-1), stream)
+        if src.nbytes != batch * n * (k // 32) * 18:
+            raise TractRocmError(f"{src.nbytes} bytes of blocks do not make a [{batch}, {n}, {k}] Q4_0 tensor")
+        h = C.c_void_p()
+        call("trocm_q4_0_weights_create", C.byref(h), src.ptr, batch, n, k, _sh(stream))
+        self.handle, self.batch, self.n, self.k = h, batch, n, k
+        synchronize() if stream is None else stream.synchronize()   # `src` may be released now
+
+    @classmethod
+    def quantize(cls, w: np.ndarray, stream=None) -> "Q40Weights":
+        """Quantise a dense [batch, n, k] (or [n, k]) tensor with Q4_0 along k (BlockQuant::quant_f32)."""
+        w = np.asarray(w)
+        if w.ndim == 2:
+            w = w[None]
+        b, n, k = w.shape
+        blob = Q4_0_FORMAT.quant_f16(w, stream) if w.dtype == np.float16 else Q4_0_FORMAT.quant_f32(w, stream)
+        return cls(blob, b, n, k, stream)
+
+    def blocks(self, stream=None) -> np.ndarray:
+        """The canonical blocks, uint8 [batch, n, k/32 * 18]."""
+        dst = DeviceTensor((self.batch, self.n, self.k // 32 * 18), np.uint8)
+        call("trocm_q4_0_weights_export", self.handle, dst.ptr, _sh(stream))
+        return dst.to_numpy(stream)
+
+    def close(self):
+        if getattr(self, "handle", None):
+            call("trocm_q4_0_weights_destroy", self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class GgmlGemm:
+    """Activations [b, m, k] x Q4_0 weights [b_w, n, k] -> [b, m, n] for m <= 8 (GgmlGemm::dispatch_eval,
+    cuda/src/kernels/matmul/mod.rs:575-627; output_shape :536-545)."""
+
+    def output_shape(self, act_shape, w_shape):
+        return tuple(act_shape[:-2]) + (act_shape[-2], w_shape[-2])
+
+    def eval(self, activs, weights: Q40Weights, stream=None, out=None) -> DeviceTensor:
+        a = _as_device(activs, stream)
+        if a.dtype not in (np.float32, np.float16):
+            raise TractRocmError("activations must be f32 or f16")
+        shape = tuple(a.shape)
+        if len(shape) == 2:
+            shape = (1,) + shape
+        if len(shape) != 3 or shape[2] != weights.k:
+            raise TractRocmError(f"activations {tuple(a.shape)} do not match weights [.., {weights.n}, {weights.k}]")
+        b, m, _ = shape
+        oshape = tuple(a.shape[:-1]) + (weights.n,)
+        if out is None:
+            out = DeviceTensor(oshape, a.dtype)
+        elif tuple(out.shape) != oshape or out.dtype != a.dtype:
+            raise TractRocmError("out must have shape [.., m, n] and the activations' datum type")
+        call("trocm_q4_0_matvec", weights.handle, a.ptr, dtype_code(a.dtype), b, m, out.ptr, _sh(stream))
+        return out
 
 
 def sdpa_decode_ragged(q: DeviceTensor, k_caches, v_caches, scale=None, workspace: Workspace | None = None,
