@@ -174,6 +174,60 @@ __device__ __forceinline__ void merge_head(const DecodeDev &p, int64_t first, in
     out_row[tid] = from_f32<T>(acc / ll);
 }
 
+// In-kernel merge by the last workgroup of a (sequence, kv head) to arrive.  Every workgroup calls this
+// after storing its partial record with agent-scope (write-through) stores: it waits for its stores,
+// signals its arrival on `counter`, and the workgroup that arrives last reads all `nsplit` records
+// (first, first + stride, ...; at most kTailMergeMax) with agent-scope loads and writes the G output
+// rows at `out`.  All loads of all splits are issued before the first use: one memory latency, not
+// one per split.  The counter is left at zero for the next launch.
+template <typename T, int D, int G>
+__device__ __forceinline__ void tail_merge(const DecodeDev &p, int *counter, int nsplit, int64_t first, int64_t stride,
+                                           T *out, int tid) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's partial stores have completed
+    __syncthreads();                                     // ... and so have the whole workgroup's
+    __shared__ int s_last;
+    if (tid == 0) {
+        const int arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = arrived == nsplit - 1;
+        if (s_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    auto aload = [](const float *a) { return __hip_atomic_load(a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    constexpr int NE = (G * D + kThreads - 1) / kThreads;
+    float mv[NE][kTailMergeMax], lv[NE][kTailMergeMax], ov[NE][kTailMergeMax];
+    const int64_t ml_step = stride * (2 * G), po_step = stride * (G * D);
+#pragma unroll
+    for (int e = 0; e < NE; e++) {
+        const int idx = min(tid + e * kThreads, G * D - 1);
+        const int h = idx / D;
+        const float *ml = p.part_ml + first * (2 * G) + h;
+        const float *po = p.part_o + first * (G * D) + idx;
+#pragma unroll
+        for (int sp = 0; sp < kTailMergeMax; sp++) {
+            const int spc = min(sp, nsplit - 1);   // splits past the last repeat it and get weight 0 below
+            mv[e][sp] = aload(ml + spc * ml_step);
+            lv[e][sp] = aload(ml + spc * ml_step + G);
+            ov[e][sp] = aload(po + spc * po_step);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < NE; e++) {
+        const int idx = tid + e * kThreads;
+        float mm = -INFINITY;
+#pragma unroll
+        for (int sp = 0; sp < kTailMergeMax; sp++) mm = fmaxf(mm, mv[e][sp]);
+        float acc = 0.0f, ll = 0.0f;
+#pragma unroll
+        for (int sp = 0; sp < kTailMergeMax; sp++) {
+            const float f = sp < nsplit ? fast_exp2(mv[e][sp] - mm) : 0.0f;
+            acc += ov[e][sp] * f;
+            ll += lv[e][sp] * f;
+        }
+        if (idx < G * D) out[idx] = from_f32<T>(acc / ll);
+    }
+}
+
 // Merge launch: grid (kv_heads, batch, G), D threads; runs after the split kernel on the same stream.
 template <typename T, int D, int G>
 __global__ __launch_bounds__(D) void sdpa_decode_merge_kernel(DecodeDev p) {

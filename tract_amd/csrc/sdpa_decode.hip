@@ -81,13 +81,6 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
     const int lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, and the compiler is told so: tile bases stay in scalar registers
 
-    // ---- stage the G query vectors of this KV head ------------------------------------
-    {
-        const u32x4 *qg = reinterpret_cast<const u32x4 *>(wk.q);
-        for (int i = tid; i < G * CPR; i += kThreads) lds_q[i] = qg[i];
-    }
-    __syncthreads();
-
     const char *kbase = wk.kbase, *vbase = wk.vbase;
     const int seq_T = wk.T;
     const int new_pos = wk.k_new ? wk.new_pos : -1;   // the token that comes from the step's input, if any
@@ -188,6 +181,12 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
         issue_k(tile);
         issue_v(tile);
     }
+    // ---- stage the G query vectors of this KV head (the first tile's K and V are already in flight) ----
+    {
+        const u32x4 *qg = reinterpret_cast<const u32x4 *>(wk.q);
+        for (int i = tid; i < G * CPR; i += kThreads) lds_q[i] = qg[i];
+    }
+    __syncthreads();
     const u32x4 *lds_krow = &lds_k[w][qk_row * CPR];
     const int qk_rot = rot<CPR>(qk_row) + qk_half * HC;
 
@@ -331,50 +330,7 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
     if (wk.direct || wk.counter == nullptr) return;
 
     // ---- the last workgroup of this sequence-head to arrive merges the splits -------------------
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's partial stores have completed
-    __syncthreads();                                     // ... and so have the whole workgroup's
-    __shared__ int s_last;
-    if (tid == 0) {
-        const int arrived = __hip_atomic_fetch_add(wk.counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = arrived == wk.nsplit - 1;
-        if (s_last) __hip_atomic_store(wk.counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
-    }
-    __syncthreads();
-    if (!s_last) return;
-    // All loads of all splits are issued before the first use: one memory latency, not one per split.
-    auto aload = [](const float *a) { return __hip_atomic_load(a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
-    constexpr int NE = (G * D + kThreads - 1) / kThreads;
-    float mv[NE][kTailMergeMax], lv[NE][kTailMergeMax], ov[NE][kTailMergeMax];
-    const int64_t ml_step = wk.part_stride * (2 * G), po_step = wk.part_stride * (G * D);
-#pragma unroll
-    for (int e = 0; e < NE; e++) {
-        const int idx = min(tid + e * kThreads, G * D - 1);
-        const int h = idx / D;
-        const float *ml = p.part_ml + wk.part_first * (2 * G) + h;
-        const float *po = p.part_o + wk.part_first * (G * D) + idx;
-#pragma unroll
-        for (int sp = 0; sp < kTailMergeMax; sp++) {
-            const int spc = min(sp, wk.nsplit - 1);   // splits past the last repeat it and get weight 0 below
-            mv[e][sp] = aload(ml + spc * ml_step);
-            lv[e][sp] = aload(ml + spc * ml_step + G);
-            ov[e][sp] = aload(po + spc * po_step);
-        }
-    }
-#pragma unroll
-    for (int e = 0; e < NE; e++) {
-        const int idx = tid + e * kThreads;
-        float mm = -INFINITY;
-#pragma unroll
-        for (int sp = 0; sp < kTailMergeMax; sp++) mm = fmaxf(mm, mv[e][sp]);
-        float acc = 0.0f, ll = 0.0f;
-#pragma unroll
-        for (int sp = 0; sp < kTailMergeMax; sp++) {
-            const float f = sp < wk.nsplit ? fast_exp2(mv[e][sp] - mm) : 0.0f;
-            acc += ov[e][sp] * f;
-            ll += lv[e][sp] * f;
-        }
-        if (idx < G * D) out[idx] = from_f32<T>(acc / ll);
-    }
+    tail_merge<T, D, G>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
 }
 
 // Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.

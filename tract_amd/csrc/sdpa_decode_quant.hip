@@ -338,21 +338,30 @@ __global__ __launch_bounds__(kThreads, G <= 4 ? 2 : 1) void sdpa_decode_q_kernel
         }
         if (p.nsplit == 1) {
             out[idx] = __float2half_rn(acc / ll);
-        } else {
+        } else if (p.counters == nullptr) {
             int64_t slot = bh * p.nsplit + split;
             p.part_o[slot * (G * D) + idx] = acc;
             if ((idx % D) == 0) {
                 p.part_ml[slot * (2 * G) + h] = mm;
                 p.part_ml[slot * (2 * G) + G + h] = ll;
             }
+        } else {   // write-through stores: visible device-wide when they complete (see tail_merge)
+            int64_t slot = bh * p.nsplit + split;
+            __hip_atomic_store(&p.part_o[slot * (G * D) + idx], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((idx % D) == 0) {
+                __hip_atomic_store(&p.part_ml[slot * (2 * G) + h], mm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&p.part_ml[slot * (2 * G) + G + h], ll, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
     }
+    if (p.nsplit == 1 || p.counters == nullptr) return;
+    tail_merge<__half, D, G>(p, p.counters + bh, p.nsplit, bh * p.nsplit, 1, out, tid);
 }
 
 template <int FMT, int G>
 int launch_one(const DecodeDev &p, dim3 grid, hipStream_t s) {
     hipLaunchKernelGGL((sdpa_decode_q_kernel<FMT, G>), grid, dim3(kThreads), 0, s, p);
-    if (p.nsplit > 1)
+    if (p.nsplit > 1 && p.counters == nullptr)
         hipLaunchKernelGGL((sdpa_decode_merge_kernel<__half, kD, G>), dim3(grid.y, grid.z, G), dim3(kD), 0, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("sdpa_decode (quantised KV) launch failed: %s", hipGetErrorString(e));
@@ -421,6 +430,9 @@ int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s) {
     p.scale_log2 = a.scale * 1.4426950408889634f;
     p.part_ml = (float *)((char *)a.workspace + kWsCounterBytes);
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * G;
+    // few splits: the last workgroup of a (batch, kv head) to arrive merges them, no second launch
+    static const int tail = getenv("TROCM_DECODE_TAIL_MERGE") ? atoi(getenv("TROCM_DECODE_TAIL_MERGE")) : 1;
+    if (tail && nsplit > 1 && nsplit <= kTailMergeMax && BH <= (int64_t)(kWsCounterBytes / sizeof(int))) p.counters = (int *)a.workspace;
     dim3 grid(nsplit, (unsigned)a.Hkv, (unsigned)a.B);
     return a.kv_fmt == TROCM_Q8_0 ? launch_fmt<TROCM_Q8_0>(p, (int)G, grid, s) : launch_fmt<TROCM_Q4_0>(p, (int)G, grid, s);
 }
