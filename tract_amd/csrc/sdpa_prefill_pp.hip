@@ -1,5 +1,6 @@
 // MFMA prefill attention for gfx950, throughput version for q_len >= 32 (GQA heads share K/V tiles).
-// f16 in/out, f32 accumulate, causal (bottom-right aligned) or unmasked, GQA, K/V read in place.
+// f16 in/out, f32 accumulate, causal (bottom-right aligned), unmasked or with an additive mask input, GQA,
+// K/V read in place.
 //
 // Same transposed formulation as sdpa_prefill.hip (S^T = K.Q^T, O^T = V^T.P^T with 32x32x16 MFMAs,
 // every softmax scalar of a query in one lane).  What differs is how a compute unit is kept busy:
