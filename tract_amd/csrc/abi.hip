@@ -1,6 +1,7 @@
 // Host side of libtract_rocm.so: the C ABI declared in include/tract_rocm.h.
 // Runtime context, error convention, device memory, the in-place capacity-doubling KV
 // cache and the dispatch of attention calls to the kernels.
+#include <atomic>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -28,7 +29,7 @@ int fail(const char *fmt, ...) {
 
 // ---- context ---------------------------------------------------------------------------------
 static std::mutex g_init_mutex;
-static int g_device = -1;
+static std::atomic<int> g_device{-1};   // written once, under g_init_mutex; read by every call
 static int g_compute_units = 0;
 static size_t g_hbm_bytes = 0;
 static char g_name[256] = "";
@@ -165,11 +166,7 @@ static int plane_free(trocm_kv_cache *c, void *ptr) {
 // over densely packed rows (57.5 us against 53.5 us, batch 8, 8226 tokens in 16384-token rows).
 // 1/32 of padding per row removes the effect (52.9 us).  TROCM_KV_PITCH_PAD=<tokens> overrides.
 static int64_t pitch_for(int64_t cap) {
-    static int64_t forced = -2;
-    if (forced == -2) {
-        const char *e = getenv("TROCM_KV_PITCH_PAD");
-        forced = e ? atoll(e) : -1;
-    }
+    static const int64_t forced = getenv("TROCM_KV_PITCH_PAD") ? atoll(getenv("TROCM_KV_PITCH_PAD")) : -1;
     if (forced >= 0) return cap + forced;
     return cap >= 2048 ? cap + ((cap / 32 + 7) & ~(int64_t)7) : cap;
 }
@@ -224,7 +221,12 @@ static int regrow(trocm_kv_cache *c, int64_t new_cap, hipStream_t s) {
     }
     if (c->data) {
         // The old buffers may still be read by work queued on the stream.
-        TROCM_HIP(hipStreamSynchronize(s));
+        hipError_t e = hipStreamSynchronize(s);
+        if (e != hipSuccess) {
+            (void)plane_free(c, nd);
+            (void)plane_free(c, ns);
+            return fail("hipStreamSynchronize failed while growing a KV cache: %s", hipGetErrorString(e));
+        }
         if (plane_free(c, c->data)) return 1;
         if (plane_free(c, c->scales)) return 1;
     }
@@ -241,7 +243,7 @@ extern "C" {
 int trocm_init(int device) {
     std::lock_guard<std::mutex> lock(g_init_mutex);
     if (g_device >= 0) {
-        TROCM_REQUIRE(g_device == device, "Context is already set on device %d", g_device);  // gpu/src/device.rs:129-137
+        TROCM_REQUIRE(g_device.load() == device, "Context is already set on device %d", g_device.load());  // gpu/src/device.rs:129-137
         return 0;
     }
     int n = 0;

@@ -451,11 +451,7 @@ size_t decode_workspace_bytes(int64_t B, int64_t Hq, int64_t D) {
 // tile per wave, bounded by the workspace.  The quantised kernels are ALU/latency-limited and
 // do better with two workgroups per compute unit (Q8_0, 16k context: 79.7 us vs 94.4 us).
 int choose_decode_splits(int64_t BH, int64_t G, int n_tiles, int wg_per_cu) {
-    static int forced = -1;
-    if (forced < 0) {
-        const char *e = getenv("TROCM_DECODE_SPLITS");  // experiment knob, like tract's declare_knob!
-        forced = e ? atoi(e) : 0;
-    }
+    static const int forced = getenv("TROCM_DECODE_SPLITS") ? atoi(getenv("TROCM_DECODE_SPLITS")) : 0;  // experiment knob, like tract's declare_knob!
     int64_t target = (int64_t)num_compute_units() * wg_per_cu;
     int64_t ns = forced > 0 ? forced : (target + BH / 2) / BH;
     int64_t max_by_tiles = (n_tiles + kWaves - 1) / kWaves;

@@ -310,11 +310,7 @@ int launch_sdpa_prefill(const SdpaArgs &a, hipStream_t s) {
     // Shapes, named WM WN HG: 4 1 1 = four waves, 128 queries of one head; 2 2 1 = four waves, 64
     // queries, keys split two ways; 4 2 1 = eight waves, 128 queries, keys split two ways.
     // TROCM_PREFILL_SHAPE=<WM><WN><HG> forces one (experiments).
-    static int forced = -1;
-    if (forced < 0) {
-        const char *e = getenv("TROCM_PREFILL_SHAPE");
-        forced = e ? atoi(e) : 0;
-    }
+    static const int forced = getenv("TROCM_PREFILL_SHAPE") ? atoi(getenv("TROCM_PREFILL_SHAPE")) : 0;
     const int64_t G = a.Hq / a.Hkv;
     int shape = forced;
     if (!shape) {
