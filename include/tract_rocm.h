@@ -216,7 +216,9 @@ int trocm_q4_0_weights_shape(const trocm_q4_weights *weights, int64_t *batch, in
 /* The canonical blocks back (byte-identical to what was loaded). */
 int trocm_q4_0_weights_export(const trocm_q4_weights *weights, void *dst_blocks_device, void *stream);
 /* out[b, i, j] = sum_k act[b, i, k] * w[b / (act_batch / batch), j, k]; act and out dense, F32 or F16,
- * act 16-byte aligned, m <= 8. */
+ * act 16-byte aligned.  Built for the m <= 8 rows of a decode step (one pass over the weights); a
+ * larger m runs as groups of 8 rows, one pass each (the reference switches to a matrix-matrix
+ * kernel there, mod.rs:607-609, which this library does not have). */
 int trocm_q4_0_matvec(const trocm_q4_weights *weights, const void *act, int act_dtype, int64_t act_batch,
                       int64_t m, void *out, void *stream);
 

@@ -826,7 +826,6 @@ int trocm_q4_0_matvec(const trocm_q4_weights *w, const void *act, int act_dtype,
     TROCM_NOT_NULL(w);
     TROCM_REQUIRE(act_dtype == TROCM_F32 || act_dtype == TROCM_F16, "q4_0_matvec: activations must be F32 or F16");
     TROCM_REQUIRE(act_batch >= 0 && m >= 0, "q4_0_matvec: negative dimension");
-    TROCM_REQUIRE(m <= 8, "q4_0_matvec: m = %lld activation rows; the matrix-vector kernel takes at most 8", (long long)m);  // mod.rs:605
     if (act_batch == 0 || m == 0) return 0;                                      // mod.rs:586-588
     TROCM_REQUIRE(act_batch % w->batch == 0, "q4_0_matvec: activation batch %lld is not a multiple of the weights' batch %lld",
                   (long long)act_batch, (long long)w->batch);                     // mod.rs:488

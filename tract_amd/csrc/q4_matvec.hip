@@ -39,6 +39,7 @@ struct MatVecDev {
     const uint16_t *scales;   // [w_batch, n, k/32]
     const void *act;          // [act_batch, m, k]
     void *out;                // [act_batch, m, n]
+    int64_t act_stride_b, out_stride_b;   // elements between consecutive batches of act and out
     int n, k, ratio;          // ratio = act_batch / w_batch
     int kc;                   // activations staged per chunk (elements of k), a multiple of 32
     int groups;               // row groups of kMvWaves * R rows
@@ -121,8 +122,8 @@ __global__ __launch_bounds__(kMvThreads) void q4_0_matvec_kernel(MatVecDev p) {
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int b = blockIdx.y, wb = b / p.ratio;
     const int nb = p.k / 32;                            // blocks per weight row
-    const T *act = reinterpret_cast<const T *>(p.act) + (int64_t)b * M * p.k;
-    T *out = reinterpret_cast<T *>(p.out) + (int64_t)b * M * p.n;
+    const T *act = reinterpret_cast<const T *>(p.act) + (int64_t)b * p.act_stride_b;
+    T *out = reinterpret_cast<T *>(p.out) + (int64_t)b * p.out_stride_b;
     const bool one_chunk = p.kc >= p.k;                 // the activations fit in LDS: staged once per workgroup
 
     // A workgroup takes row groups g, g + gridDim.x, ... (kMvWaves * R rows each).
@@ -267,16 +268,24 @@ int launch_m(const MatVecDev &p, int m, int64_t act_batch, hipStream_t s) {
 
 int launch_q4_0_matvec(const void *codes, const void *scales, int64_t w_batch, int64_t n, int64_t k, const void *act,
                        int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s) {
-    MatVecDev p;
-    memset(&p, 0, sizeof(p));
-    p.codes = (const uint8_t *)codes, p.scales = (const uint16_t *)scales;
-    p.act = act, p.out = out;
-    p.n = (int)n, p.k = (int)k, p.ratio = (int)(act_batch / w_batch);
     const int64_t es = (int64_t)elem_bytes(act_dtype);
-    int64_t kc = kLdsBytes / (m * es) / 32 * 32;       // what fits, in whole blocks
-    if (kc > k) kc = k;
-    p.kc = (int)kc;
-    return act_dtype == TROCM_F16 ? launch_m<__half>(p, (int)m, act_batch, s) : launch_m<float>(p, (int)m, act_batch, s);
+    // More than 8 activation rows run as groups of 8 (each group streams the weights once): correct
+    // for any m, efficient only for the few rows of a decode step.
+    for (int64_t i0 = 0; i0 < m; i0 += 8) {
+        const int64_t mg = m - i0 < 8 ? m - i0 : 8;
+        MatVecDev p;
+        memset(&p, 0, sizeof(p));
+        p.codes = (const uint8_t *)codes, p.scales = (const uint16_t *)scales;
+        p.act = (const char *)act + i0 * k * es, p.out = (char *)out + i0 * n * es;
+        p.act_stride_b = m * k, p.out_stride_b = m * n;
+        p.n = (int)n, p.k = (int)k, p.ratio = (int)(act_batch / w_batch);
+        int64_t kc = kLdsBytes / (mg * es) / 32 * 32;   // what fits, in whole blocks
+        if (kc > k) kc = k;
+        p.kc = (int)kc;
+        const int rc = act_dtype == TROCM_F16 ? launch_m<__half>(p, (int)mg, act_batch, s) : launch_m<float>(p, (int)mg, act_batch, s);
+        if (rc) return rc;
+    }
+    return 0;
 }
 
 }  // namespace trocm

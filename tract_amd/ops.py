@@ -621,7 +621,7 @@ class Q40Weights:
 
 
 class GgmlGemm:
-    """Activations [b, m, k] x Q4_0 weights [b_w, n, k] -> [b, m, n] for m <= 8 (GgmlGemm::dispatch_eval,
+    """Activations [b, m, k] x Q4_0 weights [b_w, n, k] -> [b, m, n]; built for m <= 8 (GgmlGemm::dispatch_eval,
     cuda/src/kernels/matmul/mod.rs:575-627; output_shape :536-545)."""
 
     def output_shape(self, act_shape, w_shape):
