@@ -363,6 +363,27 @@ def test_prefill_grouped_heads_and_key_splits(rt, B, Hq, Hkv, Sq, Sk, D, causal)
     assert max_abs(got, cases.textbook_sdpa(q, k, v, causal=causal)) <= 4e-3
 
 
+@pytest.mark.parametrize("Sq", [2, 3, 5, 8, 17, 31])
+@pytest.mark.parametrize("Hq,Hkv,D,T", [(32, 8, 128, 3000), (16, 2, 128, 1100), (8, 4, 64, 777)])
+def test_few_queries_over_a_long_cache(rt, Sq, Hq, Hkv, D, T):
+    """q_len of a few tokens (speculative decoding, tiny chunks) with grouped heads: served by the MFMA
+    kernel that reads K/V once per kv head.  Causal row r must also equal the decode step that sees the
+    first T - Sq + r + 1 keys."""
+    rng = np.random.default_rng(4000 + Sq + T)
+    B = 2
+    q = (rng.standard_normal((B, Hq, Sq, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    k = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(np.float16)
+    got = tract_amd.Sdpa(datum_type=np.float16, is_causal=True).eval(q, k, v).to_numpy()
+    assert not np.isnan(got).any()
+    assert max_abs(got, orc.flash_sdpa(q, k, v, causal=True, threads=8)) <= 2e-2
+    assert max_abs(got, cases.textbook_sdpa(q, k, v, causal=True)) <= 4e-3
+    r = Sq // 2
+    n = T - Sq + r + 1
+    step = tract_amd.Sdpa(datum_type=np.float16).eval(q[:, :, r:r + 1], k[:, :, :n].copy(), v[:, :, :n].copy()).to_numpy()
+    assert max_abs(got[:, :, r:r + 1], step) <= 2e-3
+
+
 @pytest.mark.parametrize("kind", ["random", "causal_min", "causal_inf", "window_inf"])
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,mb,mh", [
     (1, 32, 8, 512, 2048, 128, 1, 1),     # the chunked-prefill shape, one mask for all heads, key splits
