@@ -141,6 +141,57 @@ def test_decode_with_additive_mask(rt, kind, dt, B, Hq, Hkv, D, T, mb, mh):
     assert max_abs(got, cases.textbook_sdpa(q, k, v, mask)) <= (2e-3 if dt == np.float16 else 2e-5)
 
 
+@pytest.mark.parametrize("fmt_name", ["plain", "Q8_0", "Q4_0"])
+@pytest.mark.parametrize("dt,Hq,Hkv,D,T", [
+    (np.float16, 24, 8, 128, 1500), (np.float16, 14, 2, 128, 3000), (np.float16, 12, 2, 128, 700),
+    (np.float16, 10, 2, 128, 333), (np.float32, 6, 2, 64, 513), (np.float16, 21, 3, 64, 200),
+])
+def test_decode_group_sizes_that_are_not_powers_of_two(rt, fmt_name, dt, Hq, Hkv, D, T):
+    """Group sizes 3, 5, 6, 7 (24q/8kv, 14q/2kv ... of current decoders) run on the split-K kernels of the
+    next larger instantiated group size; prefill, fused decode steps, a masked step and the ragged
+    form, each against the oracle."""
+    if fmt_name != "plain" and (dt != np.float16 or D != 128):
+        pytest.skip("quantised caches: f16 queries, head_dim 128")
+    fmt = {"plain": None, "Q8_0": tract_amd.Q8_0, "Q4_0": tract_amd.Q4_0}[fmt_name]
+    tol = TOL[np.dtype(dt)] if fmt is None else 2e-2
+    rng = np.random.default_rng(300 + Hq + T)
+    B = 2
+    k = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(dt)
+    v = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(dt)
+    st = tract_amd.InPlaceKvSdpa(axis=2, causal=True, storage_format=fmt).state()
+    st.k.push(k), st.v.push(v)
+    kd, vd = k, v
+    if fmt is not None:   # the oracle attends over the dequantised blocks
+        kd = orc.dequant(fmt, orc.quant(fmt, k), dt)
+        vd = orc.dequant(fmt, orc.quant(fmt, v), dt)
+    for _ in range(3):
+        q = (rng.standard_normal((B, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(dt)
+        kn = rng.standard_normal((B, Hkv, 1, D), dtype=np.float32).astype(dt)
+        vn = rng.standard_normal((B, Hkv, 1, D), dtype=np.float32).astype(dt)
+        got = st.eval([q, kn, vn]).to_numpy()
+        kq, vq = (kn, vn) if fmt is None else (orc.dequant(fmt, orc.quant(fmt, kn), dt), orc.dequant(fmt, orc.quant(fmt, vn), dt))
+        kd, vd = np.concatenate([kd, kq], axis=2), np.concatenate([vd, vq], axis=2)
+        assert not np.isnan(got).any()
+        assert max_abs(got, orc.flash_sdpa(q, kd, vd, causal=True, threads=4)) <= tol
+    if fmt is None:
+        assert st.k.valid_contiguous().tobytes() == kd.tobytes()
+        # a per-head mask on the same shape
+        mask = (rng.standard_normal((B, Hq, 1, kd.shape[2]), dtype=np.float32) * 2).astype(dt)
+        got = tract_amd.Sdpa(datum_type=dt).eval(q, kd, vd, mask).to_numpy()
+        assert max_abs(got, orc.flash_sdpa(q, kd, vd, mask=mask, threads=4)) <= tol
+        # the ragged form: every batch entry as a sequence of its own
+        caches = []
+        for b in range(B):
+            kc, vc = tract_amd.InPlaceKvCache(2), tract_amd.InPlaceKvCache(2)
+            n = kd.shape[2] - 17 * b
+            kc.push(kd[b:b + 1, :, :n]), vc.push(vd[b:b + 1, :, :n])
+            caches.append((kc, vc, n))
+        got = tract_amd.sdpa_decode_ragged(tract_amd.DeviceTensor.from_numpy(q), [c[0] for c in caches], [c[1] for c in caches]).to_numpy()
+        for b, (_, _, n) in enumerate(caches):
+            want = orc.flash_sdpa(q[b:b + 1], kd[b:b + 1, :, :n], vd[b:b + 1, :, :n], threads=4)
+            assert max_abs(got[b:b + 1], want) <= tol
+
+
 @pytest.mark.parametrize("splits", [1, 2, 3, 7, 64])
 def test_decode_any_split_count_agrees(rt, splits, monkeypatch):
     # The split merge is exact in real arithmetic (log-sum-exp identity).

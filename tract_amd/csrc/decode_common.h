@@ -28,6 +28,9 @@ struct DecodeDev {
     int T;                                          // valid tokens
     int tiles_per_split, nsplit;
     int Hq, Hkv;
+    // Query heads per kv head.  The kernels are instantiated for G = 1, 2, 4, 8; another group size runs
+    // on the next larger one: the extra heads of a workgroup repeat its last real head and write nothing.
+    int g_real;
     float scale_log2;
     float *part_o;   // [B*Hkv*nsplit][G*D]
     float *part_ml;  // [B*Hkv*nsplit][2*G]
@@ -224,16 +227,17 @@ __device__ __forceinline__ void tail_merge(const DecodeDev &p, int *counter, int
             acc += ov[e][sp] * f;
             ll += lv[e][sp] * f;
         }
-        if (idx < G * D) out[idx] = from_f32<T>(acc / ll);
+        if (idx < p.g_real * D) out[idx] = from_f32<T>(acc / ll);
     }
 }
 
-// Merge launch: grid (kv_heads, batch, G), D threads; runs after the split kernel on the same stream.
+// Merge launch: grid (kv_heads, batch, real query heads per kv head), D threads; runs after the split
+// kernel on the same stream.
 template <typename T, int D, int G>
 __global__ __launch_bounds__(D) void sdpa_decode_merge_kernel(DecodeDev p) {
     const int kvh = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
     const int64_t bh = (int64_t)b * p.Hkv + kvh;
-    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)b * p.Hq + (int64_t)kvh * G + h) * D;
+    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)b * p.Hq + (int64_t)kvh * p.g_real + h) * D;
     merge_head<T, D, G>(p, bh * p.nsplit, 1, p.nsplit, h, out, threadIdx.x);
 }
 

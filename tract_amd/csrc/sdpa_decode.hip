@@ -133,7 +133,7 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
         // wave-uniform row bases plus one 32-bit lane offset
         const uint32_t moff = (uint32_t)min(tile * kTile + qk_row, last_tok) * (uint32_t)sizeof(T);
 #pragma unroll
-        for (int h = 0; h < G; h++) mreg[h] = *reinterpret_cast<const T *>(wk.mask + h * wk.mask_stride_h + moff);
+        for (int h = 0; h < G; h++) mreg[h] = *reinterpret_cast<const T *>(wk.mask + min(h, p.g_real - 1) * wk.mask_stride_h + moff);
     };
     auto issue_k = [&](int tile) {
         const int t0 = tile * kTile;
@@ -184,7 +184,7 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
     // ---- stage the G query vectors of this KV head (the first tile's K and V are already in flight) ----
     {
         const u32x4 *qg = reinterpret_cast<const u32x4 *>(wk.q);
-        for (int i = tid; i < G * CPR; i += kThreads) lds_q[i] = qg[i];
+        for (int i = tid; i < G * CPR; i += kThreads) lds_q[i] = qg[min(i / CPR, p.g_real - 1) * CPR + i % CPR];
     }
     __syncthreads();
     const u32x4 *lds_krow = &lds_k[w][qk_row * CPR];
@@ -308,7 +308,7 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
             ll += comb[ww * kCombStride + G * D + G + h] * f;
         }
         if (wk.direct) {
-            out[idx] = from_f32<T>(acc / ll);
+            if (h < p.g_real) out[idx] = from_f32<T>(acc / ll);
         } else if (wk.counter == nullptr) {
             int64_t slot = wk.part;
             p.part_o[slot * (G * D) + idx] = acc;
@@ -338,7 +338,7 @@ template <typename T, int D, int G, bool MASK>
 __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1) void sdpa_decode_kernel(DecodeDev p) {
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     DecodeWork wk;
-    const int64_t row = ((int64_t)b * p.Hq + (int64_t)kvh * G) * D * (int64_t)sizeof(T);
+    const int64_t row = ((int64_t)b * p.Hq + (int64_t)kvh * p.g_real) * D * (int64_t)sizeof(T);
     wk.q = p.q + row;
     wk.out = p.out + row;
     wk.kbase = p.k + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
@@ -365,7 +365,7 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     wk.nsplit = p.nsplit;
     wk.part_first = bh * p.nsplit;
     wk.part_stride = 1;
-    wk.mask = MASK ? p.mask + (int64_t)b * p.mask_stride_b + (int64_t)kvh * G * p.mask_stride_h : nullptr;
+    wk.mask = MASK ? p.mask + (int64_t)b * p.mask_stride_b + (int64_t)kvh * p.g_real * p.mask_stride_h : nullptr;
     wk.mask_stride_h = p.mask_stride_h;
     decode_body<T, D, G, MASK>(p, wk);
 }
@@ -379,7 +379,7 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     const RaggedItem it = items[blockIdx.x];
     const int kvh = blockIdx.y;
     DecodeWork wk;
-    const int64_t row = ((int64_t)it.seq * p.Hq + (int64_t)kvh * G) * D * (int64_t)sizeof(T);
+    const int64_t row = ((int64_t)it.seq * p.Hq + (int64_t)kvh * p.g_real) * D * (int64_t)sizeof(T);
     wk.q = p.q + row;
     wk.out = p.out + row;
     wk.kbase = it.k + (int64_t)kvh * it.stride_h;
@@ -409,7 +409,7 @@ __global__ __launch_bounds__(D) void sdpa_decode_ragged_merge_kernel(DecodeDev p
     const int kvh = blockIdx.x, seq = blockIdx.y, h = blockIdx.z;
     const RaggedSeqSlots ss = seqs[seq];
     if (ss.nsplit <= 1) return;
-    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)seq * p.Hq + (int64_t)kvh * G + h) * D;
+    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)seq * p.Hq + (int64_t)kvh * p.g_real + h) * D;
     merge_head<T, D, G>(p, (int64_t)ss.slot0 * p.Hkv + kvh, p.Hkv, ss.nsplit, h, out, threadIdx.x);
 }
 
@@ -420,7 +420,7 @@ void launch_both(const DecodeDev &p, dim3 grid, hipStream_t s) {
     else
         hipLaunchKernelGGL((sdpa_decode_kernel<T, D, G, false>), grid, dim3(kThreads), 0, s, p);
     if (p.nsplit > 1 && p.counters == nullptr)
-        hipLaunchKernelGGL((sdpa_decode_merge_kernel<T, D, G>), dim3(grid.y, grid.z, G), dim3(D), 0, s, p);
+        hipLaunchKernelGGL((sdpa_decode_merge_kernel<T, D, G>), dim3(grid.y, grid.z, p.g_real), dim3(D), 0, s, p);
 }
 
 template <typename T, int D>
@@ -468,8 +468,9 @@ int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
     if (a.q_dtype != a.kv_fmt) return 2;
     if (a.D != 64 && a.D != 128) return 2;
     if (a.Hq % a.Hkv) return 2;
-    int64_t G = a.Hq / a.Hkv;
-    if (G != 1 && G != 2 && G != 4 && G != 8) return 2;
+    const int64_t g_real = a.Hq / a.Hkv;
+    if (g_real > 8) return 2;
+    const int64_t G = g_real <= 2 ? g_real : g_real <= 4 ? 4 : 8;   // the instantiation that runs it
     size_t es = elem_bytes(a.kv_fmt);
     // 128-bit loads: rows and bases must be 16-byte aligned
     if ((a.kv_stride_b * es) % 16 || (a.kv_stride_h * es) % 16 || (a.kv_stride_t * es) % 16) return 2;
@@ -507,6 +508,7 @@ int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
     p.interleave = interleave;
     p.Hq = (int)a.Hq;
     p.Hkv = (int)a.Hkv;
+    p.g_real = (int)g_real;
     p.scale_log2 = a.scale * 1.4426950408889634f;
     p.k_new = (const char *)a.k_new;
     p.v_new = (const char *)a.v_new;
@@ -566,7 +568,7 @@ void launch_ragged(const DecodeDev &p, const RaggedItem *items, int n_items, con
                    bool any_split, hipStream_t s) {
     hipLaunchKernelGGL((sdpa_decode_ragged_kernel<T, D, G>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
     if (any_split)
-        hipLaunchKernelGGL((sdpa_decode_ragged_merge_kernel<T, D, G>), dim3(p.Hkv, n_seq, G), dim3(D), 0, s, p, seqs);
+        hipLaunchKernelGGL((sdpa_decode_ragged_merge_kernel<T, D, G>), dim3(p.Hkv, n_seq, p.g_real), dim3(D), 0, s, p, seqs);
 }
 
 template <typename T, int D>
@@ -617,10 +619,11 @@ int ragged_per_sequence(const void *q, void *out, int q_dtype, int kv_fmt, int64
 int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt, int64_t n_seq, int64_t Hq, int64_t Hkv,
                               int64_t D, const RaggedSeq *seqs, float scale, void *workspace, size_t workspace_bytes,
                               const void *k_new, const void *v_new, hipStream_t s) {
-    const int64_t G = Hq / Hkv;
+    const int64_t g_real = Hq / Hkv;
+    const int64_t G = g_real <= 2 ? g_real : g_real <= 4 ? 4 : 8;   // the instantiation that runs it
     const size_t es = elem_bytes(kv_fmt);
     bool fast = (kv_fmt == TROCM_F16 || kv_fmt == TROCM_F32) && q_dtype == kv_fmt && (D == 64 || D == 128) &&
-                (G == 1 || G == 2 || G == 4 || G == 8) && workspace != nullptr && (uintptr_t)q % 16 == 0 &&
+                g_real >= 1 && g_real <= 8 && workspace != nullptr && (uintptr_t)q % 16 == 0 &&
                 n_seq <= 2048 && Hkv <= 65535;
     for (int64_t i = 0; i < n_seq && fast; i++)
         fast = (uintptr_t)seqs[i].k % 16 == 0 && (uintptr_t)seqs[i].v % 16 == 0 && seqs[i].len < (1ll << 30) &&
@@ -635,7 +638,7 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     int64_t total_tiles = 0;
     for (int64_t i = 0; i < n_seq; i++) total_tiles += (seqs[i].len + kTile - 1) / kTile;
     const int64_t rows_cap = (int64_t)((workspace_bytes - kWsCounterBytes) / ((D + 2) * sizeof(float)));
-    const int64_t max_items_ws = rows_cap / Hq;  // every item may need a partial record per q head
+    const int64_t max_items_ws = rows_cap / (Hkv * G);  // every item may need a partial record per (padded) q head
     const int64_t max_items_tbl =
         ((int64_t)kWsCounterBytes - n_seq * (int64_t)sizeof(RaggedSeqSlots)) / (int64_t)sizeof(RaggedItem);
     const int64_t max_items = max_items_ws < max_items_tbl ? max_items_ws : max_items_tbl;
@@ -694,6 +697,7 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     p.kv_stride_t = D * (int64_t)es;
     p.Hq = (int)Hq;
     p.Hkv = (int)Hkv;
+    p.g_real = (int)g_real;
     p.scale_log2 = scale * 1.4426950408889634f;
     p.k_new = (const char *)k_new;
     p.v_new = (const char *)v_new;

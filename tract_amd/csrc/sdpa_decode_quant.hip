@@ -78,10 +78,11 @@ __global__ __launch_bounds__(kThreads, G <= 4 ? 2 : 1) void sdpa_decode_q_kernel
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
 
     {
-        const u32x4 *qg = reinterpret_cast<const u32x4 *>(p.q + ((int64_t)b * p.Hq + (int64_t)kvh * G) * (D * 2));
-        for (int i = tid; i < G * QC; i += kThreads) lds_q[i] = qg[i];
+        const u32x4 *qg = reinterpret_cast<const u32x4 *>(p.q + ((int64_t)b * p.Hq + (int64_t)kvh * p.g_real) * (D * 2));
+        for (int i = tid; i < G * QC; i += kThreads) lds_q[i] = qg[min(i / QC, p.g_real - 1) * QC + i % QC];
         if (tid < G * kNB) {
-            const __half *qh = reinterpret_cast<const __half *>(p.q) + ((int64_t)b * p.Hq + (int64_t)kvh * G) * D + tid * 32;
+            const __half *qh = reinterpret_cast<const __half *>(p.q) + ((int64_t)b * p.Hq + (int64_t)kvh * p.g_real) * D +
+                               min(tid / kNB, p.g_real - 1) * D + (tid % kNB) * 32;
             float sum = 0.0f;
             for (int i = 0; i < 32; i++) sum += __half2float(qh[i]);
             lds_qsum[tid] = sum * Q::kBias;
@@ -323,7 +324,7 @@ __global__ __launch_bounds__(kThreads, G <= 4 ? 2 : 1) void sdpa_decode_q_kernel
     __syncthreads();
 
     const int64_t bh = (int64_t)b * p.Hkv + kvh;
-    __half *out = reinterpret_cast<__half *>(p.out) + ((int64_t)b * p.Hq + (int64_t)kvh * G) * D;
+    __half *out = reinterpret_cast<__half *>(p.out) + ((int64_t)b * p.Hq + (int64_t)kvh * p.g_real) * D;
     for (int idx = tid; idx < G * D; idx += kThreads) {
         int h = idx / D;
         float mm = -INFINITY;
@@ -337,7 +338,7 @@ __global__ __launch_bounds__(kThreads, G <= 4 ? 2 : 1) void sdpa_decode_q_kernel
             ll += comb[ww][G * D + G + h] * f;
         }
         if (p.nsplit == 1) {
-            out[idx] = __float2half_rn(acc / ll);
+            if (h < p.g_real) out[idx] = __float2half_rn(acc / ll);
         } else if (p.counters == nullptr) {
             int64_t slot = bh * p.nsplit + split;
             p.part_o[slot * (G * D) + idx] = acc;
@@ -362,7 +363,7 @@ template <int FMT, int G>
 int launch_one(const DecodeDev &p, dim3 grid, hipStream_t s) {
     hipLaunchKernelGGL((sdpa_decode_q_kernel<FMT, G>), grid, dim3(kThreads), 0, s, p);
     if (p.nsplit > 1 && p.counters == nullptr)
-        hipLaunchKernelGGL((sdpa_decode_merge_kernel<__half, kD, G>), dim3(grid.y, grid.z, G), dim3(kD), 0, s, p);
+        hipLaunchKernelGGL((sdpa_decode_merge_kernel<__half, kD, G>), dim3(grid.y, grid.z, p.g_real), dim3(kD), 0, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("sdpa_decode (quantised KV) launch failed: %s", hipGetErrorString(e));
     return 0;
@@ -386,8 +387,9 @@ int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s) {
     if (a.kv_fmt != TROCM_Q8_0 && a.kv_fmt != TROCM_Q4_0) return 2;
     if (a.q_dtype != TROCM_F16 || a.D != kD) return 2;
     if (a.Hq % a.Hkv) return 2;
-    int64_t G = a.Hq / a.Hkv;
-    if (G != 1 && G != 2 && G != 4 && G != 8) return 2;
+    const int64_t g_real = a.Hq / a.Hkv;
+    if (g_real > 8) return 2;
+    const int64_t G = g_real <= 2 ? g_real : g_real <= 4 ? 4 : 8;   // the instantiation that runs it
     if (a.kv_stride_t != a.D) return 2;  // cache planes: token rows are dense
     if ((uintptr_t)a.k % 16 || (uintptr_t)a.v % 16 || (uintptr_t)a.q % 16 || (uintptr_t)a.k_scales % 4 ||
         (uintptr_t)a.v_scales % 4)
@@ -427,6 +429,7 @@ int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s) {
     p.nsplit = nsplit;
     p.Hq = (int)a.Hq;
     p.Hkv = (int)a.Hkv;
+    p.g_real = (int)g_real;
     p.scale_log2 = a.scale * 1.4426950408889634f;
     p.part_ml = (float *)((char *)a.workspace + kWsCounterBytes);
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * G;
