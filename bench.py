@@ -435,6 +435,13 @@ def run_ops(ta, args):
     res["prefill_512x4096_causal_as_mask_input"] = {"us": round(us, 2), "tflops": round(fl / us / 1e6, 1)}
     us = time_calls(ta, lambda: sc.eval(qp, kp, vp, out=op), 50)
     res["prefill_512x4096_is_causal"] = {"us": round(us, 2), "tflops": round(fl / us / 1e6, 1)}
+    # the same chunk over Q8_0 / Q4_0 caches of 4096 tokens (blocks dequantised while the tiles are staged)
+    for name, fmt in (("q8_0", ta.Q8_0), ("q4_0", ta.Q4_0)):
+        stq = ta.InPlaceKvSdpa(axis=2, causal=True, storage_format=fmt).state()
+        stq.k.push(kp), stq.v.push(vp)
+        us = time_calls(ta, lambda: stq.attend(qp, out=op), 50)
+        res[f"prefill_512x4096_{name}_cache"] = {"us": round(us, 2), "tflops": round(fl / us / 1e6, 1)}
+        del stq
     del kvs, kp, vp
     # Q4_0 weights x one activation row (the decode-time projections of an 8B-class decoder), f16; each
     # shape rotates over 8 weight matrices so that launches read HBM

@@ -475,6 +475,40 @@ def test_prefill_with_additive_mask(rt, kind, B, Hq, Hkv, Sq, Sk, D, mb, mh):
         assert max_abs(got, same) <= 2e-3
 
 
+@pytest.mark.parametrize("fmt_name", ["Q8_0", "Q4_0"])
+@pytest.mark.parametrize("B,Hq,Hkv,D,chunks", [
+    (1, 32, 8, 128, (512, 512, 300)),     # chunked prefill into a quantised cache, key splits
+    (2, 8, 2, 128, (100, 77, 33)), (1, 4, 4, 128, (64, 200)), (2, 6, 2, 128, (40, 130)),
+    (1, 8, 2, 64, (96, 160)), (3, 16, 16, 64, (70,)),
+])
+def test_prefill_over_a_quantised_cache(rt, fmt_name, B, Hq, Hkv, D, chunks):
+    """Chunks of a prompt appended to a Q8_0 / Q4_0 cache (quantised on append), each attending causally
+    over the cache so far: the MFMA kernel dequantises the blocks while staging its K/V tiles.  The
+    oracle attends over the dequantised blocks (the reference states attention over a block-quantised
+    tensor through simulate_precision_loss, block_quant/mod.rs:110-155)."""
+    fmt = {"Q8_0": tract_amd.Q8_0, "Q4_0": tract_amd.Q4_0}[fmt_name]
+    rng = np.random.default_rng(5000 + Hq + sum(chunks))
+    st = tract_amd.InPlaceKvSdpa(axis=2, causal=True, storage_format=fmt).state()
+    kd = vd = None
+    for S in chunks:
+        q = (rng.standard_normal((B, Hq, S, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+        k = rng.standard_normal((B, Hkv, S, D), dtype=np.float32).astype(np.float16)
+        v = rng.standard_normal((B, Hkv, S, D), dtype=np.float32).astype(np.float16)
+        k[:, :, :, 5] *= 12.0   # an outlier channel: blocks with very different scales
+        got = st.eval([q, k, v]).to_numpy()
+        kq = orc.dequant(fmt, orc.quant(fmt, k), np.float16)
+        vq = orc.dequant(fmt, orc.quant(fmt, v), np.float16)
+        kd = kq if kd is None else np.concatenate([kd, kq], axis=2)
+        vd = vq if vd is None else np.concatenate([vd, vq], axis=2)
+        assert not np.isnan(got).any()
+        assert max_abs(got, orc.flash_sdpa(q, kd, vd, causal=True, threads=8)) <= 2e-2
+        assert max_abs(got, cases.textbook_sdpa(q, kd, vd, causal=True)) <= 4e-3
+    # the stored blocks are the oracle's, bit for bit
+    want_blocks = orc.quant(fmt, k)   # last chunk
+    got_blocks = st.k.valid_contiguous()[:, :, -chunks[-1]:]
+    assert got_blocks.tobytes() == want_blocks.tobytes()
+
+
 _PREFILL_ENV_CODE = """
 import os, sys, numpy as np
 import tract_amd

@@ -56,6 +56,10 @@ struct PrefillPP {
     // != NULL: arrival counters, one per (batch, query tile, head group, kv head), zero between launches;
     // the last key split of a tile to arrive merges the partials itself and no merge launch follows
     int *counters;
+    // Q8_0 / Q4_0 caches (kernels with FMT != TROCM_F16): code planes [B, Hkv, pitch, D or D/2] bytes at
+    // k / v, f16 scale planes [B, Hkv, pitch, D/32]; strides in token rows
+    const uint16_t *k_scales, *v_scales;
+    int64_t row_stride_b, row_stride_h;
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -70,7 +74,24 @@ __device__ __forceinline__ half4_t lds_read_tr16(const _Float16 *lds_ptr) {
 
 constexpr int kWavesPP = 8, kThreadsPP = 64 * kWavesPP, kTileN = 64;
 
-template <int D, int HG, bool MASK>
+__device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+// bytes (b0, b1) / (b2, b3) of a word as the half pairs (1024 + b): the byte under exponent byte 0x64
+__device__ __forceinline__ half2_t magic_lo(uint32_t w) { return __builtin_bit_cast(half2_t, perm(0x64646464u, w, 0x04010400u)); }
+__device__ __forceinline__ half2_t magic_hi(uint32_t w) { return __builtin_bit_cast(half2_t, perm(0x64646464u, w, 0x04030402u)); }
+
+// Eight code bytes -> the reference's f16 dequantised values (code - zero) * d, each rounded once to
+// f16 (q4_0.rs:82-95): (1024 + u) - (1024 + zero) is exact, the product rounds.
+__device__ __forceinline__ u32x4 dequant8(uint32_t b0123, uint32_t b4567, half2_t zero1024, half2_t d2) {
+    u32x4 r;
+    r.x = __builtin_bit_cast(uint32_t, (magic_lo(b0123) - zero1024) * d2);
+    r.y = __builtin_bit_cast(uint32_t, (magic_hi(b0123) - zero1024) * d2);
+    r.z = __builtin_bit_cast(uint32_t, (magic_lo(b4567) - zero1024) * d2);
+    r.w = __builtin_bit_cast(uint32_t, (magic_hi(b4567) - zero1024) * d2);
+    return r;
+}
+
+template <int D, int HG, bool MASK, int FMT>
 __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p) {
     constexpr int QB = kWavesPP / HG;     // 32-query blocks per workgroup
     constexpr int BLOCK_M = 32 * QB;
@@ -127,23 +148,80 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
 
     half8_t qf[KS];
     u32x4 kpre[NL], vpre[NL];
+    // Quantised caches: a thread fetches one unit of 16 elements of a key row per tile and tensor -- 16
+    // code bytes (Q8_0) or the 8 bytes that hold elements j..j+7 and 16+j..16+j+7 of a block (Q4_0) --
+    // plus the block's scale, and dequantises while staging.
+    constexpr bool QUANT = FMT != TROCM_F16;
+    constexpr int UPR = D / 16;                        // units per key row
+    const bool q_active = tid < kTileN * UPR;          // D = 64: half the threads
+    const int q_key = tid / UPR, q_unit = tid % UPR;
+    uint16_t ksc = 0, vsc = 0;
+    const uint8_t *kq = nullptr, *vq = nullptr;
+    const uint16_t *ksp = nullptr, *vsp = nullptr;
+    if constexpr (QUANT) {
+        const int64_t plane_row = (int64_t)b * p.row_stride_b + (int64_t)kvh * p.row_stride_h;
+        constexpr int RB = FMT == TROCM_Q8_0 ? D : D / 2;   // code bytes per token row
+        kq = reinterpret_cast<const uint8_t *>(p.k) + plane_row * RB;
+        vq = reinterpret_cast<const uint8_t *>(p.v) + plane_row * RB;
+        ksp = p.k_scales + plane_row * (D / 32);
+        vsp = p.v_scales + plane_row * (D / 32);
+    }
     auto prefetch = [&](int kt) {
+        if constexpr (!QUANT) {
 #pragma unroll
-        for (int j = 0; j < NL; j++) {
-            int c = j * kThreadsPP + tid;
-            int key = c / (D / 8), dc = c % (D / 8);
-            int64_t row = min(kt * kTileN + key, p.Sk - 1);
-            kpre[j] = *reinterpret_cast<const u32x4 *>(kbase + row * p.kv_stride_t + dc * 8);
-            vpre[j] = *reinterpret_cast<const u32x4 *>(vbase + row * p.kv_stride_t + dc * 8);
+            for (int j = 0; j < NL; j++) {
+                int c = j * kThreadsPP + tid;
+                int key = c / (D / 8), dc = c % (D / 8);
+                int64_t row = min(kt * kTileN + key, p.Sk - 1);
+                kpre[j] = *reinterpret_cast<const u32x4 *>(kbase + row * p.kv_stride_t + dc * 8);
+                vpre[j] = *reinterpret_cast<const u32x4 *>(vbase + row * p.kv_stride_t + dc * 8);
+            }
+        } else if (q_active) {
+            const int64_t row = min(kt * kTileN + q_key, p.Sk - 1);
+            if constexpr (FMT == TROCM_Q8_0) {
+                kpre[0] = *reinterpret_cast<const u32x4 *>(kq + row * D + q_unit * 16);
+                vpre[0] = *reinterpret_cast<const u32x4 *>(vq + row * D + q_unit * 16);
+            } else {   // unit u of a row: block u / 2, bytes 8 * (u % 2) .. + 8 of its 16 code bytes
+                const uint2 kk = *reinterpret_cast<const uint2 *>(kq + row * (D / 2) + q_unit * 8);
+                const uint2 vv = *reinterpret_cast<const uint2 *>(vq + row * (D / 2) + q_unit * 8);
+                kpre[0].x = kk.x, kpre[0].y = kk.y, vpre[0].x = vv.x, vpre[0].y = vv.y;
+            }
+            ksc = ksp[row * (D / 32) + q_unit / 2];
+            vsc = vsp[row * (D / 32) + q_unit / 2];
         }
     };
     auto stage = [&](int kbuf, int vbuf) {
+        if constexpr (!QUANT) {
 #pragma unroll
-        for (int j = 0; j < NL; j++) {
-            int c = j * kThreadsPP + tid;
-            int key = c / (D / 8), dc = c % (D / 8);
-            *reinterpret_cast<u32x4 *>(&lds_k[kbuf][key * KROW + dc * 8]) = kpre[j];
-            *reinterpret_cast<u32x4 *>(&lds_v[vbuf][key * VROW + dc * 8]) = vpre[j];
+            for (int j = 0; j < NL; j++) {
+                int c = j * kThreadsPP + tid;
+                int key = c / (D / 8), dc = c % (D / 8);
+                *reinterpret_cast<u32x4 *>(&lds_k[kbuf][key * KROW + dc * 8]) = kpre[j];
+                *reinterpret_cast<u32x4 *>(&lds_v[vbuf][key * VROW + dc * 8]) = vpre[j];
+            }
+        } else if (q_active) {
+            const half2_t kd = {__builtin_bit_cast(_Float16, ksc), __builtin_bit_cast(_Float16, ksc)};
+            const half2_t vd = {__builtin_bit_cast(_Float16, vsc), __builtin_bit_cast(_Float16, vsc)};
+            u32x4 ka, kb2, va, vb2;     // two chunks of 8 halves per tensor
+            int dc_a, dc_b;             // their 16-byte chunk indices in the row
+            if constexpr (FMT == TROCM_Q8_0) {
+                const half2_t zero = {(_Float16)1152.0f, (_Float16)1152.0f};   // 1024 + 128: codes are stored as code ^ 0x80
+                const uint32_t x = 0x80808080u;
+                ka = dequant8(kpre[0].x ^ x, kpre[0].y ^ x, zero, kd), kb2 = dequant8(kpre[0].z ^ x, kpre[0].w ^ x, zero, kd);
+                va = dequant8(vpre[0].x ^ x, vpre[0].y ^ x, zero, vd), vb2 = dequant8(vpre[0].z ^ x, vpre[0].w ^ x, zero, vd);
+                dc_a = 2 * q_unit, dc_b = 2 * q_unit + 1;
+            } else {
+                const half2_t zero = {(_Float16)1032.0f, (_Float16)1032.0f};   // 1024 + 8
+                // low nibbles: elements j..j+7 of the block, high nibbles: elements 16+j..16+j+7
+                const uint32_t m = 0x0F0F0F0Fu;
+                ka = dequant8(kpre[0].x & m, kpre[0].y & m, zero, kd), kb2 = dequant8((kpre[0].x >> 4) & m, (kpre[0].y >> 4) & m, zero, kd);
+                va = dequant8(vpre[0].x & m, vpre[0].y & m, zero, vd), vb2 = dequant8((vpre[0].x >> 4) & m, (vpre[0].y >> 4) & m, zero, vd);
+                dc_a = 4 * (q_unit / 2) + (q_unit % 2), dc_b = dc_a + 2;
+            }
+            *reinterpret_cast<u32x4 *>(&lds_k[kbuf][q_key * KROW + dc_a * 8]) = ka;
+            *reinterpret_cast<u32x4 *>(&lds_k[kbuf][q_key * KROW + dc_b * 8]) = kb2;
+            *reinterpret_cast<u32x4 *>(&lds_v[vbuf][q_key * VROW + dc_a * 8]) = va;
+            *reinterpret_cast<u32x4 *>(&lds_v[vbuf][q_key * VROW + dc_b * 8]) = vb2;
         }
     };
 
@@ -480,11 +558,15 @@ __global__ __launch_bounds__(256) void sdpa_prefill_merge_kernel(PrefillPP p) {
 }
 
 template <int D, int HG>
-int launch_cfg(const PrefillPP &p, int64_t wgs, hipStream_t s) {
-    if (p.mask)
-        hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG, true>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
+int launch_cfg(const PrefillPP &p, int fmt, int64_t wgs, hipStream_t s) {
+    if (fmt == TROCM_Q8_0)
+        hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG, false, TROCM_Q8_0>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
+    else if (fmt == TROCM_Q4_0)
+        hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG, false, TROCM_Q4_0>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
+    else if (p.mask)
+        hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG, true, TROCM_F16>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
     else
-        hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG, false>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
+        hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG, false, TROCM_F16>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("sdpa_prefill_pp launch failed: %s", hipGetErrorString(e));
     if (p.nsplit > 1 && p.counters == nullptr) {
@@ -496,11 +578,11 @@ int launch_cfg(const PrefillPP &p, int64_t wgs, hipStream_t s) {
 }
 
 template <int D>
-int launch_hg(const PrefillPP &p, int hg, int64_t wgs, hipStream_t s) {
+int launch_hg(const PrefillPP &p, int fmt, int hg, int64_t wgs, hipStream_t s) {
     switch (hg) {
-        case 4: return launch_cfg<D, 4>(p, wgs, s);
-        case 2: return launch_cfg<D, 2>(p, wgs, s);
-        default: return launch_cfg<D, 1>(p, wgs, s);
+        case 4: return launch_cfg<D, 4>(p, fmt, wgs, s);
+        case 2: return launch_cfg<D, 2>(p, fmt, wgs, s);
+        default: return launch_cfg<D, 1>(p, fmt, wgs, s);
     }
 }
 
@@ -525,7 +607,10 @@ size_t prefill_workspace_bytes(int64_t B, int64_t Hq, int64_t Sq, int64_t D) {
 }
 
 int launch_sdpa_prefill_pp(const SdpaArgs &a, hipStream_t s) {
-    if (a.q_dtype != TROCM_F16 || a.kv_fmt != TROCM_F16) return 2;
+    if (a.q_dtype != TROCM_F16) return 2;
+    const bool quant = is_quant(a.kv_fmt);
+    if (!quant && a.kv_fmt != TROCM_F16) return 2;
+    if (quant && (a.mask || a.kv_stride_t != a.D || !a.k_scales || !a.v_scales)) return 2;   // cache planes: dense token rows
     if (a.mask && a.causal) return 2;
     if (a.D != 128 && a.D != 64) return 2;
     if (a.Sq < 2 || a.Sk < 1 || a.Hq % a.Hkv) return 2;
@@ -534,6 +619,12 @@ int launch_sdpa_prefill_pp(const SdpaArgs &a, hipStream_t s) {
     if (a.Sk >= (1ll << 30) || a.Sq >= (1ll << 30) || a.B >= (1ll << 20)) return 2;
     if ((a.kv_stride_b % 8) || (a.kv_stride_h % 8) || (a.kv_stride_t % 8)) return 2;  // 128-bit row loads
     if ((uintptr_t)a.q % 16 || (uintptr_t)a.k % 16 || (uintptr_t)a.v % 16 || (uintptr_t)a.out % 8) return 2;
+    if (quant) {   // strides arrive in elements of the logical [.., D] rows: whole token rows per head and batch
+        if (a.kv_stride_h % a.D || a.kv_stride_b % a.D) return 2;
+        const int64_t rb = a.kv_fmt == TROCM_Q8_0 ? a.D : a.D / 2;
+        if (((a.kv_stride_h / a.D) * rb) % 16 || ((a.kv_stride_b / a.D) * rb) % 16) return 2;
+        if ((uintptr_t)a.k_scales % 2 || (uintptr_t)a.v_scales % 2) return 2;
+    }
     static const int enabled = env_int("TROCM_PREFILL_PP", 1);
     if (!enabled) return 2;
     static const int forced_hg = env_int("TROCM_PREFILL_HG", 0);
@@ -556,6 +647,10 @@ int launch_sdpa_prefill_pp(const SdpaArgs &a, hipStream_t s) {
     p.k = (const _Float16 *)a.k;
     p.v = (const _Float16 *)a.v;
     p.kv_stride_b = a.kv_stride_b, p.kv_stride_h = a.kv_stride_h, p.kv_stride_t = a.kv_stride_t;
+    if (quant) {
+        p.k_scales = (const uint16_t *)a.k_scales, p.v_scales = (const uint16_t *)a.v_scales;
+        p.row_stride_b = a.kv_stride_b / a.D, p.row_stride_h = a.kv_stride_h / a.D;
+    }
     p.B = (int)a.B, p.Hq = (int)a.Hq, p.Hkv = (int)a.Hkv, p.Sq = (int)a.Sq, p.Sk = (int)a.Sk;
     p.causal = a.causal;
     p.scale_log2 = a.scale * 1.4426950408889634f;
@@ -596,7 +691,7 @@ int launch_sdpa_prefill_pp(const SdpaArgs &a, hipStream_t s) {
     }
     const int64_t wgs = wgs1 * ns;
     if (wgs >= (1ll << 31)) return 2;
-    return a.D == 128 ? launch_hg<128>(p, hg, wgs, s) : launch_hg<64>(p, hg, wgs, s);
+    return a.D == 128 ? launch_hg<128>(p, a.kv_fmt, hg, wgs, s) : launch_hg<64>(p, a.kv_fmt, hg, wgs, s);
 }
 
 }  // namespace trocm
