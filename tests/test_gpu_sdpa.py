@@ -480,6 +480,7 @@ def test_prefill_with_additive_mask(rt, kind, B, Hq, Hkv, Sq, Sk, D, mb, mh):
     (1, 32, 8, 128, (512, 512, 300)),     # chunked prefill into a quantised cache, key splits
     (2, 8, 2, 128, (100, 77, 33)), (1, 4, 4, 128, (64, 200)), (2, 6, 2, 128, (40, 130)),
     (1, 8, 2, 64, (96, 160)), (3, 16, 16, 64, (70,)),
+    (1, 8, 8, 128, (300, 5, 2)), (1, 6, 2, 128, (200, 9)),   # a few queries, one head per workgroup
 ])
 def test_prefill_over_a_quantised_cache(rt, fmt_name, B, Hq, Hkv, D, chunks):
     """Chunks of a prompt appended to a Q8_0 / Q4_0 cache (quantised on append), each attending causally

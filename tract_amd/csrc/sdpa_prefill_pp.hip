@@ -638,7 +638,8 @@ int launch_sdpa_prefill_pp(const SdpaArgs &a, hipStream_t s) {
     // the better kernel for a few queries over a long cache (speculative decoding, tiny chunks): the
     // K/V tiles are read once per kv head instead of once per query head (8 x 32 heads x 4 queries over
     // 8192 tokens: 66 us against 183 us).  With one head per workgroup short prompts go to the smaller kernel.
-    if (hg == 1 && a.Sq * 2 < n_qtiles * block_m) return 2;
+    // (Quantised caches have no smaller kernel: they stay here whatever the prompt length.)
+    if (hg == 1 && !quant && a.Sq * 2 < n_qtiles * block_m) return 2;
 
     PrefillPP p;
     memset(&p, 0, sizeof(p));
