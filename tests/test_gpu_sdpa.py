@@ -141,17 +141,16 @@ def test_decode_with_additive_mask(rt, kind, dt, B, Hq, Hkv, D, T, mb, mh):
     assert max_abs(got, cases.textbook_sdpa(q, k, v, mask)) <= (2e-3 if dt == np.float16 else 2e-5)
 
 
-@pytest.mark.parametrize("fmt_name", ["plain", "Q8_0", "Q4_0"])
-@pytest.mark.parametrize("dt,Hq,Hkv,D,T", [
-    (np.float16, 24, 8, 128, 1500), (np.float16, 14, 2, 128, 3000), (np.float16, 12, 2, 128, 700),
-    (np.float16, 10, 2, 128, 333), (np.float32, 6, 2, 64, 513), (np.float16, 21, 3, 64, 200),
-])
+_ODD_GROUPS = [(np.float16, 24, 8, 128, 1500), (np.float16, 14, 2, 128, 3000), (np.float16, 12, 2, 128, 700),
+               (np.float16, 10, 2, 128, 333), (np.float32, 6, 2, 64, 513), (np.float16, 21, 3, 64, 200)]
+
+
+@pytest.mark.parametrize("fmt_name,dt,Hq,Hkv,D,T", [("plain",) + c for c in _ODD_GROUPS] +
+                         [(f,) + c for f in ("Q8_0", "Q4_0") for c in _ODD_GROUPS if c[0] == np.float16 and c[3] == 128])
 def test_decode_group_sizes_that_are_not_powers_of_two(rt, fmt_name, dt, Hq, Hkv, D, T):
     """Group sizes 3, 5, 6, 7 (24q/8kv, 14q/2kv ... of current decoders) run on the split-K kernels of the
     next larger instantiated group size; prefill, fused decode steps, a masked step and the ragged
     form, each against the oracle."""
-    if fmt_name != "plain" and (dt != np.float16 or D != 128):
-        pytest.skip("quantised caches: f16 queries, head_dim 128")
     fmt = {"plain": None, "Q8_0": tract_amd.Q8_0, "Q4_0": tract_amd.Q4_0}[fmt_name]
     tol = TOL[np.dtype(dt)] if fmt is None else 2e-2
     rng = np.random.default_rng(300 + Hq + T)
