@@ -509,6 +509,26 @@ def test_prefill_over_a_quantised_cache(rt, fmt_name, B, Hq, Hkv, D, chunks):
     assert got_blocks.tobytes() == want_blocks.tobytes()
 
 
+def test_f32_prompt_through_the_f16_kernels_like_the_cuda_translator(rt):
+    """convert_sdpa_to_cuda_flash_attn (cuda/src/transform.rs:358-406) casts Q, K, V and the mask to f16
+    around its kernel and casts the result back: the same option on the Sdpa mirror, held to the f16
+    tolerance; without it an f32 prompt keeps f32 arithmetic (generic kernel) and the f32 tolerance."""
+    rng = np.random.default_rng(6000)
+    B, Hq, Hkv, Sq, Sk, D = 1, 8, 2, 96, 300, 128
+    q = (rng.standard_normal((B, Hq, Sq, D), dtype=np.float32) / np.sqrt(D)).astype(np.float32)
+    k = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32)
+    v = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32)
+    want = cases.textbook_sdpa(q, k, v, causal=True)
+    exact = tract_amd.Sdpa(is_causal=True).eval(q, k, v).to_numpy()
+    fast = tract_amd.Sdpa(is_causal=True, f16_flash_attention=True).eval(q, k, v).to_numpy()
+    assert exact.dtype == fast.dtype == np.float32
+    assert max_abs(exact, want) <= 2e-5
+    assert 2e-5 < max_abs(fast, want) <= 2e-2     # f16 arithmetic, as on the reference's GPU path
+    mask = (rng.standard_normal((1, 1, Sq, Sk), dtype=np.float32))
+    fast = tract_amd.Sdpa(f16_flash_attention=True).eval(q, k, v, mask).to_numpy()
+    assert max_abs(fast, cases.textbook_sdpa(q, k, v, mask)) <= 2e-2
+
+
 _PREFILL_ENV_CODE = """
 import os, sys, numpy as np
 import tract_amd

@@ -275,8 +275,14 @@ def _scale_arg(scale) -> float:
 class Sdpa:
     """Scaled dot-product attention on plain device tensors (sdpa.rs:83-89)."""
 
-    def __init__(self, scale=None, datum_type=np.float32, acc_datum_type=np.float32, is_causal=False):
+    def __init__(self, scale=None, datum_type=np.float32, acc_datum_type=np.float32, is_causal=False,
+                 f16_flash_attention=False):
+        """`f16_flash_attention=True` is what the reference's CUDA translator does to every Sdpa
+        (convert_sdpa_to_cuda_flash_attn, cuda/src/transform.rs:358-406): Q, K, V and the mask are cast
+        to f16, the f16 kernel runs, the output is cast back.  f32 inputs then take the MFMA kernels
+        (and the f16 tolerance) instead of the generic f32 kernel; off by default (CPU parity)."""
         self.scale, self.datum_type, self.acc_datum_type, self.is_causal = scale, datum_type, acc_datum_type, is_causal
+        self.f16_flash_attention = f16_flash_attention
         self._ws = None
 
     def output_facts(self, q_shape, k_shape, v_shape, mask_shape=None):
@@ -302,6 +308,18 @@ class Sdpa:
         _, Hkv, Sk, Dk = _canon4(k.shape)
         if _canon4(v.shape) != (B, Hkv, Sk, D) or Dk != D:
             raise TractRocmError("K/V shape mismatch")
+        if self.f16_flash_attention and q.dtype == np.float32:
+            half = Cast(np.float16)
+            inner = Sdpa(self.scale, np.float16, self.acc_datum_type, self.is_causal)
+            o16 = inner.eval(half.eval(q, stream), half.eval(k, stream), half.eval(v, stream),
+                             None if m is None else half.eval(m, stream), stream)
+            if out is None:
+                out = DeviceTensor(q.shape, np.float32)
+            elif tuple(out.shape) != tuple(q.shape) or out.dtype != np.float32:
+                raise TractRocmError("out must have Q's shape and datum type")
+            call("trocm_cast", o16.ptr, dtype_code(np.float16), out.ptr, dtype_code(np.float32),
+                 int(np.prod(q.shape, dtype=np.int64)), _sh(stream))
+            return out   # (the f16 temporaries are released by hipFree, which waits for the work that uses them)
         mb = mh = 1
         if m is not None:
             ms = _canon4(m.shape)
