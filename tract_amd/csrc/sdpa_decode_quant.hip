@@ -53,6 +53,22 @@ __device__ __forceinline__ int qrot(int row) {
     return CPR == 8 ? (row >> 1) : (row >> 2);
 }
 
+// Streaming (non-temporal) loads of the code planes: K and V are read once per launch, and keeping them
+// out of the caches' replacement order is worth 8-9 % of a decode launch.
+template <typename V>
+__device__ __forceinline__ V stream_load(const char *ptr);
+template <>
+__device__ __forceinline__ uint32_t stream_load<uint32_t>(const char *ptr) {
+    return __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(ptr));
+}
+template <>
+__device__ __forceinline__ uint2 stream_load<uint2>(const char *ptr) {
+    const uint64_t raw = __builtin_nontemporal_load(reinterpret_cast<const uint64_t *>(ptr));
+    uint2 v;
+    v.x = (uint32_t)raw, v.y = (uint32_t)(raw >> 32);
+    return v;
+}
+
 template <int FMT, int G>
 __global__ __launch_bounds__(kThreads, G <= 4 ? 2 : 1) void sdpa_decode_q_kernel(DecodeDev p) {
     typedef QTraits<FMT> Q;
@@ -129,7 +145,7 @@ __global__ __launch_bounds__(kThreads, G <= 4 ? 2 : 1) void sdpa_decode_q_kernel
         const char *base = kbase + (int64_t)t0 * RB;
         if (t0 + kTile <= p.T) {
 #pragma unroll
-            for (int j = 0; j < KL; j++) kreg[j] = *reinterpret_cast<const u32x4 *>(base + k_off[j]);
+            for (int j = 0; j < KL; j++) kreg[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + k_off[j]));
             ksreg = *reinterpret_cast<const uint32_t *>(ksbase + (int64_t)(t0 + qk_row) * SB + qk_half * 4);
         } else {
 #pragma unroll
@@ -146,7 +162,7 @@ __global__ __launch_bounds__(kThreads, G <= 4 ? 2 : 1) void sdpa_decode_q_kernel
 #pragma unroll
         for (int i = 0; i < VI; i++) {
             int tok = min(t0 + 4 * i + rg, last_tok);
-            vreg[i] = *reinterpret_cast<const vcode_t *>(vbase + (int64_t)tok * RB + j16 * (int)sizeof(vcode_t));
+            vreg[i] = stream_load<vcode_t>(vbase + (int64_t)tok * RB + j16 * (int)sizeof(vcode_t));
             vsreg[i] = *reinterpret_cast<const uint16_t *>(vsbase + (int64_t)tok * SB + vblk * 2);
         }
     };
