@@ -15,6 +15,24 @@ struct CopyDev {
     int64_t src_stride[6];  // bytes
 };
 
+// One element of BYTES bytes, read and written once: non-temporal accesses keep a large copy out of
+// the caches' replacement order.
+typedef uint32_t cp_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t cp_u32x2 __attribute__((ext_vector_type(2)));
+template <int BYTES>
+__device__ __forceinline__ void stream_copy(char *dst, const char *src) {
+    if constexpr (BYTES == 16)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(reinterpret_cast<const cp_u32x4 *>(src)), reinterpret_cast<cp_u32x4 *>(dst));
+    else if constexpr (BYTES == 8)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(reinterpret_cast<const cp_u32x2 *>(src)), reinterpret_cast<cp_u32x2 *>(dst));
+    else if constexpr (BYTES == 4)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(src)), reinterpret_cast<uint32_t *>(dst));
+    else if constexpr (BYTES == 2)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(reinterpret_cast<const uint16_t *>(src)), reinterpret_cast<uint16_t *>(dst));
+    else
+        __builtin_nontemporal_store(__builtin_nontemporal_load(reinterpret_cast<const uint8_t *>(src)), reinterpret_cast<uint8_t *>(dst));
+}
+
 template <typename V, typename Index>
 __global__ __launch_bounds__(256) void copy_nd_kernel(char *__restrict__ dst, const char *__restrict__ src,
                                                       CopyDev p, Index total) {
@@ -32,7 +50,7 @@ __global__ __launch_bounds__(256) void copy_nd_kernel(char *__restrict__ dst, co
                 soff += (int64_t)i * p.src_stride[d];
             }
         }
-        *reinterpret_cast<V *>(dst + doff) = *reinterpret_cast<const V *>(src + soff);
+        stream_copy<sizeof(V)>(dst + doff, src + soff);
     }
 }
 

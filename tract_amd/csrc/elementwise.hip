@@ -67,6 +67,25 @@ __global__ __launch_bounds__(256) void apply_rope_kernel(const T *__restrict__ x
     st(y + yo + (i + p.half) * p.out_s[3], hi);
 }
 
+// Streaming accesses for data that is read or written once: non-temporal loads and stores keep it out
+// of the caches' replacement order.
+typedef uint32_t nt_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t nt_u32x2 __attribute__((ext_vector_type(2)));
+template <int BYTES>
+__device__ __forceinline__ void stream_copy_in(void *regs, const void *src) {
+    if constexpr (BYTES == 16)
+        *reinterpret_cast<nt_u32x4 *>(regs) = __builtin_nontemporal_load(reinterpret_cast<const nt_u32x4 *>(src));
+    else
+        *reinterpret_cast<nt_u32x2 *>(regs) = __builtin_nontemporal_load(reinterpret_cast<const nt_u32x2 *>(src));
+}
+template <int BYTES>
+__device__ __forceinline__ void stream_copy_out(void *dst, const void *regs) {
+    if constexpr (BYTES == 16)
+        __builtin_nontemporal_store(*reinterpret_cast<const nt_u32x4 *>(regs), reinterpret_cast<nt_u32x4 *>(dst));
+    else
+        __builtin_nontemporal_store(*reinterpret_cast<const nt_u32x2 *>(regs), reinterpret_cast<nt_u32x2 *>(dst));
+}
+
 // The same with 16-byte accesses: one thread per VW consecutive rotation pairs (VW = 8 halfs or 4
 // floats).  Used when the innermost strides are 1 and everything is 16-byte aligned, which is every
 // layout an exported decoder produces; the scalar kernel above moved 1.4 TB/s on a prefill chunk.
@@ -87,8 +106,8 @@ __global__ __launch_bounds__(256) void apply_rope_vec_kernel(const T *__restrict
     const T *xr = x + i0 * p.in_s[0] + i1 * p.in_s[1] + i2 * p.in_s[2];
     T *yr = y + i0 * p.out_s[0] + i1 * p.out_s[1] + i2 * p.out_s[2];
     T a[VW], b[VW], c_lo[VW], s_lo[VW], c_hi[VW], s_hi[VW], lo[VW], hi[VW];
-    *reinterpret_cast<uint4 *>(a) = *reinterpret_cast<const uint4 *>(xr + i);
-    *reinterpret_cast<uint4 *>(b) = *reinterpret_cast<const uint4 *>(xr + i + p.half);
+    stream_copy_in<16>(a, xr + i);
+    stream_copy_in<16>(b, xr + i + p.half);
     if (!p.rotate_only) {
         const int64_t co = i0 * p.cs_s[0] + i1 * p.cs_s[1] + i2 * p.cs_s[2];
         *reinterpret_cast<uint4 *>(c_lo) = *reinterpret_cast<const uint4 *>(cs + co + i);
@@ -110,8 +129,8 @@ __global__ __launch_bounds__(256) void apply_rope_vec_kernel(const T *__restrict
         st(&lo[j], l);
         st(&hi[j], h);
     }
-    *reinterpret_cast<uint4 *>(yr + i) = *reinterpret_cast<const uint4 *>(lo);
-    *reinterpret_cast<uint4 *>(yr + i + p.half) = *reinterpret_cast<const uint4 *>(hi);
+    stream_copy_out<16>(yr + i, lo);
+    stream_copy_out<16>(yr + i + p.half, hi);
 }
 
 template <typename S, typename Dd>
@@ -120,15 +139,13 @@ __global__ __launch_bounds__(256) void cast_kernel(const S *__restrict__ src, Dd
     if (i + 4 <= n && ((uintptr_t)src % (4 * sizeof(S)) == 0) && ((uintptr_t)dst % (4 * sizeof(Dd)) == 0)) {
         S in[4];
         Dd out[4];
-        *reinterpret_cast<typename std::conditional<sizeof(S) == 4, uint4, uint2>::type *>(in) =
-            *reinterpret_cast<const typename std::conditional<sizeof(S) == 4, uint4, uint2>::type *>(src + i);
+        stream_copy_in<4 * sizeof(S)>(in, src + i);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             float f = ld(&in[j]);
             st(&out[j], f);   // f32 -> f16 rounds to nearest even; f16 -> f32 is exact
         }
-        *reinterpret_cast<typename std::conditional<sizeof(Dd) == 4, uint4, uint2>::type *>(dst + i) =
-            *reinterpret_cast<const typename std::conditional<sizeof(Dd) == 4, uint4, uint2>::type *>(out);
+        stream_copy_out<4 * sizeof(Dd)>(dst + i, out);
     } else {
         for (size_t j = i; j < n && j < i + 4; j++) st(dst + j, ld(src + j));
     }
