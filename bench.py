@@ -171,9 +171,15 @@ def cpu_baseline(B, budget_s=20.0):
 
 
 def time_calls(ta, fn, iters):
-    """Average microseconds of fn() over `iters` back-to-back calls (HIP events on the stream)."""
-    for _ in range(3):
+    """Average microseconds of fn() over `iters` back-to-back calls (HIP events on the stream), after
+    at least 3 calls and about 10 ms of untimed calls (the device's clocks settle)."""
+    t0 = time.perf_counter()
+    calls = 0
+    while calls < 3 or (time.perf_counter() - t0 < 0.010 and calls < 2000):
         fn()
+        calls += 1
+        if calls % 16 == 0:
+            ta.synchronize()
     ta.synchronize()
     e0, e1 = ta.Event(), ta.Event()
     e0.record()
