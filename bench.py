@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 
 HQ, HKV, D, CTX = 32, 8, 128, 8192
 LAYERS = 4
-PREWARM_LAUNCHES = 200   # untimed attention launches before the warm-up steps (clock ramp), see run_batch
+PREWARM_LAUNCHES = 1000   # untimed attention launches before the warm-up steps (clock ramp), see run_batch
 HBM_PEAK_GBS = 8000.0
 # HBM traffic of one decode-attention launch at the default arguments (batch 8, context 8226 in the
 # kernel loop), from two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE), each
