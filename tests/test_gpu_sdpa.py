@@ -191,6 +191,42 @@ def test_decode_group_sizes_that_are_not_powers_of_two(rt, fmt_name, dt, Hq, Hkv
             assert max_abs(got[b:b + 1], want) <= tol
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,D,T", [
+    (1, 64, 8, 128, 4097), (2, 64, 8, 128, 1000), (1, 128, 8, 128, 3000), (2, 16, 1, 128, 777), (1, 32, 1, 128, 2050),
+    (3, 40, 8, 64, 513), (1, 96, 8, 64, 1500), (2, 24, 2, 128, 31), (1, 64, 8, 128, 1), (8, 64, 8, 128, 300),
+    (1, 22, 2, 128, 640),
+])
+def test_decode_with_large_head_groups(rt, B, Hq, Hkv, D, T):
+    """8, 16 or up to 32 query heads per kv head (the 70B / 405B class of decoders): the heads are the rows
+    of MFMA tiles.  Over caches with spare capacity (NaN-filled tail), with and without key splits."""
+    rng = np.random.default_rng(7000 + Hq + T)
+    q = (rng.standard_normal((B, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    k = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(np.float16)
+    k[:, :, T // 2] *= 5.0   # an outlier key: the running maxima of waves and splits differ
+    st = tract_amd.InPlaceKvSdpa(axis=2, causal=True).state()
+    import ctypes as C
+    from tract_amd._lib import call
+    cap = T + 45
+    for c in (st.k, st.v):
+        c.reserve(cap, like=(k.shape, k.dtype))
+        data, pitch = C.c_void_p(), C.c_int64()
+        call("trocm_kv_cache_raw", c.handle, C.byref(data), None, C.byref(pitch))
+        call("trocm_memset", data, 0xFF, B * Hkv * pitch.value * D * 2, None)  # NaN fill
+    out = st.eval([q, k, v]).to_numpy()
+    assert not np.isnan(out).any()
+    assert max_abs(out, orc.flash_sdpa(q, k, v, causal=True, threads=8)) <= 2e-2
+    assert max_abs(out, cases.textbook_sdpa(q, k, v, causal=True)) <= 2e-3
+    # a decode step on top (explicit append, then the same kernel)
+    q1 = (rng.standard_normal((B, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    k1 = rng.standard_normal((B, Hkv, 1, D), dtype=np.float32).astype(np.float16)
+    v1 = rng.standard_normal((B, Hkv, 1, D), dtype=np.float32).astype(np.float16)
+    out = st.eval([q1, k1, v1]).to_numpy()
+    k2, v2 = np.concatenate([k, k1], axis=2), np.concatenate([v, v1], axis=2)
+    assert max_abs(out, cases.textbook_sdpa(q1, k2, v2)) <= 2e-3
+    assert st.k.valid_contiguous().tobytes() == k2.tobytes()
+
+
 @pytest.mark.parametrize("splits", [1, 2, 3, 7, 64])
 def test_decode_any_split_count_agrees(rt, splits, monkeypatch):
     # The split merge is exact in real arithmetic (log-sum-exp identity).

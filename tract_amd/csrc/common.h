@@ -132,6 +132,9 @@ struct SdpaArgs {
 int launch_sdpa_generic(const SdpaArgs &a, hipStream_t s);
 // Split-K decode (Sq == 1).  Returns 2 when the shape is not covered by a fast kernel.
 int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s);
+// Split-K decode for 2..32 query heads per kv head (f16): the heads are the rows of MFMA tiles.
+// Returns 2 when not covered (masks, other types).
+int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s);
 // Split-K decode over Q8_0 / Q4_0 caches with fused dequantisation.  Returns 2 when not covered.
 int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s);
 // MFMA prefill.  Returns 2 when the shape is not covered.

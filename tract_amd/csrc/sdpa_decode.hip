@@ -466,6 +466,10 @@ int choose_decode_splits(int64_t BH, int64_t G, int n_tiles, int wg_per_cu) {
 
 int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
     if (a.Sq != 1) return 2;
+    {   // large head groups: the MFMA formulation (it declines masks, the fused append and f32)
+        const int rc = launch_sdpa_decode_mfma(a, s);
+        if (rc != 2) return rc;
+    }
     if (a.kv_fmt != TROCM_F16 && a.kv_fmt != TROCM_F32) return 2;
     if (a.q_dtype != a.kv_fmt) return 2;
     if (a.D != 64 && a.D != 128) return 2;

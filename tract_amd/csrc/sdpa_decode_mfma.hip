@@ -1,0 +1,308 @@
+// Split-K flash-decode attention with grouped query heads (q_len == 1, 2..32 query heads per kv
+// head, f16): gfx950.
+//
+// The vector-ALU decode kernel (sdpa_decode.hip) spends one v_dot2 per (head, 2 features) and one fma
+// per (head, feature) of every token; with 8 heads per kv head that is about 970 vector instructions
+// per wave and 32-token tile, and the kernel is bound by them, not by HBM (batch 8, 8192 tokens:
+// 84.5 us against 47 us for 4 heads per kv head).  Here the G query heads of a kv head are the
+// *rows* of a 32-row MFMA tile: S^T = K.Q^T and O^T = V^T.P^T with v_mfma_f32_32x32x16_f16, the same
+// transposed formulation as the prefill kernel, with a head where that kernel has a query.  Only G
+// of the 32 rows are live, which the matrix pipe absorbs easily (16 MFMAs per 16 KiB of K and V);
+// what matters is that the vector work per tile drops to the softmax of 16 values per lane.
+//
+// Work decomposition: grid (splits, kv_heads, batch), 4 waves; wave w takes 32-token tiles w, w+4, ...
+// of its split.  Per tile: K rows global -> registers (one tile ahead, non-temporal) -> a wave-private
+// LDS tile -> A fragments; softmax in registers (a lane owns one head and 16 of the 32 tokens); V
+// rows the same way into the same LDS tile (K is dead by then) -> transposing LDS reads -> A
+// fragments of the second product.  Waves are merged through LDS, splits through the workspace: by the
+// last workgroup to arrive (up to 8 heads per kv head) or by the merge launch, both shared with the other
+// decode kernels.  A step's new token can be handed in and is stored to the cache by the kernel.
+//
+// Roofline: HBM-bound.  Algorithmic bytes as for sdpa_decode.hip.
+#include "decode_common.h"
+
+namespace trocm {
+namespace {
+
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef short short4_t __attribute__((ext_vector_type(4)));
+
+// Transposing 64-bit LDS load of 16-bit elements: in each block of 16 lanes, lane i receives
+// element i%4 of the four 8-byte rows addressed by lanes i/4, i/4+4, i/4+8, i/4+12.
+__device__ __forceinline__ half4_t lds_read_tr16(const _Float16 *lds_ptr) {
+    typedef __attribute__((address_space(3))) short4_t *lds_v4_ptr;
+    short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_ptr)(uintptr_t)(uint32_t)(uintptr_t)lds_ptr);
+    return __builtin_bit_cast(half4_t, r);
+}
+
+template <int D, int GP>
+__global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev p) {
+    constexpr int KS = D / 16;             // contraction steps of K.Q^T
+    constexpr int DB = D / 32;             // 32-feature blocks of the output
+    constexpr int KROW = D + 8;            // halfs per K row in LDS (128-bit reads of 16 rows hit distinct banks)
+    constexpr int VROW = D + 16;           // halfs per V row in LDS (rows of a transposing read 8 banks apart)
+    constexpr int CPR = D / 8;             // 16-byte chunks per row
+    constexpr int NLD = kTile * CPR / 64;  // 128-bit loads per lane, tile and tensor
+    constexpr int kCombStride = GP * D + 2 * GP;
+    constexpr int kTileBytes = kTile * VROW * 2;
+    constexpr int kLdsBytes = kWaves * (kTileBytes > kCombStride * 4 ? kTileBytes : kCombStride * 4);
+    __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kLdsBytes];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, hb = lane >> 5;
+    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    const int g = p.g_real;
+    _Float16 *tile = reinterpret_cast<_Float16 *>(lds_raw + w * kTileBytes);
+
+    const int64_t head0 = (int64_t)b * p.Hq + (int64_t)kvh * g;
+    const _Float16 *qrow = reinterpret_cast<const _Float16 *>(p.q) + (head0 + min(l32, g - 1)) * D;
+    const char *kbase = p.k + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+    const char *vbase = p.v + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+    const int T = p.T;
+    const int n_tiles = (T + kTile - 1) / kTile;
+    const int tile_begin = split * p.tiles_per_split, tile_end = min(n_tiles, tile_begin + p.tiles_per_split);
+
+    // this lane's chunks of a tile: chunk j*64 + lane = (row, 16-byte chunk of the row)
+    uint32_t g_off[NLD], k_slot[NLD], v_slot[NLD];
+#pragma unroll
+    for (int j = 0; j < NLD; j++) {
+        const int c = j * 64 + lane, row = c / CPR, dc = c % CPR;
+        g_off[j] = (uint32_t)row * (uint32_t)p.kv_stride_t + (uint32_t)dc * 16u;
+        k_slot[j] = row * KROW + dc * 8;
+        v_slot[j] = row * VROW + dc * 8;
+    }
+    u32x4 kpre[NLD], vpre[NLD];
+    // fused append: the row of token new_pos comes from the step's input and is stored to the cache on the way
+    const int new_pos = p.k_new ? p.new_pos : -1;
+    const int64_t new_row = ((int64_t)b * p.Hkv + kvh) * D * 2;
+    auto fetch = [&](const char *base0, const char *fresh, int t, u32x4 (&dst)[NLD]) {
+        const int t0 = t * kTile;
+        const char *base = base0 + (int64_t)t0 * p.kv_stride_t;
+        if (t0 + kTile <= T && !(new_pos >= t0 && new_pos < t0 + kTile)) {
+#pragma unroll
+            for (int j = 0; j < NLD; j++) dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + g_off[j]));
+        } else {   // the sequence's last tile (rows past the end repeat the last token, masked below) or the new token's
+#pragma unroll
+            for (int j = 0; j < NLD; j++) {
+                const int c = j * 64 + lane, row = min(c / CPR, T - 1 - t0), dc = c % CPR;
+                const char *cache_ptr = base + (uint32_t)row * (uint32_t)p.kv_stride_t + (uint32_t)dc * 16u;
+                const bool is_new = t0 + row == new_pos;
+                dst[j] = *reinterpret_cast<const u32x4 *>(is_new ? fresh + new_row + dc * 16 : cache_ptr);
+                if (is_new && c / CPR == new_pos - t0) *reinterpret_cast<u32x4 *>(const_cast<char *>(cache_ptr)) = dst[j];
+            }
+        }
+    };
+
+    int t = tile_begin + w;
+    if (t < tile_end) {
+        fetch(kbase, p.k_new, t, kpre);
+        fetch(vbase, p.v_new, t, vpre);
+    }
+    // Q^T fragments: row (head) = lane % 32, features 16*ks + 8*hb .. +8
+    half8_t qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = *reinterpret_cast<const half8_t *>(qrow + 16 * ks + 8 * hb);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) asm volatile("" : "+v"(qf[ks]));   // settled here, not at first use inside the loop
+
+    float m_run = -INFINITY, l_run = 0.0f;   // log2 domain, already scaled
+    float16_t o[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
+
+    // this lane as a SOURCE of the transposing loads: key row (lane%16)/4 of a group of four, features
+    // 16*(lane/16 % 2) + 4*(lane%4) of the 32-feature block
+    const int vsrc_off = (4 * hb + ((lane & 15) >> 2)) * VROW + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+    for (; t < tile_end; t += kWaves) {
+        const int t0 = t * kTile;
+        const bool more = t + kWaves < tile_end;
+        // ---- K tile -> LDS, the next tile's K into flight ----------------------------------------------
+#pragma unroll
+        for (int j = 0; j < NLD; j++) *reinterpret_cast<u32x4 *>(tile + k_slot[j]) = kpre[j];
+        if (more) fetch(kbase, p.k_new, t + kWaves, kpre);
+        // ---- S^T = K Q^T: 32 tokens x 32 rows ------------------------------------------------------------
+        float16_t s;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = 0.0f;
+        const _Float16 *kt = tile + l32 * KROW + 8 * hb;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const half8_t kf = *reinterpret_cast<const half8_t *>(kt + 16 * ks);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s, 0, 0, 0);
+        }
+        // ---- online softmax of this lane's head over its 16 tokens: token = t0 + 8*(r/4) + 4*hb + r%4 ----
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int tok = t0 + 8 * (r >> 2) + 4 * hb + (r & 3);
+            s[r] = (t0 + kTile <= T || tok < T) ? s[r] * p.scale_log2 : -INFINITY;
+            tmax = fmaxf(tmax, s[r]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m_run, tmax);   // finite: every tile holds at least one valid token
+        float psum = 0.0f;
+        half8_t pf[2];
+#pragma unroll
+        for (int st = 0; st < 2; st++)
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float pv = fast_exp2(s[8 * st + i] - m_new);
+                psum += pv;
+                pf[st][i] = (_Float16)pv;
+            }
+        const bool moved = m_new != m_run;
+        const float alpha = fast_exp2(m_run - m_new);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[db][r] *= alpha;
+        }
+        // ---- V tile -> the same LDS tile (every K fragment has been consumed), next V into flight ------
+#pragma unroll
+        for (int j = 0; j < NLD; j++) *reinterpret_cast<u32x4 *>(tile + v_slot[j]) = vpre[j];
+        if (more) fetch(vbase, p.v_new, t + kWaves, vpre);
+        // ---- O^T += V^T P^T ---------------------------------------------------------------------------------
+        const _Float16 *vsrc = tile + vsrc_off;
+#pragma unroll
+        for (int st = 0; st < 2; st++)
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+                const half4_t lo = lds_read_tr16(vsrc + (16 * st) * VROW + 32 * db);      // tokens 16st + 4hb + 0..3
+                const half4_t hi = lds_read_tr16(vsrc + (16 * st + 8) * VROW + 32 * db);  // tokens 16st + 8 + 4hb + 0..3
+                const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[st], o[db], 0, 0, 0);
+            }
+    }
+    l_run += __shfl_xor(l_run, 32, 64);
+
+    // ---- merge the 4 waves through LDS (the K/V tiles are dead) --------------------------------------------
+    __syncthreads();
+    float *comb = reinterpret_cast<float *>(lds_raw);   // [kWaves][GP*D + 2*GP]
+    if (l32 < GP) {
+        float *cw = comb + w * kCombStride;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int rq = 0; rq < 4; rq++) {
+                float4_t f4 = {o[db][4 * rq], o[db][4 * rq + 1], o[db][4 * rq + 2], o[db][4 * rq + 3]};
+                *reinterpret_cast<float4_t *>(cw + l32 * D + 32 * db + 8 * rq + 4 * hb) = f4;
+            }
+        if (hb == 0) {
+            cw[GP * D + l32] = m_run;
+            cw[GP * D + GP + l32] = l_run;
+        }
+    }
+    __syncthreads();
+    __half *out = reinterpret_cast<__half *>(p.out) + head0 * D;
+    const int64_t slot = ((int64_t)b * p.Hkv + kvh) * p.nsplit + split;
+    for (int idx = tid; idx < GP * D; idx += kThreads) {
+        const int h = idx / D;
+        float mm = -INFINITY;
+#pragma unroll
+        for (int ww = 0; ww < kWaves; ww++) mm = fmaxf(mm, comb[ww * kCombStride + GP * D + h]);
+        const float mm_ref = mm == -INFINITY ? 0.0f : mm;   // a wave without tiles holds (0, -inf, 0)
+        float acc = 0.0f, ll = 0.0f;
+#pragma unroll
+        for (int ww = 0; ww < kWaves; ww++) {
+            const float f = fast_exp2(comb[ww * kCombStride + GP * D + h] - mm_ref);
+            acc += comb[ww * kCombStride + idx] * f;
+            ll += comb[ww * kCombStride + GP * D + GP + h] * f;
+        }
+        if (p.nsplit == 1) {
+            if (h < g) out[idx] = __float2half_rn(acc / ll);
+        } else if (p.counters == nullptr) {
+            p.part_o[slot * (GP * D) + idx] = acc;
+            if ((idx % D) == 0) {
+                p.part_ml[slot * (2 * GP) + h] = mm;
+                p.part_ml[slot * (2 * GP) + GP + h] = ll;
+            }
+        } else {   // write-through stores: visible device-wide when they complete (see tail_merge)
+            __hip_atomic_store(&p.part_o[slot * (GP * D) + idx], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((idx % D) == 0) {
+                __hip_atomic_store(&p.part_ml[slot * (2 * GP) + h], mm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&p.part_ml[slot * (2 * GP) + GP + h], ll, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+    if constexpr (GP <= 8) {   // (larger groups: the merge launch; the in-kernel merge would need too many registers)
+        if (p.nsplit > 1 && p.counters != nullptr) {
+            const int64_t bh = (int64_t)b * p.Hkv + kvh;
+            tail_merge<__half, D, GP>(p, p.counters + bh, p.nsplit, bh * p.nsplit, 1, out, tid);
+        }
+    }
+}
+
+template <int D, int GP>
+int launch_gp(const DecodeDev &p, dim3 grid, hipStream_t s) {
+    hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, GP>), grid, dim3(kThreads), 0, s, p);
+    if (p.nsplit > 1 && p.counters == nullptr)
+        hipLaunchKernelGGL((sdpa_decode_merge_kernel<__half, D, GP>), dim3(grid.y, grid.z, p.g_real), dim3(D), 0, s, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("sdpa_decode (mfma) launch failed: %s", hipGetErrorString(e));
+    return 0;
+}
+
+template <int D>
+int launch_d(const DecodeDev &p, int gp, dim3 grid, hipStream_t s) {
+    switch (gp) {
+        case 8: return launch_gp<D, 8>(p, grid, s);
+        case 16: return launch_gp<D, 16>(p, grid, s);
+        default: return launch_gp<D, 32>(p, grid, s);
+    }
+}
+
+}  // namespace
+
+int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {
+    if (a.Sq != 1 || a.mask != nullptr) return 2;
+    if (a.kv_fmt != TROCM_F16 || a.q_dtype != TROCM_F16) return 2;
+    if (a.D != 64 && a.D != 128) return 2;
+    if (a.Hq % a.Hkv) return 2;
+    const int64_t g_real = a.Hq / a.Hkv;
+    // One head per kv head is faster on the vector-ALU kernel (batch 8, 8226 tokens: 43.4 against 47.4 us);
+    // from two heads on this one is (4 heads: 47.5 against 48.6 us with a merge launch still in it, batch 32
+    // 157 against 162 us; 8 heads: 47 against 84 us).
+    static const int min_group = getenv("TROCM_DECODE_MFMA_MIN_GROUP") ? atoi(getenv("TROCM_DECODE_MFMA_MIN_GROUP")) : 2;
+    if (g_real < min_group || g_real > 32) return 2;
+    const int gp = g_real <= 8 ? 8 : g_real <= 16 ? 16 : 32;
+    if ((a.kv_stride_b * 2) % 16 || (a.kv_stride_h * 2) % 16 || (a.kv_stride_t * 2) % 16) return 2;
+    if ((uintptr_t)a.k % 16 || (uintptr_t)a.v % 16 || (uintptr_t)a.q % 16) return 2;
+    if (a.Sk <= 0 || a.Sk > (1ll << 30) || a.kv_stride_t * 2 * kTile >= (1ll << 31)) return 2;
+    if (a.B > 65535 || a.Hkv > 65535) return 2;
+    const int64_t BH = a.B * a.Hkv;
+    const int n_tiles = (int)((a.Sk + kTile - 1) / kTile);
+    int nsplit = choose_decode_splits(BH, gp, n_tiles, 1);
+    const int tps = (n_tiles + nsplit - 1) / nsplit;
+    nsplit = (n_tiles + tps - 1) / tps;
+    if (nsplit > 1) {
+        TROCM_NOT_NULL(a.workspace);
+        const size_t need = kWsCounterBytes + (size_t)BH * nsplit * gp * (a.D + 2) * sizeof(float);
+        TROCM_REQUIRE(a.workspace_bytes >= need, "sdpa workspace too small: %zu bytes given, %zu needed", a.workspace_bytes, need);
+    }
+    DecodeDev p;
+    memset(&p, 0, sizeof(p));
+    p.q = (const char *)a.q, p.out = (char *)a.out, p.k = (const char *)a.k, p.v = (const char *)a.v;
+    p.kv_stride_b = a.kv_stride_b * 2, p.kv_stride_h = a.kv_stride_h * 2, p.kv_stride_t = a.kv_stride_t * 2;
+    p.T = (int)a.Sk;
+    p.tiles_per_split = tps, p.nsplit = nsplit;
+    p.Hq = (int)a.Hq, p.Hkv = (int)a.Hkv, p.g_real = (int)g_real;
+    p.scale_log2 = a.scale * 1.4426950408889634f;
+    p.k_new = (const char *)a.k_new, p.v_new = (const char *)a.v_new;
+    p.new_pos = a.new_pos >= 0 ? (int)a.new_pos : (int)a.Sk - 1;
+    if (p.k_new && (p.v_new == nullptr || (uintptr_t)p.k_new % 16 || (uintptr_t)p.v_new % 16)) return 2;
+    p.part_ml = (float *)((char *)a.workspace + kWsCounterBytes);
+    p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * gp;
+    static const int tail = getenv("TROCM_DECODE_TAIL_MERGE") ? atoi(getenv("TROCM_DECODE_TAIL_MERGE")) : 1;
+    if (tail && gp <= 8 && nsplit > 1 && nsplit <= kTailMergeMax && BH <= (int64_t)(kWsCounterBytes / sizeof(int))) p.counters = (int *)a.workspace;
+    dim3 grid(nsplit, (unsigned)a.Hkv, (unsigned)a.B);
+    return a.D == 128 ? launch_d<128>(p, gp, grid, s) : launch_d<64>(p, gp, grid, s);
+}
+
+}  // namespace trocm
