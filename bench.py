@@ -347,7 +347,7 @@ def run_cfg5(ta, args):
     tot = int(sum(c.len() for c in kcs))
     by = 2 * HKV * D * 2 * tot + 2 * n_seq * HQ * D * 2 + 2 * n_seq * HKV * D * 2
     us_k = time_calls(ta, lambda: ta.sdpa_decode_ragged(qs[0], kcs, vcs, workspace=ws, out=out), 20)
-    roof = {"bound": "hbm", "kernel": "sdpa_decode_ragged_kernel<f16,128,4>", "achieved": round(by / us_k / 1e3, 1),
+    roof = {"bound": "hbm", "kernel": "sdpa_decode_mfma_ragged_kernel<128,8>", "achieved": round(by / us_k / 1e3, 1),
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(by / us_k / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
             "kernel_us": round(us_k, 2), "algorithmic_bytes_per_launch": int(by)}
     st = pool.stats()
@@ -558,7 +558,7 @@ def main():
         "parity_max_abs_vs_oracle": err,
         "roofline": {
             "bound": "hbm",
-            "kernel": "sdpa_decode_kernel<f16,128,4>",
+            "kernel": "sdpa_decode_mfma_kernel<128,8>",
             "achieved": round(main_res["kernel_gbs"], 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",

@@ -379,6 +379,38 @@ def test_ragged_decode_many_sequences(rt, dt, Hq, Hkv, D, n_seq, lo, hi):
             ks[i], vs[i] = np.concatenate([ks[i], kn], axis=2), np.concatenate([vs[i], vn], axis=2)
 
 
+def test_one_workspace_shared_by_ragged_and_dense_calls(rt):
+    """A ragged call keeps its launch plan in the workspace; a dense decode that follows on the same
+    workspace counts workgroup arrivals there.  Neither may disturb the other, in either order."""
+    rng = np.random.default_rng(404)
+    Hq, Hkv, D, B, T = 32, 8, 128, 4, 2100
+    lens = [700, 2100, 1300, 4000, 64, 900]
+    kcs, vcs, ks = [], [], []
+    for n in lens:
+        k = rng.standard_normal((1, Hkv, n, D), dtype=np.float32).astype(np.float16)
+        kc, vc = tract_amd.InPlaceKvCache(2), tract_amd.InPlaceKvCache(2)
+        kc.push(k), vc.push(k)
+        kcs.append(kc), vcs.append(vc), ks.append(k)
+    kd = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(np.float16)
+    st = tract_amd.InPlaceKvSdpa(axis=2, causal=True).state()
+    st.k.push(kd), st.v.push(kd)
+    ws = tract_amd.Workspace(max(B, len(lens)), Hq, 1, D)
+    qr = (rng.standard_normal((len(lens), Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    qd = (rng.standard_normal((B, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    want_d = orc.flash_sdpa(qd, kd, kd, causal=True)
+    from tract_amd._lib import call
+    from tract_amd.runtime import dtype_code
+    qd_dev, out_d = tract_amd.DeviceTensor.from_numpy(qd), tract_amd.DeviceTensor(qd.shape, np.float16)
+    for turn in range(3):
+        got_r = tract_amd.sdpa_decode_ragged(tract_amd.DeviceTensor.from_numpy(qr), kcs, vcs, workspace=ws).to_numpy()
+        call("trocm_sdpa_cached", qd_dev.ptr, dtype_code(np.float16), Hq, 1, st.k.handle, st.v.handle, out_d.ptr,
+             float("nan"), 1, ws.ptr, ws.nbytes, None)
+        got_d = out_d.to_numpy()
+        assert max_abs(got_d, want_d) <= 2e-2, f"dense after ragged, turn {turn}"
+        for i in range(len(lens)):
+            assert max_abs(got_r[i:i + 1], orc.flash_sdpa(qr[i:i + 1], ks[i], ks[i], causal=True)) <= 2e-2, f"ragged, turn {turn}, sequence {i}"
+
+
 def test_ragged_equals_padded_batch_with_mask(rt):
     """The reference's statement of a ragged batch: a dense batch padded to the longest
     sequence with an additive mask whose padded columns are <= -65504 (flash_sdpa.rs:261-268)."""

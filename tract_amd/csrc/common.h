@@ -155,8 +155,11 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
                               int64_t Hkv, int64_t D, const RaggedSeq *seqs, float scale, void *workspace,
                               size_t workspace_bytes, const void *k_new, const void *v_new, hipStream_t s);
 
-// Workspace layout: [counters: kWsCounters ints][partials ...]
+// Workspace layout: [arrival counters][partials ...]; a ragged launch keeps its plan (work items and
+// per-sequence slot ranges) between the two, so that the counters stay zero for whichever launch comes next:
+// [arrival counters][plan][partials ...].
 constexpr size_t kWsCounterBytes = 64 * 1024;   // 16384 arrival counters
+constexpr size_t kWsPlanBytes = 64 * 1024;      // about 1100 work items
 size_t decode_workspace_bytes(int64_t B, int64_t Hq, int64_t D);
 
 }  // namespace trocm

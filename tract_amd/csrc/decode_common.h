@@ -7,18 +7,6 @@
 #include "common.h"
 
 namespace trocm {
-namespace {
-
-constexpr int kWaves = 4;
-constexpr int kThreads = kWaves * 64;
-constexpr int kTile = 32;
-
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-typedef float float4_t __attribute__((ext_vector_type(4)));
-typedef float float8_t __attribute__((ext_vector_type(8)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 struct DecodeDev {
     const char *q;
@@ -61,6 +49,19 @@ struct RaggedItem {
 struct RaggedSeqSlots {
     int slot0, nsplit;
 };
+
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+constexpr int kTile = 32;
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_f(float x) {
@@ -241,10 +242,26 @@ __global__ __launch_bounds__(D) void sdpa_decode_merge_kernel(DecodeDev p) {
     merge_head<T, D, G>(p, bh * p.nsplit, 1, p.nsplit, h, out, threadIdx.x);
 }
 
+// Merge launch of the ragged batch: grid (kv_heads, sequences, G), D threads.
+template <typename T, int D, int G>
+__global__ __launch_bounds__(D) void sdpa_decode_ragged_merge_kernel(DecodeDev p, const RaggedSeqSlots *__restrict__ seqs) {
+    const int kvh = blockIdx.x, seq = blockIdx.y, h = blockIdx.z;
+    const RaggedSeqSlots ss = seqs[seq];
+    if (ss.nsplit <= 1) return;
+    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)seq * p.Hq + (int64_t)kvh * p.g_real + h) * D;
+    merge_head<T, D, G>(p, (int64_t)ss.slot0 * p.Hkv + kvh, p.Hkv, ss.nsplit, h, out, threadIdx.x);
+}
+
 }  // namespace
 
+// The MFMA formulation of the ragged launch (sdpa_decode_mfma.hip); gp = its padded group size (8, 16, 32),
+// which is also the stride of the partial records.
+int decode_mfma_group(int64_t g_real);   // 0: not taken by the MFMA formulation
+int launch_sdpa_decode_ragged_mfma(const DecodeDev &p, int gp, int64_t D, const RaggedItem *items, int n_items,
+                                   const RaggedSeqSlots *seqs, int n_seq, bool any_split, hipStream_t s);
+
 // Partials: at most kMaxSplitRows rows of (D + 2) floats per query head.
-constexpr int64_t kMaxSplitRows = 8192;
+constexpr int64_t kMaxSplitRows = 32768;
 int choose_decode_splits(int64_t BH, int64_t G, int n_tiles, int wg_per_cu);
 
 }  // namespace trocm

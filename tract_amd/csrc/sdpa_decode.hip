@@ -29,6 +29,7 @@
 //
 // Roofline: HBM-bound.  Algorithmic bytes per launch = 2*B*Hkv*T*D*e (K and V once per KV
 // head) + Q read + O write.
+#include <algorithm>
 #include "decode_common.h"
 
 namespace trocm {
@@ -405,16 +406,6 @@ __global__ __launch_bounds__(kThreads, (D * sizeof(T) <= 256 && G <= 4) ? 2 : 1)
     decode_body<T, D, G, false>(p, wk);
 }
 
-// Merge launch of the ragged batch: grid (kv_heads, sequences, G), D threads.
-template <typename T, int D, int G>
-__global__ __launch_bounds__(D) void sdpa_decode_ragged_merge_kernel(DecodeDev p, const RaggedSeqSlots *__restrict__ seqs) {
-    const int kvh = blockIdx.x, seq = blockIdx.y, h = blockIdx.z;
-    const RaggedSeqSlots ss = seqs[seq];
-    if (ss.nsplit <= 1) return;
-    T *out = reinterpret_cast<T *>(p.out) + ((int64_t)seq * p.Hq + (int64_t)kvh * p.g_real + h) * D;
-    merge_head<T, D, G>(p, (int64_t)ss.slot0 * p.Hkv + kvh, p.Hkv, ss.nsplit, h, out, threadIdx.x);
-}
-
 template <typename T, int D, int G>
 void launch_both(const DecodeDev &p, dim3 grid, hipStream_t s) {
     if (p.mask)
@@ -443,7 +434,7 @@ int launch_g(const DecodeDev &p, int G, dim3 grid, hipStream_t s) {
 
 size_t decode_workspace_bytes(int64_t B, int64_t Hq, int64_t D) {
     int64_t rows = B * Hq > kMaxSplitRows ? B * Hq : kMaxSplitRows;
-    return kWsCounterBytes + (size_t)rows * (size_t)(D + 2) * sizeof(float) + 256;
+    return kWsCounterBytes + kWsPlanBytes + (size_t)rows * (size_t)(D + 2) * sizeof(float) + 256;
 }
 
 // Number of splits.  Measured on MI355X (8k context, f16, G=4): one workgroup per compute
@@ -545,13 +536,21 @@ namespace {
 
 // Pinned staging for the per-call plan of a ragged launch (a few KiB): a small ring per host
 // thread, each slot guarded by an event so that a slot is not rewritten while its copy is
-// still in flight.
+// still in flight.  A kernel copies the plan into the workspace: a copy command between two
+// kernels of one stream hands the stream to a DMA engine and back, which left the device idle for
+// 27..49 us per step (64 sequences, 16 KiB of plan); the copy kernel reads the pinned pages itself.
 constexpr int kStageSlots = 4;
 struct StageSlot {
     void *host = nullptr;
+    void *host_dev = nullptr;   // the same pages as the device addresses them
     hipEvent_t done = nullptr;
     bool in_flight = false;
 };
+
+__global__ __launch_bounds__(256) void plan_upload_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int n16) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n16) dst[i] = src[i];
+}
 thread_local StageSlot g_stage[kStageSlots];
 thread_local int g_stage_next = 0;
 
@@ -559,7 +558,8 @@ int acquire_stage(StageSlot **out) {
     StageSlot &sl = g_stage[g_stage_next];
     g_stage_next = (g_stage_next + 1) % kStageSlots;
     if (!sl.host) {
-        TROCM_HIP(hipHostMalloc(&sl.host, kWsCounterBytes, hipHostMallocDefault));
+        TROCM_HIP(hipHostMalloc(&sl.host, kWsPlanBytes, hipHostMallocMapped));
+        TROCM_HIP(hipHostGetDevicePointer(&sl.host_dev, sl.host, 0));
         TROCM_HIP(hipEventCreateWithFlags(&sl.done, hipEventDisableTiming));
     } else if (sl.in_flight) {
         TROCM_HIP(hipEventSynchronize(sl.done));
@@ -626,10 +626,11 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
                               int64_t D, const RaggedSeq *seqs, float scale, void *workspace, size_t workspace_bytes,
                               const void *k_new, const void *v_new, hipStream_t s) {
     const int64_t g_real = Hq / Hkv;
-    const int64_t G = g_real <= 2 ? g_real : g_real <= 4 ? 4 : 8;   // the instantiation that runs it
+    const int mfma_gp = kv_fmt == TROCM_F16 ? decode_mfma_group(g_real) : 0;   // f16 with grouped heads: the MFMA formulation
+    const int64_t G = mfma_gp ? mfma_gp : g_real <= 2 ? g_real : g_real <= 4 ? 4 : 8;   // the instantiation that runs it
     const size_t es = elem_bytes(kv_fmt);
     bool fast = (kv_fmt == TROCM_F16 || kv_fmt == TROCM_F32) && q_dtype == kv_fmt && (D == 64 || D == 128) &&
-                g_real >= 1 && g_real <= 8 && workspace != nullptr && (uintptr_t)q % 16 == 0 &&
+                g_real >= 1 && (g_real <= 8 || mfma_gp) && workspace != nullptr && (uintptr_t)q % 16 == 0 &&
                 n_seq <= 2048 && Hkv <= 65535;
     for (int64_t i = 0; i < n_seq && fast; i++)
         fast = (uintptr_t)seqs[i].k % 16 == 0 && (uintptr_t)seqs[i].v % 16 == 0 && seqs[i].len < (1ll << 30) &&
@@ -643,14 +644,21 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     // ---- plan ----------------------------------------------------------------------------------
     int64_t total_tiles = 0;
     for (int64_t i = 0; i < n_seq; i++) total_tiles += (seqs[i].len + kTile - 1) / kTile;
-    const int64_t rows_cap = (int64_t)((workspace_bytes - kWsCounterBytes) / ((D + 2) * sizeof(float)));
+    TROCM_REQUIRE(workspace_bytes > kWsCounterBytes + kWsPlanBytes, "sdpa workspace too small for a ragged launch (%zu bytes)",
+                  workspace_bytes);
+    const int64_t rows_cap = (int64_t)((workspace_bytes - kWsCounterBytes - kWsPlanBytes) / ((D + 2) * sizeof(float)));
     const int64_t max_items_ws = rows_cap / (Hkv * G);  // every item may need a partial record per (padded) q head
     const int64_t max_items_tbl =
-        ((int64_t)kWsCounterBytes - n_seq * (int64_t)sizeof(RaggedSeqSlots)) / (int64_t)sizeof(RaggedItem);
+        ((int64_t)kWsPlanBytes - n_seq * (int64_t)sizeof(RaggedSeqSlots)) / (int64_t)sizeof(RaggedItem);
     const int64_t max_items = max_items_ws < max_items_tbl ? max_items_ws : max_items_tbl;
-    TROCM_REQUIRE(workspace_bytes > kWsCounterBytes && max_items >= n_seq,
+    TROCM_REQUIRE(max_items >= n_seq,
                   "sdpa workspace too small for %lld sequences (%zu bytes)", (long long)n_seq, workspace_bytes);
-    int64_t tiles_per_item = (total_tiles + num_compute_units() - 1) / num_compute_units();
+    // Workgroups (items x kv heads) per compute unit: two are resident at a time, and the last round of
+    // them is only partly full, so more and smaller items shorten the tail at the cost of partial records.
+    static const int wg_per_cu = getenv("TROCM_RAGGED_WG_PER_CU") ? atoi(getenv("TROCM_RAGGED_WG_PER_CU")) : 0;
+    int64_t want_items = wg_per_cu > 0 ? ((int64_t)num_compute_units() * wg_per_cu + Hkv - 1) / Hkv : num_compute_units();
+    if (want_items < 1) want_items = 1;
+    int64_t tiles_per_item = (total_tiles + want_items - 1) / want_items;
     if (tiles_per_item < kWaves) tiles_per_item = kWaves;
     int64_t n_items = 0;
     for (;;) {
@@ -668,6 +676,7 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     RaggedSeqSlots *slots = (RaggedSeqSlots *)(items + n_items);
     int64_t it = 0;
     bool any_split = false;
+    int64_t max_split = 1;
     for (int64_t i = 0; i < n_seq; i++) {
         int64_t tiles = (seqs[i].len + kTile - 1) / kTile;
         int64_t ns = (tiles + tiles_per_item - 1) / tiles_per_item;
@@ -676,6 +685,7 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
         slots[i].slot0 = (int)it;
         slots[i].nsplit = (int)ns;
         any_split |= ns > 1;
+        if (ns > max_split) max_split = ns;
         for (int64_t sp = 0; sp < ns; sp++, it++) {
             RaggedItem &r = items[it];
             r.k = (const char *)seqs[i].k;
@@ -688,11 +698,21 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
         }
     }
     n_items = it;
+    // Longest items first: the workgroups that start last, when the device is no longer full, are the short ones.
+    // (An item carries its own partial slot, so the order is free.)
+    std::stable_sort(items, items + n_items, [](const RaggedItem &a, const RaggedItem &b) {
+        return a.tile_end - a.tile_begin > b.tile_end - b.tile_begin;
+    });
     // the seq table sits right after the items actually emitted
     RaggedSeqSlots *slots_packed = (RaggedSeqSlots *)(items + n_items);
     if (slots_packed != slots) memmove(slots_packed, slots, (size_t)n_seq * sizeof(RaggedSeqSlots));
     size_t plan_bytes = (size_t)n_items * sizeof(RaggedItem) + (size_t)n_seq * sizeof(RaggedSeqSlots);
-    TROCM_HIP(hipMemcpyAsync(workspace, stage->host, plan_bytes, hipMemcpyHostToDevice, s));
+    {
+        const int n16 = (int)((plan_bytes + 15) / 16);   // the slot and the plan area are both kWsPlanBytes long
+        hipLaunchKernelGGL(plan_upload_kernel, dim3((n16 + 255) / 256), dim3(256), 0, s, (const uint4 *)stage->host_dev,
+                           (uint4 *)((char *)workspace + kWsCounterBytes), n16);
+        TROCM_HIP(hipGetLastError());
+    }
     TROCM_HIP(hipEventRecord(stage->done, s));
     stage->in_flight = true;
 
@@ -707,10 +727,16 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     p.scale_log2 = scale * 1.4426950408889634f;
     p.k_new = (const char *)k_new;
     p.v_new = (const char *)v_new;
-    p.part_ml = (float *)((char *)workspace + kWsCounterBytes);
+    p.part_ml = (float *)((char *)workspace + kWsCounterBytes + kWsPlanBytes);
     p.part_o = p.part_ml + (size_t)n_items * Hkv * 2 * G;
-    const RaggedItem *d_items = (const RaggedItem *)workspace;
+    const RaggedItem *d_items = (const RaggedItem *)((char *)workspace + kWsCounterBytes);
     const RaggedSeqSlots *d_slots = (const RaggedSeqSlots *)(d_items + n_items);
+    // The MFMA kernel merges the splits of a sequence-head itself when none has more than it can hold in registers.
+    static const int tail = getenv("TROCM_DECODE_TAIL_MERGE") ? atoi(getenv("TROCM_DECODE_TAIL_MERGE")) : 1;
+    if (tail && mfma_gp && mfma_gp <= 8 && any_split && max_split <= kTailMergeMax &&
+        n_seq * Hkv <= (int64_t)(kWsCounterBytes / sizeof(int)))
+        p.counters = (int *)workspace;
+    if (mfma_gp) return launch_sdpa_decode_ragged_mfma(p, mfma_gp, D, d_items, (int)n_items, d_slots, (int)n_seq, any_split, s);
     if (kv_fmt == TROCM_F16)
         return D == 128 ? launch_ragged_g<__half, 128>(p, (int)G, d_items, (int)n_items, d_slots, (int)n_seq, any_split, s)
                         : launch_ragged_g<__half, 64>(p, (int)G, d_items, (int)n_items, d_slots, (int)n_seq, any_split, s);

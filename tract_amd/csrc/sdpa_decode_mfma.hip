@@ -35,8 +35,20 @@ __device__ __forceinline__ half4_t lds_read_tr16(const _Float16 *lds_ptr) {
     return __builtin_bit_cast(half4_t, r);
 }
 
+// What one workgroup has to do: a tile range of one (sequence, kv head), and where its result goes.
+struct MfmaWork {
+    int seq, kvh;                 // the sequence (batch entry) and kv head
+    const char *kbase, *vbase;    // K and V rows of this (sequence, kv head)
+    int T, tile_begin, tile_end;
+    int nsplit;                   // splits of this sequence-head (1: write the output rows)
+    int64_t slot;                 // partial record of this workgroup
+    int new_pos;                  // token stored by a fused append (-1: none)
+    int *counter;                 // in-kernel merge by the last workgroup to arrive (dense batches, GP <= 8)
+    int64_t part_first, part_stride;   // partial records of this sequence-head: first, first + stride, ...
+};
+
 template <int D, int GP>
-__global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev p) {
+__device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaWork &wk) {
     constexpr int KS = D / 16;             // contraction steps of K.Q^T
     constexpr int DB = D / 32;             // 32-feature blocks of the output
     constexpr int KROW = D + 8;            // halfs per K row in LDS (128-bit reads of 16 rows hit distinct banks)
@@ -51,17 +63,15 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, hb = lane >> 5;
-    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    const int kvh = wk.kvh, b = wk.seq;
     const int g = p.g_real;
     _Float16 *tile = reinterpret_cast<_Float16 *>(lds_raw + w * kTileBytes);
 
     const int64_t head0 = (int64_t)b * p.Hq + (int64_t)kvh * g;
     const _Float16 *qrow = reinterpret_cast<const _Float16 *>(p.q) + (head0 + min(l32, g - 1)) * D;
-    const char *kbase = p.k + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
-    const char *vbase = p.v + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
-    const int T = p.T;
-    const int n_tiles = (T + kTile - 1) / kTile;
-    const int tile_begin = split * p.tiles_per_split, tile_end = min(n_tiles, tile_begin + p.tiles_per_split);
+    const char *kbase = wk.kbase, *vbase = wk.vbase;
+    const int T = wk.T;
+    const int tile_begin = wk.tile_begin, tile_end = wk.tile_end;
 
     // this lane's chunks of a tile: chunk j*64 + lane = (row, 16-byte chunk of the row)
     uint32_t g_off[NLD], k_slot[NLD], v_slot[NLD];
@@ -74,7 +84,7 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev
     }
     u32x4 kpre[NLD], vpre[NLD];
     // fused append: the row of token new_pos comes from the step's input and is stored to the cache on the way
-    const int new_pos = p.k_new ? p.new_pos : -1;
+    const int new_pos = wk.new_pos;
     const int64_t new_row = ((int64_t)b * p.Hkv + kvh) * D * 2;
     auto fetch = [&](const char *base0, const char *fresh, int t, u32x4 (&dst)[NLD]) {
         const int t0 = t * kTile;
@@ -201,7 +211,7 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev
     }
     __syncthreads();
     __half *out = reinterpret_cast<__half *>(p.out) + head0 * D;
-    const int64_t slot = ((int64_t)b * p.Hkv + kvh) * p.nsplit + split;
+    const int64_t slot = wk.slot;
     for (int idx = tid; idx < GP * D; idx += kThreads) {
         const int h = idx / D;
         float mm = -INFINITY;
@@ -215,9 +225,9 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev
             acc += comb[ww * kCombStride + idx] * f;
             ll += comb[ww * kCombStride + GP * D + GP + h] * f;
         }
-        if (p.nsplit == 1) {
+        if (wk.nsplit == 1) {
             if (h < g) out[idx] = __float2half_rn(acc / ll);
-        } else if (p.counters == nullptr) {
+        } else if (wk.counter == nullptr) {
             p.part_o[slot * (GP * D) + idx] = acc;
             if ((idx % D) == 0) {
                 p.part_ml[slot * (2 * GP) + h] = mm;
@@ -232,11 +242,48 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev
         }
     }
     if constexpr (GP <= 8) {   // (larger groups: the merge launch; the in-kernel merge would need too many registers)
-        if (p.nsplit > 1 && p.counters != nullptr) {
-            const int64_t bh = (int64_t)b * p.Hkv + kvh;
-            tail_merge<__half, D, GP>(p, p.counters + bh, p.nsplit, bh * p.nsplit, 1, out, tid);
-        }
+        if (wk.nsplit > 1 && wk.counter != nullptr) tail_merge<__half, D, GP>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
     }
+}
+
+// Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.
+template <int D, int GP>
+__global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev p) {
+    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    MfmaWork wk;
+    wk.seq = b, wk.kvh = kvh;
+    wk.kbase = p.k + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+    wk.vbase = p.v + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+    wk.T = p.T;
+    const int n_tiles = (p.T + kTile - 1) / kTile;
+    wk.tile_begin = split * p.tiles_per_split;
+    wk.tile_end = min(n_tiles, wk.tile_begin + p.tiles_per_split);
+    wk.nsplit = p.nsplit;
+    const int64_t bh = (int64_t)b * p.Hkv + kvh;
+    wk.slot = bh * p.nsplit + split;
+    wk.new_pos = p.k_new ? p.new_pos : -1;
+    wk.counter = p.counters ? p.counters + bh : nullptr;
+    wk.part_first = bh * p.nsplit, wk.part_stride = 1;
+    decode_mfma_body<D, GP>(p, wk);
+}
+
+// Ragged batch: grid (work items, kv_heads); an item is a tile range of one sequence (the host's plan).
+template <int D, int GP>
+__global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_ragged_kernel(DecodeDev p, const RaggedItem *__restrict__ items) {
+    const RaggedItem it = items[blockIdx.x];
+    const int kvh = blockIdx.y;
+    MfmaWork wk;
+    wk.seq = it.seq, wk.kvh = kvh;
+    wk.kbase = it.k + (int64_t)kvh * it.stride_h;
+    wk.vbase = it.v + (int64_t)kvh * it.stride_h;
+    wk.T = it.T;
+    wk.tile_begin = it.tile_begin, wk.tile_end = it.tile_end;
+    wk.nsplit = it.nsplit;
+    wk.slot = ((int64_t)it.slot0 + it.split) * p.Hkv + kvh;
+    wk.new_pos = p.k_new ? it.T - 1 : -1;
+    wk.counter = p.counters ? p.counters + (int64_t)it.seq * p.Hkv + kvh : nullptr;
+    wk.part_first = (int64_t)it.slot0 * p.Hkv + kvh, wk.part_stride = p.Hkv;
+    decode_mfma_body<D, GP>(p, wk);
 }
 
 template <int D, int GP>
@@ -258,7 +305,44 @@ int launch_d(const DecodeDev &p, int gp, dim3 grid, hipStream_t s) {
     }
 }
 
+template <int D, int GP>
+int launch_ragged_gp(const DecodeDev &p, const RaggedItem *items, int n_items, const RaggedSeqSlots *seqs, int n_seq,
+                     bool any_split, hipStream_t s) {
+    hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<D, GP>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+    if (any_split && !p.counters)   // with counters the last workgroup of a sequence-head has merged it
+        hipLaunchKernelGGL((sdpa_decode_ragged_merge_kernel<__half, D, GP>), dim3(p.Hkv, n_seq, p.g_real), dim3(D), 0, s, p, seqs);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("ragged sdpa_decode (mfma) launch failed: %s", hipGetErrorString(e));
+    return 0;
+}
+
+template <int D>
+int launch_ragged_d(const DecodeDev &p, int gp, const RaggedItem *items, int n_items, const RaggedSeqSlots *seqs, int n_seq,
+                    bool any_split, hipStream_t s) {
+    switch (gp) {
+        case 8: return launch_ragged_gp<D, 8>(p, items, n_items, seqs, n_seq, any_split, s);
+        case 16: return launch_ragged_gp<D, 16>(p, items, n_items, seqs, n_seq, any_split, s);
+        default: return launch_ragged_gp<D, 32>(p, items, n_items, seqs, n_seq, any_split, s);
+    }
+}
+
 }  // namespace
+
+// Group sizes this formulation takes, and the padded size (rows of the partial records) that runs them.
+// One head per kv head is faster on the vector-ALU kernel (batch 8, 8226 tokens: 43.4 against 47.4 us);
+// from two heads on this one is (4 heads: 47.1 against 51.5 us, batch 32 159 against 168 us; 8 heads:
+// 47 against 88 us).  TROCM_DECODE_MFMA_MIN_GROUP overrides the threshold.
+int decode_mfma_group(int64_t g_real) {
+    static const int min_group = getenv("TROCM_DECODE_MFMA_MIN_GROUP") ? atoi(getenv("TROCM_DECODE_MFMA_MIN_GROUP")) : 2;
+    if (g_real < min_group || g_real > 32) return 0;
+    return g_real <= 8 ? 8 : g_real <= 16 ? 16 : 32;
+}
+
+int launch_sdpa_decode_ragged_mfma(const DecodeDev &p, int gp, int64_t D, const RaggedItem *items, int n_items,
+                                   const RaggedSeqSlots *seqs, int n_seq, bool any_split, hipStream_t s) {
+    return D == 128 ? launch_ragged_d<128>(p, gp, items, n_items, seqs, n_seq, any_split, s)
+                    : launch_ragged_d<64>(p, gp, items, n_items, seqs, n_seq, any_split, s);
+}
 
 int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {
     if (a.Sq != 1 || a.mask != nullptr) return 2;
@@ -266,12 +350,8 @@ int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {
     if (a.D != 64 && a.D != 128) return 2;
     if (a.Hq % a.Hkv) return 2;
     const int64_t g_real = a.Hq / a.Hkv;
-    // One head per kv head is faster on the vector-ALU kernel (batch 8, 8226 tokens: 43.4 against 47.4 us);
-    // from two heads on this one is (4 heads: 47.5 against 48.6 us with a merge launch still in it, batch 32
-    // 157 against 162 us; 8 heads: 47 against 84 us).
-    static const int min_group = getenv("TROCM_DECODE_MFMA_MIN_GROUP") ? atoi(getenv("TROCM_DECODE_MFMA_MIN_GROUP")) : 2;
-    if (g_real < min_group || g_real > 32) return 2;
-    const int gp = g_real <= 8 ? 8 : g_real <= 16 ? 16 : 32;
+    const int gp = decode_mfma_group(g_real);
+    if (gp == 0) return 2;
     if ((a.kv_stride_b * 2) % 16 || (a.kv_stride_h * 2) % 16 || (a.kv_stride_t * 2) % 16) return 2;
     if ((uintptr_t)a.k % 16 || (uintptr_t)a.v % 16 || (uintptr_t)a.q % 16) return 2;
     if (a.Sk <= 0 || a.Sk > (1ll << 30) || a.kv_stride_t * 2 * kTile >= (1ll << 31)) return 2;
