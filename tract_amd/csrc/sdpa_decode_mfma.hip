@@ -35,10 +35,26 @@ __device__ __forceinline__ half4_t lds_read_tr16(const _Float16 *lds_ptr) {
     return __builtin_bit_cast(half4_t, r);
 }
 
+__device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
+// bytes (b0, b1) / (b2, b3) of a word as the half pairs (1024 + b): the byte under exponent byte 0x64
+__device__ __forceinline__ half2_t magic_lo(uint32_t w) { return __builtin_bit_cast(half2_t, perm(0x64646464u, w, 0x04010400u)); }
+__device__ __forceinline__ half2_t magic_hi(uint32_t w) { return __builtin_bit_cast(half2_t, perm(0x64646464u, w, 0x04030402u)); }
+// Eight code bytes -> the reference's f16 dequantised values (code - zero) * d, each rounded once to
+// f16 (q4_0.rs:82-95): (1024 + u) - (1024 + zero) is exact, the product rounds.
+__device__ __forceinline__ u32x4 dequant8(uint32_t b0123, uint32_t b4567, half2_t zero1024, half2_t d2) {
+    u32x4 r;
+    r.x = __builtin_bit_cast(uint32_t, (magic_lo(b0123) - zero1024) * d2);
+    r.y = __builtin_bit_cast(uint32_t, (magic_hi(b0123) - zero1024) * d2);
+    r.z = __builtin_bit_cast(uint32_t, (magic_lo(b4567) - zero1024) * d2);
+    r.w = __builtin_bit_cast(uint32_t, (magic_hi(b4567) - zero1024) * d2);
+    return r;
+}
+
 // What one workgroup has to do: a tile range of one (sequence, kv head), and where its result goes.
 struct MfmaWork {
     int seq, kvh;                 // the sequence (batch entry) and kv head
-    const char *kbase, *vbase;    // K and V rows of this (sequence, kv head)
+    const char *kbase, *vbase;    // K and V rows of this (sequence, kv head): f16 rows or block codes
+    const char *ksbase, *vsbase;  // quantised formats: their f16 block scales, D/32 per token
     int T, tile_begin, tile_end;
     int nsplit;                   // splits of this sequence-head (1: write the output rows)
     int64_t slot;                 // partial record of this workgroup
@@ -47,14 +63,21 @@ struct MfmaWork {
     int64_t part_first, part_stride;   // partial records of this sequence-head: first, first + stride, ...
 };
 
-template <int D, int GP>
+// FMT: TROCM_F16, or a block-quantised cache (TROCM_Q8_0 / TROCM_Q4_0, 32-element blocks): the codes are
+// dequantised on the way into the LDS tile, (code - zero) * d rounded once to f16 as the reference's
+// dequantisation rounds it, and everything after the tile is the f16 kernel.
+template <int D, int GP, int FMT>
 __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaWork &wk) {
+    constexpr bool QUANT = FMT != TROCM_F16;
     constexpr int KS = D / 16;             // contraction steps of K.Q^T
     constexpr int DB = D / 32;             // 32-feature blocks of the output
     constexpr int KROW = D + 8;            // halfs per K row in LDS (128-bit reads of 16 rows hit distinct banks)
     constexpr int VROW = D + 16;           // halfs per V row in LDS (rows of a transposing read 8 banks apart)
-    constexpr int CPR = D / 8;             // 16-byte chunks per row
+    constexpr int RB = FMT == TROCM_F16 ? D * 2 : FMT == TROCM_Q8_0 ? D : D / 2;   // bytes per row in the cache
+    constexpr int CPR = RB / 16;           // 16-byte chunks per row
+    constexpr int EPC = D / CPR;           // elements per chunk: 8, 16 (Q8_0), 32 (Q4_0, one block)
     constexpr int NLD = kTile * CPR / 64;  // 128-bit loads per lane, tile and tensor
+    constexpr int SROW = D / 32 * 2;       // bytes of block scales per row
     constexpr int kCombStride = GP * D + 2 * GP;
     constexpr int kTileBytes = kTile * VROW * 2;
     constexpr int kLdsBytes = kWaves * (kTileBytes > kCombStride * 4 ? kTileBytes : kCombStride * 4);
@@ -74,18 +97,66 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
     const int tile_begin = wk.tile_begin, tile_end = wk.tile_end;
 
     // this lane's chunks of a tile: chunk j*64 + lane = (row, 16-byte chunk of the row)
-    uint32_t g_off[NLD], k_slot[NLD], v_slot[NLD];
+    uint32_t g_off[NLD], k_slot[NLD], v_slot[NLD], s_off[QUANT ? NLD : 1];
 #pragma unroll
     for (int j = 0; j < NLD; j++) {
         const int c = j * 64 + lane, row = c / CPR, dc = c % CPR;
+        s_off[QUANT ? j : 0] = row * (D / 32 * 2);
         g_off[j] = (uint32_t)row * (uint32_t)p.kv_stride_t + (uint32_t)dc * 16u;
-        k_slot[j] = row * KROW + dc * 8;
-        v_slot[j] = row * VROW + dc * 8;
+        k_slot[j] = row * KROW + dc * EPC;
+        v_slot[j] = row * VROW + dc * EPC;
     }
     u32x4 kpre[NLD], vpre[NLD];
+    // quantised: the 32-bit word that holds the scale of this lane's chunk (the chunk's place in its row, and
+    // so the word and the half of it, is the same for every j), and the byte selector that doubles that half
+    uint32_t ksc[QUANT ? NLD : 1], vsc[QUANT ? NLD : 1];
+    const int my_block = (lane % CPR) * EPC / 32;
+    const uint32_t sc_word = (my_block >> 1) * 4, sc_sel = (my_block & 1) ? 0x03020302u : 0x01000100u;
     // fused append: the row of token new_pos comes from the step's input and is stored to the cache on the way
     const int new_pos = wk.new_pos;
     const int64_t new_row = ((int64_t)b * p.Hkv + kvh) * D * 2;
+    auto fetch_q = [&](const char *base0, const char *sbase0, int t, u32x4 (&dst)[NLD], uint32_t (&sc)[QUANT ? NLD : 1]) {
+        const int t0 = t * kTile;
+        const char *base = base0 + (int64_t)t0 * RB;
+        const char *sbase = sbase0 + (int64_t)t0 * SROW + sc_word;
+        if (t0 + kTile <= T) {   // whole tile: a wave-uniform base and this lane's fixed offsets
+#pragma unroll
+            for (int j = 0; j < (QUANT ? NLD : 0); j++) {
+                dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + g_off[j]));
+                sc[j] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(sbase + s_off[QUANT ? j : 0]));
+            }
+        } else {
+            const int last = T - 1 - t0;   // rows past the end of the sequence repeat its last token (masked below)
+#pragma unroll
+            for (int j = 0; j < (QUANT ? NLD : 0); j++) {
+                const int c = j * 64 + lane, row = min(c / CPR, last), dc = c % CPR;
+                dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + row * RB + dc * 16));
+                sc[j] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(sbase + row * SROW));
+            }
+        }
+    };
+    // codes of one tile -> f16 rows in the LDS tile
+    auto stash_q = [&](const u32x4 (&codes)[NLD], const uint32_t (&sc)[QUANT ? NLD : 1], const uint32_t (&slot)[NLD]) {
+#pragma unroll
+        for (int j = 0; j < (QUANT ? NLD : 0); j++) {
+            const half2_t d2 = __builtin_bit_cast(half2_t, perm(sc[j], sc[j], sc_sel));
+            const u32x4 c = codes[j];
+            if constexpr (FMT == TROCM_Q8_0) {
+                const half2_t zero = {(_Float16)1152.0f, (_Float16)1152.0f};   // 1024 + 128: the byte read is code ^ 0x80 = code + 128
+                const uint32_t x = 0x80808080u;
+                *reinterpret_cast<u32x4 *>(tile + slot[j]) = dequant8(c.x ^ x, c.y ^ x, zero, d2);
+                *reinterpret_cast<u32x4 *>(tile + slot[j] + 8) = dequant8(c.z ^ x, c.w ^ x, zero, d2);
+            } else {
+                // byte i of a block's 16: element i in the low nibble, element 16 + i in the high one
+                const half2_t zero = {(_Float16)1032.0f, (_Float16)1032.0f};   // 1024 + 8
+                const uint32_t m = 0x0F0F0F0Fu;
+                *reinterpret_cast<u32x4 *>(tile + slot[j]) = dequant8(c.x & m, c.y & m, zero, d2);
+                *reinterpret_cast<u32x4 *>(tile + slot[j] + 8) = dequant8(c.z & m, c.w & m, zero, d2);
+                *reinterpret_cast<u32x4 *>(tile + slot[j] + 16) = dequant8((c.x >> 4) & m, (c.y >> 4) & m, zero, d2);
+                *reinterpret_cast<u32x4 *>(tile + slot[j] + 24) = dequant8((c.z >> 4) & m, (c.w >> 4) & m, zero, d2);
+            }
+        }
+    };
     auto fetch = [&](const char *base0, const char *fresh, int t, u32x4 (&dst)[NLD]) {
         const int t0 = t * kTile;
         const char *base = base0 + (int64_t)t0 * p.kv_stride_t;
@@ -106,8 +177,13 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
 
     int t = tile_begin + w;
     if (t < tile_end) {
-        fetch(kbase, p.k_new, t, kpre);
-        fetch(vbase, p.v_new, t, vpre);
+        if constexpr (QUANT) {
+            fetch_q(kbase, wk.ksbase, t, kpre, ksc);
+            fetch_q(vbase, wk.vsbase, t, vpre, vsc);
+        } else {
+            fetch(kbase, p.k_new, t, kpre);
+            fetch(vbase, p.v_new, t, vpre);
+        }
     }
     // Q^T fragments: row (head) = lane % 32, features 16*ks + 8*hb .. +8
     half8_t qf[KS];
@@ -131,9 +207,14 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
         const int t0 = t * kTile;
         const bool more = t + kWaves < tile_end;
         // ---- K tile -> LDS, the next tile's K into flight ----------------------------------------------
+        if constexpr (QUANT) {
+            stash_q(kpre, ksc, k_slot);
+            if (more) fetch_q(kbase, wk.ksbase, t + kWaves, kpre, ksc);
+        } else {
 #pragma unroll
-        for (int j = 0; j < NLD; j++) *reinterpret_cast<u32x4 *>(tile + k_slot[j]) = kpre[j];
-        if (more) fetch(kbase, p.k_new, t + kWaves, kpre);
+            for (int j = 0; j < NLD; j++) *reinterpret_cast<u32x4 *>(tile + k_slot[j]) = kpre[j];
+            if (more) fetch(kbase, p.k_new, t + kWaves, kpre);
+        }
         // ---- S^T = K Q^T: 32 tokens x 32 rows ------------------------------------------------------------
         float16_t s;
 #pragma unroll
@@ -146,11 +227,19 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
         }
         // ---- online softmax of this lane's head over its 16 tokens: token = t0 + 8*(r/4) + 4*hb + r%4 ----
         float tmax = -INFINITY;
+        if (QUANT && t0 + kTile <= T) {   // (the f16 instantiation has no register to spare for a second copy of this)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int tok = t0 + 8 * (r >> 2) + 4 * hb + (r & 3);
-            s[r] = (t0 + kTile <= T || tok < T) ? s[r] * p.scale_log2 : -INFINITY;
-            tmax = fmaxf(tmax, s[r]);
+            for (int r = 0; r < 16; r++) {
+                s[r] *= p.scale_log2;
+                tmax = fmaxf(tmax, s[r]);
+            }
+        } else {   // possibly the sequence's last tile: tokens past its end do not count
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int tok = t0 + 8 * (r >> 2) + 4 * hb + (r & 3);
+                s[r] = (t0 + kTile <= T || tok < T) ? s[r] * p.scale_log2 : -INFINITY;
+                tmax = fmaxf(tmax, s[r]);
+            }
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
         const float m_new = fmaxf(m_run, tmax);   // finite: every tile holds at least one valid token
@@ -175,9 +264,14 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
                 for (int r = 0; r < 16; r++) o[db][r] *= alpha;
         }
         // ---- V tile -> the same LDS tile (every K fragment has been consumed), next V into flight ------
+        if constexpr (QUANT) {
+            stash_q(vpre, vsc, v_slot);
+            if (more) fetch_q(vbase, wk.vsbase, t + kWaves, vpre, vsc);
+        } else {
 #pragma unroll
-        for (int j = 0; j < NLD; j++) *reinterpret_cast<u32x4 *>(tile + v_slot[j]) = vpre[j];
-        if (more) fetch(vbase, p.v_new, t + kWaves, vpre);
+            for (int j = 0; j < NLD; j++) *reinterpret_cast<u32x4 *>(tile + v_slot[j]) = vpre[j];
+            if (more) fetch(vbase, p.v_new, t + kWaves, vpre);
+        }
         // ---- O^T += V^T P^T ---------------------------------------------------------------------------------
         const _Float16 *vsrc = tile + vsrc_off;
 #pragma unroll
@@ -247,13 +341,18 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
 }
 
 // Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.
-template <int D, int GP>
+template <int D, int GP, int FMT>
 __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev p) {
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     MfmaWork wk;
     wk.seq = b, wk.kvh = kvh;
     wk.kbase = p.k + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
     wk.vbase = p.v + (int64_t)b * p.kv_stride_b + (int64_t)kvh * p.kv_stride_h;
+    wk.ksbase = wk.vsbase = nullptr;
+    if constexpr (FMT != TROCM_F16) {
+        wk.ksbase = p.k_scales + (int64_t)b * p.sc_stride_b + (int64_t)kvh * p.sc_stride_h;
+        wk.vsbase = p.v_scales + (int64_t)b * p.sc_stride_b + (int64_t)kvh * p.sc_stride_h;
+    }
     wk.T = p.T;
     const int n_tiles = (p.T + kTile - 1) / kTile;
     wk.tile_begin = split * p.tiles_per_split;
@@ -264,7 +363,7 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev
     wk.new_pos = p.k_new ? p.new_pos : -1;
     wk.counter = p.counters ? p.counters + bh : nullptr;
     wk.part_first = bh * p.nsplit, wk.part_stride = 1;
-    decode_mfma_body<D, GP>(p, wk);
+    decode_mfma_body<D, GP, FMT>(p, wk);
 }
 
 // Ragged batch: grid (work items, kv_heads); an item is a tile range of one sequence (the host's plan).
@@ -276,6 +375,7 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_ragged_kernel(De
     wk.seq = it.seq, wk.kvh = kvh;
     wk.kbase = it.k + (int64_t)kvh * it.stride_h;
     wk.vbase = it.v + (int64_t)kvh * it.stride_h;
+    wk.ksbase = wk.vsbase = nullptr;
     wk.T = it.T;
     wk.tile_begin = it.tile_begin, wk.tile_end = it.tile_end;
     wk.nsplit = it.nsplit;
@@ -283,12 +383,12 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_ragged_kernel(De
     wk.new_pos = p.k_new ? it.T - 1 : -1;
     wk.counter = p.counters ? p.counters + (int64_t)it.seq * p.Hkv + kvh : nullptr;
     wk.part_first = (int64_t)it.slot0 * p.Hkv + kvh, wk.part_stride = p.Hkv;
-    decode_mfma_body<D, GP>(p, wk);
+    decode_mfma_body<D, GP, TROCM_F16>(p, wk);
 }
 
-template <int D, int GP>
+template <int D, int GP, int FMT = TROCM_F16>
 int launch_gp(const DecodeDev &p, dim3 grid, hipStream_t s) {
-    hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, GP>), grid, dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, GP, FMT>), grid, dim3(kThreads), 0, s, p);
     if (p.nsplit > 1 && p.counters == nullptr)
         hipLaunchKernelGGL((sdpa_decode_merge_kernel<__half, D, GP>), dim3(grid.y, grid.z, p.g_real), dim3(D), 0, s, p);
     hipError_t e = hipGetLastError();
@@ -302,6 +402,15 @@ int launch_d(const DecodeDev &p, int gp, dim3 grid, hipStream_t s) {
         case 8: return launch_gp<D, 8>(p, grid, s);
         case 16: return launch_gp<D, 16>(p, grid, s);
         default: return launch_gp<D, 32>(p, grid, s);
+    }
+}
+
+template <int FMT>
+int launch_quant(const DecodeDev &p, int gp, dim3 grid, hipStream_t s) {
+    switch (gp) {
+        case 8: return launch_gp<128, 8, FMT>(p, grid, s);
+        case 16: return launch_gp<128, 16, FMT>(p, grid, s);
+        default: return launch_gp<128, 32, FMT>(p, grid, s);
     }
 }
 
@@ -342,6 +451,32 @@ int launch_sdpa_decode_ragged_mfma(const DecodeDev &p, int gp, int64_t D, const 
                                    const RaggedSeqSlots *seqs, int n_seq, bool any_split, hipStream_t s) {
     return D == 128 ? launch_ragged_d<128>(p, gp, items, n_items, seqs, n_seq, any_split, s)
                     : launch_ragged_d<64>(p, gp, items, n_items, seqs, n_seq, any_split, s);
+}
+
+// Quantised cache planes (the caller has checked formats, alignment and strides and filled p but for the
+// splits): 2 = not taken (one head per kv head).
+int launch_sdpa_decode_quant_mfma(DecodeDev &p, int kv_fmt, int64_t B, void *workspace, size_t workspace_bytes, hipStream_t s) {
+    const int gp = decode_mfma_group(p.g_real);
+    if (gp == 0) return 2;
+    const int64_t BH = B * p.Hkv;
+    const int n_tiles = (p.T + kTile - 1) / kTile;
+    static const int wg_per_cu = getenv("TROCM_DECODE_QUANT_WG_PER_CU") ? atoi(getenv("TROCM_DECODE_QUANT_WG_PER_CU")) : 2;
+    int nsplit = choose_decode_splits(BH, gp, n_tiles, wg_per_cu);
+    const int tps = (n_tiles + nsplit - 1) / nsplit;
+    nsplit = (n_tiles + tps - 1) / tps;
+    if (nsplit > 1) {
+        TROCM_NOT_NULL(workspace);
+        const size_t need = kWsCounterBytes + (size_t)BH * nsplit * gp * (128 + 2) * sizeof(float);
+        TROCM_REQUIRE(workspace_bytes >= need, "sdpa workspace too small: %zu bytes given, %zu needed", workspace_bytes, need);
+    }
+    p.tiles_per_split = tps, p.nsplit = nsplit;
+    p.part_ml = (float *)((char *)workspace + kWsCounterBytes);
+    p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * gp;
+    static const int tail = getenv("TROCM_DECODE_TAIL_MERGE") ? atoi(getenv("TROCM_DECODE_TAIL_MERGE")) : 1;
+    p.counters = nullptr;
+    if (tail && gp <= 8 && nsplit > 1 && nsplit <= kTailMergeMax && BH <= (int64_t)(kWsCounterBytes / sizeof(int))) p.counters = (int *)workspace;
+    dim3 grid(nsplit, (unsigned)p.Hkv, (unsigned)B);
+    return kv_fmt == TROCM_Q8_0 ? launch_quant<TROCM_Q8_0>(p, gp, grid, s) : launch_quant<TROCM_Q4_0>(p, gp, grid, s);
 }
 
 int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {

@@ -404,7 +404,8 @@ int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s) {
     if (a.q_dtype != TROCM_F16 || a.D != kD) return 2;
     if (a.Hq % a.Hkv) return 2;
     const int64_t g_real = a.Hq / a.Hkv;
-    if (g_real > 8) return 2;
+    const bool mfma = decode_mfma_group(g_real) != 0;   // grouped heads: the MFMA formulation (sdpa_decode_mfma.hip)
+    if (g_real > 8 && !mfma) return 2;
     const int64_t G = g_real <= 2 ? g_real : g_real <= 4 ? 4 : 8;   // the instantiation that runs it
     if (a.kv_stride_t != a.D) return 2;  // cache planes: token rows are dense
     if ((uintptr_t)a.k % 16 || (uintptr_t)a.v % 16 || (uintptr_t)a.q % 16 || (uintptr_t)a.k_scales % 4 ||
@@ -417,6 +418,19 @@ int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s) {
     int64_t cap_h = a.kv_stride_h / a.D, cap_b = a.kv_stride_b / a.D;  // in token rows
     if ((cap_h * rb) % 16 || (cap_b * rb) % 16) return 2;
 
+    if (mfma) {
+        DecodeDev p;
+        memset(&p, 0, sizeof(p));
+        p.q = (const char *)a.q, p.out = (char *)a.out, p.k = (const char *)a.k, p.v = (const char *)a.v;
+        p.kv_stride_b = cap_b * rb, p.kv_stride_h = cap_h * rb, p.kv_stride_t = rb;
+        p.k_scales = (const char *)a.k_scales, p.v_scales = (const char *)a.v_scales;
+        p.sc_stride_b = cap_b * kNB * 2, p.sc_stride_h = cap_h * kNB * 2;
+        p.T = (int)a.Sk;
+        p.Hq = (int)a.Hq, p.Hkv = (int)a.Hkv, p.g_real = (int)g_real;
+        p.scale_log2 = a.scale * 1.4426950408889634f;
+        p.new_pos = -1;
+        return launch_sdpa_decode_quant_mfma(p, a.kv_fmt, a.B, a.workspace, a.workspace_bytes, s);
+    }
     int n_tiles = (int)((a.Sk + kTile - 1) / kTile);
     int nsplit = choose_decode_splits(BH, G, n_tiles, 2);
     int tps = (n_tiles + nsplit - 1) / nsplit;
