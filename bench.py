@@ -473,6 +473,26 @@ def run_ops(ta, args):
         by = n_ * (k_ // 32) * 18 + 2 * k_ + 2 * n_
         res[f"q4_0_matvec_f16_n{n_}_k{k_}"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": by}
         del ws
+    # ragged decode step over quantised caches: 32 sequences of 512..32768 tokens, their new tokens quantised
+    # by one launch and attention by another
+    n_seq = 32
+    lens = np.random.default_rng(cfg_seed(5, "q") + 3).integers(512, 32768, size=n_seq, endpoint=True)
+    for fmt, name, rb in ((ta.Q8_0, "q8_0", 136), (ta.Q4_0, "q4_0", 72)):
+        pool = ta.KvPool(int(lens.sum()) * HKV * rb * 2 * 3 + (64 << 20))
+        kcs, vcs = [], []
+        for n_ in lens:
+            kk = rng.standard_normal((1, HKV, int(n_), D), dtype=np.float32).astype(np.float16)
+            kc, vc = ta.InPlaceKvCache(2, fmt, pool=pool), ta.InPlaceKvCache(2, fmt, pool=pool)
+            kc.push(kk), vc.push(kk)
+            kcs.append(kc), vcs.append(vc)
+        wsr = ta.Workspace(n_seq, HQ, 1, D)
+        qr = ta.DeviceTensor.from_numpy((rng.standard_normal((n_seq, HQ, 1, D)) / np.sqrt(D)).astype(np.float16))
+        knr = ta.DeviceTensor.from_numpy(rng.standard_normal((n_seq, HKV, 1, D)).astype(np.float16))
+        outr = ta.DeviceTensor((n_seq, HQ, 1, D), np.float16)
+        us = time_calls(ta, lambda: ta.inplace_kv_sdpa_eval_ragged(qr, knr, knr, kcs, vcs, workspace=wsr, out=outr), 16)
+        by = 2 * HKV * int(sum(c.len() for c in kcs)) * rb
+        res[f"ragged_step_{name}_32seq"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": by}
+        del kcs, vcs, pool
     # the oracle on the host for the same ops, on a bounded sample
     xh = rng.standard_normal((1, 4, S, D)).astype(np.float16)
     t0 = time.perf_counter()

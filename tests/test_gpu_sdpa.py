@@ -297,7 +297,7 @@ def test_ragged_decode_small(rt):
 
 @pytest.mark.parametrize("fmt_name", ["Q8_0", "Q4_0"])
 @pytest.mark.parametrize("B,Hq,Hkv,T", [(1, 32, 8, 1), (2, 32, 8, 100), (2, 32, 8, 1025), (1, 8, 8, 333), (1, 16, 2, 64),
-                                         (1, 24, 8, 77)])
+                                         (1, 24, 8, 77), (2, 32, 2, 300), (1, 32, 1, 129), (1, 22, 2, 95)])
 def test_decode_quantised_cache(rt, fmt_name, B, Hq, Hkv, T):
     """cfg4 (reduced): K/V quantised on append, 1% outlier channels x20, decode with fused
     dequantisation.  Oracle: FlashSdpaOp over the dequantised blocks (f16 dequant like
@@ -330,6 +330,43 @@ def test_decode_quantised_cache(rt, fmt_name, B, Hq, Hkv, T):
     exact = cases.textbook_sdpa(q, orc.dequant(orc_fmt, kq, np.float32), orc.dequant(orc_fmt, vq, np.float32))
     # (the output is f16: allow its rounding, half an ulp relative, on the outlier-channel magnitudes)
     assert np.allclose(out.astype(np.float64), exact, rtol=1.5e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize("fmt_name", ["Q8_0", "Q4_0"])
+@pytest.mark.parametrize("Hq,Hkv,n_seq,lo,hi", [(32, 8, 12, 1, 2500), (16, 1, 5, 20, 700), (8, 8, 4, 10, 200)])
+def test_ragged_decode_over_quantised_caches(rt, fmt_name, Hq, Hkv, n_seq, lo, hi):
+    """Independent sequences with quantised caches of their own: every sequence equals the batch-1
+    oracle over its dequantised blocks.  Two steps: attention only, then the append-and-attend step."""
+    D = 128
+    dev_fmt, orc_fmt = getattr(tract_amd, fmt_name), getattr(orc, "FMT_" + fmt_name)
+    rng = np.random.default_rng(cases.cfg_seed(5, "len") + Hq)
+    lens = rng.integers(lo, hi, size=n_seq, endpoint=True)
+    kcs, vcs, ks, vs = [], [], [], []
+    for n in lens:
+        k = rng.standard_normal((1, Hkv, int(n), D), dtype=np.float32).astype(np.float16)
+        v = rng.standard_normal((1, Hkv, int(n), D), dtype=np.float32).astype(np.float16)
+        kc, vc = tract_amd.InPlaceKvCache(2, dev_fmt), tract_amd.InPlaceKvCache(2, dev_fmt)
+        kc.push(k), vc.push(v)
+        kcs.append(kc), vcs.append(vc), ks.append(k), vs.append(v)
+    ws = tract_amd.Workspace(n_seq, Hq, 1, D)
+
+    def check(out, q):
+        assert not np.isnan(out).any()
+        for i in range(n_seq):
+            kd = orc.dequant(orc_fmt, orc.quant(orc_fmt, ks[i]), np.float16)
+            vd = orc.dequant(orc_fmt, orc.quant(orc_fmt, vs[i]), np.float16)
+            assert max_abs(out[i:i + 1], orc.flash_sdpa(q[i:i + 1], kd, vd, causal=True)) <= 2e-2, f"sequence {i} len {ks[i].shape[2]}"
+
+    q = (rng.standard_normal((n_seq, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    check(tract_amd.sdpa_decode_ragged(tract_amd.DeviceTensor.from_numpy(q), kcs, vcs, workspace=ws).to_numpy(), q)
+    kn = rng.standard_normal((n_seq, Hkv, 1, D), dtype=np.float32).astype(np.float16)
+    vn = rng.standard_normal((n_seq, Hkv, 1, D), dtype=np.float32).astype(np.float16)
+    q = (rng.standard_normal((n_seq, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    out = tract_amd.inplace_kv_sdpa_eval_ragged(tract_amd.DeviceTensor.from_numpy(q), tract_amd.DeviceTensor.from_numpy(kn),
+                                                tract_amd.DeviceTensor.from_numpy(vn), kcs, vcs, workspace=ws).to_numpy()
+    for i in range(n_seq):
+        ks[i], vs[i] = np.concatenate([ks[i], kn[i:i + 1]], axis=2), np.concatenate([vs[i], vn[i:i + 1]], axis=2)
+    check(out, q)
 
 
 def test_quantised_cache_with_f32_queries_uses_generic_kernel(rt):

@@ -1170,7 +1170,26 @@ static int ragged_common(const void *q, const void *k_new, const void *v_new, in
         }
         return 0;
     };
-    if (fused && !in_kernel && append_explicitly()) return 1;
+    // Quantised caches: one launch quantises every sequence's new token (its table travels in the plan area of
+    // the workspace, which the attention launch rewrites afterwards, in stream order).
+    auto append_quantised_at_once = [&]() -> int {
+        std::vector<QuantAppendSeq> tbl((size_t)n_seq);
+        for (int64_t i = 0; i < n_seq; i++) {
+            trocm_kv_cache *kc = k_caches[i], *vc = v_caches[i];
+            TROCM_REQUIRE(kc->pitch == vc->pitch, "K/V capacities must match (sequence %lld)", (long long)i);
+            tbl[(size_t)i] = QuantAppendSeq{kc->data, kc->scales, vc->data, vc->scales, kc->pitch, kc->len};
+        }
+        void *dev_tbl = (char *)workspace + kWsCounterBytes;
+        if (upload_table(tbl.data(), tbl.size() * sizeof(QuantAppendSeq), dev_tbl, s)) return 1;
+        if (launch_quant_append_ragged(k0->fmt, q_dtype, n_seq, k0->H, k0->D, (const QuantAppendSeq *)dev_tbl, k_new, v_new, s)) return 1;
+        for (int64_t i = 0; i < n_seq; i++) k_caches[i]->len += 1, v_caches[i]->len += 1;
+        return 0;
+    };
+    if (fused && !in_kernel) {
+        const bool at_once = is_quant(k0->fmt) && workspace != nullptr && workspace_bytes >= kWsCounterBytes + kWsPlanBytes &&
+                             (size_t)n_seq * sizeof(QuantAppendSeq) <= kWsPlanBytes && k0->D % 32 == 0;
+        if (at_once ? append_quantised_at_once() : append_explicitly()) return 1;
+    }
     for (;;) {
         for (int64_t i = 0; i < n_seq; i++) {
             const trocm_kv_cache *kc = k_caches[i], *vc = v_caches[i];

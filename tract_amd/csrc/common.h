@@ -86,6 +86,17 @@ struct QuantAppend {
     void *codes, *scales;
 };
 int launch_quant_append(const QuantAppend &a, hipStream_t s);
+// One new token for each of n_seq sequences (k_new / v_new dense [n_seq, H, 1, D], f16 or f32) quantised
+// into the sequences' own K and V planes by one launch; `table` is in device memory.
+struct QuantAppendSeq {
+    void *k_codes, *k_scales, *v_codes, *v_scales;
+    int64_t cap, t0;   // tokens between kv heads in the planes, and the token to write
+};
+int launch_quant_append_ragged(int fmt, int src_dtype, int64_t n_seq, int64_t H, int64_t D, const QuantAppendSeq *table,
+                               const void *k_new, const void *v_new, hipStream_t s);
+// A small host table (at most kWsPlanBytes) into device memory, ordered on the stream, by a kernel that reads
+// pinned pages (a copy command between two kernels hands the stream to a DMA engine and back).
+int upload_table(const void *src, size_t bytes, void *dst, hipStream_t s);
 // Canonical export of the quantised planes: dst [B,H,len, D/32 * block_bytes].
 int launch_quant_export(int fmt, int64_t B, int64_t H, int64_t len, int64_t cap, int64_t D,
                         const void *codes, const void *scales, void *dst, hipStream_t s);

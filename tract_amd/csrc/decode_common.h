@@ -41,8 +41,10 @@ struct DecodeDev {
 
 // Ragged batches: one work item = a tile range of one sequence (device copies of the host plan).
 struct RaggedItem {
-    const char *k, *v;   // planes of the sequence (kv head 0)
+    const char *k, *v;   // planes of the sequence (kv head 0): f16/f32 rows or block codes
     int64_t stride_h;    // bytes between kv heads
+    const char *ks, *vs; // quantised formats: the f16 block-scale planes (NULL otherwise)
+    int64_t sc_stride_h; // bytes between kv heads in them
     int T, tile_begin, tile_end;
     int seq, split, nsplit, slot0;
 };
@@ -258,7 +260,7 @@ __global__ __launch_bounds__(D) void sdpa_decode_ragged_merge_kernel(DecodeDev p
 // which is also the stride of the partial records.
 int decode_mfma_group(int64_t g_real);   // 0: not taken by the MFMA formulation
 int launch_sdpa_decode_quant_mfma(DecodeDev &p, int kv_fmt, int64_t B, void *workspace, size_t workspace_bytes, hipStream_t s);
-int launch_sdpa_decode_ragged_mfma(const DecodeDev &p, int gp, int64_t D, const RaggedItem *items, int n_items,
+int launch_sdpa_decode_ragged_mfma(const DecodeDev &p, int kv_fmt, int gp, int64_t D, const RaggedItem *items, int n_items,
                                    const RaggedSeqSlots *seqs, int n_seq, bool any_split, hipStream_t s);
 
 // Partials: at most kMaxSplitRows rows of (D + 2) floats per query head.

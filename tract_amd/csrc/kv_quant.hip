@@ -165,6 +165,38 @@ __global__ __launch_bounds__(256) void quant_append_kernel(QuantAppendDev a) {
     }
 }
 
+// One token per sequence into per-sequence planes: grid (sequences, 2 = K / V).
+template <typename SrcT>
+__global__ __launch_bounds__(256) void quant_append_ragged_kernel(int fmt, const QuantAppendSeq *__restrict__ table,
+                                                                  const SrcT *__restrict__ k_new, const SrcT *__restrict__ v_new,
+                                                                  int64_t H, int64_t D, int vec) {
+    const QuantAppendSeq e = table[blockIdx.x];
+    const bool is_v = blockIdx.y != 0;
+    const SrcT *src = (is_v ? v_new : k_new) + (int64_t)blockIdx.x * H * D;
+    uint8_t *codes = (uint8_t *)(is_v ? e.v_codes : e.k_codes);
+    uint16_t *scales = (uint16_t *)(is_v ? e.v_scales : e.k_scales);
+    const int64_t nb = D / 32;
+    for (int64_t idx = threadIdx.x; idx < H * nb; idx += blockDim.x) {
+        const int64_t blk = idx % nb, h = idx / nb;
+        float v[32];
+        load_block(src + h * D + blk * 32, 1, vec != 0, v);
+        const int64_t row = h * e.cap + e.t0;
+        if (fmt == TROCM_Q8_0) {
+            uint32_t c[8];
+            const uint16_t d = quant_q8(v, c);
+            uint4 *dst = reinterpret_cast<uint4 *>(codes + row * D + blk * 32);
+            dst[0] = make_uint4(c[0], c[1], c[2], c[3]);
+            dst[1] = make_uint4(c[4], c[5], c[6], c[7]);
+            scales[row * nb + blk] = d;
+        } else {
+            uint32_t c[4];
+            const uint16_t d = quant_q4(v, c);
+            *reinterpret_cast<uint4 *>(codes + row * (D / 2) + blk * 16) = make_uint4(c[0], c[1], c[2], c[3]);
+            scales[row * nb + blk] = d;
+        }
+    }
+}
+
 // Canonical export: [B,H,len, nb * (2 + code bytes)], 2-byte aligned stores.
 __global__ __launch_bounds__(256) void quant_export_kernel(int fmt, int64_t BH, int64_t len, int64_t cap, int64_t D,
                                                            const uint8_t *__restrict__ codes,
@@ -300,6 +332,20 @@ int launch_quant_append(const QuantAppend &a, hipStream_t s) {
     else
         hipLaunchKernelGGL(quant_append_kernel<float>, dim3(grid), dim3(256), 0, s, d);
     return check_launch("quant_append");
+}
+
+int launch_quant_append_ragged(int fmt, int src_dtype, int64_t n_seq, int64_t H, int64_t D, const QuantAppendSeq *table,
+                               const void *k_new, const void *v_new, hipStream_t s) {
+    if (n_seq == 0) return 0;
+    const int vec = (uintptr_t)k_new % 16 == 0 && (uintptr_t)v_new % 16 == 0;   // rows of D elements, D % 32 == 0
+    const int threads = H * (D / 32) >= 256 ? 256 : 64;
+    if (src_dtype == TROCM_F16)
+        hipLaunchKernelGGL(quant_append_ragged_kernel<__half>, dim3((unsigned)n_seq, 2), dim3(threads), 0, s, fmt, table,
+                           (const __half *)k_new, (const __half *)v_new, H, D, vec);
+    else
+        hipLaunchKernelGGL(quant_append_ragged_kernel<float>, dim3((unsigned)n_seq, 2), dim3(threads), 0, s, fmt, table,
+                           (const float *)k_new, (const float *)v_new, H, D, vec);
+    return check_launch("quant_append_ragged");
 }
 
 int launch_quant_export(int fmt, int64_t B, int64_t H, int64_t len, int64_t cap, int64_t D, const void *codes,

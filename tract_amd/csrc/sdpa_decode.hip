@@ -569,6 +569,24 @@ int acquire_stage(StageSlot **out) {
     return 0;
 }
 
+}  // namespace
+
+int upload_table(const void *src, size_t bytes, void *dst, hipStream_t s) {
+    TROCM_REQUIRE(bytes <= kWsPlanBytes, "upload_table: %zu bytes exceed the staging slot", bytes);
+    if (bytes == 0) return 0;
+    StageSlot *stage;
+    if (acquire_stage(&stage)) return 1;
+    memcpy(stage->host, src, bytes);
+    const int n16 = (int)((bytes + 15) / 16);
+    hipLaunchKernelGGL(plan_upload_kernel, dim3((n16 + 255) / 256), dim3(256), 0, s, (const uint4 *)stage->host_dev, (uint4 *)dst, n16);
+    TROCM_HIP(hipGetLastError());
+    TROCM_HIP(hipEventRecord(stage->done, s));
+    stage->in_flight = true;
+    return 0;
+}
+
+namespace {
+
 template <typename T, int D, int G>
 void launch_ragged(const DecodeDev &p, const RaggedItem *items, int n_items, const RaggedSeqSlots *seqs, int n_seq,
                    bool any_split, hipStream_t s) {
@@ -626,15 +644,22 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
                               int64_t D, const RaggedSeq *seqs, float scale, void *workspace, size_t workspace_bytes,
                               const void *k_new, const void *v_new, hipStream_t s) {
     const int64_t g_real = Hq / Hkv;
-    const int mfma_gp = kv_fmt == TROCM_F16 ? decode_mfma_group(g_real) : 0;   // f16 with grouped heads: the MFMA formulation
+    // grouped heads over f16 or block-quantised caches: the MFMA formulation (sdpa_decode_mfma.hip)
+    const bool quant = is_quant(kv_fmt);
+    const int mfma_gp = (kv_fmt == TROCM_F16 || (quant && q_dtype == TROCM_F16 && D == 128)) ? decode_mfma_group(g_real) : 0;
     const int64_t G = mfma_gp ? mfma_gp : g_real <= 2 ? g_real : g_real <= 4 ? 4 : 8;   // the instantiation that runs it
-    const size_t es = elem_bytes(kv_fmt);
-    bool fast = (kv_fmt == TROCM_F16 || kv_fmt == TROCM_F32) && q_dtype == kv_fmt && (D == 64 || D == 128) &&
-                g_real >= 1 && (g_real <= 8 || mfma_gp) && workspace != nullptr && (uintptr_t)q % 16 == 0 &&
-                n_seq <= 2048 && Hkv <= 65535;
-    for (int64_t i = 0; i < n_seq && fast; i++)
+    const int64_t rb = kv_fmt == TROCM_Q8_0 ? D : kv_fmt == TROCM_Q4_0 ? D / 2 : D * (int64_t)elem_bytes(kv_fmt);   // bytes per token row
+    bool fast = quant ? mfma_gp != 0 && k_new == nullptr
+                      : (kv_fmt == TROCM_F16 || kv_fmt == TROCM_F32) && q_dtype == kv_fmt && (D == 64 || D == 128) &&
+                            g_real >= 1 && (g_real <= 8 || mfma_gp);
+    fast = fast && workspace != nullptr && (uintptr_t)q % 16 == 0 && n_seq <= 2048 && Hkv <= 65535;
+    for (int64_t i = 0; i < n_seq && fast; i++) {
         fast = (uintptr_t)seqs[i].k % 16 == 0 && (uintptr_t)seqs[i].v % 16 == 0 && seqs[i].len < (1ll << 30) &&
-               (seqs[i].cap * D * es) % 16 == 0;
+               (seqs[i].cap * rb) % 16 == 0;
+        if (quant)
+            fast = fast && seqs[i].k_scales && seqs[i].v_scales && (uintptr_t)seqs[i].k_scales % 4 == 0 &&
+                   (uintptr_t)seqs[i].v_scales % 4 == 0;
+    }
     if (k_new && ((uintptr_t)k_new % 16 || (uintptr_t)v_new % 16)) fast = false;
     if (!fast) {
         if (k_new) return 2;  // the caller appends explicitly, then calls again without a fused append
@@ -690,7 +715,9 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
             RaggedItem &r = items[it];
             r.k = (const char *)seqs[i].k;
             r.v = (const char *)seqs[i].v;
-            r.stride_h = seqs[i].cap * D * (int64_t)es;
+            r.stride_h = seqs[i].cap * rb;
+            r.ks = (const char *)seqs[i].k_scales, r.vs = (const char *)seqs[i].v_scales;
+            r.sc_stride_h = seqs[i].cap * (D / 32) * 2;
             r.T = (int)seqs[i].len;
             r.tile_begin = (int)(sp * tps);
             r.tile_end = (int)((sp + 1) * tps < tiles ? (sp + 1) * tps : tiles);
@@ -720,7 +747,7 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     memset(&p, 0, sizeof(p));
     p.q = (const char *)q;
     p.out = (char *)out;
-    p.kv_stride_t = D * (int64_t)es;
+    p.kv_stride_t = rb;
     p.Hq = (int)Hq;
     p.Hkv = (int)Hkv;
     p.g_real = (int)g_real;
@@ -736,7 +763,7 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     if (tail && mfma_gp && mfma_gp <= 8 && any_split && max_split <= kTailMergeMax &&
         n_seq * Hkv <= (int64_t)(kWsCounterBytes / sizeof(int)))
         p.counters = (int *)workspace;
-    if (mfma_gp) return launch_sdpa_decode_ragged_mfma(p, mfma_gp, D, d_items, (int)n_items, d_slots, (int)n_seq, any_split, s);
+    if (mfma_gp) return launch_sdpa_decode_ragged_mfma(p, kv_fmt, mfma_gp, D, d_items, (int)n_items, d_slots, (int)n_seq, any_split, s);
     if (kv_fmt == TROCM_F16)
         return D == 128 ? launch_ragged_g<__half, 128>(p, (int)G, d_items, (int)n_items, d_slots, (int)n_seq, any_split, s)
                         : launch_ragged_g<__half, 64>(p, (int)G, d_items, (int)n_items, d_slots, (int)n_seq, any_split, s);

@@ -367,7 +367,7 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev
 }
 
 // Ragged batch: grid (work items, kv_heads); an item is a tile range of one sequence (the host's plan).
-template <int D, int GP>
+template <int D, int GP, int FMT>
 __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_ragged_kernel(DecodeDev p, const RaggedItem *__restrict__ items) {
     const RaggedItem it = items[blockIdx.x];
     const int kvh = blockIdx.y;
@@ -376,6 +376,10 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_ragged_kernel(De
     wk.kbase = it.k + (int64_t)kvh * it.stride_h;
     wk.vbase = it.v + (int64_t)kvh * it.stride_h;
     wk.ksbase = wk.vsbase = nullptr;
+    if constexpr (FMT != TROCM_F16) {
+        wk.ksbase = it.ks + (int64_t)kvh * it.sc_stride_h;
+        wk.vsbase = it.vs + (int64_t)kvh * it.sc_stride_h;
+    }
     wk.T = it.T;
     wk.tile_begin = it.tile_begin, wk.tile_end = it.tile_end;
     wk.nsplit = it.nsplit;
@@ -383,7 +387,7 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_ragged_kernel(De
     wk.new_pos = p.k_new ? it.T - 1 : -1;
     wk.counter = p.counters ? p.counters + (int64_t)it.seq * p.Hkv + kvh : nullptr;
     wk.part_first = (int64_t)it.slot0 * p.Hkv + kvh, wk.part_stride = p.Hkv;
-    decode_mfma_body<D, GP, TROCM_F16>(p, wk);
+    decode_mfma_body<D, GP, FMT>(p, wk);
 }
 
 template <int D, int GP, int FMT = TROCM_F16>
@@ -414,10 +418,10 @@ int launch_quant(const DecodeDev &p, int gp, dim3 grid, hipStream_t s) {
     }
 }
 
-template <int D, int GP>
+template <int D, int GP, int FMT = TROCM_F16>
 int launch_ragged_gp(const DecodeDev &p, const RaggedItem *items, int n_items, const RaggedSeqSlots *seqs, int n_seq,
                      bool any_split, hipStream_t s) {
-    hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<D, GP>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+    hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<D, GP, FMT>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
     if (any_split && !p.counters)   // with counters the last workgroup of a sequence-head has merged it
         hipLaunchKernelGGL((sdpa_decode_ragged_merge_kernel<__half, D, GP>), dim3(p.Hkv, n_seq, p.g_real), dim3(D), 0, s, p, seqs);
     hipError_t e = hipGetLastError();
@@ -447,8 +451,20 @@ int decode_mfma_group(int64_t g_real) {
     return g_real <= 8 ? 8 : g_real <= 16 ? 16 : 32;
 }
 
-int launch_sdpa_decode_ragged_mfma(const DecodeDev &p, int gp, int64_t D, const RaggedItem *items, int n_items,
+template <int FMT>
+int launch_ragged_quant(const DecodeDev &p, int gp, const RaggedItem *items, int n_items, const RaggedSeqSlots *seqs, int n_seq,
+                        bool any_split, hipStream_t s) {
+    switch (gp) {
+        case 8: return launch_ragged_gp<128, 8, FMT>(p, items, n_items, seqs, n_seq, any_split, s);
+        case 16: return launch_ragged_gp<128, 16, FMT>(p, items, n_items, seqs, n_seq, any_split, s);
+        default: return launch_ragged_gp<128, 32, FMT>(p, items, n_items, seqs, n_seq, any_split, s);
+    }
+}
+
+int launch_sdpa_decode_ragged_mfma(const DecodeDev &p, int kv_fmt, int gp, int64_t D, const RaggedItem *items, int n_items,
                                    const RaggedSeqSlots *seqs, int n_seq, bool any_split, hipStream_t s) {
+    if (kv_fmt == TROCM_Q8_0) return launch_ragged_quant<TROCM_Q8_0>(p, gp, items, n_items, seqs, n_seq, any_split, s);
+    if (kv_fmt == TROCM_Q4_0) return launch_ragged_quant<TROCM_Q4_0>(p, gp, items, n_items, seqs, n_seq, any_split, s);
     return D == 128 ? launch_ragged_d<128>(p, gp, items, n_items, seqs, n_seq, any_split, s)
                     : launch_ragged_d<64>(p, gp, items, n_items, seqs, n_seq, any_split, s);
 }
