@@ -36,8 +36,8 @@ HBM_PEAK_GBS = 8000.0
 # HBM traffic of one decode-attention launch at the default arguments (batch 8, context 8226 in the
 # kernel loop), from two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE), each
 # counter scaled by what it reads for the 128 MiB prefill copy of known size: FETCH_SIZE
-# 132105.6 x 1.9991 KiB + WRITE_SIZE 650 x 1.000 KiB.
-PMC_TRAFFIC_BYTES_B8_CTX8226 = int((132105.6 * 1.9991 + 650.0) * 1024)
+# 132350.8 x 1.9991 KiB + WRITE_SIZE 1226 x 1.000 KiB.
+PMC_TRAFFIC_BYTES_B8_CTX8226 = int((132350.8 * 1.9991 + 1226.0) * 1024)
 
 
 def cfg_seed(cfg, what):
@@ -307,7 +307,7 @@ def run_cfg4(ta, args):
             by = 2 * B * HKV * T * D * ek + 2 * B * HQ * D * 2
             res[f"{name}_ctx{T}"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by)}
     head = res["q8_0_ctx16384"]
-    roof = {"bound": "hbm", "kernel": "sdpa_decode_q_kernel<Q8_0,4>", "achieved": head["gbs"], "peak": HBM_PEAK_GBS,
+    roof = {"bound": "hbm", "kernel": "sdpa_decode_mfma_kernel<128,8,Q8_0>", "achieved": head["gbs"], "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4), "traffic": None}
     return base_line(args, "cfg4: decode over a Q8_0 / Q4_0 quantised KV cache (fused dequant), batch 8, contexts 4096 "
                      "and 16384, 1% outlier channels x20; attention launches only, rotating over 2-4 layers' caches; "
@@ -347,7 +347,7 @@ def run_cfg5(ta, args):
     tot = int(sum(c.len() for c in kcs))
     by = 2 * HKV * D * 2 * tot + 2 * n_seq * HQ * D * 2 + 2 * n_seq * HKV * D * 2
     us_k = time_calls(ta, lambda: ta.sdpa_decode_ragged(qs[0], kcs, vcs, workspace=ws, out=out), 20)
-    roof = {"bound": "hbm", "kernel": "sdpa_decode_mfma_ragged_kernel<128,8>", "achieved": round(by / us_k / 1e3, 1),
+    roof = {"bound": "hbm", "kernel": "sdpa_decode_mfma_ragged_kernel<128,8,F16>", "achieved": round(by / us_k / 1e3, 1),
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(by / us_k / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
             "kernel_us": round(us_k, 2), "algorithmic_bytes_per_launch": int(by)}
     st = pool.stats()
@@ -578,7 +578,7 @@ def main():
         "parity_max_abs_vs_oracle": err,
         "roofline": {
             "bound": "hbm",
-            "kernel": "sdpa_decode_mfma_kernel<128,8>",
+            "kernel": "sdpa_decode_mfma_kernel<128,8,F16>",
             "achieved": round(main_res["kernel_gbs"], 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
