@@ -250,7 +250,9 @@ int trocm_rotate_half(const void *input, void *out, int dtype, int rank, const i
  * owns one workspace and passes it to every call.  trocm_sdpa_workspace_init() must run
  * once on a new workspace (it zeroes the header area reserved for kernel-side counters);
  * kernels leave it ready for the next call.  Two calls that overlap in time must not share
- * a workspace.  The size covers decode for (batch, q_heads, head_dim) and, for q_len > 1,
+ * a workspace; calls that follow each other on one stream may, dense and ragged in any order
+ * (a ragged call keeps its launch plan in a second header area and refuses a workspace too
+ * small to have one).  The size covers decode for (batch, q_heads, head_dim) and, for q_len > 1,
  * the partial results of a prefill whose key range is split over workgroups; a call made
  * with a smaller (or NULL) workspace still succeeds, with fewer splits. */
 int trocm_sdpa_workspace_bytes(int64_t batch, int64_t q_heads, int64_t q_len, int64_t head_dim,
@@ -306,7 +308,9 @@ int trocm_window_kv_sdpa_eval(const void *q, const void *k_new, const void *v_ne
  * cache (batch == 1 each, same heads/head_dim/format) and its own length; one query token
  * per sequence.  q, out: [n_seq, q_heads, 1, head_dim].  The reference has no ragged batch:
  * its statement of the same result is a dense batch padded to the longest sequence with an
- * additive mask whose padded columns are <= -65504 (flash_sdpa.rs:261-268). */
+ * additive mask whose padded columns are <= -65504 (flash_sdpa.rs:261-268).  F16 and F32 caches,
+ * and Q8_0 / Q4_0 caches with 2..32 query heads per kv head, run as one launch (plus a merge launch
+ * when a sequence is cut into more than 8 pieces); other cases as one call per sequence. */
 int trocm_sdpa_decode_ragged(const void *q, int q_dtype, int64_t q_heads, int64_t n_seq,
                              trocm_kv_cache *const *k_caches, trocm_kv_cache *const *v_caches,
                              void *out, float scale, void *workspace, size_t workspace_bytes,
@@ -315,7 +319,8 @@ int trocm_sdpa_decode_ragged(const void *q, int q_dtype, int64_t q_heads, int64_
 /* One decode step of a ragged batch as one call: append k_new[i], v_new[i] (dense
  * [n_seq, kv_heads, 1, head_dim] of `dtype`) to sequence i's caches, then attend q[i] over them.
  * Per sequence this is InPlaceKvSdpaState::eval (inplace_kv_cache.rs:191-216).  On F32/F16 caches
- * the attention kernel stores the new tokens itself: one launch (plus the split merge) per step. */
+ * the attention kernel stores the new tokens itself: one launch (plus the split merge) per step;
+ * on quantised caches one launch quantises every sequence's new token and a second attends. */
 int trocm_inplace_kv_sdpa_eval_ragged(const void *q, const void *k_new, const void *v_new, int dtype,
                                       int64_t q_heads, int64_t n_seq, trocm_kv_cache *const *k_caches,
                                       trocm_kv_cache *const *v_caches, void *out, float scale,
