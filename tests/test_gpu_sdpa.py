@@ -112,6 +112,9 @@ def test_decode_split_k(rt, dt, B, Hq, Hkv, D, T):
 @pytest.mark.parametrize("dt,B,Hq,Hkv,D,T,mb,mh", [
     (np.float16, 2, 32, 8, 128, 3000, 2, 1), (np.float16, 2, 32, 8, 128, 1025, 1, 32), (np.float16, 3, 8, 8, 64, 333, 3, 8),
     (np.float32, 2, 8, 4, 64, 513, 2, 1), (np.float32, 1, 4, 2, 128, 200, 1, 4), (np.float16, 1, 16, 2, 128, 97, 1, 1),
+    # kv_len % 4 == 0 with grouped heads: the MFMA decode kernel (a partial last tile; 16 heads per kv head; group 3, d=64)
+    (np.float16, 2, 32, 8, 128, 2052, 1, 32), (np.float16, 1, 32, 2, 128, 516, 1, 1), (np.float16, 2, 24, 8, 64, 1000, 2, 24),
+    (np.float16, 8, 32, 8, 128, 8192, 8, 1),
 ])
 def test_decode_with_additive_mask(rt, kind, dt, B, Hq, Hkv, D, T, mb, mh):
     """Sq == 1 with a mask input [mask_b, mask_h, 1, T] (broadcast over batch and/or heads), the form in

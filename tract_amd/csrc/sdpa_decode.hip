@@ -457,7 +457,7 @@ int choose_decode_splits(int64_t BH, int64_t G, int n_tiles, int wg_per_cu) {
 
 int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
     if (a.Sq != 1) return 2;
-    {   // large head groups: the MFMA formulation (it declines masks, the fused append and f32)
+    {   // grouped heads: the MFMA formulation (it declines f32 and masks over rows whose length is not a multiple of 4)
         const int rc = launch_sdpa_decode_mfma(a, s);
         if (rc != 2) return rc;
     }

@@ -61,12 +61,14 @@ struct MfmaWork {
     int new_pos;                  // token stored by a fused append (-1: none)
     int *counter;                 // in-kernel merge by the last workgroup to arrive (dense batches, GP <= 8)
     int64_t part_first, part_stride;   // partial records of this sequence-head: first, first + stride, ...
+    const char *mask;             // additive mask row of this kv head's first query head, token 0 (MASK instantiations)
 };
 
 // FMT: TROCM_F16, or a block-quantised cache (TROCM_Q8_0 / TROCM_Q4_0, 32-element blocks): the codes are
 // dequantised on the way into the LDS tile, (code - zero) * d rounded once to f16 as the reference's
 // dequantisation rounds it, and everything after the tile is the f16 kernel.
-template <int D, int GP, int FMT>
+// MASK: an additive mask [mask_b, mask_h, 1, T] of f16 joins the scaled scores (f16 caches, dense batches).
+template <int D, int GP, int FMT, bool MASK = false>
 __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaWork &wk) {
     constexpr bool QUANT = FMT != TROCM_F16;
     constexpr int KS = D / 16;             // contraction steps of K.Q^T
@@ -203,9 +205,27 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
     // 16*(lane/16 % 2) + 4*(lane%4) of the 32-feature block
     const int vsrc_off = (4 * hb + ((lane & 15) >> 2)) * VROW + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
+    // this lane's mask values: its head's row, tokens 8*rq + 4*hb + 0..3 of the tile
+    const char *mask_lane = MASK ? wk.mask + (int64_t)min(l32, g - 1) * p.mask_stride_h + 8 * hb : nullptr;
     for (; t < tile_end; t += kWaves) {
         const int t0 = t * kTile;
         const bool more = t + kWaves < tile_end;
+        half4_t mk[MASK ? 4 : 1];
+        if constexpr (MASK) {   // asked for before the products with K, used after them
+            const char *mp = mask_lane + (int64_t)t0 * 2;
+            if (t0 + kTile <= T) {
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) mk[rq] = *reinterpret_cast<const half4_t *>(mp + 16 * rq);
+            } else {   // the row ends inside this tile
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int tok = t0 + 8 * rq + 4 * hb + i;
+                        mk[rq][i] = tok < T ? *reinterpret_cast<const _Float16 *>(mp + 16 * rq + 2 * i) : (_Float16)0.0f;
+                    }
+            }
+        }
         // ---- K tile -> LDS, the next tile's K into flight ----------------------------------------------
         if constexpr (QUANT) {
             stash_q(kpre, ksc, k_slot);
@@ -238,23 +258,26 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
             for (int r = 0; r < 16; r++) {
                 const int tok = t0 + 8 * (r >> 2) + 4 * hb + (r & 3);
                 s[r] = (t0 + kTile <= T || tok < T) ? s[r] * p.scale_log2 : -INFINITY;
+                if constexpr (MASK) s[r] = __builtin_fmaf((float)mk[r >> 2][r & 3], 1.4426950408889634f, s[r]);
                 tmax = fmaxf(tmax, s[r]);
             }
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float m_new = fmaxf(m_run, tmax);   // finite: every tile holds at least one valid token
+        const float m_new = fmaxf(m_run, tmax);   // finite without a mask: every tile holds at least one valid token
+        // a tile (so far: a row) masked out entirely with -inf must leave the state untouched, not NaN
+        const float m_ref = (MASK && m_new == -INFINITY) ? 0.0f : m_new;
         float psum = 0.0f;
         half8_t pf[2];
 #pragma unroll
         for (int st = 0; st < 2; st++)
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                const float pv = fast_exp2(s[8 * st + i] - m_new);
+                const float pv = fast_exp2(s[8 * st + i] - m_ref);
                 psum += pv;
                 pf[st][i] = (_Float16)pv;
             }
         const bool moved = m_new != m_run;
-        const float alpha = fast_exp2(m_run - m_new);
+        const float alpha = fast_exp2(m_run - m_ref);
         l_run = l_run * alpha + psum;
         m_run = m_new;
         if (__builtin_amdgcn_ballot_w64(moved) != 0) {
@@ -341,7 +364,7 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
 }
 
 // Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.
-template <int D, int GP, int FMT>
+template <int D, int GP, int FMT, bool MASK = false>
 __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev p) {
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     MfmaWork wk;
@@ -363,7 +386,8 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev
     wk.new_pos = p.k_new ? p.new_pos : -1;
     wk.counter = p.counters ? p.counters + bh : nullptr;
     wk.part_first = bh * p.nsplit, wk.part_stride = 1;
-    decode_mfma_body<D, GP, FMT>(p, wk);
+    wk.mask = MASK ? p.mask + (int64_t)b * p.mask_stride_b + (int64_t)kvh * p.g_real * p.mask_stride_h : nullptr;
+    decode_mfma_body<D, GP, FMT, MASK>(p, wk);
 }
 
 // Ragged batch: grid (work items, kv_heads); an item is a tile range of one sequence (the host's plan).
@@ -387,12 +411,16 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_ragged_kernel(De
     wk.new_pos = p.k_new ? it.T - 1 : -1;
     wk.counter = p.counters ? p.counters + (int64_t)it.seq * p.Hkv + kvh : nullptr;
     wk.part_first = (int64_t)it.slot0 * p.Hkv + kvh, wk.part_stride = p.Hkv;
+    wk.mask = nullptr;
     decode_mfma_body<D, GP, FMT>(p, wk);
 }
 
 template <int D, int GP, int FMT = TROCM_F16>
 int launch_gp(const DecodeDev &p, dim3 grid, hipStream_t s) {
-    hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, GP, FMT>), grid, dim3(kThreads), 0, s, p);
+    if (FMT == TROCM_F16 && p.mask)
+        hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, GP, TROCM_F16, true>), grid, dim3(kThreads), 0, s, p);
+    else
+        hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, GP, FMT>), grid, dim3(kThreads), 0, s, p);
     if (p.nsplit > 1 && p.counters == nullptr)
         hipLaunchKernelGGL((sdpa_decode_merge_kernel<__half, D, GP>), dim3(grid.y, grid.z, p.g_real), dim3(D), 0, s, p);
     hipError_t e = hipGetLastError();
@@ -496,7 +524,9 @@ int launch_sdpa_decode_quant_mfma(DecodeDev &p, int kv_fmt, int64_t B, void *wor
 }
 
 int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {
-    if (a.Sq != 1 || a.mask != nullptr) return 2;
+    if (a.Sq != 1) return 2;
+    // mask rows are read by 8-byte loads: [mask_b, mask_h, 1, Sk] with Sk % 4 == 0 (the vector-ALU kernel takes the others)
+    if (a.mask && (a.Sk % 4 != 0 || (uintptr_t)a.mask % 8 != 0 || a.k_new != nullptr)) return 2;
     if (a.kv_fmt != TROCM_F16 || a.q_dtype != TROCM_F16) return 2;
     if (a.D != 64 && a.D != 128) return 2;
     if (a.Hq % a.Hkv) return 2;
@@ -530,6 +560,11 @@ int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {
     if (p.k_new && (p.v_new == nullptr || (uintptr_t)p.k_new % 16 || (uintptr_t)p.v_new % 16)) return 2;
     p.part_ml = (float *)((char *)a.workspace + kWsCounterBytes);
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * gp;
+    if (a.mask) {   // [mask_b, mask_h, 1, Sk] dense f16
+        p.mask = (const char *)a.mask;
+        p.mask_stride_h = a.mask_h > 1 ? a.Sk * 2 : 0;
+        p.mask_stride_b = a.mask_b > 1 ? a.mask_h * a.Sk * 2 : 0;
+    }
     static const int tail = getenv("TROCM_DECODE_TAIL_MERGE") ? atoi(getenv("TROCM_DECODE_TAIL_MERGE")) : 1;
     if (tail && gp <= 8 && nsplit > 1 && nsplit <= kTailMergeMax && BH <= (int64_t)(kWsCounterBytes / sizeof(int))) p.counters = (int *)a.workspace;
     dim3 grid(nsplit, (unsigned)a.Hkv, (unsigned)a.B);
