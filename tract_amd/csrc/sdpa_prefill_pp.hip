@@ -23,6 +23,7 @@
 #include <hip/hip_fp16.h>
 #include <string.h>
 #include <stdlib.h>
+#include <type_traits>
 #include "common.h"
 
 namespace trocm {
@@ -369,7 +370,6 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
             pv(cur, pf);
         }
     }
-
     l_run += __shfl_xor(l_run, 32, 64);
     if (p.nsplit == 1) {
         if (!wave_has_queries || my_q >= p.Sq) return;
@@ -434,41 +434,15 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
     // The weights go through a wave-private corner of the (now idle) K tile buffer; the partial
     // outputs are laid out as the accumulators are, so each lane reads back exactly its own elements,
     // two splits in flight at a time.
-    constexpr int kMaxSplits = 16, kMergeBatch = 2;
+    constexpr int kMaxSplits = 16;
     auto aload_f = [](const float *a) { return __hip_atomic_load(a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
     float *wts = reinterpret_cast<float *>(&lds_k[0][0]) + w * (kMaxSplits * 32);
-    {
-        float mv[kMaxSplits], lv[kMaxSplits];
+    // One merge step for NS splits starting at s0: their outputs and, when WEIGHTS, the (m, l) records of
+    // MAXS splits are requested together; the weights go through LDS (lanes 32..63 need those of lanes 0..31).
+    auto load_outputs = [&](int s0, auto &raw, auto ns_tag) {
+        constexpr int NS = decltype(ns_tag)::value;
 #pragma unroll
-        for (int sp = 0; sp < kMaxSplits; sp++) {
-            const float *ml = p.part_ml + ((int64_t)min(sp, p.nsplit - 1) * p.n_wb + wb) * 64;
-            mv[sp] = aload_f(ml + l32);
-            lv[sp] = aload_f(ml + 32 + l32);
-        }
-        float mm = -INFINITY;
-#pragma unroll
-        for (int sp = 0; sp < kMaxSplits; sp++) mm = fmaxf(mm, mv[sp]);
-        const float m_ref = (mm == -INFINITY) ? 0.0f : mm;
-        float total = 0.0f;
-#pragma unroll
-        for (int sp = 0; sp < kMaxSplits; sp++) {
-            lv[sp] = sp < p.nsplit ? lv[sp] * fast_exp2(mv[sp] - m_ref) : 0.0f;
-            total += lv[sp];
-        }
-        const float inv = total > 0.0f ? 1.0f / total : 0.0f;
-        if (hb == 0) {
-#pragma unroll
-            for (int sp = 0; sp < kMaxSplits; sp++) wts[sp * 32 + l32] = lv[sp] * inv;
-        }
-    }
-#pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
-    for (int s0 = 0; s0 < p.nsplit; s0 += kMergeBatch) {
-        uint64_t raw[kMergeBatch][DB * 4];
-#pragma unroll
-        for (int j = 0; j < kMergeBatch; j++) {
+        for (int j = 0; j < NS; j++) {
             const _Float16 *po = p.part_o + ((int64_t)min(s0 + j, p.nsplit - 1) * p.n_wb + wb) * (32 * D) + l32 * 4;
 #pragma unroll
             for (int db = 0; db < DB; db++)
@@ -477,8 +451,36 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
                     raw[j][db * 4 + rq] = __hip_atomic_load(reinterpret_cast<const uint64_t *>(po + (8 * db + 2 * rq + hb) * 128),
                                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+    };
+    auto weights = [&](auto maxs_tag) {
+        constexpr int MAXS = decltype(maxs_tag)::value;
+        float mv[MAXS], lv[MAXS];
 #pragma unroll
-        for (int j = 0; j < kMergeBatch; j++) {
+        for (int sp = 0; sp < MAXS; sp++) {
+            const float *ml = p.part_ml + ((int64_t)min(sp, p.nsplit - 1) * p.n_wb + wb) * 64;
+            mv[sp] = aload_f(ml + l32);
+            lv[sp] = aload_f(ml + 32 + l32);
+        }
+        float mm = -INFINITY;
+#pragma unroll
+        for (int sp = 0; sp < MAXS; sp++) mm = fmaxf(mm, mv[sp]);
+        const float m_ref = (mm == -INFINITY) ? 0.0f : mm;
+        float total = 0.0f;
+#pragma unroll
+        for (int sp = 0; sp < MAXS; sp++) {
+            lv[sp] = sp < p.nsplit ? lv[sp] * fast_exp2(mv[sp] - m_ref) : 0.0f;
+            total += lv[sp];
+        }
+        const float inv = total > 0.0f ? 1.0f / total : 0.0f;
+        if (hb == 0) {
+#pragma unroll
+            for (int sp = 0; sp < MAXS; sp++) wts[sp * 32 + l32] = lv[sp] * inv;
+        }
+    };
+    auto accumulate = [&](int s0, auto &raw, auto ns_tag) {
+        constexpr int NS = decltype(ns_tag)::value;
+#pragma unroll
+        for (int j = 0; j < NS; j++) {
             const float wgt = s0 + j < p.nsplit ? wts[(s0 + j) * 32 + l32] : 0.0f;
 #pragma unroll
             for (int db = 0; db < DB; db++)
@@ -488,6 +490,27 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
 #pragma unroll
                     for (int i = 0; i < 4; i++) o[db][4 * rq + i] += wgt * (float)h4[i];
                 }
+        }
+    };
+    auto zero_o = [&]() {
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
+    };
+    if (p.nsplit <= 4) {   // the common case: everything in one round trip to the L2
+        uint64_t raw[4][DB * 4];
+        load_outputs(0, raw, std::integral_constant<int, 4>{});
+        weights(std::integral_constant<int, 4>{});
+        zero_o();
+        accumulate(0, raw, std::integral_constant<int, 4>{});
+    } else {
+        weights(std::integral_constant<int, kMaxSplits>{});
+        zero_o();
+        for (int s0 = 0; s0 < p.nsplit; s0 += 2) {
+            uint64_t raw[2][DB * 4];
+            load_outputs(s0, raw, std::integral_constant<int, 2>{});
+            accumulate(s0, raw, std::integral_constant<int, 2>{});
         }
     }
     if (my_q >= p.Sq) return;
