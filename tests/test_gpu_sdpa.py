@@ -372,6 +372,34 @@ def test_ragged_decode_over_quantised_caches(rt, fmt_name, Hq, Hkv, n_seq, lo, h
     check(out, q)
 
 
+def test_ragged_step_over_quantised_caches_with_f32_tokens(rt):
+    """f32 queries and new tokens over Q8_0 caches: no fast attention kernel takes f32 queries (one generic call
+    per sequence), but the step's tokens are still quantised by the one launch, from f32, to the oracle's blocks."""
+    rng = np.random.default_rng(91)
+    Hq, Hkv, D = 8, 2, 128
+    lens = [40, 7, 130]
+    kcs, vcs, ks, vs = [], [], [], []
+    for n in lens:
+        k = rng.standard_normal((1, Hkv, n, D), dtype=np.float32)
+        v = rng.standard_normal((1, Hkv, n, D), dtype=np.float32)
+        kc, vc = tract_amd.InPlaceKvCache(2, tract_amd.Q8_0), tract_amd.InPlaceKvCache(2, tract_amd.Q8_0)
+        kc.push(k), vc.push(v)
+        kcs.append(kc), vcs.append(vc), ks.append(k), vs.append(v)
+    q = rng.standard_normal((len(lens), Hq, 1, D), dtype=np.float32) / np.sqrt(D).astype(np.float32)
+    kn = rng.standard_normal((len(lens), Hkv, 1, D), dtype=np.float32)
+    vn = rng.standard_normal((len(lens), Hkv, 1, D), dtype=np.float32)
+    out = tract_amd.inplace_kv_sdpa_eval_ragged(tract_amd.DeviceTensor.from_numpy(q), tract_amd.DeviceTensor.from_numpy(kn),
+                                                tract_amd.DeviceTensor.from_numpy(vn), kcs, vcs).to_numpy()
+    for i, n in enumerate(lens):
+        k = np.concatenate([ks[i], kn[i:i + 1]], axis=2)
+        v = np.concatenate([vs[i], vn[i:i + 1]], axis=2)
+        kq, vq = orc.quant(orc.FMT_Q8_0, k), orc.quant(orc.FMT_Q8_0, v)
+        assert kcs[i].len() == n + 1
+        assert kcs[i].valid_contiguous().tobytes() == kq.tobytes() and vcs[i].valid_contiguous().tobytes() == vq.tobytes()
+        want = orc.flash_sdpa(q[i:i + 1], orc.dequant(orc.FMT_Q8_0, kq), orc.dequant(orc.FMT_Q8_0, vq), causal=True)
+        assert max_abs(out[i:i + 1], want) <= 1e-3, f"sequence {i}"
+
+
 def test_quantised_cache_with_f32_queries_uses_generic_kernel(rt):
     rng = np.random.default_rng(31)
     B, Hq, Hkv, T, D = 1, 4, 2, 50, 64
