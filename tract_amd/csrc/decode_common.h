@@ -234,6 +234,61 @@ __device__ __forceinline__ void tail_merge(const DecodeDev &p, int *counter, int
     }
 }
 
+// The same for up to kWideMergeMax splits (small batches: 32 splits at batch 1), with G * kWideMergeMax <=
+// kThreads: thread (h, sp) loads the (m, l) record of head h in split sp and the 32 threads of a head reduce
+// them to weights, which go through `lds_w` (G * kWideMergeMax floats of LDS that nothing else uses any more);
+// the outputs of all splits are requested before that, so the whole merge is one round trip to the L2 where
+// a merge launch costs a launch gap and a kernel.
+constexpr int kWideMergeMax = 32;
+template <typename T, int D, int G>
+__device__ __forceinline__ void tail_merge_wide(const DecodeDev &p, int *counter, int nsplit, int64_t first, int64_t stride,
+                                                T *out, int tid, float *lds_w) {
+    static_assert(G * kWideMergeMax <= kThreads, "one thread per (head, split)");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's partial stores have completed
+    __syncthreads();                                     // ... and so have the whole workgroup's
+    __shared__ int s_last_wide;
+    if (tid == 0) {
+        const int arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last_wide = arrived == nsplit - 1;
+        if (s_last_wide) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last_wide) return;
+    auto aload = [](const float *a) { return __hip_atomic_load(a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    constexpr int NE = (G * D + kThreads - 1) / kThreads;
+    const int64_t ml_step = stride * (2 * G), po_step = stride * (G * D);
+    float ov[NE][kWideMergeMax];
+#pragma unroll
+    for (int e = 0; e < NE; e++) {
+        const float *po = p.part_o + first * (G * D) + min(tid + e * kThreads, G * D - 1);
+#pragma unroll
+        for (int sp = 0; sp < kWideMergeMax; sp++) ov[e][sp] = aload(po + min(sp, nsplit - 1) * po_step);
+    }
+    if (tid < G * kWideMergeMax) {
+        const int h = tid / kWideMergeMax, sp = tid % kWideMergeMax;
+        const float *ml = p.part_ml + first * (2 * G) + min(sp, nsplit - 1) * ml_step + h;
+        const float m = aload(ml), l = aload(ml + G);
+        float mm = m;
+#pragma unroll
+        for (int d = 1; d < kWideMergeMax; d <<= 1) mm = fmaxf(mm, __shfl_xor(mm, d, 64));
+        const float f = sp < nsplit ? fast_exp2(m - (mm == -INFINITY ? 0.0f : mm)) : 0.0f;
+        float ll = l * f;
+#pragma unroll
+        for (int d = 1; d < kWideMergeMax; d <<= 1) ll += __shfl_xor(ll, d, 64);
+        lds_w[tid] = f / ll;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < NE; e++) {
+        const int idx = tid + e * kThreads;
+        const float *wh = lds_w + min(idx / D, G - 1) * kWideMergeMax;
+        float acc = 0.0f;
+#pragma unroll
+        for (int sp = 0; sp < kWideMergeMax; sp++) acc += ov[e][sp] * wh[sp];
+        if (idx < p.g_real * D) out[idx] = from_f32<T>(acc);
+    }
+}
+
 // Merge launch: grid (kv_heads, batch, real query heads per kv head), D threads; runs after the split
 // kernel on the same stream.
 template <typename T, int D, int G>

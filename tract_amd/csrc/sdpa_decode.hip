@@ -760,7 +760,7 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     const RaggedSeqSlots *d_slots = (const RaggedSeqSlots *)(d_items + n_items);
     // The MFMA kernel merges the splits of a sequence-head itself when none has more than it can hold in registers.
     static const int tail = getenv("TROCM_DECODE_TAIL_MERGE") ? atoi(getenv("TROCM_DECODE_TAIL_MERGE")) : 1;
-    if (tail && mfma_gp && mfma_gp <= 8 && any_split && max_split <= kTailMergeMax &&
+    if (tail && mfma_gp && mfma_gp <= 8 && any_split && max_split <= kWideMergeMax &&
         n_seq * Hkv <= (int64_t)(kWsCounterBytes / sizeof(int)))
         p.counters = (int *)workspace;
     if (mfma_gp) return launch_sdpa_decode_ragged_mfma(p, kv_fmt, mfma_gp, D, d_items, (int)n_items, d_slots, (int)n_seq, any_split, s);

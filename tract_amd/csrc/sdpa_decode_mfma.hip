@@ -359,7 +359,10 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
         }
     }
     if constexpr (GP <= 8) {   // (larger groups: the merge launch; the in-kernel merge would need too many registers)
-        if (wk.nsplit > 1 && wk.counter != nullptr) tail_merge<__half, D, GP>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
+        if (wk.nsplit > kTailMergeMax && wk.counter != nullptr)
+            tail_merge_wide<__half, D, GP>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid, reinterpret_cast<float *>(lds_raw));
+        else if (wk.nsplit > 1 && wk.counter != nullptr)
+            tail_merge<__half, D, GP>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
     }
 }
 
@@ -518,7 +521,7 @@ int launch_sdpa_decode_quant_mfma(DecodeDev &p, int kv_fmt, int64_t B, void *wor
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * gp;
     static const int tail = getenv("TROCM_DECODE_TAIL_MERGE") ? atoi(getenv("TROCM_DECODE_TAIL_MERGE")) : 1;
     p.counters = nullptr;
-    if (tail && gp <= 8 && nsplit > 1 && nsplit <= kTailMergeMax && BH <= (int64_t)(kWsCounterBytes / sizeof(int))) p.counters = (int *)workspace;
+    if (tail && gp <= 8 && nsplit > 1 && nsplit <= kWideMergeMax && BH <= (int64_t)(kWsCounterBytes / sizeof(int))) p.counters = (int *)workspace;
     dim3 grid(nsplit, (unsigned)p.Hkv, (unsigned)B);
     return kv_fmt == TROCM_Q8_0 ? launch_quant<TROCM_Q8_0>(p, gp, grid, s) : launch_quant<TROCM_Q4_0>(p, gp, grid, s);
 }
@@ -566,7 +569,7 @@ int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {
         p.mask_stride_b = a.mask_b > 1 ? a.mask_h * a.Sk * 2 : 0;
     }
     static const int tail = getenv("TROCM_DECODE_TAIL_MERGE") ? atoi(getenv("TROCM_DECODE_TAIL_MERGE")) : 1;
-    if (tail && gp <= 8 && nsplit > 1 && nsplit <= kTailMergeMax && BH <= (int64_t)(kWsCounterBytes / sizeof(int))) p.counters = (int *)a.workspace;
+    if (tail && gp <= 8 && nsplit > 1 && nsplit <= kWideMergeMax && BH <= (int64_t)(kWsCounterBytes / sizeof(int))) p.counters = (int *)a.workspace;
     dim3 grid(nsplit, (unsigned)a.Hkv, (unsigned)a.B);
     return a.D == 128 ? launch_d<128>(p, gp, grid, s) : launch_d<64>(p, gp, grid, s);
 }
