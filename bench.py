@@ -307,7 +307,7 @@ def run_cfg4(ta, args):
             by = 2 * B * HKV * T * D * ek + 2 * B * HQ * D * 2
             res[f"{name}_ctx{T}"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by)}
     head = res["q8_0_ctx16384"]
-    roof = {"bound": "hbm", "kernel": "sdpa_decode_mfma_kernel<128,8,Q8_0>", "achieved": head["gbs"], "peak": HBM_PEAK_GBS,
+    roof = {"bound": "hbm", "kernel": "sdpa_decode_mfma_kernel<128,8,Q8_0,false,true>", "achieved": head["gbs"], "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4), "traffic": None}
     return base_line(args, "cfg4: decode over a Q8_0 / Q4_0 quantised KV cache (fused dequant), batch 8, contexts 4096 "
                      "and 16384, 1% outlier channels x20; attention launches only, rotating over 2-4 layers' caches; "
@@ -347,7 +347,7 @@ def run_cfg5(ta, args):
     tot = int(sum(c.len() for c in kcs))
     by = 2 * HKV * D * 2 * tot + 2 * n_seq * HQ * D * 2 + 2 * n_seq * HKV * D * 2
     us_k = time_calls(ta, lambda: ta.sdpa_decode_ragged(qs[0], kcs, vcs, workspace=ws, out=out), 20)
-    roof = {"bound": "hbm", "kernel": "sdpa_decode_mfma_ragged_kernel<128,8,F16>", "achieved": round(by / us_k / 1e3, 1),
+    roof = {"bound": "hbm", "kernel": "sdpa_decode_mfma_ragged_kernel<128,8,F16,true>", "achieved": round(by / us_k / 1e3, 1),
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(by / us_k / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
             "kernel_us": round(us_k, 2), "algorithmic_bytes_per_launch": int(by)}
     st = pool.stats()
@@ -578,7 +578,7 @@ def main():
         "parity_max_abs_vs_oracle": err,
         "roofline": {
             "bound": "hbm",
-            "kernel": "sdpa_decode_mfma_kernel<128,8,F16>",
+            "kernel": "sdpa_decode_mfma_kernel<128,8,F16,false,true>",
             "achieved": round(main_res["kernel_gbs"], 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",

@@ -68,8 +68,13 @@ struct MfmaWork {
 // dequantised on the way into the LDS tile, (code - zero) * d rounded once to f16 as the reference's
 // dequantisation rounds it, and everything after the tile is the f16 kernel.
 // MASK: an additive mask [mask_b, mask_h, 1, T] of f16 joins the scaled scores (f16 caches, dense batches).
-template <int D, int GP, int FMT, bool MASK = false>
+// W16: the tiles are 16 heads wide (v_mfma_f32_16x16x32_f16, up to 16 heads per kv head): half the matrix time,
+// half the accumulator and query registers, and a lane exponentiates 8 scores instead of 16.  A lane then owns
+// head lane % 16 and, of a 32-token tile, tokens 4*(lane/16) + 0..3 and 16 + 4*(lane/16) + 0..3; of the output,
+// features 16*fb + 4*(lane/16) + 0..3 of every 16-feature block fb.
+template <int D, int GP, int FMT, bool MASK = false, bool W16 = false>
 __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaWork &wk) {
+    static_assert(!(W16 && MASK) && (!W16 || GP <= 16), "the 16-wide layout: no mask input, at most 16 heads");
     constexpr bool QUANT = FMT != TROCM_F16;
     constexpr int KS = D / 16;             // contraction steps of K.Q^T
     constexpr int DB = D / 32;             // 32-feature blocks of the output
@@ -88,12 +93,14 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, hb = lane >> 5;
+    const int l16 = lane & 15, q4 = lane >> 4;
+    const int hcol = W16 ? l16 : l32;   // the head (column of the score tile) of this lane
     const int kvh = wk.kvh, b = wk.seq;
     const int g = p.g_real;
     _Float16 *tile = reinterpret_cast<_Float16 *>(lds_raw + w * kTileBytes);
 
     const int64_t head0 = (int64_t)b * p.Hq + (int64_t)kvh * g;
-    const _Float16 *qrow = reinterpret_cast<const _Float16 *>(p.q) + (head0 + min(l32, g - 1)) * D;
+    const _Float16 *qrow = reinterpret_cast<const _Float16 *>(p.q) + (head0 + min(hcol, g - 1)) * D;
     const char *kbase = wk.kbase, *vbase = wk.vbase;
     const int T = wk.T;
     const int tile_begin = wk.tile_begin, tile_end = wk.tile_end;
@@ -187,23 +194,29 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
             fetch(vbase, p.v_new, t, vpre);
         }
     }
-    // Q^T fragments: row (head) = lane % 32, features 16*ks + 8*hb .. +8
-    half8_t qf[KS];
+    // Q^T fragments: row (head) = lane % 32, features 16*ks + 8*hb .. +8 (16-wide: lane % 16, 32*ks + 8*(lane/16) .. +8)
+    constexpr int NQF = W16 ? D / 32 : KS;
+    half8_t qf[NQF];
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) qf[ks] = *reinterpret_cast<const half8_t *>(qrow + 16 * ks + 8 * hb);
+    for (int ks = 0; ks < NQF; ks++)
+        qf[ks] = *reinterpret_cast<const half8_t *>(W16 ? qrow + 32 * ks + 8 * q4 : qrow + 16 * ks + 8 * hb);
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) asm volatile("" : "+v"(qf[ks]));   // settled here, not at first use inside the loop
+    for (int ks = 0; ks < NQF; ks++) asm volatile("" : "+v"(qf[ks]));   // settled here, not at first use inside the loop
 
     float m_run = -INFINITY, l_run = 0.0f;   // log2 domain, already scaled
-    float16_t o[DB];
+    float16_t o[W16 ? 1 : DB];
+    float4_t o16[W16 ? D / 16 : 1];
 #pragma unroll
-    for (int db = 0; db < DB; db++)
+    for (int db = 0; db < (W16 ? 1 : DB); db++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
+#pragma unroll
+    for (int fb = 0; fb < (W16 ? D / 16 : 1); fb++) o16[fb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
     // this lane as a SOURCE of the transposing loads: key row (lane%16)/4 of a group of four, features
-    // 16*(lane/16 % 2) + 4*(lane%4) of the 32-feature block
-    const int vsrc_off = (4 * hb + ((lane & 15) >> 2)) * VROW + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    // 16*(lane/16 % 2) + 4*(lane%4) of the 32-feature block (16-wide: token group lane/16, features 4*(lane%4))
+    const int vsrc_off = W16 ? (4 * q4 + (l16 >> 2)) * VROW + 4 * (l16 & 3)
+                             : (4 * hb + ((lane & 15) >> 2)) * VROW + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
     // this lane's mask values: its head's row, tokens 8*rq + 4*hb + 0..3 of the tile
     const char *mask_lane = MASK ? wk.mask + (int64_t)min(l32, g - 1) * p.mask_stride_h + 8 * hb : nullptr;
@@ -235,7 +248,50 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
             for (int j = 0; j < NLD; j++) *reinterpret_cast<u32x4 *>(tile + k_slot[j]) = kpre[j];
             if (more) fetch(kbase, p.k_new, t + kWaves, kpre);
         }
+        half8_t pf16;
+        if constexpr (W16) {
+            // ---- S^T = K Q^T: two blocks of 16 tokens x 16 heads --------------------------------------------
+            float4_t s16[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+            const _Float16 *kt16 = tile + l16 * KROW + 8 * q4;
+#pragma unroll
+            for (int ks = 0; ks < D / 32; ks++)
+#pragma unroll
+                for (int mb = 0; mb < 2; mb++) {
+                    const half8_t kf = *reinterpret_cast<const half8_t *>(kt16 + 16 * mb * KROW + 32 * ks);
+                    s16[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[ks], s16[mb], 0, 0, 0);
+                }
+            // ---- online softmax of this lane's head over its 8 tokens: t0 + 16*mb + 4*(lane/16) + r ---------
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int tok = t0 + 16 * mb + 4 * q4 + r;
+                    s16[mb][r] = (t0 + kTile <= T || tok < T) ? s16[mb][r] * p.scale_log2 : -INFINITY;
+                    tmax = fmaxf(tmax, s16[mb][r]);
+                }
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+            const float m_new = fmaxf(m_run, tmax);   // finite: every tile holds at least one valid token
+            float psum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float pv = fast_exp2(s16[i >> 2][i & 3] - m_new);
+                psum += pv;
+                pf16[i] = (_Float16)pv;
+            }
+            const bool moved = m_new != m_run;
+            const float alpha = fast_exp2(m_run - m_new);
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
+            if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+                for (int fb = 0; fb < D / 16; fb++) o16[fb] *= alpha;
+            }
+        }
         // ---- S^T = K Q^T: 32 tokens x 32 rows ------------------------------------------------------------
+        half8_t pf[2];
+        if constexpr (!W16) {
         float16_t s;
 #pragma unroll
         for (int r = 0; r < 16; r++) s[r] = 0.0f;
@@ -267,7 +323,6 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
         // a tile (so far: a row) masked out entirely with -inf must leave the state untouched, not NaN
         const float m_ref = (MASK && m_new == -INFINITY) ? 0.0f : m_new;
         float psum = 0.0f;
-        half8_t pf[2];
 #pragma unroll
         for (int st = 0; st < 2; st++)
 #pragma unroll
@@ -286,6 +341,7 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
 #pragma unroll
                 for (int r = 0; r < 16; r++) o[db][r] *= alpha;
         }
+        }
         // ---- V tile -> the same LDS tile (every K fragment has been consumed), next V into flight ------
         if constexpr (QUANT) {
             stash_q(vpre, vsc, v_slot);
@@ -297,22 +353,43 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
         }
         // ---- O^T += V^T P^T ---------------------------------------------------------------------------------
         const _Float16 *vsrc = tile + vsrc_off;
+        if constexpr (W16) {
 #pragma unroll
-        for (int st = 0; st < 2; st++)
-#pragma unroll
-            for (int db = 0; db < DB; db++) {
-                const half4_t lo = lds_read_tr16(vsrc + (16 * st) * VROW + 32 * db);      // tokens 16st + 4hb + 0..3
-                const half4_t hi = lds_read_tr16(vsrc + (16 * st + 8) * VROW + 32 * db);  // tokens 16st + 8 + 4hb + 0..3
+            for (int fb = 0; fb < D / 16; fb++) {
+                const half4_t lo = lds_read_tr16(vsrc + 16 * fb);               // tokens 4*(lane/16) + 0..3
+                const half4_t hi = lds_read_tr16(vsrc + 16 * VROW + 16 * fb);   // tokens 16 + 4*(lane/16) + 0..3
                 const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[st], o[db], 0, 0, 0);
+                o16[fb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf16, o16[fb], 0, 0, 0);
             }
+        } else {
+#pragma unroll
+            for (int st = 0; st < 2; st++)
+#pragma unroll
+                for (int db = 0; db < DB; db++) {
+                    const half4_t lo = lds_read_tr16(vsrc + (16 * st) * VROW + 32 * db);      // tokens 16st + 4hb + 0..3
+                    const half4_t hi = lds_read_tr16(vsrc + (16 * st + 8) * VROW + 32 * db);  // tokens 16st + 8 + 4hb + 0..3
+                    const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[st], o[db], 0, 0, 0);
+                }
+        }
     }
+    if constexpr (W16) l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
 
     // ---- merge the 4 waves through LDS (the K/V tiles are dead) --------------------------------------------
     __syncthreads();
     float *comb = reinterpret_cast<float *>(lds_raw);   // [kWaves][GP*D + 2*GP]
-    if (l32 < GP) {
+    if constexpr (W16) {
+        if (l16 < GP) {
+            float *cw = comb + w * kCombStride;
+#pragma unroll
+            for (int fb = 0; fb < D / 16; fb++) *reinterpret_cast<float4_t *>(cw + l16 * D + 16 * fb + 4 * q4) = o16[fb];
+            if (q4 == 0) {
+                cw[GP * D + l16] = m_run;
+                cw[GP * D + GP + l16] = l_run;
+            }
+        }
+    } else if (l32 < GP) {
         float *cw = comb + w * kCombStride;
 #pragma unroll
         for (int db = 0; db < DB; db++)
@@ -367,7 +444,7 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
 }
 
 // Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.
-template <int D, int GP, int FMT, bool MASK = false>
+template <int D, int GP, int FMT, bool MASK = false, bool W16 = false>
 __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev p) {
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     MfmaWork wk;
@@ -390,11 +467,11 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev
     wk.counter = p.counters ? p.counters + bh : nullptr;
     wk.part_first = bh * p.nsplit, wk.part_stride = 1;
     wk.mask = MASK ? p.mask + (int64_t)b * p.mask_stride_b + (int64_t)kvh * p.g_real * p.mask_stride_h : nullptr;
-    decode_mfma_body<D, GP, FMT, MASK>(p, wk);
+    decode_mfma_body<D, GP, FMT, MASK, W16>(p, wk);
 }
 
 // Ragged batch: grid (work items, kv_heads); an item is a tile range of one sequence (the host's plan).
-template <int D, int GP, int FMT>
+template <int D, int GP, int FMT, bool W16 = false>
 __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_ragged_kernel(DecodeDev p, const RaggedItem *__restrict__ items) {
     const RaggedItem it = items[blockIdx.x];
     const int kvh = blockIdx.y;
@@ -415,13 +492,24 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_ragged_kernel(De
     wk.counter = p.counters ? p.counters + (int64_t)it.seq * p.Hkv + kvh : nullptr;
     wk.part_first = (int64_t)it.slot0 * p.Hkv + kvh, wk.part_stride = p.Hkv;
     wk.mask = nullptr;
-    decode_mfma_body<D, GP, FMT>(p, wk);
+    decode_mfma_body<D, GP, FMT, false, W16>(p, wk);
+}
+
+// Up to 16 heads per kv head: the 16-wide tiles (batch 8, 8226 tokens, f16: 49.3 -> 48.5 us; batch 1 15.4 -> 14.5 us;
+// Q8_0 at 16384 tokens 57-59 -> 55.5 us, Q4_0 46-48 -> 45 us; three workgroups per CU, which the Q8_0 variant reaches
+// at 168 registers, gain nothing: the loop is bound by instruction issue).  TROCM_DECODE_MFMA16 = 0 / 1 / 2 selects
+// never / quantised formats only / always.
+bool use_16_wide(int fmt) {
+    static const int mode = getenv("TROCM_DECODE_MFMA16") ? atoi(getenv("TROCM_DECODE_MFMA16")) : 2;
+    return mode == 2 || (mode == 1 && fmt != TROCM_F16);
 }
 
 template <int D, int GP, int FMT = TROCM_F16>
 int launch_gp(const DecodeDev &p, dim3 grid, hipStream_t s) {
     if (FMT == TROCM_F16 && p.mask)
         hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, GP, TROCM_F16, true>), grid, dim3(kThreads), 0, s, p);
+    else if (GP <= 16 && use_16_wide(FMT))
+        hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, (GP <= 16 ? GP : 16), FMT, false, true>), grid, dim3(kThreads), 0, s, p);
     else
         hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, GP, FMT>), grid, dim3(kThreads), 0, s, p);
     if (p.nsplit > 1 && p.counters == nullptr)
@@ -452,7 +540,10 @@ int launch_quant(const DecodeDev &p, int gp, dim3 grid, hipStream_t s) {
 template <int D, int GP, int FMT = TROCM_F16>
 int launch_ragged_gp(const DecodeDev &p, const RaggedItem *items, int n_items, const RaggedSeqSlots *seqs, int n_seq,
                      bool any_split, hipStream_t s) {
-    hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<D, GP, FMT>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+    if (GP <= 16 && use_16_wide(FMT))
+        hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<D, (GP <= 16 ? GP : 16), FMT, true>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+    else
+        hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<D, GP, FMT>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
     if (any_split && !p.counters)   // with counters the last workgroup of a sequence-head has merged it
         hipLaunchKernelGGL((sdpa_decode_ragged_merge_kernel<__half, D, GP>), dim3(p.Hkv, n_seq, p.g_real), dim3(D), 0, s, p, seqs);
     hipError_t e = hipGetLastError();
