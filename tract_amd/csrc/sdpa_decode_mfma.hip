@@ -74,7 +74,7 @@ struct MfmaWork {
 // features 16*fb + 4*(lane/16) + 0..3 of every 16-feature block fb.
 template <int D, int GP, int FMT, bool MASK = false, bool W16 = false>
 __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaWork &wk) {
-    static_assert(!(W16 && MASK) && (!W16 || GP <= 16), "the 16-wide layout: no mask input, at most 16 heads");
+    static_assert(!W16 || GP <= 16, "the 16-wide layout: at most 16 heads");
     constexpr bool QUANT = FMT != TROCM_F16;
     constexpr int KS = D / 16;             // contraction steps of K.Q^T
     constexpr int DB = D / 32;             // 32-feature blocks of the output
@@ -219,23 +219,26 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
                              : (4 * hb + ((lane & 15) >> 2)) * VROW + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
     // this lane's mask values: its head's row, tokens 8*rq + 4*hb + 0..3 of the tile
-    const char *mask_lane = MASK ? wk.mask + (int64_t)min(l32, g - 1) * p.mask_stride_h + 8 * hb : nullptr;
+    // (16-wide: tokens 16*mb + 4*(lane/16) + 0..3)
+    const char *mask_lane = MASK ? wk.mask + (int64_t)min(hcol, g - 1) * p.mask_stride_h + 8 * (W16 ? q4 : hb) : nullptr;
     for (; t < tile_end; t += kWaves) {
         const int t0 = t * kTile;
         const bool more = t + kWaves < tile_end;
-        half4_t mk[MASK ? 4 : 1];
+        constexpr int NMK = W16 ? 2 : 4;          // groups of 4 consecutive tokens this lane owns in a tile
+        constexpr int kMkStep = W16 ? 16 : 8;     // tokens between them
+        half4_t mk[MASK ? NMK : 1];
         if constexpr (MASK) {   // asked for before the products with K, used after them
             const char *mp = mask_lane + (int64_t)t0 * 2;
             if (t0 + kTile <= T) {
 #pragma unroll
-                for (int rq = 0; rq < 4; rq++) mk[rq] = *reinterpret_cast<const half4_t *>(mp + 16 * rq);
+                for (int rq = 0; rq < NMK; rq++) mk[rq] = *reinterpret_cast<const half4_t *>(mp + 2 * kMkStep * rq);
             } else {   // the row ends inside this tile
 #pragma unroll
-                for (int rq = 0; rq < 4; rq++)
+                for (int rq = 0; rq < NMK; rq++)
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        const int tok = t0 + 8 * rq + 4 * hb + i;
-                        mk[rq][i] = tok < T ? *reinterpret_cast<const _Float16 *>(mp + 16 * rq + 2 * i) : (_Float16)0.0f;
+                        const int tok = t0 + kMkStep * rq + 4 * (W16 ? q4 : hb) + i;
+                        mk[rq][i] = tok < T ? *reinterpret_cast<const _Float16 *>(mp + 2 * kMkStep * rq + 2 * i) : (_Float16)0.0f;
                     }
             }
         }
@@ -268,20 +271,22 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
                 for (int r = 0; r < 4; r++) {
                     const int tok = t0 + 16 * mb + 4 * q4 + r;
                     s16[mb][r] = (t0 + kTile <= T || tok < T) ? s16[mb][r] * p.scale_log2 : -INFINITY;
+                    if constexpr (MASK) s16[mb][r] = __builtin_fmaf((float)mk[mb][r], 1.4426950408889634f, s16[mb][r]);
                     tmax = fmaxf(tmax, s16[mb][r]);
                 }
             tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-            const float m_new = fmaxf(m_run, tmax);   // finite: every tile holds at least one valid token
+            const float m_new = fmaxf(m_run, tmax);   // finite without a mask: every tile holds at least one valid token
+            const float m_ref16 = (MASK && m_new == -INFINITY) ? 0.0f : m_new;   // masked out entirely with -inf: no NaN
             float psum = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                const float pv = fast_exp2(s16[i >> 2][i & 3] - m_new);
+                const float pv = fast_exp2(s16[i >> 2][i & 3] - m_ref16);
                 psum += pv;
                 pf16[i] = (_Float16)pv;
             }
             const bool moved = m_new != m_run;
-            const float alpha = fast_exp2(m_run - m_new);
+            const float alpha = fast_exp2(m_run - m_ref16);
             l_run = l_run * alpha + psum;
             m_run = m_new;
             if (__builtin_amdgcn_ballot_w64(moved) != 0) {
@@ -506,7 +511,9 @@ bool use_16_wide(int fmt) {
 
 template <int D, int GP, int FMT = TROCM_F16>
 int launch_gp(const DecodeDev &p, dim3 grid, hipStream_t s) {
-    if (FMT == TROCM_F16 && p.mask)
+    if (FMT == TROCM_F16 && p.mask && GP <= 16 && use_16_wide(FMT))
+        hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, (GP <= 16 ? GP : 16), TROCM_F16, true, true>), grid, dim3(kThreads), 0, s, p);
+    else if (FMT == TROCM_F16 && p.mask)
         hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, GP, TROCM_F16, true>), grid, dim3(kThreads), 0, s, p);
     else if (GP <= 16 && use_16_wide(FMT))
         hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, (GP <= 16 ? GP : 16), FMT, false, true>), grid, dim3(kThreads), 0, s, p);
