@@ -304,8 +304,15 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
             for (int i = 0; i < 8; i++) {
                 const float sx = s[st >> 1][8 * (st & 1) + i];
                 float pv = fast_exp2(MASK ? sx - m_ref : __builtin_fmaf(sx, p.scale_log2, -m_ref));
-                psum += pv;
                 pf[st][i] = (_Float16)pv;
+            }
+            // the row sum is taken over the f16 values that enter the product with V (one v_dot2 per pair
+            // instead of two additions, and numerator and denominator see the same rounding)
+            const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const half2_t pair = {pf[st][2 * i], pf[st][2 * i + 1]};
+                psum = __builtin_amdgcn_fdot2(pair, ones, psum, false);
             }
         }
         const bool moved = m_new != m_run;
