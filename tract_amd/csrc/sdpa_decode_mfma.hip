@@ -1,24 +1,26 @@
-// Split-K flash-decode attention with grouped query heads (q_len == 1, 2..32 query heads per kv
-// head, f16): gfx950.
+// Split-K flash-decode attention with grouped query heads (q_len == 1, 2..32 query heads per kv head, f16
+// queries) over f16, Q8_0 or Q4_0 caches, dense or ragged batches: gfx950.
 //
 // The vector-ALU decode kernel (sdpa_decode.hip) spends one v_dot2 per (head, 2 features) and one fma
 // per (head, feature) of every token; with 8 heads per kv head that is about 970 vector instructions
 // per wave and 32-token tile, and the kernel is bound by them, not by HBM (batch 8, 8192 tokens:
 // 84.5 us against 47 us for 4 heads per kv head).  Here the G query heads of a kv head are the
-// *rows* of a 32-row MFMA tile: S^T = K.Q^T and O^T = V^T.P^T with v_mfma_f32_32x32x16_f16, the same
-// transposed formulation as the prefill kernel, with a head where that kernel has a query.  Only G
-// of the 32 rows are live, which the matrix pipe absorbs easily (16 MFMAs per 16 KiB of K and V);
-// what matters is that the vector work per tile drops to the softmax of 16 values per lane.
+// *columns* of MFMA tiles: S^T = K.Q^T and O^T = V^T.P^T, the same transposed formulation as the prefill
+// kernel, with a head where that kernel has a query.  Only G of a tile's 16 (v_mfma_f32_16x16x32_f16, up
+// to 16 heads) or 32 (v_mfma_f32_32x32x16_f16) columns are live, which the matrix pipe absorbs easily;
+// what matters is that the vector work per tile drops to the softmax of 8 or 16 values per lane.
 //
-// Work decomposition: grid (splits, kv_heads, batch), 4 waves; wave w takes 32-token tiles w, w+4, ...
-// of its split.  Per tile: K rows global -> registers (one tile ahead, non-temporal) -> a wave-private
-// LDS tile -> A fragments; softmax in registers (a lane owns one head and 16 of the 32 tokens); V
-// rows the same way into the same LDS tile (K is dead by then) -> transposing LDS reads -> A
-// fragments of the second product.  Waves are merged through LDS, splits through the workspace: by the
-// last workgroup to arrive (up to 8 heads per kv head) or by the merge launch, both shared with the other
-// decode kernels.  A step's new token can be handed in and is stored to the cache by the kernel.
+// Work decomposition: grid (splits, kv_heads, batch) or (work items, kv_heads), 4 waves; wave w takes
+// 32-token tiles w, w+4, ... of its range.  Per tile: K rows global -> registers (one tile ahead,
+// non-temporal) -> a wave-private LDS tile (block-quantised rows are dequantised on the way) -> A
+// fragments; softmax in registers; V rows the same way into the same LDS tile (K is dead by then) ->
+// transposing LDS reads -> A fragments of the second product.  Waves are merged through LDS, splits through
+// the workspace: by the last workgroup to arrive (up to 8 heads per kv head, up to 32 splits) or by the merge
+// launch, both shared with the other decode kernels.  A step's new token can be handed in and is stored to
+// the cache by the kernel (f16 caches); an additive mask row per head can join the scores (f16 caches).
 //
-// Roofline: HBM-bound.  Algorithmic bytes as for sdpa_decode.hip.
+// Roofline: HBM-bound (f16) / bound by vector-instruction issue (quantised).  Algorithmic bytes as for
+// sdpa_decode.hip and sdpa_decode_quant.hip.
 #include "decode_common.h"
 
 namespace trocm {
