@@ -433,6 +433,13 @@ def run_ops(ta, args):
     for name, masked in (("decode_b8_ctx8192_padding_mask", True), ("decode_b8_ctx8192_no_mask", False)):
         us = time_calls(ta, lambda: one_masked(masked), 100)
         res[name] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by)}
+    # the reference's statement of a ragged batch: padded to 8192 tokens, sequence b holds 8192 - 1024 * b of them
+    pad2 = np.zeros((B, 1, 1, T), np.float16)
+    for b in range(B):
+        pad2[b, :, :, T - 1024 * b:] = np.finfo(np.float16).min
+    pad, by2 = ta.DeviceTensor.from_numpy(pad2), sum(algorithmic_bytes(1, T - 1024 * b) for b in range(B))
+    us = time_calls(ta, lambda: one_masked(True), 100)
+    res["decode_b8_padded_to_8192_lens_8192_down_to_1024"] = {"us": round(us, 2), "gbs": round(by2 / us / 1e3, 1), "bytes": int(by2)}
     Sq, Sk = 512, 4096
     qp = ta.DeviceTensor.from_numpy((rng.standard_normal((1, HQ, Sq, D)) / np.sqrt(D)).astype(np.float16))
     op = ta.DeviceTensor((1, HQ, Sq, D), np.float16)

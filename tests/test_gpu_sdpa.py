@@ -144,6 +144,38 @@ def test_decode_with_additive_mask(rt, kind, dt, B, Hq, Hkv, D, T, mb, mh):
     assert max_abs(got, cases.textbook_sdpa(q, k, v, mask)) <= (2e-3 if dt == np.float16 else 2e-5)
 
 
+def test_padded_batch_mask_skips_the_padding(rt):
+    """A batch padded to its longest sequence with one mask row per sequence (finite minimum or -inf on the
+    padded columns, flash_sdpa.rs:261-268): the decode kernel divides only the unpadded tokens among its
+    workgroups; results as for any mask.  A row masked out entirely keeps all its tokens (uniform weights)."""
+    rng = np.random.default_rng(515)
+    B, Hq, Hkv, D, T = 6, 32, 8, 128, 4096
+    lens = [4096, 1, 37, 2048, 4095, 0]     # 0: the whole row is masked
+    q = (rng.standard_normal((B, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    k = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(np.float16)
+    for lo in (float(np.finfo(np.float16).min), -np.inf):
+        mask = np.zeros((B, 1, 1, T), dtype=np.float32)
+        for b, n in enumerate(lens):
+            mask[b, 0, 0, n:] = lo
+        if lo == -np.inf:
+            mask[5] = float(np.finfo(np.float16).min)   # (all -inf would be NaN in the reference too)
+        mask = mask.astype(np.float16)
+        got = tract_amd.Sdpa(datum_type=np.float16).eval(q, k, v, mask).to_numpy()
+        assert not np.isnan(got).any()
+        # (the reference's flash kernel skips key tiles masked below -65503 and returns zeros for the row that is
+        # masked out entirely, flash_sdpa.rs:261-268, where its naive Sdpa and the textbook weigh that row's
+        # tokens alike: the row is compared with the textbook only)
+        assert max_abs(got[:5], orc.flash_sdpa(q, k, v, mask=mask)[:5]) <= 2e-2
+        assert max_abs(got, cases.textbook_sdpa(q, k, v, mask)) <= 2e-3
+        # a hole in the middle of the kept part stays a hole, and a token that counts after padding is kept
+        mask2 = mask.copy()
+        mask2[3, 0, 0, 100:1000] = lo
+        mask2[2, 0, 0, 3000] = 0
+        got = tract_amd.Sdpa(datum_type=np.float16).eval(q, k, v, mask2).to_numpy()
+        assert max_abs(got, cases.textbook_sdpa(q, k, v, mask2)) <= 2e-3
+
+
 _ODD_GROUPS = [(np.float16, 24, 8, 128, 1500), (np.float16, 14, 2, 128, 3000), (np.float16, 12, 2, 128, 700),
                (np.float16, 10, 2, 128, 333), (np.float32, 6, 2, 64, 513), (np.float16, 21, 3, 64, 200)]
 

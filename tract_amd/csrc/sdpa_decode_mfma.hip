@@ -450,6 +450,33 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
     }
 }
 
+// The reference states a ragged batch as a dense batch padded to the longest sequence, with a mask row per
+// sequence whose padded columns hold the format's minimum or -inf (flash_sdpa.rs:261-268).  The tokens of such a
+// suffix weigh exactly nothing (their exponentials underflow to zero next to any token that counts), so the
+// workgroups of a sequence find where it starts and divide only the tokens before it among themselves.
+// Returns the number of leading columns to keep: one past the last column of `row` above -60000, or T when no
+// column is (a row masked out entirely keeps its tokens: they then weigh the same, as in the reference).
+// All threads of the workgroup call it; `red` is kWaves ints of LDS.
+__device__ __forceinline__ int mask_row_len(const _Float16 *__restrict__ row, int T, int tid, int *red) {
+    int best = -1;   // (T % 4 == 0 and 8-byte aligned rows: checked on the host)
+#pragma unroll 8
+    for (int c = tid * 4; c < T; c += kThreads * 4) {
+        const half4_t v = *reinterpret_cast<const half4_t *>(row + c);
+        const _Float16 big = fmaxf(fmaxf((float)v[0], (float)v[1]), fmaxf((float)v[2], (float)v[3]));
+        if (big > (_Float16)-60000.0f) {   // the highest column of these four that counts
+            const int i = v[3] > (_Float16)-60000.0f ? 3 : v[2] > (_Float16)-60000.0f ? 2 : v[1] > (_Float16)-60000.0f ? 1 : 0;
+            best = c + i;   // columns grow with the loop: the last one found is the highest
+        }
+    }
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) best = max(best, __shfl_xor(best, d, 64));
+    if ((tid & 63) == 0) red[tid >> 6] = best;
+    __syncthreads();
+#pragma unroll
+    for (int ww = 0; ww < kWaves; ww++) best = max(best, red[ww]);
+    return best < 0 ? T : best + 1;
+}
+
 // Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.
 template <int D, int GP, int FMT, bool MASK = false, bool W16 = false>
 __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev p) {
@@ -464,9 +491,17 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev
         wk.vsbase = p.v_scales + (int64_t)b * p.sc_stride_b + (int64_t)kvh * p.sc_stride_h;
     }
     wk.T = p.T;
-    const int n_tiles = (p.T + kTile - 1) / kTile;
-    wk.tile_begin = split * p.tiles_per_split;
-    wk.tile_end = min(n_tiles, wk.tile_begin + p.tiles_per_split);
+    int tiles_per_split = p.tiles_per_split;
+    if constexpr (MASK && (W16 || D == 64)) {   // (the 32-wide instantiation at head_dim 128 has no register left for it)
+        if (p.mask_stride_h == 0) {   // one mask row for all heads of the sequence: a padded suffix is skipped
+            __shared__ int red[kWaves];
+            wk.T = mask_row_len(reinterpret_cast<const _Float16 *>(p.mask + (int64_t)b * p.mask_stride_b), p.T, threadIdx.x, red);
+            tiles_per_split = ((wk.T + kTile - 1) / kTile + p.nsplit - 1) / p.nsplit;
+        }
+    }
+    const int n_tiles = (wk.T + kTile - 1) / kTile;
+    wk.tile_begin = split * tiles_per_split;
+    wk.tile_end = min(n_tiles, wk.tile_begin + tiles_per_split);
     wk.nsplit = p.nsplit;
     const int64_t bh = (int64_t)b * p.Hkv + kvh;
     wk.slot = bh * p.nsplit + split;
