@@ -58,6 +58,8 @@ struct MfmaWork {
     const char *kbase, *vbase;    // K and V rows of this (sequence, kv head): f16 rows or block codes
     const char *ksbase, *vsbase;  // quantised formats: their f16 block scales, D/32 per token
     int T, tile_begin, tile_end;
+    int tile_step;                // a wave's next tile: kWaves (a contiguous range) or kWaves * splits (the splits of a
+                                  // dense sequence-head take groups of kWaves tiles in turn)
     int nsplit;                   // splits of this sequence-head (1: write the output rows)
     int64_t slot;                 // partial record of this workgroup
     int new_pos;                  // token stored by a fused append (-1: none)
@@ -223,9 +225,10 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
     // this lane's mask values: its head's row, tokens 8*rq + 4*hb + 0..3 of the tile
     // (16-wide: tokens 16*mb + 4*(lane/16) + 0..3)
     const char *mask_lane = MASK ? wk.mask + (int64_t)min(hcol, g - 1) * p.mask_stride_h + 8 * (W16 ? q4 : hb) : nullptr;
-    for (; t < tile_end; t += kWaves) {
+    const int tstep = wk.tile_step;
+    for (; t < tile_end; t += tstep) {
         const int t0 = t * kTile;
-        const bool more = t + kWaves < tile_end;
+        const bool more = t + tstep < tile_end;
         constexpr int NMK = W16 ? 2 : 4;          // groups of 4 consecutive tokens this lane owns in a tile
         constexpr int kMkStep = W16 ? 16 : 8;     // tokens between them
         half4_t mk[MASK ? NMK : 1];
@@ -247,11 +250,11 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
         // ---- K tile -> LDS, the next tile's K into flight ----------------------------------------------
         if constexpr (QUANT) {
             stash_q(kpre, ksc, k_slot);
-            if (more) fetch_q(kbase, wk.ksbase, t + kWaves, kpre, ksc);
+            if (more) fetch_q(kbase, wk.ksbase, t + tstep, kpre, ksc);
         } else {
 #pragma unroll
             for (int j = 0; j < NLD; j++) *reinterpret_cast<u32x4 *>(tile + k_slot[j]) = kpre[j];
-            if (more) fetch(kbase, p.k_new, t + kWaves, kpre);
+            if (more) fetch(kbase, p.k_new, t + tstep, kpre);
         }
         half8_t pf16;
         if constexpr (W16) {
@@ -352,11 +355,11 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
         // ---- V tile -> the same LDS tile (every K fragment has been consumed), next V into flight ------
         if constexpr (QUANT) {
             stash_q(vpre, vsc, v_slot);
-            if (more) fetch_q(vbase, wk.vsbase, t + kWaves, vpre, vsc);
+            if (more) fetch_q(vbase, wk.vsbase, t + tstep, vpre, vsc);
         } else {
 #pragma unroll
             for (int j = 0; j < NLD; j++) *reinterpret_cast<u32x4 *>(tile + v_slot[j]) = vpre[j];
-            if (more) fetch(vbase, p.v_new, t + kWaves, vpre);
+            if (more) fetch(vbase, p.v_new, t + tstep, vpre);
         }
         // ---- O^T += V^T P^T ---------------------------------------------------------------------------------
         const _Float16 *vsrc = tile + vsrc_off;
@@ -500,8 +503,13 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev
         }
     }
     const int n_tiles = (wk.T + kTile - 1) / kTile;
-    wk.tile_begin = split * tiles_per_split;
-    wk.tile_end = min(n_tiles, wk.tile_begin + tiles_per_split);
+    if (p.interleave) {   // concurrent workgroups read neighbouring addresses
+        wk.tile_begin = split * kWaves, wk.tile_end = n_tiles, wk.tile_step = kWaves * p.nsplit;
+    } else {
+        wk.tile_begin = split * tiles_per_split;
+        wk.tile_end = min(n_tiles, wk.tile_begin + tiles_per_split);
+        wk.tile_step = kWaves;
+    }
     wk.nsplit = p.nsplit;
     const int64_t bh = (int64_t)b * p.Hkv + kvh;
     wk.slot = bh * p.nsplit + split;
@@ -527,7 +535,7 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_ragged_kernel(De
         wk.vsbase = it.vs + (int64_t)kvh * it.sc_stride_h;
     }
     wk.T = it.T;
-    wk.tile_begin = it.tile_begin, wk.tile_end = it.tile_end;
+    wk.tile_begin = it.tile_begin, wk.tile_end = it.tile_end, wk.tile_step = kWaves;
     wk.nsplit = it.nsplit;
     wk.slot = ((int64_t)it.slot0 + it.split) * p.Hkv + kvh;
     wk.new_pos = p.k_new ? it.T - 1 : -1;
@@ -652,6 +660,8 @@ int launch_sdpa_decode_quant_mfma(DecodeDev &p, int kv_fmt, int64_t B, void *wor
         TROCM_REQUIRE(workspace_bytes >= need, "sdpa workspace too small: %zu bytes given, %zu needed", workspace_bytes, need);
     }
     p.tiles_per_split = tps, p.nsplit = nsplit;
+    static const int interleave = getenv("TROCM_DECODE_INTERLEAVE") ? atoi(getenv("TROCM_DECODE_INTERLEAVE")) : 1;
+    p.interleave = interleave;
     p.part_ml = (float *)((char *)workspace + kWsCounterBytes);
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * gp;
     static const int tail = getenv("TROCM_DECODE_TAIL_MERGE") ? atoi(getenv("TROCM_DECODE_TAIL_MERGE")) : 1;
@@ -698,6 +708,8 @@ int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {
     if (p.k_new && (p.v_new == nullptr || (uintptr_t)p.k_new % 16 || (uintptr_t)p.v_new % 16)) return 2;
     p.part_ml = (float *)((char *)a.workspace + kWsCounterBytes);
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * gp;
+    static const int interleave = getenv("TROCM_DECODE_INTERLEAVE") ? atoi(getenv("TROCM_DECODE_INTERLEAVE")) : 1;
+    p.interleave = interleave;
     if (a.mask) {   // [mask_b, mask_h, 1, Sk] dense f16
         p.mask = (const char *)a.mask;
         p.mask_stride_h = a.mask_h > 1 ? a.Sk * 2 : 0;
