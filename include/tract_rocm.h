@@ -309,7 +309,7 @@ int trocm_window_kv_sdpa_eval(const void *q, const void *k_new, const void *v_ne
  * per sequence.  q, out: [n_seq, q_heads, 1, head_dim].  The reference has no ragged batch:
  * its statement of the same result is a dense batch padded to the longest sequence with an
  * additive mask whose padded columns are <= -65504 (flash_sdpa.rs:261-268).  F16 and F32 caches,
- * and Q8_0 / Q4_0 caches with 2..32 query heads per kv head, run as one launch (plus a merge launch
+ * and Q8_0 / Q4_0 caches with 1..32 query heads per kv head (head_dim 128, f16 queries), run as one launch (plus a merge launch
  * when a sequence is cut into more than 8 pieces); other cases as one call per sequence. */
 int trocm_sdpa_decode_ragged(const void *q, int q_dtype, int64_t q_heads, int64_t n_seq,
                              trocm_kv_cache *const *k_caches, trocm_kv_cache *const *v_caches,

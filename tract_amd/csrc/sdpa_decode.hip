@@ -646,7 +646,10 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     const int64_t g_real = Hq / Hkv;
     // grouped heads over f16 or block-quantised caches: the MFMA formulation (sdpa_decode_mfma.hip)
     const bool quant = is_quant(kv_fmt);
-    const int mfma_gp = (kv_fmt == TROCM_F16 || (quant && q_dtype == TROCM_F16 && D == 128)) ? decode_mfma_group(g_real) : 0;
+    int mfma_gp = (kv_fmt == TROCM_F16 || (quant && q_dtype == TROCM_F16 && D == 128)) ? decode_mfma_group(g_real) : 0;
+    // one head per kv head over quantised caches: the vector-ALU kernel has no ragged form, and one launch on the
+    // matrix cores beats a launch per sequence
+    if (quant && q_dtype == TROCM_F16 && D == 128 && g_real == 1) mfma_gp = 8;
     const int64_t G = mfma_gp ? mfma_gp : g_real <= 2 ? g_real : g_real <= 4 ? 4 : 8;   // the instantiation that runs it
     const int64_t rb = kv_fmt == TROCM_Q8_0 ? D : kv_fmt == TROCM_Q4_0 ? D / 2 : D * (int64_t)elem_bytes(kv_fmt);   // bytes per token row
     bool fast = quant ? mfma_gp != 0 && k_new == nullptr
