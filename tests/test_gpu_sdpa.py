@@ -511,6 +511,26 @@ def test_one_workspace_shared_by_ragged_and_dense_calls(rt):
             assert max_abs(got_r[i:i + 1], orc.flash_sdpa(qr[i:i + 1], ks[i], ks[i], causal=True)) <= 2e-2, f"ragged, turn {turn}, sequence {i}"
 
 
+def test_ragged_decode_with_a_thousand_short_sequences(rt):
+    """More sequences than compute units: every sequence is one work item, the plan holds a thousand of them."""
+    rng = np.random.default_rng(1000)
+    Hq, Hkv, D, n_seq = 8, 2, 64, 1000
+    lens = rng.integers(1, 40, size=n_seq, endpoint=True)
+    pool = tract_amd.KvPool(64 << 20)
+    kcs, vcs, ks, vs = [], [], [], []
+    for n in lens:
+        k = rng.standard_normal((1, Hkv, int(n), D), dtype=np.float32).astype(np.float16)
+        v = rng.standard_normal((1, Hkv, int(n), D), dtype=np.float32).astype(np.float16)
+        kc, vc = tract_amd.InPlaceKvCache(2, pool=pool), tract_amd.InPlaceKvCache(2, pool=pool)
+        kc.push(k), vc.push(v)
+        kcs.append(kc), vcs.append(vc), ks.append(k), vs.append(v)
+    q = (rng.standard_normal((n_seq, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    out = tract_amd.sdpa_decode_ragged(tract_amd.DeviceTensor.from_numpy(q), kcs, vcs).to_numpy()
+    assert not np.isnan(out).any()
+    for i in range(0, n_seq, 7):
+        assert max_abs(out[i:i + 1], orc.flash_sdpa(q[i:i + 1], ks[i], vs[i], causal=True)) <= 2e-2, f"sequence {i}"
+
+
 def test_ragged_equals_padded_batch_with_mask(rt):
     """The reference's statement of a ragged batch: a dense batch padded to the longest
     sequence with an additive mask whose padded columns are <= -65504 (flash_sdpa.rs:261-268)."""

@@ -170,7 +170,7 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
 // per-sequence slot ranges) between the two, so that the counters stay zero for whichever launch comes next:
 // [arrival counters][plan][partials ...].
 constexpr size_t kWsCounterBytes = 64 * 1024;   // 16384 arrival counters
-constexpr size_t kWsPlanBytes = 64 * 1024;      // about 1100 work items
+constexpr size_t kWsPlanBytes = 256 * 1024;     // about 3000 work items: the 2048 sequences a ragged launch takes, cut at most once each
 size_t decode_workspace_bytes(int64_t B, int64_t Hq, int64_t D);
 
 }  // namespace trocm
