@@ -479,6 +479,31 @@ def test_ragged_decode_many_sequences(rt, dt, Hq, Hkv, D, n_seq, lo, hi):
             ks[i], vs[i] = np.concatenate([ks[i], kn], axis=2), np.concatenate([vs[i], vn], axis=2)
 
 
+@pytest.mark.parametrize("fmt_name", ["plain", "Q8_0"])
+@pytest.mark.parametrize("ws_bytes", [0, 70_000, 400_000])
+def test_decode_with_a_small_or_no_workspace(rt, fmt_name, ws_bytes):
+    """A decode call whose workspace has no room for the splits it would like runs with fewer, down to one
+    (no workspace at all): the result does not change."""
+    from tract_amd._lib import call
+    from tract_amd.runtime import dtype_code
+    rng = np.random.default_rng(88)
+    B, Hq, Hkv, D, T = 1, 32, 8, 128, 3000
+    fmt = None if fmt_name == "plain" else tract_amd.Q8_0
+    k = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(np.float16)
+    q = (rng.standard_normal((B, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    st = tract_amd.InPlaceKvSdpa(axis=2, causal=True, storage_format=fmt).state()
+    st.k.push(k), st.v.push(v)
+    qd, out = tract_amd.DeviceTensor.from_numpy(q), tract_amd.DeviceTensor(q.shape, np.float16)
+    want = st.attend(qd).to_numpy()
+    ws = tract_amd.DeviceTensor((max(ws_bytes, 16),), np.uint8)
+    if ws_bytes:
+        call("trocm_sdpa_workspace_init", ws.ptr, ws_bytes, None)
+    call("trocm_sdpa_cached", qd.ptr, dtype_code(np.float16), Hq, 1, st.k.handle, st.v.handle, out.ptr,
+         float("nan"), 1, ws.ptr if ws_bytes else None, ws_bytes, None)
+    assert max_abs(out.to_numpy(), want) <= 2e-3
+
+
 def test_one_workspace_shared_by_ragged_and_dense_calls(rt):
     """A ragged call keeps its launch plan in the workspace; a dense decode that follows on the same
     workspace counts workgroup arrivals there.  Neither may disturb the other, in either order."""

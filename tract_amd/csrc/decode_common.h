@@ -321,5 +321,13 @@ int launch_sdpa_decode_ragged_mfma(const DecodeDev &p, int kv_fmt, int gp, int64
 // Partials: at most kMaxSplitRows rows of (D + 2) floats per query head.
 constexpr int64_t kMaxSplitRows = 32768;
 int choose_decode_splits(int64_t BH, int64_t G, int n_tiles, int wg_per_cu);
+// The splits that the caller's workspace has room for (records of BH x splits x G rows of D + 2 floats behind the
+// counter area), at least one: a call with a small or no workspace runs with fewer splits, it does not fail.
+inline int fit_decode_splits(int nsplit, int64_t BH, int64_t G, int64_t D, const void *workspace, size_t workspace_bytes) {
+    if (nsplit <= 1 || workspace == nullptr || workspace_bytes <= kWsCounterBytes) return 1;
+    const int64_t per_split = BH * G * (D + 2) * (int64_t)sizeof(float);
+    const int64_t fit = (int64_t)(workspace_bytes - kWsCounterBytes) / per_split;
+    return (int)(fit < 1 ? 1 : fit < nsplit ? fit : nsplit);
+}
 
 }  // namespace trocm

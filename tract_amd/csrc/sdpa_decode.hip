@@ -477,15 +477,9 @@ int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
     if (BH > (int64_t)(kWsCounterBytes / sizeof(int)) || a.B > 65535 || a.Hkv > 65535) return 2;
 
     int n_tiles = (int)((a.Sk + kTile - 1) / kTile);
-    int nsplit = choose_decode_splits(BH, G, n_tiles, 1);
+    int nsplit = fit_decode_splits(choose_decode_splits(BH, G, n_tiles, 1), BH, G, a.D, a.workspace, a.workspace_bytes);
     int tps = (n_tiles + nsplit - 1) / nsplit;
     nsplit = (n_tiles + tps - 1) / tps;  // no empty split
-    if (nsplit > 1) {
-        TROCM_NOT_NULL(a.workspace);
-        size_t need = kWsCounterBytes + (size_t)BH * nsplit * G * (a.D + 2) * sizeof(float);
-        TROCM_REQUIRE(a.workspace_bytes >= need, "sdpa workspace too small: %zu bytes given, %zu needed",
-                      a.workspace_bytes, need);
-    }
     DecodeDev p;
     memset(&p, 0, sizeof(p));
     p.q = (const char *)a.q;

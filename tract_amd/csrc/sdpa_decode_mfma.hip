@@ -651,14 +651,9 @@ int launch_sdpa_decode_quant_mfma(DecodeDev &p, int kv_fmt, int64_t B, void *wor
     const int64_t BH = B * p.Hkv;
     const int n_tiles = (p.T + kTile - 1) / kTile;
     static const int wg_per_cu = getenv("TROCM_DECODE_QUANT_WG_PER_CU") ? atoi(getenv("TROCM_DECODE_QUANT_WG_PER_CU")) : 2;
-    int nsplit = choose_decode_splits(BH, gp, n_tiles, wg_per_cu);
+    int nsplit = fit_decode_splits(choose_decode_splits(BH, gp, n_tiles, wg_per_cu), BH, gp, 128, workspace, workspace_bytes);
     const int tps = (n_tiles + nsplit - 1) / nsplit;
     nsplit = (n_tiles + tps - 1) / tps;
-    if (nsplit > 1) {
-        TROCM_NOT_NULL(workspace);
-        const size_t need = kWsCounterBytes + (size_t)BH * nsplit * gp * (128 + 2) * sizeof(float);
-        TROCM_REQUIRE(workspace_bytes >= need, "sdpa workspace too small: %zu bytes given, %zu needed", workspace_bytes, need);
-    }
     p.tiles_per_split = tps, p.nsplit = nsplit;
     static const int interleave = getenv("TROCM_DECODE_INTERLEAVE") ? atoi(getenv("TROCM_DECODE_INTERLEAVE")) : 1;
     p.interleave = interleave;
@@ -687,14 +682,9 @@ int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {
     if (a.B > 65535 || a.Hkv > 65535) return 2;
     const int64_t BH = a.B * a.Hkv;
     const int n_tiles = (int)((a.Sk + kTile - 1) / kTile);
-    int nsplit = choose_decode_splits(BH, gp, n_tiles, 1);
+    int nsplit = fit_decode_splits(choose_decode_splits(BH, gp, n_tiles, 1), BH, gp, a.D, a.workspace, a.workspace_bytes);
     const int tps = (n_tiles + nsplit - 1) / nsplit;
     nsplit = (n_tiles + tps - 1) / tps;
-    if (nsplit > 1) {
-        TROCM_NOT_NULL(a.workspace);
-        const size_t need = kWsCounterBytes + (size_t)BH * nsplit * gp * (a.D + 2) * sizeof(float);
-        TROCM_REQUIRE(a.workspace_bytes >= need, "sdpa workspace too small: %zu bytes given, %zu needed", a.workspace_bytes, need);
-    }
     DecodeDev p;
     memset(&p, 0, sizeof(p));
     p.q = (const char *)a.q, p.out = (char *)a.out, p.k = (const char *)a.k, p.v = (const char *)a.v;

@@ -432,15 +432,9 @@ int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s) {
         return launch_sdpa_decode_quant_mfma(p, a.kv_fmt, a.B, a.workspace, a.workspace_bytes, s);
     }
     int n_tiles = (int)((a.Sk + kTile - 1) / kTile);
-    int nsplit = choose_decode_splits(BH, G, n_tiles, 2);
+    int nsplit = fit_decode_splits(choose_decode_splits(BH, G, n_tiles, 2), BH, G, a.D, a.workspace, a.workspace_bytes);
     int tps = (n_tiles + nsplit - 1) / nsplit;
     nsplit = (n_tiles + tps - 1) / tps;
-    if (nsplit > 1) {
-        TROCM_NOT_NULL(a.workspace);
-        size_t need = kWsCounterBytes + (size_t)BH * nsplit * G * (a.D + 2) * sizeof(float);
-        TROCM_REQUIRE(a.workspace_bytes >= need, "sdpa workspace too small: %zu bytes given, %zu needed",
-                      a.workspace_bytes, need);
-    }
     DecodeDev p;
     memset(&p, 0, sizeof(p));
     p.q = (const char *)a.q;
