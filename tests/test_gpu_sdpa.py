@@ -776,7 +776,8 @@ def test_prefill_any_split_count_and_head_grouping_agree(rt, env):
 
 
 def test_prefill_with_a_workspace_too_small_for_key_splits(rt):
-    """A caller may hand over a workspace sized for decode only: prefill then runs unsplit."""
+    """A caller may hand over a workspace with room for fewer key splits than the prefill would like, for none
+    at all, or no workspace: prefill then runs with fewer splits or unsplit."""
     from tract_amd._lib import call
     from tract_amd.runtime import DeviceTensor, Workspace
     B, Hq, Hkv, Sq, Sk, D = 1, 32, 8, 512, 1024, 128
@@ -784,11 +785,13 @@ def test_prefill_with_a_workspace_too_small_for_key_splits(rt):
     q = (rng.standard_normal((B, Hq, Sq, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
     k = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(np.float16)
     v = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(np.float16)
-    ws = Workspace(B, Hq, 1, D)
-    assert ws.nbytes < Workspace.bytes_for(B, Hq, Sq, D)
+    full = Workspace.bytes_for(B, Hq, Sq, D)
+    small = [DeviceTensor((n,), np.uint8) for n in (full // 2, 80_000)]
+    for t in small:
+        call("trocm_sdpa_workspace_init", t.ptr, t.shape[0], None)
     dq, dk, dv = (DeviceTensor.from_numpy(t) for t in (q, k, v))
     out = DeviceTensor(q.shape, q.dtype)
-    for wsp, wsn in ((ws.ptr, ws.nbytes), (None, 0)):
+    for wsp, wsn in ((small[0].ptr, small[0].shape[0]), (small[1].ptr, small[1].shape[0]), (None, 0)):
         call("trocm_sdpa", dq.ptr, dk.ptr, dv.ptr, None, out.ptr, 1, B, Hq, Hkv, Sq, Sk, D, None, 1, 1,
              float("nan"), 1, wsp, wsn, None)
         assert max_abs(out.to_numpy(), cases.textbook_sdpa(q, k, v, causal=True)) <= 4e-3
