@@ -270,7 +270,10 @@ int trocm_sdpa_workspace_init(void *workspace, size_t bytes, void *stream);
  *            dispatch expresses with zero strides, cuda/src/kernels/flash_attn.rs:138-143);
  *            must be NULL when causal (sdpa.rs:297-299).  Values may be finite minima
  *            (sdpa.rs:550-553) or -inf; a row masked entirely with -inf yields NaN, as on the
- *            CPU.  The split-K decode and MFMA prefill kernels take the mask themselves.
+ *            CPU.  The split-K decode and MFMA prefill kernels take the mask themselves; with
+ *            q_len == 1 and mask_heads == 1 (a batch padded to its longest sequence,
+ *            flash_sdpa.rs:261-268) the columns after the last one above -60000 weigh nothing and
+ *            are not read.
  *   scale  : NaN selects the default 1/sqrt(head_dim) (sdpa.rs:177-181)
  *   causal : key j visible to query i iff j <= i + (kv_len - q_len) (flash_sdpa.rs:279-288) */
 int trocm_sdpa(const void *q, const void *k, const void *v, const void *mask, void *out, int dtype,
