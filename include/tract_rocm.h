@@ -289,6 +289,22 @@ int trocm_sdpa_cached(const void *q, int q_dtype, int64_t q_heads, int64_t q_len
                       const trocm_kv_cache *k_cache, const trocm_kv_cache *v_cache, void *out,
                       float scale, int causal, void *workspace, size_t workspace_bytes, void *stream);
 
+/* trocm_sdpa_cached for callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same
+ * arguments, result and kernels as trocm_sdpa_cached, but the split-K scratch is a static device
+ * array of TROCM_STATIC_SCRATCH_BYTES inside the library (held on the library's device until the
+ * process ends) and the call reaches no hipMalloc, hipFree or other allocating routine.
+ *   - `stream` must not be NULL (the library's per-thread stream is created on first use).
+ *   - a shape whose trocm_sdpa_workspace_bytes(batch, q_heads, q_len, head_dim) exceeds
+ *     TROCM_STATIC_SCRATCH_BYTES is refused with a message (decode: batch * q_heads <= 32768 at
+ *     head_dim <= 128 fits; prefill: the split partials of q_len > 1 must fit).
+ *   - every call shares the one array: calls that overlap in time on the device race on it;
+ *     calls ordered by one stream, or by events, do not. */
+#define TROCM_STATIC_SCRATCH_BYTES (24u << 20)
+int trocm_sdpa_cached_noalloc(const void *q, int q_dtype, int64_t q_heads, int64_t q_len,
+                              const trocm_kv_cache *k_cache, const trocm_kv_cache *v_cache, void *out,
+                              float scale, int causal, void *stream);
+
 /* InPlaceKvSdpaState::eval (inplace_kv_cache.rs:191-216) as one call: push k_new and v_new
  * ([batch, kv_heads, n_new, head_dim] of `dtype`, element strides kv_new_strides[4] or NULL for
  * dense) into the caches, then attend q ([batch, q_heads, n_new, head_dim] dense) over them. */

@@ -80,6 +80,7 @@ SIGNATURES = {
     "trocm_sdpa": [_vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i64, _i64, _i64, _i64, _pi64, _i64, _i64, _f, _i,
                    _vp, _sz, _vp],
     "trocm_sdpa_cached": [_vp, _i, _i64, _i64, _vp, _vp, _vp, _f, _i, _vp, _sz, _vp],
+    "trocm_sdpa_cached_noalloc": [_vp, _i, _i64, _i64, _vp, _vp, _vp, _f, _i, _vp],
     "trocm_kv_cache_create_window": [C.POINTER(_vp), _i, _i64, _i64, _i64, _i64],
     "trocm_kv_cache_window": [_vp, _pi64, _pi64],
     "trocm_window_kv_sdpa_eval": [_vp, _vp, _vp, _i, _i64, _i64, _pi64, _vp, _vp, _vp, _f, _vp, _sz, _vp],

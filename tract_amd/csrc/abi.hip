@@ -34,6 +34,13 @@ static int g_compute_units = 0;
 static size_t g_hbm_bytes = 0;
 static char g_name[256] = "";
 
+// Split-K scratch of trocm_sdpa_cached_noalloc, the entry point that allocates nothing: the workspace its
+// kernels would otherwise take from the caller.  The array's name is a host-side stand-in, not a device
+// address; trocm_init asks the runtime where the array lives on the library's device, and every use on the
+// host goes through that pointer.  All calls share the one array: calls that overlap in time race on it.
+static __device__ __align__(256) unsigned char scratch[TROCM_STATIC_SCRATCH_BYTES];
+static void *g_scratch_ptr = nullptr;   // written once, under g_init_mutex, before g_device is published
+
 struct ThreadStream {
     hipStream_t s = nullptr;
     ~ThreadStream() {
@@ -259,6 +266,14 @@ int trocm_init(int device) {
     g_compute_units = prop.multiProcessorCount;
     g_hbm_bytes = prop.totalGlobalMem;
     snprintf(g_name, sizeof(g_name), "%s (%s)", prop.name, prop.gcnArchName);
+    // The device address of the static scratch on this device, and its counter area cleared once: the
+    // kernels leave the counters at zero after every launch.
+    void *sp = nullptr;
+    TROCM_HIP(hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)));
+    TROCM_REQUIRE(sp != nullptr, "hipGetSymbolAddress returned no address for the static scratch");
+    TROCM_HIP(hipMemset(sp, 0, kWsCounterBytes));
+    TROCM_HIP(hipDeviceSynchronize());
+    g_scratch_ptr = sp;
     g_device = device;
     return 0;
 }
@@ -985,9 +1000,9 @@ int trocm_sdpa(const void *q, const void *k, const void *v, const void *mask, vo
     return dispatch_sdpa(a, s);
 }
 
-int trocm_sdpa_cached(const void *q, int q_dtype, int64_t q_heads, int64_t q_len, const trocm_kv_cache *kc,
-                      const trocm_kv_cache *vc, void *out, float scale, int causal, void *workspace,
-                      size_t workspace_bytes, void *stream) {
+// Argument checks of an attention call over two caches (none of them touches the device).
+static int sdpa_cached_check(const void *q, int q_dtype, int64_t q_heads, const trocm_kv_cache *kc, const trocm_kv_cache *vc,
+                             const void *out) {
     TROCM_NOT_NULL(q);
     TROCM_NOT_NULL(kc);
     TROCM_NOT_NULL(vc);
@@ -998,12 +1013,16 @@ int trocm_sdpa_cached(const void *q, int q_dtype, int64_t q_heads, int64_t q_len
     TROCM_REQUIRE(kc->len == vc->len, "K/V lengths must match (%lld vs %lld)", (long long)kc->len, (long long)vc->len);
     TROCM_REQUIRE(kc->cap == vc->cap, "K/V capacities must match (%lld vs %lld)", (long long)kc->cap, (long long)vc->cap);
     TROCM_REQUIRE(kc->len > 0, "empty kv-cache");  // inplace_kv_cache.rs:91
-    TROCM_REQUIRE(q_heads % kc->H == 0, "Q heads (%lld) must be a multiple of K/V heads (%lld)", (long long)q_heads,
+    TROCM_REQUIRE(q_heads >= 1 && q_heads % kc->H == 0, "Q heads (%lld) must be a multiple of K/V heads (%lld)", (long long)q_heads,
                   (long long)kc->H);
     TROCM_REQUIRE(is_quant(kc->fmt) || kc->fmt == q_dtype, "q dtype %d does not match the cache format %d", q_dtype,
                   kc->fmt);
-    hipStream_t s;
-    if (resolve_stream(stream, &s)) return 1;
+    return 0;
+}
+
+static int sdpa_cached_run(const void *q, int q_dtype, int64_t q_heads, int64_t q_len, const trocm_kv_cache *kc,
+                           const trocm_kv_cache *vc, void *out, float scale, int causal, void *workspace,
+                           size_t workspace_bytes, hipStream_t s) {
     SdpaArgs a;
     memset(&a, 0, sizeof(a));
     a.q = q, a.out = out, a.q_dtype = q_dtype, a.kv_fmt = kc->fmt;
@@ -1015,6 +1034,34 @@ int trocm_sdpa_cached(const void *q, int q_dtype, int64_t q_heads, int64_t q_len
     a.causal = causal;
     a.workspace = workspace, a.workspace_bytes = workspace_bytes;
     return dispatch_sdpa(a, s);
+}
+
+int trocm_sdpa_cached(const void *q, int q_dtype, int64_t q_heads, int64_t q_len, const trocm_kv_cache *kc,
+                      const trocm_kv_cache *vc, void *out, float scale, int causal, void *workspace,
+                      size_t workspace_bytes, void *stream) {
+    if (sdpa_cached_check(q, q_dtype, q_heads, kc, vc, out)) return 1;
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    return sdpa_cached_run(q, q_dtype, q_heads, q_len, kc, vc, out, scale, causal, workspace, workspace_bytes, s);
+}
+
+// trocm_sdpa_cached for callers that cannot allocate: the split-K scratch is the library's static device
+// array instead of a caller's workspace, and nothing on this path calls an allocating routine (the caller's
+// stream is required because the library's own per-thread stream is created on first use).
+int trocm_sdpa_cached_noalloc(const void *q, int q_dtype, int64_t q_heads, int64_t q_len, const trocm_kv_cache *kc,
+                              const trocm_kv_cache *vc, void *out, float scale, int causal, void *stream) {
+    if (ensure_init()) return 1;
+    TROCM_REQUIRE(stream != nullptr, "sdpa_cached_noalloc: a stream is required (the library's per-thread stream would be created here)");
+    if (sdpa_cached_check(q, q_dtype, q_heads, kc, vc, out)) return 1;
+    TROCM_REQUIRE(q_len >= 0, "sdpa: negative dimension");
+    size_t need = 0;
+    if (trocm_sdpa_workspace_bytes(kc->B, q_heads, q_len, kc->D, &need)) return 1;
+    TROCM_REQUIRE(need <= (size_t)TROCM_STATIC_SCRATCH_BYTES,
+                  "sdpa_cached_noalloc: batch %lld x %lld query heads x %lld queries at head_dim %lld asks for %zu bytes of split-K "
+                  "scratch, the static buffer holds %zu; call trocm_sdpa_cached with a workspace of that size instead",
+                  (long long)kc->B, (long long)q_heads, (long long)q_len, (long long)kc->D, need, (size_t)TROCM_STATIC_SCRATCH_BYTES);
+    return sdpa_cached_run(q, q_dtype, q_heads, q_len, kc, vc, out, scale, causal, g_scratch_ptr, (size_t)TROCM_STATIC_SCRATCH_BYTES,
+                           (hipStream_t)stream);
 }
 
 // Shared argument block of an attention call over two caches.

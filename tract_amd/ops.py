@@ -407,6 +407,16 @@ class InPlaceKvSdpaState:
              _scale_arg(self.scale), int(self.causal), self._ws.ptr, self._ws.nbytes, _sh(stream))
         return out
 
+    def attend_noalloc(self, q: DeviceTensor, out: DeviceTensor, stream) -> DeviceTensor:
+        """`attend` through the entry point that allocates nothing (the library's static split-K
+        scratch): `out` and `stream` are the caller's; calls that overlap in time race on the scratch."""
+        B, Hq, Sq, D = _canon4(q.shape)
+        if self.k.handle is None:
+            raise TractRocmError("empty kv-cache")
+        call("trocm_sdpa_cached_noalloc", q.ptr, dtype_code(q.dtype), Hq, Sq, self.k.handle, self.v.handle, out.ptr,
+             _scale_arg(self.scale), int(self.causal), _sh(stream))
+        return out
+
     def save_to(self, states: list) -> None:
         if not self.k.is_empty():
             states.append(self.k.valid_contiguous())
