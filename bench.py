@@ -38,6 +38,7 @@ HBM_PEAK_GBS = 8000.0
 # counter scaled by what it reads for the 128 MiB prefill copy of known size: FETCH_SIZE
 # 132347.9 x 1.9991 KiB + WRITE_SIZE 1226 x 1.000 KiB.
 PMC_TRAFFIC_BYTES_B8_CTX8226 = int((132347.9 * 1.9991 + 1226.0) * 1024)
+PMC_ALGORITHMIC_BYTES_B8_CTX8226 = 2 * 8 * 8 * 8226 * 128 * 2 + 2 * 8 * 32 * 128 * 2
 
 
 def cfg_seed(cfg, what):
@@ -54,7 +55,7 @@ def seeded_f16(seed, shape):
     return g.standard_normal(shape, dtype=np.float32).astype(np.float16)
 
 
-def run_batch(ta, B, steps, warmup, kernel_iters, layers=LAYERS):
+def run_batch(ta, B, steps, warmup, kernel_iters, layers=LAYERS, windows=5):
     """Returns a dict of measurements for batch size B."""
     sts = [ta.InPlaceKvSdpa(axis=2, causal=True, scale=None).state() for _ in range(layers)]
     # prefill: one append of 8192 seeded tokens per sequence (the same values in every layer)
@@ -67,7 +68,7 @@ def run_batch(ta, B, steps, warmup, kernel_iters, layers=LAYERS):
         st.k.push(kp)
         st.v.push(vp)
     del kp, vp
-    n = steps + warmup
+    n = warmup + windows * steps
     scale_q = np.float32(1.0 / np.sqrt(D))
     q_all = (seeded_f16(cfg_seed(2, "q"), (n, B, HQ, 1, D)).astype(np.float32) * scale_q).astype(np.float16)
     k_all = seeded_f16(cfg_seed(2, "k") + 7, (n, B, HKV, 1, D))
@@ -86,20 +87,42 @@ def run_batch(ta, B, steps, warmup, kernel_iters, layers=LAYERS):
         sts[j % layers].attend(dq[0], out=out)
     for i in range(warmup):
         step(i)  # a layer's first step doubles its capacity 8192 -> 16384 (one reallocation)
-    ta.synchronize()
-    t0 = time.perf_counter()
-    for i in range(warmup, n):
-        step(i)
-    ta.synchronize()
-    dt = time.perf_counter() - t0
-    # context length seen by timed step i: the layer's prefill plus its earlier visits plus this token
-    ctx_sum = sum(CTX + i // layers + 1 for i in range(warmup, n))
-    step_bytes = algorithmic_bytes(B, ctx_sum / steps)
+    # The timed region is `steps` steps between two device synchronisations, taken `windows` times on
+    # fresh inputs (every step appends, so the caches keep growing).  Each window is timed twice over:
+    # by the host's clock around the synchronisations, and by two HIP events recorded on the stream just
+    # before the first and just after the last step.  The event time is the device's time for the steps;
+    # the host's clock adds one launch latency and one synchronisation latency (together 40-80 us), which
+    # a short window (20 steps are 1 ms at batch 8) does not amortise and a decoder that keeps its stream
+    # fed never pays.  The median window by event time gives `value`; the host's clock is reported beside it.
+    wins = []
+    e0, e1 = ta.Event(), ta.Event()
+    for w in range(windows):
+        first = warmup + w * steps
+        ta.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(first, first + steps):
+            step(i)
+        e1.record()
+        ta.synchronize()
+        wall = time.perf_counter() - t0
+        ev = ta.Event.elapsed_ms(e0, e1) * 1e-3
+        # context length seen by timed step i: the layer's prefill plus its earlier visits plus this token
+        ctx_sum = sum(CTX + i // layers + 1 for i in range(first, first + steps))
+        wins.append({"event_s": ev, "wall_s": wall, "bytes": algorithmic_bytes(B, ctx_sum / steps)})
+    wins.sort(key=lambda x: x["event_s"])
+    med = wins[len(wins) // 2]
+    dt = med["event_s"]
+    wall_med = sorted(x["wall_s"] for x in wins)[len(wins) // 2]
     res = {
         "batch": B,
         "ms_per_step": dt / steps * 1e3,
         "us_per_token": dt / steps * 1e6,
-        "step_gbs": step_bytes / (dt / steps) / 1e9,
+        "step_gbs": med["bytes"] / (dt / steps) / 1e9,
+        "wall_ms_per_step": wall_med / steps * 1e3,
+        "wall_step_gbs": med["bytes"] / (wall_med / steps) / 1e9,
+        "windows": windows,
+        "window_ms_per_step_min_max": [round(wins[0]["event_s"] / steps * 1e3, 5), round(wins[-1]["event_s"] / steps * 1e3, 5)],
         "reallocs": sts[0].k.reallocs(),
         "context_end": sts[0].k.len(),
         "prewarm_launches": PREWARM_LAUNCHES,
@@ -525,6 +548,7 @@ def main():
     ap.add_argument("--batch", type=int, default=8, help="headline batch size")
     ap.add_argument("--other-batches", type=str, default="1,32")
     ap.add_argument("--kernel-iters", type=int, default=200)
+    ap.add_argument("--windows", type=int, default=5, help="how many times the timed window of --steps steps is taken (median reported)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "ops"],
                     help="cfg2 (default) is the configuration the metric is quoted on; the others print one line "
@@ -542,7 +566,7 @@ def main():
         line["device"] = rt.device_name
         print(json.dumps(line))
         return
-    main_res = run_batch(ta, args.batch, args.steps, args.warmup, args.kernel_iters)
+    main_res = run_batch(ta, args.batch, args.steps, args.warmup, args.kernel_iters, windows=args.windows)
 
     # parity spot check of the last output against the oracle (checker only)
     from oracle import oracle as orc
@@ -555,11 +579,20 @@ def main():
 
     others = {}
     for b in [int(x) for x in args.other_batches.split(",") if x]:
-        r = run_batch(ta, b, args.steps, args.warmup, args.kernel_iters)
+        r = run_batch(ta, b, args.steps, args.warmup, args.kernel_iters, windows=args.windows)
         for key in ("state", "last_out", "last_q"):
             r.pop(key)
         others[str(b)] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in r.items()}
 
+    # HBM traffic of a launch: counted at batch 8 with 8226 tokens in the kernel loop; K and V make up all but
+    # 0.3 % of it, so another context at batch 8 is that figure scaled by the algorithmic bytes.  Not counted for
+    # other batch sizes.
+    traffic, traffic_note = None, "counted at batch 8 only"
+    if args.batch == 8:
+        traffic = int(PMC_TRAFFIC_BYTES_B8_CTX8226 * main_res["kernel_bytes"] / PMC_ALGORITHMIC_BYTES_B8_CTX8226)
+        traffic_note = ("rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE per launch at batch 8, 8226 tokens "
+                        f"({PMC_TRAFFIC_BYTES_B8_CTX8226} bytes for {PMC_ALGORITHMIC_BYTES_B8_CTX8226} algorithmic), scaled by this run's "
+                        "algorithmic bytes per launch")
     line = {
         "metric": "decode-attn over KV cache: achieved HBM GB/s (% of peak) + us/token at 8k ctx",
         "value": round(main_res["step_gbs"], 2),
@@ -569,6 +602,12 @@ def main():
         "warmup": args.warmup,
         "ms_per_step": round(main_res["ms_per_step"], 5),
         "us_per_token": round(main_res["us_per_token"], 2),
+        "wall_ms_per_step": round(main_res["wall_ms_per_step"], 5),
+        "wall_value": round(main_res["wall_step_gbs"], 2),
+        "timing": {"value_clock": "HIP events on the stream around each window of --steps steps, median window",
+                   "windows": main_res["windows"], "window_ms_per_step_min_max": main_res["window_ms_per_step_min_max"],
+                   "wall_clock": "time.perf_counter around the same window between two device synchronisations "
+                                 "(adds one launch + one synchronisation latency per window)"},
         "pct_of_hbm_peak": round(100 * main_res["step_gbs"] / HBM_PEAK_GBS, 2),
         "higher_is_better": True,
         "scaling": "weak",
@@ -578,7 +617,9 @@ def main():
         "config": {"workload": f"cfg2: GQA decode layer 32q/8kv d=128 f16, batch {args.batch}, KV caches of {LAYERS} layers "
                                f"prefilled to {CTX} tokens, {args.steps} steps (single-token append + decode "
                                f"attention) visiting the layers round-robin; {PREWARM_LAUNCHES} untimed attention launches "
-                               f"before the warm-up steps bring the device to steady clocks",
+                               f"before the warm-up steps bring the device to steady clocks; value = algorithmic bytes of a "
+                               f"step / device time per step (HIP events on the stream around the {args.steps} steps, median of "
+                               f"{args.windows} such windows); wall_value = the same over the host's clock",
                    "batch": args.batch, "layers": LAYERS, "context": CTX, "q_heads": HQ, "kv_heads": HKV, "head_dim": D,
                    "prewarm_launches": PREWARM_LAUNCHES},
         "device": rt.device_name,
@@ -590,7 +631,8 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(main_res["kernel_gbs"] / HBM_PEAK_GBS, 4),
-            "traffic": PMC_TRAFFIC_BYTES_B8_CTX8226 if (args.batch, args.steps, args.warmup) == (8, 128, 8) else None,
+            "traffic": traffic,
+            "traffic_note": traffic_note,
             "kernel_us": round(main_res["kernel_us"], 3),
             "algorithmic_bytes_per_launch": main_res["kernel_bytes"],
             "cache_resident_achieved": round(main_res["cache_resident_kernel_gbs"], 2),
