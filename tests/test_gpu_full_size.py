@@ -102,27 +102,44 @@ def test_cfg3_full_size_chunked_prefill(rt):
     assert max_abs(got, want) <= 2e-2
 
 
-@pytest.mark.parametrize("fmt_name,T", [("Q8_0", 16384), ("Q4_0", 16384), ("Q8_0", 4096)])
+def _with_outlier_channels(x, chan):
+    """1 % of the kv_heads * head_dim channels scaled by 20, the same channels for every token."""
+    B, H, T, Dh = x.shape
+    f = x.transpose(0, 2, 1, 3).reshape(B, T, H * Dh).copy()
+    f[:, :, chan] *= 20
+    return np.ascontiguousarray(f.reshape(B, T, H, Dh).transpose(0, 2, 1, 3)).astype(np.float16)
+
+
+@pytest.mark.parametrize("fmt_name,T", [("Q8_0", 16384), ("Q4_0", 16384), ("Q8_0", 4096), ("Q4_0", 4096)])
 def test_cfg4_full_size_quantised(rt, fmt_name, T):
-    """cfg4 at full size (batch 8): blocks bit-exact via a checksum of checksums per sequence,
-    decode vs the oracle over the dequantised blocks."""
+    """cfg4 at full size (batch 8), K and V different tensors: blocks bit-exact via a checksum of
+    checksums per sequence and tensor, decode vs the oracle over the dequantised blocks (a swap of the
+    K and V planes or of their scales would fail either)."""
     B = 8
     dev_fmt, orc_fmt = getattr(tract_amd, fmt_name), getattr(orc, "FMT_" + fmt_name)
     rng = np.random.default_rng(cases.cfg_seed(4, "chan"))
     chan = rng.choice(HKV * D, size=10, replace=False)
-    k = cases.seeded_normal(cases.cfg_seed(4, "k"), (B, HKV, T, D)).transpose(0, 2, 1, 3).reshape(B, T, HKV * D).copy()
-    k[:, :, chan] *= 20
-    k = np.ascontiguousarray(k.reshape(B, T, HKV, D).transpose(0, 2, 1, 3)).astype(np.float16)
+    k = _with_outlier_channels(cases.seeded_normal(cases.cfg_seed(4, "k"), (B, HKV, T, D)), chan)
+    v = _with_outlier_channels(cases.seeded_normal(cases.cfg_seed(4, "v"), (B, HKV, T, D)), chan)
     st = tract_amd.InPlaceKvSdpa(axis=2, causal=True, storage_format=dev_fmt).state()
-    st.k.push(k), st.v.push(k)
-    kq = orc.quant(orc_fmt, k)
-    got = st.k.valid_contiguous()
-    for b in range(B):
-        assert hashlib.sha256(got[b].tobytes()).digest() == hashlib.sha256(kq[b].tobytes()).digest(), f"sequence {b}"
+    st.k.push(k), st.v.push(v)
+    kq, vq = orc.quant(orc_fmt, k), orc.quant(orc_fmt, v)
+    for name, got, want in (("K", st.k.valid_contiguous(), kq), ("V", st.v.valid_contiguous(), vq)):
+        for b in range(B):
+            assert hashlib.sha256(got[b].tobytes()).digest() == hashlib.sha256(want[b].tobytes()).digest(), f"{name}, sequence {b}"
     q = (cases.seeded_normal(cases.cfg_seed(4, "q"), (B, HQ, 1, D)) / np.sqrt(D)).astype(np.float16)
     out = st.attend(tract_amd.DeviceTensor.from_numpy(q)).to_numpy()
-    kd = orc.dequant(orc_fmt, kq, np.float16)
-    assert max_abs(out, orc.flash_sdpa(q, kd, kd, causal=True, threads=8)) <= 2e-2
+    kd, vd = orc.dequant(orc_fmt, kq, np.float16), orc.dequant(orc_fmt, vq, np.float16)
+    assert max_abs(out, orc.flash_sdpa(q, kd, vd, causal=True, threads=8)) <= 2e-2
+    # and a fused step on top: the new token quantised on append, then attended to
+    kn = _with_outlier_channels(cases.seeded_normal(31, (B, HKV, 1, D)), chan)
+    vn = _with_outlier_channels(cases.seeded_normal(32, (B, HKV, 1, D)), chan)
+    out = st.eval([q, kn, vn]).to_numpy()
+    kd = np.concatenate([kd, orc.dequant(orc_fmt, orc.quant(orc_fmt, kn), np.float16)], axis=2)
+    vd = np.concatenate([vd, orc.dequant(orc_fmt, orc.quant(orc_fmt, vn), np.float16)], axis=2)
+    assert max_abs(out, orc.flash_sdpa(q, kd, vd, causal=True, threads=8)) <= 2e-2
+    assert st.k.valid_contiguous()[:, :, T:].tobytes() == orc.quant(orc_fmt, kn).tobytes()
+    assert st.v.valid_contiguous()[:, :, T:].tobytes() == orc.quant(orc_fmt, vn).tobytes()
 
 
 def test_cfg5_ragged_long_sequences(rt):
