@@ -212,6 +212,21 @@ def time_calls(ta, fn, iters):
     return ta.Event.elapsed_ms(e0, e1) / iters * 1e3
 
 
+def parity_sample(out, q, k, v, heads, seqs=None, k_dequant=None):
+    """Max-abs difference between the GPU's `out` and the oracle's flash SDPA on a sample: query heads `heads` of
+    batch entries `seqs` (default: the first).  Runs after the timed region; the oracle is the checker only."""
+    from oracle import oracle as orc
+    g = q.shape[1] // k.shape[1]
+    worst = 0.0
+    for b in (seqs if seqs is not None else [0]):
+        for h in heads:
+            kh = h // g
+            want = orc.flash_sdpa(q[b:b + 1, h:h + 1], np.ascontiguousarray(k[b:b + 1, kh:kh + 1]),
+                                  np.ascontiguousarray(v[b:b + 1, kh:kh + 1]), causal=True, threads=8)
+            worst = max(worst, float(np.abs(want.astype(np.float32) - out[b:b + 1, h:h + 1].astype(np.float32)).max()))
+    return worst
+
+
 def base_line(args, workload, value, unit, ms_per_step, dtype, roofline, extra):
     line = {
         "metric": "decode-attn over KV cache: achieved HBM GB/s (% of peak) + us/token at 8k ctx",
@@ -279,13 +294,18 @@ def run_cfg3(ta, args):
     S, C = 512, 8
     st = ta.InPlaceKvSdpa(axis=2, causal=True).state()
     per_chunk, tot_us, tot_fl = [], 0.0, 0.0
+    ks, vs, err = [], [], 0.0
     for c in range(1, C + 1):
         k = seeded_f16(cfg_seed(3, "k") + c, (1, HKV, S, D))
         v = seeded_f16(cfg_seed(3, "v") + c, (1, HKV, S, D))
         st.k.push(k), st.v.push(v)
-        q = ta.DeviceTensor.from_numpy((seeded_f16(cfg_seed(3, "q") + c, (1, HQ, S, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16))
+        ks.append(k), vs.append(v)
+        qh = (seeded_f16(cfg_seed(3, "q") + c, (1, HQ, S, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16)
+        q = ta.DeviceTensor.from_numpy(qh)
         out = ta.DeviceTensor((1, HQ, S, D), np.float16)
         us = time_calls(ta, lambda: st.attend(q, out=out), 20)
+        if c in (1, 4, C):   # after the timing: the chunk's output against the oracle on three query heads (checker only)
+            err = max(err, parity_sample(out.to_numpy(), qh, np.concatenate(ks, axis=2), np.concatenate(vs, axis=2), [0, 13, 31]))
         pairs = S * (S * c) - S * (S - 1) // 2
         fl = 4.0 * HQ * D * pairs
         per_chunk.append({"kv_len": S * c, "us": round(us, 2), "tflops": round(fl / us / 1e6, 1)})
@@ -296,7 +316,9 @@ def run_cfg3(ta, args):
             "unit": "TFLOP/s", "frac": round(tf / 2500.0, 4), "traffic": None}
     return base_line(args, "cfg3: chunked prefill, 8 x 512 tokens into an empty cache, causal SDPA of each chunk over "
                      "the cache so far (32q/8kv d=128 f16, batch 1); attention launches only", round(tf, 1), "TFLOP/s",
-                     round(tot_us / C / 1e3, 5), "f16", roof, {"chunks": per_chunk, "total_us": round(tot_us, 1)})
+                     round(tot_us / C / 1e3, 5), "f16", roof,
+                     {"chunks": per_chunk, "total_us": round(tot_us, 1), "parity_max_abs_vs_oracle": err,
+                      "parity_sample": "chunks 1, 4 and 8, query heads 0, 13 and 31, all 512 queries, against the oracle"})
 
 
 def run_cfg4(ta, args):
@@ -317,7 +339,8 @@ def run_cfg4(ta, args):
                 for c in (st.k, st.v):
                     c.reserve(T + 128, like=(k.shape, k.dtype))
                     c.push(k)
-            q = ta.DeviceTensor.from_numpy((seeded_f16(cfg_seed(4, "q"), (B, HQ, 1, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16))
+            qh = (seeded_f16(cfg_seed(4, "q"), (B, HQ, 1, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16)
+            q = ta.DeviceTensor.from_numpy(qh)
             out = ta.DeviceTensor((B, HQ, 1, D), np.float16)
             turn = [0]
 
@@ -326,16 +349,27 @@ def run_cfg4(ta, args):
                 turn[0] += 1
 
             us = time_calls(ta, one, 100)
+            # after the timing: sequences 0 and 7, four query heads, against the oracle over the dequantised blocks
+            from oracle import oracle as orc
+            sts[0].attend(q, out=out)
+            kd = k[[0, 7]]
+            if fmt is not None:
+                ofmt = getattr(orc, "FMT_" + name.upper())
+                kd = orc.dequant(ofmt, orc.quant(ofmt, kd), np.float16)
+            o = out.to_numpy()[[0, 7]]
+            err = parity_sample(o, qh[[0, 7]], kd, kd, [0, 9, 18, 31], seqs=[0, 1])
             del sts
             by = 2 * B * HKV * T * D * ek + 2 * B * HQ * D * 2
-            res[f"{name}_ctx{T}"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by)}
+            res[f"{name}_ctx{T}"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by), "parity_max_abs_vs_oracle": err}
     head = res["q8_0_ctx16384"]
     roof = {"bound": "hbm", "kernel": "sdpa_decode_mfma_kernel<128,8,Q8_0,false,true>", "achieved": head["gbs"], "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4), "traffic": None}
     return base_line(args, "cfg4: decode over a Q8_0 / Q4_0 quantised KV cache (fused dequant), batch 8, contexts 4096 "
                      "and 16384, 1% outlier channels x20; attention launches only, rotating over 2-4 layers' caches; "
                      "headline = Q8_0 at 16384",
-                     head["gbs"], "GB/s", round(head["us"] / 1e3, 5), "q8_0/f16", roof, {"cases": res})
+                     head["gbs"], "GB/s", round(head["us"] / 1e3, 5), "q8_0/f16", roof,
+                     {"cases": res, "parity_max_abs_vs_oracle": max(c["parity_max_abs_vs_oracle"] for c in res.values()),
+                      "parity_sample": "every case: sequences 0 and 7, query heads 0, 9, 18, 31, against the oracle's attention over the dequantised blocks"})
 
 
 def run_cfg5(ta, args):
@@ -370,6 +404,11 @@ def run_cfg5(ta, args):
     tot = int(sum(c.len() for c in kcs))
     by = 2 * HKV * D * 2 * tot + 2 * n_seq * HQ * D * 2 + 2 * n_seq * HKV * D * 2
     us_k = time_calls(ta, lambda: ta.sdpa_decode_ragged(qs[0], kcs, vcs, workspace=ws, out=out), 20)
+    # after the timing: the last launch's output for the shortest, the longest and two other sequences against the
+    # oracle over those sequences' caches as they now are (read back from the device)
+    o, q0 = out.to_numpy(), qs[0].to_numpy()
+    sample = sorted({int(np.argmin(lens)), int(np.argmax(lens)), 7, 40})
+    err = max(parity_sample(o[i:i + 1], q0[i:i + 1], kcs[i].valid_contiguous(), vcs[i].valid_contiguous(), [0, 13, 31]) for i in sample)
     roof = {"bound": "hbm", "kernel": "sdpa_decode_mfma_ragged_kernel<128,8,F16,true>", "achieved": round(by / us_k / 1e3, 1),
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(by / us_k / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
             "kernel_us": round(us_k, 2), "algorithmic_bytes_per_launch": int(by)}
@@ -378,7 +417,9 @@ def run_cfg5(ta, args):
                      "capacity-doubling caches in one pool, one fused append+attention call per step",
                      round(by / dt / 1e9, 1), "GB/s", round(dt * 1e3, 5), "f16", roof,
                      {"steps": steps, "us_per_step": round(dt * 1e6, 1), "pool_bytes": st["bytes_total"],
-                      "pool_in_use": st["bytes_in_use"], "pct_of_hbm_peak": round(100 * by / dt / 1e9 / HBM_PEAK_GBS, 2)})
+                      "pool_in_use": st["bytes_in_use"], "pct_of_hbm_peak": round(100 * by / dt / 1e9 / HBM_PEAK_GBS, 2),
+                      "parity_max_abs_vs_oracle": err,
+                      "parity_sample": f"sequences {sample} (shortest, longest, two others), query heads 0, 13, 31, after the timed steps"})
 
 
 def run_ops(ta, args):
