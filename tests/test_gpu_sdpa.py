@@ -556,6 +556,42 @@ def test_ragged_decode_with_a_thousand_short_sequences(rt):
         assert max_abs(out[i:i + 1], orc.flash_sdpa(q[i:i + 1], ks[i], vs[i], causal=True)) <= 2e-2, f"sequence {i}"
 
 
+@pytest.mark.parametrize("n_seq", [600, 2048])
+def test_ragged_decode_with_many_sequences_of_a_grouped_head_model(rt, n_seq):
+    """32 query heads on 8 kv heads at head_dim 128 (padded groups of 8 rows per record) with a workspace of exactly
+    the size the library asks for: many short sequences that are one work item each (they need no partial record)
+    next to a few long ones that are cut."""
+    rng = np.random.default_rng(n_seq)
+    Hq, Hkv, D = 32, 8, 128
+    lens = rng.integers(1, 48, size=n_seq, endpoint=True)
+    lens[[3, n_seq // 2, n_seq - 1]] = [9000, 5000, 2500]
+    pool = tract_amd.KvPool(int(lens.sum()) * Hkv * D * 2 * 2 * 2 + (128 << 20))
+    kcs, vcs, ks, vs = [], [], [], []
+    for n in lens:
+        k = rng.standard_normal((1, Hkv, int(n), D), dtype=np.float32).astype(np.float16)
+        v = rng.standard_normal((1, Hkv, int(n), D), dtype=np.float32).astype(np.float16)
+        kc, vc = tract_amd.InPlaceKvCache(2, pool=pool), tract_amd.InPlaceKvCache(2, pool=pool)
+        kc.push(k), vc.push(v)
+        kcs.append(kc), vcs.append(vc), ks.append(k), vs.append(v)
+    q = (rng.standard_normal((n_seq, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    ws = tract_amd.Workspace(n_seq, Hq, 1, D)
+    assert ws.nbytes == tract_amd.Workspace.bytes_for(n_seq, Hq, 1, D)
+    qd = tract_amd.DeviceTensor.from_numpy(q)
+    out = tract_amd.sdpa_decode_ragged(qd, kcs, vcs, workspace=ws).to_numpy()
+    assert not np.isnan(out).any()
+    for i in sorted(set(range(0, n_seq, 41)) | {3, n_seq // 2, n_seq - 1}):
+        assert max_abs(out[i:i + 1], orc.flash_sdpa(q[i:i + 1], ks[i], vs[i], causal=True)) <= 2e-2, f"sequence {i}"
+    # a fused step on the same workspace
+    kn = rng.standard_normal((n_seq, Hkv, 1, D), dtype=np.float32).astype(np.float16)
+    vn = rng.standard_normal((n_seq, Hkv, 1, D), dtype=np.float32).astype(np.float16)
+    out = tract_amd.inplace_kv_sdpa_eval_ragged(qd, tract_amd.DeviceTensor.from_numpy(kn), tract_amd.DeviceTensor.from_numpy(vn),
+                                                kcs, vcs, workspace=ws).to_numpy()
+    for i in sorted(set(range(0, n_seq, 97)) | {3, n_seq - 1}):
+        kk, vv = np.concatenate([ks[i], kn[i:i + 1]], 2), np.concatenate([vs[i], vn[i:i + 1]], 2)
+        assert max_abs(out[i:i + 1], orc.flash_sdpa(q[i:i + 1], kk, vv, causal=True)) <= 2e-2, f"fused step, sequence {i}"
+        assert kcs[i].valid_contiguous().tobytes() == kk.tobytes()
+
+
 def test_ragged_equals_padded_batch_with_mask(rt):
     """The reference's statement of a ragged batch: a dense batch padded to the longest
     sequence with an additive mask whose padded columns are <= -65504 (flash_sdpa.rs:261-268)."""

@@ -668,13 +668,14 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     for (int64_t i = 0; i < n_seq; i++) total_tiles += (seqs[i].len + kTile - 1) / kTile;
     TROCM_REQUIRE(workspace_bytes > kWsCounterBytes + kWsPlanBytes, "sdpa workspace too small for a ragged launch (%zu bytes)",
                   workspace_bytes);
+    // Partial records are needed only by the items of sequences that are cut: a sequence that is one item writes its
+    // output rows itself.  (Two limits, then: items in the plan table, records in the rest of the workspace.)
     const int64_t rows_cap = (int64_t)((workspace_bytes - kWsCounterBytes - kWsPlanBytes) / ((D + 2) * sizeof(float)));
-    const int64_t max_items_ws = rows_cap / (Hkv * G);  // every item may need a partial record per (padded) q head
+    const int64_t max_slots_ws = rows_cap / (Hkv * G);  // a record has a row per (padded) query head of every kv head
     const int64_t max_items_tbl =
         ((int64_t)kWsPlanBytes - n_seq * (int64_t)sizeof(RaggedSeqSlots)) / (int64_t)sizeof(RaggedItem);
-    const int64_t max_items = max_items_ws < max_items_tbl ? max_items_ws : max_items_tbl;
-    TROCM_REQUIRE(max_items >= n_seq,
-                  "sdpa workspace too small for %lld sequences (%zu bytes)", (long long)n_seq, workspace_bytes);
+    TROCM_REQUIRE(max_items_tbl >= n_seq, "ragged decode: the plan area holds %lld work items, fewer than the %lld sequences",
+                  (long long)max_items_tbl, (long long)n_seq);
     // Workgroups (items x kv heads) per compute unit: two are resident at a time, and the last round of
     // them is only partly full, so more and smaller items shorten the tail at the cost of partial records.
     static const int wg_per_cu = getenv("TROCM_RAGGED_WG_PER_CU") ? atoi(getenv("TROCM_RAGGED_WG_PER_CU")) : 0;
@@ -682,21 +683,23 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     if (want_items < 1) want_items = 1;
     int64_t tiles_per_item = (total_tiles + want_items - 1) / want_items;
     if (tiles_per_item < kWaves) tiles_per_item = kWaves;
-    int64_t n_items = 0;
-    for (;;) {
-        n_items = 0;
+    int64_t n_items = 0, n_slots = 0;
+    for (;;) {   // ends at the latest when no sequence is cut: n_seq items, no records
+        n_items = n_slots = 0;
         for (int64_t i = 0; i < n_seq; i++) {
             int64_t tiles = (seqs[i].len + kTile - 1) / kTile;
-            n_items += (tiles + tiles_per_item - 1) / tiles_per_item;
+            int64_t ns = (tiles + tiles_per_item - 1) / tiles_per_item;
+            n_items += ns;
+            if (ns > 1) n_slots += ns;
         }
-        if (n_items <= max_items) break;
+        if (n_items <= max_items_tbl && n_slots <= max_slots_ws) break;
         tiles_per_item += (tiles_per_item + 3) / 4;
     }
     StageSlot *stage;
     if (acquire_stage(&stage)) return 1;
     RaggedItem *items = (RaggedItem *)stage->host;
     RaggedSeqSlots *slots = (RaggedSeqSlots *)(items + n_items);
-    int64_t it = 0;
+    int64_t it = 0, slot_it = 0;
     bool any_split = false;
     int64_t max_split = 1;
     for (int64_t i = 0; i < n_seq; i++) {
@@ -704,8 +707,9 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
         int64_t ns = (tiles + tiles_per_item - 1) / tiles_per_item;
         int64_t tps = (tiles + ns - 1) / ns;
         ns = (tiles + tps - 1) / tps;
-        slots[i].slot0 = (int)it;
+        slots[i].slot0 = (int)slot_it;   // first partial record of the sequence (unused when it is not cut)
         slots[i].nsplit = (int)ns;
+        if (ns > 1) slot_it += ns;
         any_split |= ns > 1;
         if (ns > max_split) max_split = ns;
         for (int64_t sp = 0; sp < ns; sp++, it++) {
@@ -752,7 +756,7 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     p.k_new = (const char *)k_new;
     p.v_new = (const char *)v_new;
     p.part_ml = (float *)((char *)workspace + kWsCounterBytes + kWsPlanBytes);
-    p.part_o = p.part_ml + (size_t)n_items * Hkv * 2 * G;
+    p.part_o = p.part_ml + (size_t)slot_it * Hkv * 2 * G;
     const RaggedItem *d_items = (const RaggedItem *)((char *)workspace + kWsCounterBytes);
     const RaggedSeqSlots *d_slots = (const RaggedSeqSlots *)(d_items + n_items);
     // The MFMA kernel merges the splits of a sequence-head itself when none has more than it can hold in registers.
