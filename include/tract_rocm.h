@@ -269,8 +269,10 @@ int trocm_sdpa_workspace_init(void *workspace, size_t bytes, void *stream);
  *            mask_batch in {1, batch}, mask_heads in {1, q_heads} (the broadcast the CUDA
  *            dispatch expresses with zero strides, cuda/src/kernels/flash_attn.rs:138-143);
  *            must be NULL when causal (sdpa.rs:297-299).  Values may be finite minima
- *            (sdpa.rs:550-553) or -inf; a row masked entirely with -inf yields NaN, as on the
- *            CPU.  The split-K decode and MFMA prefill kernels take the mask themselves; with
+ *            (sdpa.rs:550-553) or -inf; a query row masked entirely with -inf yields zeros in every
+ *            kernel: what the CPU op returns when its tile skip drops all of the row's key tiles
+ *            (flash_sdpa.rs:267-274, :253; always so for q_len == 1), where its NaN for such a row
+ *            inside a partly visible query tile (:309-316) is not reproduced.  The split-K decode and MFMA prefill kernels take the mask themselves; with
  *            q_len == 1 and mask_heads == 1 (a batch padded to its longest sequence,
  *            flash_sdpa.rs:261-268) the columns after the last one above -60000 weigh nothing and
  *            are not read.

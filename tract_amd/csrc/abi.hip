@@ -141,9 +141,80 @@ struct trocm_kv_cache {
     int64_t window, cursor;
 };
 
+// Planes that a growing cache has left behind.  Work queued on the stream may still read them, so they are not
+// freed at once (that would take a stream synchronisation inside an asynchronous append): an event recorded on the
+// stream after the copy into the new planes guards them, and they are released by a later call that finds the
+// event complete (growth, reserve, destroy, pool statistics), or that needs the memory and waits for it.
+struct DeferredFree {
+    void *data, *scales;
+    trocm_kv_pool *pool;   // NULL: planes of their own (hipFree)
+    hipEvent_t done;
+};
+static std::mutex g_deferred_mu;
+static std::vector<DeferredFree> g_deferred;
+
+static void release_planes(trocm_kv_pool *pool, void *data, void *scales) {
+    if (pool) {
+        if (data) pool_free(pool, data);
+        if (scales) pool_free(pool, scales);
+    } else {
+        if (data) (void)hipFree(data);
+        if (scales) (void)hipFree(scales);
+    }
+}
+
+// Release the deferred planes whose event has completed; with `wait`, all of them (of `only_pool`, if given).
+// hipFree waits for the whole device, so planes outside a pool are released only where the host is waiting anyway
+// (`unpooled`: the synchronising calls, destroy, a failed allocation); a pool's bookkeeping costs nothing.
+static void reap_deferred(bool wait, trocm_kv_pool *only_pool = nullptr, bool unpooled = true) {
+    std::vector<DeferredFree> ready;
+    {
+        std::lock_guard<std::mutex> lock(g_deferred_mu);
+        for (size_t i = 0; i < g_deferred.size();) {
+            DeferredFree &d = g_deferred[i];
+            const bool mine = (only_pool == nullptr || d.pool == only_pool) && (unpooled || d.pool != nullptr);
+            bool done = mine && hipEventQuery(d.done) == hipSuccess;
+            if (mine && !done && wait) done = hipEventSynchronize(d.done) == hipSuccess;
+            if (done) {
+                ready.push_back(d);
+                g_deferred[i] = g_deferred.back();
+                g_deferred.pop_back();
+            } else {
+                i++;
+            }
+        }
+        (void)hipGetLastError();   // "not ready" is an answer, not a failure: keep it away from the launch checks
+    }
+    for (DeferredFree &d : ready) {
+        (void)hipEventDestroy(d.done);
+        release_planes(d.pool, d.data, d.scales);
+    }
+}
+
+// Hand the planes over to the deferred list, guarded by an event recorded on `s` now.
+static int defer_free(trocm_kv_pool *pool, void *data, void *scales, hipStream_t s) {
+    if (!data && !scales) return 0;
+    DeferredFree d{data, scales, pool, nullptr};
+    hipError_t e = hipEventCreateWithFlags(&d.done, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventRecord(d.done, s);
+    if (e != hipSuccess) {   // no event: fall back to waiting for the stream
+        if (d.done) (void)hipEventDestroy(d.done);
+        TROCM_HIP(hipStreamSynchronize(s));
+        release_planes(pool, data, scales);
+        return 0;
+    }
+    std::lock_guard<std::mutex> lock(g_deferred_mu);
+    g_deferred.push_back(d);
+    return 0;
+}
+
 static int plane_alloc(trocm_kv_cache *c, void **ptr, size_t bytes, const char *what) {
     if (c->pool) {
         *ptr = pool_alloc(c->pool, bytes);
+        if (!*ptr) {   // planes of this pool that wait for their event may make the room
+            reap_deferred(true, c->pool);
+            *ptr = pool_alloc(c->pool, bytes);
+        }
         if (!*ptr) {
             std::lock_guard<std::mutex> lock(c->pool->mu);
             return fail("KV pool exhausted: %s of %zu bytes does not fit (%zu of %zu bytes in use)", what, bytes,
@@ -152,6 +223,11 @@ static int plane_alloc(trocm_kv_cache *c, void **ptr, size_t bytes, const char *
         return 0;
     }
     hipError_t e = hipMalloc(ptr, bytes ? bytes : 16);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        reap_deferred(true);
+        e = hipMalloc(ptr, bytes ? bytes : 16);
+    }
     if (e != hipSuccess) return fail("allocating %s (%zu bytes) failed: %s", what, bytes, hipGetErrorString(e));
     return 0;
 }
@@ -211,6 +287,7 @@ static int copy_valid(const trocm_kv_cache *c, void *dst, void *dst_scales, int6
 // Replace the buffers by ones of `new_cap` tokens holding the valid region
 // (grow(), transformers/src/ops/inplace_kv_cache.rs:106-113; the tail stays uninitialised).
 static int regrow(trocm_kv_cache *c, int64_t new_cap, hipStream_t s) {
+    reap_deferred(false, nullptr, false);
     void *nd = nullptr, *ns = nullptr;
     const int64_t new_pitch = pitch_for(new_cap);
     size_t pb = plane_bytes(c, new_pitch), sb = scale_plane_bytes(c, new_pitch);
@@ -226,21 +303,27 @@ static int regrow(trocm_kv_cache *c, int64_t new_cap, hipStream_t s) {
             return 1;
         }
     }
-    if (c->data) {
-        // The old buffers may still be read by work queued on the stream.
-        hipError_t e = hipStreamSynchronize(s);
-        if (e != hipSuccess) {
-            (void)plane_free(c, nd);
-            (void)plane_free(c, ns);
-            return fail("hipStreamSynchronize failed while growing a KV cache: %s", hipGetErrorString(e));
-        }
-        if (plane_free(c, c->data)) return 1;
-        if (plane_free(c, c->scales)) return 1;
+    // The old planes may still be read by work queued on the stream (the copy above, earlier attention calls):
+    // they are released once an event recorded here has completed, by a later call; the host does not wait.
+    if (c->data && defer_free(c->pool, c->data, c->scales, s)) {
+        (void)plane_free(c, nd);
+        (void)plane_free(c, ns);
+        return 1;
     }
     c->data = nd;
     c->scales = ns;
     c->cap = new_cap;
     c->pitch = new_pitch;
+    return 0;
+}
+
+// A call that grew K and then failed to grow V (a pool that ran out) leaves the two capacities apart, and attention
+// takes one row pitch for both: the next call brings the smaller cache up to the larger before anything else.
+static int equalise_capacities(trocm_kv_cache *kc, trocm_kv_cache *vc, hipStream_t s) {
+    if (kc->cap == vc->cap || kc->window || vc->window) return 0;
+    trocm_kv_cache *small = kc->cap < vc->cap ? kc : vc, *big = kc->cap < vc->cap ? vc : kc;
+    if (regrow(small, big->cap, s)) return 1;
+    small->reallocs += 1;   // the growth that the failed call owed
     return 0;
 }
 
@@ -352,12 +435,14 @@ int trocm_stream_sync(void *stream) {
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
     TROCM_HIP(hipStreamSynchronize(s));
+    reap_deferred(false);   // planes that growing caches left behind and nothing reads any more
     return 0;
 }
 
 int trocm_device_sync(void) {
     if (ensure_init()) return 1;
     TROCM_HIP(hipDeviceSynchronize());
+    reap_deferred(false);
     return 0;
 }
 
@@ -461,6 +546,11 @@ int trocm_kv_cache_create_in_pool(trocm_kv_cache **out, trocm_kv_pool *pool, int
 
 int trocm_kv_cache_destroy(trocm_kv_cache *c) {
     if (!c) return 0;
+    reap_deferred(false);
+    // No stream is known here and kernels queued anywhere may still read the planes: hipFree waits for the device
+    // by itself, the pool's bookkeeping does not, so a pooled cache waits explicitly before its planes can be
+    // handed to another cache.
+    if (c->pool && (c->data || c->scales)) (void)hipDeviceSynchronize();
     int rc = plane_free(c, c->data);
     rc |= plane_free(c, c->scales);
     if (c->pool) {
@@ -491,6 +581,7 @@ int trocm_kv_pool_create(trocm_kv_pool **out, size_t bytes) {
 
 int trocm_kv_pool_destroy(trocm_kv_pool *p) {
     if (!p) return 0;
+    reap_deferred(true, p);
     TROCM_REQUIRE(p->live_caches == 0, "kv pool still has %lld live caches", (long long)p->live_caches);
     TROCM_HIP(hipFree(p->base));
     delete p;
@@ -500,6 +591,7 @@ int trocm_kv_pool_destroy(trocm_kv_pool *p) {
 int trocm_kv_pool_stats(trocm_kv_pool *p, size_t *bytes_total, size_t *bytes_in_use, size_t *largest_free,
                         void **base) {
     TROCM_NOT_NULL(p);
+    reap_deferred(true, p);   // planes left behind by growth count as free once their last reader has finished
     std::lock_guard<std::mutex> lock(p->mu);
     if (bytes_total) *bytes_total = p->bytes;
     if (bytes_in_use) *bytes_in_use = p->in_use;
@@ -644,6 +736,9 @@ int trocm_kv_append_pair(trocm_kv_cache *kc, trocm_kv_cache *vc, const void *k_s
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
     TROCM_REQUIRE(kc->window == vc->window, "K and V caches differ in window");
+    TROCM_NOT_NULL(k_src);
+    TROCM_NOT_NULL(v_src);
+    if (kc->len == vc->len && equalise_capacities(kc, vc, s)) return 1;
     if (append_prepare(kc, k_src, src_dtype, src_strides, n_new, s)) return 1;
     if (append_prepare(vc, v_src, src_dtype, src_strides, n_new, s)) return 1;
     if (kc->window) {
@@ -1079,12 +1174,41 @@ static void cached_args(SdpaArgs &a, const void *q, int q_dtype, int64_t q_heads
     a.workspace = workspace, a.workspace_bytes = workspace_bytes;
 }
 
+// Everything an append + attention call can be refused for, checked before either cache is touched: a call that
+// fails leaves the caches as they were and can be repeated.
+static int inplace_eval_check(const char *what, const void *q, const void *k_new, const void *v_new, const void *out, int dtype,
+                              int64_t q_heads, int64_t n_new, const trocm_kv_cache *kc, const trocm_kv_cache *vc) {
+    TROCM_NOT_NULL(kc);
+    TROCM_NOT_NULL(vc);
+    TROCM_NOT_NULL(q);
+    TROCM_NOT_NULL(k_new);
+    TROCM_NOT_NULL(v_new);
+    TROCM_NOT_NULL(out);
+    TROCM_REQUIRE(dtype == TROCM_F32 || dtype == TROCM_F16, "%s: dtype must be F32 or F16", what);
+    TROCM_REQUIRE(n_new >= 0, "append: negative token count");
+    TROCM_REQUIRE(kc->fmt == vc->fmt && kc->B == vc->B && kc->H == vc->H && kc->D == vc->D,
+                  "K and V caches differ in format or shape");
+    TROCM_REQUIRE(kc->window == vc->window, "K and V caches differ in window");
+    TROCM_REQUIRE(kc->len == vc->len, "K/V lengths must match (%lld vs %lld)", (long long)kc->len, (long long)vc->len);
+    TROCM_REQUIRE(is_quant(kc->fmt) || kc->fmt == dtype, "q dtype %d does not match the cache format %d", dtype, kc->fmt);
+    TROCM_REQUIRE(q_heads >= 1 && q_heads % kc->H == 0, "Q heads (%lld) must be a multiple of K/V heads (%lld)", (long long)q_heads,
+                  (long long)kc->H);
+    TROCM_REQUIRE(kc->len + n_new > 0, "empty kv-cache");  // inplace_kv_cache.rs:91
+    return 0;
+}
+
 int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_new, int dtype, int64_t q_heads,
                                int64_t n_new, const int64_t *kv_new_strides, trocm_kv_cache *kc, trocm_kv_cache *vc,
                                void *out, float scale, int causal, void *workspace, size_t workspace_bytes,
                                void *stream) {
-    TROCM_NOT_NULL(kc);
-    TROCM_NOT_NULL(vc);
+    if (inplace_eval_check("inplace_kv_sdpa", q, k_new, v_new, out, dtype, q_heads, n_new, kc, vc)) return 1;
+    if (kv_new_strides)
+        for (int i = 0; i < 4; i++) TROCM_REQUIRE(kv_new_strides[i] >= 0, "append: negative source strides are not supported");
+    {
+        hipStream_t s0;
+        if (resolve_stream(stream, &s0)) return 1;
+        if (equalise_capacities(kc, vc, s0)) return 1;
+    }
     int64_t dense[4];
     dense[3] = 1, dense[2] = kc->D, dense[1] = n_new * kc->D, dense[0] = kc->H * n_new * kc->D;
     bool is_dense = kv_new_strides == nullptr;
@@ -1129,6 +1253,10 @@ int trocm_window_kv_sdpa_eval(const void *q, const void *k_new, const void *v_ne
     TROCM_NOT_NULL(kc);
     TROCM_NOT_NULL(vc);
     TROCM_REQUIRE(kc->window > 0 && vc->window == kc->window, "window_kv_sdpa: K and V must be sliding-window caches of one window");
+    if (inplace_eval_check("window_kv_sdpa", q, k_new, v_new, out, dtype, q_heads, n_new, kc, vc)) return 1;
+    TROCM_REQUIRE(kc->cursor == vc->cursor, "K and V ring cursors must match");
+    if (kv_new_strides)
+        for (int i = 0; i < 4; i++) TROCM_REQUIRE(kv_new_strides[i] >= 0, "append: negative source strides are not supported");
     int64_t dense[4];
     dense[3] = 1, dense[2] = kc->D, dense[1] = n_new * kc->D, dense[0] = kc->H * n_new * kc->D;
     bool is_dense = kv_new_strides == nullptr;

@@ -164,7 +164,8 @@ __device__ __forceinline__ void merge_head(const DecodeDev &p, int64_t first, in
         float cm = -INFINITY;
         for (int sp = 0; sp < n; sp++) cm = fmaxf(cm, lds_m[sp]);
         const float m_new = fmaxf(m_run, cm);
-        const float keep = fast_exp2(m_run - m_new);   // 0 on the first chunk
+        const float m_ref = m_new == -INFINITY ? 0.0f : m_new;   // every split masked out with -inf so far: weights 0, not NaN
+        const float keep = fast_exp2(m_run - m_ref);   // 0 on the first chunk
         acc *= keep;
         ll *= keep;
         m_run = m_new;
@@ -172,12 +173,12 @@ __device__ __forceinline__ void merge_head(const DecodeDev &p, int64_t first, in
         const int64_t po_step = stride * (G * D);
 #pragma unroll 8
         for (int sp = 0; sp < n; sp++) {
-            const float f = fast_exp2(lds_m[sp] - m_new);
+            const float f = fast_exp2(lds_m[sp] - m_ref);
             acc += po[sp * po_step] * f;
             ll += lds_l[sp] * f;
         }
     }
-    out_row[tid] = from_f32<T>(acc / ll);
+    out_row[tid] = from_f32<T>(ll > 0.0f ? acc / ll : 0.0f);   // a row masked out entirely with -inf: zeros
 }
 
 // In-kernel merge by the last workgroup of a (sequence, kv head) to arrive.  Every workgroup calls this
@@ -223,6 +224,7 @@ __device__ __forceinline__ void tail_merge(const DecodeDev &p, int *counter, int
         float mm = -INFINITY;
 #pragma unroll
         for (int sp = 0; sp < kTailMergeMax; sp++) mm = fmaxf(mm, mv[e][sp]);
+        if (mm == -INFINITY) mm = 0.0f;   // a row masked out entirely with -inf: weights 0, not NaN
         float acc = 0.0f, ll = 0.0f;
 #pragma unroll
         for (int sp = 0; sp < kTailMergeMax; sp++) {
@@ -230,7 +232,7 @@ __device__ __forceinline__ void tail_merge(const DecodeDev &p, int *counter, int
             acc += ov[e][sp] * f;
             ll += lv[e][sp] * f;
         }
-        if (idx < p.g_real * D) out[idx] = from_f32<T>(acc / ll);
+        if (idx < p.g_real * D) out[idx] = from_f32<T>(ll > 0.0f ? acc / ll : 0.0f);
     }
 }
 
@@ -275,7 +277,7 @@ __device__ __forceinline__ void tail_merge_wide(const DecodeDev &p, int *counter
         float ll = l * f;
 #pragma unroll
         for (int d = 1; d < kWideMergeMax; d <<= 1) ll += __shfl_xor(ll, d, 64);
-        lds_w[tid] = f / ll;
+        lds_w[tid] = ll > 0.0f ? f / ll : 0.0f;
     }
     __syncthreads();
 #pragma unroll

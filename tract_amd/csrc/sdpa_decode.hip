@@ -311,7 +311,7 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
             ll += comb[ww * kCombStride + G * D + G + h] * f;
         }
         if (wk.direct) {
-            if (h < p.g_real) out[idx] = from_f32<T>(acc / ll);
+            if (h < p.g_real) out[idx] = from_f32<T>(ll > 0.0f ? acc / ll : 0.0f);
         } else if (wk.counter == nullptr) {
             int64_t slot = wk.part;
             p.part_o[slot * (G * D) + idx] = acc;

@@ -430,7 +430,7 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
             ll += comb[ww * kCombStride + GP * D + GP + h] * f;
         }
         if (wk.nsplit == 1) {
-            if (h < g) out[idx] = __float2half_rn(acc / ll);
+            if (h < g) out[idx] = __float2half_rn(ll > 0.0f ? acc / ll : 0.0f);
         } else if (wk.counter == nullptr) {
             p.part_o[slot * (GP * D) + idx] = acc;
             if ((idx % D) == 0) {

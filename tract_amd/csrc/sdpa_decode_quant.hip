@@ -354,7 +354,7 @@ __global__ __launch_bounds__(kThreads, G <= 4 ? 2 : 1) void sdpa_decode_q_kernel
             ll += comb[ww][G * D + G + h] * f;
         }
         if (p.nsplit == 1) {
-            if (h < p.g_real) out[idx] = __float2half_rn(acc / ll);
+            if (h < p.g_real) out[idx] = __float2half_rn(ll > 0.0f ? acc / ll : 0.0f);
         } else if (p.counters == nullptr) {
             int64_t slot = bh * p.nsplit + split;
             p.part_o[slot * (G * D) + idx] = acc;
