@@ -422,6 +422,57 @@ def run_cfg5(ta, args):
                       "parity_sample": f"sequences {sample} (shortest, longest, two others), query heads 0, 13, 31, after the timed steps"})
 
 
+def run_append(ta, args):
+    """Kernels (1) and (2) on their own: the bulk append of a prefill (8 sequences x 8 kv heads x 16384 tokens x 128,
+    f16 source) into a reserved cache, as plain f16 rows and quantised to Q8_0 / Q4_0 on the way, and the append of one
+    decode token per sequence.  Two sources and two caches in turn (each pair moves more than the 256 MB Infinity Cache).
+    Algorithmic bytes per element: 2 read + 2, 34/32 or 18/32 written."""
+    from oracle import oracle as orc
+    B, T = 8, 16384
+    n_el = B * HKV * T * D
+    srcs = [ta.DeviceTensor.from_numpy(seeded_f16(cfg_seed(4, "k") + i, (B, HKV, T, D))) for i in range(2)]
+    tok = ta.DeviceTensor.from_numpy(seeded_f16(cfg_seed(4, "k") + 9, (B, HKV, 1, D)))
+    res, turn = {}, [0]
+    for name, fmt, wb in (("f16", None, 2.0), ("q8_0", ta.Q8_0, 34 / 32), ("q4_0", ta.Q4_0, 18 / 32)):
+        caches = [ta.InPlaceKvCache(2, storage_format=fmt) for _ in range(2)]
+        for c in caches:
+            c.reserve(T + 64, like=((B, HKV, T, D), np.float16))
+            c.push(srcs[0])
+
+        def bulk():
+            c = caches[turn[0] % 2]
+            c.truncate(0)
+            c.push(srcs[turn[0] % 2])
+            turn[0] += 1
+
+        us = time_calls(ta, bulk, 20)
+        by = n_el * (2 + wb)
+        res[f"bulk_append_{name}_8x8x16384x128"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by)}
+
+        def one_token():
+            c = caches[turn[0] % 2]
+            c.truncate(T)
+            c.push(tok)
+            turn[0] += 1
+
+        us1 = time_calls(ta, one_token, 200)
+        res[f"token_append_{name}_8x8x1x128"] = {"us": round(us1, 2)}
+        if fmt is not None:   # after the timing: the stored blocks of two heads against the oracle's, bit for bit
+            c = caches[(turn[0] + 1) % 2]
+            c.truncate(0)
+            c.push(srcs[1])
+            got = c.valid_contiguous()[3, 5]
+            want = orc.quant(getattr(orc, "FMT_" + name.upper()), srcs[1].to_numpy()[3, 5])
+            res[f"bulk_append_{name}_8x8x16384x128"]["blocks_bit_exact_vs_oracle"] = bool(got.tobytes() == want.tobytes())
+        del caches
+    head = res["bulk_append_q8_0_8x8x16384x128"]
+    roof = {"bound": "hbm", "kernel": "quant_append_kernel<f16> (Q8_0)", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(head["gbs"] / HBM_PEAK_GBS, 4), "traffic": None}
+    return base_line(args, "append: bulk append of a 16384-token prefill (batch 8, 8 kv heads, d=128, f16 source) into a reserved "
+                     "cache as f16 rows, Q8_0 and Q4_0 blocks, and the append of one token per sequence; headline = Q8_0 bulk append",
+                     head["gbs"], "GB/s", round(head["us"] / 1e3, 5), "f16->q8_0", roof, {"cases": res})
+
+
 def run_ops(ta, args):
     """The ops either side of the cache (RoPE, cast) and the sliding-window decode step, each against
     its HBM roofline, with the oracle timed on the host for the same ops (smaller sample)."""
@@ -591,7 +642,7 @@ def main():
     ap.add_argument("--kernel-iters", type=int, default=200)
     ap.add_argument("--windows", type=int, default=5, help="how many times the timed window of --steps steps is taken (median reported)")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "ops"],
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "ops", "append"],
                     help="cfg2 (default) is the configuration the metric is quoted on; the others print one line "
                          "of the same shape for the remaining configurations")
     args = ap.parse_args()
@@ -603,7 +654,7 @@ def main():
     import tract_amd as ta
     rt = ta.runtime_for_name("rocm")
     if args.workload != "cfg2":
-        line = {"cfg1": run_cfg1, "cfg3": run_cfg3, "cfg4": run_cfg4, "cfg5": run_cfg5, "ops": run_ops}[args.workload](ta, args)
+        line = {"cfg1": run_cfg1, "cfg3": run_cfg3, "cfg4": run_cfg4, "cfg5": run_cfg5, "ops": run_ops, "append": run_append}[args.workload](ta, args)
         line["device"] = rt.device_name
         print(json.dumps(line))
         return
