@@ -19,8 +19,13 @@
 // launch, both shared with the other decode kernels.  A step's new token can be handed in and is stored to
 // the cache by the kernel (f16 caches); an additive mask row per head can join the scores (f16 caches).
 //
-// Roofline: HBM-bound (f16) / bound by vector-instruction issue (quantised).  Algorithmic bytes as for
-// sdpa_decode.hip and sdpa_decode_quant.hip.
+// Block-quantised caches at head_dim 128 with up to 16 heads per kv head do not dequantise at all: the raw codes go
+// into the matrix cores as exact f16 integers, one 32-deep product per quantisation block, and the block scales are
+// applied to the products (decode_mfma_qblock_body).
+//
+// Roofline: HBM-bound (f16) / bound by vector-instruction issue and the latency of a tile's dependent chain
+// (quantised).  Algorithmic bytes as for sdpa_decode.hip and sdpa_decode_quant.hip.
+#include <type_traits>
 #include "decode_common.h"
 
 namespace trocm {
@@ -28,6 +33,7 @@ namespace {
 
 typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 // Transposing 64-bit LDS load of 16-bit elements: in each block of 16 lanes, lane i receives
 // element i%4 of the four 8-byte rows addressed by lanes i/4, i/4+4, i/4+8, i/4+12.
@@ -67,6 +73,54 @@ struct MfmaWork {
     int64_t part_first, part_stride;   // partial records of this sequence-head: first, first + stride, ...
     const char *mask;             // additive mask row of this kv head's first query head, token 0 (MASK instantiations)
 };
+
+// The tail every formulation shares: the four waves' records (O[GP][D], m[GP], l[GP], in `lds_raw`, kCombStride floats
+// each) become the output rows (one split), or this workgroup's partial record, merged by the last workgroup to
+// arrive or by the merge launch.
+template <int D, int GP>
+__device__ __forceinline__ void wave_records_to_output(const DecodeDev &p, const MfmaWork &wk, unsigned char *lds_raw, int64_t head0,
+                                                       int g, int tid) {
+    constexpr int kCombStride = GP * D + 2 * GP;
+    float *comb = reinterpret_cast<float *>(lds_raw);   // [kWaves][GP*D + 2*GP]
+    __syncthreads();
+    __half *out = reinterpret_cast<__half *>(p.out) + head0 * D;
+    const int64_t slot = wk.slot;
+    for (int idx = tid; idx < GP * D; idx += kThreads) {
+        const int h = idx / D;
+        float mm = -INFINITY;
+#pragma unroll
+        for (int ww = 0; ww < kWaves; ww++) mm = fmaxf(mm, comb[ww * kCombStride + GP * D + h]);
+        const float mm_ref = mm == -INFINITY ? 0.0f : mm;   // a wave without tiles holds (0, -inf, 0)
+        float acc = 0.0f, ll = 0.0f;
+#pragma unroll
+        for (int ww = 0; ww < kWaves; ww++) {
+            const float f = fast_exp2(comb[ww * kCombStride + GP * D + h] - mm_ref);
+            acc += comb[ww * kCombStride + idx] * f;
+            ll += comb[ww * kCombStride + GP * D + GP + h] * f;
+        }
+        if (wk.nsplit == 1) {
+            if (h < g) out[idx] = __float2half_rn(ll > 0.0f ? acc / ll : 0.0f);
+        } else if (wk.counter == nullptr) {
+            p.part_o[slot * (GP * D) + idx] = acc;
+            if ((idx % D) == 0) {
+                p.part_ml[slot * (2 * GP) + h] = mm;
+                p.part_ml[slot * (2 * GP) + GP + h] = ll;
+            }
+        } else {   // write-through stores: visible device-wide when they complete (see tail_merge)
+            __hip_atomic_store(&p.part_o[slot * (GP * D) + idx], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((idx % D) == 0) {
+                __hip_atomic_store(&p.part_ml[slot * (2 * GP) + h], mm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&p.part_ml[slot * (2 * GP) + GP + h], ll, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+    if constexpr (GP <= 8) {   // (larger groups: the merge launch; the in-kernel merge would need too many registers)
+        if (wk.nsplit > kTailMergeMax && wk.counter != nullptr)
+            tail_merge_wide<__half, D, GP>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid, reinterpret_cast<float *>(lds_raw));
+        else if (wk.nsplit > 1 && wk.counter != nullptr)
+            tail_merge<__half, D, GP>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
+    }
+}
 
 // FMT: TROCM_F16, or a block-quantised cache (TROCM_Q8_0 / TROCM_Q4_0, 32-element blocks): the codes are
 // dequantised on the way into the LDS tile, (code - zero) * d rounded once to f16 as the reference's
@@ -413,44 +467,349 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
             cw[GP * D + GP + l32] = l_run;
         }
     }
+    wave_records_to_output<D, GP>(p, wk, lds_raw, head0, g, tid);
+}
+
+// Transposing 64-bit LDS load of 8-bit elements: in each block of 16 lanes, lane i receives byte i%8 of the eight
+// 8-byte rows addressed by lanes i/8, i/8 + 2, ..., i/8 + 14 of the block, in that order.
+__device__ __forceinline__ void lds_read_tr8(const unsigned char *lds_ptr, uint32_t &w0, uint32_t &w1) {
+    typedef int int2_t __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(3))) int2_t *lds_v2_ptr;
+    const int2_t r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2_ptr)(uintptr_t)(uint32_t)(uintptr_t)lds_ptr);
+    w0 = (uint32_t)r[0], w1 = (uint32_t)r[1];
+}
+// eight unsigned bytes as the eight halves 1024 + b (exact integers in f16)
+__device__ __forceinline__ half8_t magic8(uint32_t w0, uint32_t w1) {
+    u32x4 r;
+    r.x = perm(0x64646464u, w0, 0x04010400u), r.y = perm(0x64646464u, w0, 0x04030402u);
+    r.z = perm(0x64646464u, w1, 0x04010400u), r.w = perm(0x64646464u, w1, 0x04030402u);
+    return __builtin_bit_cast(half8_t, r);
+}
+
+// Block-quantised caches (Q8_0 / Q4_0, head_dim 128, up to 16 heads per kv head) without dequantising any element.
+// The contraction of v_mfma_f32_16x16x32_f16 is 32 features deep, exactly one quantisation block, so the raw codes go
+// into the matrix cores as the exact f16 integers 1024 + u (one v_perm per two codes puts the byte under the exponent
+// byte 0x64; Q4_0's high nibbles stay where they are, as 16 u, against query features divided by 16) and the block
+// scales are applied outside the products:
+//   scores:  S[t, h] = sum_blk d_k[t, blk] * (acc_blk[t, h] - bias[h, blk]);  the bias, (1024 + zero) * sum of the
+//            block's query features, is a constant of the lane's head and rides in as the accumulator's initial value;
+//   outputs: O[f, h] = sum_t (u_v[t, f] - zero) * (P[t, h] * d_v[t, blk(f)]): the scale is folded into the probabilities
+//            (one packed multiply per block and token pair), and the zero point is taken out once at the end through
+//            SP[h, blk] = sum_t P[t, h] * d_v[t, blk], accumulated beside the outputs.
+// The products are exact in f32 where the reference rounds every dequantised element to f16 first (q4_0.rs:82-95):
+// the two differ by at most half an f16 unit per element, inside the tolerance of the path.
+// Per wave and 32-token tile: code rows global -> registers (one tile ahead, non-temporal 128-bit loads) -> raw bytes in
+// a wave-private LDS tile (consecutive lanes write consecutive 16-byte slots) -> K fragments by 8-byte (Q4_0: 4-byte)
+// reads, V^T fragments by transposing byte reads; the f16 block scales of the tile (256 bytes per tensor) go through
+// LDS too.
+template <int GP, int FMT, int PF>
+__device__ __forceinline__ void decode_mfma_qblock_body(const DecodeDev &p, const MfmaWork &wk) {
+    static_assert(GP <= 16, "the 16-wide layout: at most 16 heads");
+    static_assert(FMT == TROCM_Q8_0 || FMT == TROCM_Q4_0, "block-quantised caches only");
+    constexpr int D = 128;
+    constexpr bool Q8 = FMT == TROCM_Q8_0;
+    constexpr int NB = D / 32;                 // blocks per token row
+    constexpr int RB = Q8 ? D : D / 2;         // code bytes per token row
+    constexpr int NLD = kTile * RB / 1024;     // 128-bit loads per lane, tile and tensor: 4 / 2
+    constexpr int CPR = RB / 16;               // 16-byte chunks per row: 8 / 4
+    constexpr int SROW = NB * 2;               // bytes of block scales per row
+    constexpr int kCodeBytes = kTile * RB;     // one tensor's tile in LDS
+    constexpr int kScaleBytes = kTile * SROW;
+    constexpr int kWaveBytes = 2 * kCodeBytes + 2 * kScaleBytes;
+    constexpr int kCombStride = GP * D + 2 * GP;
+    constexpr int kLdsBytes = kWaves * (kWaveBytes > kCombStride * 4 ? kWaveBytes : kCombStride * 4);
+    __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kLdsBytes];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l16 = lane & 15, q4 = lane >> 4;
+    const int kvh = wk.kvh, b = wk.seq;
+    const int g = p.g_real;
+    unsigned char *lds_k = lds_raw + w * kWaveBytes, *lds_v = lds_k + kCodeBytes;
+    unsigned char *lds_ks = lds_v + kCodeBytes, *lds_vs = lds_ks + kScaleBytes;
+
+    const int64_t head0 = (int64_t)b * p.Hq + (int64_t)kvh * g;
+    const _Float16 *qrow = reinterpret_cast<const _Float16 *>(p.q) + (head0 + min(l16, g - 1)) * D;
+    const int T = wk.T;
+    const int tile_begin = wk.tile_begin, tile_end = wk.tile_end;
+
+    // one tile ahead in registers: NLD chunks of 16 code bytes (chunk j*64 + lane of the tile, rows are dense) and,
+    // in lanes 0..31, the 8 bytes of block scales of token `lane`
+    // (PF tiles ahead: a wave's tile of Q4_0 codes is 2 KiB per tensor, and 2048 waves with one tile each in flight do
+    // not cover the memory latency at full bandwidth)
+    u32x4 kpre[PF][NLD], vpre[PF][NLD];
+    u32x2 kspre[PF], vspre[PF];
+    auto fetch = [&](const char *base0, const char *sbase0, int t, u32x4 (&dst)[NLD], u32x2 &sc) {
+        const int t0 = t * kTile;
+        const char *base = base0 + (int64_t)t0 * RB;
+        const char *sbase = sbase0 + (int64_t)t0 * SROW;
+        if (t0 + kTile <= T) {
+#pragma unroll
+            for (int j = 0; j < NLD; j++)
+                dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + (j * 64 + lane) * 16));
+            if (lane < kTile) sc = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(sbase + lane * SROW));
+        } else {   // rows past the end of the sequence repeat its last token (their scores are masked below)
+            const int last = T - 1 - t0;
+#pragma unroll
+            for (int j = 0; j < NLD; j++) {
+                const int c = j * 64 + lane, row = min(c / CPR, last), dc = c % CPR;
+                dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + row * RB + dc * 16));
+            }
+            if (lane < kTile) sc = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(sbase + min(lane, last) * SROW));
+        }
+    };
+    // Where this lane's chunks go in the LDS tiles.  The 16-byte chunks of a row are permuted (xor with a key of the row)
+    // so that the fragment reads below, which walk down the rows at a fixed place in the row, spread over the banks: the
+    // K tile is read 16 consecutive tokens at a time (key: the token's low bits), the V tile 4 + 4 tokens 16 apart (key:
+    // low bits and bit 4 of the token).  A row stays one contiguous 128- or 64-byte run, so the writes stay conflict-free.
+    auto key_k = [](int row) { return Q8 ? (row & 7) : ((row >> 1) & 3); };
+    auto key_v = [](int row) { return Q8 ? ((row & 3) | (((row >> 4) & 1) << 2)) : (((row >> 1) & 1) | (((row >> 4) & 1) << 1)); };
+    uint32_t k_slot[NLD], v_slot[NLD];
+#pragma unroll
+    for (int j = 0; j < NLD; j++) {
+        const int c = j * 64 + lane, row = c / CPR, dc = c % CPR;
+        k_slot[j] = row * RB + 16 * (dc ^ key_k(row));
+        v_slot[j] = row * RB + 16 * (dc ^ key_v(row));
+    }
+    const int tstep = wk.tile_step;
+    int t = tile_begin + w;
+#pragma unroll
+    for (int st = 0; st < PF; st++) {
+        kspre[st] = vspre[st] = u32x2{0u, 0u};
+        if (t + st * tstep < tile_end) {
+            fetch(wk.kbase, wk.ksbase, t + st * tstep, kpre[st], kspre[st]);
+            fetch(wk.vbase, wk.vsbase, t + st * tstep, vpre[st], vspre[st]);
+        }
+    }
+
+    // Q^T fragments of this lane's head, one per block: the 8 features that lane group q4 contributes.
+    //   Q8_0: features 32 blk + 8 q4 + 0..7
+    //   Q4_0: features 32 blk + 4 q4 + 0..3 (low nibbles) and 32 blk + 16 + 4 q4 + 0..3 (high nibbles: the codes arrive
+    //         as 16 u, so these features are divided by 16 -- exact but for subnormal results)
+    half8_t qf[NB];
+    float bias[NB];   // (1024 + zero) * (what the products add up for a block of all-zero-point codes), negated
+#pragma unroll
+    for (int blk = 0; blk < NB; blk++) {
+        float part;
+        if constexpr (Q8) {
+            qf[blk] = *reinterpret_cast<const half8_t *>(qrow + 32 * blk + 8 * q4);
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) sum += (float)qf[blk][i];
+            part = 1152.0f * sum;   // byte ^ 0x80 = code + 128 under 1024
+        } else {
+            const half4_t lo = *reinterpret_cast<const half4_t *>(qrow + 32 * blk + 4 * q4);
+            const half4_t hi = *reinterpret_cast<const half4_t *>(qrow + 32 * blk + 16 + 4 * q4);
+            float s_lo = 0.0f, s_hi = 0.0f, s_hi16 = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const _Float16 h16 = hi[i] * (_Float16)0.0625f;
+                qf[blk][i] = lo[i], qf[blk][4 + i] = h16;
+                s_lo += (float)lo[i], s_hi16 += (float)h16, s_hi += 16.0f * (float)h16;
+            }
+            part = 1024.0f * (s_lo + s_hi16) + 8.0f * (s_lo + s_hi);
+        }
+        part += __shfl_xor(part, 16, 64);
+        part += __shfl_xor(part, 32, 64);
+        bias[blk] = -part;
+    }
+#pragma unroll
+    for (int blk = 0; blk < NB; blk++) asm volatile("" : "+v"(qf[blk]));   // settled here, not at first use inside the loop
+
+    float m_run = -INFINITY, l_run = 0.0f;   // log2 domain, already scaled
+    float4_t o16[D / 16];
+    float sp[NB];
+#pragma unroll
+    for (int fb = 0; fb < D / 16; fb++) o16[fb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int blk = 0; blk < NB; blk++) sp[blk] = 0.0f;
+
+    // K fragment of this lane: token 16 mb + l16 (its key does not depend on mb), the bytes of block blk that lane group
+    // q4 contributes: Q8_0 chunk 2 blk + q4 / 2, half q4 % 2; Q4_0 chunk blk, word q4
+    uint32_t k_frag[NB];
+#pragma unroll
+    for (int blk = 0; blk < NB; blk++)
+        k_frag[blk] = Q8 ? l16 * RB + 16 * ((2 * blk + (q4 >> 1)) ^ key_k(l16)) + 8 * (q4 & 1) : l16 * RB + 16 * (blk ^ key_k(l16)) + 4 * q4;
+    // V^T fragments: this lane as a SOURCE of the transposing reads addresses token (4 q4 + k, or 16 + 4 q4 + k - 4: the
+    // order of the probabilities in the B fragment), bytes 8 (l16 % 2) .. + 8 of a 16-byte group; k = l16 / 2
+    const int vk = l16 >> 1, v_tok = vk < 4 ? 4 * q4 + vk : 12 + 4 * q4 + vk;
+    const unsigned char *v_row = lds_v + v_tok * RB + 8 * (l16 & 1);
+    const uint32_t v_key16 = 16 * key_v(v_tok);   // (16 c) ^ v_key16 = 16 (c ^ key)
+    // block scales of this lane's tokens 16 mb + 4 q4 + 0..3: 32 contiguous bytes per mb
+    const unsigned char *ks_frag = lds_ks + 4 * q4 * SROW, *vs_frag = lds_vs + 4 * q4 * SROW;
+    const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+
+    const float c_log2 = p.scale_log2;   // > 0 (checked on the host): the maximum is taken before scaling
+    // one tile, whose codes wait in stage ST of the prefetch registers
+    auto do_tile = [&](auto stage_tag, int t) {
+        constexpr int ST = decltype(stage_tag)::value;
+        const int t0 = t * kTile;
+        const bool more = t + PF * tstep < tile_end;
+        // ---- this tile's codes and scales -> LDS, the tile PF steps on into flight --------------------------------
+#pragma unroll
+        for (int j = 0; j < NLD; j++) {
+            *reinterpret_cast<u32x4 *>(lds_k + k_slot[j]) = kpre[ST][j];
+            *reinterpret_cast<u32x4 *>(lds_v + v_slot[j]) = vpre[ST][j];
+        }
+        if (lane < kTile) {
+            *reinterpret_cast<u32x2 *>(lds_ks + lane * SROW) = kspre[ST];
+            *reinterpret_cast<u32x2 *>(lds_vs + lane * SROW) = vspre[ST];
+        }
+        if (more) {
+            fetch(wk.kbase, wk.ksbase, t + PF * tstep, kpre[ST], kspre[ST]);
+            fetch(wk.vbase, wk.vsbase, t + PF * tstep, vpre[ST], vspre[ST]);
+        }
+        // ---- per block: codes x query features, the bias riding in the accumulator -------------------------------
+        float4_t acc[2][NB];
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+            for (int blk = 0; blk < NB; blk++) {
+                half8_t kf;
+                if constexpr (Q8) {
+                    const u32x2 c = *reinterpret_cast<const u32x2 *>(lds_k + k_frag[blk] + 16 * mb * RB);
+                    kf = magic8(c.x ^ 0x80808080u, c.y ^ 0x80808080u);
+                } else {
+                    const uint32_t c = *reinterpret_cast<const uint32_t *>(lds_k + k_frag[blk] + 16 * mb * RB);
+                    kf = magic8(c & 0x0F0F0F0Fu, c & 0xF0F0F0F0u);
+                }
+                const float4_t c0 = {bias[blk], bias[blk], bias[blk], bias[blk]};
+                acc[mb][blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[blk], c0, 0, 0, 0);
+            }
+        // ---- scores (before the softmax scale): the block scales of this lane's tokens 16 mb + 4 q4 + r ---------------
+        float sc8[8];
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++) {
+            const u32x4 d01 = *reinterpret_cast<const u32x4 *>(ks_frag + 16 * mb * SROW);        // tokens r = 0, 1: (d0 d1)(d2 d3) each
+            const u32x4 d23 = *reinterpret_cast<const u32x4 *>(ks_frag + 16 * mb * SROW + 16);   // tokens r = 2, 3
+            const uint32_t dw[4][2] = {{d01.x, d01.y}, {d01.z, d01.w}, {d23.x, d23.y}, {d23.z, d23.w}};
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const half2_t da = as_half2(dw[r][0]), db = as_half2(dw[r][1]);
+                float sv = __builtin_fmaf((float)da[0], acc[mb][0][r], 0.0f);
+                sv = __builtin_fmaf((float)da[1], acc[mb][1][r], sv);
+                sv = __builtin_fmaf((float)db[0], acc[mb][2][r], sv);
+                sv = __builtin_fmaf((float)db[1], acc[mb][3][r], sv);
+                sc8[4 * mb + r] = sv;
+            }
+        }
+        if (t0 + kTile > T) {   // the sequence's last tile: tokens past its end do not count
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (t0 + 16 * (i >> 2) + 4 * q4 + (i & 3) >= T) sc8[i] = -INFINITY;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) tmax = fmaxf(tmax, sc8[i]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m_run, tmax * c_log2);   // finite: every tile holds at least one valid token
+        float psum = 0.0f;
+        half2_t pf[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float p0 = fast_exp2(__builtin_fmaf(sc8[2 * i], c_log2, -m_new)), p1 = fast_exp2(__builtin_fmaf(sc8[2 * i + 1], c_log2, -m_new));
+            psum += p0 + p1;
+            pf[i] = half2_t{(_Float16)p0, (_Float16)p1};
+        }
+        const bool moved = m_new != m_run;
+        const float alpha = fast_exp2(m_run - m_new);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+            for (int fb = 0; fb < D / 16; fb++) o16[fb] *= alpha;
+#pragma unroll
+            for (int blk = 0; blk < NB; blk++) sp[blk] *= alpha;
+        }
+        // ---- probabilities times the V block scales of their tokens, per block -----------------------------------------
+        // pf[i] holds tokens (4 q4 + 2i, + 1) for i < 2 and (16 + 4 q4 + 2(i - 2), + 1) for i >= 2
+        half8_t pb[NB];
+        {
+            const u32x4 e0 = *reinterpret_cast<const u32x4 *>(vs_frag);                       // mb 0: tokens r = 0, 1
+            const u32x4 e1 = *reinterpret_cast<const u32x4 *>(vs_frag + 16);                  //       r = 2, 3
+            const u32x4 e2 = *reinterpret_cast<const u32x4 *>(vs_frag + 16 * SROW);           // mb 1: r = 0, 1
+            const u32x4 e3 = *reinterpret_cast<const u32x4 *>(vs_frag + 16 * SROW + 16);      //       r = 2, 3
+            const u32x4 ev[4] = {e0, e1, e2, e3};   // ev[i] = rows of the token pair of pf[i]: (x y) first token, (z w) second
+#pragma unroll
+            for (int blk = 0; blk < NB; blk++) {
+                u32x4 pw;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t first = (blk < 2) ? ev[i].x : ev[i].y, second = (blk < 2) ? ev[i].z : ev[i].w;
+                    const half2_t dd = as_half2(perm(second, first, (blk & 1) ? 0x07060302u : 0x05040100u));
+                    const half2_t pp = pf[i] * dd;
+                    sp[blk] = __builtin_amdgcn_fdot2(pp, ones, sp[blk], false);
+                    pw[i] = __builtin_bit_cast(uint32_t, pp);
+                }
+                pb[blk] = __builtin_bit_cast(half8_t, pw);
+            }
+        }
+        // ---- O^T += codes^T x scaled probabilities -----------------------------------------------------------------------
+#pragma unroll
+        for (int blk = 0; blk < NB; blk++) {
+            if constexpr (Q8) {
+#pragma unroll
+                for (int hf = 0; hf < 2; hf++) {
+                    uint32_t w0, w1;
+                    lds_read_tr8(v_row + ((32 * blk + 16 * hf) ^ v_key16), w0, w1);
+                    const half8_t vf = magic8(w0 ^ 0x80808080u, w1 ^ 0x80808080u);
+                    o16[2 * blk + hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pb[blk], o16[2 * blk + hf], 0, 0, 0);
+                }
+            } else {
+                uint32_t w0, w1;   // byte l16 of the block's 16: feature l16 in the low nibble, 16 + l16 in the high one
+                lds_read_tr8(v_row + ((16 * blk) ^ v_key16), w0, w1);
+                const half8_t vlo = magic8(w0 & 0x0F0F0F0Fu, w1 & 0x0F0F0F0Fu);
+                const half8_t vhi = magic8(w0 & 0xF0F0F0F0u, w1 & 0xF0F0F0F0u);
+                o16[2 * blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vlo, pb[blk], o16[2 * blk], 0, 0, 0);
+                o16[2 * blk + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vhi, pb[blk], o16[2 * blk + 1], 0, 0, 0);
+            }
+        }
+    };
+    static_assert(PF <= 4, "stages are written out");
+    while (t < tile_end) {
+        do_tile(std::integral_constant<int, 0>{}, t);
+        t += tstep;
+        if constexpr (PF > 1) {
+            if (t < tile_end) do_tile(std::integral_constant<int, 1>{}, t), t += tstep;
+        }
+        if constexpr (PF > 2) {
+            if (t < tile_end) do_tile(std::integral_constant<int, 2>{}, t), t += tstep;
+        }
+        if constexpr (PF > 3) {
+            if (t < tile_end) do_tile(std::integral_constant<int, 3>{}, t), t += tstep;
+        }
+    }
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    // the zero points: O[f, h] -= (1024 + zero) * SP[h, blk(f)] (Q4_0's high features arrived 16 times too large)
+#pragma unroll
+    for (int blk = 0; blk < NB; blk++) {
+        float s_all = sp[blk];
+        s_all += __shfl_xor(s_all, 16, 64);
+        s_all += __shfl_xor(s_all, 32, 64);
+        if constexpr (Q8) {
+            o16[2 * blk] -= 1152.0f * s_all;
+            o16[2 * blk + 1] -= 1152.0f * s_all;
+        } else {
+            o16[2 * blk] -= 1032.0f * s_all;
+            o16[2 * blk + 1] = o16[2 * blk + 1] * 0.0625f - 72.0f * s_all;
+        }
+    }
+
+    // ---- merge the 4 waves through LDS (the tiles are dead) ------------------------------------------------------------
     __syncthreads();
-    __half *out = reinterpret_cast<__half *>(p.out) + head0 * D;
-    const int64_t slot = wk.slot;
-    for (int idx = tid; idx < GP * D; idx += kThreads) {
-        const int h = idx / D;
-        float mm = -INFINITY;
+    float *comb = reinterpret_cast<float *>(lds_raw);   // [kWaves][GP*D + 2*GP]
+    if (l16 < GP) {
+        float *cw = comb + w * kCombStride;
 #pragma unroll
-        for (int ww = 0; ww < kWaves; ww++) mm = fmaxf(mm, comb[ww * kCombStride + GP * D + h]);
-        const float mm_ref = mm == -INFINITY ? 0.0f : mm;   // a wave without tiles holds (0, -inf, 0)
-        float acc = 0.0f, ll = 0.0f;
-#pragma unroll
-        for (int ww = 0; ww < kWaves; ww++) {
-            const float f = fast_exp2(comb[ww * kCombStride + GP * D + h] - mm_ref);
-            acc += comb[ww * kCombStride + idx] * f;
-            ll += comb[ww * kCombStride + GP * D + GP + h] * f;
-        }
-        if (wk.nsplit == 1) {
-            if (h < g) out[idx] = __float2half_rn(ll > 0.0f ? acc / ll : 0.0f);
-        } else if (wk.counter == nullptr) {
-            p.part_o[slot * (GP * D) + idx] = acc;
-            if ((idx % D) == 0) {
-                p.part_ml[slot * (2 * GP) + h] = mm;
-                p.part_ml[slot * (2 * GP) + GP + h] = ll;
-            }
-        } else {   // write-through stores: visible device-wide when they complete (see tail_merge)
-            __hip_atomic_store(&p.part_o[slot * (GP * D) + idx], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if ((idx % D) == 0) {
-                __hip_atomic_store(&p.part_ml[slot * (2 * GP) + h], mm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(&p.part_ml[slot * (2 * GP) + GP + h], ll, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
+        for (int fb = 0; fb < D / 16; fb++) *reinterpret_cast<float4_t *>(cw + l16 * D + 16 * fb + 4 * q4) = o16[fb];
+        if (q4 == 0) {
+            cw[GP * D + l16] = m_run;
+            cw[GP * D + GP + l16] = l_run;
         }
     }
-    if constexpr (GP <= 8) {   // (larger groups: the merge launch; the in-kernel merge would need too many registers)
-        if (wk.nsplit > kTailMergeMax && wk.counter != nullptr)
-            tail_merge_wide<__half, D, GP>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid, reinterpret_cast<float *>(lds_raw));
-        else if (wk.nsplit > 1 && wk.counter != nullptr)
-            tail_merge<__half, D, GP>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
-    }
+    wave_records_to_output<D, GP>(p, wk, lds_raw, head0, g, tid);
 }
 
 // The reference states a ragged batch as a dense batch padded to the longest sequence, with a mask row per
@@ -481,8 +840,9 @@ __device__ __forceinline__ int mask_row_len(const _Float16 *__restrict__ row, in
 }
 
 // Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.
-template <int D, int GP, int FMT, bool MASK = false, bool W16 = false>
-__global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev p) {
+// QB: quantised caches on the 16-wide tiles run the body that scales per block outside the products.
+template <int D, int GP, int FMT, bool MASK = false, bool W16 = false, int QB = 0>
+__global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma_kernel(DecodeDev p) {
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     MfmaWork wk;
     wk.seq = b, wk.kvh = kvh;
@@ -517,12 +877,15 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(DecodeDev
     wk.counter = p.counters ? p.counters + bh : nullptr;
     wk.part_first = bh * p.nsplit, wk.part_stride = 1;
     wk.mask = MASK ? p.mask + (int64_t)b * p.mask_stride_b + (int64_t)kvh * p.g_real * p.mask_stride_h : nullptr;
-    decode_mfma_body<D, GP, FMT, MASK, W16>(p, wk);
+    if constexpr (QB != 0)
+        decode_mfma_qblock_body<GP, FMT, QB / 10>(p, wk);
+    else
+        decode_mfma_body<D, GP, FMT, MASK, W16>(p, wk);
 }
 
 // Ragged batch: grid (work items, kv_heads); an item is a tile range of one sequence (the host's plan).
-template <int D, int GP, int FMT, bool W16 = false>
-__global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_ragged_kernel(DecodeDev p, const RaggedItem *__restrict__ items) {
+template <int D, int GP, int FMT, bool W16 = false, int QB = 0>
+__global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma_ragged_kernel(DecodeDev p, const RaggedItem *__restrict__ items) {
     const RaggedItem it = items[blockIdx.x];
     const int kvh = blockIdx.y;
     MfmaWork wk;
@@ -542,7 +905,10 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_ragged_kernel(De
     wk.counter = p.counters ? p.counters + (int64_t)it.seq * p.Hkv + kvh : nullptr;
     wk.part_first = (int64_t)it.slot0 * p.Hkv + kvh, wk.part_stride = p.Hkv;
     wk.mask = nullptr;
-    decode_mfma_body<D, GP, FMT, false, W16>(p, wk);
+    if constexpr (QB != 0)
+        decode_mfma_qblock_body<GP, FMT, QB / 10>(p, wk);
+    else
+        decode_mfma_body<D, GP, FMT, false, W16>(p, wk);
 }
 
 // Up to 16 heads per kv head: the 16-wide tiles (batch 8, 8226 tokens, f16: 49.3 -> 48.5 us; batch 1 15.4 -> 14.5 us;
@@ -554,12 +920,29 @@ bool use_16_wide(int fmt) {
     return mode == 2 || (mode == 1 && fmt != TROCM_F16);
 }
 
+// Quantised caches on the 16-wide tiles: block scales applied outside the products (decode_mfma_qblock_body) unless
+// TROCM_DECODE_QBLOCK=0 asks for the kernel that dequantises every element on the way into the LDS tile.
+bool use_block_scaling() {
+    static const int on = getenv("TROCM_DECODE_QBLOCK") ? atoi(getenv("TROCM_DECODE_QBLOCK")) : 1;
+    return on != 0;
+}
+
+// The block-scaling kernel keeps one tile (Q8_0) or two (Q4_0: half the bytes per tile) ahead in registers, two
+// workgroups per compute unit.  Measured at batch 8, 16384 tokens: a tile more ahead 52.1 -> 54.6 us (Q8_0) and 37.7 ->
+// 39.2 us (Q4_0); three workgroups per compute unit (Q4_0, 162 registers) 39.2 us.
+template <int GP, int FMT>
+void launch_qblock(const DecodeDev &p, dim3 grid, hipStream_t s) {
+    hipLaunchKernelGGL((sdpa_decode_mfma_kernel<128, GP, FMT, false, true, (FMT == TROCM_Q8_0 ? 12 : 22)>), grid, dim3(kThreads), 0, s, p);
+}
+
 template <int D, int GP, int FMT = TROCM_F16>
 int launch_gp(const DecodeDev &p, dim3 grid, hipStream_t s) {
     if (FMT == TROCM_F16 && p.mask && GP <= 16 && use_16_wide(FMT))
         hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, (GP <= 16 ? GP : 16), TROCM_F16, true, true>), grid, dim3(kThreads), 0, s, p);
     else if (FMT == TROCM_F16 && p.mask)
         hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, GP, TROCM_F16, true>), grid, dim3(kThreads), 0, s, p);
+    else if (FMT != TROCM_F16 && D == 128 && GP <= 16 && use_16_wide(FMT) && use_block_scaling() && p.scale_log2 > 0.0f)
+        launch_qblock<(GP <= 16 ? GP : 16), (FMT != TROCM_F16 ? FMT : TROCM_Q8_0)>(p, grid, s);
     else if (GP <= 16 && use_16_wide(FMT))
         hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, (GP <= 16 ? GP : 16), FMT, false, true>), grid, dim3(kThreads), 0, s, p);
     else
@@ -592,7 +975,9 @@ int launch_quant(const DecodeDev &p, int gp, dim3 grid, hipStream_t s) {
 template <int D, int GP, int FMT = TROCM_F16>
 int launch_ragged_gp(const DecodeDev &p, const RaggedItem *items, int n_items, const RaggedSeqSlots *seqs, int n_seq,
                      bool any_split, hipStream_t s) {
-    if (GP <= 16 && use_16_wide(FMT))
+    if (FMT != TROCM_F16 && D == 128 && GP <= 16 && use_16_wide(FMT) && use_block_scaling() && p.scale_log2 > 0.0f)
+        hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<128, (GP <= 16 ? GP : 16), (FMT != TROCM_F16 ? FMT : TROCM_Q8_0), true, (FMT == TROCM_Q4_0 ? 22 : 12)>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+    else if (GP <= 16 && use_16_wide(FMT))
         hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<D, (GP <= 16 ? GP : 16), FMT, true>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
     else
         hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<D, GP, FMT>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
