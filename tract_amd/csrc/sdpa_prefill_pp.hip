@@ -74,6 +74,7 @@ __device__ __forceinline__ half4_t lds_read_tr16(const _Float16 *lds_ptr) {
 }
 
 constexpr int kWavesPP = 8, kThreadsPP = 64 * kWavesPP, kTileN = 64;
+constexpr float kLazyMax = 8.0f;
 
 __device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
@@ -295,7 +296,12 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
 #pragma unroll
             for (int r = 0; r < 16; r++) tmax = fmaxf(tmax, s[kb][r]);
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float m_new = fmaxf(m_run, MASK ? tmax : tmax * p.scale_log2);  // scale > 0: the maximum commutes with the scaling
+        // The reference of the exponentials follows the maximum lazily: it moves only when this tile's maximum exceeds it
+        // by more than kLazyMax (the exponentials then reach 2^kLazyMax at most, far inside f16 and f32 range), so the
+        // accumulators are rescaled a few times per sequence instead of at most tiles; o / l does not depend on it.
+        const float t_scaled = MASK ? tmax : tmax * p.scale_log2;   // scale > 0: the maximum commutes with the scaling
+        const bool moved = t_scaled > m_run + kLazyMax;   // also the first visible key (reference -inf); never for a maximum of -inf
+        const float m_new = moved ? t_scaled : m_run;
         const float m_ref = (m_new == -INFINITY) ? 0.0f : m_new;  // nothing visible yet: keep everything at zero
         float psum = 0.0f;
 #pragma unroll
@@ -315,8 +321,7 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
                 psum = __builtin_amdgcn_fdot2(pair, ones, psum, false);
             }
         }
-        const bool moved = m_new != m_run;
-        const float alpha = fast_exp2(m_run - m_ref);
+        const float alpha = moved ? fast_exp2(m_run - m_ref) : 1.0f;   // 0 from a reference of -inf
         l_run = l_run * alpha + psum;
         m_run = m_new;
         if (__builtin_amdgcn_ballot_w64(moved) != 0) {
