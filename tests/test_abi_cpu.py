@@ -29,6 +29,30 @@ def test_library_exports_every_declared_symbol():
     assert exported == set(names)
 
 
+def test_rust_binding_matches_header():
+    """The Rust `extern "C"` block a maintainer pastes into rocm/src/ffi.rs declares every entry point of the
+    header with the same arguments: the copy in INTEGRATION.md is the generator's output for today's header."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("gen_rust_ffi", os.path.join(ROOT, "include", "gen_rust_ffi.py"))
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    header = open(os.path.join(ROOT, "include", "tract_rocm.h")).read()
+    decls = gen.declarations(header)
+    assert [d[0] for d in decls] == sorted(set(d[0] for d in decls), key=[d[0] for d in decls].index)   # no duplicates
+    assert sorted(d[0] for d in decls) == _header_symbols()
+    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    block = re.search(r'extern "C" \{\n.*?\n\}', doc, flags=re.S).group(0)
+    assert block == gen.rust_block(header)
+    # argument counts, independently of the generator's type mapping
+    doc_fns = dict((m.group(1), m.group(2)) for m in re.finditer(r"pub fn (trocm_[a-z0-9_]+)\((.*?)\) ->", block))
+    for name, _ret, params in decls:
+        n_doc = 0 if not doc_fns[name].strip() else doc_fns[name].count(":")
+        assert n_doc == len(params), name
+    # every opaque handle the block mentions is declared beside it
+    for opaque in set(re.findall(r"\b(trocm_[a-z0-9_]+)\b(?!\()", block)) - set(doc_fns):
+        assert f"pub struct {opaque}" in doc, opaque
+
+
 def test_header_is_plain_c():
     src = '#include "tract_rocm.h"\nint main(void){return (int)sizeof(trocm_dtype) == 0;}\n'
     subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"), "-x", "c", "-",
