@@ -195,6 +195,12 @@ int trocm_block_quant(int format, const void *src, int src_dtype, size_t n_elems
                       void *stream);
 int trocm_block_dequant(int format, const void *src_blocks, size_t n_elems, void *dst, int dst_dtype,
                         void *stream);
+/* BlockQuant::simulate_precision_loss (linalg/src/frame/block_quant/mod.rs:130-154; the matmul tests build
+ * their expected values with it, test-rt/suite-unit/src/matmul_q40.rs:119-126): `n_elems` (multiple of 32)
+ * contiguous elements of `dtype` (F32 / F16), blocked along the innermost axis, are quantised and dequantised
+ * back into `dst` in one pass; `dst` may be `src`. */
+int trocm_block_simulate_precision_loss(int format, const void *src, void *dst, int dtype, size_t n_elems,
+                                        void *stream);
 
 /* ---- Q4_0 weights x a few activation rows: the decode-time projections ------------------------
  *

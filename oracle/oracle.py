@@ -58,6 +58,7 @@ def lib() -> C.CDLL:
         L.orc_quant.argtypes = [i, i, vp, sz, vp]
         L.orc_dequant.argtypes = [i, i, vp, sz, vp]
         L.orc_q4_0_matvec.argtypes = [vp, sz, sz, sz, vp, i, sz, sz, vp]
+        L.orc_streamed_sdpa_f32.argtypes = [vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, i, i, f, sz, vp]
         L.orc_kv_new.restype = vp
         L.orc_kv_new.argtypes = [sz, sz]
         L.orc_kv_free.argtypes = [vp]
@@ -124,6 +125,12 @@ def dequant(fmt: int, q: np.ndarray, dtype=np.float32) -> np.ndarray:
     rc = lib().orc_dequant(fmt, int(dtype == np.float16), _p(q), out.size, _p(out))
     assert rc == 0
     return out
+
+
+def simulate_precision_loss(fmt: int, x: np.ndarray) -> np.ndarray:
+    """BlockQuant::simulate_precision_loss (block_quant/mod.rs:130-154): every block of 32 along the last axis is
+    quantised and dequantised in the tensor's own type."""
+    return dequant(fmt, quant(fmt, x), dtype=x.dtype).reshape(x.shape)
 
 
 def q4_0_matvec(blocks: np.ndarray, act: np.ndarray) -> np.ndarray:
@@ -232,6 +239,28 @@ def flash_sdpa(q, k, v, mask=None, causal=False, scale=None, threads=1):
         out = np.empty(q.shape, dtype=np.float32)
         lib().orc_flash_sdpa_f32(_p(qq), _p(kk), _p(vv), _p(mm), B, Hq, Hkv, Sq, Sk, D,
                                  Hkv * Sk * D, Sk * D, D, mb, mh, int(causal), hs, sc, _p(out), threads)
+    return out[:, 0] if r3 else out
+
+
+def streamed_sdpa(q, k, v, mask=None, causal=False, scale=None, block_k=64):
+    """StreamedSdpaOp::eval (streamed_sdpa.rs:95-160): f32 or f16 inputs of rank 3 or 4, optional rank-2 mask
+    [q_len, kv_len]; computed in f32, returned in Q's type and shape."""
+    dt = q.dtype
+    r3 = q.ndim == 3
+    q4, k4, v4 = ((a[:, None] if r3 else a) for a in (q, k, v))
+    qq, kk, vv = (np.ascontiguousarray(a, dtype=np.float32) for a in (q4, k4, v4))
+    B, Hq, Sq, D = qq.shape
+    _, Hkv, Sk, _ = kk.shape
+    mm = None
+    if mask is not None:
+        assert mask.shape == (Sq, Sk)
+        mm = np.ascontiguousarray(mask, dtype=np.float32)
+    out = np.empty(qq.shape, dtype=np.float32)
+    hs, sc = (0, 0.0) if scale is None else (1, float(scale))
+    rc = lib().orc_streamed_sdpa_f32(_p(qq), _p(kk), _p(vv), _p(mm), B, Hq, Hkv, Sq, Sk, D, int(causal), hs, sc,
+                                     int(block_k), _p(out))
+    assert rc == 0
+    out = out.astype(dt)
     return out[:, 0] if r3 else out
 
 

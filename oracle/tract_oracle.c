@@ -34,6 +34,9 @@
  *                          concatenate form, the rotation closed forms (norm of each
  *                          pair kept, angles add); f16 arithmetic is the `half` crate's
  *                          (operate in f32, round to f16 after every operation)
+ *   StreamedSdpaOp          pinned (tolerance): f64 brute force with its own mask rules (top-left causal,
+ *                          rank-2 mask that overrides the causal flag), independence of block_k, rows that
+ *                          see nothing are zero; equals the flash path where their rules coincide
  *   Q4_0 matrix-vector      pinned (tolerance): == numpy's product with the (pinned) dequantised
  *                          weights in f64, a hand-built block whose dot product is known in
  *                          closed form, linearity in the activations; exact f32 bits unpinned
@@ -822,4 +825,72 @@ ORC_API void orc_win_valid(const orc_win *c, void *dstv) {
     unsigned char *dst = (unsigned char *)dstv;
     for (size_t o = 0; o < c->outer; o++)
         memcpy(dst + o * c->len * c->row_bytes, c->buf + o * c->window * c->row_bytes, c->len * c->row_bytes);
+}
+
+/* ------------------------------------------------------------------------- */
+/* StreamedSdpaOp                                                               */
+/* ------------------------------------------------------------------------- */
+
+/* StreamedSdpaOp::flash_attention_gqa (transformers/src/ops/streamed_sdpa.rs:164-272): one query row at a
+ * time over key blocks of `block_k`, f32 throughout (eval casts f16 inputs to f32 and the result back,
+ * :112-160).  mask: optional [q_len, kv_len] shared by every batch and head (:143-152); with a mask the
+ * causal flag is not consulted (:216-222); causal hides key i_k > t_q, counted from the first key whatever
+ * kv_len is (:218).  A block whose largest score is not finite is skipped whole (:231-234), a score that is
+ * not finite contributes nothing (:247-249), a row that saw nothing is zero (:263). */
+ORC_API int orc_streamed_sdpa_f32(const float *q, const float *k, const float *v, const float *mask, size_t B, size_t Hq,
+                          size_t Hkv, size_t Sq, size_t Sk, size_t D, int causal, int has_scale, float scale_in,
+                          size_t block_k, float *out) {
+    if (Hkv == 0 || Hq % Hkv) return 1;
+    const float scale = has_scale ? scale_in : sqrtf(1.0f / (float)D); /* :183: recip().sqrt() */
+    if (block_k < 1) block_k = 1;                                       /* :184 */
+    const size_t group = Hq / Hkv;
+    float *acc = (float *)malloc(D * sizeof(float));
+    float *scores = (float *)malloc(block_k * sizeof(float));
+    for (size_t b = 0; b < B; b++)
+        for (size_t kh = 0; kh < Hkv; kh++) {
+            const float *kbh = k + (b * Hkv + kh) * Sk * D, *vbh = v + (b * Hkv + kh) * Sk * D;
+            for (size_t g = 0; g < group; g++) {
+                const size_t qh = kh * group + g; /* :195 */
+                for (size_t tq = 0; tq < Sq; tq++) {
+                    const float *qv = q + ((b * Hq + qh) * Sq + tq) * D;
+                    float m = -INFINITY, l = 0.0f; /* :203-205 */
+                    for (size_t e = 0; e < D; e++) acc[e] = 0.0f;
+                    for (size_t kb = 0; kb < Sk; kb += block_k) {
+                        const size_t kend = kb + block_k < Sk ? kb + block_k : Sk;
+                        float block_max = -INFINITY;
+                        for (size_t ik = kb; ik < kend; ik++) {
+                            const float mk = mask ? mask[tq * Sk + ik] : (causal && ik > tq) ? -INFINITY : 0.0f;
+                            float dot = 0.0f; /* dot1d :275-282: serial f32 sum */
+                            for (size_t e = 0; e < D; e++) dot += qv[e] * kbh[ik * D + e];
+                            const float s = dot * scale + mk; /* :223 */
+                            if (s > block_max) block_max = s;
+                            scores[ik - kb] = s;
+                        }
+                        if (!isfinite(block_max)) continue; /* :231-234 */
+                        const float new_m = m > block_max ? m : block_max;
+                        const float alpha = isfinite(m) ? expf(m - new_m) : 0.0f; /* :237 */
+                        if (alpha != 1.0f) {
+                            for (size_t e = 0; e < D; e++) acc[e] *= alpha;
+                            l *= alpha;
+                        }
+                        float block_l = 0.0f;
+                        for (size_t ik = kb; ik < kend; ik++) {
+                            const float s = scores[ik - kb];
+                            if (!isfinite(s)) continue; /* :247-249 */
+                            const float w = expf(s - new_m);
+                            block_l += w;
+                            for (size_t e = 0; e < D; e++) acc[e] += w * vbh[ik * D + e];
+                        }
+                        l += block_l;
+                        m = new_m;
+                    }
+                    const float inv_l = l > 0.0f ? 1.0f / l : 0.0f; /* :263 */
+                    float *o = out + ((b * Hq + qh) * Sq + tq) * D;
+                    for (size_t e = 0; e < D; e++) o[e] = acc[e] * inv_l;
+                }
+            }
+        }
+    free(acc);
+    free(scores);
+    return 0;
 }

@@ -48,6 +48,32 @@ def test_block_quant_op_bit_exact(rt, dt, dev_fmt, orc_fmt, bq):
 
 @pytest.mark.parametrize("dt", [np.float32, np.float16])
 @pytest.mark.parametrize("dev_fmt,orc_fmt,bq", FMTS)
+def test_simulate_precision_loss_bit_exact(rt, dt, dev_fmt, orc_fmt, bq):
+    """BlockQuant::simulate_precision_loss (block_quant/mod.rs:130-154): one pass on the device gives the bits of
+    quantising and dequantising in the tensor's own type, on a rank-3 tensor blocked along its last axis."""
+    rng = np.random.default_rng(12)
+    with np.errstate(over="ignore", invalid="ignore"):
+        x = _nasty(rng, 6 * 50 * 4, dt).reshape(6, 50, 128)
+        got = bq.simulate_precision_loss(x, 2)
+        want = orc.simulate_precision_loss(orc_fmt, x)
+    assert got.shape == x.shape and got.dtype == x.dtype
+    u = np.uint16 if dt == np.float16 else np.uint32
+    ok = (got.view(u) == want.view(u)) | (np.isnan(got) & np.isnan(want))
+    assert ok.all(), np.argwhere(~ok)[:5]
+    # the reference's own round trips (q4_0.rs:505-535): small integers survive Q4_0 exactly
+    if dev_fmt == tract_amd.Q4_0:
+        for head in ([1, 2, 3, 4], [-1, -2, -3, -4], [1234], [-1234]):
+            y = np.zeros((1, 32), dtype=dt)
+            y[0, : len(head)] = head
+            assert np.array_equal(bq.simulate_precision_loss(y, 1), y)
+    with pytest.raises(tract_amd.TractRocmError):
+        bq.simulate_precision_loss(x, 1)                      # blocks run along the last axis only
+    with pytest.raises(tract_amd.TractRocmError):
+        bq.simulate_precision_loss(x[:, :, :48], 2)           # 48 is not a multiple of the block length
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+@pytest.mark.parametrize("dev_fmt,orc_fmt,bq", FMTS)
 def test_quantised_cache_append_bit_exact(rt, dt, dev_fmt, orc_fmt, bq):
     """cfg4 shape (reduced): GQA [B,8,T,128], 1% outlier channels x20, appended in chunks
     with growth; export must equal quant(concat(chunks))."""

@@ -62,6 +62,42 @@ def test_generic_shapes(rt, dt, B, Hq, Hkv, Sq, Sk, D, causal):
     assert max_abs(got, cases.textbook_sdpa(q, k, v, causal=causal)) <= TOL[np.dtype(dt)]
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+@pytest.mark.parametrize("shape_q,shape_kv,causal,with_mask,scale", [
+    ((2, 4, 9, 16), (2, 2, 9, 16), True, False, None),           # generic kernel shapes
+    ((1, 6, 5, 8), (1, 2, 23, 8), True, False, 0.7),             # kv_len > q_len: diagonal from the FIRST key
+    ((1, 2, 17, 8), (1, 1, 6, 8), True, False, None),            # kv_len < q_len: the rule goes in as a mask
+    ((1, 4, 6, 16), (1, 2, 11, 16), True, True, None),           # a mask overrides the causal flag
+    ((1, 32, 256, 128), (1, 8, 256, 128), True, False, None),    # MFMA prefill, square causal
+    ((1, 32, 128, 128), (1, 8, 640, 128), True, False, None),    # MFMA prefill over the first 128 of 640 keys
+    ((2, 32, 1, 128), (2, 8, 1500, 128), False, True, None),     # split-K decode with a rank-2 mask row
+    ((2, 40, 64), (2, 100, 64), False, False, None),             # rank 3
+])
+def test_streamed_sdpa_op(rt, dt, shape_q, shape_kv, causal, with_mask, scale):
+    """StreamedSdpaOp (streamed_sdpa.rs:95-272) against the oracle's restatement of its row-streaming loop."""
+    rng = np.random.default_rng(len(shape_q) * 100 + shape_q[-2] + shape_kv[-2])
+    q = (rng.standard_normal(shape_q) / 3).astype(dt)
+    k, v = (rng.standard_normal(shape_kv).astype(dt) for _ in range(2))
+    Sq, Sk = shape_q[-2], shape_kv[-2]
+    mask = None
+    if with_mask:
+        mask = rng.standard_normal((Sq, Sk)).astype(np.float32)   # any float type: the op casts it (:143-152)
+        mask[rng.random((Sq, Sk)) < 0.3] = -np.inf
+        mask[:, 0] = 0.0
+        mask[Sq // 2, :] = -np.inf                                 # a row that sees nothing: zeros
+        mask[0, 0] = 0.0 if Sq > 1 else -np.inf
+    op = tract_amd.StreamedSdpaOp(causal=causal, block_k=32, scale=scale)
+    assert op.output_facts(shape_q, shape_kv, shape_kv, None if mask is None else mask.shape) == tuple(shape_q)
+    got = op.eval(q, k, v, mask).to_numpy()
+    want = orc.streamed_sdpa(q, k, v, mask=mask, causal=causal, scale=scale, block_k=32)
+    assert got.shape == want.shape and got.dtype == np.dtype(dt)
+    assert max_abs(got, want) <= TOL[np.dtype(dt)]
+    if with_mask:
+        assert not got[..., Sq // 2, :].any()
+    with pytest.raises(tract_amd.TractRocmError):
+        op.output_facts(shape_q, shape_kv, shape_kv, (1, Sq, Sk))   # the mask is of rank 2 (:58-60)
+
+
 def test_padding_mask_equals_shorter_sequence(rt):
     rng = np.random.default_rng(8)
     B, Hq, Hkv, Sq, Sk, D = 2, 4, 2, 3, 80, 16

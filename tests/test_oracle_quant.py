@@ -53,6 +53,33 @@ def test_q4_0_reference_round_trips(dt, head):
     assert np.array_equal(_cycle(orc.FMT_Q4_0, x), x)
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+@pytest.mark.parametrize("fmt", [orc.FMT_Q4_0, orc.FMT_Q8_0])
+def test_simulate_precision_loss_is_quant_then_dequant_in_the_tensors_type(fmt, dt):
+    # block_quant/mod.rs:130-154; the reference's matmul tests build their expected values with it
+    # (test-rt/suite-unit/src/matmul_q40.rs:119-126).  Checked here against the round trip spelled out per block
+    # with the formulas of q4_0.rs:27-45,82-95 and q8_1.rs:36-63 in numpy.
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((3, 7, 64)) * 4).astype(dt)
+    got = orc.simulate_precision_loss(fmt, x)
+    assert got.shape == x.shape and got.dtype == x.dtype
+    xb = x.astype(np.float32).reshape(-1, 32)
+    first_max = np.abs(xb).argmax(axis=1)                                  # first index of the largest magnitude
+    mx = xb[np.arange(len(xb)), first_max]
+    if fmt == orc.FMT_Q4_0:
+        d = (mx / np.float32(-8)).astype(np.float32)
+        r = np.where(d == 0, np.float32(0), np.float32(1) / d).astype(np.float32)
+        codes = np.minimum((xb * r[:, None] + np.float32(8.5)).astype(np.float32).astype(np.int8), 15).astype(np.float32) - 8
+    else:
+        d = (mx / np.float32(127)).astype(np.float32)
+        r = np.where(d == 0, np.float32(0), np.float32(1) / d).astype(np.float32)
+        t = (xb * r[:, None]).astype(np.float32)
+        codes = np.trunc(t + np.copysign(np.float32(0.5), t)).astype(np.float32)   # f32::round: half away from zero
+    d16 = d.astype(np.float16).astype(np.float32)
+    want = (codes * d16[:, None]).astype(np.float32).astype(dt).reshape(x.shape)
+    assert np.array_equal(got, want)
+
+
 def test_q4_0_ramp_extracts_exactly():
     # q4_0.rs:589-593: ((i % 14) - 6) survives quant/dequant after .round()
     x = np.array([(i % 14) - 6 for i in range(64)], dtype=np.float32)

@@ -135,3 +135,62 @@ def test_invariants():
     vb = np.full((B, Hkv, cap, D), np.nan, dtype=np.float32)
     kb[:, :, :Sk], vb[:, :, :Sk] = k, v
     assert np.array_equal(orc.flash_sdpa_view(qs, kb, vb, Sk), a)
+
+
+# ------------------------------------------------------------------ StreamedSdpaOp (streamed_sdpa.rs:164-272)
+def _streamed_f64(q, k, v, mask, causal, scale):
+    """The operator's definition, vectorised in f64: its own mask rules and a row that sees nothing is zero."""
+    q, k, v = (np.asarray(a, dtype=np.float64) for a in (q, k, v))
+    B, Hq, Sq, D = q.shape
+    Hkv, Sk = k.shape[1], k.shape[2]
+    g = Hq // Hkv
+    sc = (1.0 / D) ** 0.5 if scale is None else scale
+    s = np.einsum("bhqd,bhkd->bhqk", q, np.repeat(k, g, axis=1)) * sc
+    if mask is not None:
+        s = s + np.asarray(mask, dtype=np.float64)[None, None]
+    elif causal:
+        s = np.where(np.arange(Sk)[None, :] > np.arange(Sq)[:, None], -np.inf, s)
+    mx = s.max(axis=-1, keepdims=True)
+    with np.errstate(invalid="ignore"):
+        p = np.where(np.isfinite(s), np.exp(s - np.where(np.isfinite(mx), mx, 0.0)), 0.0)
+    l = p.sum(axis=-1, keepdims=True)
+    p = np.where(l > 0, p / np.where(l > 0, l, 1.0), 0.0)
+    return np.einsum("bhqk,bhkd->bhqd", p, np.repeat(v, g, axis=1))
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,with_mask,scale", [
+    (2, 4, 2, 9, 9, 16, True, False, None),      # square causal
+    (1, 6, 2, 5, 23, 8, True, False, 0.7),       # kv_len > q_len: the diagonal starts at the FIRST key
+    (1, 2, 1, 17, 6, 8, True, False, None),      # kv_len < q_len: late queries see every key
+    (2, 3, 3, 7, 13, 32, False, False, None),
+    (1, 4, 2, 6, 11, 16, True, True, None),      # a mask overrides the causal flag
+    (1, 2, 2, 1, 40, 64, False, True, 1.1),
+])
+def test_streamed_sdpa_vs_f64_definition(B, Hq, Hkv, Sq, Sk, D, causal, with_mask, scale):
+    rng = np.random.default_rng(B * 1000 + Sq * 10 + Sk)
+    q, k, v = (rng.standard_normal(sh).astype(np.float32) for sh in ((B, Hq, Sq, D), (B, Hkv, Sk, D), (B, Hkv, Sk, D)))
+    mask = None
+    if with_mask:
+        mask = rng.standard_normal((Sq, Sk)).astype(np.float32)
+        mask[rng.random((Sq, Sk)) < 0.3] = -np.inf
+        mask[Sq // 2, :] = -np.inf               # a row that sees nothing
+    want = _streamed_f64(q, k, v, mask, causal, scale)
+    for bk in (1, 5, 64, 1000):                  # block_k changes the order of the sums only
+        got = orc.streamed_sdpa(q, k, v, mask=mask, causal=causal, scale=scale, block_k=bk)
+        assert got.shape == q.shape and got.dtype == np.float32
+        assert np.abs(got - want).max() < 2e-6, bk
+    if with_mask:
+        assert not got[:, :, Sq // 2].any()
+    if causal and not with_mask and Sk > Sq:     # keys past the q_len-th are invisible to every query
+        trunc = orc.streamed_sdpa(q, k[:, :, :Sq], v[:, :, :Sq], causal=True, scale=scale)
+        assert np.abs(got - trunc).max() < 1e-6
+    if causal and not with_mask and Sk == Sq:    # where the two operators' rules coincide, so do they
+        assert np.abs(got - orc.flash_sdpa(q, k, v, causal=True, scale=scale)).max() < 2e-6
+
+
+def test_streamed_sdpa_rank3_f16_and_first_key_only():
+    rng = np.random.default_rng(3)
+    q, k, v = (rng.standard_normal(sh).astype(np.float16) for sh in ((2, 1, 32), (2, 9, 32), (2, 9, 32)))
+    got = orc.streamed_sdpa(q, k, v, causal=True)
+    assert got.shape == q.shape and got.dtype == np.float16
+    assert np.array_equal(got[:, 0], v[:, 0])    # one query, causal: it sees key 0 alone (streamed_sdpa.rs:218)

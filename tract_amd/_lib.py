@@ -67,6 +67,7 @@ SIGNATURES = {
     "trocm_q8_0_to_q8_1": [_vp, _vp, _sz],
     "trocm_block_quant": [_i, _vp, _i, _sz, _vp, _vp],
     "trocm_block_dequant": [_i, _vp, _sz, _vp, _i, _vp],
+    "trocm_block_simulate_precision_loss": [_i, _vp, _vp, _i, _sz, _vp],
     "trocm_q4_0_weights_create": [C.POINTER(_vp), _vp, _i64, _i64, _i64, _vp],
     "trocm_q4_0_weights_destroy": [_vp],
     "trocm_q4_0_weights_shape": [_vp, _pi64, _pi64, _pi64],

@@ -973,6 +973,18 @@ int trocm_block_dequant(int format, const void *src_blocks, size_t n_elems, void
     return launch_block_dequant(format, src_blocks, n_elems, dst, dst_dtype, s);
 }
 
+int trocm_block_simulate_precision_loss(int format, const void *src, void *dst, int dtype, size_t n_elems, void *stream) {
+    TROCM_REQUIRE(format == TROCM_Q8_0 || format == TROCM_Q4_0, "simulate_precision_loss: format must be Q8_0 or Q4_0");
+    TROCM_REQUIRE(dtype == TROCM_F32 || dtype == TROCM_F16, "simulate_precision_loss: dtype must be F32 or F16");
+    TROCM_REQUIRE(n_elems % 32 == 0, "simulate_precision_loss: %zu elements is not a multiple of the block length 32", n_elems);
+    if (n_elems == 0) return 0;
+    TROCM_NOT_NULL(src);
+    TROCM_NOT_NULL(dst);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    return launch_block_simulate(format, src, dst, dtype, n_elems, s);
+}
+
 // ---- element-wise neighbours: cast, RotateHalf, ApplyRope ---------------------------------------
 int trocm_cast(const void *src, int src_dtype, void *dst, int dst_dtype, size_t n_elems, void *stream) {
     TROCM_REQUIRE((src_dtype == TROCM_F32 || src_dtype == TROCM_F16) && (dst_dtype == TROCM_F32 || dst_dtype == TROCM_F16),

@@ -106,6 +106,8 @@ int launch_quant_import(int fmt, int64_t B, int64_t H, int64_t n, int64_t pitch,
 // Dequantise canonical blocks to a dense f32/f16 tensor.
 int launch_block_quant(int fmt, const void *src, int src_dtype, size_t n_elems, void *dst, hipStream_t s);
 int launch_block_dequant(int fmt, const void *blocks, size_t n_elems, void *dst, int dst_dtype, hipStream_t s);
+// Quantise and dequantise in one pass (dst may be src): BlockQuant::simulate_precision_loss.
+int launch_block_simulate(int fmt, const void *src, void *dst, int dtype, size_t n_elems, hipStream_t s);
 
 // Element-wise neighbours of the cache: cast f32 <-> f16, RotateHalf, ApplyRope (rank <= 4, element
 // strides, NULL = dense; cos/sin strides are 0 on broadcast axes).

@@ -294,6 +294,35 @@ __global__ __launch_bounds__(256) void block_dequant_kernel(int fmt, const uint8
     }
 }
 
+// BlockQuant::simulate_precision_loss (block_quant/mod.rs:130-154): every block of 32 goes through the quantiser and
+// straight back through the dequantiser of the tensor's own type; no block bytes are written.  In place when dst == src
+// (a thread has read its whole block before it stores).
+template <typename T>
+__global__ __launch_bounds__(256) void block_simulate_kernel(int fmt, const T *__restrict__ src, int64_t n_blocks, bool vec,
+                                                             T *__restrict__ dst) {
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n_blocks;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        float v[32];
+        load_block(src + idx * 32, 1, vec, v);
+        T *o = dst + idx * 32;
+        if (fmt == TROCM_Q8_0) {
+            uint32_t c[8];
+            const float d = __half2float(__ushort_as_half(quant_q8(v, c)));
+#pragma unroll
+            for (int i = 0; i < 32; i++) store_out(o + i, __fmul_rn((float)(int8_t)((c[i >> 2] >> (8 * (i & 3))) & 0xff), d));
+        } else {
+            uint32_t c[4];
+            const float d = __half2float(__ushort_as_half(quant_q4(v, c)));
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                const int byte = (c[j >> 2] >> (8 * (j & 3))) & 0xff;
+                store_out(o + j, __fmul_rn((float)((byte & 0xf) - 8), d));
+                store_out(o + j + 16, __fmul_rn((float)((byte >> 4) - 8), d));
+            }
+        }
+    }
+}
+
 int grid_for(int64_t n) {
     int64_t blocks = (n + 255) / 256;
     int64_t cap = (int64_t)num_compute_units() * 16;
@@ -377,6 +406,19 @@ int launch_block_quant(int fmt, const void *src, int src_dtype, size_t n_elems, 
         hipLaunchKernelGGL(block_quant_kernel<float>, dim3(grid_for(nb)), dim3(256), 0, s, fmt, (const float *)src, nb,
                            vec, (uint16_t *)dst);
     return check_launch("block_quant");
+}
+
+int launch_block_simulate(int fmt, const void *src, void *dst, int dtype, size_t n_elems, hipStream_t s) {
+    int64_t nb = (int64_t)(n_elems / 32);
+    if (nb == 0) return 0;
+    bool vec = (uintptr_t)src % 16 == 0;
+    if (dtype == TROCM_F16)
+        hipLaunchKernelGGL(block_simulate_kernel<__half>, dim3(grid_for(nb)), dim3(256), 0, s, fmt, (const __half *)src, nb, vec,
+                           (__half *)dst);
+    else
+        hipLaunchKernelGGL(block_simulate_kernel<float>, dim3(grid_for(nb)), dim3(256), 0, s, fmt, (const float *)src, nb, vec,
+                           (float *)dst);
+    return check_launch("block_simulate");
 }
 
 int launch_block_dequant(int fmt, const void *blocks, size_t n_elems, void *dst, int dst_dtype, hipStream_t s) {

@@ -338,6 +338,83 @@ class Sdpa:
         return out
 
 
+class StreamedSdpaOp:
+    """The row-streaming attention operator (streamed_sdpa.rs:6-10): Q, K, V of rank 3 or 4 and an optional rank-2
+    mask [q_len, kv_len] shared by every batch and head; the output has Q's shape and datum type.
+
+    It is served by the same kernels as Sdpa; what differs is stated here as the reference states it:
+    * a mask takes precedence and the causal flag is then not consulted (streamed_sdpa.rs:216-222);
+    * `causal` hides key i_k > t_q counted from the FIRST key (:218), whatever kv_len is, where Sdpa aligns the
+      diagonal with the last key: with kv_len > q_len only the first q_len keys are ever visible and the kernels
+      are given exactly those (no copy: a shorter kv_len over the same strides); with kv_len < q_len the rule is
+      passed as a mask;
+    * `block_k` (:8) only sets the order of the f32 sums on the CPU and is not used.
+    Scores that are NaN or +inf, which the CPU loop steps over (:231-234, :247-249), are not given that treatment."""
+
+    def __init__(self, causal: bool = False, block_k: int = 64, scale=None):
+        self.causal, self.block_k, self.scale = bool(causal), int(block_k), scale
+        self._ws = None
+
+    def name(self) -> str:
+        return "StreamedSDPA"
+
+    def info(self):
+        return [f"causal={self.causal}, block_k={self.block_k}, scale={self.scale}"]
+
+    def output_facts(self, q_shape, k_shape, v_shape, mask_shape=None):
+        """streamed_sdpa.rs:29-91."""
+        if not (len(q_shape) == len(k_shape) == len(v_shape)):
+            raise TractRocmError(f"Q, K and V must have the same rank, found {len(q_shape)}, {len(k_shape)}, {len(v_shape)} resp.")
+        if len(q_shape) not in (3, 4):
+            raise TractRocmError(f"Inputs must be of rank 3 or 4, found {len(q_shape)}")
+        if mask_shape is not None and len(mask_shape) != 2:
+            raise TractRocmError(f"Mask must be of rank 2, found mask {tuple(mask_shape)}")
+        (bq, hq, _tq, dq), (bk, hkv, tk, dk), (bv, hkv2, tk2, dv) = _canon4(q_shape), _canon4(k_shape), _canon4(v_shape)
+        if not (bq == bk == bv):
+            raise TractRocmError("Batch dims must match for Q/K/V")
+        if hkv != hkv2:
+            raise TractRocmError("K/V head counts must match")
+        if tk != tk2:
+            raise TractRocmError("K/V lengths must match")
+        if not (dq == dk == dv):
+            raise TractRocmError("Head dims (D) must match across Q/K/V")
+        if hq % hkv:
+            raise TractRocmError("num_q_heads must be a multiple of num_kv_heads for GQA")
+        return tuple(q_shape)
+
+    def eval(self, q, k, v, mask=None, stream=None, out=None) -> DeviceTensor:
+        q, k, v = (_as_device(t, stream) for t in (q, k, v))
+        m = None if mask is None else _as_device(mask, stream)
+        self.output_facts(q.shape, k.shape, v.shape, None if m is None else m.shape)
+        if q.dtype not in (np.float32, np.float16) or not (q.dtype == k.dtype == v.dtype):
+            raise TractRocmError("Q, K and V must be f32 or f16 and share a datum type")
+        B, Hq, Sq, D = _canon4(q.shape)
+        _, Hkv, Sk, _ = _canon4(k.shape)
+        causal, kv_len = 0, Sk
+        if m is not None:
+            if tuple(m.shape) != (Sq, Sk):
+                raise TractRocmError(f"mask shape {tuple(m.shape)} is not [q_len, kv_len] = [{Sq}, {Sk}]")
+            if m.dtype != q.dtype:   # the reference casts any float mask to f32 (:143-152); here to the kernels' type
+                m = Cast(q.dtype).eval(m, stream)
+        elif self.causal:
+            if Sk >= Sq:
+                causal, kv_len = 1, Sq   # keys past the q_len-th are hidden from every query
+            else:
+                rule = np.where(np.arange(Sk)[None, :] > np.arange(Sq)[:, None], -np.inf, 0.0).astype(q.dtype)
+                m = DeviceTensor.from_numpy(rule, stream)
+        if out is None:
+            out = DeviceTensor(q.shape, q.dtype)
+        elif tuple(out.shape) != tuple(q.shape) or out.dtype != q.dtype:
+            raise TractRocmError("out must have Q's shape and datum type")
+        if self._ws is None or self._ws_key != (B, Hq, D) or self._ws.nbytes < Workspace.bytes_for(B, Hq, Sq, D):
+            self._ws, self._ws_key = Workspace(B, Hq, Sq, D, stream), (B, Hq, D)
+        strides = (C.c_int64 * 3)(Hkv * Sk * D, Sk * D, D)
+        call("trocm_sdpa", q.ptr, k.ptr, v.ptr, None if m is None else m.ptr, out.ptr, dtype_code(q.dtype),
+             B, Hq, Hkv, Sq, kv_len, D, strides, 1, 1, _scale_arg(self.scale), causal,
+             self._ws.ptr, self._ws.nbytes, _sh(stream))
+        return out
+
+
 class InPlaceKvSdpa:
     """Fused in-place KV-cache + attention op: inputs [Q, K_new, V_new], output Q-shaped."""
 
@@ -590,6 +667,20 @@ class BlockQuant:
         dst = DeviceTensor((n,), dtype)
         call("trocm_block_dequant", self.fmt, src.ptr, n, dst.ptr, dtype_code(dtype), _sh(stream))
         return dst.to_numpy(stream)
+
+    def simulate_precision_loss(self, tensor, block_axis: int, stream=None) -> np.ndarray:
+        """block_quant/mod.rs:130-154: the tensor after a round trip through the format, in its own type (f32 or
+        f16); blocks run along `block_axis`, which must be the last axis."""
+        x = np.ascontiguousarray(tensor)
+        if x.dtype not in (np.float32, np.float16):
+            raise TractRocmError(f"simulate_precision_loss takes f32 or f16 tensors, got {x.dtype}")
+        if block_axis != x.ndim - 1:
+            raise TractRocmError(f"block axis {block_axis} is not the last axis of a rank {x.ndim} tensor")
+        if x.shape[-1] % 32:
+            raise TractRocmError(f"{x.shape[-1]} elements along the block axis is not a multiple of the block length 32")
+        t = DeviceTensor.from_numpy(x, stream)
+        call("trocm_block_simulate_precision_loss", self.fmt, t.ptr, t.ptr, dtype_code(x.dtype), x.size, _sh(stream))
+        return t.to_numpy(stream)
 
     def dequant_f32(self, blob, stream=None) -> np.ndarray:
         return self._dequant(blob, np.float32, stream)
