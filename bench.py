@@ -594,6 +594,18 @@ def run_ops(ta, args):
         us = time_calls(ta, one_mv, 200)
         by = n_ * (k_ // 32) * 18 + 2 * k_ + 2 * n_
         res[f"q4_0_matvec_f16_n{n_}_k{k_}"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": by}
+        if (n_, k_) != (4096, 14336):
+            # the same weights x the 512 rows of a prefill chunk: the matrix-matrix arm, on the matrix cores
+            m_ = 512
+            xm = ta.DeviceTensor.from_numpy(rng.standard_normal((1, m_, k_)).astype(np.float16))
+            om = ta.DeviceTensor((1, m_, n_), np.float16)
+
+            def one_mm():
+                gemm.eval(xm, ws[turn[0] % 8], out=om)
+                turn[0] += 1
+
+            us = time_calls(ta, one_mm, 50)
+            res[f"q4_0_matmul_f16_m{m_}_n{n_}_k{k_}"] = {"us": round(us, 2), "tflops": round(2.0 * m_ * n_ * k_ / us / 1e6, 1)}
         del ws
     # ragged decode step over quantised caches: 32 sequences of 512..32768 tokens, their new tokens quantised
     # by one launch and attention by another

@@ -31,7 +31,8 @@ def f64_product(blocks, act, dt):
     (1, 1, 1, 1, 32), (2, 2, 1, 2, 64), (2, 2, 2, 7, 128), (1, 4, 1, 1, 64), (1, 1, 5, 1, 32), (1, 2, 8, 2, 64),
     (1, 1, 1, 4096, 4096), (1, 1, 1, 1000, 2080), (1, 1, 3, 515, 4096), (1, 2, 4, 130, 1024), (1, 1, 6, 77, 2048),
     (1, 1, 7, 33, 992), (1, 1, 8, 200, 8192), (1, 1, 1, 64, 20480), (2, 4, 2, 50, 14336),
-    (1, 1, 9, 40, 128), (1, 2, 21, 70, 256), (2, 2, 64, 33, 512),   # more than 8 rows: groups of 8
+    (1, 1, 9, 40, 128), (1, 2, 21, 70, 256), (2, 2, 64, 33, 512),   # more than 8 rows: the matrix-matrix arm (f16) / groups of 8
+    (1, 1, 9, 40, 96), (2, 4, 9, 129, 128), (1, 2, 130, 300, 1024), (1, 1, 257, 131, 2048), (1, 1, 512, 1024, 4096),
 ])
 def test_matvec_matches_the_oracle(rt, dt, wb, ab, m, n, k):
     rng = np.random.default_rng(n + k + m)

@@ -269,7 +269,11 @@ int launch_m(const MatVecDev &p, int m, int64_t act_batch, hipStream_t s) {
 int launch_q4_0_matvec(const void *codes, const void *scales, int64_t w_batch, int64_t n, int64_t k, const void *act,
                        int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s) {
     const int64_t es = (int64_t)elem_bytes(act_dtype);
-    // More than 8 activation rows run as groups of 8 (each group streams the weights once): correct
+    if (m > 8) {   // the matrix-matrix arm (q4_matmul.hip) for f16 activations
+        const int rc = launch_q4_0_matmul(codes, scales, w_batch, n, k, act, act_dtype, act_batch, m, out, s);
+        if (rc != 2) return rc;
+    }
+    // What it does not take runs as groups of 8 rows (each group streams the weights once): correct
     // for any m, efficient only for the few rows of a decode step.
     for (int64_t i0 = 0; i0 < m; i0 += 8) {
         const int64_t mg = m - i0 < 8 ? m - i0 : 8;
