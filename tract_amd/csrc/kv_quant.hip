@@ -33,20 +33,21 @@ __device__ __forceinline__ uint16_t f32_to_f16_bits(float x) {
 __device__ __forceinline__ void store_out(float *p, float x) { *p = x; }
 __device__ __forceinline__ void store_out(__half *p, float x) { *p = __ushort_as_half(f32_to_f16_bits(x)); }
 
-// Rust `f32 as i8`: truncate toward zero, saturate, NaN -> 0.
-__device__ __forceinline__ int sat_i8(float x) {
-    if (x != x) return 0;
-    if (x <= -128.0f) return -128;
-    if (x >= 127.0f) return 127;
-    return (int)x;
+// Rust `f32 as i8`: truncate toward zero, saturate, NaN -> 0.  v_cvt_i32_f32 does the first and the last itself
+// (it truncates, saturates at the 32-bit range and turns NaN into 0); what is left is the clamp to 8 bits.
+__device__ __forceinline__ int cvt_i32_rz_sat(float x) {
+    int r;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(x));   // (a C cast may assume the value is in range)
+    return r;
 }
+__device__ __forceinline__ int sat_i8(float x) { return max(-128, min(127, cvt_i32_rz_sat(x))); }   // (one v_med3_i32)
 
-// f32::round(): half away from zero.  x - trunc(x) is exact, so the comparison is too.
+// f32::round(): half away from zero.  d = x - trunc(x) is exact and |d| < 1, so d + d is exact too and its
+// truncation is the unit to add: +-1 exactly when |d| >= 0.5, with the sign of x.
 __device__ __forceinline__ float round_half_away(float x) {
-    float t = truncf(x);
-    float d = __fsub_rn(x, t);
-    if (fabsf(d) >= 0.5f) t = __fadd_rn(t, copysignf(1.0f, x));
-    return t;
+    const float t = truncf(x);
+    const float d = __fsub_rn(x, t);
+    return __fadd_rn(t, truncf(__fadd_rn(d, d)));
 }
 
 // Signed value of the first element with strictly largest magnitude (q4_0.rs:27-34).
@@ -132,35 +133,43 @@ struct QuantAppendDev {
     uint8_t *codes;
     uint16_t *scales;
     int64_t n_blocks;
+    int nb_shift;   // log2(D / 32) when that is a power of two, else -1
 };
 
 template <typename SrcT>
+__device__ __forceinline__ void quant_one_block(const QuantAppendDev &a, const SrcT *p, int64_t row, int64_t nb, int64_t blk) {
+    float v[32];
+    load_block(p, a.ss[3], a.vec != 0, v);
+    if (a.fmt == TROCM_Q8_0) {
+        uint32_t c[8];
+        uint16_t d = quant_q8(v, c);
+        uint4 *dst = reinterpret_cast<uint4 *>(a.codes + row * a.D + blk * 32);
+        dst[0] = make_uint4(c[0], c[1], c[2], c[3]);
+        dst[1] = make_uint4(c[4], c[5], c[6], c[7]);
+        a.scales[row * nb + blk] = d;
+    } else {
+        uint32_t c[4];
+        uint16_t d = quant_q4(v, c);
+        *reinterpret_cast<uint4 *>(a.codes + row * (a.D / 2) + blk * 16) = make_uint4(c[0], c[1], c[2], c[3]);
+        a.scales[row * nb + blk] = d;
+    }
+}
+
+// Grid (chunks of a (batch, head) row's blocks, batch * heads): the position of a block inside its row is one 32-bit
+// division (a shift when head_dim / 32 is a power of two); with a flat index over all blocks the three 64-bit
+// divisions were 45 % of the kernel's instructions, and the kernel is bound by them, not by HBM.
+template <typename SrcT>
 __global__ __launch_bounds__(256) void quant_append_kernel(QuantAppendDev a) {
-    int64_t nb = a.D / 32;
-    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < a.n_blocks;
-         idx += (int64_t)gridDim.x * blockDim.x) {
-        int64_t blk = idx % nb;
-        int64_t rem = idx / nb;
-        int64_t t = rem % a.S;
-        rem /= a.S;
-        int64_t h = rem % a.H;
-        int64_t b = rem / a.H;
-        const SrcT *p = (const SrcT *)a.src + b * a.ss[0] + h * a.ss[1] + t * a.ss[2] + blk * 32 * a.ss[3];
-        float v[32];
-        load_block(p, a.ss[3], a.vec != 0, v);
-        int64_t row = (b * a.H + h) * a.cap + a.t0 + t;
-        if (a.fmt == TROCM_Q8_0) {
-            uint32_t c[8];
-            uint16_t d = quant_q8(v, c);
-            uint4 *dst = reinterpret_cast<uint4 *>(a.codes + row * a.D + blk * 32);
-            dst[0] = make_uint4(c[0], c[1], c[2], c[3]);
-            dst[1] = make_uint4(c[4], c[5], c[6], c[7]);
-            a.scales[row * nb + blk] = d;
-        } else {
-            uint32_t c[4];
-            uint16_t d = quant_q4(v, c);
-            *reinterpret_cast<uint4 *>(a.codes + row * (a.D / 2) + blk * 16) = make_uint4(c[0], c[1], c[2], c[3]);
-            a.scales[row * nb + blk] = d;
+    const uint32_t nb = (uint32_t)(a.D / 32);
+    const uint32_t per_row = (uint32_t)a.S * nb;
+    for (int64_t bh = blockIdx.y; bh < a.B * a.H; bh += gridDim.y) {
+        const int64_t b = bh / a.H, h = bh % a.H;   // (scalar: once per workgroup trip)
+        const SrcT *src_row = (const SrcT *)a.src + b * a.ss[0] + h * a.ss[1];
+        const int64_t row0 = bh * a.cap + a.t0;
+        for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < per_row; i += gridDim.x * blockDim.x) {
+            const uint32_t t = a.nb_shift >= 0 ? i >> a.nb_shift : i / nb;
+            const uint32_t blk = i - t * nb;
+            quant_one_block(a, src_row + (int64_t)t * a.ss[2] + (int64_t)blk * 32 * a.ss[3], row0 + t, nb, blk);
         }
     }
 }
@@ -355,11 +364,22 @@ int launch_quant_append(const QuantAppend &a, hipStream_t s) {
     bool vec = a.ss[3] == 1 && ((uintptr_t)a.src % 16 == 0);
     for (int i = 0; i < 3 && vec; i++) vec = (a.ss[i] * (int64_t)es) % 16 == 0;
     d.vec = vec;
-    int grid = grid_for(d.n_blocks);
+    TROCM_REQUIRE(a.S * (a.D / 32) < (1ll << 31), "quant_append: %lld tokens of %lld blocks per (batch, head) row exceed the 32-bit index",
+                  (long long)a.S, (long long)(a.D / 32));
+    const int64_t nb = a.D / 32;
+    d.nb_shift = -1;
+    for (int sh = 0; sh < 16; sh++)
+        if (nb == (1ll << sh)) d.nb_shift = sh;
+    const int64_t per_row = a.S * nb, bh = a.B * a.H;
+    const int64_t want = (int64_t)num_compute_units() * 16;              // workgroups that keep the device busy
+    int64_t gx = (per_row + 255) / 256;
+    int64_t gy = bh < 65535 ? bh : 65535;
+    if (gx * gy > want) gx = gx * gy / want > 0 ? (gx + (gx * gy / want) - 1) / (gx * gy / want) : gx;   // several blocks per thread
+    if (gx < 1) gx = 1;
     if (a.src_dtype == TROCM_F16)
-        hipLaunchKernelGGL(quant_append_kernel<__half>, dim3(grid), dim3(256), 0, s, d);
+        hipLaunchKernelGGL(quant_append_kernel<__half>, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, d);
     else
-        hipLaunchKernelGGL(quant_append_kernel<float>, dim3(grid), dim3(256), 0, s, d);
+        hipLaunchKernelGGL(quant_append_kernel<float>, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, d);
     return check_launch("quant_append");
 }
 
