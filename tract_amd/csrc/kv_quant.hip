@@ -373,9 +373,11 @@ int launch_quant_append(const QuantAppend &a, hipStream_t s) {
     const int64_t per_row = a.S * nb, bh = a.B * a.H;
     const int64_t want = (int64_t)num_compute_units() * 16;              // workgroups that keep the device busy
     int64_t gx = (per_row + 255) / 256;
-    int64_t gy = bh < 65535 ? bh : 65535;
-    if (gx * gy > want) gx = gx * gy / want > 0 ? (gx + (gx * gy / want) - 1) / (gx * gy / want) : gx;   // several blocks per thread
-    if (gx < 1) gx = 1;
+    const int64_t gy = bh < 65535 ? bh : 65535;
+    if (gx * gy > want) {   // more workgroups than that: every thread takes several blocks
+        const int64_t per_thread = gx * gy / want;
+        gx = (gx + per_thread - 1) / per_thread;
+    }
     if (a.src_dtype == TROCM_F16)
         hipLaunchKernelGGL(quant_append_kernel<__half>, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, d);
     else
