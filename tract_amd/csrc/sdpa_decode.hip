@@ -146,8 +146,7 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
             for (int j = 0; j < KL; j++) kreg[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + k_off[j]));
         } else {
             // the sequence's last tile and the tile of a fused new token: rows past the end repeat the
-            // last token; the new token comes from the step's input and is written to its place in
-            // the cache on the way
+            // last token; the new token comes from the step's input
 #pragma unroll
             for (int j = 0; j < KL; j++) {
                 int L = j * 64 + lane;
@@ -155,7 +154,6 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
                 const char *cache_ptr = base + (uint32_t)row * stride_t + (uint32_t)c * 16u;
                 const bool is_new = t0 + row == new_pos;
                 kreg[j] = *reinterpret_cast<const u32x4 *>(is_new ? wk.k_new + c * 16 : cache_ptr);
-                if (is_new && L / CPR == new_pos - t0) *reinterpret_cast<u32x4 *>(const_cast<char *>(cache_ptr)) = kreg[j];
             }
         }
     };
@@ -172,11 +170,20 @@ __device__ __forceinline__ void decode_body(const DecodeDev &p, const DecodeWork
                 const char *cache_ptr = base + (uint32_t)row * stride_t + (uint32_t)j16 * (uint32_t)sizeof(vslice_t);
                 const bool is_new = t0 + row == new_pos;
                 vreg[i] = *reinterpret_cast<const vslice_t *>(is_new ? wk.v_new + j16 * (int)sizeof(vslice_t) : cache_ptr);
-                if (is_new && 4 * i + rg == new_pos - t0)
-                    *reinterpret_cast<vslice_t *>(const_cast<char *>(cache_ptr)) = vreg[i];
             }
         }
     };
+
+    // A fused new token is stored to its place in the cache here, by the first wave of the sequence-head's first
+    // workgroup, ahead of the tile loop: stored from inside the loop, the store shared the vector-memory counter with
+    // the prefetches, and the waits the compiler sizes for the path with the fewest operations in flight made every tile
+    // wait for its newest loads as well.
+    if (new_pos >= 0 && w == 0 && tile_begin == 0 && lane < 2 * CPR) {
+        const int c = lane % CPR;
+        const char *src = (lane < CPR ? wk.k_new : wk.v_new) + c * 16;
+        char *dst = const_cast<char *>(lane < CPR ? kbase : vbase) + (int64_t)new_pos * p.kv_stride_t + c * 16;
+        *reinterpret_cast<u32x4 *>(dst) = *reinterpret_cast<const u32x4 *>(src);
+    }
 
     int tile = tile_begin + w;
     if (tile < tile_end) {

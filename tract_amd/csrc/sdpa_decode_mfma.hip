@@ -179,9 +179,21 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
     uint32_t ksc[QUANT ? NLD : 1], vsc[QUANT ? NLD : 1];
     const int my_block = (lane % CPR) * EPC / 32;
     const uint32_t sc_word = (my_block >> 1) * 4, sc_sel = (my_block & 1) ? 0x03020302u : 0x01000100u;
-    // fused append: the row of token new_pos comes from the step's input and is stored to the cache on the way
+    // fused append: the row of token new_pos comes from the step's input wherever a tile holds it, and the first wave
+    // of the sequence-head's first workgroup stores it to the cache here, ahead of the tile loop.  (Stored from inside
+    // the loop, by the wave whose tile holds it, the store shared the vector-memory counter with the prefetches: the
+    // compiler sizes a wait for the path with the fewest operations in flight, so every tile of every wave waited for
+    // its newest loads as well -- 1.6 us of a 47.6 us launch, with or without a new token.)
     const int new_pos = wk.new_pos;
     const int64_t new_row = ((int64_t)b * p.Hkv + kvh) * D * 2;
+    if constexpr (!QUANT) {
+        if (new_pos >= 0 && w == 0 && wk.tile_begin == 0 && lane < 2 * CPR) {
+            const int dc = lane % CPR;
+            const char *src = (lane < CPR ? p.k_new : p.v_new) + new_row + dc * 16;
+            char *dst = const_cast<char *>(lane < CPR ? kbase : vbase) + (int64_t)new_pos * p.kv_stride_t + dc * 16;
+            *reinterpret_cast<u32x4 *>(dst) = *reinterpret_cast<const u32x4 *>(src);
+        }
+    }
     auto fetch_q = [&](const char *base0, const char *sbase0, int t, u32x4 (&dst)[NLD], uint32_t (&sc)[QUANT ? NLD : 1]) {
         const int t0 = t * kTile;
         const char *base = base0 + (int64_t)t0 * RB;
@@ -237,7 +249,6 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
                 const char *cache_ptr = base + (uint32_t)row * (uint32_t)p.kv_stride_t + (uint32_t)dc * 16u;
                 const bool is_new = t0 + row == new_pos;
                 dst[j] = *reinterpret_cast<const u32x4 *>(is_new ? fresh + new_row + dc * 16 : cache_ptr);
-                if (is_new && c / CPR == new_pos - t0) *reinterpret_cast<u32x4 *>(const_cast<char *>(cache_ptr)) = dst[j];
             }
         }
     };
