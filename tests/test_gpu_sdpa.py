@@ -698,6 +698,31 @@ def test_prefill_grouped_heads_and_key_splits(rt, B, Hq, Hkv, Sq, Sk, D, causal)
     assert max_abs(got, cases.textbook_sdpa(q, k, v, causal=causal)) <= 4e-3
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,masked", [
+    (1, 32, 8, 512, 2048, 128, False),    # four key splits merged by whichever workgroup arrives last
+    (2, 32, 8, 848, 848, 128, False),     # two splits
+    (2, 32, 8, 848, 848, 128, True),      # the mask-input instantiation
+    (1, 8, 2, 64, 4096, 128, False),      # 16 splits: merged two at a time
+    (1, 16, 4, 96, 1500, 64, False),
+])
+def test_prefill_key_splits_give_the_same_bits_every_time(rt, B, Hq, Hkv, Sq, Sk, D, masked):
+    """The split that arrives last merges the others and takes its own partial from registers; which one that is
+    changes from launch to launch, the output bits must not."""
+    rng = np.random.default_rng(2100 + Sq + Sk + Hq)
+    q = (rng.standard_normal((B, Hq, Sq, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+    k = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32).astype(np.float16)
+    if masked:
+        mask = np.where(np.arange(Sk)[None, :] <= np.arange(Sq)[:, None] + (Sk - Sq), 0.0, -np.inf).astype(np.float16)[None, None]
+        op, inputs = tract_amd.Sdpa(datum_type=np.float16), (q, k, v, mask)
+    else:
+        op, inputs = tract_amd.Sdpa(datum_type=np.float16, is_causal=True), (q, k, v)
+    first = op.eval(*inputs).to_numpy()
+    assert max_abs(first, cases.textbook_sdpa(q, k, v, causal=True)) <= 4e-3
+    for _ in range(12):
+        assert op.eval(*inputs).to_numpy().tobytes() == first.tobytes()
+
+
 @pytest.mark.parametrize("Sq", [2, 3, 5, 8, 17, 31])
 @pytest.mark.parametrize("Hq,Hkv,D,T", [(32, 8, 128, 3000), (16, 2, 128, 1100), (8, 4, 64, 777)])
 def test_few_queries_over_a_long_cache(rt, Sq, Hq, Hkv, D, T):

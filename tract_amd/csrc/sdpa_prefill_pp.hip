@@ -368,10 +368,6 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
     for (int it = 0; it < n_it; it++) {
         __syncthreads();   // tile `it` is in LDS; every wave is done with the buffers about to be overwritten
         const int cur = it & 1;
-        if (it + 1 < n_it) {
-            stage(cur ^ 1, cur ^ 1);
-            if (it + 2 < n_it) prefetch(t_begin + it + 2);
-        }
         const int kt = t_begin + it;
         if (tile_active(kt)) {
             float16_t s[2];
@@ -381,22 +377,55 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
             if (it + 1 < n_it) prefetch_mask(kt + 1);
             pv(cur, pf);
         }
+        // The next tile goes to LDS after this one's arithmetic, not before it: its loads were issued a whole
+        // iteration ago in the steady state and right before the loop for the first iteration, whose arithmetic
+        // then covers their latency.
+        if (it + 1 < n_it) {
+            stage(cur ^ 1, cur ^ 1);
+            if (it + 2 < n_it) prefetch(t_begin + it + 2);
+        }
     }
     l_run += __shfl_xor(l_run, 32, 64);
-    if (p.nsplit == 1) {
-        if (!wave_has_queries || my_q >= p.Sq) return;
-        const int64_t row = ((int64_t)b * p.Hq + qh) * p.Sq + my_q;
-        const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
-        _Float16 *orow = p.out + row * D;
+    // Output rows of this wave (32 queries of one head: one contiguous block of 32 * D halves).  A lane holds
+    // 4-feature pieces of its own query's row, which stored as they stand would touch 32 rows per instruction;
+    // they go through a wave-private corner of the (idle) V tile buffers instead, half of the features at a
+    // time, and leave as 16-byte pieces of consecutive addresses.  Callers make sure every wave of the
+    // workgroup is past the tile loop.
+    auto wave_sync = []() {   // orders this wave's LDS accesses across its lanes (no instruction: the LDS serves a wave in order)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    auto write_output = [&](float mul) {
+        constexpr int FP = D / 2, TROW = FP + 8, CPRW = FP / 8, RPI = 64 / CPRW;   // features per pass, LDS row, 16-byte pieces per row, rows per instruction
+        static_assert(kWavesPP * 32 * TROW <= 2 * kTileN * VROW, "transposition area exceeds the V tile buffers");
+        _Float16 *tr = &lds_v[0][0] + w * (32 * TROW);
+        _Float16 *obase = p.out + (((int64_t)b * p.Hq + qh) * p.Sq + q0) * D;
 #pragma unroll
-        for (int db = 0; db < DB; db++)
+        for (int h = 0; h < 2; h++) {
 #pragma unroll
-            for (int rq = 0; rq < 4; rq++) {
-                half4_t h4;
+            for (int d2 = 0; d2 < DB / 2; d2++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) h4[i] = (_Float16)(o[db][4 * rq + i] * inv);
-                *reinterpret_cast<half4_t *>(orow + 32 * db + 8 * rq + 4 * hb) = h4;
+                for (int rq = 0; rq < 4; rq++) {
+                    half4_t h4;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) h4[i] = (_Float16)(o[h * (DB / 2) + d2][4 * rq + i] * mul);
+                    *reinterpret_cast<half4_t *>(tr + l32 * TROW + 32 * d2 + 8 * rq + 4 * hb) = h4;
+                }
+            wave_sync();   // lanes read what other lanes of the wave wrote
+#pragma unroll
+            for (int i = 0; i < 32 / RPI; i++) {
+                const int row = i * RPI + lane / CPRW, ch = lane % CPRW;
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(tr + row * TROW + ch * 8);
+                if (q0 + row < p.Sq) *reinterpret_cast<u32x4 *>(obase + (int64_t)row * D + h * FP + ch * 8) = v;
             }
+            wave_sync();   // ... and are done reading before the second half overwrites it
+        }
+    };
+    if (p.nsplit == 1) {
+        __syncthreads();   // the V tile buffers are idle from here on
+        if (!wave_has_queries) return;
+        write_output(l_run > 0.0f ? 1.0f / l_run : 0.0f);
         return;
     }
     // ---- key splits: store this split's normalised partial -----------------------------------------
@@ -405,8 +434,18 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
     // workgroup signals its arrival.
     const bool tail_merge = p.counters != nullptr;
     const int64_t wb = ((int64_t)b * p.Hq + qh) * p.n_qb32 + (q0 >> 5);
+    const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+    // An element of this split's normalised partial, as it is stored.  The product is rounded to f32 on its own
+    // and then to f16, here and wherever the value is formed again (the merge below takes the own split's
+    // values from the accumulators): the multiplication is written out so that the compiler cannot fuse the two
+    // steps in one place and not in the other, which would round differently in rare cases (and, being volatile,
+    // stays where it is used instead of being hoisted, all 64 products at once, above the merge's loads).
+    auto partial_elem = [&](float acc) {
+        float pr;
+        asm volatile("v_mul_f32 %0, %1, %2" : "=v"(pr) : "v"(acc), "v"(inv));
+        return (_Float16)pr;
+    };
     if (wave_has_queries) {
-        const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
         _Float16 *po = p.part_o + ((int64_t)split * p.n_wb + wb) * (32 * D) + l32 * 4;
         float *pml = p.part_ml + ((int64_t)split * p.n_wb + wb) * 64 + lane;
 #pragma unroll
@@ -415,7 +454,7 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
             for (int rq = 0; rq < 4; rq++) {
                 half4_t h4;
 #pragma unroll
-                for (int i = 0; i < 4; i++) h4[i] = (_Float16)(o[db][4 * rq + i] * inv);
+                for (int i = 0; i < 4; i++) h4[i] = partial_elem(o[db][4 * rq + i]);
                 _Float16 *dst = po + (8 * db + 2 * rq + hb) * 128;
                 if (tail_merge)
                     __hip_atomic_store(reinterpret_cast<uint64_t *>(dst), __builtin_bit_cast(uint64_t, h4), __ATOMIC_RELAXED,
@@ -448,6 +487,7 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
     // two splits in flight at a time.
     constexpr int kMaxSplits = 16;
     auto aload_f = [](const float *a) { return __hip_atomic_load(a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    static_assert(kWavesPP * kMaxSplits * 32 * sizeof(float) <= sizeof(lds_k), "merge weights exceed the K tile buffers");
     float *wts = reinterpret_cast<float *>(&lds_k[0][0]) + w * (kMaxSplits * 32);
     // One merge step for NS splits starting at s0: their outputs and, when WEIGHTS, the (m, l) records of
     // MAXS splits are requested together; the weights go through LDS (lanes 32..63 need those of lanes 0..31).
@@ -464,9 +504,11 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
                                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     };
-    auto weights = [&](auto maxs_tag) {
+    // Every lane works out the weights of its query into lv (lanes l and l + 32 the same ones, from the same
+    // loads): nothing is handed from lane to lane.
+    auto weights = [&](auto maxs_tag, auto &lv) {
         constexpr int MAXS = decltype(maxs_tag)::value;
-        float mv[MAXS], lv[MAXS];
+        float mv[MAXS];
 #pragma unroll
         for (int sp = 0; sp < MAXS; sp++) {
             const float *ml = p.part_ml + ((int64_t)min(sp, p.nsplit - 1) * p.n_wb + wb) * 64;
@@ -483,11 +525,9 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
             lv[sp] = sp < p.nsplit ? lv[sp] * fast_exp2(mv[sp] - m_ref) : 0.0f;
             total += lv[sp];
         }
-        const float inv = total > 0.0f ? 1.0f / total : 0.0f;
-        if (hb == 0) {
+        const float inv_total = total > 0.0f ? 1.0f / total : 0.0f;
 #pragma unroll
-            for (int sp = 0; sp < MAXS; sp++) wts[sp * 32 + l32] = lv[sp] * inv;
-        }
+        for (int sp = 0; sp < MAXS; sp++) lv[sp] *= inv_total;
     };
     auto accumulate = [&](int s0, auto &raw, auto ns_tag) {
         constexpr int NS = decltype(ns_tag)::value;
@@ -510,14 +550,59 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
 #pragma unroll
             for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
     };
-    if (p.nsplit <= 4) {   // the common case: everything in one round trip to the L2
-        uint64_t raw[4][DB * 4];
-        load_outputs(0, raw, std::integral_constant<int, 4>{});
-        weights(std::integral_constant<int, 4>{});
-        zero_o();
-        accumulate(0, raw, std::integral_constant<int, 4>{});
+    if (p.nsplit <= 4) {
+        // The common case: everything in one round trip to the L2, and this workgroup's own partial, still in
+        // its accumulators, is not read back.  Every element is the chain fma(w3, O3, fma(w2, O2, fma(w1, O1,
+        // w0 O0))) over the splits in their order, the own term entering at its place with the f16 value that
+        // was stored: the result does not depend on which split arrived last.
+        uint64_t raw[3][DB * 4];   // the other splits in their order
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            const int sj = min(j + (j >= split), p.nsplit - 1);
+            const _Float16 *po = p.part_o + ((int64_t)sj * p.n_wb + wb) * (32 * D) + l32 * 4;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++)
+                    raw[j][db * 4 + rq] = __hip_atomic_load(reinterpret_cast<const uint64_t *>(po + (8 * db + 2 * rq + hb) * 128),
+                                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        float wv[4];   // 0 past the last split
+        weights(std::integral_constant<int, 4>{}, wv);
+        auto chain = [&](auto own_tag) {
+            constexpr int K = decltype(own_tag)::value;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    half4_t h[3];
+#pragma unroll
+                    for (int j = 0; j < 3; j++) h[j] = __builtin_bit_cast(half4_t, raw[j][db * 4 + rq]);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const float mine = (float)partial_elem(o[db][4 * rq + i]);
+                        float acc = 0.0f;
+#pragma unroll
+                        for (int sp = 0; sp < 4; sp++) {
+                            const float term = sp == K ? mine : (float)h[sp < K ? sp : sp - 1][i];
+                            acc = sp == 0 ? wv[0] * term : __builtin_fmaf(wv[sp], term, acc);
+                        }
+                        o[db][4 * rq + i] = acc;
+                    }
+                    __builtin_amdgcn_sched_barrier(0);   // piece by piece: hoisting all the own-term products at once spills
+                }
+        };
+        switch (split) {
+            case 0: chain(std::integral_constant<int, 0>{}); break;
+            case 1: chain(std::integral_constant<int, 1>{}); break;
+            case 2: chain(std::integral_constant<int, 2>{}); break;
+            default: chain(std::integral_constant<int, 3>{}); break;
+        }
     } else {
-        weights(std::integral_constant<int, kMaxSplits>{});
+        float wv[kMaxSplits];
+        weights(std::integral_constant<int, kMaxSplits>{}, wv);
+#pragma unroll
+        for (int sp = 0; sp < kMaxSplits; sp++) wts[sp * 32 + l32] = wv[sp];   // lanes l and l + 32 write the same value and read it back
         zero_o();
         for (int s0 = 0; s0 < p.nsplit; s0 += 2) {
             uint64_t raw[2][DB * 4];
@@ -525,17 +610,7 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
             accumulate(s0, raw, std::integral_constant<int, 2>{});
         }
     }
-    if (my_q >= p.Sq) return;
-    _Float16 *orow = p.out + (((int64_t)b * p.Hq + qh) * p.Sq + my_q) * D;
-#pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int rq = 0; rq < 4; rq++) {
-            half4_t h4;
-#pragma unroll
-            for (int i = 0; i < 4; i++) h4[i] = (_Float16)o[db][4 * rq + i];
-            *reinterpret_cast<half4_t *>(orow + 32 * db + 8 * rq + 4 * hb) = h4;
-        }
+    write_output(1.0f);
 }
 
 // Merge of the key splits, one workgroup per 32-query block:
@@ -653,7 +728,7 @@ int launch_sdpa_prefill_pp(const SdpaArgs &a, hipStream_t s) {
     if (a.causal && a.Sk < a.Sq) return 2;  // some queries would see nothing: the generic kernel owns that case
     if (a.Sk >= (1ll << 30) || a.Sq >= (1ll << 30) || a.B >= (1ll << 20)) return 2;
     if ((a.kv_stride_b % 8) || (a.kv_stride_h % 8) || (a.kv_stride_t % 8)) return 2;  // 128-bit row loads
-    if ((uintptr_t)a.q % 16 || (uintptr_t)a.k % 16 || (uintptr_t)a.v % 16 || (uintptr_t)a.out % 8) return 2;
+    if ((uintptr_t)a.q % 16 || (uintptr_t)a.k % 16 || (uintptr_t)a.v % 16 || (uintptr_t)a.out % 16) return 2;
     if (quant) {   // strides arrive in elements of the logical [.., D] rows: whole token rows per head and batch
         if (a.kv_stride_h % a.D || a.kv_stride_b % a.D) return 2;
         const int64_t rb = a.kv_fmt == TROCM_Q8_0 ? a.D : a.D / 2;
