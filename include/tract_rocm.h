@@ -356,6 +356,57 @@ int trocm_inplace_kv_sdpa_eval_ragged(const void *q, const void *k_new, const vo
                                       trocm_kv_cache *const *v_caches, void *out, float scale,
                                       void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- KIVI-style affine quantised caches (the reference's own storage-quantised cache ops) ----------
+ *
+ * A different scheme from Q8_0 / Q4_0: u8 or u4 codes with f32 (lo, scale) parameters, Values per token,
+ * Keys per channel.  One object holds one tensor [batch, heads, len, head_dim]; stored codes and
+ * parameters are bit-identical to the CPU op's.
+ *   TROCM_KIVI_PER_TOKEN        PerTokenStore (transformers/src/ops/quant_dyn_kv_cache.rs:97-151) and, with 8 bits
+ *                               and no sink tokens, QuantValueCache (transformers/src/ops/kv_quant.rs:121-163)
+ *   TROCM_KIVI_BLOCK_CHANNEL    BlockChannelStore (quant_dyn_kv_cache.rs:153-250): per-channel parameters frozen
+ *                               per block of 32 tokens, the partial block kept in f32
+ *   TROCM_KIVI_RUNNING_CHANNEL  QuantKeyCache (kv_quant.rs:171-236): running per-channel lo / scale, 8 bits; old
+ *                               codes are read back with the current parameters, as the CPU op does
+ * The first `sink_tokens` tokens stay in f32 (SINK_TOKENS = 4 in quant_dyn_kv_cache.rs:92; 0 in kv_quant.rs). */
+typedef struct trocm_kivi_cache trocm_kivi_cache;
+enum { TROCM_KIVI_PER_TOKEN = 0, TROCM_KIVI_BLOCK_CHANNEL = 1, TROCM_KIVI_RUNNING_CHANNEL = 2 };
+enum { TROCM_KIVI_PART_SINK = 0, TROCM_KIVI_PART_CODES = 1, TROCM_KIVI_PART_LO = 2, TROCM_KIVI_PART_SCALE = 3,
+       TROCM_KIVI_PART_RESIDUAL = 4 };
+
+/* HeadCache::new for every (batch, head) (quant_dyn_kv_cache.rs:259-266, :401-406; kv_quant.rs:301-305).  bits is 4
+ * or 8 (quant_dyn_kv_cache.rs:706).  Allocates at the first append. */
+int trocm_kivi_cache_create(trocm_kivi_cache **out, int layout, int bits, int64_t sink_tokens, int64_t batch,
+                            int64_t heads, int64_t head_dim);
+int trocm_kivi_cache_destroy(trocm_kivi_cache *cache);
+int trocm_kivi_cache_len(const trocm_kivi_cache *cache, int64_t *len);
+/* Tokens held as f32 sinks, as coded rows and in the partial key block; bytes of a coded row (row_bytes, :58-60). */
+int trocm_kivi_cache_counts(const trocm_kivi_cache *cache, int64_t *n_sink, int64_t *n_rows, int64_t *n_res,
+                            int64_t *row_bytes);
+/* Resident bytes of the state: codes + 8 per parameter pair (memory_bytes, kv_quant.rs:160-162, :233-235) + the f32
+ * sink and partial-block rows. */
+int trocm_kivi_cache_memory_bytes(const trocm_kivi_cache *cache, size_t *bytes);
+/* QuantizedDynKvCacheState::ingest (quant_dyn_kv_cache.rs:393-423): push every new token of `src`
+ * ([batch, heads, n_new, head_dim] dense, F32 or F16; F16 is widened exactly like cast_to::<f32>, :487). */
+int trocm_kivi_cache_append(trocm_kivi_cache *cache, const void *src, int src_dtype, int64_t n_new, void *stream);
+/* QuantizedDynKvCacheState::dequantized + cast_to_dt (:426-449, :489): the whole cache as
+ * [batch, heads, len, head_dim] dense of dst_dtype (F16 rounds to nearest even).  This is the op's output and
+ * what save_to stores (:467-470). */
+int trocm_kivi_cache_dequantize(const trocm_kivi_cache *cache, void *dst, int dst_dtype, void *stream);
+/* One part of the raw state, dense per (batch, head): SINK [n_sink, head_dim] f32, CODES [n_rows, row_bytes],
+ * LO / SCALE f32 ([n_rows] per token, [n_rows / 32, head_dim] per block and channel, [head_dim] running),
+ * RESIDUAL [n_res, head_dim] f32.  `bytes` receives the size; a NULL dst only asks for it. */
+int trocm_kivi_cache_export(const trocm_kivi_cache *cache, int part, void *dst_device, size_t *bytes, void *stream);
+/* OpStateFreeze::freeze (quant_dyn_kv_cache.rs:510-524; kv_quant.rs:345-355): an independent deep copy. */
+int trocm_kivi_cache_clone(const trocm_kivi_cache *cache, trocm_kivi_cache **out, void *stream);
+
+/* QuantizedKvSdpaState::eval (kv_quant.rs:283-330): push k_new and v_new ([batch, kv_heads, n_new, head_dim] dense
+ * of `dtype`) into a RUNNING_CHANNEL key store and a PER_TOKEN value store (8 bits, no sink tokens), dequantise
+ * both and attend q ([batch, q_heads, n_new, head_dim]) over every stored token WITHOUT a causal mask (:326).  The
+ * dequantised copies live in buffers the stores own and grow by doubling. */
+int trocm_quantized_kv_sdpa_eval(const void *q, const void *k_new, const void *v_new, int dtype, int64_t q_heads,
+                                 int64_t n_new, trocm_kivi_cache *k_cache, trocm_kivi_cache *v_cache, void *out,
+                                 float scale, void *workspace, size_t workspace_bytes, void *stream);
+
 #if defined(__GNUC__)
 #pragma GCC visibility pop
 #endif

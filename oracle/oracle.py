@@ -20,8 +20,8 @@ BLOCK_BYTES = {FMT_Q8_0: 34, FMT_Q4_0: 18, FMT_Q8_1: 36}
 
 def build(force: bool = False) -> str:
     """Compile the oracle with gcc (a few hundred ms)."""
-    src = os.path.join(_HERE, "tract_oracle.c")
-    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+    srcs = [os.path.join(_HERE, f) for f in ("tract_oracle.c", "kivi_oracle.c")]
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < max(os.path.getmtime(s) for s in srcs):
         subprocess.check_call(["make", "-s", "-C", _HERE, "-B" if force else "-s"])
     return _SO
 
@@ -78,6 +78,19 @@ def lib() -> C.CDLL:
         L.orc_naive_sdpa_f64.argtypes = [vp, vp, vp, vp] + [sz] * 6 + [sz, sz, i, i, f, vp]
         L.orc_max_threads.restype = i
         L.orc_decode_step_f16.argtypes = [vp] * 5 + [sz] * 5 + [i, vp, C.POINTER(vp), C.POINTER(vp)]
+        L.orc_kivi_quant_dequant.argtypes = [vp, sz, sz, C.c_uint, i, vp]
+        L.orc_kivi_new.restype = vp
+        L.orc_kivi_new.argtypes = [i, sz, C.c_uint, sz]
+        L.orc_kivi_clone.restype = vp
+        L.orc_kivi_clone.argtypes = [vp]
+        L.orc_kivi_free.argtypes = [vp]
+        L.orc_kivi_push.argtypes = [vp, vp]
+        for n in ("len", "n_sink", "n_rows", "n_res", "n_params", "row_bytes", "memory_bytes"):
+            fn = getattr(L, "orc_kivi_" + n)
+            fn.restype = sz
+            fn.argtypes = [vp]
+        L.orc_kivi_state.argtypes = [vp] * 6
+        L.orc_kivi_dequant_all.argtypes = [vp, vp]
         _lib = L
     return _lib
 
@@ -426,3 +439,94 @@ def q4_0_legacy_to_gguf(blocks: np.ndarray) -> np.ndarray:
             msb = ((second[i // 2] & 0x0F) << 4) if i % 2 == 0 else (second[i // 2] & 0xF0)
             nibbles[i] = msb | lsb
     return out.reshape(blocks.shape)
+
+
+# ---- KIVI-style affine KV quantisation (kv_quant.rs, quant_dyn_kv_cache.rs) --------------------------
+KIVI_PER_TOKEN, KIVI_BLOCK_CHANNEL, KIVI_RUNNING_CHANNEL = 0, 1, 2
+KIVI_SINK_TOKENS, KIVI_KEY_BLOCK = 4, 32   # quant_dyn_kv_cache.rs:92, :153
+
+
+def kivi_quant_dequant(x: np.ndarray, bits: int, by_row: bool) -> np.ndarray:
+    """quant_dequant (kv_quant.rs:73-98) of a [rows, cols] f32 matrix."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    lib().orc_kivi_quant_dequant(_p(x), x.shape[0], x.shape[1], bits, int(by_row), _p(out))
+    return out
+
+
+class KiviStore:
+    """One head's store: PerTokenStore / BlockChannelStore (quant_dyn_kv_cache.rs:97-250, sink_tokens=4) or
+    QuantValueCache / QuantKeyCache (kv_quant.rs:121-236: KIVI_PER_TOKEN / KIVI_RUNNING_CHANNEL, 8 bits, no sinks)."""
+
+    def __init__(self, layout: int, d: int, bits: int = 8, sink_tokens: int = KIVI_SINK_TOKENS, _h=None):
+        self.layout, self.d, self.bits, self.sink_tokens = layout, d, bits, sink_tokens
+        self._h = _h if _h is not None else lib().orc_kivi_new(layout, d, bits, sink_tokens)
+
+    def push_token(self, row: np.ndarray) -> None:
+        row = np.ascontiguousarray(row, dtype=np.float32)
+        assert row.shape == (self.d,)
+        lib().orc_kivi_push(self._h, _p(row))
+
+    def clone(self) -> "KiviStore":
+        return KiviStore(self.layout, self.d, self.bits, self.sink_tokens, _h=lib().orc_kivi_clone(self._h))
+
+    def len(self) -> int:
+        return lib().orc_kivi_len(self._h)
+
+    def memory_bytes(self) -> int:
+        return lib().orc_kivi_memory_bytes(self._h)
+
+    def dequant_all(self) -> np.ndarray:
+        out = np.empty((self.len(), self.d), np.float32)
+        lib().orc_kivi_dequant_all(self._h, _p(out))
+        return out
+
+    def state(self) -> dict:
+        """Raw state: sink [n_sink, d] f32, packed [n_rows, row_bytes] u8, lo / scale f32, residual [n_res, d] f32."""
+        L = lib()
+        ns, nr, nres, npar, rb = (getattr(L, "orc_kivi_" + n)(self._h) for n in ("n_sink", "n_rows", "n_res", "n_params", "row_bytes"))
+        st = {"sink": np.empty((ns, self.d), np.float32), "packed": np.empty((nr, rb), np.uint8),
+              "lo": np.empty(npar, np.float32), "scale": np.empty(npar, np.float32),
+              "residual": np.empty((nres, self.d), np.float32)}
+        L.orc_kivi_state(self._h, _p(st["sink"]), _p(st["packed"]), _p(st["lo"]), _p(st["scale"]), _p(st["residual"]))
+        return st
+
+    def __del__(self):
+        if self._h is not None and _lib is not None:
+            _lib.orc_kivi_free(self._h)
+            self._h = None
+
+
+class KiviCache:
+    """QuantizedDynKvCacheState (quant_dyn_kv_cache.rs:334-449): one store per (batch, head) of a
+    [B, H, S, D] tensor, Keys block x channel (per_channel) or Values per token; `running` selects the
+    stores of QuantizedKvSdpaState (kv_quant.rs:270-330: no sink tokens, 8 bits, Keys with running scales)."""
+
+    def __init__(self, per_channel: bool, bits: int = 8, running: bool = False):
+        self.per_channel, self.bits, self.running = per_channel, bits, running
+        self.stores: list[KiviStore] = []
+        self.lead = None
+        self.length = 0
+
+    def ingest(self, x: np.ndarray) -> None:
+        x = np.ascontiguousarray(x).astype(np.float32)
+        b, h, s, d = x.shape
+        if not self.stores:
+            self.lead = (b, h)
+            layout = (KIVI_RUNNING_CHANNEL if self.running else KIVI_BLOCK_CHANNEL) if self.per_channel else KIVI_PER_TOKEN
+            self.stores = [KiviStore(layout, d, 8 if self.running else self.bits, 0 if self.running else KIVI_SINK_TOKENS)
+                           for _ in range(b * h)]
+        assert self.lead == (b, h), "cache shape changed between steps"
+        for bi in range(b):
+            for hi in range(h):
+                for t in range(s):
+                    self.stores[bi * h + hi].push_token(x[bi, hi, t])
+        self.length += s
+
+    def dequantized(self) -> np.ndarray:
+        b, h = self.lead
+        return np.stack([st.dequant_all() for st in self.stores]).reshape(b, h, self.length, -1)
+
+    def state(self) -> dict:
+        sts = [st.state() for st in self.stores]
+        return {k: np.stack([s[k] for s in sts]) for k in sts[0]}

@@ -1,0 +1,220 @@
+"""KIVI-style quantised caches on the GPU against the oracle (oracle/kivi_oracle.c): stored codes, parameters,
+sink and partial-block rows and the dequantised cache bit-exact; the fused QuantizedKvSdpa within the path's
+attention tolerance (1e-3 in f32, 2e-2 in f16).  The reference's own unit tests are replayed on the device ops."""
+import numpy as np
+import pytest
+
+import tract_amd
+from tract_amd import kivi
+from oracle import oracle as orc
+from tests.gpu_util import max_abs, rt  # noqa: F401
+from tests.test_oracle_kivi import close_enough_super, lcg, take
+
+pytestmark = pytest.mark.gpu
+
+
+def same_state(gpu: dict, cpu: dict, where=""):
+    for key in ("sink", "packed", "residual"):
+        assert gpu[key].shape == cpu[key].shape, (where, key, gpu[key].shape, cpu[key].shape)
+        assert gpu[key].tobytes() == cpu[key].tobytes(), (where, key)
+    for key in ("lo", "scale"):
+        # numerically equal (a zero `lo` may differ in sign: the CPU op leaves min(+0, -0) to the platform)
+        g, c = gpu[key].reshape(-1), cpu[key].reshape(-1)
+        assert g.shape == c.shape, (where, key)
+        assert np.array_equal(g, c, equal_nan=True), (where, key)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_quantized_dyn_kv_cache_state_and_output_equal_the_oracle(rt, dt, bits, per_channel):
+    rng = np.random.default_rng(bits + 10 * per_channel)
+    B, H, D = 2, 3, 64
+    op = tract_amd.QuantizedDynKeyValueCache("kv0", 2, bits, per_channel)
+    st = op.state()
+    ref = orc.KiviCache(per_channel, bits)
+    outliers = rng.choice([1.0, 1.0, 1.0, 20.0], D)
+    for step, n in enumerate([1, 2, 3, 1, 30, 1, 1, 64, 5, 100, 1, 27, 32, 1]):
+        x = (rng.standard_normal((B, H, n, D)) * outliers).astype(dt)
+        out = st.eval(x).to_numpy()
+        ref.ingest(x)
+        want = ref.dequantized().astype(dt)            # cast_to_dt(input_dt): round to nearest even
+        assert out.shape == want.shape and out.dtype == dt
+        assert out.tobytes() == want.tobytes(), f"step {step}"
+        same_state(st.cache.state(), ref.state(), f"step {step}")
+        assert st.resolve_symbols() == ref.length
+    c = st.cache.counts()
+    assert c["n_sink"] == 4 and c["row_bytes"] == D * bits // 8
+    if per_channel:
+        assert c["n_rows"] == (ref.length - 4) // 32 * 32 and c["n_res"] == (ref.length - 4) % 32
+
+
+@pytest.mark.parametrize("D", [8, 16, 3, 130])
+def test_odd_head_sizes_and_tiny_caches(rt, D):
+    rng = np.random.default_rng(D)
+    for per_channel in (False, True):
+        for bits in (4, 8):
+            st = tract_amd.QuantizedDynKeyValueCache("c", 2, bits, per_channel).state()
+            ref = orc.KiviCache(per_channel, bits)
+            for n in (1, 1, 1, 1, 1, 31, 1, 40):
+                x = rng.standard_normal((1, 2, n, D)).astype(np.float32)
+                out = st.eval(x).to_numpy()
+                ref.ingest(x)
+                assert out.tobytes() == ref.dequantized().tobytes()
+            same_state(st.cache.state(), ref.state(), f"D={D} bits={bits} per_channel={per_channel}")
+
+
+def test_nan_inf_and_constant_rows(rt):
+    D = 32
+    x = np.random.default_rng(0).standard_normal((1, 1, 4 + 64, D)).astype(np.float32)
+    x[0, 0, 5, 3] = np.nan
+    x[0, 0, 6, :] = np.nan
+    x[0, 0, 7, 2] = np.inf
+    x[0, 0, 8, 9] = -np.inf
+    x[0, 0, 9, :] = 2.5
+    x[0, 0, 40, 1] = np.nan
+    x[0, 0, 41, 2] = np.inf
+    for per_channel in (False, True):
+        for bits in (4, 8):
+            st = tract_amd.QuantizedDynKeyValueCache("c", 2, bits, per_channel).state()
+            ref = orc.KiviCache(per_channel, bits)
+            out = st.eval(x).to_numpy()
+            ref.ingest(x)
+            assert out.tobytes() == ref.dequantized().tobytes(), (per_channel, bits)
+            same_state(st.cache.state(), ref.state())
+
+
+def test_load_from_save_to_freeze(rt):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((1, 2, 50, 16)).astype(np.float32)
+    st = tract_amd.QuantizedDynKeyValueCache("c", 2, 8, True).state()
+    st.load_from([x])                                    # quant_dyn_kv_cache.rs:455-465
+    assert st.resolve_symbols() == 50
+    saved = []
+    st.save_to(saved)                                    # :467-470: the dequantised cache
+    ref = orc.KiviCache(True, 8)
+    ref.ingest(x)
+    assert saved[0].tobytes() == ref.dequantized().tobytes()
+    frozen = st.freeze()                                 # :510-541
+    y = rng.standard_normal((1, 2, 20, 16)).astype(np.float32)
+    a = st.eval(y).to_numpy()
+    assert frozen.resolve_symbols() == 50                # the copy did not move
+    b = frozen.unfreeze().eval(y).to_numpy()
+    ref.ingest(y)
+    assert a.tobytes() == b.tobytes() == ref.dequantized().tobytes()
+    with pytest.raises(tract_amd.TractRocmError, match="cache shape changed between steps"):
+        st.eval(np.zeros((1, 3, 1, 16), np.float32))
+    with pytest.raises(tract_amd.TractRocmError, match="rank-4"):
+        tract_amd.QuantizedDynKeyValueCache("c", 2, 8, True).state().eval(np.zeros((2, 1, 16), np.float32))
+    with pytest.raises(tract_amd.TractRocmError, match="bits must be 4 or 8"):
+        tract_amd.QuantizedDynKeyValueCache("c", 2, 3, True)
+
+
+# ---- the reference's unit tests on the device ops -----------------------------------------------------------------
+def test_ref_quant_dequant_cases(rt):
+    x = np.array([[0, 1, 2, 3], [-1, 0.5, 4, 9], [2, 2, 2, 2.1]], np.float32)       # kv_quant.rs:454-478
+    for bits in (4, 8):
+        for by_row in (False, True):
+            assert kivi.quant_dequant(x, bits, by_row).tobytes() == orc.kivi_quant_dequant(x, bits, by_row).tobytes()
+    e4 = np.abs(x - kivi.quant_dequant(x, 4, False)).max()
+    e8 = np.abs(x - kivi.quant_dequant(x, 8, False)).max()
+    assert e8 < e4
+    x = np.array([[100, 0.10, -0.20, 0.05], [-90, 0.02, 0.30, -0.08], [120, -0.15, 0.10, 0.20],    # :483-505
+                  [-110, 0.07, -0.05, 0.12]], np.float32)
+    pc = np.abs(x - kivi.quant_dequant(x, 4, False))[:, 1:].max()
+    pt = np.abs(x - kivi.quant_dequant(x, 4, True))[:, 1:].max()
+    assert pc < pt * 0.2
+
+
+def test_ref_quant_cache_accumulates_near_lossless_int8(rt):   # quant_dyn_kv_cache.rs:728-756
+    for per_channel in (False, True):
+        gen = lcg(3)
+        st = tract_amd.QuantizedDynKeyValueCache("kv0", 2, 8, per_channel).state()
+        acc = None
+        for _ in range(40):
+            step = take(gen, 1, 2, 1, 8)
+            out = st.eval(step).to_numpy()
+            acc = step if acc is None else np.concatenate([acc, step], axis=2)
+            assert out.shape == acc.shape and close_enough_super(out, acc)
+
+
+def test_ref_block_per_channel_key_consistent_over_growing_range(rt):   # quant_dyn_kv_cache.rs:758-778
+    d = 16
+    rows = np.array([[t * 2.0 if c == 0 else np.sin(np.float32((t * 7 + c) * 0.013)) * 0.1 for c in range(d)]
+                     for t in range(80)], np.float32)
+    st = tract_amd.QuantizedDynKeyValueCache("k", 2, 8, True).state()
+    for r in rows:
+        out = st.eval(r.reshape(1, 1, 1, d))
+    assert st.resolve_symbols() == 80
+    assert np.abs(out.to_numpy()[0, 0] - rows).max() < 1.0
+
+
+def test_ref_quantized_kv_sdpa_runs_in_model(rt):              # kv_quant.rs:568-650
+    b, h, d = 1, 2, 16
+    st = tract_amd.QuantizedKvSdpa(axis=2, scale=None).state()
+    kc, vc = orc.KiviCache(True, running=True), orc.KiviCache(False, running=True)
+    kf = vf = None
+
+    def mk(base):
+        return (np.float32(base) + np.sin(np.arange(b * h * d, dtype=np.float32) * np.float32(0.013))).astype(np.float32).reshape(b, h, 1, d)
+
+    for t in range(10):
+        qi, ki, vi = mk(9.0 + t * 0.1), mk(1.0 + t * 0.07), mk(5.0 - t * 0.05)
+        got = st.eval([qi, ki, vi]).to_numpy()
+        kf = ki if kf is None else np.concatenate([kf, ki], axis=2)
+        vf = vi if vf is None else np.concatenate([vf, vi], axis=2)
+        want = orc.naive_sdpa_f64(qi, kf, vf, causal=False).astype(np.float32)
+        assert close_enough_super(got, want), t
+        kc.ingest(ki)
+        vc.ingest(vi)
+        assert max_abs(got, orc.flash_sdpa(qi, kc.dequantized(), vc.dequantized(), causal=False)) <= 1e-3
+    same_state(st.k.state(), kc.state(), "K")
+    same_state(st.v.state(), vc.state(), "V")
+    assert st.k.memory_bytes() == b * h * (10 * d + d * 8) and st.v.memory_bytes() == b * h * (10 * d + 10 * 8)
+
+
+@pytest.mark.parametrize("dt,tol", [(np.float32, 1e-3), (np.float16, 2e-2)])
+def test_quantized_kv_sdpa_gqa_prefill_then_decode(rt, dt, tol):
+    rng = np.random.default_rng(11)
+    B, Hq, Hkv, D = 2, 8, 2, 128
+    st = tract_amd.QuantizedKvSdpa(axis=2, scale=0.11).state()
+    kc, vc = orc.KiviCache(True, running=True), orc.KiviCache(False, running=True)
+    chan = rng.choice([1.0, 1.0, 1.0, 20.0], D)
+    for n in (37, 1, 1, 8, 1, 200, 1):
+        q = (rng.standard_normal((B, Hq, n, D)) / np.sqrt(D)).astype(dt)
+        k = (rng.standard_normal((B, Hkv, n, D)) * chan).astype(dt)
+        v = rng.standard_normal((B, Hkv, n, D)).astype(dt)
+        got = st.eval([q, k, v]).to_numpy()
+        kc.ingest(k)
+        vc.ingest(v)
+        want = orc.flash_sdpa(q.astype(np.float32), kc.dequantized(), vc.dequantized(), causal=False, scale=0.11)   # kv_quant.rs:326
+        assert got.dtype == dt and max_abs(got, want) <= tol, n
+    same_state(st.k.state(), kc.state(), "K")
+    same_state(st.v.state(), vc.state(), "V")
+    frozen = st.freeze()
+    q = (rng.standard_normal((B, Hq, 1, D)) / np.sqrt(D)).astype(dt)
+    k = rng.standard_normal((B, Hkv, 1, D)).astype(dt)
+    assert st.eval([q, k, k]).to_numpy().tobytes() == frozen.eval([q, k, k]).to_numpy().tobytes()
+
+
+def test_cache_of_the_decode_layer_shape(rt):
+    """32q/8kv, d=128 at batch 8: a 2048-token prefill and decode steps; sampled heads against the oracle."""
+    rng = np.random.default_rng(2)
+    B, H, D, T = 8, 8, 128, 2048
+    x = rng.standard_normal((B, H, T, D)).astype(np.float16)
+    x[:, :, :, 5] *= 20
+    for per_channel in (False, True):
+        st = tract_amd.QuantizedDynKeyValueCache("kv", 2, 8, per_channel).state()
+        out = st.eval(x).to_numpy()
+        steps = [rng.standard_normal((B, H, 1, D)).astype(np.float16) for _ in range(3)]
+        for s in steps:
+            out = st.eval(s).to_numpy()
+        assert out.shape == (B, H, T + 3, D)
+        state = st.cache.state()
+        for (b, h) in ((0, 0), (3, 5), (7, 7)):
+            ref = orc.KiviCache(per_channel, 8)
+            ref.ingest(x[b:b + 1, h:h + 1])
+            for s in steps:
+                ref.ingest(s[b:b + 1, h:h + 1])
+            assert out[b, h].tobytes() == ref.dequantized()[0, 0].astype(np.float16).tobytes()
+            same_state({k: v[b * H + h:b * H + h + 1] for k, v in state.items()}, ref.state(), f"head {b},{h}")

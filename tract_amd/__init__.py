@@ -12,3 +12,5 @@ from .runtime import (DeviceTensor, Event, RocmRuntime, Stream, Workspace, runti
 from .ops import (ApplyRope, BlockQuant, Cast, GgmlGemm, Q40Weights, RotateHalf, DynKeyValueCache, DynKeyValueCacheState, InPlaceKvCache, KvPool,  # noqa: F401
                   InPlaceKvSdpa, InPlaceKvSdpaState, Sdpa, StreamedSdpaOp, WindowKvCache, WindowKvSdpa, WindowKvSdpaState, Q4_0_FORMAT, Q8_0_FORMAT, inplace_kv_sdpa_eval_ragged,
                   sdpa_decode_ragged)
+from .kivi import (KiviCache, QuantizedDynKeyValueCache, QuantizedDynKvCacheState, QuantizedKvSdpa,  # noqa: F401
+                   QuantizedKvSdpaState, KIVI_BLOCK_CHANNEL, KIVI_PER_TOKEN, KIVI_RUNNING_CHANNEL)

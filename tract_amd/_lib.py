@@ -88,6 +88,16 @@ SIGNATURES = {
     "trocm_inplace_kv_sdpa_eval": [_vp, _vp, _vp, _i, _i64, _i64, _pi64, _vp, _vp, _vp, _f, _i, _vp, _sz, _vp],
     "trocm_inplace_kv_sdpa_eval_ragged": [_vp, _vp, _vp, _i, _i64, _i64, C.POINTER(_vp), C.POINTER(_vp), _vp, _f, _vp,
                                           _sz, _vp],
+    "trocm_kivi_cache_create": [C.POINTER(_vp), _i, _i, _i64, _i64, _i64, _i64],
+    "trocm_kivi_cache_destroy": [_vp],
+    "trocm_kivi_cache_len": [_vp, _pi64],
+    "trocm_kivi_cache_counts": [_vp, _pi64, _pi64, _pi64, _pi64],
+    "trocm_kivi_cache_memory_bytes": [_vp, C.POINTER(_sz)],
+    "trocm_kivi_cache_append": [_vp, _vp, _i, _i64, _vp],
+    "trocm_kivi_cache_dequantize": [_vp, _vp, _i, _vp],
+    "trocm_kivi_cache_export": [_vp, _i, _vp, C.POINTER(_sz), _vp],
+    "trocm_kivi_cache_clone": [_vp, C.POINTER(_vp), _vp],
+    "trocm_quantized_kv_sdpa_eval": [_vp, _vp, _vp, _i, _i64, _i64, _vp, _vp, _vp, _f, _vp, _sz, _vp],
     "trocm_sdpa_decode_ragged": [_vp, _i, _i64, _i64, C.POINTER(_vp), C.POINTER(_vp), _vp, _f, _vp, _sz, _vp],
 }
 _RESTYPES = {"trocm_last_error": C.c_char_p}

@@ -1,0 +1,607 @@
+// KIVI-style affine KV-cache quantisation: tract's storage-quantised cache op and its fused variant.
+//
+//   QuantizedDynKeyValueCache  transformers/src/ops/quant_dyn_kv_cache.rs:92-250, :334-495
+//       Values per token (PerTokenStore), Keys per channel in frozen blocks of 32 tokens
+//       (BlockChannelStore), the first 4 "sink" tokens and the partial key block kept in f32,
+//       4 or 8 bits per code; the op's output is the whole cache dequantised to the input type.
+//   QuantizedKvSdpa            transformers/src/ops/kv_quant.rs:105-236, :242-330
+//       u8 codes, Values per token, Keys per channel with RUNNING lo / scale (old codes are read
+//       back with the current parameters), followed by non-causal attention over the
+//       dequantised cache.
+//
+// The stored bytes and parameters must equal the CPU op's, so every floating-point step is spelled
+// out (this file is compiled with -ffp-contract=off): f32 subtraction, IEEE division, f32::round
+// (half away from zero), clamp, saturating `as u8` with NaN -> 0; `lo + code * scale` with two
+// roundings.  min / max ignore NaN like f32::min / f32::max (v_min_f32 / v_max_f32 in IEEE mode).
+//
+// Device layout, one object per tensor, BH = batch * heads rows of everything:
+//   sink      [BH, sink_tokens, D] f32
+//   codes     [BH, cap_rows, row_bytes] u8, row_bytes = ceil(D * bits / 8) (4 bits: even index -> low nibble)
+//   lo, scale per token [BH, cap_rows] / per block and channel [BH, cap_rows / 32, D] / per channel [BH, D]
+//   residual  [BH, 32, D] f32 (block layout: the partial block)
+// cap_rows doubles (multiples of 32).  All of it is HBM-bound byte work: a token costs its own bytes on
+// append, the dequantising read costs row_bytes + 2 or 4 bytes per element.
+#include <hip/hip_fp16.h>
+#include <new>
+#include "common.h"
+
+namespace trocm {
+namespace {
+
+constexpr int kKeyBlock = 32;   // quant_dyn_kv_cache.rs:153
+
+__device__ __forceinline__ float ld(const float *p) { return *p; }
+__device__ __forceinline__ float ld(const __half *p) { return __half2float(*p); }
+
+// f32 -> f16 as its own instruction: without the barrier the compiler may fold the preceding multiply and add
+// into one mixed-precision fma, which rounds once where the CPU op rounds three times.
+__device__ __forceinline__ void st(float *p, float x) { *p = x; }
+__device__ __forceinline__ void st(__half *p, float x) {
+    asm volatile("" : "+v"(x));
+    *p = __float2half_rn(x);
+}
+
+// f32::round(): half away from zero.  Values of magnitude >= 2^23 (and inf, NaN) are their own rounding;
+// below that d = x - trunc(x) is exact, so is d + d, whose truncation is the unit to add.
+__device__ __forceinline__ float round_half_away(float x) {
+    if (!(fabsf(x) < 8388608.0f)) return x;
+    const float t = truncf(x);
+    const float d = __fsub_rn(x, t);
+    return __fadd_rn(t, truncf(__fadd_rn(d, d)));
+}
+
+// ((x - lo) / scale).round().clamp(0.0, lv) as u8   (quant_dyn_kv_cache.rs:128, :190; kv_quant.rs:110, :219)
+__device__ __forceinline__ uint32_t affine_code(float x, float lo, float scale, float lv) {
+    float q = round_half_away(__fdiv_rn(__fsub_rn(x, lo), scale));
+    if (!(q == q)) return 0;            // clamp keeps NaN, the cast turns it into 0
+    q = q < 0.0f ? 0.0f : (q > lv ? lv : q);
+    return (uint32_t)q;
+}
+__device__ __forceinline__ float affine_scale(float lo, float hi, float lv) {   // :127, :186
+    return hi > lo ? __fdiv_rn(__fsub_rn(hi, lo), lv) : 1.0f;
+}
+
+// dst[bh][dst_t0 + i][c] = (f32) src[bh][src_t0 + i][c], i < n: sink tokens and the partial key block.
+template <typename SrcT>
+__global__ void kivi_rows_to_f32_kernel(const SrcT *__restrict__ src, int64_t S, int64_t src_t0, float *__restrict__ dst,
+                                        int64_t dst_pitch, int64_t dst_t0, int n, int D) {
+    const int bh = blockIdx.y;
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n * D) return;
+    const int i = e / D, c = e - i * D;
+    dst[((int64_t)bh * dst_pitch + dst_t0 + i) * D + c] = ld(src + ((int64_t)bh * S + src_t0 + i) * D + c);
+}
+
+// Values, one wave per (head row, token): lo / hi over the token's D channels, then its codes (PerTokenStore::push_token).
+template <typename SrcT, int BITS>
+__global__ void __launch_bounds__(256) kivi_quant_tokens_kernel(const SrcT *__restrict__ src, int64_t S, int64_t src_t0, int n, int D,
+                                                                uint8_t *__restrict__ codes, int64_t cap_rows, int row_bytes,
+                                                                int64_t row0, float *__restrict__ lo_out, float *__restrict__ scale_out) {
+    const int bh = blockIdx.y;
+    const int i = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (i >= n) return;
+    const SrcT *row = src + ((int64_t)bh * S + src_t0 + i) * D;
+    float lo = INFINITY, hi = -INFINITY;
+    for (int c = lane; c < D; c += 64) {
+        const float v = ld(row + c);
+        lo = fminf(lo, v);
+        hi = fmaxf(hi, v);
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        lo = fminf(lo, __shfl_xor(lo, m, 64));
+        hi = fmaxf(hi, __shfl_xor(hi, m, 64));
+    }
+    constexpr float lv = (float)((1u << BITS) - 1u);
+    const float scale = affine_scale(lo, hi, lv);
+    uint8_t *out = codes + ((int64_t)bh * cap_rows + row0 + i) * row_bytes;
+    for (int u = lane; u < row_bytes; u += 64) {
+        uint32_t byte;
+        if (BITS == 8) {
+            byte = affine_code(ld(row + u), lo, scale, lv);
+        } else {
+            const int c0 = 2 * u, c1 = 2 * u + 1;
+            byte = affine_code(ld(row + c0), lo, scale, lv) & 15u;
+            if (c1 < D) byte |= (affine_code(ld(row + c1), lo, scale, lv) & 15u) << 4;
+        }
+        out[u] = (uint8_t)byte;
+    }
+    if (lane == 0) {
+        lo_out[(int64_t)bh * cap_rows + row0 + i] = lo;
+        scale_out[(int64_t)bh * cap_rows + row0 + i] = scale;
+    }
+}
+
+// Keys, one workgroup per (block that becomes full, head row), a thread per byte column of the rows: lo / hi of its
+// channel(s) over the block's 32 tokens, the frozen parameters, then the 32 codes (BlockChannelStore::finalize_block).
+// Row k of the run of blocks comes from the partial block when k < n_res_old, else from the new tokens.
+template <typename SrcT, int BITS>
+__global__ void __launch_bounds__(256) kivi_finalize_blocks_kernel(const SrcT *__restrict__ src, int64_t S, int64_t src_t0,
+                                                                   const float *__restrict__ residual, int n_res_old, int D,
+                                                                   uint8_t *__restrict__ codes, int64_t cap_rows, int row_bytes,
+                                                                   int64_t row0, float *__restrict__ lo_out, float *__restrict__ scale_out) {
+    const int j = blockIdx.x, bh = blockIdx.y;
+    constexpr float lv = (float)((1u << BITS) - 1u);
+    constexpr int CH = BITS == 8 ? 1 : 2;
+    const int64_t blk = row0 / kKeyBlock + j;
+    const float *res = residual + (int64_t)bh * kKeyBlock * D;
+    const SrcT *fresh = src + ((int64_t)bh * S + src_t0 - n_res_old) * D;   // row k >= n_res_old of the run sits at fresh + k * D
+    for (int u = threadIdx.x; u < row_bytes; u += blockDim.x) {
+        float lo[CH], scale[CH];
+#pragma unroll
+        for (int h = 0; h < CH; h++) {
+            const int c = CH * u + h;
+            float l = INFINITY, hi = -INFINITY;
+            if (c < D) {
+#pragma unroll 1
+                for (int r = 0; r < kKeyBlock; r++) {
+                    const int k = j * kKeyBlock + r;
+                    const float x = k < n_res_old ? res[(int64_t)k * D + c] : ld(fresh + (int64_t)k * D + c);
+                    l = fminf(l, x);
+                    hi = fmaxf(hi, x);
+                }
+                const int64_t at = ((int64_t)bh * (cap_rows / kKeyBlock) + blk) * D + c;
+                lo_out[at] = l;
+                scale_out[at] = affine_scale(l, hi, lv);
+            }
+            lo[h] = l;
+            scale[h] = affine_scale(l, hi, lv);
+        }
+        // second pass over the block's rows (they are in the cache now): the codes
+#pragma unroll 1
+        for (int r = 0; r < kKeyBlock; r++) {
+            const int k = j * kKeyBlock + r;
+            uint32_t byte = 0;
+#pragma unroll
+            for (int h = 0; h < CH; h++) {
+                const int c = CH * u + h;
+                if (c < D) {
+                    const float x = k < n_res_old ? res[(int64_t)k * D + c] : ld(fresh + (int64_t)k * D + c);
+                    const uint32_t code = affine_code(x, lo[h], scale[h], lv);
+                    byte |= CH == 1 ? code : (code & 15u) << (4 * h);
+                }
+            }
+            codes[((int64_t)bh * cap_rows + row0 + k) * row_bytes + u] = (uint8_t)byte;
+        }
+    }
+}
+
+// Keys with running parameters, a thread per (head row, channel), tokens in order (QuantKeyCache::push_token):
+// lo follows the minimum, scale only grows, each token is coded under the parameters current at its push.
+template <typename SrcT>
+__global__ void kivi_running_push_kernel(const SrcT *__restrict__ src, int64_t S, int n, int D, uint8_t *__restrict__ codes,
+                                         int64_t cap_rows, int64_t row0, float *__restrict__ lo_io, float *__restrict__ scale_io) {
+    const int bh = blockIdx.y;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= D) return;
+    float lo = lo_io[(int64_t)bh * D + c], scale = scale_io[(int64_t)bh * D + c];
+    for (int t = 0; t < n; t++) {
+        const float val = ld(src + ((int64_t)bh * S + t) * D + c);
+        if (val < lo) lo = val;
+        const float range = __fsub_rn(val, lo);
+        if (range > 0.0f) {
+            const float ns = __fdiv_rn(range, 255.0f);
+            if (ns > scale) scale = ns;
+        }
+        codes[((int64_t)bh * cap_rows + row0 + t) * D + c] = (uint8_t)affine_code(val, lo, scale, 255.0f);
+    }
+    lo_io[(int64_t)bh * D + c] = lo;
+    scale_io[(int64_t)bh * D + c] = scale;
+}
+
+struct KiviView {
+    int layout, D, row_bytes, len, n_sink, n_rows;
+    int64_t sink_tokens, cap_rows;
+    const float *sink, *residual, *lo, *scale;
+    const uint8_t *codes;
+};
+
+// dequant_all (quant_dyn_kv_cache.rs:132-150, :200-229; kv_quant.rs:148-159, :224-234): dst [BH, len, D] dense.
+template <typename DstT, int BITS>
+__global__ void kivi_dequant_kernel(KiviView a, DstT *__restrict__ dst) {
+    const int bh = blockIdx.y;
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= a.len * a.D) return;
+    const int t = e / a.D, c = e - t * a.D;
+    float x;
+    if (t < a.n_sink) {
+        x = a.sink[((int64_t)bh * a.sink_tokens + t) * a.D + c];
+    } else if (t - a.n_sink < a.n_rows) {
+        const int r = t - a.n_sink;
+        const uint8_t *row = a.codes + ((int64_t)bh * a.cap_rows + r) * a.row_bytes;
+        uint32_t code;
+        if (BITS == 8) {
+            code = row[c];
+        } else {
+            const uint32_t b = row[c >> 1];
+            code = (c & 1) ? (b >> 4) : (b & 15u);
+        }
+        int64_t p;
+        if (a.layout == TROCM_KIVI_PER_TOKEN) p = (int64_t)bh * a.cap_rows + r;
+        else if (a.layout == TROCM_KIVI_BLOCK_CHANNEL) p = ((int64_t)bh * (a.cap_rows / kKeyBlock) + r / kKeyBlock) * a.D + c;
+        else p = (int64_t)bh * a.D + c;
+        x = __fadd_rn(a.lo[p], __fmul_rn((float)code, a.scale[p]));
+    } else {
+        x = a.residual[((int64_t)bh * kKeyBlock + (t - a.n_sink - a.n_rows)) * a.D + c];
+    }
+    st(dst + ((int64_t)bh * a.len + t) * a.D + c, x);
+}
+
+__global__ void kivi_fill_running_kernel(float *lo, float *scale, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        lo[i] = INFINITY;    // kv_quant.rs:187-188
+        scale[i] = 1.0f;
+    }
+}
+
+}  // namespace
+}  // namespace trocm
+
+using namespace trocm;
+
+struct trocm_kivi_cache {
+    int layout = 0, bits = 8;
+    int64_t sink_tokens = 0, B = 0, H = 0, D = 0, BH = 0, row_bytes = 0;
+    int64_t len = 0, n_sink = 0, n_rows = 0, n_res = 0, cap_rows = 0;
+    float *sink = nullptr, *residual = nullptr, *lo = nullptr, *scale = nullptr;
+    uint8_t *codes = nullptr;
+    void *deq = nullptr;      // dequantised copy handed to attention by trocm_quantized_kv_sdpa_eval
+    size_t deq_bytes = 0;
+};
+
+static int64_t param_pitch(const trocm_kivi_cache *c, int64_t cap_rows) {
+    switch (c->layout) {
+        case TROCM_KIVI_PER_TOKEN: return cap_rows;
+        case TROCM_KIVI_BLOCK_CHANNEL: return cap_rows / kKeyBlock * c->D;
+        default: return c->D;
+    }
+}
+static int64_t n_params(const trocm_kivi_cache *c) {
+    switch (c->layout) {
+        case TROCM_KIVI_PER_TOKEN: return c->n_rows;
+        case TROCM_KIVI_BLOCK_CHANNEL: return c->n_rows / kKeyBlock * c->D;
+        default: return c->D;
+    }
+}
+
+// [BH rows of width_bytes] between two pitched planes.
+static int copy_rows(void *dst, int64_t dpitch, const void *src, int64_t spitch, int64_t width, int64_t rows, hipStream_t s) {
+    if (width == 0 || rows == 0) return 0;
+    CopyNd d;
+    d.rank = 2;
+    d.shape[0] = rows;
+    d.shape[1] = width;
+    d.dst_stride[0] = dpitch;
+    d.dst_stride[1] = 1;
+    d.src_stride[0] = spitch;
+    d.src_stride[1] = 1;
+    return launch_copy_nd(dst, src, d, 1, s);
+}
+
+static int kivi_alloc_fixed(trocm_kivi_cache *c, hipStream_t s) {
+    if (c->sink_tokens && !c->sink) TROCM_HIP(hipMalloc((void **)&c->sink, (size_t)c->BH * c->sink_tokens * c->D * 4));
+    if (c->layout == TROCM_KIVI_BLOCK_CHANNEL && !c->residual)
+        TROCM_HIP(hipMalloc((void **)&c->residual, (size_t)c->BH * kKeyBlock * c->D * 4));
+    if (c->layout == TROCM_KIVI_RUNNING_CHANNEL && !c->lo) {
+        const int64_t n = c->BH * c->D;
+        TROCM_HIP(hipMalloc((void **)&c->lo, (size_t)n * 4));
+        TROCM_HIP(hipMalloc((void **)&c->scale, (size_t)n * 4));
+        kivi_fill_running_kernel<<<dim3((unsigned)((n + 255) / 256)), 256, 0, s>>>(c->lo, c->scale, n);
+        TROCM_HIP(hipGetLastError());
+    }
+    return 0;
+}
+
+// Room for `need` coded rows: capacities are multiples of 32 and at least double.  The valid region moves on the
+// stream; the old planes are freed after the stream has drained (the CPU op is synchronous as well).
+static int kivi_ensure_rows(trocm_kivi_cache *c, int64_t need, hipStream_t s) {
+    if (need <= c->cap_rows) return 0;
+    int64_t cap = c->cap_rows * 2 > need ? c->cap_rows * 2 : need;
+    cap = (cap + kKeyBlock - 1) / kKeyBlock * kKeyBlock;
+    uint8_t *codes = nullptr;
+    float *lo = nullptr, *scale = nullptr;
+    TROCM_HIP(hipMalloc((void **)&codes, (size_t)c->BH * cap * c->row_bytes));
+    const bool own_params = c->layout != TROCM_KIVI_RUNNING_CHANNEL;
+    if (own_params) {
+        if (hipMalloc((void **)&lo, (size_t)c->BH * param_pitch(c, cap) * 4) != hipSuccess ||
+            hipMalloc((void **)&scale, (size_t)c->BH * param_pitch(c, cap) * 4) != hipSuccess) {
+            (void)hipFree(codes);
+            if (lo) (void)hipFree(lo);
+            return fail("hipMalloc failed for the parameters of a quantised cache of %lld rows", (long long)cap);
+        }
+    }
+    int rc = 0;
+    if (c->n_rows) {
+        rc = copy_rows(codes, cap * c->row_bytes, c->codes, c->cap_rows * c->row_bytes, c->n_rows * c->row_bytes, c->BH, s);
+        if (!rc && own_params) {
+            rc = copy_rows(lo, param_pitch(c, cap) * 4, c->lo, param_pitch(c, c->cap_rows) * 4, n_params(c) * 4, c->BH, s);
+            if (!rc) rc = copy_rows(scale, param_pitch(c, cap) * 4, c->scale, param_pitch(c, c->cap_rows) * 4, n_params(c) * 4, c->BH, s);
+        }
+    }
+    if (rc) {
+        (void)hipFree(codes);
+        if (lo) (void)hipFree(lo);
+        if (scale) (void)hipFree(scale);
+        return rc;
+    }
+    if (c->codes) {
+        TROCM_HIP(hipStreamSynchronize(s));
+        (void)hipFree(c->codes);
+        if (own_params) {
+            (void)hipFree(c->lo);
+            (void)hipFree(c->scale);
+        }
+    }
+    c->codes = codes;
+    if (own_params) {
+        c->lo = lo;
+        c->scale = scale;
+    }
+    c->cap_rows = cap;
+    return 0;
+}
+
+template <typename SrcT>
+static int kivi_append_t(trocm_kivi_cache *c, const SrcT *src, int64_t S, hipStream_t s) {
+    const int D = (int)c->D;
+    const unsigned BH = (unsigned)c->BH;
+    if (kivi_alloc_fixed(c, s)) return 1;
+    int64_t t0 = 0;
+    const int64_t ns = c->sink_tokens - c->n_sink < S ? c->sink_tokens - c->n_sink : S;
+    if (ns > 0) {   // quant_dyn_kv_cache.rs:118-122, :170-174
+        kivi_rows_to_f32_kernel<SrcT><<<dim3((unsigned)((ns * D + 255) / 256), BH), 256, 0, s>>>(src, S, 0, c->sink, c->sink_tokens, c->n_sink, (int)ns, D);
+        TROCM_HIP(hipGetLastError());
+        c->n_sink += ns;
+        t0 = ns;
+    }
+    const int64_t rem = S - t0;
+    if (rem > 0 && c->layout == TROCM_KIVI_PER_TOKEN) {
+        if (kivi_ensure_rows(c, c->n_rows + rem, s)) return 1;
+        const dim3 grid((unsigned)((rem + 3) / 4), BH);
+        if (c->bits == 8)
+            kivi_quant_tokens_kernel<SrcT, 8><<<grid, 256, 0, s>>>(src, S, t0, (int)rem, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
+        else
+            kivi_quant_tokens_kernel<SrcT, 4><<<grid, 256, 0, s>>>(src, S, t0, (int)rem, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
+        TROCM_HIP(hipGetLastError());
+        c->n_rows += rem;
+    } else if (rem > 0 && c->layout == TROCM_KIVI_BLOCK_CHANNEL) {
+        const int64_t nb = (c->n_res + rem) / kKeyBlock;
+        if (nb > 0) {
+            if (kivi_ensure_rows(c, c->n_rows + nb * kKeyBlock, s)) return 1;
+            const dim3 grid((unsigned)nb, BH);
+            const int threads = c->row_bytes >= 256 ? 256 : (int)((c->row_bytes + 63) / 64 * 64);
+            if (c->bits == 8)
+                kivi_finalize_blocks_kernel<SrcT, 8><<<grid, threads, 0, s>>>(src, S, t0, c->residual, (int)c->n_res, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
+            else
+                kivi_finalize_blocks_kernel<SrcT, 4><<<grid, threads, 0, s>>>(src, S, t0, c->residual, (int)c->n_res, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
+            TROCM_HIP(hipGetLastError());
+            const int64_t used = nb * kKeyBlock - c->n_res, tail = rem - used;
+            c->n_rows += nb * kKeyBlock;
+            if (tail > 0) {
+                kivi_rows_to_f32_kernel<SrcT><<<dim3((unsigned)((tail * D + 255) / 256), BH), 256, 0, s>>>(src, S, t0 + used, c->residual, kKeyBlock, 0, (int)tail, D);
+                TROCM_HIP(hipGetLastError());
+            }
+            c->n_res = tail;
+        } else {
+            kivi_rows_to_f32_kernel<SrcT><<<dim3((unsigned)((rem * D + 255) / 256), BH), 256, 0, s>>>(src, S, t0, c->residual, kKeyBlock, c->n_res, (int)rem, D);
+            TROCM_HIP(hipGetLastError());
+            c->n_res += rem;
+        }
+    } else if (rem > 0) {
+        if (kivi_ensure_rows(c, c->n_rows + rem, s)) return 1;
+        kivi_running_push_kernel<SrcT><<<dim3((unsigned)((D + 127) / 128), BH), 128, 0, s>>>(src + t0 * D, S, (int)rem, D, c->codes, c->cap_rows, c->n_rows, c->lo, c->scale);
+        TROCM_HIP(hipGetLastError());
+        c->n_rows += rem;
+    }
+    c->len += S;
+    return 0;
+}
+
+static int kivi_dequantize(const trocm_kivi_cache *c, void *dst, int dst_dtype, hipStream_t s) {
+    if (c->len == 0) return 0;
+    KiviView a;
+    a.layout = c->layout;
+    a.D = (int)c->D;
+    a.row_bytes = (int)c->row_bytes;
+    a.len = (int)c->len;
+    a.n_sink = (int)c->n_sink;
+    a.n_rows = (int)c->n_rows;
+    a.sink_tokens = c->sink_tokens;
+    a.cap_rows = c->cap_rows;
+    a.sink = c->sink;
+    a.residual = c->residual;
+    a.lo = c->lo;
+    a.scale = c->scale;
+    a.codes = c->codes;
+    const dim3 grid((unsigned)((c->len * c->D + 255) / 256), (unsigned)c->BH);
+    if (dst_dtype == TROCM_F32) {
+        if (c->bits == 8) kivi_dequant_kernel<float, 8><<<grid, 256, 0, s>>>(a, (float *)dst);
+        else kivi_dequant_kernel<float, 4><<<grid, 256, 0, s>>>(a, (float *)dst);
+    } else {
+        if (c->bits == 8) kivi_dequant_kernel<__half, 8><<<grid, 256, 0, s>>>(a, (__half *)dst);
+        else kivi_dequant_kernel<__half, 4><<<grid, 256, 0, s>>>(a, (__half *)dst);
+    }
+    TROCM_HIP(hipGetLastError());
+    return 0;
+}
+
+extern "C" {
+
+int trocm_kivi_cache_create(trocm_kivi_cache **out, int layout, int bits, int64_t sink_tokens, int64_t batch,
+                            int64_t heads, int64_t head_dim) {
+    TROCM_NOT_NULL(out);
+    if (ensure_init()) return 1;
+    TROCM_REQUIRE(layout == TROCM_KIVI_PER_TOKEN || layout == TROCM_KIVI_BLOCK_CHANNEL || layout == TROCM_KIVI_RUNNING_CHANNEL,
+                  "unknown quantised-cache layout %d", layout);
+    TROCM_REQUIRE(bits == 4 || bits == 8, "KV quantization bits must be 4 or 8");   // quant_dyn_kv_cache.rs:706
+    TROCM_REQUIRE(layout != TROCM_KIVI_RUNNING_CHANNEL || bits == 8, "the running per-channel key store holds 8-bit codes");
+    TROCM_REQUIRE(batch > 0 && heads > 0 && head_dim > 0 && sink_tokens >= 0, "quantised cache: invalid shape");
+    TROCM_REQUIRE(batch * heads <= 65535, "quantised cache: batch * heads = %lld exceeds 65535", (long long)(batch * heads));
+    trocm_kivi_cache *c = new (std::nothrow) trocm_kivi_cache();
+    TROCM_REQUIRE(c, "out of host memory");
+    c->layout = layout;
+    c->bits = bits;
+    c->sink_tokens = sink_tokens;
+    c->B = batch;
+    c->H = heads;
+    c->D = head_dim;
+    c->BH = batch * heads;
+    c->row_bytes = (head_dim * bits + 7) / 8;   // quant_dyn_kv_cache.rs:58-60
+    *out = c;
+    return 0;
+}
+
+int trocm_kivi_cache_destroy(trocm_kivi_cache *c) {
+    if (!c) return 0;
+    (void)hipFree(c->sink);
+    (void)hipFree(c->residual);
+    (void)hipFree(c->lo);
+    (void)hipFree(c->scale);
+    (void)hipFree(c->codes);
+    (void)hipFree(c->deq);
+    delete c;
+    return 0;
+}
+
+int trocm_kivi_cache_len(const trocm_kivi_cache *c, int64_t *len) {
+    TROCM_NOT_NULL(c);
+    TROCM_NOT_NULL(len);
+    *len = c->len;
+    return 0;
+}
+
+int trocm_kivi_cache_counts(const trocm_kivi_cache *c, int64_t *n_sink, int64_t *n_rows, int64_t *n_res, int64_t *row_bytes) {
+    TROCM_NOT_NULL(c);
+    if (n_sink) *n_sink = c->n_sink;
+    if (n_rows) *n_rows = c->n_rows;
+    if (n_res) *n_res = c->n_res;
+    if (row_bytes) *row_bytes = c->row_bytes;
+    return 0;
+}
+
+int trocm_kivi_cache_memory_bytes(const trocm_kivi_cache *c, size_t *bytes) {
+    TROCM_NOT_NULL(c);
+    TROCM_NOT_NULL(bytes);
+    const size_t per_head = (size_t)(c->n_rows * c->row_bytes) + (size_t)n_params(c) * 8 + (size_t)(c->n_sink + c->n_res) * c->D * 4;
+    *bytes = per_head * (size_t)c->BH;
+    return 0;
+}
+
+int trocm_kivi_cache_append(trocm_kivi_cache *c, const void *src, int src_dtype, int64_t n_new, void *stream) {
+    TROCM_NOT_NULL(c);
+    TROCM_REQUIRE(src_dtype == TROCM_F32 || src_dtype == TROCM_F16, "quantised cache: the input must be f32 or f16");
+    TROCM_REQUIRE(n_new >= 0, "quantised cache: negative token count");
+    if (n_new == 0) return 0;
+    TROCM_NOT_NULL(src);
+    TROCM_REQUIRE((c->len + n_new) * c->D < (1ll << 31) && n_new * c->D < (1ll << 31), "quantised cache: %lld tokens of %lld channels exceed the index range",
+                  (long long)(c->len + n_new), (long long)c->D);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    return src_dtype == TROCM_F32 ? kivi_append_t(c, (const float *)src, n_new, s) : kivi_append_t(c, (const __half *)src, n_new, s);
+}
+
+int trocm_kivi_cache_dequantize(const trocm_kivi_cache *c, void *dst, int dst_dtype, void *stream) {
+    TROCM_NOT_NULL(c);
+    TROCM_REQUIRE(dst_dtype == TROCM_F32 || dst_dtype == TROCM_F16, "quantised cache: the output must be f32 or f16");
+    if (c->len == 0) return 0;
+    TROCM_NOT_NULL(dst);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    return kivi_dequantize(c, dst, dst_dtype, s);
+}
+
+int trocm_kivi_cache_export(const trocm_kivi_cache *c, int part, void *dst, size_t *bytes, void *stream) {
+    TROCM_NOT_NULL(c);
+    int64_t width = 0, pitch = 0;
+    const void *src = nullptr;
+    switch (part) {
+        case TROCM_KIVI_PART_SINK: width = c->n_sink * c->D * 4; pitch = c->sink_tokens * c->D * 4; src = c->sink; break;
+        case TROCM_KIVI_PART_CODES: width = c->n_rows * c->row_bytes; pitch = c->cap_rows * c->row_bytes; src = c->codes; break;
+        case TROCM_KIVI_PART_LO: width = n_params(c) * 4; pitch = param_pitch(c, c->cap_rows) * 4; src = c->lo; break;
+        case TROCM_KIVI_PART_SCALE: width = n_params(c) * 4; pitch = param_pitch(c, c->cap_rows) * 4; src = c->scale; break;
+        case TROCM_KIVI_PART_RESIDUAL: width = c->n_res * c->D * 4; pitch = (int64_t)kKeyBlock * c->D * 4; src = c->residual; break;
+        default: return fail("quantised cache: unknown part %d", part);
+    }
+    if (c->layout == TROCM_KIVI_RUNNING_CHANNEL && (part == TROCM_KIVI_PART_LO || part == TROCM_KIVI_PART_SCALE) && !c->lo) width = 0;
+    if (bytes) *bytes = (size_t)width * (size_t)c->BH;
+    if (!dst || width == 0) return 0;
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    return copy_rows(dst, width, src, pitch, width, c->BH, s);
+}
+
+int trocm_kivi_cache_clone(const trocm_kivi_cache *c, trocm_kivi_cache **out, void *stream) {
+    TROCM_NOT_NULL(c);
+    TROCM_NOT_NULL(out);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    trocm_kivi_cache *n = nullptr;
+    if (trocm_kivi_cache_create(&n, c->layout, c->bits, c->sink_tokens, c->B, c->H, c->D)) return 1;
+    int rc = 0;
+    if (c->len > 0) {
+        rc = kivi_alloc_fixed(n, s);
+        if (!rc && c->n_rows) rc = kivi_ensure_rows(n, c->cap_rows, s);
+        n->len = c->len;
+        n->n_sink = c->n_sink;
+        n->n_rows = c->n_rows;
+        n->n_res = c->n_res;
+        if (!rc && c->n_sink) rc = copy_rows(n->sink, c->sink_tokens * c->D * 4, c->sink, c->sink_tokens * c->D * 4, c->n_sink * c->D * 4, c->BH, s);
+        if (!rc && c->n_res) rc = copy_rows(n->residual, (int64_t)kKeyBlock * c->D * 4, c->residual, (int64_t)kKeyBlock * c->D * 4, c->n_res * c->D * 4, c->BH, s);
+        if (!rc && c->n_rows) rc = copy_rows(n->codes, n->cap_rows * c->row_bytes, c->codes, c->cap_rows * c->row_bytes, c->n_rows * c->row_bytes, c->BH, s);
+        if (!rc && c->lo && n_params(c)) {
+            rc = copy_rows(n->lo, param_pitch(n, n->cap_rows) * 4, c->lo, param_pitch(c, c->cap_rows) * 4, n_params(c) * 4, c->BH, s);
+            if (!rc) rc = copy_rows(n->scale, param_pitch(n, n->cap_rows) * 4, c->scale, param_pitch(c, c->cap_rows) * 4, n_params(c) * 4, c->BH, s);
+        }
+    }
+    if (rc) {
+        trocm_kivi_cache_destroy(n);
+        return rc;
+    }
+    *out = n;
+    return 0;
+}
+
+int trocm_quantized_kv_sdpa_eval(const void *q, const void *k_new, const void *v_new, int dtype, int64_t q_heads,
+                                 int64_t n_new, trocm_kivi_cache *k_cache, trocm_kivi_cache *v_cache, void *out,
+                                 float scale, void *workspace, size_t workspace_bytes, void *stream) {
+    TROCM_NOT_NULL(q);
+    TROCM_NOT_NULL(k_new);
+    TROCM_NOT_NULL(v_new);
+    TROCM_NOT_NULL(k_cache);
+    TROCM_NOT_NULL(v_cache);
+    TROCM_NOT_NULL(out);
+    TROCM_REQUIRE(dtype == TROCM_F32 || dtype == TROCM_F16, "QuantizedKvSdpa: inputs must be f32 or f16");
+    TROCM_REQUIRE(n_new > 0, "QuantizedKvSdpa: no new token");
+    TROCM_REQUIRE(k_cache->B == v_cache->B && k_cache->H == v_cache->H && k_cache->D == v_cache->D && k_cache->len == v_cache->len,
+                  "QuantizedKvSdpa: the K and V stores differ in shape or length");
+    TROCM_REQUIRE(q_heads > 0 && q_heads % k_cache->H == 0, "QuantizedKvSdpa: %lld query heads over %lld kv heads",
+                  (long long)q_heads, (long long)k_cache->H);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    if (trocm_kivi_cache_append(k_cache, k_new, dtype, n_new, s)) return 1;
+    if (trocm_kivi_cache_append(v_cache, v_new, dtype, n_new, s)) return 1;
+    const int64_t T = k_cache->len, D = k_cache->D;
+    const size_t need = (size_t)k_cache->BH * T * D * elem_bytes(dtype);
+    for (trocm_kivi_cache *c : {k_cache, v_cache}) {
+        if (c->deq_bytes < need) {
+            size_t cap = c->deq_bytes * 2 > need ? c->deq_bytes * 2 : need;
+            if (c->deq) {
+                TROCM_HIP(hipStreamSynchronize(s));
+                (void)hipFree(c->deq);
+                c->deq = nullptr;
+                c->deq_bytes = 0;
+            }
+            TROCM_HIP(hipMalloc(&c->deq, cap));
+            c->deq_bytes = cap;
+        }
+        if (kivi_dequantize(c, c->deq, dtype, s)) return 1;
+    }
+    const int64_t strides[3] = {k_cache->H * T * D, T * D, D};
+    // kv_quant.rs:326-327: FlashSdpaOp { causal: false, scale }
+    return trocm_sdpa(q, k_cache->deq, v_cache->deq, nullptr, out, dtype, k_cache->B, q_heads, k_cache->H, n_new, T, D, strides, 1, 1,
+                      scale, 0, workspace, workspace_bytes, s);
+}
+
+}  // extern "C"
