@@ -473,6 +473,78 @@ def run_append(ta, args):
                      head["gbs"], "GB/s", round(head["us"] / 1e3, 5), "f16->q8_0", roof, {"cases": res})
 
 
+def run_kivi(ta, args):
+    """The KIVI-style quantised caches on their own: the ingest of a 16384-token prefill (8 x 8 kv heads x 128, f16 source)
+    into per-token Value stores and block x channel Key stores at 8 and 4 bits, the dequantising read of the whole cache
+    (the QuantizedDynKeyValueCache op's output) and one QuantizedKvSdpa decode step over 8192 tokens.  Algorithmic bytes
+    per element: ingest reads 2 and writes bits / 8 (+ parameters); the read moves bits / 8 in and 2 out."""
+    from oracle import oracle as orc
+    from tract_amd import kivi
+    B, T = 8, 16384
+    n_el = B * HKV * T * D
+    srcs = [ta.DeviceTensor.from_numpy(seeded_f16(cfg_seed(4, "k") + i, (B, HKV, T, D))) for i in range(2)]
+    tok = ta.DeviceTensor.from_numpy(seeded_f16(cfg_seed(4, "k") + 9, (B, HKV, 1, D)))
+    res, turn = {}, [0]
+    for name, layout in (("value_per_token", kivi.KIVI_PER_TOKEN), ("key_block_channel", kivi.KIVI_BLOCK_CHANNEL)):
+        for bits in (8, 4):
+            caches = [kivi.KiviCache(layout, bits, kivi.SINK_TOKENS, B, HKV, D) for _ in range(2)]
+            for c in caches:
+                c.append(srcs[0])
+
+            def bulk():
+                c = caches[turn[0] % 2]
+                c.reset()
+                c.append(srcs[turn[0] % 2])
+                turn[0] += 1
+
+            us = time_calls(ta, bulk, 20)
+            params = (B * HKV * T * 8) if layout == kivi.KIVI_PER_TOKEN else (B * HKV * (T // 32) * D * 8)
+            by = n_el * (2 + bits / 8) + params
+            res[f"ingest_{name}_{bits}bit_8x8x16384x128"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by)}
+            outs = [ta.DeviceTensor((B, HKV, caches[0].len(), D), np.float16) for _ in range(2)]
+
+            def read():
+                caches[turn[0] % 2].dequantize(out=outs[turn[0] % 2])
+                turn[0] += 1
+
+            us = time_calls(ta, read, 20)
+            by = n_el * (bits / 8 + 2) + params
+            res[f"dequantize_{name}_{bits}bit_8x8x16384x128"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by)}
+            us1 = time_calls(ta, lambda: caches[0].append(tok), 64)
+            res[f"token_ingest_{name}_{bits}bit"] = {"us": round(us1, 2)}
+            # after the timing: one head's state against the oracle's, bit for bit
+            c = caches[1]
+            c.reset()
+            c.append(srcs[1])
+            ref = orc.KiviStore(orc.KIVI_PER_TOKEN if layout == kivi.KIVI_PER_TOKEN else orc.KIVI_BLOCK_CHANNEL, D, bits)
+            for row in srcs[1].to_numpy()[3, 5].astype(np.float32):
+                ref.push_token(row)
+            got, want = c.state(), ref.state()
+            at = 3 * HKV + 5
+            res[f"ingest_{name}_{bits}bit_8x8x16384x128"]["state_bit_exact_vs_oracle"] = bool(
+                got["packed"][at].tobytes() == want["packed"].tobytes() and np.array_equal(got["lo"][at], want["lo"])
+                and np.array_equal(got["scale"][at], want["scale"]) and got["sink"][at].tobytes() == want["sink"].tobytes())
+            del caches, outs
+    # QuantizedKvSdpa: one decode step over an 8192-token cache (append, two dequantising reads, attention)
+    Tc = 8192
+    st = ta.QuantizedKvSdpa(axis=2).state()
+    kq = ta.DeviceTensor.from_numpy(seeded_f16(cfg_seed(2, "k"), (B, HKV, Tc, D)))
+    st.k = kivi.KiviCache(kivi.KIVI_RUNNING_CHANNEL, 8, 0, B, HKV, D)
+    st.v = kivi.KiviCache(kivi.KIVI_PER_TOKEN, 8, 0, B, HKV, D)
+    st.k.append(kq), st.v.append(kq)
+    q1 = ta.DeviceTensor.from_numpy((seeded_f16(cfg_seed(2, "q") + 1, (B, HQ, 1, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16))
+    out = ta.DeviceTensor((B, HQ, 1, D), np.float16)
+    us = time_calls(ta, lambda: st.eval([q1, tok, tok], out=out), 32)
+    res["quantized_kv_sdpa_step_b8_ctx8192"] = {"us": round(us, 2), "note": "append + dequantise K and V (u8 -> f16) + f16 decode attention"}
+    head = res["dequantize_key_block_channel_8bit_8x8x16384x128"]
+    roof = {"bound": "hbm", "kernel": "kivi_dequant_kernel<f16, 8>", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(head["gbs"] / HBM_PEAK_GBS, 4), "traffic": None}
+    return base_line(args, "kivi: KIVI-style affine quantised caches (8 x 8 kv heads x 16384 tokens x 128, f16): ingest into per-token "
+                     "Value and block x channel Key stores at 8 / 4 bits, the dequantising read of the whole cache, one QuantizedKvSdpa "
+                     "decode step at 8192 tokens; headline = the 8-bit Key cache read", head["gbs"], "GB/s", round(head["us"] / 1e3, 5),
+                     "u8->f16", roof, {"cases": res})
+
+
 def run_ops(ta, args):
     """The ops either side of the cache (RoPE, cast) and the sliding-window decode step, each against
     its HBM roofline, with the oracle timed on the host for the same ops (smaller sample)."""
@@ -654,7 +726,7 @@ def main():
     ap.add_argument("--kernel-iters", type=int, default=200)
     ap.add_argument("--windows", type=int, default=5, help="how many times the timed window of --steps steps is taken (median reported)")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "ops", "append"],
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "ops", "append", "kivi"],
                     help="cfg2 (default) is the configuration the metric is quoted on; the others print one line "
                          "of the same shape for the remaining configurations")
     args = ap.parse_args()
@@ -666,7 +738,7 @@ def main():
     import tract_amd as ta
     rt = ta.runtime_for_name("rocm")
     if args.workload != "cfg2":
-        line = {"cfg1": run_cfg1, "cfg3": run_cfg3, "cfg4": run_cfg4, "cfg5": run_cfg5, "ops": run_ops, "append": run_append}[args.workload](ta, args)
+        line = {"cfg1": run_cfg1, "cfg3": run_cfg3, "cfg4": run_cfg4, "cfg5": run_cfg5, "ops": run_ops, "append": run_append, "kivi": run_kivi}[args.workload](ta, args)
         line["device"] = rt.device_name
         print(json.dumps(line))
         return

@@ -378,6 +378,9 @@ enum { TROCM_KIVI_PART_SINK = 0, TROCM_KIVI_PART_CODES = 1, TROCM_KIVI_PART_LO =
 int trocm_kivi_cache_create(trocm_kivi_cache **out, int layout, int bits, int64_t sink_tokens, int64_t batch,
                             int64_t heads, int64_t head_dim);
 int trocm_kivi_cache_destroy(trocm_kivi_cache *cache);
+/* Back to the empty state a new session starts from (EvalOp::state, quant_dyn_kv_cache.rs:301-314), keeping the
+ * device buffers. */
+int trocm_kivi_cache_reset(trocm_kivi_cache *cache, void *stream);
 int trocm_kivi_cache_len(const trocm_kivi_cache *cache, int64_t *len);
 /* Tokens held as f32 sinks, as coded rows and in the partial key block; bytes of a coded row (row_bytes, :58-60). */
 int trocm_kivi_cache_counts(const trocm_kivi_cache *cache, int64_t *n_sink, int64_t *n_rows, int64_t *n_res,

@@ -90,6 +90,7 @@ SIGNATURES = {
                                           _sz, _vp],
     "trocm_kivi_cache_create": [C.POINTER(_vp), _i, _i, _i64, _i64, _i64, _i64],
     "trocm_kivi_cache_destroy": [_vp],
+    "trocm_kivi_cache_reset": [_vp, _vp],
     "trocm_kivi_cache_len": [_vp, _pi64],
     "trocm_kivi_cache_counts": [_vp, _pi64, _pi64, _pi64, _pi64],
     "trocm_kivi_cache_memory_bytes": [_vp, C.POINTER(_sz)],

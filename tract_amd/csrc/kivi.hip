@@ -190,6 +190,146 @@ __global__ void kivi_running_push_kernel(const SrcT *__restrict__ src, int64_t S
     scale_io[(int64_t)bh * D + c] = scale;
 }
 
+// ---- the same three steps for head sizes that are a multiple of 8 (and, for the two quantising kernels, 64, 128,
+// ---- 256 or 512 with 16-byte aligned sources): a lane owns 8 consecutive channels, so rows move as 128-bit words
+struct F8 {
+    float v[8];
+};
+__device__ __forceinline__ F8 ld8(const float *p) {
+    const float4 a = reinterpret_cast<const float4 *>(p)[0], b = reinterpret_cast<const float4 *>(p)[1];
+    return F8{{a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w}};
+}
+__device__ __forceinline__ F8 ld8(const __half *p) {
+    const uint4 w = *reinterpret_cast<const uint4 *>(p);
+    const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+    F8 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        r.v[2 * i] = __half2float(__ushort_as_half((unsigned short)(u[i] & 0xffffu)));
+        r.v[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(u[i] >> 16)));
+    }
+    return r;
+}
+__device__ __forceinline__ void st8(float *p, const F8 &x) {
+    reinterpret_cast<float4 *>(p)[0] = make_float4(x.v[0], x.v[1], x.v[2], x.v[3]);
+    reinterpret_cast<float4 *>(p)[1] = make_float4(x.v[4], x.v[5], x.v[6], x.v[7]);
+}
+__device__ __forceinline__ void st8(__half *p, const F8 &x) {
+    uint32_t u[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float a = x.v[2 * i], b = x.v[2 * i + 1];
+        asm volatile("" : "+v"(a), "+v"(b));   // conversions stay their own instructions (see st)
+        u[i] = (uint32_t)__half_as_ushort(__float2half_rn(a)) | ((uint32_t)__half_as_ushort(__float2half_rn(b)) << 16);
+    }
+    *reinterpret_cast<uint4 *>(p) = make_uint4(u[0], u[1], u[2], u[3]);
+}
+// 8 codes of one lane's channels packed as the row stores them: 8 bytes, or 4 bytes of nibble pairs (even index low).
+template <int BITS>
+__device__ __forceinline__ void store_codes8(uint8_t *row, int sub, const uint32_t (&code)[8]) {
+    if (BITS == 8) {
+        const uint32_t w0 = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
+        const uint32_t w1 = code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24);
+        *reinterpret_cast<uint2 *>(row + sub * 8) = make_uint2(w0, w1);
+    } else {
+        uint32_t w = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) w |= (code[i] & 15u) << (4 * i);
+        *reinterpret_cast<uint32_t *>(row + sub * 4) = w;
+    }
+}
+
+// Values: LPR = D / 8 lanes per token, 64 / LPR tokens per wave.
+template <typename SrcT, int BITS, int LPR>
+__global__ void __launch_bounds__(256) kivi_quant_tokens_vec_kernel(const SrcT *__restrict__ src, int64_t S, int64_t src_t0, int n,
+                                                                    uint8_t *__restrict__ codes, int64_t cap_rows, int64_t row0,
+                                                                    float *__restrict__ lo_out, float *__restrict__ scale_out) {
+    constexpr int D = LPR * 8, TPW = 64 / LPR, RB = D * BITS / 8;
+    constexpr float lv = (float)((1u << BITS) - 1u);
+    const int bh = blockIdx.y, lane = threadIdx.x & 63, sub = lane % LPR;
+    const int i = (blockIdx.x * 4 + (threadIdx.x >> 6)) * TPW + lane / LPR;
+    if (i >= n) return;   // whole groups of LPR lanes leave together; the exchanges below stay inside a group
+    const F8 x = ld8(src + ((int64_t)bh * S + src_t0 + i) * D + sub * 8);
+    float lo = INFINITY, hi = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        lo = fminf(lo, x.v[e]);
+        hi = fmaxf(hi, x.v[e]);
+    }
+#pragma unroll
+    for (int m = LPR / 2; m >= 1; m >>= 1) {
+        lo = fminf(lo, __shfl_xor(lo, m, 64));
+        hi = fmaxf(hi, __shfl_xor(hi, m, 64));
+    }
+    const float scale = affine_scale(lo, hi, lv);
+    uint32_t code[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) code[e] = affine_code(x.v[e], lo, scale, lv);
+    store_codes8<BITS>(codes + ((int64_t)bh * cap_rows + row0 + i) * RB, sub, code);
+    if (sub == 0) {
+        lo_out[(int64_t)bh * cap_rows + row0 + i] = lo;
+        scale_out[(int64_t)bh * cap_rows + row0 + i] = scale;
+    }
+}
+
+// Keys: one wave per block whose 32 rows all come from the new tokens; the wave's 64 / LPR lane groups take the rows
+// in turn, join their lo / hi, and code their rows in a second pass (the rows are in the cache by then).
+template <typename SrcT, int BITS, int LPR>
+__global__ void __launch_bounds__(256) kivi_finalize_blocks_vec_kernel(const SrcT *__restrict__ src, int64_t S, int64_t src_t0, int nb,
+                                                                       uint8_t *__restrict__ codes, int64_t cap_rows, int64_t row0,
+                                                                       float *__restrict__ lo_out, float *__restrict__ scale_out) {
+    constexpr int D = LPR * 8, G = 64 / LPR, RB = D * BITS / 8;
+    constexpr float lv = (float)((1u << BITS) - 1u);
+    const int bh = blockIdx.y, lane = threadIdx.x & 63, sub = lane % LPR, g = lane / LPR;
+    const int j = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (j >= nb) return;   // wave-uniform
+    const SrcT *rows = src + ((int64_t)bh * S + src_t0 + (int64_t)j * kKeyBlock) * D + sub * 8;
+    float lo[8], hi[8], scale[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        lo[e] = INFINITY;
+        hi[e] = -INFINITY;
+    }
+#pragma unroll 4
+    for (int r = g; r < kKeyBlock; r += G) {
+        const F8 x = ld8(rows + (int64_t)r * D);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            lo[e] = fminf(lo[e], x.v[e]);
+            hi[e] = fmaxf(hi[e], x.v[e]);
+        }
+    }
+#pragma unroll
+    for (int m = LPR; m < 64; m <<= 1) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            lo[e] = fminf(lo[e], __shfl_xor(lo[e], m, 64));
+            hi[e] = fmaxf(hi[e], __shfl_xor(hi[e], m, 64));
+        }
+    }
+    F8 ls, ss;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        scale[e] = affine_scale(lo[e], hi[e], lv);
+        ls.v[e] = lo[e];
+        ss.v[e] = scale[e];
+    }
+    if (g == 0) {
+        const int64_t at = ((int64_t)bh * (cap_rows / kKeyBlock) + row0 / kKeyBlock + j) * D + sub * 8;
+        st8(lo_out + at, ls);
+        st8(scale_out + at, ss);
+    }
+    uint8_t *out = codes + ((int64_t)bh * cap_rows + row0 + (int64_t)j * kKeyBlock) * RB;
+#pragma unroll 4
+    for (int r = g; r < kKeyBlock; r += G) {
+        const F8 x = ld8(rows + (int64_t)r * D);
+        uint32_t code[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) code[e] = affine_code(x.v[e], lo[e], scale[e], lv);
+        store_codes8<BITS>(out + (int64_t)r * RB, sub, code);
+    }
+}
+
 struct KiviView {
     int layout, D, row_bytes, len, n_sink, n_rows;
     int64_t sink_tokens, cap_rows;
@@ -226,6 +366,50 @@ __global__ void kivi_dequant_kernel(KiviView a, DstT *__restrict__ dst) {
         x = a.residual[((int64_t)bh * kKeyBlock + (t - a.n_sink - a.n_rows)) * a.D + c];
     }
     st(dst + ((int64_t)bh * a.len + t) * a.D + c, x);
+}
+
+// dequant_all for head sizes that are a multiple of 8: a thread owns 8 consecutive channels of one token.
+template <typename DstT, int BITS>
+__global__ void __launch_bounds__(256) kivi_dequant_vec_kernel(KiviView a, DstT *__restrict__ dst) {
+    const int bh = blockIdx.y;
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    const int d8 = a.D >> 3;
+    if (e >= a.len * d8) return;
+    const int t = e / d8, c = (e - t * d8) * 8;
+    F8 x;
+    if (t < a.n_sink) {
+        x = ld8(a.sink + ((int64_t)bh * a.sink_tokens + t) * a.D + c);
+    } else if (t - a.n_sink < a.n_rows) {
+        const int r = t - a.n_sink;
+        const uint8_t *row = a.codes + ((int64_t)bh * a.cap_rows + r) * a.row_bytes;
+        uint32_t code[8];
+        if (BITS == 8) {
+            const uint2 w = *reinterpret_cast<const uint2 *>(row + c);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                code[i] = (w.x >> (8 * i)) & 255u;
+                code[4 + i] = (w.y >> (8 * i)) & 255u;
+            }
+        } else {
+            const uint32_t w = *reinterpret_cast<const uint32_t *>(row + (c >> 1));
+#pragma unroll
+            for (int i = 0; i < 8; i++) code[i] = (w >> (4 * i)) & 15u;
+        }
+        if (a.layout == TROCM_KIVI_PER_TOKEN) {
+            const float lo = a.lo[(int64_t)bh * a.cap_rows + r], sc = a.scale[(int64_t)bh * a.cap_rows + r];
+#pragma unroll
+            for (int i = 0; i < 8; i++) x.v[i] = __fadd_rn(lo, __fmul_rn((float)code[i], sc));
+        } else {
+            const int64_t p = a.layout == TROCM_KIVI_BLOCK_CHANNEL ? ((int64_t)bh * (a.cap_rows / kKeyBlock) + r / kKeyBlock) * a.D + c
+                                                                   : (int64_t)bh * a.D + c;
+            const F8 lo = ld8(a.lo + p), sc = ld8(a.scale + p);
+#pragma unroll
+            for (int i = 0; i < 8; i++) x.v[i] = __fadd_rn(lo.v[i], __fmul_rn((float)code[i], sc.v[i]));
+        }
+    } else {
+        x = ld8(a.residual + ((int64_t)bh * kKeyBlock + (t - a.n_sink - a.n_rows)) * a.D + c);
+    }
+    st8(dst + ((int64_t)bh * a.len + t) * a.D + c, x);
 }
 
 __global__ void kivi_fill_running_kernel(float *lo, float *scale, int64_t n) {
@@ -359,24 +543,56 @@ static int kivi_append_t(trocm_kivi_cache *c, const SrcT *src, int64_t S, hipStr
     const int64_t rem = S - t0;
     if (rem > 0 && c->layout == TROCM_KIVI_PER_TOKEN) {
         if (kivi_ensure_rows(c, c->n_rows + rem, s)) return 1;
-        const dim3 grid((unsigned)((rem + 3) / 4), BH);
-        if (c->bits == 8)
-            kivi_quant_tokens_kernel<SrcT, 8><<<grid, 256, 0, s>>>(src, S, t0, (int)rem, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
-        else
-            kivi_quant_tokens_kernel<SrcT, 4><<<grid, 256, 0, s>>>(src, S, t0, (int)rem, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
+        const bool vec = ((uintptr_t)src & 15) == 0 && (D == 64 || D == 128 || D == 256 || D == 512);
+#define KIVI_TOKENS_VEC(BITS, LPR)                                                                                              \
+    kivi_quant_tokens_vec_kernel<SrcT, BITS, LPR><<<dim3((unsigned)((rem + 4 * (64 / LPR) - 1) / (4 * (64 / LPR))), BH), 256, 0, s>>>( \
+        src, S, t0, (int)rem, c->codes, c->cap_rows, c->n_rows, c->lo, c->scale)
+        if (vec && c->bits == 8) {
+            if (D == 64) KIVI_TOKENS_VEC(8, 8); else if (D == 128) KIVI_TOKENS_VEC(8, 16); else if (D == 256) KIVI_TOKENS_VEC(8, 32); else KIVI_TOKENS_VEC(8, 64);
+        } else if (vec) {
+            if (D == 64) KIVI_TOKENS_VEC(4, 8); else if (D == 128) KIVI_TOKENS_VEC(4, 16); else if (D == 256) KIVI_TOKENS_VEC(4, 32); else KIVI_TOKENS_VEC(4, 64);
+        } else {
+            const dim3 grid((unsigned)((rem + 3) / 4), BH);
+            if (c->bits == 8)
+                kivi_quant_tokens_kernel<SrcT, 8><<<grid, 256, 0, s>>>(src, S, t0, (int)rem, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
+            else
+                kivi_quant_tokens_kernel<SrcT, 4><<<grid, 256, 0, s>>>(src, S, t0, (int)rem, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
+        }
+#undef KIVI_TOKENS_VEC
         TROCM_HIP(hipGetLastError());
         c->n_rows += rem;
     } else if (rem > 0 && c->layout == TROCM_KIVI_BLOCK_CHANNEL) {
         const int64_t nb = (c->n_res + rem) / kKeyBlock;
         if (nb > 0) {
             if (kivi_ensure_rows(c, c->n_rows + nb * kKeyBlock, s)) return 1;
-            const dim3 grid((unsigned)nb, BH);
-            const int threads = c->row_bytes >= 256 ? 256 : (int)((c->row_bytes + 63) / 64 * 64);
-            if (c->bits == 8)
-                kivi_finalize_blocks_kernel<SrcT, 8><<<grid, threads, 0, s>>>(src, S, t0, c->residual, (int)c->n_res, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
-            else
-                kivi_finalize_blocks_kernel<SrcT, 4><<<grid, threads, 0, s>>>(src, S, t0, c->residual, (int)c->n_res, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
-            TROCM_HIP(hipGetLastError());
+            // the block that the partial block completes (if any) takes the general kernel; blocks made of new tokens only
+            // take the 128-bit one when the head size allows
+            const bool vec = ((uintptr_t)src & 15) == 0 && (D == 64 || D == 128 || D == 256 || D == 512);
+            const int64_t nb_gen = !vec ? nb : (c->n_res > 0 ? 1 : 0), nb_vec = nb - nb_gen;
+            if (nb_gen > 0) {
+                const dim3 grid((unsigned)nb_gen, BH);
+                const int threads = c->row_bytes >= 256 ? 256 : (int)((c->row_bytes + 63) / 64 * 64);
+                if (c->bits == 8)
+                    kivi_finalize_blocks_kernel<SrcT, 8><<<grid, threads, 0, s>>>(src, S, t0, c->residual, (int)c->n_res, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
+                else
+                    kivi_finalize_blocks_kernel<SrcT, 4><<<grid, threads, 0, s>>>(src, S, t0, c->residual, (int)c->n_res, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
+                TROCM_HIP(hipGetLastError());
+            }
+            if (nb_vec > 0) {
+                // rows of these blocks start after the tokens the general launch consumed
+                const int64_t skip = nb_gen * kKeyBlock - (nb_gen ? c->n_res : 0);
+                const int64_t vt0 = t0 + skip, vrow0 = c->n_rows + nb_gen * kKeyBlock;
+#define KIVI_BLOCKS_VEC(BITS, LPR)                                                                                   \
+    kivi_finalize_blocks_vec_kernel<SrcT, BITS, LPR><<<dim3((unsigned)((nb_vec + 3) / 4), BH), 256, 0, s>>>(         \
+        src, S, vt0, (int)nb_vec, c->codes, c->cap_rows, vrow0, c->lo, c->scale)
+                if (c->bits == 8) {
+                    if (D == 64) KIVI_BLOCKS_VEC(8, 8); else if (D == 128) KIVI_BLOCKS_VEC(8, 16); else if (D == 256) KIVI_BLOCKS_VEC(8, 32); else KIVI_BLOCKS_VEC(8, 64);
+                } else {
+                    if (D == 64) KIVI_BLOCKS_VEC(4, 8); else if (D == 128) KIVI_BLOCKS_VEC(4, 16); else if (D == 256) KIVI_BLOCKS_VEC(4, 32); else KIVI_BLOCKS_VEC(4, 64);
+                }
+#undef KIVI_BLOCKS_VEC
+                TROCM_HIP(hipGetLastError());
+            }
             const int64_t used = nb * kKeyBlock - c->n_res, tail = rem - used;
             c->n_rows += nb * kKeyBlock;
             if (tail > 0) {
@@ -415,6 +631,18 @@ static int kivi_dequantize(const trocm_kivi_cache *c, void *dst, int dst_dtype, 
     a.lo = c->lo;
     a.scale = c->scale;
     a.codes = c->codes;
+    if (c->D % 8 == 0 && ((uintptr_t)dst & 15) == 0) {
+        const dim3 grid8((unsigned)((c->len * (c->D / 8) + 255) / 256), (unsigned)c->BH);
+        if (dst_dtype == TROCM_F32) {
+            if (c->bits == 8) kivi_dequant_vec_kernel<float, 8><<<grid8, 256, 0, s>>>(a, (float *)dst);
+            else kivi_dequant_vec_kernel<float, 4><<<grid8, 256, 0, s>>>(a, (float *)dst);
+        } else {
+            if (c->bits == 8) kivi_dequant_vec_kernel<__half, 8><<<grid8, 256, 0, s>>>(a, (__half *)dst);
+            else kivi_dequant_vec_kernel<__half, 4><<<grid8, 256, 0, s>>>(a, (__half *)dst);
+        }
+        TROCM_HIP(hipGetLastError());
+        return 0;
+    }
     const dim3 grid((unsigned)((c->len * c->D + 255) / 256), (unsigned)c->BH);
     if (dst_dtype == TROCM_F32) {
         if (c->bits == 8) kivi_dequant_kernel<float, 8><<<grid, 256, 0, s>>>(a, (float *)dst);
@@ -462,6 +690,19 @@ int trocm_kivi_cache_destroy(trocm_kivi_cache *c) {
     (void)hipFree(c->codes);
     (void)hipFree(c->deq);
     delete c;
+    return 0;
+}
+
+int trocm_kivi_cache_reset(trocm_kivi_cache *c, void *stream) {
+    TROCM_NOT_NULL(c);
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    c->len = c->n_sink = c->n_rows = c->n_res = 0;
+    if (c->layout == TROCM_KIVI_RUNNING_CHANNEL && c->lo) {
+        const int64_t n = c->BH * c->D;
+        kivi_fill_running_kernel<<<dim3((unsigned)((n + 255) / 256)), 256, 0, s>>>(c->lo, c->scale, n);
+        TROCM_HIP(hipGetLastError());
+    }
     return 0;
 }
 

@@ -52,6 +52,10 @@ class KiviCache:
         call("trocm_kivi_cache_len", self.handle, C.byref(n))
         return n.value
 
+    def reset(self, stream=None) -> None:
+        """The empty state of a new session, keeping the device buffers."""
+        call("trocm_kivi_cache_reset", self.handle, _sh(stream))
+
     def counts(self) -> dict:
         a, b, c, d = C.c_int64(), C.c_int64(), C.c_int64(), C.c_int64()
         call("trocm_kivi_cache_counts", self.handle, C.byref(a), C.byref(b), C.byref(c), C.byref(d))
