@@ -134,7 +134,7 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_kernel(const SrcT *_
             const int c = CH * u + h;
             float l = INFINITY, hi = -INFINITY;
             if (c < D) {
-#pragma unroll 1
+#pragma unroll 4
                 for (int r = 0; r < kKeyBlock; r++) {
                     const int k = j * kKeyBlock + r;
                     const float x = k < n_res_old ? res[(int64_t)k * D + c] : ld(fresh + (int64_t)k * D + c);
@@ -149,7 +149,7 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_kernel(const SrcT *_
             scale[h] = affine_scale(l, hi, lv);
         }
         // second pass over the block's rows (they are in the cache now): the codes
-#pragma unroll 1
+#pragma unroll 2
         for (int r = 0; r < kKeyBlock; r++) {
             const int k = j * kKeyBlock + r;
             uint32_t byte = 0;
@@ -276,6 +276,7 @@ __global__ void __launch_bounds__(256) kivi_quant_tokens_vec_kernel(const SrcT *
 // in turn, join their lo / hi, and code their rows in a second pass (the rows are in the cache by then).
 template <typename SrcT, int BITS, int LPR>
 __global__ void __launch_bounds__(256) kivi_finalize_blocks_vec_kernel(const SrcT *__restrict__ src, int64_t S, int64_t src_t0, int nb,
+                                                                       const float *__restrict__ residual, int n_res_old,
                                                                        uint8_t *__restrict__ codes, int64_t cap_rows, int64_t row0,
                                                                        float *__restrict__ lo_out, float *__restrict__ scale_out) {
     constexpr int D = LPR * 8, G = 64 / LPR, RB = D * BITS / 8;
@@ -283,7 +284,10 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_vec_kernel(const Src
     const int bh = blockIdx.y, lane = threadIdx.x & 63, sub = lane % LPR, g = lane / LPR;
     const int j = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (j >= nb) return;   // wave-uniform
-    const SrcT *rows = src + ((int64_t)bh * S + src_t0 + (int64_t)j * kKeyBlock) * D + sub * 8;
+    // row r of block j is row k = 32 j + r of the run: from the partial block when k < n_res_old, else new token k - n_res_old
+    const SrcT *rows = src + ((int64_t)bh * S + src_t0 + (int64_t)j * kKeyBlock - n_res_old) * D + sub * 8;
+    const float *res = residual + (int64_t)bh * kKeyBlock * D + sub * 8;
+    const int n_old = j == 0 ? n_res_old : 0;
     float lo[8], hi[8], scale[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) {
@@ -292,7 +296,7 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_vec_kernel(const Src
     }
 #pragma unroll 4
     for (int r = g; r < kKeyBlock; r += G) {
-        const F8 x = ld8(rows + (int64_t)r * D);
+        const F8 x = r < n_old ? ld8(res + (int64_t)r * D) : ld8(rows + (int64_t)r * D);
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             lo[e] = fminf(lo[e], x.v[e]);
@@ -322,7 +326,7 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_vec_kernel(const Src
     uint8_t *out = codes + ((int64_t)bh * cap_rows + row0 + (int64_t)j * kKeyBlock) * RB;
 #pragma unroll 4
     for (int r = g; r < kKeyBlock; r += G) {
-        const F8 x = ld8(rows + (int64_t)r * D);
+        const F8 x = r < n_old ? ld8(res + (int64_t)r * D) : ld8(rows + (int64_t)r * D);
         uint32_t code[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) code[e] = affine_code(x.v[e], lo[e], scale[e], lv);
@@ -565,34 +569,24 @@ static int kivi_append_t(trocm_kivi_cache *c, const SrcT *src, int64_t S, hipStr
         const int64_t nb = (c->n_res + rem) / kKeyBlock;
         if (nb > 0) {
             if (kivi_ensure_rows(c, c->n_rows + nb * kKeyBlock, s)) return 1;
-            // the block that the partial block completes (if any) takes the general kernel; blocks made of new tokens only
-            // take the 128-bit one when the head size allows
             const bool vec = ((uintptr_t)src & 15) == 0 && (D == 64 || D == 128 || D == 256 || D == 512);
-            const int64_t nb_gen = !vec ? nb : (c->n_res > 0 ? 1 : 0), nb_vec = nb - nb_gen;
-            if (nb_gen > 0) {
-                const dim3 grid((unsigned)nb_gen, BH);
+#define KIVI_BLOCKS_VEC(BITS, LPR)                                                                               \
+    kivi_finalize_blocks_vec_kernel<SrcT, BITS, LPR><<<dim3((unsigned)((nb + 3) / 4), BH), 256, 0, s>>>(         \
+        src, S, t0, (int)nb, c->residual, (int)c->n_res, c->codes, c->cap_rows, c->n_rows, c->lo, c->scale)
+            if (vec && c->bits == 8) {
+                if (D == 64) KIVI_BLOCKS_VEC(8, 8); else if (D == 128) KIVI_BLOCKS_VEC(8, 16); else if (D == 256) KIVI_BLOCKS_VEC(8, 32); else KIVI_BLOCKS_VEC(8, 64);
+            } else if (vec) {
+                if (D == 64) KIVI_BLOCKS_VEC(4, 8); else if (D == 128) KIVI_BLOCKS_VEC(4, 16); else if (D == 256) KIVI_BLOCKS_VEC(4, 32); else KIVI_BLOCKS_VEC(4, 64);
+            } else {
+                const dim3 grid((unsigned)nb, BH);
                 const int threads = c->row_bytes >= 256 ? 256 : (int)((c->row_bytes + 63) / 64 * 64);
                 if (c->bits == 8)
                     kivi_finalize_blocks_kernel<SrcT, 8><<<grid, threads, 0, s>>>(src, S, t0, c->residual, (int)c->n_res, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
                 else
                     kivi_finalize_blocks_kernel<SrcT, 4><<<grid, threads, 0, s>>>(src, S, t0, c->residual, (int)c->n_res, D, c->codes, c->cap_rows, (int)c->row_bytes, c->n_rows, c->lo, c->scale);
-                TROCM_HIP(hipGetLastError());
             }
-            if (nb_vec > 0) {
-                // rows of these blocks start after the tokens the general launch consumed
-                const int64_t skip = nb_gen * kKeyBlock - (nb_gen ? c->n_res : 0);
-                const int64_t vt0 = t0 + skip, vrow0 = c->n_rows + nb_gen * kKeyBlock;
-#define KIVI_BLOCKS_VEC(BITS, LPR)                                                                                   \
-    kivi_finalize_blocks_vec_kernel<SrcT, BITS, LPR><<<dim3((unsigned)((nb_vec + 3) / 4), BH), 256, 0, s>>>(         \
-        src, S, vt0, (int)nb_vec, c->codes, c->cap_rows, vrow0, c->lo, c->scale)
-                if (c->bits == 8) {
-                    if (D == 64) KIVI_BLOCKS_VEC(8, 8); else if (D == 128) KIVI_BLOCKS_VEC(8, 16); else if (D == 256) KIVI_BLOCKS_VEC(8, 32); else KIVI_BLOCKS_VEC(8, 64);
-                } else {
-                    if (D == 64) KIVI_BLOCKS_VEC(4, 8); else if (D == 128) KIVI_BLOCKS_VEC(4, 16); else if (D == 256) KIVI_BLOCKS_VEC(4, 32); else KIVI_BLOCKS_VEC(4, 64);
-                }
 #undef KIVI_BLOCKS_VEC
-                TROCM_HIP(hipGetLastError());
-            }
+            TROCM_HIP(hipGetLastError());
             const int64_t used = nb * kKeyBlock - c->n_res, tail = rem - used;
             c->n_rows += nb * kKeyBlock;
             if (tail > 0) {
