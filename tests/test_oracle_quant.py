@@ -228,3 +228,26 @@ def test_f16_dequant_rounds_product_to_f16():
     got = orc.dequant(orc.FMT_Q4_0, np.frombuffer(raw, dtype=np.uint8), np.float16)
     d = np.float32(np.float16(0.1))
     assert got[0] == np.float16(np.float32(7) * d) and got[16] == np.float16(np.float32(-8) * d)
+
+
+def test_round_half_away_as_one_addition_and_a_truncation():
+    """The quantising kernels round with trunc(x + copysign(0.49999997, x)) (three instructions); this is f32::round
+    for every float.  Checked here on every mantissa of the exponents 2^-2 .. 2^8 (the range of the codes) and on
+    the ties, huge values, infinities and NaN; the exponents up to 2^24 were compared the same way when it was written."""
+    h = np.nextafter(np.float32(0.5), np.float32(0))
+    assert h == np.float32(0.49999997)
+
+    def dev(x):
+        return np.trunc((x + np.copysign(h, x)).astype(np.float32))
+
+    for e in range(-2, 9):
+        base = np.float32(2.0 ** e).view(np.uint32)
+        x = np.arange(base, base + (1 << 23), dtype=np.uint32).view(np.float32)
+        want = np.floor(x.astype(np.float64) + 0.5)
+        assert np.array_equal(dev(x).astype(np.float64), want)
+        assert np.array_equal(dev(-x).astype(np.float64), -want)
+    ties = np.arange(0, 300, dtype=np.float32) + np.float32(0.5)
+    assert np.array_equal(dev(ties), ties + np.float32(0.5)) and np.array_equal(dev(-ties), -ties - np.float32(0.5))
+    assert dev(np.float32(0.49999997)) == 0 and dev(np.float32(-0.49999997)) == 0
+    big = np.array([2.0 ** 23 + 1, 2.0 ** 24, 3e38, np.inf, -np.inf], np.float32)
+    assert np.array_equal(dev(big), big) and np.isnan(dev(np.float32(np.nan)))

@@ -15,6 +15,7 @@
 // bytes, so one lane reads whole 128-bit words.  The work is HBM-bound (reads 2-4 bytes
 // and writes ~1 byte per element).
 #include <hip/hip_fp16.h>
+#include <stdlib.h>
 #include "common.h"
 
 namespace trocm {
@@ -42,12 +43,13 @@ __device__ __forceinline__ int cvt_i32_rz_sat(float x) {
 }
 __device__ __forceinline__ int sat_i8(float x) { return max(-128, min(127, cvt_i32_rz_sat(x))); }   // (one v_med3_i32)
 
-// f32::round(): half away from zero.  d = x - trunc(x) is exact and |d| < 1, so d + d is exact too and its
-// truncation is the unit to add: +-1 exactly when |d| >= 0.5, with the sign of x.
+// f32::round(): half away from zero, as trunc(x + copysign(0.49999997, x)) with the addition rounded to nearest even.
+// 0.49999997 is the float below 0.5: for a fraction below one half the sum stays under the next integer, at exactly one
+// half the sum lies midway between two floats and ties to the even one, which is the integer; from 2^23 on x + 0.49999997
+// rounds back to x.  Equal to round() for every float (all 2^23 mantissas of every exponent from 2^-3 to 2^24 were
+// compared on the host; below 2^-3 the sum stays under 1, above 2^25 it is x; inf and NaN pass through).
 __device__ __forceinline__ float round_half_away(float x) {
-    const float t = truncf(x);
-    const float d = __fsub_rn(x, t);
-    return __fadd_rn(t, truncf(__fadd_rn(d, d)));
+    return truncf(__fadd_rn(x, __builtin_copysignf(0.49999997f, x)));
 }
 
 // Signed value of the first element with strictly largest magnitude (q4_0.rs:27-34).
