@@ -532,6 +532,13 @@ def run_kivi(ta, args):
     st.k = kivi.KiviCache(kivi.KIVI_RUNNING_CHANNEL, 8, 0, B, HKV, D)
     st.v = kivi.KiviCache(kivi.KIVI_PER_TOKEN, 8, 0, B, HKV, D)
     st.k.append(kq), st.v.append(kq)
+
+    def prompt():
+        st.k.reset()
+        st.k.append(kq)
+
+    res["prompt_push_running_keys_8x8x8192x128"] = {"us": round(time_calls(ta, prompt, 8), 2),
+                                                    "note": "chunked scan over 64-token chunks; incl. the scratch allocation and the wait before it is freed"}
     q1 = ta.DeviceTensor.from_numpy((seeded_f16(cfg_seed(2, "q") + 1, (B, HQ, 1, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16))
     out = ta.DeviceTensor((B, HQ, 1, D), np.float16)
     us = time_calls(ta, lambda: st.eval([q1, tok, tok], out=out), 32)

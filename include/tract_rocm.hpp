@@ -5,6 +5,8 @@
 //   InPlaceKvSdpa / State     transformers/src/ops/inplace_kv_cache.rs:131-290
 //   Sdpa                      transformers/src/ops/sdpa.rs:83-89, 296-356
 //   runtime_for_name          core/src/runtime.rs:223-250
+//   QuantizedDynKeyValueCache / State   transformers/src/ops/quant_dyn_kv_cache.rs:283-495
+//   QuantizedKvSdpa / State             transformers/src/ops/kv_quant.rs:242-355
 // Every failing ABI call becomes a trocm::Error carrying the library's message, the way a
 // TractResult Err carries its context.
 #pragma once
@@ -314,6 +316,150 @@ struct WindowKvSdpa {
     std::string name() const { return "WindowKvSdpa"; }
     bool is_stateless() const { return false; }
     WindowKvSdpaState state() const { return WindowKvSdpaState(axis, window, scale); }
+};
+
+// One KIVI-style quantised tensor on the device (HeadCache of every (batch, head), quant_dyn_kv_cache.rs:252-281).
+class KiviCache {
+   public:
+    KiviCache() = default;
+    KiviCache(int layout, int bits, int64_t sink_tokens, int64_t batch, int64_t heads, int64_t head_dim) {
+        check(trocm_kivi_cache_create(&h_, layout, bits, sink_tokens, batch, heads, head_dim));
+    }
+    KiviCache(const KiviCache &) = delete;
+    KiviCache &operator=(const KiviCache &) = delete;
+    KiviCache(KiviCache &&o) noexcept { std::swap(h_, o.h_); }
+    KiviCache &operator=(KiviCache &&o) noexcept {
+        std::swap(h_, o.h_);
+        return *this;
+    }
+    ~KiviCache() {
+        if (h_) trocm_kivi_cache_destroy(h_);
+    }
+    bool is_some() const { return h_ != nullptr; }
+    int64_t len() const {
+        int64_t n = 0;
+        if (h_) check(trocm_kivi_cache_len(h_, &n));
+        return n;
+    }
+    size_t memory_bytes() const {
+        size_t n = 0;
+        check(trocm_kivi_cache_memory_bytes(h_, &n));
+        return n;
+    }
+    void append(const DeviceTensor &x) {
+        check(trocm_kivi_cache_append(h_, x.ptr(), (int)x.datum_type(), x.shape()[2], nullptr));
+    }
+    DeviceTensor dequantize(std::vector<int64_t> lead, int64_t head_dim, DatumType dt) const {
+        DeviceTensor out({lead[0], lead[1], len(), head_dim}, dt);
+        check(trocm_kivi_cache_dequantize(h_, out.ptr(), (int)dt, nullptr));
+        return out;
+    }
+    KiviCache clone() const {
+        KiviCache c;
+        check(trocm_kivi_cache_clone(h_, &c.h_, nullptr));
+        return c;
+    }
+    trocm_kivi_cache *handle() const { return h_; }
+
+   private:
+    trocm_kivi_cache *h_ = nullptr;
+};
+
+// quant_dyn_kv_cache.rs:334-495: the state ingests every new token and returns the whole cache, dequantised, in the
+// input's datum type.  Keys (per_channel) freeze per-channel parameters per block of 32 tokens, Values quantise per
+// token; the first 4 tokens stay f32.
+class QuantizedDynKvCacheState {
+   public:
+    QuantizedDynKvCacheState(std::string name, size_t axis, uint32_t bits, bool per_channel)
+        : name_(std::move(name)), axis_(axis), bits_(bits), per_channel_(per_channel) {}
+    DeviceTensor eval(const DeviceTensor &input) {
+        ingest(input);
+        return cache_.dequantize(lead_, d_, input.datum_type());
+    }
+    void load_from(const DeviceTensor &init) { ingest(init); }             // :455-465
+    DeviceTensor save_to() const { return cache_.dequantize(lead_, d_, DatumType::F32); }   // :467-470
+    int64_t resolve_symbols() const { return cache_.len(); }              // :472-474: the past-length symbol
+    QuantizedDynKvCacheState freeze() const {                            // :510-541
+        QuantizedDynKvCacheState f(name_, axis_, bits_, per_channel_);
+        f.lead_ = lead_, f.d_ = d_;
+        if (cache_.is_some()) f.cache_ = cache_.clone();
+        return f;
+    }
+
+   private:
+    void ingest(const DeviceTensor &x) {                                  // :393-423
+        const auto &s = x.shape();
+        if (s.size() != 4) throw Error("quantized KV cache supports rank-4 [B, H, S, D] caches");
+        if (axis_ != 2) throw Error("seq axis must be 2 ([B, H, S, D])");
+        if (!cache_.is_some()) {
+            lead_ = {s[0], s[1]}, d_ = s[3];
+            cache_ = KiviCache(per_channel_ ? TROCM_KIVI_BLOCK_CHANNEL : TROCM_KIVI_PER_TOKEN, (int)bits_, 4, s[0], s[1], s[3]);
+        }
+        if (s[3] != d_ || s[0] != lead_[0] || s[1] != lead_[1]) throw Error("cache shape changed between steps");
+        cache_.append(x);
+    }
+    std::string name_;
+    size_t axis_;
+    uint32_t bits_;
+    bool per_channel_;
+    std::vector<int64_t> lead_;
+    int64_t d_ = 0;
+    KiviCache cache_;
+};
+
+struct QuantizedDynKeyValueCache {
+    std::string name;
+    size_t axis = 2;
+    uint32_t bits = 8;
+    bool per_channel = false;
+    std::string op_name() const { return "QuantizedDynKeyValueCache"; }
+    bool is_stateless() const { return false; }
+    QuantizedDynKvCacheState state() const {
+        if (bits != 4 && bits != 8) throw Error("KV quantization bits must be 4 or 8");
+        return QuantizedDynKvCacheState(name, axis, bits, per_channel);
+    }
+};
+
+// kv_quant.rs:270-355: Keys in per-channel u8 with running parameters, Values in per-token u8, attention over the
+// dequantised cache without a causal mask.  Inputs [Q, K_new, V_new], each [B, H, S, D].
+class QuantizedKvSdpaState {
+   public:
+    explicit QuantizedKvSdpaState(std::optional<float> scale) : scale_(scale) {}
+    DeviceTensor eval(const DeviceTensor &q, const DeviceTensor &k_new, const DeviceTensor &v_new) {
+        const auto &ks = k_new.shape();
+        const auto &qs = q.shape();
+        if (!k.is_some()) {
+            k = KiviCache(TROCM_KIVI_RUNNING_CHANNEL, 8, 0, ks[0], ks[1], ks[3]);
+            v = KiviCache(TROCM_KIVI_PER_TOKEN, 8, 0, ks[0], ks[1], ks[3]);
+        }
+        size_t need = 0;
+        check(trocm_sdpa_workspace_bytes(qs[0], qs[1], qs[2], qs[3], &need));
+        if (!ws_ || ws_->bytes() < need) ws_ = std::make_unique<Workspace>(qs[0], qs[1], qs[2], qs[3]);
+        DeviceTensor out(qs, q.datum_type());
+        check(trocm_quantized_kv_sdpa_eval(q.ptr(), k_new.ptr(), v_new.ptr(), (int)q.datum_type(), qs[1], ks[2], k.handle(),
+                                           v.handle(), out.ptr(), scale_.value_or(NAN), ws_->ptr(), ws_->bytes(), nullptr));
+        return out;
+    }
+    QuantizedKvSdpaState freeze() const {
+        QuantizedKvSdpaState f(scale_);
+        if (k.is_some()) f.k = k.clone(), f.v = v.clone();
+        return f;
+    }
+
+   private:
+    std::optional<float> scale_;
+    std::unique_ptr<Workspace> ws_;
+
+   public:
+    KiviCache k, v;
+};
+
+struct QuantizedKvSdpa {
+    size_t axis = 2;
+    std::optional<float> scale;
+    std::string name() const { return "QuantizedKvSdpa"; }
+    bool is_stateless() const { return false; }
+    QuantizedKvSdpaState state() const { return QuantizedKvSdpaState(scale); }
 };
 
 // RotateHalf / ApplyRope (transformers/src/ops/apply_rope.rs:58-76, 169-176) and Cast on dense tensors;

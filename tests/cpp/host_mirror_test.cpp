@@ -278,6 +278,63 @@ int main() {
             GgmlGemm{}.eval(DeviceTensor::from_host(e.data(), {1, 1, K}, DatumType::F32), w).to_host(got.data());
             for (int j = 0; j < N; j++) EXPECT(got[j] == scales[j] * -8.0f);
         }
+        // quant_cache_accumulates_near_lossless_int8 (quant_dyn_kv_cache.rs:728-756): 40 single-token steps through the
+        // quantised cache op, Values then Keys; every output is the concatenation so far within SuperApproximate
+        // (atol 0.1, rtol 0.05), and here within half an 8-bit step of data in [-0.5, 0.5)
+        for (int per_channel = 0; per_channel < 2; per_channel++) {
+            const int B = 1, H = 2, D = 8;
+            QuantizedDynKvCacheState st = QuantizedDynKeyValueCache{"kv0", 2, 8, per_channel != 0}.state();
+            uint64_t lcg = 3;
+            auto nf = [&]() {
+                lcg = lcg * 6364136223846793005ull + 1;
+                return (float)(lcg >> 40) / (float)(1ull << 24) - 0.5f;
+            };
+            std::vector<float> acc;
+            int len = 0;
+            for (int t = 0; t < 40; t++) {
+                std::vector<float> step((size_t)B * H * D);
+                for (auto &x : step) x = nf();
+                DeviceTensor out = st.eval(DeviceTensor::from_host(step.data(), {B, H, 1, D}, DatumType::F32));
+                concat(acc, len, step, B, H, 1, D);
+                EXPECT(out.shape()[2] == len && st.resolve_symbols() == len);
+                std::vector<float> got(out.len());
+                out.to_host(got.data());
+                for (size_t i = 0; i < got.size(); i++) {
+                    EXPECT(std::fabs(got[i] - acc[i]) <= 0.1f + 0.05f * std::fabs(acc[i]));
+                    EXPECT(std::fabs(got[i] - acc[i]) <= 0.5f / 255.0f + 1e-6f);
+                }
+                if (t < 4) for (size_t i = 0; i < got.size(); i++) EXPECT(got[i] == acc[i]);   // sink tokens are kept in f32
+            }
+            QuantizedDynKvCacheState frozen = st.freeze();
+            EXPECT(frozen.resolve_symbols() == 40);
+        }
+        // quantized_kv_sdpa_runs_in_model (kv_quant.rs:568-650): 10 decode steps of the fused op against f32 attention
+        // over the growing cache, within SuperApproximate
+        {
+            const int B = 1, H = 2, D = 16;
+            QuantizedKvSdpaState st = QuantizedKvSdpa{2, std::nullopt}.state();
+            auto mk = [&](float base) {
+                std::vector<float> v((size_t)B * H * D);
+                for (size_t i = 0; i < v.size(); i++) v[i] = base + std::sin((float)i * 0.013f);
+                return v;
+            };
+            std::vector<float> kf, vf;
+            int len = 0, vlen = 0;
+            for (int t = 0; t < 10; t++) {
+                auto q = mk(9.0f + t * 0.1f), k = mk(1.0f + t * 0.07f), v = mk(5.0f - t * 0.05f);
+                DeviceTensor o = st.eval(DeviceTensor::from_host(q.data(), {B, H, 1, D}, DatumType::F32),
+                                         DeviceTensor::from_host(k.data(), {B, H, 1, D}, DatumType::F32),
+                                         DeviceTensor::from_host(v.data(), {B, H, 1, D}, DatumType::F32));
+                std::vector<float> got(o.len());
+                o.to_host(got.data());
+                concat(kf, len, k, B, H, 1, D);
+                concat(vf, vlen, v, B, H, 1, D);
+                auto want = naive(q, kf, vf, B, H, H, 1, len, D, false);
+                for (size_t i = 0; i < want.size(); i++) EXPECT(std::fabs(want[i] - got[i]) <= 0.1f + 0.05f * std::fabs(want[i]));
+            }
+            EXPECT(st.k.memory_bytes() == (size_t)B * H * (10 * D + D * 8));    // memory_bytes, kv_quant.rs:233-235
+            EXPECT(st.v.memory_bytes() == (size_t)B * H * (10 * D + 10 * 8));   // kv_quant.rs:160-162
+        }
         std::printf("host_mirror_test: all checks passed\n");
         return 0;
     } catch (const std::exception &e) {

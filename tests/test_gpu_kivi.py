@@ -218,3 +218,27 @@ def test_cache_of_the_decode_layer_shape(rt):
                 ref.ingest(s[b:b + 1, h:h + 1])
             assert out[b, h].tobytes() == ref.dequantized()[0, 0].astype(np.float16).tobytes()
             same_state({k: v[b * H + h:b * H + h + 1] for k, v in state.items()}, ref.state(), f"head {b},{h}")
+
+
+def test_running_key_store_prompt_push_equals_token_by_token(rt):
+    """A long run of tokens takes the chunked scan (three passes over 64-token chunks); its codes and parameters are
+    those of the token-by-token push, also on top of earlier state, with NaN, infinities and signed zeros in the data."""
+    rng = np.random.default_rng(8)
+    B, H, D = 1, 3, 40
+    cache = kivi.KiviCache(kivi.KIVI_RUNNING_CHANNEL, 8, 0, B, H, D)
+    ref = orc.KiviCache(True, running=True)
+    for n, mag in ((5, 1.0), (300, 1.0), (1, 1.0), (1000, 3.0), (256, 0.1), (257, 30.0)):
+        x = (rng.standard_normal((B, H, n, D)) * mag).astype(np.float32)
+        x[0, 0, n // 2, 3] = np.nan
+        x[0, 1, n // 3, 4] = 0.0
+        x[0, 1, n // 3 + 1 if n > 1 else 0, 4] = -0.0
+        if n > 600:
+            x[0, 2, 600, 7] = np.inf
+            x[0, 2, 100:200, 9] = np.linspace(5, -50, 100)     # the minimum keeps moving inside and across chunks
+            x[0, 2, 200:, 9] = np.linspace(-50, 400, n - 200)  # then the range keeps growing
+        cache.append(x)
+        ref.ingest(x)
+        got, want = cache.state(), ref.state()
+        assert got["packed"].tobytes() == want["packed"].tobytes(), n
+        assert got["lo"].tobytes() == want["lo"].tobytes() and got["scale"].tobytes() == want["scale"].tobytes(), n
+    assert cache.dequantize(np.float32).to_numpy().tobytes() == ref.dequantized().tobytes()

@@ -188,6 +188,93 @@ __global__ void kivi_running_push_kernel(const SrcT *__restrict__ src, int64_t S
     scale_io[(int64_t)bh * D + c] = scale;
 }
 
+// The same push for a long run of tokens (a prompt), in chunks of kRunChunk tokens that are scanned side by side.
+// The running parameters are prefix results: lo after token t is the first minimal value among lo_before and the tokens
+// up to t (`val < lo` never takes a NaN and keeps the earlier of two equal values), scale after token t is the largest
+// of scale_before and (val_s - lo_s) / 255 over the tokens s <= t whose range is positive.  Three passes over the
+// chunks with two short scans over the chunk results between them give every token the parameters the token-by-token
+// loop would have had at its push.
+constexpr int kRunChunk = 64;
+
+// pass 1: first minimal value of each chunk and channel (+inf for a chunk of NaNs)
+template <typename SrcT>
+__global__ void kivi_run_chunk_min_kernel(const SrcT *__restrict__ src, int64_t S, int n, int D, int n_chunks, float *__restrict__ cmin) {
+    const int bh = blockIdx.z, k = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= D) return;
+    float lo = INFINITY;
+    const int t1 = min(n, (k + 1) * kRunChunk);
+    for (int t = k * kRunChunk; t < t1; t++) {
+        const float val = ld(src + ((int64_t)bh * S + t) * D + c);
+        if (val < lo) lo = val;
+    }
+    cmin[((int64_t)bh * n_chunks + k) * D + c] = lo;
+}
+// scan 1: lo at the start of every chunk (in place), and the final lo into the store
+__global__ void kivi_run_scan_min_kernel(float *__restrict__ cmin, int D, int n_chunks, float *__restrict__ lo_io) {
+    const int bh = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= D) return;
+    float lo = lo_io[(int64_t)bh * D + c];
+    for (int k = 0; k < n_chunks; k++) {
+        float *at = cmin + ((int64_t)bh * n_chunks + k) * D + c;
+        const float m = *at;
+        *at = lo;
+        if (m < lo) lo = m;
+    }
+    lo_io[(int64_t)bh * D + c] = lo;
+}
+// pass 2: the largest scale candidate of each chunk and channel (0 when no token of the chunk has a positive range)
+template <typename SrcT>
+__global__ void kivi_run_chunk_scale_kernel(const SrcT *__restrict__ src, int64_t S, int n, int D, int n_chunks,
+                                            const float *__restrict__ lo_start, float *__restrict__ cmax) {
+    const int bh = blockIdx.z, k = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= D) return;
+    float lo = lo_start[((int64_t)bh * n_chunks + k) * D + c], best = 0.0f;
+    const int t1 = min(n, (k + 1) * kRunChunk);
+    for (int t = k * kRunChunk; t < t1; t++) {
+        const float val = ld(src + ((int64_t)bh * S + t) * D + c);
+        if (val < lo) lo = val;
+        const float range = __fsub_rn(val, lo);
+        if (range > 0.0f) {
+            const float ns = __fdiv_rn(range, 255.0f);
+            if (ns > best) best = ns;
+        }
+    }
+    cmax[((int64_t)bh * n_chunks + k) * D + c] = best;
+}
+// scan 2: scale at the start of every chunk (in place), and the final scale into the store
+__global__ void kivi_run_scan_scale_kernel(float *__restrict__ cmax, int D, int n_chunks, float *__restrict__ scale_io) {
+    const int bh = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= D) return;
+    float scale = scale_io[(int64_t)bh * D + c];
+    for (int k = 0; k < n_chunks; k++) {
+        float *at = cmax + ((int64_t)bh * n_chunks + k) * D + c;
+        const float m = *at;
+        *at = scale;
+        if (m > scale) scale = m;
+    }
+    scale_io[(int64_t)bh * D + c] = scale;
+}
+// pass 3: the codes, every chunk starting from its own parameters
+template <typename SrcT>
+__global__ void kivi_run_chunk_codes_kernel(const SrcT *__restrict__ src, int64_t S, int n, int D, int n_chunks,
+                                            const float *__restrict__ lo_start, const float *__restrict__ scale_start,
+                                            uint8_t *__restrict__ codes, int64_t cap_rows, int64_t row0) {
+    const int bh = blockIdx.z, k = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= D) return;
+    float lo = lo_start[((int64_t)bh * n_chunks + k) * D + c], scale = scale_start[((int64_t)bh * n_chunks + k) * D + c];
+    const int t1 = min(n, (k + 1) * kRunChunk);
+    for (int t = k * kRunChunk; t < t1; t++) {
+        const float val = ld(src + ((int64_t)bh * S + t) * D + c);
+        if (val < lo) lo = val;
+        const float range = __fsub_rn(val, lo);
+        if (range > 0.0f) {
+            const float ns = __fdiv_rn(range, 255.0f);
+            if (ns > scale) scale = ns;
+        }
+        codes[((int64_t)bh * cap_rows + row0 + t) * D + c] = (uint8_t)affine_code(val, lo, scale, 255.0f);
+    }
+}
+
 // ---- the same three steps for head sizes that are a multiple of 8 (and, for the two quantising kernels, 64, 128,
 // ---- 256 or 512 with 16-byte aligned sources): a lane owns 8 consecutive channels, so rows move as 128-bit words
 struct F8 {
@@ -599,8 +686,26 @@ static int kivi_append_t(trocm_kivi_cache *c, const SrcT *src, int64_t S, hipStr
         }
     } else if (rem > 0) {
         if (kivi_ensure_rows(c, c->n_rows + rem, s)) return 1;
-        kivi_running_push_kernel<SrcT><<<dim3((unsigned)((D + 127) / 128), BH), 128, 0, s>>>(src + t0 * D, S, (int)rem, D, c->codes, c->cap_rows, c->n_rows, c->lo, c->scale);
-        TROCM_HIP(hipGetLastError());
+        const int64_t n_chunks = (rem + kRunChunk - 1) / kRunChunk;
+        if (rem >= 4 * kRunChunk && n_chunks <= 65535) {   // a prompt: chunks side by side (scratch: two floats per chunk and channel)
+            float *tmp = nullptr;
+            const size_t plane = (size_t)c->BH * n_chunks * D;
+            TROCM_HIP(hipMalloc((void **)&tmp, plane * 2 * sizeof(float)));
+            const dim3 grid((unsigned)((D + 63) / 64), (unsigned)n_chunks, BH), scan((unsigned)((D + 63) / 64), BH);
+            kivi_run_chunk_min_kernel<SrcT><<<grid, 64, 0, s>>>(src + t0 * D, S, (int)rem, D, (int)n_chunks, tmp);
+            kivi_run_scan_min_kernel<<<scan, 64, 0, s>>>(tmp, D, (int)n_chunks, c->lo);
+            kivi_run_chunk_scale_kernel<SrcT><<<grid, 64, 0, s>>>(src + t0 * D, S, (int)rem, D, (int)n_chunks, tmp, tmp + plane);
+            kivi_run_scan_scale_kernel<<<scan, 64, 0, s>>>(tmp + plane, D, (int)n_chunks, c->scale);
+            kivi_run_chunk_codes_kernel<SrcT><<<grid, 64, 0, s>>>(src + t0 * D, S, (int)rem, D, (int)n_chunks, tmp, tmp + plane, c->codes, c->cap_rows, c->n_rows);
+            const hipError_t launched = hipGetLastError();
+            const hipError_t drained = hipStreamSynchronize(s);   // the scratch is freed here, so the stream drains first
+            (void)hipFree(tmp);
+            TROCM_HIP(launched);
+            TROCM_HIP(drained);
+        } else {
+            kivi_running_push_kernel<SrcT><<<dim3((unsigned)((D + 127) / 128), BH), 128, 0, s>>>(src + t0 * D, S, (int)rem, D, c->codes, c->cap_rows, c->n_rows, c->lo, c->scale);
+            TROCM_HIP(hipGetLastError());
+        }
         c->n_rows += rem;
     }
     c->len += S;
