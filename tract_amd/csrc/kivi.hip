@@ -309,6 +309,23 @@ __device__ __forceinline__ void st8(__half *p, const F8 &x) {
     }
     *reinterpret_cast<uint4 *>(p) = make_uint4(u[0], u[1], u[2], u[3]);
 }
+// streaming stores for the dequantised cache (written once, read by the next kernel from HBM anyway)
+__device__ __forceinline__ void st8_stream(float *p, const F8 &x) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    __builtin_nontemporal_store(f32x4{x.v[0], x.v[1], x.v[2], x.v[3]}, reinterpret_cast<f32x4 *>(p));
+    __builtin_nontemporal_store(f32x4{x.v[4], x.v[5], x.v[6], x.v[7]}, reinterpret_cast<f32x4 *>(p) + 1);
+}
+__device__ __forceinline__ void st8_stream(__half *p, const F8 &x) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    uint32_t u[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float a = x.v[2 * i], b = x.v[2 * i + 1];
+        asm volatile("" : "+v"(a), "+v"(b));
+        u[i] = (uint32_t)__half_as_ushort(__float2half_rn(a)) | ((uint32_t)__half_as_ushort(__float2half_rn(b)) << 16);
+    }
+    __builtin_nontemporal_store(u32x4{u[0], u[1], u[2], u[3]}, reinterpret_cast<u32x4 *>(p));
+}
 // 8 codes of one lane's channels packed as the row stores them: 8 bytes, or 4 bytes of nibble pairs (even index low).
 template <int BITS>
 __device__ __forceinline__ void store_codes8(uint8_t *row, int sub, const uint32_t (&code)[8]) {
@@ -458,7 +475,9 @@ __global__ void kivi_dequant_kernel(KiviView a, DstT *__restrict__ dst) {
 }
 
 // dequant_all for head sizes that are a multiple of 8: a thread owns 8 consecutive channels of one token.
-template <typename DstT, int BITS>
+// STREAM: the output leaves with streaming stores (the op's output, read much later); without it the stores stay in the
+// caches for the attention launch that follows inside trocm_quantized_kv_sdpa_eval.
+template <typename DstT, int BITS, bool STREAM>
 __global__ void __launch_bounds__(256) kivi_dequant_vec_kernel(KiviView a, DstT *__restrict__ dst) {
     const int bh = blockIdx.y;
     const int e = blockIdx.x * blockDim.x + threadIdx.x;
@@ -473,14 +492,11 @@ __global__ void __launch_bounds__(256) kivi_dequant_vec_kernel(KiviView a, DstT 
         const uint8_t *row = a.codes + ((int64_t)bh * a.cap_rows + r) * a.row_bytes;
         uint32_t code[8];
         if (BITS == 8) {
-            const uint2 w = *reinterpret_cast<const uint2 *>(row + c);
+            const uint64_t w = __builtin_nontemporal_load(reinterpret_cast<const uint64_t *>(row + c));
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                code[i] = (w.x >> (8 * i)) & 255u;
-                code[4 + i] = (w.y >> (8 * i)) & 255u;
-            }
+            for (int i = 0; i < 8; i++) code[i] = (uint32_t)(w >> (8 * i)) & 255u;
         } else {
-            const uint32_t w = *reinterpret_cast<const uint32_t *>(row + (c >> 1));
+            const uint32_t w = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(row + (c >> 1)));
 #pragma unroll
             for (int i = 0; i < 8; i++) code[i] = (w >> (4 * i)) & 15u;
         }
@@ -498,7 +514,8 @@ __global__ void __launch_bounds__(256) kivi_dequant_vec_kernel(KiviView a, DstT 
     } else {
         x = ld8(a.residual + ((int64_t)bh * kKeyBlock + (t - a.n_sink - a.n_rows)) * a.D + c);
     }
-    st8(dst + ((int64_t)bh * a.len + t) * a.D + c, x);
+    if (STREAM) st8_stream(dst + ((int64_t)bh * a.len + t) * a.D + c, x);
+    else st8(dst + ((int64_t)bh * a.len + t) * a.D + c, x);
 }
 
 __global__ void kivi_fill_running_kernel(float *lo, float *scale, int64_t n) {
@@ -712,7 +729,7 @@ static int kivi_append_t(trocm_kivi_cache *c, const SrcT *src, int64_t S, hipStr
     return 0;
 }
 
-static int kivi_dequantize(const trocm_kivi_cache *c, void *dst, int dst_dtype, hipStream_t s) {
+static int kivi_dequantize(const trocm_kivi_cache *c, void *dst, int dst_dtype, hipStream_t s, bool stream_out = true) {
     if (c->len == 0) return 0;
     KiviView a;
     a.layout = c->layout;
@@ -730,13 +747,19 @@ static int kivi_dequantize(const trocm_kivi_cache *c, void *dst, int dst_dtype, 
     a.codes = c->codes;
     if (c->D % 8 == 0 && ((uintptr_t)dst & 15) == 0) {
         const dim3 grid8((unsigned)((c->len * (c->D / 8) + 255) / 256), (unsigned)c->BH);
+#define KIVI_DEQ(T, BITS)                                                                          \
+    do {                                                                                           \
+        if (stream_out) kivi_dequant_vec_kernel<T, BITS, true><<<grid8, 256, 0, s>>>(a, (T *)dst); \
+        else kivi_dequant_vec_kernel<T, BITS, false><<<grid8, 256, 0, s>>>(a, (T *)dst);          \
+    } while (0)
         if (dst_dtype == TROCM_F32) {
-            if (c->bits == 8) kivi_dequant_vec_kernel<float, 8><<<grid8, 256, 0, s>>>(a, (float *)dst);
-            else kivi_dequant_vec_kernel<float, 4><<<grid8, 256, 0, s>>>(a, (float *)dst);
+            if (c->bits == 8) KIVI_DEQ(float, 8);
+            else KIVI_DEQ(float, 4);
         } else {
-            if (c->bits == 8) kivi_dequant_vec_kernel<__half, 8><<<grid8, 256, 0, s>>>(a, (__half *)dst);
-            else kivi_dequant_vec_kernel<__half, 4><<<grid8, 256, 0, s>>>(a, (__half *)dst);
+            if (c->bits == 8) KIVI_DEQ(__half, 8);
+            else KIVI_DEQ(__half, 4);
         }
+#undef KIVI_DEQ
         TROCM_HIP(hipGetLastError());
         return 0;
     }
@@ -934,7 +957,7 @@ int trocm_quantized_kv_sdpa_eval(const void *q, const void *k_new, const void *v
             TROCM_HIP(hipMalloc(&c->deq, cap));
             c->deq_bytes = cap;
         }
-        if (kivi_dequantize(c, c->deq, dtype, s)) return 1;
+        if (kivi_dequantize(c, c->deq, dtype, s, false)) return 1;
     }
     const int64_t strides[3] = {k_cache->H * T * D, T * D, D};
     // kv_quant.rs:326-327: FlashSdpaOp { causal: false, scale }
