@@ -823,6 +823,343 @@ __device__ __forceinline__ void decode_mfma_qblock_body(const DecodeDev &p, cons
     wave_records_to_output<D, GP>(p, wk, lds_raw, head0, g, tid);
 }
 
+// The same block-scaling arithmetic for up to 4 heads per kv head, with no idle column in the 16-wide tiles: column
+// c = 4 blk + h of a score tile stands for (quantisation block blk, head h).  The 32-deep contraction of one
+// v_mfma_f32_16x16x32_f16 takes 8 features of EACH of a token's four blocks (lane group q4 feeds block q4), and the
+// query operand is block diagonal: column (blk, h) holds head h's features of block blk in the lanes of group blk and
+// zeros elsewhere.  Four such products (one per 8-feature slice j of the blocks) leave, in column (blk, h), the sum
+// over block blk alone -- what the block-scaling body keeps in four accumulators -- so that
+//   * a lane scales its four tokens' sums by ONE block's scales (4 multiplications per 16 tokens instead of 16), and the
+//     four blocks of a head are added across lanes (two row rotations);
+//   * the probabilities times the V block scales are ONE operand for all four blocks (column (blk, h) carries
+//     P[t, h] d_v[t, blk]; an output tile of block b is read off the columns (b, h)): 4 packed multiplications and 4
+//     dot products per tile where the block-scaling body needs 16 + 16, and no shuffling of scales at all, because
+//     the scale tiles are kept transposed in LDS ([block][token]: a lane's four tokens are one 8-byte read).
+// Matrix instructions, code unpacking and LDS traffic per tile are those of the block-scaling body.
+// Eight nibbles of a word as eight halves with one shift and four and-or: (w & 0x000F000F) | 0x64006400 is the pair
+// (1024 + n0, 1024 + n4), (w & 0x00F000F0) | 0x64006400 the pair (1024 + 16 n1, 1024 + 16 n5), and w >> 8 brings n2, n6
+// and n3, n7 to the same places.  For a word of four Q4_0 bytes b0..b3 (low nibble = one element, high nibble = another):
+// halves (lo0, lo2), 16 (hi0, hi2), (lo1, lo3), 16 (hi1, hi3).
+__device__ __forceinline__ void nibbles8(uint32_t w, uint32_t &lo02, uint32_t &hi02, uint32_t &lo13, uint32_t &hi13) {
+    const uint32_t t = w >> 8;
+    lo02 = (w & 0x000F000Fu) | 0x64006400u, hi02 = (w & 0x00F000F0u) | 0x64006400u;
+    lo13 = (t & 0x000F000Fu) | 0x64006400u, hi13 = (t & 0x00F000F0u) | 0x64006400u;
+}
+
+template <int GP, int FMT, int PF>
+__device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const MfmaWork &wk) {
+    static_assert(GP == 8, "partial records are 8 rows wide; rows 0..3 are used");
+    static_assert(FMT == TROCM_Q8_0 || FMT == TROCM_Q4_0, "block-quantised caches only");
+    constexpr int D = 128;
+    constexpr bool Q8 = FMT == TROCM_Q8_0;
+    constexpr int NB = D / 32;                 // blocks per token row
+    constexpr int RB = Q8 ? D : D / 2;         // code bytes per token row
+    constexpr int NLD = kTile * RB / 1024;     // 128-bit loads per lane, tile and tensor: 4 / 2
+    constexpr int CPR = RB / 16;               // 16-byte chunks per row: 8 / 4
+    constexpr int SROW = NB * 2;               // bytes of block scales per row
+    constexpr int kCodeBytes = kTile * RB;     // one tensor's tile in LDS
+    constexpr int kScaleBytes = kTile * SROW;
+    constexpr int kWaveBytes = 2 * kCodeBytes + 2 * kScaleBytes;
+    constexpr int kCombStride = GP * D + 2 * GP;
+    constexpr int kLdsBytes = kWaves * (kWaveBytes > kCombStride * 4 ? kWaveBytes : kCombStride * 4);
+    __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kLdsBytes];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l16 = lane & 15, q4 = lane >> 4;
+    const int blk_c = l16 >> 2, h_c = l16 & 3;   // this lane's column: (block, head)
+    const int kvh = wk.kvh, b = wk.seq;
+    const int g = p.g_real;
+    unsigned char *lds_k = lds_raw + w * kWaveBytes, *lds_v = lds_k + kCodeBytes;
+    unsigned char *lds_ks = lds_v + kCodeBytes, *lds_vs = lds_ks + kScaleBytes;   // scales, transposed: [block][token] f16
+
+    const int64_t head0 = (int64_t)b * p.Hq + (int64_t)kvh * g;
+    const _Float16 *qrow = reinterpret_cast<const _Float16 *>(p.q) + (head0 + min(h_c, g - 1)) * D;
+    const int T = wk.T;
+    const int tile_begin = wk.tile_begin, tile_end = wk.tile_end;
+
+    u32x4 kpre[PF][NLD], vpre[PF][NLD];
+    u32x2 kspre[PF], vspre[PF];
+    auto fetch = [&](const char *base0, const char *sbase0, int t, u32x4 (&dst)[NLD], u32x2 &sc) {
+        const int t0 = t * kTile;
+        const char *base = base0 + (int64_t)t0 * RB;
+        const char *sbase = sbase0 + (int64_t)t0 * SROW;
+        if (t0 + kTile <= T) {
+#pragma unroll
+            for (int j = 0; j < NLD; j++)
+                dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + (j * 64 + lane) * 16));
+            if (lane < kTile) sc = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(sbase + lane * SROW));
+        } else {   // rows past the end of the sequence repeat its last token (their scores are masked below)
+            const int last = T - 1 - t0;
+#pragma unroll
+            for (int j = 0; j < NLD; j++) {
+                const int c = j * 64 + lane, row = min(c / CPR, last), dc = c % CPR;
+                dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + row * RB + dc * 16));
+            }
+            if (lane < kTile) sc = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(sbase + min(lane, last) * SROW));
+        }
+    };
+    // code tiles in LDS exactly as in the block-scaling body (16-byte chunks of a row permuted by a key of the row)
+    auto key_k = [](int row) { return Q8 ? (row & 7) : ((row >> 1) & 3); };
+    auto key_v = [](int row) { return Q8 ? ((row & 3) | (((row >> 4) & 1) << 2)) : (((row >> 1) & 1) | (((row >> 4) & 1) << 1)); };
+    uint32_t k_slot[NLD], v_slot[NLD];
+#pragma unroll
+    for (int j = 0; j < NLD; j++) {
+        const int c = j * 64 + lane, row = c / CPR, dc = c % CPR;
+        k_slot[j] = row * RB + 16 * (dc ^ key_k(row));
+        v_slot[j] = row * RB + 16 * (dc ^ key_v(row));
+    }
+    const int tstep = wk.tile_step;
+    int t = tile_begin + w;
+#pragma unroll
+    for (int st = 0; st < PF; st++) {
+        kspre[st] = vspre[st] = u32x2{0u, 0u};
+        if (t + st * tstep < tile_end) {
+            fetch(wk.kbase, wk.ksbase, t + st * tstep, kpre[st], kspre[st]);
+            fetch(wk.vbase, wk.vsbase, t + st * tstep, vpre[st], vspre[st]);
+        }
+    }
+
+    // Query operands, one per slice j: in the lanes of group blk_c the 8 features of slice j of block blk_c of head h_c,
+    // zeros in the other lane groups.
+    //   Q8_0: features 32 blk + 8 j + 0..7
+    //   Q4_0: features 32 blk + 4 j + 0..3 (low nibbles) and 32 blk + 16 + 4 j + 0..3 (high nibbles: the codes arrive as
+    //         16 u, so these features are divided by 16 -- exact but for subnormal results)
+    half8_t qf[4];
+    float part = 0.0f;   // what the products add up for a block of all-zero-point codes
+    const bool mine = q4 == blk_c;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        half8_t f = {0, 0, 0, 0, 0, 0, 0, 0};
+        if constexpr (Q8) {
+            const half8_t x = *reinterpret_cast<const half8_t *>(qrow + 32 * blk_c + 8 * j);
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) sum += (float)x[i];
+            if (mine) f = x, part += 1152.0f * sum;   // byte ^ 0x80 = code + 128 under 1024
+        } else {
+            const half4_t lo = *reinterpret_cast<const half4_t *>(qrow + 32 * blk_c + 4 * j);
+            const half4_t hi = *reinterpret_cast<const half4_t *>(qrow + 32 * blk_c + 16 + 4 * j);
+            half8_t x;
+            float s_lo = 0.0f, s_hi = 0.0f, s_hi16 = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const _Float16 h16 = hi[i] * (_Float16)0.0625f;
+                // the order in which nibbles8() delivers the codes of a word: (lo0, lo2), (hi0, hi2), (lo1, lo3), (hi1, hi3)
+                const int at = 4 * (i & 1) + (i >> 1);
+                x[at] = lo[i], x[2 + at] = h16;
+                s_lo += (float)lo[i], s_hi16 += (float)h16, s_hi += 16.0f * (float)h16;
+            }
+            if (mine) f = x, part += 1024.0f * (s_lo + s_hi16) + 8.0f * (s_lo + s_hi);
+        }
+        qf[j] = f;
+    }
+    part += __shfl_xor(part, 16, 64);   // the one lane group that holds the column's features hands the sum to the others
+    part += __shfl_xor(part, 32, 64);
+    const float bias = -part;
+#pragma unroll
+    for (int j = 0; j < 4; j++) asm volatile("" : "+v"(qf[j]));   // settled here, not at first use inside the loop
+
+    float m_run = -INFINITY, l_run = 0.0f;   // log2 domain, already scaled
+    float4_t o16[D / 16];
+    float sp = 0.0f;
+#pragma unroll
+    for (int fb = 0; fb < D / 16; fb++) o16[fb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // K fragment of this lane for slice j: token 16 mb + l16 (its key does not depend on mb), block q4, the bytes of
+    // slice j: Q8_0 chunk 2 q4 + j / 2, half j % 2; Q4_0 chunk q4, word j
+    uint32_t k_frag[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        k_frag[j] = Q8 ? l16 * RB + 16 * ((2 * q4 + (j >> 1)) ^ key_k(l16)) + 8 * (j & 1) : l16 * RB + 16 * (q4 ^ key_k(l16)) + 4 * j;
+    // V^T fragments: as in the block-scaling body
+    const int vk = l16 >> 1, v_tok = vk < 4 ? 4 * q4 + vk : 12 + 4 * q4 + vk;
+    const unsigned char *v_row = lds_v + v_tok * RB + 8 * (l16 & 1);
+    const uint32_t v_key16 = 16 * key_v(v_tok);
+    // block scales of this lane's tokens 16 mb + 4 q4 + 0..3 in its block blk_c: 8 contiguous bytes per mb
+    const unsigned char *ks_frag = lds_ks + (blk_c * kTile + 4 * q4) * 2, *vs_frag = lds_vs + (blk_c * kTile + 4 * q4) * 2;
+    // where token `lane` goes in a row of the scale tiles: Q4_0 pairs tokens (0, 2) and (1, 3) of a group of four, the
+    // order in which nibbles8() delivers the V codes (and so the order of the probabilities in their operand)
+    const int sc_pos = Q8 ? lane : ((lane & ~3) | ((lane & 1) << 1) | ((lane >> 1) & 1));
+    const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+    auto ror_add = [](float x, auto ctrl_tag) {   // x + (x of the lane `n` places on in its row of 16 lanes)
+        constexpr int ctrl = decltype(ctrl_tag)::value;
+        const int y = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), ctrl, 0xf, 0xf, false);
+        return x + __builtin_bit_cast(float, y);
+    };
+
+    const float c_log2 = p.scale_log2;   // > 0 (checked on the host): the maximum is taken before scaling
+    auto do_tile = [&](auto stage_tag, int t) {
+        constexpr int ST = decltype(stage_tag)::value;
+        const int t0 = t * kTile;
+        const bool more = t + PF * tstep < tile_end;
+        // ---- this tile's codes and scales -> LDS, the tile PF steps on into flight --------------------------------
+#pragma unroll
+        for (int j = 0; j < NLD; j++) {
+            *reinterpret_cast<u32x4 *>(lds_k + k_slot[j]) = kpre[ST][j];
+            *reinterpret_cast<u32x4 *>(lds_v + v_slot[j]) = vpre[ST][j];
+        }
+        if (lane < kTile) {   // token `lane`: its four block scales to the four block rows of the transposed tiles
+            uint16_t *ksT = reinterpret_cast<uint16_t *>(lds_ks) + sc_pos, *vsT = reinterpret_cast<uint16_t *>(lds_vs) + sc_pos;
+            ksT[0] = (uint16_t)kspre[ST].x, ksT[kTile] = (uint16_t)(kspre[ST].x >> 16);
+            ksT[2 * kTile] = (uint16_t)kspre[ST].y, ksT[3 * kTile] = (uint16_t)(kspre[ST].y >> 16);
+            vsT[0] = (uint16_t)vspre[ST].x, vsT[kTile] = (uint16_t)(vspre[ST].x >> 16);
+            vsT[2 * kTile] = (uint16_t)vspre[ST].y, vsT[3 * kTile] = (uint16_t)(vspre[ST].y >> 16);
+        }
+        if (more) {
+            fetch(wk.kbase, wk.ksbase, t + PF * tstep, kpre[ST], kspre[ST]);
+            fetch(wk.vbase, wk.vsbase, t + PF * tstep, vpre[ST], vspre[ST]);
+        }
+        // ---- codes x block-diagonal query operands: column (blk, h) receives the sum over block blk ----------------------
+        float4_t acc[2];
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++) {
+            acc[mb] = float4_t{bias, bias, bias, bias};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                half8_t kf;
+                if constexpr (Q8) {
+                    const u32x2 c = *reinterpret_cast<const u32x2 *>(lds_k + k_frag[j] + 16 * mb * RB);
+                    kf = magic8(c.x ^ 0x80808080u, c.y ^ 0x80808080u);
+                } else {
+                    const uint32_t c = *reinterpret_cast<const uint32_t *>(lds_k + k_frag[j] + 16 * mb * RB);
+                    uint32_t r0, r1, r2, r3;
+                    nibbles8(c, r0, r1, r2, r3);
+                    kf = __builtin_bit_cast(half8_t, u32x4{r0, r1, r2, r3});
+                }
+                acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[j], acc[mb], 0, 0, 0);
+            }
+        }
+        // ---- scores (before the softmax scale) of tokens 16 mb + 4 q4 + r for head h_c: this block's share, then all four --
+        float sc8[8];
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++) {
+            const u32x2 dk = *reinterpret_cast<const u32x2 *>(ks_frag + 32 * mb);   // scales of tokens r = 0, 1 | 2, 3
+            const half2_t da = as_half2(dk.x), db = as_half2(dk.y);
+            // (Q4_0: the scale tiles hold a group of four tokens in the order 0, 2, 1, 3)
+            const _Float16 dv[4] = {da[0], Q8 ? da[1] : db[0], Q8 ? db[0] : da[1], db[1]};
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                float sv = __builtin_fmaf((float)dv[r], acc[mb][r], 0.0f);
+                sv = ror_add(sv, std::integral_constant<int, 0x124>{});   // row_ror:4
+                sv = ror_add(sv, std::integral_constant<int, 0x128>{});   // row_ror:8
+                sc8[4 * mb + r] = sv;
+            }
+        }
+        if (t0 + kTile > T) {   // the sequence's last tile: tokens past its end do not count
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (t0 + 16 * (i >> 2) + 4 * q4 + (i & 3) >= T) sc8[i] = -INFINITY;
+        }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; i++) tmax = fmaxf(tmax, sc8[i]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m_run, tmax * c_log2);   // finite: every tile holds at least one valid token
+        float psum = 0.0f;
+        half2_t pf[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            // Q8_0: tokens (2i, 2i + 1) of the lane's eight; Q4_0: (0, 2), (1, 3), (4, 6), (5, 7)
+            const int ia = Q8 ? 2 * i : 4 * (i >> 1) + (i & 1), ib = Q8 ? 2 * i + 1 : ia + 2;
+            const float p0 = fast_exp2(__builtin_fmaf(sc8[ia], c_log2, -m_new)), p1 = fast_exp2(__builtin_fmaf(sc8[ib], c_log2, -m_new));
+            psum += p0 + p1;
+            pf[i] = half2_t{(_Float16)p0, (_Float16)p1};
+        }
+        const bool moved = m_new != m_run;
+        const float alpha = fast_exp2(m_run - m_new);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+            for (int fb = 0; fb < D / 16; fb++) o16[fb] *= alpha;
+            sp *= alpha;
+        }
+        // ---- probabilities times the V scales of their tokens in block blk_c: one operand for all four blocks ---------------
+        // pf[i] holds two tokens of 4 q4 + 0..3 for i < 2 and of 16 + 4 q4 + 0..3 for i >= 2, the scale tiles the same pairs
+        u32x4 pw;
+        {
+            const u32x2 e0 = *reinterpret_cast<const u32x2 *>(vs_frag), e1 = *reinterpret_cast<const u32x2 *>(vs_frag + 32);
+            const uint32_t ev[4] = {e0.x, e0.y, e1.x, e1.y};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const half2_t pp = pf[i] * as_half2(ev[i]);
+                sp = __builtin_amdgcn_fdot2(pp, ones, sp, false);
+                pw[i] = __builtin_bit_cast(uint32_t, pp);
+            }
+        }
+        const half8_t pb = __builtin_bit_cast(half8_t, pw);
+        // ---- O^T += codes^T x scaled probabilities: the tile of block blk is right in the columns (blk, h) -------------------
+#pragma unroll
+        for (int blk = 0; blk < NB; blk++) {
+            if constexpr (Q8) {
+#pragma unroll
+                for (int hf = 0; hf < 2; hf++) {
+                    uint32_t w0, w1;
+                    lds_read_tr8(v_row + ((32 * blk + 16 * hf) ^ v_key16), w0, w1);
+                    const half8_t vf = magic8(w0 ^ 0x80808080u, w1 ^ 0x80808080u);
+                    o16[2 * blk + hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pb, o16[2 * blk + hf], 0, 0, 0);
+                }
+            } else {
+                uint32_t w0, w1;   // byte l16 of the block's 16: feature l16 in the low nibble, 16 + l16 in the high one
+                lds_read_tr8(v_row + ((16 * blk) ^ v_key16), w0, w1);
+                uint32_t la, ha, lb, hb2, lc, hc, ld2, hd;   // tokens (0, 2), (1, 3) of w0's four, then of w1's
+                nibbles8(w0, la, ha, lb, hb2);
+                nibbles8(w1, lc, hc, ld2, hd);
+                const half8_t vlo = __builtin_bit_cast(half8_t, u32x4{la, lb, lc, ld2}), vhi = __builtin_bit_cast(half8_t, u32x4{ha, hb2, hc, hd});
+                o16[2 * blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vlo, pb, o16[2 * blk], 0, 0, 0);
+                o16[2 * blk + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vhi, pb, o16[2 * blk + 1], 0, 0, 0);
+            }
+        }
+    };
+    static_assert(PF <= 2, "stages are written out");
+    while (t < tile_end) {
+        do_tile(std::integral_constant<int, 0>{}, t);
+        t += tstep;
+        if constexpr (PF > 1) {
+            if (t < tile_end) do_tile(std::integral_constant<int, 1>{}, t), t += tstep;
+        }
+    }
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    // the zero points of this lane's column: O[f, h] -= (1024 + zero) * SP[h, blk] (Q4_0's high features arrived 16 times
+    // too large); only the tiles of block blk_c are read off this column
+    sp += __shfl_xor(sp, 16, 64);
+    sp += __shfl_xor(sp, 32, 64);
+#pragma unroll
+    for (int blk = 0; blk < NB; blk++) {
+        if constexpr (Q8) {
+            o16[2 * blk] -= 1152.0f * sp;
+            o16[2 * blk + 1] -= 1152.0f * sp;
+        } else {
+            o16[2 * blk] -= 1032.0f * sp;
+            o16[2 * blk + 1] = o16[2 * blk + 1] * 0.0625f - 72.0f * sp;
+        }
+    }
+
+    // ---- merge the 4 waves through LDS (the tiles are dead): rows 0..3 are the heads, rows 4..7 neutral records -----------
+    __syncthreads();
+    float *comb = reinterpret_cast<float *>(lds_raw);   // [kWaves][GP*D + 2*GP]
+    {
+        float *cw = comb + w * kCombStride;
+        const float4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int fb = 0; fb < D / 16; fb++)
+            if ((fb >> 1) == blk_c) {
+                *reinterpret_cast<float4_t *>(cw + h_c * D + 16 * fb + 4 * q4) = o16[fb];
+                *reinterpret_cast<float4_t *>(cw + (4 + h_c) * D + 16 * fb + 4 * q4) = zero4;
+            }
+        if (q4 == 0 && blk_c == 0) {
+            cw[GP * D + h_c] = m_run;
+            cw[GP * D + GP + h_c] = l_run;
+            cw[GP * D + 4 + h_c] = -INFINITY;
+            cw[GP * D + GP + 4 + h_c] = 0.0f;
+        }
+    }
+    wave_records_to_output<D, GP>(p, wk, lds_raw, head0, g, tid);
+}
+
 // The reference states a ragged batch as a dense batch padded to the longest sequence, with a mask row per
 // sequence whose padded columns hold the format's minimum or -inf (flash_sdpa.rs:261-268).  The tokens of such a
 // suffix weigh exactly nothing (their exponentials underflow to zero next to any token that counts), so the
@@ -853,7 +1190,7 @@ __device__ __forceinline__ int mask_row_len(const _Float16 *__restrict__ row, in
 // Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.
 // QB: quantised caches on the 16-wide tiles run the body that scales per block outside the products.
 template <int D, int GP, int FMT, bool MASK = false, bool W16 = false, int QB = 0>
-__global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma_kernel(DecodeDev p) {
+__global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma_kernel(DecodeDev p) {   // QB = 100 * diagonal + 10 * tiles ahead + workgroups per CU
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     MfmaWork wk;
     wk.seq = b, wk.kvh = kvh;
@@ -888,7 +1225,9 @@ __global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma
     wk.counter = p.counters ? p.counters + bh : nullptr;
     wk.part_first = bh * p.nsplit, wk.part_stride = 1;
     wk.mask = MASK ? p.mask + (int64_t)b * p.mask_stride_b + (int64_t)kvh * p.g_real * p.mask_stride_h : nullptr;
-    if constexpr (QB != 0)
+    if constexpr (QB >= 100)
+        decode_mfma_qdiag_body<GP, FMT, (QB / 10) % 10>(p, wk);
+    else if constexpr (QB != 0)
         decode_mfma_qblock_body<GP, FMT, QB / 10>(p, wk);
     else
         decode_mfma_body<D, GP, FMT, MASK, W16>(p, wk);
@@ -916,7 +1255,9 @@ __global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma
     wk.counter = p.counters ? p.counters + (int64_t)it.seq * p.Hkv + kvh : nullptr;
     wk.part_first = (int64_t)it.slot0 * p.Hkv + kvh, wk.part_stride = p.Hkv;
     wk.mask = nullptr;
-    if constexpr (QB != 0)
+    if constexpr (QB >= 100)
+        decode_mfma_qdiag_body<GP, FMT, (QB / 10) % 10>(p, wk);
+    else if constexpr (QB != 0)
         decode_mfma_qblock_body<GP, FMT, QB / 10>(p, wk);
     else
         decode_mfma_body<D, GP, FMT, false, W16>(p, wk);
@@ -941,8 +1282,19 @@ bool use_block_scaling() {
 // The block-scaling kernel keeps one tile (Q8_0) or two (Q4_0: half the bytes per tile) ahead in registers, two
 // workgroups per compute unit.  Measured at batch 8, 16384 tokens: a tile more ahead 52.1 -> 54.6 us (Q8_0) and 37.7 ->
 // 39.2 us (Q4_0); three workgroups per compute unit (Q4_0, 162 registers) 39.2 us.
+// Up to 4 heads per kv head take the diagonal body (decode_mfma_qdiag_body) unless TROCM_DECODE_QDIAG=0.
+bool use_diagonal() {
+    static const int on = getenv("TROCM_DECODE_QDIAG") ? atoi(getenv("TROCM_DECODE_QDIAG")) : 1;
+    return on != 0;
+}
 template <int GP, int FMT>
 void launch_qblock(const DecodeDev &p, dim3 grid, hipStream_t s) {
+    if constexpr (GP == 8) {
+        if (p.g_real <= 4 && use_diagonal()) {
+            hipLaunchKernelGGL((sdpa_decode_mfma_kernel<128, GP, FMT, false, true, (FMT == TROCM_Q8_0 ? 112 : 122)>), grid, dim3(kThreads), 0, s, p);
+            return;
+        }
+    }
     hipLaunchKernelGGL((sdpa_decode_mfma_kernel<128, GP, FMT, false, true, (FMT == TROCM_Q8_0 ? 12 : 22)>), grid, dim3(kThreads), 0, s, p);
 }
 
@@ -987,7 +1339,10 @@ template <int D, int GP, int FMT = TROCM_F16>
 int launch_ragged_gp(const DecodeDev &p, const RaggedItem *items, int n_items, const RaggedSeqSlots *seqs, int n_seq,
                      bool any_split, hipStream_t s) {
     if (FMT != TROCM_F16 && D == 128 && GP <= 16 && use_16_wide(FMT) && use_block_scaling() && p.scale_log2 > 0.0f)
-        hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<128, (GP <= 16 ? GP : 16), (FMT != TROCM_F16 ? FMT : TROCM_Q8_0), true, (FMT == TROCM_Q4_0 ? 22 : 12)>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+        if (GP == 8 && p.g_real <= 4 && use_diagonal())
+            hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<128, 8, (FMT != TROCM_F16 ? FMT : TROCM_Q8_0), true, (FMT == TROCM_Q4_0 ? 122 : 112)>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+        else
+            hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<128, (GP <= 16 ? GP : 16), (FMT != TROCM_F16 ? FMT : TROCM_Q8_0), true, (FMT == TROCM_Q4_0 ? 22 : 12)>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
     else if (GP <= 16 && use_16_wide(FMT))
         hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<D, (GP <= 16 ? GP : 16), FMT, true>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
     else
