@@ -839,11 +839,21 @@ __device__ __forceinline__ void decode_mfma_qblock_body(const DecodeDev &p, cons
 // Eight nibbles of a word as eight halves with one shift and four and-or: (w & 0x000F000F) | 0x64006400 is the pair
 // (1024 + n0, 1024 + n4), (w & 0x00F000F0) | 0x64006400 the pair (1024 + 16 n1, 1024 + 16 n5), and w >> 8 brings n2, n6
 // and n3, n7 to the same places.  For a word of four Q4_0 bytes b0..b3 (low nibble = one element, high nibble = another):
-// halves (lo0, lo2), 16 (hi0, hi2), (lo1, lo3), 16 (hi1, hi3).
-__device__ __forceinline__ void nibbles8(uint32_t w, uint32_t &lo02, uint32_t &hi02, uint32_t &lo13, uint32_t &hi13) {
+// halves (lo0, lo2), 16 (hi0, hi2), (lo1, lo3), 16 (hi1, hi3).  The three constants come in vector registers (laundered
+// through an empty asm once per kernel): as literals, v_and_or_b32 cannot take two of them and the compiler emits an and
+// and an or instead.
+struct NibbleConsts {
+    uint32_t lo, hi, magic;
+};
+__device__ __forceinline__ NibbleConsts nibble_consts() {
+    NibbleConsts c = {0x000F000Fu, 0x00F000F0u, 0x64006400u};
+    asm volatile("" : "+v"(c.lo), "+v"(c.hi), "+v"(c.magic));
+    return c;
+}
+__device__ __forceinline__ void nibbles8(const NibbleConsts &c, uint32_t w, uint32_t &lo02, uint32_t &hi02, uint32_t &lo13, uint32_t &hi13) {
     const uint32_t t = w >> 8;
-    lo02 = (w & 0x000F000Fu) | 0x64006400u, hi02 = (w & 0x00F000F0u) | 0x64006400u;
-    lo13 = (t & 0x000F000Fu) | 0x64006400u, hi13 = (t & 0x00F000F0u) | 0x64006400u;
+    lo02 = (w & c.lo) | c.magic, hi02 = (w & c.hi) | c.magic;
+    lo13 = (t & c.lo) | c.magic, hi13 = (t & c.hi) | c.magic;
 }
 
 template <int GP, int FMT, int PF>
@@ -982,6 +992,7 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
     // order in which nibbles8() delivers the V codes (and so the order of the probabilities in their operand)
     const int sc_pos = Q8 ? lane : ((lane & ~3) | ((lane & 1) << 1) | ((lane >> 1) & 1));
     const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+    const NibbleConsts nc = nibble_consts();
     auto ror_add = [](float x, auto ctrl_tag) {   // x + (x of the lane `n` places on in its row of 16 lanes)
         constexpr int ctrl = decltype(ctrl_tag)::value;
         const int y = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), ctrl, 0xf, 0xf, false);
@@ -1024,7 +1035,7 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
                 } else {
                     const uint32_t c = *reinterpret_cast<const uint32_t *>(lds_k + k_frag[j] + 16 * mb * RB);
                     uint32_t r0, r1, r2, r3;
-                    nibbles8(c, r0, r1, r2, r3);
+                    nibbles8(nc, c, r0, r1, r2, r3);
                     kf = __builtin_bit_cast(half8_t, u32x4{r0, r1, r2, r3});
                 }
                 acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[j], acc[mb], 0, 0, 0);
@@ -1039,13 +1050,16 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
             // (Q4_0: the scale tiles hold a group of four tokens in the order 0, 2, 1, 3)
             const _Float16 dv[4] = {da[0], Q8 ? da[1] : db[0], Q8 ? db[0] : da[1], db[1]};
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                float sv = __builtin_fmaf((float)dv[r], acc[mb][r], 0.0f);
-                sv = ror_add(sv, std::integral_constant<int, 0x124>{});   // row_ror:4
-                sv = ror_add(sv, std::integral_constant<int, 0x128>{});   // row_ror:8
-                sc8[4 * mb + r] = sv;
-            }
+            for (int r = 0; r < 4; r++) sc8[4 * mb + r] = __builtin_fmaf((float)dv[r], acc[mb][r], 0.0f);
         }
+        // the four blocks of a head sit 4 lanes apart in a row of 16 lanes: two rotations add them up in every lane.  (One
+        // stage at a time over all eight values: a rotation must wait two issue slots for its operand, and a value carried
+        // through both stages on its own fills them with s_nop.)
+#pragma unroll
+        for (int i = 0; i < 8; i++) sc8[i] = ror_add(sc8[i], std::integral_constant<int, 0x124>{});   // row_ror:4
+#pragma unroll
+        for (int i = 0; i < 8; i++) sc8[i] = ror_add(sc8[i], std::integral_constant<int, 0x128>{});   // row_ror:8
+
         if (t0 + kTile > T) {   // the sequence's last tile: tokens past its end do not count
 #pragma unroll
             for (int i = 0; i < 8; i++)
@@ -1105,8 +1119,8 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
                 uint32_t w0, w1;   // byte l16 of the block's 16: feature l16 in the low nibble, 16 + l16 in the high one
                 lds_read_tr8(v_row + ((16 * blk) ^ v_key16), w0, w1);
                 uint32_t la, ha, lb, hb2, lc, hc, ld2, hd;   // tokens (0, 2), (1, 3) of w0's four, then of w1's
-                nibbles8(w0, la, ha, lb, hb2);
-                nibbles8(w1, lc, hc, ld2, hd);
+                nibbles8(nc, w0, la, ha, lb, hb2);
+                nibbles8(nc, w1, lc, hc, ld2, hd);
                 const half8_t vlo = __builtin_bit_cast(half8_t, u32x4{la, lb, lc, ld2}), vhi = __builtin_bit_cast(half8_t, u32x4{ha, hb2, hc, hd});
                 o16[2 * blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vlo, pb, o16[2 * blk], 0, 0, 0);
                 o16[2 * blk + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vhi, pb, o16[2 * blk + 1], 0, 0, 0);
