@@ -823,19 +823,6 @@ __device__ __forceinline__ void decode_mfma_qblock_body(const DecodeDev &p, cons
     wave_records_to_output<D, GP>(p, wk, lds_raw, head0, g, tid);
 }
 
-// The same block-scaling arithmetic for up to 4 heads per kv head, with no idle column in the 16-wide tiles: column
-// c = 4 blk + h of a score tile stands for (quantisation block blk, head h).  The 32-deep contraction of one
-// v_mfma_f32_16x16x32_f16 takes 8 features of EACH of a token's four blocks (lane group q4 feeds block q4), and the
-// query operand is block diagonal: column (blk, h) holds head h's features of block blk in the lanes of group blk and
-// zeros elsewhere.  Four such products (one per 8-feature slice j of the blocks) leave, in column (blk, h), the sum
-// over block blk alone -- what the block-scaling body keeps in four accumulators -- so that
-//   * a lane scales its four tokens' sums by ONE block's scales (4 multiplications per 16 tokens instead of 16), and the
-//     four blocks of a head are added across lanes (two row rotations);
-//   * the probabilities times the V block scales are ONE operand for all four blocks (column (blk, h) carries
-//     P[t, h] d_v[t, blk]; an output tile of block b is read off the columns (b, h)): 4 packed multiplications and 4
-//     dot products per tile where the block-scaling body needs 16 + 16, and no shuffling of scales at all, because
-//     the scale tiles are kept transposed in LDS ([block][token]: a lane's four tokens are one 8-byte read).
-// Matrix instructions, code unpacking and LDS traffic per tile are those of the block-scaling body.
 // Eight nibbles of a word as eight halves with one shift and four and-or: (w & 0x000F000F) | 0x64006400 is the pair
 // (1024 + n0, 1024 + n4), (w & 0x00F000F0) | 0x64006400 the pair (1024 + 16 n1, 1024 + 16 n5), and w >> 8 brings n2, n6
 // and n3, n7 to the same places.  For a word of four Q4_0 bytes b0..b3 (low nibble = one element, high nibble = another):
@@ -856,6 +843,19 @@ __device__ __forceinline__ void nibbles8(const NibbleConsts &c, uint32_t w, uint
     lo13 = (t & c.lo) | c.magic, hi13 = (t & c.hi) | c.magic;
 }
 
+// The same block-scaling arithmetic for up to 4 heads per kv head, with no idle column in the 16-wide tiles: column
+// c = 4 blk + h of a score tile stands for (quantisation block blk, head h).  The 32-deep contraction of one
+// v_mfma_f32_16x16x32_f16 takes 8 features of EACH of a token's four blocks (lane group q4 feeds block q4), and the
+// query operand is block diagonal: column (blk, h) holds head h's features of block blk in the lanes of group blk and
+// zeros elsewhere.  Four such products (one per 8-feature slice j of the blocks) leave, in column (blk, h), the sum
+// over block blk alone -- what the block-scaling body keeps in four accumulators -- so that
+//   * a lane scales its four tokens' sums by ONE block's scales (4 multiplications per 16 tokens instead of 16), and the
+//     four blocks of a head are added across lanes (two row rotations);
+//   * the probabilities times the V block scales are ONE operand for all four blocks (column (blk, h) carries
+//     P[t, h] d_v[t, blk]; an output tile of block b is read off the columns (b, h)): 4 packed multiplications and 4
+//     dot products per tile where the block-scaling body needs 16 + 16, and no shuffling of scales at all, because
+//     the scale tiles are kept transposed in LDS ([block][token]: a lane's four tokens are one 8-byte read).
+// Matrix instructions, code unpacking and LDS traffic per tile are those of the block-scaling body.
 template <int GP, int FMT, int PF>
 __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const MfmaWork &wk) {
     static_assert(GP == 8, "partial records are 8 rows wide; rows 0..3 are used");
