@@ -93,7 +93,7 @@ int trocm_copy_nd(void *dst, size_t dst_offset_bytes, const int64_t *dst_strides
  * One cache holds one tensor (K or V) of logical shape [batch, kv_heads, len, head_dim]
  * in a device buffer of `capacity` tokens.  Storage formats:
  *   F32/F16  [batch, kv_heads, capacity, head_dim]
- *   Q8_0     codes [batch, kv_heads, capacity, head_dim] int8  + scales [.., capacity, head_dim/32] f16
+ *   Q8_0     codes [batch, kv_heads, capacity, head_dim] bytes (code + 128) + scales [.., capacity, head_dim/32] f16
  *   Q4_0     codes [batch, kv_heads, capacity, head_dim/2] (16 canonical nibble bytes per block)
  *            + scales [.., capacity, head_dim/32] f16
  * The device layout of the quantised formats is private; trocm_kv_export() emits the

@@ -6,7 +6,9 @@
 // file is compiled with -ffp-contract=off and uses the _rn intrinsics), IEEE division,
 // round-half-away for Q8 codes, truncation for Q4 codes, RNE for the f16 scale.
 //
-// Device layout (private): a code plane with one row per token ([D] int8 for Q8_0,
+// Device layout (private): a code plane with one row per token ([D] bytes for Q8_0, each code + 128 -- offset binary:
+// the attention kernels put a code byte under an exponent byte to make the f16 integer 1024 + byte, and with the sign
+// bit already flipped they do not have to flip it for every byte they read;
 // [D/2] bytes = 16 canonical nibble bytes per block for Q4_0) and a scale plane with
 // D/32 f16 per token, so that decode can read both with aligned 128-bit loads.
 //
@@ -146,8 +148,9 @@ __device__ __forceinline__ void quant_one_block(const QuantAppendDev &a, const S
         uint32_t c[8];
         uint16_t d = quant_q8(v, c);
         uint4 *dst = reinterpret_cast<uint4 *>(a.codes + row * a.D + blk * 32);
-        dst[0] = make_uint4(c[0], c[1], c[2], c[3]);
-        dst[1] = make_uint4(c[4], c[5], c[6], c[7]);
+        constexpr uint32_t x = 0x80808080u;   // the plane holds code + 128
+        dst[0] = make_uint4(c[0] ^ x, c[1] ^ x, c[2] ^ x, c[3] ^ x);
+        dst[1] = make_uint4(c[4] ^ x, c[5] ^ x, c[6] ^ x, c[7] ^ x);
         a.scales[row * nb + blk] = d;
     } else {
         uint32_t c[4];
@@ -196,8 +199,9 @@ __global__ __launch_bounds__(256) void quant_append_ragged_kernel(int fmt, const
             uint32_t c[8];
             const uint16_t d = quant_q8(v, c);
             uint4 *dst = reinterpret_cast<uint4 *>(codes + row * D + blk * 32);
-            dst[0] = make_uint4(c[0], c[1], c[2], c[3]);
-            dst[1] = make_uint4(c[4], c[5], c[6], c[7]);
+            constexpr uint32_t x = 0x80808080u;   // the plane holds code + 128
+            dst[0] = make_uint4(c[0] ^ x, c[1] ^ x, c[2] ^ x, c[3] ^ x);
+            dst[1] = make_uint4(c[4] ^ x, c[5] ^ x, c[6] ^ x, c[7] ^ x);
             scales[row * nb + blk] = d;
         } else {
             uint32_t c[4];
@@ -226,7 +230,8 @@ __global__ __launch_bounds__(256) void quant_export_kernel(int fmt, int64_t BH, 
         const uint16_t *c = reinterpret_cast<const uint16_t *>(codes + (row * nb + blk) * (cw * 2));
         uint16_t *o = dst + ((bh * len + t) * nb + blk) * (1 + cw);
         o[0] = scales[row * nb + blk];
-        for (int i = 0; i < cw; i++) o[1 + i] = c[i];
+        const uint16_t flip = fmt == TROCM_Q8_0 ? 0x8080 : 0;   // Q8_0 planes hold code + 128
+        for (int i = 0; i < cw; i++) o[1 + i] = c[i] ^ flip;
     }
 }
 
@@ -248,7 +253,8 @@ __global__ __launch_bounds__(256) void quant_import_kernel(int fmt, int64_t BH, 
         const uint16_t *i16 = src + ((bh * n + t) * nb + blk) * (1 + cw);
         uint16_t *c = reinterpret_cast<uint16_t *>(codes + (row * nb + blk) * (cw * 2));
         scales[row * nb + blk] = i16[0];
-        for (int i = 0; i < cw; i++) c[i] = i16[1 + i];
+        const uint16_t flip = fmt == TROCM_Q8_0 ? 0x8080 : 0;   // Q8_0 planes hold code + 128
+        for (int i = 0; i < cw; i++) c[i] = i16[1 + i] ^ flip;
     }
 }
 

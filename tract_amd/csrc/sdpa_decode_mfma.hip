@@ -221,10 +221,9 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
             const half2_t d2 = __builtin_bit_cast(half2_t, perm(sc[j], sc[j], sc_sel));
             const u32x4 c = codes[j];
             if constexpr (FMT == TROCM_Q8_0) {
-                const half2_t zero = {(_Float16)1152.0f, (_Float16)1152.0f};   // 1024 + 128: the byte read is code ^ 0x80 = code + 128
-                const uint32_t x = 0x80808080u;
-                *reinterpret_cast<u32x4 *>(tile + slot[j]) = dequant8(c.x ^ x, c.y ^ x, zero, d2);
-                *reinterpret_cast<u32x4 *>(tile + slot[j] + 8) = dequant8(c.z ^ x, c.w ^ x, zero, d2);
+                const half2_t zero = {(_Float16)1152.0f, (_Float16)1152.0f};   // 1024 + 128: the plane holds code + 128
+                *reinterpret_cast<u32x4 *>(tile + slot[j]) = dequant8(c.x, c.y, zero, d2);
+                *reinterpret_cast<u32x4 *>(tile + slot[j] + 8) = dequant8(c.z, c.w, zero, d2);
             } else {
                 // byte i of a block's 16: element i in the low nibble, element 16 + i in the high one
                 const half2_t zero = {(_Float16)1032.0f, (_Float16)1032.0f};   // 1024 + 8
@@ -607,7 +606,7 @@ __device__ __forceinline__ void decode_mfma_qblock_body(const DecodeDev &p, cons
             float sum = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; i++) sum += (float)qf[blk][i];
-            part = 1152.0f * sum;   // byte ^ 0x80 = code + 128 under 1024
+            part = 1152.0f * sum;   // the plane holds code + 128, under 1024
         } else {
             const half4_t lo = *reinterpret_cast<const half4_t *>(qrow + 32 * blk + 4 * q4);
             const half4_t hi = *reinterpret_cast<const half4_t *>(qrow + 32 * blk + 16 + 4 * q4);
@@ -679,7 +678,7 @@ __device__ __forceinline__ void decode_mfma_qblock_body(const DecodeDev &p, cons
                 half8_t kf;
                 if constexpr (Q8) {
                     const u32x2 c = *reinterpret_cast<const u32x2 *>(lds_k + k_frag[blk] + 16 * mb * RB);
-                    kf = magic8(c.x ^ 0x80808080u, c.y ^ 0x80808080u);
+                    kf = magic8(c.x, c.y);   // (the plane holds code + 128)
                 } else {
                     const uint32_t c = *reinterpret_cast<const uint32_t *>(lds_k + k_frag[blk] + 16 * mb * RB);
                     kf = magic8(c & 0x0F0F0F0Fu, c & 0xF0F0F0F0u);
@@ -764,7 +763,7 @@ __device__ __forceinline__ void decode_mfma_qblock_body(const DecodeDev &p, cons
                 for (int hf = 0; hf < 2; hf++) {
                     uint32_t w0, w1;
                     lds_read_tr8(v_row + ((32 * blk + 16 * hf) ^ v_key16), w0, w1);
-                    const half8_t vf = magic8(w0 ^ 0x80808080u, w1 ^ 0x80808080u);
+                    const half8_t vf = magic8(w0, w1);
                     o16[2 * blk + hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pb[blk], o16[2 * blk + hf], 0, 0, 0);
                 }
             } else {
@@ -946,7 +945,7 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
             float sum = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; i++) sum += (float)x[i];
-            if (mine) f = x, part += 1152.0f * sum;   // byte ^ 0x80 = code + 128 under 1024
+            if (mine) f = x, part += 1152.0f * sum;   // the plane holds code + 128, under 1024
         } else {
             const half4_t lo = *reinterpret_cast<const half4_t *>(qrow + 32 * blk_c + 4 * j);
             const half4_t hi = *reinterpret_cast<const half4_t *>(qrow + 32 * blk_c + 16 + 4 * j);
@@ -1031,7 +1030,7 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
                 half8_t kf;
                 if constexpr (Q8) {
                     const u32x2 c = *reinterpret_cast<const u32x2 *>(lds_k + k_frag[j] + 16 * mb * RB);
-                    kf = magic8(c.x ^ 0x80808080u, c.y ^ 0x80808080u);
+                    kf = magic8(c.x, c.y);   // (the plane holds code + 128)
                 } else {
                     const uint32_t c = *reinterpret_cast<const uint32_t *>(lds_k + k_frag[j] + 16 * mb * RB);
                     uint32_t r0, r1, r2, r3;
@@ -1112,7 +1111,7 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
                 for (int hf = 0; hf < 2; hf++) {
                     uint32_t w0, w1;
                     lds_read_tr8(v_row + ((32 * blk + 16 * hf) ^ v_key16), w0, w1);
-                    const half8_t vf = magic8(w0 ^ 0x80808080u, w1 ^ 0x80808080u);
+                    const half8_t vf = magic8(w0, w1);
                     o16[2 * blk + hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pb, o16[2 * blk + hf], 0, 0, 0);
                 }
             } else {

@@ -4,8 +4,8 @@
 // K codes staged through LDS for the transposed read, V codes straight from HBM.
 //
 // Codes become f16 without a per-element conversion instruction: one v_perm_b32 puts two
-// code bytes under the exponent byte 0x64, i.e. forms the halves (1024 + u), u = code ^ 0x80
-// for Q8_0 (so u = code + 128) and u = nibble for Q4_0.
+// code bytes under the exponent byte 0x64, i.e. forms the halves (1024 + u), u = code + 128 for Q8_0
+// (the cache's code plane holds exactly that byte) and u = nibble for Q4_0.
 //   QK : dot2 accumulates sum q_i (1024 + u_i) per 32-element block; the constant part
 //        (1152 or 1032 times the block sum of q, computed once per workgroup) is subtracted
 //        and the block scale d applied:  s += d * (dot - bias * qsum).
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(kThreads, G <= 4 ? 2 : 1) void sdpa_decode_q_kernel
 #pragma unroll
                 for (int cc = 0; cc < 2; cc++) {
                     u32x4 kc = lds_krow[(bl * 2 + cc + qk_rot) & (CPR - 1)];
-                    uint32_t kw[4] = {kc.x ^ 0x80808080u, kc.y ^ 0x80808080u, kc.z ^ 0x80808080u, kc.w ^ 0x80808080u};
+                    uint32_t kw[4] = {kc.x, kc.y, kc.z, kc.w};   // the plane holds code + 128
 #pragma unroll
                     for (int h = 0; h < G; h++) {
                         u32x4 q0 = lds_q[h * QC + blk * 4 + cc * 2], q1 = lds_q[h * QC + blk * 4 + cc * 2 + 1];
@@ -283,8 +283,8 @@ __global__ __launch_bounds__(kThreads, G <= 4 ? 2 : 1) void sdpa_decode_q_kernel
             }
             uint32_t wa[2], wb[2];
             if constexpr (FMT == TROCM_Q8_0) {
-                wa[0] = vreg[ia].x ^ 0x80808080u, wa[1] = vreg[ia].y ^ 0x80808080u;
-                wb[0] = vreg[ib].x ^ 0x80808080u, wb[1] = vreg[ib].y ^ 0x80808080u;
+                wa[0] = vreg[ia].x, wa[1] = vreg[ia].y;   // the plane holds code + 128
+                wb[0] = vreg[ib].x, wb[1] = vreg[ib].y;
             } else {
                 wa[0] = vreg[ia] & 0x0F0F0F0Fu, wa[1] = (vreg[ia] >> 4) & 0x0F0F0F0Fu;
                 wb[0] = vreg[ib] & 0x0F0F0F0Fu, wb[1] = (vreg[ib] >> 4) & 0x0F0F0F0Fu;

@@ -44,7 +44,7 @@ struct KvReader {
     __device__ __forceinline__ float at(int64_t j, int d) const {
         if (fmt == TROCM_Q8_0) {
             float sc = __half2float(__ushort_as_half(scales[j * (D / 32) + d / 32]));
-            return (float)(int8_t)codes[j * D + d] * sc;
+            return (float)((int)codes[j * D + d] - 128) * sc;   // the plane holds code + 128
         }
         if (fmt == TROCM_Q4_0) {
             float sc = __half2float(__ushort_as_half(scales[j * (D / 32) + d / 32]));

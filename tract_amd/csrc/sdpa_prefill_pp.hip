@@ -207,10 +207,9 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
             u32x4 ka, kb2, va, vb2;     // two chunks of 8 halves per tensor
             int dc_a, dc_b;             // their 16-byte chunk indices in the row
             if constexpr (FMT == TROCM_Q8_0) {
-                const half2_t zero = {(_Float16)1152.0f, (_Float16)1152.0f};   // 1024 + 128: codes are stored as code ^ 0x80
-                const uint32_t x = 0x80808080u;
-                ka = dequant8(kpre[0].x ^ x, kpre[0].y ^ x, zero, kd), kb2 = dequant8(kpre[0].z ^ x, kpre[0].w ^ x, zero, kd);
-                va = dequant8(vpre[0].x ^ x, vpre[0].y ^ x, zero, vd), vb2 = dequant8(vpre[0].z ^ x, vpre[0].w ^ x, zero, vd);
+                const half2_t zero = {(_Float16)1152.0f, (_Float16)1152.0f};   // 1024 + 128: the plane holds code + 128
+                ka = dequant8(kpre[0].x, kpre[0].y, zero, kd), kb2 = dequant8(kpre[0].z, kpre[0].w, zero, kd);
+                va = dequant8(vpre[0].x, vpre[0].y, zero, vd), vb2 = dequant8(vpre[0].z, vpre[0].w, zero, vd);
                 dc_a = 2 * q_unit, dc_b = 2 * q_unit + 1;
             } else {
                 const half2_t zero = {(_Float16)1032.0f, (_Float16)1032.0f};   // 1024 + 8
