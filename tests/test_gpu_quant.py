@@ -25,6 +25,18 @@ def _nasty(rng, n_blocks, dt):
     x[5, :] = np.float32(6e-8)  # f16 subnormal scale range
     x[6] = np.arange(32) - 16
     x[7] = -(np.arange(32) - 15.5)
+    # equal magnitudes of both signs: the first element decides the sign of the scale
+    x[8, 0], x[8, 1] = 3.0, -3.0
+    x[9] = -0.0
+    x[10] = np.nan
+    x[11, 3], x[11, 9] = np.inf, -np.inf
+    x[12, 3], x[12, 9] = -np.inf, np.inf
+    m = np.abs(x[13]).max()
+    x[13, 31] = -m if x[13][np.abs(x[13]).argmax()] > 0 else m
+    x[14, 20], x[14, 2] = -5000.0, 5000.0
+    x[15, 0], x[15, 4], x[15, 9] = np.nan, -7000.0, 7000.0
+    x[16, 1:] = np.nan                                   # one number among NaN
+    x[17, :] = -2.5
     return x.astype(dt)
 
 

@@ -37,9 +37,9 @@ template <typename V, typename Index>
 __global__ __launch_bounds__(256) void copy_nd_kernel(char *__restrict__ dst, const char *__restrict__ src,
                                                       CopyDev p, Index total) {
     Index step = (Index)gridDim.x * blockDim.x;
-    for (Index idx = (Index)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += step) {
+    auto offsets = [&](Index idx, int64_t &doff, int64_t &soff) {
         Index rem = idx;
-        int64_t doff = 0, soff = 0;
+        doff = 0, soff = 0;
 #pragma unroll
         for (int d = 5; d >= 0; --d) {
             if (d < p.rank) {
@@ -50,6 +50,11 @@ __global__ __launch_bounds__(256) void copy_nd_kernel(char *__restrict__ dst, co
                 soff += (int64_t)i * p.src_stride[d];
             }
         }
+    };
+    Index idx = (Index)blockIdx.x * blockDim.x + threadIdx.x;
+    for (; idx < total; idx += step) {
+        int64_t doff, soff;
+        offsets(idx, doff, soff);
         stream_copy<sizeof(V)>(dst + doff, src + soff);
     }
 }
@@ -58,7 +63,9 @@ template <typename V>
 int launch_typed(char *dst, const char *src, const CopyDev &p, uint64_t total, hipStream_t s) {
     const int block = 256;
     uint64_t blocks = (total + block - 1) / block;
-    uint64_t max_blocks = (uint64_t)num_compute_units() * 32;
+    // Workgroups per compute unit, measured on a 256 MiB copy (16 bytes per thread and trip): 8: 96.8 us, 16: 95.3, 32: 90.2,
+    // 64: 86.1, 128: 84.3, 256 (one trip per thread): 89.4; two loads in flight per thread did not help.
+    uint64_t max_blocks = (uint64_t)num_compute_units() * 128;
     if (blocks > max_blocks) blocks = max_blocks;
     if (total < (1ull << 31))
         hipLaunchKernelGGL((copy_nd_kernel<V, uint32_t>), dim3((unsigned)blocks), dim3(block), 0, s, dst, src, p,

@@ -45,17 +45,18 @@ __device__ __forceinline__ int cvt_i32_rz_sat(float x) {
 }
 __device__ __forceinline__ int sat_i8(float x) { return max(-128, min(127, cvt_i32_rz_sat(x))); }   // (one v_med3_i32)
 
-// f32::round(): half away from zero, as trunc(x + copysign(0.49999997, x)) with the addition rounded to nearest even.
-// 0.49999997 is the float below 0.5: for a fraction below one half the sum stays under the next integer, at exactly one
-// half the sum lies midway between two floats and ties to the even one, which is the integer; from 2^23 on x + 0.49999997
-// rounds back to x.  Equal to round() for every float (all 2^23 mantissas of every exponent from 2^-3 to 2^24 were
-// compared on the host; below 2^-3 the sum stays under 1, above 2^25 it is x; inf and NaN pass through).
-__device__ __forceinline__ float round_half_away(float x) {
-    return truncf(__fadd_rn(x, __builtin_copysignf(0.49999997f, x)));
+// f32::round() followed by the saturating cast: half away from zero, as the conversion (which truncates) of
+// x + copysign(0.49999997, x) with the addition rounded to nearest even.  0.49999997 is the float below 0.5: for a
+// fraction below one half the sum stays under the next integer, at exactly one half the sum lies midway between two
+// floats and ties to the even one, which is the integer; from 2^23 on x + 0.49999997 rounds back to x.  The sum truncates
+// to round(x) for every float (all 2^23 mantissas of every exponent from 2^-3 to 2^24 were compared on the host; below
+// 2^-3 the sum stays under 1, above 2^25 it is x; inf saturates and NaN gives 0 either way).
+__device__ __forceinline__ int round_half_away_sat_i8(float x) {
+    return sat_i8(__fadd_rn(x, __builtin_copysignf(0.49999997f, x)));
 }
 
-// Signed value of the first element with strictly largest magnitude (q4_0.rs:27-34).
-__device__ __forceinline__ float signed_first_absmax(const float (&v)[32]) {
+// Signed value of the first element with strictly largest magnitude (q4_0.rs:27-34): the element order decides.
+__device__ __forceinline__ float signed_first_absmax_in_order(const float (&v)[32]) {
     float amax = 0.0f, mx = 0.0f;
 #pragma unroll
     for (int i = 0; i < 32; i++) {
@@ -68,6 +69,21 @@ __device__ __forceinline__ float signed_first_absmax(const float (&v)[32]) {
     return mx;
 }
 
+// The same value without the ordered scan where the order cannot matter: the largest and the smallest element (NaN
+// ignored, as the scan's comparison ignores it) are one v_max3 / v_min3 per two elements; whichever has the larger
+// magnitude is the answer.  Equal magnitudes (a +x and a -x, all zeros, nothing but NaN) go through the scan.
+__device__ __forceinline__ float signed_first_absmax(const float (&v)[32]) {
+    float hi = v[0], lo = v[0];
+#pragma unroll
+    for (int i = 1; i < 32; i++) {
+        hi = fmaxf(hi, v[i]);
+        lo = fminf(lo, v[i]);
+    }
+    if (hi > -lo) return hi;
+    if (-lo > hi) return lo;
+    return signed_first_absmax_in_order(v);
+}
+
 // Q8: returns the f16 scale bits, codes packed 4 per word in element order.
 __device__ __forceinline__ uint16_t quant_q8(const float (&v)[32], uint32_t (&codes)[8]) {
     float mx = signed_first_absmax(v);
@@ -78,7 +94,7 @@ __device__ __forceinline__ uint16_t quant_q8(const float (&v)[32], uint32_t (&co
         uint32_t word = 0;
 #pragma unroll
         for (int b = 0; b < 4; b++) {
-            int c = sat_i8(round_half_away(__fmul_rn(v[w * 4 + b], r)));  // q8_1.rs:45
+            int c = round_half_away_sat_i8(__fmul_rn(v[w * 4 + b], r));  // q8_1.rs:45
             word |= (uint32_t)(c & 0xff) << (8 * b);
         }
         codes[w] = word;
@@ -140,10 +156,7 @@ struct QuantAppendDev {
     int nb_shift;   // log2(D / 32) when that is a power of two, else -1
 };
 
-template <typename SrcT>
-__device__ __forceinline__ void quant_one_block(const QuantAppendDev &a, const SrcT *p, int64_t row, int64_t nb, int64_t blk) {
-    float v[32];
-    load_block(p, a.ss[3], a.vec != 0, v);
+__device__ __forceinline__ void quant_store_block(const QuantAppendDev &a, const float (&v)[32], int64_t row, int64_t nb, int64_t blk) {
     if (a.fmt == TROCM_Q8_0) {
         uint32_t c[8];
         uint16_t d = quant_q8(v, c);
@@ -160,18 +173,49 @@ __device__ __forceinline__ void quant_one_block(const QuantAppendDev &a, const S
     }
 }
 
-// Grid (chunks of a (batch, head) row's blocks, batch * heads): the position of a block inside its row is one 32-bit
-// division (a shift when head_dim / 32 is a power of two); with a flat index over all blocks the three 64-bit
-// divisions were 45 % of the kernel's instructions, and the kernel is bound by them, not by HBM.
+template <typename SrcT>
+__device__ __forceinline__ void quant_one_block(const QuantAppendDev &a, const SrcT *p, int64_t row, int64_t nb, int64_t blk) {
+    float v[32];
+    load_block(p, a.ss[3], a.vec != 0, v);
+    quant_store_block(a, v, row, nb, blk);
+}
+
+// Grid (chunks of a (batch, head) row's blocks, batch * heads), one block per thread: the position of a block inside
+// its row is one 32-bit division (a shift when head_dim / 32 is a power of two); with a flat index over all blocks the
+// three 64-bit divisions were 45 % of the kernel's instructions.  Dense sources have a loop of their own: with the
+// choice between 128-bit and element loads inside one loop the same launch measured 82 us instead of 75 us.
 template <typename SrcT>
 __global__ __launch_bounds__(256) void quant_append_kernel(QuantAppendDev a) {
     const uint32_t nb = (uint32_t)(a.D / 32);
     const uint32_t per_row = (uint32_t)a.S * nb;
+    const uint32_t first = blockIdx.x * blockDim.x + threadIdx.x, step = gridDim.x * blockDim.x;
+    constexpr int kWords = 32 * sizeof(SrcT) / 16;
     for (int64_t bh = blockIdx.y; bh < a.B * a.H; bh += gridDim.y) {
         const int64_t b = bh / a.H, h = bh % a.H;   // (scalar: once per workgroup trip)
         const SrcT *src_row = (const SrcT *)a.src + b * a.ss[0] + h * a.ss[1];
         const int64_t row0 = bh * a.cap + a.t0;
-        for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < per_row; i += gridDim.x * blockDim.x) {
+        if (a.vec) {
+            if (first >= per_row) continue;
+            for (uint32_t i = first; i < per_row; i += step) {
+                const uint32_t t = a.nb_shift >= 0 ? i >> a.nb_shift : i / nb;
+                const uint32_t blk = i - t * nb;
+                const uint4 *p = reinterpret_cast<const uint4 *>(src_row + (int64_t)t * a.ss[2] + (int64_t)blk * 32);
+                uint4 w[kWords];
+#pragma unroll
+                for (int k = 0; k < kWords; k++) w[k] = p[k];
+                float v[32];
+                constexpr int kPerWord = 16 / sizeof(SrcT);
+#pragma unroll
+                for (int k = 0; k < kWords; k++) {
+                    const SrcT *e = reinterpret_cast<const SrcT *>(&w[k]);
+#pragma unroll
+                    for (int q = 0; q < kPerWord; q++) v[k * kPerWord + q] = load_elem(e + q);
+                }
+                quant_store_block(a, v, row0 + t, nb, blk);
+            }
+            continue;
+        }
+        for (uint32_t i = first; i < per_row; i += step) {
             const uint32_t t = a.nb_shift >= 0 ? i >> a.nb_shift : i / nb;
             const uint32_t blk = i - t * nb;
             quant_one_block(a, src_row + (int64_t)t * a.ss[2] + (int64_t)blk * 32 * a.ss[3], row0 + t, nb, blk);
@@ -379,13 +423,13 @@ int launch_quant_append(const QuantAppend &a, hipStream_t s) {
     for (int sh = 0; sh < 16; sh++)
         if (nb == (1ll << sh)) d.nb_shift = sh;
     const int64_t per_row = a.S * nb, bh = a.B * a.H;
-    const int64_t want = (int64_t)num_compute_units() * 16;              // workgroups that keep the device busy
-    int64_t gx = (per_row + 255) / 256;
+    // One block per thread whatever the size.  A fixed number of workgroups whose threads walk over several blocks was
+    // measured against it on a 16384-token prefill (8 x 8 heads): 16 workgroups per compute unit and 4 blocks per thread
+    // 82.6 us (Q8_0) / 66.6 us (Q4_0), with the next block requested before the current one is worked on 81.8 / 67.1
+    // (two blocks ahead 86 / 72: fewer waves fit), a contiguous run of blocks per workgroup 87.5 / 70.3, one block per
+    // thread 75-76 / 62-63.  The loops in the kernel only serve launches beyond the grid limits.
+    const int64_t gx = std::min<int64_t>((per_row + 255) / 256, 1 << 22);
     const int64_t gy = bh < 65535 ? bh : 65535;
-    if (gx * gy > want) {   // more workgroups than that: every thread takes several blocks
-        const int64_t per_thread = gx * gy / want;
-        gx = (gx + per_thread - 1) / per_thread;
-    }
     if (a.src_dtype == TROCM_F16)
         hipLaunchKernelGGL(quant_append_kernel<__half>, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, d);
     else
