@@ -525,13 +525,14 @@ def run_kivi(ta, args):
                 got["packed"][at].tobytes() == want["packed"].tobytes() and np.array_equal(got["lo"][at], want["lo"])
                 and np.array_equal(got["scale"][at], want["scale"]) and got["sink"][at].tobytes() == want["sink"].tobytes())
             del caches, outs
-    # QuantizedKvSdpa: one decode step over an 8192-token cache (append, two dequantising reads, attention)
+    # QuantizedKvSdpa: one decode step over an 8192-token cache (two single-token appends, attention straight over the codes)
     Tc = 8192
     st = ta.QuantizedKvSdpa(axis=2).state()
-    kq = ta.DeviceTensor.from_numpy(seeded_f16(cfg_seed(2, "k"), (B, HKV, Tc, D)))
+    kq_np, vq_np = seeded_f16(cfg_seed(2, "k"), (B, HKV, Tc, D)), seeded_f16(cfg_seed(2, "v"), (B, HKV, Tc, D))
+    kq, vq = ta.DeviceTensor.from_numpy(kq_np), ta.DeviceTensor.from_numpy(vq_np)
     st.k = kivi.KiviCache(kivi.KIVI_RUNNING_CHANNEL, 8, 0, B, HKV, D)
     st.v = kivi.KiviCache(kivi.KIVI_PER_TOKEN, 8, 0, B, HKV, D)
-    st.k.append(kq), st.v.append(kq)
+    st.k.append(kq), st.v.append(vq)
 
     def prompt():
         st.k.reset()
@@ -539,16 +540,30 @@ def run_kivi(ta, args):
 
     res["prompt_push_running_keys_8x8x8192x128"] = {"us": round(time_calls(ta, prompt, 8), 2),
                                                     "note": "chunked scan over 64-token chunks; incl. the scratch allocation and the wait before it is freed"}
-    q1 = ta.DeviceTensor.from_numpy((seeded_f16(cfg_seed(2, "q") + 1, (B, HQ, 1, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16))
+    q1_np = (seeded_f16(cfg_seed(2, "q") + 1, (B, HQ, 1, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16)
+    q1 = ta.DeviceTensor.from_numpy(q1_np)
     out = ta.DeviceTensor((B, HQ, 1, D), np.float16)
     us = time_calls(ta, lambda: st.eval([q1, tok, tok], out=out), 32)
-    res["quantized_kv_sdpa_step_b8_ctx8192"] = {"us": round(us, 2), "note": "append + dequantise K and V (u8 -> f16) + f16 decode attention"}
+    T_end = st.k.len()
+    step_bytes = B * HKV * (Tc + (T_end - Tc) // 2) * (2 * D + 8) + B * HKV * D * 8 + 2 * B * HQ * D * 2
+    case = {"us": round(us, 2), "bytes": step_bytes, "gbs": round(step_bytes / us / 1e3, 1),
+            "note": "two single-token appends + attention straight over the u8 codes (TROCM_KIVI_FUSED=0: append + dequantise K and V + f16 attention)"}
+    # after the timing: the last step's output for one kv head against the oracle's attention over its own stores
+    b0, h0, g = 5, 3, HQ // HKV
+    tok_np = tok.to_numpy()
+    kc, vc = orc.KiviCache(True, running=True), orc.KiviCache(False, running=True)
+    kc.ingest(kq_np[b0:b0 + 1, h0:h0 + 1]), vc.ingest(vq_np[b0:b0 + 1, h0:h0 + 1])
+    for _ in range(T_end - Tc):
+        kc.ingest(tok_np[b0:b0 + 1, h0:h0 + 1]), vc.ingest(tok_np[b0:b0 + 1, h0:h0 + 1])
+    want = orc.flash_sdpa(q1_np[b0:b0 + 1, h0 * g:(h0 + 1) * g].astype(np.float32), kc.dequantized(), vc.dequantized(), causal=False)
+    case["parity_max_abs_vs_oracle"] = float(np.abs(out.to_numpy()[b0:b0 + 1, h0 * g:(h0 + 1) * g].astype(np.float32) - want).max())
+    res["quantized_kv_sdpa_step_b8_ctx8192"] = case
     head = res["dequantize_key_block_channel_8bit_8x8x16384x128"]
     roof = {"bound": "hbm", "kernel": "kivi_dequant_kernel<f16, 8>", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(head["gbs"] / HBM_PEAK_GBS, 4), "traffic": None}
     return base_line(args, "kivi: KIVI-style affine quantised caches (8 x 8 kv heads x 16384 tokens x 128, f16): ingest into per-token "
                      "Value and block x channel Key stores at 8 / 4 bits, the dequantising read of the whole cache, one QuantizedKvSdpa "
-                     "decode step at 8192 tokens; headline = the 8-bit Key cache read", head["gbs"], "GB/s", round(head["us"] / 1e3, 5),
+                     "decode step at 8192 tokens (attention over the codes); headline = the 8-bit Key cache read", head["gbs"], "GB/s", round(head["us"] / 1e3, 5),
                      "u8->f16", roof, {"cases": res})
 
 

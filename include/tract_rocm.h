@@ -403,9 +403,11 @@ int trocm_kivi_cache_export(const trocm_kivi_cache *cache, int part, void *dst_d
 int trocm_kivi_cache_clone(const trocm_kivi_cache *cache, trocm_kivi_cache **out, void *stream);
 
 /* QuantizedKvSdpaState::eval (kv_quant.rs:283-330): push k_new and v_new ([batch, kv_heads, n_new, head_dim] dense
- * of `dtype`) into a RUNNING_CHANNEL key store and a PER_TOKEN value store (8 bits, no sink tokens), dequantise
- * both and attend q ([batch, q_heads, n_new, head_dim]) over every stored token WITHOUT a causal mask (:326).  The
- * dequantised copies live in buffers the stores own and grow by doubling. */
+ * of `dtype`) into a RUNNING_CHANNEL key store and a PER_TOKEN value store (8 bits, no sink tokens) and attend q
+ * ([batch, q_heads, n_new, head_dim]) over every stored token WITHOUT a causal mask (:326).  One F16 query token at
+ * head_dim 128 with up to 16 query heads per kv head attends straight over the codes (needs the workspace of
+ * trocm_sdpa_workspace_bytes); every other case dequantises both stores into buffers they own (grown by doubling,
+ * released again at the next step that does not need them) and runs trocm_sdpa over the copies. */
 int trocm_quantized_kv_sdpa_eval(const void *q, const void *k_new, const void *v_new, int dtype, int64_t q_heads,
                                  int64_t n_new, trocm_kivi_cache *k_cache, trocm_kivi_cache *v_cache, void *out,
                                  float scale, void *workspace, size_t workspace_bytes, void *stream);

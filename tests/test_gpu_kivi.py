@@ -197,6 +197,50 @@ def test_quantized_kv_sdpa_gqa_prefill_then_decode(rt, dt, tol):
     assert st.eval([q, k, k]).to_numpy().tobytes() == frozen.eval([q, k, k]).to_numpy().tobytes()
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,T0", [(4, 32, 8, 4100), (1, 32, 8, 8192), (2, 32, 2, 1500), (3, 6, 2, 700)])
+def test_quantized_kv_sdpa_decode_steps_over_the_codes(rt, B, Hq, Hkv, T0):
+    """One f16 query token per step at head_dim 128: attention runs straight over the u8 codes (key features scaled
+    once per launch, token scales folded into the probabilities), several key splits merged in the kernel.  Sampled kv
+    heads against the oracle's attention over its dequantised stores; the stores stay bit-exact."""
+    rng = np.random.default_rng(T0)
+    D, g = 128, Hq // Hkv
+    st = tract_amd.QuantizedKvSdpa(axis=2, scale=None).state()
+    chan = rng.choice([1.0, 1.0, 1.0, 20.0], D)
+    k0 = (rng.standard_normal((B, Hkv, T0, D)) * chan).astype(np.float16)
+    v0 = rng.standard_normal((B, Hkv, T0, D)).astype(np.float16)
+    v0[:, :, 5::97] += 40.0                      # tokens whose lo dominates
+    v0[:, :, 11::131] = np.float16(-3.25)        # constant tokens: hi == lo, scale 1
+    q0 = (rng.standard_normal((B, Hq, T0, D)) / np.sqrt(D)).astype(np.float16)
+    st.eval([q0, k0, v0])
+    sample = sorted({(0, 0), (B - 1, Hkv - 1), (B // 2, Hkv // 2)})
+    refs = {}
+    for (b, h) in sample:
+        kc, vc = orc.KiviCache(True, running=True), orc.KiviCache(False, running=True)
+        kc.ingest(k0[b:b + 1, h:h + 1])
+        vc.ingest(v0[b:b + 1, h:h + 1])
+        refs[(b, h)] = (kc, vc)
+    worst = 0.0
+    for step in range(4):
+        q = (rng.standard_normal((B, Hq, 1, D)) * (3.0 if step == 2 else 1.0) / np.sqrt(D)).astype(np.float16)
+        k = (rng.standard_normal((B, Hkv, 1, D)) * chan * (1.0 if step != 1 else 4.0)).astype(np.float16)   # step 1 widens the key ranges
+        v = rng.standard_normal((B, Hkv, 1, D)).astype(np.float16)
+        got = st.eval([q, k, v]).to_numpy()
+        assert got.dtype == np.float16 and got.shape == (B, Hq, 1, D)
+        for (b, h), (kc, vc) in refs.items():
+            kc.ingest(k[b:b + 1, h:h + 1])
+            vc.ingest(v[b:b + 1, h:h + 1])
+            want = orc.flash_sdpa(q[b:b + 1, h * g:(h + 1) * g].astype(np.float32), kc.dequantized(), vc.dequantized(), causal=False)
+            err = max_abs(got[b:b + 1, h * g:(h + 1) * g], want)
+            worst = max(worst, err)
+            assert err <= 2e-2, (step, b, h, err)
+    state_k, state_v = st.k.state(), st.v.state()
+    for (b, h), (kc, vc) in refs.items():
+        i = b * Hkv + h
+        same_state({n: a[i:i + 1] for n, a in state_k.items()}, kc.state(), f"K {b},{h}")
+        same_state({n: a[i:i + 1] for n, a in state_v.items()}, vc.state(), f"V {b},{h}")
+    assert worst <= 8e-3, worst   # what f16 outputs and f16 probabilities leave
+
+
 def test_cache_of_the_decode_layer_shape(rt):
     """32q/8kv, d=128 at batch 8: a 2048-token prefill and decode steps; sampled heads against the oracle."""
     rng = np.random.default_rng(2)

@@ -153,6 +153,22 @@ int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s);
 int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s);
 // Split-K decode over Q8_0 / Q4_0 caches with fused dequantisation.  Returns 2 when not covered.
 int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s);
+// Split-K decode straight over the affine u8 stores of QuantizedKvSdpa (kv_quant.rs:105-236): Keys coded per channel
+// under one (lo, scale) per channel, Values per token.  f16 queries, head_dim 128, up to 16 query heads per kv head;
+// returns 2 when not covered.
+struct KiviSdpaArgs {
+    const void *q;
+    void *out;
+    const uint8_t *k_codes, *v_codes;    // [B * Hkv, cap_rows, 128]
+    int64_t k_cap_rows, v_cap_rows;
+    const float *k_chan_scale;           // [B * Hkv, 128]
+    const float *v_tok_scale, *v_tok_lo; // [B * Hkv, v_cap_rows]
+    int64_t B, Hq, Hkv, T;
+    float scale;
+    void *workspace;
+    size_t workspace_bytes;
+};
+int launch_sdpa_decode_kivi(const KiviSdpaArgs &a, hipStream_t s);
 // MFMA prefill.  Returns 2 when the shape is not covered.
 int launch_sdpa_prefill(const SdpaArgs &a, hipStream_t s);
 // MFMA prefill for q_len >= 32: staggered waves, GQA heads sharing K/V tiles, key splits across

@@ -37,6 +37,9 @@ struct DecodeDev {
     // additive mask of the q/out dtype, [mask_b, mask_h, 1, T] (NULL = none); byte strides, 0 on a broadcast axis
     const char *mask;
     int64_t mask_stride_b, mask_stride_h;
+    // affine u8 caches (decode_mfma_kivi_body): the Keys' per-channel scales, f32 [B * Hkv, D]; k_scales / v_scales then
+    // point at the Values' per-token scale and lo planes, f32 [B, Hkv, cap_rows], sc_stride_* their byte strides
+    const float *chan_scale;
 };
 
 // Ragged batches: one work item = a tile range of one sequence (device copies of the host plan).

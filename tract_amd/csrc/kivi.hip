@@ -944,6 +944,33 @@ int trocm_quantized_kv_sdpa_eval(const void *q, const void *k_new, const void *v
     if (trocm_kivi_cache_append(k_cache, k_new, dtype, n_new, s)) return 1;
     if (trocm_kivi_cache_append(v_cache, v_new, dtype, n_new, s)) return 1;
     const int64_t T = k_cache->len, D = k_cache->D;
+    // One token of f16 queries over the op's own stores (Keys under running per-channel parameters, Values per token, u8
+    // codes, nothing kept in f32): attention straight over the codes, no dequantised copy.  TROCM_KIVI_FUSED=0 keeps
+    // the dequantising path below, which serves every other case.
+    static const int fused = getenv("TROCM_KIVI_FUSED") ? atoi(getenv("TROCM_KIVI_FUSED")) : 1;
+    if (fused && dtype == TROCM_F16 && n_new == 1 && D == 128 && k_cache->layout == TROCM_KIVI_RUNNING_CHANNEL &&
+        v_cache->layout == TROCM_KIVI_PER_TOKEN && k_cache->bits == 8 && v_cache->bits == 8 && k_cache->n_sink == 0 &&
+        v_cache->n_sink == 0 && k_cache->n_res == 0 && v_cache->n_res == 0 && k_cache->n_rows == T && v_cache->n_rows == T) {
+        KiviSdpaArgs a;
+        a.q = q, a.out = out;
+        a.k_codes = k_cache->codes, a.v_codes = v_cache->codes;
+        a.k_cap_rows = k_cache->cap_rows, a.v_cap_rows = v_cache->cap_rows;
+        a.k_chan_scale = k_cache->scale;
+        a.v_tok_scale = v_cache->scale, a.v_tok_lo = v_cache->lo;
+        a.B = k_cache->B, a.Hq = q_heads, a.Hkv = k_cache->H, a.T = T;
+        a.scale = scale == scale ? scale : 1.0f / sqrtf((float)D);   // NaN asks for the default (sdpa.rs:93-95)
+        a.workspace = workspace, a.workspace_bytes = workspace_bytes;
+        const int rc = workspace ? launch_sdpa_decode_kivi(a, s) : 2;
+        if (rc == 0) {   // the dequantised copies a prompt left behind are not needed again (hipFree waits for the device)
+            for (trocm_kivi_cache *c : {k_cache, v_cache})
+                if (c->deq) {
+                    (void)hipFree(c->deq);
+                    c->deq = nullptr;
+                    c->deq_bytes = 0;
+                }
+        }
+        if (rc != 2) return rc;
+    }
     const size_t need = (size_t)k_cache->BH * T * D * elem_bytes(dtype);
     for (trocm_kivi_cache *c : {k_cache, v_cache}) {
         if (c->deq_bytes < need) {

@@ -1173,6 +1173,231 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
     wave_records_to_output<D, GP>(p, wk, lds_raw, head0, g, tid);
 }
 
+// Affine u8 caches as QuantizedKvSdpa keeps them (kv_quant.rs:105-236): K[t, c] = lo_k[c] + u_k[t, c] * s_k[c] with one
+// (lo, scale) per channel for the whole sequence, V[t, f] = lo_v[t] + u_v[t, f] * s_v[t] per token.  Nothing is
+// dequantised:
+//   S[t, h] = sum_c (q[h, c] s_k[c]) u_k[t, c]  +  sum_c q[h, c] lo_k[c]
+// and the second term is the same for every token of a head, so the softmax does not see it: the query features are
+// scaled once per launch and the raw codes go into the matrix cores as the exact halves 1024 + u (the 1024 leaves through
+// the accumulator's initial value);
+//   O[h, f] = sum_t (P[t, h] s_v[t]) u_v[t, f]  +  sum_t P[t, h] lo_v[t]
+// with the token scales folded into the probabilities (one operand for the whole row) and the second term one scalar per
+// head, added to every feature after the loop.  Lane layout, LDS tiles and the combine are those of the block-scaling
+// body; wk.ksbase / wk.vsbase are the Values' per-token scale and lo rows (f32).
+template <int GP, int PF>
+__device__ __forceinline__ void decode_mfma_kivi_body(const DecodeDev &p, const MfmaWork &wk) {
+    static_assert(GP <= 16, "the 16-wide layout: at most 16 heads");
+    constexpr int D = 128;
+    constexpr int NB = D / 32;
+    constexpr int RB = D;                      // code bytes per token row
+    constexpr int NLD = kTile * RB / 1024;     // 128-bit loads per lane, tile and tensor
+    constexpr int CPR = RB / 16;
+    constexpr int kCodeBytes = kTile * RB;
+    constexpr int kParamBytes = 2 * kTile * 4; // the tile's token scales, then its token los
+    constexpr int kWaveBytes = 2 * kCodeBytes + kParamBytes;
+    constexpr int kCombStride = GP * D + 2 * GP;
+    constexpr int kLdsBytes = kWaves * (kWaveBytes > kCombStride * 4 ? kWaveBytes : kCombStride * 4);
+    __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kLdsBytes];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l16 = lane & 15, q4 = lane >> 4;
+    const int kvh = wk.kvh, b = wk.seq;
+    const int g = p.g_real;
+    unsigned char *lds_k = lds_raw + w * kWaveBytes, *lds_v = lds_k + kCodeBytes;
+    float *lds_vp = reinterpret_cast<float *>(lds_v + kCodeBytes);
+
+    const int64_t head0 = (int64_t)b * p.Hq + (int64_t)kvh * g;
+    const _Float16 *qrow = reinterpret_cast<const _Float16 *>(p.q) + (head0 + min(l16, g - 1)) * D;
+    const float *ksc = p.chan_scale + ((int64_t)b * p.Hkv + kvh) * D;
+    const int T = wk.T;
+    const int tile_begin = wk.tile_begin, tile_end = wk.tile_end;
+    // lanes 0..31 carry the scale of token `lane` of a tile, lanes 32..63 the lo of token `lane - 32`
+    const float *par_row = reinterpret_cast<const float *>(lane < kTile ? wk.ksbase : wk.vsbase);
+
+    u32x4 kpre[PF][NLD], vpre[PF][NLD];
+    float ppre[PF];
+    auto fetch = [&](int t, u32x4 (&kd)[NLD], u32x4 (&vd)[NLD], float &par) {
+        const int t0 = t * kTile;
+        const char *kb = wk.kbase + (int64_t)t0 * RB, *vb = wk.vbase + (int64_t)t0 * RB;
+        if (t0 + kTile <= T) {
+#pragma unroll
+            for (int j = 0; j < NLD; j++) {
+                kd[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(kb + (j * 64 + lane) * 16));
+                vd[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(vb + (j * 64 + lane) * 16));
+            }
+            par = par_row[t0 + (lane & (kTile - 1))];
+        } else {   // rows past the end of the sequence repeat its last token (their scores are masked below)
+            const int last = T - 1 - t0;
+#pragma unroll
+            for (int j = 0; j < NLD; j++) {
+                const int c = j * 64 + lane, row = min(c / CPR, last), dc = c % CPR;
+                kd[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(kb + row * RB + dc * 16));
+                vd[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(vb + row * RB + dc * 16));
+            }
+            par = par_row[t0 + min(lane & (kTile - 1), last)];
+        }
+    };
+    auto key_k = [](int row) { return row & 7; };
+    auto key_v = [](int row) { return (row & 3) | (((row >> 4) & 1) << 2); };
+    uint32_t k_slot[NLD], v_slot[NLD];
+#pragma unroll
+    for (int j = 0; j < NLD; j++) {
+        const int c = j * 64 + lane, row = c / CPR, dc = c % CPR;
+        k_slot[j] = row * RB + 16 * (dc ^ key_k(row));
+        v_slot[j] = row * RB + 16 * (dc ^ key_v(row));
+    }
+    const int tstep = wk.tile_step;
+    int t = tile_begin + w;
+#pragma unroll
+    for (int st = 0; st < PF; st++) {
+        ppre[st] = 0.0f;
+        if (t + st * tstep < tile_end) fetch(t + st * tstep, kpre[st], vpre[st], ppre[st]);
+    }
+
+    // Q^T fragments of this lane's head, one per 32 channels: channels 32 blk + 8 q4 + 0..7, times their key scales
+    half8_t qf[NB];
+    float part = 0.0f;
+#pragma unroll
+    for (int blk = 0; blk < NB; blk++) {
+        const half8_t x = *reinterpret_cast<const half8_t *>(qrow + 32 * blk + 8 * q4);
+        const float4_t s0 = *reinterpret_cast<const float4_t *>(ksc + 32 * blk + 8 * q4), s1 = *reinterpret_cast<const float4_t *>(ksc + 32 * blk + 8 * q4 + 4);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            qf[blk][i] = (_Float16)((float)x[i] * (i < 4 ? s0[i] : s1[i - 4]));
+            part += (float)qf[blk][i];
+        }
+    }
+    part += __shfl_xor(part, 16, 64);
+    part += __shfl_xor(part, 32, 64);
+    const float bias = -1024.0f * part;
+#pragma unroll
+    for (int blk = 0; blk < NB; blk++) asm volatile("" : "+v"(qf[blk]));   // settled here, not at first use inside the loop
+
+    float m_run = -INFINITY, l_run = 0.0f;   // log2 domain, already scaled
+    float4_t o16[D / 16];
+    float sp = 0.0f, sl = 0.0f;              // sum of P s_v (as the halves the matrix cores saw), sum of P lo_v
+#pragma unroll
+    for (int fb = 0; fb < D / 16; fb++) o16[fb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    uint32_t k_frag[NB];
+#pragma unroll
+    for (int blk = 0; blk < NB; blk++) k_frag[blk] = l16 * RB + 16 * ((2 * blk + (q4 >> 1)) ^ key_k(l16)) + 8 * (q4 & 1);
+    const int vk = l16 >> 1, v_tok = vk < 4 ? 4 * q4 + vk : 12 + 4 * q4 + vk;
+    const unsigned char *v_row = lds_v + v_tok * RB + 8 * (l16 & 1);
+    const uint32_t v_key16 = 16 * key_v(v_tok);
+    const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+
+    const float c_log2 = p.scale_log2;   // > 0 (checked on the host): the maximum is taken before scaling
+    auto do_tile = [&](auto stage_tag, int t) {
+        constexpr int ST = decltype(stage_tag)::value;
+        const int t0 = t * kTile;
+        const bool more = t + PF * tstep < tile_end;
+#pragma unroll
+        for (int j = 0; j < NLD; j++) {
+            *reinterpret_cast<u32x4 *>(lds_k + k_slot[j]) = kpre[ST][j];
+            *reinterpret_cast<u32x4 *>(lds_v + v_slot[j]) = vpre[ST][j];
+        }
+        lds_vp[lane] = ppre[ST];
+        if (more) fetch(t + PF * tstep, kpre[ST], vpre[ST], ppre[ST]);
+        // ---- codes x scaled query features, all 128 channels into one accumulator ------------------------------------
+        float sc8[8];
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++) {
+            float4_t acc = {bias, bias, bias, bias};
+#pragma unroll
+            for (int blk = 0; blk < NB; blk++) {
+                const u32x2 c = *reinterpret_cast<const u32x2 *>(lds_k + k_frag[blk] + 16 * mb * RB);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(magic8(c.x, c.y), qf[blk], acc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; r++) sc8[4 * mb + r] = acc[r];   // tokens 16 mb + 4 q4 + r, head l16
+        }
+        if (t0 + kTile > T) {   // the sequence's last tile: tokens past its end do not count
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (t0 + 16 * (i >> 2) + 4 * q4 + (i & 3) >= T) sc8[i] = -INFINITY;
+        }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; i++) tmax = fmaxf(tmax, sc8[i]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m_run, tmax * c_log2);   // finite: every tile holds at least one valid token
+        float pe[8], psum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            pe[i] = fast_exp2(__builtin_fmaf(sc8[i], c_log2, -m_new));
+            psum += pe[i];
+        }
+        const bool moved = m_new != m_run;
+        const float alpha = fast_exp2(m_run - m_new);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+            for (int fb = 0; fb < D / 16; fb++) o16[fb] *= alpha;
+            sp *= alpha;
+            sl *= alpha;
+        }
+        // ---- probabilities times the scales of their tokens: one operand for the whole row ---------------------------------
+        u32x4 pw;
+        {
+            const float4_t sa = *reinterpret_cast<const float4_t *>(lds_vp + 4 * q4), sb = *reinterpret_cast<const float4_t *>(lds_vp + 16 + 4 * q4);
+            const float4_t la = *reinterpret_cast<const float4_t *>(lds_vp + kTile + 4 * q4), lb = *reinterpret_cast<const float4_t *>(lds_vp + kTile + 16 + 4 * q4);
+            const float sv[8] = {sa[0], sa[1], sa[2], sa[3], sb[0], sb[1], sb[2], sb[3]};
+            const float lv[8] = {la[0], la[1], la[2], la[3], lb[0], lb[1], lb[2], lb[3]};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const half2_t pp = {(_Float16)(pe[2 * i] * sv[2 * i]), (_Float16)(pe[2 * i + 1] * sv[2 * i + 1])};
+                sp = __builtin_amdgcn_fdot2(pp, ones, sp, false);
+                sl = __builtin_fmaf(pe[2 * i], lv[2 * i], sl);
+                sl = __builtin_fmaf(pe[2 * i + 1], lv[2 * i + 1], sl);
+                pw[i] = __builtin_bit_cast(uint32_t, pp);
+            }
+        }
+        const half8_t pb = __builtin_bit_cast(half8_t, pw);
+        // ---- O^T += codes^T x scaled probabilities -----------------------------------------------------------------------
+#pragma unroll
+        for (int fb = 0; fb < D / 16; fb++) {
+            uint32_t w0, w1;
+            lds_read_tr8(v_row + ((16 * fb) ^ v_key16), w0, w1);
+            o16[fb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(magic8(w0, w1), pb, o16[fb], 0, 0, 0);
+        }
+    };
+    static_assert(PF <= 2, "stages are written out");
+    while (t < tile_end) {
+        do_tile(std::integral_constant<int, 0>{}, t);
+        t += tstep;
+        if constexpr (PF > 1) {
+            if (t < tile_end) do_tile(std::integral_constant<int, 1>{}, t), t += tstep;
+        }
+    }
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    sp += __shfl_xor(sp, 16, 64);
+    sp += __shfl_xor(sp, 32, 64);
+    sl += __shfl_xor(sl, 16, 64);
+    sl += __shfl_xor(sl, 32, 64);
+    const float shift = sl - 1024.0f * sp;   // the 1024 under every code leaves, the tokens' los arrive
+#pragma unroll
+    for (int fb = 0; fb < D / 16; fb++) o16[fb] += shift;
+
+    // ---- merge the 4 waves through LDS (the tiles are dead) ------------------------------------------------------------
+    __syncthreads();
+    float *comb = reinterpret_cast<float *>(lds_raw);   // [kWaves][GP*D + 2*GP]
+    if (l16 < GP) {
+        float *cw = comb + w * kCombStride;
+#pragma unroll
+        for (int fb = 0; fb < D / 16; fb++) *reinterpret_cast<float4_t *>(cw + l16 * D + 16 * fb + 4 * q4) = o16[fb];
+        if (q4 == 0) {
+            cw[GP * D + l16] = m_run;
+            cw[GP * D + GP + l16] = l_run;
+        }
+    }
+    wave_records_to_output<D, GP>(p, wk, lds_raw, head0, g, tid);
+}
+
 // The reference states a ragged batch as a dense batch padded to the longest sequence, with a mask row per
 // sequence whose padded columns hold the format's minimum or -inf (flash_sdpa.rs:261-268).  The tokens of such a
 // suffix weigh exactly nothing (their exponentials underflow to zero next to any token that counts), so the
@@ -1203,7 +1428,7 @@ __device__ __forceinline__ int mask_row_len(const _Float16 *__restrict__ row, in
 // Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.
 // QB: quantised caches on the 16-wide tiles run the body that scales per block outside the products.
 template <int D, int GP, int FMT, bool MASK = false, bool W16 = false, int QB = 0>
-__global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma_kernel(DecodeDev p) {   // QB = 100 * diagonal + 10 * tiles ahead + workgroups per CU
+__global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma_kernel(DecodeDev p) {   // QB = 100 * (1: diagonal, 2: affine u8) + 10 * tiles ahead + workgroups per CU
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     MfmaWork wk;
     wk.seq = b, wk.kvh = kvh;
@@ -1238,7 +1463,9 @@ __global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma
     wk.counter = p.counters ? p.counters + bh : nullptr;
     wk.part_first = bh * p.nsplit, wk.part_stride = 1;
     wk.mask = MASK ? p.mask + (int64_t)b * p.mask_stride_b + (int64_t)kvh * p.g_real * p.mask_stride_h : nullptr;
-    if constexpr (QB >= 100)
+    if constexpr (QB >= 200)
+        decode_mfma_kivi_body<GP, (QB / 10) % 10>(p, wk);
+    else if constexpr (QB >= 100)
         decode_mfma_qdiag_body<GP, FMT, (QB / 10) % 10>(p, wk);
     else if constexpr (QB != 0)
         decode_mfma_qblock_body<GP, FMT, QB / 10>(p, wk);
@@ -1428,6 +1655,53 @@ int launch_sdpa_decode_quant_mfma(DecodeDev &p, int kv_fmt, int64_t B, void *wor
     if (tail && gp <= 8 && nsplit > 1 && nsplit <= kWideMergeMax && BH <= (int64_t)(kWsCounterBytes / sizeof(int))) p.counters = (int *)workspace;
     dim3 grid(nsplit, (unsigned)p.Hkv, (unsigned)B);
     return kv_fmt == TROCM_Q8_0 ? launch_quant<TROCM_Q8_0>(p, gp, grid, s) : launch_quant<TROCM_Q4_0>(p, gp, grid, s);
+}
+
+int launch_sdpa_decode_kivi(const KiviSdpaArgs &a, hipStream_t s) {
+    if (a.Hq % a.Hkv) return 2;
+    const int64_t g_real = a.Hq / a.Hkv;
+    const int gp = decode_mfma_group(g_real);
+    if (gp == 0 || gp > 16) return 2;
+    if (a.T <= 0 || a.T > (1ll << 30) || a.B > 65535 || a.Hkv > 65535 || !(a.scale > 0.0f)) return 2;
+    if ((uintptr_t)a.q % 16 || (uintptr_t)a.k_codes % 16 || (uintptr_t)a.v_codes % 16 || (uintptr_t)a.k_chan_scale % 16) return 2;
+    const int64_t BH = a.B * a.Hkv;
+    const int n_tiles = (int)((a.T + kTile - 1) / kTile);
+    int nsplit = fit_decode_splits(choose_decode_splits(BH, gp, n_tiles, 2), BH, gp, 128, a.workspace, a.workspace_bytes);
+    const int tps = (n_tiles + nsplit - 1) / nsplit;
+    nsplit = (n_tiles + tps - 1) / tps;
+    DecodeDev p;
+    memset(&p, 0, sizeof(p));
+    p.q = (const char *)a.q, p.out = (char *)a.out;
+    p.k = (const char *)a.k_codes, p.v = (const char *)a.v_codes;
+    if (a.k_cap_rows != a.v_cap_rows) return 2;   // one pair of strides serves both code planes
+    p.kv_stride_h = a.k_cap_rows * 128, p.kv_stride_b = a.Hkv * p.kv_stride_h, p.kv_stride_t = 128;
+    p.k_scales = (const char *)a.v_tok_scale, p.v_scales = (const char *)a.v_tok_lo;
+    p.sc_stride_h = a.v_cap_rows * 4, p.sc_stride_b = a.Hkv * p.sc_stride_h;
+    p.chan_scale = a.k_chan_scale;
+    p.T = (int)a.T;
+    p.tiles_per_split = tps, p.nsplit = nsplit;
+    p.Hq = (int)a.Hq, p.Hkv = (int)a.Hkv, p.g_real = (int)g_real;
+    p.scale_log2 = a.scale * 1.4426950408889634f;
+    p.new_pos = (int)a.T - 1;
+    static const int interleave = getenv("TROCM_DECODE_INTERLEAVE") ? atoi(getenv("TROCM_DECODE_INTERLEAVE")) : 1;
+    p.interleave = interleave;
+    p.part_ml = (float *)((char *)a.workspace + kWsCounterBytes);
+    p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * gp;
+    static const int tail = getenv("TROCM_DECODE_TAIL_MERGE") ? atoi(getenv("TROCM_DECODE_TAIL_MERGE")) : 1;
+    if (tail && gp <= 8 && nsplit > 1 && nsplit <= kWideMergeMax && BH <= (int64_t)(kWsCounterBytes / sizeof(int))) p.counters = (int *)a.workspace;
+    dim3 grid(nsplit, (unsigned)a.Hkv, (unsigned)a.B);
+    if (gp == 8) {
+        hipLaunchKernelGGL((sdpa_decode_mfma_kernel<128, 8, TROCM_Q8_0, false, true, 212>), grid, dim3(kThreads), 0, s, p);
+        if (p.nsplit > 1 && p.counters == nullptr)
+            hipLaunchKernelGGL((sdpa_decode_merge_kernel<__half, 128, 8>), dim3(grid.y, grid.z, p.g_real), dim3(128), 0, s, p);
+    } else {
+        hipLaunchKernelGGL((sdpa_decode_mfma_kernel<128, 16, TROCM_Q8_0, false, true, 212>), grid, dim3(kThreads), 0, s, p);
+        if (p.nsplit > 1 && p.counters == nullptr)
+            hipLaunchKernelGGL((sdpa_decode_merge_kernel<__half, 128, 16>), dim3(grid.y, grid.z, p.g_real), dim3(128), 0, s, p);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("sdpa_decode (affine u8) launch failed: %s", hipGetErrorString(e));
+    return 0;
 }
 
 int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {
