@@ -49,6 +49,49 @@ def test_quantized_dyn_kv_cache_state_and_output_equal_the_oracle(rt, dt, bits, 
         assert c["n_rows"] == (ref.length - 4) // 32 * 32 and c["n_res"] == (ref.length - 4) % 32
 
 
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_quotients_on_and_beside_the_rounding_boundaries(rt, bits, per_channel):
+    """Values whose quotient (x - lo) / scale is exactly k + 1/2, or one to three floats beside it, for scales that are
+    and are not powers of two, and scales outside the range where a reciprocal may stand in for the division: the codes
+    must be the ones the division gives (the device codes most elements by a product and falls back near a boundary)."""
+    rng = np.random.default_rng(bits)
+    D, lv = 128, (1 << bits) - 1
+    n_groups = 64
+    scales = np.concatenate([[1.0, 3.0, 0.75, 1e-3, 7.0, 2.0 ** -20, 1e30, 1e-38, 3e-41, 1e38 / lv],
+                             rng.uniform(1e-3, 50.0, n_groups - 10)]).astype(np.float32)
+    # a group: lo = 0, hi = lv * s (so that scale = RN(hi / lv), close to s), 126 more values at and around the boundaries
+    groups = np.zeros((n_groups, D), np.float32)
+    for gi, s in enumerate(scales):
+        hi = np.float32(lv) * s
+        sc = np.float32(hi / np.float32(lv)) if np.isfinite(hi) and hi > 0 else np.float32(1.0)
+        ks = rng.integers(0, lv, D - 2).astype(np.float32)
+        with np.errstate(over="ignore", invalid="ignore"):
+            vals = ((ks + np.float32(0.5)) * sc).astype(np.float32)
+            for j in range(D - 2):
+                steps = (j % 7) - 3
+                for _ in range(abs(steps)):
+                    vals[j] = np.nextafter(vals[j], np.float32(np.inf if steps > 0 else 0.0), dtype=np.float32)
+            vals = np.clip(np.nan_to_num(vals, nan=0.0, posinf=float(hi), neginf=0.0), 0.0, hi)
+        groups[gi, 0], groups[gi, 1], groups[gi, 2:] = 0.0, hi, vals
+    if per_channel:     # a group is a channel over one 32-token block: blocks [32, D] with D groups side by side
+        n_blocks = n_groups * D // (32 * D) * 4
+        x = np.zeros((1, 1, 4 + 32 * n_blocks, D), np.float32)
+        flat = groups.reshape(-1)
+        for b in range(n_blocks):
+            for c in range(D):
+                g = groups[(b * D + c) % n_groups]
+                x[0, 0, 4 + 32 * b:4 + 32 * (b + 1), c] = np.concatenate([g[:2], g[2 + (b * 30) % 96:2 + (b * 30) % 96 + 30]])
+    else:               # a group is a token
+        x = np.concatenate([np.zeros((4, D), np.float32), groups]).reshape(1, 1, 4 + n_groups, D)
+    st = tract_amd.QuantizedDynKeyValueCache("kv", 2, bits, per_channel).state()
+    ref = orc.KiviCache(per_channel, bits)
+    out = st.eval(x).to_numpy()
+    ref.ingest(x)
+    same_state(st.cache.state(), ref.state(), f"bits={bits} per_channel={per_channel}")
+    assert out.tobytes() == ref.dequantized().tobytes()
+
+
 @pytest.mark.parametrize("D", [8, 16, 3, 130])
 def test_odd_head_sizes_and_tiny_caches(rt, D):
     rng = np.random.default_rng(D)

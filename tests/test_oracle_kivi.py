@@ -261,3 +261,34 @@ def test_ref_quantized_kv_sdpa_near_f32_attention():           # kv_quant.rs:568
         vf = vi if vf is None else orc.concat_append(vf, vi, 2)
         want = orc.naive_sdpa_f64(qi, kf, vf, causal=False).astype(np.float32)
         assert close_enough_super(got, want), t
+
+
+def test_codes_by_a_product_equal_codes_by_the_division_away_from_the_boundaries():
+    """The device codes (x - lo) * RN(1 / scale) instead of (x - lo) / scale and falls back to the division when the
+    product's fraction is within 2^-13 of one half.  Here in numpy: on quotients placed on and a few floats beside the
+    boundaries k + 1/2 and on random ones, for power-of-two and other scales, the two codes agree wherever the rule does
+    not ask for the fallback, and without the rule they would differ somewhere (so the rule is needed)."""
+    rng = np.random.default_rng(8)
+    half = np.float32(0.49999997)
+    differ = checked = 0
+    for lv in (255, 15):
+        scales = np.concatenate([[1.0, 3.0, 0.75, 1e-3, 7.0, 2.0 ** -20], rng.uniform(1e-3, 50.0, 200)]).astype(np.float32)
+        for s in scales:
+            sc = np.float32(np.float32(lv) * s / np.float32(lv))
+            ks = rng.integers(0, lv, 256).astype(np.float32)
+            vals = ((ks + np.float32(0.5)) * sc).astype(np.float32)
+            for j in range(vals.size):
+                steps = (j % 7) - 3
+                for _ in range(abs(steps)):
+                    vals[j] = np.nextafter(vals[j], np.float32(np.inf if steps > 0 else 0.0), dtype=np.float32)
+            vals = np.concatenate([vals, rng.uniform(0, lv * float(sc), 256).astype(np.float32)])
+            q = (vals / sc).astype(np.float32)
+            exact = np.clip(np.trunc((q + np.copysign(half, q)).astype(np.float32)), 0, lv)
+            q0 = (vals * np.float32(np.float32(1.0) / sc)).astype(np.float32)
+            fast = np.clip(np.trunc((q0 + half).astype(np.float32)), 0, lv)
+            near = np.abs((q0 - np.floor(q0)).astype(np.float32) - np.float32(0.5))
+            safe = near >= np.float32(2.0 ** -13)
+            assert (fast[safe] == exact[safe]).all(), (lv, s)
+            differ += int((fast != exact).sum())
+            checked += int(safe.sum())
+    assert differ > 0 and checked > 50000

@@ -23,6 +23,7 @@
 // append, the dequantising read costs row_bytes + 2 or 4 bytes per element.
 #include <hip/hip_fp16.h>
 #include <new>
+#include <type_traits>
 #include "common.h"
 
 namespace trocm {
@@ -57,6 +58,43 @@ __device__ __forceinline__ uint32_t affine_code(float x, float lo, float scale, 
 }
 __device__ __forceinline__ float affine_scale(float lo, float hi, float lv) {   // :127, :186
     return hi > lo ? __fdiv_rn(__fsub_rn(hi, lo), lv) : 1.0f;
+}
+
+// The same codes without a division per element.  With inv = RN(1 / scale) the product q0 = RN((x - lo) * inv) lies
+// within 2^-22 relative of the reference's quotient q = RN((x - lo) / scale) (three roundings of 2^-24 between them),
+// i.e. within 2^-14 absolute wherever a rounding decision is still open (q below lv + 1/2 <= 255.5; from there on
+// both clamp to lv, and every negative quotient rounds to a code of 0).  So when the fraction of q0 is at least 2^-13
+// away from one half, trunc(q0 + 0.49999997) is the reference's round(q) (see round_half_away); otherwise, and for a
+// scale whose reciprocal is not an ordinary float, the eight codes are computed again with the division.  NaN gives 0
+// and +inf gives lv on both paths.
+__device__ __forceinline__ float affine_inv(float scale) {   // 0: do not use the product
+    return (scale >= 0x1p-100f && scale <= 0x1p100f) ? __fdiv_rn(1.0f, scale) : 0.0f;
+}
+__device__ __forceinline__ int cvt_i32_rz_sat(float x) {   // truncates, saturates, NaN -> 0 (a C cast may assume the value is in range)
+    int r;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(x));
+    return r;
+}
+template <typename Params>   // Params: float (one group for the 8 values) or float[8] (a group per value)
+__device__ __forceinline__ void affine_codes8(const float (&x)[8], const Params &lo, const Params &scale, const Params &inv, float lv,
+                                              uint32_t (&code)[8]) {
+    auto at = [](const Params &p, int e) -> float {
+        if constexpr (std::is_same<Params, float>::value) return p;
+        else return p[e];
+    };
+    float near = 1.0f;   // the smallest distance of a fraction from one half (fminf drops a NaN)
+    bool usable = true;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const float q0 = __fmul_rn(__fsub_rn(x[e], at(lo, e)), at(inv, e));
+        near = fminf(near, fabsf(__fsub_rn(__builtin_amdgcn_fractf(q0), 0.5f)));
+        code[e] = (uint32_t)max(0, min((int)lv, cvt_i32_rz_sat(__fadd_rn(q0, 0.49999997f))));
+        usable = usable && at(inv, e) != 0.0f;
+    }
+    if (!(usable && near >= 0x1p-13f)) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) code[e] = affine_code(x[e], at(lo, e), at(scale, e), lv);
+    }
 }
 
 // dst[bh][dst_t0 + i][c] = (f32) src[bh][src_t0 + i][c], i < n: sink tokens and the partial key block.
@@ -363,10 +401,9 @@ __global__ void __launch_bounds__(256) kivi_quant_tokens_vec_kernel(const SrcT *
         lo = fminf(lo, __shfl_xor(lo, m, 64));
         hi = fmaxf(hi, __shfl_xor(hi, m, 64));
     }
-    const float scale = affine_scale(lo, hi, lv);
+    const float scale = affine_scale(lo, hi, lv), inv = affine_inv(scale);
     uint32_t code[8];
-#pragma unroll
-    for (int e = 0; e < 8; e++) code[e] = affine_code(x.v[e], lo, scale, lv);
+    affine_codes8(x.v, lo, scale, inv, lv, code);
     store_codes8<BITS>(codes + ((int64_t)bh * cap_rows + row0 + i) * RB, sub, code);
     if (sub == 0) {
         lo_out[(int64_t)bh * cap_rows + row0 + i] = lo;
@@ -390,7 +427,7 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_vec_kernel(const Src
     const SrcT *rows = src + ((int64_t)bh * S + src_t0 + (int64_t)j * kKeyBlock - n_res_old) * D + sub * 8;
     const float *res = residual + (int64_t)bh * kKeyBlock * D + sub * 8;
     const int n_old = j == 0 ? n_res_old : 0;
-    float lo[8], hi[8], scale[8];
+    float lo[8], hi[8], scale[8], inv[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) {
         lo[e] = INFINITY;
@@ -417,6 +454,7 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_vec_kernel(const Src
 #pragma unroll
     for (int e = 0; e < 8; e++) {
         scale[e] = affine_scale(lo[e], hi[e], lv);
+        inv[e] = affine_inv(scale[e]);
         ls.v[e] = lo[e];
         ss.v[e] = scale[e];
     }
@@ -430,8 +468,7 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_vec_kernel(const Src
     for (int r = g; r < kKeyBlock; r += G) {
         const F8 x = r < n_old ? ld8(res + (int64_t)r * D) : ld8(rows + (int64_t)r * D);
         uint32_t code[8];
-#pragma unroll
-        for (int e = 0; e < 8; e++) code[e] = affine_code(x.v[e], lo[e], scale[e], lv);
+        affine_codes8(x.v, lo, scale, inv, lv, code);
         store_codes8<BITS>(out + (int64_t)r * RB, sub, code);
     }
 }
