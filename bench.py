@@ -312,7 +312,7 @@ def run_cfg3(ta, args):
         tot_us += us
         tot_fl += fl
     tf = tot_fl / tot_us / 1e6
-    roof = {"bound": "mfma", "kernel": "sdpa_prefill_pp_kernel<128,4> (+ sdpa_prefill_merge_kernel<128>)", "achieved": round(tf, 1), "peak": 2500.0,
+    roof = {"bound": "mfma", "kernel": "sdpa_prefill_pp_kernel<128,4,false,F16> (key splits merged in the kernel)", "achieved": round(tf, 1), "peak": 2500.0,
             "unit": "TFLOP/s", "frac": round(tf / 2500.0, 4), "traffic": None}
     return base_line(args, "cfg3: chunked prefill, 8 x 512 tokens into an empty cache, causal SDPA of each chunk over "
                      "the cache so far (32q/8kv d=128 f16, batch 1); attention launches only", round(tf, 1), "TFLOP/s",
@@ -335,10 +335,11 @@ def run_cfg4(ta, args):
             kf = k.transpose(0, 2, 1, 3).reshape(B, T, HKV * D)
             kf[:, :, chan] *= 20.0
             k = kf.reshape(B, T, HKV, D).transpose(0, 2, 1, 3).astype(np.float16)
+            v = seeded_f16(cfg_seed(4, "v") + T, (B, HKV, T, D))   # (not K again: swapped planes or scales would show)
             for st in sts:
-                for c in (st.k, st.v):
-                    c.reserve(T + 128, like=(k.shape, k.dtype))
-                    c.push(k)
+                for c, x in ((st.k, k), (st.v, v)):
+                    c.reserve(T + 128, like=(x.shape, x.dtype))
+                    c.push(x)
             qh = (seeded_f16(cfg_seed(4, "q"), (B, HQ, 1, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16)
             q = ta.DeviceTensor.from_numpy(qh)
             out = ta.DeviceTensor((B, HQ, 1, D), np.float16)
@@ -352,17 +353,18 @@ def run_cfg4(ta, args):
             # after the timing: sequences 0 and 7, four query heads, against the oracle over the dequantised blocks
             from oracle import oracle as orc
             sts[0].attend(q, out=out)
-            kd = k[[0, 7]]
+            kd, vd = k[[0, 7]], v[[0, 7]]
             if fmt is not None:
                 ofmt = getattr(orc, "FMT_" + name.upper())
                 kd = orc.dequant(ofmt, orc.quant(ofmt, kd), np.float16)
+                vd = orc.dequant(ofmt, orc.quant(ofmt, vd), np.float16)
             o = out.to_numpy()[[0, 7]]
-            err = parity_sample(o, qh[[0, 7]], kd, kd, [0, 9, 18, 31], seqs=[0, 1])
+            err = parity_sample(o, qh[[0, 7]], kd, vd, [0, 9, 18, 31], seqs=[0, 1])
             del sts
             by = 2 * B * HKV * T * D * ek + 2 * B * HQ * D * 2
             res[f"{name}_ctx{T}"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by), "parity_max_abs_vs_oracle": err}
     head = res["q8_0_ctx16384"]
-    roof = {"bound": "hbm", "kernel": "sdpa_decode_mfma_kernel<128,8,Q8_0,false,true>", "achieved": head["gbs"], "peak": HBM_PEAK_GBS,
+    roof = {"bound": "hbm", "kernel": "sdpa_decode_mfma_kernel<128,8,Q8_0,false,true,112>", "achieved": head["gbs"], "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4), "traffic": None}
     return base_line(args, "cfg4: decode over a Q8_0 / Q4_0 quantised KV cache (fused dequant), batch 8, contexts 4096 "
                      "and 16384, 1% outlier channels x20; attention launches only, rotating over 2-4 layers' caches; "
