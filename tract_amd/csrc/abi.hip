@@ -757,6 +757,19 @@ int trocm_kv_append_pair(trocm_kv_cache *kc, trocm_kv_cache *vc, const void *k_s
         a.dst_stride[0] = kc->H * kc->pitch * kc->D * es, a.dst_stride[1] = kc->pitch * kc->D * es, a.dst_stride[2] = kc->D * es;
         rc = launch_append_pair(a, s);
     }
+    if (is_quant(kc->fmt)) {   // both tensors quantised by one launch
+        QuantAppend a[2];
+        trocm_kv_cache *cs[2] = {kc, vc};
+        const void *srcs[2] = {k_src, v_src};
+        for (int t = 0; t < 2; t++) {
+            a[t].fmt = cs[t]->fmt, a[t].src_dtype = src_dtype;
+            a[t].B = cs[t]->B, a[t].H = cs[t]->H, a[t].S = n_new, a[t].D = cs[t]->D;
+            for (int i = 0; i < 4; i++) a[t].ss[i] = src_strides[i];
+            a[t].cap = cs[t]->pitch, a[t].t0 = cs[t]->len;
+            a[t].src = srcs[t], a[t].codes = cs[t]->data, a[t].scales = cs[t]->scales;
+        }
+        rc = launch_quant_append_pair(a[0], a[1], s);
+    }
     if (rc == 2) {
         rc = append_write(kc, k_src, src_dtype, src_strides, n_new, s);
         if (!rc) rc = append_write(vc, v_src, src_dtype, src_strides, n_new, s);

@@ -86,6 +86,8 @@ struct QuantAppend {
     void *codes, *scales;
 };
 int launch_quant_append(const QuantAppend &a, hipStream_t s);
+// K and V of one shape and source type in one launch; returns 2 when they differ.
+int launch_quant_append_pair(const QuantAppend &k, const QuantAppend &v, hipStream_t s);
 // One new token for each of n_seq sequences (k_new / v_new dense [n_seq, H, 1, D], f16 or f32) quantised
 // into the sequences' own K and V planes by one launch; `table` is in device memory.
 struct QuantAppendSeq {

@@ -517,9 +517,8 @@ __global__ void kivi_dequant_kernel(KiviView a, DstT *__restrict__ dst) {
 template <typename DstT, int BITS, bool STREAM>
 __global__ void __launch_bounds__(256) kivi_dequant_vec_kernel(KiviView a, DstT *__restrict__ dst) {
     const int bh = blockIdx.y;
-    const int e = blockIdx.x * blockDim.x + threadIdx.x;
     const int d8 = a.D >> 3;
-    if (e >= a.len * d8) return;
+    for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < a.len * d8; e += gridDim.x * blockDim.x) {
     const int t = e / d8, c = (e - t * d8) * 8;
     F8 x;
     if (t < a.n_sink) {
@@ -553,6 +552,7 @@ __global__ void __launch_bounds__(256) kivi_dequant_vec_kernel(KiviView a, DstT 
     }
     if (STREAM) st8_stream(dst + ((int64_t)bh * a.len + t) * a.D + c, x);
     else st8(dst + ((int64_t)bh * a.len + t) * a.D + c, x);
+    }
 }
 
 __global__ void kivi_fill_running_kernel(float *lo, float *scale, int64_t n) {
@@ -783,7 +783,12 @@ static int kivi_dequantize(const trocm_kivi_cache *c, void *dst, int dst_dtype, 
     a.scale = c->scale;
     a.codes = c->codes;
     if (c->D % 8 == 0 && ((uintptr_t)dst & 15) == 0) {
-        const dim3 grid8((unsigned)((c->len * (c->D / 8) + 255) / 256), (unsigned)c->BH);
+        int64_t gx = (c->len * (c->D / 8) + 255) / 256;
+        // at most 128 workgroups per compute unit, whose threads then take several trips (8 x 8 x 16384 x 128 to f16: one
+        // trip per thread 84 us, 128 per compute unit 78, 64: 79, 32: 82, 16: 93)
+        const int64_t want = (int64_t)num_compute_units() * 128;
+        if (gx * c->BH > want) gx = (want + c->BH - 1) / c->BH;
+        const dim3 grid8((unsigned)gx, (unsigned)c->BH);
 #define KIVI_DEQ(T, BITS)                                                                          \
     do {                                                                                           \
         if (stream_out) kivi_dequant_vec_kernel<T, BITS, true><<<grid8, 256, 0, s>>>(a, (T *)dst); \

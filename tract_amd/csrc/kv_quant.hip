@@ -185,7 +185,7 @@ __device__ __forceinline__ void quant_one_block(const QuantAppendDev &a, const S
 // three 64-bit divisions were 45 % of the kernel's instructions.  Dense sources have a loop of their own: with the
 // choice between 128-bit and element loads inside one loop the same launch measured 82 us instead of 75 us.
 template <typename SrcT>
-__global__ __launch_bounds__(256) void quant_append_kernel(QuantAppendDev a) {
+__device__ __forceinline__ void quant_append_body(const QuantAppendDev &a) {
     const uint32_t nb = (uint32_t)(a.D / 32);
     const uint32_t per_row = (uint32_t)a.S * nb;
     const uint32_t first = blockIdx.x * blockDim.x + threadIdx.x, step = gridDim.x * blockDim.x;
@@ -221,6 +221,17 @@ __global__ __launch_bounds__(256) void quant_append_kernel(QuantAppendDev a) {
             quant_one_block(a, src_row + (int64_t)t * a.ss[2] + (int64_t)blk * 32 * a.ss[3], row0 + t, nb, blk);
         }
     }
+}
+
+template <typename SrcT>
+__global__ __launch_bounds__(256) void quant_append_kernel(QuantAppendDev a) {
+    quant_append_body<SrcT>(a);
+}
+// K and V of the same shape in one launch: blockIdx.z selects the tensor.
+template <typename SrcT>
+__global__ __launch_bounds__(256) void quant_append_pair_kernel(QuantAppendDev k, QuantAppendDev v) {
+    if (blockIdx.z == 0) quant_append_body<SrcT>(k);
+    else quant_append_body<SrcT>(v);
 }
 
 // One token per sequence into per-sequence planes: grid (sequences, 2 = K / V).
@@ -398,9 +409,9 @@ int check_launch(const char *what) {
 
 }  // namespace
 
-int launch_quant_append(const QuantAppend &a, hipStream_t s) {
+// The device-side description of one append, and the grid (gx, gy) that covers it.
+static int describe_quant_append(const QuantAppend &a, QuantAppendDev &d, int64_t &gx, int64_t &gy) {
     TROCM_REQUIRE(a.D % 32 == 0, "quantised KV cache needs head_dim %% 32 == 0, got %lld", (long long)a.D);
-    QuantAppendDev d;
     d.fmt = a.fmt;
     d.B = a.B, d.H = a.H, d.S = a.S, d.D = a.D;
     for (int i = 0; i < 4; i++) d.ss[i] = a.ss[i];
@@ -409,7 +420,6 @@ int launch_quant_append(const QuantAppend &a, hipStream_t s) {
     d.codes = (uint8_t *)a.codes;
     d.scales = (uint16_t *)a.scales;
     d.n_blocks = a.B * a.H * a.S * (a.D / 32);
-    if (d.n_blocks == 0) return 0;
     size_t es = elem_bytes(a.src_dtype);
     // 128-bit loads need a dense innermost axis and every block start on a 16-byte boundary
     // (blocks are 32 elements = 64 or 128 bytes, so only the base and outer strides matter).
@@ -428,13 +438,34 @@ int launch_quant_append(const QuantAppend &a, hipStream_t s) {
     // 82.6 us (Q8_0) / 66.6 us (Q4_0), with the next block requested before the current one is worked on 81.8 / 67.1
     // (two blocks ahead 86 / 72: fewer waves fit), a contiguous run of blocks per workgroup 87.5 / 70.3, one block per
     // thread 75-76 / 62-63.  The loops in the kernel only serve launches beyond the grid limits.
-    const int64_t gx = std::min<int64_t>((per_row + 255) / 256, 1 << 22);
-    const int64_t gy = bh < 65535 ? bh : 65535;
+    gx = std::min<int64_t>((per_row + 255) / 256, 1 << 22);
+    gy = bh < 65535 ? bh : 65535;
+    return 0;
+}
+
+int launch_quant_append(const QuantAppend &a, hipStream_t s) {
+    QuantAppendDev d;
+    int64_t gx, gy;
+    if (describe_quant_append(a, d, gx, gy)) return 1;
+    if (d.n_blocks == 0) return 0;
     if (a.src_dtype == TROCM_F16)
         hipLaunchKernelGGL(quant_append_kernel<__half>, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, d);
     else
         hipLaunchKernelGGL(quant_append_kernel<float>, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, d);
     return check_launch("quant_append");
+}
+
+int launch_quant_append_pair(const QuantAppend &k, const QuantAppend &v, hipStream_t s) {
+    if (k.src_dtype != v.src_dtype || k.B != v.B || k.H != v.H || k.S != v.S || k.D != v.D) return 2;
+    QuantAppendDev dk, dv;
+    int64_t gx, gy, gx2, gy2;
+    if (describe_quant_append(k, dk, gx, gy) || describe_quant_append(v, dv, gx2, gy2)) return 1;
+    if (dk.n_blocks == 0) return 0;
+    if (k.src_dtype == TROCM_F16)
+        hipLaunchKernelGGL(quant_append_pair_kernel<__half>, dim3((unsigned)gx, (unsigned)gy, 2), dim3(256), 0, s, dk, dv);
+    else
+        hipLaunchKernelGGL(quant_append_pair_kernel<float>, dim3((unsigned)gx, (unsigned)gy, 2), dim3(256), 0, s, dk, dv);
+    return check_launch("quant_append_pair");
 }
 
 int launch_quant_append_ragged(int fmt, int src_dtype, int64_t n_seq, int64_t H, int64_t D, const QuantAppendSeq *table,
