@@ -404,6 +404,47 @@ def test_decode_quantised_cache(rt, fmt_name, B, Hq, Hkv, T):
 
 
 @pytest.mark.parametrize("fmt_name", ["Q8_0", "Q4_0"])
+@pytest.mark.parametrize("B,Hq,Hkv,T0", [(2, 32, 8, 61), (1, 16, 2, 30), (2, 32, 2, 95), (1, 6, 2, 0), (8, 32, 8, 2047), (1, 8, 8, 40)])
+def test_decode_steps_quantise_the_new_token_in_the_attention_launch(rt, fmt_name, B, Hq, Hkv, T0):
+    """Single-token steps on a quantised cache (f16 inputs): the attention kernel quantises the step's K and V rows
+    itself, stores them and attends over them.  After every step the cache's canonical blocks equal the CPU quantiser's
+    on all tokens so far, and the output the oracle's attention over the dequantised blocks; the steps cross a tile
+    boundary, and the new rows carry an outlier channel, a zero block and a block with +x and -x of equal magnitude.
+    (One head per kv head takes the separate append launch: same checks.)"""
+    D = 128
+    dev_fmt, orc_fmt = getattr(tract_amd, fmt_name), getattr(orc, "FMT_" + fmt_name)
+    rng = np.random.default_rng(T0 + Hq)
+    st = tract_amd.InPlaceKvSdpa(axis=2, causal=True, storage_format=dev_fmt).state()
+    ks = rng.standard_normal((B, Hkv, T0, D), dtype=np.float32).astype(np.float16)
+    vs = rng.standard_normal((B, Hkv, T0, D), dtype=np.float32).astype(np.float16)
+    if T0:
+        st.k.push(ks), st.v.push(vs)
+    for step in range(5):
+        q = (rng.standard_normal((B, Hq, 1, D), dtype=np.float32) / np.sqrt(D)).astype(np.float16)
+        kn = rng.standard_normal((B, Hkv, 1, D), dtype=np.float32).astype(np.float16)
+        vn = rng.standard_normal((B, Hkv, 1, D), dtype=np.float32).astype(np.float16)
+        kn[..., 7] *= 20
+        vn[:, :, :, 32:64] = 0
+        kn[:, :, :, 64], kn[:, :, :, 65] = np.float16(-30.0), np.float16(30.0)
+        vn[:, :, :, 100], vn[:, :, :, 97] = np.float16(9.5), np.float16(-9.5)
+        # products that round onto a rounding boundary (x = mx / 2: x * (1 / scale) is 63.49999.. before its rounding, 63.5
+        # after): a multiply fused with the addition that follows it would code them differently
+        kn[:, :, :, 96:128] *= np.float16(0.05)
+        mx = np.float16(2.3476562 + 0.001 * step)
+        kn[:, :, :, 96], kn[:, :, :, 97], kn[:, :, :, 98], kn[:, :, :, 99] = mx, mx / np.float16(2), mx / np.float16(16), np.float16(3) * mx / np.float16(16)
+        vn[:, :, :, 0:32] *= np.float16(0.05)
+        vn[:, :, :, 0], vn[:, :, :, 1], vn[:, :, :, 2] = -mx, -mx / np.float16(2), mx / np.float16(2)
+        out = st.eval([q, kn, vn]).to_numpy()
+        ks, vs = np.concatenate([ks, kn], axis=2), np.concatenate([vs, vn], axis=2)
+        kq, vq = orc.quant(orc_fmt, ks), orc.quant(orc_fmt, vs)
+        assert st.k.valid_contiguous().tobytes() == kq.tobytes(), step
+        assert st.v.valid_contiguous().tobytes() == vq.tobytes(), step
+        want = orc.flash_sdpa(q, orc.dequant(orc_fmt, kq, np.float16), orc.dequant(orc_fmt, vq, np.float16), causal=True)
+        assert not np.isnan(out).any() and max_abs(out, want) <= 2e-2, step
+    assert st.k.len() == T0 + 5
+
+
+@pytest.mark.parametrize("fmt_name", ["Q8_0", "Q4_0"])
 @pytest.mark.parametrize("Hq,Hkv,n_seq,lo,hi", [(32, 8, 12, 1, 2500), (16, 1, 5, 20, 700), (8, 8, 4, 10, 200)])
 def test_ragged_decode_over_quantised_caches(rt, fmt_name, Hq, Hkv, n_seq, lo, hi):
     """Independent sequences with quantised caches of their own: every sequence equals the batch-1
@@ -438,6 +479,9 @@ def test_ragged_decode_over_quantised_caches(rt, fmt_name, Hq, Hkv, n_seq, lo, h
     for i in range(n_seq):
         ks[i], vs[i] = np.concatenate([ks[i], kn[i:i + 1]], axis=2), np.concatenate([vs[i], vn[i:i + 1]], axis=2)
     check(out, q)
+    for i in range(n_seq):   # the new tokens' blocks (quantised by the attention launch where it takes them) are the CPU quantiser's
+        assert kcs[i].valid_contiguous().tobytes() == orc.quant(orc_fmt, ks[i]).tobytes(), i
+        assert vcs[i].valid_contiguous().tobytes() == orc.quant(orc_fmt, vs[i]).tobytes(), i
 
 
 def test_ragged_step_over_quantised_caches_with_f32_tokens(rt):

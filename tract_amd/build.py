@@ -82,7 +82,7 @@ def resource_usage() -> dict:
 
 def build(force: bool = False, verbose: bool = True) -> str:
     os.makedirs(OBJ, exist_ok=True)
-    headers = [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "decode_common.h"), os.path.join(HERE, "..", "include", "tract_rocm.h"), __file__]
+    headers = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")) + [os.path.join(HERE, "..", "include", "tract_rocm.h"), __file__]
     jobs = []
     objs = []
     for src in SOURCES:

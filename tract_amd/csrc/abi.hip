@@ -1243,9 +1243,9 @@ int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_n
     } else {
         kv_new_strides = dense;
     }
-    // Decode step on a plain-format cache: the attention kernel reads the new token from the
-    // inputs and stores it into the cache itself -- one launch instead of append + attention.
-    if (n_new == 1 && is_dense && !is_quant(kc->fmt) && dtype == kc->fmt && q && k_new && v_new && out &&
+    // Decode step: the attention kernel reads the new token from the inputs and stores it into the cache itself (a
+    // block-quantised cache: quantises it, f16 inputs) -- one launch instead of append + attention.
+    if (n_new == 1 && is_dense && (is_quant(kc->fmt) ? dtype == TROCM_F16 : dtype == kc->fmt) && q && k_new && v_new && out &&
         kc->window == 0 && vc->window == 0 && kc->fmt == vc->fmt && kc->B == vc->B && kc->H == vc->H && kc->D == vc->D && kc->len == vc->len &&
         q_heads % kc->H == 0) {
         hipStream_t s;
@@ -1256,7 +1256,7 @@ int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_n
             SdpaArgs a;
             cached_args(a, q, dtype, q_heads, 1, kc, vc, kc->len + 1, out, scale, causal, workspace, workspace_bytes);
             a.k_new = k_new, a.v_new = v_new, a.new_pos = -1;
-            int rc = launch_sdpa_decode(a, s);
+            int rc = is_quant(kc->fmt) ? launch_sdpa_decode_quant(a, s) : launch_sdpa_decode(a, s);
             if (rc == 0) {
                 kc->len += 1;
                 vc->len += 1;
@@ -1352,7 +1352,7 @@ static int ragged_common(const void *q, const void *k_new, const void *v_new, in
     const int64_t row_elems = k0->H * k0->D;  // one sequence's new token, all kv heads
     const size_t es = elem_bytes(q_dtype);
     int64_t dense[4] = {row_elems, k0->D, k0->D, 1};
-    bool in_kernel = fused && !is_quant(k0->fmt);
+    bool in_kernel = fused && (!is_quant(k0->fmt) || q_dtype == TROCM_F16);   // (quantised caches: f16 rows, quantised by the attention kernel)
     if (fused) {  // growth first (may reallocate), for every sequence
         for (int64_t i = 0; i < n_seq; i++) {
             const char *kn = (const char *)k_new + (size_t)i * row_elems * es, *vn = (const char *)v_new + (size_t)i * row_elems * es;
@@ -1407,7 +1407,9 @@ static int ragged_common(const void *q, const void *k_new, const void *v_new, in
         if (!in_kernel) return fail("ragged decode: no kernel covers this shape");
         // the kernel cannot append in place for this shape: append explicitly, then attend
         in_kernel = false;
-        if (append_explicitly()) return 1;
+        const bool at_once = is_quant(k0->fmt) && workspace != nullptr && workspace_bytes >= kWsCounterBytes + kWsPlanBytes &&
+                             (size_t)n_seq * sizeof(QuantAppendSeq) <= kWsPlanBytes && k0->D % 32 == 0;
+        if (at_once ? append_quantised_at_once() : append_explicitly()) return 1;
     }
 }
 

@@ -653,7 +653,7 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     if (quant && q_dtype == TROCM_F16 && D == 128 && g_real == 1) mfma_gp = 8;
     const int64_t G = mfma_gp ? mfma_gp : g_real <= 2 ? g_real : g_real <= 4 ? 4 : 8;   // the instantiation that runs it
     const int64_t rb = kv_fmt == TROCM_Q8_0 ? D : kv_fmt == TROCM_Q4_0 ? D / 2 : D * (int64_t)elem_bytes(kv_fmt);   // bytes per token row
-    bool fast = quant ? mfma_gp != 0 && k_new == nullptr
+    bool fast = quant ? mfma_gp != 0 && (k_new == nullptr || (g_real > 1 && decode_quant_appends_in_kernel(g_real, scale)))
                       : (kv_fmt == TROCM_F16 || kv_fmt == TROCM_F32) && q_dtype == kv_fmt && (D == 64 || D == 128) &&
                             g_real >= 1 && (g_real <= 8 || mfma_gp);
     fast = fast && workspace != nullptr && (uintptr_t)q % 16 == 0 && n_seq <= 2048 && Hkv <= 65535;

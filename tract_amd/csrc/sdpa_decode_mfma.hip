@@ -27,6 +27,7 @@
 // (quantised).  Algorithmic bytes as for sdpa_decode.hip and sdpa_decode_quant.hip.
 #include <type_traits>
 #include "decode_common.h"
+#include "quant_block.h"
 
 namespace trocm {
 namespace {
@@ -512,6 +513,52 @@ __device__ __forceinline__ half8_t magic8(uint32_t w0, uint32_t w1) {
 // a wave-private LDS tile (consecutive lanes write consecutive 16-byte slots) -> K fragments by 8-byte (Q4_0: 4-byte)
 // reads, V^T fragments by transposing byte reads; the f16 block scales of the tile (256 bytes per tensor) go through
 // LDS too.
+// A decode step's new token on a block-quantised cache (the fused append): quantised once, by the wave whose tiles
+// include the sequence's last one, exactly as the append kernel would (quant_block.h), written to the cache planes and
+// kept in `lds_new` (K codes, V codes, the K scales, the V scales), from where that wave's tile takes the row -- no other
+// wave of the launch reads it.  Lanes 0..3 take the four K blocks of the row, lanes 4..7 the V blocks.
+template <int FMT>
+__device__ __forceinline__ void quantise_new_token(const DecodeDev &p, const MfmaWork &wk, int lane, unsigned char *lds_new) {
+    constexpr bool Q8 = FMT == TROCM_Q8_0;
+    constexpr int D = 128, RB = Q8 ? D : D / 2, BB = Q8 ? 32 : 16, SROW = (D / 32) * 2;
+    if (lane < 8) {
+        const int blk = lane & 3;
+        const bool is_v = lane >= 4;
+        const __half *src = reinterpret_cast<const __half *>(is_v ? p.v_new : p.k_new) + ((int64_t)wk.seq * p.Hkv + wk.kvh) * D + 32 * blk;
+        float v[32];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint4 x = reinterpret_cast<const uint4 *>(src)[i];
+            const __half *e = reinterpret_cast<const __half *>(&x);
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[8 * i + j] = __half2float(e[j]);
+        }
+        unsigned char *codes_lds = lds_new + (is_v ? RB : 0) + blk * BB;
+        char *codes_mem = const_cast<char *>(is_v ? wk.vbase : wk.kbase) + (int64_t)wk.new_pos * RB + blk * BB;
+        uint16_t d;
+        if constexpr (Q8) {
+            uint32_t c[8];
+            d = quant_q8(v, c);
+            constexpr uint32_t x = 0x80808080u;   // the plane holds code + 128
+            const u32x4 lo4 = {c[0] ^ x, c[1] ^ x, c[2] ^ x, c[3] ^ x}, hi4 = {c[4] ^ x, c[5] ^ x, c[6] ^ x, c[7] ^ x};
+            reinterpret_cast<u32x4 *>(codes_lds)[0] = lo4, reinterpret_cast<u32x4 *>(codes_lds)[1] = hi4;
+            reinterpret_cast<u32x4 *>(codes_mem)[0] = lo4, reinterpret_cast<u32x4 *>(codes_mem)[1] = hi4;
+        } else {
+            uint32_t c[4];
+            d = quant_q4(v, c);
+            const u32x4 c4 = {c[0], c[1], c[2], c[3]};
+            *reinterpret_cast<u32x4 *>(codes_lds) = c4;
+            *reinterpret_cast<u32x4 *>(codes_mem) = c4;
+        }
+        reinterpret_cast<uint16_t *>(lds_new + 2 * RB)[lane] = d;   // K scales 0..3, V scales 4..7
+        *reinterpret_cast<uint16_t *>(const_cast<char *>(is_v ? wk.vsbase : wk.ksbase) + (int64_t)wk.new_pos * SROW + blk * 2) = d;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the wave's other lanes read the row back from LDS
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+constexpr int kNewTokenLdsBytes = 2 * 128 + 16;   // two rows of codes (Q8_0: 128 bytes each) and eight scales
+
 template <int GP, int FMT, int PF>
 __device__ __forceinline__ void decode_mfma_qblock_body(const DecodeDev &p, const MfmaWork &wk) {
     static_assert(GP <= 16, "the 16-wide layout: at most 16 heads");
@@ -525,7 +572,7 @@ __device__ __forceinline__ void decode_mfma_qblock_body(const DecodeDev &p, cons
     constexpr int SROW = NB * 2;               // bytes of block scales per row
     constexpr int kCodeBytes = kTile * RB;     // one tensor's tile in LDS
     constexpr int kScaleBytes = kTile * SROW;
-    constexpr int kWaveBytes = 2 * kCodeBytes + 2 * kScaleBytes;
+    constexpr int kWaveBytes = 2 * kCodeBytes + 2 * kScaleBytes + kNewTokenLdsBytes;
     constexpr int kCombStride = GP * D + 2 * GP;
     constexpr int kLdsBytes = kWaves * (kWaveBytes > kCombStride * 4 ? kWaveBytes : kCombStride * 4);
     __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kLdsBytes];
@@ -549,11 +596,14 @@ __device__ __forceinline__ void decode_mfma_qblock_body(const DecodeDev &p, cons
     // not cover the memory latency at full bandwidth)
     u32x4 kpre[PF][NLD], vpre[PF][NLD];
     u32x2 kspre[PF], vspre[PF];
-    auto fetch = [&](const char *base0, const char *sbase0, int t, u32x4 (&dst)[NLD], u32x2 &sc) {
+    // (a fused append's new token is the sequence's last: its tile takes the row from lds_new, see quantise_new_token)
+    const int new_pos = wk.new_pos;
+    unsigned char *lds_new = lds_raw + w * kWaveBytes + 2 * kCodeBytes + 2 * kScaleBytes;
+    auto fetch = [&](const char *base0, const char *sbase0, int which, int t, u32x4 (&dst)[NLD], u32x2 &sc) {
         const int t0 = t * kTile;
         const char *base = base0 + (int64_t)t0 * RB;
         const char *sbase = sbase0 + (int64_t)t0 * SROW;
-        if (t0 + kTile <= T) {
+        if (t0 + kTile <= T && !(new_pos >= t0 && new_pos < t0 + kTile)) {
 #pragma unroll
             for (int j = 0; j < NLD; j++)
                 dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + (j * 64 + lane) * 16));
@@ -563,9 +613,14 @@ __device__ __forceinline__ void decode_mfma_qblock_body(const DecodeDev &p, cons
 #pragma unroll
             for (int j = 0; j < NLD; j++) {
                 const int c = j * 64 + lane, row = min(c / CPR, last), dc = c % CPR;
-                dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + row * RB + dc * 16));
+                if (t0 + row == new_pos) dst[j] = *reinterpret_cast<const u32x4 *>(lds_new + which * RB + dc * 16);
+                else dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + row * RB + dc * 16));
             }
-            if (lane < kTile) sc = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(sbase + min(lane, last) * SROW));
+            if (lane < kTile) {
+                const int row = min(lane, last);
+                if (t0 + row == new_pos) sc = *reinterpret_cast<const u32x2 *>(lds_new + 2 * RB + which * 8);
+                else sc = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(sbase + row * SROW));
+            }
         }
     };
     // Where this lane's chunks go in the LDS tiles.  The 16-byte chunks of a row are permuted (xor with a key of the row)
@@ -583,12 +638,16 @@ __device__ __forceinline__ void decode_mfma_qblock_body(const DecodeDev &p, cons
     }
     const int tstep = wk.tile_step;
     int t = tile_begin + w;
+    if (new_pos >= 0) {   // (wave-uniform) the wave whose tiles include the new token's quantises and stores it
+        const int nt = new_pos / kTile;
+        if (nt >= t && nt < tile_end && (nt - t) % tstep == 0) quantise_new_token<FMT>(p, wk, lane, lds_new);
+    }
 #pragma unroll
     for (int st = 0; st < PF; st++) {
         kspre[st] = vspre[st] = u32x2{0u, 0u};
         if (t + st * tstep < tile_end) {
-            fetch(wk.kbase, wk.ksbase, t + st * tstep, kpre[st], kspre[st]);
-            fetch(wk.vbase, wk.vsbase, t + st * tstep, vpre[st], vspre[st]);
+            fetch(wk.kbase, wk.ksbase, 0, t + st * tstep, kpre[st], kspre[st]);
+            fetch(wk.vbase, wk.vsbase, 1, t + st * tstep, vpre[st], vspre[st]);
         }
     }
 
@@ -666,8 +725,8 @@ __device__ __forceinline__ void decode_mfma_qblock_body(const DecodeDev &p, cons
             *reinterpret_cast<u32x2 *>(lds_vs + lane * SROW) = vspre[ST];
         }
         if (more) {
-            fetch(wk.kbase, wk.ksbase, t + PF * tstep, kpre[ST], kspre[ST]);
-            fetch(wk.vbase, wk.vsbase, t + PF * tstep, vpre[ST], vspre[ST]);
+            fetch(wk.kbase, wk.ksbase, 0, t + PF * tstep, kpre[ST], kspre[ST]);
+            fetch(wk.vbase, wk.vsbase, 1, t + PF * tstep, vpre[ST], vspre[ST]);
         }
         // ---- per block: codes x query features, the bias riding in the accumulator -------------------------------
         float4_t acc[2][NB];
@@ -868,7 +927,7 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
     constexpr int SROW = NB * 2;               // bytes of block scales per row
     constexpr int kCodeBytes = kTile * RB;     // one tensor's tile in LDS
     constexpr int kScaleBytes = kTile * SROW;
-    constexpr int kWaveBytes = 2 * kCodeBytes + 2 * kScaleBytes;
+    constexpr int kWaveBytes = 2 * kCodeBytes + 2 * kScaleBytes + kNewTokenLdsBytes;
     constexpr int kCombStride = GP * D + 2 * GP;
     constexpr int kLdsBytes = kWaves * (kWaveBytes > kCombStride * 4 ? kWaveBytes : kCombStride * 4);
     __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kLdsBytes];
@@ -889,11 +948,14 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
 
     u32x4 kpre[PF][NLD], vpre[PF][NLD];
     u32x2 kspre[PF], vspre[PF];
-    auto fetch = [&](const char *base0, const char *sbase0, int t, u32x4 (&dst)[NLD], u32x2 &sc) {
+    // (a fused append's new token is the sequence's last: its tile takes the row from lds_new, see quantise_new_token)
+    const int new_pos = wk.new_pos;
+    unsigned char *lds_new = lds_raw + w * kWaveBytes + 2 * kCodeBytes + 2 * kScaleBytes;
+    auto fetch = [&](const char *base0, const char *sbase0, int which, int t, u32x4 (&dst)[NLD], u32x2 &sc) {
         const int t0 = t * kTile;
         const char *base = base0 + (int64_t)t0 * RB;
         const char *sbase = sbase0 + (int64_t)t0 * SROW;
-        if (t0 + kTile <= T) {
+        if (t0 + kTile <= T && !(new_pos >= t0 && new_pos < t0 + kTile)) {
 #pragma unroll
             for (int j = 0; j < NLD; j++)
                 dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + (j * 64 + lane) * 16));
@@ -903,9 +965,14 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
 #pragma unroll
             for (int j = 0; j < NLD; j++) {
                 const int c = j * 64 + lane, row = min(c / CPR, last), dc = c % CPR;
-                dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + row * RB + dc * 16));
+                if (t0 + row == new_pos) dst[j] = *reinterpret_cast<const u32x4 *>(lds_new + which * RB + dc * 16);
+                else dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + row * RB + dc * 16));
             }
-            if (lane < kTile) sc = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(sbase + min(lane, last) * SROW));
+            if (lane < kTile) {
+                const int row = min(lane, last);
+                if (t0 + row == new_pos) sc = *reinterpret_cast<const u32x2 *>(lds_new + 2 * RB + which * 8);
+                else sc = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(sbase + row * SROW));
+            }
         }
     };
     // code tiles in LDS exactly as in the block-scaling body (16-byte chunks of a row permuted by a key of the row)
@@ -920,12 +987,16 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
     }
     const int tstep = wk.tile_step;
     int t = tile_begin + w;
+    if (new_pos >= 0) {   // (wave-uniform) the wave whose tiles include the new token's quantises and stores it
+        const int nt = new_pos / kTile;
+        if (nt >= t && nt < tile_end && (nt - t) % tstep == 0) quantise_new_token<FMT>(p, wk, lane, lds_new);
+    }
 #pragma unroll
     for (int st = 0; st < PF; st++) {
         kspre[st] = vspre[st] = u32x2{0u, 0u};
         if (t + st * tstep < tile_end) {
-            fetch(wk.kbase, wk.ksbase, t + st * tstep, kpre[st], kspre[st]);
-            fetch(wk.vbase, wk.vsbase, t + st * tstep, vpre[st], vspre[st]);
+            fetch(wk.kbase, wk.ksbase, 0, t + st * tstep, kpre[st], kspre[st]);
+            fetch(wk.vbase, wk.vsbase, 1, t + st * tstep, vpre[st], vspre[st]);
         }
     }
 
@@ -1017,8 +1088,8 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
             vsT[2 * kTile] = (uint16_t)vspre[ST].y, vsT[3 * kTile] = (uint16_t)(vspre[ST].y >> 16);
         }
         if (more) {
-            fetch(wk.kbase, wk.ksbase, t + PF * tstep, kpre[ST], kspre[ST]);
-            fetch(wk.vbase, wk.vsbase, t + PF * tstep, vpre[ST], vspre[ST]);
+            fetch(wk.kbase, wk.ksbase, 0, t + PF * tstep, kpre[ST], kspre[ST]);
+            fetch(wk.vbase, wk.vsbase, 1, t + PF * tstep, vpre[ST], vspre[ST]);
         }
         // ---- codes x block-diagonal query operands: column (blk, h) receives the sum over block blk ----------------------
         float4_t acc[2];
@@ -1636,6 +1707,13 @@ int launch_sdpa_decode_ragged_mfma(const DecodeDev &p, int kv_fmt, int gp, int64
 
 // Quantised cache planes (the caller has checked formats, alignment and strides and filled p but for the
 // splits): 2 = not taken (one head per kv head).
+// Whether the launch below would run one of the two bodies that take a step's new token from the step's inputs.
+bool decode_quant_appends_in_kernel(int64_t g_real, float scale) {
+    static const int on = getenv("TROCM_DECODE_QUANT_FUSED_APPEND") ? atoi(getenv("TROCM_DECODE_QUANT_FUSED_APPEND")) : 1;
+    const int gp = decode_mfma_group(g_real);
+    return on && gp != 0 && gp <= 16 && use_16_wide(TROCM_Q8_0) && use_block_scaling() && scale > 0.0f;
+}
+
 int launch_sdpa_decode_quant_mfma(DecodeDev &p, int kv_fmt, int64_t B, void *workspace, size_t workspace_bytes, hipStream_t s) {
     const int gp = decode_mfma_group(p.g_real);
     if (gp == 0) return 2;

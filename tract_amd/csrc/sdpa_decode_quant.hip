@@ -406,6 +406,10 @@ int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s) {
     const int64_t g_real = a.Hq / a.Hkv;
     const bool mfma = decode_mfma_group(g_real) != 0;   // grouped heads: the MFMA formulation (sdpa_decode_mfma.hip)
     if (g_real > 8 && !mfma) return 2;
+    // a fused append (the step's new token, f16 rows [B, Hkv, 1, D] like q): only the block-scaling MFMA bodies take it
+    if (a.k_new && (!mfma || !decode_quant_appends_in_kernel(g_real, a.scale) || a.v_new == nullptr || a.new_pos >= 0 ||
+                    (uintptr_t)a.k_new % 16 || (uintptr_t)a.v_new % 16))
+        return 2;
     const int64_t G = g_real <= 2 ? g_real : g_real <= 4 ? 4 : 8;   // the instantiation that runs it
     if (a.kv_stride_t != a.D) return 2;  // cache planes: token rows are dense
     if ((uintptr_t)a.k % 16 || (uintptr_t)a.v % 16 || (uintptr_t)a.q % 16 || (uintptr_t)a.k_scales % 4 ||
@@ -428,7 +432,8 @@ int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s) {
         p.T = (int)a.Sk;
         p.Hq = (int)a.Hq, p.Hkv = (int)a.Hkv, p.g_real = (int)g_real;
         p.scale_log2 = a.scale * 1.4426950408889634f;
-        p.new_pos = -1;
+        p.k_new = (const char *)a.k_new, p.v_new = (const char *)a.v_new;
+        p.new_pos = a.k_new ? (int)a.Sk - 1 : -1;
         return launch_sdpa_decode_quant_mfma(p, a.kv_fmt, a.B, a.workspace, a.workspace_bytes, s);
     }
     int n_tiles = (int)((a.Sk + kTile - 1) / kTile);
