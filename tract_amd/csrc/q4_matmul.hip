@@ -10,7 +10,7 @@
 //
 // C^T[n, m] = W[n, k] . act^T[k, m] with v_mfma_f32_32x32x16_f16: both operands are rows of k, so every fragment
 // is one 128-bit LDS read.  A workgroup of 4 waves owns a 128 x 128 tile of C^T (each wave 64 x 64: four
-// accumulators), walks k in chunks of 64 (two quantisation blocks), and keeps the next chunk in registers while
+// accumulators; 128 x 64 with two accumulators per wave when the larger tiles would be fewer than the compute units), walks k in chunks of 64 (two quantisation blocks), and keeps the next chunk in registers while
 // it multiplies the current one: a thread fetches the 16 code bytes and the scale of one weight block and four
 // 16-byte pieces of the activations, dequantises its block on the way into LDS (one v_perm per two codes puts the
 // nibble under the exponent byte 0x64: 1024 + u; minus 1032 is exact; times d rounds once).
@@ -31,7 +31,7 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kMmThreads = 256;
-constexpr int BN = 128, BM = 128, BK = 64;
+constexpr int BN = 128, BK = 64;   // (the tile's m extent BM is 128, or 64 when 128 would leave compute units without a tile)
 constexpr int ROW = BK + 8;   // halves per tile row in LDS: the 16 rows of a 128-bit read pass fall into 16 distinct bank groups
 
 struct MatMulDev {
@@ -52,14 +52,17 @@ __device__ __forceinline__ void dequant4(uint32_t w, half2_t d2, uint32_t &lo, u
     hi = __builtin_bit_cast(uint32_t, (as_half2(perm(0x64646464u, w, 0x04030402u)) - zero) * d2);
 }
 
+template <int BM>
 __global__ __launch_bounds__(kMmThreads, 2) void q4_0_matmul_kernel(MatMulDev p) {
+    constexpr int MJ = BM / 64;        // 32-row halves of m per wave: the wave's corner is 64 (n) x 32 MJ (m)
+    constexpr int AP = BM * 8 / kMmThreads;   // 16-byte activation pieces per thread and chunk
     __shared__ __attribute__((aligned(16))) _Float16 lds_w[2][BN * ROW];
     __shared__ __attribute__((aligned(16))) _Float16 lds_a[2][BM * ROW];
 
     const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hb = lane >> 5, l32 = lane & 31;
     const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM, b = blockIdx.z, wb = b / p.ratio;
-    const int wn = 64 * (w & 1), wm = 64 * (w >> 1);   // this wave's 64 x 64 corner of the tile
+    const int wn = 64 * (w & 1), wm = 32 * MJ * (w >> 1);   // this wave's corner of the tile
     const int nb = p.k / 32;
 
     // staging roles: weight block (row tid / 2, block tid % 2 of the chunk); activation pieces j * 256 + tid
@@ -68,20 +71,20 @@ __global__ __launch_bounds__(kMmThreads, 2) void q4_0_matmul_kernel(MatMulDev p)
     const uint8_t *w_codes = p.codes + w_grow * (p.k / 2) + w_blk * 16;
     const uint16_t *w_scales = p.scales + w_grow * nb + w_blk;
     const _Float16 *a_base = p.act + (int64_t)b * p.m * p.k;
-    int a_row[4], a_col[4];
+    int a_row[AP], a_col[AP];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < AP; j++) {
         const int c = j * kMmThreads + tid;
         a_row[j] = c >> 3, a_col[j] = (c & 7) * 8;
     }
 
-    u32x4 cpre, apre[4];
+    u32x4 cpre, apre[AP];
     uint16_t spre;
     auto prefetch = [&](int k0) {
         cpre = *reinterpret_cast<const u32x4 *>(w_codes + (k0 / 32) * 16);
         spre = w_scales[k0 / 32];
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < AP; j++)
             apre[j] = *reinterpret_cast<const u32x4 *>(a_base + (int64_t)min(m0 + a_row[j], p.m - 1) * p.k + k0 + a_col[j]);
     };
     auto stage = [&](int buf) {
@@ -100,14 +103,14 @@ __global__ __launch_bounds__(kMmThreads, 2) void q4_0_matmul_kernel(MatMulDev p)
         dst[2] = u32x4{hi[0], hi[1], hi[2], hi[3]};
         dst[3] = u32x4{hi[4], hi[5], hi[6], hi[7]};
 #pragma unroll
-        for (int j = 0; j < 4; j++) *reinterpret_cast<u32x4 *>(&lds_a[buf][a_row[j] * ROW + a_col[j]]) = apre[j];
+        for (int j = 0; j < AP; j++) *reinterpret_cast<u32x4 *>(&lds_a[buf][a_row[j] * ROW + a_col[j]]) = apre[j];
     };
 
-    float16_t acc[2][2];   // [n half][m half] of the wave's corner
+    float16_t acc[2][MJ];   // [n half][m half] of the wave's corner
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < MJ; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
@@ -126,16 +129,15 @@ __global__ __launch_bounds__(kMmThreads, 2) void q4_0_matmul_kernel(MatMulDev p)
         const _Float16 *at = &lds_a[cur][(wm + l32) * ROW + 8 * hb];
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ks++) {
-            half8_t wf[2], af[2];
+            half8_t wf[2], af[MJ];
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                wf[i] = *reinterpret_cast<const half8_t *>(wt + (32 * i) * ROW + 16 * ks);
-                af[i] = *reinterpret_cast<const half8_t *>(at + (32 * i) * ROW + 16 * ks);
-            }
+            for (int i = 0; i < 2; i++) wf[i] = *reinterpret_cast<const half8_t *>(wt + (32 * i) * ROW + 16 * ks);
+#pragma unroll
+            for (int j = 0; j < MJ; j++) af[j] = *reinterpret_cast<const half8_t *>(at + (32 * j) * ROW + 16 * ks);
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[i], af[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < MJ; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[i], af[j], acc[i][j], 0, 0, 0);
         }
     }
 
@@ -143,7 +145,7 @@ __global__ __launch_bounds__(kMmThreads, 2) void q4_0_matmul_kernel(MatMulDev p)
     _Float16 *out = p.out + (int64_t)b * p.m * p.n;
     const bool vec = (p.n % 4) == 0;
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
+    for (int j = 0; j < MJ; j++) {
         const int mi = m0 + wm + 32 * j + l32;
         if (mi >= p.m) continue;
         _Float16 *orow = out + (int64_t)mi * p.n;
@@ -181,9 +183,15 @@ int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, i
     p.codes = (const uint8_t *)codes, p.scales = (const uint16_t *)scales;
     p.act = (const _Float16 *)act, p.out = (_Float16 *)out;
     p.n = (int)n, p.k = (int)k, p.m = (int)m, p.ratio = (int)(act_batch / w_batch);
-    const int64_t gx = (n + BN - 1) / BN, gy = (m + BM - 1) / BM;
+    // 128 x 128 tiles unless they are fewer than the compute units: then 128 (n) x 64 (m), twice as many workgroups
+    const int64_t gx = (n + BN - 1) / BN;
+    const bool half_m = gx * ((m + 127) / 128) * act_batch < num_compute_units() && m > 64;
+    const int64_t gy = half_m ? (m + 63) / 64 : (m + 127) / 128;
     if (gy > 65535) return 2;
-    hipLaunchKernelGGL(q4_0_matmul_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)act_batch), dim3(kMmThreads), 0, s, p);
+    if (half_m)
+        hipLaunchKernelGGL(q4_0_matmul_kernel<64>, dim3((unsigned)gx, (unsigned)gy, (unsigned)act_batch), dim3(kMmThreads), 0, s, p);
+    else
+        hipLaunchKernelGGL(q4_0_matmul_kernel<128>, dim3((unsigned)gx, (unsigned)gy, (unsigned)act_batch), dim3(kMmThreads), 0, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("q4_0_matmul launch failed: %s", hipGetErrorString(e));
     return 0;
