@@ -538,7 +538,7 @@ def run_kivi(ta, args):
                 got["packed"][at].tobytes() == want["packed"].tobytes() and np.array_equal(got["lo"][at], want["lo"])
                 and np.array_equal(got["scale"][at], want["scale"]) and got["sink"][at].tobytes() == want["sink"].tobytes())
             del caches, outs
-    # QuantizedKvSdpa: one decode step over an 8192-token cache (two single-token appends, attention straight over the codes)
+    # QuantizedKvSdpa: one decode step over an 8192-token cache (one launch pushes the token, one attends over the codes)
     Tc = 8192
     st = ta.QuantizedKvSdpa(axis=2).state()
     kq_np, vq_np = seeded_f16(cfg_seed(2, "k"), (B, HKV, Tc, D)), seeded_f16(cfg_seed(2, "v"), (B, HKV, Tc, D))
@@ -560,7 +560,7 @@ def run_kivi(ta, args):
     T_end = st.k.len()
     step_bytes = B * HKV * (Tc + (T_end - Tc) // 2) * (2 * D + 8) + B * HKV * D * 8 + 2 * B * HQ * D * 2
     case = {"us": round(us, 2), "bytes": step_bytes, "gbs": round(step_bytes / us / 1e3, 1),
-            "note": "two single-token appends + attention straight over the u8 codes (TROCM_KIVI_FUSED=0: append + dequantise K and V + f16 attention)"}
+            "note": "the new token's K and V rows pushed by one launch + attention straight over the u8 codes (TROCM_KIVI_FUSED=0: push + dequantise K and V + f16 attention)"}
     # after the timing: the last step's output for one kv head against the oracle's attention over its own stores
     b0, h0, g = 5, 3, HQ // HKV
     tok_np = tok.to_numpy()

@@ -411,6 +411,56 @@ __global__ void __launch_bounds__(256) kivi_quant_tokens_vec_kernel(const SrcT *
     }
 }
 
+// One decode step of QuantizedKvSdpa in one launch (head_dim 128, u8 codes): the new token's Key row into the running
+// per-channel store (a thread per channel, as kivi_running_push_kernel) and its Value row into the per-token store (16
+// lanes of 8 channels, as kivi_quant_tokens_vec_kernel).  Grid (batch * heads, 2) x 128 threads; sources [BH, 1, 128].
+template <typename SrcT>
+__global__ void __launch_bounds__(128) kivi_step_push_kernel(const SrcT *__restrict__ k_src, const SrcT *__restrict__ v_src,
+                                                             uint8_t *__restrict__ k_codes, int64_t k_cap_rows, int64_t k_row0,
+                                                             float *__restrict__ k_lo_io, float *__restrict__ k_scale_io,
+                                                             uint8_t *__restrict__ v_codes, int64_t v_cap_rows, int64_t v_row0,
+                                                             float *__restrict__ v_lo_out, float *__restrict__ v_scale_out) {
+    constexpr int D = 128;
+    const int bh = blockIdx.x;
+    if (blockIdx.y == 0) {
+        const int c = threadIdx.x;
+        float lo = k_lo_io[(int64_t)bh * D + c], scale = k_scale_io[(int64_t)bh * D + c];
+        const float val = ld(k_src + (int64_t)bh * D + c);
+        if (val < lo) lo = val;
+        const float range = __fsub_rn(val, lo);
+        if (range > 0.0f) {
+            const float ns = __fdiv_rn(range, 255.0f);
+            if (ns > scale) scale = ns;
+        }
+        k_codes[((int64_t)bh * k_cap_rows + k_row0) * D + c] = (uint8_t)affine_code(val, lo, scale, 255.0f);
+        k_lo_io[(int64_t)bh * D + c] = lo;
+        k_scale_io[(int64_t)bh * D + c] = scale;
+    } else {
+        const int sub = threadIdx.x;
+        if (sub >= 16) return;   // (the exchanges below stay inside the first 16 lanes)
+        const F8 x = ld8(v_src + (int64_t)bh * D + sub * 8);
+        float lo = INFINITY, hi = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            lo = fminf(lo, x.v[e]);
+            hi = fmaxf(hi, x.v[e]);
+        }
+#pragma unroll
+        for (int m = 8; m >= 1; m >>= 1) {
+            lo = fminf(lo, __shfl_xor(lo, m, 64));
+            hi = fmaxf(hi, __shfl_xor(hi, m, 64));
+        }
+        const float scale = affine_scale(lo, hi, 255.0f), inv = affine_inv(scale);
+        uint32_t code[8];
+        affine_codes8(x.v, lo, scale, inv, 255.0f, code);
+        store_codes8<8>(v_codes + ((int64_t)bh * v_cap_rows + v_row0) * D, sub, code);
+        if (sub == 0) {
+            v_lo_out[(int64_t)bh * v_cap_rows + v_row0] = lo;
+            v_scale_out[(int64_t)bh * v_cap_rows + v_row0] = scale;
+        }
+    }
+}
+
 // Keys: one wave per block whose 32 rows all come from the new tokens; the wave's 64 / LPR lane groups take the rows
 // in turn, join their lo / hi, and code their rows in a second pass (the rows are in the cache by then).
 template <typename SrcT, int BITS, int LPR>
@@ -983,8 +1033,27 @@ int trocm_quantized_kv_sdpa_eval(const void *q, const void *k_new, const void *v
                   (long long)q_heads, (long long)k_cache->H);
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
-    if (trocm_kivi_cache_append(k_cache, k_new, dtype, n_new, s)) return 1;
-    if (trocm_kivi_cache_append(v_cache, v_new, dtype, n_new, s)) return 1;
+    // a decode step on the op's own stores: both rows pushed by one launch
+    if (n_new == 1 && k_cache->D == 128 && k_cache->layout == TROCM_KIVI_RUNNING_CHANNEL && v_cache->layout == TROCM_KIVI_PER_TOKEN &&
+        k_cache->bits == 8 && v_cache->bits == 8 && k_cache->sink_tokens == 0 && v_cache->sink_tokens == 0 &&
+        ((uintptr_t)v_new & 15) == 0 && (k_cache->len + 1) * 128 < (1ll << 31)) {
+        for (trocm_kivi_cache *c : {k_cache, v_cache}) {
+            if (kivi_alloc_fixed(c, s)) return 1;
+            if (kivi_ensure_rows(c, c->n_rows + 1, s)) return 1;
+        }
+        const dim3 grid((unsigned)k_cache->BH, 2);
+        if (dtype == TROCM_F16)
+            kivi_step_push_kernel<__half><<<grid, 128, 0, s>>>((const __half *)k_new, (const __half *)v_new, k_cache->codes, k_cache->cap_rows, k_cache->n_rows,
+                                                               k_cache->lo, k_cache->scale, v_cache->codes, v_cache->cap_rows, v_cache->n_rows, v_cache->lo, v_cache->scale);
+        else
+            kivi_step_push_kernel<float><<<grid, 128, 0, s>>>((const float *)k_new, (const float *)v_new, k_cache->codes, k_cache->cap_rows, k_cache->n_rows,
+                                                              k_cache->lo, k_cache->scale, v_cache->codes, v_cache->cap_rows, v_cache->n_rows, v_cache->lo, v_cache->scale);
+        TROCM_HIP(hipGetLastError());
+        for (trocm_kivi_cache *c : {k_cache, v_cache}) c->n_rows += 1, c->len += 1;
+    } else {
+        if (trocm_kivi_cache_append(k_cache, k_new, dtype, n_new, s)) return 1;
+        if (trocm_kivi_cache_append(v_cache, v_new, dtype, n_new, s)) return 1;
+    }
     const int64_t T = k_cache->len, D = k_cache->D;
     // One token of f16 queries over the op's own stores (Keys under running per-channel parameters, Values per token, u8
     // codes, nothing kept in f32): attention straight over the codes, no dequantised copy.  TROCM_KIVI_FUSED=0 keeps
