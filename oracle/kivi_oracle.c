@@ -13,8 +13,8 @@
  *
  * Every float step is the reference's: f32 subtraction, IEEE division, f32::round (half away from
  * zero), clamp, saturating `as u8` (NaN -> 0); dequantisation is `lo + code * scale` with two
- * roundings (compiled with -ffp-contract=off).  f32::min / f32::max ignore a NaN operand, as fminf /
- * fmaxf do.  Parity unpinned: the sign of a zero `lo` (Rust leaves min(+0, -0) to the platform).
+ * roundings (compiled with -ffp-contract=off).  f32::min / f32::max ignore a NaN operand of either kind
+ * (rust_min / rust_max below; the C library's fminf / fmaxf answer NaN for a signalling one).  Parity unpinned: the sign of a zero `lo` (Rust leaves min(+0, -0) to the platform).
  */
 #include <math.h>
 #include <stdint.h>
@@ -35,6 +35,10 @@ static uint8_t code_of(float x, float lo, float scale, float lv) {
     return (uint8_t)q;
 }
 
+/* f32::min / f32::max (core::f32): the other operand when one is NaN, quiet or signalling. */
+static float rust_min(float a, float b) { return a != a ? b : (b != b ? a : (b < a ? b : a)); }
+static float rust_max(float a, float b) { return a != a ? b : (b != b ? a : (b > a ? b : a)); }
+
 /* kv_quant.rs:73-98 */
 ORC_API void orc_kivi_quant_dequant(const float *x, size_t r, size_t c, unsigned bits, int by_row, float *out) {
     float levels = (float)((1u << bits) - 1u);
@@ -43,8 +47,8 @@ ORC_API void orc_kivi_quant_dequant(const float *x, size_t r, size_t c, unsigned
         float lo = INFINITY, hi = -INFINITY;
         for (size_t k = 0; k < n_in; k++) {
             float v = by_row ? x[g * c + k] : x[k * c + g];
-            lo = fminf(lo, v);
-            hi = fmaxf(hi, v);
+            lo = rust_min(lo, v);
+            hi = rust_max(hi, v);
         }
         float scale = hi > lo ? (hi - lo) / levels : 1.0f;
         for (size_t k = 0; k < n_in; k++) {
@@ -164,8 +168,8 @@ static void finalize_block(orc_kivi *s) {
         float l = INFINITY, h = -INFINITY;
         for (size_t t = 0; t < s->n_res; t++) {
             float v = s->residual[t * d + c];
-            l = fminf(l, v);
-            h = fmaxf(h, v);
+            l = rust_min(l, v);
+            h = rust_max(h, v);
         }
         lo[c] = l;
         sc[c] = h > l ? (h - l) / lv : 1.0f;
@@ -194,8 +198,8 @@ ORC_API void orc_kivi_push(void *p, const float *row) {
         float lv = (float)((1u << s->bits) - 1u);
         float lo = INFINITY, hi = -INFINITY;
         for (size_t c = 0; c < d; c++) {
-            lo = fminf(lo, row[c]);
-            hi = fmaxf(hi, row[c]);
+            lo = rust_min(lo, row[c]);
+            hi = rust_max(hi, row[c]);
         }
         float scale = hi > lo ? (hi - lo) / lv : 1.0f;
         uint8_t *codes = (uint8_t *)malloc(d);

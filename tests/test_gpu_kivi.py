@@ -116,6 +116,10 @@ def test_nan_inf_and_constant_rows(rt):
     x[0, 0, 8, 9] = -np.inf
     x[0, 0, 9, :] = 2.5
     x[0, 0, 40, 1] = np.nan
+    x.view(np.uint32)[0, 0, 42, 2] = 0x7FA00000   # signalling NaNs: skipped like the quiet ones, in a token and in a channel
+    x[0, 0, 42, 3], x[0, 0, 42, 1] = 50.0, -60.0
+    x.view(np.uint32)[0, 0, 50, 7] = 0xFFA00001
+    x[0, 0, 49, 7], x[0, 0, 51, 7] = 70.0, -80.0
     x[0, 0, 41, 2] = np.inf
     for per_channel in (False, True):
         for bits in (4, 8):

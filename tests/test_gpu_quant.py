@@ -37,6 +37,10 @@ def _nasty(rng, n_blocks, dt):
     x[15, 0], x[15, 4], x[15, 9] = np.nan, -7000.0, 7000.0
     x[16, 1:] = np.nan                                   # one number among NaN
     x[17, :] = -2.5
+    x[18, 0], x[18, 1], x[18, 2] = 1.0, 900.0, 3.0          # a signalling NaN beside the block's largest value:
+    x.view(np.uint32)[18, 3] = 0x7FA00000                     # ignored like any NaN, and it must not take its neighbours along
+    x[19, 5], x[19, 6], x[19, 7] = -700.0, 2.0, 1.0
+    x.view(np.uint32)[19, 4] = 0xFFA00001
     return x.astype(dt)
 
 

@@ -83,6 +83,26 @@ def test_nan_and_inf_rows_by_hand():
     assert np.isposinf(st["lo"][0]) and st["scale"].tolist() == [1.0] and st["packed"].tolist() == [[0, 0]]
 
 
+def test_signalling_nan_is_ignored_like_a_quiet_one():
+    # f32::min / f32::max return the other operand for ANY NaN (core::f32: "handles all NaNs the same way"); C's fminf /
+    # fmaxf answer NaN for a signalling one, after which the running minimum would forget what it had seen
+    row = np.array([-60.0, 0.0, 50.0, 1.0], np.float32)
+    row.view(np.uint32)[1] = 0x7FA00000
+    s = orc.KiviStore(orc.KIVI_PER_TOKEN, 4, 8, 0)
+    s.push_token(row)
+    st = s.state()
+    assert st["lo"].tolist() == [-60.0] and st["scale"][0] == np.float32(np.float32(110.0) / np.float32(255.0))
+    assert st["packed"].tolist() == [[0, 0, 255, 141]]          # 61 / (110 / 255) = 141.4
+    blk = np.zeros((32, 1), np.float32)
+    blk[3, 0], blk[5, 0] = 70.0, -80.0
+    blk.view(np.uint32)[4, 0] = 0xFFA00001
+    s = orc.KiviStore(orc.KIVI_BLOCK_CHANNEL, 1, 8, 0)
+    for r in blk:
+        s.push_token(r)
+    st = s.state()
+    assert st["lo"].reshape(-1).tolist() == [-80.0] and st["scale"].reshape(-1)[0] == np.float32(np.float32(150.0) / np.float32(255.0))
+
+
 def test_running_channel_by_hand():
     # kv_quant.rs:200-222 with one channel: lo follows the minimum, scale only grows, old codes are kept and
     # read back with the CURRENT parameters (:224-234)

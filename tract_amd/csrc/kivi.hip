@@ -32,6 +32,10 @@ namespace {
 constexpr int kKeyBlock = 32;   // quant_dyn_kv_cache.rs:153
 
 __device__ __forceinline__ float ld(const float *p) { return *p; }
+// A value on its way into fminf / fmaxf: a signalling NaN is quieted first.  v_min_f32 / v_max_f32 answer NaN for a
+// signalling one, and the next operation of the chain, which ignores that NaN, has then lost what came before it;
+// f32::min / f32::max skip every NaN alike.
+__device__ __forceinline__ float quiet(float x) { return __builtin_canonicalizef(x); }
 __device__ __forceinline__ float ld(const __half *p) { return __half2float(*p); }
 
 // f32 -> f16 as its own instruction: without the barrier the compiler may fold the preceding multiply and add
@@ -121,8 +125,8 @@ __global__ void __launch_bounds__(256) kivi_quant_tokens_kernel(const SrcT *__re
     float lo = INFINITY, hi = -INFINITY;
     for (int c = lane; c < D; c += 64) {
         const float v = ld(row + c);
-        lo = fminf(lo, v);
-        hi = fmaxf(hi, v);
+        lo = fminf(lo, quiet(v));
+        hi = fmaxf(hi, quiet(v));
     }
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) {
@@ -174,8 +178,8 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_kernel(const SrcT *_
                 for (int r = 0; r < kKeyBlock; r++) {
                     const int k = j * kKeyBlock + r;
                     const float x = k < n_res_old ? res[(int64_t)k * D + c] : ld(fresh + (int64_t)k * D + c);
-                    l = fminf(l, x);
-                    hi = fmaxf(hi, x);
+                    l = fminf(l, quiet(x));
+                    hi = fmaxf(hi, quiet(x));
                 }
                 const int64_t at = ((int64_t)bh * (cap_rows / kKeyBlock) + blk) * D + c;
                 lo_out[at] = l;
@@ -393,8 +397,8 @@ __global__ void __launch_bounds__(256) kivi_quant_tokens_vec_kernel(const SrcT *
     float lo = INFINITY, hi = -INFINITY;
 #pragma unroll
     for (int e = 0; e < 8; e++) {
-        lo = fminf(lo, x.v[e]);
-        hi = fmaxf(hi, x.v[e]);
+        lo = fminf(lo, quiet(x.v[e]));
+        hi = fmaxf(hi, quiet(x.v[e]));
     }
 #pragma unroll
     for (int m = LPR / 2; m >= 1; m >>= 1) {
@@ -442,8 +446,8 @@ __global__ void __launch_bounds__(128) kivi_step_push_kernel(const SrcT *__restr
         float lo = INFINITY, hi = -INFINITY;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            lo = fminf(lo, x.v[e]);
-            hi = fmaxf(hi, x.v[e]);
+            lo = fminf(lo, quiet(x.v[e]));
+            hi = fmaxf(hi, quiet(x.v[e]));
         }
 #pragma unroll
         for (int m = 8; m >= 1; m >>= 1) {
@@ -488,8 +492,8 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_vec_kernel(const Src
         const F8 x = r < n_old ? ld8(res + (int64_t)r * D) : ld8(rows + (int64_t)r * D);
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            lo[e] = fminf(lo[e], x.v[e]);
-            hi[e] = fmaxf(hi[e], x.v[e]);
+            lo[e] = fminf(lo[e], quiet(x.v[e]));
+            hi[e] = fmaxf(hi[e], quiet(x.v[e]));
         }
     }
 #pragma unroll

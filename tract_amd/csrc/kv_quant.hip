@@ -24,7 +24,10 @@
 namespace trocm {
 namespace {
 
-__device__ __forceinline__ float load_elem(const float *p) { return *p; }
+// (A signalling NaN is quieted on the way in: v_max3_f32 / v_min3_f32 answer NaN for one, and the next instruction of
+// the chain, ignoring that NaN, would have lost the two values that shared an instruction with it.  Quiet or
+// signalling, a NaN is skipped by the scan and codes as 0, so nothing else changes.)
+__device__ __forceinline__ float load_elem(const float *p) { return __builtin_canonicalizef(*p); }
 __device__ __forceinline__ float load_elem(const __half *p) { return __half2float(*p); }
 
 __device__ __forceinline__ void store_out(float *p, float x) { *p = x; }
