@@ -1,7 +1,7 @@
 """Prints the Rust `extern "C"` block for every entry point that tract_rocm.h declares.
 
-Usage: ``python include/gen_rust_ffi.py`` (the block goes to stdout; INTEGRATION.md holds a copy, and
-tests/test_abi_cpu.py checks that copy against the header, name by name and argument by argument).
+Usage: ``python include/gen_rust_ffi.py`` (the block goes to stdout; the integration notes at the repository
+root hold a copy, and tests/test_abi_cpu.py checks that copy against the header, name by name and argument by argument).
 """
 from __future__ import annotations
 

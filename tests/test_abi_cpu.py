@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_rust_binding_matches_header():
     """The Rust `extern "C"` block a maintainer pastes into rocm/src/ffi.rs declares every entry point of the
-    header with the same arguments: the copy in INTEGRATION.md is the generator's output for today's header."""
+    header with the same arguments: the copy in the integration notes is the generator's output for today's header."""
     import importlib.util
     spec = importlib.util.spec_from_file_location("gen_rust_ffi", os.path.join(ROOT, "include", "gen_rust_ffi.py"))
     gen = importlib.util.module_from_spec(spec)
