@@ -459,6 +459,10 @@ int choose_decode_splits(int64_t BH, int64_t G, int n_tiles, int wg_per_cu) {
     int64_t max_by_ws = kMaxSplitRows / (BH * G);
     if (ns > max_by_ws) ns = max_by_ws;
     if (ns < 1) ns = 1;
+    if (forced <= 0) {   // no more splits than shorten the longest wave's run: the same critical path with fewer partial records
+        const int64_t groups = max_by_tiles, longest = (groups + ns - 1) / ns;   // groups of kWaves tiles; groups per split
+        ns = (groups + longest - 1) / longest;
+    }
     return (int)ns;
 }
 
