@@ -33,6 +33,7 @@ def f64_product(blocks, act, dt):
     (1, 1, 7, 33, 992), (1, 1, 8, 200, 8192), (1, 1, 1, 64, 20480), (2, 4, 2, 50, 14336),
     (1, 1, 9, 40, 128), (1, 2, 21, 70, 256), (2, 2, 64, 33, 512),   # more than 8 rows: the matrix-matrix arm (f16) / groups of 8
     (1, 1, 9, 40, 96), (2, 4, 9, 129, 128), (1, 2, 130, 300, 1024), (1, 1, 257, 131, 2048), (1, 1, 512, 1024, 4096),
+    (1, 1, 300, 14336, 256), (2, 2, 129, 8250, 128),   # enough 128 x 128 tiles for every compute unit (the shapes above run 128 x 64 tiles)
 ])
 def test_matvec_matches_the_oracle(rt, dt, wb, ab, m, n, k):
     rng = np.random.default_rng(n + k + m)
