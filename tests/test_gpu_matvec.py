@@ -34,6 +34,10 @@ def f64_product(blocks, act, dt):
     (1, 1, 9, 40, 128), (1, 2, 21, 70, 256), (2, 2, 64, 33, 512),   # more than 8 rows: the matrix-matrix arm (f16) / groups of 8
     (1, 1, 9, 40, 96), (2, 4, 9, 129, 128), (1, 2, 130, 300, 1024), (1, 1, 257, 131, 2048), (1, 1, 512, 1024, 4096),
     (1, 1, 300, 14336, 256), (2, 2, 129, 8250, 128),   # enough 128 x 128 tiles for every compute unit (the shapes above run 128 x 64 tiles)
+    # 4..16 f16 rows against 16 weight rows per matrix instruction: one staged chunk (2 and 4 sets of waves per
+    # workgroup, more than 64 KB of LDS), k beyond one chunk, ragged n, batches that share weights
+    (1, 1, 5, 2050, 256), (1, 1, 8, 2048, 4096), (1, 1, 6, 2100, 8320), (1, 1, 4, 12300, 128), (1, 1, 7, 12290, 384),
+    (1, 1, 16, 40, 384), (2, 4, 12, 70, 256), (1, 2, 9, 129, 1024), (1, 1, 13, 3000, 2176), (1, 1, 16, 2049, 4096),
 ])
 def test_matvec_matches_the_oracle(rt, dt, wb, ab, m, n, k):
     rng = np.random.default_rng(n + k + m)

@@ -122,6 +122,9 @@ int launch_apply_rope(const void *x, const void *cos, const void *sin, void *y, 
 // rows: out[b, i, j] = sum_k act[b, i, k] * w[b * w_batch / act_batch, j, k]; act and out of act_dtype.
 int launch_q4_0_matvec(const void *codes, const void *scales, int64_t w_batch, int64_t n, int64_t k, const void *act,
                        int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s);
+// Q4_0 weights x 2..16 f16 activation rows on the matrix cores (q4_matvec_mfma.hip); 2 = not taken.
+int launch_q4_0_matvec_mfma(const void *codes, const void *scales, int64_t w_batch, int64_t n, int64_t k, const void *act,
+                            int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s);
 // The same product for m > 8 rows of f16 activations on the matrix cores.  Returns 2 when not covered.
 int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, int64_t n, int64_t k, const void *act,
                        int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s);

@@ -269,6 +269,10 @@ int launch_m(const MatVecDev &p, int m, int64_t act_batch, hipStream_t s) {
 int launch_q4_0_matvec(const void *codes, const void *scales, int64_t w_batch, int64_t n, int64_t k, const void *act,
                        int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s) {
     const int64_t es = (int64_t)elem_bytes(act_dtype);
+    if (m >= 2 && m <= 16) {   // a few f16 rows: 16 weight rows x 16 activation rows per matrix instruction (q4_matvec_mfma.hip)
+        const int rc = launch_q4_0_matvec_mfma(codes, scales, w_batch, n, k, act, act_dtype, act_batch, m, out, s);
+        if (rc != 2) return rc;
+    }
     if (m > 8) {   // the matrix-matrix arm (q4_matmul.hip) for f16 activations
         const int rc = launch_q4_0_matmul(codes, scales, w_batch, n, k, act, act_dtype, act_batch, m, out, s);
         if (rc != 2) return rc;

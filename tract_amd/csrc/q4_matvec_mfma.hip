@@ -1,0 +1,258 @@
+// Q4_0 weights x 2..16 f16 activation rows on the matrix cores: gfx950.
+//
+//   out[b, i, j] = sum_k act[b, i, k] * dequant(W[b / ratio, j, k]),   2 <= i-count m <= 16
+//
+// the rows of a batched decode step or of a short speculative run through GgmlGemm
+// (cuda/src/kernels/matmul/mod.rs:575-627).  The vector-ALU kernel of q4_matvec.hip multiplies every
+// weight by each of the m rows in turn (its time grows with m: 9.5 us for one row of a 14336 x 4096
+// matrix, 39.5 us for eight); here one v_mfma_f32_16x16x32_f16 multiplies a block of 16 weight rows by up
+// to 16 activation rows, so the launch stays bound by the weights' bytes.
+//
+// Arithmetic: the contraction of the instruction is 32 deep, exactly one quantisation block.  The codes enter
+// as the exact f16 integers -8..7, the products accumulate in f32 inside the instruction from zero, and the
+// block's sum is scaled by its f16 scale with one fma per output: the definition the vector-ALU kernel
+// computes, in another order of additions.
+//
+// Work: four waves own 16 R weight rows (a workgroup holds S such sets of four behind one staged chunk of the
+// activations); the four split the features of a chunk between them and add their partial sums through LDS
+// at the end.  Lane l = (r, g) (r = l % 16, g = l / 16) loads the 16
+// bytes of block 4 i + g of row r, a 4 x 4 transpose over the lane groups (v_permlane32_swap,
+// v_permlane16_swap) hands it byte group g of blocks 4 i .. 4 i + 3, i.e. codes 4g..4g+3 and 16+4g..16+4g+3
+// of each block: the B operand of one instruction per block.  The activations are staged in LDS in that
+// feature order (16-byte vectors XOR-swizzled by row, so that the 16 rows of one read fall into different
+// banks) and read as the A operand.
+//
+// Roofline: HBM-bound on the weights: 18 bytes per 32 weights, read once.
+#include <hip/hip_fp16.h>
+#include <string.h>
+#include <stdlib.h>
+#include "common.h"
+
+namespace trocm {
+namespace {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kQuarters = 4;   // waves that split the features of one set of 16 R rows
+#ifndef MVM_PD
+#define MVM_PD 4
+#endif
+constexpr int PD = MVM_PD;   // groups of four blocks per row in flight ahead of the arithmetic
+
+struct MvMfmaDev {
+    const uint8_t *codes;     // [w_batch, n, k/2]
+    const uint16_t *scales;   // [w_batch, n, k/32]
+    const _Float16 *act;      // [act_batch, m, k]
+    _Float16 *out;            // [act_batch, m, n]
+    int64_t act_stride_b, out_stride_b;   // elements between consecutive batches of act and out
+    int n, k, m, ratio;       // ratio = act_batch / w_batch
+    int kc;                   // features staged per chunk, a multiple of 128
+    int groups;               // row groups of 16 R rows
+};
+
+__device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
+
+// The four bytes of `c` hold codes (low nibbles) e..e+3 and (high nibbles) 16+e..16+e+3 of a block: the eight
+// values code - 8 as f16, in that order.  0x6400 | v is the half 1024 + v; 1032 comes off exactly.
+__device__ __forceinline__ half8_t codes_as_halves(uint32_t c) {
+    const uint32_t lo = c & 0x0F0F0F0Fu, hi = (c >> 4) & 0x0F0F0F0Fu;
+    const half2_t off = {(_Float16)1032.0f, (_Float16)1032.0f};
+    const half2_t a = __builtin_bit_cast(half2_t, perm(0x64646464u, lo, 0x04010400u)) - off;
+    const half2_t b = __builtin_bit_cast(half2_t, perm(0x64646464u, lo, 0x04030402u)) - off;
+    const half2_t c2 = __builtin_bit_cast(half2_t, perm(0x64646464u, hi, 0x04010400u)) - off;
+    const half2_t d = __builtin_bit_cast(half2_t, perm(0x64646464u, hi, 0x04030402u)) - off;
+    return half8_t{a[0], a[1], b[0], b[1], c2[0], c2[1], d[0], d[1]};
+}
+
+// Register j of lane group g <-> register g of lane group j (lane groups of 16 lanes).
+__device__ __forceinline__ void transpose_lane_groups(u32x4 &w) {
+    auto s02 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);   // upper half of [0] <-> lower half of [2]
+    auto s13 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
+    auto t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);   // odd groups of [0] <-> even groups of [1]
+    auto t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+    w[0] = t01[0], w[1] = t01[1], w[2] = t23[0], w[3] = t23[1];
+}
+
+template <int R, int S>
+__global__ __launch_bounds__(256 * S) void q4_0_matvec_mfma_kernel(MvMfmaDev p) {
+    constexpr int kThreads = 256 * S;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    _Float16 *lds_x = reinterpret_cast<_Float16 *>(lds_raw);                                   // [m][kc], swizzled
+    float *red = reinterpret_cast<float *>(lds_raw + (size_t)p.m * p.kc * sizeof(_Float16));    // [4 S waves][R][4][64]
+    const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int q = w & 3, st = w >> 2;        // this wave's quarter of the features, its set of rows
+    const int b = blockIdx.y, wb = b / p.ratio;
+    const int nb = p.k / 32;
+    const _Float16 *act = p.act + (int64_t)b * p.act_stride_b;
+    _Float16 *out = p.out + (int64_t)b * p.out_stride_b;
+    const int arow = min(r16, p.m - 1);      // output rows m..15 of the instruction are never stored: any row serves
+    const bool one_chunk = p.kc >= p.k;      // the activations fit in LDS: staged once per workgroup
+
+    for (int grp = blockIdx.x; grp < p.groups; grp += gridDim.x) {
+        int64_t rows[R];
+#pragma unroll
+        for (int rr = 0; rr < R; rr++) rows[rr] = (int64_t)wb * p.n + min(((grp * S + st) * R + rr) * 16 + r16, p.n - 1);
+        float4_t acc[R];
+#pragma unroll
+        for (int rr = 0; rr < R; rr++) acc[rr] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+        for (int k0 = 0; k0 < p.k; k0 += p.kc) {
+            const int kn = min(p.kc, p.k - k0);                 // a multiple of 128
+            const int nit = kn / 128;                           // groups of four blocks in this chunk
+            const int it_lo = q * nit / kQuarters, ni = (q + 1) * nit / kQuarters - it_lo;   // this wave's share
+            const int blk_lo = k0 / 32 + 4 * it_lo;             // its first block in the row
+            u32x4 cn[PD][R];
+            uint64_t sn[PD][R];                                 // four f16 scales
+            auto fetch = [&](int slot, int it) {
+#pragma unroll
+                for (int rr = 0; rr < R; rr++) {
+                    cn[slot][rr] = *reinterpret_cast<const u32x4 *>(p.codes + rows[rr] * (p.k / 2) + (int64_t)(blk_lo + 4 * it + g) * 16);
+                    sn[slot][rr] = *reinterpret_cast<const uint64_t *>(p.scales + rows[rr] * nb + blk_lo + 4 * it);
+                }
+            };
+#pragma unroll
+            for (int d = 0; d < PD; d++)                        // in flight while the activations are staged
+                if (d < ni) fetch(d, d);
+            if (!one_chunk || grp == (int)blockIdx.x) {
+                if (k0 || grp != (int)blockIdx.x) __syncthreads();
+                // act[:, k0 .. k0+kn) in pieces of 4 halves; piece pos of a block goes to 16-byte vector pos % 4,
+                // half pos / 4 of it, so that vector e holds features 4e..4e+3 and 16+4e..16+4e+3.
+                const int pieces = kn / 4;
+                for (int v = tid; v < p.m * pieces; v += kThreads) {
+                    const int i = v / pieces, c = v % pieces;
+                    const int vec = (c >> 3) * 4 + (c & 3), half = (c >> 2) & 1;
+                    *reinterpret_cast<u32x2 *>(lds_x + (int64_t)i * p.kc + ((vec ^ (i & 15)) * 8) + half * 4) =
+                        *reinterpret_cast<const u32x2 *>(act + (int64_t)i * p.k + k0 + 4 * c);
+                }
+                __syncthreads();
+            }
+            for (int it0 = 0; it0 < ni; it0 += PD)
+#pragma unroll
+                for (int d = 0; d < PD; d++) {
+                    const int it = it0 + d;
+                    if (it >= ni) break;
+                    u32x4 c[R];
+                    uint64_t sc[R];
+#pragma unroll
+                    for (int rr = 0; rr < R; rr++) c[rr] = cn[d][rr], sc[rr] = sn[d][rr];
+                    if (it + PD < ni) fetch(d, it + PD);
+#pragma unroll
+                    for (int rr = 0; rr < R; rr++) transpose_lane_groups(c[rr]);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const int vec = ((it_lo + it) * 4 + j) * 4 + g;
+                        const half8_t a = *reinterpret_cast<const half8_t *>(lds_x + (int64_t)arow * p.kc + ((vec ^ arow) * 8));
+#pragma unroll
+                        for (int rr = 0; rr < R; rr++) {
+                            const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, codes_as_halves(c[rr][j]),
+                                                                                         float4_t{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+                            const float dsc = (float)__builtin_bit_cast(_Float16, (uint16_t)(sc[rr] >> (16 * j)));
+#pragma unroll
+                            for (int e = 0; e < 4; e++) acc[rr][e] = __builtin_fmaf(dsc, part[e], acc[rr][e]);
+                        }
+                    }
+                }
+        }
+        // acc[rr][e] = partial out[4 g + e][row rr * 16 + r16] of this wave's set: the wave of quarter q adds the
+        // set's four values of e = q.
+        __syncthreads();
+#pragma unroll
+        for (int rr = 0; rr < R; rr++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) red[((w * R + rr) * 4 + e) * 64 + lane] = acc[rr][e];
+        __syncthreads();
+#pragma unroll
+        for (int rr = 0; rr < R; rr++) {
+            float sum = 0.0f;
+#pragma unroll
+            for (int ww = 0; ww < kQuarters; ww++) sum += red[(((st * 4 + ww) * R + rr) * 4 + q) * 64 + lane];
+            const int i = 4 * g + q, row = ((grp * S + st) * R + rr) * 16 + r16;
+            if (i < p.m && row < p.n) out[(int64_t)i * p.n + row] = (_Float16)sum;
+        }
+    }
+}
+
+template <int R, int S>
+int launch_rs(MvMfmaDev p, int64_t act_batch, size_t x_bytes, hipStream_t s) {
+    p.groups = (p.n + 16 * R * S - 1) / (16 * R * S);
+    const size_t lds = x_bytes + (size_t)kQuarters * S * R * 4 * 64 * sizeof(float);
+    if (lds > 64 * 1024 &&      // beyond the default limit of dynamic LDS: allowed per kernel (and device) on request
+        hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_0_matvec_mfma_kernel<R, S>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess) {
+        (void)hipGetLastError();
+        return 2;
+    }
+    // When the activations fit in LDS a workgroup stages them once and walks several row groups: as many
+    // workgroups as are resident at once (by LDS, at most 32 waves per compute unit), each with the same number of groups.
+    static const int wg_per_cu = getenv("TROCM_MVM_WG_PER_CU") ? atoi(getenv("TROCM_MVM_WG_PER_CU")) : 0;
+    int64_t wgs = p.groups;
+    int64_t per_cu = (160 * 1024) / (int64_t)lds;
+    if (per_cu > 8 / S) per_cu = 8 / S;
+    if (per_cu < 1) per_cu = 1;
+    if (wg_per_cu > 0) per_cu = wg_per_cu;
+    const int64_t resident = (int64_t)num_compute_units() * per_cu / act_batch;
+    if (p.kc >= p.k && wgs > resident && resident >= 1) {
+        const int64_t turns = (wgs + resident - 1) / resident;
+        wgs = (wgs + turns - 1) / turns;
+    }
+    hipLaunchKernelGGL((q4_0_matvec_mfma_kernel<R, S>), dim3((unsigned)wgs, (unsigned)act_batch), dim3(256 * S), lds, s, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("q4_0_matvec (matrix cores) launch failed: %s", hipGetErrorString(e));
+    return 0;
+}
+
+template <int R>
+int launch_r(const MvMfmaDev &p, int sets, int64_t act_batch, size_t x_bytes, hipStream_t s) {
+    if constexpr (R == 1)     // (16 waves of two row blocks each would not fit the register file)
+        if (sets == 4) return launch_rs<R, 4>(p, act_batch, x_bytes, s);
+    return sets >= 2 ? launch_rs<R, 2>(p, act_batch, x_bytes, s) : launch_rs<R, 1>(p, act_batch, x_bytes, s);
+}
+
+}  // namespace
+
+// 2 = not taken (the caller runs the vector-ALU kernel): f32 activations (their products stay in f32 there), k that
+// is not a whole number of 128-feature groups, misaligned operands, and the row counts and matrix sizes at which the
+// vector-ALU kernel measured faster (up to 4 rows; up to 8 rows against fewer than 2048 weight rows).
+int launch_q4_0_matvec_mfma(const void *codes, const void *scales, int64_t w_batch, int64_t n, int64_t k, const void *act,
+                            int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s) {
+    static const int enabled = getenv("TROCM_MV_MFMA") ? atoi(getenv("TROCM_MV_MFMA")) : 1;
+    static const int forced_min_m = getenv("TROCM_MV_MFMA_MIN_M") ? atoi(getenv("TROCM_MV_MFMA_MIN_M")) : 0;
+    static const int lds_kb = getenv("TROCM_MV_MFMA_LDS_KB") ? atoi(getenv("TROCM_MV_MFMA_LDS_KB")) : 64;
+    static const int forced_r = getenv("TROCM_MV_MFMA_ROWS") ? atoi(getenv("TROCM_MV_MFMA_ROWS")) : 0;
+    static const int forced_sets = getenv("TROCM_MV_MFMA_SETS") ? atoi(getenv("TROCM_MV_MFMA_SETS")) : 0;
+    if (!enabled || act_dtype != TROCM_F16 || m < 2 || m > 16 || k % 128 != 0 || k < 128) return 2;
+    if ((uintptr_t)codes % 16 || (uintptr_t)scales % 8 || (uintptr_t)act % 8 || (uintptr_t)out % 2) return 2;
+    if (n < 1 || n >= (1ll << 30) || k >= (1ll << 30) || act_batch < 1 || act_batch > 65535) return 2;
+    const int64_t cus = num_compute_units();
+    const int64_t blocks16 = (n + 15) / 16 * act_batch;          // blocks of 16 weight rows in the launch
+    // Measured against the vector-ALU kernel (14336 x 4096: 4 rows 13.9 vs 16.7 us, 8 rows 15.2 vs 38.8 us;
+    // 4096 x 4096: 4 rows 9.2 vs 6.9 us, 8 rows 10.7 vs 14.2 us; 1024 x 4096, 8 rows: 10.1 vs 7.4 us).
+    const int64_t min_m = forced_min_m > 0 ? forced_min_m : blocks16 >= 3 * cus ? 4 : 5;
+    if (m < min_m || (m <= 8 && forced_min_m == 0 && blocks16 * 2 < cus)) return 2;
+    MvMfmaDev p;
+    memset(&p, 0, sizeof(p));
+    p.codes = (const uint8_t *)codes, p.scales = (const uint16_t *)scales;
+    p.act = (const _Float16 *)act, p.out = (_Float16 *)out;
+    p.act_stride_b = m * k, p.out_stride_b = m * n;
+    p.n = (int)n, p.k = (int)k, p.m = (int)m, p.ratio = (int)(act_batch / w_batch);
+    int64_t kc = (int64_t)lds_kb * 1024 / (m * 2) / 128 * 128;   // what the budget holds, in whole groups of four blocks
+    if (kc < 128) kc = 128;
+    if (kc > k) kc = k;
+    p.kc = (int)kc;
+    const size_t x_bytes = (size_t)m * kc * 2;
+    // One block of 16 rows per wave (two, sharing each read of the activations, measured slower: 105 vs 91 us for
+    // 128256 x 4096 and 8 rows).  Sets of 4 waves behind one staged chunk: four when that still leaves about a
+    // workgroup per compute unit (14336 rows, 8 activation rows: 15.2 us; two sets 16.6 us; one 21.8 us), else two
+    // (4096 rows: 10.7 us; four sets 14.0 us; one 11.5 us).
+    const int r = forced_r == 2 ? 2 : 1;
+    int sets = blocks16 >= 3 * cus ? 4 : 2;
+    if (forced_sets == 1 || forced_sets == 2 || forced_sets == 4) sets = forced_sets;
+    return r == 2 ? launch_r<2>(p, sets, act_batch, x_bytes, s) : launch_r<1>(p, sets, act_batch, x_bytes, s);
+}
+
+}  // namespace trocm
