@@ -20,7 +20,9 @@
 // v_permlane16_swap) hands it byte group g of blocks 4 i .. 4 i + 3, i.e. codes 4g..4g+3 and 16+4g..16+4g+3
 // of each block: the B operand of one instruction per block.  The activations are staged in LDS in that
 // feature order (16-byte vectors XOR-swizzled by row, so that the 16 rows of one read fall into different
-// banks) and read as the A operand.
+// banks) and read as the A operand.  When they do not fit, they are staged in chunks that hold a piece of
+// every wave's quarter of k, so that a wave's weights stay one contiguous stream that is prefetched across the
+// chunks, and the next chunk's activations wait in registers while this chunk is multiplied.
 //
 // Roofline: HBM-bound on the weights: 18 bytes per 32 weights, read once.
 #include <hip/hip_fp16.h>
@@ -37,11 +39,8 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kQuarters = 4;   // waves that split the features of one set of 16 R rows
-#ifndef MVM_PD
-#define MVM_PD 4
-#endif
-constexpr int PD = MVM_PD;   // groups of four blocks per row in flight ahead of the arithmetic
+// KS waves split the features of one set of 16 R rows (4, or 8 when the matrix has few rows); each keeps PD = 16 / KS
+// groups of four blocks per row in flight ahead of the arithmetic.
 
 struct MvMfmaDev {
     const uint8_t *codes;     // [w_batch, n, k/2]
@@ -50,9 +49,13 @@ struct MvMfmaDev {
     _Float16 *out;            // [act_batch, m, n]
     int64_t act_stride_b, out_stride_b;   // elements between consecutive batches of act and out
     int n, k, m, ratio;       // ratio = act_batch / w_batch
-    int kc;                   // features staged per chunk, a multiple of 128
-    int groups;               // row groups of 16 R rows
+    int cq;                   // groups of four blocks (128 features) per quarter of k in one staged chunk
+    int nch;                  // chunks; 1 = the activations fit in LDS and are staged once per workgroup
+    int prefetch;             // the next chunk's activations wait in registers during this chunk's arithmetic
+    int groups;               // row groups of 16 R S rows
 };
+constexpr int kStageRegs = 8;   // 8-byte pieces of the next chunk a thread holds (prefetch mode)
+// cq in prefetch mode is PD: a chunk is 2048 features, 512 pieces per row, and piece indices split by shifts
 
 __device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
 
@@ -77,21 +80,43 @@ __device__ __forceinline__ void transpose_lane_groups(u32x4 &w) {
     w[0] = t01[0], w[1] = t01[1], w[2] = t23[0], w[3] = t23[1];
 }
 
-template <int R, int S>
-__global__ __launch_bounds__(256 * S) void q4_0_matvec_mfma_kernel(MvMfmaDev p) {
-    constexpr int kThreads = 256 * S;
+template <int R, int S, bool PF, int KS>
+__global__ __launch_bounds__(64 * KS * S) void q4_0_matvec_mfma_kernel(MvMfmaDev p) {
+    constexpr int kThreads = 64 * KS * S, PD = 16 / KS, kPrefetchCq = PD;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    _Float16 *lds_x = reinterpret_cast<_Float16 *>(lds_raw);                                   // [m][kc], swizzled
-    float *red = reinterpret_cast<float *>(lds_raw + (size_t)p.m * p.kc * sizeof(_Float16));    // [4 S waves][R][4][64]
+    const int kc = KS * p.cq * 128;          // features per staged row: cq groups of each wave's share of k
+    _Float16 *lds_x = reinterpret_cast<_Float16 *>(lds_raw);                                 // [m][kc], swizzled
+    float *red = reinterpret_cast<float *>(lds_raw + (size_t)p.m * kc * sizeof(_Float16));    // [KS S waves][R][4][64]
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int q = w & 3, st = w >> 2;        // this wave's quarter of the features, its set of rows
+    const int q = w % KS, st = w / KS;       // this wave's share of the features, its set of rows
     const int b = blockIdx.y, wb = b / p.ratio;
-    const int nb = p.k / 32;
+    const int nb = p.k / 32, nit = p.k / 128;
+    const int it_lo = q * nit / KS, ni = (q + 1) * nit / KS - it_lo;   // this wave's groups of four blocks
     const _Float16 *act = p.act + (int64_t)b * p.act_stride_b;
     _Float16 *out = p.out + (int64_t)b * p.out_stride_b;
     const int arow = min(r16, p.m - 1);      // output rows m..15 of the instruction are never stored: any row serves
-    const bool one_chunk = p.kc >= p.k;      // the activations fit in LDS: staged once per workgroup
+    const bool one_chunk = p.nch == 1;
+
+    // Piece v of chunk c: 4 halves of activation row i, quarter qq, group li of the chunk.  A group's 16 vectors of
+    // 16 bytes are XOR-swizzled by the row; piece pos of a block goes to vector pos % 4, half pos / 4 of it, so that
+    // vector e of a block holds features 4e..4e+3 and 16+4e..16+4e+3.
+    auto piece_at = [&](int pc, int li, int qq, int i, int c, const _Float16 *&src, int &dst) -> bool {
+        const int lo = qq * nit / KS, have = (qq + 1) * nit / KS - lo, t = c * p.cq + li;
+        if (i >= p.m || t >= have) return false;
+        src = act + (int64_t)i * p.k + (int64_t)(lo + t) * 128 + pc * 4;
+        const int vecg = (pc >> 3) * 4 + (pc & 3), hi = (pc >> 2) & 1;
+        dst = i * kc + ((qq * p.cq + li) * 16 + (vecg ^ (i & 15))) * 8 + hi * 4;
+        return true;
+    };
+    // Prefetch mode (PF; cq = kPrefetchCq, at least 512 threads): piece u of a thread is the same 4 halves of row
+    // i0 + u * kThreads / 512, so one source pointer and one LDS offset serve all of them.
+    const int pf_pc = tid & 31, pf_li = (tid >> 5) & (PD - 1), pf_qq = ((tid >> 5) / PD) & (KS - 1), pf_i0 = tid >> 9;
+    const int pf_lo = pf_qq * nit / KS, pf_have = (pf_qq + 1) * nit / KS - pf_lo;
+    const _Float16 *pf_src = act + (int64_t)pf_i0 * p.k + (int64_t)(pf_lo + pf_li) * 128 + pf_pc * 4;
+    const int pf_vecg = (pf_pc >> 3) * 4 + (pf_pc & 3);
+    const int pf_dst = (pf_qq * kPrefetchCq + pf_li) * 128 + ((pf_pc >> 2) & 1) * 4;
+    constexpr int kRowStep = kThreads >> 9;
 
     for (int grp = blockIdx.x; grp < p.groups; grp += gridDim.x) {
         int64_t rows[R];
@@ -101,55 +126,90 @@ __global__ __launch_bounds__(256 * S) void q4_0_matvec_mfma_kernel(MvMfmaDev p) 
 #pragma unroll
         for (int rr = 0; rr < R; rr++) acc[rr] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-        for (int k0 = 0; k0 < p.k; k0 += p.kc) {
-            const int kn = min(p.kc, p.k - k0);                 // a multiple of 128
-            const int nit = kn / 128;                           // groups of four blocks in this chunk
-            const int it_lo = q * nit / kQuarters, ni = (q + 1) * nit / kQuarters - it_lo;   // this wave's share
-            const int blk_lo = k0 / 32 + 4 * it_lo;             // its first block in the row
-            u32x4 cn[PD][R];
-            uint64_t sn[PD][R];                                 // four f16 scales
-            auto fetch = [&](int slot, int it) {
+        // PD groups of four blocks per row ahead, across the chunks: the weights do not wait for a chunk's staging.
+        u32x4 cn[PD][R];
+        uint64_t sn[PD][R];                                     // four f16 scales
+        auto fetch = [&](int slot, int t) {
 #pragma unroll
-                for (int rr = 0; rr < R; rr++) {
-                    cn[slot][rr] = *reinterpret_cast<const u32x4 *>(p.codes + rows[rr] * (p.k / 2) + (int64_t)(blk_lo + 4 * it + g) * 16);
-                    sn[slot][rr] = *reinterpret_cast<const uint64_t *>(p.scales + rows[rr] * nb + blk_lo + 4 * it);
-                }
-            };
+            for (int rr = 0; rr < R; rr++) {
+                cn[slot][rr] = *reinterpret_cast<const u32x4 *>(p.codes + rows[rr] * (p.k / 2) + (int64_t)((it_lo + t) * 4 + g) * 16);
+                sn[slot][rr] = *reinterpret_cast<const uint64_t *>(p.scales + rows[rr] * nb + (it_lo + t) * 4);
+            }
+        };
 #pragma unroll
-            for (int d = 0; d < PD; d++)                        // in flight while the activations are staged
-                if (d < ni) fetch(d, d);
-            if (!one_chunk || grp == (int)blockIdx.x) {
-                if (k0 || grp != (int)blockIdx.x) __syncthreads();
-                // act[:, k0 .. k0+kn) in pieces of 4 halves; piece pos of a block goes to 16-byte vector pos % 4,
-                // half pos / 4 of it, so that vector e holds features 4e..4e+3 and 16+4e..16+4e+3.
-                const int pieces = kn / 4;
-                for (int v = tid; v < p.m * pieces; v += kThreads) {
-                    const int i = v / pieces, c = v % pieces;
-                    const int vec = (c >> 3) * 4 + (c & 3), half = (c >> 2) & 1;
-                    *reinterpret_cast<u32x2 *>(lds_x + (int64_t)i * p.kc + ((vec ^ (i & 15)) * 8) + half * 4) =
-                        *reinterpret_cast<const u32x2 *>(act + (int64_t)i * p.k + k0 + 4 * c);
+        for (int d = 0; d < PD; d++)
+            if (d < ni) fetch(d, d);
+
+        const bool stage_here = !one_chunk || grp == (int)blockIdx.x;
+        u32x2 held[kStageRegs];
+        auto hold = [&](int c) {                                // chunk c's pieces of this thread into registers
+            if (c * kPrefetchCq + pf_li < pf_have) {
+#pragma unroll
+                for (int u = 0; u < kStageRegs; u++)
+                    if (pf_i0 + u * kRowStep < p.m)
+                        held[u] = *reinterpret_cast<const u32x2 *>(pf_src + (int64_t)u * kRowStep * p.k + c * (kPrefetchCq * 128));
+            }
+        };
+        if constexpr (PF) hold(0);
+
+        for (int c = 0; c < p.nch; c++) {
+            if (stage_here) {
+                if (c || grp != (int)blockIdx.x) __syncthreads();           // the previous chunk has been read
+                if constexpr (PF) {
+                    if (c * kPrefetchCq + pf_li < pf_have) {
+#pragma unroll
+                        for (int u = 0; u < kStageRegs; u++) {
+                            const int i = pf_i0 + u * kRowStep;
+                            if (i < p.m) *reinterpret_cast<u32x2 *>(lds_x + i * kc + pf_dst + ((pf_vecg ^ (i & 15)) * 8)) = held[u];
+                        }
+                    }
+                } else if (kc == p.k) {
+                    // every quarter of k is whole: the one chunk is the rows in their natural order of blocks
+                    const int pieces = p.k / 4;
+                    for (int v = tid; v < p.m * pieces; v += kThreads) {
+                        const int i = v / pieces, cc = v % pieces;
+                        const int vec = (cc >> 3) * 4 + (cc & 3), hi = (cc >> 2) & 1;
+                        *reinterpret_cast<u32x2 *>(lds_x + i * kc + ((vec ^ (i & 15)) * 8) + hi * 4) =
+                            *reinterpret_cast<const u32x2 *>(act + (int64_t)i * p.k + 4 * cc);
+                    }
+                } else {
+                    // piece v = ((i * KS + qq) * cq + li) * 32 + pc for v = tid, tid + kThreads, ...: li and i * KS + qq
+                    // are carried along instead of divided out
+                    int li = (tid >> 5) % p.cq, iq = (tid >> 5) / p.cq;
+                    while (iq < p.m * KS) {
+                        const _Float16 *src;
+                        int dst;
+                        if (piece_at(tid & 31, li, iq % KS, iq / KS, c, src, dst))
+                            *reinterpret_cast<u32x2 *>(lds_x + dst) = *reinterpret_cast<const u32x2 *>(src);
+                        li += kThreads / 32;
+                        while (li >= p.cq) li -= p.cq, iq++;
+                    }
                 }
                 __syncthreads();
+                if constexpr (PF)
+                    if (c + 1 < p.nch) hold(c + 1);               // in flight during this chunk's arithmetic
             }
-            for (int it0 = 0; it0 < ni; it0 += PD)
+            const int cnt = min(max(ni - c * p.cq, 0), p.cq);               // this wave's groups in the chunk
+            for (int l0 = 0; l0 < cnt; l0 += PD)
 #pragma unroll
                 for (int d = 0; d < PD; d++) {
-                    const int it = it0 + d;
-                    if (it >= ni) break;
-                    u32x4 c[R];
+                    const int l = l0 + d;
+                    if (l >= cnt) break;
+                    const int t = c * p.cq + l;                             // t % PD == d: cq is a multiple of PD when nch > 1
+                    u32x4 cw[R];
                     uint64_t sc[R];
 #pragma unroll
-                    for (int rr = 0; rr < R; rr++) c[rr] = cn[d][rr], sc[rr] = sn[d][rr];
-                    if (it + PD < ni) fetch(d, it + PD);
+                    for (int rr = 0; rr < R; rr++) cw[rr] = cn[d][rr], sc[rr] = sn[d][rr];
+                    if (t + PD < ni) fetch(d, t + PD);
 #pragma unroll
-                    for (int rr = 0; rr < R; rr++) transpose_lane_groups(c[rr]);
+                    for (int rr = 0; rr < R; rr++) transpose_lane_groups(cw[rr]);
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
-                        const int vec = ((it_lo + it) * 4 + j) * 4 + g;
-                        const half8_t a = *reinterpret_cast<const half8_t *>(lds_x + (int64_t)arow * p.kc + ((vec ^ arow) * 8));
+                        const int vec = (q * p.cq + l) * 16 + ((j * 4 + g) ^ arow);
+                        const half8_t a = *reinterpret_cast<const half8_t *>(lds_x + arow * kc + vec * 8);
 #pragma unroll
                         for (int rr = 0; rr < R; rr++) {
-                            const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, codes_as_halves(c[rr][j]),
+                            const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, codes_as_halves(cw[rr][j]),
                                                                                          float4_t{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
                             const float dsc = (float)__builtin_bit_cast(_Float16, (uint16_t)(sc[rr] >> (16 * j)));
 #pragma unroll
@@ -158,31 +218,32 @@ __global__ __launch_bounds__(256 * S) void q4_0_matvec_mfma_kernel(MvMfmaDev p) 
                     }
                 }
         }
-        // acc[rr][e] = partial out[4 g + e][row rr * 16 + r16] of this wave's set: the wave of quarter q adds the
-        // set's four values of e = q.
+        // acc[rr][e] = partial out[4 g + e][row rr * 16 + r16] of this wave's set: wave q < 4 of the set adds its KS
+        // values of e = q.
         __syncthreads();
 #pragma unroll
         for (int rr = 0; rr < R; rr++)
 #pragma unroll
             for (int e = 0; e < 4; e++) red[((w * R + rr) * 4 + e) * 64 + lane] = acc[rr][e];
         __syncthreads();
+        if (q < 4) {
 #pragma unroll
-        for (int rr = 0; rr < R; rr++) {
-            float sum = 0.0f;
+            for (int rr = 0; rr < R; rr++) {
+                float sum = 0.0f;
 #pragma unroll
-            for (int ww = 0; ww < kQuarters; ww++) sum += red[(((st * 4 + ww) * R + rr) * 4 + q) * 64 + lane];
-            const int i = 4 * g + q, row = ((grp * S + st) * R + rr) * 16 + r16;
-            if (i < p.m && row < p.n) out[(int64_t)i * p.n + row] = (_Float16)sum;
+                for (int ww = 0; ww < KS; ww++) sum += red[(((st * KS + ww) * R + rr) * 4 + q) * 64 + lane];
+                const int i = 4 * g + q, row = ((grp * S + st) * R + rr) * 16 + r16;
+                if (i < p.m && row < p.n) out[(int64_t)i * p.n + row] = (_Float16)sum;
+            }
         }
     }
 }
 
-template <int R, int S>
-int launch_rs(MvMfmaDev p, int64_t act_batch, size_t x_bytes, hipStream_t s) {
-    p.groups = (p.n + 16 * R * S - 1) / (16 * R * S);
-    const size_t lds = x_bytes + (size_t)kQuarters * S * R * 4 * 64 * sizeof(float);
+template <int R, int S, bool PF, int KS>
+int launch_rsp(const MvMfmaDev &p, int64_t act_batch, hipStream_t s) {
+    const size_t lds = (size_t)p.m * KS * p.cq * 128 * 2 + (size_t)KS * S * R * 4 * 64 * sizeof(float);
     if (lds > 64 * 1024 &&      // beyond the default limit of dynamic LDS: allowed per kernel (and device) on request
-        hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_0_matvec_mfma_kernel<R, S>), hipFuncAttributeMaxDynamicSharedMemorySize,
+        hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_0_matvec_mfma_kernel<R, S, PF, KS>), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
         (void)hipGetLastError();
         return 2;
@@ -192,25 +253,39 @@ int launch_rs(MvMfmaDev p, int64_t act_batch, size_t x_bytes, hipStream_t s) {
     static const int wg_per_cu = getenv("TROCM_MVM_WG_PER_CU") ? atoi(getenv("TROCM_MVM_WG_PER_CU")) : 0;
     int64_t wgs = p.groups;
     int64_t per_cu = (160 * 1024) / (int64_t)lds;
-    if (per_cu > 8 / S) per_cu = 8 / S;
+    if (per_cu > 32 / (KS * S)) per_cu = 32 / (KS * S);
     if (per_cu < 1) per_cu = 1;
     if (wg_per_cu > 0) per_cu = wg_per_cu;
     const int64_t resident = (int64_t)num_compute_units() * per_cu / act_batch;
-    if (p.kc >= p.k && wgs > resident && resident >= 1) {
+    if (p.nch == 1 && wgs > resident && resident >= 1) {
         const int64_t turns = (wgs + resident - 1) / resident;
         wgs = (wgs + turns - 1) / turns;
     }
-    hipLaunchKernelGGL((q4_0_matvec_mfma_kernel<R, S>), dim3((unsigned)wgs, (unsigned)act_batch), dim3(256 * S), lds, s, p);
+    hipLaunchKernelGGL((q4_0_matvec_mfma_kernel<R, S, PF, KS>), dim3((unsigned)wgs, (unsigned)act_batch), dim3(64 * KS * S), lds, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("q4_0_matvec (matrix cores) launch failed: %s", hipGetErrorString(e));
     return 0;
 }
 
+template <int R, int S, int KS>
+int launch_rs(MvMfmaDev p, int64_t act_batch, hipStream_t s) {
+    p.groups = (p.n + 16 * R * S - 1) / (16 * R * S);
+    constexpr int kThreads = 64 * KS * S;
+    if constexpr (kThreads >= 512) {
+        static const int allowed = getenv("TROCM_MV_MFMA_PREFETCH") ? atoi(getenv("TROCM_MV_MFMA_PREFETCH")) : 1;
+        p.prefetch = allowed && p.nch > 1 && p.cq == 16 / KS && (p.m + (kThreads >> 9) - 1) / (kThreads >> 9) <= kStageRegs;
+        if (p.prefetch) return launch_rsp<R, S, true, KS>(p, act_batch, s);
+    }
+    p.prefetch = 0;
+    return launch_rsp<R, S, false, KS>(p, act_batch, s);
+}
+
 template <int R>
-int launch_r(const MvMfmaDev &p, int sets, int64_t act_batch, size_t x_bytes, hipStream_t s) {
+int launch_r(const MvMfmaDev &p, int splits, int sets, int64_t act_batch, hipStream_t s) {
+    if (splits == 8) return sets >= 2 ? launch_rs<R, 2, 8>(p, act_batch, s) : launch_rs<R, 1, 8>(p, act_batch, s);
     if constexpr (R == 1)     // (16 waves of two row blocks each would not fit the register file)
-        if (sets == 4) return launch_rs<R, 4>(p, act_batch, x_bytes, s);
-    return sets >= 2 ? launch_rs<R, 2>(p, act_batch, x_bytes, s) : launch_rs<R, 1>(p, act_batch, x_bytes, s);
+        if (sets == 4) return launch_rs<R, 4, 4>(p, act_batch, s);
+    return sets >= 2 ? launch_rs<R, 2, 4>(p, act_batch, s) : launch_rs<R, 1, 4>(p, act_batch, s);
 }
 
 }  // namespace
@@ -222,7 +297,7 @@ int launch_q4_0_matvec_mfma(const void *codes, const void *scales, int64_t w_bat
                             int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s) {
     static const int enabled = getenv("TROCM_MV_MFMA") ? atoi(getenv("TROCM_MV_MFMA")) : 1;
     static const int forced_min_m = getenv("TROCM_MV_MFMA_MIN_M") ? atoi(getenv("TROCM_MV_MFMA_MIN_M")) : 0;
-    static const int lds_kb = getenv("TROCM_MV_MFMA_LDS_KB") ? atoi(getenv("TROCM_MV_MFMA_LDS_KB")) : 64;
+    static const int forced_lds_kb = getenv("TROCM_MV_MFMA_LDS_KB") ? atoi(getenv("TROCM_MV_MFMA_LDS_KB")) : 0;
     static const int forced_r = getenv("TROCM_MV_MFMA_ROWS") ? atoi(getenv("TROCM_MV_MFMA_ROWS")) : 0;
     static const int forced_sets = getenv("TROCM_MV_MFMA_SETS") ? atoi(getenv("TROCM_MV_MFMA_SETS")) : 0;
     if (!enabled || act_dtype != TROCM_F16 || m < 2 || m > 16 || k % 128 != 0 || k < 128) return 2;
@@ -240,19 +315,37 @@ int launch_q4_0_matvec_mfma(const void *codes, const void *scales, int64_t w_bat
     p.act = (const _Float16 *)act, p.out = (_Float16 *)out;
     p.act_stride_b = m * k, p.out_stride_b = m * n;
     p.n = (int)n, p.k = (int)k, p.m = (int)m, p.ratio = (int)(act_batch / w_batch);
-    int64_t kc = (int64_t)lds_kb * 1024 / (m * 2) / 128 * 128;   // what the budget holds, in whole groups of four blocks
-    if (kc < 128) kc = 128;
-    if (kc > k) kc = k;
-    p.kc = (int)kc;
-    const size_t x_bytes = (size_t)m * kc * 2;
+    // Every wave walks one quarter of k.  If the whole of the activations fits the LDS budget they are staged once per
+    // workgroup; else in chunks of 4 groups of 128 features per quarter (2048 features, a multiple of the weights'
+    // prefetch depth), the next chunk waiting in registers.
+    // Every wave walks one share of k: a quarter, or an eighth when the matrix has too few rows to give every SIMD a
+    // wave otherwise.  If the whole of the activations fits the LDS budget they are staged once per workgroup; else in
+    // chunks of 2048 features (512 or 256 of every share, a multiple of the weights' prefetch depth), the next chunk
+    // waiting in registers.
+    static const int forced_cq = getenv("TROCM_MV_MFMA_CQ") ? atoi(getenv("TROCM_MV_MFMA_CQ")) : 0;
+    static const int forced_splits = getenv("TROCM_MV_MFMA_SPLITS") ? atoi(getenv("TROCM_MV_MFMA_SPLITS")) : 0;
+    int splits = blocks16 < 2 * cus && k >= 2048 ? 8 : 4;
+    if (forced_splits == 4 || forced_splits == 8) splits = forced_splits;
+    const int64_t per_split = (k / 128 + splits - 1) / splits;
+    // (budget: 64 KB, two workgroups per compute unit; 136 KB when every workgroup walks many row groups behind
+    // one staging: 128256 x 4096 with 16 rows 95 us, in chunks 125 us; 14336 x 4096 20.0 us, in chunks 16.5 us)
+    const int64_t budget = forced_lds_kb > 0 ? (int64_t)forced_lds_kb * 1024 : blocks16 / 4 >= 4 * cus ? 136 * 1024 : 64 * 1024;
+    if (m * splits * per_split * 128 * 2 <= budget) {
+        p.cq = (int)per_split, p.nch = 1;
+    } else {
+        const int pd = 16 / splits;
+        p.cq = forced_cq > 0 && forced_cq % pd == 0 ? forced_cq : pd;
+        p.nch = (int)((per_split + p.cq - 1) / p.cq);
+    }
     // One block of 16 rows per wave (two, sharing each read of the activations, measured slower: 105 vs 91 us for
     // 128256 x 4096 and 8 rows).  Sets of 4 waves behind one staged chunk: four when that still leaves about a
     // workgroup per compute unit (14336 rows, 8 activation rows: 15.2 us; two sets 16.6 us; one 21.8 us), else two
     // (4096 rows: 10.7 us; four sets 14.0 us; one 11.5 us).
     const int r = forced_r == 2 ? 2 : 1;
-    int sets = blocks16 >= 3 * cus ? 4 : 2;
+    int sets = splits == 8 ? 1 : blocks16 >= 3 * cus ? 4 : 2;
     if (forced_sets == 1 || forced_sets == 2 || forced_sets == 4) sets = forced_sets;
-    return r == 2 ? launch_r<2>(p, sets, act_batch, x_bytes, s) : launch_r<1>(p, sets, act_batch, x_bytes, s);
+    if (p.nch > 1 && m > 8 && forced_sets == 0) sets = splits == 8 ? 2 : 4;    // 1024 threads hold a chunk of 16 rows in their registers
+    return r == 2 ? launch_r<2>(p, splits, sets, act_batch, s) : launch_r<1>(p, splits, sets, act_batch, s);
 }
 
 }  // namespace trocm
