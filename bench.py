@@ -701,6 +701,18 @@ def run_ops(ta, args):
         us = time_calls(ta, one_mv, 200)
         by = n_ * (k_ // 32) * 18 + 2 * k_ + 2 * n_
         res[f"q4_0_matvec_f16_n{n_}_k{k_}"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": by}
+        # the same weights x the 8 rows of a batch-8 decode step: 16 weight rows x 8 activation rows per matrix
+        # instruction, still bound by the weights' bytes
+        x8 = ta.DeviceTensor.from_numpy(rng.standard_normal((1, 8, k_)).astype(np.float16))
+        o8 = ta.DeviceTensor((1, 8, n_), np.float16)
+
+        def one_mv8():
+            gemm.eval(x8, ws[turn[0] % 8], out=o8)
+            turn[0] += 1
+
+        us = time_calls(ta, one_mv8, 200)
+        by8 = n_ * (k_ // 32) * 18 + 8 * 2 * k_ + 8 * 2 * n_
+        res[f"q4_0_matvec_f16_m8_n{n_}_k{k_}"] = {"us": round(us, 2), "gbs": round(by8 / us / 1e3, 1), "bytes": by8}
         if (n_, k_) != (4096, 14336):
             # the same weights x the 512 rows of a prefill chunk: the matrix-matrix arm, on the matrix cores
             m_ = 512

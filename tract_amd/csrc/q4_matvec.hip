@@ -18,7 +18,8 @@
 // of the current k chunk, whose activations sit in LDS (read once per lane and block, used for R
 // rows).  Accumulators are reduced across the wave at the end.
 //
-// Roofline: HBM-bound on the weights: 18 bytes per 32 weights, read once.
+// Roofline: HBM-bound on the weights: 18 bytes per 32 weights, read once.  (From about 4 f16 rows on the arithmetic
+// of this kernel, which repeats per row, takes longer than the weights: those calls go to q4_matvec_mfma.hip.)
 #include <hip/hip_fp16.h>
 #include <string.h>
 #include <stdlib.h>

@@ -13,16 +13,16 @@
 // block's sum is scaled by its f16 scale with one fma per output: the definition the vector-ALU kernel
 // computes, in another order of additions.
 //
-// Work: four waves own 16 R weight rows (a workgroup holds S such sets of four behind one staged chunk of the
-// activations); the four split the features of a chunk between them and add their partial sums through LDS
-// at the end.  Lane l = (r, g) (r = l % 16, g = l / 16) loads the 16
+// Work: KS waves (4, or 8 when the matrix has too few rows to occupy every SIMD otherwise) own 16 R weight rows; each
+// walks one contiguous share of k, and they add their partial sums through LDS at the end.  A workgroup holds S
+// such sets behind one staged chunk of the activations.  Lane l = (r, g) (r = l % 16, g = l / 16) loads the 16
 // bytes of block 4 i + g of row r, a 4 x 4 transpose over the lane groups (v_permlane32_swap,
 // v_permlane16_swap) hands it byte group g of blocks 4 i .. 4 i + 3, i.e. codes 4g..4g+3 and 16+4g..16+4g+3
 // of each block: the B operand of one instruction per block.  The activations are staged in LDS in that
 // feature order (16-byte vectors XOR-swizzled by row, so that the 16 rows of one read fall into different
-// banks) and read as the A operand.  When they do not fit, they are staged in chunks that hold a piece of
-// every wave's quarter of k, so that a wave's weights stay one contiguous stream that is prefetched across the
-// chunks, and the next chunk's activations wait in registers while this chunk is multiplied.
+// banks) and read as the A operand.  When they do not fit, they are staged in chunks of 2048 features that hold a
+// piece of every wave's share of k, so that a wave's weights stay one contiguous stream that is prefetched across
+// the chunks, and the next chunk's activations wait in registers while this chunk is multiplied.
 //
 // Roofline: HBM-bound on the weights: 18 bytes per 32 weights, read once.
 #include <hip/hip_fp16.h>
