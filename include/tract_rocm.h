@@ -225,9 +225,10 @@ int trocm_q4_0_weights_shape(const trocm_q4_weights *weights, int64_t *batch, in
 /* The canonical blocks back (byte-identical to what was loaded). */
 int trocm_q4_0_weights_export(const trocm_q4_weights *weights, void *dst_blocks_device, void *stream);
 /* out[b, i, j] = sum_k act[b, i, k] * w[b / (act_batch / batch), j, k]; act and out dense, F32 or F16,
- * act 16-byte aligned.  Built for the m <= 8 rows of a decode step (one pass over the weights); a
- * larger m runs as groups of 8 rows, one pass each (the reference switches to a matrix-matrix
- * kernel there, mod.rs:607-609, which this library does not have). */
+ * act 16-byte aligned.  One pass over the weights for the m <= 8 rows of a decode step (from about
+ * 4 f16 rows on, and up to 16, on the matrix cores when k is a multiple of 128); a larger m of F16 rows
+ * (k a multiple of 64) runs on a matrix-matrix kernel as the reference does (mod.rs:607-609), anything
+ * else as groups of 8 rows, one pass each. */
 int trocm_q4_0_matvec(const trocm_q4_weights *weights, const void *act, int act_dtype, int64_t act_batch,
                       int64_t m, void *out, void *stream);
 

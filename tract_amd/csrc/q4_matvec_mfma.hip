@@ -283,8 +283,7 @@ int launch_rs(MvMfmaDev p, int64_t act_batch, hipStream_t s) {
 template <int R>
 int launch_r(const MvMfmaDev &p, int splits, int sets, int64_t act_batch, hipStream_t s) {
     if (splits == 8) return sets >= 2 ? launch_rs<R, 2, 8>(p, act_batch, s) : launch_rs<R, 1, 8>(p, act_batch, s);
-    if constexpr (R == 1)     // (16 waves of two row blocks each would not fit the register file)
-        if (sets == 4) return launch_rs<R, 4, 4>(p, act_batch, s);
+    if (sets == 4) return launch_rs<R, 4, 4>(p, act_batch, s);
     return sets >= 2 ? launch_rs<R, 2, 4>(p, act_batch, s) : launch_rs<R, 1, 4>(p, act_batch, s);
 }
 
@@ -298,7 +297,6 @@ int launch_q4_0_matvec_mfma(const void *codes, const void *scales, int64_t w_bat
     static const int enabled = getenv("TROCM_MV_MFMA") ? atoi(getenv("TROCM_MV_MFMA")) : 1;
     static const int forced_min_m = getenv("TROCM_MV_MFMA_MIN_M") ? atoi(getenv("TROCM_MV_MFMA_MIN_M")) : 0;
     static const int forced_lds_kb = getenv("TROCM_MV_MFMA_LDS_KB") ? atoi(getenv("TROCM_MV_MFMA_LDS_KB")) : 0;
-    static const int forced_r = getenv("TROCM_MV_MFMA_ROWS") ? atoi(getenv("TROCM_MV_MFMA_ROWS")) : 0;
     static const int forced_sets = getenv("TROCM_MV_MFMA_SETS") ? atoi(getenv("TROCM_MV_MFMA_SETS")) : 0;
     if (!enabled || act_dtype != TROCM_F16 || m < 2 || m > 16 || k % 128 != 0 || k < 128) return 2;
     if ((uintptr_t)codes % 16 || (uintptr_t)scales % 8 || (uintptr_t)act % 8 || (uintptr_t)out % 2) return 2;
@@ -337,15 +335,14 @@ int launch_q4_0_matvec_mfma(const void *codes, const void *scales, int64_t w_bat
         p.cq = forced_cq > 0 && forced_cq % pd == 0 ? forced_cq : pd;
         p.nch = (int)((per_split + p.cq - 1) / p.cq);
     }
-    // One block of 16 rows per wave (two, sharing each read of the activations, measured slower: 105 vs 91 us for
-    // 128256 x 4096 and 8 rows).  Sets of 4 waves behind one staged chunk: four when that still leaves about a
-    // workgroup per compute unit (14336 rows, 8 activation rows: 15.2 us; two sets 16.6 us; one 21.8 us), else two
-    // (4096 rows: 10.7 us; four sets 14.0 us; one 11.5 us).
-    const int r = forced_r == 2 ? 2 : 1;
+    // One block of 16 rows per wave (R = 1; two, sharing each read of the activations, measured slower: 105 vs 91 us
+    // for 128256 x 4096 and 8 rows, and are not instantiated).  Sets of waves behind one staged chunk: one of 8 waves
+    // for matrices of few rows; of 4 waves, four when that still leaves about a workgroup per compute unit (14336
+    // rows, 8 activation rows: 15.2 us; two sets 16.6 us; one 21.8 us), else two.
     int sets = splits == 8 ? 1 : blocks16 >= 3 * cus ? 4 : 2;
     if (forced_sets == 1 || forced_sets == 2 || forced_sets == 4) sets = forced_sets;
     if (p.nch > 1 && m > 8 && forced_sets == 0) sets = splits == 8 ? 2 : 4;    // 1024 threads hold a chunk of 16 rows in their registers
-    return r == 2 ? launch_r<2>(p, splits, sets, act_batch, s) : launch_r<1>(p, splits, sets, act_batch, s);
+    return launch_r<1>(p, splits, sets, act_batch, s);
 }
 
 }  // namespace trocm
