@@ -128,17 +128,28 @@ __global__ __launch_bounds__(64 * KS * S) void q4_0_matvec_mfma_kernel(MvMfmaDev
 
         // PD groups of four blocks per row ahead, across the chunks: the weights do not wait for a chunk's staging.
         u32x4 cn[PD][R];
-        uint64_t sn[PD][R];                                     // four f16 scales
+        // The f16 scales of a round of PD groups come with one load per round: lane group g takes those of group
+        // g % PD of the round (8 bytes: four blocks), and ds_bpermute hands them round at use.  (Every load
+        // instruction that touches 16 rows costs the compute unit's address path 16 cache lines, whatever it takes
+        // from them: without the weights' loads the launch took 61 of 94 us, without the scales' 76.)
+        uint64_t sr[R], sr_next[R];
+        auto fetch_scales = [&](uint64_t (&dst)[R], int t0) {
+            const int t = min(t0 + (g & (PD - 1)), ni - 1);     // (past the end: the last group's again, unused)
+#pragma unroll
+            for (int rr = 0; rr < R; rr++) dst[rr] = *reinterpret_cast<const uint64_t *>(p.scales + rows[rr] * nb + (it_lo + t) * 4);
+        };
         auto fetch = [&](int slot, int t) {
 #pragma unroll
             for (int rr = 0; rr < R; rr++) {
                 cn[slot][rr] = *reinterpret_cast<const u32x4 *>(p.codes + rows[rr] * (p.k / 2) + (int64_t)((it_lo + t) * 4 + g) * 16);
-                sn[slot][rr] = *reinterpret_cast<const uint64_t *>(p.scales + rows[rr] * nb + (it_lo + t) * 4);
             }
         };
 #pragma unroll
         for (int d = 0; d < PD; d++)
             if (d < ni) fetch(d, d);
+        if (ni > 0) fetch_scales(sr, 0);
+#pragma unroll
+        for (int rr = 0; rr < R; rr++) sr_next[rr] = 0;
 
         const bool stage_here = !one_chunk || grp == (int)blockIdx.x;
         u32x2 held[kStageRegs];
@@ -190,7 +201,8 @@ __global__ __launch_bounds__(64 * KS * S) void q4_0_matvec_mfma_kernel(MvMfmaDev
                     if (c + 1 < p.nch) hold(c + 1);               // in flight during this chunk's arithmetic
             }
             const int cnt = min(max(ni - c * p.cq, 0), p.cq);               // this wave's groups in the chunk
-            for (int l0 = 0; l0 < cnt; l0 += PD)
+            for (int l0 = 0; l0 < cnt; l0 += PD) {
+                if (c * p.cq + l0 + PD < ni) fetch_scales(sr_next, c * p.cq + l0 + PD);
 #pragma unroll
                 for (int d = 0; d < PD; d++) {
                     const int l = l0 + d;
@@ -199,7 +211,12 @@ __global__ __launch_bounds__(64 * KS * S) void q4_0_matvec_mfma_kernel(MvMfmaDev
                     u32x4 cw[R];
                     uint64_t sc[R];
 #pragma unroll
-                    for (int rr = 0; rr < R; rr++) cw[rr] = cn[d][rr], sc[rr] = sn[d][rr];
+                    for (int rr = 0; rr < R; rr++) {
+                        cw[rr] = cn[d][rr];
+                        const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute((r16 + 16 * d) * 4, (int)(uint32_t)sr[rr]);
+                        const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute((r16 + 16 * d) * 4, (int)(uint32_t)(sr[rr] >> 32));
+                        sc[rr] = lo | (uint64_t)hi << 32;
+                    }
                     if (t + PD < ni) fetch(d, t + PD);
 #pragma unroll
                     for (int rr = 0; rr < R; rr++) transpose_lane_groups(cw[rr]);
@@ -217,6 +234,9 @@ __global__ __launch_bounds__(64 * KS * S) void q4_0_matvec_mfma_kernel(MvMfmaDev
                         }
                     }
                 }
+#pragma unroll
+                for (int rr = 0; rr < R; rr++) sr[rr] = sr_next[rr];
+            }
         }
         // acc[rr][e] = partial out[4 g + e][row rr * 16 + r16] of this wave's set: wave q < 4 of the set adds its KS
         // values of e = q.
