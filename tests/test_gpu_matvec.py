@@ -37,7 +37,7 @@ def f64_product(blocks, act, dt):
     # 4..16 f16 rows against 16 weight rows per matrix instruction: one staged chunk (2 and 4 sets of waves per
     # workgroup, more than 64 KB of LDS), k beyond one chunk, ragged n, batches that share weights
     (1, 1, 5, 2050, 256), (1, 1, 8, 2048, 4096), (1, 1, 6, 2100, 8320), (1, 1, 4, 12300, 128), (1, 1, 7, 12290, 384),
-    (1, 1, 16, 40, 384), (2, 4, 12, 70, 256), (1, 2, 9, 129, 1024), (1, 1, 13, 3000, 2176), (1, 1, 16, 2049, 4096),
+    (1, 1, 16, 40, 384), (2, 4, 12, 70, 256), (1, 1, 4, 2064, 512), (1, 2, 9, 129, 1024), (1, 1, 13, 3000, 2176), (1, 1, 16, 2049, 4096),
 ])
 def test_matvec_matches_the_oracle(rt, dt, wb, ab, m, n, k):
     rng = np.random.default_rng(n + k + m)

@@ -311,7 +311,7 @@ int launch_r(const MvMfmaDev &p, int splits, int sets, int64_t act_batch, hipStr
 
 // 2 = not taken (the caller runs the vector-ALU kernel): f32 activations (their products stay in f32 there), k that
 // is not a whole number of 128-feature groups, misaligned operands, and the row counts and matrix sizes at which the
-// vector-ALU kernel measured faster (up to 4 rows; up to 8 rows against fewer than 2048 weight rows).
+// vector-ALU kernel measured faster (up to 3 rows; up to 8 rows against fewer than 2048 weight rows).
 int launch_q4_0_matvec_mfma(const void *codes, const void *scales, int64_t w_batch, int64_t n, int64_t k, const void *act,
                             int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s) {
     static const int enabled = getenv("TROCM_MV_MFMA") ? atoi(getenv("TROCM_MV_MFMA")) : 1;
@@ -323,9 +323,10 @@ int launch_q4_0_matvec_mfma(const void *codes, const void *scales, int64_t w_bat
     if (n < 1 || n >= (1ll << 30) || k >= (1ll << 30) || act_batch < 1 || act_batch > 65535) return 2;
     const int64_t cus = num_compute_units();
     const int64_t blocks16 = (n + 15) / 16 * act_batch;          // blocks of 16 weight rows in the launch
-    // Measured against the vector-ALU kernel (14336 x 4096: 4 rows 13.9 vs 16.7 us, 8 rows 15.2 vs 38.8 us;
-    // 4096 x 4096: 4 rows 9.2 vs 6.9 us, 8 rows 10.7 vs 14.2 us; 1024 x 4096, 8 rows: 10.1 vs 7.4 us).
-    const int64_t min_m = forced_min_m > 0 ? forced_min_m : blocks16 >= 3 * cus ? 4 : 5;
+    // Measured against the vector-ALU kernel (us; 14336 x 4096: 3 rows 12.1 vs 13.2, 4 rows 12.5 vs 16.7, 8 rows 13.6 vs
+    // 38.8; 4096 x 4096: 3 rows 6.4 vs 6.0, 4 rows 6.8 vs 6.9, 8 rows 8.3 vs 14.2; 128256 x 4096: 3 rows 80.5 vs 78.2,
+    // 4 rows 78 vs 98; 1024 x 4096, 8 rows: 10.1 vs 7.4).
+    const int64_t min_m = forced_min_m > 0 ? forced_min_m : 4;
     if (m < min_m || (m <= 8 && forced_min_m == 0 && blocks16 * 2 < cus)) return 2;
     MvMfmaDev p;
     memset(&p, 0, sizeof(p));
