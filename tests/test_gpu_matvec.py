@@ -54,6 +54,26 @@ def test_matvec_matches_the_oracle(rt, dt, wb, ab, m, n, k):
         assert rel_err(got, orc.q4_0_matvec(blocks, act).astype(np.float64)) <= tol
 
 
+@pytest.mark.parametrize("m,k", [(16, 3584), (8, 4096)])
+def test_tall_matrix_of_repeated_rows(rt, m, k):
+    """65536 weight rows (the output matrix of a large vocabulary), built by repeating 512 quantised rows: every
+    workgroup walks several row groups behind one staged copy of the activations.  16 rows of 3584 features
+    leave the waves no LDS for their code buffers (the kernel that loads 64 bytes per row and transposes over the
+    lane groups runs), 8 rows do.  Expected: the f64 product of the 512 rows, repeated."""
+    rng = np.random.default_rng(m + k)
+    base_n, reps = 512, 128
+    w = (rng.standard_normal((1, base_n, k)) * 0.05).astype(np.float32)
+    w[:, :, ::97] *= 8.0
+    act = rng.standard_normal((1, m, k)).astype(np.float16)
+    base = orc.quant(Q4, w)
+    blocks = np.ascontiguousarray(np.tile(base, (1, reps, 1)))
+    wq = tract_amd.Q40Weights(blocks, 1, base_n * reps, k)
+    got = tract_amd.GgmlGemm().eval(act, wq).to_numpy()
+    want = np.tile(f64_product(base, act, np.float16), (1, 1, reps))
+    assert got.shape == want.shape and rel_err(got, want) <= 4e-3
+    assert np.array_equal(got[:, :, :base_n], got[:, :, -base_n:])
+
+
 def test_closed_form_blocks(rt):
     """Nibbles i % 16 in every block (the table of q4_0.rs:722-739): sums of whole blocks and single
     elements are known exactly, low and high nibbles alike."""

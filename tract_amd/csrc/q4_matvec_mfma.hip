@@ -52,8 +52,10 @@ struct MvMfmaDev {
     int cq;                   // groups of four blocks (128 features) per quarter of k in one staged chunk
     int nch;                  // chunks; 1 = the activations fit in LDS and are staged once per workgroup
     int prefetch;             // the next chunk's activations wait in registers during this chunk's arithmetic
+    int wide;                 // 128-byte loads of 8 rows through the waves' code buffers (host-side choice of the kernel)
     int groups;               // row groups of 16 R S rows
 };
+constexpr int kCodeRow = 144;   // bytes between the rows of a wave's pair of code groups in LDS (128 + 16: no bank conflicts)
 constexpr int kStageRegs = 8;   // 8-byte pieces of the next chunk a thread holds (prefetch mode)
 // cq in prefetch mode is PD: a chunk is 2048 features, 512 pieces per row, and piece indices split by shifts
 
@@ -80,7 +82,7 @@ __device__ __forceinline__ void transpose_lane_groups(u32x4 &w) {
     w[0] = t01[0], w[1] = t01[1], w[2] = t23[0], w[3] = t23[1];
 }
 
-template <int R, int S, bool PF, int KS>
+template <int R, int S, bool PF, int KS, bool WIDE>
 __global__ __launch_bounds__(64 * KS * S) void q4_0_matvec_mfma_kernel(MvMfmaDev p) {
     constexpr int kThreads = 64 * KS * S, PD = 16 / KS, kPrefetchCq = PD;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -95,6 +97,7 @@ __global__ __launch_bounds__(64 * KS * S) void q4_0_matvec_mfma_kernel(MvMfmaDev
     const int it_lo = q * nit / KS, ni = (q + 1) * nit / KS - it_lo;   // this wave's groups of four blocks
     const _Float16 *act = p.act + (int64_t)b * p.act_stride_b;
     _Float16 *out = p.out + (int64_t)b * p.out_stride_b;
+    unsigned char *wave_codes = lds_raw + (size_t)p.m * kc * sizeof(_Float16) + (size_t)KS * S * R * 4 * 64 * sizeof(float) + w * (16 * kCodeRow);   // (WIDE)
     const int arow = min(r16, p.m - 1);      // output rows m..15 of the instruction are never stored: any row serves
     const bool one_chunk = p.nch == 1;
 
@@ -138,15 +141,31 @@ __global__ __launch_bounds__(64 * KS * S) void q4_0_matvec_mfma_kernel(MvMfmaDev
 #pragma unroll
             for (int rr = 0; rr < R; rr++) dst[rr] = *reinterpret_cast<const uint64_t *>(p.scales + rows[rr] * nb + (it_lo + t) * 4);
         };
-        auto fetch = [&](int slot, int t) {
+        // WIDE: a load instruction takes 128 contiguous bytes (8 blocks: a pair of groups) of 8 rows: lane = (row
+        // lane / 8, block lane % 8); slot s of a round holds rows (s & 1) * 8 .. + 7 of pair s / 2.  Half as many cache
+        // lines per byte as 64 bytes of 16 rows; the wave passes the pair through its own 16 x 144 bytes of LDS to the
+        // lanes that feed the matrix instruction.  Else lane (r, g) loads block g of a group of row r, and the lane
+        // groups transpose.
+        static_assert(!WIDE || R == 1, "one block of 16 rows per wave");
+        const int ra = lane >> 3, b8 = lane & 7;
+        int64_t rows_h[2];
 #pragma unroll
-            for (int rr = 0; rr < R; rr++) {
-                cn[slot][rr] = *reinterpret_cast<const u32x4 *>(p.codes + rows[rr] * (p.k / 2) + (int64_t)((it_lo + t) * 4 + g) * 16);
+        for (int h = 0; h < 2; h++) rows_h[h] = (int64_t)wb * p.n + min((grp * S + st) * R * 16 + h * 8 + ra, p.n - 1);
+        auto fetch = [&](int slot, int t) {                     // t: the group; WIDE: the pair's first group
+            if constexpr (WIDE) {
+                const int blk = min((it_lo + t) * 4 + b8, (it_lo + ni) * 4 - 1);   // (an odd share's last pair: the last block again, unused)
+                cn[slot][0] = *reinterpret_cast<const u32x4 *>(p.codes + rows_h[slot & 1] * (p.k / 2) + (int64_t)blk * 16);
+            } else {
+#pragma unroll
+                for (int rr = 0; rr < R; rr++)
+                    cn[slot][rr] = *reinterpret_cast<const u32x4 *>(p.codes + rows[rr] * (p.k / 2) + (int64_t)((it_lo + t) * 4 + g) * 16);
             }
         };
 #pragma unroll
-        for (int d = 0; d < PD; d++)
-            if (d < ni) fetch(d, d);
+        for (int d = 0; d < PD; d++) {
+            const int t = WIDE ? (d & ~1) : d;
+            if (t < ni) fetch(d, t);
+        }
         if (ni > 0) fetch_scales(sr, 0);
 #pragma unroll
         for (int rr = 0; rr < R; rr++) sr_next[rr] = 0;
@@ -203,6 +222,38 @@ __global__ __launch_bounds__(64 * KS * S) void q4_0_matvec_mfma_kernel(MvMfmaDev
             const int cnt = min(max(ni - c * p.cq, 0), p.cq);               // this wave's groups in the chunk
             for (int l0 = 0; l0 < cnt; l0 += PD) {
                 if (c * p.cq + l0 + PD < ni) fetch_scales(sr_next, c * p.cq + l0 + PD);
+                if constexpr (WIDE) {
+#pragma unroll
+                for (int pr = 0; pr < PD / 2; pr++) {
+                    const int lp = l0 + 2 * pr;
+                    if (lp >= cnt) break;
+                    const int tp = c * p.cq + lp;                           // even: pairs do not straddle rounds or chunks
+#pragma unroll
+                    for (int h = 0; h < 2; h++)
+                        *reinterpret_cast<u32x4 *>(wave_codes + (h * 8 + ra) * kCodeRow + b8 * 16) = cn[2 * pr + h][0];
+                    if (tp + PD < ni) fetch(2 * pr, tp + PD), fetch(2 * pr + 1, tp + PD);
+#pragma unroll
+                    for (int i2 = 0; i2 < 2; i2++) {
+                        const int l = lp + i2;
+                        if (l >= cnt) break;
+                        const int d = 2 * pr + i2;
+                        const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute((r16 + 16 * d) * 4, (int)(uint32_t)sr[0]);
+                        const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute((r16 + 16 * d) * 4, (int)(uint32_t)(sr[0] >> 32));
+                        const uint64_t sc = lo | (uint64_t)hi << 32;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const int vec = (q * p.cq + l) * 16 + ((j * 4 + g) ^ arow);
+                            const half8_t a = *reinterpret_cast<const half8_t *>(lds_x + arow * kc + vec * 8);
+                            const uint32_t code = *reinterpret_cast<const uint32_t *>(wave_codes + r16 * kCodeRow + (i2 * 4 + j) * 16 + g * 4);
+                            const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, codes_as_halves(code),
+                                                                                         float4_t{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+                            const float dsc = (float)__builtin_bit_cast(_Float16, (uint16_t)(sc >> (16 * j)));
+#pragma unroll
+                            for (int e = 0; e < 4; e++) acc[0][e] = __builtin_fmaf(dsc, part[e], acc[0][e]);
+                        }
+                    }
+                }
+                } else {
 #pragma unroll
                 for (int d = 0; d < PD; d++) {
                     const int l = l0 + d;
@@ -234,6 +285,7 @@ __global__ __launch_bounds__(64 * KS * S) void q4_0_matvec_mfma_kernel(MvMfmaDev
                         }
                     }
                 }
+                }
 #pragma unroll
                 for (int rr = 0; rr < R; rr++) sr[rr] = sr_next[rr];
             }
@@ -259,11 +311,11 @@ __global__ __launch_bounds__(64 * KS * S) void q4_0_matvec_mfma_kernel(MvMfmaDev
     }
 }
 
-template <int R, int S, bool PF, int KS>
+template <int R, int S, bool PF, int KS, bool WIDE>
 int launch_rsp(const MvMfmaDev &p, int64_t act_batch, hipStream_t s) {
-    const size_t lds = (size_t)p.m * KS * p.cq * 128 * 2 + (size_t)KS * S * R * 4 * 64 * sizeof(float);
+    const size_t lds = (size_t)p.m * KS * p.cq * 128 * 2 + (size_t)KS * S * R * 4 * 64 * sizeof(float) + (WIDE ? (size_t)KS * S * 16 * kCodeRow : 0);
     if (lds > 64 * 1024 &&      // beyond the default limit of dynamic LDS: allowed per kernel (and device) on request
-        hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_0_matvec_mfma_kernel<R, S, PF, KS>), hipFuncAttributeMaxDynamicSharedMemorySize,
+        hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_0_matvec_mfma_kernel<R, S, PF, KS, WIDE>), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
         (void)hipGetLastError();
         return 2;
@@ -281,7 +333,7 @@ int launch_rsp(const MvMfmaDev &p, int64_t act_batch, hipStream_t s) {
         const int64_t turns = (wgs + resident - 1) / resident;
         wgs = (wgs + turns - 1) / turns;
     }
-    hipLaunchKernelGGL((q4_0_matvec_mfma_kernel<R, S, PF, KS>), dim3((unsigned)wgs, (unsigned)act_batch), dim3(64 * KS * S), lds, s, p);
+    hipLaunchKernelGGL((q4_0_matvec_mfma_kernel<R, S, PF, KS, WIDE>), dim3((unsigned)wgs, (unsigned)act_batch), dim3(64 * KS * S), lds, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("q4_0_matvec (matrix cores) launch failed: %s", hipGetErrorString(e));
     return 0;
@@ -294,10 +346,12 @@ int launch_rs(MvMfmaDev p, int64_t act_batch, hipStream_t s) {
     if constexpr (kThreads >= 512) {
         static const int allowed = getenv("TROCM_MV_MFMA_PREFETCH") ? atoi(getenv("TROCM_MV_MFMA_PREFETCH")) : 1;
         p.prefetch = allowed && p.nch > 1 && p.cq == 16 / KS && (p.m + (kThreads >> 9) - 1) / (kThreads >> 9) <= kStageRegs;
-        if (p.prefetch) return launch_rsp<R, S, true, KS>(p, act_batch, s);
+        if (p.prefetch) return launch_rsp<R, S, true, KS, true>(p, act_batch, s);
     }
     p.prefetch = 0;
-    return launch_rsp<R, S, false, KS>(p, act_batch, s);
+    if constexpr (S == 4 && KS == 4)      // (the one shape whose activations may leave no room for the code buffers)
+        if (!p.wide) return launch_rsp<R, S, false, KS, false>(p, act_batch, s);
+    return launch_rsp<R, S, false, KS, true>(p, act_batch, s);
 }
 
 template <int R>
@@ -334,34 +388,41 @@ int launch_q4_0_matvec_mfma(const void *codes, const void *scales, int64_t w_bat
     p.act = (const _Float16 *)act, p.out = (_Float16 *)out;
     p.act_stride_b = m * k, p.out_stride_b = m * n;
     p.n = (int)n, p.k = (int)k, p.m = (int)m, p.ratio = (int)(act_batch / w_batch);
-    // Every wave walks one quarter of k.  If the whole of the activations fits the LDS budget they are staged once per
-    // workgroup; else in chunks of 4 groups of 128 features per quarter (2048 features, a multiple of the weights'
-    // prefetch depth), the next chunk waiting in registers.
     // Every wave walks one share of k: a quarter, or an eighth when the matrix has too few rows to give every SIMD a
-    // wave otherwise.  If the whole of the activations fits the LDS budget they are staged once per workgroup; else in
-    // chunks of 2048 features (512 or 256 of every share, a multiple of the weights' prefetch depth), the next chunk
-    // waiting in registers.
+    // wave otherwise.
     static const int forced_cq = getenv("TROCM_MV_MFMA_CQ") ? atoi(getenv("TROCM_MV_MFMA_CQ")) : 0;
     static const int forced_splits = getenv("TROCM_MV_MFMA_SPLITS") ? atoi(getenv("TROCM_MV_MFMA_SPLITS")) : 0;
     int splits = blocks16 < 2 * cus && k >= 2048 ? 8 : 4;
     if (forced_splits == 4 || forced_splits == 8) splits = forced_splits;
     const int64_t per_split = (k / 128 + splits - 1) / splits;
-    // (budget: 64 KB, two workgroups per compute unit; 136 KB when every workgroup walks many row groups behind
-    // one staging: 128256 x 4096 with 16 rows 95 us, in chunks 125 us; 14336 x 4096 20.0 us, in chunks 16.5 us)
-    const int64_t budget = forced_lds_kb > 0 ? (int64_t)forced_lds_kb * 1024 : blocks16 / 4 >= 4 * cus ? 136 * 1024 : 64 * 1024;
-    if (m * splits * per_split * 128 * 2 <= budget) {
-        p.cq = (int)per_split, p.nch = 1;
-    } else {
-        const int pd = 16 / splits;
-        p.cq = forced_cq > 0 && forced_cq % pd == 0 ? forced_cq : pd;
-        p.nch = (int)((per_split + p.cq - 1) / p.cq);
-    }
     // One block of 16 rows per wave (R = 1; two, sharing each read of the activations, measured slower: 105 vs 91 us
     // for 128256 x 4096 and 8 rows, and are not instantiated).  Sets of waves behind one staged chunk: one of 8 waves
     // for matrices of few rows; of 4 waves, four when that still leaves about a workgroup per compute unit (14336
     // rows, 8 activation rows: 15.2 us; two sets 16.6 us; one 21.8 us), else two.
     int sets = splits == 8 ? 1 : blocks16 >= 3 * cus ? 4 : 2;
     if (forced_sets == 1 || forced_sets == 2 || forced_sets == 4) sets = forced_sets;
+    // If the whole of the activations fits the LDS budget they are staged once per workgroup; else in chunks of 2048
+    // features (512 or 256 of every share, a multiple of the weights' prefetch depth), the next chunk waiting in
+    // registers.  Budget: what leaves room for two workgroups of 8 waves or one of 16 on a compute unit beside the
+    // partial sums and the waves' code buffers; all of the LDS when every workgroup walks many row groups behind one
+    // staging (128256 x 4096 with 16 rows: 95 us, in chunks 125 us; 14336 x 4096: 20.0 us, in chunks 16.5 us), with
+    // without the code buffers if that is what makes it fit.
+    const int64_t x_bytes = m * splits * per_split * 128 * 2;
+    auto beside = [&](int st, bool wide = true) { return (int64_t)splits * st * (4 * 64 * 4 + (wide ? 16 * kCodeRow : 0)); };
+    const int64_t lds_all = 160 * 1024;
+    const bool walks_many = blocks16 / 4 >= 4 * cus;
+    // (16 activation rows of 4096 features leave the 16 waves no room for code buffers: the 64-byte loads then)
+    p.wide = !(walks_many && splits * sets == 16 && x_bytes + beside(sets) > lds_all && x_bytes + beside(sets, false) <= lds_all);
+    const int64_t budget = forced_lds_kb > 0 ? (int64_t)forced_lds_kb * 1024
+                         : walks_many        ? lds_all - beside(sets, p.wide)
+                         : splits * sets >= 16 ? 64 * 1024 : lds_all / 2 - beside(sets);
+    if (x_bytes <= budget) {
+        p.cq = (int)per_split, p.nch = 1;
+    } else {
+        const int pd = 16 / splits;
+        p.cq = forced_cq > 0 && forced_cq % pd == 0 ? forced_cq : pd;
+        p.nch = (int)((per_split + p.cq - 1) / p.cq);
+    }
     if (p.nch > 1 && m > 8 && forced_sets == 0) sets = splits == 8 ? 2 : 4;    // 1024 threads hold a chunk of 16 rows in their registers
     return launch_r<1>(p, splits, sets, act_batch, s);
 }
