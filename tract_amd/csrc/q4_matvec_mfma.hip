@@ -15,10 +15,13 @@
 //
 // Work: KS waves (4, or 8 when the matrix has too few rows to occupy every SIMD otherwise) own 16 R weight rows; each
 // walks one contiguous share of k, and they add their partial sums through LDS at the end.  A workgroup holds S
-// such sets behind one staged chunk of the activations.  Lane l = (r, g) (r = l % 16, g = l / 16) loads the 16
-// bytes of block 4 i + g of row r, a 4 x 4 transpose over the lane groups (v_permlane32_swap,
-// v_permlane16_swap) hands it byte group g of blocks 4 i .. 4 i + 3, i.e. codes 4g..4g+3 and 16+4g..16+4g+3
-// of each block: the B operand of one instruction per block.  The activations are staged in LDS in that
+// such sets behind one staged chunk of the activations.  The instruction wants from lane (r, g) (r = l % 16,
+// g = l / 16) byte group g of a block of weight row r, i.e. its codes 4g..4g+3 and 16+4g..16+4g+3.  The codes are
+// loaded 128 contiguous bytes (8 blocks) of 8 rows per instruction and passed through 16 x 144 bytes of LDS of the
+// wave's own, from which every lane reads its four bytes per instruction (a load instruction costs the compute
+// unit's address path one step per cache line it touches, whatever it uses of the line); where LDS has no room for
+// that, lane (r, g) loads the 16 bytes of block 4 i + g of row r and a 4 x 4 transpose over the lane groups
+// (v_permlane32_swap, v_permlane16_swap) hands it byte group g of blocks 4 i .. 4 i + 3.  The activations are staged in LDS in that
 // feature order (16-byte vectors XOR-swizzled by row, so that the 16 rows of one read fall into different
 // banks) and read as the A operand.  When they do not fit, they are staged in chunks of 2048 features that hold a
 // piece of every wave's share of k, so that a wave's weights stay one contiguous stream that is prefetched across
