@@ -899,10 +899,14 @@ sys.stdout.buffer.write(o.tobytes())
 @pytest.mark.parametrize("env", [{"TROCM_PREFILL_SPLITS": "1"}, {"TROCM_PREFILL_SPLITS": "2"},
                                  {"TROCM_PREFILL_SPLITS": "5"}, {"TROCM_PREFILL_SPLITS": "16"},
                                  {"TROCM_PREFILL_HG": "1"}, {"TROCM_PREFILL_HG": "2"}, {"TROCM_PREFILL_PP": "0"},
-                                 {"TROCM_PREFILL_TAIL_MERGE": "0"}, {"TROCM_PREFILL_TAIL_MERGE": "0", "TROCM_PREFILL_SPLITS": "7"}])
+                                 {"TROCM_PREFILL_TAIL_MERGE": "0"}, {"TROCM_PREFILL_TAIL_MERGE": "0", "TROCM_PREFILL_SPLITS": "7"},
+                                 {"TROCM_PREFILL_PING": "1"}, {"TROCM_PREFILL_PING": "1", "TROCM_PREFILL_SPLITS": "1"},
+                                 {"TROCM_PREFILL_PING": "1", "TROCM_PREFILL_HG": "1"}, {"TROCM_PREFILL_PING": "1", "TROCM_PREFILL_HG": "2", "TROCM_PREFILL_SPLITS": "3"}])
 def test_prefill_any_split_count_and_head_grouping_agree(rt, env):
     """The key-split merge is exact in real arithmetic and the head grouping only changes which
-    workgroup computes a head: every setting must agree with the textbook form."""
+    workgroup computes a head: every setting must agree with the textbook form.  TROCM_PREFILL_PING=1
+    selects the tile loop that loads K/V straight into LDS and alternates two groups of waves between the
+    matrix and the vector half of a tile."""
     import subprocess, sys
     e = dict(os.environ)
     e.update(env)

@@ -18,12 +18,20 @@
 //    workspace, laid out exactly as the accumulator registers are (so every store instruction
 //    covers 512 contiguous bytes), and a small kernel merges them.
 //  * The output accumulators are rescaled only when some query's running maximum moved.
+//  * A second tile loop (template argument PING, chosen with TROCM_PREFILL_PING=1, f16 caches without a mask
+//    input) loads K/V tiles straight into LDS (global_load_lds_dwordx4, swizzled rows) and runs waves 0..3 and
+//    4..7 half a tile apart, one group on the matrix cores while the other computes its softmax.  It gives the
+//    same results and, measured, the same speed (within 2 %) as the loop that stages through registers, which
+//    stays the default: removing the barriers, the load waits or the priorities from it changes nothing, while
+//    removing the MFMAs, the LDS fragment reads, the softmax or the direct loads shortens it by 36, 26, 18
+//    and 12 %: the parts add up, because an MFMA in flight blocks most of the other wave's vector issue slots.
 //
 // Roofline: MFMA-bound.  FLOPs = 4 * B * Hq * D * (visible query-key pairs).
 #include <hip/hip_fp16.h>
 #include <string.h>
 #include <stdlib.h>
 #include <type_traits>
+#include <utility>
 #include "common.h"
 
 namespace trocm {
@@ -74,7 +82,22 @@ __device__ __forceinline__ half4_t lds_read_tr16(const _Float16 *lds_ptr) {
 }
 
 constexpr int kWavesPP = 8, kThreadsPP = 64 * kWavesPP, kTileN = 64;
+
+template <class F, int... Is>
+__device__ __attribute__((always_inline)) inline void static_for_impl(F &&f, std::integer_sequence<int, Is...>) { (f(std::integral_constant<int, Is>{}), ...); }
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression
+template <int N, class F>
+__device__ __attribute__((always_inline)) inline void static_for(F &&f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
 constexpr float kLazyMax = 8.0f;
+#ifndef TROCM_PING_PRIO_MFMA
+#define TROCM_PING_PRIO_MFMA 1
+#endif
+#ifndef TROCM_PING_DEPTH
+#define TROCM_PING_DEPTH 4   // fragments requested ahead of the MFMA that uses them
+#endif
+#ifndef TROCM_PING_PRIO_VALU
+#define TROCM_PING_PRIO_VALU 0
+#endif
 
 __device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
@@ -93,8 +116,10 @@ __device__ __forceinline__ u32x4 dequant8(uint32_t b0123, uint32_t b4567, half2_
     return r;
 }
 
-template <int D, int HG, bool MASK, int FMT>
+
+template <int D, int HG, bool MASK, int FMT, bool PING = false>
 __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p) {
+    static_assert(!PING || (!MASK && FMT == TROCM_F16), "the ping-pong loop serves f16 caches without a mask input");
     constexpr int QB = kWavesPP / HG;     // 32-query blocks per workgroup
     constexpr int BLOCK_M = 32 * QB;
     constexpr int KS = D / 16;            // contraction steps of Q K^T
@@ -104,8 +129,17 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
     constexpr int NL = kTileN * D / 8 / kThreadsPP;  // 128-bit loads per thread per tile and tensor
     static_assert(NL >= 1 && NL * 8 * kThreadsPP == kTileN * D, "tile loads must divide evenly");
 
-    __shared__ __attribute__((aligned(16))) _Float16 lds_k[2][kTileN * KROW];
-    __shared__ __attribute__((aligned(16))) _Float16 lds_v[2][kTileN * VROW];
+    // One LDS block: two K tiles, then two V tiles.  The ping-pong loop keeps rows unpadded (the direct loads write
+    // 1024 contiguous bytes per instruction) and swizzles their 16-byte pieces instead.
+    constexpr int K_TILE = PING ? kTileN * D : kTileN * KROW;   // halves
+    constexpr int V_TILE = PING ? kTileN * D : kTileN * VROW;
+    constexpr int TR_HALVES = kWavesPP * 32 * (D / 2 + 8);      // output transposition area of the epilogue
+    constexpr int WTS_HALVES = kWavesPP * 16 * 32 * 2;          // merge weights of the epilogue (floats)
+    constexpr int LDS_HALVES = PING ? (2 * K_TILE + 2 * V_TILE > WTS_HALVES + TR_HALVES ? 2 * K_TILE + 2 * V_TILE : WTS_HALVES + TR_HALVES)
+                                    : 2 * K_TILE + 2 * V_TILE;
+    __shared__ __attribute__((aligned(1024))) _Float16 lds_all[LDS_HALVES];
+    _Float16 (*lds_k)[K_TILE] = reinterpret_cast<_Float16 (*)[K_TILE]>(&lds_all[0]);
+    _Float16 (*lds_v)[V_TILE] = reinterpret_cast<_Float16 (*)[V_TILE]>(&lds_all[2 * K_TILE]);
 
     const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hb = lane >> 5, l32 = lane & 31;
@@ -248,7 +282,7 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
     };
 
     // does this wave have anything to do on tile kt?
-    auto tile_active = [&](int kt) { return wave_has_queries && (!p.causal || kt * kTileN <= wave_q_last + off); };
+    auto tile_active = [&](int kt) __attribute__((always_inline)) { return wave_has_queries && (!p.causal || kt * kTileN <= wave_q_last + off); };
 
     // ---- S^T = K Q^T : 2 key blocks of 32 x 32 queries ---------------------------------------------
     auto qk = [&](int kbuf, float16_t (&s)[2]) {
@@ -268,7 +302,7 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
     };
 
     // ---- online softmax for query lane%32 over this lane's 32 keys; leaves P^T fragments in pf ----
-    auto softmax = [&](int kt, float16_t (&s)[2], half8_t (&pf)[4]) {
+    auto softmax = [&](int kt, float16_t (&s)[2], half8_t (&pf)[4]) __attribute__((always_inline)) {
         const int k_lo = kt * kTileN;
         if constexpr (MASK) {
             // logits in the log2 domain, mask added: the maximum below is then taken after the scaling
@@ -280,14 +314,12 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
         }
         const bool need_mask = (k_lo + kTileN > p.Sk) || (p.causal && (k_lo + kTileN - 1 > q0 + off));
         if (need_mask) {
+            // key k_lo + 4 hb + c, c = 32 kb + 8 (r / 4) + r % 4, is visible when c <= lim
+            const int lim = (p.causal ? min(p.Sk - 1, my_q + off) : p.Sk - 1) - k_lo - 4 * hb;
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    int key = k_lo + 32 * kb + 8 * (r >> 2) + 4 * hb + (r & 3);
-                    bool vis = key < p.Sk && (!p.causal || key <= my_q + off);
-                    s[kb][r] = vis ? s[kb][r] : -INFINITY;
-                }
+                for (int r = 0; r < 16; r++) s[kb][r] = (32 * kb + 8 * (r >> 2) + (r & 3)) <= lim ? s[kb][r] : -INFINITY;
         }
         float tmax = -INFINITY;
 #pragma unroll
@@ -349,40 +381,224 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
         }
     };
 
-    if (n_it > 0) prefetch(t_begin);   // issued before the Q loads: both latencies overlap
-    // Q^T fragments: query = lane % 32, features 16*ks + 8*hb .. +8
+    if constexpr (!PING) {
+        if (n_it > 0) prefetch(t_begin);   // issued before the Q loads: both latencies overlap
+        // Q^T fragments: query = lane % 32, features 16*ks + 8*hb .. +8
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) qf[ks] = *reinterpret_cast<const half8_t *>(qrow + 16 * ks + 8 * hb);
-    // Settle the Q loads here.  Otherwise the compiler must assume they may still be in flight at
-    // the top of the tile loop and waits for vmcnt(0) at their first use there, which also waits
-    // for the K/V prefetch issued a few instructions earlier and exposes its whole latency.
+        for (int ks = 0; ks < KS; ks++) qf[ks] = *reinterpret_cast<const half8_t *>(qrow + 16 * ks + 8 * hb);
+        // Settle the Q loads here.  Otherwise the compiler must assume they may still be in flight at
+        // the top of the tile loop and waits for vmcnt(0) at their first use there, which also waits
+        // for the K/V prefetch issued a few instructions earlier and exposes its whole latency.
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) asm volatile("" : "+v"(qf[ks]));
+        for (int ks = 0; ks < KS; ks++) asm volatile("" : "+v"(qf[ks]));
 
-    if (n_it > 0) {
-        stage(0, 0);
-        if (n_it > 1) prefetch(t_begin + 1);
-        prefetch_mask(t_begin);
-    }
-    for (int it = 0; it < n_it; it++) {
-        __syncthreads();   // tile `it` is in LDS; every wave is done with the buffers about to be overwritten
-        const int cur = it & 1;
-        const int kt = t_begin + it;
-        if (tile_active(kt)) {
-            float16_t s[2];
-            half8_t pf[4];
-            qk(cur, s);
-            softmax(kt, s, pf);
-            if (it + 1 < n_it) prefetch_mask(kt + 1);
-            pv(cur, pf);
+        if (n_it > 0) {
+            stage(0, 0);
+            if (n_it > 1) prefetch(t_begin + 1);
+            prefetch_mask(t_begin);
         }
-        // The next tile goes to LDS after this one's arithmetic, not before it: its loads were issued a whole
-        // iteration ago in the steady state and right before the loop for the first iteration, whose arithmetic
-        // then covers their latency.
-        if (it + 1 < n_it) {
-            stage(cur ^ 1, cur ^ 1);
-            if (it + 2 < n_it) prefetch(t_begin + it + 2);
+        for (int it = 0; it < n_it; it++) {
+            __syncthreads();   // tile `it` is in LDS; every wave is done with the buffers about to be overwritten
+            const int cur = it & 1;
+            const int kt = t_begin + it;
+            if (tile_active(kt)) {
+                float16_t s[2];
+                half8_t pf[4];
+                qk(cur, s);
+                softmax(kt, s, pf);
+                if (it + 1 < n_it) prefetch_mask(kt + 1);
+                pv(cur, pf);
+            }
+            // The next tile goes to LDS after this one's arithmetic, not before it: its loads were issued a whole
+            // iteration ago in the steady state and right before the loop for the first iteration, whose arithmetic
+            // then covers their latency.
+            if (it + 1 < n_it) {
+                stage(cur ^ 1, cur ^ 1);
+                if (it + 2 < n_it) prefetch(t_begin + it + 2);
+            }
         }
+    } else {
+        // ---- ping-pong loop -----------------------------------------------------------------------------
+        // Waves 0..3 and waves 4..7 (one of each per SIMD) run half a tile apart: while one group issues the 32 MFMAs
+        // of P.V (previous tile) and K.Q^T (this tile), the other computes its softmax on the vector ALUs, and the
+        // two swap at a barrier (two barriers per tile).  K and V tiles go from global memory straight into LDS
+        // (global_load_lds_dwordx4: each lane fetches 16 bytes from its own address, the 64 pieces of an
+        // instruction land in 1024 consecutive bytes), so rows are unpadded and bank conflicts are avoided by
+        // storing the 16-byte piece p of row r at piece p ^ f(r): the lane that fills physical piece pp of row r
+        // fetches logical piece pp ^ f(r).  f_k(r) = r % 16 (a K fragment read takes one piece of 16
+        // consecutive rows per quarter wave), f_v(r) = 4 (r % 4) (a transposing V read takes 64 consecutive
+        // bytes of 4 consecutive rows per half wave); with 128-byte rows (head size 64) r / 2 takes r's place.
+        constexpr int ROWB = 2 * D, PPR = D / 8, RSH = D == 128 ? 0 : 1;
+        constexpr int NLD = kTileN * PPR / 64 / kWavesPP;   // direct loads per wave, tile and tensor
+        static_assert(NLD >= 1 && NLD * 64 * kWavesPP == kTileN * PPR, "tile pieces must divide over the waves");
+        typedef __attribute__((address_space(3))) void *lds_void_ptr;
+        typedef __attribute__((address_space(1))) const void *global_void_ptr;
+        const int grp = w >> 2;
+        const uint32_t lds0 = (uint32_t)(uintptr_t)&lds_all[0];
+        // This lane's pieces of a tile: instruction n of wave w fills LDS bytes [(w NLD + n) 1024, + 1024) of the
+        // tile, lane i the 16 bytes at 16 i: row (w NLD + n) (64 / PPR) + i / PPR, physical piece i % PPR.
+        const int64_t row_bytes = p.kv_stride_t * 2;
+        uint32_t koff[NLD], voff[NLD];   // byte offsets from the tile's first row (the host admits rows of less than 2^25 bytes)
+#pragma unroll
+        for (int n = 0; n < NLD; n++) {
+            const int row = (w * NLD + n) * (64 / PPR) + lane / PPR, pp = lane % PPR;
+            koff[n] = (uint32_t)row * (uint32_t)row_bytes + (pp ^ ((row >> RSH) & (PPR - 1))) * 16;
+            voff[n] = (uint32_t)row * (uint32_t)row_bytes + (pp ^ (4 * ((row >> RSH) & (PPR / 4 - 1)))) * 16;
+        }
+        // rows past the last key repeat the last key's row (their scores are masked; V must stay finite)
+        auto clamped_off = [&](int kt, int n, bool is_v) __attribute__((always_inline)) {
+            const int row = (w * NLD + n) * (64 / PPR) + lane / PPR, pp = lane % PPR;
+            const int f = is_v ? 4 * ((row >> RSH) & (PPR / 4 - 1)) : (row >> RSH) & (PPR - 1);
+            return (uint32_t)min(row, p.Sk - 1 - kt * kTileN) * (uint32_t)row_bytes + (uint32_t)((pp ^ f) * 16);
+        };
+        // keeps the 32-bit offset a 32-bit register up to the load (hoisted out of the loop it becomes a 64-bit one)
+        auto opaque = [](uint32_t v) __attribute__((always_inline)) {
+            asm volatile("" : "+v"(v));
+            return v;
+        };
+        auto issue_k = [&](int kt, int buf) __attribute__((always_inline)) {
+            const char *tile = reinterpret_cast<const char *>(kbase) + (int64_t)kt * kTileN * row_bytes;
+            const bool whole = (kt + 1) * kTileN <= p.Sk;
+#pragma unroll
+            for (int n = 0; n < NLD; n++)
+                __builtin_amdgcn_global_load_lds((global_void_ptr)(tile + opaque(whole ? koff[n] : clamped_off(kt, n, false))),
+                                                 (lds_void_ptr)(uintptr_t)(lds0 + (uint32_t)((buf * K_TILE) * 2 + (w * NLD + n) * 1024)), 16, 0, 0);
+        };
+        auto issue_v = [&](int kt, int buf) __attribute__((always_inline)) {
+            const char *tile = reinterpret_cast<const char *>(vbase) + (int64_t)kt * kTileN * row_bytes;
+            const bool whole = (kt + 1) * kTileN <= p.Sk;
+#pragma unroll
+            for (int n = 0; n < NLD; n++)
+                __builtin_amdgcn_global_load_lds((global_void_ptr)(tile + opaque(whole ? voff[n] : clamped_off(kt, n, true))),
+                                                 (lds_void_ptr)(uintptr_t)(lds0 + (uint32_t)((2 * K_TILE + buf * V_TILE) * 2 + (w * NLD + n) * 1024)), 16, 0, 0);
+        };
+        // tile it + 1's K and tile it's V: both buffers were last read two barriers ago
+        auto issue_loads = [&](int it) __attribute__((always_inline)) {
+            if (it + 1 < n_it) issue_k(t_begin + it + 1, (it + 1) & 1);
+            if (it < n_it) issue_v(t_begin + it, it & 1);
+        };
+        auto loads_landed = []() __attribute__((always_inline)) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        };
+
+        // K fragment of (key block kb, step ks): row 32 kb + lane % 32, logical piece 2 ks + hb
+        const uint32_t kfrag = lds0 + l32 * ROWB + ((hb ^ ((l32 >> RSH) & (PPR - 1))) << 4);
+        // Per-lane LDS byte addresses of the K fragments of step ks (key block 0) and of the V^T fragments of
+        // feature block db (keys 0..7) in the buffers the next matrix half reads; they flip after every iteration.
+        uint32_t kx[KS], vx[DB];
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) kx[ks] = kfrag ^ (uint32_t)(ks << 5);
+        // V^T fragments: this lane as a source of the transposing loads addresses key row 4 hb + (lane % 16) / 4 of
+        // a group of 8, features 16 (lane / 16 % 2) + 4 (lane % 4) of the 32-feature block db
+        const int vrl = 4 * hb + ((lane & 15) >> 2);
+        const uint32_t vfrag = lds0 + (2 * K_TILE + V_TILE) * 2 + vrl * ROWB +
+                               (((2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) ^ (4 * ((vrl >> RSH) & (PPR / 4 - 1)))) << 4) + 8 * (lane & 1);
+#pragma unroll
+        for (int db = 0; db < DB; db++) vx[db] = vfrag ^ (uint32_t)(db << 6);   // iteration 1 reads tile 0 in buffer 0 after one flip
+        int kflip = K_TILE * 2, vflip = -V_TILE * 2;   // bytes to the other buffer
+        auto flip_buffers = [&]() __attribute__((always_inline)) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) kx[ks] += (uint32_t)kflip;
+#pragma unroll
+            for (int db = 0; db < DB; db++) vx[db] += (uint32_t)vflip;
+            kflip = -kflip, vflip = -vflip;
+        };
+
+        float16_t s[2];
+        half8_t pf[4];
+        // The matrix half of an iteration: the 4 DB fragments of V^T and the MFMAs of P.V (when DO_PV), then the 2 KS
+        // fragments of K and the MFMAs of K.Q^T (when DO_QK).  The LDS reads are written out (with their waits)
+        // because the compiler, which cannot tell the direct loads' LDS writes from the tiles being read, would
+        // wait for every direct load before the first read, and because it keeps only one or two reads in flight:
+        // here fragment i + kDepth is requested before fragment i is used.  LDS reads return in order, so the wait
+        // before fragment i's MFMA allows as many outstanding reads as were issued after its own.
+        auto matrix_half = [&](auto pv_tag, auto qk_tag) __attribute__((always_inline)) {
+            constexpr bool DO_PV = decltype(pv_tag)::value, DO_QK = decltype(qk_tag)::value;
+            constexpr int NV = DO_PV ? 4 * DB : 0, NK = DO_QK ? 2 * KS : 0, NF = NV + NK;
+            constexpr int PD = TROCM_PING_DEPTH < NF ? TROCM_PING_DEPTH : NF;
+            half4_t vlo[DO_PV ? 4 * DB : 1], vhi[DO_PV ? 4 * DB : 1];
+            half8_t kf[DO_QK ? 2 * KS : 1];
+            auto request = [&](auto ic) __attribute__((always_inline)) {
+                (void)vlo, (void)vhi, (void)kf, (void)vx, (void)kx;   // named outside the dependent branches, so that they are captured
+                constexpr int i = decltype(ic)::value;
+                if constexpr (i < NV) {
+                    constexpr int off = 16 * (i / DB) * ROWB;
+                    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(vlo[i]) : "v"(vx[i % DB]), "n"(off));
+                    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(vhi[i]) : "v"(vx[i % DB]), "n"(off + 8 * ROWB));
+                } else {
+                    constexpr int j = i - NV;
+                    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(kf[j]) : "v"(kx[j / 2]), "n"((j % 2) * 32 * ROWB));
+                }
+            };
+            static_for<PD>(request);
+            static_for<NF>([&](auto ic) __attribute__((always_inline)) {
+                (void)vlo, (void)vhi, (void)kf, (void)s, (void)pf, (void)qf, (void)o;
+                constexpr int i = decltype(ic)::value;
+                if constexpr (i + PD < NF) request(std::integral_constant<int, i + PD>{});
+                constexpr int last = i + PD < NF ? i + PD : NF - 1;      // the last fragment requested so far
+                constexpr int behind = (last < NV ? 2 * (last - i) : i < NV ? 2 * (NV - 1 - i) + (last - NV + 1) : last - i);
+                if constexpr (i < NV) {
+                    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(vlo[i]), "+v"(vhi[i]) : "n"(behind));
+                    const half8_t vf = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);
+                    o[i % DB] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[i / DB], o[i % DB], 0, 0, 0);
+                } else {
+                    constexpr int j = i - NV;
+                    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(kf[j]) : "n"(behind));
+                    if constexpr (j < 2) {
+#pragma unroll
+                        for (int r = 0; r < 16; r++) s[j % 2][r] = 0.0f;
+                    }
+                    s[j % 2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[j], qf[j / 2], s[j % 2], 0, 0, 0);
+                }
+            });
+        };
+        // barrier without a fence: a fence would wait for the direct loads in flight (they count as LDS writes)
+        auto half_barrier = []() __attribute__((always_inline)) {
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        };
+
+        if (n_it > 0) issue_k(t_begin, 0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) qf[ks] = *reinterpret_cast<const half8_t *>(qrow + 16 * ks + 8 * hb);
+        loads_landed();
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) asm volatile("" : "+v"(qf[ks]));
+        half_barrier();   // the first K tile is in LDS
+        if (grp == 1) {    // the second group starts half a tile late
+            issue_loads(0);
+            half_barrier();
+        }
+        // Iteration `it`, matrix half: P.V of tile it - 1, then K.Q^T of tile it; vector half: softmax of tile it.
+        // Every wave issues its share of the loads of (K of tile it + 1, V of tile it) at the start of the first
+        // group's matrix half and waits for them before the barrier that ends the second group's: they have two
+        // half-tiles to land.  Every wave takes every tile of the workgroup: a tile that a wave's queries do not see
+        // (or a wave without queries) comes out of the softmax as all zeros.  The first and the last iteration,
+        // which lack one of the two products, are written out on their own, so that no two versions of the
+        // accumulators meet after a branch.
+        auto iteration = [&](int it, auto pv_tag, auto qk_tag) __attribute__((always_inline)) {
+            if (grp == 0) issue_loads(it);
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(TROCM_PING_PRIO_MFMA);
+            matrix_half(pv_tag, qk_tag);
+            __builtin_amdgcn_s_setprio(TROCM_PING_PRIO_VALU);
+            if (grp == 1) loads_landed();
+            half_barrier();
+            if (grp == 1) issue_loads(it + 1);
+            if constexpr (decltype(qk_tag)::value) softmax(t_begin + it, s, pf);
+            flip_buffers();
+            if (grp == 0) loads_landed();
+            half_barrier();
+        };
+        if (n_it > 0) {
+            iteration(0, std::false_type{}, std::true_type{});
+            for (int it = 1; it < n_it; it++) iteration(it, std::true_type{}, std::true_type{});
+            iteration(n_it, std::true_type{}, std::false_type{});
+        }
+        if (grp == 0) half_barrier();   // as many barriers as the second group
     }
     l_run += __shfl_xor(l_run, 32, 64);
     // Output rows of this wave (32 queries of one head: one contiguous block of 32 * D halves).  A lane holds
@@ -397,8 +613,8 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
     };
     auto write_output = [&](float mul) {
         constexpr int FP = D / 2, TROW = FP + 8, CPRW = FP / 8, RPI = 64 / CPRW;   // features per pass, LDS row, 16-byte pieces per row, rows per instruction
-        static_assert(kWavesPP * 32 * TROW <= 2 * kTileN * VROW, "transposition area exceeds the V tile buffers");
-        _Float16 *tr = &lds_v[0][0] + w * (32 * TROW);
+        static_assert(kWavesPP * 32 * TROW == TR_HALVES && (PING || TR_HALVES <= 2 * V_TILE), "transposition area exceeds the V tile buffers");
+        _Float16 *tr = (PING ? &lds_all[WTS_HALVES] : &lds_v[0][0]) + w * (32 * TROW);
         _Float16 *obase = p.out + (((int64_t)b * p.Hq + qh) * p.Sq + q0) * D;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
@@ -486,8 +702,8 @@ __global__ __launch_bounds__(kThreadsPP) void sdpa_prefill_pp_kernel(PrefillPP p
     // two splits in flight at a time.
     constexpr int kMaxSplits = 16;
     auto aload_f = [](const float *a) { return __hip_atomic_load(a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
-    static_assert(kWavesPP * kMaxSplits * 32 * sizeof(float) <= sizeof(lds_k), "merge weights exceed the K tile buffers");
-    float *wts = reinterpret_cast<float *>(&lds_k[0][0]) + w * (kMaxSplits * 32);
+    static_assert(kWavesPP * kMaxSplits * 32 * sizeof(float) == WTS_HALVES * sizeof(_Float16) && WTS_HALVES <= 2 * K_TILE, "merge weights exceed the K tile buffers");
+    float *wts = reinterpret_cast<float *>(&lds_all[0]) + w * (kMaxSplits * 32);
     // One merge step for NS splits starting at s0: their outputs and, when WEIGHTS, the (m, l) records of
     // MAXS splits are requested together; the weights go through LDS (lanes 32..63 need those of lanes 0..31).
     auto load_outputs = [&](int s0, auto &raw, auto ns_tag) {
@@ -666,6 +882,17 @@ __global__ __launch_bounds__(256) void sdpa_prefill_merge_kernel(PrefillPP p) {
     }
 }
 
+int env_int(const char *name, int dflt) {
+    const char *e = getenv(name);
+    return e ? atoi(e) : dflt;
+}
+
+// TROCM_PREFILL_PING=0 keeps the loop that stages tiles through registers for f16 caches as well
+bool ping_enabled() {
+    static const int on = env_int("TROCM_PREFILL_PING", 0);
+    return on != 0;
+}
+
 template <int D, int HG>
 int launch_cfg(const PrefillPP &p, int fmt, int64_t wgs, hipStream_t s) {
     if (fmt == TROCM_Q8_0)
@@ -674,6 +901,8 @@ int launch_cfg(const PrefillPP &p, int fmt, int64_t wgs, hipStream_t s) {
         hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG, false, TROCM_Q4_0>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
     else if (p.mask)
         hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG, true, TROCM_F16>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
+    else if (ping_enabled())
+        hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG, false, TROCM_F16, true>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
     else
         hipLaunchKernelGGL((sdpa_prefill_pp_kernel<D, HG, false, TROCM_F16>), dim3((unsigned)wgs), dim3(kThreadsPP), 0, s, p);
     hipError_t e = hipGetLastError();
@@ -693,11 +922,6 @@ int launch_hg(const PrefillPP &p, int fmt, int hg, int64_t wgs, hipStream_t s) {
         case 2: return launch_cfg<D, 2>(p, fmt, wgs, s);
         default: return launch_cfg<D, 1>(p, fmt, wgs, s);
     }
-}
-
-int env_int(const char *name, int dflt) {
-    const char *e = getenv(name);
-    return e ? atoi(e) : dflt;
 }
 
 }  // namespace
@@ -727,6 +951,7 @@ int launch_sdpa_prefill_pp(const SdpaArgs &a, hipStream_t s) {
     if (a.causal && a.Sk < a.Sq) return 2;  // some queries would see nothing: the generic kernel owns that case
     if (a.Sk >= (1ll << 30) || a.Sq >= (1ll << 30) || a.B >= (1ll << 20)) return 2;
     if ((a.kv_stride_b % 8) || (a.kv_stride_h % 8) || (a.kv_stride_t % 8)) return 2;  // 128-bit row loads
+    if (a.kv_stride_t >= (1ll << 24)) return 2;  // byte offsets within a tile are 32-bit
     if ((uintptr_t)a.q % 16 || (uintptr_t)a.k % 16 || (uintptr_t)a.v % 16 || (uintptr_t)a.out % 16) return 2;
     if (quant) {   // strides arrive in elements of the logical [.., D] rows: whole token rows per head and batch
         if (a.kv_stride_h % a.D || a.kv_stride_b % a.D) return 2;
