@@ -763,6 +763,72 @@ def run_ops(ta, args):
     return line
 
 
+def run_floors(ta, args):
+    """What a short launch costs before any kernel logic: an empty kernel and a read-only streaming kernel
+    (non-temporal 128-bit loads, eight in flight per thread, nothing written) on the decode kernels' launch
+    shapes, over the byte counts of the short decode launches; then those decode launches themselves as a
+    fraction of the streaming kernel's time on the same bytes."""
+    from tract_amd._lib import call
+    res = {}
+    rng = np.random.default_rng(11)
+    sizes = {"33.6MB (f16, batch 1, 8192 tokens)": 2 * 1 * HKV * 8192 * D * 2 + 2 * HQ * D * 2,
+             "37.8MB (Q4_0, batch 8, 4096 tokens)": 2 * 8 * HKV * 4096 * D * 18 // 32 + 2 * 8 * HQ * D * 2,
+             "71.3MB (Q8_0, batch 8, 4096 tokens)": 2 * 8 * HKV * 4096 * D * 34 // 32 + 2 * 8 * HQ * D * 2,
+             "268.6MB (f16, batch 8, 8192 tokens)": 2 * 8 * HKV * 8192 * D * 2 + 2 * 8 * HQ * D * 2}
+    big = max(sizes.values())
+    n_buf = 4   # every launch reads another buffer; short sizes stride through all of them: nothing is found in a cache
+    bufs = [ta.DeviceTensor.from_numpy(rng.integers(0, 255, ((big + 15) // 16 * 16,), dtype=np.uint8)) for _ in range(n_buf)]
+    sink = ta.DeviceTensor((4,), np.uint8)
+    turn = [0]
+    shapes = [(256, 256), (512, 256), (1024, 256), (2048, 256), (512, 512), (256, 1024)]
+    for wg, th in shapes:
+        us = time_calls(ta, lambda: call("trocm_launch_floor", 0, None, 0, wg, th, None, None), 200)
+        res[f"empty_kernel_{wg}x{th}"] = {"us": round(us, 2)}
+    floor = {}
+    for name, nbytes in sizes.items():
+        nb16 = nbytes // 16 * 16
+        per_buf = max(1, big // nb16)   # disjoint windows of one buffer, then the next buffer
+        best = None
+        for wg, th in shapes:
+            def one():
+                i = turn[0]
+                turn[0] += 1
+                b = bufs[(i // per_buf) % n_buf]
+                call("trocm_launch_floor", 1, b.ptr.value + (i % per_buf) * nb16, nb16, wg, th, sink.ptr, None)
+            us = time_calls(ta, one, 100)
+            res[f"stream_read_{name.split(' ')[0]}_{wg}x{th}"] = {"us": round(us, 2), "gbs": round(nb16 / us / 1e3, 1)}
+            best = us if best is None else min(best, us)
+        floor[name] = best
+    del bufs
+    # the decode launches over the same bytes (attention launch only; caches of several layers in turn)
+    def decode_case(B, T, fmt, layers):
+        sts = [ta.InPlaceKvSdpa(axis=2, causal=True, storage_format=fmt).state() for _ in range(layers)]
+        k = seeded_f16(cfg_seed(4, "k") + T + B, (B, HKV, T, D))
+        for st in sts:
+            for c in (st.k, st.v):
+                c.reserve(T + 1024, like=(k.shape, k.dtype))
+                c.push(k)
+        q = ta.DeviceTensor.from_numpy((seeded_f16(cfg_seed(4, "q"), (B, HQ, 1, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16))
+        out = ta.DeviceTensor((B, HQ, 1, D), np.float16)
+
+        def one():
+            sts[turn[0] % layers].attend(q, out=out)
+            turn[0] += 1
+        return time_calls(ta, one, 200)
+    cases = {"33.6MB (f16, batch 1, 8192 tokens)": (1, 8192, None, 10), "37.8MB (Q4_0, batch 8, 4096 tokens)": (8, 4096, ta.Q4_0, 8),
+             "71.3MB (Q8_0, batch 8, 4096 tokens)": (8, 4096, ta.Q8_0, 5), "268.6MB (f16, batch 8, 8192 tokens)": (8, 8192, None, 2)}
+    for name, (B, T, fmt, layers) in cases.items():
+        us = decode_case(B, T, fmt, layers)
+        res[f"decode_{name.split(' ')[0]}"] = {"us": round(us, 2), "gbs": round(sizes[name] / us / 1e3, 1), "best_stream_read_us": round(floor[name], 2),
+                                                "stream_read_time_over_decode_time": round(floor[name] / us, 3)}
+    head = res["decode_33.6MB"]
+    roof = {"bound": "hbm", "kernel": "sdpa_decode_mfma_kernel<128,8,F16,false,true,0> at batch 1", "achieved": head["gbs"], "peak": HBM_PEAK_GBS,
+            "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4), "traffic": None}
+    return base_line(args, "floors: an empty kernel and a read-only streaming kernel on the decode launch shapes over the byte counts "
+                     "of the short decode launches, and those launches beside them (headline: batch-1 decode over 8192 tokens)",
+                     head["gbs"], "GB/s", round(head["us"] / 1e3, 5), "f16", roof, {"cases": res})
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -773,7 +839,7 @@ def main():
     ap.add_argument("--kernel-iters", type=int, default=200)
     ap.add_argument("--windows", type=int, default=5, help="how many times the timed window of --steps steps is taken (median reported)")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "ops", "append", "kivi"],
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "ops", "append", "kivi", "floors"],
                     help="cfg2 (default) is the configuration the metric is quoted on; the others print one line "
                          "of the same shape for the remaining configurations")
     args = ap.parse_args()
@@ -785,7 +851,7 @@ def main():
     import tract_amd as ta
     rt = ta.runtime_for_name("rocm")
     if args.workload != "cfg2":
-        line = {"cfg1": run_cfg1, "cfg3": run_cfg3, "cfg4": run_cfg4, "cfg5": run_cfg5, "ops": run_ops, "append": run_append, "kivi": run_kivi}[args.workload](ta, args)
+        line = {"cfg1": run_cfg1, "cfg3": run_cfg3, "cfg4": run_cfg4, "cfg5": run_cfg5, "ops": run_ops, "append": run_append, "kivi": run_kivi, "floors": run_floors}[args.workload](ta, args)
         line["device"] = rt.device_name
         print(json.dumps(line))
         return

@@ -234,6 +234,14 @@ int trocm_q4_0_matvec(const trocm_q4_weights *weights, const void *act, int act_
 
 /* ---- element-wise neighbours of the cache ------------------------------------------------- */
 
+/* A measurement aid with no counterpart in the reference: the floor under a launch of a given shape.
+ * kind 0 launches a kernel that does nothing; kind 1 a kernel in which `workgroups` workgroups of `threads`
+ * threads read `bytes` bytes at `src` once (non-temporal 128-bit loads) and write nothing (`sink`, 4 bytes of
+ * device memory or NULL, is never written in practice).  Timed between two events on the stream, they say how
+ * much of a short attention launch is the machine's launch and streaming time rather than the kernel's. */
+int trocm_launch_floor(int kind, const void *src, size_t bytes, int workgroups, int threads, void *sink,
+                       void *stream);
+
 /* Cast between F32 and F16 (core `Cast` as the GPU backends run it,
  * cuda/src/kernels/array/cast.rs:21-47, :92): F32 -> F16 rounds to nearest even, F16 -> F32
  * is exact, same type copies.  n_elems dense elements. */

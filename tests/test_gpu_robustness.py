@@ -159,3 +159,21 @@ def test_a_row_masked_out_entirely_with_minus_infinity_yields_zeros(rt, dt, B, H
     keep = np.ones((B, Hq, Sq), bool)
     keep[0, 1, 0] = keep[B - 1, Hq - 1, Sq - 1] = False
     assert max_abs(got[keep], want[keep]) <= (1e-3 if dt == np.float32 else 2e-2)
+
+
+def test_launch_floor_kernels_run_and_refuse_bad_shapes(rt):
+    """The measurement aid: an empty kernel and a read-only streaming kernel on a given launch shape.  They write
+    nothing (the buffer and the 4-byte sink stay as they were) and refuse shapes that are not launches."""
+    src = DeviceTensor.from_numpy(np.arange(1 << 20, dtype=np.uint32))
+    sink = DeviceTensor.from_numpy(np.array([7], dtype=np.uint32))
+    for wg, th in ((1, 64), (256, 256), (2048, 256), (256, 1024)):
+        call("trocm_launch_floor", 0, None, 0, wg, th, None, None)
+        call("trocm_launch_floor", 1, src.ptr, 4 << 20, wg, th, sink.ptr, None)
+    call("trocm_launch_floor", 1, src.ptr, 16 * 1000 + 16, 512, 256, None, None)   # a size that is no multiple of the grid
+    ta.synchronize()
+    assert sink.to_numpy()[0] == 7 and np.array_equal(src.to_numpy(), np.arange(1 << 20, dtype=np.uint32))
+    lib = load()
+    for args in ((2, src.ptr, 16, 1, 64, None, None), (1, None, 16, 1, 64, None, None), (1, src.ptr, 24, 1, 64, None, None),
+                 (0, None, 0, 0, 64, None, None), (0, None, 0, 1, 96, None, None), (0, None, 0, 1, 2048, None, None)):
+        assert lib.trocm_launch_floor(*args) == 1
+        assert b"launch_floor" in lib.trocm_last_error() or b"null pointer" in lib.trocm_last_error()

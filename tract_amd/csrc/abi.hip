@@ -998,6 +998,22 @@ int trocm_block_simulate_precision_loss(int format, const void *src, void *dst, 
     return launch_block_simulate(format, src, dst, dtype, n_elems, s);
 }
 
+// ---- launch floors -----------------------------------------------------------------------------
+int trocm_launch_floor(int kind, const void *src, size_t bytes, int workgroups, int threads, void *sink, void *stream) {
+    if (ensure_init()) return 1;
+    TROCM_REQUIRE(kind == 0 || kind == 1, "launch_floor: kind is 0 (empty kernel) or 1 (streaming read), got %d", kind);
+    TROCM_REQUIRE(workgroups >= 1 && workgroups <= (1 << 20) && threads >= 64 && threads <= 1024 && threads % 64 == 0,
+                  "launch_floor: %d workgroups of %d threads is not a launch shape (1..2^20 workgroups of 64..1024 threads in whole waves)",
+                  workgroups, threads);
+    if (kind == 1) {
+        TROCM_NOT_NULL(src);
+        TROCM_REQUIRE((uintptr_t)src % 16 == 0 && bytes % 16 == 0, "launch_floor: the buffer must be 16-byte aligned and a multiple of 16 bytes");
+    }
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    return launch_floor(kind, src, bytes, workgroups, threads, sink, s);
+}
+
 // ---- element-wise neighbours: cast, RotateHalf, ApplyRope ---------------------------------------
 int trocm_cast(const void *src, int src_dtype, void *dst, int dst_dtype, size_t n_elems, void *stream) {
     TROCM_REQUIRE((src_dtype == TROCM_F32 || src_dtype == TROCM_F16) && (dst_dtype == TROCM_F32 || dst_dtype == TROCM_F16),

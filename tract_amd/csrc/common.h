@@ -74,6 +74,8 @@ struct AppendPair {
     int64_t dst_stride[3];
 };
 int launch_append_pair(const AppendPair &a, hipStream_t s);
+// empty kernel (kind 0) or read-only streaming kernel (kind 1) on a given launch shape
+int launch_floor(int kind, const void *src, size_t bytes, int workgroups, int threads, void *sink, hipStream_t s);
 
 // Quantise [rows, d] (row r of the source at src + b*ss[0] + h*ss[1] + t*ss[2] elements, element
 // stride ss[3]) into the code/scale planes of a cache at token offset t0.

@@ -213,4 +213,42 @@ int launch_copy_nd(void *dst_v, const void *src_v, const CopyNd &in, int elem_si
     }
 }
 
+// ---- launch floors: what a launch of a given shape costs before any kernel logic ---------------------------
+// kind 0: a kernel that does nothing; kind 1: every workgroup reads its contiguous share of `bytes` with
+// non-temporal 128-bit loads, eight in flight per thread, and adds the words up (the sum leaves through `sink`
+// only if it is the impossible value, so the loads cannot be dropped and nothing is written).
+namespace {
+__global__ void floor_null_kernel() {}
+
+__global__ __launch_bounds__(1024) void floor_read_kernel(const cp_u32x4 *__restrict__ src, size_t n_vec, uint32_t *sink) {
+    const size_t per_wg = (n_vec + gridDim.x - 1) / gridDim.x;
+    const size_t begin = per_wg * blockIdx.x, end = begin + per_wg < n_vec ? begin + per_wg : n_vec;
+    uint32_t acc = 0;
+    size_t i = begin + threadIdx.x;
+    for (; i + 7 * (size_t)blockDim.x < end; i += 8 * (size_t)blockDim.x) {
+        cp_u32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = __builtin_nontemporal_load(src + i + j * (size_t)blockDim.x);
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc += v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
+    }
+    for (; i < end; i += blockDim.x) {
+        const cp_u32x4 v = __builtin_nontemporal_load(src + i);
+        acc += v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (acc == 0x9E3779B9u && sink) *sink = acc;
+}
+}  // namespace
+
+int launch_floor(int kind, const void *src, size_t bytes, int workgroups, int threads, void *sink, hipStream_t s) {
+    if (kind == 0)
+        hipLaunchKernelGGL(floor_null_kernel, dim3((unsigned)workgroups), dim3((unsigned)threads), 0, s);
+    else
+        hipLaunchKernelGGL(floor_read_kernel, dim3((unsigned)workgroups), dim3((unsigned)threads), 0, s,
+                           reinterpret_cast<const cp_u32x4 *>(src), bytes / 16, reinterpret_cast<uint32_t *>(sink));
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("launch floor kernel failed: %s", hipGetErrorString(e));
+    return 0;
+}
+
 }  // namespace trocm

@@ -1821,8 +1821,16 @@ int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {
         p.mask_stride_h = a.mask_h > 1 ? a.Sk * 2 : 0;
         p.mask_stride_b = a.mask_b > 1 ? a.mask_h * a.Sk * 2 : 0;
     }
+    // The last workgroup to arrive merges the splits, except in a short launch with many splits per sequence-head
+    // (one or two sequences over up to 16384 tokens: more than kTailMergeMax partial records per head, merged by
+    // one workgroup per kv head): there the merge launch, one workgroup per query head, is the shorter way in
+    // spite of the launch gap (batch 1, 8192 tokens: 13.6 us against 14.9 us; batch 2: 18.0 against 19.0; from
+    // 32768 tokens or 3 sequences on the two are level or the in-kernel merge wins).  TROCM_DECODE_TAIL_MERGE:
+    // 0 = always the launch, 2 = always in the kernel.
     static const int tail = getenv("TROCM_DECODE_TAIL_MERGE") ? atoi(getenv("TROCM_DECODE_TAIL_MERGE")) : 1;
-    if (tail && gp <= 8 && nsplit > 1 && nsplit <= kWideMergeMax && BH <= (int64_t)(kWsCounterBytes / sizeof(int))) p.counters = (int *)a.workspace;
+    const bool short_and_wide = nsplit > kTailMergeMax && a.B <= 2 && a.Sk <= 16384;
+    if (tail && (tail == 2 || !short_and_wide) && gp <= 8 && nsplit > 1 && nsplit <= kWideMergeMax && BH <= (int64_t)(kWsCounterBytes / sizeof(int)))
+        p.counters = (int *)a.workspace;
     dim3 grid(nsplit, (unsigned)a.Hkv, (unsigned)a.B);
     return a.D == 128 ? launch_d<128>(p, gp, grid, s) : launch_d<64>(p, gp, grid, s);
 }
