@@ -234,6 +234,13 @@ int trocm_q4_0_matvec(const trocm_q4_weights *weights, const void *act, int act_
 
 /* ---- element-wise neighbours of the cache ------------------------------------------------- */
 
+/* Planes that a growing cache or store has left behind are released behind an event by a later call of the library
+ * (growth of a pooled cache, trocm_stream_sync, trocm_device_sync, a destroy, an allocation that fails at first).
+ * A host that synchronises with its own HIP calls and never meets one of those can release them here: what the
+ * device has finished with (wait == 0, never blocks on the stream) or everything (wait != 0).  No counterpart in
+ * the reference, whose caches are freed by Rust's ownership (gpu/src/ops/dyn_kv_cache.rs:58-113). */
+int trocm_release_unused(int wait);
+
 /* A measurement aid with no counterpart in the reference: the floor under a launch of a given shape.
  * kind 0 launches a kernel that does nothing; kind 1 a kernel in which `workgroups` workgroups of `threads`
  * threads read `bytes` bytes at `src` once (non-temporal 128-bit loads) and write nothing (`sink`, 4 bytes of
@@ -309,8 +316,10 @@ int trocm_sdpa_cached(const void *q, int q_dtype, int64_t q_heads, int64_t q_len
                       const trocm_kv_cache *k_cache, const trocm_kv_cache *v_cache, void *out,
                       float scale, int causal, void *workspace, size_t workspace_bytes, void *stream);
 
-/* trocm_sdpa_cached for callers that cannot allocate device memory: code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same
+/* trocm_sdpa_cached for callers that cannot allocate device memory: tight serving loops, harnesses
+ * that forbid hipMalloc.  (Recording it into a HIP graph is not tested, and of limited use: like every
+ * attention entry point it passes the cache length to its kernels as an argument, so a replayed launch
+ * would attend over the length it was recorded with.)  No counterpart in the reference.  Same
  * arguments, result and kernels as trocm_sdpa_cached, but the split-K scratch is a static device
  * array of TROCM_STATIC_SCRATCH_BYTES inside the library (held on the library's device until the
  * process ends) and the call reaches no hipMalloc, hipFree or other allocating routine.

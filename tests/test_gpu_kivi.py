@@ -1,6 +1,8 @@
 """KIVI-style quantised caches on the GPU against the oracle (oracle/kivi_oracle.c): stored codes, parameters,
 sink and partial-block rows and the dequantised cache bit-exact; the fused QuantizedKvSdpa within the path's
 attention tolerance (1e-3 in f32, 2e-2 in f16).  The reference's own unit tests are replayed on the device ops."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -333,3 +335,146 @@ def test_running_key_store_prompt_push_equals_token_by_token(rt):
         assert got["packed"].tobytes() == want["packed"].tobytes(), n
         assert got["lo"].tobytes() == want["lo"].tobytes() and got["scale"].tobytes() == want["scale"].tobytes(), n
     assert cache.dequantize(np.float32).to_numpy().tobytes() == ref.dequantized().tobytes()
+
+
+@pytest.mark.parametrize("D,dt", [(128, np.float16), (128, np.float32), (64, np.float16), (256, np.float32)])
+def test_running_key_store_prompt_push_with_128_bit_rows(rt, D, dt):
+    """Head sizes 64 / 128 / 256 take the chunk passes in which a lane owns 8 channels and rows move as 128-bit words:
+    the same codes and parameters as the token-by-token push, over several prompts, on top of earlier state, with a
+    ragged last chunk, NaN, infinities, signed zeros and a minimum / range that keep moving."""
+    rng = np.random.default_rng(D)
+    B, H = 2, 3
+    cache = kivi.KiviCache(kivi.KIVI_RUNNING_CHANNEL, 8, 0, B, H, D)
+    refs = {(b, h): orc.KiviCache(True, running=True) for b in range(B) for h in (0, H - 1)}
+    for n, mag in ((3, 1.0), (700, 1.0), (1, 1.0), (257, 4.0), (1024, 0.2)):
+        x = (rng.standard_normal((B, H, n, D)) * mag).astype(dt)
+        x[0, 0, n // 2, 3] = np.nan
+        x[1, H - 1, n // 3, D - 1] = 0.0
+        x[1, H - 1, n // 3 + 1 if n > 1 else 0, D - 1] = -0.0
+        if n > 600:
+            x[0, H - 1, 600, 7] = np.inf
+            x[0, H - 1, 100:200, 9] = np.linspace(5, -50, 100).astype(dt)
+            x[0, H - 1, 200:, 9] = np.linspace(-50, 400, n - 200).astype(dt)
+        cache.append(x)
+        got = cache.state()
+        for (b, h), ref in refs.items():
+            ref.ingest(x[b:b + 1, h:h + 1].astype(np.float32))
+            want, i = ref.state(), b * H + h
+            assert got["packed"][i:i + 1].tobytes() == want["packed"].tobytes(), (n, b, h)
+            assert got["lo"][i:i + 1].tobytes() == want["lo"].tobytes() and got["scale"][i:i + 1].tobytes() == want["scale"].tobytes(), (n, b, h)
+
+
+def test_growing_stores_then_attention_without_a_host_sync(rt):
+    """A prompt into the running Key store and the per-token Value store, then decode steps that grow both stores,
+    all queued behind other work on one stream: no call waits for the stream (growth and the prompt's scratch
+    release their old memory behind events), and the state is what the synchronous order gives."""
+    import time
+    from tract_amd.runtime import Stream
+    B, Hq, Hkv, D, T = 1, 8, 2, 128, 300
+    rng = np.random.default_rng(12)
+    k = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((B, Hkv, T, D), dtype=np.float32).astype(np.float16)
+    steps = [(rng.standard_normal((B, Hq, 1, D), dtype=np.float32).astype(np.float16) * np.float16(0.1),
+              rng.standard_normal((B, Hkv, 1, D), dtype=np.float32).astype(np.float16),
+              rng.standard_normal((B, Hkv, 1, D), dtype=np.float32).astype(np.float16)) for _ in range(40)]
+    stream = Stream()
+    ref_state = kivi.QuantizedKvSdpa(axis=2).state()
+    qp = rng.standard_normal((B, Hq, T, D), dtype=np.float32).astype(np.float16) * np.float16(0.1)
+    want = [ref_state.eval([qp, k, v]).to_numpy()] + [ref_state.eval(list(s)).to_numpy() for s in steps]
+    tract_amd.synchronize()
+    st = kivi.QuantizedKvSdpa(axis=2).state()
+    from tract_amd.runtime import Workspace
+    st._ws = Workspace(B, Hq, T, D, stream)   # (the host mirror synchronises when it makes a workspace: made ahead of the queue)
+    dev = [tract_amd.DeviceTensor.from_numpy(a, stream) for a in (qp, k, v)]
+    dsteps = [[tract_amd.DeviceTensor.from_numpy(a, stream) for a in s] for s in steps]
+    big = tract_amd.DeviceTensor((1 << 30,), np.uint8)   # 1 GiB, one half copied onto the other many times: ~60 ms of queued work
+    half = 1 << 29
+    shape, st1 = (C.c_int64 * 1)(half // 16), (C.c_int64 * 1)(1)
+    stream.synchronize()
+    from tract_amd._lib import call
+    for _ in range(300):
+        call("trocm_copy_nd", big.ptr, half, st1, big.ptr, 0, st1, shape, 1, 16, stream.handle)
+    t0 = time.perf_counter()
+    got = [st.eval(dev, stream=stream)] + [st.eval(s, stream=stream) for s in dsteps]   # 300 + 40 tokens: both stores double several times
+    queued = time.perf_counter() - t0
+    stream.synchronize()
+    total = time.perf_counter() - t0
+    assert queued < 0.5 * total, (queued, total)   # the calls returned while the stream was still busy
+    for g, w in zip(got, want):
+        assert g.to_numpy().tobytes() == w.tobytes()
+    a, b = st.k.state(), ref_state.k.state()
+    assert all(a[n].tobytes() == b[n].tobytes() for n in a)
+
+
+def test_a_refused_append_changes_nothing_and_can_be_repeated(rt):
+    """An append that cannot get its memory (more than the device has) fails before anything is counted: length, sink
+    and row counts stay, and the next append works.  The same for a QuantizedKvSdpa step: K and V stay level."""
+    import ctypes as C2
+    from tract_amd._lib import load
+    lib = load()
+    B, H, D = 8, 512, 512                       # 4096 (batch, head) rows of 512 channels
+    hbm = C2.c_size_t()
+    assert lib.trocm_device_info(None, C2.byref(hbm), None, 0) == 0
+    n_huge = (1 << 31) // D - 64                # the index range's limit: 4096 x 4 Mi x 512 bytes of codes = 8.8 TB
+    assert B * H * n_huge * D > 4 * hbm.value
+    for layout, bits, sink in ((kivi.KIVI_PER_TOKEN, 8, 4), (kivi.KIVI_BLOCK_CHANNEL, 4, 4), (kivi.KIVI_RUNNING_CHANNEL, 8, 0)):
+        cache = kivi.KiviCache(layout, bits, sink, B, H, D)
+        x = np.random.default_rng(1).standard_normal((B, H, 2, D)).astype(np.float32)
+        cache.append(x)
+        before = (cache.len(), cache.counts())
+        small = tract_amd.DeviceTensor.from_numpy(x)   # never read: the call fails while it allocates
+        assert lib.trocm_kivi_cache_append(cache.handle, small.ptr, 0, n_huge, None) == 1
+        assert b"failed" in lib.trocm_last_error() or b"hipMalloc" in lib.trocm_last_error() or b"memory" in lib.trocm_last_error()
+        assert (cache.len(), cache.counts()) == before
+        cache.append(x)
+        assert cache.len() == 4
+    kc = kivi.KiviCache(kivi.KIVI_RUNNING_CHANNEL, 8, 0, B, H, D)
+    vc = kivi.KiviCache(kivi.KIVI_PER_TOKEN, 8, 0, B, H, D)
+    q = tract_amd.DeviceTensor.from_numpy(np.zeros((B, H, 1, D), np.float32))
+    out = tract_amd.DeviceTensor((B, H, 1, D), np.float32)
+    kn = tract_amd.DeviceTensor.from_numpy(np.ones((B, H, 1, D), np.float32))
+    nan = C2.c_float(float("nan"))
+    assert lib.trocm_quantized_kv_sdpa_eval(q.ptr, kn.ptr, kn.ptr, 0, H, 1, kc.handle, vc.handle, out.ptr, nan, None, 0, None) == 0
+    assert lib.trocm_quantized_kv_sdpa_eval(q.ptr, kn.ptr, kn.ptr, 0, H, n_huge, kc.handle, vc.handle, out.ptr, nan, None, 0, None) == 1
+    assert kc.len() == 1 and vc.len() == 1 and kc.counts() == {**kc.counts(), "n_rows": 1} and vc.counts()["n_rows"] == 1
+    assert lib.trocm_quantized_kv_sdpa_eval(q.ptr, kn.ptr, kn.ptr, 0, H, 1, kc.handle, vc.handle, out.ptr, nan, None, 0, None) == 0
+    assert kc.len() == 2 and vc.len() == 2
+
+
+@pytest.mark.parametrize("k_mag,v_mag", [(1.0, 1e-3), (1.0, 1e-5), (1e-3, 1.0), (1e-3, 1e-4), (30.0, 200.0)])
+def test_quantized_kv_sdpa_over_the_codes_with_small_and_large_magnitudes(rt, k_mag, v_mag):
+    """Keys and Values far from unit magnitude: their scales (range / 255) fall below the smallest normal half, or grow
+    large.  The products q * s_k and P * s_v that the matrix cores take as halves are first brought into range by a
+    power of two, so the output keeps the accuracy it has at unit magnitude, relative to its own size.  Some tokens are
+    20x larger than the rest, and come late, so that the running factor of the Values has to move."""
+    rng = np.random.default_rng(5)
+    B, Hq, Hkv, D, T0 = 2, 8, 2, 128, 1000
+    g = Hq // Hkv
+    st = tract_amd.QuantizedKvSdpa(axis=2, scale=None).state()
+    k0 = (rng.standard_normal((B, Hkv, T0, D)) * k_mag).astype(np.float16)
+    v0 = (rng.standard_normal((B, Hkv, T0, D)) * v_mag).astype(np.float32)
+    v0[:, :, 700::50] *= 20.0
+    v0 = v0.astype(np.float16)
+    q_mag = 1.0 / (np.sqrt(D) * k_mag)    # logits of unit size whatever the keys' magnitude
+    q0 = (rng.standard_normal((B, Hq, T0, D)) * q_mag).astype(np.float16)
+    st.eval([q0, k0, v0])
+    refs = {}
+    for (b, h) in ((0, 0), (1, 1)):
+        kc, vc = orc.KiviCache(True, running=True), orc.KiviCache(False, running=True)
+        kc.ingest(k0[b:b + 1, h:h + 1])
+        vc.ingest(v0[b:b + 1, h:h + 1])
+        refs[(b, h)] = (kc, vc)
+    for step in range(3):
+        q = (rng.standard_normal((B, Hq, 1, D)) * q_mag).astype(np.float16)
+        k = (rng.standard_normal((B, Hkv, 1, D)) * k_mag).astype(np.float16)
+        v = (rng.standard_normal((B, Hkv, 1, D)) * v_mag).astype(np.float16)
+        got = st.eval([q, k, v]).to_numpy().astype(np.float64)
+        for (b, h), (kc, vc) in refs.items():
+            kc.ingest(k[b:b + 1, h:h + 1])
+            vc.ingest(v[b:b + 1, h:h + 1])
+            want = orc.flash_sdpa(q[b:b + 1, h * g:(h + 1) * g].astype(np.float32), kc.dequantized(), vc.dequantized(), causal=False).astype(np.float64)
+            size = float(np.abs(want).max())
+            err = float(np.abs(got[b:b + 1, h * g:(h + 1) * g] - want).max())
+            # 8e-3 is what f16 outputs and f16 probabilities leave at unit magnitude; outputs below the halves'
+            # normal range (6e-5) are also limited by the output type's own subnormal step (6e-8)
+            assert err <= 8e-3 * size + 6e-8, (step, b, h, err, size)

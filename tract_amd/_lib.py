@@ -73,6 +73,7 @@ SIGNATURES = {
     "trocm_q4_0_weights_shape": [_vp, _pi64, _pi64, _pi64],
     "trocm_q4_0_weights_export": [_vp, _vp, _vp],
     "trocm_q4_0_matvec": [_vp, _vp, _i, _i64, _i64, _vp, _vp],
+    "trocm_release_unused": [_i],
     "trocm_launch_floor": [_i, _vp, _sz, _i, _i, _vp, _vp],
     "trocm_cast": [_vp, _i, _vp, _i, _sz, _vp],
     "trocm_apply_rope": [_vp, _vp, _vp, _vp, _i, _i, _pi64, _pi64, _pi64, _pi64, _vp],

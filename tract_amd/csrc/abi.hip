@@ -165,25 +165,33 @@ static void release_planes(trocm_kv_pool *pool, void *data, void *scales) {
 
 // Release the deferred planes whose event has completed; with `wait`, all of them (of `only_pool`, if given).
 // hipFree waits for the whole device, so planes outside a pool are released only where the host is waiting anyway
-// (`unpooled`: the synchronising calls, destroy, a failed allocation); a pool's bookkeeping costs nothing.
+// (`unpooled`: the synchronising calls, destroy, a failed allocation, trocm_release_unused); a pool's bookkeeping
+// costs nothing.  The list's lock is not held while an event is waited for.
 static void reap_deferred(bool wait, trocm_kv_pool *only_pool = nullptr, bool unpooled = true) {
-    std::vector<DeferredFree> ready;
+    std::vector<DeferredFree> mine, ready;
     {
         std::lock_guard<std::mutex> lock(g_deferred_mu);
         for (size_t i = 0; i < g_deferred.size();) {
-            DeferredFree &d = g_deferred[i];
-            const bool mine = (only_pool == nullptr || d.pool == only_pool) && (unpooled || d.pool != nullptr);
-            bool done = mine && hipEventQuery(d.done) == hipSuccess;
-            if (mine && !done && wait) done = hipEventSynchronize(d.done) == hipSuccess;
-            if (done) {
-                ready.push_back(d);
+            const DeferredFree &d = g_deferred[i];
+            if ((only_pool == nullptr || d.pool == only_pool) && (unpooled || d.pool != nullptr)) {
+                mine.push_back(d);
                 g_deferred[i] = g_deferred.back();
                 g_deferred.pop_back();
             } else {
                 i++;
             }
         }
-        (void)hipGetLastError();   // "not ready" is an answer, not a failure: keep it away from the launch checks
+    }
+    std::vector<DeferredFree> pending;
+    for (DeferredFree &d : mine) {
+        bool done = hipEventQuery(d.done) == hipSuccess;
+        if (!done && wait) done = hipEventSynchronize(d.done) == hipSuccess;
+        (done ? ready : pending).push_back(d);
+    }
+    (void)hipGetLastError();   // "not ready" is an answer, not a failure: keep it away from the launch checks
+    if (!pending.empty()) {
+        std::lock_guard<std::mutex> lock(g_deferred_mu);
+        g_deferred.insert(g_deferred.end(), pending.begin(), pending.end());
     }
     for (DeferredFree &d : ready) {
         (void)hipEventDestroy(d.done);
@@ -207,6 +215,13 @@ static int defer_free(trocm_kv_pool *pool, void *data, void *scales, hipStream_t
     g_deferred.push_back(d);
     return 0;
 }
+
+// The same service for the other stateful objects of the library (the affine-quantised stores): device memory that
+// work queued on `s` may still read is released by a later call, not by waiting for the stream here.
+namespace trocm {
+int defer_device_free(void *a, void *b, hipStream_t s) { return defer_free(nullptr, a, b, s); }
+void reap_device_frees(bool wait) { reap_deferred(wait); }
+}  // namespace trocm
 
 static int plane_alloc(trocm_kv_cache *c, void **ptr, size_t bytes, const char *what) {
     if (c->pool) {
@@ -996,6 +1011,12 @@ int trocm_block_simulate_precision_loss(int format, const void *src, void *dst, 
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
     return launch_block_simulate(format, src, dst, dtype, n_elems, s);
+}
+
+int trocm_release_unused(int wait) {
+    if (ensure_init()) return 1;
+    reap_deferred(wait != 0);
+    return 0;
 }
 
 // ---- launch floors -----------------------------------------------------------------------------

@@ -74,6 +74,10 @@ struct AppendPair {
     int64_t dst_stride[3];
 };
 int launch_append_pair(const AppendPair &a, hipStream_t s);
+// Device memory that work queued on `s` may still read: released by a later call, once an event recorded on `s` now has
+// completed (abi.hip).  reap_device_frees(wait) releases what has completed (wait: everything).
+int defer_device_free(void *a, void *b, hipStream_t s);
+void reap_device_frees(bool wait);
 // empty kernel (kind 0) or read-only streaming kernel (kind 1) on a given launch shape
 int launch_floor(int kind, const void *src, size_t bytes, int workgroups, int threads, void *sink, hipStream_t s);
 

@@ -383,6 +383,57 @@ __device__ __forceinline__ void store_codes8(uint8_t *row, int sub, const uint32
     }
 }
 
+// The three chunk passes of the running Key store for head sizes 64 / 128 / 256 / 512 and 16-byte aligned sources: a lane
+// owns 8 consecutive channels of one chunk and walks the chunk's tokens with 128-bit loads; LPR = D / 8 lanes cover a row,
+// 256 / LPR chunks share a workgroup.  PASS 1: first minimal value per chunk and channel into `a`; PASS 2: largest scale
+// candidate into `b`, starting from the chunk's lo in `a`; PASS 3: the codes, starting from the parameters in `a`, `b`.
+// Arithmetic, order and tie-breaking are those of kivi_run_chunk_{min,scale,codes}_kernel.
+template <typename SrcT, int LPR, int PASS>
+__global__ void __launch_bounds__(256) kivi_run_chunk_vec_kernel(const SrcT *__restrict__ src, int64_t S, int n, int n_chunks,
+                                                                 float *__restrict__ a, float *__restrict__ b,
+                                                                 uint8_t *__restrict__ codes, int64_t cap_rows, int64_t row0) {
+    constexpr int D = LPR * 8, CPW = 256 / LPR;
+    const int bh = blockIdx.y, k = blockIdx.x * CPW + (int)threadIdx.x / LPR, sub = (int)threadIdx.x % LPR;
+    if (k >= n_chunks) return;
+    const int64_t at = ((int64_t)bh * n_chunks + k) * D + sub * 8;
+    const int t0 = k * kRunChunk, t1 = min(n, t0 + kRunChunk);
+    const SrcT *row = src + ((int64_t)bh * S + t0) * D + sub * 8;
+    F8 lo, sc;
+    if (PASS == 1) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) lo.v[e] = INFINITY;
+    } else {
+        lo = ld8(a + at);
+    }
+    if (PASS == 2) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) sc.v[e] = 0.0f;
+    } else if (PASS == 3) {
+        sc = ld8(b + at);
+    }
+#pragma unroll 4
+    for (int t = t0; t < t1; t++, row += D) {
+        const F8 x = ld8(row);
+        uint32_t code[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float val = x.v[e];
+            if (val < lo.v[e]) lo.v[e] = val;
+            if (PASS >= 2) {
+                const float range = __fsub_rn(val, lo.v[e]);
+                if (range > 0.0f) {
+                    const float ns = __fdiv_rn(range, 255.0f);
+                    if (ns > sc.v[e]) sc.v[e] = ns;
+                }
+            }
+            if (PASS == 3) code[e] = affine_code(val, lo.v[e], sc.v[e], 255.0f);
+        }
+        if (PASS == 3) store_codes8<8>(codes + ((int64_t)bh * cap_rows + row0 + t) * D, sub, code);
+    }
+    if (PASS == 1) st8(a + at, lo);
+    if (PASS == 2) st8(b + at, sc);
+}
+
 // Values: LPR = D / 8 lanes per token, 64 / LPR tokens per wave.
 template <typename SrcT, int BITS, int LPR>
 __global__ void __launch_bounds__(256) kivi_quant_tokens_vec_kernel(const SrcT *__restrict__ src, int64_t S, int64_t src_t0, int n,
@@ -630,6 +681,8 @@ struct trocm_kivi_cache {
     uint8_t *codes = nullptr;
     void *deq = nullptr;      // dequantised copy handed to attention by trocm_quantized_kv_sdpa_eval
     size_t deq_bytes = 0;
+    float *scan = nullptr;    // chunk results of a prompt pushed into the running Key store (kept for the next prompt)
+    size_t scan_bytes = 0;
 };
 
 static int64_t param_pitch(const trocm_kivi_cache *c, int64_t cap_rows) {
@@ -661,14 +714,38 @@ static int copy_rows(void *dst, int64_t dpitch, const void *src, int64_t spitch,
     return launch_copy_nd(dst, src, d, 1, s);
 }
 
+// hipMalloc that first gives memory waiting for its event a chance, and leaves no stale error behind when it fails (the
+// next launch check would report it).
+static int kivi_malloc(void **ptr, size_t bytes, const char *what) {
+    *ptr = nullptr;
+    hipError_t e = hipMalloc(ptr, bytes ? bytes : 16);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        reap_device_frees(true);
+        e = hipMalloc(ptr, bytes ? bytes : 16);
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        *ptr = nullptr;
+        return fail("allocating %s (%zu bytes) failed: %s", what, bytes, hipGetErrorString(e));
+    }
+    return 0;
+}
+
 static int kivi_alloc_fixed(trocm_kivi_cache *c, hipStream_t s) {
-    if (c->sink_tokens && !c->sink) TROCM_HIP(hipMalloc((void **)&c->sink, (size_t)c->BH * c->sink_tokens * c->D * 4));
-    if (c->layout == TROCM_KIVI_BLOCK_CHANNEL && !c->residual)
-        TROCM_HIP(hipMalloc((void **)&c->residual, (size_t)c->BH * kKeyBlock * c->D * 4));
+    if (c->sink_tokens && !c->sink && kivi_malloc((void **)&c->sink, (size_t)c->BH * c->sink_tokens * c->D * 4, "the unquantised first tokens")) return 1;
+    if (c->layout == TROCM_KIVI_BLOCK_CHANNEL && !c->residual &&
+        kivi_malloc((void **)&c->residual, (size_t)c->BH * kKeyBlock * c->D * 4, "the partial key block"))
+        return 1;
     if (c->layout == TROCM_KIVI_RUNNING_CHANNEL && !c->lo) {
         const int64_t n = c->BH * c->D;
-        TROCM_HIP(hipMalloc((void **)&c->lo, (size_t)n * 4));
-        TROCM_HIP(hipMalloc((void **)&c->scale, (size_t)n * 4));
+        float *lo = nullptr, *scale = nullptr;
+        if (kivi_malloc((void **)&lo, (size_t)n * 4, "running key parameters")) return 1;
+        if (kivi_malloc((void **)&scale, (size_t)n * 4, "running key parameters")) {
+            (void)hipFree(lo);
+            return 1;
+        }
+        c->lo = lo, c->scale = scale;
         kivi_fill_running_kernel<<<dim3((unsigned)((n + 255) / 256)), 256, 0, s>>>(c->lo, c->scale, n);
         TROCM_HIP(hipGetLastError());
     }
@@ -676,21 +753,21 @@ static int kivi_alloc_fixed(trocm_kivi_cache *c, hipStream_t s) {
 }
 
 // Room for `need` coded rows: capacities are multiples of 32 and at least double.  The valid region moves on the
-// stream; the old planes are freed after the stream has drained (the CPU op is synchronous as well).
+// stream; the old planes are released behind an event by a later call (the host does not wait for the stream).
 static int kivi_ensure_rows(trocm_kivi_cache *c, int64_t need, hipStream_t s) {
     if (need <= c->cap_rows) return 0;
     int64_t cap = c->cap_rows * 2 > need ? c->cap_rows * 2 : need;
     cap = (cap + kKeyBlock - 1) / kKeyBlock * kKeyBlock;
     uint8_t *codes = nullptr;
     float *lo = nullptr, *scale = nullptr;
-    TROCM_HIP(hipMalloc((void **)&codes, (size_t)c->BH * cap * c->row_bytes));
+    if (kivi_malloc((void **)&codes, (size_t)c->BH * cap * c->row_bytes, "the codes of a quantised store")) return 1;
     const bool own_params = c->layout != TROCM_KIVI_RUNNING_CHANNEL;
     if (own_params) {
-        if (hipMalloc((void **)&lo, (size_t)c->BH * param_pitch(c, cap) * 4) != hipSuccess ||
-            hipMalloc((void **)&scale, (size_t)c->BH * param_pitch(c, cap) * 4) != hipSuccess) {
+        if (kivi_malloc((void **)&lo, (size_t)c->BH * param_pitch(c, cap) * 4, "the parameters of a quantised store") ||
+            kivi_malloc((void **)&scale, (size_t)c->BH * param_pitch(c, cap) * 4, "the parameters of a quantised store")) {
             (void)hipFree(codes);
             if (lo) (void)hipFree(lo);
-            return fail("hipMalloc failed for the parameters of a quantised cache of %lld rows", (long long)cap);
+            return 1;
         }
     }
     int rc = 0;
@@ -707,13 +784,9 @@ static int kivi_ensure_rows(trocm_kivi_cache *c, int64_t need, hipStream_t s) {
         if (scale) (void)hipFree(scale);
         return rc;
     }
-    if (c->codes) {
-        TROCM_HIP(hipStreamSynchronize(s));
-        (void)hipFree(c->codes);
-        if (own_params) {
-            (void)hipFree(c->lo);
-            (void)hipFree(c->scale);
-        }
+    if (c->codes) {   // the copies above (and whatever the stream still runs over the old planes) finish first
+        if (defer_device_free(c->codes, nullptr, s)) return 1;
+        if (own_params && defer_device_free(c->lo, c->scale, s)) return 1;
     }
     c->codes = codes;
     if (own_params) {
@@ -724,11 +797,44 @@ static int kivi_ensure_rows(trocm_kivi_cache *c, int64_t need, hipStream_t s) {
     return 0;
 }
 
+// A scratch buffer that only grows (by doubling); the one it replaces is released behind an event.
+static int kivi_grow_buffer(void **buf, size_t *have, size_t need, hipStream_t s, const char *what) {
+    if (*have >= need) return 0;
+    const size_t cap = *have * 2 > need ? *have * 2 : need;
+    void *fresh = nullptr;
+    if (kivi_malloc(&fresh, cap, what)) return 1;
+    if (*buf && defer_device_free(*buf, nullptr, s)) return 1;
+    *buf = fresh;
+    *have = cap;
+    return 0;
+}
+
+static bool kivi_prompt_scan(const trocm_kivi_cache *c, int64_t rem) {
+    return c->layout == TROCM_KIVI_RUNNING_CHANNEL && rem >= 4 * kRunChunk && (rem + kRunChunk - 1) / kRunChunk <= 65535;
+}
+
+// Everything an append of S tokens may have to allocate, before anything is launched or counted: a call that fails here
+// has changed nothing and can be repeated.
+static int kivi_prepare(trocm_kivi_cache *c, int64_t S, hipStream_t s) {
+    if (kivi_alloc_fixed(c, s)) return 1;
+    const int64_t ns = c->sink_tokens - c->n_sink < S ? c->sink_tokens - c->n_sink : S;
+    const int64_t rem = S - (ns > 0 ? ns : 0);
+    if (rem <= 0) return 0;
+    int64_t rows = c->n_rows + rem;
+    if (c->layout == TROCM_KIVI_BLOCK_CHANNEL) rows = c->n_rows + (c->n_res + rem) / kKeyBlock * kKeyBlock;
+    if (rows > c->n_rows && kivi_ensure_rows(c, rows, s)) return 1;
+    if (kivi_prompt_scan(c, rem)) {
+        const size_t need = (size_t)c->BH * ((rem + kRunChunk - 1) / kRunChunk) * c->D * 2 * sizeof(float);
+        if (kivi_grow_buffer((void **)&c->scan, &c->scan_bytes, need, s, "the chunk results of a prompt")) return 1;
+    }
+    return 0;
+}
+
 template <typename SrcT>
 static int kivi_append_t(trocm_kivi_cache *c, const SrcT *src, int64_t S, hipStream_t s) {
     const int D = (int)c->D;
     const unsigned BH = (unsigned)c->BH;
-    if (kivi_alloc_fixed(c, s)) return 1;
+    if (kivi_prepare(c, S, s)) return 1;   // every allocation of this call: nothing below can run out of memory
     int64_t t0 = 0;
     const int64_t ns = c->sink_tokens - c->n_sink < S ? c->sink_tokens - c->n_sink : S;
     if (ns > 0) {   // quant_dyn_kv_cache.rs:118-122, :170-174
@@ -739,7 +845,6 @@ static int kivi_append_t(trocm_kivi_cache *c, const SrcT *src, int64_t S, hipStr
     }
     const int64_t rem = S - t0;
     if (rem > 0 && c->layout == TROCM_KIVI_PER_TOKEN) {
-        if (kivi_ensure_rows(c, c->n_rows + rem, s)) return 1;
         const bool vec = ((uintptr_t)src & 15) == 0 && (D == 64 || D == 128 || D == 256 || D == 512);
 #define KIVI_TOKENS_VEC(BITS, LPR)                                                                                              \
     kivi_quant_tokens_vec_kernel<SrcT, BITS, LPR><<<dim3((unsigned)((rem + 4 * (64 / LPR) - 1) / (4 * (64 / LPR))), BH), 256, 0, s>>>( \
@@ -761,7 +866,6 @@ static int kivi_append_t(trocm_kivi_cache *c, const SrcT *src, int64_t S, hipStr
     } else if (rem > 0 && c->layout == TROCM_KIVI_BLOCK_CHANNEL) {
         const int64_t nb = (c->n_res + rem) / kKeyBlock;
         if (nb > 0) {
-            if (kivi_ensure_rows(c, c->n_rows + nb * kKeyBlock, s)) return 1;
             const bool vec = ((uintptr_t)src & 15) == 0 && (D == 64 || D == 128 || D == 256 || D == 512);
 #define KIVI_BLOCKS_VEC(BITS, LPR)                                                                               \
     kivi_finalize_blocks_vec_kernel<SrcT, BITS, LPR><<<dim3((unsigned)((nb + 3) / 4), BH), 256, 0, s>>>(         \
@@ -793,23 +897,34 @@ static int kivi_append_t(trocm_kivi_cache *c, const SrcT *src, int64_t S, hipStr
             c->n_res += rem;
         }
     } else if (rem > 0) {
-        if (kivi_ensure_rows(c, c->n_rows + rem, s)) return 1;
         const int64_t n_chunks = (rem + kRunChunk - 1) / kRunChunk;
-        if (rem >= 4 * kRunChunk && n_chunks <= 65535) {   // a prompt: chunks side by side (scratch: two floats per chunk and channel)
-            float *tmp = nullptr;
+        if (kivi_prompt_scan(c, rem)) {   // a prompt: chunks side by side (scratch: two floats per chunk and channel)
+            float *tmp = c->scan;
             const size_t plane = (size_t)c->BH * n_chunks * D;
-            TROCM_HIP(hipMalloc((void **)&tmp, plane * 2 * sizeof(float)));
-            const dim3 grid((unsigned)((D + 63) / 64), (unsigned)n_chunks, BH), scan((unsigned)((D + 63) / 64), BH);
-            kivi_run_chunk_min_kernel<SrcT><<<grid, 64, 0, s>>>(src + t0 * D, S, (int)rem, D, (int)n_chunks, tmp);
-            kivi_run_scan_min_kernel<<<scan, 64, 0, s>>>(tmp, D, (int)n_chunks, c->lo);
-            kivi_run_chunk_scale_kernel<SrcT><<<grid, 64, 0, s>>>(src + t0 * D, S, (int)rem, D, (int)n_chunks, tmp, tmp + plane);
-            kivi_run_scan_scale_kernel<<<scan, 64, 0, s>>>(tmp + plane, D, (int)n_chunks, c->scale);
-            kivi_run_chunk_codes_kernel<SrcT><<<grid, 64, 0, s>>>(src + t0 * D, S, (int)rem, D, (int)n_chunks, tmp, tmp + plane, c->codes, c->cap_rows, c->n_rows);
-            const hipError_t launched = hipGetLastError();
-            const hipError_t drained = hipStreamSynchronize(s);   // the scratch is freed here, so the stream drains first
-            (void)hipFree(tmp);
-            TROCM_HIP(launched);
-            TROCM_HIP(drained);
+            const SrcT *from = src + t0 * D;
+            const dim3 scan((unsigned)((D + 63) / 64), BH);
+            const bool vec = ((uintptr_t)from & 15) == 0 && (D == 64 || D == 128 || D == 256 || D == 512);
+#define KIVI_RUN_VEC(LPR)                                                                                                              \
+    do {                                                                                                                               \
+        const dim3 vgrid((unsigned)((n_chunks + 256 / LPR - 1) / (256 / LPR)), BH);                                                    \
+        kivi_run_chunk_vec_kernel<SrcT, LPR, 1><<<vgrid, 256, 0, s>>>(from, S, (int)rem, (int)n_chunks, tmp, tmp + plane, c->codes, c->cap_rows, c->n_rows); \
+        kivi_run_scan_min_kernel<<<scan, 64, 0, s>>>(tmp, D, (int)n_chunks, c->lo);                                                   \
+        kivi_run_chunk_vec_kernel<SrcT, LPR, 2><<<vgrid, 256, 0, s>>>(from, S, (int)rem, (int)n_chunks, tmp, tmp + plane, c->codes, c->cap_rows, c->n_rows); \
+        kivi_run_scan_scale_kernel<<<scan, 64, 0, s>>>(tmp + plane, D, (int)n_chunks, c->scale);                                      \
+        kivi_run_chunk_vec_kernel<SrcT, LPR, 3><<<vgrid, 256, 0, s>>>(from, S, (int)rem, (int)n_chunks, tmp, tmp + plane, c->codes, c->cap_rows, c->n_rows); \
+    } while (0)
+            if (vec) {
+                if (D == 64) KIVI_RUN_VEC(8); else if (D == 128) KIVI_RUN_VEC(16); else if (D == 256) KIVI_RUN_VEC(32); else KIVI_RUN_VEC(64);
+            } else {
+                const dim3 grid((unsigned)((D + 63) / 64), (unsigned)n_chunks, BH);
+                kivi_run_chunk_min_kernel<SrcT><<<grid, 64, 0, s>>>(from, S, (int)rem, D, (int)n_chunks, tmp);
+                kivi_run_scan_min_kernel<<<scan, 64, 0, s>>>(tmp, D, (int)n_chunks, c->lo);
+                kivi_run_chunk_scale_kernel<SrcT><<<grid, 64, 0, s>>>(from, S, (int)rem, D, (int)n_chunks, tmp, tmp + plane);
+                kivi_run_scan_scale_kernel<<<scan, 64, 0, s>>>(tmp + plane, D, (int)n_chunks, c->scale);
+                kivi_run_chunk_codes_kernel<SrcT><<<grid, 64, 0, s>>>(from, S, (int)rem, D, (int)n_chunks, tmp, tmp + plane, c->codes, c->cap_rows, c->n_rows);
+            }
+#undef KIVI_RUN_VEC
+            TROCM_HIP(hipGetLastError());
         } else {
             kivi_running_push_kernel<SrcT><<<dim3((unsigned)((D + 127) / 128), BH), 128, 0, s>>>(src + t0 * D, S, (int)rem, D, c->codes, c->cap_rows, c->n_rows, c->lo, c->scale);
             TROCM_HIP(hipGetLastError());
@@ -905,6 +1020,7 @@ int trocm_kivi_cache_destroy(trocm_kivi_cache *c) {
     (void)hipFree(c->scale);
     (void)hipFree(c->codes);
     (void)hipFree(c->deq);
+    (void)hipFree(c->scan);
     delete c;
     return 0;
 }
@@ -1020,6 +1136,17 @@ int trocm_kivi_cache_clone(const trocm_kivi_cache *c, trocm_kivi_cache **out, vo
     return 0;
 }
 
+// One token of f16 queries over the op's own stores (Keys under running per-channel parameters, Values per token, u8
+// codes, nothing kept in f32): attention straight over the codes, no dequantised copy.  TROCM_KIVI_FUSED=0 keeps the
+// dequantising path, which serves every other case.  (Evaluated before the step's tokens are appended: the stores
+// hold whole coded rows only, so the conditions on their counts hold afterwards as well.)
+static bool kivi_fused_step(int dtype, int64_t n_new, const trocm_kivi_cache *k, const trocm_kivi_cache *v) {
+    static const int fused = getenv("TROCM_KIVI_FUSED") ? atoi(getenv("TROCM_KIVI_FUSED")) : 1;
+    return fused && dtype == TROCM_F16 && n_new == 1 && k->D == 128 && k->layout == TROCM_KIVI_RUNNING_CHANNEL &&
+           v->layout == TROCM_KIVI_PER_TOKEN && k->bits == 8 && v->bits == 8 && k->sink_tokens == 0 && v->sink_tokens == 0 &&
+           k->n_res == 0 && v->n_res == 0 && k->n_rows == k->len && v->n_rows == v->len;
+}
+
 int trocm_quantized_kv_sdpa_eval(const void *q, const void *k_new, const void *v_new, int dtype, int64_t q_heads,
                                  int64_t n_new, trocm_kivi_cache *k_cache, trocm_kivi_cache *v_cache, void *out,
                                  float scale, void *workspace, size_t workspace_bytes, void *stream) {
@@ -1035,16 +1162,24 @@ int trocm_quantized_kv_sdpa_eval(const void *q, const void *k_new, const void *v
                   "QuantizedKvSdpa: the K and V stores differ in shape or length");
     TROCM_REQUIRE(q_heads > 0 && q_heads % k_cache->H == 0, "QuantizedKvSdpa: %lld query heads over %lld kv heads",
                   (long long)q_heads, (long long)k_cache->H);
+    TROCM_REQUIRE((k_cache->len + n_new) * k_cache->D < (1ll << 31) && n_new * k_cache->D < (1ll << 31),
+                  "QuantizedKvSdpa: %lld tokens of %lld channels exceed the index range", (long long)(k_cache->len + n_new), (long long)k_cache->D);
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
+    // Every allocation of the step, for both stores, before either is touched: a call that fails for want of memory
+    // leaves K and V as they were (same length, same counts) and can be repeated.
+    const bool fused_attention = kivi_fused_step(dtype, n_new, k_cache, v_cache);
+    for (trocm_kivi_cache *c : {k_cache, v_cache})
+        if (kivi_prepare(c, n_new, s)) return 1;
+    if (!(fused_attention && workspace)) {
+        const size_t need = (size_t)k_cache->BH * (k_cache->len + n_new) * k_cache->D * elem_bytes(dtype);
+        for (trocm_kivi_cache *c : {k_cache, v_cache})
+            if (kivi_grow_buffer(&c->deq, &c->deq_bytes, need, s, "the dequantised copy of a quantised store")) return 1;
+    }
     // a decode step on the op's own stores: both rows pushed by one launch
     if (n_new == 1 && k_cache->D == 128 && k_cache->layout == TROCM_KIVI_RUNNING_CHANNEL && v_cache->layout == TROCM_KIVI_PER_TOKEN &&
         k_cache->bits == 8 && v_cache->bits == 8 && k_cache->sink_tokens == 0 && v_cache->sink_tokens == 0 &&
         ((uintptr_t)v_new & 15) == 0 && (k_cache->len + 1) * 128 < (1ll << 31)) {
-        for (trocm_kivi_cache *c : {k_cache, v_cache}) {
-            if (kivi_alloc_fixed(c, s)) return 1;
-            if (kivi_ensure_rows(c, c->n_rows + 1, s)) return 1;
-        }
         const dim3 grid((unsigned)k_cache->BH, 2);
         if (dtype == TROCM_F16)
             kivi_step_push_kernel<__half><<<grid, 128, 0, s>>>((const __half *)k_new, (const __half *)v_new, k_cache->codes, k_cache->cap_rows, k_cache->n_rows,
@@ -1062,10 +1197,7 @@ int trocm_quantized_kv_sdpa_eval(const void *q, const void *k_new, const void *v
     // One token of f16 queries over the op's own stores (Keys under running per-channel parameters, Values per token, u8
     // codes, nothing kept in f32): attention straight over the codes, no dequantised copy.  TROCM_KIVI_FUSED=0 keeps
     // the dequantising path below, which serves every other case.
-    static const int fused = getenv("TROCM_KIVI_FUSED") ? atoi(getenv("TROCM_KIVI_FUSED")) : 1;
-    if (fused && dtype == TROCM_F16 && n_new == 1 && D == 128 && k_cache->layout == TROCM_KIVI_RUNNING_CHANNEL &&
-        v_cache->layout == TROCM_KIVI_PER_TOKEN && k_cache->bits == 8 && v_cache->bits == 8 && k_cache->n_sink == 0 &&
-        v_cache->n_sink == 0 && k_cache->n_res == 0 && v_cache->n_res == 0 && k_cache->n_rows == T && v_cache->n_rows == T) {
+    if (fused_attention) {
         KiviSdpaArgs a;
         a.q = q, a.out = out;
         a.k_codes = k_cache->codes, a.v_codes = v_cache->codes;
@@ -1076,31 +1208,22 @@ int trocm_quantized_kv_sdpa_eval(const void *q, const void *k_new, const void *v
         a.scale = scale == scale ? scale : 1.0f / sqrtf((float)D);   // NaN asks for the default (sdpa.rs:93-95)
         a.workspace = workspace, a.workspace_bytes = workspace_bytes;
         const int rc = workspace ? launch_sdpa_decode_kivi(a, s) : 2;
-        if (rc == 0) {   // the dequantised copies a prompt left behind are not needed again (hipFree waits for the device)
+        if (rc == 0) {   // the dequantised copies a prompt left behind are not needed again: released behind an event
             for (trocm_kivi_cache *c : {k_cache, v_cache})
                 if (c->deq) {
-                    (void)hipFree(c->deq);
+                    if (defer_device_free(c->deq, nullptr, s)) return 1;
                     c->deq = nullptr;
                     c->deq_bytes = 0;
                 }
         }
         if (rc != 2) return rc;
+        // (the launch declined: the dequantising path needs its buffers after all)
+        const size_t need = (size_t)k_cache->BH * T * D * elem_bytes(dtype);
+        for (trocm_kivi_cache *c : {k_cache, v_cache})
+            if (kivi_grow_buffer(&c->deq, &c->deq_bytes, need, s, "the dequantised copy of a quantised store")) return 1;
     }
-    const size_t need = (size_t)k_cache->BH * T * D * elem_bytes(dtype);
-    for (trocm_kivi_cache *c : {k_cache, v_cache}) {
-        if (c->deq_bytes < need) {
-            size_t cap = c->deq_bytes * 2 > need ? c->deq_bytes * 2 : need;
-            if (c->deq) {
-                TROCM_HIP(hipStreamSynchronize(s));
-                (void)hipFree(c->deq);
-                c->deq = nullptr;
-                c->deq_bytes = 0;
-            }
-            TROCM_HIP(hipMalloc(&c->deq, cap));
-            c->deq_bytes = cap;
-        }
+    for (trocm_kivi_cache *c : {k_cache, v_cache})
         if (kivi_dequantize(c, c->deq, dtype, s, false)) return 1;
-    }
     const int64_t strides[3] = {k_cache->H * T * D, T * D, D};
     // kv_quant.rs:326-327: FlashSdpaOp { causal: false, scale }
     return trocm_sdpa(q, k_cache->deq, v_cache->deq, nullptr, out, dtype, k_cache->B, q_heads, k_cache->H, n_new, T, D, strides, 1, 1,

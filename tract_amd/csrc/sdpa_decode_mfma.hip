@@ -59,6 +59,15 @@ __device__ __forceinline__ u32x4 dequant8(uint32_t b0123, uint32_t b4567, half2_
     return r;
 }
 
+// The power of two 2^-e that takes a positive finite x = m 2^e (m in [1/2, 1)) into [1/2, 1); 1 for zero, infinities and NaN.
+__device__ __forceinline__ float pow2_normaliser(float x) {
+    if (!(x > 0.0f) || x > 3.0e38f) return 1.0f;
+    int e;
+    (void)frexpf(x, &e);
+    e = e > 126 ? 126 : (e < -126 ? -126 : e);   // the factor itself stays an ordinary float
+    return ldexpf(1.0f, -e);
+}
+
 // What one workgroup has to do: a tile range of one (sequence, kv head), and where its result goes.
 struct MfmaWork {
     int seq, kvh;                 // the sequence (batch entry) and kv head
@@ -1327,15 +1336,29 @@ __device__ __forceinline__ void decode_mfma_kivi_body(const DecodeDev &p, const 
     }
 
     // Q^T fragments of this lane's head, one per 32 channels: channels 32 blk + 8 q4 + 0..7, times their key scales
+    // The products q * s_k go to the matrix cores as halves: a power of two takes the largest key scale of this kv head
+    // into [1/2, 1) first and leaves through the score scale below, so that keys of any magnitude keep the halves'
+    // 11 bits (scales under 6e-5 would otherwise make every product a subnormal half).
     half8_t qf[NB];
+    float ks_max = 0.0f;
+    float4_t ksv[NB][2];
+#pragma unroll
+    for (int blk = 0; blk < NB; blk++) {
+        ksv[blk][0] = *reinterpret_cast<const float4_t *>(ksc + 32 * blk + 8 * q4);
+        ksv[blk][1] = *reinterpret_cast<const float4_t *>(ksc + 32 * blk + 8 * q4 + 4);
+#pragma unroll
+        for (int i = 0; i < 8; i++) ks_max = fmaxf(ks_max, fabsf(ksv[blk][i >> 2][i & 3]));
+    }
+    ks_max = fmaxf(ks_max, __shfl_xor(ks_max, 16, 64));
+    ks_max = fmaxf(ks_max, __shfl_xor(ks_max, 32, 64));
+    const float k_norm = pow2_normaliser(ks_max), k_denorm = 1.0f / k_norm;   // exact powers of two
     float part = 0.0f;
 #pragma unroll
     for (int blk = 0; blk < NB; blk++) {
         const half8_t x = *reinterpret_cast<const half8_t *>(qrow + 32 * blk + 8 * q4);
-        const float4_t s0 = *reinterpret_cast<const float4_t *>(ksc + 32 * blk + 8 * q4), s1 = *reinterpret_cast<const float4_t *>(ksc + 32 * blk + 8 * q4 + 4);
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            qf[blk][i] = (_Float16)((float)x[i] * (i < 4 ? s0[i] : s1[i - 4]));
+            qf[blk][i] = (_Float16)((float)x[i] * (ksv[blk][i >> 2][i & 3] * k_norm));
             part += (float)qf[blk][i];
         }
     }
@@ -1359,7 +1382,10 @@ __device__ __forceinline__ void decode_mfma_kivi_body(const DecodeDev &p, const 
     const uint32_t v_key16 = 16 * key_v(v_tok);
     const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
 
-    const float c_log2 = p.scale_log2;   // > 0 (checked on the host): the maximum is taken before scaling
+    const float c_log2 = p.scale_log2 * k_denorm;   // > 0 (checked on the host): the maximum is taken before scaling
+    // Likewise P * s_v: v_norm is the power of two that takes the largest Value scale seen so far into [1/2, 1); when a
+    // tile brings a larger one the accumulated products move to the new factor (exact), like the running maximum.
+    float v_norm = 0.0f;   // 0: no tile yet
     auto do_tile = [&](auto stage_tag, int t) {
         constexpr int ST = decltype(stage_tag)::value;
         const int t0 = t * kTile;
@@ -1418,9 +1444,24 @@ __device__ __forceinline__ void decode_mfma_kivi_body(const DecodeDev &p, const 
             const float4_t la = *reinterpret_cast<const float4_t *>(lds_vp + kTile + 4 * q4), lb = *reinterpret_cast<const float4_t *>(lds_vp + kTile + 16 + 4 * q4);
             const float sv[8] = {sa[0], sa[1], sa[2], sa[3], sb[0], sb[1], sb[2], sb[3]};
             const float lv[8] = {la[0], la[1], la[2], la[3], lb[0], lb[1], lb[2], lb[3]};
+            float sv_max = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) sv_max = fmaxf(sv_max, fabsf(sv[i]));
+            sv_max = fmaxf(sv_max, __shfl_xor(sv_max, 16, 64));
+            sv_max = fmaxf(sv_max, __shfl_xor(sv_max, 32, 64));   // the tile's 32 tokens: the same value in every lane
+            const float want = pow2_normaliser(sv_max);
+            if (v_norm == 0.0f) {
+                v_norm = want;
+            } else if (want < v_norm) {   // a larger scale than any before (wave-uniform)
+                const float f = want / v_norm;   // a power of two below 1
+#pragma unroll
+                for (int fb = 0; fb < D / 16; fb++) o16[fb] *= f;
+                sp *= f;
+                v_norm = want;
+            }
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const half2_t pp = {(_Float16)(pe[2 * i] * sv[2 * i]), (_Float16)(pe[2 * i + 1] * sv[2 * i + 1])};
+                const half2_t pp = {(_Float16)(pe[2 * i] * (sv[2 * i] * v_norm)), (_Float16)(pe[2 * i + 1] * (sv[2 * i + 1] * v_norm))};
                 sp = __builtin_amdgcn_fdot2(pp, ones, sp, false);
                 sl = __builtin_fmaf(pe[2 * i], lv[2 * i], sl);
                 sl = __builtin_fmaf(pe[2 * i + 1], lv[2 * i + 1], sl);
@@ -1450,9 +1491,13 @@ __device__ __forceinline__ void decode_mfma_kivi_body(const DecodeDev &p, const 
     sp += __shfl_xor(sp, 32, 64);
     sl += __shfl_xor(sl, 16, 64);
     sl += __shfl_xor(sl, 32, 64);
-    const float shift = sl - 1024.0f * sp;   // the 1024 under every code leaves, the tokens' los arrive
+    // the 1024 under every code leaves, the power of two of the Value scales leaves, the tokens' los arrive
+    const float v_denorm = v_norm > 0.0f ? 1.0f / v_norm : 0.0f;
+    const float shift = 1024.0f * sp;
 #pragma unroll
-    for (int fb = 0; fb < D / 16; fb++) o16[fb] += shift;
+    for (int fb = 0; fb < D / 16; fb++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) o16[fb][r] = __builtin_fmaf(o16[fb][r] - shift, v_denorm, sl);
 
     // ---- merge the 4 waves through LDS (the tiles are dead) ------------------------------------------------------------
     __syncthreads();
