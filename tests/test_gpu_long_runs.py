@@ -61,6 +61,40 @@ def test_cfg2_128_steps_at_8192(rt, B, check_every):
     assert worst <= 2e-3   # in practice an order of magnitude inside the bar
 
 
+def test_cfg2_batch_32_fused_steps_at_8192(rt):
+    """cfg2's largest batch: 32 sequences prefilled to 8192 tokens (1 GiB of K and V), 32 fused steps (the first one
+    doubles both capacities).  Sequences 3 and 29 against the oracle on their own caches every 16 steps and at the
+    end, the final caches of all 32 sequences against the concatenation by hash."""
+    B, T, steps, watch = 32, 8192, 32, (3, 29)
+    kh = np.empty((B, HKV, T + steps, D), np.float16)
+    vh = np.empty((B, HKV, T + steps, D), np.float16)
+    for b in range(B):
+        kh[b, :, :T] = cases.seeded_normal(cases.cfg_seed(2, "k") + 1000 * b, (HKV, T, D), np.float16)
+        vh[b, :, :T] = cases.seeded_normal(cases.cfg_seed(2, "v") + 1000 * b, (HKV, T, D), np.float16)
+    st = ta.InPlaceKvSdpa(axis=2, causal=True).state()
+    st.k.push(np.ascontiguousarray(kh[:, :, :T])), st.v.push(np.ascontiguousarray(vh[:, :, :T]))
+    q_all = (cases.seeded_normal(cases.cfg_seed(2, "q") + 32, (steps, B, HQ, 1, D)) / np.sqrt(D)).astype(np.float16)
+    k_all = cases.seeded_normal(cases.cfg_seed(2, "k") + 39, (steps, B, HKV, 1, D), np.float16)
+    v_all = cases.seeded_normal(cases.cfg_seed(2, "v") + 39, (steps, B, HKV, 1, D), np.float16)
+    worst = 0.0
+    for s in range(steps):
+        out = st.eval([q_all[s], k_all[s], v_all[s]]).to_numpy()
+        kh[:, :, T + s], vh[:, :, T + s] = k_all[s][:, :, 0], v_all[s][:, :, 0]
+        if s % 16 == 0 or s == steps - 1:
+            n = T + s + 1
+            for b in watch:
+                want = orc.flash_sdpa(q_all[s][b:b + 1], np.ascontiguousarray(kh[b:b + 1, :, :n]), np.ascontiguousarray(vh[b:b + 1, :, :n]),
+                                      causal=True, threads=8)
+                err = max_abs(out[b:b + 1], want)
+                worst = max(worst, err)
+                assert err <= 2e-2, f"step {s}, sequence {b}: {err}"
+    assert (st.k.len(), st.k.capacity(), st.k.reallocs()) == (T + steps, 2 * T, 1)
+    assert (st.v.len(), st.v.capacity(), st.v.reallocs()) == (T + steps, 2 * T, 1)
+    assert _sha(st.k.valid_contiguous()) == _sha(kh)
+    assert _sha(st.v.valid_contiguous()) == _sha(vh)
+    assert worst <= 2e-3
+
+
 def test_cfg5_64_sequences_64_fused_steps(rt):
     n_seq, steps, per_step = 64, 64, 3
     rng = np.random.default_rng(cases.cfg_seed(5, "len"))

@@ -177,3 +177,19 @@ def test_launch_floor_kernels_run_and_refuse_bad_shapes(rt):
                  (0, None, 0, 0, 64, None, None), (0, None, 0, 1, 96, None, None), (0, None, 0, 1, 2048, None, None)):
         assert lib.trocm_launch_floor(*args) == 1
         assert b"launch_floor" in lib.trocm_last_error() or b"null pointer" in lib.trocm_last_error()
+
+
+def test_release_unused_frees_what_growth_left_behind(rt):
+    """A cache that grows outside a pool leaves its old planes on a list guarded by an event; a host that never calls
+    one of the library's synchronising entry points releases them with trocm_release_unused.  Contents stay."""
+    B, H, D = 1, 2, 64
+    rng = np.random.default_rng(9)
+    c = ta.InPlaceKvCache(2)
+    chunks = [rng.standard_normal((B, H, n, D), dtype=np.float32).astype(np.float16) for n in (16, 16, 40, 200)]
+    for x in chunks:
+        c.push(x)                       # 16 -> 32 -> 72 -> 272: three reallocations
+        call("trocm_release_unused", 0)  # never waits: frees what the device has finished with
+    call("trocm_release_unused", 1)      # waits for the rest
+    call("trocm_release_unused", 1)      # nothing left: still fine
+    assert c.reallocs() == 3
+    assert c.valid_contiguous().tobytes() == np.concatenate(chunks, axis=2).tobytes()

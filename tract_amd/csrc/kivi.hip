@@ -251,16 +251,22 @@ __global__ void kivi_run_chunk_min_kernel(const SrcT *__restrict__ src, int64_t 
     }
     cmin[((int64_t)bh * n_chunks + k) * D + c] = lo;
 }
-// scan 1: lo at the start of every chunk (in place), and the final lo into the store
+// scan 1: lo at the start of every chunk (in place), and the final lo into the store.  Sixteen chunk results are
+// requested together: one dependent load per chunk made this a chain of memory latencies (32 us for 128 chunks).
 __global__ void kivi_run_scan_min_kernel(float *__restrict__ cmin, int D, int n_chunks, float *__restrict__ lo_io) {
     const int bh = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= D) return;
     float lo = lo_io[(int64_t)bh * D + c];
-    for (int k = 0; k < n_chunks; k++) {
-        float *at = cmin + ((int64_t)bh * n_chunks + k) * D + c;
-        const float m = *at;
-        *at = lo;
-        if (m < lo) lo = m;
+    float *col = cmin + (int64_t)bh * n_chunks * D + c;
+    for (int k0 = 0; k0 < n_chunks; k0 += 16) {
+        float m[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) m[i] = k0 + i < n_chunks ? col[(int64_t)(k0 + i) * D] : INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            if (k0 + i < n_chunks) col[(int64_t)(k0 + i) * D] = lo;
+            if (m[i] < lo) lo = m[i];
+        }
     }
     lo_io[(int64_t)bh * D + c] = lo;
 }
@@ -288,11 +294,16 @@ __global__ void kivi_run_scan_scale_kernel(float *__restrict__ cmax, int D, int 
     const int bh = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= D) return;
     float scale = scale_io[(int64_t)bh * D + c];
-    for (int k = 0; k < n_chunks; k++) {
-        float *at = cmax + ((int64_t)bh * n_chunks + k) * D + c;
-        const float m = *at;
-        *at = scale;
-        if (m > scale) scale = m;
+    float *col = cmax + (int64_t)bh * n_chunks * D + c;
+    for (int k0 = 0; k0 < n_chunks; k0 += 16) {
+        float m[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) m[i] = k0 + i < n_chunks ? col[(int64_t)(k0 + i) * D] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            if (k0 + i < n_chunks) col[(int64_t)(k0 + i) * D] = scale;
+            if (m[i] > scale) scale = m[i];
+        }
     }
     scale_io[(int64_t)bh * D + c] = scale;
 }
@@ -411,24 +422,40 @@ __global__ void __launch_bounds__(256) kivi_run_chunk_vec_kernel(const SrcT *__r
     } else if (PASS == 3) {
         sc = ld8(b + at);
     }
+    // A channel's scale is the largest RN(range / 255) so far, and that quotient grows with the range: the division is
+    // only needed for a range larger than any before it (the same result as dividing every time).  The codes take the
+    // reciprocal of the scale with its re-check (affine_codes8), refreshed when the scale moves.
+    float widest[8];
+    F8 inv;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        widest[e] = 0.0f;
+        inv.v[e] = PASS == 3 ? affine_inv(sc.v[e]) : 0.0f;
+    }
 #pragma unroll 4
     for (int t = t0; t < t1; t++, row += D) {
         const F8 x = ld8(row);
-        uint32_t code[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             const float val = x.v[e];
             if (val < lo.v[e]) lo.v[e] = val;
             if (PASS >= 2) {
                 const float range = __fsub_rn(val, lo.v[e]);
-                if (range > 0.0f) {
+                if (range > widest[e]) {
+                    widest[e] = range;
                     const float ns = __fdiv_rn(range, 255.0f);
-                    if (ns > sc.v[e]) sc.v[e] = ns;
+                    if (ns > sc.v[e]) {
+                        sc.v[e] = ns;
+                        if (PASS == 3) inv.v[e] = affine_inv(ns);
+                    }
                 }
             }
-            if (PASS == 3) code[e] = affine_code(val, lo.v[e], sc.v[e], 255.0f);
         }
-        if (PASS == 3) store_codes8<8>(codes + ((int64_t)bh * cap_rows + row0 + t) * D, sub, code);
+        if (PASS == 3) {
+            uint32_t code[8];
+            affine_codes8(x.v, lo.v, sc.v, inv.v, 255.0f, code);
+            store_codes8<8>(codes + ((int64_t)bh * cap_rows + row0 + t) * D, sub, code);
+        }
     }
     if (PASS == 1) st8(a + at, lo);
     if (PASS == 2) st8(b + at, sc);
