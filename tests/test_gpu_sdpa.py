@@ -368,7 +368,9 @@ def test_ragged_decode_small(rt):
 
 @pytest.mark.parametrize("fmt_name", ["Q8_0", "Q4_0"])
 @pytest.mark.parametrize("B,Hq,Hkv,T", [(1, 32, 8, 1), (2, 32, 8, 100), (2, 32, 8, 1025), (1, 8, 8, 333), (1, 16, 2, 64),
-                                         (1, 24, 8, 77), (2, 32, 2, 300), (1, 32, 1, 129), (1, 22, 2, 95)])
+                                         (1, 24, 8, 77), (2, 32, 2, 300), (1, 32, 1, 129), (1, 22, 2, 95),
+                                         # 5..8 heads per kv head: two sets of four heads in the diagonal body
+                                         (2, 64, 8, 1025), (1, 10, 2, 1), (3, 12, 2, 257), (1, 14, 2, 4100), (2, 16, 2, 33)])
 def test_decode_quantised_cache(rt, fmt_name, B, Hq, Hkv, T):
     """cfg4 (reduced): K/V quantised on append, 1% outlier channels x20, decode with fused
     dequantisation.  Oracle: FlashSdpaOp over the dequantised blocks (f16 dequant like
@@ -404,7 +406,8 @@ def test_decode_quantised_cache(rt, fmt_name, B, Hq, Hkv, T):
 
 
 @pytest.mark.parametrize("fmt_name", ["Q8_0", "Q4_0"])
-@pytest.mark.parametrize("B,Hq,Hkv,T0", [(2, 32, 8, 61), (1, 16, 2, 30), (2, 32, 2, 95), (1, 6, 2, 0), (8, 32, 8, 2047), (1, 8, 8, 40)])
+@pytest.mark.parametrize("B,Hq,Hkv,T0", [(2, 32, 8, 61), (1, 16, 2, 30), (2, 32, 2, 95), (1, 6, 2, 0), (8, 32, 8, 2047), (1, 8, 8, 40),
+                                          (2, 14, 2, 95), (1, 40, 8, 1021)])
 def test_decode_steps_quantise_the_new_token_in_the_attention_launch(rt, fmt_name, B, Hq, Hkv, T0):
     """Single-token steps on a quantised cache (f16 inputs): the attention kernel quantises the step's K and V rows
     itself, stores them and attends over them.  After every step the cache's canonical blocks equal the CPU quantiser's
@@ -445,7 +448,8 @@ def test_decode_steps_quantise_the_new_token_in_the_attention_launch(rt, fmt_nam
 
 
 @pytest.mark.parametrize("fmt_name", ["Q8_0", "Q4_0"])
-@pytest.mark.parametrize("Hq,Hkv,n_seq,lo,hi", [(32, 8, 12, 1, 2500), (16, 1, 5, 20, 700), (8, 8, 4, 10, 200)])
+@pytest.mark.parametrize("Hq,Hkv,n_seq,lo,hi", [(32, 8, 12, 1, 2500), (16, 1, 5, 20, 700), (8, 8, 4, 10, 200), (16, 2, 9, 1, 3000),
+                                                 (12, 2, 5, 30, 900)])
 def test_ragged_decode_over_quantised_caches(rt, fmt_name, Hq, Hkv, n_seq, lo, hi):
     """Independent sequences with quantised caches of their own: every sequence equals the batch-1
     oracle over its dequantised blocks.  Two steps: attention only, then the append-and-attend step."""

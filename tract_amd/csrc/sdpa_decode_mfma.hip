@@ -923,9 +923,28 @@ __device__ __forceinline__ void nibbles8(const NibbleConsts &c, uint32_t w, uint
 //     dot products per tile where the block-scaling body needs 16 + 16, and no shuffling of scales at all, because
 //     the scale tiles are kept transposed in LDS ([block][token]: a lane's four tokens are one 8-byte read).
 // Matrix instructions, code unpacking and LDS traffic per tile are those of the block-scaling body.
-template <int GP, int FMT, int PF>
+//
+// H = 8 (5..8 heads per kv head): column c = 8 blk' + h stands for (block blk' of a PAIR of blocks, head h).  One product
+// then takes 16 features of each of two blocks (lane groups 2 blk', 2 blk' + 1 feed block blk' of the pair), a token's
+// four blocks take two sets of products (X = 0: blocks 0, 1; X = 1: blocks 2, 3) into two accumulators, a lane scales
+// the sums of two blocks and adds them in place, and one row rotation joins the pair.  The probabilities need one
+// operand per set (column (blk', h) carries P[t, h] d_v[t, 2 X + blk']).  Products, unpacking and LDS traffic per tile
+// stay what they are for H = 4; 16 vector instructions per tile are added.
+//
+// RS: the lanes that hold a head's blocks are neighbours (column c = BPC h + blk) and the sum over the blocks is a
+// reduce-scatter instead of an all-reduce.  The lanes that feed block blk of a set read token row (l ^ blk) of a
+// 16-token half where the others read row l, so register r of lane (h, blk) holds token (r ^ blk) of its group of four.
+// H = 4:  y = x0 + swap1(x1),  w = x2 + swap1(x3),  z = y + swap2(w)  (swap1 / swap2: the lane 1 / 2 places across in
+// the quad, DPP quad_perm) is, in lane blk, the whole score of token blk: three additions per half instead of eight,
+// every register index static; a lane exponentiates TWO scores (one per half) instead of eight.  H = 8:  x0 + swap1(x1)
+// and x2 + swap1(x3) are the scores of tokens blk and 2 + blk: two additions per half instead of four, four
+// exponentials instead of eight.  The pairs (token j of the first half, of the second) are then handed round with four
+// quad broadcasts, which put token j's pair into register j of every lane.
+template <int GP, int FMT, int PF, int H = 4, bool RS = false>
 __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const MfmaWork &wk) {
-    static_assert(GP == 8, "partial records are 8 rows wide; rows 0..3 are used");
+
+    static_assert(GP == 8, "partial records are 8 rows wide; with H = 4 rows 0..3 are used");
+    static_assert(H == 4 || H == 8, "4 or 8 heads across the 16 columns");
     static_assert(FMT == TROCM_Q8_0 || FMT == TROCM_Q4_0, "block-quantised caches only");
     constexpr int D = 128;
     constexpr bool Q8 = FMT == TROCM_Q8_0;
@@ -944,7 +963,12 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l16 = lane & 15, q4 = lane >> 4;
-    const int blk_c = l16 >> 2, h_c = l16 & 3;   // this lane's column: (block, head)
+    constexpr int BPC = 16 / H;                // blocks per product: 4 | 2
+    constexpr int LG = 4 / BPC;                // lane groups that feed one block of a product: 1 | 2
+    constexpr int NX = NB / BPC;               // sets of products per token: 1 | 2
+    constexpr int NJ = 4 / LG;                 // 8-code slices of a block per lane: 4 | 2
+    const int blk_c = RS ? l16 % BPC : l16 / H, h_c = RS ? l16 / BPC : l16 % H;  // this lane's column: (block within a set, head)
+    const int qb = q4 / LG, qs = q4 % LG;      // as a feeder: block within a set, and which slices of it (qs NJ + j)
     const int kvh = wk.kvh, b = wk.seq;
     const int g = p.g_real;
     unsigned char *lds_k = lds_raw + w * kWaveBytes, *lds_v = lds_k + kCodeBytes;
@@ -1014,62 +1038,86 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
     //   Q8_0: features 32 blk + 8 j + 0..7
     //   Q4_0: features 32 blk + 4 j + 0..3 (low nibbles) and 32 blk + 16 + 4 j + 0..3 (high nibbles: the codes arrive as
     //         16 u, so these features are divided by 16 -- exact but for subnormal results)
-    half8_t qf[4];
-    float part = 0.0f;   // what the products add up for a block of all-zero-point codes
-    const bool mine = q4 == blk_c;
+    half8_t qf[NX][NJ];
+    float bias[NX];      // minus what the products add up for a block of all-zero-point codes
+    const bool mine = qb == blk_c;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        half8_t f = {0, 0, 0, 0, 0, 0, 0, 0};
-        if constexpr (Q8) {
-            const half8_t x = *reinterpret_cast<const half8_t *>(qrow + 32 * blk_c + 8 * j);
-            float sum = 0.0f;
+    for (int X = 0; X < NX; X++) {
+        float part = 0.0f;
+        const _Float16 *qblk = qrow + 32 * (X * BPC + blk_c);
 #pragma unroll
-            for (int i = 0; i < 8; i++) sum += (float)x[i];
-            if (mine) f = x, part += 1152.0f * sum;   // the plane holds code + 128, under 1024
-        } else {
-            const half4_t lo = *reinterpret_cast<const half4_t *>(qrow + 32 * blk_c + 4 * j);
-            const half4_t hi = *reinterpret_cast<const half4_t *>(qrow + 32 * blk_c + 16 + 4 * j);
-            half8_t x;
-            float s_lo = 0.0f, s_hi = 0.0f, s_hi16 = 0.0f;
+        for (int j = 0; j < NJ; j++) {
+            const int sl = qs * NJ + j;   // slice of the block
+            half8_t f = {0, 0, 0, 0, 0, 0, 0, 0};
+            if constexpr (Q8) {
+                const half8_t x = *reinterpret_cast<const half8_t *>(qblk + 8 * sl);
+                float sum = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const _Float16 h16 = hi[i] * (_Float16)0.0625f;
-                // the order in which nibbles8() delivers the codes of a word: (lo0, lo2), (hi0, hi2), (lo1, lo3), (hi1, hi3)
-                const int at = 4 * (i & 1) + (i >> 1);
-                x[at] = lo[i], x[2 + at] = h16;
-                s_lo += (float)lo[i], s_hi16 += (float)h16, s_hi += 16.0f * (float)h16;
+                for (int i = 0; i < 8; i++) sum += (float)x[i];
+                if (mine) f = x, part += 1152.0f * sum;   // the plane holds code + 128, under 1024
+            } else {
+                const half4_t lo = *reinterpret_cast<const half4_t *>(qblk + 4 * sl);
+                const half4_t hi = *reinterpret_cast<const half4_t *>(qblk + 16 + 4 * sl);
+                half8_t x;
+                float s_lo = 0.0f, s_hi = 0.0f, s_hi16 = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const _Float16 h16 = hi[i] * (_Float16)0.0625f;
+                    // the order in which nibbles8() delivers the codes of a word: (lo0, lo2), (hi0, hi2), (lo1, lo3), (hi1, hi3)
+                    const int at = 4 * (i & 1) + (i >> 1);
+                    x[at] = lo[i], x[2 + at] = h16;
+                    s_lo += (float)lo[i], s_hi16 += (float)h16, s_hi += 16.0f * (float)h16;
+                }
+                if (mine) f = x, part += 1024.0f * (s_lo + s_hi16) + 8.0f * (s_lo + s_hi);
             }
-            if (mine) f = x, part += 1024.0f * (s_lo + s_hi16) + 8.0f * (s_lo + s_hi);
+            qf[X][j] = f;
         }
-        qf[j] = f;
+        part += __shfl_xor(part, 16, 64);   // the lane groups that hold the column's features hand their sums to the others
+        part += __shfl_xor(part, 32, 64);
+        bias[X] = -part;
     }
-    part += __shfl_xor(part, 16, 64);   // the one lane group that holds the column's features hands the sum to the others
-    part += __shfl_xor(part, 32, 64);
-    const float bias = -part;
 #pragma unroll
-    for (int j = 0; j < 4; j++) asm volatile("" : "+v"(qf[j]));   // settled here, not at first use inside the loop
+    for (int X = 0; X < NX; X++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++) asm volatile("" : "+v"(qf[X][j]));   // settled here, not at first use inside the loop
 
     float m_run = -INFINITY, l_run = 0.0f;   // log2 domain, already scaled
     float4_t o16[D / 16];
-    float sp = 0.0f;
+    float sp[NX];
+#pragma unroll
+    for (int X = 0; X < NX; X++) sp[X] = 0.0f;
 #pragma unroll
     for (int fb = 0; fb < D / 16; fb++) o16[fb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    // K fragment of this lane for slice j: token 16 mb + l16 (its key does not depend on mb), block q4, the bytes of
-    // slice j: Q8_0 chunk 2 q4 + j / 2, half j % 2; Q4_0 chunk q4, word j
-    uint32_t k_frag[4];
+    // K fragment of this lane for set X, slice j: token 16 mb + l16 (its key does not depend on mb), block X BPC + qb, the
+    // bytes of slice sl = qs NJ + j: Q8_0 chunk 2 block + sl / 2, half sl % 2; Q4_0 chunk block, word sl
+    uint32_t k_frag[NX][NJ];
 #pragma unroll
-    for (int j = 0; j < 4; j++)
-        k_frag[j] = Q8 ? l16 * RB + 16 * ((2 * q4 + (j >> 1)) ^ key_k(l16)) + 8 * (j & 1) : l16 * RB + 16 * (q4 ^ key_k(l16)) + 4 * j;
+    for (int X = 0; X < NX; X++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            const int blk = X * BPC + qb, sl = qs * NJ + j;
+            const int row = RS ? (l16 ^ qb) : l16;   // (RS: the feeders of block blk take the tokens of a group of four in the order t ^ blk)
+            k_frag[X][j] = Q8 ? row * RB + 16 * ((2 * blk + (sl >> 1)) ^ key_k(row)) + 8 * (sl & 1) : row * RB + 16 * (blk ^ key_k(row)) + 4 * sl;
+        }
     // V^T fragments: as in the block-scaling body
-    const int vk = l16 >> 1, v_tok = vk < 4 ? 4 * q4 + vk : 12 + 4 * q4 + vk;
+    // (RS: position 2 j + mb of the contraction is token 16 mb + 4 q4 + j; Q4_0's nibbles8() delivers byte p of the eight at
+    // position (0, 2, 1, 3, 4, 6, 5, 7)[p])
+    const int vk = l16 >> 1;
+    const int v_tok = !RS ? (vk < 4 ? 4 * q4 + vk : 12 + 4 * q4 + vk)
+                          : Q8 ? 16 * (vk & 1) + 4 * q4 + (vk >> 1) : 16 * ((vk >> 1) & 1) + 4 * q4 + 2 * (vk >> 2) + (vk & 1);
     const unsigned char *v_row = lds_v + v_tok * RB + 8 * (l16 & 1);
     const uint32_t v_key16 = 16 * key_v(v_tok);
-    // block scales of this lane's tokens 16 mb + 4 q4 + 0..3 in its block blk_c: 8 contiguous bytes per mb
-    const unsigned char *ks_frag = lds_ks + (blk_c * kTile + 4 * q4) * 2, *vs_frag = lds_vs + (blk_c * kTile + 4 * q4) * 2;
+    // block scales of this lane's tokens 16 mb + 4 q4 + 0..3 in its block blk_c of set 0 (set X: X BPC block rows on): 8
+    // contiguous bytes per mb
+    // (RS: the V scales of a lane's eight tokens are 16 contiguous bytes, pairs (token j of the first half, of the second))
+    const unsigned char *ks_frag = lds_ks + (blk_c * kTile + 4 * q4) * 2, *vs_frag = lds_vs + (blk_c * kTile + (RS ? 8 : 4) * q4) * 2;
     // where token `lane` goes in a row of the scale tiles: Q4_0 pairs tokens (0, 2) and (1, 3) of a group of four, the
     // order in which nibbles8() delivers the V codes (and so the order of the probabilities in their operand)
     const int sc_pos = Q8 ? lane : ((lane & ~3) | ((lane & 1) << 1) | ((lane >> 1) & 1));
+    // RS: in block row blk of the K scales token t sits at t ^ (blk % BPC), the order of the score registers; in
+    // every block row of the V scales token 16 mb + 4 q + j sits at 8 q + 2 j + mb
+    const int vs_pos = 8 * ((lane & 15) >> 2) + 2 * (lane & 3) + ((lane >> 4) & 1);
     const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
     const NibbleConsts nc = nibble_consts();
     auto ror_add = [](float x, auto ctrl_tag) {   // x + (x of the lane `n` places on in its row of 16 lanes)
@@ -1090,9 +1138,14 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
             *reinterpret_cast<u32x4 *>(lds_v + v_slot[j]) = vpre[ST][j];
         }
         if (lane < kTile) {   // token `lane`: its four block scales to the four block rows of the transposed tiles
-            uint16_t *ksT = reinterpret_cast<uint16_t *>(lds_ks) + sc_pos, *vsT = reinterpret_cast<uint16_t *>(lds_vs) + sc_pos;
-            ksT[0] = (uint16_t)kspre[ST].x, ksT[kTile] = (uint16_t)(kspre[ST].x >> 16);
-            ksT[2 * kTile] = (uint16_t)kspre[ST].y, ksT[3 * kTile] = (uint16_t)(kspre[ST].y >> 16);
+            uint16_t *ksT = reinterpret_cast<uint16_t *>(lds_ks) + (RS ? 0 : sc_pos), *vsT = reinterpret_cast<uint16_t *>(lds_vs) + (RS ? vs_pos : sc_pos);
+            if constexpr (RS) {
+                ksT[lane] = (uint16_t)kspre[ST].x, ksT[kTile + (lane ^ (1 % BPC))] = (uint16_t)(kspre[ST].x >> 16);
+                ksT[2 * kTile + (lane ^ (2 % BPC))] = (uint16_t)kspre[ST].y, ksT[3 * kTile + (lane ^ (3 % BPC))] = (uint16_t)(kspre[ST].y >> 16);
+            } else {
+                ksT[0] = (uint16_t)kspre[ST].x, ksT[kTile] = (uint16_t)(kspre[ST].x >> 16);
+                ksT[2 * kTile] = (uint16_t)kspre[ST].y, ksT[3 * kTile] = (uint16_t)(kspre[ST].y >> 16);
+            }
             vsT[0] = (uint16_t)vspre[ST].x, vsT[kTile] = (uint16_t)(vspre[ST].x >> 16);
             vsT[2 * kTile] = (uint16_t)vspre[ST].y, vsT[3 * kTile] = (uint16_t)(vspre[ST].y >> 16);
         }
@@ -1100,42 +1153,150 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
             fetch(wk.kbase, wk.ksbase, 0, t + PF * tstep, kpre[ST], kspre[ST]);
             fetch(wk.vbase, wk.vsbase, 1, t + PF * tstep, vpre[ST], vspre[ST]);
         }
-        // ---- codes x block-diagonal query operands: column (blk, h) receives the sum over block blk ----------------------
-        float4_t acc[2];
+        // ---- codes x block-diagonal query operands: column (blk, h) receives the sum over block X BPC + blk ----------------
+        float4_t acc[NX][2];
 #pragma unroll
         for (int mb = 0; mb < 2; mb++) {
-            acc[mb] = float4_t{bias, bias, bias, bias};
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                half8_t kf;
-                if constexpr (Q8) {
-                    const u32x2 c = *reinterpret_cast<const u32x2 *>(lds_k + k_frag[j] + 16 * mb * RB);
-                    kf = magic8(c.x, c.y);   // (the plane holds code + 128)
-                } else {
-                    const uint32_t c = *reinterpret_cast<const uint32_t *>(lds_k + k_frag[j] + 16 * mb * RB);
-                    uint32_t r0, r1, r2, r3;
-                    nibbles8(nc, c, r0, r1, r2, r3);
-                    kf = __builtin_bit_cast(half8_t, u32x4{r0, r1, r2, r3});
+            for (int X = 0; X < NX; X++) {
+                acc[X][mb] = float4_t{bias[X], bias[X], bias[X], bias[X]};
+#pragma unroll
+                for (int j = 0; j < NJ; j++) {
+                    half8_t kf;
+                    if constexpr (Q8) {
+                        const u32x2 c = *reinterpret_cast<const u32x2 *>(lds_k + k_frag[X][j] + 16 * mb * RB);
+                        kf = magic8(c.x, c.y);   // (the plane holds code + 128)
+                    } else {
+                        const uint32_t c = *reinterpret_cast<const uint32_t *>(lds_k + k_frag[X][j] + 16 * mb * RB);
+                        uint32_t r0, r1, r2, r3;
+                        nibbles8(nc, c, r0, r1, r2, r3);
+                        kf = __builtin_bit_cast(half8_t, u32x4{r0, r1, r2, r3});
+                    }
+                    acc[X][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[X][j], acc[X][mb], 0, 0, 0);
                 }
-                acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[j], acc[mb], 0, 0, 0);
             }
         }
-        // ---- scores (before the softmax scale) of tokens 16 mb + 4 q4 + r for head h_c: this block's share, then all four --
+        half2_t pf[4];
+        if constexpr (RS) {
+            // ---- this block's share of the scores of tokens 16 mb + 4 q4 + (r ^ blk_c), then the reduce-scatter over the quad ---
+            auto quad_add = [](float x, float y, auto ctrl_tag) {   // x + (y of the lane across in the quad)
+                constexpr int ctrl = decltype(ctrl_tag)::value;
+                const int o = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, y), ctrl, 0xf, 0xf, false);
+                return x + __builtin_bit_cast(float, o);
+            };
+            // Maxima as the bare instruction: fmaxf first copies every operand that might be a signalling NaN through a
+            // canonicalising v_max (nine more instructions per tile here).  The quad steps read their operand through DPP;
+            // the two wait states such a read needs after the write of its register are in the asm, because the compiler
+            // does not count wait states for registers that an asm writes.
+            auto vmax = [](float a, float b) {
+                float r;
+                asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+                return r;
+            };
+            auto quad_max_swap1 = [](float x) {
+                float r;
+                asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "=v"(r) : "v"(x));
+                return r;
+            };
+            auto quad_max_swap2 = [](float x) {
+                float r;
+                asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "=v"(r) : "v"(x));
+                return r;
+            };
+            using Swap1 = std::integral_constant<int, 0xB1>;   // quad_perm:[1,0,3,2]
+            using Swap2 = std::integral_constant<int, 0x4E>;   // quad_perm:[2,3,0,1]
+            constexpr int NS = 4 / BPC;   // scores per lane and half: tokens blk_c + BPC i
+            float x[2][4];
+#pragma unroll
+            for (int mb = 0; mb < 2; mb++) {
+#pragma unroll
+                for (int X = 0; X < NX; X++) {
+                    const u32x2 dk = *reinterpret_cast<const u32x2 *>(ks_frag + X * BPC * kTile * 2 + 32 * mb);
+                    const half2_t da = as_half2(dk.x), db = as_half2(dk.y);
+                    const _Float16 dv[4] = {da[0], da[1], db[0], db[1]};
+#pragma unroll
+                    for (int r = 0; r < 4; r++) x[mb][r] = __builtin_fmaf((float)dv[r], acc[X][mb][r], X == 0 ? 0.0f : x[mb][r]);
+                }
+            }
+            float z[2][NS];
+            {
+                float y[2], wv[2];
+#pragma unroll
+                for (int mb = 0; mb < 2; mb++) y[mb] = quad_add(x[mb][0], x[mb][1], Swap1{}), wv[mb] = quad_add(x[mb][2], x[mb][3], Swap1{});
+#pragma unroll
+                for (int mb = 0; mb < 2; mb++) {
+                    if constexpr (H == 4) z[mb][0] = quad_add(y[mb], wv[mb], Swap2{});   // token 16 mb + 4 q4 + blk_c, head h_c
+                    else z[mb][0] = y[mb], z[mb][NS - 1] = wv[mb];                       // tokens 16 mb + 4 q4 + blk_c (+ 2)
+                }
+            }
+            if (t0 + kTile > T) {   // the sequence's last tile: tokens past its end do not count
+                asm volatile("");   // (a branch, not selects in every tile)
+#pragma unroll
+                for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                    for (int i = 0; i < NS; i++)
+                        if (t0 + 16 * mb + 4 * q4 + blk_c + BPC * i >= T) z[mb][i] = -INFINITY;
+            }
+            float tmax = vmax(z[0][0], z[1][0]);
+            if constexpr (NS == 2) tmax = vmax(tmax, vmax(z[0][NS - 1], z[1][NS - 1]));
+            tmax = quad_max_swap1(tmax);
+            if constexpr (H == 4) tmax = quad_max_swap2(tmax);
+            tmax = vmax(tmax, __shfl_xor(tmax, 16, 64));
+            tmax = vmax(tmax, __shfl_xor(tmax, 32, 64));
+            const float m_new = vmax(m_run, tmax * c_log2);   // finite: every tile holds at least one valid token
+            float psum = 0.0f;
+            uint32_t mine2[NS];
+#pragma unroll
+            for (int i = 0; i < NS; i++) {
+                const float p0 = fast_exp2(__builtin_fmaf(z[0][i], c_log2, -m_new)), p1 = fast_exp2(__builtin_fmaf(z[1][i], c_log2, -m_new));
+                psum += p0 + p1;
+                mine2[i] = __builtin_bit_cast(uint32_t, half2_t{(_Float16)p0, (_Float16)p1});
+            }
+            // register j of every lane: the pair of token j of the lane's group of four (quad broadcasts from the lane that
+            // holds it: lane j of the quad; with two lanes per head lane j % 2 of the head's pair, its register j / 2)
+            if constexpr (H == 4) {
+                pf[0] = as_half2((uint32_t)__builtin_amdgcn_mov_dpp((int)mine2[0], 0x00, 0xf, 0xf, true));
+                pf[1] = as_half2((uint32_t)__builtin_amdgcn_mov_dpp((int)mine2[0], 0x55, 0xf, 0xf, true));
+                pf[2] = as_half2((uint32_t)__builtin_amdgcn_mov_dpp((int)mine2[0], 0xAA, 0xf, 0xf, true));
+                pf[3] = as_half2((uint32_t)__builtin_amdgcn_mov_dpp((int)mine2[0], 0xFF, 0xf, 0xf, true));
+            } else {
+                pf[0] = as_half2((uint32_t)__builtin_amdgcn_mov_dpp((int)mine2[0], 0xA0, 0xf, 0xf, true));        // quad_perm:[0,0,2,2]
+                pf[1] = as_half2((uint32_t)__builtin_amdgcn_mov_dpp((int)mine2[0], 0xF5, 0xf, 0xf, true));        // quad_perm:[1,1,3,3]
+                pf[2] = as_half2((uint32_t)__builtin_amdgcn_mov_dpp((int)mine2[NS - 1], 0xA0, 0xf, 0xf, true));
+                pf[3] = as_half2((uint32_t)__builtin_amdgcn_mov_dpp((int)mine2[NS - 1], 0xF5, 0xf, 0xf, true));
+            }
+            const bool moved = m_new != m_run;
+            const float alpha = fast_exp2(m_run - m_new);
+            l_run = l_run * alpha + psum;   // this lane's own tokens; the lanes of a head are added up after the loop
+            m_run = m_new;
+            if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+                for (int fb = 0; fb < D / 16; fb++) o16[fb] *= alpha;
+#pragma unroll
+                for (int X = 0; X < NX; X++) sp[X] *= alpha;
+            }
+        } else {
+        // ---- scores (before the softmax scale) of tokens 16 mb + 4 q4 + r for head h_c: this lane's blocks, then all four --
         float sc8[8];
 #pragma unroll
         for (int mb = 0; mb < 2; mb++) {
-            const u32x2 dk = *reinterpret_cast<const u32x2 *>(ks_frag + 32 * mb);   // scales of tokens r = 0, 1 | 2, 3
-            const half2_t da = as_half2(dk.x), db = as_half2(dk.y);
-            // (Q4_0: the scale tiles hold a group of four tokens in the order 0, 2, 1, 3)
-            const _Float16 dv[4] = {da[0], Q8 ? da[1] : db[0], Q8 ? db[0] : da[1], db[1]};
 #pragma unroll
-            for (int r = 0; r < 4; r++) sc8[4 * mb + r] = __builtin_fmaf((float)dv[r], acc[mb][r], 0.0f);
+            for (int X = 0; X < NX; X++) {
+                const u32x2 dk = *reinterpret_cast<const u32x2 *>(ks_frag + X * BPC * kTile * 2 + 32 * mb);   // scales of tokens r = 0, 1 | 2, 3
+                const half2_t da = as_half2(dk.x), db = as_half2(dk.y);
+                // (Q4_0: the scale tiles hold a group of four tokens in the order 0, 2, 1, 3)
+                const _Float16 dv[4] = {da[0], Q8 ? da[1] : db[0], Q8 ? db[0] : da[1], db[1]};
+#pragma unroll
+                for (int r = 0; r < 4; r++) sc8[4 * mb + r] = __builtin_fmaf((float)dv[r], acc[X][mb][r], X == 0 ? 0.0f : sc8[4 * mb + r]);
+            }
         }
-        // the four blocks of a head sit 4 lanes apart in a row of 16 lanes: two rotations add them up in every lane.  (One
-        // stage at a time over all eight values: a rotation must wait two issue slots for its operand, and a value carried
-        // through both stages on its own fills them with s_nop.)
+        // the blocks of a head sit H lanes apart in a row of 16 lanes: rotations add them up in every lane.  (One stage at a
+        // time over all eight values: a rotation must wait two issue slots for its operand, and a value carried through
+        // both stages on its own fills them with s_nop.)
+        if constexpr (H == 4) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) sc8[i] = ror_add(sc8[i], std::integral_constant<int, 0x124>{});   // row_ror:4
+            for (int i = 0; i < 8; i++) sc8[i] = ror_add(sc8[i], std::integral_constant<int, 0x124>{});   // row_ror:4
+        }
 #pragma unroll
         for (int i = 0; i < 8; i++) sc8[i] = ror_add(sc8[i], std::integral_constant<int, 0x128>{});   // row_ror:8
 
@@ -1151,7 +1312,6 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
         const float m_new = fmaxf(m_run, tmax * c_log2);   // finite: every tile holds at least one valid token
         float psum = 0.0f;
-        half2_t pf[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             // Q8_0: tokens (2i, 2i + 1) of the lane's eight; Q4_0: (0, 2), (1, 3), (4, 6), (5, 7)
@@ -1167,23 +1327,34 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
         if (__builtin_amdgcn_ballot_w64(moved) != 0) {
 #pragma unroll
             for (int fb = 0; fb < D / 16; fb++) o16[fb] *= alpha;
-            sp *= alpha;
+#pragma unroll
+            for (int X = 0; X < NX; X++) sp[X] *= alpha;
         }
-        // ---- probabilities times the V scales of their tokens in block blk_c: one operand for all four blocks ---------------
+        }
+        // ---- probabilities times the V scales of their tokens in block X BPC + blk_c: one operand per set of blocks ---------
         // pf[i] holds two tokens of 4 q4 + 0..3 for i < 2 and of 16 + 4 q4 + 0..3 for i >= 2, the scale tiles the same pairs
-        u32x4 pw;
-        {
-            const u32x2 e0 = *reinterpret_cast<const u32x2 *>(vs_frag), e1 = *reinterpret_cast<const u32x2 *>(vs_frag + 32);
-            const uint32_t ev[4] = {e0.x, e0.y, e1.x, e1.y};
+        half8_t pb[NX];
+#pragma unroll
+        for (int X = 0; X < NX; X++) {
+            const unsigned char *vsx = vs_frag + X * BPC * kTile * 2;
+            uint32_t ev[4];
+            if constexpr (RS) {
+                const u32x4 e = *reinterpret_cast<const u32x4 *>(vsx);
+                ev[0] = e.x, ev[1] = e.y, ev[2] = e.z, ev[3] = e.w;
+            } else {
+                const u32x2 e0 = *reinterpret_cast<const u32x2 *>(vsx), e1 = *reinterpret_cast<const u32x2 *>(vsx + 32);
+                ev[0] = e0.x, ev[1] = e0.y, ev[2] = e1.x, ev[3] = e1.y;
+            }
+            u32x4 pw;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const half2_t pp = pf[i] * as_half2(ev[i]);
-                sp = __builtin_amdgcn_fdot2(pp, ones, sp, false);
+                sp[X] = __builtin_amdgcn_fdot2(pp, ones, sp[X], false);
                 pw[i] = __builtin_bit_cast(uint32_t, pp);
             }
+            pb[X] = __builtin_bit_cast(half8_t, pw);
         }
-        const half8_t pb = __builtin_bit_cast(half8_t, pw);
-        // ---- O^T += codes^T x scaled probabilities: the tile of block blk is right in the columns (blk, h) -------------------
+        // ---- O^T += codes^T x scaled probabilities: the tile of block blk is right in the columns (blk % BPC, h) -------------
 #pragma unroll
         for (int blk = 0; blk < NB; blk++) {
             if constexpr (Q8) {
@@ -1192,7 +1363,7 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
                     uint32_t w0, w1;
                     lds_read_tr8(v_row + ((32 * blk + 16 * hf) ^ v_key16), w0, w1);
                     const half8_t vf = magic8(w0, w1);
-                    o16[2 * blk + hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pb, o16[2 * blk + hf], 0, 0, 0);
+                    o16[2 * blk + hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pb[blk / BPC], o16[2 * blk + hf], 0, 0, 0);
                 }
             } else {
                 uint32_t w0, w1;   // byte l16 of the block's 16: feature l16 in the low nibble, 16 + l16 in the high one
@@ -1201,8 +1372,8 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
                 nibbles8(nc, w0, la, ha, lb, hb2);
                 nibbles8(nc, w1, lc, hc, ld2, hd);
                 const half8_t vlo = __builtin_bit_cast(half8_t, u32x4{la, lb, lc, ld2}), vhi = __builtin_bit_cast(half8_t, u32x4{ha, hb2, hc, hd});
-                o16[2 * blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vlo, pb, o16[2 * blk], 0, 0, 0);
-                o16[2 * blk + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vhi, pb, o16[2 * blk + 1], 0, 0, 0);
+                o16[2 * blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vlo, pb[blk / BPC], o16[2 * blk], 0, 0, 0);
+                o16[2 * blk + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vhi, pb[blk / BPC], o16[2 * blk + 1], 0, 0, 0);
             }
         }
     };
@@ -1214,24 +1385,32 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
             if (t < tile_end) do_tile(std::integral_constant<int, 1>{}, t), t += tstep;
         }
     }
+    if constexpr (RS) {   // a lane has summed its own tokens of every tile
+        l_run += __shfl_xor(l_run, 1, 64);
+        if constexpr (H == 4) l_run += __shfl_xor(l_run, 2, 64);
+    }
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
     // the zero points of this lane's column: O[f, h] -= (1024 + zero) * SP[h, blk] (Q4_0's high features arrived 16 times
-    // too large); only the tiles of block blk_c are read off this column
-    sp += __shfl_xor(sp, 16, 64);
-    sp += __shfl_xor(sp, 32, 64);
+    // too large); only the tiles of the blocks X BPC + blk_c are read off this column
+#pragma unroll
+    for (int X = 0; X < NX; X++) {
+        sp[X] += __shfl_xor(sp[X], 16, 64);
+        sp[X] += __shfl_xor(sp[X], 32, 64);
+    }
 #pragma unroll
     for (int blk = 0; blk < NB; blk++) {
+        const float spb = sp[blk / BPC];
         if constexpr (Q8) {
-            o16[2 * blk] -= 1152.0f * sp;
-            o16[2 * blk + 1] -= 1152.0f * sp;
+            o16[2 * blk] -= 1152.0f * spb;
+            o16[2 * blk + 1] -= 1152.0f * spb;
         } else {
-            o16[2 * blk] -= 1032.0f * sp;
-            o16[2 * blk + 1] = o16[2 * blk + 1] * 0.0625f - 72.0f * sp;
+            o16[2 * blk] -= 1032.0f * spb;
+            o16[2 * blk + 1] = o16[2 * blk + 1] * 0.0625f - 72.0f * spb;
         }
     }
 
-    // ---- merge the 4 waves through LDS (the tiles are dead): rows 0..3 are the heads, rows 4..7 neutral records -----------
+    // ---- merge the 4 waves through LDS (the tiles are dead): rows 0..H-1 are the heads, with H = 4 rows 4..7 neutral records -
     __syncthreads();
     float *comb = reinterpret_cast<float *>(lds_raw);   // [kWaves][GP*D + 2*GP]
     {
@@ -1239,15 +1418,17 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
         const float4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int fb = 0; fb < D / 16; fb++)
-            if ((fb >> 1) == blk_c) {
+            if ((fb >> 1) % BPC == blk_c) {
                 *reinterpret_cast<float4_t *>(cw + h_c * D + 16 * fb + 4 * q4) = o16[fb];
-                *reinterpret_cast<float4_t *>(cw + (4 + h_c) * D + 16 * fb + 4 * q4) = zero4;
+                if constexpr (H == 4) *reinterpret_cast<float4_t *>(cw + (4 + h_c) * D + 16 * fb + 4 * q4) = zero4;
             }
         if (q4 == 0 && blk_c == 0) {
             cw[GP * D + h_c] = m_run;
             cw[GP * D + GP + h_c] = l_run;
-            cw[GP * D + 4 + h_c] = -INFINITY;
-            cw[GP * D + GP + 4 + h_c] = 0.0f;
+            if constexpr (H == 4) {
+                cw[GP * D + 4 + h_c] = -INFINITY;
+                cw[GP * D + GP + 4 + h_c] = 0.0f;
+            }
         }
     }
     wave_records_to_output<D, GP>(p, wk, lds_raw, head0, g, tid);
@@ -1544,7 +1725,7 @@ __device__ __forceinline__ int mask_row_len(const _Float16 *__restrict__ row, in
 // Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.
 // QB: quantised caches on the 16-wide tiles run the body that scales per block outside the products.
 template <int D, int GP, int FMT, bool MASK = false, bool W16 = false, int QB = 0>
-__global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma_kernel(DecodeDev p) {   // QB = 100 * (1: diagonal, 2: affine u8) + 10 * tiles ahead + workgroups per CU
+__global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma_kernel(DecodeDev p) {   // QB = 100 * (1: diagonal, 2: affine u8, 3: diagonal with 8 heads across the columns, 4 / 5: 1 / 3 with the reduce-scatter) + 10 * tiles ahead + workgroups per CU
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     MfmaWork wk;
     wk.seq = b, wk.kvh = kvh;
@@ -1579,10 +1760,10 @@ __global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma
     wk.counter = p.counters ? p.counters + bh : nullptr;
     wk.part_first = bh * p.nsplit, wk.part_stride = 1;
     wk.mask = MASK ? p.mask + (int64_t)b * p.mask_stride_b + (int64_t)kvh * p.g_real * p.mask_stride_h : nullptr;
-    if constexpr (QB >= 200)
+    if constexpr (QB / 100 == 2)
         decode_mfma_kivi_body<GP, (QB / 10) % 10>(p, wk);
     else if constexpr (QB >= 100)
-        decode_mfma_qdiag_body<GP, FMT, (QB / 10) % 10>(p, wk);
+        decode_mfma_qdiag_body<GP, FMT, (QB / 10) % 10, (QB / 100 == 3 || QB / 100 == 5 ? 8 : 4), (QB / 100 >= 4)>(p, wk);
     else if constexpr (QB != 0)
         decode_mfma_qblock_body<GP, FMT, QB / 10>(p, wk);
     else
@@ -1612,7 +1793,7 @@ __global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma
     wk.part_first = (int64_t)it.slot0 * p.Hkv + kvh, wk.part_stride = p.Hkv;
     wk.mask = nullptr;
     if constexpr (QB >= 100)
-        decode_mfma_qdiag_body<GP, FMT, (QB / 10) % 10>(p, wk);
+        decode_mfma_qdiag_body<GP, FMT, (QB / 10) % 10, (QB / 100 == 3 || QB / 100 == 5 ? 8 : 4), (QB / 100 >= 4)>(p, wk);
     else if constexpr (QB != 0)
         decode_mfma_qblock_body<GP, FMT, QB / 10>(p, wk);
     else
@@ -1643,11 +1824,36 @@ bool use_diagonal() {
     static const int on = getenv("TROCM_DECODE_QDIAG") ? atoi(getenv("TROCM_DECODE_QDIAG")) : 1;
     return on != 0;
 }
+// 5..8 heads per kv head: the diagonal body with 8 heads and a pair of blocks across the columns (batch 8, 16384 tokens,
+// Q4_0, 8 heads per kv head: 37.8 us on the 16 columns of heads -> 34.2 us) unless TROCM_DECODE_QDIAG_PAIRS=0.  (Two sets
+// of four heads in the 4 x 4 arrangement, every unpacked fragment feeding two products, were measured first: 42.2 us,
+// the score-side instructions double.)
+bool use_diagonal_pairs() {
+    static const int on = getenv("TROCM_DECODE_QDIAG_PAIRS") ? atoi(getenv("TROCM_DECODE_QDIAG_PAIRS")) : 1;
+    return on != 0;
+}
+// The diagonal bodies sum a head's blocks with a reduce-scatter over neighbouring lanes and exponentiate each score once
+// per head instead of once per block column (batch 8, 16384 tokens, Q4_0: 4 heads per kv head 32.3 -> 30.9 us, 8 heads
+// 34.5 -> 33 us; Q8_0 49.3 -> 48.8 us) unless TROCM_DECODE_QDIAG_RS=0.
+bool use_diagonal_rs() {
+    static const int on = getenv("TROCM_DECODE_QDIAG_RS") ? atoi(getenv("TROCM_DECODE_QDIAG_RS")) : 1;
+    return on != 0;
+}
 template <int GP, int FMT>
 void launch_qblock(const DecodeDev &p, dim3 grid, hipStream_t s) {
     if constexpr (GP == 8) {
         if (p.g_real <= 4 && use_diagonal()) {
-            hipLaunchKernelGGL((sdpa_decode_mfma_kernel<128, GP, FMT, false, true, (FMT == TROCM_Q8_0 ? 112 : 122)>), grid, dim3(kThreads), 0, s, p);
+            if (use_diagonal_rs())
+                hipLaunchKernelGGL((sdpa_decode_mfma_kernel<128, GP, FMT, false, true, (FMT == TROCM_Q8_0 ? 412 : 422)>), grid, dim3(kThreads), 0, s, p);
+            else
+                hipLaunchKernelGGL((sdpa_decode_mfma_kernel<128, GP, FMT, false, true, (FMT == TROCM_Q8_0 ? 112 : 122)>), grid, dim3(kThreads), 0, s, p);
+            return;
+        }
+        if (use_diagonal() && use_diagonal_pairs()) {   // 5..8 heads per kv head: 8 heads x a pair of blocks across the columns
+            if (use_diagonal_rs())
+                hipLaunchKernelGGL((sdpa_decode_mfma_kernel<128, GP, FMT, false, true, (FMT == TROCM_Q8_0 ? 512 : 522)>), grid, dim3(kThreads), 0, s, p);
+            else
+                hipLaunchKernelGGL((sdpa_decode_mfma_kernel<128, GP, FMT, false, true, (FMT == TROCM_Q8_0 ? 312 : 322)>), grid, dim3(kThreads), 0, s, p);
             return;
         }
     }
@@ -1695,8 +1901,14 @@ template <int D, int GP, int FMT = TROCM_F16>
 int launch_ragged_gp(const DecodeDev &p, const RaggedItem *items, int n_items, const RaggedSeqSlots *seqs, int n_seq,
                      bool any_split, hipStream_t s) {
     if (FMT != TROCM_F16 && D == 128 && GP <= 16 && use_16_wide(FMT) && use_block_scaling() && p.scale_log2 > 0.0f)
-        if (GP == 8 && p.g_real <= 4 && use_diagonal())
+        if (GP == 8 && p.g_real <= 4 && use_diagonal() && use_diagonal_rs())
+            hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<128, 8, (FMT != TROCM_F16 ? FMT : TROCM_Q8_0), true, (FMT == TROCM_Q4_0 ? 422 : 412)>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+        else if (GP == 8 && p.g_real <= 4 && use_diagonal())
             hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<128, 8, (FMT != TROCM_F16 ? FMT : TROCM_Q8_0), true, (FMT == TROCM_Q4_0 ? 122 : 112)>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+        else if (GP == 8 && use_diagonal() && use_diagonal_pairs() && use_diagonal_rs())
+            hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<128, 8, (FMT != TROCM_F16 ? FMT : TROCM_Q8_0), true, (FMT == TROCM_Q4_0 ? 522 : 512)>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+        else if (GP == 8 && use_diagonal() && use_diagonal_pairs())
+            hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<128, 8, (FMT != TROCM_F16 ? FMT : TROCM_Q8_0), true, (FMT == TROCM_Q4_0 ? 322 : 312)>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
         else
             hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<128, (GP <= 16 ? GP : 16), (FMT != TROCM_F16 ? FMT : TROCM_Q8_0), true, (FMT == TROCM_Q4_0 ? 22 : 12)>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
     else if (GP <= 16 && use_16_wide(FMT))
