@@ -660,6 +660,57 @@ def run_ops(ta, args):
     by = algorithmic_bytes(B, W)
     res["window_kv_sdpa_step_b8_w4096"] = {"us": round(us, 2), "gbs": round(by / us / 1e3, 1), "bytes": int(by)}
     del sts, xs, cs
+    # the attention block of a decoder layer's step as an exported graph states it: ApplyRope on Q, ApplyRope on K_new,
+    # InPlaceKvSdpa -- as three calls (three launches) and through the entry point that rotates both inside the attention
+    # launch; cfg2's shape at 8192 tokens over 4 layers' caches, batch 8 and batch 1
+    for Bs in (8, 1):
+        T0 = 8192
+        lay = [ta.InPlaceKvSdpa(axis=2, causal=True).state() for _ in range(4)]
+        kk = rng.standard_normal((Bs, HKV, T0, D)).astype(np.float16)
+        for st in lay:
+            for c in (st.k, st.v):
+                c.reserve(T0 + 1024, like=(kk.shape, kk.dtype))
+                c.push(kk)
+        del kk
+        qd = ta.DeviceTensor.from_numpy((rng.standard_normal((Bs, HQ, 1, D)) / np.sqrt(D)).astype(np.float16))
+        kd = ta.DeviceTensor.from_numpy(rng.standard_normal((Bs, HKV, 1, D)).astype(np.float16))
+        angs = rng.uniform(-3, 3, (Bs, 1, 1, D)).astype(np.float32)
+        cd, sd = ta.DeviceTensor.from_numpy(np.cos(angs).astype(np.float16)), ta.DeviceTensor.from_numpy(np.sin(angs).astype(np.float16))
+        qr, kr = ta.DeviceTensor(qd.shape, np.float16), ta.DeviceTensor(kd.shape, np.float16)
+        od = ta.DeviceTensor(qd.shape, np.float16)
+
+        # (raw C calls with their arguments built once: at batch 1 the host mirror's Python would be what is timed)
+        import ctypes as C
+        ws = ta.Workspace(Bs, HQ, 1, D)
+        nanf = C.c_float(float("nan"))
+        qshape, kshape = (C.c_int64 * 4)(Bs, HQ, 1, D), (C.c_int64 * 4)(Bs, HKV, 1, D)
+        cstr = (C.c_int64 * 4)(D, 0, D, 1)
+        hk, hv = [st.k.handle for st in lay], [st.v.handle for st in lay]
+
+        def three_calls():
+            i = turn[0] % 4
+            call("trocm_apply_rope", qd.ptr, cd.ptr, sd.ptr, qr.ptr, 1, 4, qshape, None, cstr, None, None)
+            call("trocm_apply_rope", kd.ptr, cd.ptr, sd.ptr, kr.ptr, 1, 4, kshape, None, cstr, None, None)
+            call("trocm_inplace_kv_sdpa_eval", qr.ptr, kr.ptr, kd.ptr, 1, HQ, 1, None, hk[i], hv[i], od.ptr, nanf, 1, ws.ptr, ws.nbytes, None)
+            turn[0] += 1
+
+        def one_call():
+            i = turn[0] % 4
+            call("trocm_inplace_kv_sdpa_eval_rope", qd.ptr, kd.ptr, kd.ptr, cd.ptr, sd.ptr, D, 1, HQ, 1, hk[i], hv[i], od.ptr, nanf, 1,
+                 ws.ptr, ws.nbytes, None, 0, None)
+            turn[0] += 1
+
+        def plain_step():   # the step without any rotation, for scale
+            i = turn[0] % 4
+            call("trocm_inplace_kv_sdpa_eval", qd.ptr, kd.ptr, kd.ptr, 1, HQ, 1, None, hk[i], hv[i], od.ptr, nanf, 1, ws.ptr, ws.nbytes, None)
+            turn[0] += 1
+
+        us3 = time_calls(ta, three_calls, 100)
+        us1 = time_calls(ta, one_call, 100)
+        us0 = time_calls(ta, plain_step, 100)
+        res[f"rope_rope_step_b{Bs}_ctx8192"] = {"three_calls_us": round(us3, 2), "fused_us": round(us1, 2), "step_without_rope_us": round(us0, 2),
+                                                "note": "ApplyRope(Q), ApplyRope(K_new), InPlaceKvSdpa step: three launches against one"}
+        del lay
     # mask inputs on the fast attention kernels: decode (batch 8, 8192 tokens, padding mask [8,1,1,T]) over
     # 4 layers' K/V, and a 512-query chunk over 4096 keys with the causal mask stated as an input [1,1,512,4096]
     T = 8192

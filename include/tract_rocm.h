@@ -342,6 +342,22 @@ int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_n
                                trocm_kv_cache *k_cache, trocm_kv_cache *v_cache, void *out, float scale,
                                int causal, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ApplyRope (transformers/src/ops/apply_rope.rs:169-176) on q and k_new followed by InPlaceKvSdpaState::eval
+ * (inplace_kv_cache.rs:191-216) as one call: the two ApplyRope nodes an exported decoder puts between its
+ * projections and the cache (the pattern transformers/src/ops/sdpa.rs:453-458 looks through).  q, k_new, v_new and out
+ * dense as in trocm_inplace_kv_sdpa_eval; cos and sin are [n_new, head_dim] rows of `dtype` per sequence,
+ * `cos_sin_batch_stride` elements apart (0: one set of rows for every sequence); v_new is not rotated.  The appended
+ * keys and the output are bit-identical to trocm_apply_rope on q and k_new followed by trocm_inplace_kv_sdpa_eval.
+ * A single-token step on an F16 cache with 2..16 query heads per kv head is one launch and touches no scratch;
+ * every other call rotates into `rot_scratch` (16-byte aligned), which must then hold
+ * round_up(batch * q_heads * n_new * head_dim * elem, 256) + batch * kv_heads * n_new * head_dim * elem bytes
+ * (a call that needs it and finds it too small fails before anything is changed). */
+int trocm_inplace_kv_sdpa_eval_rope(const void *q, const void *k_new, const void *v_new, const void *cos,
+                                    const void *sin, int64_t cos_sin_batch_stride, int dtype, int64_t q_heads,
+                                    int64_t n_new, trocm_kv_cache *k_cache, trocm_kv_cache *v_cache, void *out,
+                                    float scale, int causal, void *workspace, size_t workspace_bytes,
+                                    void *rot_scratch, size_t rot_scratch_bytes, void *stream);
+
 /* WindowKvSdpaState::eval (transformers/src/ops/window_kv_cache.rs:216-239): append K_new and
  * V_new to the two sliding-window caches, then attend Q to every valid slot without a causal
  * mask (the ring buffer is the window).  Arguments as trocm_inplace_kv_sdpa_eval.  A

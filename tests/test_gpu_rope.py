@@ -105,3 +105,79 @@ def test_rope_then_cache_then_attention_matches_oracle(rt):
         assert np.abs(out.astype(np.float32) - want.astype(np.float32)).max() <= 2e-2
         pos += S
     assert st.k.valid_contiguous().tobytes() == np.concatenate(ks, 2).tobytes()
+
+
+def _rope_step_inputs(rng, B, Hq, Hkv, n, D, dt, per_sequence):
+    q = (rng.standard_normal((B, Hq, n, D)) / np.sqrt(D)).astype(dt)
+    k = rng.standard_normal((B, Hkv, n, D)).astype(dt)
+    v = rng.standard_normal((B, Hkv, n, D)).astype(dt)
+    ang = rng.uniform(-7, 7, (B if per_sequence else 1, 1, n, D))
+    return q, k, v, np.cos(ang).astype(dt), np.sin(ang).astype(dt)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,D,T0,per_sequence", [(2, 32, 8, 128, 61, True), (1, 16, 2, 128, 2050, False), (3, 12, 2, 64, 30, True),
+                                                        (8, 32, 8, 128, 2047, True), (1, 14, 2, 128, 95, False)])
+def test_decode_steps_rotate_q_and_k_in_the_attention_launch(rt, B, Hq, Hkv, D, T0, per_sequence):
+    """Single-token steps through the entry point that fuses ApplyRope on Q and K_new into the append + attention launch:
+    after every step the cache's keys are the oracle's rope of the step's keys, bit for bit, and the output equals the
+    unfused sequence (ApplyRope, ApplyRope, InPlaceKvSdpa) bit for bit and the oracle within the path's tolerance."""
+    rng = np.random.default_rng(B * 1000 + Hq + T0)
+    op = tract_amd.InPlaceKvSdpa(axis=2, causal=True)
+    fused, plain = op.state(), op.state()
+    k0, v0 = rng.standard_normal((B, Hkv, T0, D)).astype(np.float16), rng.standard_normal((B, Hkv, T0, D)).astype(np.float16)
+    for st in (fused, plain):
+        st.k.reserve(T0 + 3, like=(k0.shape, k0.dtype)), st.v.reserve(T0 + 3, like=(v0.shape, v0.dtype))   # two steps in place, then growth
+        st.k.push(k0), st.v.push(v0)
+    ks, vs = k0, v0
+    for step in range(5):
+        q, k, v, cos, sin = _rope_step_inputs(rng, B, Hq, Hkv, 1, D, np.float16, per_sequence)
+        dq, dk, dv, dc, ds = (tract_amd.DeviceTensor.from_numpy(a) for a in (q, k, v, cos, sin))
+        got = fused.eval_rope_into(dq, dk, dv, dc, ds).to_numpy()
+        rq, rk = orc.apply_rope(q, cos, sin), orc.apply_rope(k, cos, sin)
+        want_plain = plain.eval([tract_amd.ApplyRope().eval(q, cos, sin), tract_amd.ApplyRope().eval(k, cos, sin), v]).to_numpy()
+        ks, vs = np.concatenate([ks, rk], axis=2), np.concatenate([vs, v], axis=2)
+        assert fused.k.valid_contiguous().tobytes() == ks.tobytes(), step
+        assert fused.v.valid_contiguous().tobytes() == vs.tobytes(), step
+        assert got.tobytes() == want_plain.tobytes(), step
+        want = orc.flash_sdpa(rq, ks, vs, causal=True)
+        assert np.abs(got.astype(np.float32) - want.astype(np.float32)).max() <= 2e-2, step
+    assert fused.k.len() == T0 + 5
+
+
+@pytest.mark.parametrize("dt,B,Hq,Hkv,D,n", [(np.float16, 2, 32, 8, 128, 5), (np.float32, 2, 8, 2, 64, 1), (np.float16, 1, 8, 8, 128, 1),
+                                             (np.float16, 1, 40, 2, 128, 1)])
+def test_rope_steps_that_rotate_into_the_scratch(rt, dt, B, Hq, Hkv, D, n):
+    """Chunks of several tokens, f32, one head per kv head and more than 16 heads per kv head have no fused kernel: the call
+    rotates into its scratch and goes on as the plain step; same bits as the unfused sequence."""
+    rng = np.random.default_rng(Hq * 7 + n)
+    op = tract_amd.InPlaceKvSdpa(axis=2, causal=True)
+    fused, plain = op.state(), op.state()
+    k0, v0 = rng.standard_normal((B, Hkv, 40, D)).astype(dt), rng.standard_normal((B, Hkv, 40, D)).astype(dt)
+    for st in (fused, plain):
+        st.k.push(k0), st.v.push(v0)
+    for step in range(3):
+        q, k, v, cos, sin = _rope_step_inputs(rng, B, Hq, Hkv, n, D, dt, step % 2 == 0)
+        got = fused.eval_rope_into(*(tract_amd.DeviceTensor.from_numpy(a) for a in (q, k, v, cos, sin))).to_numpy()
+        want = plain.eval([tract_amd.ApplyRope().eval(q, cos, sin), tract_amd.ApplyRope().eval(k, cos, sin), v]).to_numpy()
+        assert got.tobytes() == want.tobytes(), step
+        assert fused.k.valid_contiguous().tobytes() == plain.k.valid_contiguous().tobytes()
+
+
+def test_rope_step_refused_for_its_scratch_changes_nothing(rt):
+    import ctypes as C
+    from tract_amd._lib import call
+    rng = np.random.default_rng(5)
+    st = tract_amd.InPlaceKvSdpa(axis=2, causal=True).state()
+    k0 = rng.standard_normal((1, 2, 33, 128)).astype(np.float16)
+    st.k.push(k0), st.v.push(k0)
+    q, k, v, cos, sin = _rope_step_inputs(rng, 1, 8, 2, 4, 128, np.float16, False)
+    dq, dk, dv, dc, ds = (tract_amd.DeviceTensor.from_numpy(a) for a in (q, k, v, cos, sin))
+    out = tract_amd.DeviceTensor(q.shape, q.dtype)
+    ws = tract_amd.Workspace(1, 8, 4, 128)
+    before = st.k.valid_contiguous().tobytes()
+    with pytest.raises(tract_amd.TractRocmError, match="rot_scratch"):
+        call("trocm_inplace_kv_sdpa_eval_rope", dq.ptr, dk.ptr, dv.ptr, dc.ptr, ds.ptr, 0, 1, 8, 4, st.k.handle, st.v.handle, out.ptr,
+             C.c_float(float("nan")), 1, ws.ptr, ws.nbytes, None, 0, None)
+    assert st.k.len() == 33 and st.k.valid_contiguous().tobytes() == before
+    got = st.eval_rope_into(dq, dk, dv, dc, ds).to_numpy()   # the same call with its scratch goes through
+    assert st.k.len() == 37 and not np.isnan(got).any()

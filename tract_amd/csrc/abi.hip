@@ -1306,6 +1306,62 @@ int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_n
     return trocm_sdpa_cached(q, dtype, q_heads, n_new, kc, vc, out, scale, causal, workspace, workspace_bytes, stream);
 }
 
+// ApplyRope on q and k_new, then InPlaceKvSdpaState::eval: what an exported decoder's graph does with the two ApplyRope
+// nodes between the projections and the cache.  A single-token step on an f16 cache is ONE launch (the attention
+// kernel rotates both on the way in); every other call rotates into `rot_scratch` and goes on as trocm_inplace_kv_sdpa_eval.
+int trocm_inplace_kv_sdpa_eval_rope(const void *q, const void *k_new, const void *v_new, const void *cos, const void *sin,
+                                    int64_t cos_sin_batch_stride, int dtype, int64_t q_heads, int64_t n_new,
+                                    trocm_kv_cache *kc, trocm_kv_cache *vc, void *out, float scale, int causal,
+                                    void *workspace, size_t workspace_bytes, void *rot_scratch, size_t rot_scratch_bytes,
+                                    void *stream) {
+    if (inplace_eval_check("inplace_kv_sdpa_rope", q, k_new, v_new, out, dtype, q_heads, n_new, kc, vc)) return 1;
+    TROCM_NOT_NULL(cos);
+    TROCM_NOT_NULL(sin);
+    TROCM_REQUIRE(kc->D % 2 == 0, "apply_rope: the head dimension must be even");
+    TROCM_REQUIRE(cos_sin_batch_stride == 0 || cos_sin_batch_stride >= n_new * kc->D,
+                  "apply_rope: cos / sin rows of one sequence overlap the next one's (batch stride %lld < %lld)",
+                  (long long)cos_sin_batch_stride, (long long)(n_new * kc->D));
+    hipStream_t s;
+    if (resolve_stream(stream, &s)) return 1;
+    if (n_new == 1 && dtype == TROCM_F16 && kc->fmt == TROCM_F16 && kc->window == 0 && vc->window == 0 && q_heads % kc->H == 0) {
+        if (equalise_capacities(kc, vc, s)) return 1;
+        int64_t dense[4];
+        dense[3] = 1, dense[2] = kc->D, dense[1] = kc->D, dense[0] = kc->H * kc->D;
+        if (append_prepare(kc, k_new, dtype, dense, 1, s)) return 1;
+        if (append_prepare(vc, v_new, dtype, dense, 1, s)) return 1;
+        if (kc->cap == vc->cap) {
+            SdpaArgs a;
+            cached_args(a, q, dtype, q_heads, 1, kc, vc, kc->len + 1, out, scale, causal, workspace, workspace_bytes);
+            a.k_new = k_new, a.v_new = v_new, a.new_pos = -1;
+            a.rope_cos = cos, a.rope_sin = sin, a.rope_stride_b = cos_sin_batch_stride;
+            int rc = launch_sdpa_decode(a, s);
+            if (rc == 0) {
+                kc->len += 1;
+                vc->len += 1;
+                return 0;
+            }
+            if (rc != 2) return rc;
+        }
+    }
+    // rotate into the caller's scratch: q first, then k_new
+    const size_t es = elem_bytes(dtype);
+    const size_t q_bytes = (size_t)kc->B * q_heads * n_new * kc->D * es, k_bytes = (size_t)kc->B * kc->H * n_new * kc->D * es;
+    const size_t q_room = (q_bytes + 255) & ~(size_t)255;
+    TROCM_REQUIRE(rot_scratch != nullptr && rot_scratch_bytes >= q_room + k_bytes,
+                  "inplace_kv_sdpa_rope: this call rotates q and k_new into rot_scratch, which must hold %zu bytes (%zu given)",
+                  q_room + k_bytes, rot_scratch_bytes);
+    TROCM_REQUIRE((uintptr_t)rot_scratch % 16 == 0, "rot_scratch must be 16-byte aligned");
+    void *q_rot = rot_scratch, *k_rot = (char *)rot_scratch + q_room;
+    const int64_t cs[4] = {cos_sin_batch_stride, 0, kc->D, 1};
+    const int64_t qs[4] = {kc->B, q_heads, n_new, kc->D}, ks[4] = {kc->B, kc->H, n_new, kc->D};
+    if (n_new > 0) {
+        if (trocm_apply_rope(q, cos, sin, q_rot, dtype, 4, qs, nullptr, cs, nullptr, stream)) return 1;
+        if (trocm_apply_rope(k_new, cos, sin, k_rot, dtype, 4, ks, nullptr, cs, nullptr, stream)) return 1;
+    }
+    return trocm_inplace_kv_sdpa_eval(q_rot, k_rot, v_new, dtype, q_heads, n_new, nullptr, kc, vc, out, scale, causal, workspace,
+                                      workspace_bytes, stream);
+}
+
 // WindowKvSdpaState::eval (window_kv_cache.rs:216-239): push K_new / V_new into the ring buffers,
 // then attend to every valid slot in physical order without a causal mask -- the ring buffer
 // already bounds which keys are visible, and attention does not depend on the order of the keys.

@@ -155,6 +155,11 @@ struct SdpaArgs {
     int causal;
     void *workspace;
     size_t workspace_bytes;
+    // fused append with RoPE (f16 decode on the matrix cores only): q and k_new are rotated on the way in,
+    // out = x * cos + RotateHalf(x) * sin with every product and the sum rounded to f16 like ApplyRope; rows of D
+    // elements of q_dtype, one per batch entry `rope_stride_b` elements apart (0: one row for all)
+    const void *rope_cos, *rope_sin;
+    int64_t rope_stride_b;
 };
 int launch_sdpa_generic(const SdpaArgs &a, hipStream_t s);
 // Split-K decode (Sq == 1).  Returns 2 when the shape is not covered by a fast kernel.

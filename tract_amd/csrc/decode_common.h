@@ -40,6 +40,9 @@ struct DecodeDev {
     // affine u8 caches (decode_mfma_kivi_body): the Keys' per-channel scales, f32 [B * Hkv, D]; k_scales / v_scales then
     // point at the Values' per-token scale and lo planes, f32 [B, Hkv, cap_rows], sc_stride_* their byte strides
     const float *chan_scale;
+    // fused append with RoPE (f16, 16-wide tiles): cos / sin rows of D halves, one per sequence rope_stride_b bytes apart
+    const char *rope_cos, *rope_sin;
+    int64_t rope_stride_b;
 };
 
 // Ragged batches: one work item = a tile range of one sequence (device copies of the host plan).

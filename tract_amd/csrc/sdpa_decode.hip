@@ -472,6 +472,7 @@ int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s) {
         const int rc = launch_sdpa_decode_mfma(a, s);
         if (rc != 2) return rc;
     }
+    if (a.rope_cos) return 2;   // the rotation of q and k_new is built into the MFMA kernel only
     if (a.kv_fmt != TROCM_F16 && a.kv_fmt != TROCM_F32) return 2;
     if (a.q_dtype != a.kv_fmt) return 2;
     if (a.D != 64 && a.D != 128) return 2;

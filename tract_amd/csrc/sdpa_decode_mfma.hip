@@ -140,9 +140,27 @@ __device__ __forceinline__ void wave_records_to_output(const DecodeDev &p, const
 // half the accumulator and query registers, and a lane exponentiates 8 scores instead of 16.  A lane then owns
 // head lane % 16 and, of a 32-token tile, tokens 4*(lane/16) + 0..3 and 16 + 4*(lane/16) + 0..3; of the output,
 // features 16*fb + 4*(lane/16) + 0..3 of every 16-feature block fb.
-template <int D, int GP, int FMT, bool MASK = false, bool W16 = false>
+// Eight consecutive elements of a row rotated as ApplyRope does (apply_rope.rs:169-176): y = x * cos + RotateHalf(x) * sin,
+// RotateHalf(x)[i] = -x[i + D/2] in the first half of the row and x[i - D/2] in the second, every product and the sum
+// rounded to f16 (the products pass through an empty asm: this file is compiled with contraction on, and a fused
+// multiply-add would round once where the CPU op rounds twice).  `row` / `cosr` / `sinr`: the D halves of the row and of
+// its cos / sin rows; dc: which 16-byte chunk.
+template <int D>
+__device__ __forceinline__ u32x4 rope_chunk(const char *row, const char *cosr, const char *sinr, int dc) {
+    constexpr int CPR = D / 8;
+    const bool first = dc < CPR / 2;
+    const half8_t x = *reinterpret_cast<const half8_t *>(row + dc * 16);
+    const half8_t y = *reinterpret_cast<const half8_t *>(row + (first ? dc + CPR / 2 : dc - CPR / 2) * 16);
+    const half8_t c = *reinterpret_cast<const half8_t *>(cosr + dc * 16), sn = *reinterpret_cast<const half8_t *>(sinr + dc * 16);
+    half8_t a = x * c, b = (first ? -y : y) * sn;
+    asm volatile("" : "+v"(a), "+v"(b));
+    return __builtin_bit_cast(u32x4, a + b);
+}
+
+template <int D, int GP, int FMT, bool MASK = false, bool W16 = false, bool ROPE = false>
 __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaWork &wk) {
     static_assert(!W16 || GP <= 16, "the 16-wide layout: at most 16 heads");
+    static_assert(!ROPE || (W16 && FMT == TROCM_F16 && !MASK), "the rotation is built for f16 rows on the 16-wide tiles");
     constexpr bool QUANT = FMT != TROCM_F16;
     constexpr int KS = D / 16;             // contraction steps of K.Q^T
     constexpr int DB = D / 32;             // 32-feature blocks of the output
@@ -196,12 +214,19 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
     // its newest loads as well -- 1.6 us of a 47.6 us launch, with or without a new token.)
     const int new_pos = wk.new_pos;
     const int64_t new_row = ((int64_t)b * p.Hkv + kvh) * D * 2;
+    // (ROPE: the step's q and k_new rows are rotated on the way in, with the sequence's cos / sin rows)
+    const char *cos_row = ROPE ? p.rope_cos + (int64_t)b * p.rope_stride_b : nullptr;
+    const char *sin_row = ROPE ? p.rope_sin + (int64_t)b * p.rope_stride_b : nullptr;
     if constexpr (!QUANT) {
         if (new_pos >= 0 && w == 0 && wk.tile_begin == 0 && lane < 2 * CPR) {
             const int dc = lane % CPR;
             const char *src = (lane < CPR ? p.k_new : p.v_new) + new_row + dc * 16;
             char *dst = const_cast<char *>(lane < CPR ? kbase : vbase) + (int64_t)new_pos * p.kv_stride_t + dc * 16;
-            *reinterpret_cast<u32x4 *>(dst) = *reinterpret_cast<const u32x4 *>(src);
+            u32x4 val = *reinterpret_cast<const u32x4 *>(src);
+            if constexpr (ROPE) {
+                if (lane < CPR) val = rope_chunk<D>(p.k_new + new_row, cos_row, sin_row, dc);
+            }
+            *reinterpret_cast<u32x4 *>(dst) = val;
         }
     }
     auto fetch_q = [&](const char *base0, const char *sbase0, int t, u32x4 (&dst)[NLD], uint32_t (&sc)[QUANT ? NLD : 1]) {
@@ -245,7 +270,12 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
             }
         }
     };
-    auto fetch = [&](const char *base0, const char *fresh, int t, u32x4 (&dst)[NLD]) {
+    static_assert(64 % CPR == 0, "a lane's chunk of a row is the same in every load of a tile");
+    u32x4 new_k_chunk = {0u, 0u, 0u, 0u};
+    if constexpr (ROPE) {
+        if (new_pos >= 0) new_k_chunk = rope_chunk<D>(p.k_new + new_row, cos_row, sin_row, lane % CPR);
+    }
+    auto fetch = [&](const char *base0, const char *fresh, int t, u32x4 (&dst)[NLD], bool rotate = false) {
         const int t0 = t * kTile;
         const char *base = base0 + (int64_t)t0 * p.kv_stride_t;
         if (t0 + kTile <= T && !(new_pos >= t0 && new_pos < t0 + kTile)) {
@@ -257,27 +287,63 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
                 const int c = j * 64 + lane, row = min(c / CPR, T - 1 - t0), dc = c % CPR;
                 const char *cache_ptr = base + (uint32_t)row * (uint32_t)p.kv_stride_t + (uint32_t)dc * 16u;
                 const bool is_new = t0 + row == new_pos;
-                dst[j] = *reinterpret_cast<const u32x4 *>(is_new ? fresh + new_row + dc * 16 : cache_ptr);
+                const u32x4 ld = *reinterpret_cast<const u32x4 *>(is_new ? fresh + new_row + dc * 16 : cache_ptr);
+                // (ROPE: the lane's chunk of the rotated new key, made once ahead of the loop; dc = lane % CPR for every j.
+                // A select after the load, not a branch around it: with a load that some lanes skip the compiler can no
+                // longer count what is in flight and every wait of the loop becomes a wait for everything.)
+                if constexpr (ROPE) {
+                    const bool take = rotate && is_new;
+                    dst[j] = u32x4{take ? new_k_chunk.x : ld.x, take ? new_k_chunk.y : ld.y, take ? new_k_chunk.z : ld.z, take ? new_k_chunk.w : ld.w};
+                } else {
+                    dst[j] = ld;
+                }
             }
         }
     };
 
+    // Q^T fragments: row (head) = lane % 32, features 16*ks + 8*hb .. +8 (16-wide: lane % 16, 32*ks + 8*(lane/16) .. +8)
+    constexpr int NQF = W16 ? D / 32 : KS;
+    half8_t qf[NQF];
+    // ROPE: the query's features and their cos / sin are asked for AHEAD of the first tile (the vector-memory counter
+    // returns in order: asked for after it, they would arrive after 16 KiB of K and V and the rotation would sit between
+    // the tile's arrival and its first product); the partner of features 32 ks + 8 q4 + i, D/2 further on or back, is
+    // this lane's own fragment ks +- NQF/2
+    half8_t rc[ROPE ? NQF : 1], rs[ROPE ? NQF : 1];
+    if constexpr (ROPE) {
+#pragma unroll
+        for (int ks = 0; ks < NQF; ks++) {
+            qf[ks] = *reinterpret_cast<const half8_t *>(qrow + 32 * ks + 8 * q4);
+            rc[ks] = *reinterpret_cast<const half8_t *>(cos_row + (32 * ks + 8 * q4) * 2);
+            rs[ks] = *reinterpret_cast<const half8_t *>(sin_row + (32 * ks + 8 * q4) * 2);
+        }
+    }
     int t = tile_begin + w;
     if (t < tile_end) {
         if constexpr (QUANT) {
             fetch_q(kbase, wk.ksbase, t, kpre, ksc);
             fetch_q(vbase, wk.vsbase, t, vpre, vsc);
         } else {
-            fetch(kbase, p.k_new, t, kpre);
+            fetch(kbase, p.k_new, t, kpre, true);
             fetch(vbase, p.v_new, t, vpre);
         }
     }
-    // Q^T fragments: row (head) = lane % 32, features 16*ks + 8*hb .. +8 (16-wide: lane % 16, 32*ks + 8*(lane/16) .. +8)
-    constexpr int NQF = W16 ? D / 32 : KS;
-    half8_t qf[NQF];
+    if constexpr (ROPE) {
+        half8_t a[NQF], bb[NQF];
 #pragma unroll
-    for (int ks = 0; ks < NQF; ks++)
-        qf[ks] = *reinterpret_cast<const half8_t *>(W16 ? qrow + 32 * ks + 8 * q4 : qrow + 16 * ks + 8 * hb);
+        for (int ks = 0; ks < NQF; ks++) {
+            const bool first = ks < NQF / 2;
+            const half8_t y = qf[first ? ks + NQF / 2 : ks - NQF / 2];
+            a[ks] = qf[ks] * rc[ks], bb[ks] = (first ? -y : y) * rs[ks];
+        }
+#pragma unroll
+        for (int ks = 0; ks < NQF; ks++) asm volatile("" : "+v"(a[ks]), "+v"(bb[ks]));   // two roundings, not a fused multiply-add
+#pragma unroll
+        for (int ks = 0; ks < NQF; ks++) qf[ks] = a[ks] + bb[ks];
+    } else {
+#pragma unroll
+        for (int ks = 0; ks < NQF; ks++)
+            qf[ks] = *reinterpret_cast<const half8_t *>(W16 ? qrow + 32 * ks + 8 * q4 : qrow + 16 * ks + 8 * hb);
+    }
 #pragma unroll
     for (int ks = 0; ks < NQF; ks++) asm volatile("" : "+v"(qf[ks]));   // settled here, not at first use inside the loop
 
@@ -328,7 +394,7 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
         } else {
 #pragma unroll
             for (int j = 0; j < NLD; j++) *reinterpret_cast<u32x4 *>(tile + k_slot[j]) = kpre[j];
-            if (more) fetch(kbase, p.k_new, t + tstep, kpre);
+            if (more) fetch(kbase, p.k_new, t + tstep, kpre, true);
         }
         half8_t pf16;
         if constexpr (W16) {
@@ -1725,7 +1791,7 @@ __device__ __forceinline__ int mask_row_len(const _Float16 *__restrict__ row, in
 // Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.
 // QB: quantised caches on the 16-wide tiles run the body that scales per block outside the products.
 template <int D, int GP, int FMT, bool MASK = false, bool W16 = false, int QB = 0>
-__global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma_kernel(DecodeDev p) {   // QB = 100 * (1: diagonal, 2: affine u8, 3: diagonal with 8 heads across the columns, 4 / 5: 1 / 3 with the reduce-scatter) + 10 * tiles ahead + workgroups per CU
+__global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma_kernel(DecodeDev p) {   // QB = 100 * (1: diagonal, 2: affine u8, 3: diagonal with 8 heads across the columns, 4 / 5: 1 / 3 with the reduce-scatter, 9: the f16 body rotating q and k_new (RoPE)) + 10 * tiles ahead + workgroups per CU
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     MfmaWork wk;
     wk.seq = b, wk.kvh = kvh;
@@ -1760,7 +1826,9 @@ __global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma
     wk.counter = p.counters ? p.counters + bh : nullptr;
     wk.part_first = bh * p.nsplit, wk.part_stride = 1;
     wk.mask = MASK ? p.mask + (int64_t)b * p.mask_stride_b + (int64_t)kvh * p.g_real * p.mask_stride_h : nullptr;
-    if constexpr (QB / 100 == 2)
+    if constexpr (QB / 100 == 9)
+        decode_mfma_body<D, GP, FMT, MASK, W16, true>(p, wk);
+    else if constexpr (QB / 100 == 2)
         decode_mfma_kivi_body<GP, (QB / 10) % 10>(p, wk);
     else if constexpr (QB >= 100)
         decode_mfma_qdiag_body<GP, FMT, (QB / 10) % 10, (QB / 100 == 3 || QB / 100 == 5 ? 8 : 4), (QB / 100 >= 4)>(p, wk);
@@ -1862,7 +1930,9 @@ void launch_qblock(const DecodeDev &p, dim3 grid, hipStream_t s) {
 
 template <int D, int GP, int FMT = TROCM_F16>
 int launch_gp(const DecodeDev &p, dim3 grid, hipStream_t s) {
-    if (FMT == TROCM_F16 && p.mask && GP <= 16 && use_16_wide(FMT))
+    if (FMT == TROCM_F16 && p.rope_cos)   // (the caller has checked: 16-wide tiles, no mask)
+        hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, (GP <= 16 ? GP : 16), TROCM_F16, false, true, 902>), grid, dim3(kThreads), 0, s, p);
+    else if (FMT == TROCM_F16 && p.mask && GP <= 16 && use_16_wide(FMT))
         hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, (GP <= 16 ? GP : 16), TROCM_F16, true, true>), grid, dim3(kThreads), 0, s, p);
     else if (FMT == TROCM_F16 && p.mask)
         hipLaunchKernelGGL((sdpa_decode_mfma_kernel<D, GP, TROCM_F16, true>), grid, dim3(kThreads), 0, s, p);
@@ -2069,6 +2139,11 @@ int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {
     p.k_new = (const char *)a.k_new, p.v_new = (const char *)a.v_new;
     p.new_pos = a.new_pos >= 0 ? (int)a.new_pos : (int)a.Sk - 1;
     if (p.k_new && (p.v_new == nullptr || (uintptr_t)p.k_new % 16 || (uintptr_t)p.v_new % 16)) return 2;
+    if (a.rope_cos) {   // q and k_new rotated on the way in: the 16-wide f16 body only
+        if (!a.rope_sin || a.mask || !p.k_new || gp > 16 || !use_16_wide(TROCM_F16)) return 2;
+        if ((uintptr_t)a.rope_cos % 16 || (uintptr_t)a.rope_sin % 16 || (a.rope_stride_b * 2) % 16) return 2;
+        p.rope_cos = (const char *)a.rope_cos, p.rope_sin = (const char *)a.rope_sin, p.rope_stride_b = a.rope_stride_b * 2;
+    }
     p.part_ml = (float *)((char *)a.workspace + kWsCounterBytes);
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * gp;
     static const int interleave = getenv("TROCM_DECODE_INTERLEAVE") ? atoi(getenv("TROCM_DECODE_INTERLEAVE")) : 1;

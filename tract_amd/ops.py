@@ -472,6 +472,38 @@ class InPlaceKvSdpaState:
              self._ws.ptr, self._ws.nbytes, _sh(stream))
         return out
 
+    def eval_rope_into(self, q: DeviceTensor, k_new: DeviceTensor, v_new: DeviceTensor, cos: DeviceTensor, sin: DeviceTensor,
+                       out: DeviceTensor | None = None, stream=None) -> DeviceTensor:
+        """ApplyRope on Q and K_new (Cos and Sin of shape [1 or batch, 1, n_new, head_dim]), then `eval`: one C call, and
+        for a single-token step on an f16 cache one launch."""
+        if not (q.dtype == k_new.dtype == v_new.dtype == cos.dtype == sin.dtype):
+            raise TractRocmError("input, cos and sin must share a datum type")
+        if tuple(cos.shape) != tuple(sin.shape):
+            raise TractRocmError("cos and sin must have the same shape")
+        B, Hq, Sq, D = _canon4(q.shape)
+        Hkv = _canon4(k_new.shape)[1]
+        cb = _canon4(cos.shape)
+        if cb[1] != 1 or cb[2] != Sq or cb[3] != D or cb[0] not in (1, B):
+            raise TractRocmError(f"cos / sin of shape {tuple(cos.shape)} do not broadcast against Q {tuple(q.shape)} over heads")
+        if self.k.handle is None:   # first chunk: the caches take their shape from it
+            rq = ApplyRope().eval(q, cos, sin, stream)
+            rk = ApplyRope().eval(k_new, cos, sin, stream)
+            return self.eval_into(rq, rk, v_new, out, stream)
+        self.k._check_push_shape(k_new.shape)
+        if out is None:
+            out = DeviceTensor(q.shape, q.dtype)
+        if self._ws is None or self._ws_key != (B, Hq, D) or self._ws.nbytes < Workspace.bytes_for(B, Hq, Sq, D):
+            self._ws, self._ws_key = Workspace(B, Hq, Sq, D, stream), (B, Hq, D)
+        es = np.dtype(q.dtype).itemsize
+        need = ((B * Hq * Sq * D * es + 255) & ~255) + B * Hkv * Sq * D * es
+        rot = getattr(self, "_rot", None)
+        if rot is None or rot.nbytes < need:
+            rot = self._rot = DeviceTensor((need,), np.uint8)
+        call("trocm_inplace_kv_sdpa_eval_rope", q.ptr, k_new.ptr, v_new.ptr, cos.ptr, sin.ptr, 0 if cb[0] == 1 else Sq * D,
+             dtype_code(q.dtype), Hq, Sq, self.k.handle, self.v.handle, out.ptr, _scale_arg(self.scale), int(self.causal),
+             self._ws.ptr, self._ws.nbytes, rot.ptr, rot.nbytes, _sh(stream))
+        return out
+
     def attend(self, q: DeviceTensor, stream=None, out: DeviceTensor | None = None) -> DeviceTensor:
         B, Hq, Sq, D = _canon4(q.shape)
         if out is None:
