@@ -1,6 +1,8 @@
 //! `InPlaceKvSdpa` and `WindowKvSdpa` on the device (transformers/src/ops/inplace_kv_cache.rs:131-290,
 //! window_kv_cache.rs:161-237): one stateful op, inputs `[Q, K_new, V_new]`, output Q-shaped.  The two caches
 //! never leave the state; a decode step is ONE launch that stores the new token and attends over the cache.
+//! With `rope` set the op has the inputs `[Q, K_new, V_new, Cos, Sin]` and stands for ApplyRope(Q), ApplyRope(K_new),
+//! InPlaceKvSdpa (the translator folds the two rotations in, transform.rs): still one launch per decode step.
 use std::os::raw::c_int;
 
 use tract_core::internal::*;
@@ -88,17 +90,24 @@ pub struct RocmInPlaceKvSdpa {
     pub scale_bits: Option<u32>, // f32 bits: the op must be Eq + Hash
     pub window: Option<usize>,
     pub storage: KvStorage,
+    /// Inputs 3 and 4 are Cos and Sin: Q and K_new are rotated (apply_rope.rs:169-176) before the append.
+    pub rope: bool,
 }
 
 pub type RocmWindowKvSdpa = RocmInPlaceKvSdpa;
 
 impl RocmInPlaceKvSdpa {
     pub fn from_inplace(op: &InPlaceKvSdpa, storage: KvStorage) -> Self {
-        Self { axis: op.axis, causal: op.causal, scale_bits: op.scale.map(f32::to_bits), window: None, storage }
+        Self { axis: op.axis, causal: op.causal, scale_bits: op.scale.map(f32::to_bits), window: None, storage, rope: false }
+    }
+    /// The same op with ApplyRope on Q and K_new folded in (growing f32 / f16 caches only).
+    pub fn with_rope(mut self) -> Self {
+        self.rope = true;
+        self
     }
     pub fn from_window(op: &WindowKvSdpa, storage: KvStorage) -> Self {
         // the ring buffer is the mask: window_kv_cache.rs:212-237 attends over every token it still holds
-        Self { axis: op.axis, causal: false, scale_bits: op.scale.map(f32::to_bits), window: Some(op.window), storage }
+        Self { axis: op.axis, causal: false, scale_bits: op.scale.map(f32::to_bits), window: Some(op.window), storage, rope: false }
     }
     fn scale(&self) -> Option<f32> {
         self.scale_bits.map(f32::from_bits)
@@ -107,10 +116,19 @@ impl RocmInPlaceKvSdpa {
 
 impl Op for RocmInPlaceKvSdpa {
     fn name(&self) -> StaticName {
-        if self.window.is_some() { "RocmWindowKvSdpa".into() } else { "RocmInPlaceKvSdpa".into() }
+        if self.window.is_some() {
+            "RocmWindowKvSdpa".into()
+        } else if self.rope {
+            "RocmRopeInPlaceKvSdpa".into()
+        } else {
+            "RocmInPlaceKvSdpa".into()
+        }
     }
     fn info(&self) -> TractResult<Vec<String>> {
-        Ok(vec![format!("axis={}, causal={}, scale={:?}, window={:?}, storage={:?}", self.axis, self.causal, self.scale(), self.window, self.storage)])
+        Ok(vec![format!(
+            "axis={}, causal={}, scale={:?}, window={:?}, storage={:?}, rope={}",
+            self.axis, self.causal, self.scale(), self.window, self.storage, self.rope
+        )])
     }
     op_as_typed_op!();
 }
@@ -121,13 +139,18 @@ impl EvalOp for RocmInPlaceKvSdpa {
     }
     fn state(&self, _session: &TurnState, node_id: usize) -> TractResult<Option<Box<dyn OpState>>> {
         ensure!(self.axis == 2, "tract-rocm caches grow along axis 2 of [B, H, S, D], got axis {}", self.axis);
-        Ok(Some(Box::new(RocmInPlaceKvSdpaState { node_id, op: self.clone(), k: None, v: None, workspace: Workspace::default() })))
+        ensure!(!self.rope || (self.window.is_none() && self.storage == KvStorage::AsInput), "the rotation is folded into growing f32 / f16 caches only");
+        Ok(Some(Box::new(RocmInPlaceKvSdpaState { node_id, op: self.clone(), k: None, v: None, workspace: Workspace::default(), rot_scratch: None })))
     }
 }
 
 impl TypedOp for RocmInPlaceKvSdpa {
     fn output_facts(&self, inputs: &[&TypedFact]) -> TractResult<TVec<TypedFact>> {
-        ensure!(inputs.len() == 3, "{} expects [Q, K_new, V_new]", self.name());
+        if self.rope {
+            ensure!(inputs.len() == 5, "{} expects [Q, K_new, V_new, Cos, Sin]", self.name());
+        } else {
+            ensure!(inputs.len() == 3, "{} expects [Q, K_new, V_new]", self.name());
+        }
         // Q's shape and dtype, as a device fact.  The caches are op state: nothing here is `state_owned`.
         tract_gpu::utils::facts_to_device_facts(inputs, |facts| Ok(tvec!(facts[0].without_value())))
             .with_context(|| format!("Error while computing facts for {:?}", self.name()))
@@ -142,12 +165,14 @@ pub struct RocmInPlaceKvSdpaState {
     k: Option<CacheHandle>,
     v: Option<CacheHandle>,
     workspace: Workspace,
+    /// `rope` only: where a call that has no fused kernel (several tokens, f32, one head per kv head) rotates Q and K_new
+    rot_scratch: Option<crate::tensor::RocmBuffer>,
 }
 
 impl Clone for RocmInPlaceKvSdpaState {
     fn clone(&self) -> Self {
         let dup = |c: &Option<CacheHandle>| c.as_ref().map(|c| c.try_clone().expect("cloning a device KV cache"));
-        Self { node_id: self.node_id, op: self.op.clone(), k: dup(&self.k), v: dup(&self.v), workspace: Workspace::default() }
+        Self { node_id: self.node_id, op: self.op.clone(), k: dup(&self.k), v: dup(&self.v), workspace: Workspace::default(), rot_scratch: None }
     }
 }
 
@@ -180,7 +205,7 @@ impl RocmInPlaceKvSdpaState {
 
 impl OpState for RocmInPlaceKvSdpaState {
     fn eval(&mut self, session: &mut TurnState, _op: &dyn Op, inputs: TVec<TValue>) -> TractResult<TVec<TValue>> {
-        ensure!(inputs.len() == 3, "{} expects [Q, K_new, V_new]", self.op.name());
+        ensure!(inputs.len() == if self.op.rope { 5 } else { 3 }, "{}: wrong number of inputs", self.op.name());
         let (q, k_new, v_new) = (inputs[0].to_device_tensor()?, inputs[1].to_device_tensor()?, inputs[2].to_device_tensor()?);
         ensure!(k_new.datum_type() == q.datum_type() && v_new.datum_type() == q.datum_type(), "Q, K and V of one type");
         ensure!(k_new.shape() == v_new.shape() && k_new.strides() == v_new.strides(), "K_new and V_new of one layout");
@@ -195,6 +220,39 @@ impl OpState for RocmInPlaceKvSdpaState {
         let (scale, causal, window) = (scale_arg(self.op.scale()), self.op.causal as c_int, self.op.window);
         let dt = dt_code(q.datum_type())?;
         let workspace = &mut self.workspace;
+        if self.op.rope {
+            // Cos and Sin: [1 or B, 1, n_new, D] of Q's type, dense (what an exported decoder slices out of its tables)
+            let (cos, sin) = (inputs[3].to_device_tensor()?, inputs[4].to_device_tensor()?);
+            ensure!(cos.datum_type() == q.datum_type() && sin.datum_type() == q.datum_type(), "Cos and Sin of Q's type");
+            ensure!(cos.shape() == sin.shape(), "Cos and Sin of one shape");
+            let [cb, ch, cn, cd] = bhsd(cos.shape())?;
+            ensure!(ch == 1 && cn == n_new && cd == d && (cb == 1 || cb == b), "Cos / Sin {:?} do not broadcast over the heads of Q {:?}", cos.shape(), q.shape());
+            for t in [cos, sin, k_new] {
+                ensure!(t.strides() == Tensor::natural_strides(t.shape()).as_slice(), "the rotating step takes dense operands");
+            }
+            let es = q.datum_type().size_of();
+            let q_room = ((b * hq * n_new * d) as usize * es + 255) & !255;
+            let need = q_room + (b * hkv * n_new * d) as usize * es;
+            if self.rot_scratch.as_ref().map(|r| r.len() < need).unwrap_or(true) {
+                // (an older, smaller scratch may still be read by launches in flight: drain the stream before it is dropped)
+                if self.rot_scratch.is_some() {
+                    with_rocm_stream(|s| s.synchronize())?;
+                }
+                self.rot_scratch = Some(crate::tensor::RocmBuffer::alloc(need)?);
+            }
+            let rot = self.rot_scratch.as_ref().unwrap();
+            let batch_stride = if cb == 1 { 0 } else { n_new * d };
+            with_rocm_stream(|s| {
+                let (ws, ws_bytes) = workspace.for_shape(b, hq, sq, d, s.raw())?;
+                ffi::check(unsafe {
+                    ffi::trocm_inplace_kv_sdpa_eval_rope(
+                        data_ptr(q), data_ptr(k_new), data_ptr(v_new), data_ptr(cos), data_ptr(sin), batch_stride, dt, hq, n_new, kc, vc,
+                        data_ptr(&out) as *mut _, scale, causal, ws, ws_bytes, rot.ptr_mut(), rot.len(), s.raw(),
+                    )
+                })
+            })?;
+            return Ok(tvec!(out.into_tensor().into_tvalue()));
+        }
         with_rocm_stream(|s| {
             let (ws, ws_bytes) = workspace.for_shape(b, hq, sq, d, s.raw())?;
             ffi::check(unsafe {

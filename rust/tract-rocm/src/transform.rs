@@ -38,6 +38,13 @@ tract_core::declare_knob!(
     "Comma-separated node-name substrings kept on the CPU."
 );
 
+tract_core::declare_knob!(
+    TRACT_ROCM_FUSE_ROPE,
+    bool,
+    true,
+    "Fold ApplyRope on Q and K_new into the fused cache + attention op when both rotations share their Cos and Sin."
+);
+
 fn kv_storage() -> TractResult<KvStorage> {
     match TRACT_ROCM_KV_FORMAT.get().as_str() {
         "" | "f16" | "f32" => Ok(KvStorage::AsInput),
@@ -77,11 +84,44 @@ impl RocmTransform {
             return Ok(());
         }
         *model = self.translate_model(model)?;
+        model.compact()?; // (drops the rotations whose work moved into a fused op)
         if stop_at_phase == 1 {
             return Ok(());
         }
         rewire_syncs(model)
     }
+}
+
+/// `InPlaceKvSdpa` whose Q and K_new both come out of `ApplyRope` nodes that share their Cos and Sin (what an exported
+/// decoder's attention block looks like, sdpa.rs:453-458): the outlets `[Q, K, V_new, Cos, Sin]` of the fused device op,
+/// Q and K as they enter the rotations.  The rotations must feed nothing else, or they would run anyway.
+fn rope_feeding(source: &TypedModel, node: &TypedNode) -> Option<TVec<OutletId>> {
+    let op = node.op_as::<InPlaceKvSdpa>()?;
+    if op.axis != 2 || kv_storage().ok()? != KvStorage::AsInput {
+        return None;
+    }
+    let (rq, rk) = (source.node(node.inputs[0].node), source.node(node.inputs[1].node));
+    if !rq.op_is::<ApplyRope>() || !rk.op_is::<ApplyRope>() || rq.id == rk.id {
+        return None;
+    }
+    if rq.inputs[1] != rk.inputs[1] || rq.inputs[2] != rk.inputs[2] {
+        return None;
+    }
+    if rq.outputs[0].successors.len() != 1 || rk.outputs[0].successors.len() != 1 {
+        return None;
+    }
+    if source.outputs.iter().any(|o| o.node == rq.id || o.node == rk.id) {
+        return None;
+    }
+    // Cos / Sin that broadcast over the heads: [1 or B, 1, S, D] against Q [B, H, S, D]
+    let (qf, cf) = (source.outlet_fact(rq.inputs[0]).ok()?, source.outlet_fact(rq.inputs[1]).ok()?);
+    if qf.rank() != 4 || cf.rank() != 4 || cf.shape[1] != 1.to_dim() || cf.shape[3] != qf.shape[3] || cf.shape[2] != qf.shape[2] {
+        return None;
+    }
+    if cf.shape[0] != 1.to_dim() && cf.shape[0] != qf.shape[0] {
+        return None;
+    }
+    Some(tvec!(rq.inputs[0], rk.inputs[0], node.inputs[2], rq.inputs[1], rq.inputs[2]))
 }
 
 /// The device op for `node`, or None when the node stays on the CPU.
@@ -142,6 +182,22 @@ impl Translate<TypedFact, Box<dyn TypedOp>, TypedFact, Box<dyn TypedOp>> for Roc
     ) -> TractResult<TVec<OutletId>> {
         // (constant inputs of a device op are uploaded by sync_inputs_if_required itself, gpu/src/sync.rs:117-128)
         let forced_cpu = TRACT_ROCM_FORCE_CPU.get().split(',').any(|pat| !pat.is_empty() && node.name.contains(pat));
+        // ApplyRope(Q), ApplyRope(K_new), InPlaceKvSdpa as one device op (one launch per decode step).  The two rotation
+        // nodes were translated when the walk passed them; with their only consumer gone they are dead and the
+        // compaction that follows the translation drops them.
+        if !forced_cpu && TRACT_ROCM_FUSE_ROPE.get() {
+            if let Some(fused_inputs) = rope_feeding(source, node) {
+                let facts: TVec<&TypedFact> = fused_inputs.iter().map(|o| source.outlet_fact(*o)).collect::<TractResult<_>>()?;
+                if facts.iter().all(|f| matches!(f.datum_type, DatumType::F32 | DatumType::F16)) && facts.iter().all(|f| f.datum_type == facts[0].datum_type) {
+                    let op = RocmInPlaceKvSdpa::from_inplace(node.op_as::<InPlaceKvSdpa>().unwrap(), KvStorage::AsInput).with_rope();
+                    let mut as_fused = node.clone();
+                    as_fused.inputs = fused_inputs;
+                    let inputs = sync_inputs_if_required(target, &as_fused, mapping, DeviceSyncKind::ToDevice)?;
+                    let outlets = target.wire_node(node.name.clone(), op, &inputs)?;
+                    return sync_model_outputs_if_required(source, node, target, outlets);
+                }
+            }
+        }
         let device_op = if forced_cpu { None } else { try_make_rocm_op(source, node)? };
         // The op must accept the facts it will really see: every input as a device fact (what the ToDevice syncs
         // produce).  An op that refuses them stays on the CPU instead of aborting the translation.
