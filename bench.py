@@ -663,9 +663,9 @@ def run_ops(ta, args):
     # the attention block of a decoder layer's step as an exported graph states it: ApplyRope on Q, ApplyRope on K_new,
     # InPlaceKvSdpa -- as three calls (three launches) and through the entry point that rotates both inside the attention
     # launch; cfg2's shape at 8192 tokens over 4 layers' caches, batch 8 and batch 1
-    for Bs in (8, 1):
+    for Bs, fmt, tag in ((8, None, ""), (1, None, ""), (8, ta.Q4_0, "_q4_0")):
         T0 = 8192
-        lay = [ta.InPlaceKvSdpa(axis=2, causal=True).state() for _ in range(4)]
+        lay = [ta.InPlaceKvSdpa(axis=2, causal=True, storage_format=fmt).state() for _ in range(4)]
         kk = rng.standard_normal((Bs, HKV, T0, D)).astype(np.float16)
         for st in lay:
             for c in (st.k, st.v):
@@ -708,7 +708,7 @@ def run_ops(ta, args):
         us3 = time_calls(ta, three_calls, 100)
         us1 = time_calls(ta, one_call, 100)
         us0 = time_calls(ta, plain_step, 100)
-        res[f"rope_rope_step_b{Bs}_ctx8192"] = {"three_calls_us": round(us3, 2), "fused_us": round(us1, 2), "step_without_rope_us": round(us0, 2),
+        res[f"rope_rope_step_b{Bs}_ctx8192{tag}"] = {"three_calls_us": round(us3, 2), "fused_us": round(us1, 2), "step_without_rope_us": round(us0, 2),
                                                 "note": "ApplyRope(Q), ApplyRope(K_new), InPlaceKvSdpa step: three launches against one"}
         del lay
     # mask inputs on the fast attention kernels: decode (batch 8, 8192 tokens, padding mask [8,1,1,T]) over

@@ -348,7 +348,8 @@ int trocm_inplace_kv_sdpa_eval(const void *q, const void *k_new, const void *v_n
  * dense as in trocm_inplace_kv_sdpa_eval; cos and sin are [n_new, head_dim] rows of `dtype` per sequence,
  * `cos_sin_batch_stride` elements apart (0: one set of rows for every sequence); v_new is not rotated.  The appended
  * keys and the output are bit-identical to trocm_apply_rope on q and k_new followed by trocm_inplace_kv_sdpa_eval.
- * A single-token step on an F16 cache with 2..16 query heads per kv head is one launch and touches no scratch;
+ * A single-token F16 step on an F16 cache with 2..16 query heads per kv head, or on a Q8_0 / Q4_0 cache (head_dim 128)
+ * with 2..8, is one launch and touches no scratch (the key is rotated before it is quantised);
  * every other call rotates into `rot_scratch` (16-byte aligned), which must then hold
  * round_up(batch * q_heads * n_new * head_dim * elem, 256) + batch * kv_heads * n_new * head_dim * elem bytes
  * (a call that needs it and finds it too small fails before anything is changed). */

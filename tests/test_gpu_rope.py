@@ -181,3 +181,31 @@ def test_rope_step_refused_for_its_scratch_changes_nothing(rt):
     assert st.k.len() == 33 and st.k.valid_contiguous().tobytes() == before
     got = st.eval_rope_into(dq, dk, dv, dc, ds).to_numpy()   # the same call with its scratch goes through
     assert st.k.len() == 37 and not np.isnan(got).any()
+
+
+@pytest.mark.parametrize("fmt_name", ["Q8_0", "Q4_0"])
+@pytest.mark.parametrize("B,Hq,Hkv,T0,per_sequence", [(2, 32, 8, 61, True), (1, 16, 2, 2050, False), (3, 12, 2, 30, True), (1, 10, 2, 127, True),
+                                                      (1, 32, 2, 40, False)])
+def test_rope_steps_over_quantised_caches(rt, fmt_name, B, Hq, Hkv, T0, per_sequence):
+    """The same over Q8_0 / Q4_0 caches: the key is rotated, then quantised, inside the attention launch (2..8 heads per kv
+    head; 16 heads per kv head rotate into the scratch).  The cache's canonical blocks are the CPU quantiser's blocks of the
+    oracle's rotated keys, the output equals the unfused sequence bit for bit."""
+    fmt = {"Q8_0": tract_amd.Q8_0, "Q4_0": tract_amd.Q4_0}[fmt_name]
+    orc_fmt = {"Q8_0": orc.FMT_Q8_0, "Q4_0": orc.FMT_Q4_0}[fmt_name]
+    D = 128
+    rng = np.random.default_rng(B * 100 + Hq + T0)
+    op = tract_amd.InPlaceKvSdpa(axis=2, causal=True, storage_format=fmt)
+    fused, plain = op.state(), op.state()
+    k0, v0 = rng.standard_normal((B, Hkv, T0, D)).astype(np.float16), rng.standard_normal((B, Hkv, T0, D)).astype(np.float16)
+    for st in (fused, plain):
+        st.k.push(k0), st.v.push(v0)
+    ks = k0
+    for step in range(4):
+        q, k, v, cos, sin = _rope_step_inputs(rng, B, Hq, Hkv, 1, D, np.float16, per_sequence)
+        got = fused.eval_rope_into(*(tract_amd.DeviceTensor.from_numpy(a) for a in (q, k, v, cos, sin))).to_numpy()
+        want = plain.eval([tract_amd.ApplyRope().eval(q, cos, sin), tract_amd.ApplyRope().eval(k, cos, sin), v]).to_numpy()
+        ks = np.concatenate([ks, orc.apply_rope(k, cos, sin)], axis=2)
+        assert fused.k.valid_contiguous().tobytes() == orc.quant(orc_fmt, ks).tobytes(), step
+        assert fused.v.valid_contiguous().tobytes() == plain.v.valid_contiguous().tobytes(), step
+        assert got.tobytes() == want.tobytes(), step
+    assert fused.k.len() == T0 + 4

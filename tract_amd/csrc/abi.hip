@@ -1323,7 +1323,7 @@ int trocm_inplace_kv_sdpa_eval_rope(const void *q, const void *k_new, const void
                   (long long)cos_sin_batch_stride, (long long)(n_new * kc->D));
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
-    if (n_new == 1 && dtype == TROCM_F16 && kc->fmt == TROCM_F16 && kc->window == 0 && vc->window == 0 && q_heads % kc->H == 0) {
+    if (n_new == 1 && dtype == TROCM_F16 && (kc->fmt == TROCM_F16 || is_quant(kc->fmt)) && kc->window == 0 && vc->window == 0 && q_heads % kc->H == 0) {
         if (equalise_capacities(kc, vc, s)) return 1;
         int64_t dense[4];
         dense[3] = 1, dense[2] = kc->D, dense[1] = kc->D, dense[0] = kc->H * kc->D;
@@ -1334,7 +1334,7 @@ int trocm_inplace_kv_sdpa_eval_rope(const void *q, const void *k_new, const void
             cached_args(a, q, dtype, q_heads, 1, kc, vc, kc->len + 1, out, scale, causal, workspace, workspace_bytes);
             a.k_new = k_new, a.v_new = v_new, a.new_pos = -1;
             a.rope_cos = cos, a.rope_sin = sin, a.rope_stride_b = cos_sin_batch_stride;
-            int rc = launch_sdpa_decode(a, s);
+            int rc = is_quant(kc->fmt) ? launch_sdpa_decode_quant(a, s) : launch_sdpa_decode(a, s);
             if (rc == 0) {
                 kc->len += 1;
                 vc->len += 1;

@@ -324,6 +324,7 @@ __global__ __launch_bounds__(D) void sdpa_decode_ragged_merge_kernel(DecodeDev p
 int decode_mfma_group(int64_t g_real);   // 0: not taken by the MFMA formulation
 int launch_sdpa_decode_quant_mfma(DecodeDev &p, int kv_fmt, int64_t B, void *workspace, size_t workspace_bytes, hipStream_t s);
 bool decode_quant_appends_in_kernel(int64_t g_real, float scale);
+bool decode_quant_rotates_in_kernel(int64_t g_real);
 int launch_sdpa_decode_ragged_mfma(const DecodeDev &p, int kv_fmt, int gp, int64_t D, const RaggedItem *items, int n_items,
                                    const RaggedSeqSlots *seqs, int n_seq, bool any_split, hipStream_t s);
 

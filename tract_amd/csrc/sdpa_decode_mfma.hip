@@ -153,8 +153,36 @@ __device__ __forceinline__ u32x4 rope_chunk(const char *row, const char *cosr, c
     const half8_t y = *reinterpret_cast<const half8_t *>(row + (first ? dc + CPR / 2 : dc - CPR / 2) * 16);
     const half8_t c = *reinterpret_cast<const half8_t *>(cosr + dc * 16), sn = *reinterpret_cast<const half8_t *>(sinr + dc * 16);
     half8_t a = x * c, b = (first ? -y : y) * sn;
-    asm volatile("" : "+v"(a), "+v"(b));
+    asm("" : "+v"(a), "+v"(b));   // (not volatile: several pieces' loads may be in flight together)
     return __builtin_bit_cast(u32x4, a + b);
+}
+
+// N consecutive elements (N = 4 or 8, not straddling the middle of the row) of a row of 128 halves, rotated the same way.
+template <int N>
+struct RopeRaw {
+    typedef _Float16 vec_t __attribute__((ext_vector_type(N)));
+    vec_t x, y, c, sn;   // the piece, its partner half a row away (sign applied), its cos and sin
+};
+template <int N>
+__device__ __forceinline__ RopeRaw<N> rope_load128(const _Float16 *row, const char *cosr, const char *sinr, int f0) {
+    typedef typename RopeRaw<N>::vec_t vec_t;
+    const bool first = f0 < 64;
+    RopeRaw<N> r;
+    r.x = *reinterpret_cast<const vec_t *>(row + f0);
+    const vec_t y = *reinterpret_cast<const vec_t *>(row + (first ? f0 + 64 : f0 - 64));
+    r.y = first ? -y : y;
+    r.c = *reinterpret_cast<const vec_t *>(cosr + 2 * f0), r.sn = *reinterpret_cast<const vec_t *>(sinr + 2 * f0);
+    return r;
+}
+template <int N>
+__device__ __forceinline__ typename RopeRaw<N>::vec_t rope_finish(const RopeRaw<N> &r) {
+    typename RopeRaw<N>::vec_t a = r.x * r.c, b = r.y * r.sn;
+    asm("" : "+v"(a), "+v"(b));   // (not volatile: volatile statements keep their order, and eight pieces would be eight round trips)
+    return a + b;
+}
+template <int N>
+__device__ __forceinline__ auto rope_piece128(const _Float16 *row, const char *cosr, const char *sinr, int f0) {
+    return rope_finish<N>(rope_load128<N>(row, cosr, sinr, f0));
 }
 
 template <int D, int GP, int FMT, bool MASK = false, bool W16 = false, bool ROPE = false>
@@ -592,7 +620,7 @@ __device__ __forceinline__ half8_t magic8(uint32_t w0, uint32_t w1) {
 // include the sequence's last one, exactly as the append kernel would (quant_block.h), written to the cache planes and
 // kept in `lds_new` (K codes, V codes, the K scales, the V scales), from where that wave's tile takes the row -- no other
 // wave of the launch reads it.  Lanes 0..3 take the four K blocks of the row, lanes 4..7 the V blocks.
-template <int FMT>
+template <int FMT, bool ROPE = false>
 __device__ __forceinline__ void quantise_new_token(const DecodeDev &p, const MfmaWork &wk, int lane, unsigned char *lds_new) {
     constexpr bool Q8 = FMT == TROCM_Q8_0;
     constexpr int D = 128, RB = Q8 ? D : D / 2, BB = Q8 ? 32 : 16, SROW = (D / 32) * 2;
@@ -603,7 +631,13 @@ __device__ __forceinline__ void quantise_new_token(const DecodeDev &p, const Mfm
         float v[32];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint4 x = reinterpret_cast<const uint4 *>(src)[i];
+            uint4 x = reinterpret_cast<const uint4 *>(src)[i];
+            if constexpr (ROPE) {   // the key is rotated (ApplyRope, rounded to f16) before it is quantised
+                if (!is_v) {
+                    const char *cs = p.rope_cos + (int64_t)wk.seq * p.rope_stride_b, *sn = p.rope_sin + (int64_t)wk.seq * p.rope_stride_b;
+                    x = __builtin_bit_cast(uint4, rope_piece128<8>(reinterpret_cast<const _Float16 *>(src) - 32 * blk, cs, sn, 32 * blk + 8 * i));
+                }
+            }
             const __half *e = reinterpret_cast<const __half *>(&x);
 #pragma unroll
             for (int j = 0; j < 8; j++) v[8 * i + j] = __half2float(e[j]);
@@ -1006,7 +1040,7 @@ __device__ __forceinline__ void nibbles8(const NibbleConsts &c, uint32_t w, uint
 // and x2 + swap1(x3) are the scores of tokens blk and 2 + blk: two additions per half instead of four, four
 // exponentials instead of eight.  The pairs (token j of the first half, of the second) are then handed round with four
 // quad broadcasts, which put token j's pair into register j of every lane.
-template <int GP, int FMT, int PF, int H = 4, bool RS = false>
+template <int GP, int FMT, int PF, int H = 4, bool RS = false, bool ROPE = false>
 __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const MfmaWork &wk) {
 
     static_assert(GP == 8, "partial records are 8 rows wide; with H = 4 rows 0..3 are used");
@@ -1086,18 +1120,28 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
     }
     const int tstep = wk.tile_step;
     int t = tile_begin + w;
-    if (new_pos >= 0) {   // (wave-uniform) the wave whose tiles include the new token's quantises and stores it
-        const int nt = new_pos / kTile;
-        if (nt >= t && nt < tile_end && (nt - t) % tstep == 0) quantise_new_token<FMT>(p, wk, lane, lds_new);
-    }
-#pragma unroll
-    for (int st = 0; st < PF; st++) {
-        kspre[st] = vspre[st] = u32x2{0u, 0u};
-        if (t + st * tstep < tile_end) {
-            fetch(wk.kbase, wk.ksbase, 0, t + st * tstep, kpre[st], kspre[st]);
-            fetch(wk.vbase, wk.vsbase, 1, t + st * tstep, vpre[st], vspre[st]);
+    auto new_token = [&]() {
+        if (new_pos >= 0) {   // (wave-uniform) the wave whose tiles include the new token's quantises and stores it
+            const int nt = new_pos / kTile;
+            if (nt >= t && nt < tile_end && (nt - t) % tstep == 0) quantise_new_token<FMT, ROPE>(p, wk, lane, lds_new);
         }
-    }
+    };
+    if constexpr (!ROPE) new_token();
+    auto first_tiles = [&]() {
+#pragma unroll
+        for (int st = 0; st < PF; st++) {
+            kspre[st] = vspre[st] = u32x2{0u, 0u};
+            if (t + st * tstep < tile_end) {
+                fetch(wk.kbase, wk.ksbase, 0, t + st * tstep, kpre[st], kspre[st]);
+                fetch(wk.vbase, wk.vsbase, 1, t + st * tstep, vpre[st], vspre[st]);
+            }
+        }
+    };
+    // (ROPE: the query's features are rotated as they are loaded, with the sequence's cos / sin rows; four loads per piece
+    // instead of one, asked for AHEAD of the first tiles: behind them they would arrive after two tiles of codes)
+    const char *cos_row = ROPE ? p.rope_cos + (int64_t)b * p.rope_stride_b : nullptr;
+    const char *sin_row = ROPE ? p.rope_sin + (int64_t)b * p.rope_stride_b : nullptr;
+    if constexpr (!ROPE) first_tiles();
 
     // Query operands, one per slice j: in the lanes of group blk_c the 8 features of slice j of block blk_c of head h_c,
     // zeros in the other lane groups.
@@ -1107,6 +1151,25 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
     half8_t qf[NX][NJ];
     float bias[NX];      // minus what the products add up for a block of all-zero-point codes
     const bool mine = qb == blk_c;
+    // ROPE: every piece's four loads first, then the first tiles', then the arithmetic (the loads return in order)
+    constexpr int NPC = Q8 ? 1 : 2;
+    RopeRaw<Q8 ? 8 : 4> raw[ROPE ? NX : 1][ROPE ? NJ : 1][NPC];
+    if constexpr (ROPE) {
+#pragma unroll
+        for (int X = 0; X < NX; X++)
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                const int sl = qs * NJ + j, f0 = 32 * (X * BPC + blk_c);
+                if constexpr (Q8) {
+                    raw[X][j][0] = rope_load128<8>(qrow, cos_row, sin_row, f0 + 8 * sl);
+                } else {
+                    raw[X][j][0] = rope_load128<4>(qrow, cos_row, sin_row, f0 + 4 * sl);
+                    raw[X][j][NPC - 1] = rope_load128<4>(qrow, cos_row, sin_row, f0 + 16 + 4 * sl);
+                }
+            }
+        new_token();   // (its own loads join the query's in flight)
+        first_tiles();
+    }
 #pragma unroll
     for (int X = 0; X < NX; X++) {
         float part = 0.0f;
@@ -1116,14 +1179,22 @@ __device__ __forceinline__ void decode_mfma_qdiag_body(const DecodeDev &p, const
             const int sl = qs * NJ + j;   // slice of the block
             half8_t f = {0, 0, 0, 0, 0, 0, 0, 0};
             if constexpr (Q8) {
-                const half8_t x = *reinterpret_cast<const half8_t *>(qblk + 8 * sl);
+                half8_t x;
+                if constexpr (ROPE && Q8) x = rope_finish<8>(raw[X][j][0]);
+                else x = *reinterpret_cast<const half8_t *>(qblk + 8 * sl);
                 float sum = 0.0f;
 #pragma unroll
                 for (int i = 0; i < 8; i++) sum += (float)x[i];
                 if (mine) f = x, part += 1152.0f * sum;   // the plane holds code + 128, under 1024
             } else {
-                const half4_t lo = *reinterpret_cast<const half4_t *>(qblk + 4 * sl);
-                const half4_t hi = *reinterpret_cast<const half4_t *>(qblk + 16 + 4 * sl);
+                half4_t lo, hi;
+                if constexpr (ROPE && !Q8) {
+                    lo = rope_finish<4>(raw[X][j][0]);
+                    hi = rope_finish<4>(raw[X][j][NPC - 1]);
+                } else {
+                    lo = *reinterpret_cast<const half4_t *>(qblk + 4 * sl);
+                    hi = *reinterpret_cast<const half4_t *>(qblk + 16 + 4 * sl);
+                }
                 half8_t x;
                 float s_lo = 0.0f, s_hi = 0.0f, s_hi16 = 0.0f;
 #pragma unroll
@@ -1791,7 +1862,7 @@ __device__ __forceinline__ int mask_row_len(const _Float16 *__restrict__ row, in
 // Dense batch: grid (splits, kv_heads, batch); every sequence has the same length.
 // QB: quantised caches on the 16-wide tiles run the body that scales per block outside the products.
 template <int D, int GP, int FMT, bool MASK = false, bool W16 = false, int QB = 0>
-__global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma_kernel(DecodeDev p) {   // QB = 100 * (1: diagonal, 2: affine u8, 3: diagonal with 8 heads across the columns, 4 / 5: 1 / 3 with the reduce-scatter, 9: the f16 body rotating q and k_new (RoPE)) + 10 * tiles ahead + workgroups per CU
+__global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma_kernel(DecodeDev p) {   // QB = 100 * (1: diagonal, 2: affine u8, 3: diagonal with 8 heads across the columns, 4 / 5: 1 / 3 with the reduce-scatter, 6 / 7: 4 / 5 rotating q and k_new (RoPE), 9: the f16 body doing so) + 10 * tiles ahead + workgroups per CU
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     MfmaWork wk;
     wk.seq = b, wk.kvh = kvh;
@@ -1831,7 +1902,7 @@ __global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma
     else if constexpr (QB / 100 == 2)
         decode_mfma_kivi_body<GP, (QB / 10) % 10>(p, wk);
     else if constexpr (QB >= 100)
-        decode_mfma_qdiag_body<GP, FMT, (QB / 10) % 10, (QB / 100 == 3 || QB / 100 == 5 ? 8 : 4), (QB / 100 >= 4)>(p, wk);
+        decode_mfma_qdiag_body<GP, FMT, (QB / 10) % 10, (QB / 100 == 3 || QB / 100 == 5 || QB / 100 == 7 ? 8 : 4), (QB / 100 >= 4), (QB / 100 >= 6)>(p, wk);
     else if constexpr (QB != 0)
         decode_mfma_qblock_body<GP, FMT, QB / 10>(p, wk);
     else
@@ -1861,7 +1932,7 @@ __global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma
     wk.part_first = (int64_t)it.slot0 * p.Hkv + kvh, wk.part_stride = p.Hkv;
     wk.mask = nullptr;
     if constexpr (QB >= 100)
-        decode_mfma_qdiag_body<GP, FMT, (QB / 10) % 10, (QB / 100 == 3 || QB / 100 == 5 ? 8 : 4), (QB / 100 >= 4)>(p, wk);
+        decode_mfma_qdiag_body<GP, FMT, (QB / 10) % 10, (QB / 100 == 3 || QB / 100 == 5 || QB / 100 == 7 ? 8 : 4), (QB / 100 >= 4), (QB / 100 >= 6)>(p, wk);
     else if constexpr (QB != 0)
         decode_mfma_qblock_body<GP, FMT, QB / 10>(p, wk);
     else
@@ -1910,6 +1981,13 @@ bool use_diagonal_rs() {
 template <int GP, int FMT>
 void launch_qblock(const DecodeDev &p, dim3 grid, hipStream_t s) {
     if constexpr (GP == 8) {
+        if (p.rope_cos) {   // (the caller has asked decode_quant_rotates_in_kernel)
+            if (p.g_real <= 4)
+                hipLaunchKernelGGL((sdpa_decode_mfma_kernel<128, GP, FMT, false, true, (FMT == TROCM_Q8_0 ? 612 : 622)>), grid, dim3(kThreads), 0, s, p);
+            else
+                hipLaunchKernelGGL((sdpa_decode_mfma_kernel<128, GP, FMT, false, true, (FMT == TROCM_Q8_0 ? 712 : 722)>), grid, dim3(kThreads), 0, s, p);
+            return;
+        }
         if (p.g_real <= 4 && use_diagonal()) {
             if (use_diagonal_rs())
                 hipLaunchKernelGGL((sdpa_decode_mfma_kernel<128, GP, FMT, false, true, (FMT == TROCM_Q8_0 ? 412 : 422)>), grid, dim3(kThreads), 0, s, p);
@@ -2035,6 +2113,13 @@ int launch_sdpa_decode_ragged_mfma(const DecodeDev &p, int kv_fmt, int gp, int64
 // Quantised cache planes (the caller has checked formats, alignment and strides and filled p but for the
 // splits): 2 = not taken (one head per kv head).
 // Whether the launch below would run one of the two bodies that take a step's new token from the step's inputs.
+// Whether a step over a quantised cache can rotate q and the new key inside the attention launch: the (head, block) bodies
+// with the reduce-scatter, i.e. up to 8 heads per kv head.
+bool decode_quant_rotates_in_kernel(int64_t g_real) {
+    return g_real >= 2 && g_real <= 8 && decode_mfma_group(g_real) == 8 && use_16_wide(TROCM_Q8_0) && use_block_scaling() && use_diagonal() &&
+           use_diagonal_pairs() && use_diagonal_rs();
+}
+
 bool decode_quant_appends_in_kernel(int64_t g_real, float scale) {
     static const int on = getenv("TROCM_DECODE_QUANT_FUSED_APPEND") ? atoi(getenv("TROCM_DECODE_QUANT_FUSED_APPEND")) : 1;
     const int gp = decode_mfma_group(g_real);

@@ -410,6 +410,10 @@ int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s) {
     if (a.k_new && (!mfma || !decode_quant_appends_in_kernel(g_real, a.scale) || a.v_new == nullptr || a.new_pos >= 0 ||
                     (uintptr_t)a.k_new % 16 || (uintptr_t)a.v_new % 16))
         return 2;
+    // q and the new key rotated on the way in: the (head, block) bodies of the MFMA formulation only
+    if (a.rope_cos && (!a.rope_sin || !a.k_new || !mfma || !decode_quant_rotates_in_kernel(g_real) || (uintptr_t)a.rope_cos % 16 ||
+                       (uintptr_t)a.rope_sin % 16 || (a.rope_stride_b * 2) % 16))
+        return 2;
     const int64_t G = g_real <= 2 ? g_real : g_real <= 4 ? 4 : 8;   // the instantiation that runs it
     if (a.kv_stride_t != a.D) return 2;  // cache planes: token rows are dense
     if ((uintptr_t)a.k % 16 || (uintptr_t)a.v % 16 || (uintptr_t)a.q % 16 || (uintptr_t)a.k_scales % 4 ||
@@ -434,8 +438,10 @@ int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s) {
         p.scale_log2 = a.scale * 1.4426950408889634f;
         p.k_new = (const char *)a.k_new, p.v_new = (const char *)a.v_new;
         p.new_pos = a.k_new ? (int)a.Sk - 1 : -1;
+        if (a.rope_cos) p.rope_cos = (const char *)a.rope_cos, p.rope_sin = (const char *)a.rope_sin, p.rope_stride_b = a.rope_stride_b * 2;
         return launch_sdpa_decode_quant_mfma(p, a.kv_fmt, a.B, a.workspace, a.workspace_bytes, s);
     }
+    if (a.rope_cos) return 2;
     int n_tiles = (int)((a.Sk + kTile - 1) / kTile);
     int nsplit = fit_decode_splits(choose_decode_splits(BH, G, n_tiles, 2), BH, G, a.D, a.workspace, a.workspace_bytes);
     int tps = (n_tiles + nsplit - 1) / nsplit;
