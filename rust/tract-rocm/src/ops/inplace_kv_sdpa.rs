@@ -100,7 +100,7 @@ impl RocmInPlaceKvSdpa {
     pub fn from_inplace(op: &InPlaceKvSdpa, storage: KvStorage) -> Self {
         Self { axis: op.axis, causal: op.causal, scale_bits: op.scale.map(f32::to_bits), window: None, storage, rope: false }
     }
-    /// The same op with ApplyRope on Q and K_new folded in (growing f32 / f16 caches only).
+    /// The same op with ApplyRope on Q and K_new folded in (growing caches of any storage format).
     pub fn with_rope(mut self) -> Self {
         self.rope = true;
         self
@@ -139,7 +139,7 @@ impl EvalOp for RocmInPlaceKvSdpa {
     }
     fn state(&self, _session: &TurnState, node_id: usize) -> TractResult<Option<Box<dyn OpState>>> {
         ensure!(self.axis == 2, "tract-rocm caches grow along axis 2 of [B, H, S, D], got axis {}", self.axis);
-        ensure!(!self.rope || (self.window.is_none() && self.storage == KvStorage::AsInput), "the rotation is folded into growing f32 / f16 caches only");
+        ensure!(!self.rope || self.window.is_none(), "the rotation is folded into growing caches only");
         Ok(Some(Box::new(RocmInPlaceKvSdpaState { node_id, op: self.clone(), k: None, v: None, workspace: Workspace::default(), rot_scratch: None })))
     }
 }

@@ -97,7 +97,7 @@ impl RocmTransform {
 /// Q and K as they enter the rotations.  The rotations must feed nothing else, or they would run anyway.
 fn rope_feeding(source: &TypedModel, node: &TypedNode) -> Option<TVec<OutletId>> {
     let op = node.op_as::<InPlaceKvSdpa>()?;
-    if op.axis != 2 || kv_storage().ok()? != KvStorage::AsInput {
+    if op.axis != 2 {
         return None;
     }
     let (rq, rk) = (source.node(node.inputs[0].node), source.node(node.inputs[1].node));
@@ -189,7 +189,7 @@ impl Translate<TypedFact, Box<dyn TypedOp>, TypedFact, Box<dyn TypedOp>> for Roc
             if let Some(fused_inputs) = rope_feeding(source, node) {
                 let facts: TVec<&TypedFact> = fused_inputs.iter().map(|o| source.outlet_fact(*o)).collect::<TractResult<_>>()?;
                 if facts.iter().all(|f| matches!(f.datum_type, DatumType::F32 | DatumType::F16)) && facts.iter().all(|f| f.datum_type == facts[0].datum_type) {
-                    let op = RocmInPlaceKvSdpa::from_inplace(node.op_as::<InPlaceKvSdpa>().unwrap(), KvStorage::AsInput).with_rope();
+                    let op = RocmInPlaceKvSdpa::from_inplace(node.op_as::<InPlaceKvSdpa>().unwrap(), kv_storage()?).with_rope();
                     let mut as_fused = node.clone();
                     as_fused.inputs = fused_inputs;
                     let inputs = sync_inputs_if_required(target, &as_fused, mapping, DeviceSyncKind::ToDevice)?;
