@@ -577,7 +577,7 @@ def run_kivi(ta, args):
         st.k.append(kq)
 
     res["prompt_push_running_keys_8x8x8192x128"] = {"us": round(time_calls(ta, prompt, 8), 2),
-                                                    "note": "chunked scan over 64-token chunks (three passes with 128-bit rows, two scans of the chunk results), incl. the reset of the running parameters; the scratch belongs to the store"}
+                                                    "note": "chunked scan over 64-token chunks (two passes with 128-bit rows, one scan of the chunk results between them), incl. the reset of the running parameters; the scratch belongs to the store"}
     q1_np = (seeded_f16(cfg_seed(2, "q") + 1, (B, HQ, 1, D)).astype(np.float32) / np.sqrt(D)).astype(np.float16)
     q1 = ta.DeviceTensor.from_numpy(q1_np)
     out = ta.DeviceTensor((B, HQ, 1, D), np.float16)

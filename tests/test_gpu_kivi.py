@@ -346,7 +346,8 @@ def test_running_key_store_prompt_push_with_128_bit_rows(rt, D, dt):
     B, H = 2, 3
     cache = kivi.KiviCache(kivi.KIVI_RUNNING_CHANNEL, 8, 0, B, H, D)
     refs = {(b, h): orc.KiviCache(True, running=True) for b in range(B) for h in (0, H - 1)}
-    for n, mag in ((3, 1.0), (700, 1.0), (1, 1.0), (257, 4.0), (1024, 0.2)):
+    # (chunk counts 11, 5, 16, 35 and 49: the scan of the chunk results walks whole groups of 16 chunks, pairs of groups, and a tail)
+    for n, mag in ((3, 1.0), (700, 1.0), (1, 1.0), (257, 4.0), (1024, 0.2), (2200, 1.0), (3100, 2.0)):
         x = (rng.standard_normal((B, H, n, D)) * mag).astype(dt)
         x[0, 0, n // 2, 3] = np.nan
         x[1, H - 1, n // 3, D - 1] = 0.0

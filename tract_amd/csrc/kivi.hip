@@ -307,6 +307,77 @@ __global__ void kivi_run_scan_scale_kernel(float *__restrict__ cmax, int D, int 
     }
     scale_io[(int64_t)bh * D + c] = scale;
 }
+// The 128-bit path makes one pass for both scans.  Per chunk and channel it leaves the first minimal value (`cmin`), the
+// largest value (`cmax`) and the widest range against the chunk's own running minimum (`cown`).  A token's range is
+// taken against the smaller of the incoming lo and the chunk's running minimum, i.e. it is the LARGER of RN(x - lo_in)
+// and RN(x - own minimum) (the subtraction grows as what is subtracted shrinks), so the chunk's widest range is
+// max(RN(cmax - lo_in), cown), its largest scale candidate RN(that / 255), and both running parameters of every chunk's
+// start come out of one walk over the chunks.  NaN values take part in nothing (every comparison with them is false),
+// exactly as in the token-by-token loop.  In place: cmin becomes the chunk's starting lo, cmax its starting scale.
+__global__ void kivi_run_scan_both_kernel(float *__restrict__ cmin, float *__restrict__ cmax, const float *__restrict__ cown, int D,
+                                          int n_chunks, float *__restrict__ lo_io, float *__restrict__ scale_io) {
+    const int bh = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= D) return;
+    float lo = lo_io[(int64_t)bh * D + c];
+    const float scale0 = scale_io[(int64_t)bh * D + c];
+    // The walk carries the widest RANGE so far, not the scale: the quotient by 255 grows with the range, so the largest
+    // quotient is the quotient of the widest range, and the divisions (one per chunk, for the scale its tokens start
+    // from) stay off the chain from chunk to chunk, which is a subtraction and two comparisons.  Sixteen chunks'
+    // results are in registers while the next sixteen are on their way.
+    float widest = 0.0f;
+    const int64_t base = (int64_t)bh * n_chunks * D + c;
+    constexpr int G = 16;
+    // (Whole groups of sixteen without a condition anywhere: a load or a store behind a condition becomes a branch, and the
+    // compiler then waits for every load where the paths meet.  The prefetch past the last group reads the last chunk again.)
+    float mn[2][G], mx[2][G], own[2][G];
+    auto load = [&](int k0, float (&a)[G], float (&b)[G], float (&o)[G]) {
+#pragma unroll
+        for (int i = 0; i < G; i++) {
+            const int64_t at = base + (int64_t)min(k0 + i, n_chunks - 1) * D;
+            a[i] = cmin[at], b[i] = cmax[at], o[i] = cown[at];
+        }
+    };
+    auto step = [&](float a, float b, float o, float &lo_in, float &w_in) {
+        lo_in = lo, w_in = widest;
+        const float r = __fsub_rn(b, lo);           // the chunk's largest value against the incoming lo
+        widest = r > widest ? r : widest;           // (a NaN range is never wider)
+        widest = o > widest ? o : widest;
+        lo = a < lo ? a : lo;
+    };
+    auto start_scale = [&](float w_in) {
+        const float ns = w_in > 0.0f ? __fdiv_rn(w_in, 255.0f) : 0.0f;
+        return ns > scale0 ? ns : scale0;
+    };
+    auto walk = [&](int k0, const float (&a)[G], const float (&b)[G], const float (&o)[G]) {
+        float lo_in[G], w_in[G];
+#pragma unroll
+        for (int i = 0; i < G; i++) step(a[i], b[i], o[i], lo_in[i], w_in[i]);
+#pragma unroll
+        for (int i = 0; i < G; i++) {
+            const int64_t at = base + (int64_t)(k0 + i) * D;
+            cmin[at] = lo_in[i], cmax[at] = start_scale(w_in[i]);
+        }
+    };
+    const int whole = n_chunks / G * G;
+    int k0 = 0;
+    if (whole > 0) load(0, mn[0], mx[0], own[0]);
+    for (; k0 + 2 * G <= whole; k0 += 2 * G) {
+        load(k0 + G, mn[1], mx[1], own[1]);
+        walk(k0, mn[0], mx[0], own[0]);
+        load(k0 + 2 * G, mn[0], mx[0], own[0]);
+        walk(k0 + G, mn[1], mx[1], own[1]);
+    }
+    if (k0 < whole) walk(k0, mn[0], mx[0], own[0]), k0 += G;
+    for (; k0 < n_chunks; k0++) {   // the chunks past the last whole group
+        const int64_t at = base + (int64_t)k0 * D;
+        float lo_in, w_in;
+        step(cmin[at], cmax[at], cown[at], lo_in, w_in);
+        cmin[at] = lo_in, cmax[at] = start_scale(w_in);
+    }
+    lo_io[(int64_t)bh * D + c] = lo;
+    const float ns = widest > 0.0f ? __fdiv_rn(widest, 255.0f) : 0.0f;
+    scale_io[(int64_t)bh * D + c] = ns > scale0 ? ns : scale0;
+}
 // pass 3: the codes, every chunk starting from its own parameters
 template <typename SrcT>
 __global__ void kivi_run_chunk_codes_kernel(const SrcT *__restrict__ src, int64_t S, int n, int D, int n_chunks,
@@ -402,13 +473,33 @@ __device__ __forceinline__ void store_codes8(uint8_t *row, int sub, const uint32
 template <typename SrcT, int LPR, int PASS>
 __global__ void __launch_bounds__(256) kivi_run_chunk_vec_kernel(const SrcT *__restrict__ src, int64_t S, int n, int n_chunks,
                                                                  float *__restrict__ a, float *__restrict__ b,
-                                                                 uint8_t *__restrict__ codes, int64_t cap_rows, int64_t row0) {
+                                                                 uint8_t *__restrict__ codes, int64_t cap_rows, int64_t row0,
+                                                                 float *__restrict__ c3 = nullptr) {
     constexpr int D = LPR * 8, CPW = 256 / LPR;
     const int bh = blockIdx.y, k = blockIdx.x * CPW + (int)threadIdx.x / LPR, sub = (int)threadIdx.x % LPR;
     if (k >= n_chunks) return;
     const int64_t at = ((int64_t)bh * n_chunks + k) * D + sub * 8;
     const int t0 = k * kRunChunk, t1 = min(n, t0 + kRunChunk);
     const SrcT *row = src + ((int64_t)bh * S + t0) * D + sub * 8;
+    if constexpr (PASS == 12) {   // one pass for both scans (kivi_run_scan_both_kernel): first minimum, maximum, widest own range
+        F8 mn, mx, own;
+#pragma unroll
+        for (int e = 0; e < 8; e++) mn.v[e] = INFINITY, mx.v[e] = -INFINITY, own.v[e] = 0.0f;
+#pragma unroll 4
+        for (int t = t0; t < t1; t++, row += D) {
+            const F8 x = ld8(row);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float val = x.v[e];
+                mn.v[e] = val < mn.v[e] ? val : mn.v[e];
+                mx.v[e] = val > mx.v[e] ? val : mx.v[e];
+                const float range = __fsub_rn(val, mn.v[e]);
+                own.v[e] = range > own.v[e] ? range : own.v[e];   // (a NaN range is never wider)
+            }
+        }
+        st8(a + at, mn), st8(b + at, mx), st8(c3 + at, own);
+        return;
+    }
     F8 lo, sc;
     if (PASS == 1) {
 #pragma unroll
@@ -422,40 +513,56 @@ __global__ void __launch_bounds__(256) kivi_run_chunk_vec_kernel(const SrcT *__r
     } else if (PASS == 3) {
         sc = ld8(b + at);
     }
-    // A channel's scale is the largest RN(range / 255) so far, and that quotient grows with the range: the division is
-    // only needed for a range larger than any before it (the same result as dividing every time).  The codes take the
-    // reciprocal of the scale with its re-check (affine_codes8), refreshed when the scale moves.
+    // A channel's scale is the largest RN(range / 255) so far, and that quotient grows with the range.  PASS 2 therefore
+    // keeps the widest range of the chunk (compare and select, no branch) and divides once at the end: the same value as
+    // the largest of the tokens' quotients.  PASS 3 needs the scale token by token, but only a range wider than any before
+    // it can move it, and none below 254.9 times the incoming scale can (its quotient is below that scale): `widest`
+    // starts there, and the division sits behind one branch per token that is taken when some lane of the wave has such
+    // a range in one of its 8 channels -- rarely, once the first tokens of the sequence have set the scale.  The codes
+    // take the reciprocal of the scale with its re-check (affine_codes8), refreshed when the scale moves.
     float widest[8];
     F8 inv;
 #pragma unroll
     for (int e = 0; e < 8; e++) {
-        widest[e] = 0.0f;
+        widest[e] = PASS == 3 ? sc.v[e] * 254.9f : 0.0f;
         inv.v[e] = PASS == 3 ? affine_inv(sc.v[e]) : 0.0f;
     }
 #pragma unroll 4
     for (int t = t0; t < t1; t++, row += D) {
         const F8 x = ld8(row);
+        bool wider = false;
+        float range[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             const float val = x.v[e];
-            if (val < lo.v[e]) lo.v[e] = val;
+            lo.v[e] = val < lo.v[e] ? val : lo.v[e];
             if (PASS >= 2) {
-                const float range = __fsub_rn(val, lo.v[e]);
-                if (range > widest[e]) {
-                    widest[e] = range;
-                    const float ns = __fdiv_rn(range, 255.0f);
-                    if (ns > sc.v[e]) {
-                        sc.v[e] = ns;
-                        if (PASS == 3) inv.v[e] = affine_inv(ns);
-                    }
-                }
+                range[e] = __fsub_rn(val, lo.v[e]);
+                if (PASS == 2) widest[e] = range[e] > widest[e] ? range[e] : widest[e];   // (a NaN range is never wider)
+                else wider = wider || range[e] > widest[e];
             }
         }
         if (PASS == 3) {
+            if (__builtin_amdgcn_ballot_w64(wider) != 0) {
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    if (range[e] > widest[e]) {
+                        widest[e] = range[e];
+                        const float ns = __fdiv_rn(range[e], 255.0f);
+                        if (ns > sc.v[e]) {
+                            sc.v[e] = ns;
+                            inv.v[e] = affine_inv(ns);
+                        }
+                    }
+            }
             uint32_t code[8];
             affine_codes8(x.v, lo.v, sc.v, inv.v, 255.0f, code);
             store_codes8<8>(codes + ((int64_t)bh * cap_rows + row0 + t) * D, sub, code);
         }
+    }
+    if (PASS == 2) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) sc.v[e] = widest[e] > 0.0f ? __fdiv_rn(widest[e], 255.0f) : 0.0f;
     }
     if (PASS == 1) st8(a + at, lo);
     if (PASS == 2) st8(b + at, sc);
@@ -851,7 +958,7 @@ static int kivi_prepare(trocm_kivi_cache *c, int64_t S, hipStream_t s) {
     if (c->layout == TROCM_KIVI_BLOCK_CHANNEL) rows = c->n_rows + (c->n_res + rem) / kKeyBlock * kKeyBlock;
     if (rows > c->n_rows && kivi_ensure_rows(c, rows, s)) return 1;
     if (kivi_prompt_scan(c, rem)) {
-        const size_t need = (size_t)c->BH * ((rem + kRunChunk - 1) / kRunChunk) * c->D * 2 * sizeof(float);
+        const size_t need = (size_t)c->BH * ((rem + kRunChunk - 1) / kRunChunk) * c->D * 3 * sizeof(float);   // (three results per chunk and channel on the 128-bit path)
         if (kivi_grow_buffer((void **)&c->scan, &c->scan_bytes, need, s, "the chunk results of a prompt")) return 1;
     }
     return 0;
@@ -934,10 +1041,8 @@ static int kivi_append_t(trocm_kivi_cache *c, const SrcT *src, int64_t S, hipStr
 #define KIVI_RUN_VEC(LPR)                                                                                                              \
     do {                                                                                                                               \
         const dim3 vgrid((unsigned)((n_chunks + 256 / LPR - 1) / (256 / LPR)), BH);                                                    \
-        kivi_run_chunk_vec_kernel<SrcT, LPR, 1><<<vgrid, 256, 0, s>>>(from, S, (int)rem, (int)n_chunks, tmp, tmp + plane, c->codes, c->cap_rows, c->n_rows); \
-        kivi_run_scan_min_kernel<<<scan, 64, 0, s>>>(tmp, D, (int)n_chunks, c->lo);                                                   \
-        kivi_run_chunk_vec_kernel<SrcT, LPR, 2><<<vgrid, 256, 0, s>>>(from, S, (int)rem, (int)n_chunks, tmp, tmp + plane, c->codes, c->cap_rows, c->n_rows); \
-        kivi_run_scan_scale_kernel<<<scan, 64, 0, s>>>(tmp + plane, D, (int)n_chunks, c->scale);                                      \
+        kivi_run_chunk_vec_kernel<SrcT, LPR, 12><<<vgrid, 256, 0, s>>>(from, S, (int)rem, (int)n_chunks, tmp, tmp + plane, c->codes, c->cap_rows, c->n_rows, tmp + 2 * plane); \
+        kivi_run_scan_both_kernel<<<scan, 64, 0, s>>>(tmp, tmp + plane, tmp + 2 * plane, D, (int)n_chunks, c->lo, c->scale);         \
         kivi_run_chunk_vec_kernel<SrcT, LPR, 3><<<vgrid, 256, 0, s>>>(from, S, (int)rem, (int)n_chunks, tmp, tmp + plane, c->codes, c->cap_rows, c->n_rows); \
     } while (0)
             if (vec) {
