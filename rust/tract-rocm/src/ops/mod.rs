@@ -2,6 +2,7 @@
 pub mod dyn_kv_cache;
 pub mod elementwise;
 pub mod inplace_kv_sdpa;
+pub mod q40_gemm;
 pub mod quant_kv;
 pub mod sdpa;
 
@@ -16,6 +17,7 @@ use crate::tensor::RocmBuffer;
 pub use dyn_kv_cache::RocmDynKVCache;
 pub use elementwise::{RocmApplyRope, RocmCast, RocmRotateHalf};
 pub use inplace_kv_sdpa::{RocmInPlaceKvSdpa, RocmWindowKvSdpa};
+pub use q40_gemm::{Q40DeviceWeights, RocmQ40Gemm};
 pub use quant_kv::{RocmQuantDynKVCache, RocmQuantizedKvSdpa};
 pub use sdpa::RocmSdpa;
 

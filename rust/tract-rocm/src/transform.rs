@@ -9,6 +9,8 @@ use std::collections::HashMap;
 use tract_core::internal::*;
 use tract_core::model::translator::Translate;
 use tract_core::ops::cast::Cast;
+use tract_core::ops::einsum::prefix_matmul::{rewrite_einsum_to_prefix_matmul, PrefixMatMul};
+use tract_core::tract_linalg::block_quant::Q4_0;
 use tract_core::transform::ModelTransform;
 use tract_gpu::fact::DeviceTypedFactExt;
 use tract_gpu::rewrite_rules::rewire_syncs::rewire_syncs;
@@ -75,6 +77,8 @@ impl RocmTransform {
         // {DynKeyValueCache(K), DynKeyValueCache(V), Sdpa} -> InPlaceKvSdpa, after the repeat-interleave of GQA has
         // been folded away (transformers/src/ops/inplace_kv_cache.rs:336-350).  Models whose caches were already
         // rewritten (window, KIVI) arrive with those ops in place and are left alone.
+        // matrix products as PrefixMatMul, the form in which the Q4_0-weight ones are recognised (cuda/src/transform.rs:92)
+        rewrite_einsum_to_prefix_matmul(model, false)?;
         Rewriter::default()
             .with_rule_for("fuse-kv-broadcast", fuse_kv_cache_broadcast_rule)
             .with_rule_for("fuse-inplace-kv-sdpa", fuse_inplace_kv_sdpa_rule)
@@ -182,6 +186,34 @@ impl Translate<TypedFact, Box<dyn TypedOp>, TypedFact, Box<dyn TypedOp>> for Roc
     ) -> TractResult<TVec<OutletId>> {
         // (constant inputs of a device op are uploaded by sync_inputs_if_required itself, gpu/src/sync.rs:117-128)
         let forced_cpu = TRACT_ROCM_FORCE_CPU.get().split(',').any(|pat| !pat.is_empty() && node.name.contains(pat));
+        // activations x constant Q4_0 weights [n, k] (PrefixMatMul with transpose_b, the shape exported decoders have,
+        // cuda/src/transform.rs:204-270): the weights go to the library now, the node keeps the activations as its input
+        if !forced_cpu {
+            if let Some(op) = node.op_as::<PrefixMatMul>() {
+                let facts = source.node_input_facts(node.id)?;
+                let weights = facts[1].konst.as_ref().filter(|_| tract_gpu::utils::as_quant_fact(facts[1], &Q4_0).is_some());
+                if let (Some(weights), true, false, true) = (
+                    weights,
+                    matches!(facts[0].datum_type, DatumType::F32 | DatumType::F16),
+                    op.transpose_a || op.transpose_c,
+                    op.transpose_b && op.quantize_output.is_none(),
+                ) {
+                    let device_op = RocmQ40Gemm { weights: Q40DeviceWeights::from_konst(weights)? };
+                    let mut as_unary = node.clone();
+                    as_unary.inputs = tvec!(node.inputs[0]);
+                    let inputs = sync_inputs_if_required(target, &as_unary, mapping, DeviceSyncKind::ToDevice)?;
+                    let mut outlets = target.wire_node(node.name.clone(), device_op, &inputs)?;
+                    // (the CPU op may promise another float type than the activations': cast, as the reference does at :287-297)
+                    let want = source.node_output_facts(node.id)?[0].datum_type;
+                    if want != facts[0].datum_type {
+                        if let Some(cast) = RocmCast::new(want) {
+                            outlets = target.wire_node(format!("{}.out_cast", node.name), cast, &outlets)?;
+                        }
+                    }
+                    return sync_model_outputs_if_required(source, node, target, outlets);
+                }
+            }
+        }
         // ApplyRope(Q), ApplyRope(K_new), InPlaceKvSdpa as one device op (one launch per decode step).  The two rotation
         // nodes were translated when the walk passed them; with their only consumer gone they are dead and the
         // compaction that follows the translation drops them.
