@@ -391,6 +391,18 @@ int trocm_inplace_kv_sdpa_eval_ragged(const void *q, const void *k_new, const vo
                                       trocm_kv_cache *const *v_caches, void *out, float scale,
                                       void *workspace, size_t workspace_bytes, void *stream);
 
+/* The same step with ApplyRope (apply_rope.rs:169-176) on q and k_new folded in, as trocm_inplace_kv_sdpa_eval_rope does
+ * for a dense batch: cos and sin are [n_seq, head_dim] rows of `dtype`, one per sequence (its position).  F16 steps over
+ * F16 caches with 2..16 query heads per kv head, and over Q8_0 / Q4_0 caches with 2..8, rotate inside the attention
+ * launch and touch no scratch; every other call rotates into `rot_scratch` (16-byte aligned,
+ * round_up(n_seq * q_heads * head_dim * elem, 256) + n_seq * kv_heads * head_dim * elem bytes) first, and is refused
+ * before anything changes when that is missing.  Bit-identical to trocm_apply_rope twice + the step above. */
+int trocm_inplace_kv_sdpa_eval_ragged_rope(const void *q, const void *k_new, const void *v_new, const void *cos,
+                                           const void *sin, int dtype, int64_t q_heads, int64_t n_seq,
+                                           trocm_kv_cache *const *k_caches, trocm_kv_cache *const *v_caches, void *out,
+                                           float scale, void *workspace, size_t workspace_bytes, void *rot_scratch,
+                                           size_t rot_scratch_bytes, void *stream);
+
 /* ---- KIVI-style affine quantised caches (the reference's own storage-quantised cache ops) ----------
  *
  * A different scheme from Q8_0 / Q4_0: u8 or u4 codes with f32 (lo, scale) parameters, Values per token,

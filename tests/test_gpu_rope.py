@@ -209,3 +209,38 @@ def test_rope_steps_over_quantised_caches(rt, fmt_name, B, Hq, Hkv, T0, per_sequ
         assert fused.v.valid_contiguous().tobytes() == plain.v.valid_contiguous().tobytes(), step
         assert got.tobytes() == want.tobytes(), step
     assert fused.k.len() == T0 + 4
+
+
+@pytest.mark.parametrize("fmt_name,Hq,Hkv,D", [("plain", 32, 8, 128), ("plain", 12, 2, 64), ("Q8_0", 32, 8, 128), ("Q4_0", 16, 2, 128),
+                                              ("plain", 8, 8, 128), ("Q4_0", 32, 2, 128)])
+def test_ragged_steps_with_rope(rt, fmt_name, Hq, Hkv, D):
+    """Independent sequences of different lengths, every one rotated by its own position's cos / sin: the ragged step with its
+    RoPE folded in (in the attention launch where a kernel rotates, through the scratch otherwise: one head per kv head, 16
+    heads per kv head over a quantised cache) equals ApplyRope twice + the plain ragged step bit for bit, caches included."""
+    fmt = {"plain": None, "Q8_0": tract_amd.Q8_0, "Q4_0": tract_amd.Q4_0}[fmt_name]
+    rng = np.random.default_rng(Hq + D)
+    lens = [1, 700, 33, 2049, 128, 5]
+    n = len(lens)
+
+    def caches():
+        ks, vs = [], []
+        for ln in lens:
+            kc, vc = tract_amd.InPlaceKvCache(2, fmt), tract_amd.InPlaceKvCache(2, fmt)
+            r = np.random.default_rng(ln)
+            kc.push(r.standard_normal((1, Hkv, ln, D)).astype(np.float16)), vc.push(r.standard_normal((1, Hkv, ln, D)).astype(np.float16))
+            ks.append(kc), vs.append(vc)
+        return ks, vs
+
+    (fk, fv), (pk, pv) = caches(), caches()
+    for step in range(3):
+        q = (rng.standard_normal((n, Hq, 1, D)) / np.sqrt(D)).astype(np.float16)
+        k, v = rng.standard_normal((n, Hkv, 1, D)).astype(np.float16), rng.standard_normal((n, Hkv, 1, D)).astype(np.float16)
+        ang = rng.uniform(-7, 7, (n, 1, 1, D))
+        cos, sin = np.cos(ang).astype(np.float16), np.sin(ang).astype(np.float16)
+        dq, dk, dv, dc, ds = (tract_amd.DeviceTensor.from_numpy(a) for a in (q, k, v, cos, sin))
+        got = tract_amd.inplace_kv_sdpa_eval_ragged_rope(dq, dk, dv, dc, ds, fk, fv).to_numpy()
+        want = tract_amd.inplace_kv_sdpa_eval_ragged(tract_amd.ApplyRope().eval(dq, dc, ds), tract_amd.ApplyRope().eval(dk, dc, ds), dv, pk, pv).to_numpy()
+        assert got.tobytes() == want.tobytes(), step
+        for a, b in zip(fk + fv, pk + pv):
+            assert a.valid_contiguous().tobytes() == b.valid_contiguous().tobytes(), step
+    assert fk[0].len() == 4

@@ -10,7 +10,7 @@ from ._lib import F16, F32, Q4_0, Q8_0, TractRocmError  # noqa: F401
 from .runtime import (DeviceTensor, Event, RocmRuntime, Stream, Workspace, runtime_for_name,  # noqa: F401
                       synchronize)
 from .ops import (ApplyRope, BlockQuant, Cast, GgmlGemm, Q40Weights, RotateHalf, DynKeyValueCache, DynKeyValueCacheState, InPlaceKvCache, KvPool,  # noqa: F401
-                  InPlaceKvSdpa, InPlaceKvSdpaState, Sdpa, StreamedSdpaOp, WindowKvCache, WindowKvSdpa, WindowKvSdpaState, Q4_0_FORMAT, Q8_0_FORMAT, inplace_kv_sdpa_eval_ragged,
+                  InPlaceKvSdpa, InPlaceKvSdpaState, Sdpa, StreamedSdpaOp, WindowKvCache, WindowKvSdpa, WindowKvSdpaState, Q4_0_FORMAT, Q8_0_FORMAT, inplace_kv_sdpa_eval_ragged, inplace_kv_sdpa_eval_ragged_rope,
                   sdpa_decode_ragged)
 from .kivi import (KiviCache, QuantizedDynKeyValueCache, QuantizedDynKvCacheState, QuantizedKvSdpa,  # noqa: F401
                    QuantizedKvSdpaState, KIVI_BLOCK_CHANNEL, KIVI_PER_TOKEN, KIVI_RUNNING_CHANNEL)

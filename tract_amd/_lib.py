@@ -88,6 +88,7 @@ SIGNATURES = {
     "trocm_kv_cache_window": [_vp, _pi64, _pi64],
     "trocm_window_kv_sdpa_eval": [_vp, _vp, _vp, _i, _i64, _i64, _pi64, _vp, _vp, _vp, _f, _vp, _sz, _vp],
     "trocm_inplace_kv_sdpa_eval": [_vp, _vp, _vp, _i, _i64, _i64, _pi64, _vp, _vp, _vp, _f, _i, _vp, _sz, _vp],
+    "trocm_inplace_kv_sdpa_eval_ragged_rope": [_vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, C.POINTER(_vp), C.POINTER(_vp), _vp, _f, _vp, _sz, _vp, _sz, _vp],
     "trocm_inplace_kv_sdpa_eval_rope": [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i64, _i64, _vp, _vp, _vp, _f, _i, _vp, _sz, _vp, _sz, _vp],
     "trocm_inplace_kv_sdpa_eval_ragged": [_vp, _vp, _vp, _i, _i64, _i64, C.POINTER(_vp), C.POINTER(_vp), _vp, _f, _vp,
                                           _sz, _vp],

@@ -1413,7 +1413,8 @@ int trocm_window_kv_sdpa_eval(const void *q, const void *k_new, const void *v_ne
 
 static int ragged_common(const void *q, const void *k_new, const void *v_new, int q_dtype, int64_t q_heads,
                          int64_t n_seq, trocm_kv_cache *const *k_caches, trocm_kv_cache *const *v_caches, void *out,
-                         float scale, void *workspace, size_t workspace_bytes, void *stream) {
+                         float scale, void *workspace, size_t workspace_bytes, void *stream, const void *rope_cos = nullptr,
+                         const void *rope_sin = nullptr, void *rot_scratch = nullptr, size_t rot_scratch_bytes = 0) {
     TROCM_NOT_NULL(q);
     TROCM_NOT_NULL(k_caches);
     TROCM_NOT_NULL(v_caches);
@@ -1446,6 +1447,33 @@ static int ragged_common(const void *q, const void *k_new, const void *v_new, in
     const size_t es = elem_bytes(q_dtype);
     int64_t dense[4] = {row_elems, k0->D, k0->D, 1};
     bool in_kernel = fused && (!is_quant(k0->fmt) || q_dtype == TROCM_F16);   // (quantised caches: f16 rows, quantised by the attention kernel)
+    // RoPE on q and k_new: inside the attention launch where a kernel does it, else into the caller's scratch first
+    const size_t rot_q_room = ((size_t)n_seq * q_heads * k0->D * es + 255) & ~(size_t)255;
+    const size_t rot_need = rot_q_room + (size_t)n_seq * row_elems * es;
+    auto rotate_into_scratch = [&]() -> int {
+        void *q_rot = rot_scratch, *k_rot = (char *)rot_scratch + rot_q_room;
+        const int64_t cs[4] = {k0->D, 0, k0->D, 1};
+        const int64_t qs[4] = {n_seq, q_heads, 1, k0->D}, ks[4] = {n_seq, k0->H, 1, k0->D};
+        if (trocm_apply_rope(q, rope_cos, rope_sin, q_rot, q_dtype, 4, qs, nullptr, cs, nullptr, stream)) return 1;
+        if (trocm_apply_rope(k_new, rope_cos, rope_sin, k_rot, q_dtype, 4, ks, nullptr, cs, nullptr, stream)) return 1;
+        q = q_rot, k_new = k_rot, rope_cos = rope_sin = nullptr;
+        return 0;
+    };
+    if (rope_cos) {
+        TROCM_REQUIRE(fused && rope_sin, "RoPE is folded into the step that appends (k_new, v_new, cos and sin)");
+        TROCM_REQUIRE(k0->D % 2 == 0, "apply_rope: the head dimension must be even");
+        // Whether a kernel takes the rotation is known when the launcher answers, after the caches may have grown: a call
+        // that could need the scratch and has none is refused here, before anything is changed.
+        const bool kernel_rotates = in_kernel && q_dtype == TROCM_F16 && q_heads % k0->H == 0 && q_heads / k0->H >= 2 &&
+                                    (k0->fmt == TROCM_F16 ? q_heads / k0->H <= 16 && (k0->D == 64 || k0->D == 128)
+                                                          : is_quant(k0->fmt) && decode_quant_rotates_in_kernel(q_heads / k0->H));
+        if (!kernel_rotates) {
+            TROCM_REQUIRE(rot_scratch != nullptr && rot_scratch_bytes >= rot_need && (uintptr_t)rot_scratch % 16 == 0,
+                          "ragged step with RoPE: this call rotates q and k_new into rot_scratch, which must be 16-byte aligned and hold %zu bytes (%zu given)",
+                          rot_need, rot_scratch_bytes);
+            if (rotate_into_scratch()) return 1;
+        }
+    }
     if (fused) {  // growth first (may reallocate), for every sequence
         for (int64_t i = 0; i < n_seq; i++) {
             const char *kn = (const char *)k_new + (size_t)i * row_elems * es, *vn = (const char *)v_new + (size_t)i * row_elems * es;
@@ -1493,11 +1521,17 @@ static int ragged_common(const void *q, const void *k_new, const void *v_new, in
         }
         int rc = launch_sdpa_decode_ragged(q, out, q_dtype, k0->fmt, n_seq, q_heads, k0->H, k0->D, seqs.data(), sc,
                                            workspace, workspace_bytes, in_kernel ? k_new : nullptr,
-                                           in_kernel ? v_new : nullptr, s);
+                                           in_kernel ? v_new : nullptr, s, in_kernel ? rope_cos : nullptr, in_kernel ? rope_sin : nullptr);
         if (rc == 0 && in_kernel)
             for (int64_t i = 0; i < n_seq; i++) k_caches[i]->len += 1, v_caches[i]->len += 1;
         if (rc != 2) return rc;
         if (!in_kernel) return fail("ragged decode: no kernel covers this shape");
+        if (rope_cos) {   // (alignment, a workspace too small ...) no kernel rotates after all: rotate first if there is room, then go on
+            if (rot_scratch == nullptr || rot_scratch_bytes < rot_need || (uintptr_t)rot_scratch % 16)
+                return fail("ragged step with RoPE: no kernel rotates for this call and rot_scratch does not hold %zu bytes", rot_need);
+            if (rotate_into_scratch()) return 1;
+            continue;
+        }
         // the kernel cannot append in place for this shape: append explicitly, then attend
         in_kernel = false;
         const bool at_once = is_quant(k0->fmt) && workspace != nullptr && workspace_bytes >= kWsCounterBytes + kWsPlanBytes &&
@@ -1520,6 +1554,19 @@ int trocm_inplace_kv_sdpa_eval_ragged(const void *q, const void *k_new, const vo
     TROCM_NOT_NULL(v_new);
     return ragged_common(q, k_new, v_new, dtype, q_heads, n_seq, k_caches, v_caches, out, scale, workspace,
                          workspace_bytes, stream);
+}
+
+// The ragged step with its RoPE folded in: cos and sin are [n_seq, head_dim] rows of `dtype` (each sequence's position).
+int trocm_inplace_kv_sdpa_eval_ragged_rope(const void *q, const void *k_new, const void *v_new, const void *cos, const void *sin,
+                                           int dtype, int64_t q_heads, int64_t n_seq, trocm_kv_cache *const *k_caches,
+                                           trocm_kv_cache *const *v_caches, void *out, float scale, void *workspace,
+                                           size_t workspace_bytes, void *rot_scratch, size_t rot_scratch_bytes, void *stream) {
+    TROCM_NOT_NULL(k_new);
+    TROCM_NOT_NULL(v_new);
+    TROCM_NOT_NULL(cos);
+    TROCM_NOT_NULL(sin);
+    return ragged_common(q, k_new, v_new, dtype, q_heads, n_seq, k_caches, v_caches, out, scale, workspace, workspace_bytes,
+                         stream, cos, sin, rot_scratch, rot_scratch_bytes);
 }
 
 }  // extern "C"

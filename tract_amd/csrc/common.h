@@ -169,6 +169,9 @@ int launch_sdpa_decode(const SdpaArgs &a, hipStream_t s);
 int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s);
 // Split-K decode over Q8_0 / Q4_0 caches with fused dequantisation.  Returns 2 when not covered.
 int launch_sdpa_decode_quant(const SdpaArgs &a, hipStream_t s);
+// Whether a step over a Q8_0 / Q4_0 cache with g_real query heads per kv head can rotate q and the new key (RoPE) inside the
+// attention launch (sdpa_decode_mfma.hip).
+bool decode_quant_rotates_in_kernel(int64_t g_real);
 // Split-K decode straight over the affine u8 stores of QuantizedKvSdpa (kv_quant.rs:105-236): Keys coded per channel
 // under one (lo, scale) per channel, Values per token.  f16 queries, head_dim 128, up to 16 query heads per kv head;
 // returns 2 when not covered.
@@ -199,9 +202,12 @@ struct RaggedSeq {
 };
 // k_new/v_new: optional fused append, dense [n_seq, Hkv, 1, D] (then seqs[i].len already counts
 // the new token).  Returns 2 when a fused append was asked for but the fast kernel does not apply.
+// rope_cos / rope_sin: with a fused append, rows [n_seq, D] of q_dtype by which q and k_new are rotated on the way in
+// (2 when no kernel that does so covers the shape).
 int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt, int64_t n_seq, int64_t Hq,
                               int64_t Hkv, int64_t D, const RaggedSeq *seqs, float scale, void *workspace,
-                              size_t workspace_bytes, const void *k_new, const void *v_new, hipStream_t s);
+                              size_t workspace_bytes, const void *k_new, const void *v_new, hipStream_t s,
+                              const void *rope_cos = nullptr, const void *rope_sin = nullptr);
 
 // Workspace layout: [arrival counters][partials ...]; a ragged launch keeps its plan (work items and
 // per-sequence slot ranges) between the two, so that the counters stay zero for whichever launch comes next:

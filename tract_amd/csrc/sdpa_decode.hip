@@ -648,7 +648,7 @@ int ragged_per_sequence(const void *q, void *out, int q_dtype, int kv_fmt, int64
 // head of the workspace, and the kernels index it by blockIdx.
 int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt, int64_t n_seq, int64_t Hq, int64_t Hkv,
                               int64_t D, const RaggedSeq *seqs, float scale, void *workspace, size_t workspace_bytes,
-                              const void *k_new, const void *v_new, hipStream_t s) {
+                              const void *k_new, const void *v_new, hipStream_t s, const void *rope_cos, const void *rope_sin) {
     const int64_t g_real = Hq / Hkv;
     // grouped heads over f16 or block-quantised caches: the MFMA formulation (sdpa_decode_mfma.hip)
     const bool quant = is_quant(kv_fmt);
@@ -670,6 +670,12 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
                    (uintptr_t)seqs[i].v_scales % 4 == 0;
     }
     if (k_new && ((uintptr_t)k_new % 16 || (uintptr_t)v_new % 16)) fast = false;
+    if (rope_cos) {   // q and k_new rotated on the way in: the 16-wide f16 body, or the (head, block) bodies over quantised caches
+        const bool covered = k_new && rope_sin && q_dtype == TROCM_F16 && mfma_gp != 0 && (uintptr_t)rope_cos % 16 == 0 &&
+                             (uintptr_t)rope_sin % 16 == 0 && (D * 2) % 16 == 0 &&
+                             (quant ? decode_quant_rotates_in_kernel(g_real) : kv_fmt == TROCM_F16 && mfma_gp <= 16);
+        if (!covered) return 2;
+    }
     if (!fast) {
         if (k_new) return 2;  // the caller appends explicitly, then calls again without a fused append
         return ragged_per_sequence(q, out, q_dtype, kv_fmt, n_seq, Hq, Hkv, D, seqs, scale, workspace, workspace_bytes, s);
@@ -767,6 +773,7 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     p.scale_log2 = scale * 1.4426950408889634f;
     p.k_new = (const char *)k_new;
     p.v_new = (const char *)v_new;
+    if (rope_cos) p.rope_cos = (const char *)rope_cos, p.rope_sin = (const char *)rope_sin, p.rope_stride_b = D * 2;
     p.part_ml = (float *)((char *)workspace + kWsCounterBytes + kWsPlanBytes);
     p.part_o = p.part_ml + (size_t)slot_it * Hkv * 2 * G;
     const RaggedItem *d_items = (const RaggedItem *)((char *)workspace + kWsCounterBytes);

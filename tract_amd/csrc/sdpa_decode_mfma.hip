@@ -1931,7 +1931,9 @@ __global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma
     wk.counter = p.counters ? p.counters + (int64_t)it.seq * p.Hkv + kvh : nullptr;
     wk.part_first = (int64_t)it.slot0 * p.Hkv + kvh, wk.part_stride = p.Hkv;
     wk.mask = nullptr;
-    if constexpr (QB >= 100)
+    if constexpr (QB / 100 == 9)
+        decode_mfma_body<D, GP, FMT, false, W16, true>(p, wk);
+    else if constexpr (QB >= 100)
         decode_mfma_qdiag_body<GP, FMT, (QB / 10) % 10, (QB / 100 == 3 || QB / 100 == 5 || QB / 100 == 7 ? 8 : 4), (QB / 100 >= 4), (QB / 100 >= 6)>(p, wk);
     else if constexpr (QB != 0)
         decode_mfma_qblock_body<GP, FMT, QB / 10>(p, wk);
@@ -2048,7 +2050,13 @@ int launch_quant(const DecodeDev &p, int gp, dim3 grid, hipStream_t s) {
 template <int D, int GP, int FMT = TROCM_F16>
 int launch_ragged_gp(const DecodeDev &p, const RaggedItem *items, int n_items, const RaggedSeqSlots *seqs, int n_seq,
                      bool any_split, hipStream_t s) {
-    if (FMT != TROCM_F16 && D == 128 && GP <= 16 && use_16_wide(FMT) && use_block_scaling() && p.scale_log2 > 0.0f)
+    if (p.rope_cos && FMT == TROCM_F16)   // (the caller has checked: 16-wide tiles)
+        hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<D, (GP <= 16 ? GP : 16), TROCM_F16, true, 902>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+    else if (p.rope_cos && GP == 8 && p.g_real <= 4)   // (... and decode_quant_rotates_in_kernel)
+        hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<128, 8, (FMT != TROCM_F16 ? FMT : TROCM_Q8_0), true, (FMT == TROCM_Q4_0 ? 622 : 612)>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+    else if (p.rope_cos && GP == 8)
+        hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<128, 8, (FMT != TROCM_F16 ? FMT : TROCM_Q8_0), true, (FMT == TROCM_Q4_0 ? 722 : 712)>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
+    else if (FMT != TROCM_F16 && D == 128 && GP <= 16 && use_16_wide(FMT) && use_block_scaling() && p.scale_log2 > 0.0f)
         if (GP == 8 && p.g_real <= 4 && use_diagonal() && use_diagonal_rs())
             hipLaunchKernelGGL((sdpa_decode_mfma_ragged_kernel<128, 8, (FMT != TROCM_F16 ? FMT : TROCM_Q8_0), true, (FMT == TROCM_Q4_0 ? 422 : 412)>), dim3(n_items, p.Hkv), dim3(kThreads), 0, s, p, items);
         else if (GP == 8 && p.g_real <= 4 && use_diagonal())

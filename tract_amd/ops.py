@@ -834,6 +834,34 @@ def inplace_kv_sdpa_eval_ragged(q: DeviceTensor, k_new: DeviceTensor, v_new: Dev
     return out
 
 
+def inplace_kv_sdpa_eval_ragged_rope(q: DeviceTensor, k_new: DeviceTensor, v_new: DeviceTensor, cos: DeviceTensor, sin: DeviceTensor,
+                                     k_caches, v_caches, scale=None, workspace: Workspace | None = None, stream=None,
+                                     out: DeviceTensor | None = None, rot_scratch: DeviceTensor | None = None) -> DeviceTensor:
+    """`inplace_kv_sdpa_eval_ragged` with ApplyRope on q and k_new folded in; cos and sin are [n_seq, 1, 1, head_dim] (every
+    sequence's own position)."""
+    n, Hq, _, D = q.shape
+    if len(k_caches) != n or len(v_caches) != n:
+        raise TractRocmError("ragged decode: one K and one V cache per sequence expected")
+    if k_new.shape != v_new.shape or k_new.shape[0] != n or k_new.shape[2] != 1:
+        raise TractRocmError("ragged decode: k_new / v_new must be [n_seq, kv_heads, 1, head_dim]")
+    if tuple(cos.shape) != tuple(sin.shape) or int(np.prod(cos.shape)) != n * D or cos.shape[0] != n or cos.shape[-1] != D:
+        raise TractRocmError("ragged decode with RoPE: cos and sin must be [n_seq, 1, 1, head_dim]")
+    if not (q.dtype == k_new.dtype == cos.dtype == sin.dtype):
+        raise TractRocmError("input, cos and sin must share a datum type")
+    if out is None:
+        out = DeviceTensor(q.shape, q.dtype)
+    ws = workspace or Workspace(n, Hq, 1, D, stream)
+    es = np.dtype(q.dtype).itemsize
+    need = ((n * Hq * D * es + 255) & ~255) + n * k_new.shape[1] * D * es
+    if rot_scratch is None:
+        rot_scratch = DeviceTensor((need,), np.uint8)
+    ks = (C.c_void_p * n)(*[c.handle for c in k_caches])
+    vs = (C.c_void_p * n)(*[c.handle for c in v_caches])
+    call("trocm_inplace_kv_sdpa_eval_ragged_rope", q.ptr, k_new.ptr, v_new.ptr, cos.ptr, sin.ptr, dtype_code(q.dtype), Hq, n, ks, vs,
+         out.ptr, _scale_arg(scale), ws.ptr, ws.nbytes, rot_scratch.ptr, rot_scratch.nbytes, _sh(stream))
+    return out
+
+
 def _broadcast_strides(x_shape, c_shape):
     """Element strides of a dense tensor of shape ``c_shape`` broadcast against ``x_shape``
     (0 on broadcast axes), for x's rank: cuda/src/kernels/utils.rs compute_broadcast_strides."""
