@@ -43,7 +43,14 @@ struct DecodeDev {
     // fused append with RoPE (f16, 16-wide tiles): cos / sin rows of D halves, one per sequence rope_stride_b bytes apart
     const char *rope_cos, *rope_sin;
     int64_t rope_stride_b;
+    // matrix-core kernels, 8-row records with at most 4 real heads, in-kernel merge of up to 8 splits: rows 4..7 are neither
+    // combined, stored nor merged (TROCM_DECODE_LIVE_TRIM=0 keeps them)
+    int live_trim;
 };
+inline int decode_live_trim() {
+    static const int on = getenv("TROCM_DECODE_LIVE_TRIM") ? atoi(getenv("TROCM_DECODE_LIVE_TRIM")) : 1;
+    return on;
+}
 
 // Ragged batches: one work item = a tile range of one sequence (device copies of the host plan).
 struct RaggedItem {
@@ -193,7 +200,9 @@ __device__ __forceinline__ void merge_head(const DecodeDev &p, int64_t first, in
 // (first, first + stride, ...; at most kTailMergeMax) with agent-scope loads and writes the G output
 // rows at `out`.  All loads of all splits are issued before the first use: one memory latency, not
 // one per split.  The counter is left at zero for the next launch.
-template <typename T, int D, int G>
+// LIVE: how many of a record's G rows are read (the rows of real heads come first; the matrix-core kernels pad their
+// groups, and with up to half the rows real they skip the rest).
+template <typename T, int D, int G, int LIVE = G>
 __device__ __forceinline__ void tail_merge(const DecodeDev &p, int *counter, int nsplit, int64_t first, int64_t stride,
                                            T *out, int tid) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's partial stores have completed
@@ -207,7 +216,7 @@ __device__ __forceinline__ void tail_merge(const DecodeDev &p, int *counter, int
     __syncthreads();
     if (!s_last) return;
     auto aload = [](const float *a) { return __hip_atomic_load(a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
-    constexpr int NE = (G * D + kThreads - 1) / kThreads;
+    constexpr int NE = (LIVE * D + kThreads - 1) / kThreads;
     float mv[NE][kTailMergeMax], lv[NE][kTailMergeMax], ov[NE][kTailMergeMax];
     const int64_t ml_step = stride * (2 * G), po_step = stride * (G * D);
 #pragma unroll

@@ -774,6 +774,7 @@ int launch_sdpa_decode_ragged(const void *q, void *out, int q_dtype, int kv_fmt,
     p.k_new = (const char *)k_new;
     p.v_new = (const char *)v_new;
     if (rope_cos) p.rope_cos = (const char *)rope_cos, p.rope_sin = (const char *)rope_sin, p.rope_stride_b = D * 2;
+    p.live_trim = decode_live_trim();
     p.part_ml = (float *)((char *)workspace + kWsCounterBytes + kWsPlanBytes);
     p.part_o = p.part_ml + (size_t)slot_it * Hkv * 2 * G;
     const RaggedItem *d_items = (const RaggedItem *)((char *)workspace + kWsCounterBytes);

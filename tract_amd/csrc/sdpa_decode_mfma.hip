@@ -95,7 +95,12 @@ __device__ __forceinline__ void wave_records_to_output(const DecodeDev &p, const
     __syncthreads();
     __half *out = reinterpret_cast<__half *>(p.out) + head0 * D;
     const int64_t slot = wk.slot;
-    for (int idx = tid; idx < GP * D; idx += kThreads) {
+    // Rows of padded heads are neither combined nor stored when at most half the rows are real.  The merges of up to
+    // kTailMergeMax splits then skip them too; the merge launch reads the rows of real heads only anyway; the wide merge
+    // reads every row (its loads carry no condition) and writes the real ones: what it finds in rows 4..7 goes nowhere.
+    const bool half_live = p.live_trim && GP == 8 && g <= GP / 2;
+    const int rows_end = half_live ? (GP / 2) * D : GP * D;
+    for (int idx = tid; idx < rows_end; idx += kThreads) {
         const int h = idx / D;
         float mm = -INFINITY;
 #pragma unroll
@@ -127,6 +132,8 @@ __device__ __forceinline__ void wave_records_to_output(const DecodeDev &p, const
     if constexpr (GP <= 8) {   // (larger groups: the merge launch; the in-kernel merge would need too many registers)
         if (wk.nsplit > kTailMergeMax && wk.counter != nullptr)
             tail_merge_wide<__half, D, GP>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid, reinterpret_cast<float *>(lds_raw));
+        else if (wk.nsplit > 1 && wk.counter != nullptr && half_live)
+            tail_merge<__half, D, GP, GP / 2>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
         else if (wk.nsplit > 1 && wk.counter != nullptr)
             tail_merge<__half, D, GP>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
     }
@@ -2146,6 +2153,7 @@ int launch_sdpa_decode_quant_mfma(DecodeDev &p, int kv_fmt, int64_t B, void *wor
     p.tiles_per_split = tps, p.nsplit = nsplit;
     static const int interleave = getenv("TROCM_DECODE_INTERLEAVE") ? atoi(getenv("TROCM_DECODE_INTERLEAVE")) : 1;
     p.interleave = interleave;
+    p.live_trim = decode_live_trim();
     p.part_ml = (float *)((char *)workspace + kWsCounterBytes);
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * gp;
     static const int tail = getenv("TROCM_DECODE_TAIL_MERGE") ? atoi(getenv("TROCM_DECODE_TAIL_MERGE")) : 1;
@@ -2183,6 +2191,7 @@ int launch_sdpa_decode_kivi(const KiviSdpaArgs &a, hipStream_t s) {
     p.new_pos = (int)a.T - 1;
     static const int interleave = getenv("TROCM_DECODE_INTERLEAVE") ? atoi(getenv("TROCM_DECODE_INTERLEAVE")) : 1;
     p.interleave = interleave;
+    p.live_trim = decode_live_trim();
     p.part_ml = (float *)((char *)a.workspace + kWsCounterBytes);
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * gp;
     static const int tail = getenv("TROCM_DECODE_TAIL_MERGE") ? atoi(getenv("TROCM_DECODE_TAIL_MERGE")) : 1;
@@ -2241,6 +2250,7 @@ int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * gp;
     static const int interleave = getenv("TROCM_DECODE_INTERLEAVE") ? atoi(getenv("TROCM_DECODE_INTERLEAVE")) : 1;
     p.interleave = interleave;
+    p.live_trim = decode_live_trim();
     if (a.mask) {   // [mask_b, mask_h, 1, Sk] dense f16
         p.mask = (const char *)a.mask;
         p.mask_stride_h = a.mask_h > 1 ? a.Sk * 2 : 0;
