@@ -200,9 +200,10 @@ __device__ __forceinline__ void merge_head(const DecodeDev &p, int64_t first, in
 // (first, first + stride, ...; at most kTailMergeMax) with agent-scope loads and writes the G output
 // rows at `out`.  All loads of all splits are issued before the first use: one memory latency, not
 // one per split.  The counter is left at zero for the next launch.
+// MAXS: the most splits this instantiation merges (nsplit <= MAXS).
 // LIVE: how many of a record's G rows are read (the rows of real heads come first; the matrix-core kernels pad their
 // groups, and with up to half the rows real they skip the rest).
-template <typename T, int D, int G, int LIVE = G>
+template <typename T, int D, int G, int LIVE = G, int MAXS = kTailMergeMax>
 __device__ __forceinline__ void tail_merge(const DecodeDev &p, int *counter, int nsplit, int64_t first, int64_t stride,
                                            T *out, int tid) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's partial stores have completed
@@ -217,7 +218,7 @@ __device__ __forceinline__ void tail_merge(const DecodeDev &p, int *counter, int
     if (!s_last) return;
     auto aload = [](const float *a) { return __hip_atomic_load(a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
     constexpr int NE = (LIVE * D + kThreads - 1) / kThreads;
-    float mv[NE][kTailMergeMax], lv[NE][kTailMergeMax], ov[NE][kTailMergeMax];
+    float mv[NE][MAXS], lv[NE][MAXS], ov[NE][MAXS];
     const int64_t ml_step = stride * (2 * G), po_step = stride * (G * D);
 #pragma unroll
     for (int e = 0; e < NE; e++) {
@@ -226,7 +227,7 @@ __device__ __forceinline__ void tail_merge(const DecodeDev &p, int *counter, int
         const float *ml = p.part_ml + first * (2 * G) + h;
         const float *po = p.part_o + first * (G * D) + idx;
 #pragma unroll
-        for (int sp = 0; sp < kTailMergeMax; sp++) {
+        for (int sp = 0; sp < MAXS; sp++) {
             const int spc = min(sp, nsplit - 1);   // splits past the last repeat it and get weight 0 below
             mv[e][sp] = aload(ml + spc * ml_step);
             lv[e][sp] = aload(ml + spc * ml_step + G);
@@ -238,11 +239,11 @@ __device__ __forceinline__ void tail_merge(const DecodeDev &p, int *counter, int
         const int idx = tid + e * kThreads;
         float mm = -INFINITY;
 #pragma unroll
-        for (int sp = 0; sp < kTailMergeMax; sp++) mm = fmaxf(mm, mv[e][sp]);
+        for (int sp = 0; sp < MAXS; sp++) mm = fmaxf(mm, mv[e][sp]);
         if (mm == -INFINITY) mm = 0.0f;   // a row masked out entirely with -inf: weights 0, not NaN
         float acc = 0.0f, ll = 0.0f;
 #pragma unroll
-        for (int sp = 0; sp < kTailMergeMax; sp++) {
+        for (int sp = 0; sp < MAXS; sp++) {
             const float f = sp < nsplit ? fast_exp2(mv[e][sp] - mm) : 0.0f;
             acc += ov[e][sp] * f;
             ll += lv[e][sp] * f;

@@ -132,6 +132,8 @@ __device__ __forceinline__ void wave_records_to_output(const DecodeDev &p, const
     if constexpr (GP <= 8) {   // (larger groups: the merge launch; the in-kernel merge would need too many registers)
         if (wk.nsplit > kTailMergeMax && wk.counter != nullptr)
             tail_merge_wide<__half, D, GP>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid, reinterpret_cast<float *>(lds_raw));
+        else if (wk.nsplit > 1 && wk.nsplit <= 4 && wk.counter != nullptr && half_live)   // (cfg2's shape: 4 splits of 4 heads)
+            tail_merge<__half, D, GP, GP / 2, 4>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
         else if (wk.nsplit > 1 && wk.counter != nullptr && half_live)
             tail_merge<__half, D, GP, GP / 2>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
         else if (wk.nsplit > 1 && wk.counter != nullptr)
