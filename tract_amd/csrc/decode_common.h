@@ -252,6 +252,66 @@ __device__ __forceinline__ void tail_merge(const DecodeDev &p, int *counter, int
     }
 }
 
+// tail_merge with two consecutive elements per thread: 64-bit agent-scope loads, half the instructions, and for 4 live
+// rows of 128 one element pair per thread.  The records must have been stored the same way (two floats at a time).
+template <typename T, int D, int G, int LIVE, int MAXS>
+__device__ __forceinline__ void tail_merge_pairs(const DecodeDev &p, int *counter, int nsplit, int64_t first, int64_t stride,
+                                                 T *out, int tid) {
+    static_assert(D % 2 == 0, "pairs of elements of one row");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's partial stores have completed
+    __syncthreads();                                     // ... and so have the whole workgroup's
+    __shared__ int s_last_pairs;
+    if (tid == 0) {
+        const int arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last_pairs = arrived == nsplit - 1;
+        if (s_last_pairs) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last_pairs) return;
+    auto aload = [](const float *a) { return __hip_atomic_load(a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    auto aload2 = [](const float *a) {
+        return __hip_atomic_load(reinterpret_cast<const uint64_t *>(a), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+    constexpr int NE = (LIVE * D + 2 * kThreads - 1) / (2 * kThreads);
+    float mv[NE][MAXS], lv[NE][MAXS];
+    uint64_t ov[NE][MAXS];
+    const int64_t ml_step = stride * (2 * G), po_step = stride * (G * D);
+#pragma unroll
+    for (int e = 0; e < NE; e++) {
+        const int idx = min(2 * (tid + e * kThreads), LIVE * D - 2);
+        const int h = idx / D;
+        const float *ml = p.part_ml + first * (2 * G) + h;
+        const float *po = p.part_o + first * (G * D) + idx;
+#pragma unroll
+        for (int sp = 0; sp < MAXS; sp++) {
+            const int spc = min(sp, nsplit - 1);   // splits past the last repeat it and get weight 0 below
+            mv[e][sp] = aload(ml + spc * ml_step);
+            lv[e][sp] = aload(ml + spc * ml_step + G);
+            ov[e][sp] = aload2(po + spc * po_step);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < NE; e++) {
+        const int idx = 2 * (tid + e * kThreads);
+        float mm = -INFINITY;
+#pragma unroll
+        for (int sp = 0; sp < MAXS; sp++) mm = fmaxf(mm, mv[e][sp]);
+        if (mm == -INFINITY) mm = 0.0f;   // a row masked out entirely with -inf: weights 0, not NaN
+        float acc0 = 0.0f, acc1 = 0.0f, ll = 0.0f;
+#pragma unroll
+        for (int sp = 0; sp < MAXS; sp++) {
+            const float f = sp < nsplit ? fast_exp2(mv[e][sp] - mm) : 0.0f;
+            acc0 += __builtin_bit_cast(float, (uint32_t)ov[e][sp]) * f;
+            acc1 += __builtin_bit_cast(float, (uint32_t)(ov[e][sp] >> 32)) * f;
+            ll += lv[e][sp] * f;
+        }
+        if (idx < p.g_real * D && idx < LIVE * D) {
+            out[idx] = from_f32<T>(ll > 0.0f ? acc0 / ll : 0.0f);
+            out[idx + 1] = from_f32<T>(ll > 0.0f ? acc1 / ll : 0.0f);
+        }
+    }
+}
+
 // The same for up to kWideMergeMax splits (small batches: 32 splits at batch 1), with G * kWideMergeMax <=
 // kThreads: thread (h, sp) loads the (m, l) record of head h in split sp and the 32 threads of a head reduce
 // them to weights, which go through `lds_w` (G * kWideMergeMax floats of LDS that nothing else uses any more);

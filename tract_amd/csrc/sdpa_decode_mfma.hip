@@ -100,29 +100,37 @@ __device__ __forceinline__ void wave_records_to_output(const DecodeDev &p, const
     // reads every row (its loads carry no condition) and writes the real ones: what it finds in rows 4..7 goes nowhere.
     const bool half_live = p.live_trim && GP == 8 && g <= GP / 2;
     const int rows_end = half_live ? (GP / 2) * D : GP * D;
-    for (int idx = tid; idx < rows_end; idx += kThreads) {
+    // two consecutive elements per thread: 64-bit LDS reads and 64-bit stores (the in-kernel merges of up to kTailMergeMax
+    // splits read the records the same way)
+    for (int idx = 2 * tid; idx < rows_end; idx += 2 * kThreads) {
         const int h = idx / D;
         float mm = -INFINITY;
 #pragma unroll
         for (int ww = 0; ww < kWaves; ww++) mm = fmaxf(mm, comb[ww * kCombStride + GP * D + h]);
         const float mm_ref = mm == -INFINITY ? 0.0f : mm;   // a wave without tiles holds (0, -inf, 0)
-        float acc = 0.0f, ll = 0.0f;
+        float acc0 = 0.0f, acc1 = 0.0f, ll = 0.0f;
 #pragma unroll
         for (int ww = 0; ww < kWaves; ww++) {
             const float f = fast_exp2(comb[ww * kCombStride + GP * D + h] - mm_ref);
-            acc += comb[ww * kCombStride + idx] * f;
+            const float2 o2 = *reinterpret_cast<const float2 *>(comb + ww * kCombStride + idx);
+            acc0 += o2.x * f, acc1 += o2.y * f;
             ll += comb[ww * kCombStride + GP * D + GP + h] * f;
         }
         if (wk.nsplit == 1) {
-            if (h < g) out[idx] = __float2half_rn(ll > 0.0f ? acc / ll : 0.0f);
+            if (h < g) {
+                const float inv = ll > 0.0f ? 1.0f : 0.0f;
+                out[idx] = __float2half_rn(inv != 0.0f ? acc0 / ll : 0.0f);
+                out[idx + 1] = __float2half_rn(inv != 0.0f ? acc1 / ll : 0.0f);
+            }
         } else if (wk.counter == nullptr) {
-            p.part_o[slot * (GP * D) + idx] = acc;
+            *reinterpret_cast<float2 *>(p.part_o + slot * (GP * D) + idx) = float2{acc0, acc1};
             if ((idx % D) == 0) {
                 p.part_ml[slot * (2 * GP) + h] = mm;
                 p.part_ml[slot * (2 * GP) + GP + h] = ll;
             }
         } else {   // write-through stores: visible device-wide when they complete (see tail_merge)
-            __hip_atomic_store(&p.part_o[slot * (GP * D) + idx], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint64_t both = (uint64_t)__builtin_bit_cast(uint32_t, acc0) | ((uint64_t)__builtin_bit_cast(uint32_t, acc1) << 32);
+            __hip_atomic_store(reinterpret_cast<uint64_t *>(p.part_o + slot * (GP * D) + idx), both, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if ((idx % D) == 0) {
                 __hip_atomic_store(&p.part_ml[slot * (2 * GP) + h], mm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 __hip_atomic_store(&p.part_ml[slot * (2 * GP) + GP + h], ll, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -133,11 +141,11 @@ __device__ __forceinline__ void wave_records_to_output(const DecodeDev &p, const
         if (wk.nsplit > kTailMergeMax && wk.counter != nullptr)
             tail_merge_wide<__half, D, GP>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid, reinterpret_cast<float *>(lds_raw));
         else if (wk.nsplit > 1 && wk.nsplit <= 4 && wk.counter != nullptr && half_live)   // (cfg2's shape: 4 splits of 4 heads)
-            tail_merge<__half, D, GP, GP / 2, 4>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
+            tail_merge_pairs<__half, D, GP, GP / 2, 4>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
         else if (wk.nsplit > 1 && wk.counter != nullptr && half_live)
-            tail_merge<__half, D, GP, GP / 2>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
+            tail_merge_pairs<__half, D, GP, GP / 2, kTailMergeMax>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
         else if (wk.nsplit > 1 && wk.counter != nullptr)
-            tail_merge<__half, D, GP>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
+            tail_merge_pairs<__half, D, GP, GP, kTailMergeMax>(p, wk.counter, wk.nsplit, wk.part_first, wk.part_stride, out, tid);
     }
 }
 
