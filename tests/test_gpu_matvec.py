@@ -54,12 +54,64 @@ def test_matvec_matches_the_oracle(rt, dt, wb, ab, m, n, k):
         assert rel_err(got, orc.q4_0_matvec(blocks, act).astype(np.float64)) <= tol
 
 
+# Weights whose rows are a multiple of 16 and whose features a multiple of 128 are held as tiles of 16 rows x 128
+# features: one wave per row group and k share (1, 2, 4 or 8 shares by the matrix's size), activations whole in LDS or
+# in chunks (8 rows of 14336 features, 16 of 8192), row groups that do not fill a workgroup's set, several rounds per
+# workgroup (20000 rows x 128 features), batches that share weights, and more than 16 rows (the matrix-matrix kernel
+# reading tiles; 17 rows of f32 in groups of 8).
+TILED_SHAPES = [
+    (1, 1, 1, 16, 128), (1, 1, 1, 48, 256), (2, 2, 1, 80, 384), (1, 3, 2, 4096, 1024), (1, 1, 1, 14336, 4096), (1, 1, 3, 4096, 14336),
+    (1, 1, 8, 14336, 4096), (1, 1, 8, 4096, 14336), (1, 1, 16, 1040, 8192), (2, 4, 5, 272, 2176), (1, 1, 7, 20000, 128),
+    (1, 1, 12, 6000 * 16, 256), (1, 1, 17, 160, 640), (1, 2, 40, 4112, 1152), (1, 1, 130, 2048, 4096),
+]
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+@pytest.mark.parametrize("wb,ab,m,n,k", TILED_SHAPES)
+def test_tiled_weights_match_the_f64_product(rt, dt, wb, ab, m, n, k):
+    rng = np.random.default_rng(n + k + m)
+    w = (rng.standard_normal((wb, n, k)) * 0.05).astype(np.float32)
+    w[:, :, ::97] *= 8.0
+    act = rng.standard_normal((ab, m, k)).astype(dt)
+    blocks = orc.quant(Q4, w)
+    wq = tract_amd.Q40Weights(blocks, wb, n, k)
+    assert np.array_equal(wq.blocks(), blocks)              # the tiles give the canonical bytes back
+    got = tract_amd.GgmlGemm().eval(act, wq).to_numpy()
+    assert got.dtype == dt and got.shape == (ab, m, n)
+    tol = 1e-4 if dt == np.float32 else 4e-3
+    assert rel_err(got, f64_product(blocks, act, dt)) <= tol
+
+
+def test_tiles_and_planes_hold_the_same_weights(rt, monkeypatch):
+    """The same matrix as tiles and (TROCM_Q4_TILED=0 at creation) as planes of codes and scales: equal exports, and
+    products that agree to the tolerance of either."""
+    rng = np.random.default_rng(5)
+    n, k = 2048, 1024
+    w = (rng.standard_normal((1, n, k)) * 0.05).astype(np.float32)
+    blocks = orc.quant(Q4, w)
+    tiles = tract_amd.Q40Weights(blocks, 1, n, k)
+    monkeypatch.setenv("TROCM_Q4_TILED", "0")
+    planes = tract_amd.Q40Weights(blocks, 1, n, k)
+    monkeypatch.delenv("TROCM_Q4_TILED")
+    assert np.array_equal(tiles.blocks(), planes.blocks())
+    for dt, tol in ((np.float16, 4e-3), (np.float32, 1e-4)):
+        for m in (1, 6, 24):
+            act = rng.standard_normal((1, m, k)).astype(dt)
+            a = tract_amd.GgmlGemm().eval(act, tiles).to_numpy()
+            b = tract_amd.GgmlGemm().eval(act, planes).to_numpy()
+            assert rel_err(a, b.astype(np.float64)) <= 2 * tol
+            assert rel_err(a, f64_product(blocks, act, dt)) <= tol
+
+
+@pytest.mark.parametrize("tiled", [1, 0])
 @pytest.mark.parametrize("m,k", [(16, 3584), (8, 4096)])
-def test_tall_matrix_of_repeated_rows(rt, m, k):
+def test_tall_matrix_of_repeated_rows(rt, monkeypatch, m, k, tiled):
     """65536 weight rows (the output matrix of a large vocabulary), built by repeating 512 quantised rows: every
-    workgroup walks several row groups behind one staged copy of the activations.  16 rows of 3584 features
-    leave the waves no LDS for their code buffers (the kernel that loads 64 bytes per row and transposes over the
-    lane groups runs), 8 rows do.  Expected: the f64 product of the 512 rows, repeated."""
+    workgroup walks several row groups behind one staged copy of the activations, as tiles and as planes of codes
+    and scales.  As planes, 16 rows of 3584 features leave the waves no LDS for their code buffers (the kernel that
+    loads 64 bytes per row and transposes over the lane groups runs), 8 rows do.  Expected: the f64 product of the
+    512 rows, repeated."""
+    monkeypatch.setenv("TROCM_Q4_TILED", str(tiled))
     rng = np.random.default_rng(m + k)
     base_n, reps = 512, 128
     w = (rng.standard_normal((1, base_n, k)) * 0.05).astype(np.float32)

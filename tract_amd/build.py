@@ -28,7 +28,7 @@ COMMON = [
 # per-file extra flags: the quantiser must not contract a*b+c into an fma
 EXTRA = {"kv_quant.hip": ["-ffp-contract=off"], "elementwise.hip": ["-ffp-contract=off"], "kivi.hip": ["-ffp-contract=off"]}
 SOURCES = ["abi.hip", "copy.hip", "kv_quant.hip", "sdpa_generic.hip", "sdpa_decode.hip", "sdpa_decode_quant.hip",
-           "sdpa_prefill.hip", "sdpa_prefill_pp.hip", "elementwise.hip", "dat_format.hip", "q4_matvec.hip", "q4_matvec_mfma.hip", "q4_matmul.hip", "sdpa_decode_mfma.hip", "kivi.hip"]
+           "sdpa_prefill.hip", "sdpa_prefill_pp.hip", "elementwise.hip", "dat_format.hip", "q4_matvec.hip", "q4_matvec_mfma.hip", "q4_matmul.hip", "q4_tiled.hip", "sdpa_decode_mfma.hip", "kivi.hip"]
 
 
 def _newer(target: str, deps: list[str]) -> bool:

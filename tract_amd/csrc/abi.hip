@@ -896,6 +896,7 @@ int trocm_kv_cache_raw(const trocm_kv_cache *c, void **data, void **scales, int6
 struct trocm_q4_weights {
     int64_t batch, n, k;
     void *codes, *scales;   // [batch * n, k/2] bytes and [batch * n, k/32] f16
+    int tiled;              // codes = tiles of 16 rows x 128 features with their scales (q4_tiled.hip), scales = NULL
 };
 
 extern "C" {
@@ -916,16 +917,21 @@ int trocm_q4_0_weights_create(trocm_q4_weights **out, const void *blocks, int64_
     TROCM_REQUIRE(w != nullptr, "out of host memory");
     w->batch = batch, w->n = n, w->k = k;
     const int64_t rows = batch * n;
-    hipError_t e = hipMalloc(&w->codes, (size_t)rows * (size_t)(k / 2));
-    if (e == hipSuccess) e = hipMalloc(&w->scales, (size_t)rows * (size_t)(k / 32) * 2);
+    // The matrices of a decoder (rows a multiple of 16, features of 128) are tiled for the matrix instruction;
+    // TROCM_Q4_TILED=0 (read at every call) keeps the planes of codes and scales for them too.
+    const char *tiled_env = getenv("TROCM_Q4_TILED");
+    w->tiled = q4_0_tiled_layout_fits(n, k) && !(tiled_env && atoi(tiled_env) == 0);
+    hipError_t e = hipMalloc(&w->codes, w->tiled ? q4_0_tiled_bytes(rows, k) : (size_t)rows * (size_t)(k / 2));
+    if (e == hipSuccess && !w->tiled) e = hipMalloc(&w->scales, (size_t)rows * (size_t)(k / 32) * 2);
     if (e != hipSuccess) {
         if (w->codes) (void)hipFree(w->codes);
         delete w;
         return fail("q4_0 weights: hipMalloc failed: %s", hipGetErrorString(e));
     }
-    if (launch_quant_import(TROCM_Q4_0, 1, 1, rows, rows, 0, k, blocks, w->codes, w->scales, s)) {
+    if (w->tiled ? launch_q4_0_tiled_import(blocks, w->codes, rows, k, s)
+                 : launch_quant_import(TROCM_Q4_0, 1, 1, rows, rows, 0, k, blocks, w->codes, w->scales, s)) {
         (void)hipFree(w->codes);
-        (void)hipFree(w->scales);
+        if (w->scales) (void)hipFree(w->scales);
         delete w;
         return 1;
     }
@@ -937,7 +943,7 @@ int trocm_q4_0_weights_destroy(trocm_q4_weights *w) {
     if (!w) return 0;
     TROCM_HIP(hipDeviceSynchronize());
     TROCM_HIP(hipFree(w->codes));
-    TROCM_HIP(hipFree(w->scales));
+    if (w->scales) TROCM_HIP(hipFree(w->scales));
     delete w;
     return 0;
 }
@@ -956,6 +962,7 @@ int trocm_q4_0_weights_export(const trocm_q4_weights *w, void *dst_blocks, void 
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
     const int64_t rows = w->batch * w->n;
+    if (w->tiled) return launch_q4_0_tiled_export(w->codes, dst_blocks, rows, w->k, s);
     return launch_quant_export(TROCM_Q4_0, 1, 1, rows, rows, w->k, w->codes, w->scales, dst_blocks, s);
 }
 
@@ -973,6 +980,7 @@ int trocm_q4_0_matvec(const trocm_q4_weights *w, const void *act, int act_dtype,
     TROCM_REQUIRE((uintptr_t)act % 16 == 0, "q4_0_matvec: activations must be 16-byte aligned");
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
+    if (w->tiled) return launch_q4_0_tiled_matvec(w->codes, w->batch, w->n, w->k, act, act_dtype, act_batch, m, out, s);
     return launch_q4_0_matvec(w->codes, w->scales, w->batch, w->n, w->k, act, act_dtype, act_batch, m, out, s);
 }
 

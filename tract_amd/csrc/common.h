@@ -132,8 +132,17 @@ int launch_q4_0_matvec(const void *codes, const void *scales, int64_t w_batch, i
 int launch_q4_0_matvec_mfma(const void *codes, const void *scales, int64_t w_batch, int64_t n, int64_t k, const void *act,
                             int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s);
 // The same product for m > 8 rows of f16 activations on the matrix cores.  Returns 2 when not covered.
+// tiled: `codes` are tiles of 16 rows x 128 features (q4_tiled.hip), `scales` is unused.
 int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, int64_t n, int64_t k, const void *act,
-                       int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s);
+                       int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s, int tiled = 0);
+// Q4_0 weights tiled by 16 rows x 128 features (n a multiple of 16, k of 128): the layout, its inverse, and the product
+// with m rows of f16 or f32 activations (q4_tiled.hip).
+bool q4_0_tiled_layout_fits(int64_t n, int64_t k);
+size_t q4_0_tiled_bytes(int64_t rows, int64_t k);
+int launch_q4_0_tiled_import(const void *blocks, void *tiles, int64_t rows, int64_t k, hipStream_t s);
+int launch_q4_0_tiled_export(const void *tiles, void *blocks, int64_t rows, int64_t k, hipStream_t s);
+int launch_q4_0_tiled_matvec(const void *tiles, int64_t w_batch, int64_t n, int64_t k, const void *act, int act_dtype,
+                             int64_t act_batch, int64_t m, void *out, hipStream_t s);
 
 // Attention.  One description for every kernel.
 struct SdpaArgs {

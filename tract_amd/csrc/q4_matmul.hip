@@ -29,14 +29,15 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kMmThreads = 256;
 constexpr int BN = 128, BK = 64;   // (the tile's m extent BM is 128, or 64 when 128 would leave compute units without a tile)
 constexpr int ROW = BK + 8;   // halves per tile row in LDS: the 16 rows of a 128-bit read pass fall into 16 distinct bank groups
 
 struct MatMulDev {
-    const uint8_t *codes;     // [w_batch, n, k/2]
-    const uint16_t *scales;   // [w_batch, n, k/32]
+    const uint8_t *codes;     // [w_batch, n, k/2]; TILED: [w_batch, n / 16, k / 128] records of 1152 bytes (q4_tiled.hip)
+    const uint16_t *scales;   // [w_batch, n, k/32]; TILED: unused (the scales are in the records)
     const _Float16 *act;      // [act_batch, m, k]
     _Float16 *out;            // [act_batch, m, n]
     int n, k, m, ratio;       // ratio = act_batch / w_batch
@@ -52,7 +53,7 @@ __device__ __forceinline__ void dequant4(uint32_t w, half2_t d2, uint32_t &lo, u
     hi = __builtin_bit_cast(uint32_t, (as_half2(perm(0x64646464u, w, 0x04030402u)) - zero) * d2);
 }
 
-template <int BM>
+template <int BM, bool TILED>
 __global__ __launch_bounds__(kMmThreads, 2) void q4_0_matmul_kernel(MatMulDev p) {
     constexpr int MJ = BM / 64;        // 32-row halves of m per wave: the wave's corner is 64 (n) x 32 MJ (m)
     constexpr int AP = BM * 8 / kMmThreads;   // 16-byte activation pieces per thread and chunk
@@ -78,16 +79,54 @@ __global__ __launch_bounds__(kMmThreads, 2) void q4_0_matmul_kernel(MatMulDev p)
         a_row[j] = c >> 3, a_col[j] = (c & 7) * 8;
     }
 
+    // TILED: a chunk is one half (blocks 2 hh, 2 hh + 1) of a tile of each of the 8 row groups of the workgroup's 128
+    // rows; this thread stages slot `lane` (row lane % 16, bytes 4 g .. 4 g + 3 of each block, g = lane / 16) of row
+    // groups w and w + 4: 8 bytes of codes and two scales each.
+    const int t_r = lane & 15, t_g = lane >> 4;
+    const uint8_t *t_rec[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const int64_t grp = (int64_t)wb * (p.n / 16) + min(n0 / 16 + w + 4 * h, p.n / 16 - 1);   // groups past the end repeat the last one
+        t_rec[h] = p.codes + grp * (p.k / 128) * 1152;
+    }
+    u32x2 tpre[2];
+    uint32_t tspre[2];
+
     u32x4 cpre, apre[AP];
     uint16_t spre;
     auto prefetch = [&](int k0) {
-        cpre = *reinterpret_cast<const u32x4 *>(w_codes + (k0 / 32) * 16);
-        spre = w_scales[k0 / 32];
+        if constexpr (TILED) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const uint8_t *rec = t_rec[h] + (int64_t)(k0 / 128) * 1152;
+                tpre[h] = *reinterpret_cast<const u32x2 *>(rec + 16 * lane + 8 * ((k0 / 64) & 1));
+                tspre[h] = *reinterpret_cast<const uint32_t *>(rec + 1024 + 8 * t_r + 4 * ((k0 / 64) & 1));
+            }
+        } else {
+            cpre = *reinterpret_cast<const u32x4 *>(w_codes + (k0 / 32) * 16);
+            spre = w_scales[k0 / 32];
+        }
 #pragma unroll
         for (int j = 0; j < AP; j++)
             apre[j] = *reinterpret_cast<const u32x4 *>(a_base + (int64_t)min(m0 + a_row[j], p.m - 1) * p.k + k0 + a_col[j]);
     };
     auto stage = [&](int buf) {
+        if constexpr (TILED) {
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int jj = 0; jj < 2; jj++) {
+                    const _Float16 d = __builtin_bit_cast(_Float16, (uint16_t)(tspre[h] >> (16 * jj)));
+                    const half2_t d2 = {d, d};
+                    const uint32_t word = tpre[h][jj];
+                    uint32_t lo0, lo1, hi0, hi1;   // elements 4 g .. 4 g + 3 and 16 + 4 g .. 16 + 4 g + 3 of block jj of the chunk
+                    dequant4(word & 0x0F0F0F0Fu, d2, lo0, lo1);
+                    dequant4((word >> 4) & 0x0F0F0F0Fu, d2, hi0, hi1);
+                    _Float16 *dst = &lds_w[buf][((w + 4 * h) * 16 + t_r) * ROW + jj * 32 + 4 * t_g];
+                    *reinterpret_cast<u32x2 *>(dst) = u32x2{lo0, lo1};
+                    *reinterpret_cast<u32x2 *>(dst + 16) = u32x2{hi0, hi1};
+                }
+        } else {
         const _Float16 d = __builtin_bit_cast(_Float16, spre);
         const half2_t d2 = {d, d};
         const uint32_t cw[4] = {cpre.x, cpre.y, cpre.z, cpre.w};
@@ -102,6 +141,7 @@ __global__ __launch_bounds__(kMmThreads, 2) void q4_0_matmul_kernel(MatMulDev p)
         dst[1] = u32x4{lo[4], lo[5], lo[6], lo[7]};
         dst[2] = u32x4{hi[0], hi[1], hi[2], hi[3]};
         dst[3] = u32x4{hi[4], hi[5], hi[6], hi[7]};
+        }
 #pragma unroll
         for (int j = 0; j < AP; j++) *reinterpret_cast<u32x4 *>(&lds_a[buf][a_row[j] * ROW + a_col[j]]) = apre[j];
     };
@@ -173,7 +213,7 @@ __global__ __launch_bounds__(kMmThreads, 2) void q4_0_matmul_kernel(MatMulDev p)
 // 2 = not taken (the caller runs the rows in groups of 8 on the vector-ALU kernel): f32 activations (their products
 // stay in f32 there), k that is not a whole number of 64-element chunks, misaligned operands.
 int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, int64_t n, int64_t k, const void *act,
-                       int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s) {
+                       int act_dtype, int64_t act_batch, int64_t m, void *out, hipStream_t s, int tiled) {
     static const int enabled = getenv("TROCM_Q4_MATMUL") ? atoi(getenv("TROCM_Q4_MATMUL")) : 1;
     if (!enabled || act_dtype != TROCM_F16 || m <= 8 || k % BK != 0) return 2;
     if ((uintptr_t)codes % 16 || (uintptr_t)act % 16 || (uintptr_t)out % 8) return 2;
@@ -188,10 +228,15 @@ int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, i
     const bool half_m = gx * ((m + 127) / 128) * act_batch < num_compute_units() && m > 64;
     const int64_t gy = half_m ? (m + 63) / 64 : (m + 127) / 128;
     if (gy > 65535) return 2;
-    if (half_m)
-        hipLaunchKernelGGL(q4_0_matmul_kernel<64>, dim3((unsigned)gx, (unsigned)gy, (unsigned)act_batch), dim3(kMmThreads), 0, s, p);
+    const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)act_batch);
+    if (tiled && half_m)
+        hipLaunchKernelGGL((q4_0_matmul_kernel<64, true>), grid, dim3(kMmThreads), 0, s, p);
+    else if (tiled)
+        hipLaunchKernelGGL((q4_0_matmul_kernel<128, true>), grid, dim3(kMmThreads), 0, s, p);
+    else if (half_m)
+        hipLaunchKernelGGL((q4_0_matmul_kernel<64, false>), grid, dim3(kMmThreads), 0, s, p);
     else
-        hipLaunchKernelGGL(q4_0_matmul_kernel<128>, dim3((unsigned)gx, (unsigned)gy, (unsigned)act_batch), dim3(kMmThreads), 0, s, p);
+        hipLaunchKernelGGL((q4_0_matmul_kernel<128, false>), grid, dim3(kMmThreads), 0, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("q4_0_matmul launch failed: %s", hipGetErrorString(e));
     return 0;

@@ -1,0 +1,536 @@
+// Q4_0 weights in tiles of 16 rows x 128 features, and their products with a few activation rows: gfx950.
+//
+//   out[b, i, j] = sum_k act[b, i, k] * dequant(W[b / ratio, j, k])
+//
+// the matrix-vector arm of GgmlGemm (cuda/src/kernels/matmul/mod.rs:575-627) for weights whose row count is a
+// multiple of 16 and whose row length is a multiple of 128: the matrices of a decoder.
+//
+// Layout.  The weights are constant, so they are laid out once, at load time, in the order in which the matrix
+// instruction consumes them.  Tile (G, t) = rows 16 G .. 16 G + 15, features 128 t .. 128 t + 127 (4 blocks per row)
+// is one record of 1152 bytes, the records of a row group consecutive in t:
+//   bytes [0, 1024): slot l = r + 16 g (r = row in the group, g = 0..3) holds 16 bytes: word j = code bytes
+//                    4 g .. 4 g + 3 of block 4 t + j of the row, i.e. its elements 4 g .. 4 g + 3 (low nibbles) and
+//                    16 + 4 g .. 16 + 4 g + 3 (high nibbles) -- what lane l feeds v_mfma_f32_16x16x32_f16 as the B
+//                    operand of block j;
+//   bytes [1024, 1152): the f16 scales [r][j].
+// A wave's loads are then one 128-bit and one 64-bit load per lane and tile, from nine consecutive cache lines of
+// which every byte is used: a load instruction costs the compute unit's address path one step per cache line it
+// touches, and rows of the [n, k/2] code plane put every lane group of a load on 16 different lines.
+// trocm_q4_0_weights_export undoes the layout: the canonical 18-byte blocks come back unchanged.
+//
+// f16 activations, 1..16 rows (q4_0_tiled_mfma_kernel): KS waves share the tiles of a row group (wave q takes
+// tiles q, q + KS, ...), a workgroup of 8 waves holds 8 / KS row groups behind one staged copy of the activations and
+// walks `rounds` such sets.  Every wave keeps a ring of PD tiles in flight that runs on across the end of a round into
+// the next round's first tiles, so that neither the reduction over the KS waves nor the barrier in front of it leaves
+// the memory pipe idle.  Arithmetic: the contraction of the instruction is 32 deep, one quantisation block; the codes
+// enter as the exact f16 integers -8 .. 7, the products accumulate in f32 inside the instruction from zero, and the
+// block's sum is scaled by its f16 scale with one fma per output.
+//
+// f32 activations, 1..8 rows (q4_0_tiled_vec_f32_kernel): the same tiles on the vector ALU, products and sums in f32
+// (the codes are exact in f32), one wave per row group, lane (r, g) the 32 weights of its slot per tile.
+//
+// Roofline: HBM-bound on the weights: 18 bytes per 32 weights, read once.
+#include <hip/hip_fp16.h>
+#include <string.h>
+#include <stdlib.h>
+#include <type_traits>
+#include "common.h"
+
+namespace trocm {
+namespace {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kTile = 1152;        // bytes per tile record
+constexpr int kTileScales = 1024;  // offset of the scales in a record
+constexpr int kW = 8;              // waves per workgroup of the f16 kernel
+
+// ---- layout ---------------------------------------------------------------------------------------------------------
+// Canonical blocks [rows, nb, 18 bytes] (f16 scale, 16 code bytes; 2-byte aligned) <-> tiles.  One thread per block.
+__global__ __launch_bounds__(256) void q4_0_tiled_import_kernel(const uint16_t *__restrict__ src, uint8_t *__restrict__ tiles,
+                                                                int64_t rows, int64_t nb) {
+    const int64_t total = rows * nb, T = nb / 4;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t blk = idx % nb, row = idx / nb;
+        const int r = (int)(row % 16), j = (int)(blk % 4);
+        uint8_t *rec = tiles + ((row / 16) * T + blk / 4) * kTile;
+        const uint16_t *i16 = src + idx * 9;
+        *reinterpret_cast<uint16_t *>(rec + kTileScales + (r * 4 + j) * 2) = i16[0];
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+            *reinterpret_cast<uint32_t *>(rec + 16 * (r + 16 * g) + 4 * j) = (uint32_t)i16[1 + 2 * g] | ((uint32_t)i16[2 + 2 * g] << 16);
+    }
+}
+
+__global__ __launch_bounds__(256) void q4_0_tiled_export_kernel(const uint8_t *__restrict__ tiles, uint16_t *__restrict__ dst,
+                                                                int64_t rows, int64_t nb) {
+    const int64_t total = rows * nb, T = nb / 4;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t blk = idx % nb, row = idx / nb;
+        const int r = (int)(row % 16), j = (int)(blk % 4);
+        const uint8_t *rec = tiles + ((row / 16) * T + blk / 4) * kTile;
+        uint16_t *o = dst + idx * 9;
+        o[0] = *reinterpret_cast<const uint16_t *>(rec + kTileScales + (r * 4 + j) * 2);
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const uint32_t w = *reinterpret_cast<const uint32_t *>(rec + 16 * (r + 16 * g) + 4 * j);
+            o[1 + 2 * g] = (uint16_t)w, o[2 + 2 * g] = (uint16_t)(w >> 16);
+        }
+    }
+}
+
+// ---- products ---------------------------------------------------------------------------------------------------------
+struct TiledDev {
+    const uint8_t *tiles;     // [w_batch, n / 16, k / 128] records
+    const void *act;          // [act_batch, m, k]
+    void *out;                // [act_batch, m, n]
+    int64_t act_stride_b, out_stride_b;   // elements between consecutive batches of act and out
+    int n, k, m, ratio;       // ratio = act_batch / w_batch
+    int T, groups;            // tiles per row group (k / 128), row groups per weight matrix (n / 16)
+    int cq, nch;              // tiles per staged chunk of the activations, chunks (1: staged once per workgroup)
+    int rounds;               // sets of row groups a workgroup walks
+};
+
+__device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
+
+// The four bytes of `c` hold codes (low nibbles) e..e+3 and (high nibbles) 16+e..16+e+3 of a block: the eight
+// values 64 + code as f16, in that order.  0x5400 is the half 64, whose last place between 64 and 128 is 1/16: a
+// code in the high nibble of the low byte adds exactly the code.  The 72 too many per weight come off in a second
+// matrix instruction (its B operand the constant -72): 7 vector instructions per 8 weights instead of 11.
+__device__ __forceinline__ half8_t codes_plus_64(uint32_t c) {
+    const uint32_t lo = (c << 4) & 0xF0F0F0F0u, hi = c & 0xF0F0F0F0u;
+    const uint32_t a = perm(0x54545454u, lo, 0x04010400u), b = perm(0x54545454u, lo, 0x04030402u);
+    const uint32_t c2 = perm(0x54545454u, hi, 0x04010400u), d = perm(0x54545454u, hi, 0x04030402u);
+    return __builtin_bit_cast(half8_t, u32x4{a, b, c2, d});
+}
+
+// CHUNKED: the activations do not fit LDS and are staged in nch chunks per round.  (A kernel of its own: with loads
+// for the staging inside the loop over the rounds, the compiler drains every load at the head of the tile loop.)
+template <int KS, int PD, bool CHUNKED>
+__global__ __launch_bounds__(64 * kW, 4) void q4_0_tiled_mfma_kernel(TiledDev p) {
+    constexpr int kThreads = 64 * kW, S = kW / KS;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const int kc = p.cq * 128;                       // staged features per activation row
+    _Float16 *lds_x = reinterpret_cast<_Float16 *>(lds_raw);                               // [m][kc], 16-byte vectors swizzled
+    float *red = reinterpret_cast<float *>(lds_raw + (size_t)p.m * kc * sizeof(_Float16));  // [2][kW][4][64] (KS > 1)
+    const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int q = w % KS, st = w / KS;               // this wave's share of a row group's tiles, its row group of the set
+    const int b = blockIdx.y, wb = b / p.ratio;
+    const _Float16 *act = reinterpret_cast<const _Float16 *>(p.act) + (int64_t)b * p.act_stride_b;
+    _Float16 *out = reinterpret_cast<_Float16 *>(p.out) + (int64_t)b * p.out_stride_b;
+    const int arow = min(r16, p.m - 1);              // output rows m..15 of the instruction are never stored: any row serves
+    const int ni = p.T > q ? (p.T - q + KS - 1) / KS : 0;   // this wave's tiles of a row group: q + KS tt, tt < ni
+    const int cqw = p.cq / KS;                       // ... of which a full chunk holds cqw (a multiple of PD when nch > 1)
+    const uint8_t *wbase = p.tiles + (int64_t)wb * p.groups * p.T * kTile;
+    const uint32_t lane_codes = 16 * lane, lane_scales = 8 * r16;
+
+    // Slot d of the ring holds tile tt = d (mod PD) of some round.  The tiles are read through a buffer descriptor
+    // per row group (base = the group's first record, size = its T records): a load past the group's end -- a wave's
+    // share that is not a multiple of PD, a round that does not exist -- is still issued, returns zeros and moves no
+    // data, so that no load sits behind a branch (which would turn every later wait for one load into a wait for all).
+    u32x4 cn[PD];
+    u32x2 sn[PD];
+    const half8_t minus_72 = __builtin_bit_cast(half8_t, u32x4{0xD480D480u, 0xD480D480u, 0xD480D480u, 0xD480D480u});
+    struct Group { const uint8_t *base; uint32_t bytes; };
+    auto group_of = [&](int round) {
+        const int64_t gi = (blockIdx.x + (int64_t)round * gridDim.x) * S + st;
+        const bool valid = round < p.rounds && gi < p.groups;
+        return Group{wbase + (valid ? gi : 0) * p.T * kTile, valid ? (uint32_t)p.T * kTile : 0u};
+    };
+    auto rsrc_of = [&](const Group &grp) { return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(grp.base), 0, grp.bytes, 0x00020000); };
+    auto fetch = [&](int d, __amdgpu_buffer_rsrc_t rsrc, int tt) {
+        const uint32_t rec = (uint32_t)(q + KS * tt) * kTile;       // tt >= ni: past the end
+        cn[d] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, rec + lane_codes, 0, 0);
+        sn[d] = __builtin_amdgcn_raw_buffer_load_b64(rsrc, rec + kTileScales + lane_scales, 0, 0);
+    };
+
+    // Chunk c of the activations: tiles c cq .. c cq + cq - 1 of every row, loaded 16 bytes (8 features) at a time, 8
+    // loads of a thread in flight.  A tile's 16 vectors of 16 bytes are XOR-swizzled by the row, and features
+    // 4 pb .. 4 pb + 3 of a block go to vector pb % 4, half pb / 4 of it, so that vector e of a block holds features
+    // 4e..4e+3 and 16+4e..16+4e+3: the A operand of lane group e.  Every workgroup of the launch reads the same bytes:
+    // each starts at another place of the chunk, so that at any moment the compute units ask different channels of the L2.
+    constexpr int NP = 8;
+    auto stage = [&](int c, auto &&after_last_loads) {
+        const int ntl = min(p.cq, p.T - c * p.cq), per_row = ntl * 16, total = p.m * per_row;
+        const int start = (int)(((int64_t)blockIdx.x * 37 % 64) * total / 64);
+        const uint32_t inv_per_row = 0xFFFFFFFFu / (uint32_t)per_row + 1;   // v / per_row = high word of v * this (v * per_row < 2^32)
+        for (int base = 0; base < total; base += kThreads * NP) {   // (uniform: every thread runs every pass)
+            const int v0 = base + tid;
+            u32x4 x[NP];
+            // piece v: row i, tile tl of the chunk, features 8 pp .. 8 pp + 7 of the tile (computed twice rather than kept)
+            auto where = [&](int u, int &i, int &tl, int &pp) {
+                int v = min(v0 + u * kThreads, total - 1) + start;      // (past the end: the last piece again, not stored)
+                if (v >= total) v -= total;
+                i = (int)__umulhi((uint32_t)v, inv_per_row);
+                const int rem = v - i * per_row;
+                tl = rem >> 4, pp = rem & 15;
+            };
+#pragma unroll
+            for (int u = 0; u < NP; u++) {
+                int i, tl, pp;
+                where(u, i, tl, pp);
+                x[u] = *reinterpret_cast<const u32x4 *>(act + (int64_t)i * p.k + (int64_t)(c * p.cq + tl) * 128 + pp * 8);
+            }
+            if (base + kThreads * NP >= total) after_last_loads();
+#pragma unroll
+            for (int u = 0; u < NP; u++) {
+                if (v0 + u * kThreads < total) {
+                    int i, tl, pp;
+                    where(u, i, tl, pp);
+                    const int vecg = (pp >> 2) * 4 + ((2 * pp) & 3), hi = (pp >> 1) & 1;
+                    const int dst = i * kc + tl * 128 + hi * 4 + (vecg ^ (i & 15)) * 8;
+                    *reinterpret_cast<u32x2 *>(lds_x + dst) = u32x2{x[u][0], x[u][1]};
+                    *reinterpret_cast<u32x2 *>(lds_x + (dst ^ 8)) = u32x2{x[u][2], x[u][3]};   // vector vecg + 1 (vecg is even)
+                }
+            }
+        }
+    };
+
+    // The ring's first two tiles, the activations, the rest of the ring: loads return in order, and what waits for
+    // the activations must not wait for the whole ring (by then half of a small matrix).
+    Group g_cur = group_of(0);
+    const __amdgpu_buffer_rsrc_t rs0 = rsrc_of(g_cur);
+    fetch(0, rs0, 0);
+    fetch(1, rs0, 1);
+    auto rest_of_ring = [&]() {
+#pragma unroll
+        for (int d = 2; d < PD; d++) fetch(d, rs0, d);
+    };
+    if constexpr (!CHUNKED) {
+        stage(0, rest_of_ring);
+        __syncthreads();
+    } else {
+        rest_of_ring();
+    }
+
+    for (int round = 0; round < p.rounds; round++) {
+        const int64_t unit = blockIdx.x + (int64_t)round * gridDim.x;
+        const bool gvalid = unit * S + st < p.groups;
+        const int64_t gi = unit * S + st;
+        const Group g_next = group_of(round + 1);
+        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+
+        for (int c = 0; c < (CHUNKED ? p.nch : 1); c++) {
+            if constexpr (CHUNKED) {
+                if (c || round) __syncthreads();   // the previous chunk has been read
+                stage(c, []() {});
+                __syncthreads();
+            }
+            const int tt0 = CHUNKED ? c * cqw : 0, tt_end = CHUNKED ? min(ni, tt0 + cqw) : ni;
+            const int tl_off = q - c * p.cq;                      // tile tt of the wave sits at tl_off + KS tt of the chunk
+            for (int l0 = tt0; l0 < tt_end; l0 += PD) {
+                const bool more_here = l0 + PD < ni;              // the round has another batch (maybe in the next chunk)
+                const __amdgpu_buffer_rsrc_t rs = rsrc_of(more_here ? g_cur : g_next);
+#pragma unroll
+                for (int d = 0; d < PD; d++) {
+                    const int tt = l0 + d;
+                    if (tt < ni) {                                // (a share that is not a multiple of PD: zeros were loaded)
+                        // The four blocks side by side: reads, then the instructions that need only the activations,
+                        // then those that need the codes.  (Reading a tile's activations during the tile before it
+                        // measured slower: 9.4 against 8.9 us for one row of 14336 x 4096.)
+                        const int tl = tl_off + KS * tt;
+                        half8_t a[4];
+                        float4_t part[4];
+#pragma unroll
+                        for (int j = 0; j < 4; j++) a[j] = *reinterpret_cast<const half8_t *>(lds_x + (size_t)arow * kc + (tl * 16 + ((j * 4 + g) ^ arow)) * 8);
+#pragma unroll
+                        for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], minus_72, float4_t{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+#pragma unroll
+                        for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], codes_plus_64(cn[d][j]), part[j], 0, 0, 0);
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const float dsc = (float)__builtin_bit_cast(_Float16, (uint16_t)(sn[d][j >> 1] >> (16 * (j & 1))));
+#pragma unroll
+                            for (int e = 0; e < 4; e++) acc[e] = __builtin_fmaf(dsc, part[j][e], acc[e]);
+                        }
+                    }
+                    // The slot is refilled once its tile has been used, into the same registers, and the refills stay
+                    // where they are written (moved to the top of the batch, the ring would need a second set).
+                    asm volatile("" ::: "memory");
+                    fetch(d, rs, more_here ? tt + PD : d);
+                }
+            }
+        }
+        g_cur = g_next;
+
+        // acc[e] = partial out[4 g + e][16 gi + r16]
+        const int64_t row = gi * 16 + r16;
+        if constexpr (KS == 1) {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (gvalid && 4 * g + e < p.m) out[(int64_t)(4 * g + e) * p.n + row] = (_Float16)acc[e];
+        } else {
+            // Two buffers by the round's parity: the barrier of the next round separates this round's reads from the
+            // writes of the round after it.
+            float *rb = red + (round & 1) * (kW * 4 * 64);
+#pragma unroll
+            for (int e = 0; e < 4; e++) rb[(w * 4 + e) * 64 + lane] = acc[e];
+            __syncthreads();
+#pragma unroll
+            for (int e0 = 0; e0 < 4; e0 += KS) {
+                const int e = e0 + q;
+                if (e < 4) {
+                    float sum = 0.0f;
+#pragma unroll
+                    for (int ww = 0; ww < KS; ww++) sum += rb[((st * KS + ww) * 4 + e) * 64 + lane];
+                    if (gvalid && 4 * g + e < p.m) out[(int64_t)(4 * g + e) * p.n + row] = (_Float16)sum;
+                }
+            }
+        }
+        // Loads and stores share one counter and are not ordered against each other: with a store outstanding the
+        // compiler makes every wait for a tile a wait for all memory traffic, and it places its waits for every path
+        // at once.  So the path that has stored waits here, once per round, for its stores (and the next round's
+        // first tiles): what enters the tile loop has only loads outstanding, and the ring's waits count tiles.
+        if (round + 1 < p.rounds) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    }
+}
+
+// f32 activations: 4 waves, one row group per wave and round; lane (r, g) multiplies the 32 weights of its slot.
+constexpr int kVecLds = 32 * 1024;
+
+template <int M>
+__global__ __launch_bounds__(256) void q4_0_tiled_vec_f32_kernel(TiledDev p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    float *lds_x = reinterpret_cast<float *>(lds_raw);   // [M][kc]
+    const int kc = p.cq * 128;
+    const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int b = blockIdx.y, wb = b / p.ratio;
+    const float *act = reinterpret_cast<const float *>(p.act) + (int64_t)b * p.act_stride_b;
+    float *out = reinterpret_cast<float *>(p.out) + (int64_t)b * p.out_stride_b;
+    const uint8_t *wbase = p.tiles + (int64_t)wb * p.groups * p.T * kTile;
+
+    for (int round = 0; round < p.rounds; round++) {
+        const int64_t gi64 = (blockIdx.x + (int64_t)round * gridDim.x) * 4 + w;
+        const bool gvalid = gi64 < p.groups;
+        const int gi = (int)min(gi64, (int64_t)p.groups - 1);
+        const uint8_t *grp = wbase + (int64_t)gi * p.T * kTile;
+        float acc[M];
+#pragma unroll
+        for (int i = 0; i < M; i++) acc[i] = 0.0f;
+        u32x4 cnext = *reinterpret_cast<const u32x4 *>(grp + 16 * lane);
+        u32x2 snext = *reinterpret_cast<const u32x2 *>(grp + kTileScales + 8 * r16);
+        for (int c = 0; c < p.nch; c++) {
+            const int ntl = min(p.cq, p.T - c * p.cq);
+            if (p.nch > 1 || round == 0) {
+                if (c || round) __syncthreads();
+                const int vec_per_row = ntl * 32;   // 16-byte vectors
+                for (int v = tid; v < M * vec_per_row; v += 256) {
+                    const int i = v / vec_per_row, cc = v - i * vec_per_row;
+                    *reinterpret_cast<float4_t *>(lds_x + (size_t)i * kc + cc * 4) =
+                        *reinterpret_cast<const float4_t *>(act + (int64_t)i * p.k + (int64_t)c * kc + cc * 4);
+                }
+                __syncthreads();
+            }
+            for (int tl = 0; tl < ntl; tl++) {
+                const u32x4 cw = cnext;
+                const u32x2 sw = snext;
+                const int tn = min(c * p.cq + tl + 1, p.T - 1);
+                cnext = *reinterpret_cast<const u32x4 *>(grp + (int64_t)tn * kTile + 16 * lane);
+                snext = *reinterpret_cast<const u32x2 *>(grp + (int64_t)tn * kTile + kTileScales + 8 * r16);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint32_t word = cw[j];
+                    float wl[4], wh[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        wl[e] = (float)((word >> (8 * e)) & 0xFu) - 8.0f;
+                        wh[e] = (float)((word >> (8 * e + 4)) & 0xFu) - 8.0f;
+                    }
+                    const float dsc = (float)__builtin_bit_cast(_Float16, (uint16_t)(sw[j >> 1] >> (16 * (j & 1))));
+#pragma unroll
+                    for (int i = 0; i < M; i++) {
+                        const float4_t xl = *reinterpret_cast<const float4_t *>(lds_x + (size_t)i * kc + tl * 128 + j * 32 + 4 * g);
+                        const float4_t xh = *reinterpret_cast<const float4_t *>(lds_x + (size_t)i * kc + tl * 128 + j * 32 + 16 + 4 * g);
+                        float part = 0.0f;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            part = __builtin_fmaf(wl[e], xl[e], part);
+                            part = __builtin_fmaf(wh[e], xh[e], part);
+                        }
+                        acc[i] = __builtin_fmaf(dsc, part, acc[i]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < M; i++) {
+            float v = acc[i];
+            v += __shfl_xor(v, 16);
+            v += __shfl_xor(v, 32);
+            if (gvalid && g == 0) out[(int64_t)i * p.n + (int64_t)gi * 16 + r16] = v;
+        }
+    }
+}
+
+int env_int(const char *name, int dflt) {
+    const char *v = getenv(name);
+    return v ? atoi(v) : dflt;
+}
+
+template <int KS, int PD, bool CHUNKED>
+int launch_mfma_ks(TiledDev p, int64_t act_batch, int per_cu_forced, hipStream_t s) {
+    constexpr int S = kW / KS;
+    const size_t lds = (size_t)p.m * p.cq * 128 * 2 + (KS > 1 ? (size_t)2 * kW * 4 * 64 * sizeof(float) : 0);
+    if (lds > 64 * 1024 &&      // beyond the default limit of dynamic LDS: allowed per kernel (and device) on request
+        hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_0_tiled_mfma_kernel<KS, PD, CHUNKED>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail("q4_0_matvec (tiled weights): %zu bytes of LDS were refused", lds);
+    }
+    int64_t per_cu = (160 * 1024) / (int64_t)lds;
+    if (per_cu > 32 / kW) per_cu = 32 / kW;
+    if (per_cu < 1) per_cu = 1;
+    if (per_cu_forced > 0) per_cu = per_cu_forced;
+    const int64_t units = (p.groups + S - 1) / S;
+    int64_t resident = (int64_t)num_compute_units() * per_cu / act_batch;
+    if (resident < 1) resident = 1;
+    int64_t wgs = units, rounds = 1;
+    if (units > resident) {
+        rounds = (units + resident - 1) / resident;
+        wgs = (units + rounds - 1) / rounds;
+    }
+    p.rounds = (int)rounds;
+    hipLaunchKernelGGL((q4_0_tiled_mfma_kernel<KS, PD, CHUNKED>), dim3((unsigned)wgs, (unsigned)act_batch), dim3(64 * kW), lds, s, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("q4_0_matvec (tiled weights) launch failed: %s", hipGetErrorString(e));
+    return 0;
+}
+
+int launch_tiled_mfma(TiledDev p, int64_t act_batch, hipStream_t s) {
+    static const int forced_ks = env_int("TROCM_Q4T_KS", 0);
+    static const int forced_per_cu = env_int("TROCM_Q4T_WG_PER_CU", 0);
+    static const int forced_lds_kb = env_int("TROCM_Q4T_LDS_KB", 0);
+    const int64_t cus = num_compute_units();
+    // The fewest waves per row group that still give (nearly) every compute unit a workgroup, each wave then walking
+    // the longest stream of tiles: 128256 x 4096: 1; 14336 x 4096: 2 (224 workgroups; one row 8.9 us, 8 rows 10.0 us;
+    // with 4: 9.3 / 10.7; with 8: 9.1 / 10.3); 4096 x 4096 and 4096 x 14336: 8.
+    int ks = 8;
+    for (int c = 1; c <= 8; c *= 2)
+        if (((int64_t)p.groups * c + kW - 1) / kW * act_batch * 8 >= cus * 7) {
+            ks = c;
+            break;
+        }
+    while (ks > 1 && ks > p.T) ks /= 2;
+    if (forced_ks == 1 || forced_ks == 2 || forced_ks == 4 || forced_ks == 8) ks = forced_ks;
+    const int pd = ks == 8 ? 4 : 8;
+    // The activations whole in LDS if they fit beside the partial sums; else in chunks of a multiple of KS PD tiles:
+    // 64 KB (two workgroups per compute unit cover each other's staging), or 128 KB where 64 KB hold no such chunk.
+    const int64_t red = ks > 1 ? 2 * kW * 4 * 64 * 4 : 0;
+    const int64_t whole = (int64_t)p.m * p.k * 2;
+    const int64_t lds_all = forced_lds_kb > 0 ? (int64_t)forced_lds_kb * 1024 : 160 * 1024;
+    if (whole + red <= lds_all) {
+        p.cq = p.T, p.nch = 1;
+    } else {
+        const int64_t step = ks * pd;
+        int64_t cq = (64 * 1024) / ((int64_t)p.m * 256) / step * step;
+        if (cq < step) cq = (128 * 1024) / ((int64_t)p.m * 256) / step * step;
+        if (cq < step) return fail("q4_0_matvec (tiled weights): %d activation rows leave no room for a chunk", p.m);
+        p.cq = (int)cq, p.nch = (int)((p.T + cq - 1) / cq);
+    }
+    if (p.nch > 1) switch (ks) {
+        case 1: return launch_mfma_ks<1, 8, true>(p, act_batch, forced_per_cu, s);
+        case 2: return launch_mfma_ks<2, 8, true>(p, act_batch, forced_per_cu, s);
+        case 4: return launch_mfma_ks<4, 8, true>(p, act_batch, forced_per_cu, s);
+        default: return launch_mfma_ks<8, 4, true>(p, act_batch, forced_per_cu, s);
+    }
+    switch (ks) {
+        case 1: return launch_mfma_ks<1, 8, false>(p, act_batch, forced_per_cu, s);
+        case 2: return launch_mfma_ks<2, 8, false>(p, act_batch, forced_per_cu, s);
+        case 4: return launch_mfma_ks<4, 8, false>(p, act_batch, forced_per_cu, s);
+        default: return launch_mfma_ks<8, 4, false>(p, act_batch, forced_per_cu, s);
+    }
+}
+
+template <int M>
+int launch_vec_m(TiledDev p, int64_t act_batch, hipStream_t s) {
+    int64_t cq = kVecLds / ((int64_t)M * 128 * 4);
+    if (cq > p.T) cq = p.T;
+    p.cq = (int)cq, p.nch = (int)((p.T + cq - 1) / cq);
+    const int64_t units = (p.groups + 3) / 4;
+    int64_t resident = (int64_t)num_compute_units() * 4 / act_batch;
+    if (resident < 1) resident = 1;
+    int64_t wgs = units, rounds = 1;
+    if (units > resident) {
+        rounds = (units + resident - 1) / resident;
+        wgs = (units + rounds - 1) / rounds;
+    }
+    p.rounds = (int)rounds;
+    hipLaunchKernelGGL((q4_0_tiled_vec_f32_kernel<M>), dim3((unsigned)wgs, (unsigned)act_batch), dim3(256), (size_t)M * p.cq * 128 * 4, s, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("q4_0_matvec (tiled weights, f32) launch failed: %s", hipGetErrorString(e));
+    return 0;
+}
+
+int launch_tiled_vec(const TiledDev &p, int64_t act_batch, hipStream_t s) {
+    switch (p.m) {
+        case 1: return launch_vec_m<1>(p, act_batch, s);
+        case 2: return launch_vec_m<2>(p, act_batch, s);
+        case 3: return launch_vec_m<3>(p, act_batch, s);
+        case 4: return launch_vec_m<4>(p, act_batch, s);
+        case 5: return launch_vec_m<5>(p, act_batch, s);
+        case 6: return launch_vec_m<6>(p, act_batch, s);
+        case 7: return launch_vec_m<7>(p, act_batch, s);
+        case 8: return launch_vec_m<8>(p, act_batch, s);
+    }
+    return fail("q4_0_matvec (tiled weights, f32): m = %d activation rows (1..8 are handled per launch)", p.m);
+}
+
+}  // namespace
+
+bool q4_0_tiled_layout_fits(int64_t n, int64_t k) { return n % 16 == 0 && k % 128 == 0 && n >= 16 && k >= 128; }
+size_t q4_0_tiled_bytes(int64_t rows, int64_t k) { return (size_t)(rows / 16) * (size_t)(k / 128) * kTile; }
+
+int launch_q4_0_tiled_import(const void *blocks, void *tiles, int64_t rows, int64_t k, hipStream_t s) {
+    const int64_t total = rows * (k / 32);
+    if (total == 0) return 0;
+    int64_t grid = (total + 255) / 256;
+    if (grid > 65535 * 16) grid = 65535 * 16;
+    hipLaunchKernelGGL(q4_0_tiled_import_kernel, dim3((unsigned)grid), dim3(256), 0, s, (const uint16_t *)blocks, (uint8_t *)tiles, rows, k / 32);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("q4_0 weights (tiling) launch failed: %s", hipGetErrorString(e));
+    return 0;
+}
+
+int launch_q4_0_tiled_export(const void *tiles, void *blocks, int64_t rows, int64_t k, hipStream_t s) {
+    const int64_t total = rows * (k / 32);
+    if (total == 0) return 0;
+    int64_t grid = (total + 255) / 256;
+    if (grid > 65535 * 16) grid = 65535 * 16;
+    hipLaunchKernelGGL(q4_0_tiled_export_kernel, dim3((unsigned)grid), dim3(256), 0, s, (const uint8_t *)tiles, (uint16_t *)blocks, rows, k / 32);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("q4_0 weights (export of tiles) launch failed: %s", hipGetErrorString(e));
+    return 0;
+}
+
+// Tiled weights x activations for any m: f16 rows in groups of up to 16 on the matrix cores (more than 16 rows go to the
+// matrix-matrix kernel first, which reads the same tiles, when it takes the call), f32 rows in groups of 8 on the
+// vector ALU.
+int launch_q4_0_tiled_matvec(const void *tiles, int64_t w_batch, int64_t n, int64_t k, const void *act, int act_dtype,
+                             int64_t act_batch, int64_t m, void *out, hipStream_t s) {
+    if (n >= (1ll << 30) || k >= (1ll << 30) || act_batch > 65535) return fail("q4_0_matvec: shape too large");
+    if (act_dtype == TROCM_F16 && m > 16) {
+        const int rc = launch_q4_0_matmul(tiles, nullptr, w_batch, n, k, act, act_dtype, act_batch, m, out, s, 1);
+        if (rc != 2) return rc;
+    }
+    const int64_t es = act_dtype == TROCM_F16 ? 2 : 4, step = act_dtype == TROCM_F16 ? 16 : 8;
+    for (int64_t i0 = 0; i0 < m; i0 += step) {
+        TiledDev p;
+        memset(&p, 0, sizeof(p));
+        p.tiles = (const uint8_t *)tiles;
+        p.act = (const char *)act + i0 * k * es, p.out = (char *)out + i0 * n * es;
+        p.act_stride_b = m * k, p.out_stride_b = m * n;
+        p.n = (int)n, p.k = (int)k, p.m = (int)(m - i0 < step ? m - i0 : step), p.ratio = (int)(act_batch / w_batch);
+        p.T = (int)(k / 128), p.groups = (int)(n / 16);
+        const int rc = act_dtype == TROCM_F16 ? launch_tiled_mfma(p, act_batch, s) : launch_tiled_vec(p, act_batch, s);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+}  // namespace trocm
