@@ -149,12 +149,12 @@ __global__ __launch_bounds__(64 * kW, 4) void q4_0_tiled_mfma_kernel(TiledDev p)
         sn[d] = __builtin_amdgcn_raw_buffer_load_b64(rsrc, rec + kTileScales + lane_scales, 0, 0);
     };
 
-    // Chunk c of the activations: tiles c cq .. c cq + cq - 1 of every row, loaded 16 bytes (8 features) at a time, 8
+    // Chunk c of the activations: tiles c cq .. c cq + cq - 1 of every row, loaded 16 bytes (8 features) at a time, 8 (4)
     // loads of a thread in flight.  A tile's 16 vectors of 16 bytes are XOR-swizzled by the row, and features
     // 4 pb .. 4 pb + 3 of a block go to vector pb % 4, half pb / 4 of it, so that vector e of a block holds features
     // 4e..4e+3 and 16+4e..16+4e+3: the A operand of lane group e.  Every workgroup of the launch reads the same bytes:
     // each starts at another place of the chunk, so that at any moment the compute units ask different channels of the L2.
-    constexpr int NP = 8;
+    constexpr int NP = CHUNKED ? 4 : 8;   // (registers)
     auto stage = [&](int c, auto &&after_last_loads) {
         const int ntl = min(p.cq, p.T - c * p.cq), per_row = ntl * 16, total = p.m * per_row;
         const int start = (int)(((int64_t)blockIdx.x * 37 % 64) * total / 64);
@@ -384,7 +384,7 @@ int launch_mfma_ks(TiledDev p, int64_t act_batch, int per_cu_forced, hipStream_t
         return fail("q4_0_matvec (tiled weights): %zu bytes of LDS were refused", lds);
     }
     int64_t per_cu = (160 * 1024) / (int64_t)lds;
-    if (per_cu > 32 / kW) per_cu = 32 / kW;
+    if (per_cu > 2) per_cu = 2;     // (by registers: 4 or 5 waves per SIMD)
     if (per_cu < 1) per_cu = 1;
     if (per_cu_forced > 0) per_cu = per_cu_forced;
     const int64_t units = (p.groups + S - 1) / S;
@@ -416,6 +416,7 @@ int launch_tiled_mfma(TiledDev p, int64_t act_batch, hipStream_t s) {
             ks = c;
             break;
         }
+    if (p.m <= 2) ks = 8;   // (one or two rows: never slower, 14336 x 4096 8.9 against 9.2 us)
     while (ks > 1 && ks > p.T) ks /= 2;
     if (forced_ks == 1 || forced_ks == 2 || forced_ks == 4 || forced_ks == 8) ks = forced_ks;
     const int pd = ks == 8 ? 4 : 8;
