@@ -26,8 +26,10 @@
 // enter as the exact f16 integers -8 .. 7, the products accumulate in f32 inside the instruction from zero, and the
 // block's sum is scaled by its f16 scale with one fma per output.
 //
-// f32 activations, 1..8 rows (q4_0_tiled_vec_f32_kernel): the same tiles on the vector ALU, products and sums in f32
-// (the codes are exact in f32), one wave per row group, lane (r, g) the 32 weights of its slot per tile.
+// f32 activations, 1..8 rows: the same kernel with v_mfma_f32_16x16x32_bf16.  Staging splits every activation into
+// three bf16 numbers of 8 significant bits each (x = b1 + b2 + b3 exactly, by truncation and exact remainders), kept as
+// three planes in LDS; the codes 64 + code are exact in bf16, so every product is exact and the sums are taken in f32
+// inside the instructions, smallest parts first: the arithmetic of an f32 kernel, over the whole range of f32.
 //
 // Roofline: HBM-bound on the weights: 18 bytes per 32 weights, read once.
 #include <hip/hip_fp16.h>
@@ -41,6 +43,7 @@ namespace {
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -110,19 +113,31 @@ __device__ __forceinline__ half8_t codes_plus_64(uint32_t c) {
 
 // CHUNKED: the activations do not fit LDS and are staged in nch chunks per round.  (A kernel of its own: with loads
 // for the staging inside the loop over the rounds, the compiler drains every load at the head of the tile loop.)
-template <int KS, int PD, bool CHUNKED>
-__global__ __launch_bounds__(64 * kW, 4) void q4_0_tiled_mfma_kernel(TiledDev p) {
+// The same as bf16: 0x4280 is 64, whose last place between 64 and 128 is 1/2: the code shifted left by one.
+__device__ __forceinline__ bf16x8_t codes_plus_64_bf16(uint32_t c) {
+    const uint32_t lo = ((c << 1) & 0x1E1E1E1Eu) | 0x80808080u, hi = ((c >> 3) & 0x1E1E1E1Eu) | 0x80808080u;
+    const uint32_t a = perm(0x42424242u, lo, 0x04010400u), b = perm(0x42424242u, lo, 0x04030402u);
+    const uint32_t c2 = perm(0x42424242u, hi, 0x04010400u), d = perm(0x42424242u, hi, 0x04030402u);
+    return __builtin_bit_cast(bf16x8_t, u32x4{a, b, c2, d});
+}
+
+// F32: f32 activations and output, three bf16 planes in LDS (else f16 activations and output).
+template <int KS, int PD, bool CHUNKED, bool F32>
+__global__ __launch_bounds__(64 * kW, F32 ? 2 : 4) void q4_0_tiled_mfma_kernel(TiledDev p) {
+    using ActT = typename std::conditional<F32, float, _Float16>::type;
+    constexpr int NPL = F32 ? 3 : 1;                 // planes of 16-bit numbers per activation
     constexpr int kThreads = 64 * kW, S = kW / KS;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const int kc = p.cq * 128;                       // staged features per activation row
-    _Float16 *lds_x = reinterpret_cast<_Float16 *>(lds_raw);                               // [m][kc], 16-byte vectors swizzled
-    float *red = reinterpret_cast<float *>(lds_raw + (size_t)p.m * kc * sizeof(_Float16));  // [2][kW][4][64] (KS > 1)
+    uint16_t *lds_x = reinterpret_cast<uint16_t *>(lds_raw);                                // [NPL][m][kc], 16-byte vectors swizzled
+    const int plane = p.m * kc;                      // 16-bit numbers per plane
+    float *red = reinterpret_cast<float *>(lds_raw + (size_t)NPL * plane * 2);              // [2][kW][4][64] (KS > 1)
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int q = w % KS, st = w / KS;               // this wave's share of a row group's tiles, its row group of the set
     const int b = blockIdx.y, wb = b / p.ratio;
-    const _Float16 *act = reinterpret_cast<const _Float16 *>(p.act) + (int64_t)b * p.act_stride_b;
-    _Float16 *out = reinterpret_cast<_Float16 *>(p.out) + (int64_t)b * p.out_stride_b;
+    const ActT *act = reinterpret_cast<const ActT *>(p.act) + (int64_t)b * p.act_stride_b;
+    ActT *out = reinterpret_cast<ActT *>(p.out) + (int64_t)b * p.out_stride_b;
     const int arow = min(r16, p.m - 1);              // output rows m..15 of the instruction are never stored: any row serves
     const int ni = p.T > q ? (p.T - q + KS - 1) / KS : 0;   // this wave's tiles of a row group: q + KS tt, tt < ni
     const int cqw = p.cq / KS;                       // ... of which a full chunk holds cqw (a multiple of PD when nch > 1)
@@ -135,7 +150,8 @@ __global__ __launch_bounds__(64 * kW, 4) void q4_0_tiled_mfma_kernel(TiledDev p)
     // data, so that no load sits behind a branch (which would turn every later wait for one load into a wait for all).
     u32x4 cn[PD];
     u32x2 sn[PD];
-    const half8_t minus_72 = __builtin_bit_cast(half8_t, u32x4{0xD480D480u, 0xD480D480u, 0xD480D480u, 0xD480D480u});
+    const uint32_t m72 = F32 ? 0xC290C290u : 0xD480D480u;      // -72 as two bf16 or two f16
+    const u32x4 minus_72 = {m72, m72, m72, m72};
     struct Group { const uint8_t *base; uint32_t bytes; };
     auto group_of = [&](int round) {
         const int64_t gi = (blockIdx.x + (int64_t)round * gridDim.x) * S + st;
@@ -155,26 +171,27 @@ __global__ __launch_bounds__(64 * kW, 4) void q4_0_tiled_mfma_kernel(TiledDev p)
     // 4e..4e+3 and 16+4e..16+4e+3: the A operand of lane group e.  Every workgroup of the launch reads the same bytes:
     // each starts at another place of the chunk, so that at any moment the compute units ask different channels of the L2.
     constexpr int NP = CHUNKED ? 4 : 8;   // (registers)
+    constexpr int PPT = F32 ? 32 : 16;    // 16-byte pieces of the source per tile and row: 4 f32 or 8 f16 features each
     auto stage = [&](int c, auto &&after_last_loads) {
-        const int ntl = min(p.cq, p.T - c * p.cq), per_row = ntl * 16, total = p.m * per_row;
+        const int ntl = min(p.cq, p.T - c * p.cq), per_row = ntl * PPT, total = p.m * per_row;
         const int start = (int)(((int64_t)blockIdx.x * 37 % 64) * total / 64);
         const uint32_t inv_per_row = 0xFFFFFFFFu / (uint32_t)per_row + 1;   // v / per_row = high word of v * this (v * per_row < 2^32)
         for (int base = 0; base < total; base += kThreads * NP) {   // (uniform: every thread runs every pass)
             const int v0 = base + tid;
             u32x4 x[NP];
-            // piece v: row i, tile tl of the chunk, features 8 pp .. 8 pp + 7 of the tile (computed twice rather than kept)
+            // piece v: row i, tile tl of the chunk, piece pp of the tile (computed twice rather than kept)
             auto where = [&](int u, int &i, int &tl, int &pp) {
                 int v = min(v0 + u * kThreads, total - 1) + start;      // (past the end: the last piece again, not stored)
                 if (v >= total) v -= total;
                 i = (int)__umulhi((uint32_t)v, inv_per_row);
                 const int rem = v - i * per_row;
-                tl = rem >> 4, pp = rem & 15;
+                tl = rem / PPT, pp = rem % PPT;
             };
 #pragma unroll
             for (int u = 0; u < NP; u++) {
                 int i, tl, pp;
                 where(u, i, tl, pp);
-                x[u] = *reinterpret_cast<const u32x4 *>(act + (int64_t)i * p.k + (int64_t)(c * p.cq + tl) * 128 + pp * 8);
+                x[u] = *reinterpret_cast<const u32x4 *>(act + (int64_t)i * p.k + (int64_t)(c * p.cq + tl) * 128 + pp * (F32 ? 4 : 8));
             }
             if (base + kThreads * NP >= total) after_last_loads();
 #pragma unroll
@@ -182,10 +199,34 @@ __global__ __launch_bounds__(64 * kW, 4) void q4_0_tiled_mfma_kernel(TiledDev p)
                 if (v0 + u * kThreads < total) {
                     int i, tl, pp;
                     where(u, i, tl, pp);
-                    const int vecg = (pp >> 2) * 4 + ((2 * pp) & 3), hi = (pp >> 1) & 1;
-                    const int dst = i * kc + tl * 128 + hi * 4 + (vecg ^ (i & 15)) * 8;
-                    *reinterpret_cast<u32x2 *>(lds_x + dst) = u32x2{x[u][0], x[u][1]};
-                    *reinterpret_cast<u32x2 *>(lds_x + (dst ^ 8)) = u32x2{x[u][2], x[u][3]};   // vector vecg + 1 (vecg is even)
+                    if constexpr (F32) {
+                        // features 4 pp .. 4 pp + 3 of the tile: vector (pp / 8) * 4 + pp % 4, half (pp / 4) % 2 of it, in each plane
+                        const int vecg = (pp >> 3) * 4 + (pp & 3), hi = (pp >> 2) & 1;
+                        const int dst = i * kc + tl * 128 + hi * 4 + (vecg ^ (i & 15)) * 8;
+                        // (the elements by name: indexed by the counter of an unrolled loop, this compiler has been seen
+                        // to read element 0 of an ext-vector every time)
+                        const uint32_t xe[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
+                        uint32_t part[3][4];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float x0 = __builtin_bit_cast(float, xe[e]);
+                            part[0][e] = xe[e] & 0xFFFF0000u;                                     // the first 8 bits of x
+                            const float r1 = x0 - __builtin_bit_cast(float, part[0][e]);          // exact
+                            part[1][e] = __builtin_bit_cast(uint32_t, r1) & 0xFFFF0000u;
+                            const float r2 = r1 - __builtin_bit_cast(float, part[1][e]);          // exact, at most 8 bits left
+                            part[2][e] = __builtin_bit_cast(uint32_t, r2);
+                        }
+#pragma unroll
+                        for (int pl = 0; pl < 3; pl++)
+                            *reinterpret_cast<u32x2 *>(lds_x + pl * plane + dst) =
+                                u32x2{perm(part[pl][1], part[pl][0], 0x07060302u), perm(part[pl][3], part[pl][2], 0x07060302u)};
+                    } else {
+                        // features 8 pp .. 8 pp + 7 of the tile: the halves of two neighbouring vectors
+                        const int vecg = (pp >> 2) * 4 + ((2 * pp) & 3), hi = (pp >> 1) & 1;
+                        const int dst = i * kc + tl * 128 + hi * 4 + (vecg ^ (i & 15)) * 8;
+                        *reinterpret_cast<u32x2 *>(lds_x + dst) = u32x2{x[u][0], x[u][1]};
+                        *reinterpret_cast<u32x2 *>(lds_x + (dst ^ 8)) = u32x2{x[u][2], x[u][3]};   // vector vecg + 1 (vecg is even)
+                    }
                 }
             }
         }
@@ -234,14 +275,29 @@ __global__ __launch_bounds__(64 * kW, 4) void q4_0_tiled_mfma_kernel(TiledDev p)
                         // then those that need the codes.  (Reading a tile's activations during the tile before it
                         // measured slower: 9.4 against 8.9 us for one row of 14336 x 4096.)
                         const int tl = tl_off + KS * tt;
-                        half8_t a[4];
+                        u32x4 a[4];
                         float4_t part[4];
+                        if constexpr (F32) {
+                            bf16x8_t codes[4];
 #pragma unroll
-                        for (int j = 0; j < 4; j++) a[j] = *reinterpret_cast<const half8_t *>(lds_x + (size_t)arow * kc + (tl * 16 + ((j * 4 + g) ^ arow)) * 8);
+                            for (int j = 0; j < 4; j++) codes[j] = codes_plus_64_bf16(cn[d][j]), part[j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                        for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], minus_72, float4_t{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+                            for (int pl = 2; pl >= 0; pl--) {     // the smallest parts first
 #pragma unroll
-                        for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], codes_plus_64(cn[d][j]), part[j], 0, 0, 0);
+                                for (int j = 0; j < 4; j++) a[j] = *reinterpret_cast<const u32x4 *>(lds_x + pl * plane + arow * kc + (tl * 16 + ((j * 4 + g) ^ arow)) * 8);
+#pragma unroll
+                                for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[j]), __builtin_bit_cast(bf16x8_t, minus_72), part[j], 0, 0, 0);
+#pragma unroll
+                                for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[j]), codes[j], part[j], 0, 0, 0);
+                            }
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < 4; j++) a[j] = *reinterpret_cast<const u32x4 *>(lds_x + arow * kc + (tl * 16 + ((j * 4 + g) ^ arow)) * 8);
+#pragma unroll
+                            for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a[j]), __builtin_bit_cast(half8_t, minus_72), float4_t{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+#pragma unroll
+                            for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a[j]), codes_plus_64(cn[d][j]), part[j], 0, 0, 0);
+                        }
 #pragma unroll
                         for (int j = 0; j < 4; j++) {
                             const float dsc = (float)__builtin_bit_cast(_Float16, (uint16_t)(sn[d][j >> 1] >> (16 * (j & 1))));
@@ -263,7 +319,7 @@ __global__ __launch_bounds__(64 * kW, 4) void q4_0_tiled_mfma_kernel(TiledDev p)
         if constexpr (KS == 1) {
 #pragma unroll
             for (int e = 0; e < 4; e++)
-                if (gvalid && 4 * g + e < p.m) out[(int64_t)(4 * g + e) * p.n + row] = (_Float16)acc[e];
+                if (gvalid && 4 * g + e < p.m) out[(int64_t)(4 * g + e) * p.n + row] = (ActT)acc[e];
         } else {
             // Two buffers by the round's parity: the barrier of the next round separates this round's reads from the
             // writes of the round after it.
@@ -278,7 +334,7 @@ __global__ __launch_bounds__(64 * kW, 4) void q4_0_tiled_mfma_kernel(TiledDev p)
                     float sum = 0.0f;
 #pragma unroll
                     for (int ww = 0; ww < KS; ww++) sum += rb[((st * KS + ww) * 4 + e) * 64 + lane];
-                    if (gvalid && 4 * g + e < p.m) out[(int64_t)(4 * g + e) * p.n + row] = (_Float16)sum;
+                    if (gvalid && 4 * g + e < p.m) out[(int64_t)(4 * g + e) * p.n + row] = (ActT)sum;
                 }
             }
         }
@@ -290,101 +346,23 @@ __global__ __launch_bounds__(64 * kW, 4) void q4_0_tiled_mfma_kernel(TiledDev p)
     }
 }
 
-// f32 activations: 4 waves, one row group per wave and round; lane (r, g) multiplies the 32 weights of its slot.
-constexpr int kVecLds = 32 * 1024;
-
-template <int M>
-__global__ __launch_bounds__(256) void q4_0_tiled_vec_f32_kernel(TiledDev p) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    float *lds_x = reinterpret_cast<float *>(lds_raw);   // [M][kc]
-    const int kc = p.cq * 128;
-    const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
-    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int b = blockIdx.y, wb = b / p.ratio;
-    const float *act = reinterpret_cast<const float *>(p.act) + (int64_t)b * p.act_stride_b;
-    float *out = reinterpret_cast<float *>(p.out) + (int64_t)b * p.out_stride_b;
-    const uint8_t *wbase = p.tiles + (int64_t)wb * p.groups * p.T * kTile;
-
-    for (int round = 0; round < p.rounds; round++) {
-        const int64_t gi64 = (blockIdx.x + (int64_t)round * gridDim.x) * 4 + w;
-        const bool gvalid = gi64 < p.groups;
-        const int gi = (int)min(gi64, (int64_t)p.groups - 1);
-        const uint8_t *grp = wbase + (int64_t)gi * p.T * kTile;
-        float acc[M];
-#pragma unroll
-        for (int i = 0; i < M; i++) acc[i] = 0.0f;
-        u32x4 cnext = *reinterpret_cast<const u32x4 *>(grp + 16 * lane);
-        u32x2 snext = *reinterpret_cast<const u32x2 *>(grp + kTileScales + 8 * r16);
-        for (int c = 0; c < p.nch; c++) {
-            const int ntl = min(p.cq, p.T - c * p.cq);
-            if (p.nch > 1 || round == 0) {
-                if (c || round) __syncthreads();
-                const int vec_per_row = ntl * 32;   // 16-byte vectors
-                for (int v = tid; v < M * vec_per_row; v += 256) {
-                    const int i = v / vec_per_row, cc = v - i * vec_per_row;
-                    *reinterpret_cast<float4_t *>(lds_x + (size_t)i * kc + cc * 4) =
-                        *reinterpret_cast<const float4_t *>(act + (int64_t)i * p.k + (int64_t)c * kc + cc * 4);
-                }
-                __syncthreads();
-            }
-            for (int tl = 0; tl < ntl; tl++) {
-                const u32x4 cw = cnext;
-                const u32x2 sw = snext;
-                const int tn = min(c * p.cq + tl + 1, p.T - 1);
-                cnext = *reinterpret_cast<const u32x4 *>(grp + (int64_t)tn * kTile + 16 * lane);
-                snext = *reinterpret_cast<const u32x2 *>(grp + (int64_t)tn * kTile + kTileScales + 8 * r16);
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const uint32_t word = cw[j];
-                    float wl[4], wh[4];
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        wl[e] = (float)((word >> (8 * e)) & 0xFu) - 8.0f;
-                        wh[e] = (float)((word >> (8 * e + 4)) & 0xFu) - 8.0f;
-                    }
-                    const float dsc = (float)__builtin_bit_cast(_Float16, (uint16_t)(sw[j >> 1] >> (16 * (j & 1))));
-#pragma unroll
-                    for (int i = 0; i < M; i++) {
-                        const float4_t xl = *reinterpret_cast<const float4_t *>(lds_x + (size_t)i * kc + tl * 128 + j * 32 + 4 * g);
-                        const float4_t xh = *reinterpret_cast<const float4_t *>(lds_x + (size_t)i * kc + tl * 128 + j * 32 + 16 + 4 * g);
-                        float part = 0.0f;
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            part = __builtin_fmaf(wl[e], xl[e], part);
-                            part = __builtin_fmaf(wh[e], xh[e], part);
-                        }
-                        acc[i] = __builtin_fmaf(dsc, part, acc[i]);
-                    }
-                }
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < M; i++) {
-            float v = acc[i];
-            v += __shfl_xor(v, 16);
-            v += __shfl_xor(v, 32);
-            if (gvalid && g == 0) out[(int64_t)i * p.n + (int64_t)gi * 16 + r16] = v;
-        }
-    }
-}
-
 int env_int(const char *name, int dflt) {
     const char *v = getenv(name);
     return v ? atoi(v) : dflt;
 }
 
-template <int KS, int PD, bool CHUNKED>
+template <int KS, int PD, bool CHUNKED, bool F32>
 int launch_mfma_ks(TiledDev p, int64_t act_batch, int per_cu_forced, hipStream_t s) {
     constexpr int S = kW / KS;
-    const size_t lds = (size_t)p.m * p.cq * 128 * 2 + (KS > 1 ? (size_t)2 * kW * 4 * 64 * sizeof(float) : 0);
+    const size_t lds = (size_t)p.m * p.cq * 128 * 2 * (F32 ? 3 : 1) + (KS > 1 ? (size_t)2 * kW * 4 * 64 * sizeof(float) : 0);
     if (lds > 64 * 1024 &&      // beyond the default limit of dynamic LDS: allowed per kernel (and device) on request
-        hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_0_tiled_mfma_kernel<KS, PD, CHUNKED>), hipFuncAttributeMaxDynamicSharedMemorySize,
+        hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_0_tiled_mfma_kernel<KS, PD, CHUNKED, F32>), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
         (void)hipGetLastError();
         return fail("q4_0_matvec (tiled weights): %zu bytes of LDS were refused", lds);
     }
     int64_t per_cu = (160 * 1024) / (int64_t)lds;
-    if (per_cu > 2) per_cu = 2;     // (by registers: 4 or 5 waves per SIMD)
+    if (per_cu > (F32 ? 1 : 2)) per_cu = F32 ? 1 : 2;     // (by registers: 4 or 5 waves per SIMD; 2 or 3 with f32 activations)
     if (per_cu < 1) per_cu = 1;
     if (per_cu_forced > 0) per_cu = per_cu_forced;
     const int64_t units = (p.groups + S - 1) / S;
@@ -396,13 +374,23 @@ int launch_mfma_ks(TiledDev p, int64_t act_batch, int per_cu_forced, hipStream_t
         wgs = (units + rounds - 1) / rounds;
     }
     p.rounds = (int)rounds;
-    hipLaunchKernelGGL((q4_0_tiled_mfma_kernel<KS, PD, CHUNKED>), dim3((unsigned)wgs, (unsigned)act_batch), dim3(64 * kW), lds, s, p);
+    hipLaunchKernelGGL((q4_0_tiled_mfma_kernel<KS, PD, CHUNKED, F32>), dim3((unsigned)wgs, (unsigned)act_batch), dim3(64 * kW), lds, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("q4_0_matvec (tiled weights) launch failed: %s", hipGetErrorString(e));
     return 0;
 }
 
-int launch_tiled_mfma(TiledDev p, int64_t act_batch, hipStream_t s) {
+template <bool CHUNKED, bool F32>
+int launch_mfma_cf(const TiledDev &p, int ks, int64_t act_batch, int per_cu_forced, hipStream_t s) {
+    switch (ks) {
+        case 1: return launch_mfma_ks<1, 8, CHUNKED, F32>(p, act_batch, per_cu_forced, s);
+        case 2: return launch_mfma_ks<2, 8, CHUNKED, F32>(p, act_batch, per_cu_forced, s);
+        case 4: return launch_mfma_ks<4, 8, CHUNKED, F32>(p, act_batch, per_cu_forced, s);
+        default: return launch_mfma_ks<8, 4, CHUNKED, F32>(p, act_batch, per_cu_forced, s);
+    }
+}
+
+int launch_tiled_mfma(TiledDev p, bool f32, int64_t act_batch, hipStream_t s) {
     static const int forced_ks = env_int("TROCM_Q4T_KS", 0);
     static const int forced_per_cu = env_int("TROCM_Q4T_WG_PER_CU", 0);
     static const int forced_lds_kb = env_int("TROCM_Q4T_LDS_KB", 0);
@@ -419,67 +407,26 @@ int launch_tiled_mfma(TiledDev p, int64_t act_batch, hipStream_t s) {
     if (p.m <= 2) ks = 8;   // (one or two rows: never slower, 14336 x 4096 8.9 against 9.2 us)
     while (ks > 1 && ks > p.T) ks /= 2;
     if (forced_ks == 1 || forced_ks == 2 || forced_ks == 4 || forced_ks == 8) ks = forced_ks;
-    const int pd = ks == 8 ? 4 : 8;
-    // The activations whole in LDS if they fit beside the partial sums; else in chunks of a multiple of KS PD tiles:
-    // 64 KB (two workgroups per compute unit cover each other's staging), or 128 KB where 64 KB hold no such chunk.
+    int pd = ks == 8 ? 4 : 8;
+    // The activations whole in LDS if they fit beside the partial sums (2 bytes per feature; 6 as three bf16 planes of
+    // f32 activations); else in chunks of a multiple of KS PD tiles: 64 KB (two workgroups per compute unit cover each
+    // other's staging), or 128 KB where 64 KB hold no such chunk.
     const int64_t red = ks > 1 ? 2 * kW * 4 * 64 * 4 : 0;
-    const int64_t whole = (int64_t)p.m * p.k * 2;
+    const int64_t per_tile = (int64_t)p.m * 256 * (f32 ? 3 : 1);
     const int64_t lds_all = forced_lds_kb > 0 ? (int64_t)forced_lds_kb * 1024 : 160 * 1024;
-    if (whole + red <= lds_all) {
+    if (per_tile * p.T + red <= lds_all) {
         p.cq = p.T, p.nch = 1;
     } else {
+        while (ks > 1 && (int64_t)ks * (ks == 8 ? 4 : 8) * per_tile > 128 * 1024) ks /= 2;   // (a chunk holds KS PD tiles at least)
+        pd = ks == 8 ? 4 : 8;
         const int64_t step = ks * pd;
-        int64_t cq = (64 * 1024) / ((int64_t)p.m * 256) / step * step;
-        if (cq < step) cq = (128 * 1024) / ((int64_t)p.m * 256) / step * step;
+        int64_t cq = (64 * 1024) / per_tile / step * step;
+        if (cq < step) cq = (128 * 1024) / per_tile / step * step;
         if (cq < step) return fail("q4_0_matvec (tiled weights): %d activation rows leave no room for a chunk", p.m);
         p.cq = (int)cq, p.nch = (int)((p.T + cq - 1) / cq);
     }
-    if (p.nch > 1) switch (ks) {
-        case 1: return launch_mfma_ks<1, 8, true>(p, act_batch, forced_per_cu, s);
-        case 2: return launch_mfma_ks<2, 8, true>(p, act_batch, forced_per_cu, s);
-        case 4: return launch_mfma_ks<4, 8, true>(p, act_batch, forced_per_cu, s);
-        default: return launch_mfma_ks<8, 4, true>(p, act_batch, forced_per_cu, s);
-    }
-    switch (ks) {
-        case 1: return launch_mfma_ks<1, 8, false>(p, act_batch, forced_per_cu, s);
-        case 2: return launch_mfma_ks<2, 8, false>(p, act_batch, forced_per_cu, s);
-        case 4: return launch_mfma_ks<4, 8, false>(p, act_batch, forced_per_cu, s);
-        default: return launch_mfma_ks<8, 4, false>(p, act_batch, forced_per_cu, s);
-    }
-}
-
-template <int M>
-int launch_vec_m(TiledDev p, int64_t act_batch, hipStream_t s) {
-    int64_t cq = kVecLds / ((int64_t)M * 128 * 4);
-    if (cq > p.T) cq = p.T;
-    p.cq = (int)cq, p.nch = (int)((p.T + cq - 1) / cq);
-    const int64_t units = (p.groups + 3) / 4;
-    int64_t resident = (int64_t)num_compute_units() * 4 / act_batch;
-    if (resident < 1) resident = 1;
-    int64_t wgs = units, rounds = 1;
-    if (units > resident) {
-        rounds = (units + resident - 1) / resident;
-        wgs = (units + rounds - 1) / rounds;
-    }
-    p.rounds = (int)rounds;
-    hipLaunchKernelGGL((q4_0_tiled_vec_f32_kernel<M>), dim3((unsigned)wgs, (unsigned)act_batch), dim3(256), (size_t)M * p.cq * 128 * 4, s, p);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return fail("q4_0_matvec (tiled weights, f32) launch failed: %s", hipGetErrorString(e));
-    return 0;
-}
-
-int launch_tiled_vec(const TiledDev &p, int64_t act_batch, hipStream_t s) {
-    switch (p.m) {
-        case 1: return launch_vec_m<1>(p, act_batch, s);
-        case 2: return launch_vec_m<2>(p, act_batch, s);
-        case 3: return launch_vec_m<3>(p, act_batch, s);
-        case 4: return launch_vec_m<4>(p, act_batch, s);
-        case 5: return launch_vec_m<5>(p, act_batch, s);
-        case 6: return launch_vec_m<6>(p, act_batch, s);
-        case 7: return launch_vec_m<7>(p, act_batch, s);
-        case 8: return launch_vec_m<8>(p, act_batch, s);
-    }
-    return fail("q4_0_matvec (tiled weights, f32): m = %d activation rows (1..8 are handled per launch)", p.m);
+    if (p.nch > 1) return f32 ? launch_mfma_cf<true, true>(p, ks, act_batch, forced_per_cu, s) : launch_mfma_cf<true, false>(p, ks, act_batch, forced_per_cu, s);
+    return f32 ? launch_mfma_cf<false, true>(p, ks, act_batch, forced_per_cu, s) : launch_mfma_cf<false, false>(p, ks, act_batch, forced_per_cu, s);
 }
 
 }  // namespace
@@ -509,9 +456,8 @@ int launch_q4_0_tiled_export(const void *tiles, void *blocks, int64_t rows, int6
     return 0;
 }
 
-// Tiled weights x activations for any m: f16 rows in groups of up to 16 on the matrix cores (more than 16 rows go to the
-// matrix-matrix kernel first, which reads the same tiles, when it takes the call), f32 rows in groups of 8 on the
-// vector ALU.
+// Tiled weights x activations for any m: f16 rows in groups of up to 16 (more than 16 rows go to the matrix-matrix
+// kernel first, which reads the same tiles, when it takes the call), f32 rows in groups of up to 8.
 int launch_q4_0_tiled_matvec(const void *tiles, int64_t w_batch, int64_t n, int64_t k, const void *act, int act_dtype,
                              int64_t act_batch, int64_t m, void *out, hipStream_t s) {
     if (n >= (1ll << 30) || k >= (1ll << 30) || act_batch > 65535) return fail("q4_0_matvec: shape too large");
@@ -528,7 +474,7 @@ int launch_q4_0_tiled_matvec(const void *tiles, int64_t w_batch, int64_t n, int6
         p.act_stride_b = m * k, p.out_stride_b = m * n;
         p.n = (int)n, p.k = (int)k, p.m = (int)(m - i0 < step ? m - i0 : step), p.ratio = (int)(act_batch / w_batch);
         p.T = (int)(k / 128), p.groups = (int)(n / 16);
-        const int rc = act_dtype == TROCM_F16 ? launch_tiled_mfma(p, act_batch, s) : launch_tiled_vec(p, act_batch, s);
+        const int rc = launch_tiled_mfma(p, act_dtype != TROCM_F16, act_batch, s);
         if (rc) return rc;
     }
     return 0;
