@@ -767,6 +767,31 @@ def run_ops(ta, args):
         blob = rng.integers(0, 256, (n_, k_ // 32 * 18), dtype=np.uint8)
         blob[:, 1::18] = (blob[:, 1::18] & 0x03) | 0x28      # scales: small finite f16 values
         ws = [ta.Q40Weights(blob, 1, n_, k_) for _ in range(8)]
+        # the same matrices as planes of codes and scales (what a matrix that is not whole tiles of 16 rows x 128
+        # features is held as), for comparison: one and eight f16 rows
+        os.environ["TROCM_Q4_TILED"] = "0"
+        wp = [ta.Q40Weights(blob, 1, n_, k_) for _ in range(8)]
+        del os.environ["TROCM_Q4_TILED"]
+        for m_ in (1, 8):
+            xp = ta.DeviceTensor.from_numpy(rng.standard_normal((1, m_, k_)).astype(np.float16))
+            op = ta.DeviceTensor((1, m_, n_), np.float16)
+
+            def one_planes():
+                gemm.eval(xp, wp[turn[0] % 8], out=op)
+                turn[0] += 1
+
+            res[f"q4_0_matvec_f16_m{m_}_n{n_}_k{k_}_planes"] = {"us": round(time_calls(ta, one_planes, 200), 2)}
+        del wp
+        # f32 activations: one and four rows (three bf16 planes per activation on the matrix cores)
+        for m_ in (1, 4):
+            xf = ta.DeviceTensor.from_numpy(rng.standard_normal((1, m_, k_)).astype(np.float32))
+            of = ta.DeviceTensor((1, m_, n_), np.float32)
+
+            def one_f32():
+                gemm.eval(xf, ws[turn[0] % 8], out=of)
+                turn[0] += 1
+
+            res[f"q4_0_matvec_f32_m{m_}_n{n_}_k{k_}"] = {"us": round(time_calls(ta, one_f32, 200), 2)}
         xa = ta.DeviceTensor.from_numpy(rng.standard_normal((1, 1, k_)).astype(np.float16))
         oa = ta.DeviceTensor((1, 1, n_), np.float16)
 

@@ -28,8 +28,8 @@
 //
 // f32 activations, 1..8 rows: the same kernel with v_mfma_f32_16x16x32_bf16.  Staging splits every activation into
 // three bf16 numbers of 8 significant bits each (x = b1 + b2 + b3 exactly, by truncation and exact remainders), kept as
-// three planes in LDS; the codes 64 + code are exact in bf16, so every product is exact and the sums are taken in f32
-// inside the instructions, smallest parts first: the arithmetic of an f32 kernel, over the whole range of f32.
+// three planes in LDS; the codes enter as 16 + code, exact in bf16, so every product is exact and the sums are taken in
+// f32 inside the instructions, smallest parts first: the arithmetic of an f32 kernel, over the whole range of f32.
 //
 // Roofline: HBM-bound on the weights: 18 bytes per 32 weights, read once.
 #include <hip/hip_fp16.h>
@@ -113,11 +113,13 @@ __device__ __forceinline__ half8_t codes_plus_64(uint32_t c) {
 
 // CHUNKED: the activations do not fit LDS and are staged in nch chunks per round.  (A kernel of its own: with loads
 // for the staging inside the loop over the rounds, the compiler drains every load at the head of the tile loop.)
-// The same as bf16: 0x4280 is 64, whose last place between 64 and 128 is 1/2: the code shifted left by one.
-__device__ __forceinline__ bf16x8_t codes_plus_64_bf16(uint32_t c) {
-    const uint32_t lo = ((c << 1) & 0x1E1E1E1Eu) | 0x80808080u, hi = ((c >> 3) & 0x1E1E1E1Eu) | 0x80808080u;
-    const uint32_t a = perm(0x42424242u, lo, 0x04010400u), b = perm(0x42424242u, lo, 0x04030402u);
-    const uint32_t c2 = perm(0x42424242u, hi, 0x04010400u), d = perm(0x42424242u, hi, 0x04030402u);
+// As bf16 the offset can be smaller (the sums then round at a third of the magnitude): 0x4180 is 16, whose last place
+// between 16 and 32 is 1/8: the code shifted left by three stays inside the low byte.  16 + code, and -24 in the
+// second instruction.
+__device__ __forceinline__ bf16x8_t codes_plus_16_bf16(uint32_t c) {
+    const uint32_t lo = ((c << 3) & 0x78787878u) | 0x80808080u, hi = ((c >> 1) & 0x78787878u) | 0x80808080u;
+    const uint32_t a = perm(0x41414141u, lo, 0x04010400u), b = perm(0x41414141u, lo, 0x04030402u);
+    const uint32_t c2 = perm(0x41414141u, hi, 0x04010400u), d = perm(0x41414141u, hi, 0x04030402u);
     return __builtin_bit_cast(bf16x8_t, u32x4{a, b, c2, d});
 }
 
@@ -150,8 +152,8 @@ __global__ __launch_bounds__(64 * kW, F32 ? 2 : 4) void q4_0_tiled_mfma_kernel(T
     // data, so that no load sits behind a branch (which would turn every later wait for one load into a wait for all).
     u32x4 cn[PD];
     u32x2 sn[PD];
-    const uint32_t m72 = F32 ? 0xC290C290u : 0xD480D480u;      // -72 as two bf16 or two f16
-    const u32x4 minus_72 = {m72, m72, m72, m72};
+    const uint32_t m72 = F32 ? 0xC1C0C1C0u : 0xD480D480u;      // -24 as two bf16, -72 as two f16
+    const u32x4 minus_72 = {m72, m72, m72, m72};                 // (the offset that the second instruction takes off)
     struct Group { const uint8_t *base; uint32_t bytes; };
     auto group_of = [&](int round) {
         const int64_t gi = (blockIdx.x + (int64_t)round * gridDim.x) * S + st;
@@ -280,7 +282,7 @@ __global__ __launch_bounds__(64 * kW, F32 ? 2 : 4) void q4_0_tiled_mfma_kernel(T
                         if constexpr (F32) {
                             bf16x8_t codes[4];
 #pragma unroll
-                            for (int j = 0; j < 4; j++) codes[j] = codes_plus_64_bf16(cn[d][j]), part[j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                            for (int j = 0; j < 4; j++) codes[j] = codes_plus_16_bf16(cn[d][j]), part[j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                             for (int pl = 2; pl >= 0; pl--) {     // the smallest parts first
 #pragma unroll
