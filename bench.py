@@ -763,24 +763,28 @@ def run_ops(ta, args):
     # Q4_0 weights x one activation row (the decode-time projections of an 8B-class decoder), f16; each
     # shape rotates over 8 weight matrices so that launches read HBM
     gemm = ta.GgmlGemm()
-    for n_, k_ in ((14336, 4096), (4096, 14336), (4096, 4096)):
+    for n_, k_ in ((14336, 4096), (4096, 14336), (4096, 4096), (128256, 4096)):
+        nw = 8 if n_ < 100000 else 3
         blob = rng.integers(0, 256, (n_, k_ // 32 * 18), dtype=np.uint8)
         blob[:, 1::18] = (blob[:, 1::18] & 0x03) | 0x28      # scales: small finite f16 values
-        ws = [ta.Q40Weights(blob, 1, n_, k_) for _ in range(8)]
-        # the same matrices as planes of codes and scales (what a matrix that is not whole tiles of 16 rows x 128
-        # features is held as), for comparison: one and eight f16 rows
+        ws = [ta.Q40Weights(blob, 1, n_, k_) for _ in range(nw)]
+        # 1..16 f16 rows against the tiles, and against the same matrices as planes of codes and scales (what a matrix
+        # that is not whole tiles of 16 rows x 128 features is held as)
         os.environ["TROCM_Q4_TILED"] = "0"
-        wp = [ta.Q40Weights(blob, 1, n_, k_) for _ in range(8)]
+        wp = [ta.Q40Weights(blob, 1, n_, k_) for _ in range(nw)]
         del os.environ["TROCM_Q4_TILED"]
-        for m_ in (1, 8):
+        for m_ in (1, 2, 4, 8, 16):
             xp = ta.DeviceTensor.from_numpy(rng.standard_normal((1, m_, k_)).astype(np.float16))
             op = ta.DeviceTensor((1, m_, n_), np.float16)
+            row = {}
+            for tag, mats in (("tiles_us", ws), ("planes_us", wp)):
+                def one_rows():
+                    gemm.eval(xp, mats[turn[0] % nw], out=op)
+                    turn[0] += 1
 
-            def one_planes():
-                gemm.eval(xp, wp[turn[0] % 8], out=op)
-                turn[0] += 1
-
-            res[f"q4_0_matvec_f16_m{m_}_n{n_}_k{k_}_planes"] = {"us": round(time_calls(ta, one_planes, 200), 2)}
+                row[tag] = round(time_calls(ta, one_rows, 200), 2)
+            row["tiles_gbs"] = round((n_ * (k_ // 32) * 18 + m_ * 2 * (k_ + n_)) / row["tiles_us"] / 1e3, 1)
+            res[f"q4_0_rows_f16_m{m_}_n{n_}_k{k_}"] = row
         del wp
         # f32 activations: one and four rows (three bf16 planes per activation on the matrix cores)
         for m_ in (1, 4):
@@ -788,10 +792,13 @@ def run_ops(ta, args):
             of = ta.DeviceTensor((1, m_, n_), np.float32)
 
             def one_f32():
-                gemm.eval(xf, ws[turn[0] % 8], out=of)
+                gemm.eval(xf, ws[turn[0] % nw], out=of)
                 turn[0] += 1
 
             res[f"q4_0_matvec_f32_m{m_}_n{n_}_k{k_}"] = {"us": round(time_calls(ta, one_f32, 200), 2)}
+        if n_ > 100000:
+            del ws
+            continue
         xa = ta.DeviceTensor.from_numpy(rng.standard_normal((1, 1, k_)).astype(np.float16))
         oa = ta.DeviceTensor((1, 1, n_), np.float16)
 
