@@ -36,8 +36,8 @@ HBM_PEAK_GBS = 8000.0
 # HBM traffic of one decode-attention launch at the default arguments (batch 8, context 8226 in the
 # kernel loop), from two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE), each
 # counter scaled by what it reads for the 128 MiB prefill copy of known size: FETCH_SIZE
-# 134394.6 x 1.9991 KiB + WRITE_SIZE 1226 x 1.000 KiB.
-PMC_TRAFFIC_BYTES_B8_CTX8226 = int((134394.6 * 1.9991 + 1226.0) * 1024)
+# 134135.5 x 1.9991 KiB + WRITE_SIZE 650 x 0.9993 KiB.
+PMC_TRAFFIC_BYTES_B8_CTX8226 = int((134135.5 * 1.9991 + 650.0 * 0.9993) * 1024)
 PMC_ALGORITHMIC_BYTES_B8_CTX8226 = 2 * 8 * 8 * 8226 * 128 * 2 + 2 * 8 * 32 * 128 * 2
 
 
