@@ -325,6 +325,48 @@ print(json.dumps(o.astype(np.float32).reshape(-1).tolist()))
     assert max_abs(got, cases.textbook_sdpa(q, k, v)) <= 2e-3
 
 
+@pytest.mark.parametrize("period,splits", [(2, 4), (3, 2), (5, 8), (16, 4)])
+def test_decode_with_unequal_shares_of_the_splits(rt, period, splits):
+    """Odd splits (they run on the odd XCDs, which stream slower) leave every `period`-th round of tile groups to their
+    even neighbours.  Small periods make many such rounds at a test's size; steps with the fused append and RoPE go
+    through the same tile sequence.  Expected: the textbook result, and the same cache contents as without."""
+    import subprocess, sys, json
+    code = f"""
+import os, json, numpy as np
+os.environ['TROCM_DECODE_XCD_SKEW']='{period}'
+os.environ['TROCM_DECODE_SPLITS']='{splits}'
+import tract_amd
+tract_amd.runtime_for_name('rocm')
+rng=np.random.default_rng(17)
+T=5000
+q=(rng.standard_normal((3,2,32,1,128),dtype=np.float32)/11.3).astype(np.float16)
+k=rng.standard_normal((2,8,T,128),dtype=np.float32).astype(np.float16)
+v=rng.standard_normal((2,8,T,128),dtype=np.float32).astype(np.float16)
+kn=rng.standard_normal((3,2,8,1,128),dtype=np.float32).astype(np.float16)
+vn=rng.standard_normal((3,2,8,1,128),dtype=np.float32).astype(np.float16)
+st=tract_amd.InPlaceKvSdpa(2,True).state()
+st.eval([q[0][:, :, :1], k, v])
+outs=[st.eval([q[i], kn[i], vn[i]]).to_numpy().astype(np.float32).reshape(-1).tolist() for i in range(3)]
+tail=st.k.valid_contiguous()[:, :, -3:].astype(np.float32).reshape(-1).tolist()
+print(json.dumps([outs, tail]))
+"""
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, check=True,
+                         cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__)))).stdout
+    outs, tail = json.loads(out.strip().splitlines()[-1])
+    rng = np.random.default_rng(17)
+    T = 5000
+    q = (rng.standard_normal((3, 2, 32, 1, 128), dtype=np.float32) / 11.3).astype(np.float16)
+    k = rng.standard_normal((2, 8, T, 128), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((2, 8, T, 128), dtype=np.float32).astype(np.float16)
+    kn = rng.standard_normal((3, 2, 8, 1, 128), dtype=np.float32).astype(np.float16)
+    vn = rng.standard_normal((3, 2, 8, 1, 128), dtype=np.float32).astype(np.float16)
+    for i in range(3):
+        k, v = np.concatenate([k, kn[i]], axis=2), np.concatenate([v, vn[i]], axis=2)
+        got = np.array(outs[i], dtype=np.float32).reshape(2, 32, 1, 128)
+        assert max_abs(got, cases.textbook_sdpa(q[i], k, v)) <= 2e-3
+    assert np.array_equal(np.array(tail, dtype=np.float32).reshape(2, 8, 3, 128), k[:, :, -3:].astype(np.float32))
+
+
 def test_inplace_kv_sdpa_decode_loop_cfg1(rt):
     """cfg1: B=1, 32 q heads = 32 kv heads, D=64, f32, cache grows 0 -> 256 one token per
     step with causal attention at each step; fused op vs {concat cache, FlashSdpaOp}."""

@@ -31,6 +31,7 @@ struct DecodeDev {
     // dense f16/f32 kernel: 1 = the splits of a sequence take groups of kWaves tiles round-robin
     // (concurrent workgroups then read neighbouring addresses), 0 = contiguous tile ranges
     int interleave;
+    int xcd_skew;                 // period (in rounds of groups) of the rounds that odd splits leave to even ones; 0: none
     // != NULL: arrival counters (one int per (batch, kv head), zero between launches); the last
     // workgroup of a sequence-head to arrive merges the splits itself and no merge launch follows
     int *counters;

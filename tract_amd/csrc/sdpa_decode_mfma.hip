@@ -76,6 +76,9 @@ struct MfmaWork {
     int T, tile_begin, tile_end;
     int tile_step;                // a wave's next tile: kWaves (a contiguous range) or kWaves * splits (the splits of a
                                   // dense sequence-head take groups of kWaves tiles in turn)
+    int skew_period, skew_split;  // > 0 (f16 body, interleaved splits, an even number of them): in every skew_period-th
+                                  // round of groups the odd splits take none and their even neighbours two.  Workgroups go
+                                  // to the 8 XCDs in turn, so odd splits run on odd XCDs, which stream about a tenth slower.
     int nsplit;                   // splits of this sequence-head (1: write the output rows)
     int64_t slot;                 // partial record of this workgroup
     int new_pos;                  // token stored by a fused append (-1: none)
@@ -410,10 +413,26 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
     // this lane's mask values: its head's row, tokens 8*rq + 4*hb + 0..3 of the tile
     // (16-wide: tokens 16*mb + 4*(lane/16) + 0..3)
     const char *mask_lane = MASK ? wk.mask + (int64_t)min(hcol, g - 1) * p.mask_stride_h + 8 * (W16 ? q4 : hb) : nullptr;
-    const int tstep = wk.tile_step;
-    for (; t < tile_end; t += tstep) {
+    // The wave's tiles in order: t, then tn.  Plain: a fixed step.  Skewed: round r of nsplit groups gives split s group
+    // nsplit r + s, except that in the rounds r % R == R - 1 an even split takes its odd neighbour's group as well
+    // (e = 1) and the odd split none.
+    const int tstep = wk.tile_step, R = wk.skew_period, nsp = wk.nsplit, sp = wk.skew_split;
+    int sr = 0, se = 0, sj = 0;               // round, extra group, r % R of the tile AFTER t
+    auto advance = [&](int from) {
+        if (R == 0) return from + tstep;
+        if ((sp & 1) == 0) {
+            if (se == 0 && sj == R - 1) se = 1;
+            else sr++, se = 0, sj = sj + 1 == R ? 0 : sj + 1;
+        } else {
+            sr++, sj = sj + 1 == R ? 0 : sj + 1;
+            if (sj == R - 1) sr++, sj = 0;
+        }
+        return (nsp * sr + sp + se) * kWaves + w;
+    };
+    int tn = advance(t);
+    for (; t < tile_end; t = tn, tn = advance(tn)) {
         const int t0 = t * kTile;
-        const bool more = t + tstep < tile_end;
+        const bool more = tn < tile_end;
         constexpr int NMK = W16 ? 2 : 4;          // groups of 4 consecutive tokens this lane owns in a tile
         constexpr int kMkStep = W16 ? 16 : 8;     // tokens between them
         half4_t mk[MASK ? NMK : 1];
@@ -435,11 +454,11 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
         // ---- K tile -> LDS, the next tile's K into flight ----------------------------------------------
         if constexpr (QUANT) {
             stash_q(kpre, ksc, k_slot);
-            if (more) fetch_q(kbase, wk.ksbase, t + tstep, kpre, ksc);
+            if (more) fetch_q(kbase, wk.ksbase, tn, kpre, ksc);
         } else {
 #pragma unroll
             for (int j = 0; j < NLD; j++) *reinterpret_cast<u32x4 *>(tile + k_slot[j]) = kpre[j];
-            if (more) fetch(kbase, p.k_new, t + tstep, kpre, true);
+            if (more) fetch(kbase, p.k_new, tn, kpre, true);
         }
         half8_t pf16;
         if constexpr (W16) {
@@ -540,11 +559,11 @@ __device__ __forceinline__ void decode_mfma_body(const DecodeDev &p, const MfmaW
         // ---- V tile -> the same LDS tile (every K fragment has been consumed), next V into flight ------
         if constexpr (QUANT) {
             stash_q(vpre, vsc, v_slot);
-            if (more) fetch_q(vbase, wk.vsbase, t + tstep, vpre, vsc);
+            if (more) fetch_q(vbase, wk.vsbase, tn, vpre, vsc);
         } else {
 #pragma unroll
             for (int j = 0; j < NLD; j++) *reinterpret_cast<u32x4 *>(tile + v_slot[j]) = vpre[j];
-            if (more) fetch(vbase, p.v_new, t + tstep, vpre);
+            if (more) fetch(vbase, p.v_new, tn, vpre);
         }
         // ---- O^T += V^T P^T ---------------------------------------------------------------------------------
         const _Float16 *vsrc = tile + vsrc_off;
@@ -1900,8 +1919,11 @@ __global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma
         }
     }
     const int n_tiles = (wk.T + kTile - 1) / kTile;
+    wk.skew_period = 0, wk.skew_split = split;
     if (p.interleave) {   // concurrent workgroups read neighbouring addresses
         wk.tile_begin = split * kWaves, wk.tile_end = n_tiles, wk.tile_step = kWaves * p.nsplit;
+        if constexpr (QB == 0 || QB / 100 == 9)
+            if (p.xcd_skew >= 2 && p.nsplit % 2 == 0) wk.skew_period = p.xcd_skew;
     } else {
         wk.tile_begin = split * tiles_per_split;
         wk.tile_end = min(n_tiles, wk.tile_begin + tiles_per_split);
@@ -1942,6 +1964,7 @@ __global__ __launch_bounds__(kThreads, (QB ? QB % 10 : 2)) void sdpa_decode_mfma
     }
     wk.T = it.T;
     wk.tile_begin = it.tile_begin, wk.tile_end = it.tile_end, wk.tile_step = kWaves;
+    wk.skew_period = 0, wk.skew_split = 0;
     wk.nsplit = it.nsplit;
     wk.slot = ((int64_t)it.slot0 + it.split) * p.Hkv + kvh;
     wk.new_pos = p.k_new ? it.T - 1 : -1;
@@ -2260,6 +2283,13 @@ int launch_sdpa_decode_mfma(const SdpaArgs &a, hipStream_t s) {
     p.part_o = p.part_ml + (size_t)BH * nsplit * 2 * gp;
     static const int interleave = getenv("TROCM_DECODE_INTERLEAVE") ? atoi(getenv("TROCM_DECODE_INTERLEAVE")) : 1;
     p.interleave = interleave;
+    // Workgroups are handed to the 8 XCDs in turn and the odd XCDs stream about a tenth slower than the even ones
+    // (time stamps per workgroup: the tile loops of a launch of equal shares end at 33 - 36 us on XCDs 0, 2, 4, 6 and
+    // at 37 - 40 us on 1, 3, 5, 7, whatever the shares' addresses): with an even number of splits the odd splits sit
+    // on odd XCDs, and in every 16th round of groups they leave their group to their even neighbour (17 : 15).
+    // TROCM_DECODE_XCD_SKEW: the period in rounds, 0 = equal shares.
+    static const int xcd_skew = getenv("TROCM_DECODE_XCD_SKEW") ? atoi(getenv("TROCM_DECODE_XCD_SKEW")) : 16;
+    p.xcd_skew = xcd_skew;
     p.live_trim = decode_live_trim();
     if (a.mask) {   // [mask_b, mask_h, 1, Sk] dense f16
         p.mask = (const char *)a.mask;
