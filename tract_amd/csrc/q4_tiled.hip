@@ -463,6 +463,8 @@ int launch_q4_0_tiled_export(const void *tiles, void *blocks, int64_t rows, int6
 int launch_q4_0_tiled_matvec(const void *tiles, int64_t w_batch, int64_t n, int64_t k, const void *act, int act_dtype,
                              int64_t act_batch, int64_t m, void *out, hipStream_t s) {
     if (n >= (1ll << 30) || k >= (1ll << 30) || act_batch > 65535) return fail("q4_0_matvec: shape too large");
+    // (a row group's records are addressed through one buffer descriptor: 32-bit offsets)
+    if ((k / 128) * kTile >= (1ll << 31)) return fail("q4_0_matvec: rows of %lld features are too long for the tiled layout", (long long)k);
     if (act_dtype == TROCM_F16 && m > 16) {
         const int rc = launch_q4_0_matmul(tiles, nullptr, w_batch, n, k, act, act_dtype, act_batch, m, out, s, 1);
         if (rc != 2) return rc;
