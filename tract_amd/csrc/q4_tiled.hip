@@ -433,7 +433,9 @@ int launch_tiled_mfma(TiledDev p, bool f32, int64_t act_batch, hipStream_t s) {
 
 }  // namespace
 
-bool q4_0_tiled_layout_fits(int64_t n, int64_t k) { return n % 16 == 0 && k % 128 == 0 && n >= 16 && k >= 128; }
+bool q4_0_tiled_layout_fits(int64_t n, int64_t k) {
+    return n % 16 == 0 && k % 128 == 0 && n >= 16 && k >= 128 && (k / 128) * kTile < (1ll << 31);   // (32-bit offsets within a row group)
+}
 size_t q4_0_tiled_bytes(int64_t rows, int64_t k) { return (size_t)(rows / 16) * (size_t)(k / 128) * kTile; }
 
 int launch_q4_0_tiled_import(const void *blocks, void *tiles, int64_t rows, int64_t k, hipStream_t s) {
