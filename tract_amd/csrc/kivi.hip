@@ -36,6 +36,43 @@ __device__ __forceinline__ float ld(const float *p) { return *p; }
 // signalling one, and the next operation of the chain, which ignores that NaN, has then lost what came before it;
 // f32::min / f32::max skip every NaN alike.
 __device__ __forceinline__ float quiet(float x) { return __builtin_canonicalizef(x); }
+
+// Exchanges between lanes on the vector ALU (DPP modifiers and the lane-swap instructions) instead of through the LDS
+// crossbar (`__shfl_xor` = ds_bpermute_b32: the per-token ingest spent 14 of its 101 us on eight of those per lane).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+// x of lane (l ^ M) for M = 8, 16, 32 combined with this lane's by OP (min or max): exact partners.
+template <int M, typename Op>
+__device__ __forceinline__ float xor_combine(float x, Op op) {
+    static_assert(M == 8 || M == 16 || M == 32, "lane distances 8, 16, 32");
+    if constexpr (M == 8) {
+        return op(x, dpp_move<0x128>(x));                       // row_ror:8 within a row of 16 lanes
+    } else {   // rows 2k and 2k + 1 (halves of the wave) trade places between the two results: one of them is this lane's own
+        unsigned a = __builtin_bit_cast(unsigned, x), b = a;
+        asm("" : "+v"(b));   // two registers: the instruction swaps in place, and both results are read
+        const auto sw = M == 16 ? __builtin_amdgcn_permlane16_swap(a, b, false, false) : __builtin_amdgcn_permlane32_swap(a, b, false, false);
+        unsigned s0 = sw[0], s1 = sw[1];
+        asm("" : "+v"(s0), "+v"(s1));   // (this compiler folds op(sw[0], sw[1]) to sw[0] when both operands were one value: the minimum was lost)
+        return op(__builtin_bit_cast(float, s0), __builtin_bit_cast(float, s1));
+    }
+}
+// Minimum and maximum over aligned groups of N lanes (8, 16, 32, 64), left in every lane of the group.  (Any order of
+// exchanges gives the same bits: both are exact.)  Quads, halves of a row and rows by DPP, then pairs of rows, then the
+// two halves of the wave.
+template <int N>
+__device__ __forceinline__ void group_min_max(float &lo, float &hi) {
+    static_assert(N == 8 || N == 16 || N == 32 || N == 64, "groups of 8, 16, 32 or 64 lanes");
+    auto mn = [](float a, float b) { return fminf(a, b); };
+    auto mx = [](float a, float b) { return fmaxf(a, b); };
+    lo = fminf(lo, dpp_move<0xB1>(lo)), hi = fmaxf(hi, dpp_move<0xB1>(hi));       // quad_perm [1,0,3,2]
+    lo = fminf(lo, dpp_move<0x4E>(lo)), hi = fmaxf(hi, dpp_move<0x4E>(hi));       // quad_perm [2,3,0,1]
+    lo = fminf(lo, dpp_move<0x141>(lo)), hi = fmaxf(hi, dpp_move<0x141>(hi));     // row_half_mirror: the other quad of 8 lanes
+    if constexpr (N >= 16) lo = fminf(lo, dpp_move<0x140>(lo)), hi = fmaxf(hi, dpp_move<0x140>(hi));   // row_mirror: the other half of the row
+    if constexpr (N >= 32) lo = xor_combine<16>(lo, mn), hi = xor_combine<16>(hi, mx);
+    if constexpr (N >= 64) lo = xor_combine<32>(lo, mn), hi = xor_combine<32>(hi, mx);
+}
 __device__ __forceinline__ float ld(const __half *p) { return __half2float(*p); }
 
 // f32 -> f16 as its own instruction: without the barrier the compiler may fold the preceding multiply and add
@@ -128,11 +165,7 @@ __global__ void __launch_bounds__(256) kivi_quant_tokens_kernel(const SrcT *__re
         lo = fminf(lo, quiet(v));
         hi = fmaxf(hi, quiet(v));
     }
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) {
-        lo = fminf(lo, __shfl_xor(lo, m, 64));
-        hi = fmaxf(hi, __shfl_xor(hi, m, 64));
-    }
+    group_min_max<64>(lo, hi);
     constexpr float lv = (float)((1u << BITS) - 1u);
     const float scale = affine_scale(lo, hi, lv);
     uint8_t *out = codes + ((int64_t)bh * cap_rows + row0 + i) * row_bytes;
@@ -585,11 +618,7 @@ __global__ void __launch_bounds__(256) kivi_quant_tokens_vec_kernel(const SrcT *
         lo = fminf(lo, quiet(x.v[e]));
         hi = fmaxf(hi, quiet(x.v[e]));
     }
-#pragma unroll
-    for (int m = LPR / 2; m >= 1; m >>= 1) {
-        lo = fminf(lo, __shfl_xor(lo, m, 64));
-        hi = fmaxf(hi, __shfl_xor(hi, m, 64));
-    }
+    group_min_max<LPR>(lo, hi);
     const float scale = affine_scale(lo, hi, lv), inv = affine_inv(scale);
     uint32_t code[8];
     affine_codes8(x.v, lo, scale, inv, lv, code);
@@ -634,11 +663,7 @@ __global__ void __launch_bounds__(128) kivi_step_push_kernel(const SrcT *__restr
             lo = fminf(lo, quiet(x.v[e]));
             hi = fmaxf(hi, quiet(x.v[e]));
         }
-#pragma unroll
-        for (int m = 8; m >= 1; m >>= 1) {
-            lo = fminf(lo, __shfl_xor(lo, m, 64));
-            hi = fmaxf(hi, __shfl_xor(hi, m, 64));
-        }
+        group_min_max<16>(lo, hi);
         const float scale = affine_scale(lo, hi, 255.0f), inv = affine_inv(scale);
         uint32_t code[8];
         affine_codes8(x.v, lo, scale, inv, 255.0f, code);
@@ -681,12 +706,14 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_vec_kernel(const Src
             hi[e] = fmaxf(hi[e], quiet(x.v[e]));
         }
     }
-#pragma unroll
-    for (int m = LPR; m < 64; m <<= 1) {
+    {   // the lane groups' rows joined: lanes LPR, 2 LPR, ... apart hold the same channels
+        auto mn = [](float a, float b) { return fminf(a, b); };
+        auto mx = [](float a, float b) { return fmaxf(a, b); };
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            lo[e] = fminf(lo[e], __shfl_xor(lo[e], m, 64));
-            hi[e] = fmaxf(hi[e], __shfl_xor(hi[e], m, 64));
+            if constexpr (LPR <= 8) lo[e] = xor_combine<8>(lo[e], mn), hi[e] = xor_combine<8>(hi[e], mx);
+            if constexpr (LPR <= 16) lo[e] = xor_combine<16>(lo[e], mn), hi[e] = xor_combine<16>(hi[e], mx);
+            if constexpr (LPR <= 32) lo[e] = xor_combine<32>(lo[e], mn), hi[e] = xor_combine<32>(hi[e], mx);
         }
     }
     F8 ls, ss;
