@@ -23,8 +23,10 @@
 // walks `rounds` such sets.  Every wave keeps a ring of PD tiles in flight that runs on across the end of a round into
 // the next round's first tiles, so that neither the reduction over the KS waves nor the barrier in front of it leaves
 // the memory pipe idle.  Arithmetic: the contraction of the instruction is 32 deep, one quantisation block; the codes
-// enter as the exact f16 integers -8 .. 7, the products accumulate in f32 inside the instruction from zero, and the
-// block's sum is scaled by its f16 scale with one fma per output.
+// enter as the exact f16 numbers 64 + code (one v_perm_b32 per two codes, no subtraction), a second instruction per
+// block with the constant operand -72 takes the offset off, both accumulate in f32 inside the instructions from zero,
+// and the block's sum is scaled by its f16 scale with one fma per output.  Every product is exact; the sums round at
+// the magnitude 72 |x| (1e-5 of a block's sum, below the f16 result's own rounding).
 //
 // f32 activations, 1..8 rows: the same kernel with v_mfma_f32_16x16x32_bf16.  Staging splits every activation into
 // three bf16 numbers of 8 significant bits each (x = b1 + b2 + b3 exactly, by truncation and exact remainders), kept as
@@ -111,8 +113,6 @@ __device__ __forceinline__ half8_t codes_plus_64(uint32_t c) {
     return __builtin_bit_cast(half8_t, u32x4{a, b, c2, d});
 }
 
-// CHUNKED: the activations do not fit LDS and are staged in nch chunks per round.  (A kernel of its own: with loads
-// for the staging inside the loop over the rounds, the compiler drains every load at the head of the tile loop.)
 // As bf16 the offset can be smaller (the sums then round at a third of the magnitude): 0x4180 is 16, whose last place
 // between 16 and 32 is 1/8: the code shifted left by three stays inside the low byte.  16 + code, and -24 in the
 // second instruction.
@@ -123,6 +123,8 @@ __device__ __forceinline__ bf16x8_t codes_plus_16_bf16(uint32_t c) {
     return __builtin_bit_cast(bf16x8_t, u32x4{a, b, c2, d});
 }
 
+// CHUNKED: the activations do not fit LDS and are staged in nch chunks per round.  (A kernel of its own: with loads
+// for the staging inside the loop over the rounds, the compiler drains every load at the head of the tile loop.)
 // F32: f32 activations and output, three bf16 planes in LDS (else f16 activations and output).
 template <int KS, int PD, bool CHUNKED, bool F32>
 __global__ __launch_bounds__(64 * kW, F32 ? 2 : 4) void q4_0_tiled_mfma_kernel(TiledDev p) {
