@@ -424,7 +424,9 @@ int launch_tiled_mfma(TiledDev p, bool f32, int64_t act_batch, hipStream_t s) {
         while (ks > 1 && (int64_t)ks * (ks == 8 ? 4 : 8) * per_tile > 128 * 1024) ks /= 2;   // (a chunk holds KS PD tiles at least)
         pd = ks == 8 ? 4 : 8;
         const int64_t step = ks * pd;
-        int64_t cq = (64 * 1024) / per_tile / step * step;
+        static const int forced_chunk_kb = env_int("TROCM_Q4T_CHUNK_KB", 0);
+        const int64_t first = forced_chunk_kb > 0 ? (int64_t)forced_chunk_kb * 1024 : 64 * 1024;
+        int64_t cq = first / per_tile / step * step;
         if (cq < step) cq = (128 * 1024) / per_tile / step * step;
         if (cq < step) return fail("q4_0_matvec (tiled weights): %d activation rows leave no room for a chunk", p.m);
         p.cq = (int)cq, p.nch = (int)((p.T + cq - 1) / cq);
