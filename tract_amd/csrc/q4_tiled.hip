@@ -53,6 +53,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kTile = 1152;        // bytes per tile record
 constexpr int kTileScales = 1024;  // offset of the scales in a record
 constexpr int kW = 8;              // waves per workgroup of the f16 kernel
+constexpr int kActF16 = 0, kActF32 = 1, kActF32Rows = 2;   // how the activations enter the matrix instruction (see the kernel)
 
 // ---- layout ---------------------------------------------------------------------------------------------------------
 // Canonical blocks [rows, nb, 18 bytes] (f16 scale, 16 code bytes; 2-byte aligned) <-> tiles.  One thread per block.
@@ -125,16 +126,20 @@ __device__ __forceinline__ bf16x8_t codes_plus_16_bf16(uint32_t c) {
 
 // CHUNKED: the activations do not fit LDS and are staged in nch chunks per round.  (A kernel of its own: with loads
 // for the staging inside the loop over the rounds, the compiler drains every load at the head of the tile loop.)
-// F32: f32 activations and output, three bf16 planes in LDS (else f16 activations and output).
-template <int KS, int PD, bool CHUNKED, bool F32>
-__global__ __launch_bounds__(64 * kW, F32 ? 2 : 4) void q4_0_tiled_mfma_kernel(TiledDev p) {
+// ACT: kActF16 = f16 activations and output; kActF32 = f32 activations and output, three bf16 planes in LDS, each its own
+// matrix instruction (up to 8 rows); kActF32Rows = f32 activations of up to 4 rows whose three bf16 parts are ROWS
+// 4 i, 4 i + 1, 4 i + 2 of the instruction's A operand: one instruction forms the three partial products of a row, and a
+// lane's first three outputs are summed at the end (the matrix instructions and the LDS reads of one f16 row).
+template <int KS, int PD, bool CHUNKED, int ACT>
+__global__ __launch_bounds__(64 * kW, ACT == kActF32 ? 2 : 4) void q4_0_tiled_mfma_kernel(TiledDev p) {
+    constexpr bool F32 = ACT != kActF16, FOLD = ACT == kActF32Rows;
     using ActT = typename std::conditional<F32, float, _Float16>::type;
-    constexpr int NPL = F32 ? 3 : 1;                 // planes of 16-bit numbers per activation
+    constexpr int NPL = ACT == kActF32 ? 3 : 1;      // planes of 16-bit numbers per activation
     constexpr int kThreads = 64 * kW, S = kW / KS;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const int kc = p.cq * 128;                       // staged features per activation row
-    uint16_t *lds_x = reinterpret_cast<uint16_t *>(lds_raw);                                // [NPL][m][kc], 16-byte vectors swizzled
-    const int plane = p.m * kc;                      // 16-bit numbers per plane
+    uint16_t *lds_x = reinterpret_cast<uint16_t *>(lds_raw);                                // [NPL][m][kc] ([3 m][kc]: row 3 i + part), 16-byte vectors swizzled
+    const int plane = (FOLD ? 3 : 1) * p.m * kc;     // 16-bit numbers per plane
     float *red = reinterpret_cast<float *>(lds_raw + (size_t)NPL * plane * 2);              // [2][kW][4][64] (KS > 1)
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -142,7 +147,8 @@ __global__ __launch_bounds__(64 * kW, F32 ? 2 : 4) void q4_0_tiled_mfma_kernel(T
     const int b = blockIdx.y, wb = b / p.ratio;
     const ActT *act = reinterpret_cast<const ActT *>(p.act) + (int64_t)b * p.act_stride_b;
     ActT *out = reinterpret_cast<ActT *>(p.out) + (int64_t)b * p.out_stride_b;
-    const int arow = min(r16, p.m - 1);              // output rows m..15 of the instruction are never stored: any row serves
+    // output rows m..15 of the instruction (rows 4 i + 3 and 4 m.. of the three-part rows) are never stored: any row serves
+    const int arow = FOLD ? min(3 * (r16 >> 2) + min(r16 & 3, 2), 3 * p.m - 1) : min(r16, p.m - 1);
     const int ni = p.T > q ? (p.T - q + KS - 1) / KS : 0;   // this wave's tiles of a row group: q + KS tt, tt < ni
     const int cqw = p.cq / KS;                       // ... of which a full chunk holds cqw (a multiple of PD when nch > 1)
     const uint8_t *wbase = p.tiles + (int64_t)wb * p.groups * p.T * kTile;
@@ -207,6 +213,7 @@ __global__ __launch_bounds__(64 * kW, F32 ? 2 : 4) void q4_0_tiled_mfma_kernel(T
                         // features 4 pp .. 4 pp + 3 of the tile: vector (pp / 8) * 4 + pp % 4, half (pp / 4) % 2 of it, in each plane
                         const int vecg = (pp >> 3) * 4 + (pp & 3), hi = (pp >> 2) & 1;
                         const int dst = i * kc + tl * 128 + hi * 4 + (vecg ^ (i & 15)) * 8;
+                        const int in_row = tl * 128 + hi * 4;
                         // (the elements by name: indexed by the counter of an unrolled loop, this compiler has been seen
                         // to read element 0 of an ext-vector every time)
                         const uint32_t xe[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
@@ -222,7 +229,7 @@ __global__ __launch_bounds__(64 * kW, F32 ? 2 : 4) void q4_0_tiled_mfma_kernel(T
                         }
 #pragma unroll
                         for (int pl = 0; pl < 3; pl++)
-                            *reinterpret_cast<u32x2 *>(lds_x + pl * plane + dst) =
+                            *reinterpret_cast<u32x2 *>(lds_x + (FOLD ? (3 * i + pl) * kc + in_row + (vecg ^ ((3 * i + pl) & 15)) * 8 : pl * plane + dst)) =
                                 u32x2{perm(part[pl][1], part[pl][0], 0x07060302u), perm(part[pl][3], part[pl][2], 0x07060302u)};
                     } else {
                         // features 8 pp .. 8 pp + 7 of the tile: the halves of two neighbouring vectors
@@ -281,7 +288,7 @@ __global__ __launch_bounds__(64 * kW, F32 ? 2 : 4) void q4_0_tiled_mfma_kernel(T
                         const int tl = tl_off + KS * tt;
                         u32x4 a[4];
                         float4_t part[4];
-                        if constexpr (F32) {
+                        if constexpr (ACT == kActF32) {
                             bf16x8_t codes[4];
 #pragma unroll
                             for (int j = 0; j < 4; j++) codes[j] = codes_plus_16_bf16(cn[d][j]), part[j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
@@ -294,6 +301,13 @@ __global__ __launch_bounds__(64 * kW, F32 ? 2 : 4) void q4_0_tiled_mfma_kernel(T
 #pragma unroll
                                 for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[j]), codes[j], part[j], 0, 0, 0);
                             }
+                        } else if constexpr (FOLD) {
+#pragma unroll
+                            for (int j = 0; j < 4; j++) a[j] = *reinterpret_cast<const u32x4 *>(lds_x + arow * kc + (tl * 16 + ((j * 4 + g) ^ arow)) * 8);
+#pragma unroll
+                            for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[j]), __builtin_bit_cast(bf16x8_t, minus_72), float4_t{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+#pragma unroll
+                            for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[j]), codes_plus_16_bf16(cn[d][j]), part[j], 0, 0, 0);
                         } else {
 #pragma unroll
                             for (int j = 0; j < 4; j++) a[j] = *reinterpret_cast<const u32x4 *>(lds_x + arow * kc + (tl * 16 + ((j * 4 + g) ^ arow)) * 8);
@@ -318,9 +332,24 @@ __global__ __launch_bounds__(64 * kW, F32 ? 2 : 4) void q4_0_tiled_mfma_kernel(T
         }
         g_cur = g_next;
 
-        // acc[e] = partial out[4 g + e][16 gi + r16]
+        // acc[e] = partial out[4 g + e][16 gi + r16] (three-part rows: part e of out[g][16 gi + r16], smallest part first)
         const int64_t row = gi * 16 + r16;
-        if constexpr (KS == 1) {
+        if constexpr (FOLD) {
+            const float mine = (acc[2] + acc[1]) + acc[0];
+            if constexpr (KS == 1) {
+                if (gvalid && g < p.m) out[(int64_t)g * p.n + row] = mine;
+            } else {
+                float *rb = red + (round & 1) * (kW * 4 * 64);
+                rb[(w * 4) * 64 + lane] = mine;
+                __syncthreads();
+                if (q == 0) {
+                    float sum = 0.0f;
+#pragma unroll
+                    for (int ww = 0; ww < KS; ww++) sum += rb[((st * KS + ww) * 4) * 64 + lane];
+                    if (gvalid && g < p.m) out[(int64_t)g * p.n + row] = sum;
+                }
+            }
+        } else if constexpr (KS == 1) {
 #pragma unroll
             for (int e = 0; e < 4; e++)
                 if (gvalid && 4 * g + e < p.m) out[(int64_t)(4 * g + e) * p.n + row] = (ActT)acc[e];
@@ -355,18 +384,20 @@ int env_int(const char *name, int dflt) {
     return v ? atoi(v) : dflt;
 }
 
-template <int KS, int PD, bool CHUNKED, bool F32>
+template <int KS, int PD, bool CHUNKED, int ACT>
 int launch_mfma_ks(TiledDev p, int64_t act_batch, int per_cu_forced, hipStream_t s) {
     constexpr int S = kW / KS;
+    constexpr bool F32 = ACT != kActF16;
     const size_t lds = (size_t)p.m * p.cq * 128 * 2 * (F32 ? 3 : 1) + (KS > 1 ? (size_t)2 * kW * 4 * 64 * sizeof(float) : 0);
     if (lds > 64 * 1024 &&      // beyond the default limit of dynamic LDS: allowed per kernel (and device) on request
-        hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_0_tiled_mfma_kernel<KS, PD, CHUNKED, F32>), hipFuncAttributeMaxDynamicSharedMemorySize,
+        hipFuncSetAttribute(reinterpret_cast<const void *>(&q4_0_tiled_mfma_kernel<KS, PD, CHUNKED, ACT>), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
         (void)hipGetLastError();
         return fail("q4_0_matvec (tiled weights): %zu bytes of LDS were refused", lds);
     }
     int64_t per_cu = (160 * 1024) / (int64_t)lds;
-    if (per_cu > (F32 ? 1 : 2)) per_cu = F32 ? 1 : 2;     // (by registers: 4 or 5 waves per SIMD; 2 or 3 with f32 activations)
+    constexpr int kMaxPerCu = ACT == kActF32 ? 1 : 2;     // (by registers: 4 or 5 waves per SIMD; 2 or 3 with three planes)
+    if (per_cu > kMaxPerCu) per_cu = kMaxPerCu;
     if (per_cu < 1) per_cu = 1;
     if (per_cu_forced > 0) per_cu = per_cu_forced;
     const int64_t units = (p.groups + S - 1) / S;
@@ -378,19 +409,19 @@ int launch_mfma_ks(TiledDev p, int64_t act_batch, int per_cu_forced, hipStream_t
         wgs = (units + rounds - 1) / rounds;
     }
     p.rounds = (int)rounds;
-    hipLaunchKernelGGL((q4_0_tiled_mfma_kernel<KS, PD, CHUNKED, F32>), dim3((unsigned)wgs, (unsigned)act_batch), dim3(64 * kW), lds, s, p);
+    hipLaunchKernelGGL((q4_0_tiled_mfma_kernel<KS, PD, CHUNKED, ACT>), dim3((unsigned)wgs, (unsigned)act_batch), dim3(64 * kW), lds, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("q4_0_matvec (tiled weights) launch failed: %s", hipGetErrorString(e));
     return 0;
 }
 
-template <bool CHUNKED, bool F32>
+template <bool CHUNKED, int ACT>
 int launch_mfma_cf(const TiledDev &p, int ks, int64_t act_batch, int per_cu_forced, hipStream_t s) {
     switch (ks) {
-        case 1: return launch_mfma_ks<1, 8, CHUNKED, F32>(p, act_batch, per_cu_forced, s);
-        case 2: return launch_mfma_ks<2, 8, CHUNKED, F32>(p, act_batch, per_cu_forced, s);
-        case 4: return launch_mfma_ks<4, 8, CHUNKED, F32>(p, act_batch, per_cu_forced, s);
-        default: return launch_mfma_ks<8, 4, CHUNKED, F32>(p, act_batch, per_cu_forced, s);
+        case 1: return launch_mfma_ks<1, 8, CHUNKED, ACT>(p, act_batch, per_cu_forced, s);
+        case 2: return launch_mfma_ks<2, 8, CHUNKED, ACT>(p, act_batch, per_cu_forced, s);
+        case 4: return launch_mfma_ks<4, 8, CHUNKED, ACT>(p, act_batch, per_cu_forced, s);
+        default: return launch_mfma_ks<8, 4, CHUNKED, ACT>(p, act_batch, per_cu_forced, s);
     }
 }
 
@@ -431,8 +462,16 @@ int launch_tiled_mfma(TiledDev p, bool f32, int64_t act_batch, hipStream_t s) {
         if (cq < step) return fail("q4_0_matvec (tiled weights): %d activation rows leave no room for a chunk", p.m);
         p.cq = (int)cq, p.nch = (int)((p.T + cq - 1) / cq);
     }
-    if (p.nch > 1) return f32 ? launch_mfma_cf<true, true>(p, ks, act_batch, forced_per_cu, s) : launch_mfma_cf<true, false>(p, ks, act_batch, forced_per_cu, s);
-    return f32 ? launch_mfma_cf<false, true>(p, ks, act_batch, forced_per_cu, s) : launch_mfma_cf<false, false>(p, ks, act_batch, forced_per_cu, s);
+    // f32 rows: up to 4 as three-part rows of one instruction, 5..8 as three planes (TROCM_Q4T_F32_ROWS=0: always planes)
+    static const int f32_rows = env_int("TROCM_Q4T_F32_ROWS", 1);
+    const int act = !f32 ? kActF16 : (p.m <= 4 && f32_rows) ? kActF32Rows : kActF32;
+    if (p.nch > 1)
+        return act == kActF16 ? launch_mfma_cf<true, kActF16>(p, ks, act_batch, forced_per_cu, s)
+             : act == kActF32 ? launch_mfma_cf<true, kActF32>(p, ks, act_batch, forced_per_cu, s)
+                              : launch_mfma_cf<true, kActF32Rows>(p, ks, act_batch, forced_per_cu, s);
+    return act == kActF16 ? launch_mfma_cf<false, kActF16>(p, ks, act_batch, forced_per_cu, s)
+         : act == kActF32 ? launch_mfma_cf<false, kActF32>(p, ks, act_batch, forced_per_cu, s)
+                          : launch_mfma_cf<false, kActF32Rows>(p, ks, act_batch, forced_per_cu, s);
 }
 
 }  // namespace
