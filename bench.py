@@ -786,7 +786,7 @@ def run_ops(ta, args):
             row["tiles_gbs"] = round((n_ * (k_ // 32) * 18 + m_ * 2 * (k_ + n_)) / row["tiles_us"] / 1e3, 1)
             res[f"q4_0_rows_f16_m{m_}_n{n_}_k{k_}"] = row
         del wp
-        # f32 activations: one and four rows (three bf16 planes per activation on the matrix cores)
+        # f32 activations: one and four rows (three bf16 parts per activation as rows of the matrix instruction)
         for m_ in (1, 4):
             xf = ta.DeviceTensor.from_numpy(rng.standard_normal((1, m_, k_)).astype(np.float32))
             of = ta.DeviceTensor((1, m_, n_), np.float32)

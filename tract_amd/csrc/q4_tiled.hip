@@ -29,9 +29,12 @@
 // the magnitude 72 |x| (1e-5 of a block's sum, below the f16 result's own rounding).
 //
 // f32 activations, 1..8 rows: the same kernel with v_mfma_f32_16x16x32_bf16.  Staging splits every activation into
-// three bf16 numbers of 8 significant bits each (x = b1 + b2 + b3 exactly, by truncation and exact remainders), kept as
-// three planes in LDS; the codes enter as 16 + code, exact in bf16, so every product is exact and the sums are taken in
-// f32 inside the instructions, smallest parts first: the arithmetic of an f32 kernel, over the whole range of f32.
+// three bf16 numbers of 8 significant bits each (x = b1 + b2 + b3 exactly, by truncation and exact remainders), which
+// become ROWS 4 i, 4 i + 1, 4 i + 2 of the instruction's A operand for activation row i of a set of four: one
+// instruction forms the three partial products of four rows, each summed in f32 over all of k, and a lane's first
+// three outputs are added at the end, smallest part first.  The codes enter as 16 + code, exact in bf16, so every
+// product is exact: the arithmetic of an f32 kernel, over the whole range of f32, for the matrix instructions and LDS
+// reads of an f16 row (rows 5..8: a second set, twice those).
 //
 // Roofline: HBM-bound on the weights: 18 bytes per 32 weights, read once.
 #include <hip/hip_fp16.h>
@@ -53,7 +56,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kTile = 1152;        // bytes per tile record
 constexpr int kTileScales = 1024;  // offset of the scales in a record
 constexpr int kW = 8;              // waves per workgroup of the f16 kernel
-constexpr int kActF16 = 0, kActF32 = 1, kActF32Rows = 2;   // how the activations enter the matrix instruction (see the kernel)
+constexpr int kActF16 = 0, kActF32Rows = 1, kActF32Rows2 = 2;   // how the activations enter the matrix instruction (see the kernel)
 
 // ---- layout ---------------------------------------------------------------------------------------------------------
 // Canonical blocks [rows, nb, 18 bytes] (f16 scale, 16 code bytes; 2-byte aligned) <-> tiles.  One thread per block.
@@ -126,21 +129,19 @@ __device__ __forceinline__ bf16x8_t codes_plus_16_bf16(uint32_t c) {
 
 // CHUNKED: the activations do not fit LDS and are staged in nch chunks per round.  (A kernel of its own: with loads
 // for the staging inside the loop over the rounds, the compiler drains every load at the head of the tile loop.)
-// ACT: kActF16 = f16 activations and output; kActF32 = f32 activations and output, three bf16 planes in LDS, each its own
-// matrix instruction (up to 8 rows); kActF32Rows = f32 activations of up to 4 rows whose three bf16 parts are ROWS
-// 4 i, 4 i + 1, 4 i + 2 of the instruction's A operand: one instruction forms the three partial products of a row, and a
-// lane's first three outputs are summed at the end (the matrix instructions and the LDS reads of one f16 row).
+// ACT: kActF16 = f16 activations and output (up to 16 rows); kActF32Rows = f32 activations and output, up to 4 rows
+// as three-part rows; kActF32Rows2 = 5..8 rows as two sets of them.
 template <int KS, int PD, bool CHUNKED, int ACT>
-__global__ __launch_bounds__(64 * kW, ACT == kActF32 ? 2 : 4) void q4_0_tiled_mfma_kernel(TiledDev p) {
-    constexpr bool F32 = ACT != kActF16, FOLD = ACT == kActF32Rows;
+__global__ __launch_bounds__(64 * kW, ACT == kActF32Rows2 ? 2 : 4) void q4_0_tiled_mfma_kernel(TiledDev p) {
+    constexpr bool F32 = ACT != kActF16;
+    constexpr int NSET = ACT == kActF32Rows2 ? 2 : 1;   // sets of four activation rows, an instruction per block each
     using ActT = typename std::conditional<F32, float, _Float16>::type;
-    constexpr int NPL = ACT == kActF32 ? 3 : 1;      // planes of 16-bit numbers per activation
+    constexpr int LR = F32 ? 3 : 1;                  // rows of 16-bit numbers in LDS per activation row
     constexpr int kThreads = 64 * kW, S = kW / KS;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const int kc = p.cq * 128;                       // staged features per activation row
-    uint16_t *lds_x = reinterpret_cast<uint16_t *>(lds_raw);                                // [NPL][m][kc] ([3 m][kc]: row 3 i + part), 16-byte vectors swizzled
-    const int plane = (FOLD ? 3 : 1) * p.m * kc;     // 16-bit numbers per plane
-    float *red = reinterpret_cast<float *>(lds_raw + (size_t)NPL * plane * 2);              // [2][kW][4][64] (KS > 1)
+    uint16_t *lds_x = reinterpret_cast<uint16_t *>(lds_raw);                                // [m][kc] ([3 m][kc]: row 3 i + part), 16-byte vectors swizzled
+    float *red = reinterpret_cast<float *>(lds_raw + (size_t)LR * p.m * kc * 2);            // [2][kW][4][64] (KS > 1)
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int q = w % KS, st = w / KS;               // this wave's share of a row group's tiles, its row group of the set
@@ -148,7 +149,8 @@ __global__ __launch_bounds__(64 * kW, ACT == kActF32 ? 2 : 4) void q4_0_tiled_mf
     const ActT *act = reinterpret_cast<const ActT *>(p.act) + (int64_t)b * p.act_stride_b;
     ActT *out = reinterpret_cast<ActT *>(p.out) + (int64_t)b * p.out_stride_b;
     // output rows m..15 of the instruction (rows 4 i + 3 and 4 m.. of the three-part rows) are never stored: any row serves
-    const int arow = FOLD ? min(3 * (r16 >> 2) + min(r16 & 3, 2), 3 * p.m - 1) : min(r16, p.m - 1);
+    const int arow = F32 ? min(3 * (r16 >> 2) + min(r16 & 3, 2), 3 * p.m - 1) : min(r16, p.m - 1);
+    const int arow2 = min(arow + 12, 3 * p.m - 1);   // (three-part rows: the second set of four rows)
     const int ni = p.T > q ? (p.T - q + KS - 1) / KS : 0;   // this wave's tiles of a row group: q + KS tt, tt < ni
     const int cqw = p.cq / KS;                       // ... of which a full chunk holds cqw (a multiple of PD when nch > 1)
     const uint8_t *wbase = p.tiles + (int64_t)wb * p.groups * p.T * kTile;
@@ -210,9 +212,8 @@ __global__ __launch_bounds__(64 * kW, ACT == kActF32 ? 2 : 4) void q4_0_tiled_mf
                     int i, tl, pp;
                     where(u, i, tl, pp);
                     if constexpr (F32) {
-                        // features 4 pp .. 4 pp + 3 of the tile: vector (pp / 8) * 4 + pp % 4, half (pp / 4) % 2 of it, in each plane
+                        // features 4 pp .. 4 pp + 3 of the tile: vector (pp / 8) * 4 + pp % 4, half (pp / 4) % 2 of it, in each of the row's three
                         const int vecg = (pp >> 3) * 4 + (pp & 3), hi = (pp >> 2) & 1;
-                        const int dst = i * kc + tl * 128 + hi * 4 + (vecg ^ (i & 15)) * 8;
                         const int in_row = tl * 128 + hi * 4;
                         // (the elements by name: indexed by the counter of an unrolled loop, this compiler has been seen
                         // to read element 0 of an ext-vector every time)
@@ -229,7 +230,7 @@ __global__ __launch_bounds__(64 * kW, ACT == kActF32 ? 2 : 4) void q4_0_tiled_mf
                         }
 #pragma unroll
                         for (int pl = 0; pl < 3; pl++)
-                            *reinterpret_cast<u32x2 *>(lds_x + (FOLD ? (3 * i + pl) * kc + in_row + (vecg ^ ((3 * i + pl) & 15)) * 8 : pl * plane + dst)) =
+                            *reinterpret_cast<u32x2 *>(lds_x + (3 * i + pl) * kc + in_row + (vecg ^ ((3 * i + pl) & 15)) * 8) =
                                 u32x2{perm(part[pl][1], part[pl][0], 0x07060302u), perm(part[pl][3], part[pl][2], 0x07060302u)};
                     } else {
                         // features 8 pp .. 8 pp + 7 of the tile: the halves of two neighbouring vectors
@@ -265,7 +266,7 @@ __global__ __launch_bounds__(64 * kW, ACT == kActF32 ? 2 : 4) void q4_0_tiled_mf
         const bool gvalid = unit * S + st < p.groups;
         const int64_t gi = unit * S + st;
         const Group g_next = group_of(round + 1);
-        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f}, acc2 = {0.0f, 0.0f, 0.0f, 0.0f};
 
         for (int c = 0; c < (CHUNKED ? p.nch : 1); c++) {
             if constexpr (CHUNKED) {
@@ -288,26 +289,31 @@ __global__ __launch_bounds__(64 * kW, ACT == kActF32 ? 2 : 4) void q4_0_tiled_mf
                         const int tl = tl_off + KS * tt;
                         u32x4 a[4];
                         float4_t part[4];
-                        if constexpr (ACT == kActF32) {
+                        if constexpr (F32) {
                             bf16x8_t codes[4];
 #pragma unroll
-                            for (int j = 0; j < 4; j++) codes[j] = codes_plus_16_bf16(cn[d][j]), part[j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                            for (int j = 0; j < 4; j++) codes[j] = codes_plus_16_bf16(cn[d][j]);
+                            if constexpr (NSET == 2) {   // rows 4..7 first: their sums go to acc2 before part[] is reused
+                                float4_t part2[4];
 #pragma unroll
-                            for (int pl = 2; pl >= 0; pl--) {     // the smallest parts first
+                                for (int j = 0; j < 4; j++) a[j] = *reinterpret_cast<const u32x4 *>(lds_x + arow2 * kc + (tl * 16 + ((j * 4 + g) ^ (arow2 & 15))) * 8);
 #pragma unroll
-                                for (int j = 0; j < 4; j++) a[j] = *reinterpret_cast<const u32x4 *>(lds_x + pl * plane + arow * kc + (tl * 16 + ((j * 4 + g) ^ arow)) * 8);
+                                for (int j = 0; j < 4; j++) part2[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[j]), __builtin_bit_cast(bf16x8_t, minus_72), float4_t{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
 #pragma unroll
-                                for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[j]), __builtin_bit_cast(bf16x8_t, minus_72), part[j], 0, 0, 0);
+                                for (int j = 0; j < 4; j++) part2[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[j]), codes[j], part2[j], 0, 0, 0);
 #pragma unroll
-                                for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[j]), codes[j], part[j], 0, 0, 0);
+                                for (int j = 0; j < 4; j++) {
+                                    const float dsc = (float)__builtin_bit_cast(_Float16, (uint16_t)(sn[d][j >> 1] >> (16 * (j & 1))));
+#pragma unroll
+                                    for (int e = 0; e < 4; e++) acc2[e] = __builtin_fmaf(dsc, part2[j][e], acc2[e]);
+                                }
                             }
-                        } else if constexpr (FOLD) {
 #pragma unroll
                             for (int j = 0; j < 4; j++) a[j] = *reinterpret_cast<const u32x4 *>(lds_x + arow * kc + (tl * 16 + ((j * 4 + g) ^ arow)) * 8);
 #pragma unroll
                             for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[j]), __builtin_bit_cast(bf16x8_t, minus_72), float4_t{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
 #pragma unroll
-                            for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[j]), codes_plus_16_bf16(cn[d][j]), part[j], 0, 0, 0);
+                            for (int j = 0; j < 4; j++) part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[j]), codes[j], part[j], 0, 0, 0);
                         } else {
 #pragma unroll
                             for (int j = 0; j < 4; j++) a[j] = *reinterpret_cast<const u32x4 *>(lds_x + arow * kc + (tl * 16 + ((j * 4 + g) ^ arow)) * 8);
@@ -334,19 +340,22 @@ __global__ __launch_bounds__(64 * kW, ACT == kActF32 ? 2 : 4) void q4_0_tiled_mf
 
         // acc[e] = partial out[4 g + e][16 gi + r16] (three-part rows: part e of out[g][16 gi + r16], smallest part first)
         const int64_t row = gi * 16 + r16;
-        if constexpr (FOLD) {
-            const float mine = (acc[2] + acc[1]) + acc[0];
+        if constexpr (F32) {
+            const float mine[2] = {(acc[2] + acc[1]) + acc[0], (acc2[2] + acc2[1]) + acc2[0]};
             if constexpr (KS == 1) {
-                if (gvalid && g < p.m) out[(int64_t)g * p.n + row] = mine;
+#pragma unroll
+                for (int z = 0; z < NSET; z++)
+                    if (gvalid && 4 * z + g < p.m) out[(int64_t)(4 * z + g) * p.n + row] = mine[z];
             } else {
                 float *rb = red + (round & 1) * (kW * 4 * 64);
-                rb[(w * 4) * 64 + lane] = mine;
+#pragma unroll
+                for (int z = 0; z < NSET; z++) rb[(w * 4 + z) * 64 + lane] = mine[z];
                 __syncthreads();
-                if (q == 0) {
+                if (q < NSET) {   // (KS >= 2 here: wave 0 of the row group sums the first set, wave 1 the second)
                     float sum = 0.0f;
 #pragma unroll
-                    for (int ww = 0; ww < KS; ww++) sum += rb[((st * KS + ww) * 4) * 64 + lane];
-                    if (gvalid && g < p.m) out[(int64_t)g * p.n + row] = sum;
+                    for (int ww = 0; ww < KS; ww++) sum += rb[((st * KS + ww) * 4 + q) * 64 + lane];
+                    if (gvalid && 4 * q + g < p.m) out[(int64_t)(4 * q + g) * p.n + row] = sum;
                 }
             }
         } else if constexpr (KS == 1) {
@@ -396,7 +405,7 @@ int launch_mfma_ks(TiledDev p, int64_t act_batch, int per_cu_forced, hipStream_t
         return fail("q4_0_matvec (tiled weights): %zu bytes of LDS were refused", lds);
     }
     int64_t per_cu = (160 * 1024) / (int64_t)lds;
-    constexpr int kMaxPerCu = ACT == kActF32 ? 1 : 2;     // (by registers: 4 or 5 waves per SIMD; 2 or 3 with three planes)
+    constexpr int kMaxPerCu = ACT == kActF32Rows2 ? 1 : 2;     // (by registers: 4 or 5 waves per SIMD; 2 or 3 with two sets of f32 rows)
     if (per_cu > kMaxPerCu) per_cu = kMaxPerCu;
     if (per_cu < 1) per_cu = 1;
     if (per_cu_forced > 0) per_cu = per_cu_forced;
@@ -443,7 +452,7 @@ int launch_tiled_mfma(TiledDev p, bool f32, int64_t act_batch, hipStream_t s) {
     while (ks > 1 && ks > p.T) ks /= 2;
     if (forced_ks == 1 || forced_ks == 2 || forced_ks == 4 || forced_ks == 8) ks = forced_ks;
     int pd = ks == 8 ? 4 : 8;
-    // The activations whole in LDS if they fit beside the partial sums (2 bytes per feature; 6 as three bf16 planes of
+    // The activations whole in LDS if they fit beside the partial sums (2 bytes per feature; 6 as the three bf16 parts of
     // f32 activations); else in chunks of a multiple of KS PD tiles: 64 KB (two workgroups per compute unit cover each
     // other's staging), or 128 KB where 64 KB hold no such chunk.
     const int64_t red = ks > 1 ? 2 * kW * 4 * 64 * 4 : 0;
@@ -452,7 +461,18 @@ int launch_tiled_mfma(TiledDev p, bool f32, int64_t act_batch, hipStream_t s) {
     if (per_tile * p.T + red <= lds_all) {
         p.cq = p.T, p.nch = 1;
     } else {
+        const int ks_wanted = ks;
         while (ks > 1 && (int64_t)ks * (ks == 8 ? 4 : 8) * per_tile > 128 * 1024) ks /= 2;   // (a chunk holds KS PD tiles at least)
+        if (f32 && p.m > 4 && ks < ks_wanted) {
+            // 6..8 f32 rows of many features: chunks that small hold too few tiles for the waves of a row group, and
+            // with fewer waves per group the launch has too few workgroups (8 rows of 4096 x 14336: 47.8 us; as two
+            // launches of four rows 2 x 17.6).  Activation rows are k apart, output rows n.
+            TiledDev lo = p, hi = p;
+            lo.m = 4, hi.m = p.m - 4;
+            hi.act = (const float *)p.act + 4 * (int64_t)p.k, hi.out = (float *)p.out + 4 * (int64_t)p.n;
+            const int rc = launch_tiled_mfma(lo, f32, act_batch, s);
+            return rc ? rc : launch_tiled_mfma(hi, f32, act_batch, s);
+        }
         pd = ks == 8 ? 4 : 8;
         const int64_t step = ks * pd;
         static const int forced_chunk_kb = env_int("TROCM_Q4T_CHUNK_KB", 0);
@@ -462,16 +482,13 @@ int launch_tiled_mfma(TiledDev p, bool f32, int64_t act_batch, hipStream_t s) {
         if (cq < step) return fail("q4_0_matvec (tiled weights): %d activation rows leave no room for a chunk", p.m);
         p.cq = (int)cq, p.nch = (int)((p.T + cq - 1) / cq);
     }
-    // f32 rows: up to 4 as three-part rows of one instruction, 5..8 as three planes (TROCM_Q4T_F32_ROWS=0: always planes)
-    static const int f32_rows = env_int("TROCM_Q4T_F32_ROWS", 1);
-    const int act = !f32 ? kActF16 : (p.m <= 4 && f32_rows) ? kActF32Rows : kActF32;
     if (p.nch > 1)
-        return act == kActF16 ? launch_mfma_cf<true, kActF16>(p, ks, act_batch, forced_per_cu, s)
-             : act == kActF32 ? launch_mfma_cf<true, kActF32>(p, ks, act_batch, forced_per_cu, s)
-                              : launch_mfma_cf<true, kActF32Rows>(p, ks, act_batch, forced_per_cu, s);
-    return act == kActF16 ? launch_mfma_cf<false, kActF16>(p, ks, act_batch, forced_per_cu, s)
-         : act == kActF32 ? launch_mfma_cf<false, kActF32>(p, ks, act_batch, forced_per_cu, s)
-                          : launch_mfma_cf<false, kActF32Rows>(p, ks, act_batch, forced_per_cu, s);
+        return !f32 ? launch_mfma_cf<true, kActF16>(p, ks, act_batch, forced_per_cu, s)
+             : p.m <= 4 ? launch_mfma_cf<true, kActF32Rows>(p, ks, act_batch, forced_per_cu, s)
+                        : launch_mfma_cf<true, kActF32Rows2>(p, ks, act_batch, forced_per_cu, s);
+    return !f32 ? launch_mfma_cf<false, kActF16>(p, ks, act_batch, forced_per_cu, s)
+         : p.m <= 4 ? launch_mfma_cf<false, kActF32Rows>(p, ks, act_batch, forced_per_cu, s)
+                    : launch_mfma_cf<false, kActF32Rows2>(p, ks, act_batch, forced_per_cu, s);
 }
 
 }  // namespace
