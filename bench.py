@@ -821,9 +821,8 @@ def run_ops(ta, args):
         us = time_calls(ta, one_mv8, 200)
         by8 = n_ * (k_ // 32) * 18 + 8 * 2 * k_ + 8 * 2 * n_
         res[f"q4_0_matvec_f16_m8_n{n_}_k{k_}"] = {"us": round(us, 2), "gbs": round(by8 / us / 1e3, 1), "bytes": by8}
-        if (n_, k_) != (4096, 14336):
-            # the same weights x the 512 rows of a prefill chunk: the matrix-matrix arm, on the matrix cores
-            m_ = 512
+        # the same weights x the rows of a prefill chunk (128, 512, 2048): the matrix-matrix arm, on the matrix cores
+        for m_ in (128, 512, 2048):
             xm = ta.DeviceTensor.from_numpy(rng.standard_normal((1, m_, k_)).astype(np.float16))
             om = ta.DeviceTensor((1, m_, n_), np.float16)
 
@@ -833,6 +832,7 @@ def run_ops(ta, args):
 
             us = time_calls(ta, one_mm, 50)
             res[f"q4_0_matmul_f16_m{m_}_n{n_}_k{k_}"] = {"us": round(us, 2), "tflops": round(2.0 * m_ * n_ * k_ / us / 1e6, 1)}
+            del xm, om
         del ws
     # ragged decode step over quantised caches: 32 sequences of 512..32768 tokens, their new tokens quantised
     # by one launch and attention by another

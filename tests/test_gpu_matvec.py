@@ -63,6 +63,8 @@ TILED_SHAPES = [
     (1, 1, 1, 16, 128), (1, 1, 1, 48, 256), (2, 2, 1, 80, 384), (1, 3, 2, 4096, 1024), (1, 1, 1, 14336, 4096), (1, 1, 3, 4096, 14336),
     (1, 1, 8, 14336, 4096), (1, 1, 8, 4096, 14336), (1, 1, 16, 1040, 8192), (2, 4, 5, 272, 2176), (1, 1, 7, 20000, 128),
     (1, 1, 12, 6000 * 16, 256), (1, 1, 17, 160, 640), (1, 2, 40, 4112, 1152), (1, 1, 130, 2048, 4096),
+    (1, 2, 200, 528, 384), (1, 1, 2100, 4112, 1152),   # the matrix-matrix kernel: 64 and 128 activation rows per workgroup, ragged edges
+    (1, 1, 100, 1024, 768), (1, 1, 400, 8192, 512),      # ... with k split over 2 sets of waves (130 x 2048 x 4096 above: over 4)
 ]
 
 
