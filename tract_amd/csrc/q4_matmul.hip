@@ -182,7 +182,7 @@ __global__ __launch_bounds__(kMmThreads, 2) void q4_0_matmul_kernel(MatMulDev p)
 // as long as both operands agree: the activations are staged with vector v = 4 block + g of a row holding the same
 // eight features.  A workgroup of 4 waves owns 128 NI (n) x BM (m) of C^T, each wave 32 NI x BM: with NI = 2 an
 // activation fragment read from LDS feeds two matrix instructions and a dequantised weight fragment BM / 32, so LDS
-// moves half a fragment per instruction (the kernel above: one, which is all LDS can deliver).  NI = 1 and BM = 64 are
+// moves half a fragment per instruction (the kernel above: one, which is all LDS can deliver).  BM = 64 and then NI = 1 are
 // for launches that would otherwise have fewer workgroups than compute units: each then walks all of k alone, and the
 // time of the launch is the time of one workgroup.  (BM = 256 -- half the dequantisation per matrix instruction, 256
 // accumulator registers, one wave per SIMD -- measured no faster: 8192 rows of 14336 x 4096 856 against 822 us.)
@@ -198,9 +198,9 @@ __global__ __launch_bounds__(kMmThreads * KS, KS == 1 ? 2 : 1) void q4_0_tiled_m
     constexpr int TN = 128 * NI;                 // rows of the weights per workgroup
     // Half tiles of the activations on their way from memory: two where the registers allow it -- the small tiles exist
     // for launches in which a workgroup walks k alone, and a half tile's arithmetic is shorter than a trip to the L2.
-    constexpr int PA = (BM == 128 && NI == 2) ? 1 : 2;
+    constexpr int PA = BM == 128 ? 1 : 2;
     // Tiles of the weights on their way from HBM, likewise: one tile's arithmetic of a small shape is about half of that trip.
-    constexpr int PW = (BM == 128 && NI == 2) ? 1 : 3;
+    constexpr int PW = BM == 128 ? 1 : 3;
     constexpr int AP = BM * 8 / kMmThreads;      // 16-byte activation pieces per thread and half tile
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];   // [KS][2][BM AROW] halves; then the sums
 
@@ -391,17 +391,18 @@ int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, i
     if (tiled) {
         // 32-bit byte offsets inside one weight matrix and one batch of activations (rows up to 128 past m are addressed)
         if (n % 16 || k % TK || (n / 16) * (k / TK) * 1152 >= (1ll << 32) || (m + 128) * k >= (1ll << 30)) return 2;
-        // The largest tile of C^T per workgroup -- 256 (n) x 128 (m), 256 x 64, 128 x 128, 128 x 64 -- that still gives
-        // three quarters of the compute units a workgroup; the smallest when none does, and then (or with 256 x 64) k
+        // The largest tile of C^T per workgroup -- 256 (n) x 128 (m), 256 x 64, 128 x 64 -- that still gives three
+        // quarters of the compute units a workgroup (128 x 128 never has more workgroups than 256 x 64); the smallest
+        // when none does, and then (or with 256 x 64) k
         // split over 2 or 4 sets of waves inside the workgroup while the workgroups are fewer than the compute units
         // can hold of that size.
         static const int forced_bm = getenv("TROCM_Q4_MATMUL_BM") ? atoi(getenv("TROCM_Q4_MATMUL_BM")) : 0;   // (measurements)
         static const int forced_ni = getenv("TROCM_Q4_MATMUL_NI") ? atoi(getenv("TROCM_Q4_MATMUL_NI")) : 0;
         static const int forced_ks = getenv("TROCM_Q4_MATMUL_KS") ? atoi(getenv("TROCM_Q4_MATMUL_KS")) : 0;
         const int64_t cus = num_compute_units();
-        const int shapes[4][2] = {{128, 2}, {64, 2}, {128, 1}, {64, 1}};
+        const int shapes[3][2] = {{128, 2}, {64, 2}, {64, 1}};
         int bm = 64, ni = 1;
-        for (int c = 0; c < 4; c++) {
+        for (int c = 0; c < 3; c++) {
             const int64_t wgs = ((n + 128 * shapes[c][1] - 1) / (128 * shapes[c][1])) * ((m + shapes[c][0] - 1) / shapes[c][0]) * act_batch;
             if (wgs * 4 >= cus * 3) {
                 bm = shapes[c][0], ni = shapes[c][1];
@@ -410,6 +411,7 @@ int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, i
         }
         if (forced_bm == 64 || forced_bm == 128) bm = forced_bm;
         if (forced_ni == 1 || forced_ni == 2) ni = forced_ni;
+        if (bm == 128) ni = 2;
         const int64_t tx = (n + 128 * ni - 1) / (128 * ni), ty = (m + bm - 1) / bm;
         if (ty > 65535) return 2;
         int ks = 1;
@@ -433,7 +435,6 @@ int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, i
         };
         int rc;
         if (bm == 128 && ni == 2) rc = launch(q4_0_tiled_matmul_kernel<128, 2, 1>);
-        else if (bm == 128) rc = launch(q4_0_tiled_matmul_kernel<128, 1, 1>);
         else if (ni == 2) rc = ks == 2 ? launch(q4_0_tiled_matmul_kernel<64, 2, 2>) : launch(q4_0_tiled_matmul_kernel<64, 2, 1>);
         else rc = ks == 4 ? launch(q4_0_tiled_matmul_kernel<64, 1, 4>) : ks == 2 ? launch(q4_0_tiled_matmul_kernel<64, 1, 2>) : launch(q4_0_tiled_matmul_kernel<64, 1, 1>);
         if (rc) return rc;
