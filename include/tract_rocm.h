@@ -220,8 +220,10 @@ typedef struct trocm_q4_weights trocm_q4_weights;
  * padding; the reference pads rows to 512 elements for its kernel, cuda/src/utils.rs:252-280, which
  * this layout does not need).  k must be a multiple of 32 (utils.rs:253).  The copy is laid out for the
  * kernels, not for the caller: a matrix whose n is a multiple of 16 and whose k a multiple of 128 as tiles of
- * 16 rows x 128 features in the order the matrix instruction consumes them, any other as a plane of codes and
- * a plane of scales; trocm_q4_0_weights_export returns the canonical blocks from either. */
+ * 16 rows x 128 features in the order the matrix instruction consumes them (one of up to 3072 rows -- the key
+ * and value projections of a decoder with grouped heads -- keeps the planes beside the tiles, twice its bytes,
+ * for calls with one or two activation rows), any other as a plane of codes and a plane of scales;
+ * trocm_q4_0_weights_export returns the canonical blocks from either. */
 int trocm_q4_0_weights_create(trocm_q4_weights **out, const void *blocks_device, int64_t batch, int64_t n,
                               int64_t k, void *stream);
 int trocm_q4_0_weights_destroy(trocm_q4_weights *weights);

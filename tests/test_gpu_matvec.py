@@ -60,7 +60,7 @@ def test_matvec_matches_the_oracle(rt, dt, wb, ab, m, n, k):
 # workgroup (20000 rows x 128 features), batches that share weights, and more than 16 rows (the matrix-matrix kernel
 # reading tiles; 17 rows of f32 in groups of 8).
 TILED_SHAPES = [
-    (1, 1, 1, 16, 128), (1, 1, 1, 48, 256), (2, 2, 1, 80, 384), (1, 3, 2, 4096, 1024), (1, 1, 1, 14336, 4096), (1, 1, 3, 4096, 14336),
+    (1, 1, 1, 16, 128), (1, 1, 1, 48, 256), (2, 2, 1, 80, 384), (1, 2, 2, 1024, 4096), (1, 1, 3, 1024, 4096), (1, 3, 2, 4096, 1024), (1, 1, 1, 14336, 4096), (1, 1, 3, 4096, 14336),
     (1, 1, 8, 14336, 4096), (1, 1, 8, 4096, 14336), (1, 1, 16, 1040, 8192), (2, 4, 5, 272, 2176), (1, 1, 7, 20000, 128),
     (1, 1, 12, 6000 * 16, 256), (1, 1, 17, 160, 640), (1, 2, 40, 4112, 1152), (1, 1, 130, 2048, 4096),
     (1, 2, 200, 528, 384), (1, 1, 2100, 4112, 1152),   # the matrix-matrix kernel: 64 and 128 activation rows per workgroup, ragged edges
@@ -70,7 +70,7 @@ TILED_SHAPES = [
 
 @pytest.mark.parametrize("dt", [np.float32, np.float16])
 @pytest.mark.parametrize("wb,ab,m,n,k", TILED_SHAPES)
-def test_tiled_weights_match_the_f64_product(rt, dt, wb, ab, m, n, k):
+def test_tiled_weights_match_the_f64_product(rt, monkeypatch, dt, wb, ab, m, n, k):
     rng = np.random.default_rng(n + k + m)
     w = (rng.standard_normal((wb, n, k)) * 0.05).astype(np.float32)
     w[:, :, ::97] *= 8.0
@@ -81,7 +81,16 @@ def test_tiled_weights_match_the_f64_product(rt, dt, wb, ab, m, n, k):
     got = tract_amd.GgmlGemm().eval(act, wq).to_numpy()
     assert got.dtype == dt and got.shape == (ab, m, n)
     tol = 1e-4 if dt == np.float32 else 4e-3
-    assert rel_err(got, f64_product(blocks, act, dt)) <= tol
+    want = f64_product(blocks, act, dt)
+    assert rel_err(got, want) <= tol
+    if n <= 3072 and m <= 2:
+        # a small matrix keeps planes of codes and scales beside its tiles and runs one or two rows over those:
+        # without them (the variable is read when the weights are created) the same call goes over the tiles
+        monkeypatch.setenv("TROCM_Q4_ROWS_TOO", "0")
+        only_tiles = tract_amd.Q40Weights(blocks, wb, n, k)
+        monkeypatch.delenv("TROCM_Q4_ROWS_TOO")
+        assert np.array_equal(only_tiles.blocks(), blocks)
+        assert rel_err(tract_amd.GgmlGemm().eval(act, only_tiles).to_numpy(), want) <= tol
 
 
 def test_tiles_and_planes_hold_the_same_weights(rt, monkeypatch):

@@ -897,6 +897,10 @@ struct trocm_q4_weights {
     int64_t batch, n, k;
     void *codes, *scales;   // [batch * n, k/2] bytes and [batch * n, k/32] f16
     int tiled;              // codes = tiles of 16 rows x 128 features with their scales (q4_tiled.hip), scales = NULL
+    // A small tiled matrix (up to 3072 rows: the key / value projections of a decoder with grouped heads) keeps the
+    // planes as well: its 16-row tiles give the matrix-instruction kernel too few independent pieces for the compute
+    // units, and one or two activation rows run faster over the planes, a wave per row (1024 x 4096: 3.7 against 4.8 us).
+    void *row_codes, *row_scales;
 };
 
 extern "C" {
@@ -928,10 +932,26 @@ int trocm_q4_0_weights_create(trocm_q4_weights **out, const void *blocks, int64_
         delete w;
         return fail("q4_0 weights: hipMalloc failed: %s", hipGetErrorString(e));
     }
-    if (w->tiled ? launch_q4_0_tiled_import(blocks, w->codes, rows, k, s)
-                 : launch_quant_import(TROCM_Q4_0, 1, 1, rows, rows, 0, k, blocks, w->codes, w->scales, s)) {
+    // TROCM_Q4_ROWS_TOO=0 (read at every call): tiles only, whatever the size
+    const char *rows_env = getenv("TROCM_Q4_ROWS_TOO");
+    const bool rows_too = w->tiled && n <= 3072 && !(rows_env && atoi(rows_env) == 0);
+    if (e == hipSuccess && rows_too) {
+        e = hipMalloc(&w->row_codes, (size_t)rows * (size_t)(k / 2));
+        if (e == hipSuccess) e = hipMalloc(&w->row_scales, (size_t)rows * (size_t)(k / 32) * 2);
+        if (e != hipSuccess) {
+            (void)hipFree(w->codes);
+            if (w->row_codes) (void)hipFree(w->row_codes);
+            delete w;
+            return fail("q4_0 weights: hipMalloc failed: %s", hipGetErrorString(e));
+        }
+    }
+    if ((w->tiled ? launch_q4_0_tiled_import(blocks, w->codes, rows, k, s)
+                  : launch_quant_import(TROCM_Q4_0, 1, 1, rows, rows, 0, k, blocks, w->codes, w->scales, s)) ||
+        (rows_too && launch_quant_import(TROCM_Q4_0, 1, 1, rows, rows, 0, k, blocks, w->row_codes, w->row_scales, s))) {
         (void)hipFree(w->codes);
         if (w->scales) (void)hipFree(w->scales);
+        if (w->row_codes) (void)hipFree(w->row_codes);
+        if (w->row_scales) (void)hipFree(w->row_scales);
         delete w;
         return 1;
     }
@@ -944,6 +964,8 @@ int trocm_q4_0_weights_destroy(trocm_q4_weights *w) {
     TROCM_HIP(hipDeviceSynchronize());
     TROCM_HIP(hipFree(w->codes));
     if (w->scales) TROCM_HIP(hipFree(w->scales));
+    if (w->row_codes) TROCM_HIP(hipFree(w->row_codes));
+    if (w->row_scales) TROCM_HIP(hipFree(w->row_scales));
     delete w;
     return 0;
 }
@@ -980,6 +1002,8 @@ int trocm_q4_0_matvec(const trocm_q4_weights *w, const void *act, int act_dtype,
     TROCM_REQUIRE((uintptr_t)act % 16 == 0, "q4_0_matvec: activations must be 16-byte aligned");
     hipStream_t s;
     if (resolve_stream(stream, &s)) return 1;
+    if (w->tiled && w->row_codes && m <= 2)
+        return launch_q4_0_matvec(w->row_codes, w->row_scales, w->batch, w->n, w->k, act, act_dtype, act_batch, m, out, s);
     if (w->tiled) return launch_q4_0_tiled_matvec(w->codes, w->batch, w->n, w->k, act, act_dtype, act_batch, m, out, s);
     return launch_q4_0_matvec(w->codes, w->scales, w->batch, w->n, w->k, act, act_dtype, act_batch, m, out, s);
 }
