@@ -763,8 +763,10 @@ def run_ops(ta, args):
     # Q4_0 weights x one activation row (the decode-time projections of an 8B-class decoder), f16; each
     # shape rotates over 8 weight matrices so that launches read HBM
     gemm = ta.GgmlGemm()
-    for n_, k_ in ((14336, 4096), (4096, 14336), (4096, 4096), (128256, 4096)):
-        nw = 8 if n_ < 100000 else 3
+    for n_, k_ in ((14336, 4096), (4096, 14336), (4096, 4096), (1024, 4096), (128256, 4096)):
+        # (1024 x 4096, the key / value projection: a matrix this small holds tiles and planes, rows 1 and 2 run over the
+        # planes; 64 matrices in rotation)
+        nw = 3 if n_ > 100000 else 64 if n_ < 2048 else 8
         blob = rng.integers(0, 256, (n_, k_ // 32 * 18), dtype=np.uint8)
         blob[:, 1::18] = (blob[:, 1::18] & 0x03) | 0x28      # scales: small finite f16 values
         ws = [ta.Q40Weights(blob, 1, n_, k_) for _ in range(nw)]
@@ -803,7 +805,7 @@ def run_ops(ta, args):
         oa = ta.DeviceTensor((1, 1, n_), np.float16)
 
         def one_mv():
-            gemm.eval(xa, ws[turn[0] % 8], out=oa)
+            gemm.eval(xa, ws[turn[0] % nw], out=oa)
             turn[0] += 1
 
         us = time_calls(ta, one_mv, 200)
@@ -815,7 +817,7 @@ def run_ops(ta, args):
         o8 = ta.DeviceTensor((1, 8, n_), np.float16)
 
         def one_mv8():
-            gemm.eval(x8, ws[turn[0] % 8], out=o8)
+            gemm.eval(x8, ws[turn[0] % nw], out=o8)
             turn[0] += 1
 
         us = time_calls(ta, one_mv8, 200)
@@ -827,7 +829,7 @@ def run_ops(ta, args):
             om = ta.DeviceTensor((1, m_, n_), np.float16)
 
             def one_mm():
-                gemm.eval(xm, ws[turn[0] % 8], out=om)
+                gemm.eval(xm, ws[turn[0] % nw], out=om)
                 turn[0] += 1
 
             us = time_calls(ta, one_mm, 50)
