@@ -65,6 +65,10 @@ TILED_SHAPES = [
     (1, 1, 12, 6000 * 16, 256), (1, 1, 17, 160, 640), (1, 2, 40, 4112, 1152), (1, 1, 130, 2048, 4096),
     (1, 2, 200, 528, 384), (1, 1, 2100, 4112, 1152),   # the matrix-matrix kernel: 64 and 128 activation rows per workgroup, ragged edges
     (1, 1, 100, 1024, 768), (1, 1, 400, 8192, 512),      # ... with k split over 2 sets of waves (130 x 2048 x 4096 above: over 4)
+    # ... sets of 4 waves and of 2 (64 rows of the weights per workgroup; the three small matrices above take sets of one
+    # wave), k over 4, 2 and 1 of them
+    (1, 1, 400, 4096, 512), (1, 1, 400, 4096, 768), (1, 1, 400, 4096, 384),
+    (1, 1, 200, 4096, 512), (1, 1, 200, 4096, 768), (1, 1, 200, 4096, 384),
 ]
 
 

@@ -23,6 +23,7 @@
 #include <hip/hip_fp16.h>
 #include <string.h>
 #include <stdlib.h>
+#include <type_traits>
 #include "common.h"
 
 namespace trocm {
@@ -192,20 +193,24 @@ constexpr int AROW = HK + 8;                 // halves per activation row in LDS
 // KS > 1: KS such sets of 4 waves share the workgroup's tile of C^T and split k between them (set kg takes tiles
 // kg T / KS .. of every row, in LDS buffers of its own), and their accumulators are added through LDS at the end: for
 // launches with so few workgroups that each compute unit would otherwise hold four waves that walk all of k alone.
-template <int BM, int NI, int KS>
-__global__ __launch_bounds__(kMmThreads * KS, KS == 1 ? 2 : 1) void q4_0_tiled_matmul_kernel(MatMulDev p) {
+// NW: waves per set (4; 2 or 1 -- 64 or 32 rows of the weights per workgroup -- when even the smallest tile above leaves
+// compute units without a workgroup: the time of such a launch is the work of one compute unit).
+template <int BM, int NI, int KS, int NW>
+__global__ __launch_bounds__(64 * NW * KS, NW * KS >= 8 ? 1 : 2) void q4_0_tiled_matmul_kernel(MatMulDev p) {
     constexpr int MS = BM / 32;                  // 32-row subtiles of m
-    constexpr int TN = 128 * NI;                 // rows of the weights per workgroup
+    constexpr int TS = 64 * NW;                  // threads of a set
+    constexpr int TN = 32 * NI * NW;             // rows of the weights per workgroup
     // Half tiles of the activations on their way from memory: two where the registers allow it -- the small tiles exist
     // for launches in which a workgroup walks k alone, and a half tile's arithmetic is shorter than a trip to the L2.
     constexpr int PA = BM == 128 ? 1 : 2;
     // Tiles of the weights on their way from HBM, likewise: one tile's arithmetic of a small shape is about half of that trip.
     constexpr int PW = BM == 128 ? 1 : 3;
-    constexpr int AP = BM * 8 / kMmThreads;      // 16-byte activation pieces per thread and half tile
+    constexpr int AP = BM * 8 / TS;              // 16-byte activation pieces per thread and half tile
+    constexpr int RPP = TS / 8;                  // activation rows that the set's threads stage in one pass
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];   // [KS][2][BM AROW] halves; then the sums
 
-    const int tid = threadIdx.x % kMmThreads, lane = tid & 63;
-    const int w = __builtin_amdgcn_readfirstlane((threadIdx.x >> 6) & 3), kg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8);
+    const int tid = threadIdx.x % TS, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane((threadIdx.x >> 6) % NW), kg = __builtin_amdgcn_readfirstlane(threadIdx.x / TS);
     const int hb = lane >> 5, l32 = lane & 31;
     const int n0 = blockIdx.x * TN, m0 = blockIdx.y * BM, b = blockIdx.z, wb = b / p.ratio;
     const int groups = p.n / 16, T = p.k / TK;
@@ -229,14 +234,14 @@ __global__ __launch_bounds__(kMmThreads * KS, KS == 1 ? 2 : 1) void q4_0_tiled_m
         w_slot[i] = grp * (uint32_t)T * 1152u + 16 * (l32 & 15) + 256 * hb;
         w_scale[i] = grp * (uint32_t)T * 1152u + 1024 + 8 * (l32 & 15);
     }
-    // activation piece j * 256 + tid of a half tile: row 32 j + tid / 8 of the workgroup's BM, features 8 pc .. 8 pc + 7 of
+    // activation piece j * TS + tid of a half tile: row RPP j + tid / 8 of the workgroup's BM, features 8 pc .. 8 pc + 7 of
     // the half (pc = tid % 8): features 8 pb .. 8 pb + 7 of its block pc / 4 (pb = pc % 4), which are halves pb / 2 of the
     // vectors g = 2 (pb % 2) and g + 1 of that block; vector 4 block + g of a row sits at 8 (4 block + g) halves
     const int a_row = tid >> 3, a_pc = tid & 7;
     uint32_t a_src[AP];   // bytes
 #pragma unroll
-    for (int j = 0; j < AP; j++) a_src[j] = (uint32_t)((m0 + 32 * j + a_row) * p.k + a_pc * 8) * 2;
-    const int a_dst = a_row * AROW + (4 * (a_pc >> 2) + 2 * (a_pc & 1)) * 8 + 4 * ((a_pc >> 1) & 1);   // piece j: + 32 j AROW
+    for (int j = 0; j < AP; j++) a_src[j] = (uint32_t)((m0 + RPP * j + a_row) * p.k + a_pc * 8) * 2;
+    const int a_dst = a_row * AROW + (4 * (a_pc >> 2) + 2 * (a_pc & 1)) * 8 + 4 * ((a_pc >> 1) & 1);   // piece j: + RPP j AROW
 
     struct Weights { u32x4 c[NI][2]; u32x2 s[NI]; };   // a tile's slots g = hb, 2 + hb and scales, for each 32 rows of the wave
     u32x4 apre[PA][AP];
@@ -255,8 +260,8 @@ __global__ __launch_bounds__(kMmThreads * KS, KS == 1 ? 2 : 1) void q4_0_tiled_m
     auto stage_a = [&](int set, int buf) {
 #pragma unroll
         for (int j = 0; j < AP; j++) {
-            *reinterpret_cast<u32x2 *>(&lds_a[buf * BM * AROW + a_dst + 32 * j * AROW]) = u32x2{apre[set][j].x, apre[set][j].y};
-            *reinterpret_cast<u32x2 *>(&lds_a[buf * BM * AROW + a_dst + 32 * j * AROW + 8]) = u32x2{apre[set][j].z, apre[set][j].w};   // vector g + 1
+            *reinterpret_cast<u32x2 *>(&lds_a[buf * BM * AROW + a_dst + RPP * j * AROW]) = u32x2{apre[set][j].x, apre[set][j].y};
+            *reinterpret_cast<u32x2 *>(&lds_a[buf * BM * AROW + a_dst + RPP * j * AROW + 8]) = u32x2{apre[set][j].z, apre[set][j].w};   // vector g + 1
         }
     };
 
@@ -331,7 +336,7 @@ __global__ __launch_bounds__(kMmThreads * KS, KS == 1 ? 2 : 1) void q4_0_tiled_m
         for (int half = KS / 2; half >= 1; half >>= 1) {
             __syncthreads();
             if (kg >= half && kg < 2 * half) {
-                float *dst = red + ((kg - half) * 4 + w) * PER_WAVE + lane;
+                float *dst = red + ((kg - half) * NW + w) * PER_WAVE + lane;
 #pragma unroll
                 for (int i = 0; i < NI; i++)
 #pragma unroll
@@ -341,7 +346,7 @@ __global__ __launch_bounds__(kMmThreads * KS, KS == 1 ? 2 : 1) void q4_0_tiled_m
             }
             __syncthreads();
             if (kg < half) {
-                const float *src = red + (kg * 4 + w) * PER_WAVE + lane;
+                const float *src = red + (kg * NW + w) * PER_WAVE + lane;
 #pragma unroll
                 for (int i = 0; i < NI; i++)
 #pragma unroll
@@ -412,31 +417,46 @@ int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, i
         if (forced_bm == 64 || forced_bm == 128) bm = forced_bm;
         if (forced_ni == 1 || forced_ni == 2) ni = forced_ni;
         if (bm == 128) ni = 2;
-        const int64_t tx = (n + 128 * ni - 1) / (128 * ni), ty = (m + bm - 1) / bm;
+        const int64_t ty = (m + bm - 1) / bm;
         if (ty > 65535) return 2;
+        // ... and when that smallest tile still leaves compute units idle, sets of 2 waves or 1 (64 or 32 rows of the
+        // weights per workgroup)
+        static const int forced_nw = getenv("TROCM_Q4_MATMUL_NW") ? atoi(getenv("TROCM_Q4_MATMUL_NW")) : 0;
+        int nw = 4;
+        if (bm == 64 && ni == 1) {
+            while (nw > 1 && ((n + 32 * nw - 1) / (32 * nw)) * ty * act_batch * 4 < cus * 3) nw /= 2;
+            if (forced_nw == 1 || forced_nw == 2 || forced_nw == 4) nw = forced_nw;
+        }
+        const int64_t txw = (n + 32 * ni * nw - 1) / (32 * ni * nw);
         int ks = 1;
         if (bm == 64) {
-            const int64_t wgs = tx * ty * act_batch, tiles = k / TK;
-            if (ni == 1 && wgs <= cus && tiles % 4 == 0) ks = 4;            // 16 waves of 128 registers: one workgroup per compute unit
-            else if (wgs <= 2 * cus && tiles % 2 == 0) ks = 2;
+            const int64_t wgs = txw * ty * act_batch, tiles = k / TK;
+            if (ni == 1 && wgs * nw <= cus * 4 && tiles % 4 == 0) ks = 4;            // (16 waves of 128 registers fill a compute unit)
+            else if (wgs * nw <= 2 * cus * 4 && tiles % 2 == 0) ks = 2;
         }
         if (forced_ks == 1 || ((forced_ks == 2 || (forced_ks == 4 && ni == 1)) && bm == 64 && (k / TK) % forced_ks == 0)) ks = forced_ks;
-        const dim3 tgrid((unsigned)tx, (unsigned)ty, (unsigned)act_batch);
+        const dim3 tgrid((unsigned)txw, (unsigned)ty, (unsigned)act_batch);
         const size_t lds_act = (size_t)ks * 2 * bm * AROW * sizeof(_Float16);
-        const size_t lds_red = ks > 1 ? (size_t)(ks / 2) * 4 * ni * (bm / 32) * 16 * 64 * sizeof(float) : 0;
+        const size_t lds_red = ks > 1 ? (size_t)(ks / 2) * nw * ni * (bm / 32) * 16 * 64 * sizeof(float) : 0;
         const size_t lds = lds_act > lds_red ? lds_act : lds_red;
         auto launch = [&](auto kernel) -> int {
             if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
                 (void)hipGetLastError();
                 return fail("q4_0_matmul (tiled weights): %zu bytes of LDS were refused", lds);
             }
-            hipLaunchKernelGGL(kernel, tgrid, dim3(kMmThreads * ks), lds, s, p);
+            hipLaunchKernelGGL(kernel, tgrid, dim3(64 * nw * ks), lds, s, p);
             return 0;
         };
+        auto launch_small = [&](auto nw_tag) -> int {   // 64 activation rows, 32 rows of the weights per wave
+            constexpr int NWc = decltype(nw_tag)::value;
+            return ks == 4 ? launch(q4_0_tiled_matmul_kernel<64, 1, 4, NWc>) : ks == 2 ? launch(q4_0_tiled_matmul_kernel<64, 1, 2, NWc>)
+                                                                                       : launch(q4_0_tiled_matmul_kernel<64, 1, 1, NWc>);
+        };
         int rc;
-        if (bm == 128 && ni == 2) rc = launch(q4_0_tiled_matmul_kernel<128, 2, 1>);
-        else if (ni == 2) rc = ks == 2 ? launch(q4_0_tiled_matmul_kernel<64, 2, 2>) : launch(q4_0_tiled_matmul_kernel<64, 2, 1>);
-        else rc = ks == 4 ? launch(q4_0_tiled_matmul_kernel<64, 1, 4>) : ks == 2 ? launch(q4_0_tiled_matmul_kernel<64, 1, 2>) : launch(q4_0_tiled_matmul_kernel<64, 1, 1>);
+        if (bm == 128) rc = launch(q4_0_tiled_matmul_kernel<128, 2, 1, 4>);
+        else if (ni == 2) rc = ks == 2 ? launch(q4_0_tiled_matmul_kernel<64, 2, 2, 4>) : launch(q4_0_tiled_matmul_kernel<64, 2, 1, 4>);
+        else rc = nw == 4 ? launch_small(std::integral_constant<int, 4>()) : nw == 2 ? launch_small(std::integral_constant<int, 2>())
+                                                                                      : launch_small(std::integral_constant<int, 1>());
         if (rc) return rc;
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return fail("q4_0_matmul (tiled weights) launch failed: %s", hipGetErrorString(e));
