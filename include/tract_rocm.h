@@ -210,10 +210,9 @@ int trocm_block_simulate_precision_loss(int format, const void *src, void *dst, 
  * [act_batch, m, k], output [act_batch, m, n] in the activations' type; act_batch must be a
  * multiple of the weights' batch (:488).  Result: the product with the dequantised weights, the
  * definition the reference's own test holds its kernel to (mod.rs:864-890).  More than 8 rows of f16
- * activations with k a multiple of 64 (weights held as tiles: more than 24 rows; up to there they run as
- * groups of 16 rows, one pass over the weights each) take the matrix-matrix arm (:607-610) on the matrix
- * cores, with the weights dequantised to f16 as dequant_block_f16 stores them (q4_0.rs:82-95); any other
- * m > 8 runs as groups of 8 rows. */
+ * activations with k a multiple of 64 (weights held as tiles: more than 16 rows) take the matrix-matrix
+ * arm (:607-610) on the matrix cores, with the weights dequantised to f16 as dequant_block_f16 stores them
+ * (q4_0.rs:82-95); any other m > 8 runs as groups of 8 rows. */
 typedef struct trocm_q4_weights trocm_q4_weights;
 
 /* Device copy of `batch * n` rows of k/32 canonical 18-byte blocks (device pointer, row-major, no

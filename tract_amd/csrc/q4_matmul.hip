@@ -405,8 +405,10 @@ int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, i
         static const int forced_ni = getenv("TROCM_Q4_MATMUL_NI") ? atoi(getenv("TROCM_Q4_MATMUL_NI")) : 0;
         static const int forced_ks = getenv("TROCM_Q4_MATMUL_KS") ? atoi(getenv("TROCM_Q4_MATMUL_KS")) : 0;
         const int64_t cus = num_compute_units();
-        const int shapes[3][2] = {{128, 2}, {64, 2}, {64, 1}};
-        int bm = 64, ni = 1;
+        // (up to 32 activation rows: 256 x 32, 128 x 32 -- half the matrix instructions of a tile of 64 rows)
+        const int shapes64[3][2] = {{128, 2}, {64, 2}, {64, 1}}, shapes32[3][2] = {{32, 2}, {32, 2}, {32, 1}};
+        const int (*shapes)[2] = m <= 32 ? shapes32 : shapes64;
+        int bm = shapes[2][0], ni = 1;
         for (int c = 0; c < 3; c++) {
             const int64_t wgs = ((n + 128 * shapes[c][1] - 1) / (128 * shapes[c][1])) * ((m + shapes[c][0] - 1) / shapes[c][0]) * act_batch;
             if (wgs * 4 >= cus * 3) {
@@ -414,7 +416,7 @@ int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, i
                 break;
             }
         }
-        if (forced_bm == 64 || forced_bm == 128) bm = forced_bm;
+        if (forced_bm == 32 || forced_bm == 64 || forced_bm == 128) bm = forced_bm;
         if (forced_ni == 1 || forced_ni == 2) ni = forced_ni;
         if (bm == 128) ni = 2;
         const int64_t ty = (m + bm - 1) / bm;
@@ -423,18 +425,18 @@ int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, i
         // weights per workgroup)
         static const int forced_nw = getenv("TROCM_Q4_MATMUL_NW") ? atoi(getenv("TROCM_Q4_MATMUL_NW")) : 0;
         int nw = 4;
-        if (bm == 64 && ni == 1) {
+        if (bm <= 64 && ni == 1) {
             while (nw > 1 && ((n + 32 * nw - 1) / (32 * nw)) * ty * act_batch * 4 < cus * 3) nw /= 2;
             if (forced_nw == 1 || forced_nw == 2 || forced_nw == 4) nw = forced_nw;
         }
         const int64_t txw = (n + 32 * ni * nw - 1) / (32 * ni * nw);
         int ks = 1;
-        if (bm == 64) {
+        if (bm <= 64) {
             const int64_t wgs = txw * ty * act_batch, tiles = k / TK;
             if (ni == 1 && wgs * nw <= cus * 4 && tiles % 4 == 0) ks = 4;            // (16 waves of 128 registers fill a compute unit)
             else if (wgs * nw <= 2 * cus * 4 && tiles % 2 == 0) ks = 2;
         }
-        if (forced_ks == 1 || ((forced_ks == 2 || (forced_ks == 4 && ni == 1)) && bm == 64 && (k / TK) % forced_ks == 0)) ks = forced_ks;
+        if (forced_ks == 1 || ((forced_ks == 2 || (forced_ks == 4 && ni == 1)) && bm <= 64 && (k / TK) % forced_ks == 0)) ks = forced_ks;
         const dim3 tgrid((unsigned)txw, (unsigned)ty, (unsigned)act_batch);
         const size_t lds_act = (size_t)ks * 2 * bm * AROW * sizeof(_Float16);
         const size_t lds_red = ks > 1 ? (size_t)(ks / 2) * nw * ni * (bm / 32) * 16 * 64 * sizeof(float) : 0;
@@ -447,16 +449,21 @@ int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, i
             hipLaunchKernelGGL(kernel, tgrid, dim3(64 * nw * ks), lds, s, p);
             return 0;
         };
-        auto launch_small = [&](auto nw_tag) -> int {   // 64 activation rows, 32 rows of the weights per wave
-            constexpr int NWc = decltype(nw_tag)::value;
-            return ks == 4 ? launch(q4_0_tiled_matmul_kernel<64, 1, 4, NWc>) : ks == 2 ? launch(q4_0_tiled_matmul_kernel<64, 1, 2, NWc>)
-                                                                                       : launch(q4_0_tiled_matmul_kernel<64, 1, 1, NWc>);
+        auto launch_small = [&](auto bm_tag, auto nw_tag) -> int {   // 64 or 32 activation rows, 32 rows of the weights per wave
+            constexpr int BMc = decltype(bm_tag)::value, NWc = decltype(nw_tag)::value;
+            return ks == 4 ? launch(q4_0_tiled_matmul_kernel<BMc, 1, 4, NWc>) : ks == 2 ? launch(q4_0_tiled_matmul_kernel<BMc, 1, 2, NWc>)
+                                                                                        : launch(q4_0_tiled_matmul_kernel<BMc, 1, 1, NWc>);
+        };
+        auto launch_bm = [&](auto bm_tag) -> int {
+            constexpr int BMc = decltype(bm_tag)::value;
+            if (ni == 2) return ks == 2 ? launch(q4_0_tiled_matmul_kernel<BMc, 2, 2, 4>) : launch(q4_0_tiled_matmul_kernel<BMc, 2, 1, 4>);
+            return nw == 4 ? launch_small(bm_tag, std::integral_constant<int, 4>()) : nw == 2 ? launch_small(bm_tag, std::integral_constant<int, 2>())
+                                                                                               : launch_small(bm_tag, std::integral_constant<int, 1>());
         };
         int rc;
         if (bm == 128) rc = launch(q4_0_tiled_matmul_kernel<128, 2, 1, 4>);
-        else if (ni == 2) rc = ks == 2 ? launch(q4_0_tiled_matmul_kernel<64, 2, 2, 4>) : launch(q4_0_tiled_matmul_kernel<64, 2, 1, 4>);
-        else rc = nw == 4 ? launch_small(std::integral_constant<int, 4>()) : nw == 2 ? launch_small(std::integral_constant<int, 2>())
-                                                                                      : launch_small(std::integral_constant<int, 1>());
+        else if (bm == 64) rc = launch_bm(std::integral_constant<int, 64>());
+        else rc = launch_bm(std::integral_constant<int, 32>());
         if (rc) return rc;
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return fail("q4_0_matmul (tiled weights) launch failed: %s", hipGetErrorString(e));

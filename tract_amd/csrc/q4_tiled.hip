@@ -520,17 +520,17 @@ int launch_q4_0_tiled_export(const void *tiles, void *blocks, int64_t rows, int6
     return 0;
 }
 
-// Tiled weights x activations for any m: f16 rows in groups of up to 16 (more than 24 rows go to the matrix-matrix
+// Tiled weights x activations for any m: f16 rows in groups of up to 16 (more than 16 rows go to the matrix-matrix
 // kernel first, which reads the same tiles, when it takes the call), f32 rows in groups of up to 8.
 int launch_q4_0_tiled_matvec(const void *tiles, int64_t w_batch, int64_t n, int64_t k, const void *act, int act_dtype,
                              int64_t act_batch, int64_t m, void *out, hipStream_t s) {
     if (n >= (1ll << 30) || k >= (1ll << 30) || act_batch > 65535) return fail("q4_0_matvec: shape too large");
     // (a row group's records are addressed through one buffer descriptor: 32-bit offsets)
     if ((k / 128) * kTile >= (1ll << 31)) return fail("q4_0_matvec: rows of %lld features are too long for the tiled layout", (long long)k);
-    // Up to 24 f16 rows go in groups of 16 through the kernel above, more to the matrix-matrix kernel (us, two passes
-    // here | one launch there: 24 rows of 14336 x 4096 21.3 | 16.3, of 4096 x 4096 12.9 | 12.6, of 4096 x 14336 35.5 | 40.0;
-    // 17 rows 20.5 | 15.9, 12.0 | 12.6, 29.0 | 38.7; 32 rows 23.2 | 16.2, 14.8 | 12.6, 41.8 | 40.2).
-    static const int matmul_from = env_int("TROCM_Q4_MATMUL_FROM", 25);
+    // Up to 16 f16 rows take one pass through the kernel above, more go to the matrix-matrix kernel (us, two passes here |
+    // one launch there with 32 activation rows per workgroup: 24 rows of 14336 x 4096 21.3 | 13.5, of 4096 x 4096
+    // 12.9 | 10.0, of 1024 x 4096 12.4 | 8.9, of 4096 x 14336 35.5 | 32.3; 17 rows of the last 29.0 | 32.3).
+    static const int matmul_from = env_int("TROCM_Q4_MATMUL_FROM", 17);
     if (act_dtype == TROCM_F16 && m >= matmul_from && m > 16) {
         const int rc = launch_q4_0_matmul(tiles, nullptr, w_batch, n, k, act, act_dtype, act_batch, m, out, s, 1);
         if (rc != 2) return rc;
