@@ -823,8 +823,8 @@ def run_ops(ta, args):
         us = time_calls(ta, one_mv8, 200)
         by8 = n_ * (k_ // 32) * 18 + 8 * 2 * k_ + 8 * 2 * n_
         res[f"q4_0_matvec_f16_m8_n{n_}_k{k_}"] = {"us": round(us, 2), "gbs": round(by8 / us / 1e3, 1), "bytes": by8}
-        # the same weights x the rows of a prefill chunk (128, 512, 2048): the matrix-matrix arm, on the matrix cores
-        for m_ in (128, 512, 2048):
+        # the same weights x the rows of a batch-32 step and of a prefill chunk (128, 512, 2048): the matrix-matrix arm
+        for m_ in (32, 128, 512, 2048):
             xm = ta.DeviceTensor.from_numpy(rng.standard_normal((1, m_, k_)).astype(np.float16))
             om = ta.DeviceTensor((1, m_, n_), np.float16)
 
