@@ -71,7 +71,7 @@ TILED_SHAPES = [
     (1, 1, 200, 4096, 512), (1, 1, 200, 4096, 768), (1, 1, 200, 4096, 384),
     # ... 25..32 rows: tiles of 32 activation rows
     (1, 1, 30, 4096, 512), (1, 2, 32, 14336, 256), (1, 1, 26, 32768, 128), (1, 1, 28, 50000, 256), (1, 1, 28, 50000, 128),
-    (1, 1, 30, 14336, 512),
+    (1, 1, 30, 14336, 512), (1, 1, 30, 4096, 1024),   # (the last: k over 8 sets of one wave, as 130 x 2048 x 4096 above)
 ]
 
 

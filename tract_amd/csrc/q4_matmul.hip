@@ -190,7 +190,7 @@ __global__ __launch_bounds__(kMmThreads, 2) void q4_0_matmul_kernel(MatMulDev p)
 constexpr int TK = 128, HK = 64;   // features per tile of the weights and per staged half of it
 constexpr int AROW = HK + 8;                 // halves per activation row in LDS (the 16 rows of a 128-bit read pass in 16 distinct bank groups)
 
-// KS > 1: KS such sets of 4 waves share the workgroup's tile of C^T and split k between them (set kg takes tiles
+// KS > 1: KS (2, 4; 8 of one wave) such sets of waves share the workgroup's tile of C^T and split k between them (set kg takes tiles
 // kg T / KS .. of every row, in LDS buffers of its own), and their accumulators are added through LDS at the end: for
 // launches with so few workgroups that each compute unit would otherwise hold four waves that walk all of k alone.
 // NW: waves per set (4; 2 or 1 -- 64 or 32 rows of the weights per workgroup -- when even the smallest tile above leaves
@@ -433,10 +433,11 @@ int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, i
         int ks = 1;
         if (bm <= 64) {
             const int64_t wgs = txw * ty * act_batch, tiles = k / TK;
-            if (ni == 1 && wgs * nw <= cus * 4 && tiles % 4 == 0) ks = 4;            // (16 waves of 128 registers fill a compute unit)
+            if (ni == 1 && nw == 1 && wgs <= cus * 2 && tiles % 8 == 0) ks = 8;      // (sets of one wave: 8 of them, two such workgroups per compute unit)
+            else if (ni == 1 && wgs * nw <= cus * 4 && tiles % 4 == 0) ks = 4;       // (16 waves of 128 registers fill a compute unit)
             else if (wgs * nw <= 2 * cus * 4 && tiles % 2 == 0) ks = 2;
         }
-        if (forced_ks == 1 || ((forced_ks == 2 || (forced_ks == 4 && ni == 1)) && bm <= 64 && (k / TK) % forced_ks == 0)) ks = forced_ks;
+        if (forced_ks == 1 || ((forced_ks == 2 || ((forced_ks == 4 || (forced_ks == 8 && nw == 1)) && ni == 1)) && bm <= 64 && (k / TK) % forced_ks == 0)) ks = forced_ks;
         const dim3 tgrid((unsigned)txw, (unsigned)ty, (unsigned)act_batch);
         const size_t lds_act = (size_t)ks * 2 * bm * AROW * sizeof(_Float16);
         const size_t lds_red = ks > 1 ? (size_t)(ks / 2) * nw * ni * (bm / 32) * 16 * 64 * sizeof(float) : 0;
@@ -451,6 +452,8 @@ int launch_q4_0_matmul(const void *codes, const void *scales, int64_t w_batch, i
         };
         auto launch_small = [&](auto bm_tag, auto nw_tag) -> int {   // 64 or 32 activation rows, 32 rows of the weights per wave
             constexpr int BMc = decltype(bm_tag)::value, NWc = decltype(nw_tag)::value;
+            if constexpr (NWc == 1)
+                if (ks == 8) return launch(q4_0_tiled_matmul_kernel<BMc, 1, 8, 1>);
             return ks == 4 ? launch(q4_0_tiled_matmul_kernel<BMc, 1, 4, NWc>) : ks == 2 ? launch(q4_0_tiled_matmul_kernel<BMc, 1, 2, NWc>)
                                                                                         : launch(q4_0_tiled_matmul_kernel<BMc, 1, 1, NWc>);
         };
