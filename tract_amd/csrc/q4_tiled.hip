@@ -184,20 +184,29 @@ __global__ __launch_bounds__(64 * kW, ACT == kActF32Rows2 ? 2 : 4) void q4_0_til
     // each starts at another place of the chunk, so that at any moment the compute units ask different channels of the L2.
     constexpr int NP = CHUNKED ? 4 : 8;   // (registers)
     constexpr int PPT = F32 ? 32 : 16;    // 16-byte pieces of the source per tile and row: 4 f32 or 8 f16 features each
+    // PRIVATE (every wave has tiles of its own, activations staged whole): a wave stages exactly the tiles it will read,
+    // all rows of them, and nobody waits for anybody -- no barrier between the staging and the first tile.
+    constexpr bool PRIVATE = KS == kW && !CHUNKED;
     auto stage = [&](int c, auto &&after_last_loads) {
-        const int ntl = min(p.cq, p.T - c * p.cq), per_row = ntl * PPT, total = p.m * per_row;
+        const int ntl = PRIVATE ? ni : min(p.cq, p.T - c * p.cq), per_row = ntl * PPT, total = p.m * per_row;
+        constexpr int NTH = PRIVATE ? 64 : kThreads;   // threads that share the pieces
+        if (total == 0) {
+            after_last_loads();
+            return;
+        }
         const int start = (int)(((int64_t)blockIdx.x * 37 % 64) * total / 64);
         const uint32_t inv_per_row = 0xFFFFFFFFu / (uint32_t)per_row + 1;   // v / per_row = high word of v * this (v * per_row < 2^32)
-        for (int base = 0; base < total; base += kThreads * NP) {   // (uniform: every thread runs every pass)
-            const int v0 = base + tid;
+        for (int base = 0; base < total; base += NTH * NP) {   // (uniform: every thread runs every pass)
+            const int v0 = base + (PRIVATE ? lane : tid);
             u32x4 x[NP];
             // piece v: row i, tile tl of the chunk, piece pp of the tile (computed twice rather than kept)
             auto where = [&](int u, int &i, int &tl, int &pp) {
-                int v = min(v0 + u * kThreads, total - 1) + start;      // (past the end: the last piece again, not stored)
+                int v = min(v0 + u * NTH, total - 1) + start;      // (past the end: the last piece again, not stored)
                 if (v >= total) v -= total;
                 i = (int)__umulhi((uint32_t)v, inv_per_row);
                 const int rem = v - i * per_row;
                 tl = rem / PPT, pp = rem % PPT;
+                if constexpr (PRIVATE) tl = q + KS * tl;                 // (the wave's tl-th tile)
             };
 #pragma unroll
             for (int u = 0; u < NP; u++) {
@@ -205,10 +214,10 @@ __global__ __launch_bounds__(64 * kW, ACT == kActF32Rows2 ? 2 : 4) void q4_0_til
                 where(u, i, tl, pp);
                 x[u] = *reinterpret_cast<const u32x4 *>(act + (int64_t)i * p.k + (int64_t)(c * p.cq + tl) * 128 + pp * (F32 ? 4 : 8));
             }
-            if (base + kThreads * NP >= total) after_last_loads();
+            if (base + NTH * NP >= total) after_last_loads();
 #pragma unroll
             for (int u = 0; u < NP; u++) {
-                if (v0 + u * kThreads < total) {
+                if (v0 + u * NTH < total) {
                     int i, tl, pp;
                     where(u, i, tl, pp);
                     if constexpr (F32) {
@@ -256,7 +265,7 @@ __global__ __launch_bounds__(64 * kW, ACT == kActF32Rows2 ? 2 : 4) void q4_0_til
     };
     if constexpr (!CHUNKED) {
         stage(0, rest_of_ring);
-        __syncthreads();
+        if constexpr (!PRIVATE) __syncthreads();
     } else {
         rest_of_ring();
     }
