@@ -498,6 +498,25 @@ __device__ __forceinline__ void store_codes8(uint8_t *row, int sub, const uint32
     }
 }
 
+// Eight consecutive channels as they lie in memory (the conversion to f32 happens when the row is used).
+struct RawF32x8 { float4 a, b; };
+__device__ __forceinline__ RawF32x8 ld8raw(const float *p) { return RawF32x8{reinterpret_cast<const float4 *>(p)[0], reinterpret_cast<const float4 *>(p)[1]}; }
+__device__ __forceinline__ uint4 ld8raw(const __half *p) { return *reinterpret_cast<const uint4 *>(p); }
+__device__ __forceinline__ F8 cvt8(const RawF32x8 &r) { return F8{{r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w}}; }
+__device__ __forceinline__ F8 cvt8(const uint4 &w) {
+    const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+    F8 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        r.v[2 * i] = __half2float(__ushort_as_half((unsigned short)(u[i] & 0xffffu)));
+        r.v[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(u[i] >> 16)));
+    }
+    return r;
+}
+
+__device__ __forceinline__ void settle(RawF32x8 &r) { asm volatile("" : "+v"(r.a.x), "+v"(r.a.y), "+v"(r.a.z), "+v"(r.a.w), "+v"(r.b.x), "+v"(r.b.y), "+v"(r.b.z), "+v"(r.b.w)); }
+__device__ __forceinline__ void settle(uint4 &w) { asm volatile("" : "+v"(w.x), "+v"(w.y), "+v"(w.z), "+v"(w.w)); }
+
 // The three chunk passes of the running Key store for head sizes 64 / 128 / 256 / 512 and 16-byte aligned sources: a lane
 // owns 8 consecutive channels of one chunk and walks the chunk's tokens with 128-bit loads; LPR = D / 8 lanes cover a row,
 // 256 / LPR chunks share a workgroup.  PASS 1: first minimal value per chunk and channel into `a`; PASS 2: largest scale
@@ -514,13 +533,44 @@ __global__ void __launch_bounds__(256) kivi_run_chunk_vec_kernel(const SrcT *__r
     const int64_t at = ((int64_t)bh * n_chunks + k) * D + sub * 8;
     const int t0 = k * kRunChunk, t1 = min(n, t0 + kRunChunk);
     const SrcT *row = src + ((int64_t)bh * S + t0) * D + sub * 8;
+    // PASS 3 takes the chunk's rows in groups of 8.  Loads and stores share a counter and are not ordered against each
+    // other, so a wait for a row with a store outstanding is a wait for all memory traffic: with the loads of just the
+    // tokens at hand and a store per token, every token paid a whole trip to memory (69 us).  Now the next group is
+    // requested first, this group's codes are formed into registers, the next group's rows are waited for while only
+    // loads (8 tokens old) are outstanding, and then this group's codes are stored: they have the next group's
+    // arithmetic to complete in.  (The passes that only load count their loads and are better off without the groups:
+    // 31 against 35 us.)  Rows past the chunk's end: its last row again.
+    constexpr int G = 8;
+    uint32_t cw0[G], cw1[G];   // PASS 3: the group's codes, 8 per token
+    auto for_each_token = [&](auto &&body) {
+        if constexpr (PASS != 3) {
+#pragma unroll 4
+            for (int t = t0; t < t1; t++) body(t, ld8(row + (int64_t)(t - t0) * D), 0);
+            return;
+        }
+        auto fetch = [&](int t) { return ld8raw(row + (int64_t)(min(t, t1 - 1) - t0) * D); };
+        decltype(fetch(0)) cur[G], nxt[G];
+#pragma unroll
+        for (int u = 0; u < G; u++) cur[u] = fetch(t0 + u);
+        for (int tg = t0; tg < t1; tg += G) {
+#pragma unroll
+            for (int u = 0; u < G; u++) nxt[u] = fetch(tg + G + u);
+#pragma unroll
+            for (int u = 0; u < G; u++)
+                if (tg + u < t1) body(tg + u, cvt8(cur[u]), u);
+#pragma unroll
+            for (int u = 0; u < G; u++) settle(nxt[u]), cur[u] = nxt[u];
+#pragma unroll
+            for (int u = 0; u < G; u++)
+                if (tg + u < t1)
+                    *reinterpret_cast<uint2 *>(codes + ((int64_t)bh * cap_rows + row0 + tg + u) * D + sub * 8) = make_uint2(cw0[u], cw1[u]);
+        }
+    };
     if constexpr (PASS == 12) {   // one pass for both scans (kivi_run_scan_both_kernel): first minimum, maximum, widest own range
         F8 mn, mx, own;
 #pragma unroll
         for (int e = 0; e < 8; e++) mn.v[e] = INFINITY, mx.v[e] = -INFINITY, own.v[e] = 0.0f;
-#pragma unroll 4
-        for (int t = t0; t < t1; t++, row += D) {
-            const F8 x = ld8(row);
+        for_each_token([&](int, const F8 &x, int) {
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 const float val = x.v[e];
@@ -529,7 +579,7 @@ __global__ void __launch_bounds__(256) kivi_run_chunk_vec_kernel(const SrcT *__r
                 const float range = __fsub_rn(val, mn.v[e]);
                 own.v[e] = range > own.v[e] ? range : own.v[e];   // (a NaN range is never wider)
             }
-        }
+        });
         st8(a + at, mn), st8(b + at, mx), st8(c3 + at, own);
         return;
     }
@@ -560,9 +610,7 @@ __global__ void __launch_bounds__(256) kivi_run_chunk_vec_kernel(const SrcT *__r
         widest[e] = PASS == 3 ? sc.v[e] * 254.9f : 0.0f;
         inv.v[e] = PASS == 3 ? affine_inv(sc.v[e]) : 0.0f;
     }
-#pragma unroll 4
-    for (int t = t0; t < t1; t++, row += D) {
-        const F8 x = ld8(row);
+    for_each_token([&](int, const F8 &x, int u) {
         bool wider = false;
         float range[8];
 #pragma unroll
@@ -590,9 +638,10 @@ __global__ void __launch_bounds__(256) kivi_run_chunk_vec_kernel(const SrcT *__r
             }
             uint32_t code[8];
             affine_codes8(x.v, lo.v, sc.v, inv.v, 255.0f, code);
-            store_codes8<8>(codes + ((int64_t)bh * cap_rows + row0 + t) * D, sub, code);
+            cw0[u] = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
+            cw1[u] = code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24);
         }
-    }
+    });
     if (PASS == 2) {
 #pragma unroll
         for (int e = 0; e < 8; e++) sc.v[e] = widest[e] > 0.0f ? __fdiv_rn(widest[e], 255.0f) : 0.0f;
