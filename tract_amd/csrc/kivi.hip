@@ -116,21 +116,23 @@ __device__ __forceinline__ int cvt_i32_rz_sat(float x) {   // truncates, saturat
     asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(x));
     return r;
 }
-template <typename Params>   // Params: float (one group for the 8 values) or float[8] (a group per value)
+// KNOWN: the caller keeps track of whether every inv is usable (non-zero) and passes it as `all_usable` (a walk whose
+// parameters change rarely: the 8 comparisons per token leave its loop).
+template <bool KNOWN = false, typename Params>   // Params: float (one group for the 8 values) or float[8] (a group per value)
 __device__ __forceinline__ void affine_codes8(const float (&x)[8], const Params &lo, const Params &scale, const Params &inv, float lv,
-                                              uint32_t (&code)[8]) {
+                                              uint32_t (&code)[8], bool all_usable = true) {
     auto at = [](const Params &p, int e) -> float {
         if constexpr (std::is_same<Params, float>::value) return p;
         else return p[e];
     };
     float near = 1.0f;   // the smallest distance of a fraction from one half (fminf drops a NaN)
-    bool usable = true;
+    bool usable = all_usable;
 #pragma unroll
     for (int e = 0; e < 8; e++) {
         const float q0 = __fmul_rn(__fsub_rn(x[e], at(lo, e)), at(inv, e));
         near = fminf(near, fabsf(__fsub_rn(__builtin_amdgcn_fractf(q0), 0.5f)));
         code[e] = (uint32_t)max(0, min((int)lv, cvt_i32_rz_sat(__fadd_rn(q0, 0.49999997f))));
-        usable = usable && at(inv, e) != 0.0f;
+        if constexpr (!KNOWN) usable = usable && at(inv, e) != 0.0f;
     }
     if (!(usable && near >= 0x1p-13f)) {
 #pragma unroll
@@ -605,10 +607,12 @@ __global__ void __launch_bounds__(256) kivi_run_chunk_vec_kernel(const SrcT *__r
     // take the reciprocal of the scale with its re-check (affine_codes8), refreshed when the scale moves.
     float widest[8];
     F8 inv;
+    bool inv_usable = true;   // every inv is non-zero (kept up to date where a scale moves)
 #pragma unroll
     for (int e = 0; e < 8; e++) {
         widest[e] = PASS == 3 ? sc.v[e] * 254.9f : 0.0f;
         inv.v[e] = PASS == 3 ? affine_inv(sc.v[e]) : 0.0f;
+        inv_usable = inv_usable && inv.v[e] != 0.0f;
     }
     for_each_token([&](int, const F8 &x, int u) {
         bool wider = false;
@@ -635,9 +639,12 @@ __global__ void __launch_bounds__(256) kivi_run_chunk_vec_kernel(const SrcT *__r
                             inv.v[e] = affine_inv(ns);
                         }
                     }
+                inv_usable = true;
+#pragma unroll
+                for (int e = 0; e < 8; e++) inv_usable = inv_usable && inv.v[e] != 0.0f;
             }
             uint32_t code[8];
-            affine_codes8(x.v, lo.v, sc.v, inv.v, 255.0f, code);
+            affine_codes8<true>(x.v, lo.v, sc.v, inv.v, 255.0f, code, inv_usable);
             cw0[u] = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
             cw1[u] = code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24);
         }
