@@ -140,6 +140,37 @@ __device__ __forceinline__ void affine_codes8(const float (&x)[8], const Params 
     }
 }
 
+// The same for 8-bit codes, as the two words a row stores for the 8 values: v_cvt_pk_u8_f32 rounds to the nearest integer
+// (ties to even), saturates to [0, 255], turns a NaN into 0 and puts the byte in its place -- the reference's
+// round-half-away and clamp wherever the fraction is not one half, which is exactly what the re-check excludes -- so
+// the product needs neither the add and truncation nor the clamp nor the shifts that pack the bytes.
+template <bool KNOWN = false, typename Params>
+__device__ __forceinline__ void affine_words8_u8(const float (&x)[8], const Params &lo, const Params &scale, const Params &inv,
+                                                 uint32_t &w0, uint32_t &w1, bool all_usable = true) {
+    auto at = [](const Params &p, int e) -> float {
+        if constexpr (std::is_same<Params, float>::value) return p;
+        else return p[e];
+    };
+    float near = 1.0f;
+    bool usable = all_usable;
+    w0 = 0, w1 = 0;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const float q0 = __fmul_rn(__fsub_rn(x[e], at(lo, e)), at(inv, e));
+        near = fminf(near, fabsf(__fsub_rn(__builtin_amdgcn_fractf(q0), 0.5f)));
+        if (e < 4) w0 = __builtin_amdgcn_cvt_pk_u8_f32(q0, e, w0);
+        else w1 = __builtin_amdgcn_cvt_pk_u8_f32(q0, e - 4, w1);
+        if constexpr (!KNOWN) usable = usable && at(inv, e) != 0.0f;
+    }
+    if (!(usable && near >= 0x1p-13f)) {
+        uint32_t code[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) code[e] = affine_code(x[e], at(lo, e), at(scale, e), 255.0f);
+        w0 = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
+        w1 = code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24);
+    }
+}
+
 // dst[bh][dst_t0 + i][c] = (f32) src[bh][src_t0 + i][c], i < n: sink tokens and the partial key block.
 template <typename SrcT>
 __global__ void kivi_rows_to_f32_kernel(const SrcT *__restrict__ src, int64_t S, int64_t src_t0, float *__restrict__ dst,
@@ -643,10 +674,7 @@ __global__ void __launch_bounds__(256) kivi_run_chunk_vec_kernel(const SrcT *__r
 #pragma unroll
                 for (int e = 0; e < 8; e++) inv_usable = inv_usable && inv.v[e] != 0.0f;
             }
-            uint32_t code[8];
-            affine_codes8<true>(x.v, lo.v, sc.v, inv.v, 255.0f, code, inv_usable);
-            cw0[u] = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
-            cw1[u] = code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24);
+            affine_words8_u8<true>(x.v, lo.v, sc.v, inv.v, cw0[u], cw1[u], inv_usable);
         }
     });
     if (PASS == 2) {
@@ -676,9 +704,16 @@ __global__ void __launch_bounds__(256) kivi_quant_tokens_vec_kernel(const SrcT *
     }
     group_min_max<LPR>(lo, hi);
     const float scale = affine_scale(lo, hi, lv), inv = affine_inv(scale);
-    uint32_t code[8];
-    affine_codes8(x.v, lo, scale, inv, lv, code);
-    store_codes8<BITS>(codes + ((int64_t)bh * cap_rows + row0 + i) * RB, sub, code);
+    uint8_t *out_row = codes + ((int64_t)bh * cap_rows + row0 + i) * RB;
+    if constexpr (BITS == 8) {
+        uint32_t w0, w1;
+        affine_words8_u8(x.v, lo, scale, inv, w0, w1);
+        *reinterpret_cast<uint2 *>(out_row + sub * 8) = make_uint2(w0, w1);
+    } else {
+        uint32_t code[8];
+        affine_codes8(x.v, lo, scale, inv, lv, code);
+        store_codes8<BITS>(out_row, sub, code);
+    }
     if (sub == 0) {
         lo_out[(int64_t)bh * cap_rows + row0 + i] = lo;
         scale_out[(int64_t)bh * cap_rows + row0 + i] = scale;
@@ -721,9 +756,9 @@ __global__ void __launch_bounds__(128) kivi_step_push_kernel(const SrcT *__restr
         }
         group_min_max<16>(lo, hi);
         const float scale = affine_scale(lo, hi, 255.0f), inv = affine_inv(scale);
-        uint32_t code[8];
-        affine_codes8(x.v, lo, scale, inv, 255.0f, code);
-        store_codes8<8>(v_codes + ((int64_t)bh * v_cap_rows + v_row0) * D, sub, code);
+        uint32_t w0, w1;
+        affine_words8_u8(x.v, lo, scale, inv, w0, w1);
+        *reinterpret_cast<uint2 *>(v_codes + ((int64_t)bh * v_cap_rows + v_row0) * D + sub * 8) = make_uint2(w0, w1);
         if (sub == 0) {
             v_lo_out[(int64_t)bh * v_cap_rows + v_row0] = lo;
             v_scale_out[(int64_t)bh * v_cap_rows + v_row0] = scale;
@@ -789,9 +824,15 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_vec_kernel(const Src
 #pragma unroll 4
     for (int r = g; r < kKeyBlock; r += G) {
         const F8 x = r < n_old ? ld8(res + (int64_t)r * D) : ld8(rows + (int64_t)r * D);
-        uint32_t code[8];
-        affine_codes8(x.v, lo, scale, inv, lv, code);
-        store_codes8<BITS>(out + (int64_t)r * RB, sub, code);
+        if constexpr (BITS == 8) {
+            uint32_t w0, w1;
+            affine_words8_u8(x.v, lo, scale, inv, w0, w1);
+            *reinterpret_cast<uint2 *>(out + (int64_t)r * RB + sub * 8) = make_uint2(w0, w1);
+        } else {
+            uint32_t code[8];
+            affine_codes8(x.v, lo, scale, inv, lv, code);
+            store_codes8<BITS>(out + (int64_t)r * RB, sub, code);
+        }
     }
 }
 
