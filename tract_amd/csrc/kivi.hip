@@ -788,9 +788,15 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_vec_kernel(const Src
         lo[e] = INFINITY;
         hi[e] = -INFINITY;
     }
-#pragma unroll 4
-    for (int r = g; r < kKeyBlock; r += G) {
+    // (head sizes up to 128: a lane group's 4 or 8 rows stay in registers for the second pass)
+    constexpr int RPG = kKeyBlock / G;          // rows per lane group
+    constexpr bool KEEP = RPG <= 8;
+    F8 keep[KEEP ? RPG : 1];
+#pragma unroll (KEEP ? RPG : 4)
+    for (int it = 0; it < RPG; it++) {   // row r = g + it G
+        const int r = g + it * G;
         const F8 x = r < n_old ? ld8(res + (int64_t)r * D) : ld8(rows + (int64_t)r * D);
+        if constexpr (KEEP) keep[it] = x;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             lo[e] = fminf(lo[e], quiet(x.v[e]));
@@ -821,9 +827,12 @@ __global__ void __launch_bounds__(256) kivi_finalize_blocks_vec_kernel(const Src
         st8(scale_out + at, ss);
     }
     uint8_t *out = codes + ((int64_t)bh * cap_rows + row0 + (int64_t)j * kKeyBlock) * RB;
-#pragma unroll 4
-    for (int r = g; r < kKeyBlock; r += G) {
-        const F8 x = r < n_old ? ld8(res + (int64_t)r * D) : ld8(rows + (int64_t)r * D);
+#pragma unroll (KEEP ? RPG : 4)
+    for (int it = 0; it < RPG; it++) {
+        const int r = g + it * G;
+        F8 x;
+        if constexpr (KEEP) x = keep[it];
+        else x = r < n_old ? ld8(res + (int64_t)r * D) : ld8(rows + (int64_t)r * D);
         if constexpr (BITS == 8) {
             uint32_t w0, w1;
             affine_words8_u8(x.v, lo, scale, inv, w0, w1);
